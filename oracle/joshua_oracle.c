@@ -1,0 +1,412 @@
+/* Scalar CPU oracle: see joshua_oracle.h for what this is and how it is pinned.
+ * Build with -ffp-contract=off: every fused multiply-add below is explicit. */
+#include "joshua_oracle.h"
+#include "iq2xxs_grid_codes.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+static __thread char g_err[256];
+
+const char *orc_last_error(void) { return g_err; }
+
+int orc_fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return 1;
+}
+
+/* IEEE binary16 -> binary32, exact (the `half` crate's f16::to_f32). */
+float orc_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: normalise */
+            int e = -1;
+            do {
+                man <<= 1;
+                e++;
+            } while (!(man & 0x400u));
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+static inline uint16_t rd16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+static inline uint32_t rd32(const uint8_t *p) {
+    return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+int orc_block_geometry(uint32_t type, size_t *elems, size_t *bytes) {
+    size_t e, b;
+    switch (type) { /* reference: src/gguf_ext.rs:483-512 */
+    case ORC_TYPE_Q8_0: e = 32; b = 34; break;
+    case ORC_TYPE_Q2_K: e = 256; b = 84; break;
+    case ORC_TYPE_Q4_K: e = 256; b = 144; break;
+    case ORC_TYPE_Q6_K: e = 256; b = 210; break;
+    case ORC_TYPE_IQ2_XXS: e = 256; b = 66; break;
+    case ORC_TYPE_MXFP4: e = 32; b = 17; break;
+    default: return -1;
+    }
+    if (elems) *elems = e;
+    if (bytes) *bytes = b;
+    return 0;
+}
+
+/* Q4_K 6-bit scale/min pair j of the 12 packed bytes
+ * (reference: src/kquant_dot.rs:108-118). */
+void orc_q4k_scale_min(const uint8_t *s, int j, uint8_t *sc, uint8_t *mn) {
+    if (j < 4) {
+        *sc = s[j] & 63;
+        *mn = s[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4));
+        *mn = (uint8_t)((s[j + 4] >> 4) | ((s[j] >> 6) << 4));
+    }
+}
+
+/* IQ2_XXS codebook entry `code` expanded to its 8 values. */
+void orc_iq2xxs_grid(int code, uint8_t out[8]) {
+    unsigned c = ORC_IQ2XXS_GRID_TRITS[code];
+    for (int j = 0; j < 8; j++) {
+        unsigned t = c % 3;
+        c /= 3;
+        out[j] = (uint8_t)(8 + 17 * t + (t >> 1));
+    }
+}
+
+/* Sign byte for 7-bit index i: bit 7 makes the popcount even
+ * (reference table: src/iq2xxs.rs:441-449). */
+uint8_t orc_iq2xxs_signs(unsigned i) {
+    return (uint8_t)(i | ((unsigned)(__builtin_popcount(i) & 1) << 7));
+}
+
+/* MXFP4 shared exponent (reference: src/mxfp4.rs:67-75); returns 0 and sets
+ * *ok = 0 for the reserved 0xFF code. */
+float orc_e8m0(uint8_t e, int *ok) {
+    uint32_t bits;
+    *ok = 1;
+    if (e == 0) {
+        bits = 0x00400000u;
+    } else if (e == 0xFF) {
+        *ok = 0;
+        bits = 0;
+    } else {
+        bits = (uint32_t)e << 23;
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+static const float E2M1[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f,
+                               -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+
+/* ---- canonical decode ("to_float") ------------------------------------- */
+
+/* y = q * d (candle BlockQ8_0::to_float; the fused kernel computes the same
+ * product, reference: src/kquant_dot.rs:287-302). */
+static void deq_q8_0(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b));
+    for (int j = 0; j < 32; j++) y[j] = (float)(int8_t)b[2 + j] * d;
+}
+
+/* Two rounded operations per element: dl*q - ml
+ * (element map, reference: src/kquant_dot.rs:26-29,349-385). */
+static void deq_q2_k(const uint8_t *b, float *y) {
+    const uint8_t *scales = b, *qs = b + 16;
+    float d = orc_f16_to_f32(rd16(b + 80));
+    float dmin = orc_f16_to_f32(rd16(b + 82));
+    for (int e = 0; e < 256; e++) {
+        int sg = e / 128, r = e % 128;
+        uint8_t byte = qs[32 * sg + r % 32];
+        int q = (byte >> (2 * (r / 32))) & 3;
+        uint8_t s = scales[e / 16];
+        float dl = d * (float)(s & 0xF);
+        float ml = dmin * (float)(s >> 4);
+        y[e] = dl * (float)q - ml;
+    }
+}
+
+/* (element map, reference: src/kquant_dot.rs:30-33,430-465). */
+static void deq_q4_k(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b));
+    float dmin = orc_f16_to_f32(rd16(b + 2));
+    const uint8_t *scales = b + 4, *qs = b + 16;
+    for (int e = 0; e < 256; e++) {
+        uint8_t sc, mn;
+        orc_q4k_scale_min(scales, e / 32, &sc, &mn);
+        uint8_t byte = qs[32 * (e / 64) + e % 32];
+        int q = ((e / 32) % 2 == 0) ? (byte & 0xF) : (byte >> 4);
+        float d1 = d * (float)sc;
+        float m1 = dmin * (float)mn;
+        y[e] = d1 * (float)q - m1;
+    }
+}
+
+/* ggml block_q6_K {ql[128], qh[64], scales[16] i8, d f16}
+ * (reference: vendor/candle-metal-kernels/src/metal_src/quantized.metal:
+ * 198-203,6673-6694).  Operation order (d*sc)*q is the third-party
+ * to_float's and is unpinned at ulp level. */
+static void deq_q6_k(const uint8_t *b, float *y) {
+    const uint8_t *ql = b, *qh = b + 128;
+    const int8_t *sc = (const int8_t *)(b + 192);
+    float d = orc_f16_to_f32(rd16(b + 208));
+    for (int e = 0; e < 256; e++) {
+        int h = e / 128, r = e % 128, l = r % 32, t = r / 32;
+        uint8_t lo = ql[64 * h + l + 32 * (t & 1)];
+        int nib = (t < 2) ? (lo & 0xF) : (lo >> 4);
+        int hi2 = (qh[32 * h + l] >> (2 * t)) & 3;
+        int q = (nib | (hi2 << 4)) - 32;
+        y[e] = d * (float)sc[e / 16] * (float)q;
+    }
+}
+
+/* (reference: src/iq2xxs.rs:44-71). */
+static void deq_iq2_xxs(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b));
+    const uint8_t *qs = b + 2;
+    for (int ib32 = 0; ib32 < 8; ib32++) {
+        uint32_t lo = rd32(qs + 8 * ib32);
+        uint32_t hi = rd32(qs + 8 * ib32 + 4);
+        float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
+        for (int l = 0; l < 4; l++) {
+            uint8_t grid[8];
+            orc_iq2xxs_grid((lo >> (8 * l)) & 0xFF, grid);
+            uint8_t signs = orc_iq2xxs_signs((hi >> (7 * l)) & 127);
+            for (int j = 0; j < 8; j++) {
+                float s = (signs & (1u << j)) ? -1.0f : 1.0f;
+                y[ib32 * 32 + l * 8 + j] = db * (float)grid[j] * s;
+            }
+        }
+    }
+}
+
+/* (reference: src/mxfp4.rs:83-94). */
+static void deq_mxfp4(const uint8_t *b, float *y) {
+    int ok;
+    float d = orc_e8m0(b[0], &ok);
+    if (!ok) {
+        for (int j = 0; j < 32; j++) y[j] = 0.0f;
+        return;
+    }
+    for (int j = 0; j < 16; j++) {
+        y[j] = d * E2M1[b[1 + j] & 0xF];
+        y[j + 16] = d * E2M1[b[1 + j] >> 4];
+    }
+}
+
+typedef void (*deq_fn)(const uint8_t *, float *);
+
+static deq_fn deq_for(uint32_t type) {
+    switch (type) {
+    case ORC_TYPE_Q8_0: return deq_q8_0;
+    case ORC_TYPE_Q2_K: return deq_q2_k;
+    case ORC_TYPE_Q4_K: return deq_q4_k;
+    case ORC_TYPE_Q6_K: return deq_q6_k;
+    case ORC_TYPE_IQ2_XXS: return deq_iq2_xxs;
+    case ORC_TYPE_MXFP4: return deq_mxfp4;
+    default: return NULL;
+    }
+}
+
+int orc_dequantize(uint32_t type, const void *blocks, size_t nblocks, float *out) {
+    size_t elems, bytes;
+    deq_fn f = deq_for(type);
+    if (!f || orc_block_geometry(type, &elems, &bytes)) return orc_fail("unknown tensor type %u", type);
+    const uint8_t *p = (const uint8_t *)blocks;
+    for (size_t i = 0; i < nblocks; i++) f(p + i * bytes, out + i * elems);
+    return 0;
+}
+
+/* ---- matmul in the reference's x86_64 operation order ------------------ */
+
+/* Shared shape check (reference: src/quant_matmul.rs:133-165,
+ * src/iq2xxs.rs:126-153, src/mxfp4.rs:142-172).  Returns blocks per row
+ * through *bpr. */
+int orc_validate(uint32_t type, size_t m, size_t k, size_t n, size_t lhs_len, size_t nbytes,
+                 size_t dst_len, size_t *bpr) {
+    size_t elems, bytes;
+    if (orc_block_geometry(type, &elems, &bytes)) return orc_fail("unknown tensor type %u", type);
+    if (k % elems != 0)
+        return orc_fail("quantized matmul: k=%zu is not a multiple of the block size %zu", k, elems);
+    size_t per_row = k / elems;
+    if (nbytes % bytes != 0 || nbytes / bytes != n * per_row)
+        return orc_fail("quantized matmul: rhs holds %zu bytes, expected %zu blocks of %zu", nbytes,
+                        n * per_row, bytes);
+    if (lhs_len != m * k || dst_len != m * n)
+        return orc_fail("quantized matmul: lhs/dst sized %zu/%zu expected %zu/%zu", lhs_len, dst_len,
+                        m * k, m * n);
+    *bpr = per_row;
+    return 0;
+}
+
+/* The AVX2 horizontal sum (reference: src/simd.rs:198-206). */
+static inline float hsum8(const float a[8]) {
+    float s0 = a[0] + a[4], s1 = a[1] + a[5], s2 = a[2] + a[6], s3 = a[3] + a[7];
+    return (s0 + s2) + (s1 + s3);
+}
+
+/* One output element with the 8-lane accumulate of every AVX2 row kernel:
+ * lane c%8 takes column c, in column order. */
+static float dot8(const float *x, const float *w, size_t k) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (size_t c = 0; c < k; c++) acc[c & 7] = fmaf(x[c], w[c], acc[c & 7]);
+    return hsum8(acc);
+}
+
+/* Row decode as the fused kernels do it in registers. */
+
+/* w = q*d, one rounding (reference: src/kquant_dot.rs:287-302). */
+static void fused_w_q8_0(const uint8_t *b, float *w) {
+    float d = orc_f16_to_f32(rd16(b));
+    for (int j = 0; j < 32; j++) w[j] = (float)(int8_t)b[2 + j] * d;
+}
+
+/* w = fmsub(q, d*(s&15), dmin*(s>>4)) (reference: src/kquant_dot.rs:345-385). */
+static void fused_w_q2_k(const uint8_t *b, float *w) {
+    const uint8_t *scales = b, *qs = b + 16;
+    float d = orc_f16_to_f32(rd16(b + 80));
+    float dmin = orc_f16_to_f32(rd16(b + 82));
+    for (int sg = 0; sg < 2; sg++) {
+        for (int j = 0; j < 8; j++) {
+            uint8_t s = scales[sg * 8 + j];
+            float d1 = d * (float)(s & 0xF);
+            float m1 = dmin * (float)(s >> 4);
+            int shift = 2 * (j / 2);
+            const uint8_t *win = qs + sg * 32 + ((j % 2) ? 16 : 0);
+            for (int i = 0; i < 16; i++) {
+                float q = (float)((win[i] >> shift) & 3);
+                w[sg * 128 + 16 * j + i] = fmaf(q, d1, -m1);
+            }
+        }
+    }
+}
+
+/* w = fmsub(q, d*sc, dmin*m) (reference: src/kquant_dot.rs:426-466). */
+static void fused_w_q4_k(const uint8_t *b, float *w) {
+    float d = orc_f16_to_f32(rd16(b));
+    float dmin = orc_f16_to_f32(rd16(b + 2));
+    const uint8_t *scales = b + 4, *qs = b + 16;
+    for (int c = 0; c < 4; c++) {
+        for (int r = 0; r < 2; r++) {
+            uint8_t sc, mn;
+            orc_q4k_scale_min(scales, 2 * c + r, &sc, &mn);
+            float d1 = d * (float)sc;
+            float m1 = dmin * (float)mn;
+            for (int i = 0; i < 32; i++) {
+                uint8_t byte = qs[c * 32 + i];
+                float q = (float)(r == 0 ? (byte & 0xF) : (byte >> 4));
+                w[64 * c + 32 * r + i] = fmaf(q, d1, -m1);
+            }
+        }
+    }
+}
+
+/* v = (grid*sign)*db (reference: src/iq2xxs.rs:349-380). */
+static void fused_w_iq2_xxs(const uint8_t *b, float *w) {
+    float d = orc_f16_to_f32(rd16(b));
+    const uint8_t *qs = b + 2;
+    for (int ib32 = 0; ib32 < 8; ib32++) {
+        uint32_t lo = rd32(qs + 8 * ib32);
+        uint32_t hi = rd32(qs + 8 * ib32 + 4);
+        float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
+        for (int l = 0; l < 4; l++) {
+            uint8_t grid[8];
+            orc_iq2xxs_grid((lo >> (8 * l)) & 0xFF, grid);
+            uint8_t signs = orc_iq2xxs_signs((hi >> (7 * l)) & 0x7F);
+            for (int j = 0; j < 8; j++) {
+                float s = (signs & (1u << j)) ? -1.0f : 1.0f;
+                w[ib32 * 32 + l * 8 + j] = ((float)grid[j] * s) * db;
+            }
+        }
+    }
+}
+
+int orc_matmul_t(uint32_t type, size_t m, size_t k, size_t n, const float *lhs, size_t lhs_len,
+                 const void *blocks, size_t nbytes, float *dst, size_t dst_len) {
+    size_t bpr;
+    if (orc_validate(type, m, k, n, lhs_len, nbytes, dst_len, &bpr)) return 1;
+    if (m == 0 || n == 0) return 0; /* reference: src/quant_matmul.rs:176-178 */
+    size_t elems, bytes;
+    orc_block_geometry(type, &elems, &bytes);
+    const uint8_t *base = (const uint8_t *)blocks;
+
+    if (type == ORC_TYPE_MXFP4) {
+        /* Scalar only in the reference: per block a sequential sum with two
+         * roundings per term, added into a zero-filled dst
+         * (reference: src/mxfp4.rs:185-235). */
+        memset(dst, 0, dst_len * sizeof(float));
+        float w[32];
+        for (size_t row = 0; row < n; row++) {
+            for (size_t b = 0; b < bpr; b++) {
+                deq_mxfp4(base + (row * bpr + b) * 17, w);
+                for (size_t i = 0; i < m; i++) {
+                    const float *a = lhs + i * k + b * 32;
+                    float acc = 0.0f;
+                    for (int j = 0; j < 32; j++) acc += a[j] * w[j];
+                    dst[i * n + row] += acc;
+                }
+            }
+        }
+        return 0;
+    }
+
+    void (*rowdec)(const uint8_t *, float *);
+    switch (type) {
+    case ORC_TYPE_Q8_0: rowdec = fused_w_q8_0; break;
+    case ORC_TYPE_Q2_K: rowdec = fused_w_q2_k; break;
+    case ORC_TYPE_Q4_K: rowdec = fused_w_q4_k; break;
+    case ORC_TYPE_IQ2_XXS: rowdec = fused_w_iq2_xxs; break;
+    /* No fused kernel: to_float into a k-float scratch, then the 8-lane dot
+     * (reference: src/quant_matmul.rs:228-248,292-325). */
+    case ORC_TYPE_Q6_K: rowdec = deq_q6_k; break;
+    default: return orc_fail("unknown tensor type %u", type);
+    }
+    float *w = (float *)malloc(k * sizeof(float));
+    if (!w) return orc_fail("out of memory");
+    for (size_t row = 0; row < n; row++) {
+        for (size_t b = 0; b < bpr; b++) rowdec(base + (row * bpr + b) * bytes, w + b * elems);
+        for (size_t i = 0; i < m; i++) dst[i * n + row] = dot8(lhs + i * k, w, k);
+    }
+    free(w);
+    return 0;
+}
+
+int orc_iq2xxs_matmul_scalar(size_t m, size_t k, size_t n, const float *lhs, size_t lhs_len,
+                             const void *blocks, size_t nbytes, float *dst, size_t dst_len) {
+    size_t bpr;
+    if (orc_validate(ORC_TYPE_IQ2_XXS, m, k, n, lhs_len, nbytes, dst_len, &bpr)) return 1;
+    if (m == 0 || n == 0) return 0;
+    memset(dst, 0, dst_len * sizeof(float));
+    const uint8_t *base = (const uint8_t *)blocks;
+    float w[256];
+    for (size_t row = 0; row < n; row++) {
+        for (size_t b = 0; b < bpr; b++) {
+            deq_iq2_xxs(base + (row * bpr + b) * 66, w);
+            for (size_t i = 0; i < m; i++) {
+                const float *a = lhs + i * k + b * 256;
+                float acc = 0.0f;
+                for (int j = 0; j < 256; j++) acc += a[j] * w[j];
+                dst[i * n + row] += acc;
+            }
+        }
+    }
+    return 0;
+}
