@@ -1,0 +1,118 @@
+/* joshua_hip.h — C ABI of libjoshua_hip.so: GGUF quantized matmul on one
+ * MI355X (gfx950).
+ *
+ * The entry points mirror, one to one, the operator contract the reference
+ * engine calls on its quantized-weight storage objects
+ * (reference: src/mmap_tensor.rs:127-203, trait methods dtype / matmul_t /
+ * embedding / dequantize / storage_size_in_bytes, and the free functions
+ * src/quant_matmul.rs:110-118 matmul_kquant, src/kquant_dot.rs:126-143
+ * try_matmul_fused, src/iq2xxs.rs:103-111 matmul_t, src/mxfp4.rs:120-128
+ * matmul_t).  A Rust `QuantizedType` implementation binds them with a plain
+ * `extern "C"` block; no C++ or torch types cross this boundary.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and nonzero on failure (the
+ *     convention of the reference's plugin ABI, src/npu/mod.rs:48-50).  On
+ *     failure nothing has been written to the destination and
+ *     jq_last_error() describes the problem (thread local), in the words of
+ *     the reference's `bail!` messages where one exists.
+ *   - dst[m,n] = lhs[m,k] . W[n,k]^T, all row-major, dst[i*n + j]; dst is
+ *     assigned, never accumulated into (reference: src/quant_matmul.rs:105-109,
+ *     src/mxfp4.rs:185-189).
+ *   - Blocks stay in their native packed GGUF layout in HBM; no f32 copy of a
+ *     weight is ever made.
+ *   - `stream` is a hipStream_t passed as void*; NULL means the default
+ *     stream.  Calls only enqueue work unless they take host pointers.
+ *   - A jq_weight is immutable after creation and may be used by several host
+ *     threads at once (reference: src/mmap_tensor.rs:86-91).
+ */
+#ifndef JOSHUA_HIP_H
+#define JOSHUA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Raw GGUF tensor type ids (reference: src/gguf_ext.rs:483-512,
+ * src/iq2xxs.rs:23, src/mxfp4.rs:39). */
+#define JQ_TYPE_Q8_0 8u
+#define JQ_TYPE_Q2_K 10u
+#define JQ_TYPE_Q4_K 12u
+#define JQ_TYPE_Q6_K 14u
+#define JQ_TYPE_IQ2_XXS 16u
+#define JQ_TYPE_MXFP4 39u
+
+typedef struct jq_weight jq_weight;
+
+/* Message for the last failure on the calling thread
+ * (replaces candle's Error::Msg strings). */
+const char *jq_last_error(void);
+
+/* Elements and bytes per block of a type id; nonzero for an unknown id
+ * (reference: src/gguf_ext.rs:483-512 type_size_bytes). */
+int jq_block_geometry(uint32_t ggml_type, size_t *elems, size_t *bytes);
+
+/* Selects the HIP device for this process and builds the constant tables.
+ * Optional: the first upload does it for device 0. */
+int jq_init(int device);
+
+/* Copies `nbytes` of packed blocks for an n x k weight (a tensor, or one
+ * expert's slice of the mapping) into HBM, once.  `blocks` is a host pointer
+ * when src_is_device == 0, else a device pointer.  Fails unless
+ * nbytes == n * k / block_elems * block_bytes
+ * (reference: src/mmap_tensor.rs:520-565 borrowed_qtensor_raw,
+ * src/mmap_tensor.rs:105-123 borrow bounds check). */
+int jq_upload(uint32_t ggml_type, const void *blocks, size_t nbytes, size_t n, size_t k,
+              int src_is_device, jq_weight **out);
+
+/* A weight that aliases `nbytes` at `byte_offset` inside `parent` without
+ * copying: one expert of a stacked [n_expert, n, k] tensor
+ * (reference: src/quantized_qwen3_moe.rs:596-631 split_experts,
+ * src/mmap_tensor.rs:614-655 borrowed_range).  The parent must outlive it. */
+int jq_view(const jq_weight *parent, size_t byte_offset, size_t n, size_t k, jq_weight **out);
+
+void jq_free(jq_weight *w);
+
+/* Accessors (reference: src/mmap_tensor.rs:128-130,175-189). */
+uint32_t jq_dtype(const jq_weight *w);
+size_t jq_rows(const jq_weight *w);
+size_t jq_cols(const jq_weight *w);
+size_t jq_storage_size_in_bytes(const jq_weight *w);
+const void *jq_device_ptr(const jq_weight *w);
+
+/* THE call: dst[m,n] = lhs[m,k] . W^T.  lhs_len / dst_len are element counts
+ * and must equal m*k / m*n; m == 0 or n == 0 succeeds without work
+ * (reference: src/mmap_tensor.rs:132-134 matmul_t,
+ * src/quant_matmul.rs:133-178 validate + empty case).  With
+ * ptrs_are_device == 0 the call stages lhs/dst through HBM and returns after
+ * the result has landed in dst. */
+int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, float *dst,
+                size_t dst_len, int ptrs_are_device, void *stream);
+
+/* The free-function form over raw device-resident block bytes: runs the fused
+ * kernel for `ggml_type` or declines (returns 1, dst untouched) when the type
+ * has no kernel or nbytes is not a whole number of blocks
+ * (reference: src/kquant_dot.rs:126-143 try_matmul_fused). */
+int jq_try_matmul_fused(uint32_t ggml_type, size_t m, size_t k, size_t n, const float *lhs_dev,
+                        const void *blocks_dev, size_t nbytes, float *dst_dev, void *stream);
+
+/* Canonical decode of the whole weight to f32, out_len == n*k
+ * (reference: src/mmap_tensor.rs:169-173 dequantize,
+ * src/quant_matmul.rs:36-103 decode_raw_to_f32). */
+int jq_dequantize(const jq_weight *w, float *out, size_t out_len, int out_is_device, void *stream);
+
+/* Row gather with decode: out[i, :] = decode(W[ids[i], :]); an id >= n fails
+ * (reference: src/mmap_tensor.rs:140-167 embedding). */
+int jq_embedding(const jq_weight *w, const uint32_t *ids, size_t n_ids, float *out, size_t out_len,
+                 int ptrs_are_device, void *stream);
+
+/* Blocks until everything enqueued on `stream` has finished. */
+int jq_stream_synchronize(void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

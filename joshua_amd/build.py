@@ -1,0 +1,43 @@
+"""Builds the native libraries in-tree: libjoshua_hip.so (HIP, gfx950) and the
+host-only synthetic-input library."""
+from __future__ import annotations
+
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+HIP_LIB = os.path.join(HERE, "libjoshua_hip.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+    # keep the compiler from forming packed-f32 instructions out of scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def hip_sources() -> list[str]:
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def build_hip(verbose: bool = False) -> str:
+    cmd = ["hipcc", *HIPCC_FLAGS, "-o", HIP_LIB, *hip_sources()]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed:\n{err}")
+    if verbose and err.strip():
+        print(err)
+    return HIP_LIB
+
+
+def build_all(verbose: bool = False) -> None:
+    from . import synth
+    build_hip(verbose)
+    synth.build()
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built", HIP_LIB)

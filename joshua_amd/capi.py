@@ -1,0 +1,194 @@
+"""ctypes binding of ``libjoshua_hip.so`` (C ABI in ``include/joshua_hip.h``).
+
+Everything here is plumbing: it passes plain pointers and sizes through the C
+ABI exactly as a Rust ``extern "C"`` block would.  There is no CPU fallback: a
+missing or unloadable library raises, and so does every failed call.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libjoshua_hip.so")
+
+Q8_0, Q2_K, Q4_K, Q6_K, IQ2_XXS, MXFP4 = 8, 10, 12, 14, 16, 39
+ALL_TYPES = (Q8_0, Q2_K, Q4_K, Q6_K, IQ2_XXS, MXFP4)
+TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "IQ2_XXS", MXFP4: "MXFP4"}
+
+# Every symbol include/joshua_hip.h declares.
+EXPORTS = (
+    "jq_last_error", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
+    "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_try_matmul_fused", "jq_dequantize",
+    "jq_embedding", "jq_stream_synchronize",
+)
+
+
+class JoshuaHipError(RuntimeError):
+    """A C-ABI call returned nonzero; the message is jq_last_error()."""
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise JoshuaHipError(
+                f"{LIB_PATH} is missing: build it with `python -m joshua_amd.build` (there is no CPU fallback)")
+        # One process must hold one HIP runtime.  PyTorch ships its own copy of
+        # libamdhip64 under the same soname the library links against, so when
+        # torch is installed it is loaded first and the loader binds this
+        # library to that copy; without torch the system runtime is used.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
+        L = ctypes.CDLL(LIB_PATH)
+        sz, u32, vp, i32 = ctypes.c_size_t, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_int
+        L.jq_last_error.restype = ctypes.c_char_p
+        L.jq_block_geometry.argtypes = [u32, ctypes.POINTER(sz), ctypes.POINTER(sz)]
+        L.jq_init.argtypes = [i32]
+        L.jq_upload.argtypes = [u32, vp, sz, sz, sz, i32, ctypes.POINTER(vp)]
+        L.jq_view.argtypes = [vp, sz, sz, sz, ctypes.POINTER(vp)]
+        L.jq_free.argtypes = [vp]
+        L.jq_free.restype = None
+        L.jq_dtype.argtypes = [vp]
+        L.jq_dtype.restype = u32
+        for f in (L.jq_rows, L.jq_cols, L.jq_storage_size_in_bytes):
+            f.argtypes = [vp]
+            f.restype = sz
+        L.jq_device_ptr.argtypes = [vp]
+        L.jq_device_ptr.restype = vp
+        L.jq_matmul_t.argtypes = [vp, sz, vp, sz, vp, sz, i32, vp]
+        L.jq_try_matmul_fused.argtypes = [u32, sz, sz, sz, vp, vp, sz, vp, vp]
+        L.jq_dequantize.argtypes = [vp, vp, sz, i32, vp]
+        L.jq_embedding.argtypes = [vp, vp, sz, vp, sz, i32, vp]
+        L.jq_stream_synchronize.argtypes = [vp]
+        _lib = L
+    return _lib
+
+
+def last_error() -> str:
+    return lib().jq_last_error().decode()
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise JoshuaHipError(last_error())
+
+
+def block_geometry(qtype: int) -> tuple[int, int]:
+    e, b = ctypes.c_size_t(), ctypes.c_size_t()
+    _check(lib().jq_block_geometry(qtype, ctypes.byref(e), ctypes.byref(b)))
+    return e.value, b.value
+
+
+def init(device: int = 0) -> None:
+    _check(lib().jq_init(device))
+
+
+def _host_bytes(blocks) -> np.ndarray:
+    a = blocks if isinstance(blocks, np.ndarray) else np.frombuffer(blocks, dtype=np.uint8)
+    return np.ascontiguousarray(a.view(np.uint8).reshape(-1))
+
+
+class Weight:
+    """An n x k quantized weight resident in HBM in native block layout: the
+    counterpart of the reference's borrowed storage objects
+    (reference: src/mmap_tensor.rs:54-60,127-203)."""
+
+    def __init__(self, handle: int, parent: "Weight | None" = None):
+        self._h = ctypes.c_void_p(handle)
+        self._parent = parent  # keeps the aliased allocation alive
+
+    @classmethod
+    def upload(cls, qtype: int, blocks, n: int, k: int) -> "Weight":
+        raw = _host_bytes(blocks)
+        out = ctypes.c_void_p()
+        _check(lib().jq_upload(qtype, raw.ctypes.data, raw.size, n, k, 0, ctypes.byref(out)))
+        return cls(out.value)
+
+    @classmethod
+    def upload_device(cls, qtype: int, dev_ptr: int, nbytes: int, n: int, k: int) -> "Weight":
+        out = ctypes.c_void_p()
+        _check(lib().jq_upload(qtype, dev_ptr, nbytes, n, k, 1, ctypes.byref(out)))
+        return cls(out.value)
+
+    def view(self, byte_offset: int, n: int, k: int) -> "Weight":
+        out = ctypes.c_void_p()
+        _check(lib().jq_view(self._h, byte_offset, n, k, ctypes.byref(out)))
+        return Weight(out.value, parent=self)
+
+    def close(self) -> None:
+        if self._h:
+            lib().jq_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def handle(self) -> ctypes.c_void_p:
+        return self._h
+
+    @property
+    def dtype(self) -> int:
+        return lib().jq_dtype(self._h)
+
+    @property
+    def n(self) -> int:
+        return lib().jq_rows(self._h)
+
+    @property
+    def k(self) -> int:
+        return lib().jq_cols(self._h)
+
+    @property
+    def nbytes(self) -> int:
+        return lib().jq_storage_size_in_bytes(self._h)
+
+    @property
+    def device_ptr(self) -> int:
+        return lib().jq_device_ptr(self._h)
+
+    # -- host-pointer calls (numpy in, numpy out) --------------------------------
+    def matmul_t(self, m: int, lhs: np.ndarray, dst: np.ndarray | None = None) -> np.ndarray:
+        x = np.ascontiguousarray(np.asarray(lhs, dtype=np.float32).reshape(-1))
+        if dst is None:
+            dst = np.empty(m * self.n, dtype=np.float32)
+        assert dst.dtype == np.float32 and dst.flags.c_contiguous
+        _check(lib().jq_matmul_t(self._h, m, x.ctypes.data, x.size, dst.ctypes.data, dst.size, 0, None))
+        return dst.reshape(m, self.n) if dst.size == m * self.n else dst
+
+    def dequantize(self) -> np.ndarray:
+        out = np.empty(self.n * self.k, dtype=np.float32)
+        _check(lib().jq_dequantize(self._h, out.ctypes.data, out.size, 0, None))
+        return out.reshape(self.n, self.k)
+
+    def embedding(self, ids) -> np.ndarray:
+        ids = np.ascontiguousarray(ids, dtype=np.uint32)
+        out = np.empty(ids.size * self.k, dtype=np.float32)
+        _check(lib().jq_embedding(self._h, ids.ctypes.data, ids.size, out.ctypes.data, out.size, 0, None))
+        return out.reshape(ids.size, self.k)
+
+    # -- device-pointer calls (raw addresses; inputs already in HBM) -------------
+    def matmul_t_dev(self, m: int, lhs_ptr: int, lhs_len: int, dst_ptr: int, dst_len: int, stream: int = 0) -> None:
+        _check(lib().jq_matmul_t(self._h, m, lhs_ptr, lhs_len, dst_ptr, dst_len, 1, stream or None))
+
+
+def try_matmul_fused(qtype: int, mkn, lhs_ptr: int, blocks_ptr: int, nbytes: int, dst_ptr: int, stream: int = 0) -> bool:
+    """True when a kernel ran; False when the call declined (dst untouched), as
+    the reference's free function does (src/kquant_dot.rs:120-133)."""
+    m, k, n = mkn
+    return lib().jq_try_matmul_fused(qtype, m, k, n, lhs_ptr, blocks_ptr, nbytes, dst_ptr, stream or None) == 0
+
+
+def stream_synchronize(stream: int = 0) -> None:
+    _check(lib().jq_stream_synchronize(stream or None))

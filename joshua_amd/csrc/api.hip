@@ -1,0 +1,337 @@
+// C ABI of libjoshua_hip.so (declared in include/joshua_hip.h): weight objects
+// resident in HBM in native GGUF block layout, shape validation with the
+// reference's error behaviour, and kernel dispatch.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "../../include/joshua_hip.h"
+#include "kernels_valu.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return 1;
+}
+
+#define HIP_TRY(expr)                                                                      \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess) return fail("%s: %s", #expr, hipGetErrorString(e_));         \
+    } while (0)
+
+struct Geometry {
+    size_t elems, bytes;
+};
+
+bool geometry(uint32_t t, Geometry *g) {
+    switch (t) {  // reference: src/gguf_ext.rs:483-512
+    case JQ_TYPE_Q8_0: *g = {32, 34}; return true;
+    case JQ_TYPE_Q2_K: *g = {256, 84}; return true;
+    case JQ_TYPE_Q4_K: *g = {256, 144}; return true;
+    case JQ_TYPE_Q6_K: *g = {256, 210}; return true;
+    case JQ_TYPE_IQ2_XXS: *g = {256, 66}; return true;
+    case JQ_TYPE_MXFP4: *g = {32, 17}; return true;
+    default: return false;
+    }
+}
+
+const char *type_name(uint32_t t) {
+    switch (t) {
+    case JQ_TYPE_Q8_0: return "quantized";
+    case JQ_TYPE_Q2_K: return "quantized";
+    case JQ_TYPE_Q4_K: return "quantized";
+    case JQ_TYPE_Q6_K: return "quantized";
+    case JQ_TYPE_IQ2_XXS: return "iq2_xxs";
+    case JQ_TYPE_MXFP4: return "mxfp4";
+    default: return "unknown";
+    }
+}
+
+std::once_flag g_init_once;
+int g_init_rc = 0;
+int g_device = 0;
+
+int do_init(int device) {
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail("jq_init: device %d out of range (%d visible)", device, count);
+    HIP_TRY(hipSetDevice(device));
+    g_device = device;
+    return 0;
+}
+
+int ensure_init() {
+    std::call_once(g_init_once, [] { g_init_rc = do_init(0); });
+    return g_init_rc;
+}
+
+}  // namespace
+
+struct jq_weight {
+    uint32_t type;
+    size_t n, k, nbytes, row_bytes;
+    uint8_t *dev;
+    bool owns;
+};
+
+namespace {
+
+// Shape checks of the reference entry points, in their order and wording
+// (reference: src/quant_matmul.rs:133-165, src/iq2xxs.rs:126-153,
+// src/mxfp4.rs:142-172).
+int validate(uint32_t type, size_t m, size_t k, size_t n, size_t lhs_len, size_t nbytes, size_t dst_len) {
+    Geometry g;
+    if (!geometry(type, &g)) return fail("unsupported tensor type id %u", type);
+    if (k % g.elems != 0)
+        return fail("%s matmul: k=%zu is not a multiple of the block size %zu", type_name(type), k, g.elems);
+    size_t bpr = k / g.elems;
+    if (nbytes % g.bytes != 0 || nbytes / g.bytes != n * bpr)
+        return fail("%s matmul: rhs holds %zu blocks, expected %zu", type_name(type), nbytes / g.bytes, n * bpr);
+    if (lhs_len != m * k || dst_len != m * n)
+        return fail("%s matmul: lhs/dst sized %zu/%zu expected %zu/%zu", type_name(type), lhs_len, dst_len, m * k,
+                    m * n);
+    return 0;
+}
+
+template <class Q>
+void launch_rows(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                 hipStream_t s) {
+    dim3 grid((unsigned)((n + jq::ROWS_PER_WG - 1) / jq::ROWS_PER_WG)), block(64 * jq::ROWS_PER_WG);
+    if (m == 1)
+        hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 1>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
+    else if (m == 2)
+        hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 2>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
+    else
+        hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 4>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
+}
+
+// All pointers are device pointers; shapes already validated; m, n > 0.
+int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
+                    size_t k, size_t n, hipStream_t s) {
+    if (m > 0x7FFFFFFF || k > 0x7FFFFFFF || n > 0x7FFFFFFF) return fail("matmul: dimension exceeds 2^31-1");
+    switch (type) {
+    case JQ_TYPE_Q8_0: launch_rows<jq::Q8_0>(W, row_bytes, X, Y, m, k, n, s); break;
+    case JQ_TYPE_Q2_K: launch_rows<jq::Q2_K>(W, row_bytes, X, Y, m, k, n, s); break;
+    case JQ_TYPE_Q4_K: launch_rows<jq::Q4_K>(W, row_bytes, X, Y, m, k, n, s); break;
+    case JQ_TYPE_Q6_K: launch_rows<jq::Q6_K>(W, row_bytes, X, Y, m, k, n, s); break;
+    case JQ_TYPE_IQ2_XXS: launch_rows<jq::IQ2_XXS>(W, row_bytes, X, Y, m, k, n, s); break;
+    case JQ_TYPE_MXFP4: launch_rows<jq::MXFP4>(W, row_bytes, X, Y, m, k, n, s); break;
+    default: return fail("unsupported tensor type id %u", type);
+    }
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+template <class Q>
+void launch_decode(const jq_weight *w, const uint32_t *ids, float *out, size_t rows, hipStream_t s) {
+    size_t units = rows * (w->k / Q::BLOCK_ELEMS) * Q::UNITS;
+    unsigned blocks = (unsigned)std::min<size_t>((units + 255) / 256, 65535u * 16u);
+    if (blocks == 0) return;
+    hipLaunchKernelGGL((jq::decode_rows<Q>), dim3(blocks), dim3(256), 0, s, w->dev, w->row_bytes, ids, out, rows,
+                       (int)w->k);
+}
+
+int dispatch_decode(const jq_weight *w, const uint32_t *ids, float *out, size_t rows, hipStream_t s) {
+    switch (w->type) {
+    case JQ_TYPE_Q8_0: launch_decode<jq::Q8_0>(w, ids, out, rows, s); break;
+    case JQ_TYPE_Q2_K: launch_decode<jq::Q2_K>(w, ids, out, rows, s); break;
+    case JQ_TYPE_Q4_K: launch_decode<jq::Q4_K>(w, ids, out, rows, s); break;
+    case JQ_TYPE_Q6_K: launch_decode<jq::Q6_K>(w, ids, out, rows, s); break;
+    case JQ_TYPE_IQ2_XXS: launch_decode<jq::IQ2_XXS>(w, ids, out, rows, s); break;
+    case JQ_TYPE_MXFP4: launch_decode<jq::MXFP4>(w, ids, out, rows, s); break;
+    default: return fail("unsupported tensor type id %u", w->type);
+    }
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// Frees a device allocation when it goes out of scope.
+struct DevBuf {
+    void *p = nullptr;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 1); }
+};
+
+}  // namespace
+
+extern "C" {
+
+const char *jq_last_error(void) { return g_err; }
+
+int jq_block_geometry(uint32_t ggml_type, size_t *elems, size_t *bytes) {
+    Geometry g;
+    if (!geometry(ggml_type, &g)) return fail("unsupported tensor type id %u", ggml_type);
+    if (elems) *elems = g.elems;
+    if (bytes) *bytes = g.bytes;
+    return 0;
+}
+
+int jq_init(int device) {
+    bool first = false;
+    std::call_once(g_init_once, [&] {
+        first = true;
+        g_init_rc = do_init(device);
+    });
+    if (!first && g_init_rc == 0 && device != g_device)
+        return fail("jq_init: already initialised on device %d", g_device);
+    return g_init_rc;
+}
+
+int jq_upload(uint32_t ggml_type, const void *blocks, size_t nbytes, size_t n, size_t k, int src_is_device,
+              jq_weight **out) {
+    if (!out) return fail("jq_upload: out is null");
+    *out = nullptr;
+    Geometry g;
+    if (!geometry(ggml_type, &g)) return fail("unsupported tensor type id %u", ggml_type);
+    if (k % g.elems != 0)
+        return fail("%s tensor: k=%zu is not a multiple of the block size %zu", type_name(ggml_type), k, g.elems);
+    size_t want = n * (k / g.elems) * g.bytes;
+    if (nbytes != want)
+        return fail("%s tensor: %zu bytes for %zu x %zu elements (expected %zu)", type_name(ggml_type), nbytes, n, k,
+                    want);
+    if (nbytes && !blocks) return fail("jq_upload: blocks is null");
+    if (ensure_init()) return 1;
+    uint8_t *dev = nullptr;
+    // Kernels read a row in 16-byte pieces that may start before the unit they
+    // need; 64 spare bytes keep every such read inside the allocation.
+    HIP_TRY(hipMalloc((void **)&dev, nbytes + 64));
+    hipError_t e = hipMemcpy(dev, blocks, nbytes, src_is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemset(dev + nbytes, 0, 64);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return fail("jq_upload: copy to device failed: %s", hipGetErrorString(e));
+    }
+    *out = new jq_weight{ggml_type, n, k, nbytes, (k / g.elems) * g.bytes, dev, true};
+    return 0;
+}
+
+int jq_view(const jq_weight *parent, size_t byte_offset, size_t n, size_t k, jq_weight **out) {
+    if (!out) return fail("jq_view: out is null");
+    *out = nullptr;
+    if (!parent) return fail("jq_view: parent is null");
+    Geometry g;
+    geometry(parent->type, &g);
+    if (k % g.elems != 0)
+        return fail("%s tensor: k=%zu is not a multiple of the block size %zu", type_name(parent->type), k, g.elems);
+    size_t need = n * (k / g.elems) * g.bytes;
+    // reference: src/mmap_tensor.rs:105-110 (range must lie inside the mapping)
+    if (byte_offset > parent->nbytes || need > parent->nbytes - byte_offset)
+        return fail("jq_view: range %zu+%zu exceeds the parent's %zu bytes", byte_offset, need, parent->nbytes);
+    if (byte_offset % g.bytes != 0) return fail("jq_view: offset %zu is not a whole number of blocks", byte_offset);
+    *out = new jq_weight{parent->type, n, k, need, (k / g.elems) * g.bytes, parent->dev + byte_offset, false};
+    return 0;
+}
+
+void jq_free(jq_weight *w) {
+    if (!w) return;
+    if (w->owns && w->dev) (void)hipFree(w->dev);
+    delete w;
+}
+
+uint32_t jq_dtype(const jq_weight *w) { return w ? w->type : 0; }
+size_t jq_rows(const jq_weight *w) { return w ? w->n : 0; }
+size_t jq_cols(const jq_weight *w) { return w ? w->k : 0; }
+size_t jq_storage_size_in_bytes(const jq_weight *w) { return w ? w->nbytes : 0; }
+const void *jq_device_ptr(const jq_weight *w) { return w ? w->dev : nullptr; }
+
+int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, float *dst, size_t dst_len,
+                int ptrs_are_device, void *stream) {
+    if (!w) return fail("jq_matmul_t: weight is null");
+    if (validate(w->type, m, w->k, w->n, lhs_len, w->nbytes, dst_len)) return 1;
+    if (m == 0 || w->n == 0) return 0;  // reference: src/quant_matmul.rs:176-178
+    if (!lhs || !dst) return fail("jq_matmul_t: lhs/dst is null");
+    hipStream_t s = (hipStream_t)stream;
+    if (ptrs_are_device) return dispatch_matmul(w->type, w->dev, w->row_bytes, lhs, dst, m, w->k, w->n, s);
+    DevBuf x, y;
+    HIP_TRY(x.alloc(lhs_len * sizeof(float)));
+    HIP_TRY(y.alloc(dst_len * sizeof(float)));
+    HIP_TRY(hipMemcpyAsync(x.p, lhs, lhs_len * sizeof(float), hipMemcpyHostToDevice, s));
+    if (dispatch_matmul(w->type, w->dev, w->row_bytes, (const float *)x.p, (float *)y.p, m, w->k, w->n, s)) return 1;
+    HIP_TRY(hipMemcpyAsync(dst, y.p, dst_len * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int jq_try_matmul_fused(uint32_t ggml_type, size_t m, size_t k, size_t n, const float *lhs_dev,
+                        const void *blocks_dev, size_t nbytes, float *dst_dev, void *stream) {
+    Geometry g;
+    // reference: src/kquant_dot.rs:158-163 (unknown dtype declines),
+    // :217-224 (ragged byte length or k shorter than a block declines)
+    if (!geometry(ggml_type, &g)) return fail("declined: no fused kernel for tensor type id %u", ggml_type);
+    if (nbytes % g.bytes != 0) return fail("declined: %zu bytes is not a whole number of %zu byte blocks", nbytes, g.bytes);
+    if (k / g.elems == 0 || k % g.elems != 0) return fail("declined: k=%zu is not a positive multiple of %zu", k, g.elems);
+    if (nbytes / g.bytes != n * (k / g.elems))
+        return fail("declined: rhs holds %zu blocks, expected %zu", nbytes / g.bytes, n * (k / g.elems));
+    if (m == 0 || n == 0) return 0;
+    if (!lhs_dev || !blocks_dev || !dst_dev) return fail("declined: null pointer");
+    if (ensure_init()) return 1;
+    return dispatch_matmul(ggml_type, (const uint8_t *)blocks_dev, (k / g.elems) * g.bytes, lhs_dev, dst_dev, m, k, n,
+                           (hipStream_t)stream);
+}
+
+int jq_dequantize(const jq_weight *w, float *out, size_t out_len, int out_is_device, void *stream) {
+    if (!w) return fail("jq_dequantize: weight is null");
+    if (out_len != w->n * w->k)
+        return fail("%s: output holds %zu values, expected %zu", type_name(w->type), out_len, w->n * w->k);
+    if (out_len == 0) return 0;
+    if (!out) return fail("jq_dequantize: out is null");
+    hipStream_t s = (hipStream_t)stream;
+    if (out_is_device) return dispatch_decode(w, nullptr, out, w->n, s);
+    DevBuf y;
+    HIP_TRY(y.alloc(out_len * sizeof(float)));
+    if (dispatch_decode(w, nullptr, (float *)y.p, w->n, s)) return 1;
+    HIP_TRY(hipMemcpyAsync(out, y.p, out_len * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int jq_embedding(const jq_weight *w, const uint32_t *ids, size_t n_ids, float *out, size_t out_len,
+                 int ptrs_are_device, void *stream) {
+    if (!w) return fail("jq_embedding: weight is null");
+    if (out_len != n_ids * w->k)
+        return fail("quantized embedding: output holds %zu values, expected %zu", out_len, n_ids * w->k);
+    if (n_ids == 0) return 0;
+    if (!ids || !out) return fail("jq_embedding: ids/out is null");
+    hipStream_t s = (hipStream_t)stream;
+    // The id check happens on the host, as in the reference
+    // (src/mmap_tensor.rs:157-161); device-resident ids are read back for it.
+    std::vector<uint32_t> host_ids;
+    const uint32_t *check = ids;
+    if (ptrs_are_device) {
+        host_ids.resize(n_ids);
+        HIP_TRY(hipMemcpyAsync(host_ids.data(), ids, n_ids * sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+        check = host_ids.data();
+    }
+    for (size_t i = 0; i < n_ids; i++)
+        if (check[i] >= w->n) return fail("embedding id %u is out of range for %zu rows", check[i], w->n);
+    if (ptrs_are_device) return dispatch_decode(w, ids, out, n_ids, s);
+    DevBuf di, y;
+    HIP_TRY(di.alloc(n_ids * sizeof(uint32_t)));
+    HIP_TRY(y.alloc(out_len * sizeof(float)));
+    HIP_TRY(hipMemcpyAsync(di.p, ids, n_ids * sizeof(uint32_t), hipMemcpyHostToDevice, s));
+    if (dispatch_decode(w, (const uint32_t *)di.p, (float *)y.p, n_ids, s)) return 1;
+    HIP_TRY(hipMemcpyAsync(out, y.p, out_len * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int jq_stream_synchronize(void *stream) {
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,228 @@
+// GGUF block formats decoded in registers (gfx950 device code).
+//
+// A block is cut into "units": the piece one lane decodes at a time, chosen
+// so that a unit reads 16-byte runs of packed values and covers 32 or 64
+// consecutive-ish elements.  Every decoder writes the same f32 weights the
+// reference's fused CPU kernels build in registers, with the same rounding
+// steps (products d*sc and dmin*m rounded to f32 first, then one fused
+// multiply-subtract per element).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "iq2xxs_grid_codes.h"
+
+namespace jq {
+
+template <class T>
+__device__ __forceinline__ T ld(const uint8_t *p) {
+    T v;
+    __builtin_memcpy(&v, p, sizeof(T));
+    return v;
+}
+
+__device__ __forceinline__ float f16_bits(uint32_t h) {
+    return __half2float(__ushort_as_half((unsigned short)(h & 0xFFFFu)));
+}
+
+// byte i (0..11) of the 12 packed Q4_K scale bytes held in three dwords
+__device__ __forceinline__ uint32_t q4k_byte(uint32_t s0, uint32_t s1, uint32_t s2, int i) {
+    uint32_t w = i < 4 ? s0 : (i < 8 ? s1 : s2);
+    return (w >> (8 * (i & 3))) & 0xFFu;
+}
+
+// 6-bit (scale, min) pair j of a Q4_K block (reference: src/kquant_dot.rs:108-118)
+__device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j, uint32_t &sc,
+                                              uint32_t &mn) {
+    if (j < 4) {
+        sc = q4k_byte(s0, s1, s2, j) & 63u;
+        mn = q4k_byte(s0, s1, s2, j + 4) & 63u;
+    } else {
+        uint32_t hi = q4k_byte(s0, s1, s2, j + 4);
+        sc = (hi & 0xFu) | ((q4k_byte(s0, s1, s2, j - 4) >> 6) << 4);
+        mn = (hi >> 4) | ((q4k_byte(s0, s1, s2, j) >> 6) << 4);
+    }
+}
+
+// IQ2_XXS codebook expanded at compile time to 256 x 8 bytes (value j of entry
+// c in byte j), from the base-3 packed form in iq2xxs_grid_codes.h.
+struct Tables {
+    uint64_t iq2xxs_grid[256];
+    constexpr Tables() : iq2xxs_grid{} {
+        for (int i = 0; i < 256; i++) {
+            unsigned c = JQ_IQ2XXS_GRID_TRITS[i];
+            uint64_t v = 0;
+            for (int j = 0; j < 8; j++) {
+                unsigned t = c % 3;
+                c /= 3;
+                v |= (uint64_t)(8 + 17 * t + (t >> 1)) << (8 * j);
+            }
+            iq2xxs_grid[i] = v;
+        }
+    }
+};
+__device__ const Tables g_tables{};
+
+// ---------------------------------------------------------------------------
+// Every format exposes:
+//   BLOCK_ELEMS, BLOCK_BYTES  geometry of one block
+//   UNITS                     units per block
+//   SEGS, SEGLEN, SEG_STRIDE  a unit covers SEGS runs of SEGLEN consecutive
+//                             elements, SEG_STRIDE elements apart
+//   elem_base(u)              first element (within the block) of unit u
+//   decode(blk, u, w)         w[s*SEGLEN + i] = weight of element
+//                             elem_base(u) + s*SEG_STRIDE + i
+// ---------------------------------------------------------------------------
+
+struct Q8_0 {  // d:f16 | qs[32] i8   (reference: src/kquant_dot.rs:53-61,287-302)
+    static constexpr int BLOCK_ELEMS = 32, BLOCK_BYTES = 34, UNITS = 1;
+    static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
+    __device__ static int elem_base(int) { return 0; }
+    __device__ static void decode(const uint8_t *blk, int, float *w) {
+        float d = f16_bits(ld<uint16_t>(blk));
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t v = ld<uint32_t>(blk + 2 + 4 * i);
+#pragma unroll
+            for (int b = 0; b < 4; b++) w[4 * i + b] = (float)(int8_t)(v >> (8 * b)) * d;
+        }
+    }
+};
+
+struct Q4_K {  // d | dmin | scales[12] | qs[128]   (reference: src/kquant_dot.rs:78-93,426-466)
+    static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 144, UNITS = 4;
+    static constexpr int SEGS = 1, SEGLEN = 64, SEG_STRIDE = 0;
+    __device__ static int elem_base(int u) { return 64 * u; }
+    __device__ static void decode(const uint8_t *blk, int c, float *w) {
+        uint4 hdr = ld<uint4>(blk);
+        float d = f16_bits(hdr.x), dmin = f16_bits(hdr.x >> 16);
+        uint32_t sc0, mn0, sc1, mn1;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc0, mn0);
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc1, mn1);
+        float d0 = d * (float)sc0, m0 = dmin * (float)mn0;
+        float d1 = d * (float)sc1, m1 = dmin * (float)mn1;
+        uint4 qa = ld<uint4>(blk + 16 + 32 * c), qb = ld<uint4>(blk + 32 + 32 * c);
+        uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t lo = q[i] & 0x0F0F0F0Fu, hi = (q[i] >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                w[4 * i + b] = fmaf((float)((lo >> (8 * b)) & 0xFFu), d0, -m0);
+                w[32 + 4 * i + b] = fmaf((float)((hi >> (8 * b)) & 0xFFu), d1, -m1);
+            }
+        }
+    }
+};
+
+struct Q2_K {  // scales[16] | qs[64] | d | dmin   (reference: src/kquant_dot.rs:63-76,345-385)
+    // unit u = (super-group sg = u/2, byte half hf = u%2): 16 bytes, four
+    // 2-bit fields -> elements 128*sg + 32*f + 16*hf + [0,16), f = 0..3,
+    // scale byte scales[8*sg + 2*f + hf].
+    static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 84, UNITS = 4;
+    static constexpr int SEGS = 4, SEGLEN = 16, SEG_STRIDE = 32;
+    __device__ static int elem_base(int u) { return 128 * (u >> 1) + 16 * (u & 1); }
+    __device__ static void decode(const uint8_t *blk, int u, float *w) {
+        int sg = u >> 1, hf = u & 1;
+        uint32_t dd = ld<uint32_t>(blk + 80);
+        float d = f16_bits(dd), dmin = f16_bits(dd >> 16);
+        uint4 qv = ld<uint4>(blk + 16 + 32 * sg + 16 * hf);
+        uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int f = 0; f < 4; f++) {
+            uint32_t s = blk[8 * sg + 2 * f + hf];
+            float d1 = d * (float)(s & 0xFu), m1 = dmin * (float)(s >> 4);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t v = (q[i] >> (2 * f)) & 0x03030303u;
+#pragma unroll
+                for (int b = 0; b < 4; b++) w[16 * f + 4 * i + b] = fmaf((float)((v >> (8 * b)) & 0xFFu), d1, -m1);
+            }
+        }
+    }
+};
+
+struct Q6_K {  // ql[128] | qh[64] | scales[16] i8 | d
+    // (reference: vendor/candle-metal-kernels/src/metal_src/quantized.metal:198-203,6673-6694;
+    //  the reference decodes it through candle's to_float, src/quant_matmul.rs:228-248)
+    // unit u = (half h = u/2, lq = u%2): l in [16*lq, 16*lq+16); quarter t
+    // covers elements 128*h + 32*t + l, scale scales[8*h + 2*t + lq].
+    static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 210, UNITS = 4;
+    static constexpr int SEGS = 4, SEGLEN = 16, SEG_STRIDE = 32;
+    __device__ static int elem_base(int u) { return 128 * (u >> 1) + 16 * (u & 1); }
+    __device__ static void decode(const uint8_t *blk, int u, float *w) {
+        int h = u >> 1, lq = u & 1;
+        float d = f16_bits(ld<uint16_t>(blk + 208));
+        uint4 la = ld<uint4>(blk + 64 * h + 16 * lq);        // ql[64h + l]
+        uint4 lb = ld<uint4>(blk + 64 * h + 32 + 16 * lq);   // ql[64h + 32 + l]
+        uint4 hv = ld<uint4>(blk + 128 + 32 * h + 16 * lq);  // qh[32h + l]
+        uint32_t a[4] = {la.x, la.y, la.z, la.w}, b[4] = {lb.x, lb.y, lb.z, lb.w}, hh[4] = {hv.x, hv.y, hv.z, hv.w};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            float ds = d * (float)(int8_t)blk[192 + 8 * h + 2 * t + lq];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t lo = (t & 1) ? b[i] : a[i];
+                uint32_t nib = (t < 2) ? (lo & 0x0F0F0F0Fu) : ((lo >> 4) & 0x0F0F0F0Fu);
+                uint32_t q = nib | (((hh[i] >> (2 * t)) & 0x03030303u) << 4);
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++)
+                    w[16 * t + 4 * i + bb] = ds * (float)((int)((q >> (8 * bb)) & 0xFFu) - 32);
+            }
+        }
+    }
+};
+
+struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: src/iq2xxs.rs:34-71,349-380)
+    static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 66, UNITS = 8;
+    static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
+    __device__ static int elem_base(int u) { return 32 * u; }
+    __device__ static void decode(const uint8_t *blk, int u, float *w) {
+        float d = f16_bits(ld<uint16_t>(blk));
+        uint2 g = ld<uint2>(blk + 2 + 8 * u);
+        uint32_t lo = g.x, hi = g.y;
+        float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            uint64_t grid = g_tables.iq2xxs_grid[(lo >> (8 * l)) & 0xFFu];
+            uint32_t s7 = (hi >> (7 * l)) & 127u;
+            uint32_t signs = s7 | ((__popc(s7) & 1u) << 7);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                float gv = (float)(uint32_t)((grid >> (8 * j)) & 0xFFu);
+                w[8 * l + j] = ((signs >> j) & 1u ? -gv : gv) * db;
+            }
+        }
+    }
+};
+
+struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
+    static constexpr int BLOCK_ELEMS = 32, BLOCK_BYTES = 17, UNITS = 1;
+    static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
+    __device__ static int elem_base(int) { return 0; }
+    __device__ static float e2m1(uint32_t c) {
+        // magnitude: code 0 -> 0, 1 -> 0.5 (subnormal), else 2^(exp-1) * (1 + mant/2)
+        uint32_t mag = c & 7u;
+        float v = mag == 0 ? 0.0f : (mag == 1 ? 0.5f : __uint_as_float(((126u + (mag >> 1)) << 23) | ((mag & 1u) << 22)));
+        return (c & 8u) ? -v : v;
+    }
+    __device__ static void decode(const uint8_t *blk, int, float *w) {
+        uint32_t e = blk[0];
+        // 2^(e-127); e == 0 is the f32 denormal 2^-127; 0xFF (reserved) decodes the block to zeros
+        float d = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
+        bool dead = e == 0xFFu;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t v = ld<uint32_t>(blk + 1 + 4 * i);
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                uint32_t byte = (v >> (8 * b)) & 0xFFu;
+                w[4 * i + b] = dead ? 0.0f : d * e2m1(byte & 0xFu);
+                w[16 + 4 * i + b] = dead ? 0.0f : d * e2m1(byte >> 4);
+            }
+        }
+    }
+};
+
+}  // namespace jq

@@ -1,0 +1,135 @@
+// Row-per-wavefront fused dequant+dot kernels on the vector ALU, plus the
+// decode-only kernels (dequantize, embedding).  One wave64 owns one weight
+// row: its lanes take the row's units in turn, decode each unit in registers
+// and multiply-accumulate it against up to MT activation rows; a cross-lane
+// butterfly finishes the sum.  Per element the arithmetic is the reference's
+// (decode with one fused multiply-subtract, then one fused multiply-add into
+// the running sum; reference: src/kquant_dot.rs:426-476); only the order in
+// which a row's products are added differs from the 8-lane CPU order.
+//
+// These kernels serve every format and every m.  They are the general path;
+// the MFMA kernels take over where they apply.
+#pragma once
+#include "blocks.hpp"
+
+namespace jq {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+constexpr int ROWS_PER_WG = 4;  // one wave per row, 256 threads
+
+template <class Q, int MT>
+__global__ __launch_bounds__(64 * ROWS_PER_WG) void matmul_rows_valu(const uint8_t *__restrict__ W, size_t row_bytes,
+                                                                      const float *__restrict__ X,
+                                                                      float *__restrict__ Y, int m, int k, int n) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * ROWS_PER_WG + (threadIdx.x >> 6);
+    if (row >= n) return;  // wave-uniform
+    const uint8_t *rp = W + (size_t)row * row_bytes;
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    constexpr int UE = Q::SEGS * Q::SEGLEN;
+    for (int m0 = 0; m0 < m; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        for (int u = lane; u < units; u += 64) {
+            const int b = u / Q::UNITS, ub = u % Q::UNITS;
+            float w[UE];
+            Q::decode(rp + (size_t)b * Q::BLOCK_BYTES, ub, w);
+            const int xoff = b * Q::BLOCK_ELEMS + Q::elem_base(ub);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                if (m0 + i < m) {
+                    const float *xp = X + (size_t)(m0 + i) * k + xoff;
+#pragma unroll
+                    for (int s = 0; s < Q::SEGS; s++) {
+#pragma unroll
+                        for (int e = 0; e < Q::SEGLEN; e += 4) {
+                            float4 xv = ld<float4>((const uint8_t *)(xp + s * Q::SEG_STRIDE + e));
+                            acc[i] = fmaf(xv.x, w[s * Q::SEGLEN + e + 0], acc[i]);
+                            acc[i] = fmaf(xv.y, w[s * Q::SEGLEN + e + 1], acc[i]);
+                            acc[i] = fmaf(xv.z, w[s * Q::SEGLEN + e + 2], acc[i]);
+                            acc[i] = fmaf(xv.w, w[s * Q::SEGLEN + e + 3], acc[i]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < m) Y[(size_t)(m0 + i) * n + row] = s;
+        }
+    }
+}
+
+// Canonical decode ("to_float"): differs from the in-dot decode only for the
+// formats whose to_float uses two rounded operations instead of one fused
+// multiply-subtract (Q2_K, Q4_K; reference: src/kquant_dot.rs:258-260).
+template <class Q>
+struct ToFloat {
+    __device__ static void decode(const uint8_t *blk, int u, float *w) { Q::decode(blk, u, w); }
+};
+
+template <>
+struct ToFloat<Q4_K> {
+    __device__ static void decode(const uint8_t *blk, int c, float *w) {
+        uint4 hdr = ld<uint4>(blk);
+        float d = f16_bits(hdr.x), dmin = f16_bits(hdr.x >> 16);
+        uint32_t sc0, mn0, sc1, mn1;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc0, mn0);
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc1, mn1);
+        float d0 = d * (float)sc0, m0 = dmin * (float)mn0;
+        float d1 = d * (float)sc1, m1 = dmin * (float)mn1;
+        for (int i = 0; i < 32; i++) {
+            uint32_t byte = blk[16 + 32 * c + i];
+            w[i] = __fsub_rn(__fmul_rn(d0, (float)(byte & 0xFu)), m0);
+            w[32 + i] = __fsub_rn(__fmul_rn(d1, (float)(byte >> 4)), m1);
+        }
+    }
+};
+
+template <>
+struct ToFloat<Q2_K> {
+    __device__ static void decode(const uint8_t *blk, int u, float *w) {
+        int sg = u >> 1, hf = u & 1;
+        float d = f16_bits(ld<uint16_t>(blk + 80)), dmin = f16_bits(ld<uint16_t>(blk + 82));
+        for (int f = 0; f < 4; f++) {
+            uint32_t s = blk[8 * sg + 2 * f + hf];
+            float dl = d * (float)(s & 0xFu), ml = dmin * (float)(s >> 4);
+            for (int i = 0; i < 16; i++) {
+                uint32_t q = (blk[16 + 32 * sg + 16 * hf + i] >> (2 * f)) & 3u;
+                w[16 * f + i] = __fsub_rn(__fmul_rn(dl, (float)q), ml);
+            }
+        }
+    }
+};
+
+// out[r*k + ...] = decode(row ids[r]) (ids == nullptr: row r itself).
+template <class Q>
+__global__ __launch_bounds__(256) void decode_rows(const uint8_t *__restrict__ W, size_t row_bytes,
+                                                    const uint32_t *__restrict__ ids, float *__restrict__ out,
+                                                    size_t n_out_rows, int k) {
+    const int units_per_row = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    const size_t total = n_out_rows * (size_t)units_per_row;
+    constexpr int UE = Q::SEGS * Q::SEGLEN;
+    for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = g / units_per_row;
+        const int u = (int)(g % units_per_row);
+        const size_t src_row = ids ? ids[r] : r;
+        const int b = u / Q::UNITS, ub = u % Q::UNITS;
+        float w[UE];
+        ToFloat<Q>::decode(W + src_row * row_bytes + (size_t)b * Q::BLOCK_BYTES, ub, w);
+        float *o = out + r * (size_t)k + (size_t)b * Q::BLOCK_ELEMS + Q::elem_base(ub);
+#pragma unroll
+        for (int s = 0; s < Q::SEGS; s++)
+#pragma unroll
+            for (int e = 0; e < Q::SEGLEN; e++) o[s * Q::SEG_STRIDE + e] = w[s * Q::SEGLEN + e];
+    }
+}
+
+}  // namespace jq

@@ -1,0 +1,231 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on
+identical seeded block bytes and activations.  Tolerance for f32 results is the
+reference's own form, |gpu - ref| <= 1e-3 * max(|ref|, 1)
+(reference: src/kquant_dot.rs:853); decode is compared bit for bit."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from joshua_amd import capi, synth
+from tests.test_oracle_matmul import fixture_iq2xxs_rhs, mxfp4_pattern, ref_lhs, ref_weights
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+
+
+def close(got, want):
+    return np.all(np.abs(got - want) <= TOL * np.maximum(np.abs(want), 1.0))
+
+
+def make_blocks(qtype, n, k, seed, sigma=0.02):
+    return synth.normal_quantized(qtype, seed, n * k, sigma)
+
+
+@pytest.mark.parametrize("qtype", capi.ALL_TYPES)
+def test_dequantize_bit_exact(qtype):
+    n, k = 37, 1024
+    blocks = make_blocks(qtype, n, k, 11)
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    got = w.dequantize()
+    want = oracle.dequantize(qtype, blocks).reshape(n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("qtype", capi.ALL_TYPES)
+def test_dequantize_random_bytes_bit_exact(qtype):
+    """Every byte pattern is a valid block (reference: src/kquant_dot.rs:37-40)."""
+    elems, nbytes = capi.block_geometry(qtype)
+    n, k = 9, 4 * 256
+    rng = np.random.default_rng(qtype)
+    raw = rng.integers(0, 256, size=n * (k // elems) * nbytes, dtype=np.uint8)
+    blk = raw.reshape(-1, nbytes)
+    for off in {capi.Q8_0: (0,), capi.Q2_K: (80, 82), capi.Q4_K: (0, 2), capi.Q6_K: (208,), capi.IQ2_XXS: (0,),
+                capi.MXFP4: ()}[qtype]:
+        blk[:, off + 1] &= 0x7B  # finite f16 scales
+    if qtype == capi.MXFP4:
+        blk[:, 0] = np.clip(blk[:, 0], 90, 160)
+        blk[::5, 0] = 0xFF
+        blk[1::5, 0] = 0
+    w = capi.Weight.upload(qtype, raw, n, k)
+    got, want = w.dequantize(), oracle.dequantize(qtype, raw).reshape(n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_iq2xxs_golden_vectors_on_gpu(golden_dir):
+    blocks = np.fromfile(os.path.join(golden_dir, "iq2xxs_blocks.bin"), dtype=np.uint8)
+    want = np.loadtxt(os.path.join(golden_dir, "iq2xxs_ref.txt"))
+    got = capi.Weight.upload(capi.IQ2_XXS, blocks, 1, 1024).dequantize().reshape(-1)
+    assert np.all(np.abs(got - want) <= 1e-6 * np.maximum(np.abs(want), 1.0))
+
+
+REF_SHAPES = [  # reference: src/kquant_dot.rs:894-901, src/quant_matmul.rs:499-515
+    (capi.Q8_0, 1, 256, 40), (capi.Q8_0, 3, 512, 17), (capi.Q8_0, 5, 128, 9),
+    (capi.Q2_K, 1, 256, 40), (capi.Q2_K, 3, 512, 11), (capi.Q2_K, 5, 768, 9),
+    (capi.Q4_K, 1, 256, 40), (capi.Q4_K, 3, 512, 13), (capi.Q4_K, 4, 768, 25),
+    (capi.Q6_K, 1, 256, 40), (capi.Q6_K, 3, 512, 13), (capi.Q6_K, 7, 768, 10),
+]
+
+
+@pytest.mark.parametrize("qtype,m,k,n", REF_SHAPES)
+def test_matmul_reference_test_shapes(qtype, m, k, n):
+    blocks = synth.quantize(qtype, ref_weights(n, k))
+    lhs = ref_lhs(m, k)
+    got = capi.Weight.upload(qtype, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks))
+
+
+@pytest.mark.parametrize("qtype,m,k,n", [
+    (capi.Q2_K, 1, 7680, 2048), (capi.Q4_K, 1, 2048, 7680), (capi.Q8_0, 1, 4096, 4096), (capi.Q8_0, 32, 4096, 4096),
+])
+def test_matmul_reference_model_shapes(qtype, m, k, n):
+    # reference: src/kquant_dot.rs:906-914
+    blocks = make_blocks(qtype, n, k, 7)
+    lhs = synth.normal(8, (m, k))
+    got = capi.Weight.upload(qtype, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
+
+
+@pytest.mark.parametrize("qtype", capi.ALL_TYPES)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 16, 17])
+def test_matmul_small_m_all_formats(qtype, m):
+    n, k = 203, 1536
+    blocks = make_blocks(qtype, n, k, 100 + qtype)
+    lhs = synth.normal(200 + m, (m, k))
+    got = capi.Weight.upload(qtype, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
+
+
+def test_iq2xxs_fixture_matmul(golden_dir):
+    # reference: src/iq2xxs.rs:758-804
+    m, k, n = 3, 512, 7
+    rhs = fixture_iq2xxs_rhs(golden_dir, k, n)
+    lhs = ref_lhs(m, k, 7919)
+    got = capi.Weight.upload(capi.IQ2_XXS, rhs, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(capi.IQ2_XXS, (m, k, n), lhs, rhs))
+
+
+def test_mxfp4_pattern_matmul_exact():
+    # reference: src/mxfp4.rs:351-388; small integers times powers of two sum exactly in f32
+    m, k, n = 2, 64, 3
+    rhs = mxfp4_pattern(n, k)
+    lhs = (np.arange(m * k, dtype=np.float32) % np.float32(7.0) - np.float32(3.0)).reshape(m, k)
+    got = capi.Weight.upload(capi.MXFP4, rhs, n, k).matmul_t(m, lhs)
+    assert np.array_equal(got, oracle.matmul_t(capi.MXFP4, (m, k, n), lhs, rhs))
+
+
+def test_matmul_assigns_into_dirty_destination():
+    # reference: src/mxfp4.rs:390-416
+    for qtype in capi.ALL_TYPES:
+        n, k = 16, 512
+        blocks = make_blocks(qtype, n, k, 3)
+        w = capi.Weight.upload(qtype, blocks, n, k)
+        lhs = synth.normal(4, (2, k))
+        fresh = w.matmul_t(2, lhs, np.zeros(2 * n, np.float32))
+        dirty = w.matmul_t(2, lhs, np.full(2 * n, 123.75, np.float32))
+        assert np.array_equal(fresh, dirty)
+
+
+def test_results_do_not_depend_on_how_rows_are_batched():
+    """The reference requires bit-identical results whatever the thread count
+    (src/kquant_dot.rs:916-929); here: a row's result must not depend on the
+    launch it is part of."""
+    for qtype in capi.ALL_TYPES:
+        n, k = 64, 1024
+        blocks = make_blocks(qtype, n, k, 5)
+        _, bb = capi.block_geometry(qtype)
+        row_bytes = bb * k // capi.block_geometry(qtype)[0]
+        lhs = synth.normal(6, (3, k))
+        w = capi.Weight.upload(qtype, blocks, n, k)
+        full = w.matmul_t(3, lhs)
+        for lo, hi in [(0, 1), (5, 16), (17, 64)]:
+            part = w.view(lo * row_bytes, hi - lo, k).matmul_t(3, lhs)
+            assert np.array_equal(part, full[:, lo:hi]), (qtype, lo, hi)
+        again = w.matmul_t(3, lhs)
+        assert np.array_equal(full, again)
+
+
+def test_rejects_bad_shapes_and_leaves_dst_alone():
+    # reference: src/quant_matmul.rs:597-608
+    blocks = synth.quantize(capi.Q8_0, ref_weights(2, 256))
+    w = capi.Weight.upload(capi.Q8_0, blocks, 2, 256)
+    for m, x, dlen in [(1, np.zeros(100, np.float32), 2), (1, np.zeros(1, np.float32), 2),
+                       (1, np.zeros(256, np.float32), 4), (2, np.zeros(256, np.float32), 4)]:
+        dst = np.full(dlen, 5.0, np.float32)
+        with pytest.raises(capi.JoshuaHipError):
+            w.matmul_t(m, x, dst)
+        assert np.all(dst == 5.0)
+    with pytest.raises(capi.JoshuaHipError):  # k not a multiple of the block size
+        capi.Weight.upload(capi.Q8_0, blocks, 2, 100)
+    with pytest.raises(capi.JoshuaHipError):  # wrong block count for (n, k)
+        capi.Weight.upload(capi.Q8_0, blocks, 4, 256)
+    with pytest.raises(capi.JoshuaHipError):
+        capi.Weight.upload(11, blocks, 2, 256)
+    with pytest.raises(capi.JoshuaHipError):  # reference: src/mmap_tensor.rs:1002-1022 (out-of-bounds borrow declines)
+        w.view(34 * 8, 2, 256)
+
+
+def test_empty_problem_is_a_no_op():
+    blocks = synth.quantize(capi.Q4_K, ref_weights(2, 256))
+    w = capi.Weight.upload(capi.Q4_K, blocks, 2, 256)
+    assert w.matmul_t(0, np.zeros(0, np.float32), np.zeros(0, np.float32)).size == 0
+
+
+def test_embedding_gathers_decoded_rows():
+    # reference: src/mmap_tensor.rs:140-167
+    for qtype in (capi.Q4_K, capi.Q6_K, capi.Q8_0):
+        n, k = 50, 512
+        blocks = make_blocks(qtype, n, k, 9)
+        w = capi.Weight.upload(qtype, blocks, n, k)
+        ids = np.array([49, 0, 7, 7, 13], np.uint32)
+        want = oracle.dequantize(qtype, blocks).reshape(n, k)[ids]
+        assert np.array_equal(w.embedding(ids), want)
+        with pytest.raises(capi.JoshuaHipError):
+            w.embedding(np.array([50], np.uint32))
+
+
+def test_expert_slices_alias_the_stacked_tensor():
+    # reference: src/quantized_qwen3_moe.rs:596-631 (expert e at base + e*per_bytes)
+    n_expert, n, k = 6, 24, 512
+    blocks = make_blocks(capi.Q4_K, n_expert * n, k, 21)
+    per = blocks.size // n_expert
+    stacked = capi.Weight.upload(capi.Q4_K, blocks, n_expert * n, k)
+    lhs = synth.normal(22, (1, k))
+    for e in (0, 3, 5):
+        ex = stacked.view(e * per, n, k)
+        assert ex.device_ptr == stacked.device_ptr + e * per
+        got = ex.matmul_t(1, lhs)
+        assert close(got, oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks[e * per:(e + 1) * per]))
+
+
+def test_try_matmul_fused_declines_like_the_reference():
+    # reference: src/kquant_dot.rs:931-959
+    import torch
+    x = torch.zeros(256, device="cuda")
+    y = torch.full((8,), 3.0, device="cuda")
+    raw = torch.zeros(34 * 8 * 8, dtype=torch.uint8, device="cuda")
+    assert not capi.try_matmul_fused(11, (1, 256, 2), x.data_ptr(), raw.data_ptr(), 34 * 16, y.data_ptr())
+    assert not capi.try_matmul_fused(capi.Q8_0, (1, 256, 8), x.data_ptr(), raw.data_ptr(), 7, y.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.all(y == 3.0)
+    assert capi.try_matmul_fused(capi.Q8_0, (1, 256, 8), x.data_ptr(), raw.data_ptr(), 34 * 8 * 8, y.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.all(y == 0.0)
+
+
+def test_headline_shape_q4k_gemv():
+    """Q4_K 14336 x 4096, M = 1 and 16, device pointers, against the AVX2 oracle."""
+    import torch
+    n, k = 14336, 4096
+    blocks = make_blocks(capi.Q4_K, n, k, 102)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    for m in (1, 16):
+        lhs = synth.normal(202, (m, k))
+        x = torch.from_numpy(lhs).cuda()
+        y = torch.full((m, n), float("nan"), device="cuda")
+        w.matmul_t_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        want = oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True)
+        assert close(y.cpu().numpy(), want)
