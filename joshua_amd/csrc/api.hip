@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "../../include/joshua_hip.h"
+#include "kernels_mfma_q4k.hpp"
 #include "kernels_valu.hpp"
 
 namespace {
@@ -116,10 +117,55 @@ void launch_rows(const uint8_t *W, size_t row_bytes, const float *X, float *Y, s
         hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 4>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
 }
 
+// Q4_K, m <= 16: the MFMA decode kernel, four activation rows per launch.
+template <int MT>
+int launch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float *Y, int m0, int m, int k, int n,
+                    hipStream_t s) {
+    size_t lds = jq::q4k_mfma_lds_bytes(k / 256, MT);
+    static std::once_flag once;
+    static hipError_t attr_rc = hipSuccess;
+    std::call_once(once, [] {
+        attr_rc = hipFuncSetAttribute((const void *)jq::q4k_gemv_mfma<MT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      160 * 1024);
+    });
+    if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
+    hipLaunchKernelGGL((jq::q4k_gemv_mfma<MT>), dim3((unsigned)((n + 15) / 16)), dim3(64 * jq::Q4K_MFMA_WAVES), lds, s,
+                       W, row_bytes, X, Y, m0, m, k, n);
+    return 0;
+}
+
+constexpr size_t Q4K_MFMA_MAX_M = 16;
+
+bool q4k_mfma_applies(size_t m, size_t k) {
+    return m <= Q4K_MFMA_MAX_M && jq::q4k_mfma_lds_bytes((int)(k / 256), m >= 4 ? 4 : (m >= 2 ? 2 : 1)) <= 160 * 1024;
+}
+
+int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                      hipStream_t s) {
+    for (size_t m0 = 0; m0 < m;) {
+        size_t left = m - m0;
+        int rc;
+        if (left >= 3) {
+            rc = launch_q4k_mfma<4>(W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s);
+            m0 += 4;
+        } else if (left == 2) {
+            rc = launch_q4k_mfma<2>(W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s);
+            m0 += 2;
+        } else {
+            rc = launch_q4k_mfma<1>(W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s);
+            m0 += 1;
+        }
+        if (rc) return rc;
+    }
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // All pointers are device pointers; shapes already validated; m, n > 0.
 int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
                     size_t k, size_t n, hipStream_t s) {
     if (m > 0x7FFFFFFF || k > 0x7FFFFFFF || n > 0x7FFFFFFF) return fail("matmul: dimension exceeds 2^31-1");
+    if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
     switch (type) {
     case JQ_TYPE_Q8_0: launch_rows<jq::Q8_0>(W, row_bytes, X, Y, m, k, n, s); break;
     case JQ_TYPE_Q2_K: launch_rows<jq::Q2_K>(W, row_bytes, X, Y, m, k, n, s); break;
