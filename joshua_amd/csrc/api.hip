@@ -5,6 +5,8 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
+#include <algorithm>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -117,45 +119,79 @@ void launch_rows(const uint8_t *W, size_t row_bytes, const float *X, float *Y, s
         hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 4>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
 }
 
-// Q4_K, m <= 16: the MFMA decode kernel, four activation rows per launch.
+// Q4_K, m <= 16: the MFMA decode kernel, up to four activation rows per launch.
+constexpr size_t Q4K_MFMA_MAX_M = 16;
+constexpr int LDS_LIMIT = 160 * 1024;
+
+struct Q4kPlan {
+    int units_per_tile, waves;
+};
+
+// Workgroup shape for a row length: all units of a tile in one workgroup, as
+// many whole tiles as fit in 16 waves (JQ_Q4K_TILES_PER_WG overrides, for tuning).
+bool q4k_plan(size_t k, size_t n, Q4kPlan *p) {
+    int bpr = (int)(k / 256);
+    int upt = (bpr + jq::Q4K_UNIT_BLOCKS - 1) / jq::Q4K_UNIT_BLOCKS;
+    if (upt < 1 || upt > jq::Q4K_MAX_WAVES) return false;
+    int tpw = std::max(1, 8 / upt);  // 8-wave workgroups measured best at 14336 x 4096
+    static const int forced = [] {
+        const char *e = getenv("JQ_Q4K_TILES_PER_WG");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced > 0 && forced * upt <= jq::Q4K_MAX_WAVES) tpw = forced;
+    int tiles = (int)((n + 15) / 16);
+    if (tpw > tiles) tpw = tiles;
+    p->units_per_tile = upt;
+    p->waves = tpw * upt;
+    return true;
+}
+
+// Activation rows for the next launch: 4 when three or more are left (a
+// fourth, absent row is masked), else what is left; fewer when LDS is short.
+int q4k_mt_that_fits(size_t left, size_t k, int waves) {
+    int first = left >= 3 ? 4 : (left == 2 ? 2 : 1);
+    for (int mt = first; mt >= 1; mt >>= 1)
+        if (jq::q4k_lds_layout((int)k, mt, waves).total <= LDS_LIMIT) return mt;
+    return 0;
+}
+
+bool q4k_mfma_applies(size_t m, size_t k, size_t n) {
+    Q4kPlan p;
+    return m <= Q4K_MFMA_MAX_M && q4k_plan(k, n, &p) && jq::q4k_lds_layout((int)k, 1, p.waves).total <= LDS_LIMIT;
+}
+
 template <int MT>
-int launch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float *Y, int m0, int m, int k, int n,
-                    hipStream_t s) {
-    size_t lds = jq::q4k_mfma_lds_bytes(k / 256, MT);
+int launch_q4k_mfma(const Q4kPlan &p, const uint8_t *W, size_t row_bytes, const float *X, float *Y, int m0, int m,
+                    int k, int n, hipStream_t s) {
     static std::once_flag once;
     static hipError_t attr_rc = hipSuccess;
     std::call_once(once, [] {
         attr_rc = hipFuncSetAttribute((const void *)jq::q4k_gemv_mfma<MT>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      160 * 1024);
+                                      LDS_LIMIT);
     });
     if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
-    hipLaunchKernelGGL((jq::q4k_gemv_mfma<MT>), dim3((unsigned)((n + 15) / 16)), dim3(64 * jq::Q4K_MFMA_WAVES), lds, s,
-                       W, row_bytes, X, Y, m0, m, k, n);
+    int tiles = (n + 15) / 16, tpw = p.waves / p.units_per_tile;
+    size_t lds = (size_t)jq::q4k_lds_layout(k, MT, p.waves).total;
+    hipLaunchKernelGGL((jq::q4k_gemv_mfma<MT>), dim3((unsigned)((tiles + tpw - 1) / tpw)), dim3(64 * p.waves), lds, s, W,
+                       row_bytes, X, Y, m0, m, k, n, p.units_per_tile);
     return 0;
-}
-
-constexpr size_t Q4K_MFMA_MAX_M = 16;
-
-bool q4k_mfma_applies(size_t m, size_t k) {
-    return m <= Q4K_MFMA_MAX_M && jq::q4k_mfma_lds_bytes((int)(k / 256), m >= 4 ? 4 : (m >= 2 ? 2 : 1)) <= 160 * 1024;
 }
 
 int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
                       hipStream_t s) {
+    Q4kPlan p;
+    if (!q4k_plan(k, n, &p)) return fail("q4k mfma: unsupported row length %zu", k);
     for (size_t m0 = 0; m0 < m;) {
-        size_t left = m - m0;
+        int mt = q4k_mt_that_fits(m - m0, k, p.waves);
         int rc;
-        if (left >= 3) {
-            rc = launch_q4k_mfma<4>(W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s);
-            m0 += 4;
-        } else if (left == 2) {
-            rc = launch_q4k_mfma<2>(W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s);
-            m0 += 2;
-        } else {
-            rc = launch_q4k_mfma<1>(W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s);
-            m0 += 1;
+        switch (mt) {
+        case 4: rc = launch_q4k_mfma<4>(p, W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s); break;
+        case 2: rc = launch_q4k_mfma<2>(p, W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s); break;
+        case 1: rc = launch_q4k_mfma<1>(p, W, row_bytes, X, Y, (int)m0, (int)m, (int)k, (int)n, s); break;
+        default: return fail("q4k mfma: activations do not fit in LDS for k=%zu", k);
         }
         if (rc) return rc;
+        m0 += (size_t)mt;
     }
     HIP_TRY(hipGetLastError());
     return 0;
@@ -165,7 +201,7 @@ int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
 int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
                     size_t k, size_t n, hipStream_t s) {
     if (m > 0x7FFFFFFF || k > 0x7FFFFFFF || n > 0x7FFFFFFF) return fail("matmul: dimension exceeds 2^31-1");
-    if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
+    if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k, n)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
     switch (type) {
     case JQ_TYPE_Q8_0: launch_rows<jq::Q8_0>(W, row_bytes, X, Y, m, k, n, s); break;
     case JQ_TYPE_Q2_K: launch_rows<jq::Q2_K>(W, row_bytes, X, Y, m, k, n, s); break;

@@ -98,6 +98,34 @@ def test_matmul_small_m_all_formats(qtype, m):
     assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (1, 256, 5), (2, 768, 33), (1, 1280, 16), (3, 5120, 100), (1, 14336, 70), (4, 12288, 48), (16, 2048, 250),
+    (5, 16384, 17), (1, 16640, 9),
+])
+def test_q4k_row_lengths_and_tails(m, k, n):
+    """Row lengths that are not a whole number of 4-block units, tiles with
+    fewer than 16 rows, and a row length beyond the MFMA kernel's reach."""
+    blocks = make_blocks(capi.Q4_K, n, k, 31 + k)
+    lhs = synth.normal(32 + m, (m, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True))
+
+
+def test_q4k_activation_scales_span_many_orders():
+    """Fixed-point activation groups: rows mixing 1e-6 .. 1e6 magnitudes, zero
+    groups and a single nonzero element still meet the f32 tolerance."""
+    n, k = 64, 4096
+    blocks = make_blocks(capi.Q4_K, n, k, 77)
+    rng = np.random.default_rng(5)
+    lhs = synth.normal(78, (3, k))
+    lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 16)).repeat(16).astype(np.float32)
+    lhs[1, :] = 0.0
+    lhs[1, 1234] = 3.5
+    lhs[2, 512:1024] = 0.0
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(3, lhs)
+    assert close(got, oracle.matmul_t(capi.Q4_K, (3, k, n), lhs, blocks, avx2=True))
+
+
 def test_iq2xxs_fixture_matmul(golden_dir):
     # reference: src/iq2xxs.rs:758-804
     m, k, n = 3, 512, 7
