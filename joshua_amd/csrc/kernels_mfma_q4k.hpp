@@ -110,10 +110,14 @@ __global__ __launch_bounds__(64 * Q4K_MAX_WAVES) void q4k_gemv_mfma(const uint8_
 
     // ---- 1. activation loads first (VMEM returns in order), then the weights ----
     const int kq = k >> 2;  // float4s per activation row
-    float4 xpre[MT];
+    constexpr int XP = 2;  // float4s per thread and row fetched ahead of the weight loads
+    float4 xpre[MT][XP];
 #pragma unroll
     for (int mi = 0; mi < MT; mi++)
-        xpre[mi] = ld<float4>((const uint8_t *)(X + (size_t)min(m0 + mi, m - 1) * k + 4 * min((int)threadIdx.x, kq - 1)));
+#pragma unroll
+        for (int j = 0; j < XP; j++)
+            xpre[mi][j] = ld<float4>((const uint8_t *)(X + (size_t)min(m0 + mi, m - 1) * k +
+                                                       4 * min((int)threadIdx.x + j * nthreads, kq - 1)));
 
     // Weight loads selected by Q4K_EARLY_MASK are issued now, the others once the
     // activations are staged.  Measured on MI355X at 14336 x 4096: issuing all
@@ -167,8 +171,11 @@ __global__ __launch_bounds__(64 * Q4K_MAX_WAVES) void q4k_gemv_mfma(const uint8_
     };
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
-        if ((int)threadIdx.x < kq) stage(mi, (int)threadIdx.x, xpre[mi]);
-        for (int fi = (int)threadIdx.x + nthreads; fi < kq; fi += nthreads)
+#pragma unroll
+        for (int j = 0; j < XP; j++)
+            if ((int)threadIdx.x + j * nthreads < kq) stage(mi, (int)threadIdx.x + j * nthreads, xpre[mi][j]);
+        // longer rows: these loads queue behind the weight loads already in flight
+        for (int fi = (int)threadIdx.x + XP * nthreads; fi < kq; fi += nthreads)
             stage(mi, fi, ld<float4>((const uint8_t *)(X + (size_t)min(m0 + mi, m - 1) * k + 4 * fi)));
     }
 
@@ -182,15 +189,15 @@ __global__ __launch_bounds__(64 * Q4K_MAX_WAVES) void q4k_gemv_mfma(const uint8_
     uint8_t *dec = lds + L.dec + wave * Q4K_DEC_WAVE;
     {
         // piece 9g sits in load 2g.  The candidates go through an empty asm so the
-        // compiler keeps this a register select instead of indexing t[] in memory.
-        uint4 h0 = t[0], h1 = t[2], h2 = t[4], h3 = t[6];
-        asm volatile("" : "+v"(h0.x), "+v"(h0.y), "+v"(h0.z), "+v"(h0.w), "+v"(h1.x), "+v"(h1.y), "+v"(h1.z), "+v"(h1.w));
-        asm volatile("" : "+v"(h2.x), "+v"(h2.y), "+v"(h2.z), "+v"(h2.w), "+v"(h3.x), "+v"(h3.y), "+v"(h3.z), "+v"(h3.w));
+        // compiler keeps this a register select instead of indexing t[] in memory
+        // (the memory clobber keeps it, and the wait for the loads, below the barrier).
+        asm volatile("" : "+v"(t[0].x), "+v"(t[0].y), "+v"(t[0].z), "+v"(t[0].w), "+v"(t[2].x), "+v"(t[2].y), "+v"(t[2].z), "+v"(t[2].w)::"memory");
+        asm volatile("" : "+v"(t[4].x), "+v"(t[4].y), "+v"(t[4].z), "+v"(t[4].w), "+v"(t[6].x), "+v"(t[6].y), "+v"(t[6].z), "+v"(t[6].w)::"memory");
         uint4 h;
-        h.x = g == 0 ? h0.x : (g == 1 ? h1.x : (g == 2 ? h2.x : h3.x));
-        h.y = g == 0 ? h0.y : (g == 1 ? h1.y : (g == 2 ? h2.y : h3.y));
-        h.z = g == 0 ? h0.z : (g == 1 ? h1.z : (g == 2 ? h2.z : h3.z));
-        h.w = g == 0 ? h0.w : (g == 1 ? h1.w : (g == 2 ? h2.w : h3.w));
+        h.x = g == 0 ? t[0].x : (g == 1 ? t[2].x : (g == 2 ? t[4].x : t[6].x));
+        h.y = g == 0 ? t[0].y : (g == 1 ? t[2].y : (g == 2 ? t[4].y : t[6].y));
+        h.z = g == 0 ? t[0].z : (g == 1 ? t[2].z : (g == 2 ? t[4].z : t[6].z));
+        h.w = g == 0 ? t[0].w : (g == 1 ? t[2].w : (g == 2 ? t[4].w : t[6].w));
         const float dd = f16_bits(h.x), dmin = f16_bits(h.x >> 16);
         const uint32_t sc_a = h.y & 0x3F3F3F3Fu, mn_a = h.z & 0x3F3F3F3Fu;  // pairs 0..3
         const uint32_t sc_b = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);          // pairs 4..7
