@@ -109,6 +109,47 @@ int jq_dequantize(const jq_weight *w, float *out, size_t out_len, int out_is_dev
 int jq_embedding(const jq_weight *w, const uint32_t *ids, size_t n_ids, float *out, size_t out_len,
                  int ptrs_are_device, void *stream);
 
+/* ---- Mixture-of-experts layer -------------------------------------------------
+ * One call per layer instead of one per expert matmul: router, gating, top-k,
+ * expert SwiGLU MLPs over the routed pairs grouped by expert id, weighted sum,
+ * optional shared expert.  Semantics follow the reference's two MoE blocks
+ * (reference: src/quantized_qwen3_moe.rs:404-528 Moe::{forward,route,dispatch,
+ * dispatch_decode}; src/quantized_deepseek2.rs:508-685 with sigmoid gating,
+ * selection bias, group-limited top-k, weight scale and shared expert). */
+typedef struct jq_moe jq_moe;
+
+typedef struct {
+    uint32_t n_expert;       /* routed experts E */
+    uint32_t n_expert_used;  /* k */
+    uint32_t hidden;         /* h */
+    uint32_t inter;          /* expert feed-forward length */
+    uint32_t gating;         /* 0 softmax, 1 sigmoid (src/quantized_deepseek2.rs:529-532) */
+    uint32_t norm_topk;      /* divide the k weights by max(sum, 6.103515625e-5) */
+    float weights_scale;     /* 0 or 1: none (src/quantized_deepseek2.rs:549-551) */
+    uint32_t n_group;        /* <= 1: no group limit (src/quantized_deepseek2.rs:563-566) */
+    uint32_t topk_group;
+} jq_moe_config;
+
+/* router_w is [E, h] row-major f32 on the host (ffn_gate_inp), router_bias [E]
+ * or NULL (exp_probs_b).  gate_exps / up_exps are stacked [E*inter, h] weights,
+ * down_exps [E*h, inter]; expert e is the e-th slice
+ * (reference: src/quantized_qwen3_moe.rs:659-667 load_moe).  The shared expert's
+ * three weights may be NULL.  The weights must outlive the layer object. */
+int jq_moe_create(const jq_moe_config *cfg, const float *router_w, const float *router_bias,
+                  const jq_weight *gate_exps, const jq_weight *up_exps, const jq_weight *down_exps,
+                  const jq_weight *shared_gate, const jq_weight *shared_up, const jq_weight *shared_down,
+                  jq_moe **out);
+void jq_moe_free(jq_moe *moe);
+
+/* Router only: ids[t, s] (descending score) and weights[t, s], s < k
+ * (reference: src/quantized_qwen3_moe.rs:424-436 route). */
+int jq_moe_route(jq_moe *moe, size_t n_tokens, const float *x, uint32_t *ids, float *weights,
+                 int ptrs_are_device, void *stream);
+
+/* y[n_tokens, h] = MoE(x[n_tokens, h]).  One call at a time per jq_moe (it owns
+ * its scratch buffers). */
+int jq_moe_forward(jq_moe *moe, size_t n_tokens, const float *x, float *y, int ptrs_are_device, void *stream);
+
 /* Blocks until everything enqueued on `stream` has finished. */
 int jq_stream_synchronize(void *stream);
 

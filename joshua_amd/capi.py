@@ -22,12 +22,19 @@ TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "
 EXPORTS = (
     "jq_last_error", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
     "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_try_matmul_fused", "jq_dequantize",
-    "jq_embedding", "jq_stream_synchronize",
+    "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
 )
 
 
 class JoshuaHipError(RuntimeError):
     """A C-ABI call returned nonzero; the message is jq_last_error()."""
+
+
+class MoeConfig(ctypes.Structure):
+    """jq_moe_config of include/joshua_hip.h."""
+    _fields_ = [("n_expert", ctypes.c_uint32), ("n_expert_used", ctypes.c_uint32), ("hidden", ctypes.c_uint32),
+                ("inter", ctypes.c_uint32), ("gating", ctypes.c_uint32), ("norm_topk", ctypes.c_uint32),
+                ("weights_scale", ctypes.c_float), ("n_group", ctypes.c_uint32), ("topk_group", ctypes.c_uint32)]
 
 
 _lib = None
@@ -68,6 +75,11 @@ def lib() -> ctypes.CDLL:
         L.jq_dequantize.argtypes = [vp, vp, sz, i32, vp]
         L.jq_embedding.argtypes = [vp, vp, sz, vp, sz, i32, vp]
         L.jq_stream_synchronize.argtypes = [vp]
+        L.jq_moe_create.argtypes = [ctypes.POINTER(MoeConfig), vp, vp, vp, vp, vp, vp, vp, vp, ctypes.POINTER(vp)]
+        L.jq_moe_free.argtypes = [vp]
+        L.jq_moe_free.restype = None
+        L.jq_moe_route.argtypes = [vp, sz, vp, vp, vp, i32, vp]
+        L.jq_moe_forward.argtypes = [vp, sz, vp, vp, i32, vp]
         _lib = L
     return _lib
 
@@ -192,3 +204,50 @@ def try_matmul_fused(qtype: int, mkn, lhs_ptr: int, blocks_ptr: int, nbytes: int
 
 def stream_synchronize(stream: int = 0) -> None:
     _check(lib().jq_stream_synchronize(stream or None))
+
+
+class Moe:
+    """A mixture-of-experts layer on the device (reference: src/quantized_qwen3_moe.rs:404-520,
+    src/quantized_deepseek2.rs:508-672)."""
+
+    def __init__(self, cfg: MoeConfig, router_w: np.ndarray, gate_exps: Weight, up_exps: Weight, down_exps: Weight,
+                 router_bias: np.ndarray | None = None, shared: "tuple[Weight, Weight, Weight] | None" = None):
+        self.cfg = cfg
+        self._keep = (gate_exps, up_exps, down_exps, shared)
+        rw = np.ascontiguousarray(router_w, dtype=np.float32)
+        assert rw.shape == (cfg.n_expert, cfg.hidden)
+        rb = None if router_bias is None else np.ascontiguousarray(router_bias, dtype=np.float32)
+        sh = [w.handle for w in shared] if shared else [None, None, None]
+        out = ctypes.c_void_p()
+        _check(lib().jq_moe_create(ctypes.byref(cfg), rw.ctypes.data, None if rb is None else rb.ctypes.data,
+                                   gate_exps.handle, up_exps.handle, down_exps.handle, sh[0], sh[1], sh[2],
+                                   ctypes.byref(out)))
+        self._h = out
+
+    def close(self) -> None:
+        if self._h:
+            lib().jq_moe_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def route(self, x: np.ndarray):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        t = x.shape[0]
+        ids = np.empty((t, self.cfg.n_expert_used), np.uint32)
+        w = np.empty((t, self.cfg.n_expert_used), np.float32)
+        _check(lib().jq_moe_route(self._h, t, x.ctypes.data, ids.ctypes.data, w.ctypes.data, 0, None))
+        return ids, w
+
+    def forward(self, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        y = np.empty_like(x)
+        _check(lib().jq_moe_forward(self._h, x.shape[0], x.ctypes.data, y.ctypes.data, 0, None))
+        return y
+
+    def forward_dev(self, n_tokens: int, x_ptr: int, y_ptr: int, stream: int = 0) -> None:
+        _check(lib().jq_moe_forward(self._h, n_tokens, x_ptr, y_ptr, 1, stream or None))

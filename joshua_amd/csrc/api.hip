@@ -13,6 +13,7 @@
 
 #include "../../include/joshua_hip.h"
 #include "kernels_mfma_q4k.hpp"
+#include "kernels_moe.hpp"
 #include "kernels_valu.hpp"
 
 namespace {
@@ -413,6 +414,280 @@ int jq_embedding(const jq_weight *w, const uint32_t *ids, size_t n_ids, float *o
 
 int jq_stream_synchronize(void *stream) {
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+
+// ---- mixture of experts -----------------------------------------------------------
+
+}  // extern "C"
+
+struct jq_moe {
+    jq_moe_config cfg;
+    const jq_weight *gate, *up, *down, *sgate, *sup, *sdown;
+    float *router_w = nullptr, *router_bias = nullptr;
+    const uint8_t **pgate = nullptr, **pup = nullptr, **pdown = nullptr;  // device tables of expert bases
+    // scratch, grown to the largest token count seen
+    size_t cap_tokens = 0;
+    float *logits = nullptr, *wts = nullptr, *G = nullptr, *U = nullptr, *out = nullptr;
+    float *sG = nullptr, *sU = nullptr, *sH = nullptr, *sOut = nullptr;
+    uint32_t *ids = nullptr;
+    int *gexp = nullptr, *offsets = nullptr, *xrow = nullptr, *yrow = nullptr;
+    std::mutex mu;
+};
+
+namespace {
+
+void moe_free_scratch(jq_moe *m) {
+    for (void *p : {(void *)m->logits, (void *)m->wts, (void *)m->G, (void *)m->U, (void *)m->out, (void *)m->sG,
+                    (void *)m->sU, (void *)m->sH, (void *)m->sOut, (void *)m->ids, (void *)m->gexp,
+                    (void *)m->offsets, (void *)m->xrow, (void *)m->yrow})
+        if (p) (void)hipFree(p);
+    m->logits = m->wts = m->G = m->U = m->out = m->sG = m->sU = m->sH = m->sOut = nullptr;
+    m->ids = nullptr;
+    m->gexp = m->offsets = m->xrow = m->yrow = nullptr;
+    m->cap_tokens = 0;
+}
+
+int moe_reserve(jq_moe *m, size_t T) {
+    if (T <= m->cap_tokens) return 0;
+    moe_free_scratch(m);
+    const jq_moe_config &c = m->cfg;
+    size_t P = T * c.n_expert_used, groups = std::max<size_t>(P, c.n_expert) + 1;
+    HIP_TRY(hipMalloc((void **)&m->logits, T * c.n_expert * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->wts, P * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->ids, P * sizeof(uint32_t)));
+    HIP_TRY(hipMalloc((void **)&m->G, P * c.inter * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->U, P * c.inter * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->out, P * c.hidden * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->gexp, groups * sizeof(int)));
+    HIP_TRY(hipMalloc((void **)&m->offsets, (groups + 1) * sizeof(int)));
+    HIP_TRY(hipMalloc((void **)&m->xrow, P * sizeof(int)));
+    HIP_TRY(hipMalloc((void **)&m->yrow, P * sizeof(int)));
+    if (m->sgate) {
+        size_t si = m->sgate->n;
+        HIP_TRY(hipMalloc((void **)&m->sG, T * si * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&m->sU, T * si * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&m->sH, T * si * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&m->sOut, T * c.hidden * sizeof(float)));
+    }
+    m->cap_tokens = T;
+    return 0;
+}
+
+template <class Q, bool SWIGLU>
+void launch_moe_rows(const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2, const int *gexp,
+                     const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n, int groups,
+                     int max_group, hipStream_t s) {
+    dim3 grid((unsigned)((n + jq::ROWS_PER_WG - 1) / jq::ROWS_PER_WG), (unsigned)groups), block(64 * jq::ROWS_PER_WG);
+    if (max_group <= 1)
+        hipLaunchKernelGGL((jq::moe_rows_valu<Q, 1, SWIGLU>), grid, block, 0, s, Wptr, row_bytes, X, X2, gexp, offsets,
+                           xsel, yrow, Y, k, n);
+    else
+        hipLaunchKernelGGL((jq::moe_rows_valu<Q, 4, SWIGLU>), grid, block, 0, s, Wptr, row_bytes, X, X2, gexp, offsets,
+                           xsel, yrow, Y, k, n);
+}
+
+template <bool SWIGLU>
+int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2,
+                      const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
+                      int groups, int max_group, hipStream_t s) {
+    switch (type) {
+#define JQ_MOE_CASE(ID, Q)                                                                                          \
+    case ID:                                                                                                        \
+        launch_moe_rows<jq::Q, SWIGLU>(Wptr, row_bytes, X, X2, gexp, offsets, xsel, yrow, Y, k, n, groups, max_group, \
+                                       s);                                                                          \
+        break;
+        JQ_MOE_CASE(JQ_TYPE_Q8_0, Q8_0)
+        JQ_MOE_CASE(JQ_TYPE_Q2_K, Q2_K)
+        JQ_MOE_CASE(JQ_TYPE_Q4_K, Q4_K)
+        JQ_MOE_CASE(JQ_TYPE_Q6_K, Q6_K)
+        JQ_MOE_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
+        JQ_MOE_CASE(JQ_TYPE_MXFP4, MXFP4)
+#undef JQ_MOE_CASE
+    default: return fail("unsupported tensor type id %u", type);
+    }
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s) {
+    const jq_moe_config &c = m->cfg;
+    hipLaunchKernelGGL(jq::moe_router_logits, dim3((c.n_expert + 3) / 4), dim3(256), 0, s, m->router_w, x, m->logits,
+                       (int)T, (int)c.hidden, (int)c.n_expert);
+    jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
+                         (int)c.n_group, (int)c.topk_group};
+    size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1)) * sizeof(float);
+    hipLaunchKernelGGL(jq::moe_gate_topk, dim3((unsigned)T), dim3(64), sm, s, m->logits, m->router_bias, gp, m->ids,
+                       m->wts);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s) {
+    const jq_moe_config &c = m->cfg;
+    if (moe_route_dev(m, T, x, s)) return 1;
+    const int P = (int)(T * c.n_expert_used);
+    int groups, max_group;
+    if ((size_t)P <= c.n_expert) {  // decode-sized: one group per pair
+        groups = P;
+        max_group = 1;
+        hipLaunchKernelGGL(jq::moe_pairs_as_groups, dim3(1), dim3(256), 0, s, m->ids, P, (int)c.n_expert_used, m->gexp,
+                           m->offsets, m->xrow, m->yrow);
+    } else {
+        groups = (int)c.n_expert;
+        max_group = (int)T;
+        hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(256), (c.n_expert + 1) * sizeof(int), s, m->ids, (int)T,
+                           (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow);
+    }
+    HIP_TRY(hipGetLastError());
+    // gate and up over the token rows, down over silu(gate)*up of each pair
+    if (dispatch_moe_rows<false>(m->gate->type, m->pgate, m->gate->row_bytes, x, nullptr, m->gexp, m->offsets, m->xrow,
+                                 m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s))
+        return 1;
+    if (dispatch_moe_rows<false>(m->up->type, m->pup, m->up->row_bytes, x, nullptr, m->gexp, m->offsets, m->xrow, m->yrow,
+                                 m->U, (int)c.hidden, (int)c.inter, groups, max_group, s))
+        return 1;
+    if (dispatch_moe_rows<true>(m->down->type, m->pdown, m->down->row_bytes, m->G, m->U, m->gexp, m->offsets, m->yrow,
+                                m->yrow, m->out, (int)c.inter, (int)c.hidden, groups, max_group, s))
+        return 1;
+    const float *shared_out = nullptr;
+    if (m->sgate) {  // shared expert over every token (reference: src/quantized_deepseek2.rs:555-557)
+        size_t si = m->sgate->n;
+        if (dispatch_matmul(m->sgate->type, m->sgate->dev, m->sgate->row_bytes, x, m->sG, T, c.hidden, si, s)) return 1;
+        if (dispatch_matmul(m->sup->type, m->sup->dev, m->sup->row_bytes, x, m->sU, T, c.hidden, si, s)) return 1;
+        size_t total = T * si;
+        hipLaunchKernelGGL(jq::swiglu_rows, dim3((unsigned)std::min<size_t>((total + 255) / 256, 4096)), dim3(256), 0, s,
+                           m->sG, m->sU, m->sH, total);
+        if (dispatch_matmul(m->sdown->type, m->sdown->dev, m->sdown->row_bytes, m->sH, m->sOut, T, si, c.hidden, s))
+            return 1;
+        shared_out = m->sOut;
+    }
+    size_t total = T * c.hidden;
+    hipLaunchKernelGGL(jq::moe_combine, dim3((unsigned)std::min<size_t>((total + 255) / 256, 4096)), dim3(256), 0, s,
+                       m->out, m->wts, (int)T, (int)c.n_expert_used, (int)c.hidden, shared_out, y);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int moe_ptr_table(const jq_weight *w, size_t n_expert, size_t rows_per_expert, const uint8_t ***out) {
+    std::vector<const uint8_t *> host(n_expert);
+    for (size_t e = 0; e < n_expert; e++) host[e] = w->dev + e * rows_per_expert * w->row_bytes;
+    HIP_TRY(hipMalloc((void **)out, n_expert * sizeof(uint8_t *)));
+    HIP_TRY(hipMemcpy((void *)*out, host.data(), n_expert * sizeof(uint8_t *), hipMemcpyHostToDevice));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int jq_moe_create(const jq_moe_config *cfg, const float *router_w, const float *router_bias,
+                  const jq_weight *gate_exps, const jq_weight *up_exps, const jq_weight *down_exps,
+                  const jq_weight *shared_gate, const jq_weight *shared_up, const jq_weight *shared_down,
+                  jq_moe **out) {
+    if (!out) return fail("jq_moe_create: out is null");
+    *out = nullptr;
+    if (!cfg || !router_w || !gate_exps || !up_exps || !down_exps) return fail("jq_moe_create: null argument");
+    const jq_moe_config &c = *cfg;
+    if (c.n_expert == 0 || c.n_expert_used == 0 || c.n_expert_used > c.n_expert)
+        return fail("moe: %u experts used of %u", c.n_expert_used, c.n_expert);
+    if (c.hidden % 4 != 0) return fail("moe: hidden size %u is not a multiple of 4", c.hidden);
+    if (c.n_group > 1 && (c.n_expert % c.n_group != 0 || c.topk_group == 0 || c.topk_group > c.n_group))
+        return fail("moe: %u experts in %u groups, %u groups kept", c.n_expert, c.n_group, c.topk_group);
+    // reference: src/quantized_qwen3_moe.rs:567-571 (expert tensor shaped [n_expert, out, in])
+    if (gate_exps->n != (size_t)c.n_expert * c.inter || gate_exps->k != c.hidden || up_exps->n != gate_exps->n ||
+        up_exps->k != c.hidden || down_exps->n != (size_t)c.n_expert * c.hidden || down_exps->k != c.inter)
+        return fail("moe: expected expert tensors shaped [%u*%u, %u], [%u*%u, %u], [%u*%u, %u]", c.n_expert, c.inter,
+                    c.hidden, c.n_expert, c.inter, c.hidden, c.n_expert, c.hidden, c.inter);
+    bool any_shared = shared_gate || shared_up || shared_down;
+    if (any_shared) {
+        if (!(shared_gate && shared_up && shared_down)) return fail("moe: shared expert needs gate, up and down");
+        if (shared_gate->k != c.hidden || shared_up->k != c.hidden || shared_up->n != shared_gate->n ||
+            shared_down->k != shared_gate->n || shared_down->n != c.hidden)
+            return fail("moe: shared expert shapes do not chain");
+    }
+    if (ensure_init()) return 1;
+    jq_moe *m = new jq_moe;
+    m->cfg = c;
+    m->gate = gate_exps;
+    m->up = up_exps;
+    m->down = down_exps;
+    m->sgate = shared_gate;
+    m->sup = shared_up;
+    m->sdown = shared_down;
+    auto cleanup = [&] {
+        jq_moe_free(m);
+        return 1;
+    };
+    size_t rbytes = (size_t)c.n_expert * c.hidden * sizeof(float);
+    if (hipMalloc((void **)&m->router_w, rbytes) != hipSuccess ||
+        hipMemcpy(m->router_w, router_w, rbytes, hipMemcpyHostToDevice) != hipSuccess) {
+        fail("moe: router upload failed");
+        return cleanup();
+    }
+    if (router_bias) {
+        if (hipMalloc((void **)&m->router_bias, c.n_expert * sizeof(float)) != hipSuccess ||
+            hipMemcpy(m->router_bias, router_bias, c.n_expert * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
+            fail("moe: router bias upload failed");
+            return cleanup();
+        }
+    }
+    if (moe_ptr_table(gate_exps, c.n_expert, c.inter, &m->pgate) || moe_ptr_table(up_exps, c.n_expert, c.inter, &m->pup) ||
+        moe_ptr_table(down_exps, c.n_expert, c.hidden, &m->pdown))
+        return cleanup();
+    *out = m;
+    return 0;
+}
+
+void jq_moe_free(jq_moe *m) {
+    if (!m) return;
+    moe_free_scratch(m);
+    for (void *p : {(void *)m->router_w, (void *)m->router_bias, (void *)m->pgate, (void *)m->pup, (void *)m->pdown})
+        if (p) (void)hipFree(p);
+    delete m;
+}
+
+int jq_moe_route(jq_moe *m, size_t n_tokens, const float *x, uint32_t *ids, float *weights, int ptrs_are_device,
+                 void *stream) {
+    if (!m) return fail("jq_moe_route: layer is null");
+    if (n_tokens == 0) return 0;
+    if (!x || !ids || !weights) return fail("jq_moe_route: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    std::lock_guard<std::mutex> lock(m->mu);
+    if (moe_reserve(m, n_tokens)) return 1;
+    size_t P = n_tokens * m->cfg.n_expert_used;
+    DevBuf xd;
+    const float *xdev = x;
+    if (!ptrs_are_device) {
+        HIP_TRY(xd.alloc(n_tokens * m->cfg.hidden * sizeof(float)));
+        HIP_TRY(hipMemcpyAsync(xd.p, x, n_tokens * m->cfg.hidden * sizeof(float), hipMemcpyHostToDevice, s));
+        xdev = (const float *)xd.p;
+    }
+    if (moe_route_dev(m, n_tokens, xdev, s)) return 1;
+    hipMemcpyKind kind = ptrs_are_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
+    HIP_TRY(hipMemcpyAsync(ids, m->ids, P * sizeof(uint32_t), kind, s));
+    HIP_TRY(hipMemcpyAsync(weights, m->wts, P * sizeof(float), kind, s));
+    if (!ptrs_are_device) HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int jq_moe_forward(jq_moe *m, size_t n_tokens, const float *x, float *y, int ptrs_are_device, void *stream) {
+    if (!m) return fail("jq_moe_forward: layer is null");
+    if (n_tokens == 0) return 0;
+    if (!x || !y) return fail("jq_moe_forward: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    std::lock_guard<std::mutex> lock(m->mu);
+    if (moe_reserve(m, n_tokens)) return 1;
+    if (ptrs_are_device) return moe_forward_dev(m, n_tokens, x, y, s);
+    size_t bytes = n_tokens * m->cfg.hidden * sizeof(float);
+    DevBuf xd, yd;
+    HIP_TRY(xd.alloc(bytes));
+    HIP_TRY(yd.alloc(bytes));
+    HIP_TRY(hipMemcpyAsync(xd.p, x, bytes, hipMemcpyHostToDevice, s));
+    if (moe_forward_dev(m, n_tokens, (const float *)xd.p, (float *)yd.p, s)) return 1;
+    HIP_TRY(hipMemcpyAsync(y, yd.p, bytes, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
     return 0;
 }
 

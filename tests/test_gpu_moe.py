@@ -1,0 +1,86 @@
+"""GPU parity of the MoE layer (router, top-k, grouped expert matmuls, combine)
+against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import oracle
+from oracle.moe import MoeOracle
+from joshua_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def build(qtype, h, inter, E, k, seed, sigma=0.02, shared_inter=0, **kw):
+    rw = synth.normal(seed, (E, h), sigma=0.02)
+    gate = synth.normal_quantized(qtype, seed + 1, E * inter * h, sigma)
+    up = synth.normal_quantized(qtype, seed + 2, E * inter * h, sigma)
+    down = synth.normal_quantized(qtype, seed + 3, E * h * inter, sigma)
+    shared_o = shared_w = None
+    if shared_inter:
+        sg = synth.normal_quantized(qtype, seed + 4, shared_inter * h, sigma)
+        su = synth.normal_quantized(qtype, seed + 5, shared_inter * h, sigma)
+        sd = synth.normal_quantized(qtype, seed + 6, h * shared_inter, sigma)
+        shared_o = (qtype, shared_inter, sg, su, sd)
+        shared_w = (capi.Weight.upload(qtype, sg, shared_inter, h), capi.Weight.upload(qtype, su, shared_inter, h),
+                    capi.Weight.upload(qtype, sd, h, shared_inter))
+    ora = MoeOracle(qtype, h, inter, E, k, rw, gate, up, down, shared=shared_o, avx2=oracle.have_avx2(), **kw)
+    cfg = capi.MoeConfig(E, k, h, inter, 1 if kw.get("gating") == "sigmoid" else 0, 1 if kw.get("norm_topk", True) else 0,
+                         float(kw.get("weights_scale", 0.0)), kw.get("n_group", 1), kw.get("topk_group", 1))
+    dev = capi.Moe(cfg, rw, capi.Weight.upload(qtype, gate, E * inter, h), capi.Weight.upload(qtype, up, E * inter, h),
+                   capi.Weight.upload(qtype, down, E * h, inter), router_bias=kw.get("router_bias"), shared=shared_w)
+    return ora, dev
+
+
+def close(got, want, tol=1e-3):
+    return np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1.0))
+
+
+@pytest.mark.parametrize("kw", [
+    dict(), dict(norm_topk=False),
+    dict(gating="sigmoid", weights_scale=2.5),
+    dict(gating="sigmoid", n_group=4, topk_group=2, router_bias=np.linspace(-0.05, 0.05, 32).astype(np.float32)),
+    dict(gating="softmax", n_group=8, topk_group=3),
+])
+def test_route_matches_oracle(kw):
+    ora, dev = build(capi.Q8_0, 512, 32, 32, 6, 40, **kw)
+    x = synth.normal(41, (9, 512))
+    ids, w = dev.route(x)
+    oid, ow = ora.route(x)
+    assert np.array_equal(ids, oid)
+    assert np.allclose(w, ow, rtol=2e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("tokens", [1, 2, 7, 64])
+def test_qwen3moe_shaped_layer_q4k(tokens):
+    """Qwen3-30B-A3B layer shape (h 2048, inter 768, top-8) with 16 experts."""
+    ora, dev = build(capi.Q4_K, 2048, 768, 16, 8, 60)
+    x = synth.normal(61 + tokens, (tokens, 2048))
+    assert close(dev.forward(x), ora.forward(x))
+
+
+def test_decode_and_grouped_dispatch_agree_on_device():
+    """reference: src/quantized_qwen3_moe.rs:912-928 (prefill vs decode path, 1e-4)."""
+    ora, dev = build(capi.Q4_K, 512, 256, 8, 2, 70)
+    row = synth.normal(71, (1, 512))
+    many = np.repeat(row, 9, axis=0)              # 18 pairs > 8 experts: grouped path
+    one = dev.forward(row)
+    assert np.all(np.abs(dev.forward(many) - one) < 1e-4)
+
+
+@pytest.mark.parametrize("qtype", [capi.IQ2_XXS, capi.MXFP4, capi.Q6_K, capi.Q2_K, capi.Q8_0])
+def test_deepseek_style_layer_with_shared_expert(qtype):
+    ora, dev = build(qtype, 1024, 512, 16, 4, 80, shared_inter=512, gating="sigmoid", n_group=4, topk_group=2,
+                     weights_scale=2.5, router_bias=np.linspace(-0.02, 0.02, 16).astype(np.float32))
+    for tokens in (1, 5):
+        x = synth.normal(81 + tokens, (tokens, 1024))
+        assert close(dev.forward(x), ora.forward(x))
+
+
+def test_moe_rejects_mismatched_shapes():
+    gate = capi.Weight.upload(capi.Q8_0, synth.normal_quantized(capi.Q8_0, 1, 4 * 32 * 256, 0.02), 4 * 32, 256)
+    down = capi.Weight.upload(capi.Q8_0, synth.normal_quantized(capi.Q8_0, 2, 4 * 256 * 32, 0.02), 4 * 256, 32)
+    rw = synth.normal(3, (4, 256))
+    with pytest.raises(capi.JoshuaHipError):
+        capi.Moe(capi.MoeConfig(4, 5, 256, 32, 0, 1, 0.0, 1, 1), rw, gate, gate, down)      # k > E
+    with pytest.raises(capi.JoshuaHipError):
+        capi.Moe(capi.MoeConfig(4, 2, 256, 64, 0, 1, 0.0, 1, 1), rw, gate, gate, down)      # wrong inter
