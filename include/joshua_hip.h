@@ -150,6 +150,46 @@ int jq_moe_route(jq_moe *moe, size_t n_tokens, const float *x, uint32_t *ids, fl
  * its scratch buffers). */
 int jq_moe_forward(jq_moe *moe, size_t n_tokens, const float *x, float *y, int ptrs_are_device, void *stream);
 
+/* ---- Dense Qwen3 decoder (end-to-end decode harness) -----------------------------
+ * The graph the reference runs for a qwen3 GGUF: embedding gather, per layer
+ * RMSNorm -> q/k/v -> per-head q/k RMSNorm -> half-split RoPE -> KV append ->
+ * causal GQA attention -> o + residual -> RMSNorm -> SwiGLU MLP + residual,
+ * then the last position's output norm and logits
+ * (reference: src/embedding.rs:297-396 for the layer, src/quantized_qwen3_moe.rs:
+ * 231-386,776-819 for attention, RoPE, KV cache and last-token logits;
+ * src/engine.rs:1149-1294 for the prefill-then-one-token-per-step contract). */
+typedef struct jq_model jq_model;
+
+typedef struct {
+    uint32_t n_layer, hidden, n_head, n_kv_head, head_dim, ffn, vocab, n_ctx;
+    float rms_eps, rope_theta;
+} jq_qwen3_config;
+
+int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out);
+void jq_qwen3_free(jq_model *model);
+
+/* Installs one tensor under its GGUF name ("token_embd.weight",
+ * "blk.3.attn_q.weight", "blk.3.attn_q_norm.weight", "output_norm.weight",
+ * "output.weight", ...).  ggml_type 0 is F32 (norm weights); the others are the
+ * JQ_TYPE_* ids, uploaded in native block layout.  The expected shape comes
+ * from the configuration; a wrong byte count fails. */
+int jq_qwen3_set_tensor(jq_model *model, const char *name, uint32_t ggml_type, const void *data,
+                        size_t nbytes);
+
+/* Appends n_tokens tokens at absolute position pos (which must equal the number
+ * of tokens fed so far) and writes vocab logits for the last one
+ * (the contract of the reference's plugin ABI, src/npu/mod.rs:44-50).  tokens is
+ * a host pointer; logits goes to host or device memory. */
+int jq_qwen3_forward(jq_model *model, const uint32_t *tokens, uint32_t n_tokens, uint32_t pos,
+                     float *logits, int logits_on_device, void *stream);
+
+/* Greedy pick over the logits of the last forward: the LAST index holding the
+ * maximum, as the reference's sampler does (src/engine.rs:2371-2378). */
+int jq_qwen3_greedy(jq_model *model, uint32_t *token, void *stream);
+
+/* Forgets the KV cache (reference: clear_kv_cache, src/quantized_qwen3_moe.rs:822-826). */
+int jq_qwen3_reset(jq_model *model);
+
 /* Blocks until everything enqueued on `stream` has finished. */
 int jq_stream_synchronize(void *stream);
 

@@ -23,6 +23,7 @@ EXPORTS = (
     "jq_last_error", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
     "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_try_matmul_fused", "jq_dequantize",
     "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
+    "jq_qwen3_create", "jq_qwen3_free", "jq_qwen3_set_tensor", "jq_qwen3_forward", "jq_qwen3_greedy", "jq_qwen3_reset",
 )
 
 
@@ -35,6 +36,14 @@ class MoeConfig(ctypes.Structure):
     _fields_ = [("n_expert", ctypes.c_uint32), ("n_expert_used", ctypes.c_uint32), ("hidden", ctypes.c_uint32),
                 ("inter", ctypes.c_uint32), ("gating", ctypes.c_uint32), ("norm_topk", ctypes.c_uint32),
                 ("weights_scale", ctypes.c_float), ("n_group", ctypes.c_uint32), ("topk_group", ctypes.c_uint32)]
+
+
+class Qwen3Config(ctypes.Structure):
+    """jq_qwen3_config of include/joshua_hip.h."""
+    _fields_ = [("n_layer", ctypes.c_uint32), ("hidden", ctypes.c_uint32), ("n_head", ctypes.c_uint32),
+                ("n_kv_head", ctypes.c_uint32), ("head_dim", ctypes.c_uint32), ("ffn", ctypes.c_uint32),
+                ("vocab", ctypes.c_uint32), ("n_ctx", ctypes.c_uint32), ("rms_eps", ctypes.c_float),
+                ("rope_theta", ctypes.c_float)]
 
 
 _lib = None
@@ -80,6 +89,13 @@ def lib() -> ctypes.CDLL:
         L.jq_moe_free.restype = None
         L.jq_moe_route.argtypes = [vp, sz, vp, vp, vp, i32, vp]
         L.jq_moe_forward.argtypes = [vp, sz, vp, vp, i32, vp]
+        L.jq_qwen3_create.argtypes = [ctypes.POINTER(Qwen3Config), ctypes.POINTER(vp)]
+        L.jq_qwen3_free.argtypes = [vp]
+        L.jq_qwen3_free.restype = None
+        L.jq_qwen3_set_tensor.argtypes = [vp, ctypes.c_char_p, u32, vp, sz]
+        L.jq_qwen3_forward.argtypes = [vp, vp, u32, u32, vp, i32, vp]
+        L.jq_qwen3_greedy.argtypes = [vp, ctypes.POINTER(u32), vp]
+        L.jq_qwen3_reset.argtypes = [vp]
         _lib = L
     return _lib
 
@@ -251,3 +267,50 @@ class Moe:
 
     def forward_dev(self, n_tokens: int, x_ptr: int, y_ptr: int, stream: int = 0) -> None:
         _check(lib().jq_moe_forward(self._h, n_tokens, x_ptr, y_ptr, 1, stream or None))
+
+
+class Qwen3:
+    """The dense Qwen3 decoder graph on the device, fed and stepped like the reference's
+    model object (reference: src/quantized_qwen3_moe.rs:792-826 forward / clear_kv_cache;
+    driver loop src/engine.rs:1149-1294)."""
+
+    def __init__(self, cfg: Qwen3Config):
+        self.cfg = cfg
+        out = ctypes.c_void_p()
+        _check(lib().jq_qwen3_create(ctypes.byref(cfg), ctypes.byref(out)))
+        self._h = out
+
+    def close(self) -> None:
+        if self._h:
+            lib().jq_qwen3_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_tensor(self, name: str, qtype: int, data) -> None:
+        """qtype 0: f32 vector; else packed blocks of that GGUF type."""
+        a = np.ascontiguousarray(data, dtype=np.float32) if qtype == 0 else _host_bytes(data)
+        _check(lib().jq_qwen3_set_tensor(self._h, name.encode(), qtype, a.ctypes.data, a.nbytes))
+
+    def forward(self, tokens, pos: int) -> np.ndarray:
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        logits = np.empty(self.cfg.vocab, np.float32)
+        _check(lib().jq_qwen3_forward(self._h, t.ctypes.data, t.size, pos, logits.ctypes.data, 0, None))
+        return logits
+
+    def forward_only(self, tokens, pos: int, stream: int = 0) -> None:
+        """Enqueues the step and leaves the logits on the device (for greedy())."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        _check(lib().jq_qwen3_forward(self._h, t.ctypes.data, t.size, pos, None, 1, stream or None))
+
+    def greedy(self, stream: int = 0) -> int:
+        tok = ctypes.c_uint32()
+        _check(lib().jq_qwen3_greedy(self._h, ctypes.byref(tok), stream or None))
+        return tok.value
+
+    def reset(self) -> None:
+        _check(lib().jq_qwen3_reset(self._h))

@@ -8,11 +8,14 @@
 #include <cstdlib>
 #include <algorithm>
 #include <cstring>
+#include <map>
 #include <mutex>
+#include <string>
 #include <vector>
 
 #include "../../include/joshua_hip.h"
 #include "kernels_mfma_q4k.hpp"
+#include "kernels_graph.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_valu.hpp"
 
@@ -688,6 +691,260 @@ int jq_moe_forward(jq_moe *m, size_t n_tokens, const float *x, float *y, int ptr
     if (moe_forward_dev(m, n_tokens, (const float *)xd.p, (float *)yd.p, s)) return 1;
     HIP_TRY(hipMemcpyAsync(y, yd.p, bytes, hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+}  // extern "C"
+
+// ---- dense Qwen3 decoder ------------------------------------------------------------
+
+struct jq_model {
+    jq_qwen3_config cfg;
+    std::map<std::string, jq_weight *> q;   // quantized matrices by GGUF name
+    std::map<std::string, float *> f;       // f32 vectors by GGUF name
+    std::vector<float *> kc, vc;            // per layer [n_kv, n_ctx, d]
+    uint32_t n_past = 0;
+    size_t cap_tokens = 0;
+    uint32_t *ids = nullptr, *pick = nullptr;
+    float *x = nullptr, *hn = nullptr, *qb = nullptr, *kb = nullptr, *vb = nullptr, *att = nullptr, *proj = nullptr,
+          *g = nullptr, *u = nullptr, *mid = nullptr, *logits = nullptr;
+    std::mutex mu;
+};
+
+namespace {
+
+void model_free_scratch(jq_model *m) {
+    for (void *p : {(void *)m->ids, (void *)m->x, (void *)m->hn, (void *)m->qb, (void *)m->kb, (void *)m->vb,
+                    (void *)m->att, (void *)m->proj, (void *)m->g, (void *)m->u, (void *)m->mid})
+        if (p) (void)hipFree(p);
+    m->ids = nullptr;
+    m->x = m->hn = m->qb = m->kb = m->vb = m->att = m->proj = m->g = m->u = m->mid = nullptr;
+    m->cap_tokens = 0;
+}
+
+int model_reserve(jq_model *m, size_t T) {
+    if (T <= m->cap_tokens) return 0;
+    model_free_scratch(m);
+    const jq_qwen3_config &c = m->cfg;
+    size_t qd = (size_t)c.n_head * c.head_dim, kd = (size_t)c.n_kv_head * c.head_dim;
+    HIP_TRY(hipMalloc((void **)&m->ids, T * sizeof(uint32_t)));
+    HIP_TRY(hipMalloc((void **)&m->x, T * c.hidden * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->hn, T * c.hidden * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->qb, T * qd * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->kb, T * kd * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->vb, T * kd * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->att, T * qd * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->proj, T * c.hidden * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->g, T * c.ffn * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->u, T * c.ffn * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->mid, T * c.ffn * sizeof(float)));
+    m->cap_tokens = T;
+    return 0;
+}
+
+// Expected [n, k] of a tensor name; k == 0 marks an f32 vector of length n.
+bool qwen3_shape(const jq_qwen3_config &c, const std::string &name, size_t *n, size_t *k) {
+    size_t qd = (size_t)c.n_head * c.head_dim, kd = (size_t)c.n_kv_head * c.head_dim;
+    auto ends = [&](const char *suf) {
+        size_t l = strlen(suf);
+        return name.size() >= l && name.compare(name.size() - l, l, suf) == 0;
+    };
+    if (name == "token_embd.weight" || name == "output.weight") { *n = c.vocab; *k = c.hidden; return true; }
+    if (name == "output_norm.weight") { *n = c.hidden; *k = 0; return true; }
+    if (name.rfind("blk.", 0) != 0) return false;
+    if (ends(".attn_norm.weight") || ends(".ffn_norm.weight")) { *n = c.hidden; *k = 0; return true; }
+    if (ends(".attn_q_norm.weight") || ends(".attn_k_norm.weight")) { *n = c.head_dim; *k = 0; return true; }
+    if (ends(".attn_q.weight")) { *n = qd; *k = c.hidden; return true; }
+    if (ends(".attn_k.weight") || ends(".attn_v.weight")) { *n = kd; *k = c.hidden; return true; }
+    if (ends(".attn_output.weight")) { *n = c.hidden; *k = qd; return true; }
+    if (ends(".ffn_gate.weight") || ends(".ffn_up.weight")) { *n = c.ffn; *k = c.hidden; return true; }
+    if (ends(".ffn_down.weight")) { *n = c.hidden; *k = c.ffn; return true; }
+    return false;
+}
+
+int model_mm(jq_model *m, const std::string &name, const float *x, float *y, size_t T, hipStream_t s) {
+    auto it = m->q.find(name);
+    if (it == m->q.end()) return fail("qwen3: missing tensor `%s`", name.c_str());
+    const jq_weight *w = it->second;
+    return dispatch_matmul(w->type, w->dev, w->row_bytes, x, y, T, w->k, w->n, s);
+}
+
+int model_vec(jq_model *m, const std::string &name, const float **out) {
+    auto it = m->f.find(name);
+    if (it == m->f.end()) return fail("qwen3: missing tensor `%s`", name.c_str());
+    *out = it->second;
+    return 0;
+}
+
+unsigned grid_for(size_t total) { return (unsigned)std::min<size_t>((total + 255) / 256, 8192); }
+
+int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
+    const jq_qwen3_config &c = m->cfg;
+    const int d = (int)c.head_dim, nh = (int)c.n_head, nkv = (int)c.n_kv_head;
+    const size_t kd = (size_t)nkv * d;
+    auto emb = m->q.find("token_embd.weight");
+    if (emb == m->q.end()) return fail("qwen3: missing tensor `token_embd.weight`");
+    if (dispatch_decode(emb->second, m->ids, m->x, T, s)) return 1;
+    const float sqrt_d = sqrtf((float)d);
+    for (uint32_t l = 0; l < c.n_layer; l++) {
+        const std::string p = "blk." + std::to_string(l);
+        const float *w_an, *w_fn, *w_qn, *w_kn;
+        if (model_vec(m, p + ".attn_norm.weight", &w_an) || model_vec(m, p + ".ffn_norm.weight", &w_fn) ||
+            model_vec(m, p + ".attn_q_norm.weight", &w_qn) || model_vec(m, p + ".attn_k_norm.weight", &w_kn))
+            return 1;
+        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(256), 0, s, m->x, w_an, c.rms_eps, m->hn, (int)c.hidden);
+        if (model_mm(m, p + ".attn_q.weight", m->hn, m->qb, T, s) || model_mm(m, p + ".attn_k.weight", m->hn, m->kb, T, s) ||
+            model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s))
+            return 1;
+        hipLaunchKernelGGL(jq::headnorm_rope, dim3(T * nh), dim3(64), 0, s, m->qb, w_qn, c.rms_eps, nh, d, (int)pos,
+                           c.rope_theta);
+        hipLaunchKernelGGL(jq::headnorm_rope, dim3(T * nkv), dim3(64), 0, s, m->kb, w_kn, c.rms_eps, nkv, d, (int)pos,
+                           c.rope_theta);
+        hipLaunchKernelGGL(jq::kv_append, dim3(grid_for(T * kd)), dim3(256), 0, s, m->kb, m->kc[l], (int)T, nkv, d,
+                           (int)pos, (int)c.n_ctx);
+        hipLaunchKernelGGL(jq::kv_append, dim3(grid_for(T * kd)), dim3(256), 0, s, m->vb, m->vc[l], (int)T, nkv, d,
+                           (int)pos, (int)c.n_ctx);
+        size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
+        hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, m->qb, m->kc[l], m->vc[l], m->att, nh, nkv,
+                           d, (int)pos, (int)c.n_ctx, sqrt_d);
+        if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
+        hipLaunchKernelGGL(jq::add_rows, dim3(grid_for((size_t)T * c.hidden)), dim3(256), 0, s, m->proj, m->x, m->x,
+                           (size_t)T * c.hidden);
+        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(256), 0, s, m->x, w_fn, c.rms_eps, m->hn, (int)c.hidden);
+        if (model_mm(m, p + ".ffn_gate.weight", m->hn, m->g, T, s) || model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s))
+            return 1;
+        hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, m->g, m->u, m->mid,
+                           (size_t)T * c.ffn);
+        if (model_mm(m, p + ".ffn_down.weight", m->mid, m->proj, T, s)) return 1;
+        hipLaunchKernelGGL(jq::add_rows, dim3(grid_for((size_t)T * c.hidden)), dim3(256), 0, s, m->proj, m->x, m->x,
+                           (size_t)T * c.hidden);
+    }
+    const float *w_on;
+    if (model_vec(m, "output_norm.weight", &w_on)) return 1;
+    // logits only for the last position (reference: src/quantized_qwen3_moe.rs:816-818)
+    hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(1), dim3(256), 0, s, m->x + (size_t)(T - 1) * c.hidden, w_on, c.rms_eps,
+                       m->hn, (int)c.hidden);
+    // tie_word_embeddings conversions ship no output head (src/quantized_qwen3_moe.rs:739-743)
+    const char *head = m->q.count("output.weight") ? "output.weight" : "token_embd.weight";
+    if (model_mm(m, head, m->hn, m->logits, 1, s)) return 1;
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out) {
+    if (!out) return fail("jq_qwen3_create: out is null");
+    *out = nullptr;
+    if (!cfg) return fail("jq_qwen3_create: cfg is null");
+    const jq_qwen3_config &c = *cfg;
+    if (!c.n_layer || !c.hidden || !c.n_head || !c.n_kv_head || !c.head_dim || !c.ffn || !c.vocab || !c.n_ctx)
+        return fail("qwen3: zero in configuration");
+    if (c.n_head % c.n_kv_head != 0) return fail("qwen3: %u query heads over %u kv heads", c.n_head, c.n_kv_head);
+    if (c.head_dim % 8 != 0 || c.hidden % 4 != 0 || c.ffn % 4 != 0) return fail("qwen3: dimensions must be multiples of 4/8");
+    if (ensure_init()) return 1;
+    jq_model *m = new jq_model;
+    m->cfg = c;
+    size_t per = (size_t)c.n_kv_head * c.n_ctx * c.head_dim * sizeof(float);
+    for (uint32_t l = 0; l < c.n_layer; l++) {
+        float *k = nullptr, *v = nullptr;
+        if (hipMalloc((void **)&k, per) != hipSuccess || hipMalloc((void **)&v, per) != hipSuccess) {
+            if (k) (void)hipFree(k);
+            jq_qwen3_free(m);
+            return fail("qwen3: KV cache allocation failed (%zu bytes per layer)", 2 * per);
+        }
+        m->kc.push_back(k);
+        m->vc.push_back(v);
+    }
+    if (hipMalloc((void **)&m->logits, c.vocab * sizeof(float)) != hipSuccess ||
+        hipMalloc((void **)&m->pick, sizeof(uint32_t)) != hipSuccess) {
+        jq_qwen3_free(m);
+        return fail("qwen3: logits allocation failed");
+    }
+    *out = m;
+    return 0;
+}
+
+void jq_qwen3_free(jq_model *m) {
+    if (!m) return;
+    model_free_scratch(m);
+    for (auto &kv : m->q) jq_free(kv.second);
+    for (auto &kv : m->f) (void)hipFree(kv.second);
+    for (float *p : m->kc) (void)hipFree(p);
+    for (float *p : m->vc) (void)hipFree(p);
+    if (m->logits) (void)hipFree(m->logits);
+    if (m->pick) (void)hipFree(m->pick);
+    delete m;
+}
+
+int jq_qwen3_set_tensor(jq_model *m, const char *name, uint32_t ggml_type, const void *data, size_t nbytes) {
+    if (!m || !name || !data) return fail("jq_qwen3_set_tensor: null argument");
+    size_t n, k;
+    if (!qwen3_shape(m->cfg, name, &n, &k)) return fail("qwen3: unknown tensor `%s`", name);
+    std::lock_guard<std::mutex> lock(m->mu);
+    if (k == 0) {
+        if (ggml_type != 0) return fail("qwen3: `%s` must be F32", name);
+        if (nbytes != n * sizeof(float)) return fail("qwen3: `%s` holds %zu bytes, expected %zu", name, nbytes, n * sizeof(float));
+        float *dev = nullptr;
+        HIP_TRY(hipMalloc((void **)&dev, nbytes));
+        hipError_t e = hipMemcpy(dev, data, nbytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(dev);
+            return fail("qwen3: upload of `%s` failed: %s", name, hipGetErrorString(e));
+        }
+        auto old = m->f.find(name);
+        if (old != m->f.end()) (void)hipFree(old->second);
+        m->f[name] = dev;
+        return 0;
+    }
+    jq_weight *w = nullptr;
+    if (jq_upload(ggml_type, data, nbytes, n, k, 0, &w)) return 1;
+    auto old = m->q.find(name);
+    if (old != m->q.end()) jq_free(old->second);
+    m->q[name] = w;
+    return 0;
+}
+
+int jq_qwen3_forward(jq_model *m, const uint32_t *tokens, uint32_t n_tokens, uint32_t pos, float *logits,
+                     int logits_on_device, void *stream) {
+    if (!m || !tokens) return fail("jq_qwen3_forward: null argument");
+    if (n_tokens == 0) return fail("qwen3: forward needs at least one token");
+    std::lock_guard<std::mutex> lock(m->mu);
+    // the KV-cache contract of the plugin boundary (reference: crates/joshua-mock-npu/src/lib.rs:89-95)
+    if (pos != m->n_past) return fail("qwen3: pos %u does not match the %u tokens fed so far", pos, m->n_past);
+    if ((uint64_t)pos + n_tokens > m->cfg.n_ctx)
+        return fail("qwen3: %u + %u tokens exceed the context of %u", pos, n_tokens, m->cfg.n_ctx);
+    for (uint32_t i = 0; i < n_tokens; i++)
+        if (tokens[i] >= m->cfg.vocab) return fail("embedding id %u is out of range for %u rows", tokens[i], m->cfg.vocab);
+    hipStream_t s = (hipStream_t)stream;
+    if (model_reserve(m, n_tokens)) return 1;
+    HIP_TRY(hipMemcpyAsync(m->ids, tokens, n_tokens * sizeof(uint32_t), hipMemcpyHostToDevice, s));
+    if (model_forward_dev(m, n_tokens, pos, s)) return 1;
+    m->n_past = pos + n_tokens;
+    if (logits) {
+        HIP_TRY(hipMemcpyAsync(logits, m->logits, m->cfg.vocab * sizeof(float),
+                               logits_on_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost, s));
+        if (!logits_on_device) HIP_TRY(hipStreamSynchronize(s));
+    }
+    return 0;
+}
+
+int jq_qwen3_greedy(jq_model *m, uint32_t *token, void *stream) {
+    if (!m || !token) return fail("jq_qwen3_greedy: null argument");
+    hipStream_t s = (hipStream_t)stream;
+    std::lock_guard<std::mutex> lock(m->mu);
+    hipLaunchKernelGGL(jq::argmax_last, dim3(1), dim3(1024), 0, s, m->logits, (int)m->cfg.vocab, m->pick);
+    HIP_TRY(hipMemcpyAsync(token, m->pick, sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int jq_qwen3_reset(jq_model *m) {
+    if (!m) return fail("jq_qwen3_reset: model is null");
+    std::lock_guard<std::mutex> lock(m->mu);
+    m->n_past = 0;
     return 0;
 }
 

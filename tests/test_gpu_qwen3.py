@@ -1,0 +1,114 @@
+"""End-to-end dense Qwen3 decode on the device against the numpy graph over the
+oracle matmul: teacher-forced logits after a prefill and on every decode step,
+the KV-cache position contract, and the greedy pick's tie order."""
+import numpy as np
+import pytest
+
+import oracle
+from oracle import qwen3 as oq
+from joshua_amd import capi
+from joshua_amd.synth.model import qwen3_tensors
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(n_layer=3, hidden=512, n_head=4, n_kv_head=2, head_dim=64, ffn=1024, vocab=768, n_ctx=48,
+           rms_eps=1e-6, rope_theta=1e6)
+
+
+def make(cfg, seed, mix="q4_k_m", override=None):
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(cfg, seed, mix)}
+    if override:
+        tensors.update(override)
+    c = capi.Qwen3Config(cfg["n_layer"], cfg["hidden"], cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"], cfg["ffn"],
+                         cfg["vocab"], cfg["n_ctx"], cfg["rms_eps"], cfg["rope_theta"])
+    m = capi.Qwen3(c)
+    for n, (qt, d) in tensors.items():
+        m.set_tensor(n, qt, d)
+    return m, oq.Qwen3Oracle(cfg, tensors, avx2=oracle.have_avx2())
+
+
+def close(got, ref, tol=1e-3):
+    # the bound the reference's acceptance uses for f32 results: |gpu - ref| <= tol * max(|ref|, 1)
+    err = np.abs(got - ref) / np.maximum(np.abs(ref), 1.0)
+    return float(err.max()) <= tol, float(err.max())
+
+
+@pytest.mark.parametrize("mix", ["q4_k_m", "8"])
+def test_teacher_forced_logits(mix):
+    m, o = make(CFG, 21, mix)
+    prompt = [3, 700, 41, 41, 256, 9, 88, 511, 2, 640, 77]
+    got, ref = m.forward(prompt, 0), o.forward(prompt, 0)
+    ok, e = close(got, ref)
+    assert ok, f"prefill: {e}"
+    pos = len(prompt)
+    for t in [5, 123, 767, 0, 350, 12]:
+        got, ref = m.forward([t], pos), o.forward([t], pos)
+        ok, e = close(got, ref)
+        assert ok, f"pos {pos}: {e}"
+        g = m.greedy()
+        top2 = np.sort(ref)[-2:]
+        if top2[1] - top2[0] > 2e-3 * max(abs(top2[1]), 1.0):
+            assert g == oq.greedy(ref)
+        assert got[g] == got.max()
+        pos += 1
+
+
+def test_prefill_in_two_chunks_matches_one():
+    m, o = make(CFG, 22)
+    toks = list(range(10, 30))
+    ref = o.forward(toks, 0)
+    m.forward(toks[:13], 0)
+    got = m.forward(toks[13:], 13)
+    ok, e = close(got, ref)
+    assert ok, e
+
+
+def test_position_contract_and_reset():
+    m, _ = make(CFG, 23)
+    a = m.forward([1, 2, 3], 0)
+    with pytest.raises(capi.JoshuaHipError, match="does not match"):
+        m.forward([4], 5)
+    with pytest.raises(capi.JoshuaHipError, match="exceed the context"):
+        m.forward(list(range(46)), 3)
+    with pytest.raises(capi.JoshuaHipError, match="out of range"):
+        m.forward([768], 3)
+    with pytest.raises(capi.JoshuaHipError, match="at least one token"):
+        m.forward([], 3)
+    m.reset()
+    b = m.forward([1, 2, 3], 0)
+    assert np.array_equal(a, b)
+
+
+def test_missing_tensor_is_reported():
+    c = capi.Qwen3Config(1, 256, 2, 1, 64, 256, 256, 8, 1e-6, 1e4)
+    m = capi.Qwen3(c)
+    with pytest.raises(capi.JoshuaHipError, match="missing tensor"):
+        m.forward([1], 0)
+    with pytest.raises(capi.JoshuaHipError, match="unknown tensor"):
+        m.set_tensor("blk.0.nope.weight", 0, np.zeros(4, np.float32))
+    with pytest.raises(capi.JoshuaHipError, match="expected"):
+        m.set_tensor("output_norm.weight", 0, np.zeros(4, np.float32))
+
+
+def test_greedy_returns_last_index_of_equal_logits():
+    # every row of the head identical -> all logits equal -> the last index wins
+    from joshua_amd.synth import normal, quantize
+    row = normal(5, (1, CFG["hidden"]), 0.05)
+    head = quantize(8, np.repeat(row, CFG["vocab"], axis=0))
+    m, _ = make(CFG, 24, override={"output.weight": (8, head)})
+    logits = m.forward([1, 2], 0)
+    assert np.all(logits == logits[0])
+    assert m.greedy() == CFG["vocab"] - 1
+
+
+def test_tied_embeddings_when_no_output_head():
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(CFG, 25)}
+    del tensors["output.weight"]
+    c = capi.Qwen3Config(CFG["n_layer"], CFG["hidden"], CFG["n_head"], CFG["n_kv_head"], CFG["head_dim"], CFG["ffn"],
+                         CFG["vocab"], CFG["n_ctx"], CFG["rms_eps"], CFG["rope_theta"])
+    m = capi.Qwen3(c)
+    for n, (qt, d) in tensors.items():
+        m.set_tensor(n, qt, d)
+    o = oq.Qwen3Oracle(CFG, tensors, avx2=oracle.have_avx2())
+    ok, e = close(m.forward([9, 8, 7], 0), o.forward([9, 8, 7], 0))
+    assert ok, e
