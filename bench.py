@@ -59,6 +59,84 @@ def cpu_baseline(blocks: np.ndarray, lhs: np.ndarray, budget_s: float) -> dict:
                       f"{threads} threads, 3 warm-up runs", "ms_per_step": round(med * 1e3, 4)}
 
 
+QWEN3_8B = dict(n_layer=36, hidden=4096, n_head=32, n_kv_head=8, head_dim=128, ffn=12288, vocab=151936, n_ctx=768,
+                rms_eps=1e-6, rope_theta=1e6)
+
+
+def decode_leg(prompt_len: int, n_decode: int, cpu_seconds: float, share_layers: bool) -> dict:
+    """End-to-end greedy decode of a random-init Qwen3-8B-shaped Q4_K_M model: prefill of
+    prompt_len uniform-random ids, then n_decode greedy tokens, one host round trip per
+    token (the engine's loop, reference: src/engine.rs:1149-1294).  The CPU leg runs the
+    same graph over the oracle's AVX2 kernels for a bounded number of tokens."""
+    from joshua_amd import capi
+    from joshua_amd.synth import uniform_u32
+    from joshua_amd.synth.model import qwen3_tensors
+
+    cfg = dict(QWEN3_8B, n_ctx=prompt_len + n_decode)
+    t0 = time.perf_counter()
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(cfg, 7, "q4_k_m", share_layers=share_layers)}
+    t_gen = time.perf_counter() - t0
+    c = capi.Qwen3Config(cfg["n_layer"], cfg["hidden"], cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"], cfg["ffn"],
+                         cfg["vocab"], cfg["n_ctx"], cfg["rms_eps"], cfg["rope_theta"])
+    model = capi.Qwen3(c)
+    wbytes = 0
+    for name, (qt, d) in tensors.items():
+        model.set_tensor(name, qt, d)
+        if qt != 0 and name != "token_embd.weight":
+            wbytes += d.nbytes
+    prompt = uniform_u32(31, prompt_len, cfg["vocab"])
+    # warm-up: a short prefill and a few steps, then start over
+    model.forward_only(prompt[:16], 0)
+    for i in range(4):
+        model.forward_only([model.greedy()], 16 + i)
+    model.reset()
+    capi.stream_synchronize()
+    t0 = time.perf_counter()
+    model.forward_only(prompt, 0)
+    tok = model.greedy()
+    t_prefill = time.perf_counter() - t0
+    out_tokens = [tok]
+    t0 = time.perf_counter()
+    for i in range(n_decode - 1):
+        model.forward_only([tok], prompt_len + i)
+        tok = model.greedy()
+        out_tokens.append(tok)
+    t_dec = time.perf_counter() - t0
+    tps = (n_decode - 1) / t_dec
+    res = {"tokens_per_s": round(tps, 2), "ms_per_token": round(1e3 / tps, 4),
+           "prefill_tokens_per_s": round(prompt_len / t_prefill, 1),
+           "workload": f"Qwen3-8B-shaped random-init model, Q4_K_M mix (Q4_K + Q6_K), {prompt_len} uniform-random "
+                       f"prompt ids then {n_decode} greedy tokens, batch 1, f32 activations and KV cache",
+           "weight_bytes_per_token": wbytes, "weights_gbs": round(wbytes * tps / 1e9, 1),
+           "hbm_frac": round(wbytes * tps / 1e9 / HBM_PEAK_GBS, 4),
+           "layers_share_bytes": share_layers, "model_gen_s": round(t_gen, 1)}
+    if cpu_seconds > 0:
+        import oracle
+        from oracle import qwen3 as oq
+        if oracle.have_avx2():
+            threads = min(oracle.default_threads(), len(os.sched_getaffinity(0)))
+            o = oq.Qwen3Oracle(cfg, tensors, avx2=True, threads=threads)
+            n_pre = 8
+            ref_logits = o.forward(list(prompt[:n_pre]), 0)
+            # parity of the graph at full size: the same 8-token prefill on the device
+            model.reset()
+            got = model.forward(prompt[:n_pre], 0)
+            res["parity_ok"] = bool(np.all(np.abs(got - ref_logits) <= 1e-3 * np.maximum(np.abs(ref_logits), 1.0)))
+            times, t = [], int(oq.greedy(ref_logits))
+            t_end = time.perf_counter() + cpu_seconds
+            while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 64):
+                t0 = time.perf_counter()
+                t = oq.greedy(o.forward([t], n_pre + len(times)))
+                times.append(time.perf_counter() - t0)
+            cpu_tps = 1.0 / float(np.median(times))
+            res["cpu_baseline"] = {"value": round(cpu_tps, 3), "unit": "tokens/s", "cores": threads, "kind": "port",
+                                   "sample": f"median of {len(times)} greedy decode steps of the same model after an "
+                                             f"{n_pre}-token prefill, AVX2 row kernels, {threads} threads"}
+            res["speedup_vs_cpu"] = round(tps / cpu_tps, 2)
+    model.close()
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,6 +145,10 @@ def main() -> int:
     ap.add_argument("--m", type=int, default=1, help="activation rows (1 = decode GEMV)")
     ap.add_argument("--copies", type=int, default=24, help="distinct weight copies rotated through (cold HBM)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline (0 = skip)")
+    ap.add_argument("--decode", type=int, default=1, help="1: also run the Qwen3-8B-shaped end-to-end decode leg")
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--share-layers", type=int, default=0, help="1: draw each layer role's bytes once (faster set-up)")
     ap.add_argument("--no-graph", action="store_true", help="enqueue launches one by one instead of a HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -164,6 +246,11 @@ def main() -> int:
     }
     if args.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(blocks, lhs, args.cpu_seconds)
+    if args.decode:
+        del weights, base
+        torch.cuda.empty_cache()
+        out["decode"] = decode_leg(args.prompt, args.new_tokens, args.cpu_seconds, bool(args.share_layers))
+        parity_ok = parity_ok and out["decode"].get("parity_ok", True)
     print(json.dumps(out))
     return 0 if parity_ok else 1
 
