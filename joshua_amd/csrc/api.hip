@@ -706,6 +706,8 @@ struct jq_model {
     uint32_t n_past = 0;
     size_t cap_tokens = 0;
     uint32_t *ids = nullptr, *pick = nullptr;
+    int *pos = nullptr;       // device copy of the position of the step being run
+    float *part = nullptr;    // split-attention partials
     float *x = nullptr, *hn = nullptr, *qb = nullptr, *kb = nullptr, *vb = nullptr, *att = nullptr, *proj = nullptr,
           *g = nullptr, *u = nullptr, *mid = nullptr, *logits = nullptr;
     std::mutex mu;
@@ -780,50 +782,52 @@ unsigned grid_for(size_t total) { return (unsigned)std::min<size_t>((total + 255
 
 int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
     const jq_qwen3_config &c = m->cfg;
-    const int d = (int)c.head_dim, nh = (int)c.n_head, nkv = (int)c.n_kv_head;
-    const size_t kd = (size_t)nkv * d;
+    const int d = (int)c.head_dim, nh = (int)c.n_head, nkv = (int)c.n_kv_head, h = (int)c.hidden;
     auto emb = m->q.find("token_embd.weight");
     if (emb == m->q.end()) return fail("qwen3: missing tensor `token_embd.weight`");
     if (dispatch_decode(emb->second, m->ids, m->x, T, s)) return 1;
+    hipLaunchKernelGGL(jq::set_int, dim3(1), dim3(1), 0, s, m->pos, (int)pos);
     const float sqrt_d = sqrtf((float)d);
+    // few query rows over a long cache: split the keys over the chip
+    const bool split = T <= 8 && d % 64 == 0 && d <= 256;
+    const int n_chunks = (int)((pos + T + jq::ATT_CHUNK - 1) / jq::ATT_CHUNK);
+    const float *pending = nullptr;  // residual not yet added into x
     for (uint32_t l = 0; l < c.n_layer; l++) {
         const std::string p = "blk." + std::to_string(l);
         const float *w_an, *w_fn, *w_qn, *w_kn;
         if (model_vec(m, p + ".attn_norm.weight", &w_an) || model_vec(m, p + ".ffn_norm.weight", &w_fn) ||
             model_vec(m, p + ".attn_q_norm.weight", &w_qn) || model_vec(m, p + ".attn_k_norm.weight", &w_kn))
             return 1;
-        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(256), 0, s, m->x, w_an, c.rms_eps, m->hn, (int)c.hidden);
+        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, m->x, pending, w_an, c.rms_eps, m->hn, h);
         if (model_mm(m, p + ".attn_q.weight", m->hn, m->qb, T, s) || model_mm(m, p + ".attn_k.weight", m->hn, m->kb, T, s) ||
             model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s))
             return 1;
-        hipLaunchKernelGGL(jq::headnorm_rope, dim3(T * nh), dim3(64), 0, s, m->qb, w_qn, c.rms_eps, nh, d, (int)pos,
-                           c.rope_theta);
-        hipLaunchKernelGGL(jq::headnorm_rope, dim3(T * nkv), dim3(64), 0, s, m->kb, w_kn, c.rms_eps, nkv, d, (int)pos,
-                           c.rope_theta);
-        hipLaunchKernelGGL(jq::kv_append, dim3(grid_for(T * kd)), dim3(256), 0, s, m->kb, m->kc[l], (int)T, nkv, d,
-                           (int)pos, (int)c.n_ctx);
-        hipLaunchKernelGGL(jq::kv_append, dim3(grid_for(T * kd)), dim3(256), 0, s, m->vb, m->vc[l], (int)T, nkv, d,
-                           (int)pos, (int)c.n_ctx);
-        size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
-        hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, m->qb, m->kc[l], m->vc[l], m->att, nh, nkv,
-                           d, (int)pos, (int)c.n_ctx, sqrt_d);
+        hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, m->qb, m->kb, m->vb, w_qn,
+                           w_kn, c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
+        if (split) {
+            hipLaunchKernelGGL(jq::attention_split, dim3(T * nh * n_chunks), dim3(256), 0, s, m->qb, m->kc[l], m->vc[l],
+                               m->part, nh, nkv, d, m->pos, (int)c.n_ctx, sqrt_d, n_chunks);
+            hipLaunchKernelGGL(jq::attention_merge, dim3(T * nh), dim3(256), 0, s, m->part, m->att, d, n_chunks);
+        } else {
+            size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
+            hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, m->qb, m->kc[l], m->vc[l], m->att, nh,
+                               nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
+        }
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
-        hipLaunchKernelGGL(jq::add_rows, dim3(grid_for((size_t)T * c.hidden)), dim3(256), 0, s, m->proj, m->x, m->x,
-                           (size_t)T * c.hidden);
-        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(256), 0, s, m->x, w_fn, c.rms_eps, m->hn, (int)c.hidden);
+        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, m->x, m->proj, w_fn, c.rms_eps, m->hn, h);
         if (model_mm(m, p + ".ffn_gate.weight", m->hn, m->g, T, s) || model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s))
             return 1;
         hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, m->g, m->u, m->mid,
                            (size_t)T * c.ffn);
         if (model_mm(m, p + ".ffn_down.weight", m->mid, m->proj, T, s)) return 1;
-        hipLaunchKernelGGL(jq::add_rows, dim3(grid_for((size_t)T * c.hidden)), dim3(256), 0, s, m->proj, m->x, m->x,
-                           (size_t)T * c.hidden);
+        pending = m->proj;
     }
     const float *w_on;
     if (model_vec(m, "output_norm.weight", &w_on)) return 1;
     // logits only for the last position (reference: src/quantized_qwen3_moe.rs:816-818)
-    hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(1), dim3(256), 0, s, m->x + (size_t)(T - 1) * c.hidden, w_on, c.rms_eps,
-                       m->hn, (int)c.hidden);
+    const size_t last = (size_t)(T - 1) * h;
+    hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(1), dim3(1024), 0, s, m->x + last, pending ? pending + last : nullptr, w_on,
+                       c.rms_eps, m->hn, h);
     // tie_word_embeddings conversions ship no output head (src/quantized_qwen3_moe.rs:739-743)
     const char *head = m->q.count("output.weight") ? "output.weight" : "token_embd.weight";
     if (model_mm(m, head, m->hn, m->logits, 1, s)) return 1;
@@ -858,8 +862,11 @@ int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out) {
         m->kc.push_back(k);
         m->vc.push_back(v);
     }
+    const size_t part_floats = (size_t)8 * c.n_head * ((c.n_ctx + jq::ATT_CHUNK - 1) / jq::ATT_CHUNK) * (c.head_dim + 2);
     if (hipMalloc((void **)&m->logits, c.vocab * sizeof(float)) != hipSuccess ||
-        hipMalloc((void **)&m->pick, sizeof(uint32_t)) != hipSuccess) {
+        hipMalloc((void **)&m->pick, sizeof(uint32_t)) != hipSuccess ||
+        hipMalloc((void **)&m->pos, sizeof(int)) != hipSuccess ||
+        hipMalloc((void **)&m->part, part_floats * sizeof(float)) != hipSuccess) {
         jq_qwen3_free(m);
         return fail("qwen3: logits allocation failed");
     }
@@ -876,6 +883,8 @@ void jq_qwen3_free(jq_model *m) {
     for (float *p : m->vc) (void)hipFree(p);
     if (m->logits) (void)hipFree(m->logits);
     if (m->pick) (void)hipFree(m->pick);
+    if (m->pos) (void)hipFree(m->pos);
+    if (m->part) (void)hipFree(m->part);
     delete m;
 }
 

@@ -18,49 +18,77 @@ __device__ __forceinline__ float block_sum(float v, float *red) {  // blockDim.x
     return t;
 }
 
-// out[r, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * w   (+ res[r, :] first when given:
-// the sum is also written to res_out so the residual stream stays materialised)
-__global__ __launch_bounds__(256) void rmsnorm_rows(const float *__restrict__ x, const float *__restrict__ w, float eps,
-                                                     float *__restrict__ out, int h) {
+// x[r, :] += res[r, :] when res is given (the residual add of the layer before), then
+// out[r, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * w.  One workgroup of 1024 per row,
+// float4 per thread, the row kept in registers between the two passes (h <= 8192),
+// so a 4096-wide row costs one memory round trip instead of sixteen.
+__global__ __launch_bounds__(1024) void rmsnorm_rows(float *__restrict__ x, const float *__restrict__ res,
+                                                      const float *__restrict__ w, float eps,
+                                                      float *__restrict__ out, int h) {
     __shared__ float red[16];
-    const float *xr = x + (size_t)blockIdx.x * h;
+    float *xr = x + (size_t)blockIdx.x * h;
+    const float *rr = res ? res + (size_t)blockIdx.x * h : nullptr;
+    const int nv = h >> 2;  // h % 4 == 0
+    float4 keep[2];
     float ss = 0.0f;
-    for (int c = threadIdx.x; c < h; c += blockDim.x) ss = fmaf(xr[c], xr[c], ss);
+    int slot = 0;
+    for (int c = threadIdx.x; c < nv; c += 1024, slot++) {
+        float4 v = ((const float4 *)xr)[c];
+        if (rr) {
+            const float4 r = ((const float4 *)rr)[c];
+            v.x += r.x, v.y += r.y, v.z += r.z, v.w += r.w;
+            ((float4 *)xr)[c] = v;
+        }
+        if (slot < 2) keep[slot] = v;
+        ss = fmaf(v.x, v.x, ss), ss = fmaf(v.y, v.y, ss), ss = fmaf(v.z, v.z, ss), ss = fmaf(v.w, v.w, ss);
+    }
     ss = block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)h + eps);
-    for (int c = threadIdx.x; c < h; c += blockDim.x) out[(size_t)blockIdx.x * h + c] = xr[c] * inv * w[c];
-}
-
-// Per-head RMSNorm over head_dim, then half-split rotary embedding at position
-// pos0 + t; one wave per (token, head).  v: [T, n_heads*d] in place.
-// inv_freq_i = theta^(-2i/d); pairs (i, i + d/2)
-// (reference: src/quantized_qwen3_moe.rs:237-262,345-354; closed form in its test :867-895).
-__global__ __launch_bounds__(64) void headnorm_rope(float *__restrict__ v, const float *__restrict__ w, float eps,
-                                                     int n_heads, int d, int pos0, float theta) {
-    const int t = blockIdx.x / n_heads, hd = blockIdx.x % n_heads, lane = threadIdx.x;
-    float *p = v + ((size_t)t * n_heads + hd) * d;
-    float ss = 0.0f;
-    for (int c = lane; c < d; c += 64) ss = fmaf(p[c], p[c], ss);
-    ss = wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
-    const int half = d / 2;
-    const float pos = (float)(pos0 + t);
-    for (int i = lane; i < half; i += 64) {
-        const float a = p[i] * inv * w[i], b = p[i + half] * inv * w[i + half];
-        const float freq = 1.0f / powf(theta, (float)(2 * i) / (float)d);
-        const float ang = pos * freq, c = cosf(ang), s = sinf(ang);
-        p[i] = a * c - b * s;
-        p[i + half] = a * s + b * c;
+    slot = 0;
+    for (int c = threadIdx.x; c < nv; c += 1024, slot++) {
+        const float4 v = slot < 2 ? keep[slot] : ((const float4 *)xr)[c];
+        const float4 g = ((const float4 *)w)[c];
+        ((float4 *)(out + (size_t)blockIdx.x * h))[c] = float4{v.x * inv * g.x, v.y * inv * g.y, v.z * inv * g.z, v.w * inv * g.w};
     }
 }
 
-// cache[kvh, pos0 + t, :] = src[t, kvh*d .. +d]
-__global__ __launch_bounds__(256) void kv_append(const float *__restrict__ src, float *__restrict__ cache, int T,
-                                                  int n_kv, int d, int pos0, int n_ctx) {
-    const size_t total = (size_t)T * n_kv * d;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const int c = (int)(i % d), kvh = (int)((i / d) % n_kv), t = (int)(i / ((size_t)d * n_kv));
-        cache[((size_t)kvh * n_ctx + pos0 + t) * d + c] = src[i];
+// Per-head RMSNorm over head_dim then half-split rotary embedding at position
+// pos0 + t, one wave per (token, head) over the q heads, the k heads and the v heads of
+// a token: q is rewritten in place, k goes normed and rotated straight into the K
+// cache, v is copied into the V cache.  inv_freq_i = theta^(-2i/d); pairs (i, i + d/2)
+// (reference: src/quantized_qwen3_moe.rs:237-262,345-364; closed form in its test :867-895).
+// cache layout [kv_head, n_ctx, d]; *pos_ptr is the number of tokens already cached.
+__global__ __launch_bounds__(64) void qkv_norm_rope_cache(float *__restrict__ q, const float *__restrict__ k,
+                                                           const float *__restrict__ v, const float *__restrict__ wq,
+                                                           const float *__restrict__ wk, float eps, int n_head, int n_kv,
+                                                           int d, const int *__restrict__ pos_ptr, float theta,
+                                                           float *__restrict__ kc, float *__restrict__ vc, int n_ctx) {
+    const int per = n_head + 2 * n_kv;
+    const int t = blockIdx.x / per, j = blockIdx.x % per, lane = threadIdx.x;
+    const int pos = *pos_ptr + t;
+    if (j >= n_head + n_kv) {  // v head: plain copy
+        const int hd = j - n_head - n_kv;
+        const float *src = v + ((size_t)t * n_kv + hd) * d;
+        float *dst = vc + ((size_t)hd * n_ctx + pos) * d;
+        for (int c = lane; c < d; c += 64) dst[c] = src[c];
+        return;
+    }
+    const bool is_q = j < n_head;
+    const int hd = is_q ? j : j - n_head;
+    const float *src = is_q ? q + ((size_t)t * n_head + hd) * d : k + ((size_t)t * n_kv + hd) * d;
+    float *dst = is_q ? q + ((size_t)t * n_head + hd) * d : kc + ((size_t)hd * n_ctx + pos) * d;
+    const float *w = is_q ? wq : wk;
+    float ss = 0.0f;
+    for (int c = lane; c < d; c += 64) ss = fmaf(src[c], src[c], ss);
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    const int half = d / 2;
+    for (int i = lane; i < half; i += 64) {
+        const float a = src[i] * inv * w[i], b = src[i + half] * inv * w[i + half];
+        const float freq = 1.0f / powf(theta, (float)(2 * i) / (float)d);
+        const float ang = (float)pos * freq, c = cosf(ang), s = sinf(ang);
+        dst[i] = a * c - b * s;
+        dst[i + half] = a * s + b * c;
     }
 }
 
@@ -69,10 +97,11 @@ __global__ __launch_bounds__(256) void kv_append(const float *__restrict__ src, 
 // (reference: src/quantized_qwen3_moe.rs:366-379; mask :776-789).
 __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ q, const float *__restrict__ kc,
                                                        const float *__restrict__ vc, float *__restrict__ out,
-                                                       int n_head, int n_kv, int d, int pos0, int n_ctx, float sqrt_d) {
+                                                       int n_head, int n_kv, int d, const int *__restrict__ pos_ptr,
+                                                       int n_ctx, float sqrt_d) {
     extern __shared__ float sm[];  // q[d], scores[n_keys], red[16]
     const int t = blockIdx.x / n_head, hq = blockIdx.x % n_head;
-    const int kvh = hq / (n_head / n_kv), n_keys = pos0 + t + 1;
+    const int kvh = hq / (n_head / n_kv), n_keys = *pos_ptr + t + 1;
     float *qs = sm, *sc = sm + d, *red = sm + d + n_keys;
     const float *qp = q + ((size_t)t * n_head + hq) * d;
     for (int c = threadIdx.x; c < d; c += blockDim.x) qs[c] = qp[c];
@@ -115,6 +144,99 @@ __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ 
         out[((size_t)t * n_head + hq) * d + c] = acc;
     }
 }
+
+// Decode-shaped attention (few query tokens, long cache), split over the keys so the
+// whole chip works on it: one workgroup per (token, query head, chunk of ATT_CHUNK keys)
+// computes its chunk's scores, their maximum m, l = sum exp(s - m) and the unnormalised
+// sum exp(s - m) v, and writes (m, l, acc[d]) to part[(t*n_head + hq)*n_chunks + chunk];
+// attention_merge rescales the chunks to the common maximum and divides by the total.
+// 16 lanes per key (4 keys per wave step), d % 64 == 0.  Chunks past the causal limit
+// write l = 0 and are skipped by the merge.
+constexpr int ATT_CHUNK = 64;
+
+__global__ __launch_bounds__(256) void attention_split(const float *__restrict__ q, const float *__restrict__ kc,
+                                                        const float *__restrict__ vc, float *__restrict__ part,
+                                                        int n_head, int n_kv, int d, const int *__restrict__ pos_ptr,
+                                                        int n_ctx, float sqrt_d, int n_chunks) {
+    __shared__ float sc[ATT_CHUNK];
+    __shared__ float red[16];
+    __shared__ float accs[4][256];  // d <= 256
+    const int chunk = blockIdx.x % n_chunks, hq = (blockIdx.x / n_chunks) % n_head, t = blockIdx.x / (n_chunks * n_head);
+    const int kvh = hq / (n_head / n_kv), n_keys = *pos_ptr + t + 1;
+    const int j0 = chunk * ATT_CHUNK, nj = min(ATT_CHUNK, n_keys - j0);
+    float *po = part + ((size_t)(t * n_head + hq) * n_chunks + chunk) * (d + 2);
+    if (nj <= 0) {
+        if (threadIdx.x == 0) po[0] = -INFINITY, po[1] = 0.0f;
+        return;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15, kq = lane >> 4;
+    const float *qp = q + ((size_t)t * n_head + hq) * d;
+    const float *kb = kc + ((size_t)kvh * n_ctx + j0) * d;
+    // this lane's slice of q: floats [4*sub + 64*i, +4), i < d/64
+    float4 qv[4];
+    for (int i = 0; i < d / 64; i++) qv[i] = *(const float4 *)(qp + 4 * sub + 64 * i);
+    for (int j = wave * 4 + kq; j < ATT_CHUNK; j += 16) {
+        float acc = 0.0f;
+        if (j < nj) {
+            const float *kr = kb + (size_t)j * d;
+            for (int i = 0; i < d / 64; i++) {
+                const float4 kv = *(const float4 *)(kr + 4 * sub + 64 * i);
+                acc = fmaf(qv[i].x, kv.x, acc), acc = fmaf(qv[i].y, kv.y, acc);
+                acc = fmaf(qv[i].z, kv.z, acc), acc = fmaf(qv[i].w, kv.w, acc);
+            }
+        }
+        acc += __shfl_xor(acc, 1, 64), acc += __shfl_xor(acc, 2, 64);
+        acc += __shfl_xor(acc, 4, 64), acc += __shfl_xor(acc, 8, 64);
+        if (sub == 0) sc[j] = j < nj ? acc / sqrt_d : -INFINITY;
+    }
+    __syncthreads();
+    float mx = sc[lane];  // ATT_CHUNK == 64: every wave holds the whole chunk
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    const float e = expf(sc[lane] - mx);  // exp(-inf) = 0 for the masked tail
+    const float l = wave_sum(e);
+    __syncthreads();
+    if (wave == 0) sc[lane] = e;
+    __syncthreads();
+    // acc[c] = sum_j e_j v[j, c]: thread (c = tid % d, part = tid / d) strides the keys
+    const int nparts = 256 / d > 0 ? 256 / d : 1;
+    const float *vb = vc + ((size_t)kvh * n_ctx + j0) * d;
+    for (int c = threadIdx.x % d, pt = threadIdx.x / d; pt < nparts && c < d; pt = nparts) {
+        float acc = 0.0f;
+        for (int j = pt; j < nj; j += nparts) acc = fmaf(sc[j], vb[(size_t)j * d + c], acc);
+        accs[pt][c] = acc;
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float a = accs[0][c];
+        for (int pt = 1; pt < nparts; pt++) a += accs[pt][c];
+        po[2 + c] = a;
+    }
+    if (threadIdx.x == 0) po[0] = mx, po[1] = l;
+    (void)red;
+}
+
+__global__ __launch_bounds__(256) void attention_merge(const float *__restrict__ part, float *__restrict__ out, int d,
+                                                        int n_chunks) {
+    const float *pp = part + (size_t)blockIdx.x * n_chunks * (d + 2);
+    float mx = -INFINITY;
+    for (int ch = 0; ch < n_chunks; ch++) mx = fmaxf(mx, pp[(size_t)ch * (d + 2)]);
+    float tot = 0.0f;
+    for (int ch = 0; ch < n_chunks; ch++) {
+        const float l = pp[(size_t)ch * (d + 2) + 1];
+        if (l > 0.0f) tot += l * expf(pp[(size_t)ch * (d + 2)] - mx);
+    }
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float a = 0.0f;
+        for (int ch = 0; ch < n_chunks; ch++) {
+            const float l = pp[(size_t)ch * (d + 2) + 1];
+            if (l > 0.0f) a = fmaf(expf(pp[(size_t)ch * (d + 2)] - mx), pp[(size_t)ch * (d + 2) + 2 + c], a);
+        }
+        out[(size_t)blockIdx.x * d + c] = a / tot;
+    }
+}
+
+__global__ void set_int(int *p, int v) { *p = v; }
 
 __global__ __launch_bounds__(256) void add_rows(const float *__restrict__ a, const float *__restrict__ b,
                                                  float *__restrict__ out, size_t total) {

@@ -126,6 +126,44 @@ def test_q4k_activation_scales_span_many_orders():
     assert close(got, oracle.matmul_t(capi.Q4_K, (3, k, n), lhs, blocks, avx2=True))
 
 
+def q4k_integer_case(n, k, seed):
+    """Q4_K blocks with d = 1, dmin = 0, every sub-block scale 1 and at most 16 nonzero
+    nibbles per row; activations are integers whose every 16-element group has maximum
+    magnitude 4161407 (the fixed-point range of the MFMA kernel, so its activation scale
+    is exactly 1) at a position whose nibble is 0.  Every product and partial sum is an
+    integer below 2^24: f32 FMA, integer MFMA and int64 arithmetic must agree exactly."""
+    rng = np.random.default_rng(seed)
+    q = np.zeros((n, k), np.int64)
+    x = rng.integers(-65535, 65536, size=k).astype(np.int64)
+    big = np.arange(0, k, 16) + int(rng.integers(0, 16))     # same slot in every group
+    x[big] = 4161407 * rng.choice([-1, 1], size=k // 16)
+    free = np.setdiff1d(np.arange(k), big)
+    for r in range(n):
+        q[r, rng.choice(free, size=16, replace=False)] = rng.integers(1, 16, size=16)
+    qb = q.reshape(n, k // 256, 4, 2, 32)                      # chunk c: low nibbles 64c.., high 64c+32..
+    packed = (qb[:, :, :, 0, :] | (qb[:, :, :, 1, :] << 4)).astype(np.uint8).reshape(n, k // 256, 128)
+    blocks = np.zeros((n, k // 256, 144), np.uint8)
+    blocks[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks[:, :, 4:8] = 1                                       # sc_0..3 = 1, m = 0
+    blocks[:, :, 12:16] = 1                                     # sc_4..7 = 1 (low 4 bits), m = 0
+    blocks[:, :, 16:] = packed
+    return blocks.reshape(-1), q, x
+
+
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_q4k_integer_dot_products_are_bit_exact(m):
+    n, k = 160, 2048
+    blocks, q, x = q4k_integer_case(n, k, 90 + m)
+    assert np.array_equal(oracle.dequantize(capi.Q4_K, blocks).reshape(n, k), q.astype(np.float32))
+    lhs = np.stack([np.roll(x, 16 * i) for i in range(m)]).astype(np.float32)
+    want = (np.stack([np.roll(x, 16 * i) for i in range(m)]) @ q.T)
+    assert np.abs(want).max() < 2 ** 24
+    ref = oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())
+    assert np.array_equal(ref, want.astype(np.float32))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
 def test_iq2xxs_fixture_matmul(golden_dir):
     # reference: src/iq2xxs.rs:758-804
     m, k, n = 3, 512, 7

@@ -63,6 +63,23 @@ def test_prefill_in_two_chunks_matches_one():
     assert ok, e
 
 
+def test_decode_over_several_key_chunks():
+    """A cache longer than one 64-key chunk of the split attention kernel, entered both by a
+    long prefill and by short multi-token steps."""
+    cfg = dict(CFG, n_ctx=224, n_layer=2)
+    m, o = make(cfg, 26)
+    rng = np.random.default_rng(3)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=190)]
+    ok, e = close(m.forward(toks[:150], 0), o.forward(toks[:150], 0))
+    assert ok, f"prefill: {e}"
+    pos = 150
+    for step in (1, 5, 8, 1, 3, 1, 1):
+        chunk = toks[pos:pos + step]
+        ok, e = close(m.forward(chunk, pos), o.forward(chunk, pos))
+        assert ok, f"pos {pos} +{step}: {e}"
+        pos += step
+
+
 def test_position_contract_and_reset():
     m, _ = make(CFG, 23)
     a = m.forward([1, 2, 3], 0)
