@@ -126,7 +126,7 @@ def test_q4k_activation_scales_span_many_orders():
     assert close(got, oracle.matmul_t(capi.Q4_K, (3, k, n), lhs, blocks, avx2=True))
 
 
-def q4k_integer_case(n, k, seed):
+def q4k_integer_case(n, k, seed, group=16, big_value=4161407, small=65535):
     """Q4_K blocks with d = 1, dmin = 0, every sub-block scale 1 and at most 16 nonzero
     nibbles per row; activations are integers whose every 16-element group has maximum
     magnitude 4161407 (the fixed-point range of the MFMA kernel, so its activation scale
@@ -134,9 +134,9 @@ def q4k_integer_case(n, k, seed):
     integer below 2^24: f32 FMA, integer MFMA and int64 arithmetic must agree exactly."""
     rng = np.random.default_rng(seed)
     q = np.zeros((n, k), np.int64)
-    x = rng.integers(-65535, 65536, size=k).astype(np.int64)
-    big = np.arange(0, k, 16) + int(rng.integers(0, 16))     # same slot in every group
-    x[big] = 4161407 * rng.choice([-1, 1], size=k // 16)
+    x = rng.integers(-small, small + 1, size=k).astype(np.int64)
+    big = np.arange(0, k, group) + int(rng.integers(0, group))     # same slot in every group
+    x[big] = big_value * rng.choice([-1, 1], size=k // group)
     free = np.setdiff1d(np.arange(k), big)
     for r in range(n):
         q[r, rng.choice(free, size=16, replace=False)] = rng.integers(1, 16, size=16)
@@ -162,6 +162,43 @@ def test_q4k_integer_dot_products_are_bit_exact(m):
     assert np.array_equal(ref, want.astype(np.float32))
     got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
     assert np.array_equal(got, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("m", [17, 64, 200])
+def test_q4k_gemm_integer_dot_products_are_bit_exact(m):
+    """The same construction for the MFMA GEMM (m > 16): its activation range is 4193279
+    per 256-element super-block; f16 products and f32 sums of integers below 2^24 are exact."""
+    n, k = 150, 1024
+    blocks, q, x = q4k_integer_case(n, k, 190 + m, group=256, big_value=4193279, small=4000)
+    xs = np.stack([np.roll(x, 256 * (i % 4)) * (1 if i % 3 else -1) for i in range(m)])
+    want = xs @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, xs.astype(np.float32))
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("m,k,n", [(17, 256, 64), (33, 512, 100), (128, 4096, 256), (130, 1024, 70),
+                                   (512, 4096, 1024), (96, 12288, 128)])
+def test_q4k_gemm_shapes(m, k, n):
+    """Prefill GEMM: ragged activation rows (not multiples of 32/128), ragged weight rows
+    (not multiples of 64), long rows."""
+    blocks = make_blocks(capi.Q4_K, n, k, 41 + n)
+    lhs = synth.normal(42 + m, (m, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True))
+
+
+def test_q4k_gemm_activation_scales_span_many_orders():
+    n, k, m = 96, 2048, 24
+    blocks = make_blocks(capi.Q4_K, n, k, 79)
+    rng = np.random.default_rng(6)
+    lhs = synth.normal(80, (m, k))
+    lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 256)).repeat(256).astype(np.float32)
+    lhs[1, :] = 0.0
+    lhs[1, 777] = -2.5
+    lhs[2, 512:1024] = 0.0
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True))
 
 
 def test_iq2xxs_fixture_matmul(golden_dir):
