@@ -206,32 +206,27 @@ int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
 // stream-ordered scratch allocation, then the MFMA GEMM.
 int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
                       hipStream_t s) {
-    constexpr int MI = 2;
-    constexpr size_t MT = 64 * MI;
-    static std::once_flag once;
-    static hipError_t attr_rc = hipSuccess;
-    std::call_once(once, [] {
-        attr_rc = hipFuncSetAttribute((const void *)jq::q4k_gemm_mfma<MI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (int)jq::q4k_gemm_lds_bytes<MI>());
-    });
-    if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
+    constexpr size_t MT = jq::QG_MT;
     const size_t m_pad = (m + MT - 1) / MT * MT, nb = k / 256;
     auto up = [](size_t v) { return (v + 255) / 256 * 256; };
-    const size_t plane_bytes = up(m_pad * k * 2 * sizeof(uint16_t)), min_bytes = up(m_pad * nb * 64),
-                 sc_bytes = up(m_pad * nb * sizeof(float));
+    const size_t plane_bytes = up(m_pad * k * 2 * sizeof(uint16_t)), min_bytes = up(m_pad * nb * 64);
     const size_t m_tiles = m_pad / MT, n_tiles = (n + jq::QG_NT - 1) / jq::QG_NT, total = m_tiles * n_tiles;
     if (total > 0x0FFFFFFFull) return fail("q4k gemm: %zu x %zu tiles exceed the grid limit", m_tiles, n_tiles);
     uint8_t *buf = nullptr;
-    HIP_TRY(hipMallocAsync((void **)&buf, plane_bytes + min_bytes + sc_bytes, s));
+    HIP_TRY(hipMallocAsync((void **)&buf, plane_bytes + min_bytes, s));
     jq::Q4kGemmActs a;
     a.planes = (_Float16 *)buf;
     a.mins = (_Float16 *)(buf + plane_bytes);
-    a.scale = (float *)(buf + plane_bytes + min_bytes);
     const size_t units = m_pad * nb;
     hipLaunchKernelGGL(jq::q4k_gemm_prep, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, X, (int)m, (int)m_pad, (int)k, a);
-    const unsigned grid = (unsigned)((total + 7) / 8 * 8);
-    hipLaunchKernelGGL((jq::q4k_gemm_mfma<MI>), dim3(grid), dim3(512), jq::q4k_gemm_lds_bytes<MI>(), s, W, row_bytes, a, Y,
-                       (int)m, (int)m_pad, (int)k, (int)n, (int)m_tiles, (int)total);
+    // 8 XCDs x the longest per-XCD work list (see the tile order at the top of the kernel)
+    size_t per_xcd;
+    if (m_tiles >= 8) per_xcd = (m_tiles + 7) / 8 * n_tiles;
+    else if (8 % m_tiles != 0) per_xcd = (total + 7) / 8;
+    else per_xcd = (n_tiles + 8 / m_tiles - 1) / (8 / m_tiles);
+    const unsigned grid = (unsigned)(8 * per_xcd);
+    hipLaunchKernelGGL(jq::q4k_gemm_mfma, dim3(grid), dim3(512), 0, s, W, row_bytes, a, Y, (int)m, (int)m_pad, (int)k, (int)n,
+                       (int)m_tiles, (int)total);
     hipError_t e = hipGetLastError();
     HIP_TRY(hipFreeAsync(buf, s));
     if (e != hipSuccess) return fail("q4k gemm launch: %s", hipGetErrorString(e));

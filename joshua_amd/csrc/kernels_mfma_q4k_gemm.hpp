@@ -26,6 +26,8 @@
 // by 64-k chunk and staged one chunk ahead; even and odd waves run their staging
 // and MFMA phases in opposite order so the two waves of a SIMD overlap them.
 #pragma once
+#include <type_traits>
+
 #include "kernels_mfma_q4k.hpp"
 
 namespace jq {
@@ -42,12 +44,10 @@ typedef uint32_t qg_u4 __attribute__((ext_vector_type(4)));
 //   planes: [m_pad/16][k/64][kstep 2][plane 2 (Xh, Xl)][lane 64][8 halves]; lane = m%16 + 16*((k%32)/8),
 //           the 8 k of a lane stored in the order 0,2,1,3,4,6,5,7 (the order the weight unpack produces)
 //   mins:   [m_pad/16][k/256][lane 64][8 halves]; lane = m%16 + 16*g, g = 0,1,2: the three f16 parts of
-//           XS_j / 4096 for j = 0..7, g = 3: zeros
-//   scale:  [m_pad][k/256]
+//           XS_j / 4096 for j = 0..7; g = 3: the f32 scale s of row m in the first four bytes
 struct Q4kGemmActs {
     _Float16 *planes;
     _Float16 *mins;
-    float *scale;
 };
 
 __device__ __forceinline__ uint32_t qg_pack_h2(int a, int b) {  // two small integers as f16
@@ -95,9 +95,13 @@ __global__ __launch_bounds__(256) void q4k_gemm_prep(const float *__restrict__ x
         const _Float16 p1 = (_Float16)r1;
         const _Float16 p2 = (_Float16)(r1 - (double)p1);
         _Float16 *o = a.mins + (((size_t)mt * nb + b) * 64 + (row & 15)) * 8 + j;
-        o[0] = p0, o[16 * 8] = p1, o[32 * 8] = p2, o[48 * 8] = (_Float16)0.0f;
+        o[0] = p0, o[16 * 8] = p1, o[32 * 8] = p2;
     }
-    if (lane == 0) a.scale[(size_t)row * nb + b] = live ? amax / QG_RANGE : 0.0f;
+    if (lane == 0) {  // lane 48 + m%16 of the block: the scale in its first dword, zeros behind it
+        uint32_t *o = (uint32_t *)(a.mins + (((size_t)mt * nb + b) * 64 + 48 + (row & 15)) * 8);
+        o[0] = __float_as_uint(live ? amax / QG_RANGE : 0.0f);
+        o[1] = o[2] = o[3] = 0;
+    }
 }
 
 // (sc * q) of the nibbles sitting in bits 0-3 and 16-19 of `two`, as two f16.
@@ -107,27 +111,70 @@ __device__ __forceinline__ uint32_t qg_scaled_h2(uint32_t two, uint32_t sc) {
     return __builtin_bit_cast(uint32_t, v);
 }
 
-template <int MI>  // 16-row activation tiles per wave
+// Asynchronous global -> LDS load: every active lane fetches `bytes` (4 or 16) from its own global
+// address, and the wave's data lands contiguously at lds_base + lane * bytes (lds_base wave-uniform).
+// Written as inline assembly so that the compiler neither tracks these loads nor inserts waits of
+// its own for them: the kernel below orders and awaits them by hand with s_waitcnt vmcnt(n).
+// M0 (the LDS base of such a load) is written here and used by nothing else in these kernels.
+__device__ __forceinline__ uint32_t qg_lds_offset(const void *p) {
+    return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void *)p);
+}
+__device__ __forceinline__ void qg_async_load16(const void *gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base)) : "memory");
+}
+__device__ __forceinline__ void qg_async_load4(const void *gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base)) : "memory");
+}
+
+// 16-row activation tiles per wave: 2 (the LDS budget below is sized for it)
+constexpr int QG_MI = 2;
+constexpr int QG_MT = 64 * QG_MI;        // activation rows per workgroup
+constexpr int QG_MT16 = 4 * QG_MI;       // 16-row activation tiles per workgroup = waves per workgroup
+constexpr int QG_A_U4 = 2 * 8 * 64;      // 16-byte slots of an unpacked A chunk: [kstep][ntile 8][lane]
+constexpr int QG_B_U4 = 2 * 2 * QG_MT16 * 64;  // of a B chunk: [kstep][plane][mtile][lane]
+
+// Every global read of the main loop is an asynchronous global->LDS load (no register in
+// between), ordered and awaited by hand: the vmcnt arithmetic in step() relies on each
+// wave issuing exactly the operations listed there, youngest last.
 __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__ W, size_t row_bytes, Q4kGemmActs acts,
                                                       float *__restrict__ Y, int m, int m_pad, int k, int n,
                                                       int m_tiles, int total_tiles) {
-    constexpr int MT = 64 * MI;          // activation rows per workgroup
-    constexpr int MT16 = 4 * MI;         // 16-row activation tiles per workgroup
-    constexpr int A_U4 = 2 * 8 * 64;     // uint4 per A buffer:  [kstep][ntile 8][lane]
-    constexpr int B_U4 = 2 * 2 * MT16 * 64;  // [kstep][plane][mtile][lane]
-    extern __shared__ uint4 qg_lds[];
-    uint4 *a_lds = qg_lds;                    // 2 buffers
-    uint4 *b_lds = qg_lds + 2 * A_U4;         // 2 buffers
-    uint4 *min_lds = b_lds + 2 * B_U4;        // [2 (super-block parity)][128 rows]: the eight mins as f16
-    float *d_lds = (float *)(min_lds + 2 * QG_NT);  // [2][128]
-    float *dmin_lds = d_lds + 2 * QG_NT;            // [2][128]
+    constexpr int MI = QG_MI, MT = QG_MT, MT16 = QG_MT16;
+    static_assert(MT16 == 8, "one activation tile of mins per wave");
+    // Rings of 64-k chunks.  The slots are separate arrays so that the compiler can tell a
+    // read of one slot from the asynchronous loads in flight into another.
+    __shared__ qg_u4 b_s0[QG_B_U4], b_s1[QG_B_U4], b_s2[QG_B_U4];   // activation planes, 3 x 32 KB
+    __shared__ uint32_t r_s0[1024], r_s1[1024], r_s2[1024];         // packed nibbles [row 128][8 dwords], 3 x 4 KB
+    __shared__ qg_u4 h_s0[QG_NT], h_s1[QG_NT], h_s2[QG_NT];          // block header of each row, per chunk slot
+    __shared__ qg_u4 x_s[QG_MT16 * 64];                              // mins operand + scales of the super-block
+    __shared__ qg_u4 a_lds[2 * QG_A_U4];                             // unpacked weights, by chunk parity
+    __shared__ qg_u4 min_lds[2 * QG_NT];   // [super-block parity][row]: the eight mins as f16
+    __shared__ float d_lds[2 * QG_NT], dmin_lds[2 * QG_NT];
 
-    // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; make the tiles
-    // an XCD works on consecutive, so the activation tiles of one weight tile share an L2.
-    const int per_xcd = (total_tiles + 7) >> 3;
-    const int logical = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    if (logical >= total_tiles) return;
-    const int mt = logical % m_tiles, nt = logical / m_tiles;
+    // XCD-aware order.  Consecutive workgroup ids go round-robin over the 8 XCDs, each with its own
+    // L2.  The activation planes are the heavy operand (4 bytes per element against 0.5 for the
+    // weights), so an XCD works on as few activation tiles as possible and keeps them in its L2,
+    // while a weight tile is fetched by the XCDs that share it.
+    const int xcd = (int)(blockIdx.x & 7), slot = (int)(blockIdx.x >> 3);
+    int mt, nt;
+    if (m_tiles >= 8 || (8 % m_tiles) != 0) {
+        // activation tiles xcd, xcd + 8, ... (or plain round-robin when the counts do not divide)
+        const int per_xcd = (total_tiles + 7) >> 3;
+        const int logical = m_tiles >= 8 ? slot : xcd * per_xcd + slot;
+        if (m_tiles >= 8) {
+            const int n_tiles = total_tiles / m_tiles;
+            mt = xcd + 8 * (logical / n_tiles), nt = logical % n_tiles;
+            if (mt >= m_tiles) return;
+        } else {
+            if (logical >= total_tiles) return;
+            mt = logical % m_tiles, nt = logical / m_tiles;
+        }
+    } else {
+        const int g = 8 / m_tiles, n_tiles = total_tiles / m_tiles;   // g XCDs share one activation tile
+        mt = xcd % m_tiles;
+        nt = xcd / m_tiles + g * slot;
+        if (nt >= n_tiles) return;
+    }
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wn = wave & 1, wm = wave >> 1;
@@ -136,58 +183,88 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
     const int m0 = mt * MT + wm * 16 * MI;       // first activation row of this wave
     const bool wave_live = m0 < m;
 
-    // staging roles
-    const int ar = tid >> 2, aq = tid & 3;        // weight row of the tile, 8-byte piece of the chunk's 32 nibble bytes
-    const uint8_t *wrow = W + (size_t)min(nt * QG_NT + ar, n - 1) * row_bytes;
-    const qg_u4 *bsrc = (const qg_u4 *)acts.planes + (size_t)(mt * MT16) * nch * 256;  // + (mtile*nch + chunk)*256 + idx
-
-    uint2 a_reg;
-    uint4 h_reg;
-    qg_u4 b_reg[2 * MI];
-
-    auto load_chunk = [&](int c) __attribute__((always_inline)) {
-        const uint8_t *blk = wrow + (size_t)(c >> 2) * 144;
-        h_reg = *(const uint4 *)blk;
-        a_reg = *(const uint2 *)(blk + 16 + 32 * (c & 3) + 8 * aq);
+    const int ar = tid >> 2, aq = tid & 3;        // unpack role: weight row of the tile, 8-byte piece of its 32 nibble bytes
+    const qg_u4 *bsrc = (const qg_u4 *)acts.planes + (size_t)(mt * MT16) * nch * 256;
+    // asynchronous-load roles: nibble rows 16 wave + 8 j + lane/8 (dword lane%8), header row 16 wave + lane/4
+    const uint8_t *nib_src[2];
 #pragma unroll
-        for (int i = 0; i < 2 * MI; i++) {
-            const int idx = tid + 512 * i;  // of MT16 * 256 uint4
-            b_reg[i] = bsrc[((size_t)(idx >> 8) * nch + c) * 256 + (idx & 255)];
+    for (int j = 0; j < 2; j++)
+        nib_src[j] = W + (size_t)min(nt * QG_NT + 16 * wave + 8 * j + (lane >> 3), n - 1) * row_bytes + 16 + 4 * (lane & 7);
+    const uint8_t *hdr_src = W + (size_t)min(nt * QG_NT + 16 * wave + (lane >> 2), n - 1) * row_bytes + 4 * (lane & 3);
+    const qg_u4 *xs_src = (const qg_u4 *)acts.mins + (size_t)(mt * MT16 + wave) * nb * 64 + lane;
+
+    auto b_slot = [&](auto S) __attribute__((always_inline)) -> qg_u4 * {
+        if constexpr (decltype(S)::value == 0) return b_s0;
+        else if constexpr (decltype(S)::value == 1) return b_s1;
+        else return b_s2;
+    };
+    auto r_slot = [&](auto S) __attribute__((always_inline)) -> uint32_t * {
+        if constexpr (decltype(S)::value == 0) return r_s0;
+        else if constexpr (decltype(S)::value == 1) return r_s1;
+        else return r_s2;
+    };
+
+    // 2 operations: packed nibbles of chunk c
+    auto dma_nibbles = [&](auto S, int c) __attribute__((always_inline)) {
+        uint32_t *rr = r_slot(S);
+        const size_t off = (size_t)(c >> 2) * 144 + 32 * (c & 3);
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            qg_async_load4(nib_src[j] + off, qg_lds_offset(rr + (wave * 2 + j) * 64));
+    };
+    auto h_slot = [&](auto S) __attribute__((always_inline)) -> qg_u4 * {
+        if constexpr (decltype(S)::value == 0) return h_s0;
+        else if constexpr (decltype(S)::value == 1) return h_s1;
+        else return h_s2;
+    };
+    // 1 operation: the 16-byte block headers of chunk c's super-block (fetched with every chunk so
+    // that the slot read by unpack_a is known at compile time)
+    auto dma_header = [&](auto S, int c) __attribute__((always_inline)) {
+        qg_async_load4(hdr_src + (size_t)(c >> 2) * 144, qg_lds_offset((uint32_t *)h_slot(S) + wave * 64));
+    };
+    auto dma_block_acts = [&](int b) __attribute__((always_inline)) {
+        qg_async_load16(xs_src + (size_t)b * 64, qg_lds_offset(x_s + wave * 64));
+    };
+    // 4 operations: activation planes of chunk c, four 1 KB blocks per wave
+    auto dma_b = [&](auto S, int c) __attribute__((always_inline)) {
+        qg_u4 *bb = b_slot(S);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int blk = wave * 4 + i;                       // LDS block = ksp * MT16 + mtile
+            const int ksp = blk / MT16, mtile = blk % MT16;
+            const qg_u4 *src = bsrc + ((size_t)mtile * nch + c) * 256 + ksp * 64 + lane;
+            qg_async_load16(src, qg_lds_offset(bb + blk * 64));
         }
     };
-    auto store_chunk = [&](int c) __attribute__((always_inline)) {
-        const int buf = c & 1, cc = c & 3;
+    // packed nibbles of chunk c (slot S) -> scaled f16 in the A buffer of its parity
+    auto unpack_a = [&](auto S, int c) __attribute__((always_inline)) {
+        const int cc = c & 3, par = (c >> 2) & 1;
+        const qg_u4 h = h_slot(S)[ar];
         uint32_t sc_lo, mn_lo, sc_hi, mn_hi;
-        q4k_scale_min(h_reg.y, h_reg.z, h_reg.w, 2 * cc, sc_lo, mn_lo);
-        q4k_scale_min(h_reg.y, h_reg.z, h_reg.w, 2 * cc + 1, sc_hi, mn_hi);
-        const uint32_t w0 = a_reg.x, w1 = a_reg.y;
+        q4k_scale_min(h.y, h.z, h.w, 2 * cc, sc_lo, mn_lo);
+        q4k_scale_min(h.y, h.z, h.w, 2 * cc + 1, sc_hi, mn_hi);
+        const uint2 raw = *(const uint2 *)(r_slot(S) + ar * 8 + aq * 2);
+        const uint32_t w0 = raw.x, w1 = raw.y;
         // operand order within the 8 k of a lane: 0,2,1,3,4,6,5,7
-        const uint4 lo = uint4{qg_scaled_h2(w0 & 0x000F000Fu, sc_lo), qg_scaled_h2((w0 >> 8) & 0x000F000Fu, sc_lo),
+        const qg_u4 lo = qg_u4{qg_scaled_h2(w0 & 0x000F000Fu, sc_lo), qg_scaled_h2((w0 >> 8) & 0x000F000Fu, sc_lo),
                                qg_scaled_h2(w1 & 0x000F000Fu, sc_lo), qg_scaled_h2((w1 >> 8) & 0x000F000Fu, sc_lo)};
-        const uint4 hi = uint4{qg_scaled_h2((w0 >> 4) & 0x000F000Fu, sc_hi), qg_scaled_h2((w0 >> 12) & 0x000F000Fu, sc_hi),
+        const qg_u4 hi = qg_u4{qg_scaled_h2((w0 >> 4) & 0x000F000Fu, sc_hi), qg_scaled_h2((w0 >> 12) & 0x000F000Fu, sc_hi),
                                qg_scaled_h2((w1 >> 4) & 0x000F000Fu, sc_hi), qg_scaled_h2((w1 >> 12) & 0x000F000Fu, sc_hi)};
-        uint4 *ab = a_lds + buf * A_U4;
+        qg_u4 *ab = a_lds + (c & 1) * QG_A_U4;
         const int tile = ar >> 4, ol = (ar & 15) + 16 * aq;
         ab[(0 * 8 + tile) * 64 + ol] = lo;   // sub-block 2cc   -> k step 0
         ab[(1 * 8 + tile) * 64 + ol] = hi;   // sub-block 2cc+1 -> k step 1
         if (cc == 0 && aq == 0) {
-            const int par = (c >> 2) & 1;
-            d_lds[par * QG_NT + ar] = f16_bits(h_reg.x);
-            dmin_lds[par * QG_NT + ar] = f16_bits(h_reg.x >> 16);
+            d_lds[par * QG_NT + ar] = f16_bits(h.x);
+            dmin_lds[par * QG_NT + ar] = f16_bits(h.x >> 16);
             uint32_t mm[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 uint32_t s_;
-                q4k_scale_min(h_reg.y, h_reg.z, h_reg.w, j, s_, mm[j]);
+                q4k_scale_min(h.y, h.z, h.w, j, s_, mm[j]);
             }
-            min_lds[par * QG_NT + ar] = uint4{qg_pack_h2((int)mm[0], (int)mm[1]), qg_pack_h2((int)mm[2], (int)mm[3]),
+            min_lds[par * QG_NT + ar] = qg_u4{qg_pack_h2((int)mm[0], (int)mm[1]), qg_pack_h2((int)mm[2], (int)mm[3]),
                                               qg_pack_h2((int)mm[4], (int)mm[5]), qg_pack_h2((int)mm[6], (int)mm[7])};
-        }
-        uint4 *bb = b_lds + buf * B_U4;
-#pragma unroll
-        for (int i = 0; i < 2 * MI; i++) {
-            const int idx = tid + 512 * i, mtile = idx >> 8, rest = idx & 255;  // rest = (kstep*2 + plane)*64 + lane
-            *(qg_u4 *)(bb + ((rest >> 6) * MT16 + mtile) * 64 + (rest & 63)) = b_reg[i];
         }
     };
 
@@ -202,9 +279,9 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
             for (int j = 0; j < 4; j++) acc[ni][mi][j] = 0.0f;
         }
 
-    auto compute_chunk = [&](int c) __attribute__((always_inline)) {
+    auto compute = [&](auto S, int c) __attribute__((always_inline)) {
         if (!wave_live) return;
-        const uint4 *ab = a_lds + (c & 1) * A_U4, *bb = b_lds + (c & 1) * B_U4;
+        const qg_u4 *ab = a_lds + (c & 1) * QG_A_U4, *bb = b_slot(S);
 #pragma unroll
         for (int ks = 0; ks < 2; ks++) {
             qg_h8 bh[MI], bl[MI];
@@ -225,61 +302,82 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
         }
     };
 
-    float s_reg[MI];
-    uint4 xs_reg[MI];
     auto close_block = [&](int b) __attribute__((always_inline)) {
         if (!wave_live) return;
         const int par = b & 1;
 #pragma unroll
         for (int mi = 0; mi < MI; mi++) {
-            const qg_h8 xm = __builtin_bit_cast(qg_h8, xs_reg[mi]);
-            const float s = s_reg[mi];
+            const qg_u4 *xt = x_s + (wm * MI + mi) * 64;
+            const qg_u4 xraw = kg < 3 ? xt[lane] : qg_u4{0, 0, 0, 0};
+            const qg_h8 xm = __builtin_bit_cast(qg_h8, xraw);
+            const float s = __uint_as_float(xt[48 + col].x);
 #pragma unroll
             for (int ni = 0; ni < 4; ni++) {
                 const int r0 = par * QG_NT + wn * 64 + 16 * ni;
-                const uint4 mraw = kg < 3 ? min_lds[r0 + col] : uint4{0, 0, 0, 0};
+                const qg_u4 mraw = kg < 3 ? min_lds[r0 + col] : qg_u4{0, 0, 0, 0};
                 const qg_f4 MM = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(qg_h8, mraw), xm,
                                                                         qg_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-                const float4 dv = *(const float4 *)(d_lds + r0 + 4 * kg);
-                const float4 mv = *(const float4 *)(dmin_lds + r0 + 4 * kg);
-                const float dj[4] = {dv.x, dv.y, dv.z, dv.w}, mj[4] = {mv.x, mv.y, mv.z, mv.w};
+                const qg_f4 dv = *(const qg_f4 *)(d_lds + r0 + 4 * kg);
+                const qg_f4 mv = *(const qg_f4 *)(dmin_lds + r0 + 4 * kg);
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const float f = fmaf(Ph[ni][mi][j], 2048.0f, Pl[ni][mi][j]);
-                    const float t = fmaf(-4096.0f * mj[j], MM[j], dj[j] * f);
+                    const float t = fmaf(-4096.0f * mv[j], MM[j], dv[j] * f);
                     acc[ni][mi][j] = fmaf(s, t, acc[ni][mi][j]);
                 }
                 Ph[ni][mi] = Pl[ni][mi] = qg_f4{0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
     };
-    auto load_block_acts = [&](int b) __attribute__((always_inline)) {
-        if (!wave_live) return;
-#pragma unroll
-        for (int mi = 0; mi < MI; mi++) {
-            s_reg[mi] = acts.scale[(size_t)(m0 + 16 * mi + col) * nb + b];
-            xs_reg[mi] = ((const uint4 *)acts.mins)[((size_t)((m0 >> 4) + mi) * nb + b) * 64 + lane];
-        }
-    };
 
-    load_chunk(0);
-    store_chunk(0);
-    if (nch > 1) load_chunk(1);
-    __syncthreads();
-    const bool stage_first = (wave & 4) == 0;  // waves 0-3 and 4-7 share SIMDs pairwise
-    for (int c = 0; c < nch; c++) {
-        if ((c & 3) == 0) load_block_acts(c >> 2);
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    const bool stage_first = (wave & 4) == 0;  // waves w and w + 4 share a SIMD
+
+    // One pipeline step: chunk c, activation planes in slot S.
+    //   on entry, in flight and oldest first: [group of step c-2], [group of step c-1]
+    //   group of step c = nibbles(c+3) x2, header(c+3), mins(c/4) if c%4 == 0, planes(c+2) x4;
+    //                     at least 7 operations while c + 3 < nch
+    //   needed now: planes(c), nibbles and header (c+1), mins issued at step c-2 or earlier
+    //   => at most the 7 youngest operations (all from step c-1) may still be in flight.
+    auto step = [&](auto S, auto S1, auto S2, int c) __attribute__((always_inline)) {
+        if (c + 4 < nch) asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (c + 3 < nch) {
+            dma_nibbles(S, c + 3);                              // slot S held chunk c, unpacked during step c-1
+            dma_header(S, c + 3);
+        }
+        if (c > 0 && (c & 3) == 0) dma_block_acts(c >> 2);      // x_s last read by close_block at step c-1; needed at c+3
+        if (c + 2 < nch) dma_b(S2, c + 2);                      // slot S2 last read by compute(c-1)
+        asm volatile("" ::: "memory");
         if (stage_first) {
-            if (c + 1 < nch) store_chunk(c + 1);
-            if (c + 2 < nch) load_chunk(c + 2);
-            compute_chunk(c);
+            if (c + 1 < nch) unpack_a(S1, c + 1);               // A buffer (c+1)&1 last read by compute(c-1)
+            compute(S, c);
         } else {
-            compute_chunk(c);
-            if (c + 1 < nch) store_chunk(c + 1);
-            if (c + 2 < nch) load_chunk(c + 2);
+            compute(S, c);
+            if (c + 1 < nch) unpack_a(S1, c + 1);
         }
         if ((c & 3) == 3) close_block(c >> 2);
-        __syncthreads();
+    };
+
+    // prologue: chunks 0..2 of nibbles, headers and mins of super-block 0, planes of chunks 0 and 1
+    dma_block_acts(0);
+    dma_nibbles(I0{}, 0), dma_header(I0{}, 0);
+    if (nch > 1) dma_nibbles(I1{}, 1), dma_header(I1{}, 1);
+    if (nch > 2) dma_nibbles(I2{}, 2), dma_header(I2{}, 2);
+    dma_b(I0{}, 0);
+    if (nch > 1) dma_b(I1{}, 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    unpack_a(I0{}, 0);
+    for (int c = 0; c < nch; c += 3) {
+        step(I0{}, I1{}, I2{}, c);
+        if (c + 1 < nch) step(I1{}, I2{}, I0{}, c + 1);
+        if (c + 2 < nch) step(I2{}, I0{}, I1{}, c + 2);
     }
 
     if (!wave_live) return;
@@ -300,11 +398,6 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
             }
         }
     }
-}
-
-template <int MI>
-constexpr size_t q4k_gemm_lds_bytes() {
-    return (size_t)(2 * (2 * 8 * 64) + 2 * (2 * 2 * 4 * MI * 64) + 2 * QG_NT) * 16 + 4 * QG_NT * sizeof(float);
 }
 
 }  // namespace jq
