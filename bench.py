@@ -59,6 +59,116 @@ def cpu_baseline(blocks: np.ndarray, lhs: np.ndarray, budget_s: float) -> dict:
                       f"{threads} threads, 3 warm-up runs", "ms_per_step": round(med * 1e3, 4)}
 
 
+BLOCK = {8: (32, 34), 10: (256, 84), 12: (256, 144), 14: (256, 210), 16: (256, 66), 39: (32, 17)}
+F16_MFMA_PEAK_TFLOPS = 2500.0
+
+
+def _time_calls(torch, stream, fn, count: int) -> float:
+    """ms per call: `count` calls of fn(i) between two events on the launch stream."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record(stream)
+    for i in range(count):
+        fn(i)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / count
+
+
+def matmul_workload(torch, capi, synth, qtype: int, n: int, k: int, m: int, seed: int, steps: int, copies: int) -> dict:
+    """One quantized matmul shape, weights rotated over `copies` distinct HBM copies."""
+    be, bb = BLOCK[qtype]
+    blocks = synth.normal_quantized(qtype, seed, n * k, 0.02)
+    lhs = synth.normal(seed + 100, (m, k))
+    dev = torch.device("cuda:0")
+    x = torch.from_numpy(lhs).to(dev)
+    y = torch.zeros((m, n), device=dev)
+    base = capi.Weight.upload(qtype, blocks, n, k)
+    ws = [base] + [capi.Weight.upload_device(qtype, base.device_ptr, base.nbytes, n, k) for _ in range(copies - 1)]
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+
+    def call(i):
+        ws[i % len(ws)].matmul_t_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), sh)
+
+    _time_calls(torch, stream, call, max(steps // 10, 3))
+    ms = _time_calls(torch, stream, call, steps)
+    abytes = n * (k // be) * bb + 4 * m * k + 4 * m * n
+    res = {"us": round(ms * 1e3, 2), "algorithmic_bytes": abytes, "gbs": round(abytes / ms / 1e6, 1),
+           "hbm_frac": round(abytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    if m > 16:
+        tflops = 2.0 * m * n * k / ms / 1e9
+        res["useful_tflops"] = round(tflops, 1)
+        res["mfma_frac_of_f16_peak"] = round(tflops / F16_MFMA_PEAK_TFLOPS, 4)
+    return res
+
+
+def moe_workload(torch, capi, synth, qtype: int, h: int, inter: int, n_expert: int, k_used: int, batch: int, seed: int,
+                 steps: int, shared: bool, gating: int) -> dict:
+    """One MoE layer call.  Every expert holds the same block bytes (one expert is drawn and repeated on the
+    device: distinct HBM addresses, identical contents); tokens rotate so the routed experts change."""
+    be, bb = BLOCK[qtype]
+    dev = torch.device("cuda:0")
+
+    def stacked(seed_, rows, cols, count):
+        one = torch.from_numpy(synth.normal_quantized(qtype, seed_, rows * cols, 0.02)).to(dev)
+        rep = one.repeat(count)
+        w = capi.Weight.upload_device(qtype, rep.data_ptr(), rep.numel(), count * rows, cols)
+        del rep, one
+        return w
+
+    gate, up, down = stacked(seed, inter, h, n_expert), stacked(seed + 1, inter, h, n_expert), stacked(seed + 2, h, inter, n_expert)
+    sh_w = None
+    if shared:
+        sh_w = (stacked(seed + 3, inter, h, 1), stacked(seed + 4, inter, h, 1), stacked(seed + 5, h, inter, 1))
+    router = synth.normal(seed + 6, (n_expert, h), 0.02)
+    cfg = capi.MoeConfig(n_expert, k_used, h, inter, gating, 1, 0.0, 1, 1)
+    moe = capi.Moe(cfg, router, gate, up, down, shared=sh_w)
+    n_sets = 16 if batch == 1 else 4
+    xs_host = [synth.normal(seed + 10 + i, (batch, h)) for i in range(n_sets)]
+    xs = [torch.from_numpy(a).to(dev) for a in xs_host]
+    y = torch.zeros((batch, h), device=dev)
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+    per_expert = 3 * inter * (h // be) * bb if qtype != 39 else 3 * inter * h // 32 * 17
+    distinct = [len(np.unique(moe.route(a)[0])) for a in xs_host]
+    abytes = float(np.mean(distinct)) * per_expert + 4 * n_expert * h + (per_expert if shared else 0) + 8 * batch * h
+
+    def call(i):
+        moe.forward_dev(batch, xs[i % n_sets].data_ptr(), y.data_ptr(), sh)
+
+    _time_calls(torch, stream, call, max(steps // 10, 3))
+    ms = _time_calls(torch, stream, call, steps)
+    res = {"us": round(ms * 1e3, 2), "distinct_experts_mean": round(float(np.mean(distinct)), 1),
+           "algorithmic_bytes": int(abytes), "gbs": round(abytes / ms / 1e6, 1),
+           "hbm_frac": round(abytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    moe.close()
+    return res
+
+
+def extra_workloads(steps: int) -> dict:
+    """The other configurations of the path, one figure each (cold HBM unless noted)."""
+    import torch
+    from joshua_amd import capi, synth
+    out = {}
+    out["q8_0_gemv_4096x4096_m1"] = matmul_workload(torch, capi, synth, 8, 4096, 4096, 1, 101, steps, 24)
+    out["q4_k_14336x4096_m16"] = matmul_workload(torch, capi, synth, 12, N, K, 16, 102, steps, 24)
+    out["q4_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 12, N, K, 512, 102, max(steps // 10, 10), 4)
+    out["q6_k_gemv_4096x12288_m1"] = matmul_workload(torch, capi, synth, 14, 4096, 12288, 1, 106, steps, 12)
+    torch.cuda.empty_cache()
+    out["moe_qwen3_30b_a3b_q4_k_b1"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 1, 104, steps, False, 0)
+    out["moe_qwen3_30b_a3b_q4_k_b64"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 64, 104, max(steps // 10, 10),
+                                                     False, 0)
+    torch.cuda.empty_cache()
+    out["moe_deepseek_v3_iq2_xxs_b1"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 1, 105, max(steps // 4, 10),
+                                                     True, 1)
+    torch.cuda.empty_cache()
+    out["moe_deepseek_v3_mxfp4_b1"] = moe_workload(torch, capi, synth, 39, 7168, 2048, 256, 8, 1, 105, max(steps // 4, 10),
+                                                   True, 1)
+    torch.cuda.empty_cache()
+    return out
+
+
 QWEN3_8B = dict(n_layer=36, hidden=4096, n_head=32, n_kv_head=8, head_dim=128, ffn=12288, vocab=151936, n_ctx=768,
                 rms_eps=1e-6, rope_theta=1e6)
 
@@ -145,6 +255,7 @@ def main() -> int:
     ap.add_argument("--m", type=int, default=1, help="activation rows (1 = decode GEMV)")
     ap.add_argument("--copies", type=int, default=24, help="distinct weight copies rotated through (cold HBM)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline (0 = skip)")
+    ap.add_argument("--extras", type=int, default=1, help="1: also time the other configurations of the path")
     ap.add_argument("--decode", type=int, default=1, help="1: also run the Qwen3-8B-shaped end-to-end decode leg")
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -246,9 +357,11 @@ def main() -> int:
     }
     if args.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(blocks, lhs, args.cpu_seconds)
+    del weights, base
+    torch.cuda.empty_cache()
+    if args.extras:
+        out["workloads"] = extra_workloads(min(steps, 200))
     if args.decode:
-        del weights, base
-        torch.cuda.empty_cache()
         out["decode"] = decode_leg(args.prompt, args.new_tokens, args.cpu_seconds, bool(args.share_layers))
         parity_ok = parity_ok and out["decode"].get("parity_ok", True)
     print(json.dumps(out))

@@ -116,12 +116,28 @@ template <class Q>
 void launch_rows(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
                  hipStream_t s) {
     dim3 grid((unsigned)((n + jq::ROWS_PER_WG - 1) / jq::ROWS_PER_WG)), block(64 * jq::ROWS_PER_WG);
-    if (m == 1)
-        hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 1>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
-    else if (m == 2)
-        hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 2>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
-    else
-        hipLaunchKernelGGL((jq::matmul_rows_valu<Q, 4>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
+    // rows staged through LDS when their starts are 16- or 4-byte aligned and four of them fit in 64 KB
+    const size_t stride = (row_bytes + 15) / 16 * 16;
+    const bool fits = stride * jq::ROWS_PER_WG <= 64 * 1024 && !getenv("JQ_NO_STAGED_ROWS");
+    const int gran = !fits ? 0 : (row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0) ? 16
+                                : (row_bytes % 4 == 0 && ((uintptr_t)W & 3) == 0)  ? 4 : 0;
+    const size_t lds = stride * jq::ROWS_PER_WG;
+#define JQ_LAUNCH_ROWS(MT)                                                                                              \
+    do {                                                                                                                 \
+        if (gran == 16)                                                                                                  \
+            hipLaunchKernelGGL((jq::matmul_rows_staged<Q, MT, 16>), grid, block, lds, s, W, row_bytes, X, Y, (int)m,     \
+                               (int)k, (int)n, (int)stride);                                                             \
+        else if (gran == 4)                                                                                              \
+            hipLaunchKernelGGL((jq::matmul_rows_staged<Q, MT, 4>), grid, block, lds, s, W, row_bytes, X, Y, (int)m,      \
+                               (int)k, (int)n, (int)stride);                                                             \
+        else                                                                                                             \
+            hipLaunchKernelGGL((jq::matmul_rows_valu<Q, MT>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k,     \
+                               (int)n);                                                                                  \
+    } while (0)
+    if (m == 1) JQ_LAUNCH_ROWS(1);
+    else if (m == 2) JQ_LAUNCH_ROWS(2);
+    else JQ_LAUNCH_ROWS(4);
+#undef JQ_LAUNCH_ROWS
 }
 
 // Q4_K, m <= 16: the MFMA decode kernel, up to four activation rows per launch.

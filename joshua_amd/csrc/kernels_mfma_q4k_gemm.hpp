@@ -22,9 +22,9 @@
 // (activation rows); a wave owns 64 x 16*MI outputs.  Weight nibbles are unpacked,
 // multiplied by their sub-block scale and converted while being staged into LDS in
 // MFMA operand order; the activation planes come prepared in operand order from
-// q4k_gemm_prep and are copied global -> registers -> LDS.  LDS is double buffered
-// by 64-k chunk and staged one chunk ahead; even and odd waves run their staging
-// and MFMA phases in opposite order so the two waves of a SIMD overlap them.
+// q4k_gemm_prep.  Everything the main loop reads from global memory travels as
+// asynchronous global -> LDS loads through rings of three 64-k chunks, two chunks
+// ahead of the MFMAs; the packed nibbles are then unpacked LDS -> LDS.
 #pragma once
 #include <type_traits>
 
@@ -333,7 +333,6 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
-    const bool stage_first = (wave & 4) == 0;  // waves w and w + 4 share a SIMD
 
     // One pipeline step: chunk c, activation planes in slot S.
     //   on entry, in flight and oldest first: [group of step c-2], [group of step c-1]
@@ -353,13 +352,8 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
         if (c > 0 && (c & 3) == 0) dma_block_acts(c >> 2);      // x_s last read by close_block at step c-1; needed at c+3
         if (c + 2 < nch) dma_b(S2, c + 2);                      // slot S2 last read by compute(c-1)
         asm volatile("" ::: "memory");
-        if (stage_first) {
-            if (c + 1 < nch) unpack_a(S1, c + 1);               // A buffer (c+1)&1 last read by compute(c-1)
-            compute(S, c);
-        } else {
-            compute(S, c);
-            if (c + 1 < nch) unpack_a(S1, c + 1);
-        }
+        compute(S, c);
+        if (c + 1 < nch) unpack_a(S1, c + 1);                   // A buffer (c+1)&1 last read by compute(c-1)
         if ((c & 3) == 3) close_block(c >> 2);
     };
 

@@ -67,6 +67,86 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void matmul_rows_valu(const uint8
     }
 }
 
+// Asynchronous global -> LDS load of `bytes` (4 or 16) per active lane; the wave's data lands
+// contiguously at lds_base + lane * bytes (lds_base wave-uniform, carried in M0, which nothing else
+// in these kernels uses).  Inline assembly: the caller awaits the loads itself with s_waitcnt vmcnt.
+__device__ __forceinline__ uint32_t lds_offset_of(const void *p) {
+    return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void *)p);
+}
+__device__ __forceinline__ void async_load16(const void *gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory");
+}
+__device__ __forceinline__ void async_load4(const void *gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory");
+}
+
+// The same arithmetic as matmul_rows_valu with the weight row staged through LDS: each wave first
+// pulls its whole packed row into LDS with fully coalesced asynchronous loads of G bytes per lane
+// (the whole row in flight at once, whatever the block size), then decodes blocks out of LDS.  A
+// block-strided global read (34-, 66-, 210-byte blocks) touches every cache line many times; this
+// touches each once.  Needs row starts and row_bytes that are multiples of G; LDS = 4 rows.
+template <class Q, int MT, int G>
+__global__ __launch_bounds__(64 * ROWS_PER_WG) void matmul_rows_staged(const uint8_t *__restrict__ W, size_t row_bytes,
+                                                                        const float *__restrict__ X,
+                                                                        float *__restrict__ Y, int m, int k, int n,
+                                                                        int lds_stride) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_rows[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = blockIdx.x * ROWS_PER_WG + wave;
+    if (row >= n) return;  // wave-uniform; the kernel has no barrier
+    uint8_t *rp = staged_rows + (size_t)wave * lds_stride;
+    {
+        const uint8_t *src = W + (size_t)row * row_bytes;
+        const int pieces = (int)(row_bytes / G);
+        for (int p0 = 0; p0 < pieces; p0 += 64) {
+            if (p0 + lane < pieces) {
+                if (G == 16) async_load16(src + (size_t)(p0 + lane) * 16, lds_offset_of(rp + (size_t)p0 * 16));
+                else async_load4(src + (size_t)(p0 + lane) * 4, lds_offset_of(rp + (size_t)p0 * 4));
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    constexpr int UE = Q::SEGS * Q::SEGLEN;
+    for (int m0 = 0; m0 < m; m0 += MT) {
+        float acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        for (int u = lane; u < units; u += 64) {
+            const int b = u / Q::UNITS, ub = u % Q::UNITS;
+            float w[UE];
+            Q::decode(rp + (size_t)b * Q::BLOCK_BYTES, ub, w);
+            const int xoff = b * Q::BLOCK_ELEMS + Q::elem_base(ub);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                if (m0 + i < m) {
+                    const float *xp = X + (size_t)(m0 + i) * k + xoff;
+#pragma unroll
+                    for (int s = 0; s < Q::SEGS; s++) {
+#pragma unroll
+                        for (int e = 0; e < Q::SEGLEN; e += 4) {
+                            float4 xv = ld<float4>((const uint8_t *)(xp + s * Q::SEG_STRIDE + e));
+                            acc[i] = fmaf(xv.x, w[s * Q::SEGLEN + e + 0], acc[i]);
+                            acc[i] = fmaf(xv.y, w[s * Q::SEGLEN + e + 1], acc[i]);
+                            acc[i] = fmaf(xv.z, w[s * Q::SEGLEN + e + 2], acc[i]);
+                            acc[i] = fmaf(xv.w, w[s * Q::SEGLEN + e + 3], acc[i]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < m) Y[(size_t)(m0 + i) * n + row] = s;
+        }
+    }
+}
+
 // Canonical decode ("to_float"): differs from the in-dot decode only for the
 // formats whose to_float uses two rounded operations instead of one fused
 // multiply-subtract (Q2_K, Q4_K; reference: src/kquant_dot.rs:258-260).
