@@ -28,6 +28,11 @@ if ROOT not in sys.path:
 
 N, K = 14336, 4096
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs
+# of this benchmark, each scaled by what the same counter reads for joshua_amd/calib/copy_kernel (a plain
+# copy of 33 030 144 bytes): FETCH_SIZE 16253.0 x 1.9987 KiB + WRITE_SIZE 56.0 x 1.0 KiB.  Only quoted for
+# the configuration it was measured on (M = 1).
+MEASURED_TRAFFIC_BYTES_M1 = 33_322_000
 SEED_W, SEED_X = 102, 202
 
 
@@ -347,7 +352,7 @@ def main() -> int:
                                f"weights N(0,0.02) quantized to Q4_K, {len(weights)} weight copies rotated (cold HBM)",
                    "launch": mode},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_M1 if m == 1 else None,
                      "algorithmic_bytes_per_launch": abytes, "kernel_us": round(ms_per_step * 1e3, 3)},
         "pct_of_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "cache_resident": {"value": round(abytes / (ms_res * 1e-3) / 1e9, 2), "unit": "GB/s",

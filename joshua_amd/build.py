@@ -32,9 +32,23 @@ def build_hip(verbose: bool = False) -> str:
     return HIP_LIB
 
 
+CALIB_SRC = os.path.join(HERE, "calib", "copy_kernel.hip")
+CALIB_BIN = os.path.join(HERE, "calib", "copy_kernel")
+
+
+def build_calibration() -> str:
+    """The copy kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
+    res = subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-o", CALIB_BIN, CALIB_SRC], capture_output=True,
+                         text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed:\n{res.stderr}")
+    return CALIB_BIN
+
+
 def build_all(verbose: bool = False) -> None:
     from . import synth
     build_hip(verbose)
+    build_calibration()
     synth.build()
 
 

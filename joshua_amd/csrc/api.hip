@@ -481,6 +481,7 @@ struct jq_moe {
     const jq_weight *gate, *up, *down, *sgate, *sup, *sdown;
     float *router_w = nullptr, *router_bias = nullptr;
     const uint8_t **pgate = nullptr, **pup = nullptr, **pdown = nullptr;  // device tables of expert bases
+    bool fold_shared = false;  // the shared expert rides along as table entry n_expert of the grouped kernels
     // scratch, grown to the largest token count seen
     size_t cap_tokens = 0;
     float *logits = nullptr, *wts = nullptr, *G = nullptr, *U = nullptr, *out = nullptr;
@@ -507,17 +508,18 @@ int moe_reserve(jq_moe *m, size_t T) {
     if (T <= m->cap_tokens) return 0;
     moe_free_scratch(m);
     const jq_moe_config &c = m->cfg;
-    size_t P = T * c.n_expert_used, groups = std::max<size_t>(P, c.n_expert) + 1;
+    // rows of the pair buffers: the routed pairs, then one per token for a folded shared expert
+    size_t P = T * c.n_expert_used, PR = P + T, groups = std::max<size_t>(PR, c.n_expert + 1) + 1;
     HIP_TRY(hipMalloc((void **)&m->logits, T * c.n_expert * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->wts, P * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->ids, P * sizeof(uint32_t)));
-    HIP_TRY(hipMalloc((void **)&m->G, P * c.inter * sizeof(float)));
-    HIP_TRY(hipMalloc((void **)&m->U, P * c.inter * sizeof(float)));
-    HIP_TRY(hipMalloc((void **)&m->out, P * c.hidden * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->G, PR * c.inter * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->U, PR * c.inter * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->out, PR * c.hidden * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->gexp, groups * sizeof(int)));
     HIP_TRY(hipMalloc((void **)&m->offsets, (groups + 1) * sizeof(int)));
-    HIP_TRY(hipMalloc((void **)&m->xrow, P * sizeof(int)));
-    HIP_TRY(hipMalloc((void **)&m->yrow, P * sizeof(int)));
+    HIP_TRY(hipMalloc((void **)&m->xrow, PR * sizeof(int)));
+    HIP_TRY(hipMalloc((void **)&m->yrow, PR * sizeof(int)));
     if (m->sgate) {
         size_t si = m->sgate->n;
         HIP_TRY(hipMalloc((void **)&m->sG, T * si * sizeof(float)));
@@ -540,6 +542,57 @@ void launch_moe_rows(const uint8_t *const *Wptr, size_t row_bytes, const float *
     else
         hipLaunchKernelGGL((jq::moe_rows_valu<Q, 4, SWIGLU>), grid, block, 0, s, Wptr, row_bytes, X, X2, gexp, offsets,
                            xsel, yrow, Y, k, n);
+}
+
+// The LDS-staged grouped kernel when the rows allow it (aligned row starts, four waves' rows within
+// 64 KB); returns -1 when they do not and the caller takes the plain kernels.
+template <class Q, bool DUAL>
+int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
+                      const float *X, const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y,
+                      int k, int n, int groups, int max_group, hipStream_t s) {
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
+    const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
+    const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
+    if (G == 0 || wave_lds * jq::ROWS_PER_WG > 64 * 1024 || getenv("JQ_NO_STAGED_ROWS")) return -1;
+    dim3 grid((unsigned)((n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R)), (unsigned)groups), block(64 * jq::ROWS_PER_WG);
+    const size_t lds = wave_lds * jq::ROWS_PER_WG;
+#define JQ_MOE_STAGED(MT, GG)                                                                                      \
+    hipLaunchKernelGGL((jq::moe_rows_staged<Q, MT, DUAL, GG>), grid, block, lds, s, Wa, Wb, row_bytes, X, gexp,     \
+                       offsets, xsel, yrow, Y, k, n, L, (int)wave_lds)
+    if (max_group <= 1) {
+        if (G == 16) JQ_MOE_STAGED(1, 16);
+        else JQ_MOE_STAGED(1, 4);
+    } else {
+        if (G == 16) JQ_MOE_STAGED(4, 16);
+        else JQ_MOE_STAGED(4, 4);
+    }
+#undef JQ_MOE_STAGED
+    return 0;
+}
+
+template <bool DUAL>
+int dispatch_moe_staged(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes,
+                        bool aligned16, const float *X, const int *gexp, const int *offsets, const int *xsel,
+                        const int *yrow, float *Y, int k, int n, int groups, int max_group, hipStream_t s) {
+    int rc;
+    switch (type) {
+#define JQ_MOE_CASE(ID, Q)                                                                                          \
+    case ID:                                                                                                        \
+        rc = launch_moe_staged<jq::Q, DUAL>(Wa, Wb, row_bytes, aligned16, X, gexp, offsets, xsel, yrow, Y, k, n,     \
+                                            groups, max_group, s);                                                  \
+        break;
+        JQ_MOE_CASE(JQ_TYPE_Q8_0, Q8_0)
+        JQ_MOE_CASE(JQ_TYPE_Q2_K, Q2_K)
+        JQ_MOE_CASE(JQ_TYPE_Q4_K, Q4_K)
+        JQ_MOE_CASE(JQ_TYPE_Q6_K, Q6_K)
+        JQ_MOE_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
+        JQ_MOE_CASE(JQ_TYPE_MXFP4, MXFP4)
+#undef JQ_MOE_CASE
+    default: return fail("unsupported tensor type id %u", type);
+    }
+    if (rc == 0) HIP_TRY(hipGetLastError());
+    return rc;
 }
 
 template <bool SWIGLU>
@@ -565,48 +618,72 @@ int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_byte
     return 0;
 }
 
-int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s) {
+int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg) {
     const jq_moe_config &c = m->cfg;
-    hipLaunchKernelGGL(jq::moe_router_logits, dim3((c.n_expert + 3) / 4), dim3(256), 0, s, m->router_w, x, m->logits,
-                       (int)T, (int)c.hidden, (int)c.n_expert);
+    hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert), dim3(256), 0, s, m->router_w, x, m->logits, (int)T,
+                       (int)c.hidden, (int)c.n_expert);
     jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
                          (int)c.n_group, (int)c.topk_group};
-    size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1)) * sizeof(float);
+    size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used) * sizeof(float);
     hipLaunchKernelGGL(jq::moe_gate_topk, dim3((unsigned)T), dim3(64), sm, s, m->logits, m->router_bias, gp, m->ids,
-                       m->wts);
+                       m->wts, pg);
     HIP_TRY(hipGetLastError());
     return 0;
 }
 
 int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s) {
     const jq_moe_config &c = m->cfg;
-    if (moe_route_dev(m, T, x, s)) return 1;
-    const int P = (int)(T * c.n_expert_used);
+    const int P = (int)(T * c.n_expert_used), extra = m->fold_shared ? 1 : 0;
     int groups, max_group;
-    if ((size_t)P <= c.n_expert) {  // decode-sized: one group per pair
-        groups = P;
+    if ((size_t)P <= c.n_expert) {  // decode-sized: one group per pair, written by the gating kernel itself
+        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra})) return 1;
+        groups = P + extra * (int)T;
         max_group = 1;
-        hipLaunchKernelGGL(jq::moe_pairs_as_groups, dim3(1), dim3(256), 0, s, m->ids, P, (int)c.n_expert_used, m->gexp,
-                           m->offsets, m->xrow, m->yrow);
     } else {
-        groups = (int)c.n_expert;
+        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{nullptr, nullptr, nullptr, nullptr, 0})) return 1;
+        groups = (int)c.n_expert + extra;
         max_group = (int)T;
         hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(256), (c.n_expert + 1) * sizeof(int), s, m->ids, (int)T,
-                           (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow);
+                           (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow, extra);
     }
     HIP_TRY(hipGetLastError());
-    // gate and up over the token rows, down over silu(gate)*up of each pair
-    if (dispatch_moe_rows<false>(m->gate->type, m->pgate, m->gate->row_bytes, x, nullptr, m->gexp, m->offsets, m->xrow,
-                                 m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s))
-        return 1;
-    if (dispatch_moe_rows<false>(m->up->type, m->pup, m->up->row_bytes, x, nullptr, m->gexp, m->offsets, m->xrow, m->yrow,
-                                 m->U, (int)c.hidden, (int)c.inter, groups, max_group, s))
-        return 1;
-    if (dispatch_moe_rows<true>(m->down->type, m->pdown, m->down->row_bytes, m->G, m->U, m->gexp, m->offsets, m->yrow,
-                                m->yrow, m->out, (int)c.inter, (int)c.hidden, groups, max_group, s))
-        return 1;
+    // silu(gate x) * (up x) of every pair into G, then down over it
+    const bool a16 = ((uintptr_t)m->gate->dev & 15) == 0 && ((uintptr_t)m->up->dev & 15) == 0 &&
+                     (!m->fold_shared || (((uintptr_t)m->sgate->dev & 15) == 0 && ((uintptr_t)m->sup->dev & 15) == 0));
+    int rc = -1;
+    if (m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes)
+        rc = dispatch_moe_staged<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, m->gexp, m->offsets,
+                                       m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s);
+    if (rc > 0) return 1;
+    const bool fused_act = rc == 0;
+    if (!fused_act) {
+        if (dispatch_moe_rows<false>(m->gate->type, m->pgate, m->gate->row_bytes, x, nullptr, m->gexp, m->offsets,
+                                     m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s))
+            return 1;
+        if (dispatch_moe_rows<false>(m->up->type, m->pup, m->up->row_bytes, x, nullptr, m->gexp, m->offsets, m->xrow,
+                                     m->yrow, m->U, (int)c.hidden, (int)c.inter, groups, max_group, s))
+            return 1;
+    }
+    const bool d16 = ((uintptr_t)m->down->dev & 15) == 0 && (!m->fold_shared || ((uintptr_t)m->sdown->dev & 15) == 0);
+    rc = fused_act ? dispatch_moe_staged<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G, m->gexp,
+                                                m->offsets, m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups,
+                                                max_group, s)
+                   : -1;
+    if (rc > 0) return 1;
+    if (rc < 0) {
+        if (fused_act) {  // G already holds the activation: plain rows over it
+            if (dispatch_moe_rows<false>(m->down->type, m->pdown, m->down->row_bytes, m->G, nullptr, m->gexp, m->offsets,
+                                         m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups, max_group, s))
+                return 1;
+        } else if (dispatch_moe_rows<true>(m->down->type, m->pdown, m->down->row_bytes, m->G, m->U, m->gexp, m->offsets,
+                                           m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups, max_group, s)) {
+            return 1;
+        }
+    }
     const float *shared_out = nullptr;
-    if (m->sgate) {  // shared expert over every token (reference: src/quantized_deepseek2.rs:555-557)
+    if (m->fold_shared) {
+        shared_out = m->out + (size_t)P * c.hidden;  // the rows the shared expert's pairs wrote
+    } else if (m->sgate) {  // shared expert over every token (reference: src/quantized_deepseek2.rs:555-557)
         size_t si = m->sgate->n;
         if (dispatch_matmul(m->sgate->type, m->sgate->dev, m->sgate->row_bytes, x, m->sG, T, c.hidden, si, s)) return 1;
         if (dispatch_matmul(m->sup->type, m->sup->dev, m->sup->row_bytes, x, m->sU, T, c.hidden, si, s)) return 1;
@@ -624,11 +701,15 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     return 0;
 }
 
-int moe_ptr_table(const jq_weight *w, size_t n_expert, size_t rows_per_expert, const uint8_t ***out) {
-    std::vector<const uint8_t *> host(n_expert);
+// Device table of expert base pointers; `extra` (the shared expert's weight, or null) becomes entry
+// n_expert.
+int moe_ptr_table(const jq_weight *w, size_t n_expert, size_t rows_per_expert, const jq_weight *extra,
+                  const uint8_t ***out) {
+    std::vector<const uint8_t *> host(n_expert + 1);
     for (size_t e = 0; e < n_expert; e++) host[e] = w->dev + e * rows_per_expert * w->row_bytes;
-    HIP_TRY(hipMalloc((void **)out, n_expert * sizeof(uint8_t *)));
-    HIP_TRY(hipMemcpy((void *)*out, host.data(), n_expert * sizeof(uint8_t *), hipMemcpyHostToDevice));
+    host[n_expert] = extra ? extra->dev : w->dev;
+    HIP_TRY(hipMalloc((void **)out, host.size() * sizeof(uint8_t *)));
+    HIP_TRY(hipMemcpy((void *)*out, host.data(), host.size() * sizeof(uint8_t *), hipMemcpyHostToDevice));
     return 0;
 }
 
@@ -687,8 +768,12 @@ int jq_moe_create(const jq_moe_config *cfg, const float *router_w, const float *
             return cleanup();
         }
     }
-    if (moe_ptr_table(gate_exps, c.n_expert, c.inter, &m->pgate) || moe_ptr_table(up_exps, c.n_expert, c.inter, &m->pup) ||
-        moe_ptr_table(down_exps, c.n_expert, c.hidden, &m->pdown))
+    // A shared expert of the routed experts' own type and shape rides along in the grouped kernels.
+    m->fold_shared = any_shared && shared_gate->type == gate_exps->type && shared_up->type == up_exps->type &&
+                     shared_down->type == down_exps->type && shared_gate->n == c.inter;
+    if (moe_ptr_table(gate_exps, c.n_expert, c.inter, m->fold_shared ? shared_gate : nullptr, &m->pgate) ||
+        moe_ptr_table(up_exps, c.n_expert, c.inter, m->fold_shared ? shared_up : nullptr, &m->pup) ||
+        moe_ptr_table(down_exps, c.n_expert, c.hidden, m->fold_shared ? shared_down : nullptr, &m->pdown))
         return cleanup();
     *out = m;
     return 0;
@@ -718,7 +803,7 @@ int jq_moe_route(jq_moe *m, size_t n_tokens, const float *x, uint32_t *ids, floa
         HIP_TRY(hipMemcpyAsync(xd.p, x, n_tokens * m->cfg.hidden * sizeof(float), hipMemcpyHostToDevice, s));
         xdev = (const float *)xd.p;
     }
-    if (moe_route_dev(m, n_tokens, xdev, s)) return 1;
+    if (moe_route_dev(m, n_tokens, xdev, s, jq::MoePairGroups{nullptr, nullptr, nullptr, nullptr, 0})) return 1;
     hipMemcpyKind kind = ptrs_are_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
     HIP_TRY(hipMemcpyAsync(ids, m->ids, P * sizeof(uint32_t), kind, s));
     HIP_TRY(hipMemcpyAsync(weights, m->wts, P * sizeof(float), kind, s));

@@ -12,13 +12,13 @@ namespace jq {
 // src/quantized_deepseek2.rs:528; an f32 matmul there too)
 __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict__ Wr, const float *__restrict__ X,
                                                           float *__restrict__ logits, int T, int h, int E) {
-    const int lane = threadIdx.x & 63;
-    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (e >= E) return;
+    // one workgroup per expert row of the router: every load of the row in flight at once
+    __shared__ float red[4][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, e = blockIdx.x;
     const float *wr = Wr + (size_t)e * h;
     for (int t0 = 0; t0 < T; t0 += 4) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int c = lane * 4; c < h; c += 256) {
+        for (int c = threadIdx.x * 4; c < h; c += 1024) {
             const float4 w = ld<float4>((const uint8_t *)(wr + c));
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -34,8 +34,13 @@ __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const float s = wave_sum(acc[i]);
-            if (lane == 0 && t0 + i < T) logits[(size_t)(t0 + i) * E + e] = s;
+            if (lane == 0) red[wave][i] = s;
         }
+        __syncthreads();
+        if (threadIdx.x < 4 && t0 + threadIdx.x < T)
+            logits[(size_t)(t0 + threadIdx.x) * E + e] =
+                (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+        __syncthreads();
     }
 }
 
@@ -52,11 +57,18 @@ struct MoeGateParams {
 // (reference: src/quantized_qwen3_moe.rs:424-436, src/quantized_deepseek2.rs:527-551,563-597).
 // Equal scores are ordered by expert index (the reference's sort order on ties
 // is that of a third-party argsort and is not pinned).
+// Where moe_gate_topk writes the pair groups itself (null gexp: a separate grouping kernel runs).
+// n_extra = 1 appends, per token, a pair for the shared expert (table index E, output row P + t).
+struct MoePairGroups {
+    int *gexp, *offsets, *xrow, *yrow;
+    int n_extra;
+};
+
 __global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ logits, const float *__restrict__ bias,
                                                      MoeGateParams p, uint32_t *__restrict__ ids,
-                                                     float *__restrict__ wts) {
-    extern __shared__ float sm[];  // probs[E], sel[E], gscore[n_group]
-    float *probs = sm, *sel = sm + p.E, *gscore = sm + 2 * p.E;
+                                                     float *__restrict__ wts, MoePairGroups pg) {
+    extern __shared__ float sm[];  // probs[E], sel[E], gscore[n_group], selw[k_used]
+    float *probs = sm, *sel = sm + p.E, *gscore = sm + 2 * p.E, *selw = gscore + (p.n_group > 1 ? p.n_group : 1);
     const int t = blockIdx.x, lane = threadIdx.x;
     const float *lg = logits + (size_t)t * p.E;
     if (p.sigmoid) {
@@ -108,20 +120,31 @@ __global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ lo
         for (int o = 0; o < p.E; o++) rank += sel[o] > v || (sel[o] == v && o < e);
         if (rank < p.k_used) {
             ids[(size_t)t * p.k_used + rank] = (uint32_t)e;
-            wts[(size_t)t * p.k_used + rank] = probs[e];
+            selw[rank] = probs[e];
+            if (pg.gexp) {  // decode-sized call: every (token, slot) pair is its own group
+                const int pidx = t * p.k_used + rank;
+                pg.gexp[pidx] = e, pg.offsets[pidx] = pidx, pg.xrow[pidx] = t, pg.yrow[pidx] = pidx;
+            }
         }
     }
     __syncthreads();
-    if (lane == 0) {
-        float *w = wts + (size_t)t * p.k_used;
+    for (int i = lane; i < p.k_used; i += 64) {
+        float w = selw[i];
         if (p.norm_topk) {
             float s = 0.0f;
-            for (int i = 0; i < p.k_used; i++) s += w[i];
-            s = fmaxf(s, 6.103515625e-5f);
-            for (int i = 0; i < p.k_used; i++) w[i] = w[i] / s;
+            for (int j = 0; j < p.k_used; j++) s += selw[j];
+            w = w / fmaxf(s, 6.103515625e-5f);
         }
-        if (p.scale != 0.0f && p.scale != 1.0f)
-            for (int i = 0; i < p.k_used; i++) w[i] = w[i] * p.scale;
+        if (p.scale != 0.0f && p.scale != 1.0f) w = w * p.scale;
+        wts[(size_t)t * p.k_used + i] = w;
+    }
+    if (pg.gexp && lane == 0) {
+        const int P = (int)gridDim.x * p.k_used, total = P + pg.n_extra * (int)gridDim.x;
+        if (t == 0) pg.offsets[total] = total;
+        if (pg.n_extra) {  // the shared expert as one more pair of this token
+            const int pidx = P + t;
+            pg.gexp[pidx] = p.E, pg.offsets[pidx] = pidx, pg.xrow[pidx] = t, pg.yrow[pidx] = pidx;
+        }
     }
 }
 
@@ -132,7 +155,8 @@ __global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ lo
 //   xrow[pos]  activation row (token) of the pair,  yrow[pos]  the pair index
 __global__ __launch_bounds__(256) void moe_group_pairs(const uint32_t *__restrict__ ids, int T, int k_used, int E,
                                                        int *__restrict__ gexp, int *__restrict__ offsets,
-                                                       int *__restrict__ xrow, int *__restrict__ yrow) {
+                                                       int *__restrict__ xrow, int *__restrict__ yrow,
+                                                       int shared_group) {
     extern __shared__ int cnt[];  // [E + 1]
     const int P = T * k_used;
     for (int e = threadIdx.x; e <= E; e += blockDim.x) cnt[e] = 0;
@@ -153,6 +177,10 @@ __global__ __launch_bounds__(256) void moe_group_pairs(const uint32_t *__restric
     }
     __syncthreads();
     for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = cnt[e];
+    if (shared_group) {  // group E: the shared expert over every token, output rows P .. P + T - 1
+        if (threadIdx.x == 0) gexp[E] = E, offsets[E + 1] = P + T;
+        for (int t = threadIdx.x; t < T; t += blockDim.x) xrow[P + t] = t, yrow[P + t] = P + t;
+    }
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         gexp[e] = e;
         int pos = cnt[e];
@@ -162,20 +190,6 @@ __global__ __launch_bounds__(256) void moe_group_pairs(const uint32_t *__restric
                 yrow[pos] = pidx;
                 pos++;
             }
-        }
-    }
-}
-
-// Few pairs (decode): every pair is its own group, its expert read from ids.
-__global__ __launch_bounds__(256) void moe_pairs_as_groups(const uint32_t *__restrict__ ids, int P, int k_used,
-                                                           int *__restrict__ gexp, int *__restrict__ offsets,
-                                                           int *__restrict__ xrow, int *__restrict__ yrow) {
-    for (int pidx = threadIdx.x; pidx <= P; pidx += blockDim.x) {
-        offsets[pidx] = pidx;
-        if (pidx < P) {
-            gexp[pidx] = (int)ids[pidx];
-            xrow[pidx] = pidx / k_used;
-            yrow[pidx] = pidx;
         }
     }
 }
@@ -245,6 +259,108 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_valu(const uint8_t 
         for (int i = 0; i < MT; i++) {
             const float s = wave_sum(acc[i]);
             if (lane == 0 && m0 + i < cnt) Y[(size_t)yrow[beg + m0 + i] * n + row] = s;
+        }
+    }
+}
+
+// The grouped expert matmul with the weight rows staged through LDS (see matmul_rows_staged): a
+// wave pulls the packed bytes of its 64 / L consecutive rows with coalesced asynchronous loads,
+// then L lanes work on each row (L = 16, 32 or 64, so that short rows still fill the wave).
+// DUAL: the same rows of two weight tables (gate and up) against one activation row, result
+// silu(gate . x) * (up . x) (reference: src/quantized_qwen3_moe.rs:397-401) without a round trip
+// of the two vectors through memory.
+template <class Q, int MT, bool DUAL, int G>
+__global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_t *const *__restrict__ Wa,
+                                                                     const uint8_t *const *__restrict__ Wb,
+                                                                     size_t row_bytes, const float *__restrict__ X,
+                                                                     const int *__restrict__ gexp,
+                                                                     const int *__restrict__ offsets,
+                                                                     const int *__restrict__ xsel,
+                                                                     const int *__restrict__ yrow,
+                                                                     float *__restrict__ Y, int k, int n, int L,
+                                                                     int wave_lds) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
+    const int grp = blockIdx.y;
+    const int beg = offsets[grp], cnt = offsets[grp + 1] - beg;
+    if (cnt == 0) return;
+    const int e = gexp[grp];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int R = 64 / L;
+    const int row0 = (blockIdx.x * ROWS_PER_WG + wave) * R;
+    if (row0 >= n) return;  // wave-uniform; the kernel has no barrier
+    const int nrows = min(R, n - row0);
+    uint8_t *ra = staged_moe + (size_t)wave * wave_lds, *rb = ra + (DUAL ? wave_lds / 2 : 0);
+    {
+        const int pieces = (int)((size_t)nrows * row_bytes / G);
+        const uint8_t *sa = Wa[e] + (size_t)row0 * row_bytes;
+        const uint8_t *sb = DUAL ? Wb[e] + (size_t)row0 * row_bytes : nullptr;
+        for (int p0 = 0; p0 < pieces; p0 += 64) {
+            if (p0 + lane < pieces) {
+                if (G == 16) {
+                    async_load16(sa + (size_t)(p0 + lane) * 16, lds_offset_of(ra + (size_t)p0 * 16));
+                    if (DUAL) async_load16(sb + (size_t)(p0 + lane) * 16, lds_offset_of(rb + (size_t)p0 * 16));
+                } else {
+                    async_load4(sa + (size_t)(p0 + lane) * 4, lds_offset_of(ra + (size_t)p0 * 4));
+                    if (DUAL) async_load4(sb + (size_t)(p0 + lane) * 4, lds_offset_of(rb + (size_t)p0 * 4));
+                }
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    const int sub = lane % L, rl = lane / L, row = row0 + rl;
+    const bool active = rl < nrows;
+    const uint8_t *rpa = ra + (size_t)rl * row_bytes, *rpb = rb + (size_t)rl * row_bytes;
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    constexpr int UE = Q::SEGS * Q::SEGLEN;
+    for (int m0 = 0; m0 < cnt; m0 += MT) {
+        float acc[MT], acc2[MT];
+        int xr[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            acc[i] = acc2[i] = 0.0f;
+            xr[i] = xsel[beg + min(m0 + i, cnt - 1)];
+        }
+        if (active) {
+            for (int u = sub; u < units; u += L) {
+                const int b = u / Q::UNITS, ub = u % Q::UNITS;
+                float w[UE], w2[DUAL ? UE : 1];
+                Q::decode(rpa + (size_t)b * Q::BLOCK_BYTES, ub, w);
+                if (DUAL) Q::decode(rpb + (size_t)b * Q::BLOCK_BYTES, ub, w2);
+                const int xoff = b * Q::BLOCK_ELEMS + Q::elem_base(ub);
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    if (m0 + i < cnt) {
+                        const float *xp = X + (size_t)xr[i] * k + xoff;
+#pragma unroll
+                        for (int s = 0; s < Q::SEGS; s++) {
+#pragma unroll
+                            for (int el = 0; el < Q::SEGLEN; el += 4) {
+                                const float4 xv = ld<float4>((const uint8_t *)(xp + s * Q::SEG_STRIDE + el));
+                                acc[i] = fmaf(xv.x, w[s * Q::SEGLEN + el + 0], acc[i]);
+                                acc[i] = fmaf(xv.y, w[s * Q::SEGLEN + el + 1], acc[i]);
+                                acc[i] = fmaf(xv.z, w[s * Q::SEGLEN + el + 2], acc[i]);
+                                acc[i] = fmaf(xv.w, w[s * Q::SEGLEN + el + 3], acc[i]);
+                                if (DUAL) {
+                                    acc2[i] = fmaf(xv.x, w2[s * Q::SEGLEN + el + 0], acc2[i]);
+                                    acc2[i] = fmaf(xv.y, w2[s * Q::SEGLEN + el + 1], acc2[i]);
+                                    acc2[i] = fmaf(xv.z, w2[s * Q::SEGLEN + el + 2], acc2[i]);
+                                    acc2[i] = fmaf(xv.w, w2[s * Q::SEGLEN + el + 3], acc2[i]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = acc[i], s2 = acc2[i];
+            for (int off = L >> 1; off > 0; off >>= 1) {
+                s += __shfl_xor(s, off, 64);
+                if (DUAL) s2 += __shfl_xor(s2, off, 64);
+            }
+            if (sub == 0 && active && m0 + i < cnt)
+                Y[(size_t)yrow[beg + m0 + i] * n + row] = DUAL ? silu(s) * s2 : s;
         }
     }
 }
