@@ -118,10 +118,10 @@ void launch_rows(const uint8_t *W, size_t row_bytes, const float *X, float *Y, s
     dim3 grid((unsigned)((n + jq::ROWS_PER_WG - 1) / jq::ROWS_PER_WG)), block(64 * jq::ROWS_PER_WG);
     // rows staged through LDS when their starts are 16- or 4-byte aligned and four of them fit in 64 KB
     const size_t stride = (row_bytes + 15) / 16 * 16;
-    const bool fits = stride * jq::ROWS_PER_WG <= 64 * 1024 && !getenv("JQ_NO_STAGED_ROWS");
+    const bool fits = stride * jq::ROWS_PER_WG + jq::table_bytes<Q>() <= 64 * 1024 && !getenv("JQ_NO_STAGED_ROWS");
     const int gran = !fits ? 0 : (row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0) ? 16
                                 : (row_bytes % 4 == 0 && ((uintptr_t)W & 3) == 0)  ? 4 : 0;
-    const size_t lds = stride * jq::ROWS_PER_WG;
+    const size_t lds = stride * jq::ROWS_PER_WG + jq::table_bytes<Q>();
 #define JQ_LAUNCH_ROWS(MT)                                                                                              \
     do {                                                                                                                 \
         if (gran == 16)                                                                                                  \
@@ -554,9 +554,9 @@ int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
     const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
     const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
-    if (G == 0 || wave_lds * jq::ROWS_PER_WG > 64 * 1024 || getenv("JQ_NO_STAGED_ROWS")) return -1;
+    if (G == 0 || wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>() > 64 * 1024 || getenv("JQ_NO_STAGED_ROWS")) return -1;
     dim3 grid((unsigned)((n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R)), (unsigned)groups), block(64 * jq::ROWS_PER_WG);
-    const size_t lds = wave_lds * jq::ROWS_PER_WG;
+    const size_t lds = wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>();
 #define JQ_MOE_STAGED(MT, GG)                                                                                      \
     hipLaunchKernelGGL((jq::moe_rows_staged<Q, MT, DUAL, GG>), grid, block, lds, s, Wa, Wb, row_bytes, X, gexp,     \
                        offsets, xsel, yrow, Y, k, n, L, (int)wave_lds)
@@ -624,8 +624,8 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
                        (int)c.hidden, (int)c.n_expert);
     jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
                          (int)c.n_group, (int)c.topk_group};
-    size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used) * sizeof(float);
-    hipLaunchKernelGGL(jq::moe_gate_topk, dim3((unsigned)T), dim3(64), sm, s, m->logits, m->router_bias, gp, m->ids,
+    size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);
+    hipLaunchKernelGGL(jq::moe_gate_topk, dim3((unsigned)T), dim3(256), sm, s, m->logits, m->router_bias, gp, m->ids,
                        m->wts, pg);
     HIP_TRY(hipGetLastError());
     return 0;
@@ -643,8 +643,10 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         if (moe_route_dev(m, T, x, s, jq::MoePairGroups{nullptr, nullptr, nullptr, nullptr, 0})) return 1;
         groups = (int)c.n_expert + extra;
         max_group = (int)T;
-        hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(256), (c.n_expert + 1) * sizeof(int), s, m->ids, (int)T,
-                           (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow, extra);
+        const int in_lds = (size_t)P <= 12288;
+        hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(256), (c.n_expert + 1 + (in_lds ? P : 0)) * sizeof(int), s,
+                           m->ids, (int)T, (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow,
+                           extra, in_lds);
     }
     HIP_TRY(hipGetLastError());
     // silu(gate x) * (up x) of every pair into G, then down over it

@@ -178,14 +178,18 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
     static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 66, UNITS = 8;
     static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
     __device__ static int elem_base(int u) { return 32 * u; }
-    __device__ static void decode(const uint8_t *blk, int u, float *w) {
+    // `grid` is the 256-entry codebook: the constant table, or a workgroup's copy of it in LDS
+    // (TABLE_BYTES), where the four lookups of a group cost LDS instead of vector-memory latency.
+    static constexpr int TABLE_BYTES = 2048;
+    __device__ static const uint64_t *table() { return g_tables.iq2xxs_grid; }
+    __device__ static void decode_with(const uint64_t *grid_table, const uint8_t *blk, int u, float *w) {
         float d = f16_bits(ld<uint16_t>(blk));
         uint2 g = ld<uint2>(blk + 2 + 8 * u);
         uint32_t lo = g.x, hi = g.y;
         float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
 #pragma unroll
         for (int l = 0; l < 4; l++) {
-            uint64_t grid = g_tables.iq2xxs_grid[(lo >> (8 * l)) & 0xFFu];
+            uint64_t grid = grid_table[(lo >> (8 * l)) & 0xFFu];
             uint32_t s7 = (hi >> (7 * l)) & 127u;
             uint32_t signs = s7 | ((__popc(s7) & 1u) << 7);
 #pragma unroll
@@ -195,23 +199,25 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
             }
         }
     }
+    __device__ static void decode(const uint8_t *blk, int u, float *w) { decode_with(g_tables.iq2xxs_grid, blk, u, w); }
 };
 
 struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
     static constexpr int BLOCK_ELEMS = 32, BLOCK_BYTES = 17, UNITS = 1;
     static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
     __device__ static int elem_base(int) { return 0; }
+    // E2M1 code c -> its value: the code's three magnitude bits placed at bit 22 of an f32 word read as
+    // (1 + mant/2) * 2^(exp - 127), or as the denormal mant * 2^-127 when exp == 0, which is 2^-126
+    // times the E2M1 value in both cases (1 exponent bit of bias against 127); the sign bit moves to
+    // bit 31.  One multiply by 2^126 then gives +-{0, .5, 1, 1.5, 2, 3, 4, 6} exactly.
     __device__ static float e2m1(uint32_t c) {
-        // magnitude: code 0 -> 0, 1 -> 0.5 (subnormal), else 2^(exp-1) * (1 + mant/2)
-        uint32_t mag = c & 7u;
-        float v = mag == 0 ? 0.0f : (mag == 1 ? 0.5f : __uint_as_float(((126u + (mag >> 1)) << 23) | ((mag & 1u) << 22)));
-        return (c & 8u) ? -v : v;
+        return __uint_as_float(((c & 7u) << 22) | ((c & 8u) << 28)) * 8.507059173023462e37f;  // 2^126
     }
     __device__ static void decode(const uint8_t *blk, int, float *w) {
         uint32_t e = blk[0];
         // 2^(e-127); e == 0 is the f32 denormal 2^-127; 0xFF (reserved) decodes the block to zeros
         float d = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
-        bool dead = e == 0xFFu;
+        const bool dead = e == 0xFFu;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             uint32_t v = ld<uint32_t>(blk + 1 + 4 * i);

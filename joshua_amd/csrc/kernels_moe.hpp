@@ -64,34 +64,43 @@ struct MoePairGroups {
     int n_extra;
 };
 
-__global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ logits, const float *__restrict__ bias,
-                                                     MoeGateParams p, uint32_t *__restrict__ ids,
-                                                     float *__restrict__ wts, MoePairGroups pg) {
-    extern __shared__ float sm[];  // probs[E], sel[E], gscore[n_group], selw[k_used]
+__global__ __launch_bounds__(256) void moe_gate_topk(const float *__restrict__ logits, const float *__restrict__ bias,
+                                                      MoeGateParams p, uint32_t *__restrict__ ids,
+                                                      float *__restrict__ wts, MoePairGroups pg) {
+    extern __shared__ float sm[];  // probs[E], sel[E], gscore[n_group], selw[k_used], red[4]
     float *probs = sm, *sel = sm + p.E, *gscore = sm + 2 * p.E, *selw = gscore + (p.n_group > 1 ? p.n_group : 1);
-    const int t = blockIdx.x, lane = threadIdx.x;
+    float *red = selw + p.k_used;
+    const int t = blockIdx.x, lane = threadIdx.x, wv = threadIdx.x >> 6;  // `lane` strides the experts by 256
+    constexpr int NT = 256;
     const float *lg = logits + (size_t)t * p.E;
     if (p.sigmoid) {
-        for (int e = lane; e < p.E; e += 64) probs[e] = 1.0f / (1.0f + expf(-lg[e]));
+        for (int e = lane; e < p.E; e += NT) probs[e] = 1.0f / (1.0f + expf(-lg[e]));
     } else {
         float mx = -INFINITY;
-        for (int e = lane; e < p.E; e += 64) mx = fmaxf(mx, lg[e]);
+        for (int e = lane; e < p.E; e += NT) mx = fmaxf(mx, lg[e]);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        if ((lane & 63) == 0) red[wv] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        __syncthreads();
         float sum = 0.0f;
-        for (int e = lane; e < p.E; e += 64) {
+        for (int e = lane; e < p.E; e += NT) {
             const float v = expf(lg[e] - mx);
             probs[e] = v;
             sum += v;
         }
         sum = wave_sum(sum);
-        for (int e = lane; e < p.E; e += 64) probs[e] = probs[e] / sum;
+        if ((lane & 63) == 0) red[wv] = sum;
+        __syncthreads();
+        sum = (red[0] + red[1]) + (red[2] + red[3]);
+        for (int e = lane; e < p.E; e += NT) probs[e] = probs[e] / sum;
     }
-    for (int e = lane; e < p.E; e += 64) sel[e] = probs[e] + (bias ? bias[e] : 0.0f);
+    for (int e = lane; e < p.E; e += NT) sel[e] = probs[e] + (bias ? bias[e] : 0.0f);
     __syncthreads();
     if (p.n_group > 1) {
         const int per = p.E / p.n_group;
-        for (int g = lane; g < p.n_group; g += 64) {
+        for (int g = lane; g < p.n_group; g += NT) {
             float b1 = -INFINITY, b2 = -INFINITY;  // two best of the group
             for (int i = 0; i < per; i++) {
                 const float v = sel[g * per + i];
@@ -105,7 +114,7 @@ __global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ lo
             gscore[g] = p.sigmoid ? b1 + b2 : b1;
         }
         __syncthreads();
-        for (int e = lane; e < p.E; e += 64) {
+        for (int e = lane; e < p.E; e += NT) {
             const int g = e / per;
             int rank = 0;
             for (int o = 0; o < p.n_group; o++) rank += gscore[o] > gscore[g] || (gscore[o] == gscore[g] && o < g);
@@ -114,7 +123,7 @@ __global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ lo
         }
         __syncthreads();
     }
-    for (int e = lane; e < p.E; e += 64) {
+    for (int e = lane; e < p.E; e += NT) {
         const float v = sel[e];
         int rank = 0;
         for (int o = 0; o < p.E; o++) rank += sel[o] > v || (sel[o] == v && o < e);
@@ -128,7 +137,7 @@ __global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ lo
         }
     }
     __syncthreads();
-    for (int i = lane; i < p.k_used; i += 64) {
+    for (int i = lane; i < p.k_used; i += NT) {
         float w = selw[i];
         if (p.norm_topk) {
             float s = 0.0f;
@@ -156,8 +165,8 @@ __global__ __launch_bounds__(64) void moe_gate_topk(const float *__restrict__ lo
 __global__ __launch_bounds__(256) void moe_group_pairs(const uint32_t *__restrict__ ids, int T, int k_used, int E,
                                                        int *__restrict__ gexp, int *__restrict__ offsets,
                                                        int *__restrict__ xrow, int *__restrict__ yrow,
-                                                       int shared_group) {
-    extern __shared__ int cnt[];  // [E + 1]
+                                                       int shared_group, int ids_in_lds) {
+    extern __shared__ int cnt[];  // [E + 1], then the pair list [P] when ids_in_lds
     const int P = T * k_used;
     for (int e = threadIdx.x; e <= E; e += blockDim.x) cnt[e] = 0;
     __syncthreads();
@@ -181,11 +190,18 @@ __global__ __launch_bounds__(256) void moe_group_pairs(const uint32_t *__restric
         if (threadIdx.x == 0) gexp[E] = E, offsets[E + 1] = P + T;
         for (int t = threadIdx.x; t < T; t += blockDim.x) xrow[P + t] = t, yrow[P + t] = P + t;
     }
+    // every expert's thread scans the pair list in order: from the LDS copy when it fits
+    uint32_t *ids_lds = (uint32_t *)(cnt + E + 1);
+    if (ids_in_lds) {
+        for (int pidx = threadIdx.x; pidx < P; pidx += blockDim.x) ids_lds[pidx] = ids[pidx];
+        __syncthreads();
+    }
+    const uint32_t *scan = ids_in_lds ? ids_lds : ids;
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         gexp[e] = e;
         int pos = cnt[e];
         for (int pidx = 0; pidx < P; pidx++) {
-            if (ids[pidx] == (uint32_t)e) {
+            if (scan[pidx] == (uint32_t)e) {
                 xrow[pos] = pidx / k_used;
                 yrow[pos] = pidx;
                 pos++;
@@ -280,6 +296,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
                                                                      float *__restrict__ Y, int k, int n, int L,
                                                                      int wave_lds) {
     extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
+    const auto *table = stage_table<Q>(staged_moe);  // before any wave leaves: it holds a barrier
     const int grp = blockIdx.y;
     const int beg = offsets[grp], cnt = offsets[grp + 1] - beg;
     if (cnt == 0) return;
@@ -289,7 +306,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
     const int row0 = (blockIdx.x * ROWS_PER_WG + wave) * R;
     if (row0 >= n) return;  // wave-uniform; the kernel has no barrier
     const int nrows = min(R, n - row0);
-    uint8_t *ra = staged_moe + (size_t)wave * wave_lds, *rb = ra + (DUAL ? wave_lds / 2 : 0);
+    uint8_t *ra = staged_moe + table_bytes<Q>() + (size_t)wave * wave_lds, *rb = ra + (DUAL ? wave_lds / 2 : 0);
     {
         const int pieces = (int)((size_t)nrows * row_bytes / G);
         const uint8_t *sa = Wa[e] + (size_t)row0 * row_bytes;
@@ -324,8 +341,8 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
             for (int u = sub; u < units; u += L) {
                 const int b = u / Q::UNITS, ub = u % Q::UNITS;
                 float w[UE], w2[DUAL ? UE : 1];
-                Q::decode(rpa + (size_t)b * Q::BLOCK_BYTES, ub, w);
-                if (DUAL) Q::decode(rpb + (size_t)b * Q::BLOCK_BYTES, ub, w2);
+                decode_staged<Q>(table, rpa + (size_t)b * Q::BLOCK_BYTES, ub, w);
+                if (DUAL) decode_staged<Q>(table, rpb + (size_t)b * Q::BLOCK_BYTES, ub, w2);
                 const int xoff = b * Q::BLOCK_ELEMS + Q::elem_base(ub);
 #pragma unroll
                 for (int i = 0; i < MT; i++) {

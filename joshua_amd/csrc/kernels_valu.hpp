@@ -10,6 +10,7 @@
 // These kernels serve every format and every m.  They are the general path;
 // the MFMA kernels take over where they apply.
 #pragma once
+#include <type_traits>
 #include "blocks.hpp"
 
 namespace jq {
@@ -84,6 +85,34 @@ __device__ __forceinline__ void async_load4(const void *gptr, uint32_t lds_base)
                  : "memory");
 }
 
+// Formats that decode through a lookup table keep a copy of it at the start of the workgroup's
+// dynamic LDS (table_bytes<Q>() bytes, 0 for the others).
+template <class Q, class = void>
+struct HasTable : std::false_type {};
+template <class Q>
+struct HasTable<Q, std::void_t<decltype(Q::TABLE_BYTES)>> : std::true_type {};
+
+template <class Q>
+__host__ __device__ constexpr int table_bytes() {
+    if constexpr (HasTable<Q>::value) return Q::TABLE_BYTES;
+    else return 0;
+}
+template <class Q>
+__device__ __forceinline__ const uint64_t *stage_table(uint8_t *lds) {
+    if constexpr (HasTable<Q>::value) {
+        for (int i = threadIdx.x; i < Q::TABLE_BYTES / 8; i += blockDim.x) ((uint64_t *)lds)[i] = Q::table()[i];
+        __syncthreads();
+        return (const uint64_t *)lds;
+    } else {
+        return nullptr;
+    }
+}
+template <class Q>
+__device__ __forceinline__ void decode_staged(const uint64_t *table, const uint8_t *blk, int u, float *w) {
+    if constexpr (HasTable<Q>::value) Q::decode_with(table, blk, u, w);
+    else Q::decode(blk, u, w);
+}
+
 // The same arithmetic as matmul_rows_valu with the weight row staged through LDS: each wave first
 // pulls its whole packed row into LDS with fully coalesced asynchronous loads of G bytes per lane
 // (the whole row in flight at once, whatever the block size), then decodes blocks out of LDS.  A
@@ -96,9 +125,10 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void matmul_rows_staged(const uin
                                                                         int lds_stride) {
     extern __shared__ __attribute__((aligned(16))) uint8_t staged_rows[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const auto *table = stage_table<Q>(staged_rows);  // before any wave leaves: it holds a barrier
     const int row = blockIdx.x * ROWS_PER_WG + wave;
-    if (row >= n) return;  // wave-uniform; the kernel has no barrier
-    uint8_t *rp = staged_rows + (size_t)wave * lds_stride;
+    if (row >= n) return;  // wave-uniform
+    uint8_t *rp = staged_rows + table_bytes<Q>() + (size_t)wave * lds_stride;
     {
         const uint8_t *src = W + (size_t)row * row_bytes;
         const int pieces = (int)(row_bytes / G);
@@ -119,7 +149,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void matmul_rows_staged(const uin
         for (int u = lane; u < units; u += 64) {
             const int b = u / Q::UNITS, ub = u % Q::UNITS;
             float w[UE];
-            Q::decode(rp + (size_t)b * Q::BLOCK_BYTES, ub, w);
+            decode_staged<Q>(table, rp + (size_t)b * Q::BLOCK_BYTES, ub, w);
             const int xoff = b * Q::BLOCK_ELEMS + Q::elem_base(ub);
 #pragma unroll
             for (int i = 0; i < MT; i++) {

@@ -76,6 +76,36 @@ def test_deepseek_style_layer_with_shared_expert(qtype):
         assert close(dev.forward(x), ora.forward(x))
 
 
+def test_shared_expert_of_another_width_runs_beside_the_groups():
+    ora, dev = build(capi.Q4_K, 512, 512, 8, 2, 90, shared_inter=256, gating="sigmoid")
+    for tokens in (1, 6):
+        x = synth.normal(91 + tokens, (tokens, 512))
+        assert close(dev.forward(x), ora.forward(x))
+
+
+@pytest.mark.parametrize("qtype,h,inter", [
+    (capi.Q6_K, 768, 256),      # 630-byte rows: no aligned staging, plain kernels; 256-wide down rows: 16 lanes a row
+    (capi.IQ2_XXS, 2560, 512),  # 660-byte rows: 4-byte staging
+    (capi.IQ2_XXS, 1792, 256),  # 462-byte rows: plain kernels
+    (capi.Q8_0, 96, 64),        # 102-byte rows, three blocks a row
+    (capi.MXFP4, 160, 96),      # 85-byte rows
+])
+def test_row_lengths_that_change_the_staging(qtype, h, inter):
+    ora, dev = build(qtype, h, inter, 8, 3, 100 + h)
+    for tokens in (1, 11):
+        x = synth.normal(101 + tokens, (tokens, h))
+        assert close(dev.forward(x), ora.forward(x))
+
+
+def test_many_tokens_group_beyond_the_lds_pair_list():
+    ora, dev = build(capi.Q8_0, 64, 32, 4, 2, 110)
+    x = synth.normal(111, (6200, 64))          # 12400 pairs
+    ids, w = dev.route(x)
+    oid, ow = ora.route(x)
+    assert np.array_equal(ids, oid)
+    assert close(dev.forward(x), ora.forward(x))
+
+
 def test_moe_rejects_mismatched_shapes():
     gate = capi.Weight.upload(capi.Q8_0, synth.normal_quantized(capi.Q8_0, 1, 4 * 32 * 256, 0.02), 4 * 32, 256)
     down = capi.Weight.upload(capi.Q8_0, synth.normal_quantized(capi.Q8_0, 2, 4 * 256 * 32, 0.02), 4 * 256, 32)
