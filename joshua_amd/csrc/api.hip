@@ -17,6 +17,7 @@
 #include "kernels_mfma_q4k.hpp"
 #include "kernels_graph.hpp"
 #include "kernels_mfma_q4k_gemm.hpp"
+#include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_valu.hpp"
 
@@ -218,6 +219,28 @@ int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
+// Q4_K, 1..16 activation rows, rows of at most 16 super-blocks: the weight-streaming MFMA kernel.
+// Returns -1 when the shape is outside its reach.
+int dispatch_q4k_stream(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                        hipStream_t s) {
+    const size_t nb = k / 256;
+    static const char *off = getenv("JQ_Q4K_NO_STREAM");
+    if (off || m > 16 || nb == 0 || nb > 16 || (nb > 8 && nb % 2 != 0) || row_bytes % 16 != 0 ||
+        ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
+        return -1;
+    const int cpw = nb > 8 ? 2 : 1, waves = (int)(nb / cpw);
+    const size_t n_tiles = (n + 15) / 16;
+    static const char *genv = getenv("JQ_Q4K_STREAM_GRID");
+    const size_t cap = genv ? (size_t)atoi(genv) : (cpw == 2 ? 256 : 512);
+    const unsigned grid = (unsigned)std::min<size_t>(n_tiles, std::max<size_t>(cap, 1));
+    if (cpw == 2)
+        hipLaunchKernelGGL(jq::q4k_stream_mfma<2>, dim3(grid), dim3(64 * waves), 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
+    else
+        hipLaunchKernelGGL(jq::q4k_stream_mfma<1>, dim3(grid), dim3(64 * waves), 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // Q4_K with more than 16 activation rows: prepare the fixed-point activation planes in a
 // stream-ordered scratch allocation, then the MFMA GEMM.
 int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
@@ -253,6 +276,12 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
 int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
                     size_t k, size_t n, hipStream_t s) {
     if (m > 0x7FFFFFFF || k > 0x7FFFFFFF || n > 0x7FFFFFFF) return fail("matmul: dimension exceeds 2^31-1");
+    // one or two activation rows: the int8 GEMV below is faster; from three on the streaming kernel,
+    // whose time hardly depends on the row count
+    if (type == JQ_TYPE_Q4_K && m > 2 && m <= Q4K_MFMA_MAX_M) {
+        const int rc = dispatch_q4k_stream(W, row_bytes, X, Y, m, k, n, s);
+        if (rc >= 0) return rc;
+    }
     if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k, n)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&
         !getenv("JQ_Q4K_NO_GEMM"))

@@ -15,8 +15,8 @@
 // super-block.  A single int8 activation plane (error 2^-8 of the group maximum)
 // cannot meet the 1e-3 bound on the results, and int8 planes of equal accuracy need
 // six MFMAs per tile and k step (two for sc q, three for X) against four here.
-// I2 is one more MFMA per tile and super-block over XS / 4096 split three ways into
-// f16.  One f32 combination per super-block applies d, dmin and s.
+// I2 is one more MFMA per tile and super-block over XS / 4096 split exactly three ways
+// into f16.  One f32 combination per super-block applies d, dmin and s.
 //
 // Workgroup: 128 weight rows x 64*MI activation rows, 8 waves = 2 (weight rows) x 4
 // (activation rows); a wave owns 64 x 16*MI outputs.  Weight nibbles are unpacked,
@@ -55,6 +55,16 @@ __device__ __forceinline__ uint32_t qg_pack_h2(int a, int b) {  // two small int
     return __builtin_bit_cast(uint32_t, v);
 }
 
+// A sub-block sum XS (|XS| < 2^27) over 4096 as three f16 values that add up to it exactly: its
+// balanced base-512 digits a0 + 512 a1 + 2^18 a2, scaled (a0 / 4096, a1 / 8, 64 a2).
+__device__ __forceinline__ void qg_split_sum(int xs, _Float16 &p0, _Float16 &p1, _Float16 &p2) {
+    const int a0 = ((xs + 256) & 511) - 256, r = (xs - a0) >> 9;
+    const int a1 = ((r + 256) & 511) - 256, a2 = (r - a1) >> 9;
+    p0 = (_Float16)((float)a0 * (1.0f / 4096.0f));
+    p1 = (_Float16)((float)a1 * 0.125f);
+    p2 = (_Float16)((float)a2 * 64.0f);
+}
+
 // One wave per (activation row, super-block).
 __global__ __launch_bounds__(256) void q4k_gemm_prep(const float *__restrict__ x, int m, int m_pad, int k,
                                                       Q4kGemmActs a) {
@@ -89,11 +99,8 @@ __global__ __launch_bounds__(256) void q4k_gemm_prep(const float *__restrict__ x
     xs += __shfl_xor(xs, 1, 64), xs += __shfl_xor(xs, 2, 64), xs += __shfl_xor(xs, 4, 64);
     if ((lane & 7) == 0) {
         const int j = lane >> 3;
-        const double val = (double)xs * (1.0 / 4096.0);
-        const _Float16 p0 = (_Float16)val;
-        const double r1 = val - (double)p0;
-        const _Float16 p1 = (_Float16)r1;
-        const _Float16 p2 = (_Float16)(r1 - (double)p1);
+        _Float16 p0, p1, p2;
+        qg_split_sum(xs, p0, p1, p2);
         _Float16 *o = a.mins + (((size_t)mt * nb + b) * 64 + (row & 15)) * 8 + j;
         o[0] = p0, o[16 * 8] = p1, o[32 * 8] = p2;
     }

@@ -150,13 +150,17 @@ def q4k_integer_case(n, k, seed, group=16, big_value=4161407, small=65535):
     return blocks.reshape(-1), q, x
 
 
-@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("m", [1, 2, 5, 16])
 def test_q4k_integer_dot_products_are_bit_exact(m):
     n, k = 160, 2048
-    blocks, q, x = q4k_integer_case(n, k, 90 + m)
+    if m <= 2:   # int8 GEMV: activation range 4161407 per 16-element group
+        blocks, q, x = q4k_integer_case(n, k, 90 + m)
+    else:        # streaming f16 MFMA kernel: 4193279 per 256-element super-block
+        blocks, q, x = q4k_integer_case(n, k, 90 + m, group=256, big_value=4193279, small=4000)
     assert np.array_equal(oracle.dequantize(capi.Q4_K, blocks).reshape(n, k), q.astype(np.float32))
-    lhs = np.stack([np.roll(x, 16 * i) for i in range(m)]).astype(np.float32)
-    want = (np.stack([np.roll(x, 16 * i) for i in range(m)]) @ q.T)
+    step = 16 if m <= 2 else 256
+    lhs = np.stack([np.roll(x, step * i) for i in range(m)]).astype(np.float32)
+    want = (np.stack([np.roll(x, step * i) for i in range(m)]) @ q.T)
     assert np.abs(want).max() < 2 ** 24
     ref = oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())
     assert np.array_equal(ref, want.astype(np.float32))
