@@ -18,6 +18,7 @@
 #include "kernels_graph.hpp"
 #include "kernels_mfma_q4k_gemm.hpp"
 #include "kernels_mfma_q4k_stream.hpp"
+#include "kernels_dot4_q4k.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_valu.hpp"
 
@@ -219,6 +220,26 @@ int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
+// Q4_K, one activation row, rows of at most 16 super-blocks: the integer-dot GEMV.
+// Returns -1 when the shape is outside its reach.
+int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
+    const size_t nb = k / 256;
+    // opt-in (JQ_Q4K_DOT4=1): on the 14336 x 4096 GEMV it streams at the same rate as the MFMA kernel
+    // below once running, but starts and drains more slowly (11.4 us against 10.2 us measured)
+    static const char *on = getenv("JQ_Q4K_DOT4");
+    if (!on || on[0] == '0' || nb == 0 || nb > jq::QD_MAX_WAVES || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 ||
+        ((uintptr_t)X & 15) != 0)
+        return -1;
+    static const char *genv = getenv("JQ_Q4K_DOT4_GRID");
+    // as many workgroups as the chip holds at once (one of 16 waves per CU, more when smaller), each
+    // with an equal share of the rows
+    const size_t cap = genv ? (size_t)atoi(genv) : 256 * std::max<size_t>(1, jq::QD_MAX_WAVES / nb);
+    const unsigned grid = (unsigned)std::min<size_t>((n + 15) / 16, std::max<size_t>(cap, 1));
+    hipLaunchKernelGGL(jq::q4k_gemv_dot4, dim3(grid), dim3((unsigned)(64 * nb)), 0, s, W, row_bytes, X, Y, (int)k, (int)n);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // Q4_K, 1..16 activation rows, rows of at most 16 super-blocks: the weight-streaming MFMA kernel.
 // Returns -1 when the shape is outside its reach.
 int dispatch_q4k_stream(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
@@ -276,6 +297,10 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
 int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
                     size_t k, size_t n, hipStream_t s) {
     if (m > 0x7FFFFFFF || k > 0x7FFFFFFF || n > 0x7FFFFFFF) return fail("matmul: dimension exceeds 2^31-1");
+    if (type == JQ_TYPE_Q4_K && m == 1) {
+        const int rc = dispatch_q4k_dot4(W, row_bytes, X, Y, k, n, s);
+        if (rc >= 0) return rc;
+    }
     // one or two activation rows: the int8 GEMV below is faster; from three on the streaming kernel,
     // whose time hardly depends on the row count
     if (type == JQ_TYPE_Q4_K && m > 2 && m <= Q4K_MFMA_MAX_M) {

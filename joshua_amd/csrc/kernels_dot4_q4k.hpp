@@ -1,0 +1,151 @@
+// Q4_K GEMV for one activation row: integer dot products on the vector ALU (v_dot4_i32_i8),
+// weights streamed once from HBM straight into registers, nothing but a 16-float reduction per
+// row tile in LDS.
+//
+// Per 32-element sub-block j of a weight row (reference arithmetic w = d sc q - dmin m,
+// src/kquant_dot.rs:440-465):
+//
+//   sum_k x_k w_k = (d sc_j) s_j S_j - (dmin m_j) s_j XS_j,   S_j = sum_k q_k X_k,  XS_j = sum_k X_k
+//
+// with X = round(x / s_j), s_j = amax_j(x) / 32639, the activation in 16-bit fixed point PER
+// SUB-BLOCK, split into two balanced byte planes X = 256 Xh + Xl.  S_j = 256 Sh + Sl with Sh, Sl
+// exact int32 sums of four-element dot products, so the integer dot product of a sub-block is
+// bit-exact; rounding the activation to 2^-16 of its own sub-block's maximum is far below the f32
+// accumulation noise of the reference and inside the 1e-3 bound on the results.
+//
+// Work split: a workgroup has one wave per 256-element super-block column of the weight matrix
+// (at most 16); lane (r = lane % 16, c = lane / 16) owns row r of the current 16-row tile and the
+// 64-element chunk c of the wave's block: 32 bytes whose low nibbles are sub-block 2c and whose high
+// nibbles are sub-block 2c+1, so a lane never shares a scale with another.  The activation planes of
+// that chunk (32 registers) are prepared once per workgroup and stay in registers; per tile a lane
+// loads its row's 16-byte block header and its 32 nibble bytes (the wave's loads cover the tile's
+// 16 x 144 bytes exactly once), two tiles ahead of use.  Each workgroup walks an equal share of the rows.
+#pragma once
+#include "kernels_valu.hpp"
+
+namespace jq {
+
+constexpr int QD_MAX_WAVES = 16;
+constexpr float QD_RANGE = 32639.0f;  // 127 * 256 + 127
+
+struct QdTile {  // what a lane holds of one 16-row tile
+    uint4 hdr, qa, qb;
+};
+
+__global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t *__restrict__ W, size_t row_bytes,
+                                                                    const float *__restrict__ X,
+                                                                    float *__restrict__ Y, int k, int n) {
+    __shared__ uint32_t xl_lds[QD_MAX_WAVES][64], xh_lds[QD_MAX_WAVES][64];  // byte planes, 4 elements a word
+    __shared__ float s_lds[QD_MAX_WAVES][8], xs_lds[QD_MAX_WAVES][8];        // per sub-block: scale, s * XS
+    __shared__ float red[2][QD_MAX_WAVES][16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int r = lane & 15, c = lane >> 4;
+    // this workgroup's share of the rows: an equal, contiguous range (not a whole number of tiles,
+    // so that every workgroup streams the same number of bytes); its last tile may be partial
+    const int G = (int)gridDim.x;
+    const int row_beg = (int)((long long)blockIdx.x * n / G), row_end = (int)((long long)(blockIdx.x + 1) * n / G);
+    const int n_tiles = (row_end - row_beg + 15) >> 4;
+    if (n_tiles == 0) return;
+
+    // loads are unconditional (tile and row indices are clamped into the range) so that every step
+    // issues the same number of loads and the compiler can wait for exactly the ones it needs
+    auto load_tile = [&](int i, QdTile &q) __attribute__((always_inline)) {
+        const int row = min(row_beg + 16 * min(i, n_tiles - 1) + r, row_end - 1);
+        const uint8_t *blk = W + (size_t)row * row_bytes + (size_t)wave * 144;
+        q.hdr = *(const uint4 *)blk;
+        q.qa = *(const uint4 *)(blk + 16 + 32 * c);
+        q.qb = *(const uint4 *)(blk + 32 + 32 * c);
+    };
+
+    // a ring of three register sets: tile i of this workgroup lives in set i % 3 and is loaded two
+    // steps before its use; the first two are on their way while the activation is prepared
+    QdTile ring0, ring1, ring2;
+    int t = 0;
+    load_tile(0, ring0);
+    load_tile(1, ring1);
+
+    // ---- activation of this wave's super-block: lane i quantises elements 4i .. 4i+3 ----
+    {
+        const float4 v = *(const float4 *)(X + 256 * wave + 4 * lane);
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));  // the 8 lanes of a sub-block
+        const bool live = amax > 0.0f && amax < INFINITY;
+        const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
+        const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                           __float2int_rn(v.w * inv)};
+        uint32_t wl = 0, wh = 0;
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int lo = ((Xq[i] + 128) & 255) - 128, hi = (Xq[i] - lo) >> 8;
+            wl |= (uint32_t)(lo & 255) << (8 * i);
+            wh |= (uint32_t)(hi & 255) << (8 * i);
+            sum += Xq[i];
+        }
+        xl_lds[wave][lane] = wl;
+        xh_lds[wave][lane] = wh;
+        sum += __shfl_xor(sum, 1, 64), sum += __shfl_xor(sum, 2, 64), sum += __shfl_xor(sum, 4, 64);
+        if ((lane & 7) == 0) {
+            s_lds[wave][lane >> 3] = s;
+            xs_lds[wave][lane >> 3] = s * (float)sum;
+        }
+    }
+    __syncthreads();
+    // chunk c: elements 64c .. 64c+31 ride on the low nibbles, 64c+32 .. 64c+63 on the high nibbles
+    uint32_t xl_lo[8], xh_lo[8], xl_hi[8], xh_hi[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        xl_lo[i] = xl_lds[wave][16 * c + i], xh_lo[i] = xh_lds[wave][16 * c + i];
+        xl_hi[i] = xl_lds[wave][16 * c + 8 + i], xh_hi[i] = xh_lds[wave][16 * c + 8 + i];
+    }
+    const float s_lo = s_lds[wave][2 * c], s_hi = s_lds[wave][2 * c + 1];
+    const float xs_lo = xs_lds[wave][2 * c], xs_hi = xs_lds[wave][2 * c + 1];
+
+    auto step = [&](QdTile &cur, QdTile &fill) __attribute__((always_inline)) {
+        load_tile(t + 2, fill);
+
+        uint32_t sc_lo, mn_lo, sc_hi, mn_hi;
+        q4k_scale_min(cur.hdr.y, cur.hdr.z, cur.hdr.w, 2 * c, sc_lo, mn_lo);
+        q4k_scale_min(cur.hdr.y, cur.hdr.z, cur.hdr.w, 2 * c + 1, sc_hi, mn_hi);
+        const uint32_t q[8] = {cur.qa.x, cur.qa.y, cur.qa.z, cur.qa.w, cur.qb.x, cur.qb.y, cur.qb.z, cur.qb.w};
+        int sl_lo = 0, sh_lo = 0, sl_hi = 0, sh_hi = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int lo4 = (int)(q[i] & 0x0F0F0F0Fu), hi4 = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+            sl_lo = __builtin_amdgcn_sdot4(lo4, (int)xl_lo[i], sl_lo, false);
+            sh_lo = __builtin_amdgcn_sdot4(lo4, (int)xh_lo[i], sh_lo, false);
+            sl_hi = __builtin_amdgcn_sdot4(hi4, (int)xl_hi[i], sl_hi, false);
+            sh_hi = __builtin_amdgcn_sdot4(hi4, (int)xh_hi[i], sh_hi, false);
+        }
+        const float d = f16_bits(cur.hdr.x), dmin = f16_bits(cur.hdr.x >> 16);
+        const float f_lo = (float)((sh_lo << 8) + sl_lo) * s_lo, f_hi = (float)((sh_hi << 8) + sl_hi) * s_hi;
+        float acc = d * fmaf((float)sc_lo, f_lo, (float)sc_hi * f_hi);
+        acc = fmaf(-dmin, fmaf((float)mn_lo, xs_lo, (float)mn_hi * xs_hi), acc);
+        acc += __shfl_xor(acc, 16, 64);
+        acc += __shfl_xor(acc, 32, 64);  // the four chunks of the block
+
+        // the waves' partial sums of the 16 rows meet in LDS; wave w then sums rows w, w + waves, ...
+        // over the waves (16 lanes, one partial each, a fixed tree), so no wave carries the whole reduction
+        const int buf = t & 1;
+        if (lane < 16) red[buf][wave][lane] = acc;
+        __syncthreads();
+        for (int rr = wave; rr < 16; rr += waves) {
+            float v = (lane < waves) ? red[buf][lane & 15][rr] : 0.0f;
+            v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
+            const int row = row_beg + 16 * t + rr;
+            if (lane == 0 && row < row_end) Y[row] = v;
+        }
+        t++;
+    };
+    while (t < n_tiles) {
+        step(ring0, ring2);
+        if (t >= n_tiles) break;
+        step(ring1, ring0);
+        if (t >= n_tiles) break;
+        step(ring2, ring1);
+    }
+}
+
+}  // namespace jq

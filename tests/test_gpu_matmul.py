@@ -153,7 +153,7 @@ def q4k_integer_case(n, k, seed, group=16, big_value=4161407, small=65535):
 @pytest.mark.parametrize("m", [1, 2, 5, 16])
 def test_q4k_integer_dot_products_are_bit_exact(m):
     n, k = 160, 2048
-    if m <= 2:   # int8 GEMV: activation range 4161407 per 16-element group
+    if m <= 2:   # int8 MFMA GEMV: activation range 4161407 per 16-element group
         blocks, q, x = q4k_integer_case(n, k, 90 + m)
     else:        # streaming f16 MFMA kernel: 4193279 per 256-element super-block
         blocks, q, x = q4k_integer_case(n, k, 90 + m, group=256, big_value=4193279, small=4000)
@@ -336,3 +336,35 @@ def test_headline_shape_q4k_gemv():
         torch.cuda.synchronize()
         want = oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True)
         assert close(y.cpu().numpy(), want)
+
+
+DOT4_CHILD = r"""
+import sys, numpy as np
+sys.path.insert(0, %r)
+import oracle
+from joshua_amd import capi, synth
+from tests.test_gpu_matmul import q4k_integer_case, close
+# exact integers: activation range 32639 per 32-element sub-block
+n, k = 150, 2048
+blocks, q, x = q4k_integer_case(n, k, 7, group=32, big_value=32639, small=4000)
+got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+assert np.array_equal(got[0], (x @ q.T).astype(np.float32)), "integer case"
+for (n, k) in [(14336, 4096), (100, 256), (4099, 1024), (33, 3840)]:
+    blocks = synth.normal_quantized(capi.Q4_K, 5 + n, n * k, 0.02)
+    lhs = synth.normal(6 + k, (1, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, lhs)
+    assert close(got, oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2())), (n, k)
+print("dot4 ok")
+"""
+
+
+def test_q4k_integer_dot_gemv_when_selected():
+    """The v_dot4 GEMV is selected by JQ_Q4K_DOT4=1 when the library first dispatches, so it runs
+    in a child process: exact on the integer construction, within tolerance on random shapes
+    (row counts that do not divide over the workgroups, short and 15-block rows)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, JQ_Q4K_DOT4="1")
+    res = subprocess.run([sys.executable, "-c", DOT4_CHILD % root], env=env, capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0 and "dot4 ok" in res.stdout, res.stdout + res.stderr
