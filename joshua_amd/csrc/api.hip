@@ -230,6 +230,14 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     if (!on || on[0] == '0' || nb == 0 || nb > jq::QD_MAX_WAVES || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 ||
         ((uintptr_t)X & 15) != 0)
         return -1;
+    static const char *lds_env = getenv("JQ_Q4K_DOT4_LDS");
+    if (lds_env && lds_env[0] != '0' && nb == 16) {
+        static const char *g2 = getenv("JQ_Q4K_DOT4_GRID");
+        const unsigned grid = (unsigned)std::min<size_t>((n + 15) / 16, g2 ? (size_t)atoi(g2) : 256);
+        hipLaunchKernelGGL(jq::q4k_gemv_dot4_lds, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
     static const char *genv = getenv("JQ_Q4K_DOT4_GRID");
     // as many workgroups as the chip holds at once (one of 16 waves per CU, more when smaller), each
     // with an equal share of the rows

@@ -148,4 +148,125 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
     }
 }
 
+// The same GEMV with the weights travelling HBM -> LDS as asynchronous, fully coalesced loads: wave w
+// copies row w of every 16-row tile (its whole packed row: three instructions of up to 1 KB) into a
+// ring of three tiles in LDS, two tiles ahead of the arithmetic; the lanes then read their header and
+// 32 nibble bytes from LDS.  Rows are padded by 16 bytes in LDS so that the 16 rows a wave reads in one
+// instruction fall into different banks.  No vector register is spent on prefetching, and every global
+// access is a contiguous kilobyte.  Needs exactly 16 super-blocks a row (one wave per row of a tile).
+constexpr int QD_ROW = 16 * 144, QD_ROW_LDS = QD_ROW + 16, QD_TILE_LDS = 16 * QD_ROW_LDS;
+
+__global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
+                                                          float *__restrict__ Y, int n) {
+    __shared__ __attribute__((aligned(16))) uint8_t ring[3][QD_TILE_LDS];
+    __shared__ uint32_t xl_lds[16][64], xh_lds[16][64];
+    __shared__ float s_lds[16][8], xs_lds[16][8];
+    __shared__ float red[2][16][16];
+    __shared__ __attribute__((aligned(16))) float x_raw[16][256];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, c = lane >> 4;
+    const int G = (int)gridDim.x;
+    const int row_beg = (int)((long long)blockIdx.x * n / G), row_end = (int)((long long)(blockIdx.x + 1) * n / G);
+    const int n_tiles = (row_end - row_beg + 15) >> 4;
+    if (n_tiles == 0) return;
+
+    // 3 asynchronous loads per wave and tile: row `wave` of tile i (clamped into the range) -> ring slot
+    auto fetch = [&](int i, int slot) __attribute__((always_inline)) {
+        const int row = min(row_beg + 16 * min(i, n_tiles - 1) + wave, row_end - 1);
+        const uint8_t *src = W + (size_t)row * QD_ROW + 16 * lane;
+        const uint32_t dst = lds_offset_of(&ring[slot][wave * QD_ROW_LDS]);
+        async_load16(src, dst);
+        async_load16(src + 1024, dst + 1024);
+        if (lane < 16) async_load16(src + 2048, dst + 2048);
+    };
+    // the activation column of this wave travels the same way, first (every global read of this kernel
+    // is an asynchronous load, counted by hand)
+    async_load16(X + 256 * wave + 4 * lane, lds_offset_of(&x_raw[wave][0]));
+    fetch(0, 0);
+    fetch(1, 1);
+    asm volatile("s_waitcnt vmcnt(6)" ::: "memory");  // the activation landed (own wave's data: no barrier needed)
+
+    {
+        const float4 v = *(const float4 *)&x_raw[wave][4 * lane];
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+        const bool live = amax > 0.0f && amax < INFINITY;
+        const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
+        const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                           __float2int_rn(v.w * inv)};
+        uint32_t wl = 0, wh = 0;
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int lo = ((Xq[i] + 128) & 255) - 128, hi = (Xq[i] - lo) >> 8;
+            wl |= (uint32_t)(lo & 255) << (8 * i);
+            wh |= (uint32_t)(hi & 255) << (8 * i);
+            sum += Xq[i];
+        }
+        xl_lds[wave][lane] = wl;
+        xh_lds[wave][lane] = wh;
+        sum += __shfl_xor(sum, 1, 64), sum += __shfl_xor(sum, 2, 64), sum += __shfl_xor(sum, 4, 64);
+        if ((lane & 7) == 0) {
+            s_lds[wave][lane >> 3] = s;
+            xs_lds[wave][lane >> 3] = s * (float)sum;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");  // tile 0 landed (tile 1 may be in flight), planes written
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    uint32_t xl_lo[8], xh_lo[8], xl_hi[8], xh_hi[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        xl_lo[i] = xl_lds[wave][16 * c + i], xh_lo[i] = xh_lds[wave][16 * c + i];
+        xl_hi[i] = xl_lds[wave][16 * c + 8 + i], xh_hi[i] = xh_lds[wave][16 * c + 8 + i];
+    }
+    const float s_lo = s_lds[wave][2 * c], s_hi = s_lds[wave][2 * c + 1];
+    const float xs_lo = xs_lds[wave][2 * c], xs_hi = xs_lds[wave][2 * c + 1];
+
+    // on entry to step t: tile t is in LDS and visible (the barrier just passed), tile t+1 in flight
+    for (int t = 0; t < n_tiles; t++) {
+        const int slot = t % 3;
+        fetch(t + 2, (t + 2) % 3);  // the slot of tile t-1, which every wave finished reading before that barrier
+
+        const uint8_t *blk = &ring[slot][r * QD_ROW_LDS + wave * 144];
+        const uint4 hdr = *(const uint4 *)blk;
+        const uint4 qa = *(const uint4 *)(blk + 16 + 32 * c), qb = *(const uint4 *)(blk + 32 + 32 * c);
+        uint32_t sc_lo, mn_lo, sc_hi, mn_hi;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc_lo, mn_lo);
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc_hi, mn_hi);
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        int sl_lo = 0, sh_lo = 0, sl_hi = 0, sh_hi = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int lo4 = (int)(q[i] & 0x0F0F0F0Fu), hi4 = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+            sl_lo = __builtin_amdgcn_sdot4(lo4, (int)xl_lo[i], sl_lo, false);
+            sh_lo = __builtin_amdgcn_sdot4(lo4, (int)xh_lo[i], sh_lo, false);
+            sl_hi = __builtin_amdgcn_sdot4(hi4, (int)xl_hi[i], sl_hi, false);
+            sh_hi = __builtin_amdgcn_sdot4(hi4, (int)xh_hi[i], sh_hi, false);
+        }
+        const float d = f16_bits(hdr.x), dmin = f16_bits(hdr.x >> 16);
+        const float f_lo = (float)((sh_lo << 8) + sl_lo) * s_lo, f_hi = (float)((sh_hi << 8) + sl_hi) * s_hi;
+        float acc = d * fmaf((float)sc_lo, f_lo, (float)sc_hi * f_hi);
+        acc = fmaf(-dmin, fmaf((float)mn_lo, xs_lo, (float)mn_hi * xs_hi), acc);
+        acc += __shfl_xor(acc, 16, 64);
+        acc += __shfl_xor(acc, 32, 64);
+
+        const int buf = t & 1;
+        if (lane < 16) red[buf][wave][lane] = acc;
+        // the partial sums are written and tile t+1 has landed: at most this step's 3 loads stay in flight
+        asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        {   // wave w sums row w of the tile over the 16 waves
+            float v = (lane < 16) ? red[buf][lane][wave] : 0.0f;
+            v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
+            const int row = row_beg + 16 * t + wave;
+            if (lane == 0 && row < row_end) Y[row] = v;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped fetches of the last two steps
+}
+
 }  // namespace jq

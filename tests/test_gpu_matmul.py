@@ -345,11 +345,11 @@ import oracle
 from joshua_amd import capi, synth
 from tests.test_gpu_matmul import q4k_integer_case, close
 # exact integers: activation range 32639 per 32-element sub-block
-n, k = 150, 2048
+n, k = 150, 4096
 blocks, q, x = q4k_integer_case(n, k, 7, group=32, big_value=32639, small=4000)
 got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
 assert np.array_equal(got[0], (x @ q.T).astype(np.float32)), "integer case"
-for (n, k) in [(14336, 4096), (100, 256), (4099, 1024), (33, 3840)]:
+for (n, k) in [(14336, 4096), (100, 256), (4099, 1024), (33, 3840), (4099, 4096), (7, 4096)]:
     blocks = synth.normal_quantized(capi.Q4_K, 5 + n, n * k, 0.02)
     lhs = synth.normal(6 + k, (1, k))
     got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, lhs)
@@ -358,13 +358,15 @@ print("dot4 ok")
 """
 
 
-def test_q4k_integer_dot_gemv_when_selected():
-    """The v_dot4 GEMV is selected by JQ_Q4K_DOT4=1 when the library first dispatches, so it runs
-    in a child process: exact on the integer construction, within tolerance on random shapes
-    (row counts that do not divide over the workgroups, short and 15-block rows)."""
+@pytest.mark.parametrize("through_lds", ["0", "1"])
+def test_q4k_integer_dot_gemv_when_selected(through_lds):
+    """The v_dot4 GEMV (weights prefetched into registers, or through an LDS ring for 4096-wide rows)
+    is selected by environment variables when the library first dispatches, so it runs in a child
+    process: exact on the integer construction, within tolerance on random shapes (row counts that
+    do not divide over the workgroups, short and 15-block rows)."""
     import subprocess
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, JQ_Q4K_DOT4="1")
+    env = dict(os.environ, JQ_Q4K_DOT4="1", JQ_Q4K_DOT4_LDS=through_lds)
     res = subprocess.run([sys.executable, "-c", DOT4_CHILD % root], env=env, capture_output=True, text=True, timeout=110)
     assert res.returncode == 0 and "dot4 ok" in res.stdout, res.stdout + res.stderr
