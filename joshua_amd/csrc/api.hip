@@ -902,6 +902,12 @@ struct jq_model {
     jq_qwen3_config cfg;
     std::map<std::string, jq_weight *> q;   // quantized matrices by GGUF name
     std::map<std::string, float *> f;       // f32 vectors by GGUF name
+    // Matrices that multiply the same activation, laid one after the other in one allocation
+    // (blk.N.qkv, blk.N.gate_up): one launch for a single-token step; q holds views of their parts.
+    std::map<std::string, jq_weight *> fused;
+    std::vector<jq_weight *> retired;  // fused allocations whose parts were replaced; views may still point into them
+    bool fused_ready = false;
+    float *cat = nullptr;     // the fused result of a single-token step (q|k|v, gate|up)
     std::vector<float *> kc, vc;            // per layer [n_kv, n_ctx, d]
     uint32_t n_past = 0;
     size_t cap_tokens = 0;
@@ -978,6 +984,70 @@ int model_vec(jq_model *m, const std::string &name, const float **out) {
     return 0;
 }
 
+// Lays the named matrices (same type, same k) one after the other in a new allocation `key`, and
+// replaces their entries in m->q by views of it.  Skipped when any is missing or the types differ.
+int model_fuse(jq_model *m, const std::string &key, const std::vector<std::string> &names) {
+    std::vector<jq_weight *> parts;
+    for (const auto &nm : names) {
+        auto it = m->q.find(nm);
+        if (it == m->q.end() || !it->second->owns) return 0;
+        parts.push_back(it->second);
+    }
+    size_t rows = 0, bytes = 0;
+    for (auto *w : parts) {
+        if (w->type != parts[0]->type || w->k != parts[0]->k) return 0;
+        rows += w->n, bytes += w->nbytes;
+    }
+    uint8_t *dev = nullptr;
+    HIP_TRY(hipMalloc((void **)&dev, bytes));
+    size_t off = 0;
+    for (auto *w : parts) {
+        hipError_t e = hipMemcpy(dev + off, w->dev, w->nbytes, hipMemcpyDeviceToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(dev);
+            return fail("qwen3: fusing `%s` failed: %s", key.c_str(), hipGetErrorString(e));
+        }
+        off += w->nbytes;
+    }
+    jq_weight *whole = new jq_weight{parts[0]->type, rows, parts[0]->k, bytes, parts[0]->row_bytes, dev, true};
+    m->fused[key] = whole;
+    off = 0;
+    for (size_t i = 0; i < parts.size(); i++) {
+        jq_weight *view = nullptr;
+        if (jq_view(whole, off, parts[i]->n, parts[i]->k, &view)) return 1;
+        off += parts[i]->nbytes;
+        jq_free(parts[i]);
+        m->q[names[i]] = view;
+    }
+    return 0;
+}
+
+int model_prepare_fused(jq_model *m) {
+    if (m->fused_ready) return 0;
+    const jq_qwen3_config &c = m->cfg;
+    for (uint32_t l = 0; l < c.n_layer; l++) {
+        const std::string p = "blk." + std::to_string(l);
+        if (!m->fused.count(p + ".qkv")) {
+            // q|k|v when all three share a type, else q|k (attn_v is often kept at more bits)
+            auto q = m->q.find(p + ".attn_q.weight"), v = m->q.find(p + ".attn_v.weight");
+            const bool with_v = q != m->q.end() && v != m->q.end() && q->second->type == v->second->type;
+            if (model_fuse(m, p + ".qkv",
+                           with_v ? std::vector<std::string>{p + ".attn_q.weight", p + ".attn_k.weight", p + ".attn_v.weight"}
+                                  : std::vector<std::string>{p + ".attn_q.weight", p + ".attn_k.weight"}))
+                return 1;
+        }
+        if (!m->fused.count(p + ".gate_up") &&
+            model_fuse(m, p + ".gate_up", {p + ".ffn_gate.weight", p + ".ffn_up.weight"}))
+            return 1;
+    }
+    if (!m->cat) {
+        const size_t widest = std::max<size_t>((size_t)(c.n_head + 2 * c.n_kv_head) * c.head_dim, 2 * (size_t)c.ffn);
+        HIP_TRY(hipMalloc((void **)&m->cat, widest * sizeof(float)));
+    }
+    m->fused_ready = true;
+    return 0;
+}
+
 unsigned grid_for(size_t total) { return (unsigned)std::min<size_t>((total + 255) / 256, 8192); }
 
 int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
@@ -999,25 +1069,44 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             model_vec(m, p + ".attn_q_norm.weight", &w_qn) || model_vec(m, p + ".attn_k_norm.weight", &w_kn))
             return 1;
         hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, m->x, pending, w_an, c.rms_eps, m->hn, h);
-        if (model_mm(m, p + ".attn_q.weight", m->hn, m->qb, T, s) || model_mm(m, p + ".attn_k.weight", m->hn, m->kb, T, s) ||
-            model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s))
+        float *qp = m->qb, *kp = m->kb, *vp = m->vb;
+        auto fq = T == 1 ? m->fused.find(p + ".qkv") : m->fused.end();
+        if (fq != m->fused.end()) {  // one launch for q|k(|v) of a single token
+            const jq_weight *w = fq->second;
+            if (dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
+            qp = m->cat, kp = m->cat + (size_t)nh * d;
+            if (w->n == (size_t)(nh + 2 * nkv) * d) vp = kp + (size_t)nkv * d;
+            else if (model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s)) return 1;
+        } else if (model_mm(m, p + ".attn_q.weight", m->hn, m->qb, T, s) ||
+                   model_mm(m, p + ".attn_k.weight", m->hn, m->kb, T, s) ||
+                   model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s)) {
             return 1;
-        hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, m->qb, m->kb, m->vb, w_qn,
-                           w_kn, c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
+        }
+        hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, qp, kp, vp, w_qn, w_kn,
+                           c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
         if (split) {
-            hipLaunchKernelGGL(jq::attention_split, dim3(T * nh * n_chunks), dim3(256), 0, s, m->qb, m->kc[l], m->vc[l],
+            hipLaunchKernelGGL(jq::attention_split, dim3(T * nh * n_chunks), dim3(256), 0, s, qp, m->kc[l], m->vc[l],
                                m->part, nh, nkv, d, m->pos, (int)c.n_ctx, sqrt_d, n_chunks);
-            hipLaunchKernelGGL(jq::attention_merge, dim3(T * nh), dim3(256), 0, s, m->part, m->att, d, n_chunks);
+            hipLaunchKernelGGL(jq::attention_merge, dim3(T * nh), dim3(128), n_chunks * sizeof(float), s, m->part, m->att, d,
+                               n_chunks);
         } else {
             size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
-            hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, m->qb, m->kc[l], m->vc[l], m->att, nh,
+            hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, qp, m->kc[l], m->vc[l], m->att, nh,
                                nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
         }
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
         hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, m->x, m->proj, w_fn, c.rms_eps, m->hn, h);
-        if (model_mm(m, p + ".ffn_gate.weight", m->hn, m->g, T, s) || model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s))
+        const float *gp = m->g, *up = m->u;
+        auto fg = T == 1 ? m->fused.find(p + ".gate_up") : m->fused.end();
+        if (fg != m->fused.end()) {
+            const jq_weight *w = fg->second;
+            if (dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
+            gp = m->cat, up = m->cat + c.ffn;
+        } else if (model_mm(m, p + ".ffn_gate.weight", m->hn, m->g, T, s) ||
+                   model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s)) {
             return 1;
-        hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, m->g, m->u, m->mid,
+        }
+        hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, gp, up, m->mid,
                            (size_t)T * c.ffn);
         if (model_mm(m, p + ".ffn_down.weight", m->mid, m->proj, T, s)) return 1;
         pending = m->proj;
@@ -1078,6 +1167,9 @@ void jq_qwen3_free(jq_model *m) {
     if (!m) return;
     model_free_scratch(m);
     for (auto &kv : m->q) jq_free(kv.second);
+    for (auto &kv : m->fused) jq_free(kv.second);
+    for (auto *w : m->retired) jq_free(w);
+    if (m->cat) (void)hipFree(m->cat);
     for (auto &kv : m->f) (void)hipFree(kv.second);
     for (float *p : m->kc) (void)hipFree(p);
     for (float *p : m->vc) (void)hipFree(p);
@@ -1113,6 +1205,23 @@ int jq_qwen3_set_tensor(jq_model *m, const char *name, uint32_t ggml_type, const
     auto old = m->q.find(name);
     if (old != m->q.end()) jq_free(old->second);
     m->q[name] = w;
+    // a replaced part: the fused copy it belonged to is retired (the other parts' views keep pointing
+    // into it) and that group runs as separate launches from now on
+    const std::string nm = name;
+    const size_t dot = nm.find('.', 4);
+    if (nm.rfind("blk.", 0) == 0 && dot != std::string::npos) {
+        const std::string layer = nm.substr(0, dot), role = nm.substr(dot);
+        const char *key = (role == ".attn_q.weight" || role == ".attn_k.weight" || role == ".attn_v.weight") ? ".qkv"
+                          : (role == ".ffn_gate.weight" || role == ".ffn_up.weight")                         ? ".gate_up"
+                                                                                                             : nullptr;
+        if (key) {
+            auto it = m->fused.find(layer + key);
+            if (it != m->fused.end()) {
+                m->retired.push_back(it->second);
+                m->fused.erase(it);
+            }
+        }
+    }
     return 0;
 }
 
@@ -1129,6 +1238,7 @@ int jq_qwen3_forward(jq_model *m, const uint32_t *tokens, uint32_t n_tokens, uin
         if (tokens[i] >= m->cfg.vocab) return fail("embedding id %u is out of range for %u rows", tokens[i], m->cfg.vocab);
     hipStream_t s = (hipStream_t)stream;
     if (model_reserve(m, n_tokens)) return 1;
+    if (n_tokens == 1 && model_prepare_fused(m)) return 1;
     HIP_TRY(hipMemcpyAsync(m->ids, tokens, n_tokens * sizeof(uint32_t), hipMemcpyHostToDevice, s));
     if (model_forward_dev(m, n_tokens, pos, s)) return 1;
     m->n_past = pos + n_tokens;

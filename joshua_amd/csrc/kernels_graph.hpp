@@ -159,8 +159,7 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
                                                         int n_head, int n_kv, int d, const int *__restrict__ pos_ptr,
                                                         int n_ctx, float sqrt_d, int n_chunks) {
     __shared__ float sc[ATT_CHUNK];
-    __shared__ float red[16];
-    __shared__ float accs[4][256];  // d <= 256
+    __shared__ float4 accs[256];    // [key part][column group of four]
     const int chunk = blockIdx.x % n_chunks, hq = (blockIdx.x / n_chunks) % n_head, t = blockIdx.x / (n_chunks * n_head);
     const int kvh = hq / (n_head / n_kv), n_keys = *pos_ptr + t + 1;
     const int j0 = chunk * ATT_CHUNK, nj = min(ATT_CHUNK, n_keys - j0);
@@ -198,40 +197,53 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
     __syncthreads();
     if (wave == 0) sc[lane] = e;
     __syncthreads();
-    // acc[c] = sum_j e_j v[j, c]: thread (c = tid % d, part = tid / d) strides the keys
-    const int nparts = 256 / d > 0 ? 256 / d : 1;
-    const float *vb = vc + ((size_t)kvh * n_ctx + j0) * d;
-    for (int c = threadIdx.x % d, pt = threadIdx.x / d; pt < nparts && c < d; pt = nparts) {
-        float acc = 0.0f;
-        for (int j = pt; j < nj; j += nparts) acc = fmaf(sc[j], vb[(size_t)j * d + c], acc);
-        accs[pt][c] = acc;
+    // acc[c] = sum_j e_j v[j, c]: thread (column group of four, key part) strides the keys of its part;
+    // the loads of a thread do not depend on each other, so several are in flight at once
+    const int ngroups = d >> 2, kparts = 256 / ngroups;  // d = 128: 32 groups x 8 parts
+    const int cg = threadIdx.x % ngroups, kp = threadIdx.x / ngroups;
+    const float *vb = vc + ((size_t)kvh * n_ctx + j0) * d + 4 * cg;
+    float4 acc = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int j = kp; j < ATT_CHUNK; j += kparts) {
+        if (j < nj) {
+            const float4 v = *(const float4 *)(vb + (size_t)j * d);
+            const float e_j = sc[j];
+            acc.x = fmaf(e_j, v.x, acc.x), acc.y = fmaf(e_j, v.y, acc.y);
+            acc.z = fmaf(e_j, v.z, acc.z), acc.w = fmaf(e_j, v.w, acc.w);
+        }
     }
+    accs[kp * ngroups + cg] = acc;
     __syncthreads();
-    for (int c = threadIdx.x; c < d; c += 256) {
-        float a = accs[0][c];
-        for (int pt = 1; pt < nparts; pt++) a += accs[pt][c];
-        po[2 + c] = a;
+    if (threadIdx.x < ngroups) {
+        float4 a = accs[threadIdx.x];
+        for (int pt = 1; pt < kparts; pt++) {
+            const float4 o = accs[pt * ngroups + threadIdx.x];
+            a.x += o.x, a.y += o.y, a.z += o.z, a.w += o.w;
+        }
+        po[2 + 4 * threadIdx.x + 0] = a.x, po[2 + 4 * threadIdx.x + 1] = a.y;
+        po[2 + 4 * threadIdx.x + 2] = a.z, po[2 + 4 * threadIdx.x + 3] = a.w;
     }
     if (threadIdx.x == 0) po[0] = mx, po[1] = l;
-    (void)red;
 }
 
+// out[(t, head), :] = sum_ch exp(m_ch - m) acc_ch / sum_ch exp(m_ch - m) l_ch over the chunks with keys
 __global__ __launch_bounds__(256) void attention_merge(const float *__restrict__ part, float *__restrict__ out, int d,
                                                         int n_chunks) {
+    extern __shared__ float wch[];  // [n_chunks] rescaling weights, then the total
     const float *pp = part + (size_t)blockIdx.x * n_chunks * (d + 2);
     float mx = -INFINITY;
     for (int ch = 0; ch < n_chunks; ch++) mx = fmaxf(mx, pp[(size_t)ch * (d + 2)]);
-    float tot = 0.0f;
-    for (int ch = 0; ch < n_chunks; ch++) {
+    for (int ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {
         const float l = pp[(size_t)ch * (d + 2) + 1];
-        if (l > 0.0f) tot += l * expf(pp[(size_t)ch * (d + 2)] - mx);
+        wch[ch] = l > 0.0f ? expf(pp[(size_t)ch * (d + 2)] - mx) : 0.0f;
     }
-    for (int c = threadIdx.x; c < d; c += 256) {
+    __syncthreads();
+    float tot = 0.0f;
+    for (int ch = 0; ch < n_chunks; ch++) tot = fmaf(pp[(size_t)ch * (d + 2) + 1], wch[ch], tot);
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
         float a = 0.0f;
-        for (int ch = 0; ch < n_chunks; ch++) {
-            const float l = pp[(size_t)ch * (d + 2) + 1];
-            if (l > 0.0f) a = fmaf(expf(pp[(size_t)ch * (d + 2)] - mx), pp[(size_t)ch * (d + 2) + 2 + c], a);
-        }
+#pragma unroll 4
+        for (int ch = 0; ch < n_chunks; ch++) a = fmaf(wch[ch], pp[(size_t)ch * (d + 2) + 2 + c], a);
         out[(size_t)blockIdx.x * d + c] = a / tot;
     }
 }

@@ -80,6 +80,25 @@ def test_decode_over_several_key_chunks():
         pos += step
 
 
+def test_replacing_a_tensor_after_decoding_takes_effect():
+    """Single-token steps run q|k|v and gate|up as fused launches; a tensor set afterwards must win."""
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(CFG, 27)}
+    m, o = make(CFG, 27)
+    m.forward([5, 6, 7], 0)
+    m.forward([8], 3)                       # builds the fused copies
+    other = {n: (qt, d) for n, qt, d in qwen3_tensors(CFG, 28)}
+    for name in ("blk.1.attn_k.weight", "blk.2.ffn_up.weight"):
+        tensors[name] = other[name]
+        m.set_tensor(name, *other[name])
+    o2 = oq.Qwen3Oracle(CFG, tensors, avx2=oracle.have_avx2())
+    m.reset()
+    ref = o2.forward([5, 6, 7], 0)
+    ok, e = close(m.forward([5, 6, 7], 0), ref)
+    assert ok, e
+    ok, e = close(m.forward([8], 3), o2.forward([8], 3))
+    assert ok, e
+
+
 def test_position_contract_and_reset():
     m, _ = make(CFG, 23)
     a = m.forward([1, 2, 3], 0)
