@@ -1059,7 +1059,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
     hipLaunchKernelGGL(jq::set_int, dim3(1), dim3(1), 0, s, m->pos, (int)pos);
     const float sqrt_d = sqrtf((float)d);
     // few query rows over a long cache: split the keys over the chip
-    const bool split = T <= 8 && d % 64 == 0 && d <= 256;
+    const bool split = T <= 8 && (d == 64 || d == 128 || d == 256);
     const int n_chunks = (int)((pos + T + jq::ATT_CHUNK - 1) / jq::ATT_CHUNK);
     const float *pending = nullptr;  // residual not yet added into x
     for (uint32_t l = 0; l < c.n_layer; l++) {
@@ -1085,8 +1085,13 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, qp, kp, vp, w_qn, w_kn,
                            c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
         if (split) {
-            hipLaunchKernelGGL(jq::attention_split, dim3(T * nh * n_chunks), dim3(256), 0, s, qp, m->kc[l], m->vc[l],
-                               m->part, nh, nkv, d, m->pos, (int)c.n_ctx, sqrt_d, n_chunks);
+#define JQ_ATT_SPLIT(D)                                                                                          \
+    hipLaunchKernelGGL(jq::attention_split<D>, dim3(T * nh * n_chunks), dim3(256), 0, s, qp, m->kc[l], m->vc[l], \
+                       m->part, nh, nkv, m->pos, (int)c.n_ctx, sqrt_d, n_chunks)
+            if (d == 64) JQ_ATT_SPLIT(64);
+            else if (d == 128) JQ_ATT_SPLIT(128);
+            else JQ_ATT_SPLIT(256);
+#undef JQ_ATT_SPLIT
             hipLaunchKernelGGL(jq::attention_merge, dim3(T * nh), dim3(128), n_chunks * sizeof(float), s, m->part, m->att, d,
                                n_chunks);
         } else {

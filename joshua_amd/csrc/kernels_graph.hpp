@@ -150,16 +150,20 @@ __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ 
 // computes its chunk's scores, their maximum m, l = sum exp(s - m) and the unnormalised
 // sum exp(s - m) v, and writes (m, l, acc[d]) to part[(t*n_head + hq)*n_chunks + chunk];
 // attention_merge rescales the chunks to the common maximum and divides by the total.
-// 16 lanes per key (4 keys per wave step), d % 64 == 0.  Chunks past the causal limit
-// write l = 0 and are skipped by the merge.
+// 16 lanes per key (4 keys per wave step), head_dim 64, 128 or 256.  Chunks past the causal
+// limit write l = 0 and are skipped by the merge.
 constexpr int ATT_CHUNK = 64;
 
+template <int D>  // head_dim: 64, 128 or 256
 __global__ __launch_bounds__(256) void attention_split(const float *__restrict__ q, const float *__restrict__ kc,
                                                         const float *__restrict__ vc, float *__restrict__ part,
-                                                        int n_head, int n_kv, int d, const int *__restrict__ pos_ptr,
-                                                        int n_ctx, float sqrt_d, int n_chunks) {
+                                                        int n_head, int n_kv, const int *__restrict__ pos_ptr, int n_ctx,
+                                                        float sqrt_d, int n_chunks) {
+    constexpr int d = D, QI = D / 64;          // float4 of q (and of a key) per lane
+    constexpr int NG = D / 4, KP = 256 / NG;   // column groups of four, key parts
+    constexpr int VI = ATT_CHUNK / KP;         // keys per thread in the value sum
     __shared__ float sc[ATT_CHUNK];
-    __shared__ float4 accs[256];    // [key part][column group of four]
+    __shared__ float4 accs[256];               // [key part][column group]
     const int chunk = blockIdx.x % n_chunks, hq = (blockIdx.x / n_chunks) % n_head, t = blockIdx.x / (n_chunks * n_head);
     const int kvh = hq / (n_head / n_kv), n_keys = *pos_ptr + t + 1;
     const int j0 = chunk * ATT_CHUNK, nj = min(ATT_CHUNK, n_keys - j0);
@@ -171,18 +175,31 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15, kq = lane >> 4;
     const float *qp = q + ((size_t)t * n_head + hq) * d;
     const float *kb = kc + ((size_t)kvh * n_ctx + j0) * d;
-    // this lane's slice of q: floats [4*sub + 64*i, +4), i < d/64
-    float4 qv[4];
-    for (int i = 0; i < d / 64; i++) qv[i] = *(const float4 *)(qp + 4 * sub + 64 * i);
-    for (int j = wave * 4 + kq; j < ATT_CHUNK; j += 16) {
+    const int cg = threadIdx.x % NG, kp = threadIdx.x / NG;
+    const float *vb = vc + ((size_t)kvh * n_ctx + j0) * d + 4 * cg;
+    // every global read of this workgroup is issued here, before any of them is needed: the query slice,
+    // this lane's slices of its four keys, this thread's VI value rows (rows past the chunk's end are
+    // read from its last valid row and not used)
+    float4 qv[QI], kv[4][QI], vv[VI];
+#pragma unroll
+    for (int i = 0; i < QI; i++) qv[i] = *(const float4 *)(qp + 4 * sub + 64 * i);
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int j = min(wave * 4 + kq + 16 * s, nj - 1);
+#pragma unroll
+        for (int i = 0; i < QI; i++) kv[s][i] = *(const float4 *)(kb + (size_t)j * d + 4 * sub + 64 * i);
+    }
+#pragma unroll
+    for (int s = 0; s < VI; s++) vv[s] = *(const float4 *)(vb + (size_t)min(kp + KP * s, nj - 1) * d);
+
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int j = wave * 4 + kq + 16 * s;
         float acc = 0.0f;
-        if (j < nj) {
-            const float *kr = kb + (size_t)j * d;
-            for (int i = 0; i < d / 64; i++) {
-                const float4 kv = *(const float4 *)(kr + 4 * sub + 64 * i);
-                acc = fmaf(qv[i].x, kv.x, acc), acc = fmaf(qv[i].y, kv.y, acc);
-                acc = fmaf(qv[i].z, kv.z, acc), acc = fmaf(qv[i].w, kv.w, acc);
-            }
+#pragma unroll
+        for (int i = 0; i < QI; i++) {
+            acc = fmaf(qv[i].x, kv[s][i].x, acc), acc = fmaf(qv[i].y, kv[s][i].y, acc);
+            acc = fmaf(qv[i].z, kv[s][i].z, acc), acc = fmaf(qv[i].w, kv[s][i].w, acc);
         }
         acc += __shfl_xor(acc, 1, 64), acc += __shfl_xor(acc, 2, 64);
         acc += __shfl_xor(acc, 4, 64), acc += __shfl_xor(acc, 8, 64);
@@ -197,27 +214,21 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
     __syncthreads();
     if (wave == 0) sc[lane] = e;
     __syncthreads();
-    // acc[c] = sum_j e_j v[j, c]: thread (column group of four, key part) strides the keys of its part;
-    // the loads of a thread do not depend on each other, so several are in flight at once
-    const int ngroups = d >> 2, kparts = 256 / ngroups;  // d = 128: 32 groups x 8 parts
-    const int cg = threadIdx.x % ngroups, kp = threadIdx.x / ngroups;
-    const float *vb = vc + ((size_t)kvh * n_ctx + j0) * d + 4 * cg;
+    // acc[c] = sum_j e_j v[j, c]: thread (column group, key part) over the keys kp, kp + KP, ...
     float4 acc = float4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-    for (int j = kp; j < ATT_CHUNK; j += kparts) {
-        if (j < nj) {
-            const float4 v = *(const float4 *)(vb + (size_t)j * d);
-            const float e_j = sc[j];
-            acc.x = fmaf(e_j, v.x, acc.x), acc.y = fmaf(e_j, v.y, acc.y);
-            acc.z = fmaf(e_j, v.z, acc.z), acc.w = fmaf(e_j, v.w, acc.w);
-        }
+#pragma unroll
+    for (int s = 0; s < VI; s++) {
+        const int j = kp + KP * s;
+        const float e_j = j < nj ? sc[j] : 0.0f;
+        acc.x = fmaf(e_j, vv[s].x, acc.x), acc.y = fmaf(e_j, vv[s].y, acc.y);
+        acc.z = fmaf(e_j, vv[s].z, acc.z), acc.w = fmaf(e_j, vv[s].w, acc.w);
     }
-    accs[kp * ngroups + cg] = acc;
+    accs[kp * NG + cg] = acc;
     __syncthreads();
-    if (threadIdx.x < ngroups) {
+    if (threadIdx.x < NG) {
         float4 a = accs[threadIdx.x];
-        for (int pt = 1; pt < kparts; pt++) {
-            const float4 o = accs[pt * ngroups + threadIdx.x];
+        for (int pt = 1; pt < KP; pt++) {
+            const float4 o = accs[pt * NG + threadIdx.x];
             a.x += o.x, a.y += o.y, a.z += o.z, a.w += o.w;
         }
         po[2 + 4 * threadIdx.x + 0] = a.x, po[2 + 4 * threadIdx.x + 1] = a.y;

@@ -63,10 +63,11 @@ def test_prefill_in_two_chunks_matches_one():
     assert ok, e
 
 
-def test_decode_over_several_key_chunks():
+@pytest.mark.parametrize("head_dim,n_head,n_kv", [(64, 4, 2), (128, 4, 1), (256, 2, 2), (192, 4, 2)])
+def test_decode_over_several_key_chunks(head_dim, n_head, n_kv):
     """A cache longer than one 64-key chunk of the split attention kernel, entered both by a
-    long prefill and by short multi-token steps."""
-    cfg = dict(CFG, n_ctx=224, n_layer=2)
+    long prefill and by short multi-token steps; head sizes with and without a split kernel."""
+    cfg = dict(CFG, n_ctx=224, n_layer=2, head_dim=head_dim, n_head=n_head, n_kv_head=n_kv)
     m, o = make(cfg, 26)
     rng = np.random.default_rng(3)
     toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=190)]
