@@ -220,29 +220,32 @@ int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
-// Q4_K, one activation row, rows of at most 16 super-blocks: the integer-dot GEMV.
-// Returns -1 when the shape is outside its reach.
+// Q4_K, one activation row: the integer-dot GEMVs.  By default the LDS-ring kernel takes rows of
+// exactly 16 super-blocks (4096 wide: 10.15 us against 10.27 us for the MFMA GEMV on 14336 rows, and
+// 2 % more decode tokens/s) and everything else is declined (-1).  JQ_Q4K_DOT4 = 0 turns them off,
+// = regs selects the register-prefetch kernel for every row length up to 16 super-blocks.
 int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
     const size_t nb = k / 256;
-    // opt-in (JQ_Q4K_DOT4=1): on the 14336 x 4096 GEMV it streams at the same rate as the MFMA kernel
-    // below once running, but starts and drains more slowly (11.4 us against 10.2 us measured)
-    static const char *on = getenv("JQ_Q4K_DOT4");
-    if (!on || on[0] == '0' || nb == 0 || nb > jq::QD_MAX_WAVES || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 ||
+    static const char *mode_env = getenv("JQ_Q4K_DOT4");
+    static const std::string mode = mode_env ? mode_env : "auto";
+    if (mode == "0" || nb == 0 || nb > jq::QD_MAX_WAVES || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 ||
         ((uintptr_t)X & 15) != 0)
         return -1;
-    static const char *lds_env = getenv("JQ_Q4K_DOT4_LDS");
-    if (lds_env && lds_env[0] != '0' && nb == 16) {
-        static const char *g2 = getenv("JQ_Q4K_DOT4_GRID");
-        const unsigned grid = (unsigned)std::min<size_t>((n + 15) / 16, g2 ? (size_t)atoi(g2) : 256);
+    static const char *genv = getenv("JQ_Q4K_DOT4_GRID");
+    const size_t tiles = (n + 15) / 16;
+    if (mode != "regs") {
+        if (nb != 16) return -1;
+        // a whole number of tiles per workgroup when the chip allows it (224 x 4 at 14336 rows)
+        const size_t rounds = (tiles + 255) / 256;
+        const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)atoi(genv) : (tiles + rounds - 1) / rounds);
         hipLaunchKernelGGL(jq::q4k_gemv_dot4_lds, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
         HIP_TRY(hipGetLastError());
         return 0;
     }
-    static const char *genv = getenv("JQ_Q4K_DOT4_GRID");
     // as many workgroups as the chip holds at once (one of 16 waves per CU, more when smaller), each
     // with an equal share of the rows
     const size_t cap = genv ? (size_t)atoi(genv) : 256 * std::max<size_t>(1, jq::QD_MAX_WAVES / nb);
-    const unsigned grid = (unsigned)std::min<size_t>((n + 15) / 16, std::max<size_t>(cap, 1));
+    const unsigned grid = (unsigned)std::min<size_t>(tiles, std::max<size_t>(cap, 1));
     hipLaunchKernelGGL(jq::q4k_gemv_dot4, dim3(grid), dim3((unsigned)(64 * nb)), 0, s, W, row_bytes, X, Y, (int)k, (int)n);
     HIP_TRY(hipGetLastError());
     return 0;

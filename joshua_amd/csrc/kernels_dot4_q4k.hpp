@@ -165,14 +165,15 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
     __shared__ __attribute__((aligned(16))) float x_raw[16][256];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, c = lane >> 4;
+    // tiles blockIdx.x, blockIdx.x + G, ...: at any moment the chip reads one contiguous stretch of the
+    // matrix (measured 5.4 TB/s against 5.1 TB/s for one contiguous range per workgroup)
     const int G = (int)gridDim.x;
-    const int row_beg = (int)((long long)blockIdx.x * n / G), row_end = (int)((long long)(blockIdx.x + 1) * n / G);
-    const int n_tiles = (row_end - row_beg + 15) >> 4;
-    if (n_tiles == 0) return;
+    const int n_tiles = (((n + 15) >> 4) - (int)blockIdx.x + G - 1) / G;
+    if (n_tiles <= 0) return;
 
     // 3 asynchronous loads per wave and tile: row `wave` of tile i (clamped into the range) -> ring slot
     auto fetch = [&](int i, int slot) __attribute__((always_inline)) {
-        const int row = min(row_beg + 16 * min(i, n_tiles - 1) + wave, row_end - 1);
+        const int row = min(16 * ((int)blockIdx.x + min(i, n_tiles - 1) * G) + wave, n - 1);
         const uint8_t *src = W + (size_t)row * QD_ROW + 16 * lane;
         const uint32_t dst = lds_offset_of(&ring[slot][wave * QD_ROW_LDS]);
         async_load16(src, dst);
@@ -262,8 +263,8 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         {   // wave w sums row w of the tile over the 16 waves
             float v = (lane < 16) ? red[buf][lane][wave] : 0.0f;
             v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
-            const int row = row_beg + 16 * t + wave;
-            if (lane == 0 && row < row_end) Y[row] = v;
+            const int row = 16 * ((int)blockIdx.x + t * G) + wave;
+            if (lane == 0 && row < n) Y[row] = v;
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped fetches of the last two steps

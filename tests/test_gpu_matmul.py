@@ -168,6 +168,15 @@ def test_q4k_integer_dot_products_are_bit_exact(m):
     assert np.array_equal(got, want.astype(np.float32))
 
 
+def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
+    """4096-wide rows, one activation row: the v_dot4 kernel, activation range 32639 per 32-element
+    sub-block."""
+    n, k = 150, 4096
+    blocks, q, x = q4k_integer_case(n, k, 7, group=32, big_value=32639, small=4000)
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+    assert np.array_equal(got[0], (x @ q.T).astype(np.float32))
+
+
 @pytest.mark.parametrize("m", [17, 64, 200])
 def test_q4k_gemm_integer_dot_products_are_bit_exact(m):
     """The same construction for the MFMA GEMM (m > 16): its activation range is 4193279
@@ -347,8 +356,10 @@ from tests.test_gpu_matmul import q4k_integer_case, close
 # exact integers: activation range 32639 per 32-element sub-block
 n, k = 150, 4096
 blocks, q, x = q4k_integer_case(n, k, 7, group=32, big_value=32639, small=4000)
-got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
-assert np.array_equal(got[0], (x @ q.T).astype(np.float32)), "integer case"
+import os
+if os.environ["JQ_Q4K_DOT4"] != "0":
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+    assert np.array_equal(got[0], (x @ q.T).astype(np.float32)), "integer case"
 for (n, k) in [(14336, 4096), (100, 256), (4099, 1024), (33, 3840), (4099, 4096), (7, 4096)]:
     blocks = synth.normal_quantized(capi.Q4_K, 5 + n, n * k, 0.02)
     lhs = synth.normal(6 + k, (1, k))
@@ -358,15 +369,16 @@ print("dot4 ok")
 """
 
 
-@pytest.mark.parametrize("through_lds", ["0", "1"])
-def test_q4k_integer_dot_gemv_when_selected(through_lds):
-    """The v_dot4 GEMV (weights prefetched into registers, or through an LDS ring for 4096-wide rows)
-    is selected by environment variables when the library first dispatches, so it runs in a child
-    process: exact on the integer construction, within tolerance on random shapes (row counts that
-    do not divide over the workgroups, short and 15-block rows)."""
+@pytest.mark.parametrize("mode", ["regs", "0"])
+def test_q4k_gemv_kernels_selected_by_environment(mode):
+    """JQ_Q4K_DOT4 picks the one-row Q4_K kernel when the library first dispatches, so the non-default
+    choices run in a child process: `regs` (v_dot4 with register prefetch, any row up to 4096) must be
+    exact on the integer construction, `0` (the MFMA GEMV also for 4096-wide rows) skips that case;
+    both within tolerance on random shapes (row counts that do not divide over the workgroups, short
+    and 15-block rows)."""
     import subprocess
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, JQ_Q4K_DOT4="1", JQ_Q4K_DOT4_LDS=through_lds)
+    env = dict(os.environ, JQ_Q4K_DOT4=mode)
     res = subprocess.run([sys.executable, "-c", DOT4_CHILD % root], env=env, capture_output=True, text=True, timeout=110)
     assert res.returncode == 0 and "dot4 ok" in res.stdout, res.stdout + res.stderr
