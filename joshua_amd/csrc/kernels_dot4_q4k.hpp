@@ -184,7 +184,7 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
     // is an asynchronous load, counted by hand)
     async_load16(X + 256 * wave + 4 * lane, lds_offset_of(&x_raw[wave][0]));
     fetch(0, 0);
-    fetch(1, 1);
+    fetch(1, 1);  // (a clamped copy of tile 0 when the workgroup has one tile only)
     asm volatile("s_waitcnt vmcnt(6)" ::: "memory");  // the activation landed (own wave's data: no barrier needed)
 
     {
@@ -229,7 +229,8 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
     // on entry to step t: tile t is in LDS and visible (the barrier just passed), tile t+1 in flight
     for (int t = 0; t < n_tiles; t++) {
         const int slot = t % 3;
-        fetch(t + 2, (t + 2) % 3);  // the slot of tile t-1, which every wave finished reading before that barrier
+        const bool more = t + 2 < n_tiles;
+        if (more) fetch(t + 2, (t + 2) % 3);  // the slot of tile t-1, which every wave finished reading before that barrier
 
         const uint8_t *blk = &ring[slot][r * QD_ROW_LDS + wave * 144];
         const uint4 hdr = *(const uint4 *)blk;
@@ -257,7 +258,8 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         const int buf = t & 1;
         if (lane < 16) red[buf][wave][lane] = acc;
         // the partial sums are written and tile t+1 has landed: at most this step's 3 loads stay in flight
-        asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+        if (more) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         {   // wave w sums row w of the tile over the 16 waves
@@ -267,7 +269,6 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
             if (lane == 0 && row < n) Y[row] = v;
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped fetches of the last two steps
 }
 
 }  // namespace jq
