@@ -20,6 +20,7 @@
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
 #include "kernels_moe.hpp"
+#include "kernels_mfma_q4k_ring.hpp"
 #include "kernels_valu.hpp"
 
 namespace {
@@ -273,6 +274,46 @@ int dispatch_q4k_stream(const uint8_t *W, size_t row_bytes, const float *X, floa
     return 0;
 }
 
+// rows x k activations -> one MFMA operand record per (row, 256-element column)
+void launch_q4k_acts_prep(const float *X, size_t rows, size_t k, uint8_t *out, hipStream_t s) {
+    const size_t units = rows * (k / 256);
+    hipLaunchKernelGGL(jq::q4k_acts_prep, dim3((unsigned)((units + 7) / 8)), dim3(256), 0, s, X, (int)rows, (int)k, out);
+}
+
+// Workgroups of the LDS-ring MFMA kernel that fit a compute unit (LDS and the 16 waves of a SIMD group).
+constexpr int ring_wgs_per_cu(int maxnb) { return maxnb == 16 ? 1 : maxnb == 8 ? 2 : 4; }
+
+// Q4_K, 1..16 activation rows, contiguous rows of at most 16 super-blocks: the LDS-ring MFMA kernel.
+// Returns -1 when the shape is outside its reach.
+int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                      hipStream_t s) {
+    const size_t nb = k / 256;
+    static const char *off = getenv("JQ_Q4K_NO_RING");
+    if (off || m > 16 || nb == 0 || nb > 16 || row_bytes != nb * 144 || ((uintptr_t)W & 15) != 0 ||
+        ((uintptr_t)X & 15) != 0 || n > 0x7FFFFFF0ull)
+        return -1;
+    const int maxnb = nb > 8 ? 16 : nb > 4 ? 8 : 4;
+    const size_t tiles = (n + 15) / 16, slots = 256 * (size_t)ring_wgs_per_cu(maxnb);
+    static const char *genv = getenv("JQ_Q4K_RING_GRID");
+    const size_t per = (tiles + slots - 1) / slots;
+    const unsigned grid = genv ? (unsigned)std::max(atoi(genv), 1) : (unsigned)((tiles + per - 1) / per);
+    // the activations as MFMA operand records, in a stream-ordered scratch allocation
+    uint8_t *acts = nullptr;
+    HIP_TRY(hipMallocAsync((void **)&acts, m * nb * jq::QS_REC, s));
+    launch_q4k_acts_prep(X, m, k, acts, s);
+#define JQ_RING(MAXNB)                                                                                              \
+    hipLaunchKernelGGL((jq::q4k_ring_mfma<MAXNB, false, false>), dim3(grid), dim3(64 * (unsigned)nb), 0, s, W, nullptr, \
+                       nullptr, acts, nullptr, nullptr, nullptr, nullptr, Y, (int)m, (int)n)
+    if (maxnb == 16) JQ_RING(16);
+    else if (maxnb == 8) JQ_RING(8);
+    else JQ_RING(4);
+#undef JQ_RING
+    hipError_t launched = hipGetLastError();
+    HIP_TRY(hipFreeAsync(acts, s));
+    HIP_TRY(launched);
+    return 0;
+}
+
 // Q4_K with more than 16 activation rows: prepare the fixed-point activation planes in a
 // stream-ordered scratch allocation, then the MFMA GEMM.
 int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
@@ -314,6 +355,12 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     }
     // one or two activation rows: the int8 GEMV below is faster; from three on the streaming kernel,
     // whose time hardly depends on the row count
+    // 3 to 16 rows against a very long matrix (a vocabulary projection): the LDS-ring kernel, whose
+    // two launches and scratch allocation only pay off from some 100 us of streaming on
+    if (type == JQ_TYPE_Q4_K && m > 2 && m <= Q4K_MFMA_MAX_M && n >= 32768) {
+        const int rc = dispatch_q4k_ring(W, row_bytes, X, Y, m, k, n, s);
+        if (rc >= 0) return rc;
+    }
     if (type == JQ_TYPE_Q4_K && m > 2 && m <= Q4K_MFMA_MAX_M) {
         const int rc = dispatch_q4k_stream(W, row_bytes, X, Y, m, k, n, s);
         if (rc >= 0) return rc;
@@ -553,6 +600,7 @@ struct jq_moe {
     float *sG = nullptr, *sU = nullptr, *sH = nullptr, *sOut = nullptr;
     uint32_t *ids = nullptr;
     int *gexp = nullptr, *offsets = nullptr, *xrow = nullptr, *yrow = nullptr;
+    uint8_t *qacts = nullptr;  // activations as MFMA operand records (Q4_K experts, grouped path)
     std::mutex mu;
 };
 
@@ -561,8 +609,9 @@ namespace {
 void moe_free_scratch(jq_moe *m) {
     for (void *p : {(void *)m->logits, (void *)m->wts, (void *)m->G, (void *)m->U, (void *)m->out, (void *)m->sG,
                     (void *)m->sU, (void *)m->sH, (void *)m->sOut, (void *)m->ids, (void *)m->gexp,
-                    (void *)m->offsets, (void *)m->xrow, (void *)m->yrow})
+                    (void *)m->offsets, (void *)m->xrow, (void *)m->yrow, (void *)m->qacts})
         if (p) (void)hipFree(p);
+    m->qacts = nullptr;
     m->logits = m->wts = m->G = m->U = m->out = m->sG = m->sU = m->sH = m->sOut = nullptr;
     m->ids = nullptr;
     m->gexp = m->offsets = m->xrow = m->yrow = nullptr;
@@ -585,6 +634,8 @@ int moe_reserve(jq_moe *m, size_t T) {
     HIP_TRY(hipMalloc((void **)&m->offsets, (groups + 1) * sizeof(int)));
     HIP_TRY(hipMalloc((void **)&m->xrow, PR * sizeof(int)));
     HIP_TRY(hipMalloc((void **)&m->yrow, PR * sizeof(int)));
+    if (m->gate->type == JQ_TYPE_Q4_K || m->down->type == JQ_TYPE_Q4_K)
+        HIP_TRY(hipMalloc((void **)&m->qacts, std::max(T * (c.hidden / 256), PR * (c.inter / 256)) * jq::QS_REC + 16));
     if (m->sgate) {
         size_t si = m->sgate->n;
         HIP_TRY(hipMalloc((void **)&m->sG, T * si * sizeof(float)));
@@ -660,6 +711,33 @@ int dispatch_moe_staged(uint32_t type, const uint8_t *const *Wa, const uint8_t *
     return rc;
 }
 
+// Q4_K experts with several tokens per group: the LDS-ring MFMA kernel per group.
+// Returns -1 when the shape is outside its reach.
+template <bool DUAL>
+int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
+                          const float *X, size_t x_rows, uint8_t *acts, const int *gexp, const int *offsets,
+                          const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s) {
+    const int nb = k / 256;
+    static const char *off = getenv("JQ_MOE_NO_RING");
+    if (off || !acts || k % 256 != 0 || nb == 0 || nb > 16 || row_bytes != (size_t)nb * 144 || !aligned16 ||
+        ((uintptr_t)X & 15) != 0)
+        return -1;
+    launch_q4k_acts_prep(X, x_rows, (size_t)k, acts, s);
+    const int maxnb = nb > 8 ? 16 : nb > 4 ? 8 : 4, n_tiles = (n + 15) / 16;
+    static const char *genv = getenv("JQ_MOE_RING_GRID");
+    const int per_group = genv ? atoi(genv) : 1024 / std::max(groups, 1);
+    dim3 grid((unsigned)std::min(n_tiles, std::max(per_group, 1)), (unsigned)groups), block(64 * nb);
+#define JQ_RING(MAXNB)                                                                                             \
+    hipLaunchKernelGGL((jq::q4k_ring_mfma<MAXNB, true, DUAL>), grid, block, 0, s, nullptr, Wa, Wb, acts, gexp,     \
+                       offsets, xsel, yrow, Y, 0, n)
+    if (maxnb == 16) JQ_RING(16);
+    else if (maxnb == 8) JQ_RING(8);
+    else JQ_RING(4);
+#undef JQ_RING
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 template <bool SWIGLU>
 int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2,
                       const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
@@ -685,8 +763,9 @@ int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_byte
 
 int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg) {
     const jq_moe_config &c = m->cfg;
-    hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert), dim3(256), 0, s, m->router_w, x, m->logits, (int)T,
-                       (int)c.hidden, (int)c.n_expert);
+    const unsigned token_runs = (unsigned)((T + jq::ROUTER_TOKENS_PER_WG - 1) / jq::ROUTER_TOKENS_PER_WG);
+    hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert, token_runs), dim3(256), 0, s, m->router_w, x, m->logits,
+                       (int)T, (int)c.hidden, (int)c.n_expert);
     jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
                          (int)c.n_group, (int)c.topk_group};
     size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);
@@ -709,7 +788,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         groups = (int)c.n_expert + extra;
         max_group = (int)T;
         const int in_lds = (size_t)P <= 12288;
-        hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(256), (c.n_expert + 1 + (in_lds ? P : 0)) * sizeof(int), s,
+        hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(jq::GROUP_PAIRS_THREADS), (c.n_expert + 1 + (in_lds ? P : 0)) * sizeof(int), s,
                            m->ids, (int)T, (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow,
                            extra, in_lds);
     }
@@ -718,7 +797,12 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     const bool a16 = ((uintptr_t)m->gate->dev & 15) == 0 && ((uintptr_t)m->up->dev & 15) == 0 &&
                      (!m->fold_shared || (((uintptr_t)m->sgate->dev & 15) == 0 && ((uintptr_t)m->sup->dev & 15) == 0));
     int rc = -1;
-    if (m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes)
+    const bool same_gu = m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes;
+    if (same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K)
+        rc = dispatch_moe_q4k_ring<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qacts, m->gexp, m->offsets,
+                                         m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s);
+    if (rc > 0) return 1;
+    if (rc < 0 && same_gu)
         rc = dispatch_moe_staged<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, m->gexp, m->offsets,
                                        m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s);
     if (rc > 0) return 1;
@@ -732,10 +816,16 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
             return 1;
     }
     const bool d16 = ((uintptr_t)m->down->dev & 15) == 0 && (!m->fold_shared || ((uintptr_t)m->sdown->dev & 15) == 0);
-    rc = fused_act ? dispatch_moe_staged<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G, m->gexp,
-                                                m->offsets, m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups,
-                                                max_group, s)
-                   : -1;
+    rc = -1;
+    if (fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K)
+        rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
+                                          m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
+                                          (int)c.hidden, groups, s);
+    if (rc > 0) return 1;
+    if (rc < 0 && fused_act)
+        rc = dispatch_moe_staged<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G, m->gexp,
+                                        m->offsets, m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups,
+                                        max_group, s);
     if (rc > 0) return 1;
     if (rc < 0) {
         if (fused_act) {  // G already holds the activation: plain rows over it

@@ -111,11 +111,42 @@ __global__ __launch_bounds__(256) void q4k_gemm_prep(const float *__restrict__ x
     }
 }
 
-// (sc * q) of the nibbles sitting in bits 0-3 and 16-19 of `two`, as two f16.
-__device__ __forceinline__ uint32_t qg_scaled_h2(uint32_t two, uint32_t sc) {
-    const uint32_t bits = (two * sc) | 0x64006400u;  // f16 of 1024 + sc q, sc q <= 945
-    const qg_h2 v = __builtin_bit_cast(qg_h2, bits) - qg_h2{(_Float16)1024.0f, (_Float16)1024.0f};
+// sc * q of two nibbles of `word`, as two exact f16, in two instructions and without moving the
+// nibbles: OR-ing the f16 exponent of 16 over the masked word makes a nibble in bits 0-3 (16-19)
+// the f16 16 + q/64, one in bits 4-7 (20-23) the f16 16 + q/4; a packed fused multiply-add with
+// (64 sc, -1024 sc), respectively (4 sc, -64 sc), leaves sc q (at most 945; every operand is an f16
+// integer, the exact result is representable, the fma rounds once).
+struct QgScaleOps {
+    qg_h2 lo, hi;  // for the nibbles in bits 0-3 / 4-7 of the bytes
+};
+
+__device__ __forceinline__ qg_h2 qg_scale_operand(uint32_t sc, float mul, float add) {
+    const _Float16 s = (_Float16)(unsigned short)sc;
+    return qg_h2{s * (_Float16)mul, s * (_Float16)add};
+}
+__device__ __forceinline__ qg_h2 qg_scale_operand_lo(uint32_t sc) { return qg_scale_operand(sc, 64.0f, -1024.0f); }
+__device__ __forceinline__ qg_h2 qg_scale_operand_hi(uint32_t sc) { return qg_scale_operand(sc, 4.0f, -64.0f); }
+
+// (word & mask) | 0x4C004C00 in one instruction: the mask in a vector register, the constant in a scalar one
+__device__ __forceinline__ uint32_t qg_mask_exp(uint32_t word, uint32_t mask) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(word), "v"(mask), "s"(0x4C004C00u));
+    return r;
+}
+
+__device__ __forceinline__ uint32_t qg_scaled_h2(uint32_t word, uint32_t mask, qg_h2 op) {
+    const qg_h2 h = __builtin_bit_cast(qg_h2, qg_mask_exp(word, mask));
+    const qg_h2 v = __builtin_elementwise_fma(h, qg_h2{op.x, op.x}, qg_h2{op.y, op.y});
     return __builtin_bit_cast(uint32_t, v);
+}
+
+// The 8 nibble bytes w0, w1 of a lane -> the MFMA A operands of the low-nibble and high-nibble
+// sub-block, element order 0,2,1,3,4,6,5,7.
+__device__ __forceinline__ void qg_unpack_words(uint32_t w0, uint32_t w1, qg_h2 op_lo, qg_h2 op_hi, qg_u4 &lo, qg_u4 &hi) {
+    const uint32_t s0 = w0 >> 8, s1 = w1 >> 8;
+    const uint32_t ml = 0x000F000Fu, mh = 0x00F000F0u;
+    lo = qg_u4{qg_scaled_h2(w0, ml, op_lo), qg_scaled_h2(s0, ml, op_lo), qg_scaled_h2(w1, ml, op_lo), qg_scaled_h2(s1, ml, op_lo)};
+    hi = qg_u4{qg_scaled_h2(w0, mh, op_hi), qg_scaled_h2(s0, mh, op_hi), qg_scaled_h2(w1, mh, op_hi), qg_scaled_h2(s1, mh, op_hi)};
 }
 
 // Asynchronous global -> LDS load: every active lane fetches `bytes` (4 or 16) from its own global
@@ -253,10 +284,8 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
         const uint2 raw = *(const uint2 *)(r_slot(S) + ar * 8 + aq * 2);
         const uint32_t w0 = raw.x, w1 = raw.y;
         // operand order within the 8 k of a lane: 0,2,1,3,4,6,5,7
-        const qg_u4 lo = qg_u4{qg_scaled_h2(w0 & 0x000F000Fu, sc_lo), qg_scaled_h2((w0 >> 8) & 0x000F000Fu, sc_lo),
-                               qg_scaled_h2(w1 & 0x000F000Fu, sc_lo), qg_scaled_h2((w1 >> 8) & 0x000F000Fu, sc_lo)};
-        const qg_u4 hi = qg_u4{qg_scaled_h2((w0 >> 4) & 0x000F000Fu, sc_hi), qg_scaled_h2((w0 >> 12) & 0x000F000Fu, sc_hi),
-                               qg_scaled_h2((w1 >> 4) & 0x000F000Fu, sc_hi), qg_scaled_h2((w1 >> 12) & 0x000F000Fu, sc_hi)};
+        qg_u4 lo, hi;
+        qg_unpack_words(w0, w1, qg_scale_operand_lo(sc_lo), qg_scale_operand_hi(sc_hi), lo, hi);
         qg_u4 *ab = a_lds + (c & 1) * QG_A_U4;
         const int tile = ar >> 4, ol = (ar & 15) + 16 * aq;
         ab[(0 * 8 + tile) * 64 + ol] = lo;   // sub-block 2cc   -> k step 0

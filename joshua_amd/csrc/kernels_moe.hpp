@@ -10,19 +10,23 @@ namespace jq {
 
 // logits[t, e] = x[t, :] . router[e, :]   (reference: src/quantized_qwen3_moe.rs:425,
 // src/quantized_deepseek2.rs:528; an f32 matmul there too)
+constexpr int ROUTER_TOKENS_PER_WG = 8;
+
 __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict__ Wr, const float *__restrict__ X,
                                                           float *__restrict__ logits, int T, int h, int E) {
-    // one workgroup per expert row of the router: every load of the row in flight at once
+    // one workgroup per (expert row of the router, run of 8 tokens): every load of the row in
+    // flight at once; a logit's arithmetic does not depend on how the tokens are split
     __shared__ float red[4][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, e = blockIdx.x;
     const float *wr = Wr + (size_t)e * h;
-    for (int t0 = 0; t0 < T; t0 += 4) {
+    const int t_begin = blockIdx.y * ROUTER_TOKENS_PER_WG, t_end = min(T, t_begin + ROUTER_TOKENS_PER_WG);
+    for (int t0 = t_begin; t0 < t_end; t0 += 4) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
         for (int c = threadIdx.x * 4; c < h; c += 1024) {
             const float4 w = ld<float4>((const uint8_t *)(wr + c));
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                if (t0 + i < T) {
+                if (t0 + i < t_end) {
                     const float4 x = ld<float4>((const uint8_t *)(X + (size_t)(t0 + i) * h + c));
                     acc[i] = fmaf(x.x, w.x, acc[i]);
                     acc[i] = fmaf(x.y, w.y, acc[i]);
@@ -37,7 +41,7 @@ __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict
             if (lane == 0) red[wave][i] = s;
         }
         __syncthreads();
-        if (threadIdx.x < 4 && t0 + threadIdx.x < T)
+        if (threadIdx.x < 4 && t0 + threadIdx.x < t_end)
             logits[(size_t)(t0 + threadIdx.x) * E + e] =
                 (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
         __syncthreads();
@@ -162,27 +166,45 @@ __global__ __launch_bounds__(256) void moe_gate_topk(const float *__restrict__ l
 // src/quantized_qwen3_moe.rs:459-480).  Group e is expert e:
 //   offsets[e] .. offsets[e+1]  positions of the expert's pairs
 //   xrow[pos]  activation row (token) of the pair,  yrow[pos]  the pair index
-__global__ __launch_bounds__(256) void moe_group_pairs(const uint32_t *__restrict__ ids, int T, int k_used, int E,
-                                                       int *__restrict__ gexp, int *__restrict__ offsets,
-                                                       int *__restrict__ xrow, int *__restrict__ yrow,
-                                                       int shared_group, int ids_in_lds) {
+constexpr int GROUP_PAIRS_THREADS = 1024;
+
+__global__ __launch_bounds__(GROUP_PAIRS_THREADS) void moe_group_pairs(const uint32_t *__restrict__ ids, int T,
+                                                                       int k_used, int E, int *__restrict__ gexp,
+                                                                       int *__restrict__ offsets,
+                                                                       int *__restrict__ xrow, int *__restrict__ yrow,
+                                                                       int shared_group, int ids_in_lds) {
     extern __shared__ int cnt[];  // [E + 1], then the pair list [P] when ids_in_lds
     const int P = T * k_used;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    uint32_t *ids_lds = (uint32_t *)(cnt + E + 1);
     for (int e = threadIdx.x; e <= E; e += blockDim.x) cnt[e] = 0;
     __syncthreads();
     for (int pidx = threadIdx.x; pidx < P; pidx += blockDim.x) {
         const uint32_t e = ids[pidx];
+        if (ids_in_lds) ids_lds[pidx] = e;
         if (e < (uint32_t)E) atomicAdd(&cnt[e], 1);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int run = 0;
-        for (int e = 0; e < E; e++) {
-            const int c = cnt[e];
-            cnt[e] = run;
-            run += c;
+    if (wave == 0) {  // counts -> start positions: each lane a run of experts, a wave scan between the runs
+        const int per = (E + 63) / 64, b = lane * per;
+        int local = 0;
+        for (int i = 0; i < per; i++)
+            if (b + i < E) local += cnt[b + i];
+        int incl = local;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
         }
-        cnt[E] = run;
+        int run = incl - local;
+        for (int i = 0; i < per; i++) {
+            if (b + i < E) {
+                const int c = cnt[b + i];
+                cnt[b + i] = run;
+                run += c;
+            }
+        }
+        if (lane == 63) cnt[E] = incl;
     }
     __syncthreads();
     for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = cnt[e];
@@ -190,22 +212,22 @@ __global__ __launch_bounds__(256) void moe_group_pairs(const uint32_t *__restric
         if (threadIdx.x == 0) gexp[E] = E, offsets[E + 1] = P + T;
         for (int t = threadIdx.x; t < T; t += blockDim.x) xrow[P + t] = t, yrow[P + t] = P + t;
     }
-    // every expert's thread scans the pair list in order: from the LDS copy when it fits
-    uint32_t *ids_lds = (uint32_t *)(cnt + E + 1);
-    if (ids_in_lds) {
-        for (int pidx = threadIdx.x; pidx < P; pidx += blockDim.x) ids_lds[pidx] = ids[pidx];
-        __syncthreads();
-    }
+    // a wave per expert walks the pair list 64 pairs at a time, in order (from the LDS copy when
+    // it fits): a pair's place is the expert's start + the matches before it
     const uint32_t *scan = ids_in_lds ? ids_lds : ids;
-    for (int e = threadIdx.x; e < E; e += blockDim.x) {
-        gexp[e] = e;
+    for (int e = wave; e < E; e += waves) {
+        if (lane == 0) gexp[e] = e;
         int pos = cnt[e];
-        for (int pidx = 0; pidx < P; pidx++) {
-            if (scan[pidx] == (uint32_t)e) {
-                xrow[pos] = pidx / k_used;
-                yrow[pos] = pidx;
-                pos++;
+        for (int base = 0; base < P; base += 64) {
+            const int pidx = base + lane;
+            const bool hit = pidx < P && scan[pidx] == (uint32_t)e;
+            const unsigned long long mask = __ballot(hit);
+            if (hit) {
+                const int at = pos + __popcll(mask & ((1ull << lane) - 1ull));
+                xrow[at] = pidx / k_used;
+                yrow[at] = pidx;
             }
+            pos += __popcll(mask);
         }
     }
 }

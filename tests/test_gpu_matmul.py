@@ -168,6 +168,26 @@ def test_q4k_integer_dot_products_are_bit_exact(m):
     assert np.array_equal(got, want.astype(np.float32))
 
 
+@pytest.mark.parametrize("m,k,n", [(16, 4096, 32768 + 5), (3, 768, 32800), (7, 1280, 33000), (4, 256, 32768)])
+def test_q4k_few_rows_against_a_very_long_matrix(m, k, n):
+    """From 32768 weight rows on, 3 to 16 activation rows take the LDS-ring MFMA kernel; rows of 16, 3,
+    5 and 1 super-blocks change how its waves share the copying of a tile."""
+    blocks = make_blocks(capi.Q4_K, n, k, 23)
+    lhs = synth.normal(24 + m, (m, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+def test_q4k_ring_kernel_integer_dot_products_are_bit_exact():
+    n, k, m = 32768 + 16, 512, 5
+    blocks, q, x = q4k_integer_case(n, k, 77, group=256, big_value=4193279, small=4000)
+    lhs = np.stack([np.roll(x, 256 * i) for i in range(m)])
+    want = lhs @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs.astype(np.float32))
+    assert np.array_equal(got, want.astype(np.float32))
+
+
 def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
     """4096-wide rows, one activation row: the v_dot4 kernel, activation range 32639 per 32-element
     sub-block."""

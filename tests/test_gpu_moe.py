@@ -83,6 +83,23 @@ def test_shared_expert_of_another_width_runs_beside_the_groups():
         assert close(dev.forward(x), ora.forward(x))
 
 
+def test_q4k_groups_of_many_tokens_with_the_shared_expert_folded_in():
+    """40 tokens: the shared expert's group holds all 40 (three passes of 16 in the grouped MFMA
+    kernel), routed groups hold 0 to about 20."""
+    ora, dev = build(capi.Q4_K, 1024, 768, 8, 2, 95, shared_inter=768, gating="sigmoid")
+    x = synth.normal(96, (40, 1024))
+    assert close(dev.forward(x), ora.forward(x))
+
+
+@pytest.mark.parametrize("h,inter", [(4096, 256), (512, 2560), (256, 3072)])
+def test_q4k_grouped_kernels_at_other_row_lengths(h, inter):
+    """16-super-block gate/up rows (outside the fused MFMA kernel's reach), and down rows of 10 and
+    12 super-blocks (two columns a wave)."""
+    ora, dev = build(capi.Q4_K, h, inter, 4, 2, 97 + inter)
+    x = synth.normal(98, (19, h))
+    assert close(dev.forward(x), ora.forward(x))
+
+
 @pytest.mark.parametrize("qtype,h,inter", [
     (capi.Q6_K, 768, 256),      # 630-byte rows: no aligned staging, plain kernels; 256-wide down rows: 16 lanes a row
     (capi.IQ2_XXS, 2560, 512),  # 660-byte rows: 4-byte staging
