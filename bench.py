@@ -30,9 +30,9 @@ N, K = 14336, 4096
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs
 # of this benchmark, each scaled by what the same counter reads for joshua_amd/calib/copy_kernel (a plain
-# copy of 33 030 144 bytes): FETCH_SIZE 16253.0 x 1.9987 KiB + WRITE_SIZE 56.0 x 1.0 KiB.  Only quoted for
-# the configuration it was measured on (M = 1).
-MEASURED_TRAFFIC_BYTES_M1 = 33_322_000
+# copy of 33 030 144 bytes): FETCH_SIZE 16223.0 x 1.9987 KiB + WRITE_SIZE 56.0 x 1.0 KiB.  Only quoted for
+# the configuration it was measured on (M = 1, the v_dot4 LDS-ring kernel).
+MEASURED_TRAFFIC_BYTES_M1 = 33_260_000
 SEED_W, SEED_X = 102, 202
 
 
@@ -347,7 +347,11 @@ def main() -> int:
         "metric": "Q4_K GEMV HBM GB/s (% of peak); decode tokens/s, 1 MI355X",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        # one row: 4-bit weights x two int8 activation planes on v_dot4 (int32 sums), f32 scales and result
+        "dtype": "int8" if m == 1 else "f16", "dtype_note": "integer dot products per 32-element sub-block "
+        "(int4 weights x 15-bit fixed-point activations in two int8 planes), f32 scales and accumulation across sub-blocks"
+        if m == 1 else "f16 MFMA on exact integers (scale x nibble, 23-bit fixed-point activations in two planes), f32 result",
+        "data": "synthetic",
         "config": {"workload": f"Q4_K matmul_t {N}x{K} (Llama-3-8B FFN-up), M={m}, f32 activations N(0,1), "
                                f"weights N(0,0.02) quantized to Q4_K, {len(weights)} weight copies rotated (cold HBM)",
                    "launch": mode},
