@@ -225,7 +225,9 @@ int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
 // exactly 16 super-blocks (4096 wide: 10.15 us against 10.27 us for the MFMA GEMV on 14336 rows, and
 // 2 % more decode tokens/s) and everything else is declined (-1).  JQ_Q4K_DOT4 = 0 turns them off,
 // = regs selects the register-prefetch kernel for every row length up to 16 super-blocks.
-int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
+// `norm`: residual add + RMSNorm in front of the product (only the LDS-ring kernel has that form).
+int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s,
+                      const jq::QdNorm *norm = nullptr) {
     const size_t nb = k / 256;
     static const char *mode_env = getenv("JQ_Q4K_DOT4");
     static const std::string mode = mode_env ? mode_env : "auto";
@@ -235,14 +237,18 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     static const char *genv = getenv("JQ_Q4K_DOT4_GRID");
     const size_t tiles = (n + 15) / 16;
     if (mode != "regs") {
-        if (nb != 16) return -1;
+        if (nb != 16 || row_bytes != jq::QD_ROW) return -1;
         // a whole number of tiles per workgroup when the chip allows it (224 x 4 at 14336 rows)
         const size_t rounds = (tiles + 255) / 256;
         const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)atoi(genv) : (tiles + rounds - 1) / rounds);
-        hipLaunchKernelGGL(jq::q4k_gemv_dot4_lds, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+        if (norm)
+            hipLaunchKernelGGL(jq::q4k_gemv_dot4_lds<true>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, *norm);
+        else
+            hipLaunchKernelGGL(jq::q4k_gemv_dot4_lds<false>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, jq::QdNorm{});
         HIP_TRY(hipGetLastError());
         return 0;
     }
+    if (norm) return -1;
     // as many workgroups as the chip holds at once (one of 16 waves per CU, more when smaller), each
     // with an equal share of the rows
     const size_t cap = genv ? (size_t)atoi(genv) : 256 * std::max<size_t>(1, jq::QD_MAX_WAVES / nb);
@@ -1007,6 +1013,7 @@ struct jq_model {
     uint32_t *ids = nullptr, *pick = nullptr;
     int *pos = nullptr;       // device copy of the position of the step being run
     float *part = nullptr;    // split-attention partials
+    float *x2 = nullptr;      // second residual row of a single-token step (the fused norm + matmul launches alternate)
     float *x = nullptr, *hn = nullptr, *qb = nullptr, *kb = nullptr, *vb = nullptr, *att = nullptr, *proj = nullptr,
           *g = nullptr, *u = nullptr, *mid = nullptr, *logits = nullptr;
     std::mutex mu;
@@ -1015,10 +1022,11 @@ struct jq_model {
 namespace {
 
 void model_free_scratch(jq_model *m) {
-    for (void *p : {(void *)m->ids, (void *)m->x, (void *)m->hn, (void *)m->qb, (void *)m->kb, (void *)m->vb,
+    for (void *p : {(void *)m->ids, (void *)m->x, (void *)m->x2, (void *)m->hn, (void *)m->qb, (void *)m->kb, (void *)m->vb,
                     (void *)m->att, (void *)m->proj, (void *)m->g, (void *)m->u, (void *)m->mid})
         if (p) (void)hipFree(p);
     m->ids = nullptr;
+    m->x2 = nullptr;
     m->x = m->hn = m->qb = m->kb = m->vb = m->att = m->proj = m->g = m->u = m->mid = nullptr;
     m->cap_tokens = 0;
 }
@@ -1030,6 +1038,7 @@ int model_reserve(jq_model *m, size_t T) {
     size_t qd = (size_t)c.n_head * c.head_dim, kd = (size_t)c.n_kv_head * c.head_dim;
     HIP_TRY(hipMalloc((void **)&m->ids, T * sizeof(uint32_t)));
     HIP_TRY(hipMalloc((void **)&m->x, T * c.hidden * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->x2, c.hidden * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->hn, T * c.hidden * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->qb, T * qd * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->kb, T * kd * sizeof(float)));
@@ -1143,6 +1152,16 @@ int model_prepare_fused(jq_model *m) {
 
 unsigned grid_for(size_t total) { return (unsigned)std::min<size_t>((total + 255) / 256, 8192); }
 
+// x_out = x + res; y = W rmsnorm(x_out) as one launch (hn_out also gets the normalised row when
+// given).  False when no kernel has that form for this weight: the caller then runs the two steps.
+bool model_norm_mm(const jq_weight *w, const float *x, const float *res, const float *norm_w, float eps, float *x_out,
+                   float *hn_out, float *y, hipStream_t s) {
+    static const char *off = getenv("JQ_NO_FUSED_NORM");
+    if (off || w->type != JQ_TYPE_Q4_K) return false;
+    const jq::QdNorm nm{res, norm_w, eps, x_out, hn_out};
+    return dispatch_q4k_dot4(w->dev, w->row_bytes, x, y, w->k, w->n, s, &nm) == 0;
+}
+
 int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
     const jq_qwen3_config &c = m->cfg;
     const int d = (int)c.head_dim, nh = (int)c.n_head, nkv = (int)c.n_kv_head, h = (int)c.hidden;
@@ -1155,20 +1174,26 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
     const bool split = T <= 8 && (d == 64 || d == 128 || d == 256);
     const int n_chunks = (int)((pos + T + jq::ATT_CHUNK - 1) / jq::ATT_CHUNK);
     const float *pending = nullptr;  // residual not yet added into x
+    float *xc = m->x, *xo = m->x2;   // the residual stream, and where a fused norm + matmul launch writes its update
     for (uint32_t l = 0; l < c.n_layer; l++) {
         const std::string p = "blk." + std::to_string(l);
         const float *w_an, *w_fn, *w_qn, *w_kn;
         if (model_vec(m, p + ".attn_norm.weight", &w_an) || model_vec(m, p + ".ffn_norm.weight", &w_fn) ||
             model_vec(m, p + ".attn_q_norm.weight", &w_qn) || model_vec(m, p + ".attn_k_norm.weight", &w_kn))
             return 1;
-        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, m->x, pending, w_an, c.rms_eps, m->hn, h);
         float *qp = m->qb, *kp = m->kb, *vp = m->vb;
         auto fq = T == 1 ? m->fused.find(p + ".qkv") : m->fused.end();
+        const bool v_fused = fq != m->fused.end() && fq->second->n == (size_t)(nh + 2 * nkv) * d;
+        // single token: residual add, norm and q|k(|v) as one launch when the kernel has that form
+        const bool normed = fq != m->fused.end() &&
+                            model_norm_mm(fq->second, xc, pending, w_an, c.rms_eps, xo, v_fused ? nullptr : m->hn, m->cat, s);
+        if (normed) std::swap(xc, xo);
+        else hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, pending, w_an, c.rms_eps, m->hn, h);
         if (fq != m->fused.end()) {  // one launch for q|k(|v) of a single token
             const jq_weight *w = fq->second;
-            if (dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
+            if (!normed && dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
             qp = m->cat, kp = m->cat + (size_t)nh * d;
-            if (w->n == (size_t)(nh + 2 * nkv) * d) vp = kp + (size_t)nkv * d;
+            if (v_fused) vp = kp + (size_t)nkv * d;
             else if (model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s)) return 1;
         } else if (model_mm(m, p + ".attn_q.weight", m->hn, m->qb, T, s) ||
                    model_mm(m, p + ".attn_k.weight", m->hn, m->kb, T, s) ||
@@ -1193,12 +1218,15 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
                                nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
         }
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
-        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, m->x, m->proj, w_fn, c.rms_eps, m->hn, h);
         const float *gp = m->g, *up = m->u;
         auto fg = T == 1 ? m->fused.find(p + ".gate_up") : m->fused.end();
+        const bool normed2 = fg != m->fused.end() &&
+                             model_norm_mm(fg->second, xc, m->proj, w_fn, c.rms_eps, xo, nullptr, m->cat, s);
+        if (normed2) std::swap(xc, xo);
+        else hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, m->proj, w_fn, c.rms_eps, m->hn, h);
         if (fg != m->fused.end()) {
             const jq_weight *w = fg->second;
-            if (dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
+            if (!normed2 && dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
             gp = m->cat, up = m->cat + c.ffn;
         } else if (model_mm(m, p + ".ffn_gate.weight", m->hn, m->g, T, s) ||
                    model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s)) {
@@ -1213,7 +1241,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
     if (model_vec(m, "output_norm.weight", &w_on)) return 1;
     // logits only for the last position (reference: src/quantized_qwen3_moe.rs:816-818)
     const size_t last = (size_t)(T - 1) * h;
-    hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(1), dim3(1024), 0, s, m->x + last, pending ? pending + last : nullptr, w_on,
+    hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(1), dim3(1024), 0, s, xc + last, pending ? pending + last : nullptr, w_on,
                        c.rms_eps, m->hn, h);
     // tie_word_embeddings conversions ship no output head (src/quantized_qwen3_moe.rs:739-743)
     const char *head = m->q.count("output.weight") ? "output.weight" : "token_embd.weight";

@@ -156,9 +156,23 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
 // access is a contiguous kilobyte.  Needs exactly 16 super-blocks a row (one wave per row of a tile).
 constexpr int QD_ROW = 16 * 144, QD_ROW_LDS = QD_ROW + 16, QD_TILE_LDS = 16 * QD_ROW_LDS;
 
+// NORM puts a residual add and an RMSNorm in front of the product (a decoder layer's
+// x += res; hn = x / sqrt(mean(x^2) + eps) * w; y = W hn as one launch): every workgroup normalises
+// the 4096-wide row for itself, workgroup 0 also stores x + res (into a buffer other than X: the
+// others are still reading X) and, when asked, the normalised row.
+struct QdNorm {
+    const float *res;  // added to X first (null: nothing to add)
+    const float *w;    // norm weight
+    float eps;
+    float *x_out;      // X + res
+    float *hn_out;     // the normalised row (null: not wanted)
+};
+
+template <bool NORM>
 __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                          float *__restrict__ Y, int n) {
+                                                          float *__restrict__ Y, int n, QdNorm nm) {
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][QD_TILE_LDS];
+    __shared__ float ss_lds[16];
     __shared__ uint32_t xl_lds[16][64], xh_lds[16][64];
     __shared__ float s_lds[16][8], xs_lds[16][8];
     __shared__ float red[2][16][16];
@@ -183,12 +197,39 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
     // the activation column of this wave travels the same way, first (every global read of this kernel
     // is an asynchronous load, counted by hand)
     async_load16(X + 256 * wave + 4 * lane, lds_offset_of(&x_raw[wave][0]));
+    // norm weight and residual columns wait in the third ring slot, which no tile enters before the main loop
+    float *w_raw = (float *)&ring[2][0] + 256 * wave, *r_raw = (float *)&ring[2][16384] + 256 * wave;
+    if (NORM) {
+        async_load16(nm.w + 256 * wave + 4 * lane, lds_offset_of(w_raw));
+        if (nm.res) async_load16(nm.res + 256 * wave + 4 * lane, lds_offset_of(r_raw));
+    }
     fetch(0, 0);
     fetch(1, 1);  // (a clamped copy of tile 0 when the workgroup has one tile only)
     asm volatile("s_waitcnt vmcnt(6)" ::: "memory");  // the activation landed (own wave's data: no barrier needed)
 
     {
-        const float4 v = *(const float4 *)&x_raw[wave][4 * lane];
+        float4 v = *(const float4 *)&x_raw[wave][4 * lane];
+        if (NORM) {
+            if (nm.res) {
+                const float4 r = *(const float4 *)&r_raw[4 * lane];
+                v.x += r.x, v.y += r.y, v.z += r.z, v.w += r.w;
+            }
+            float ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w)));
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+            if (lane == 0) ss_lds[wave] = ss;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            float tot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) tot += ss_lds[i];
+            const float inv = 1.0f / sqrtf(tot / 4096.0f + nm.eps);
+            const float4 g = *(const float4 *)&w_raw[4 * lane];
+            if (blockIdx.x == 0) *(float4 *)(nm.x_out + 256 * wave + 4 * lane) = v;
+            v = float4{v.x * inv * g.x, v.y * inv * g.y, v.z * inv * g.z, v.w * inv * g.w};
+            if (blockIdx.x == 0 && nm.hn_out) *(float4 *)(nm.hn_out + 256 * wave + 4 * lane) = v;
+        }
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
         amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
         amax = fmaxf(amax, __shfl_xor(amax, 2, 64));

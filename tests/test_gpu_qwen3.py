@@ -53,6 +53,23 @@ def test_teacher_forced_logits(mix):
         pos += 1
 
 
+@pytest.mark.parametrize("mix", ["q4_k_m", "q4_k"])
+def test_single_token_steps_with_4096_wide_rows(mix):
+    """hidden = 4096: a single-token step runs residual add + RMSNorm + q|k(|v) and + gate|up as
+    one launch each ("q4_k": every matrix Q4_K, v inside the fused launch; "q4_k_m": some layers keep
+    attn_v as Q6_K, a launch of its own over the normalised row the fused kernel leaves behind)."""
+    cfg = dict(CFG, n_layer=4, hidden=4096, n_head=4, n_kv_head=2, head_dim=128, ffn=1024, vocab=512, n_ctx=32)
+    m, o = make(cfg, 29, mix)
+    prompt = [3, 500, 41, 41, 256, 9]
+    ok, e = close(m.forward(prompt, 0), o.forward(prompt, 0))
+    assert ok, f"prefill: {e}"
+    pos = len(prompt)
+    for t in [5, 123, 511, 0, 350]:
+        ok, e = close(m.forward([t], pos), o.forward([t], pos))
+        assert ok, f"pos {pos}: {e}"
+        pos += 1
+
+
 def test_prefill_in_two_chunks_matches_one():
     m, o = make(CFG, 22)
     toks = list(range(10, 30))
