@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <cstring>
 #include <map>
+#include <set>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -225,9 +226,10 @@ int dispatch_q4k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
 // exactly 16 super-blocks (4096 wide: 10.15 us against 10.27 us for the MFMA GEMV on 14336 rows, and
 // 2 % more decode tokens/s) and everything else is declined (-1).  JQ_Q4K_DOT4 = 0 turns them off,
 // = regs selects the register-prefetch kernel for every row length up to 16 super-blocks.
-// `norm`: residual add + RMSNorm in front of the product (only the LDS-ring kernel has that form).
+// `norm`: residual add + RMSNorm in front of the product; `swiglu`: W pairs gate and up rows and Y gets
+// the n / 2 activations (only the LDS-ring kernel has these forms).
 int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s,
-                      const jq::QdNorm *norm = nullptr) {
+                      const jq::QdNorm *norm = nullptr, bool swiglu = false) {
     const size_t nb = k / 256;
     static const char *mode_env = getenv("JQ_Q4K_DOT4");
     static const std::string mode = mode_env ? mode_env : "auto";
@@ -241,14 +243,17 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
         // a whole number of tiles per workgroup when the chip allows it (224 x 4 at 14336 rows)
         const size_t rounds = (tiles + 255) / 256;
         const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)atoi(genv) : (tiles + rounds - 1) / rounds);
-        if (norm)
-            hipLaunchKernelGGL(jq::q4k_gemv_dot4_lds<true>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, *norm);
-        else
-            hipLaunchKernelGGL(jq::q4k_gemv_dot4_lds<false>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, jq::QdNorm{});
+#define JQ_DOT4_LDS(NORM, SWIGLU, NM) \
+    hipLaunchKernelGGL((jq::q4k_gemv_dot4_lds<NORM, SWIGLU>), dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, NM)
+        if (norm && swiglu) JQ_DOT4_LDS(true, true, *norm);
+        else if (norm) JQ_DOT4_LDS(true, false, *norm);
+        else if (swiglu) JQ_DOT4_LDS(false, true, jq::QdNorm{});
+        else JQ_DOT4_LDS(false, false, jq::QdNorm{});
+#undef JQ_DOT4_LDS
         HIP_TRY(hipGetLastError());
         return 0;
     }
-    if (norm) return -1;
+    if (norm || swiglu) return -1;
     // as many workgroups as the chip holds at once (one of 16 waves per CU, more when smaller), each
     // with an equal share of the rows
     const size_t cap = genv ? (size_t)atoi(genv) : 256 * std::max<size_t>(1, jq::QD_MAX_WAVES / nb);
@@ -1004,6 +1009,7 @@ struct jq_model {
     // Matrices that multiply the same activation, laid one after the other in one allocation
     // (blk.N.qkv, blk.N.gate_up): one launch for a single-token step; q holds views of their parts.
     std::map<std::string, jq_weight *> fused;
+    std::set<std::string> paired;      // fused gate|up entries whose rows alternate gate_j, up_j (see model_fuse)
     std::vector<jq_weight *> retired;  // fused allocations whose parts were replaced; views may still point into them
     bool fused_ready = false;
     float *cat = nullptr;     // the fused result of a single-token step (q|k|v, gate|up)
@@ -1088,7 +1094,9 @@ int model_vec(jq_model *m, const std::string &name, const float **out) {
 
 // Lays the named matrices (same type, same k) one after the other in a new allocation `key`, and
 // replaces their entries in m->q by views of it.  Skipped when any is missing or the types differ.
-int model_fuse(jq_model *m, const std::string &key, const std::vector<std::string> &names) {
+// With `pair_rows` (two parts of equal shape) the rows alternate instead: row 2j of the fused matrix is
+// row j of the first part, row 2j + 1 row j of the second, and the views stride over every other row.
+int model_fuse(jq_model *m, const std::string &key, const std::vector<std::string> &names, bool pair_rows = false) {
     std::vector<jq_weight *> parts;
     for (const auto &nm : names) {
         auto it = m->q.find(nm);
@@ -1100,23 +1108,32 @@ int model_fuse(jq_model *m, const std::string &key, const std::vector<std::strin
         if (w->type != parts[0]->type || w->k != parts[0]->k) return 0;
         rows += w->n, bytes += w->nbytes;
     }
+    pair_rows = pair_rows && parts.size() == 2 && parts[0]->n == parts[1]->n;
+    const size_t rb = parts[0]->row_bytes;
     uint8_t *dev = nullptr;
     HIP_TRY(hipMalloc((void **)&dev, bytes));
     size_t off = 0;
-    for (auto *w : parts) {
-        hipError_t e = hipMemcpy(dev + off, w->dev, w->nbytes, hipMemcpyDeviceToDevice);
+    for (size_t i = 0; i < parts.size(); i++) {
+        jq_weight *w = parts[i];
+        hipError_t e = pair_rows ? hipMemcpy2D(dev + i * rb, 2 * rb, w->dev, rb, rb, w->n, hipMemcpyDeviceToDevice)
+                                 : hipMemcpy(dev + off, w->dev, w->nbytes, hipMemcpyDeviceToDevice);
         if (e != hipSuccess) {
             (void)hipFree(dev);
             return fail("qwen3: fusing `%s` failed: %s", key.c_str(), hipGetErrorString(e));
         }
         off += w->nbytes;
     }
-    jq_weight *whole = new jq_weight{parts[0]->type, rows, parts[0]->k, bytes, parts[0]->row_bytes, dev, true};
+    jq_weight *whole = new jq_weight{parts[0]->type, rows, parts[0]->k, bytes, rb, dev, true};
     m->fused[key] = whole;
+    if (pair_rows) m->paired.insert(key);
     off = 0;
     for (size_t i = 0; i < parts.size(); i++) {
         jq_weight *view = nullptr;
-        if (jq_view(whole, off, parts[i]->n, parts[i]->k, &view)) return 1;
+        if (pair_rows) {
+            view = new jq_weight{whole->type, parts[i]->n, parts[i]->k, bytes - i * rb, 2 * rb, dev + i * rb, false};
+        } else if (jq_view(whole, off, parts[i]->n, parts[i]->k, &view)) {
+            return 1;
+        }
         off += parts[i]->nbytes;
         jq_free(parts[i]);
         m->q[names[i]] = view;
@@ -1138,9 +1155,13 @@ int model_prepare_fused(jq_model *m) {
                                   : std::vector<std::string>{p + ".attn_q.weight", p + ".attn_k.weight"}))
                 return 1;
         }
-        if (!m->fused.count(p + ".gate_up") &&
-            model_fuse(m, p + ".gate_up", {p + ".ffn_gate.weight", p + ".ffn_up.weight"}))
-            return 1;
+        if (!m->fused.count(p + ".gate_up")) {
+            // 4096-wide Q4_K rows: paired, for the launch that also applies SwiGLU
+            auto g = m->q.find(p + ".ffn_gate.weight");
+            const bool pair = g != m->q.end() && g->second->type == JQ_TYPE_Q4_K && g->second->k == 4096 &&
+                              g->second->row_bytes == jq::QD_ROW && !getenv("JQ_NO_PAIRED_GATE_UP");
+            if (model_fuse(m, p + ".gate_up", {p + ".ffn_gate.weight", p + ".ffn_up.weight"}, pair)) return 1;
+        }
     }
     if (!m->cat) {
         const size_t widest = std::max<size_t>((size_t)(c.n_head + 2 * c.n_kv_head) * c.head_dim, 2 * (size_t)c.ffn);
@@ -1154,12 +1175,13 @@ unsigned grid_for(size_t total) { return (unsigned)std::min<size_t>((total + 255
 
 // x_out = x + res; y = W rmsnorm(x_out) as one launch (hn_out also gets the normalised row when
 // given).  False when no kernel has that form for this weight: the caller then runs the two steps.
+// With `swiglu`, w pairs gate and up rows and y gets the w->n / 2 activations.
 bool model_norm_mm(const jq_weight *w, const float *x, const float *res, const float *norm_w, float eps, float *x_out,
-                   float *hn_out, float *y, hipStream_t s) {
+                   float *hn_out, float *y, bool swiglu, hipStream_t s) {
     static const char *off = getenv("JQ_NO_FUSED_NORM");
     if (off || w->type != JQ_TYPE_Q4_K) return false;
     const jq::QdNorm nm{res, norm_w, eps, x_out, hn_out};
-    return dispatch_q4k_dot4(w->dev, w->row_bytes, x, y, w->k, w->n, s, &nm) == 0;
+    return dispatch_q4k_dot4(w->dev, w->row_bytes, x, y, w->k, w->n, s, &nm, swiglu) == 0;
 }
 
 int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
@@ -1186,7 +1208,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         const bool v_fused = fq != m->fused.end() && fq->second->n == (size_t)(nh + 2 * nkv) * d;
         // single token: residual add, norm and q|k(|v) as one launch when the kernel has that form
         const bool normed = fq != m->fused.end() &&
-                            model_norm_mm(fq->second, xc, pending, w_an, c.rms_eps, xo, v_fused ? nullptr : m->hn, m->cat, s);
+                            model_norm_mm(fq->second, xc, pending, w_an, c.rms_eps, xo, v_fused ? nullptr : m->hn, m->cat, false, s);
         if (normed) std::swap(xc, xo);
         else hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, pending, w_an, c.rms_eps, m->hn, h);
         if (fq != m->fused.end()) {  // one launch for q|k(|v) of a single token
@@ -1220,9 +1242,11 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
         const float *gp = m->g, *up = m->u;
         auto fg = T == 1 ? m->fused.find(p + ".gate_up") : m->fused.end();
-        const bool normed2 = fg != m->fused.end() &&
-                             model_norm_mm(fg->second, xc, m->proj, w_fn, c.rms_eps, xo, nullptr, m->cat, s);
-        if (normed2) std::swap(xc, xo);
+        const bool paired = fg != m->fused.end() && m->paired.count(fg->first);  // gate and up rows alternate
+        bool activated = false;  // m->mid already holds silu(gate) * up
+        const bool normed2 = fg != m->fused.end() && model_norm_mm(fg->second, xc, m->proj, w_fn, c.rms_eps, xo, nullptr,
+                                                                   paired ? m->mid : m->cat, paired, s);
+        if (normed2) std::swap(xc, xo), activated = paired;
         else hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, m->proj, w_fn, c.rms_eps, m->hn, h);
         if (fg != m->fused.end()) {
             const jq_weight *w = fg->second;
@@ -1232,8 +1256,13 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
                    model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s)) {
             return 1;
         }
-        hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, gp, up, m->mid,
-                           (size_t)T * c.ffn);
+        if (activated) {
+        } else if (paired) {
+            hipLaunchKernelGGL(jq::swiglu_pairs, dim3(grid_for((size_t)c.ffn)), dim3(256), 0, s, m->cat, m->mid, (size_t)c.ffn);
+        } else {
+            hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, gp, up, m->mid,
+                               (size_t)T * c.ffn);
+        }
         if (model_mm(m, p + ".ffn_down.weight", m->mid, m->proj, T, s)) return 1;
         pending = m->proj;
     }
@@ -1344,6 +1373,7 @@ int jq_qwen3_set_tensor(jq_model *m, const char *name, uint32_t ggml_type, const
             auto it = m->fused.find(layer + key);
             if (it != m->fused.end()) {
                 m->retired.push_back(it->second);
+                m->paired.erase(it->first);
                 m->fused.erase(it);
             }
         }

@@ -168,7 +168,10 @@ struct QdNorm {
     float *hn_out;     // the normalised row (null: not wanted)
 };
 
-template <bool NORM>
+// SWIGLU: the matrix holds the rows of a gate and an up projection alternately (row 2j gate_j, row
+// 2j + 1 up_j) and the result is Y[j] = silu(gate_j . x) * (up_j . x), n / 2 values
+// (reference: src/quantized_qwen3_moe.rs:397-401).
+template <bool NORM, bool SWIGLU>
 __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
                                                           float *__restrict__ Y, int n, QdNorm nm) {
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][QD_TILE_LDS];
@@ -303,11 +306,17 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        {   // wave w sums row w of the tile over the 16 waves
+        if (!SWIGLU) {  // wave w sums row w of the tile over the 16 waves
             float v = (lane < 16) ? red[buf][lane][wave] : 0.0f;
             v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
             const int row = 16 * ((int)blockIdx.x + t * G) + wave;
             if (lane == 0 && row < n) Y[row] = v;
+        } else if (wave < 8) {  // wave w sums rows 2w (lanes 0..15) and 2w + 1 (lanes 16..31): a gate / up pair
+            float v = (lane < 32) ? red[buf][lane & 15][2 * wave + (lane >> 4)] : 0.0f;
+            v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
+            const float up = __shfl(v, 16, 64);
+            const int row = 16 * ((int)blockIdx.x + t * G) + 2 * wave;
+            if (lane == 0 && row + 1 < n) Y[row >> 1] = silu(v) * up;
         }
     }
 }

@@ -259,6 +259,14 @@ __global__ __launch_bounds__(256) void attention_merge(const float *__restrict__
     }
 }
 
+// out[i] = silu(gu[2i]) * gu[2i + 1]: the activation over a product with a row-paired gate|up matrix
+__global__ __launch_bounds__(256) void swiglu_pairs(const float *__restrict__ gu, float *__restrict__ out, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const float2 v = ((const float2 *)gu)[i];
+        out[i] = silu(v.x) * v.y;
+    }
+}
+
 __global__ void set_int(int *p, int v) { *p = v; }
 
 __global__ __launch_bounds__(256) void add_rows(const float *__restrict__ a, const float *__restrict__ b,

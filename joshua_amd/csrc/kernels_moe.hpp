@@ -232,7 +232,6 @@ __global__ __launch_bounds__(GROUP_PAIRS_THREADS) void moe_group_pairs(const uin
     }
 }
 
-__device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 
 // Expert matmuls over the grouped pairs: blockIdx.y = group (its expert is
 // gexp[group]), rows of the expert's weight over blockIdx.x.  The activation row of the pair at sorted

@@ -15,6 +15,8 @@
 
 namespace jq {
 
+__device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);

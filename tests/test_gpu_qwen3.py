@@ -70,6 +70,34 @@ def test_single_token_steps_with_4096_wide_rows(mix):
         pos += 1
 
 
+def test_paired_gate_up_rows_serve_prefill_and_replacement():
+    """With 4096-wide Q4_K rows the gate and up matrices are stored with alternating rows (the
+    single-token launch applies SwiGLU itself); multi-token steps read them as strided views, and a
+    replaced part sends the layer back to separate launches."""
+    cfg = dict(CFG, n_layer=2, hidden=4096, n_head=4, n_kv_head=2, head_dim=128, ffn=512, vocab=512, n_ctx=40)
+    m, o = make(cfg, 31, "q4_k")
+    toks = [7, 400, 41, 300, 256, 9, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25]
+    ok, e = close(m.forward(toks[:1], 0), o.forward(toks[:1], 0))      # fuses on the first single-token step
+    assert ok, e
+    ok, e = close(m.forward(toks[1:4], 1), o.forward(toks[1:4], 1))    # 3 rows: views under the few-row kernel
+    assert ok, e
+    ok, e = close(m.forward(toks[4:], 4), o.forward(toks[4:], 4))      # 16 rows
+    assert ok, e
+    m.reset(), o.reset()
+    ok, e = close(m.forward(toks + toks, 0), o.forward(toks + toks, 0))  # 40 rows: views under the GEMM
+    assert ok, e
+    name = "blk.1.ffn_up.weight"
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(cfg, 31, "q4_k")}
+    tensors[name] = {n: (qt, d) for n, qt, d in qwen3_tensors(cfg, 99, "q4_k")}[name]
+    m.set_tensor(name, *tensors[name])
+    o2 = oq.Qwen3Oracle(cfg, tensors, avx2=oracle.have_avx2())
+    m.reset()
+    ok, e = close(m.forward([5], 0), o2.forward([5], 0))
+    assert ok, e
+    ok, e = close(m.forward([6], 1), o2.forward([6], 1))
+    assert ok, e
+
+
 def test_prefill_in_two_chunks_matches_one():
     m, o = make(CFG, 22)
     toks = list(range(10, 30))
