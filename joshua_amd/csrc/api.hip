@@ -1017,6 +1017,8 @@ struct jq_model {
     uint32_t n_past = 0;
     size_t cap_tokens = 0;
     uint32_t *ids = nullptr, *pick = nullptr;
+    float *pick_v = nullptr;  // the greedy pick's candidates, one per slice of the logits
+    int *pick_i = nullptr;
     int *pos = nullptr;       // device copy of the position of the step being run
     float *part = nullptr;    // split-attention partials
     float *x2 = nullptr;      // second residual row of a single-token step (the fused norm + matmul launches alternate)
@@ -1232,7 +1234,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             else if (d == 128) JQ_ATT_SPLIT(128);
             else JQ_ATT_SPLIT(256);
 #undef JQ_ATT_SPLIT
-            hipLaunchKernelGGL(jq::attention_merge, dim3(T * nh), dim3(128), n_chunks * sizeof(float), s, m->part, m->att, d,
+            hipLaunchKernelGGL(jq::attention_merge, dim3(T * nh), dim3(128), 2 * n_chunks * sizeof(float), s, m->part, m->att, d,
                                n_chunks);
         } else {
             size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
@@ -1309,6 +1311,8 @@ int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out) {
     const size_t part_floats = (size_t)8 * c.n_head * ((c.n_ctx + jq::ATT_CHUNK - 1) / jq::ATT_CHUNK) * (c.head_dim + 2);
     if (hipMalloc((void **)&m->logits, c.vocab * sizeof(float)) != hipSuccess ||
         hipMalloc((void **)&m->pick, sizeof(uint32_t)) != hipSuccess ||
+        hipMalloc((void **)&m->pick_v, jq::ARGMAX_PARTS * sizeof(float)) != hipSuccess ||
+        hipMalloc((void **)&m->pick_i, jq::ARGMAX_PARTS * sizeof(int)) != hipSuccess ||
         hipMalloc((void **)&m->pos, sizeof(int)) != hipSuccess ||
         hipMalloc((void **)&m->part, part_floats * sizeof(float)) != hipSuccess) {
         jq_qwen3_free(m);
@@ -1330,6 +1334,8 @@ void jq_qwen3_free(jq_model *m) {
     for (float *p : m->vc) (void)hipFree(p);
     if (m->logits) (void)hipFree(m->logits);
     if (m->pick) (void)hipFree(m->pick);
+    if (m->pick_v) (void)hipFree(m->pick_v);
+    if (m->pick_i) (void)hipFree(m->pick_i);
     if (m->pos) (void)hipFree(m->pos);
     if (m->part) (void)hipFree(m->part);
     delete m;
@@ -1410,7 +1416,9 @@ int jq_qwen3_greedy(jq_model *m, uint32_t *token, void *stream) {
     if (!m || !token) return fail("jq_qwen3_greedy: null argument");
     hipStream_t s = (hipStream_t)stream;
     std::lock_guard<std::mutex> lock(m->mu);
-    hipLaunchKernelGGL(jq::argmax_last, dim3(1), dim3(1024), 0, s, m->logits, (int)m->cfg.vocab, m->pick);
+    hipLaunchKernelGGL(jq::argmax_last_parts, dim3(jq::ARGMAX_PARTS), dim3(256), 0, s, m->logits, (int)m->cfg.vocab,
+                       m->pick_v, m->pick_i);
+    hipLaunchKernelGGL(jq::argmax_last_merge, dim3(1), dim3(jq::ARGMAX_PARTS), 0, s, m->pick_v, m->pick_i, m->pick);
     HIP_TRY(hipMemcpyAsync(token, m->pick, sizeof(uint32_t), hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
     return 0;

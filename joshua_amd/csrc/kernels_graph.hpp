@@ -237,24 +237,35 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
     if (threadIdx.x == 0) po[0] = mx, po[1] = l;
 }
 
-// out[(t, head), :] = sum_ch exp(m_ch - m) acc_ch / sum_ch exp(m_ch - m) l_ch over the chunks with keys
-__global__ __launch_bounds__(256) void attention_merge(const float *__restrict__ part, float *__restrict__ out, int d,
+// out[(t, head), :] = sum_ch exp(m_ch - m) acc_ch / sum_ch exp(m_ch - m) l_ch over the chunks with keys.
+// Every read of the partials is issued side by side (a thread per chunk for m and l, 16 chunks at a
+// time for the sums): the kernel is a few round trips to memory long, whatever the chunk count.
+__global__ __launch_bounds__(128) void attention_merge(const float *__restrict__ part, float *__restrict__ out, int d,
                                                         int n_chunks) {
-    extern __shared__ float wch[];  // [n_chunks] rescaling weights, then the total
+    extern __shared__ float wch[];  // [n_chunks] maxima, then rescaling weights; [n_chunks] l
+    float *lch = wch + n_chunks;
     const float *pp = part + (size_t)blockIdx.x * n_chunks * (d + 2);
-    float mx = -INFINITY;
-    for (int ch = 0; ch < n_chunks; ch++) mx = fmaxf(mx, pp[(size_t)ch * (d + 2)]);
     for (int ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {
-        const float l = pp[(size_t)ch * (d + 2) + 1];
-        wch[ch] = l > 0.0f ? expf(pp[(size_t)ch * (d + 2)] - mx) : 0.0f;
+        const float2 ml = *(const float2 *)(pp + (size_t)ch * (d + 2));
+        wch[ch] = ml.x, lch[ch] = ml.y;
     }
     __syncthreads();
+    float mx = -INFINITY;
+    for (int ch = 0; ch < n_chunks; ch++) mx = fmaxf(mx, wch[ch]);
+    __syncthreads();
+    for (int ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) wch[ch] = lch[ch] > 0.0f ? expf(wch[ch] - mx) : 0.0f;
+    __syncthreads();
     float tot = 0.0f;
-    for (int ch = 0; ch < n_chunks; ch++) tot = fmaf(pp[(size_t)ch * (d + 2) + 1], wch[ch], tot);
+    for (int ch = 0; ch < n_chunks; ch++) tot = fmaf(lch[ch], wch[ch], tot);
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
         float a = 0.0f;
-#pragma unroll 4
-        for (int ch = 0; ch < n_chunks; ch++) a = fmaf(wch[ch], pp[(size_t)ch * (d + 2) + 2 + c], a);
+        for (int ch0 = 0; ch0 < n_chunks; ch0 += 16) {
+            float v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = pp[(size_t)min(ch0 + j, n_chunks - 1) * (d + 2) + 2 + c];
+#pragma unroll
+            for (int j = 0; j < 16; j++) a = fmaf(ch0 + j < n_chunks ? wch[ch0 + j] : 0.0f, v[j], a);
+        }
         out[(size_t)blockIdx.x * d + c] = a / tot;
     }
 }
@@ -276,17 +287,12 @@ __global__ __launch_bounds__(256) void add_rows(const float *__restrict__ a, con
 }
 
 // Index of the largest value; of equal values the LAST one, as the reference's
-// greedy pick does (Iterator::max_by, src/engine.rs:2371-2378).  One workgroup.
-__global__ __launch_bounds__(1024) void argmax_last(const float *__restrict__ v, int n, uint32_t *__restrict__ out) {
-    __shared__ float bv[16];
-    __shared__ int bi[16];
-    float best = -INFINITY;
-    int idx = -1;
-    for (int i = threadIdx.x; i < n; i += blockDim.x)
-        if (v[i] >= best) {  // i increases within a thread: >= keeps the last
-            best = v[i];
-            idx = i;
-        }
+// greedy pick does (Iterator::max_by, src/engine.rs:2371-2378).  Two launches: ARGMAX_PARTS
+// workgroups each find the pick of a contiguous slice, one workgroup picks among those.
+constexpr int ARGMAX_PARTS = 256;
+
+// (best, idx) over a workgroup; a later index wins among equal values.  Valid in thread 0.
+__device__ __forceinline__ void argmax_last_block(float &best, int &idx, float *bv, int *bi) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         const float ob = __shfl_xor(best, off, 64);
@@ -307,8 +313,35 @@ __global__ __launch_bounds__(1024) void argmax_last(const float *__restrict__ v,
                 best = bv[i];
                 idx = bi[i];
             }
-        out[0] = (uint32_t)(idx < 0 ? 0 : idx);
     }
+}
+
+__global__ __launch_bounds__(256) void argmax_last_parts(const float *__restrict__ v, int n, float *__restrict__ pv,
+                                                         int *__restrict__ pi) {
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    const int per = (n + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int lo = (int)blockIdx.x * per, hi = min(n, lo + per);
+    float best = -INFINITY;
+    int idx = -1;
+    for (int i = lo + (int)threadIdx.x; i < hi; i += blockDim.x)
+        if (v[i] >= best) {  // i increases within a thread: >= keeps the last
+            best = v[i];
+            idx = i;
+        }
+    argmax_last_block(best, idx, bv, bi);
+    if (threadIdx.x == 0) pv[blockIdx.x] = best, pi[blockIdx.x] = idx;
+}
+
+__global__ __launch_bounds__(ARGMAX_PARTS) void argmax_last_merge(const float *__restrict__ pv, const int *__restrict__ pi,
+                                                                  uint32_t *__restrict__ out) {
+    __shared__ float bv[ARGMAX_PARTS / 64];
+    __shared__ int bi[ARGMAX_PARTS / 64];
+    float best = pv[threadIdx.x];
+    int idx = pi[threadIdx.x];
+    if (idx < 0) best = -INFINITY;  // an empty slice, or one of NaNs only
+    argmax_last_block(best, idx, bv, bi);
+    if (threadIdx.x == 0) out[0] = (uint32_t)(idx < 0 ? 0 : idx);
 }
 
 }  // namespace jq
