@@ -20,6 +20,7 @@
 #include "kernels_mfma_q4k_gemm.hpp"
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
+#include "kernels_dot4_q6k.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
 #include "kernels_valu.hpp"
@@ -263,6 +264,24 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
+// Q6_K, one activation row, rows of 4096, 8192 or 12288: the v_dot4 LDS-ring kernel.
+// Returns -1 when the shape is outside its reach.
+int dispatch_q6k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
+    static const char *mode = getenv("JQ_Q6K_DOT4");
+    const size_t ng = k / 4096;
+    if ((mode && mode[0] == '0') || k % 4096 != 0 || ng < 1 || ng > 3 || row_bytes != ng * jq::Q6D_SLICE ||
+        ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
+        return -1;
+    const size_t tiles = (n + jq::Q6D_ROWS - 1) / jq::Q6D_ROWS, rounds = (tiles + 255) / 256;
+    static const char *genv = getenv("JQ_Q6K_DOT4_GRID");
+    const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)std::max(atoi(genv), 1) : (tiles + rounds - 1) / rounds);
+    if (ng == 1) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    else if (ng == 2) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    else hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // Q4_K, 1..16 activation rows, rows of at most 16 super-blocks: the weight-streaming MFMA kernel.
 // Returns -1 when the shape is outside its reach.
 int dispatch_q4k_stream(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
@@ -362,6 +381,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     if (m > 0x7FFFFFFF || k > 0x7FFFFFFF || n > 0x7FFFFFFF) return fail("matmul: dimension exceeds 2^31-1");
     if (type == JQ_TYPE_Q4_K && m == 1) {
         const int rc = dispatch_q4k_dot4(W, row_bytes, X, Y, k, n, s);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q6_K && m == 1) {
+        const int rc = dispatch_q6k_dot4(W, row_bytes, X, Y, k, n, s);
         if (rc >= 0) return rc;
     }
     // one or two activation rows: the int8 GEMV below is faster; from three on the streaming kernel,

@@ -1,0 +1,149 @@
+// Q6_K times one activation row on v_dot4, the weights travelling HBM -> LDS as asynchronous, fully
+// coalesced loads (the road of q4k_gemv_dot4_lds, for the 210-byte Q6_K blocks).
+//
+// Rows of 16 * NG super-blocks (k = 4096 NG).  A step is 8 weight rows x 16 super-blocks: the 16
+// waves of a workgroup copy the 8 row slices (3360 B each, half a slice a wave, two instructions)
+// into a ring of three steps in LDS, two steps ahead of the arithmetic; wave w then works on
+// super-block w of the slice, 8 lanes a row: lane (half h, eighth e) takes l in [8e, 8e + 8) of the
+// half's four 32-element quarters (24 bytes of ql and qh), builds the 6-bit values four to a
+// register and multiplies them with v_dot4_i32_i8 against the activations, which every wave keeps
+// in registers as 15-bit fixed point per 32-element block (two int8 planes, X = 256 hi + lo).  The
+// per-quarter integer sums are exact; sum (q - 32) X = sum q X - 32 sum X with the lanes' sums of X
+// prepared once.  Result per row: d * sum_quarters sc * s_x * (integer), summed over the lanes of a
+// row, the waves of a workgroup (through LDS) and the NG steps of a row tile (in a register).
+#pragma once
+#include "kernels_dot4_q4k.hpp"
+
+namespace jq {
+
+constexpr int Q6D_SLICE = 16 * 210, Q6D_SLICE_LDS = Q6D_SLICE + 16, Q6D_ROWS = 8, Q6D_STEP_LDS = Q6D_ROWS * Q6D_SLICE_LDS;
+
+template <int NG>
+__global__ __launch_bounds__(1024) void q6k_gemv_dot4_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
+                                                          float *__restrict__ Y, int n) {
+    __shared__ __attribute__((aligned(16))) uint8_t ring[3][Q6D_STEP_LDS];
+    __shared__ uint32_t xl_lds[NG][16][64], xh_lds[NG][16][64];
+    __shared__ float s_lds[NG][16][8];
+    __shared__ float red[2][16][Q6D_ROWS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane >> 3, h = (lane >> 2) & 1, e = lane & 3;  // row of the step, half of the super-block, eighth
+    const int G = (int)gridDim.x;
+    const int n_tiles = (((n + Q6D_ROWS - 1) / Q6D_ROWS) - (int)blockIdx.x + G - 1) / G;  // row tiles blockIdx.x, + G, ...
+    if (n_tiles <= 0) return;
+    const int n_steps = NG * n_tiles;
+    constexpr size_t row_bytes = (size_t)NG * Q6D_SLICE;
+
+    // step i = (row tile i / NG, column group i % NG); 2 asynchronous loads per wave: half a row slice
+    auto fetch = [&](int i, int slot) __attribute__((always_inline)) {
+        const int ii = min(i, n_steps - 1);
+        const int row = min(Q6D_ROWS * ((int)blockIdx.x + (ii / NG) * G) + (wave >> 1), n - 1);
+        const uint8_t *src = W + (size_t)row * row_bytes + (size_t)(ii % NG) * Q6D_SLICE + (wave & 1) * 1680 + 16 * lane;
+        const uint32_t dst = lds_offset_of(&ring[slot][(wave >> 1) * Q6D_SLICE_LDS + (wave & 1) * 1680]);
+        async_load16(src, dst);
+        if (lane < 41) async_load16(src + 1024, dst + 1024);  // 105 pieces of 16 bytes per half slice
+    };
+    fetch(0, 0);
+    fetch(1, 1);  // (a clamped copy of step 0 when there is one step only)
+
+    // activations of super-block 16 g + wave: 4 elements a lane, one scale per 32
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const float4 v = *(const float4 *)(X + (size_t)(16 * g + wave) * 256 + 4 * lane);
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+        const bool live = amax > 0.0f && amax < INFINITY;
+        const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
+        const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                           __float2int_rn(v.w * inv)};
+        uint32_t wl = 0, wh = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int lo = ((Xq[i] + 128) & 255) - 128, hi = (Xq[i] - lo) >> 8;
+            wl |= (uint32_t)(lo & 255) << (8 * i);
+            wh |= (uint32_t)(hi & 255) << (8 * i);
+        }
+        xl_lds[g][wave][lane] = wl;
+        xh_lds[g][wave][lane] = wh;
+        if ((lane & 7) == 0) s_lds[g][wave][lane >> 3] = s;
+    }
+    asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");  // step 0 landed (step 1 may be in flight), planes written
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // this lane's share: quarter t of half h covers elements 128 h + 32 t + 8 e .. + 7 (two registers a plane)
+    uint32_t xl[NG][4][2], xh[NG][4][2];
+    float sx[NG][4];   // activation scale of the quarter's 32-element block
+    int xs32[NG][4];   // 32 * (sum of the lane's 8 fixed-point activations of the quarter)
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int dw = 32 * h + 8 * t + 2 * e;
+            xl[g][t][0] = xl_lds[g][wave][dw], xl[g][t][1] = xl_lds[g][wave][dw + 1];
+            xh[g][t][0] = xh_lds[g][wave][dw], xh[g][t][1] = xh_lds[g][wave][dw + 1];
+            sx[g][t] = s_lds[g][wave][4 * h + t];
+            const int ones = 0x01010101;
+            const int sl = __builtin_amdgcn_sdot4(ones, (int)xl[g][t][0], __builtin_amdgcn_sdot4(ones, (int)xl[g][t][1], 0, false), false);
+            const int sh = __builtin_amdgcn_sdot4(ones, (int)xh[g][t][0], __builtin_amdgcn_sdot4(ones, (int)xh[g][t][1], 0, false), false);
+            xs32[g][t] = 32 * ((sh << 8) + sl);
+        }
+    }
+
+    // on entry to step i: step i is in LDS and visible (the barrier just passed), step i+1 in flight
+    float acc = 0.0f;
+    for (int i = 0, tile = 0; i < n_steps; i += NG, tile++) {
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            const int st = i + g;
+            const bool more = st + 2 < n_steps;
+            if (more) fetch(st + 2, (st + 2) % 3);  // the slot of step st-1, which every wave finished reading before that barrier
+
+            const uint8_t *blk = &ring[st % 3][r * Q6D_SLICE_LDS + wave * 210];
+            const uint2 qa = ld<uint2>(blk + 64 * h + 8 * e);         // ql[64h + l]
+            const uint2 qb = ld<uint2>(blk + 64 * h + 32 + 8 * e);    // ql[64h + 32 + l]
+            const uint2 qh = ld<uint2>(blk + 128 + 32 * h + 8 * e);   // qh[32h + l]
+            const float d = f16_bits(ld<uint16_t>(blk + 208));
+            const uint32_t a[2] = {qa.x, qa.y}, b[2] = {qb.x, qb.y}, hh[2] = {qh.x, qh.y};
+            float f = 0.0f;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                int sl = 0, sh = 0;
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const uint32_t lo = (t & 1) ? b[j] : a[j];
+                    const uint32_t nib = (t < 2) ? (lo & 0x0F0F0F0Fu) : ((lo >> 4) & 0x0F0F0F0Fu);
+                    const uint32_t two = t == 0 ? hh[j] << 4 : t == 1 ? hh[j] << 2 : t == 2 ? hh[j] : hh[j] >> 2;
+                    const int q = (int)(nib | (two & 0x30303030u));  // four 6-bit values, 0..63
+                    sl = __builtin_amdgcn_sdot4(q, (int)xl[g][t][j], sl, false);
+                    sh = __builtin_amdgcn_sdot4(q, (int)xh[g][t][j], sh, false);
+                }
+                const float sc = (float)(int8_t)blk[192 + 8 * h + 2 * t + (e >> 1)];
+                f = fmaf(sc * sx[g][t], (float)((sh << 8) + sl - xs32[g][t]), f);
+            }
+            acc = fmaf(d, f, acc);
+
+            const int buf = tile & 1;
+            if (g == NG - 1) {  // the row tile is complete: the lanes of a row, then the waves through LDS
+                acc += __shfl_xor(acc, 1, 64);
+                acc += __shfl_xor(acc, 2, 64);
+                acc += __shfl_xor(acc, 4, 64);
+                if ((lane & 7) == 0) red[buf][wave][r] = acc;
+                acc = 0.0f;
+            }
+            // step st+1 has landed (and the partial sums are written): at most this step's 2 loads stay in flight
+            if (more) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (g == NG - 1 && wave < Q6D_ROWS) {  // wave w sums row w of the tile over the 16 waves
+                float v = (lane < 16) ? red[buf][lane][wave] : 0.0f;
+                v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
+                const int row = Q6D_ROWS * ((int)blockIdx.x + tile * G) + wave;
+                if (lane == 0 && row < n) Y[row] = v;
+            }
+        }
+    }
+}
+
+}  // namespace jq

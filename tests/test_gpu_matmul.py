@@ -188,6 +188,48 @@ def test_q4k_ring_kernel_integer_dot_products_are_bit_exact():
     assert np.array_equal(got, want.astype(np.float32))
 
 
+@pytest.mark.parametrize("k,n", [(4096, 1024), (4096, 8 * 300 + 5), (8192, 77), (12288, 4096), (12288, 3)])
+def test_q6k_one_row_over_4096_wide_row_groups(k, n):
+    """Q6_K rows of 4096, 8192 and 12288 with one activation row take the v_dot4 kernel (8-row steps,
+    one to three column groups a row tile); row counts with a ragged last tile and below one tile."""
+    blocks = make_blocks(capi.Q6_K, n, k, 31)
+    lhs = synth.normal(32 + n % 7, (1, k))
+    got = capi.Weight.upload(capi.Q6_K, blocks, n, k).matmul_t(1, lhs)
+    assert close(got, oracle.matmul_t(capi.Q6_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+def test_q6k_dot4_integer_dot_products_are_bit_exact():
+    """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
+    scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
+    n, k = 203, 4096
+    rng = np.random.default_rng(5)
+    q = np.zeros((n, k), np.int64)
+    for r in range(n):
+        idx = rng.choice(k, size=24, replace=False)
+        q[r, idx] = rng.integers(-32, 32, size=24)
+    x = rng.integers(-3000, 3001, size=k).astype(np.int64)
+    peak = np.arange(0, k, 32) + int(rng.integers(0, 32))
+    x[peak] = 32639 * rng.choice([-1, 1], size=k // 32)
+    q[:, peak] = 0
+    qq = (q + 32).reshape(n, k // 256, 2, 4, 32)                   # [half][quarter][l]
+    ql = np.zeros((n, k // 256, 2, 64), np.uint8)
+    ql[..., :32] = (qq[:, :, :, 0, :] & 15) | ((qq[:, :, :, 2, :] & 15) << 4)
+    ql[..., 32:] = (qq[:, :, :, 1, :] & 15) | ((qq[:, :, :, 3, :] & 15) << 4)
+    qh = ((qq[:, :, :, 0, :] >> 4) | ((qq[:, :, :, 1, :] >> 4) << 2) | ((qq[:, :, :, 2, :] >> 4) << 4) |
+          ((qq[:, :, :, 3, :] >> 4) << 6)).astype(np.uint8)
+    blocks = np.zeros((n, k // 256, 210), np.uint8)
+    blocks[:, :, 0:128] = ql.reshape(n, k // 256, 128)
+    blocks[:, :, 128:192] = qh.reshape(n, k // 256, 64)
+    blocks[:, :, 192:208] = 1
+    blocks[:, :, 208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks = blocks.reshape(-1)
+    assert np.array_equal(oracle.dequantize(capi.Q6_K, blocks).reshape(n, k), q.astype(np.float32))
+    want = x @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q6_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+    assert np.array_equal(got[0], want.astype(np.float32))
+
+
 def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
     """4096-wide rows, one activation row: the v_dot4 kernel, activation range 32639 per 32-element
     sub-block."""
