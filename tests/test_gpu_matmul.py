@@ -188,7 +188,7 @@ def test_q4k_ring_kernel_integer_dot_products_are_bit_exact():
     assert np.array_equal(got, want.astype(np.float32))
 
 
-@pytest.mark.parametrize("k,n", [(4096, 1024), (4096, 8 * 300 + 5), (8192, 77), (12288, 4096), (12288, 3)])
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 8 * 600 + 5), (8192, 2048 + 77), (12288, 4096), (12288, 1368 + 3)])
 def test_q6k_one_row_over_4096_wide_row_groups(k, n):
     """Q6_K rows of 4096, 8192 and 12288 with one activation row take the v_dot4 kernel (8-row steps,
     one to three column groups a row tile); row counts with a ragged last tile and below one tile."""
@@ -201,7 +201,7 @@ def test_q6k_one_row_over_4096_wide_row_groups(k, n):
 def test_q6k_dot4_integer_dot_products_are_bit_exact():
     """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
     scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
-    n, k = 203, 4096
+    n, k = 4096 + 3, 4096
     rng = np.random.default_rng(5)
     q = np.zeros((n, k), np.int64)
     for r in range(n):
