@@ -21,6 +21,7 @@
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
 #include "kernels_dot4_q6k.hpp"
+#include "kernels_dot4_q8.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
 #include "kernels_valu.hpp"
@@ -283,6 +284,24 @@ int dispatch_q6k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
+// Q8_0, one activation row, rows of 4096, 8192 or 12288: the v_dot4 LDS-ring kernel.
+// Returns -1 when the shape is outside its reach.
+int dispatch_q8_0_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
+    static const char *mode = getenv("JQ_Q8_0_DOT4");
+    const size_t ng = k / 4096;
+    if ((mode && mode[0] == '0') || k % 4096 != 0 || ng < 1 || ng > 3 || row_bytes != ng * jq::Q8D_SLICE ||
+        ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
+        return -1;
+    const size_t tiles = (n + jq::Q8D_ROWS - 1) / jq::Q8D_ROWS, rounds = (tiles + 255) / 256;
+    if (tiles * ng < 512) return -1;  // under two steps a workgroup the staged f32 kernel is as fast
+    const unsigned grid = (unsigned)std::min<size_t>(tiles, (tiles + rounds - 1) / rounds);
+    if (ng == 1) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    else if (ng == 2) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    else hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // Q4_K, 1..16 activation rows, rows of at most 16 super-blocks: the weight-streaming MFMA kernel.
 // Returns -1 when the shape is outside its reach.
 int dispatch_q4k_stream(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
@@ -386,6 +405,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     }
     if (type == JQ_TYPE_Q6_K && m == 1) {
         const int rc = dispatch_q6k_dot4(W, row_bytes, X, Y, k, n, s);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q8_0 && m == 1) {
+        const int rc = dispatch_q8_0_dot4(W, row_bytes, X, Y, k, n, s);
         if (rc >= 0) return rc;
     }
     // one or two activation rows: the int8 GEMV below is faster; from three on the streaming kernel,

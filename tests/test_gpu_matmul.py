@@ -230,6 +230,38 @@ def test_q6k_dot4_integer_dot_products_are_bit_exact():
     assert np.array_equal(got[0], want.astype(np.float32))
 
 
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 8 * 600 + 5), (8192, 2048 + 77), (12288, 1368 + 3)])
+def test_q8_0_one_row_over_4096_wide_row_groups(k, n):
+    """Q8_0 rows of 4096, 8192 and 12288 with one activation row take the v_dot4 kernel (8-row steps,
+    one to three column groups a row tile), with ragged last tiles."""
+    blocks = make_blocks(capi.Q8_0, n, k, 41)
+    lhs = synth.normal(42 + n % 7, (1, k))
+    got = capi.Weight.upload(capi.Q8_0, blocks, n, k).matmul_t(1, lhs)
+    assert close(got, oracle.matmul_t(capi.Q8_0, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+def test_q8_0_dot4_integer_dot_products_are_bit_exact():
+    """d = 1, integer activations whose 32-element blocks peak at 32639 (activation scale exactly 1)."""
+    n, k = 4096 + 3, 4096
+    rng = np.random.default_rng(6)
+    q = np.zeros((n, k), np.int64)
+    cols = rng.integers(0, k, size=(n, 12))
+    q[np.arange(n)[:, None], cols] = rng.integers(-127, 128, size=(n, 12))
+    x = rng.integers(-3000, 3001, size=k).astype(np.int64)
+    peak = np.arange(0, k, 32) + int(rng.integers(0, 32))
+    x[peak] = 32639 * rng.choice([-1, 1], size=k // 32)
+    q[:, peak] = 0
+    blocks = np.zeros((n, k // 32, 34), np.uint8)
+    blocks[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks[:, :, 2:] = q.reshape(n, k // 32, 32).astype(np.int8).view(np.uint8)
+    blocks = blocks.reshape(-1)
+    assert np.array_equal(oracle.dequantize(capi.Q8_0, blocks).reshape(n, k), q.astype(np.float32))
+    want = x @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q8_0, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+    assert np.array_equal(got[0], want.astype(np.float32))
+
+
 def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
     """4096-wide rows, one activation row: the v_dot4 kernel, activation range 32639 per 32-element
     sub-block."""
