@@ -15,6 +15,22 @@
 
 namespace jq {
 
+// v[lane] + v[lane ^ 16] and v[lane] + v[lane ^ 32] in every lane, as one row-swap instruction and
+// one add (v_permlane16_swap / v_permlane32_swap exchange the odd rows of one operand with the even
+// rows of the other; with v in both, the two results hold the pair's values) instead of a trip
+// through LDS.
+__device__ __forceinline__ float sum_xor16(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+
+
 template <class T>
 __device__ __forceinline__ T ld(const uint8_t *p) {
     T v;

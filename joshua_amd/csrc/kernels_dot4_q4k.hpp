@@ -123,8 +123,8 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
         const float f_lo = (float)((sh_lo << 8) + sl_lo) * s_lo, f_hi = (float)((sh_hi << 8) + sl_hi) * s_hi;
         float acc = d * fmaf((float)sc_lo, f_lo, (float)sc_hi * f_hi);
         acc = fmaf(-dmin, fmaf((float)mn_lo, xs_lo, (float)mn_hi * xs_hi), acc);
-        acc += __shfl_xor(acc, 16, 64);
-        acc += __shfl_xor(acc, 32, 64);  // the four chunks of the block
+        acc = sum_xor16(acc);
+        acc = sum_xor32(acc);  // the four chunks of the block
 
         // the waves' partial sums of the 16 rows meet in LDS; wave w then sums rows w, w + waves, ...
         // over the waves (16 lanes, one partial each, a fixed tree), so no wave carries the whole reduction
@@ -296,8 +296,8 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         const float f_lo = (float)((sh_lo << 8) + sl_lo) * s_lo, f_hi = (float)((sh_hi << 8) + sl_hi) * s_hi;
         float acc = d * fmaf((float)sc_lo, f_lo, (float)sc_hi * f_hi);
         acc = fmaf(-dmin, fmaf((float)mn_lo, xs_lo, (float)mn_hi * xs_hi), acc);
-        acc += __shfl_xor(acc, 16, 64);
-        acc += __shfl_xor(acc, 32, 64);
+        acc = sum_xor16(acc);
+        acc = sum_xor32(acc);
 
         const int buf = t & 1;
         if (lane < 16) red[buf][wave][lane] = acc;

@@ -266,8 +266,8 @@ __global__ __launch_bounds__(64 * Q4K_MAX_WAVES) void q4k_gemv_mfma(const uint8_
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
         float v = acc[mi];
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
+        v = sum_xor16(v);
+        v = sum_xor32(v);
         if (lane < 16) partial[(wave * MT + mi) * 16 + lane] = v;
     }
     __syncthreads();

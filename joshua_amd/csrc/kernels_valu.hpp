@@ -18,8 +18,10 @@ namespace jq {
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 
 __device__ __forceinline__ float wave_sum(float v) {
+    v = sum_xor32(v);
+    v = sum_xor16(v);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
 }
 
