@@ -15,6 +15,43 @@
 
 namespace jq {
 
+// Sums over the aligned 16 (8) lanes around a lane, in every lane of the group, on the data-parallel
+// primitives (row rotations, half-row mirror, quad permutes): four (three) instructions with no trip
+// through LDS, where __shfl_xor costs a ds_bpermute each.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    const int u = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(u, u, CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float sum_row16(float v) {
+    v += dpp_f<0x128>(v);  // row_ror:8
+    v += dpp_f<0x124>(v);  // row_ror:4
+    v += dpp_f<0x122>(v);  // row_ror:2
+    v += dpp_f<0x121>(v);  // row_ror:1
+    return v;
+}
+__device__ __forceinline__ float sum_row8(float v) {
+    v += dpp_f<0x141>(v);  // row_half_mirror
+    v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+    return v;
+}
+
+__device__ __forceinline__ float max_row8(float v) {
+    v = fmaxf(v, dpp_f<0x141>(v));
+    v = fmaxf(v, dpp_f<0xB1>(v));
+    v = fmaxf(v, dpp_f<0x4E>(v));
+    return v;
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int u) { return __builtin_amdgcn_update_dpp(u, u, CTRL, 0xF, 0xF, false); }
+__device__ __forceinline__ int isum_row8(int v) {
+    v += dpp_i<0x141>(v);
+    v += dpp_i<0xB1>(v);
+    v += dpp_i<0x4E>(v);
+    return v;
+}
+
 // v[lane] + v[lane ^ 16] and v[lane] + v[lane ^ 32] in every lane, as one row-swap instruction and
 // one add (v_permlane16_swap / v_permlane32_swap exchange the odd rows of one operand with the even
 // rows of the other; with v in both, the two results hold the pair's values) instead of a trip

@@ -68,9 +68,7 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
     {
         const float4 v = *(const float4 *)(X + 256 * wave + 4 * lane);
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));  // the 8 lanes of a sub-block
+        amax = max_row8(amax);  // the 8 lanes of a sub-block
         const bool live = amax > 0.0f && amax < INFINITY;
         const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
         const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
@@ -86,7 +84,7 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
         }
         xl_lds[wave][lane] = wl;
         xh_lds[wave][lane] = wh;
-        sum += __shfl_xor(sum, 1, 64), sum += __shfl_xor(sum, 2, 64), sum += __shfl_xor(sum, 4, 64);
+        sum = isum_row8(sum);
         if ((lane & 7) == 0) {
             s_lds[wave][lane >> 3] = s;
             xs_lds[wave][lane >> 3] = s * (float)sum;
@@ -133,7 +131,7 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
         __syncthreads();
         for (int rr = wave; rr < 16; rr += waves) {
             float v = (lane < waves) ? red[buf][lane & 15][rr] : 0.0f;
-            v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
+            v = sum_row16(v);
             const int row = row_beg + 16 * t + rr;
             if (lane == 0 && row < row_end) Y[row] = v;
         }
@@ -218,8 +216,7 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
                 v.x += r.x, v.y += r.y, v.z += r.z, v.w += r.w;
             }
             float ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w)));
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+            ss = wave_sum(ss);
             if (lane == 0) ss_lds[wave] = ss;
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
@@ -234,9 +231,7 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
             if (blockIdx.x == 0 && nm.hn_out) *(float4 *)(nm.hn_out + 256 * wave + 4 * lane) = v;
         }
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+        amax = max_row8(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
         const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
         const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
@@ -252,7 +247,7 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         }
         xl_lds[wave][lane] = wl;
         xh_lds[wave][lane] = wh;
-        sum += __shfl_xor(sum, 1, 64), sum += __shfl_xor(sum, 2, 64), sum += __shfl_xor(sum, 4, 64);
+        sum = isum_row8(sum);
         if ((lane & 7) == 0) {
             s_lds[wave][lane >> 3] = s;
             xs_lds[wave][lane >> 3] = s * (float)sum;
@@ -308,13 +303,13 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         asm volatile("" ::: "memory");
         if (!SWIGLU) {  // wave w sums row w of the tile over the 16 waves
             float v = (lane < 16) ? red[buf][lane][wave] : 0.0f;
-            v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
+            v = sum_row16(v);
             const int row = 16 * ((int)blockIdx.x + t * G) + wave;
             if (lane == 0 && row < n) Y[row] = v;
         } else if (wave < 8) {  // wave w sums rows 2w (lanes 0..15) and 2w + 1 (lanes 16..31): a gate / up pair
             float v = (lane < 32) ? red[buf][lane & 15][2 * wave + (lane >> 4)] : 0.0f;
-            v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
-            const float up = __shfl(v, 16, 64);
+            v = sum_row16(v);
+            const float up = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
             const int row = 16 * ((int)blockIdx.x + t * G) + 2 * wave;
             if (lane == 0 && row + 1 < n) Y[row >> 1] = silu(v) * up;
         }

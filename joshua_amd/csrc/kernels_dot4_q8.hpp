@@ -49,9 +49,7 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
     for (int g = 0; g < NG; g++) {
         const float4 v = *(const float4 *)(X + (size_t)(16 * g + wave) * 256 + 4 * lane);
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+        amax = max_row8(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
         const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
         const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
@@ -102,9 +100,7 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
 
             const int buf = tile & 1;
             if (g == NG - 1) {  // the row tile is complete: the lanes of a row, then the waves through LDS
-                acc += __shfl_xor(acc, 1, 64);
-                acc += __shfl_xor(acc, 2, 64);
-                acc += __shfl_xor(acc, 4, 64);
+                acc = sum_row8(acc);
                 if (j == 0) red[buf][wave][r] = acc;
                 acc = 0.0f;
             }
@@ -115,7 +111,7 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
             asm volatile("" ::: "memory");
             if (g == NG - 1 && wave < Q8D_ROWS) {  // wave w sums row w of the tile over the 16 waves
                 float v = (lane < 16) ? red[buf][lane][wave] : 0.0f;
-                v += __shfl_xor(v, 8, 64), v += __shfl_xor(v, 4, 64), v += __shfl_xor(v, 2, 64), v += __shfl_xor(v, 1, 64);
+                v = sum_row16(v);
                 const int row = Q8D_ROWS * ((int)blockIdx.x + tile * G) + wave;
                 if (lane == 0 && row < n) Y[row] = v;
             }

@@ -20,9 +20,7 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 __device__ __forceinline__ float wave_sum(float v) {
     v = sum_xor32(v);
     v = sum_xor16(v);
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    return sum_row16(v);
 }
 
 constexpr int ROWS_PER_WG = 4;  // one wave per row, 256 threads
