@@ -37,6 +37,13 @@ __device__ __forceinline__ float sum_row8(float v) {
     return v;
 }
 
+__device__ __forceinline__ float max_row16(float v) {
+    v = fmaxf(v, dpp_f<0x128>(v));
+    v = fmaxf(v, dpp_f<0x124>(v));
+    v = fmaxf(v, dpp_f<0x122>(v));
+    v = fmaxf(v, dpp_f<0x121>(v));
+    return v;
+}
 __device__ __forceinline__ float max_row8(float v) {
     v = fmaxf(v, dpp_f<0x141>(v));
     v = fmaxf(v, dpp_f<0xB1>(v));
@@ -65,6 +72,16 @@ __device__ __forceinline__ float sum_xor32(float v) {
     const unsigned u = __builtin_bit_cast(unsigned, v);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+// The maximum over the wave, in every lane.
+__device__ __forceinline__ float wave_max(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    v = fmaxf(__builtin_bit_cast(float, (unsigned)a[0]), __builtin_bit_cast(float, (unsigned)a[1]));
+    const unsigned w = __builtin_bit_cast(unsigned, v);
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    v = fmaxf(__builtin_bit_cast(float, (unsigned)b[0]), __builtin_bit_cast(float, (unsigned)b[1]));
+    return max_row16(v);
 }
 
 

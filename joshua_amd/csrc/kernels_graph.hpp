@@ -122,8 +122,7 @@ __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ 
         sc[j] = acc;
         mx = fmaxf(mx, acc);
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = wave_max(mx);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
     __syncthreads();
@@ -201,14 +200,12 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
             acc = fmaf(qv[i].x, kv[s][i].x, acc), acc = fmaf(qv[i].y, kv[s][i].y, acc);
             acc = fmaf(qv[i].z, kv[s][i].z, acc), acc = fmaf(qv[i].w, kv[s][i].w, acc);
         }
-        acc += __shfl_xor(acc, 1, 64), acc += __shfl_xor(acc, 2, 64);
-        acc += __shfl_xor(acc, 4, 64), acc += __shfl_xor(acc, 8, 64);
+        acc = sum_row16(acc);
         if (sub == 0) sc[j] = j < nj ? acc / sqrt_d : -INFINITY;
     }
     __syncthreads();
     float mx = sc[lane];  // ATT_CHUNK == 64: every wave holds the whole chunk
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = wave_max(mx);
     const float e = expf(sc[lane] - mx);  // exp(-inf) = 0 for the masked tail
     const float l = wave_sum(e);
     __syncthreads();

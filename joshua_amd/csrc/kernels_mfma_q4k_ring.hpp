@@ -134,8 +134,8 @@ __global__ __launch_bounds__(1024) void q4k_ring_mfma(const uint8_t *__restrict_
                     const int o = idx >> pshift, p = idx & (parts - 1);
                     float s = 0.0f;
                     for (int w = p; w < waves; w += parts) s += red[buf][w][o];
-                    if (parts >= 2) s += __shfl_xor(s, 1, 64);
-                    if (parts == 4) s += __shfl_xor(s, 2, 64);
+                    if (parts >= 2) s += dpp_f<0xB1>(s);  // the neighbour: quad_perm [1,0,3,2]
+                    if (parts == 4) s += dpp_f<0x4E>(s);  // the other pair: quad_perm [2,3,0,1]
                     const int src_lane = o >> 2, jj = o & 3;
                     const int nn = 16 * row_tile_of(i) + 4 * (src_lane >> 4) + jj, mm = src_lane & 15;
                     if (DUAL && !(i & 1)) {
