@@ -115,6 +115,9 @@ __global__ __launch_bounds__(1024) void q4k_ring_mfma(const uint8_t *__restrict_
             cur[0].hdr = *(const qg_u4 *)blk;
 #pragma unroll
             for (int c = 0; c < 4; c++) cur[0].nib[c] = *(const uint2 *)(blk + 16 + 32 * c + 8 * kg);
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+                cur[0].dm[jj] = *(const uint32_t *)&ring[i % 3][(4 * kg + jj) * row_lds + wave * 144];
             float acc[4];
             qs_tile_partial<1>(cur, A, kg, acc);
 

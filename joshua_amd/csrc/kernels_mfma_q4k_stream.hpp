@@ -25,6 +25,7 @@ constexpr int QS_MAX_WAVES = 8;
 struct QsTileRegs {  // one 16-row tile of one column, as loaded
     qg_u4 hdr;       // d, dmin, 12 scale bytes of this lane's row
     uint2 nib[4];    // bytes 8*kg .. 8*kg+7 of each chunk's 32 nibble bytes
+    uint32_t dm[4];  // d | dmin of rows 4*kg .. 4*kg+3: the rows this lane holds results of
 };
 
 // The activations of a wave's CPW columns as MFMA B operands.
@@ -171,17 +172,22 @@ __device__ __forceinline__ void qs_load_acts(const uint8_t *base, int kg, QsActs
     A.sx[0] = *(const float *)(base + 16 * slot_stride + (3 - kg) * 16);
 }
 
-// Row `row` of W, the wave's columns: header and this lane group's nibble bytes into registers.
+// Rows row0 .. row0 + 15 of W (clamped to n - 1), the wave's columns: header and this lane group's
+// nibble bytes of row row0 + col, and d | dmin of the four rows whose results the lane will hold.
 template <int CPW>
-__device__ __forceinline__ void qs_load_tile(const uint8_t *__restrict__ W, size_t row_bytes, int row, int wave, int kg,
-                                             QsTileRegs (&r)[CPW]) {
-    const uint8_t *rp = W + (size_t)row * row_bytes + (size_t)(wave * CPW) * 144;
+__device__ __forceinline__ void qs_load_tile(const uint8_t *__restrict__ W, size_t row_bytes, int row0, int n, int col,
+                                             int wave, int kg, QsTileRegs (&r)[CPW]) {
+    const uint8_t *rp = W + (size_t)min(row0 + col, n - 1) * row_bytes + (size_t)(wave * CPW) * 144;
 #pragma unroll
     for (int j = 0; j < CPW; j++) {
         const uint8_t *blk = rp + 144 * j;
         r[j].hdr = *(const qg_u4 *)blk;
 #pragma unroll
         for (int c = 0; c < 4; c++) r[j].nib[c] = *(const uint2 *)(blk + 16 + 32 * c + 8 * kg);
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++)
+            r[j].dm[jj] = *(const uint32_t *)(W + (size_t)min(row0 + 4 * kg + jj, n - 1) * row_bytes +
+                                              (size_t)(wave * CPW + j) * 144);
     }
 }
 
@@ -214,12 +220,9 @@ __device__ __forceinline__ void qs_tile_partial(const QsTileRegs (&cur)[CPW], co
                        qg_pack_h2((int)mn[4], (int)mn[5]), qg_pack_h2((int)mn[6], (int)mn[7])};
         const qg_f4 MM = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(qg_h8, am), __builtin_bit_cast(qg_h8, A.Bm[j]),
                                                                 qg_f4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-        // d and dmin of weight rows 4*kg + jj sit in lanes 4*kg + jj (lanes 0..15 hold the headers
-        // of rows 0..15)
-        const float d = f16_bits(h.x), dmin = f16_bits(h.x >> 16);
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
-            const float dr = __shfl(d, 4 * kg + jj, 64), mr = __shfl(dmin, 4 * kg + jj, 64);
+            const float dr = f16_bits(cur[j].dm[jj]), mr = f16_bits(cur[j].dm[jj] >> 16);
             const float f = fmaf(Ph[jj], 2048.0f, Pl[jj]);
             const float tt = fmaf(-4096.0f * mr, MM[jj], dr * f);
             acc[jj] = fmaf(A.sx[j], tt, acc[jj]);
@@ -241,10 +244,10 @@ __global__ __launch_bounds__(64 * QS_MAX_WAVES) void q4k_stream_mfma(const uint8
 
     QsTileRegs cur[CPW], nxt[CPW];
     int t = blockIdx.x;
-    if (t < n_tiles) qs_load_tile<CPW>(W, row_bytes, min(16 * t + col, n - 1), wave, kg, cur);
+    if (t < n_tiles) qs_load_tile<CPW>(W, row_bytes, 16 * t, n, col, wave, kg, cur);
     for (int it = 0; t < n_tiles; t += gridDim.x, it++) {
         const int tn = t + gridDim.x;
-        if (tn < n_tiles) qs_load_tile<CPW>(W, row_bytes, min(16 * tn + col, n - 1), wave, kg, nxt);
+        if (tn < n_tiles) qs_load_tile<CPW>(W, row_bytes, 16 * tn, n, col, wave, kg, nxt);
 
         float acc[4];
         qs_tile_partial<CPW>(cur, A, kg, acc);
