@@ -56,8 +56,8 @@ __device__ __forceinline__ void qs_quantise_acts(const float *xrow, int wave, in
 #pragma unroll
             for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xv[ks][i]));
         }
-        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        amax = max_xor16(amax);
+        amax = max_xor32(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
         const float inv = live ? QG_RANGE / amax : 0.0f;
         A.sx[j] = live ? amax / QG_RANGE : 0.0f;
@@ -75,8 +75,8 @@ __device__ __forceinline__ void qs_quantise_acts(const float *xrow, int wave, in
             // operand order within the 8 k of a lane: 0,2,1,3,4,6,5,7 (what the weight unpack produces)
             A.Bh[j][ks] = qg_u4{qg_pack_h2(hi[0], hi[2]), qg_pack_h2(hi[1], hi[3]), qg_pack_h2(hi[4], hi[6]), qg_pack_h2(hi[5], hi[7])};
             A.Bl[j][ks] = qg_u4{qg_pack_h2(lo[0], lo[2]), qg_pack_h2(lo[1], lo[3]), qg_pack_h2(lo[4], lo[6]), qg_pack_h2(lo[5], lo[7])};
-            sum += __shfl_xor(sum, 16, 64);
-            sum += __shfl_xor(sum, 32, 64);
+            sum = isum_xor16(sum);
+            sum = isum_xor32(sum);
             xs[ks] = sum;  // the whole sub-block's sum, in all four lanes of the column
         }
         // k group g of the min operand: part g of XS_j / 4096 split three ways into f16, j = 0..7
