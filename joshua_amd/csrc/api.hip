@@ -659,6 +659,7 @@ struct jq_moe {
     uint32_t *ids = nullptr;
     int *gexp = nullptr, *offsets = nullptr, *xrow = nullptr, *yrow = nullptr;
     uint8_t *qacts = nullptr;  // activations as MFMA operand records (Q4_K experts, grouped path)
+    jq::ActsI8 qi8{nullptr, nullptr, nullptr};  // activations as int8 planes (decode path of the formats with Q::dot8)
     std::mutex mu;
 };
 
@@ -667,14 +668,19 @@ namespace {
 void moe_free_scratch(jq_moe *m) {
     for (void *p : {(void *)m->logits, (void *)m->wts, (void *)m->G, (void *)m->U, (void *)m->out, (void *)m->sG,
                     (void *)m->sU, (void *)m->sH, (void *)m->sOut, (void *)m->ids, (void *)m->gexp,
-                    (void *)m->offsets, (void *)m->xrow, (void *)m->yrow, (void *)m->qacts})
+                    (void *)m->offsets, (void *)m->xrow, (void *)m->yrow, (void *)m->qacts, (void *)m->qi8.xl,
+                    (void *)m->qi8.xh, (void *)m->qi8.sx})
         if (p) (void)hipFree(p);
     m->qacts = nullptr;
+    m->qi8 = jq::ActsI8{nullptr, nullptr, nullptr};
     m->logits = m->wts = m->G = m->U = m->out = m->sG = m->sU = m->sH = m->sOut = nullptr;
     m->ids = nullptr;
     m->gexp = m->offsets = m->xrow = m->yrow = nullptr;
     m->cap_tokens = 0;
 }
+
+// Formats whose decode-shaped expert matmuls run on integer dot products (Q::dot8).
+bool moe_has_dot8(uint32_t type) { return type == JQ_TYPE_MXFP4 && !getenv("JQ_MOE_NO_DOT8"); }
 
 int moe_reserve(jq_moe *m, size_t T) {
     if (T <= m->cap_tokens) return 0;
@@ -692,6 +698,12 @@ int moe_reserve(jq_moe *m, size_t T) {
     HIP_TRY(hipMalloc((void **)&m->offsets, (groups + 1) * sizeof(int)));
     HIP_TRY(hipMalloc((void **)&m->xrow, PR * sizeof(int)));
     HIP_TRY(hipMalloc((void **)&m->yrow, PR * sizeof(int)));
+    if (moe_has_dot8(m->gate->type) || moe_has_dot8(m->down->type)) {
+        const size_t words = PR * (std::max<size_t>(c.hidden, c.inter) / 4);
+        HIP_TRY(hipMalloc((void **)&m->qi8.xl, words * sizeof(uint32_t) + 16));
+        HIP_TRY(hipMalloc((void **)&m->qi8.xh, words * sizeof(uint32_t) + 16));
+        HIP_TRY(hipMalloc((void **)&m->qi8.sx, (words / 8 + 1) * sizeof(float)));
+    }
     if (m->gate->type == JQ_TYPE_Q4_K || m->down->type == JQ_TYPE_Q4_K)
         HIP_TRY(hipMalloc((void **)&m->qacts, std::max(T * (c.hidden / 256), PR * (c.inter / 256)) * jq::QS_REC + 16));
     if (m->sgate) {
@@ -796,6 +808,44 @@ int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, si
     return 0;
 }
 
+// One activation row a group, a format with Q::dot8: the activations become int8 planes once, the
+// expert rows are staged through LDS and multiplied on v_dot4.  Returns -1 when the shape is outside
+// its reach.
+template <class Q, bool DUAL>
+int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16, jq::ActsI8 xq,
+                    const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
+                    int groups, hipStream_t s) {
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
+    const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
+    const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
+    const size_t lds = wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>();
+    if (G == 0 || lds > 64 * 1024) return -1;
+    dim3 grid((unsigned)((n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R)), (unsigned)groups), block(64 * jq::ROWS_PER_WG);
+    if (G == 16)
+        hipLaunchKernelGGL((jq::moe_rows_dot8<Q, DUAL, 16>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp, offsets, xsel,
+                           yrow, Y, k, n, L, (int)wave_lds);
+    else
+        hipLaunchKernelGGL((jq::moe_rows_dot8<Q, DUAL, 4>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp, offsets, xsel,
+                           yrow, Y, k, n, L, (int)wave_lds);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+template <bool DUAL>
+int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
+                      const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets,
+                      const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s) {
+    if (!moe_has_dot8(type) || !xq.xl || k % 32 != 0 || ((uintptr_t)X & 15) != 0) return -1;
+    const size_t words = x_rows * (size_t)(k / 4);
+    hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
+    switch (type) {
+    case JQ_TYPE_MXFP4:
+        return launch_moe_dot8<jq::MXFP4, DUAL>(Wa, Wb, row_bytes, aligned16, xq, gexp, offsets, xsel, yrow, Y, k, n, groups, s);
+    default: return -1;
+    }
+}
+
 template <bool SWIGLU>
 int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2,
                       const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
@@ -860,6 +910,10 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         rc = dispatch_moe_q4k_ring<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qacts, m->gexp, m->offsets,
                                          m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s);
     if (rc > 0) return 1;
+    if (rc < 0 && same_gu && max_group <= 1)
+        rc = dispatch_moe_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
+                                     m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s);
+    if (rc > 0) return 1;
     if (rc < 0 && same_gu)
         rc = dispatch_moe_staged<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, m->gexp, m->offsets,
                                        m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s);
@@ -879,6 +933,11 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);
+    if (rc > 0) return 1;
+    if (rc < 0 && fused_act && max_group <= 1)
+        rc = dispatch_moe_dot8<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
+                                      m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden,
+                                      groups, s);
     if (rc > 0) return 1;
     if (rc < 0 && fused_act)
         rc = dispatch_moe_staged<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G, m->gexp,

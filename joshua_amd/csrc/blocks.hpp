@@ -301,6 +301,34 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
     __device__ static float e2m1(uint32_t c) {
         return __uint_as_float(((c & 7u) << 22) | ((c & 8u) << 28)) * 8.507059173023462e37f;  // 2^126
     }
+    // The block against its 32 activations given as 15-bit fixed point in two int8 planes (X = 256 hi +
+    // lo, eight registers a plane): v_perm_b32 looks four magnitude codes up at once in the table of
+    // doubled E2M1 values {0,1,2,3,4,6,8,12}; a negative element counts twice in a second sum instead of
+    // being negated (sum w X = sum |w| X - 2 sum_{w<0} |w| X), so the integer arithmetic is exact.
+    // Returns sum w_i X_i, the block scale applied.
+    static constexpr bool HAS_DOT8 = true;
+    __device__ static float dot8(const uint64_t *, const uint8_t *blk, int, const uint32_t *xl, const uint32_t *xh) {
+        const uint32_t e = blk[0];
+        if (e == 0xFFu) return 0.0f;
+        const float d = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
+        int pl = 0, ph = 0, nl = 0, nh = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t w = ld<uint32_t>(blk + 1 + 4 * i);
+#pragma unroll
+            for (int hi = 0; hi < 2; hi++) {  // low nibbles: elements 4i .. 4i+3; high nibbles: 16 + 4i ..
+                const uint32_t v = hi ? w >> 4 : w;
+                const int mag = (int)__builtin_amdgcn_perm(0x0C080604u, 0x03020100u, v & 0x07070707u);
+                const int neg = mag & (int)(((v >> 3) & 0x01010101u) * 0xFFu);
+                pl = __builtin_amdgcn_sdot4(mag, (int)xl[4 * hi + i], pl, false);
+                ph = __builtin_amdgcn_sdot4(mag, (int)xh[4 * hi + i], ph, false);
+                nl = __builtin_amdgcn_sdot4(neg, (int)xl[4 * hi + i], nl, false);
+                nh = __builtin_amdgcn_sdot4(neg, (int)xh[4 * hi + i], nh, false);
+            }
+        }
+        const int s2 = ((ph - 2 * nh) << 8) + (pl - 2 * nl);  // twice the sum: the table holds doubled values
+        return d * (0.5f * (float)s2);
+    }
     __device__ static void decode(const uint8_t *blk, int, float *w) {
         uint32_t e = blk[0];
         // 2^(e-127); e == 0 is the f32 denormal 2^-127; 0xFF (reserved) decodes the block to zeros

@@ -403,6 +403,106 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
     }
 }
 
+// Activations as 15-bit fixed point per 32-element block, two int8 planes (X = 256 hi + lo) and the
+// block's scale: what the formats with an integer dot product (Q::dot8) multiply against.
+struct ActsI8 {
+    uint32_t *xl, *xh;  // [rows][k / 4]: four elements a word
+    float *sx;          // [rows][k / 32]
+};
+
+__global__ __launch_bounds__(256) void acts_i8_prep(const float *__restrict__ X, size_t rows, int k, ActsI8 out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // four elements a thread, eight threads a block
+    if (i >= rows * (size_t)(k / 4)) return;  // whole groups of 8 lanes leave together (k % 32 == 0)
+    const float4 v = *(const float4 *)(X + 4 * i);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = max_row8(amax);
+    const bool live = amax > 0.0f && amax < INFINITY;
+    const float inv = live ? 32639.0f / amax : 0.0f;
+    const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                       __float2int_rn(v.w * inv)};
+    uint32_t wl = 0, wh = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int lo = ((Xq[e] + 128) & 255) - 128, hi = (Xq[e] - lo) >> 8;
+        wl |= (uint32_t)(lo & 255) << (8 * e);
+        wh |= (uint32_t)(hi & 255) << (8 * e);
+    }
+    out.xl[i] = wl;
+    out.xh[i] = wh;
+    if ((i & 7) == 0) out.sx[i >> 3] = live ? amax / 32639.0f : 0.0f;
+}
+
+// The decode-shaped grouped expert matmul (one activation row a group) on integer dot products: rows
+// staged through LDS as in moe_rows_staged, every 32-element unit multiplied by Q::dot8 against the
+// prepared activation planes.  Y[yrow[beg]] = W[e] x, or silu(Wa[e] x) * (Wb[e] x) with DUAL.
+template <class Q, bool DUAL, int G>
+__global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t *const *__restrict__ Wa,
+                                                                   const uint8_t *const *__restrict__ Wb,
+                                                                   size_t row_bytes, ActsI8 xq,
+                                                                   const int *__restrict__ gexp,
+                                                                   const int *__restrict__ offsets,
+                                                                   const int *__restrict__ xsel,
+                                                                   const int *__restrict__ yrow,
+                                                                   float *__restrict__ Y, int k, int n, int L,
+                                                                   int wave_lds) {
+    static_assert(Q::SEGS == 1 && Q::SEGLEN == 32, "units of 32 consecutive elements");
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
+    const auto *table = stage_table<Q>(staged_moe);  // before any wave leaves: it holds a barrier
+    const int grp = blockIdx.y;
+    const int beg = offsets[grp], cnt = offsets[grp + 1] - beg;
+    if (cnt == 0) return;
+    const int e = gexp[grp];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int R = 64 / L;
+    const int row0 = (blockIdx.x * ROWS_PER_WG + wave) * R;
+    if (row0 >= n) return;  // wave-uniform; the kernel has no barrier
+    const int nrows = min(R, n - row0);
+    uint8_t *ra = staged_moe + table_bytes<Q>() + (size_t)wave * wave_lds, *rb = ra + (DUAL ? wave_lds / 2 : 0);
+    {
+        const int pieces = (int)((size_t)nrows * row_bytes / G);
+        const uint8_t *sa = Wa[e] + (size_t)row0 * row_bytes;
+        const uint8_t *sb = DUAL ? Wb[e] + (size_t)row0 * row_bytes : nullptr;
+        for (int p0 = 0; p0 < pieces; p0 += 64) {
+            if (p0 + lane < pieces) {
+                if (G == 16) {
+                    async_load16(sa + (size_t)(p0 + lane) * 16, lds_offset_of(ra + (size_t)p0 * 16));
+                    if (DUAL) async_load16(sb + (size_t)(p0 + lane) * 16, lds_offset_of(rb + (size_t)p0 * 16));
+                } else {
+                    async_load4(sa + (size_t)(p0 + lane) * 4, lds_offset_of(ra + (size_t)p0 * 4));
+                    if (DUAL) async_load4(sb + (size_t)(p0 + lane) * 4, lds_offset_of(rb + (size_t)p0 * 4));
+                }
+            }
+        }
+    }
+    const int sub = lane % L, rl = lane / L, row = row0 + rl;
+    const bool active = rl < nrows;
+    const uint8_t *rpa = ra + (size_t)rl * row_bytes, *rpb = rb + (size_t)rl * row_bytes;
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    const size_t xr = (size_t)xsel[beg];
+    const uint32_t *xlp = xq.xl + xr * (size_t)(k / 4), *xhp = xq.xh + xr * (size_t)(k / 4);
+    const float *sxp = xq.sx + xr * (size_t)(k / 32);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows landed (this wave's own data)
+    float acc = 0.0f, acc2 = 0.0f;
+    if (active) {
+        for (int u = sub; u < units; u += L) {
+            const int b = u / Q::UNITS, ub = u % Q::UNITS;
+            const int el = b * Q::BLOCK_ELEMS + Q::elem_base(ub);  // a multiple of 32
+            const uint4 l0 = *(const uint4 *)(xlp + el / 4), l1 = *(const uint4 *)(xlp + el / 4 + 4);
+            const uint4 h0 = *(const uint4 *)(xhp + el / 4), h1 = *(const uint4 *)(xhp + el / 4 + 4);
+            const uint32_t xl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+            const uint32_t xh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+            const float sx = sxp[el / 32];
+            acc = fmaf(sx, Q::dot8(table, rpa + (size_t)b * Q::BLOCK_BYTES, ub, xl, xh), acc);
+            if (DUAL) acc2 = fmaf(sx, Q::dot8(table, rpb + (size_t)b * Q::BLOCK_BYTES, ub, xl, xh), acc2);
+        }
+    }
+    for (int off = L >> 1; off > 0; off >>= 1) {
+        acc += __shfl_xor(acc, off, 64);
+        if (DUAL) acc2 += __shfl_xor(acc2, off, 64);
+    }
+    if (sub == 0 && active) Y[(size_t)yrow[beg] * n + row] = DUAL ? silu(acc) * acc2 : acc;
+}
+
 // y[t, :] = sum_s w[t, s] * out[t*k + s, :]  (+ shared_out[t, :] of the shared expert),
 // slots added in order s = 0..k-1 (reference: src/quantized_qwen3_moe.rs:516-518,
 // src/quantized_deepseek2.rs:553-557).
