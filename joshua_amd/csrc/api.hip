@@ -659,7 +659,7 @@ struct jq_moe {
     uint32_t *ids = nullptr;
     int *gexp = nullptr, *offsets = nullptr, *xrow = nullptr, *yrow = nullptr;
     uint8_t *qacts = nullptr;  // activations as MFMA operand records (Q4_K experts, grouped path)
-    jq::ActsI8 qi8{nullptr, nullptr, nullptr};  // activations as int8 planes (decode path of the formats with Q::dot8)
+    jq::ActsI8 qi8{nullptr, nullptr, nullptr, nullptr};  // activations as int8 planes (decode path of the formats with Q::dot8)
     std::mutex mu;
 };
 
@@ -669,10 +669,10 @@ void moe_free_scratch(jq_moe *m) {
     for (void *p : {(void *)m->logits, (void *)m->wts, (void *)m->G, (void *)m->U, (void *)m->out, (void *)m->sG,
                     (void *)m->sU, (void *)m->sH, (void *)m->sOut, (void *)m->ids, (void *)m->gexp,
                     (void *)m->offsets, (void *)m->xrow, (void *)m->yrow, (void *)m->qacts, (void *)m->qi8.xl,
-                    (void *)m->qi8.xh, (void *)m->qi8.sx})
+                    (void *)m->qi8.xh, (void *)m->qi8.sx, (void *)m->qi8.sxs})
         if (p) (void)hipFree(p);
     m->qacts = nullptr;
-    m->qi8 = jq::ActsI8{nullptr, nullptr, nullptr};
+    m->qi8 = jq::ActsI8{nullptr, nullptr, nullptr, nullptr};
     m->logits = m->wts = m->G = m->U = m->out = m->sG = m->sU = m->sH = m->sOut = nullptr;
     m->ids = nullptr;
     m->gexp = m->offsets = m->xrow = m->yrow = nullptr;
@@ -680,7 +680,13 @@ void moe_free_scratch(jq_moe *m) {
 }
 
 // Formats whose decode-shaped expert matmuls run on integer dot products (Q::dot8).
-bool moe_has_dot8(uint32_t type) { return type == JQ_TYPE_MXFP4 && !getenv("JQ_MOE_NO_DOT8"); }
+bool moe_has_dot8(uint32_t type) {
+    static const char *env = getenv("JQ_MOE_DOT8");  // "0": none; a list of type ids ("39,16"): those only
+    if (type != JQ_TYPE_MXFP4 && type != JQ_TYPE_IQ2_XXS && type != JQ_TYPE_Q4_K) return false;
+    if (!env) return true;
+    const std::string list = std::string(",") + env + ",";
+    return list.find("," + std::to_string(type) + ",") != std::string::npos;
+}
 
 int moe_reserve(jq_moe *m, size_t T) {
     if (T <= m->cap_tokens) return 0;
@@ -703,6 +709,7 @@ int moe_reserve(jq_moe *m, size_t T) {
         HIP_TRY(hipMalloc((void **)&m->qi8.xl, words * sizeof(uint32_t) + 16));
         HIP_TRY(hipMalloc((void **)&m->qi8.xh, words * sizeof(uint32_t) + 16));
         HIP_TRY(hipMalloc((void **)&m->qi8.sx, (words / 8 + 1) * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&m->qi8.sxs, (words / 8 + 1) * sizeof(float)));
     }
     if (m->gate->type == JQ_TYPE_Q4_K || m->down->type == JQ_TYPE_Q4_K)
         HIP_TRY(hipMalloc((void **)&m->qacts, std::max(T * (c.hidden / 256), PR * (c.inter / 256)) * jq::QS_REC + 16));
@@ -842,6 +849,10 @@ int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *co
     switch (type) {
     case JQ_TYPE_MXFP4:
         return launch_moe_dot8<jq::MXFP4, DUAL>(Wa, Wb, row_bytes, aligned16, xq, gexp, offsets, xsel, yrow, Y, k, n, groups, s);
+    case JQ_TYPE_IQ2_XXS:
+        return launch_moe_dot8<jq::IQ2_XXS, DUAL>(Wa, Wb, row_bytes, aligned16, xq, gexp, offsets, xsel, yrow, Y, k, n, groups, s);
+    case JQ_TYPE_Q4_K:
+        return launch_moe_dot8<jq::Q4_K, DUAL>(Wa, Wb, row_bytes, aligned16, xq, gexp, offsets, xsel, yrow, Y, k, n, groups, s);
     default: return -1;
     }
 }

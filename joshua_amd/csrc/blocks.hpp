@@ -202,6 +202,31 @@ struct Q4_K {  // d | dmin | scales[12] | qs[128]   (reference: src/kquant_dot.r
             }
         }
     }
+    // Unit c (64 elements: the low and the high nibbles of 32 bytes) against its activations as two
+    // int8 planes, 16 registers a plane; sx, sxs: scale and scale * sum X of the two 32-element blocks.
+    static constexpr bool HAS_DOT8 = true;
+    __device__ static float dot8(const uint64_t *, const uint8_t *blk, int c, const uint32_t *xl, const uint32_t *xh,
+                                 const float *sx, const float *sxs) {
+        const uint4 hdr = ld<uint4>(blk);
+        uint32_t sc0, mn0, sc1, mn1;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc0, mn0);
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc1, mn1);
+        const uint4 qa = ld<uint4>(blk + 16 + 32 * c), qb = ld<uint4>(blk + 32 + 32 * c);
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        int l0 = 0, h0 = 0, l1 = 0, h1 = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int lo4 = (int)(q[i] & 0x0F0F0F0Fu), hi4 = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+            l0 = __builtin_amdgcn_sdot4(lo4, (int)xl[i], l0, false);
+            h0 = __builtin_amdgcn_sdot4(lo4, (int)xh[i], h0, false);
+            l1 = __builtin_amdgcn_sdot4(hi4, (int)xl[8 + i], l1, false);
+            h1 = __builtin_amdgcn_sdot4(hi4, (int)xh[8 + i], h1, false);
+        }
+        const float d = f16_bits(hdr.x), dmin = f16_bits(hdr.x >> 16);
+        const float f0 = (float)((h0 << 8) + l0) * sx[0], f1 = (float)((h1 << 8) + l1) * sx[1];
+        const float acc = d * fmaf((float)sc0, f0, (float)sc1 * f1);
+        return fmaf(-dmin, fmaf((float)mn0, sxs[0], (float)mn1 * sxs[1]), acc);
+    }
 };
 
 struct Q2_K {  // scales[16] | qs[64] | d | dmin   (reference: src/kquant_dot.rs:63-76,345-385)
@@ -288,6 +313,35 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
         }
     }
     __device__ static void decode(const uint8_t *blk, int u, float *w) { decode_with(g_tables.iq2xxs_grid, blk, u, w); }
+    // Unit u (32 elements) against its activations as two int8 planes: the codebook's magnitude bytes go
+    // to v_dot4 as they are; the 8 sign bits of a group are spread to byte masks (a multiply moves bit j
+    // of a nibble to bit 8j) and a negative element counts twice in a second sum instead of being negated.
+    static constexpr bool HAS_DOT8 = true;
+    __device__ static float dot8(const uint64_t *grid_table, const uint8_t *blk, int u, const uint32_t *xl,
+                                 const uint32_t *xh, const float *sx, const float *) {
+        const float d = f16_bits(ld<uint16_t>(blk));
+        const uint2 g = ld<uint2>(blk + 2 + 8 * u);
+        const uint32_t lo = g.x, hi = g.y;
+        int pl = 0, ph = 0, nl = 0, nh = 0;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint64_t grid = grid_table[(lo >> (8 * l)) & 0xFFu];
+            const uint32_t s7 = (hi >> (7 * l)) & 127u;
+            const uint32_t signs = s7 | ((__popc(s7) & 1u) << 7);
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {  // elements 8l + 4hf .. + 3
+                const int mag = (int)(uint32_t)(grid >> (32 * hf));
+                const uint32_t bits = ((signs >> (4 * hf)) & 15u) * 0x00204081u & 0x01010101u;
+                const int neg = mag & (int)(bits * 0xFFu);
+                pl = __builtin_amdgcn_sdot4(mag, (int)xl[2 * l + hf], pl, false);
+                ph = __builtin_amdgcn_sdot4(mag, (int)xh[2 * l + hf], ph, false);
+                nl = __builtin_amdgcn_sdot4(neg, (int)xl[2 * l + hf], nl, false);
+                nh = __builtin_amdgcn_sdot4(neg, (int)xh[2 * l + hf], nh, false);
+            }
+        }
+        const float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
+        return sx[0] * db * (float)(((ph - 2 * nh) << 8) + (pl - 2 * nl));
+    }
 };
 
 struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
@@ -305,9 +359,10 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
     // lo, eight registers a plane): v_perm_b32 looks four magnitude codes up at once in the table of
     // doubled E2M1 values {0,1,2,3,4,6,8,12}; a negative element counts twice in a second sum instead of
     // being negated (sum w X = sum |w| X - 2 sum_{w<0} |w| X), so the integer arithmetic is exact.
-    // Returns sum w_i X_i, the block scale applied.
+    // Returns sum w_i x_i over the block: sx is the activations' scale, x = sx X.
     static constexpr bool HAS_DOT8 = true;
-    __device__ static float dot8(const uint64_t *, const uint8_t *blk, int, const uint32_t *xl, const uint32_t *xh) {
+    __device__ static float dot8(const uint64_t *, const uint8_t *blk, int, const uint32_t *xl, const uint32_t *xh,
+                                 const float *sx, const float *) {
         const uint32_t e = blk[0];
         if (e == 0xFFu) return 0.0f;
         const float d = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
@@ -327,7 +382,7 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
             }
         }
         const int s2 = ((ph - 2 * nh) << 8) + (pl - 2 * nl);  // twice the sum: the table holds doubled values
-        return d * (0.5f * (float)s2);
+        return sx[0] * d * (0.5f * (float)s2);
     }
     __device__ static void decode(const uint8_t *blk, int, float *w) {
         uint32_t e = blk[0];

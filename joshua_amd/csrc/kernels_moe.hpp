@@ -407,7 +407,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
 // block's scale: what the formats with an integer dot product (Q::dot8) multiply against.
 struct ActsI8 {
     uint32_t *xl, *xh;  // [rows][k / 4]: four elements a word
-    float *sx;          // [rows][k / 32]
+    float *sx, *sxs;    // [rows][k / 32]: the block's scale, and scale * sum of its fixed-point values
 };
 
 __global__ __launch_bounds__(256) void acts_i8_prep(const float *__restrict__ X, size_t rows, int k, ActsI8 out) {
@@ -421,15 +421,22 @@ __global__ __launch_bounds__(256) void acts_i8_prep(const float *__restrict__ X,
     const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
                        __float2int_rn(v.w * inv)};
     uint32_t wl = 0, wh = 0;
+    int sum = 0;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
         const int lo = ((Xq[e] + 128) & 255) - 128, hi = (Xq[e] - lo) >> 8;
         wl |= (uint32_t)(lo & 255) << (8 * e);
         wh |= (uint32_t)(hi & 255) << (8 * e);
+        sum += Xq[e];
     }
     out.xl[i] = wl;
     out.xh[i] = wh;
-    if ((i & 7) == 0) out.sx[i >> 3] = live ? amax / 32639.0f : 0.0f;
+    sum = isum_row8(sum);
+    if ((i & 7) == 0) {
+        const float s = live ? amax / 32639.0f : 0.0f;
+        out.sx[i >> 3] = s;
+        out.sxs[i >> 3] = s * (float)sum;
+    }
 }
 
 // The decode-shaped grouped expert matmul (one activation row a group) on integer dot products: rows
@@ -445,7 +452,8 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
                                                                    const int *__restrict__ yrow,
                                                                    float *__restrict__ Y, int k, int n, int L,
                                                                    int wave_lds) {
-    static_assert(Q::SEGS == 1 && Q::SEGLEN == 32, "units of 32 consecutive elements");
+    static_assert(Q::SEGS == 1 && Q::SEGLEN % 32 == 0, "units of 32 or 64 consecutive elements");
+    constexpr int XW = Q::SEGLEN / 4, NS = Q::SEGLEN / 32;  // activation words a plane, scales a unit
     extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
     const auto *table = stage_table<Q>(staged_moe);  // before any wave leaves: it holds a barrier
     const int grp = blockIdx.y;
@@ -480,20 +488,25 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
     const size_t xr = (size_t)xsel[beg];
     const uint32_t *xlp = xq.xl + xr * (size_t)(k / 4), *xhp = xq.xh + xr * (size_t)(k / 4);
-    const float *sxp = xq.sx + xr * (size_t)(k / 32);
+    const float *sxp = xq.sx + xr * (size_t)(k / 32), *sxsp = xq.sxs + xr * (size_t)(k / 32);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows landed (this wave's own data)
     float acc = 0.0f, acc2 = 0.0f;
     if (active) {
         for (int u = sub; u < units; u += L) {
             const int b = u / Q::UNITS, ub = u % Q::UNITS;
             const int el = b * Q::BLOCK_ELEMS + Q::elem_base(ub);  // a multiple of 32
-            const uint4 l0 = *(const uint4 *)(xlp + el / 4), l1 = *(const uint4 *)(xlp + el / 4 + 4);
-            const uint4 h0 = *(const uint4 *)(xhp + el / 4), h1 = *(const uint4 *)(xhp + el / 4 + 4);
-            const uint32_t xl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
-            const uint32_t xh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
-            const float sx = sxp[el / 32];
-            acc = fmaf(sx, Q::dot8(table, rpa + (size_t)b * Q::BLOCK_BYTES, ub, xl, xh), acc);
-            if (DUAL) acc2 = fmaf(sx, Q::dot8(table, rpb + (size_t)b * Q::BLOCK_BYTES, ub, xl, xh), acc2);
+            uint32_t xl[XW], xh[XW];
+            float sx[NS], sxs[NS];
+#pragma unroll
+            for (int i = 0; i < XW; i += 4) {
+                const uint4 lw = *(const uint4 *)(xlp + el / 4 + i), hw = *(const uint4 *)(xhp + el / 4 + i);
+                xl[i] = lw.x, xl[i + 1] = lw.y, xl[i + 2] = lw.z, xl[i + 3] = lw.w;
+                xh[i] = hw.x, xh[i + 1] = hw.y, xh[i + 2] = hw.z, xh[i + 3] = hw.w;
+            }
+#pragma unroll
+            for (int i = 0; i < NS; i++) sx[i] = sxp[el / 32 + i], sxs[i] = sxsp[el / 32 + i];
+            acc += Q::dot8(table, rpa + (size_t)b * Q::BLOCK_BYTES, ub, xl, xh, sx, sxs);
+            if (DUAL) acc2 += Q::dot8(table, rpb + (size_t)b * Q::BLOCK_BYTES, ub, xl, xh, sx, sxs);
         }
     }
     for (int off = L >> 1; off > 0; off >>= 1) {
