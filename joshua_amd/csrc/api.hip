@@ -659,7 +659,7 @@ struct jq_moe {
     uint32_t *ids = nullptr;
     int *gexp = nullptr, *offsets = nullptr, *xrow = nullptr, *yrow = nullptr;
     uint8_t *qacts = nullptr;  // activations as MFMA operand records (Q4_K experts, grouped path)
-    jq::ActsI8 qi8{nullptr, nullptr, nullptr, nullptr};  // activations as int8 planes (decode path of the formats with Q::dot8)
+    jq::ActsI8 qi8{nullptr, nullptr, nullptr, nullptr};  // activations as int8 planes (decode path, long rows)
     std::mutex mu;
 };
 
@@ -815,26 +815,36 @@ int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, si
     return 0;
 }
 
-// One activation row a group, a format with Q::dot8: the activations become int8 planes once, the
-// expert rows are staged through LDS and multiplied on v_dot4.  Returns -1 when the shape is outside
-// its reach.
+// One activation row a group, a format with Q::dot8: expert rows staged through LDS and multiplied on
+// v_dot4 against the activation row as int8 planes, quantised by every workgroup itself (small
+// matrices) or once by acts_i8_prep (x_rows rows of X).  Returns -1 when the shape is outside its reach.
 template <class Q, bool DUAL>
-int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16, jq::ActsI8 xq,
-                    const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
-                    int groups, hipStream_t s) {
+int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16, const float *X,
+                    size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets, const int *xsel, const int *yrow,
+                    float *Y, int k, int n, int groups, hipStream_t s) {
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
     const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
+    // every workgroup of a group redoing the row's quantisation is cheaper than a launch up to about
+    // half a million elements a group
+    const size_t wgs = (n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R);
+    const bool own = wgs * (size_t)k <= 512 * 1024 || !xq.xl;
     const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
-    const size_t lds = wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>();
+    const size_t lds = wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>() + (own ? (size_t)k * 2 + (size_t)k / 4 : 0);
     if (G == 0 || lds > 64 * 1024) return -1;
-    dim3 grid((unsigned)((n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R)), (unsigned)groups), block(64 * jq::ROWS_PER_WG);
-    if (G == 16)
-        hipLaunchKernelGGL((jq::moe_rows_dot8<Q, DUAL, 16>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp, offsets, xsel,
-                           yrow, Y, k, n, L, (int)wave_lds);
-    else
-        hipLaunchKernelGGL((jq::moe_rows_dot8<Q, DUAL, 4>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp, offsets, xsel,
-                           yrow, Y, k, n, L, (int)wave_lds);
+    if (!own) {
+        const size_t words = x_rows * (size_t)(k / 4);
+        hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
+    }
+    dim3 grid((unsigned)wgs, (unsigned)groups), block(64 * jq::ROWS_PER_WG);
+#define JQ_DOT8(GG, OWN)                                                                                          \
+    hipLaunchKernelGGL((jq::moe_rows_dot8<Q, DUAL, GG, OWN>), grid, block, lds, s, Wa, Wb, row_bytes, X, xq, gexp,  \
+                       offsets, xsel, yrow, Y, k, n, L, (int)wave_lds)
+    if (G == 16 && own) JQ_DOT8(16, true);
+    else if (G == 16) JQ_DOT8(16, false);
+    else if (own) JQ_DOT8(4, true);
+    else JQ_DOT8(4, false);
+#undef JQ_DOT8
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -843,16 +853,16 @@ template <bool DUAL>
 int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
                       const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets,
                       const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s) {
-    if (!moe_has_dot8(type) || !xq.xl || k % 32 != 0 || ((uintptr_t)X & 15) != 0) return -1;
-    const size_t words = x_rows * (size_t)(k / 4);
-    hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
+    if (!moe_has_dot8(type) || k % 32 != 0 || ((uintptr_t)X & 15) != 0) return -1;
     switch (type) {
-    case JQ_TYPE_MXFP4:
-        return launch_moe_dot8<jq::MXFP4, DUAL>(Wa, Wb, row_bytes, aligned16, xq, gexp, offsets, xsel, yrow, Y, k, n, groups, s);
-    case JQ_TYPE_IQ2_XXS:
-        return launch_moe_dot8<jq::IQ2_XXS, DUAL>(Wa, Wb, row_bytes, aligned16, xq, gexp, offsets, xsel, yrow, Y, k, n, groups, s);
-    case JQ_TYPE_Q4_K:
-        return launch_moe_dot8<jq::Q4_K, DUAL>(Wa, Wb, row_bytes, aligned16, xq, gexp, offsets, xsel, yrow, Y, k, n, groups, s);
+#define JQ_DOT8_CASE(ID, Q)                                                                                         \
+    case ID:                                                                                                        \
+        return launch_moe_dot8<jq::Q, DUAL>(Wa, Wb, row_bytes, aligned16, X, x_rows, xq, gexp, offsets, xsel, yrow, Y, k, n, \
+                                            groups, s);
+        JQ_DOT8_CASE(JQ_TYPE_MXFP4, MXFP4)
+        JQ_DOT8_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
+        JQ_DOT8_CASE(JQ_TYPE_Q4_K, Q4_K)
+#undef JQ_DOT8_CASE
     default: return -1;
     }
 }

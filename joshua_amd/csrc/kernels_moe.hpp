@@ -440,13 +440,18 @@ __global__ __launch_bounds__(256) void acts_i8_prep(const float *__restrict__ X,
 }
 
 // The decode-shaped grouped expert matmul (one activation row a group) on integer dot products: rows
-// staged through LDS as in moe_rows_staged, every 32-element unit multiplied by Q::dot8 against the
-// prepared activation planes.  Y[yrow[beg]] = W[e] x, or silu(Wa[e] x) * (Wb[e] x) with DUAL.
-template <class Q, bool DUAL, int G>
+// staged through LDS as in moe_rows_staged, every unit of 32 or 64 elements multiplied by Q::dot8
+// against the group's activation row as 15-bit fixed point per 32-element block (ActsI8).  OWN_PREP:
+// the workgroup quantises the row itself into LDS while its rows are on their way (short rows: cheaper
+// than one more launch); otherwise the planes come from acts_i8_prep (long rows: quantising 7168
+// elements in each of thousands of workgroups costs more than it saves).
+// Y[yrow[beg]] = W[e] x, or silu(Wa[e] x) * (Wb[e] x) with DUAL.
+// Dynamic LDS: the format's table, ROWS_PER_WG * wave_lds of staged rows, with OWN_PREP 2.25 k more.
+template <class Q, bool DUAL, int G, bool OWN_PREP>
 __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t *const *__restrict__ Wa,
                                                                    const uint8_t *const *__restrict__ Wb,
-                                                                   size_t row_bytes, ActsI8 xq,
-                                                                   const int *__restrict__ gexp,
+                                                                   size_t row_bytes, const float *__restrict__ X,
+                                                                   ActsI8 xq, const int *__restrict__ gexp,
                                                                    const int *__restrict__ offsets,
                                                                    const int *__restrict__ xsel,
                                                                    const int *__restrict__ yrow,
@@ -458,15 +463,14 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
     const auto *table = stage_table<Q>(staged_moe);  // before any wave leaves: it holds a barrier
     const int grp = blockIdx.y;
     const int beg = offsets[grp], cnt = offsets[grp + 1] - beg;
-    if (cnt == 0) return;
+    if (cnt == 0) return;  // the whole workgroup
     const int e = gexp[grp];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int R = 64 / L;
     const int row0 = (blockIdx.x * ROWS_PER_WG + wave) * R;
-    if (row0 >= n) return;  // wave-uniform; the kernel has no barrier
-    const int nrows = min(R, n - row0);
+    const int nrows = min(R, n - row0);  // <= 0: this wave has no rows and only helps with the activations
     uint8_t *ra = staged_moe + table_bytes<Q>() + (size_t)wave * wave_lds, *rb = ra + (DUAL ? wave_lds / 2 : 0);
-    {
+    if (nrows > 0) {
         const int pieces = (int)((size_t)nrows * row_bytes / G);
         const uint8_t *sa = Wa[e] + (size_t)row0 * row_bytes;
         const uint8_t *sb = DUAL ? Wb[e] + (size_t)row0 * row_bytes : nullptr;
@@ -482,13 +486,47 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
             }
         }
     }
+    const size_t xr = (size_t)xsel[beg];
+    const uint32_t *xlp = xq.xl + xr * (size_t)(k / 4), *xhp = xq.xh + xr * (size_t)(k / 4);
+    const float *sxp = xq.sx + xr * (size_t)(k / 32), *sxsp = xq.sxs + xr * (size_t)(k / 32);
+    if (OWN_PREP) {  // four elements a thread, eight threads a 32-element block (k % 32 == 0)
+        uint32_t *xl_lds = (uint32_t *)(staged_moe + table_bytes<Q>() + (size_t)ROWS_PER_WG * wave_lds), *xh_lds = xl_lds + k / 4;
+        float *sx_lds = (float *)(xh_lds + k / 4), *sxs_lds = sx_lds + k / 32;
+        const float *xrow = X + xr * k;
+        for (int i = threadIdx.x; i < k / 4; i += 64 * ROWS_PER_WG) {
+            const float4 v = *(const float4 *)(xrow + 4 * i);
+            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+            amax = max_row8(amax);
+            const bool live = amax > 0.0f && amax < INFINITY;
+            const float inv = live ? 32639.0f / amax : 0.0f;
+            const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                               __float2int_rn(v.w * inv)};
+            uint32_t wl = 0, wh = 0;
+            int sum = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int lo = ((Xq[j] + 128) & 255) - 128, hi = (Xq[j] - lo) >> 8;
+                wl |= (uint32_t)(lo & 255) << (8 * j);
+                wh |= (uint32_t)(hi & 255) << (8 * j);
+                sum += Xq[j];
+            }
+            xl_lds[i] = wl;
+            xh_lds[i] = wh;
+            sum = isum_row8(sum);
+            if ((i & 7) == 0) {
+                const float s = live ? amax / 32639.0f : 0.0f;
+                sx_lds[i >> 3] = s;
+                sxs_lds[i >> 3] = s * (float)sum;
+            }
+        }
+        __syncthreads();
+        xlp = xl_lds, xhp = xh_lds, sxp = sx_lds, sxsp = sxs_lds;
+    }
+    if (nrows <= 0) return;
     const int sub = lane % L, rl = lane / L, row = row0 + rl;
     const bool active = rl < nrows;
     const uint8_t *rpa = ra + (size_t)rl * row_bytes, *rpb = rb + (size_t)rl * row_bytes;
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
-    const size_t xr = (size_t)xsel[beg];
-    const uint32_t *xlp = xq.xl + xr * (size_t)(k / 4), *xhp = xq.xh + xr * (size_t)(k / 4);
-    const float *sxp = xq.sx + xr * (size_t)(k / 32), *sxsp = xq.sxs + xr * (size_t)(k / 32);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows landed (this wave's own data)
     float acc = 0.0f, acc2 = 0.0f;
     if (active) {

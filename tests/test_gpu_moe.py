@@ -114,6 +114,15 @@ def test_row_lengths_that_change_the_staging(qtype, h, inter):
         assert close(dev.forward(x), ora.forward(x))
 
 
+@pytest.mark.parametrize("qtype", [capi.Q4_K, capi.MXFP4, capi.IQ2_XXS])
+def test_decode_sized_call_over_large_expert_matrices(qtype):
+    """One token, expert matrices large enough that the integer-dot kernels take their activations
+    from the separate quantisation launch rather than quantising them in every workgroup."""
+    ora, dev = build(qtype, 2048, 4352, 2, 1, 120)
+    x = synth.normal(121, (1, 2048))
+    assert close(dev.forward(x), ora.forward(x))
+
+
 def test_many_tokens_group_beyond_the_lds_pair_list():
     ora, dev = build(capi.Q8_0, 64, 32, 4, 2, 110)
     x = synth.normal(111, (6200, 64))          # 12400 pairs
