@@ -1148,6 +1148,7 @@ struct jq_model {
     int *pick_i = nullptr;
     int *pos = nullptr;       // device copy of the position of the step being run
     float *part = nullptr;    // split-attention partials
+    float2 *rope_cs = nullptr;  // (cos, sin) of the rotary angles of a step's tokens, [8][head_dim / 2]
     float *x2 = nullptr;      // second residual row of a single-token step (the fused norm + matmul launches alternate)
     float *x = nullptr, *hn = nullptr, *qb = nullptr, *kb = nullptr, *vb = nullptr, *att = nullptr, *proj = nullptr,
           *g = nullptr, *u = nullptr, *mid = nullptr, *logits = nullptr;
@@ -1319,10 +1320,11 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
     auto emb = m->q.find("token_embd.weight");
     if (emb == m->q.end()) return fail("qwen3: missing tensor `token_embd.weight`");
     if (dispatch_decode(emb->second, m->ids, m->x, T, s)) return 1;
-    hipLaunchKernelGGL(jq::set_int, dim3(1), dim3(1), 0, s, m->pos, (int)pos);
-    const float sqrt_d = sqrtf((float)d);
     // few query rows over a long cache: split the keys over the chip
     const bool split = T <= 8 && (d == 64 || d == 128 || d == 256);
+    // the step's position for the kernels, and with split attention the rotary angles of its tokens
+    hipLaunchKernelGGL(jq::rope_table, dim3(1), dim3(256), 0, s, m->pos, (int)pos, split ? (int)T : 0, d, c.rope_theta, m->rope_cs);
+    const float sqrt_d = sqrtf((float)d);
     const int n_chunks = (int)((pos + T + jq::ATT_CHUNK - 1) / jq::ATT_CHUNK);
     const float *pending = nullptr;  // residual not yet added into x
     float *xc = m->x, *xo = m->x2;   // the residual stream, and where a fused norm + matmul launch writes its update
@@ -1351,12 +1353,11 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
                    model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s)) {
             return 1;
         }
-        hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, qp, kp, vp, w_qn, w_kn,
-                           c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
-        if (split) {
+        if (split) {  // head norm, rotation and cache writes happen inside the attention kernel
 #define JQ_ATT_SPLIT(D)                                                                                          \
-    hipLaunchKernelGGL(jq::attention_split<D>, dim3(T * nh * n_chunks), dim3(256), 0, s, qp, m->kc[l], m->vc[l], \
-                       m->part, nh, nkv, m->pos, (int)c.n_ctx, sqrt_d, n_chunks)
+    hipLaunchKernelGGL(jq::attention_split<D>, dim3(T * nh * n_chunks), dim3(256), 0, s, qp, kp, vp, w_qn, w_kn,   \
+                       c.rms_eps, m->rope_cs, m->kc[l], m->vc[l], m->part, nh, nkv, m->pos, (int)c.n_ctx, sqrt_d, \
+                       n_chunks)
             if (d == 64) JQ_ATT_SPLIT(64);
             else if (d == 128) JQ_ATT_SPLIT(128);
             else JQ_ATT_SPLIT(256);
@@ -1364,6 +1365,8 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             hipLaunchKernelGGL(jq::attention_merge, dim3(T * nh), dim3(128), 2 * n_chunks * sizeof(float), s, m->part, m->att, d,
                                n_chunks);
         } else {
+            hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, qp, kp, vp, w_qn, w_kn,
+                               c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
             size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
             hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, qp, m->kc[l], m->vc[l], m->att, nh,
                                nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
@@ -1441,7 +1444,8 @@ int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out) {
         hipMalloc((void **)&m->pick_v, jq::ARGMAX_PARTS * sizeof(float)) != hipSuccess ||
         hipMalloc((void **)&m->pick_i, jq::ARGMAX_PARTS * sizeof(int)) != hipSuccess ||
         hipMalloc((void **)&m->pos, sizeof(int)) != hipSuccess ||
-        hipMalloc((void **)&m->part, part_floats * sizeof(float)) != hipSuccess) {
+        hipMalloc((void **)&m->part, part_floats * sizeof(float)) != hipSuccess ||
+        hipMalloc((void **)&m->rope_cs, (size_t)8 * (c.head_dim / 2) * sizeof(float2)) != hipSuccess) {
         jq_qwen3_free(m);
         return fail("qwen3: logits allocation failed");
     }
@@ -1465,6 +1469,7 @@ void jq_qwen3_free(jq_model *m) {
     if (m->pick_i) (void)hipFree(m->pick_i);
     if (m->pos) (void)hipFree(m->pos);
     if (m->part) (void)hipFree(m->part);
+    if (m->rope_cs) (void)hipFree(m->rope_cs);
     delete m;
 }
 

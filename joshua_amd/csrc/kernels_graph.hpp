@@ -144,6 +144,64 @@ __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ 
     }
 }
 
+// *pos = p, and the rotary angles of the T positions p .. p + T - 1 of a step: cs[t][i] = (cos, sin) of
+// (p + t) * theta^(-2i/d), i < d/2 — the arithmetic of qkv_norm_rope_cache, done once a step for the
+// attention kernel that applies head norm and rotation itself.
+__global__ __launch_bounds__(256) void rope_table(int *pos, int p, int T, int d, float theta, float2 *__restrict__ cs) {
+    if (threadIdx.x == 0) *pos = p;
+    const int half = d / 2;
+    for (int e = threadIdx.x; e < T * half; e += blockDim.x) {
+        const int t = e / half, i = e % half;
+        const float freq = 1.0f / powf(theta, (float)(2 * i) / (float)d);
+        const float ang = (float)(p + t) * freq;
+        cs[e] = float2{cosf(ang), sinf(ang)};
+    }
+}
+
+// One head row held by 16 lanes (lane `sub` has elements 4 sub + 64 i + c, i < D / 64, c < 4):
+// RMSNorm over the head with weight w, then the half-split rotation by the angles cs[0 .. D/2)
+// (reference: src/quantized_qwen3_moe.rs:237-262,345-364).  Same arithmetic as qkv_norm_rope_cache.
+template <int D>
+__device__ __forceinline__ void head_norm_rope(float4 (&x)[D / 64], const float *__restrict__ w, float eps,
+                                               const float2 *__restrict__ cs, int sub) {
+    constexpr int QI = D / 64;
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < QI; i++)
+        ss = fmaf(x[i].x, x[i].x, ss), ss = fmaf(x[i].y, x[i].y, ss), ss = fmaf(x[i].z, x[i].z, ss), ss = fmaf(x[i].w, x[i].w, ss);
+    ss = sum_row16(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+    float v[QI][4];
+#pragma unroll
+    for (int i = 0; i < QI; i++) {
+        const float4 g = *(const float4 *)(w + 4 * sub + 64 * i);
+        v[i][0] = x[i].x * inv * g.x, v[i][1] = x[i].y * inv * g.y, v[i][2] = x[i].z * inv * g.z, v[i][3] = x[i].w * inv * g.w;
+    }
+    if constexpr (QI >= 2) {  // element e < D/2 and its partner e + D/2 sit in the same lane
+#pragma unroll
+        for (int i = 0; i < QI / 2; i++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const float2 r = cs[4 * sub + 64 * i + c];
+                const float a = v[i][c], b = v[i + QI / 2][c];
+                v[i][c] = a * r.x - b * r.y;
+                v[i + QI / 2][c] = a * r.y + b * r.x;
+            }
+        }
+    } else {  // D = 64: the partner is 8 lanes away
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const float other = dpp_f<0x128>(v[0][c]);  // row_ror:8
+            const bool low = sub < 8;
+            const float2 r = cs[(4 * sub + c) & 31];
+            const float a = low ? v[0][c] : other, b = low ? other : v[0][c];
+            v[0][c] = low ? a * r.x - b * r.y : a * r.y + b * r.x;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < QI; i++) x[i] = float4{v[i][0], v[i][1], v[i][2], v[i][3]};
+}
+
 // Decode-shaped attention (few query tokens, long cache), split over the keys so the
 // whole chip works on it: one workgroup per (token, query head, chunk of ATT_CHUNK keys)
 // computes its chunk's scores, their maximum m, l = sum exp(s - m) and the unnormalised
@@ -151,45 +209,69 @@ __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ 
 // attention_merge rescales the chunks to the common maximum and divides by the total.
 // 16 lanes per key (4 keys per wave step), head_dim 64, 128 or 256.  Chunks past the causal
 // limit write l = 0 and are skipped by the merge.
+// q, k, v are the step's raw projections: the kernel applies the per-head RMSNorm and the rotation to
+// its query row and to the keys of the step's own tokens (positions *pos_ptr and up, not in the cache
+// yet) itself, and the workgroups of a kv head's first query head store the new key and value rows
+// into the cache for the steps to come.
 constexpr int ATT_CHUNK = 64;
 
 template <int D>  // head_dim: 64, 128 or 256
-__global__ __launch_bounds__(256) void attention_split(const float *__restrict__ q, const float *__restrict__ kc,
-                                                        const float *__restrict__ vc, float *__restrict__ part,
-                                                        int n_head, int n_kv, const int *__restrict__ pos_ptr, int n_ctx,
-                                                        float sqrt_d, int n_chunks) {
+__global__ __launch_bounds__(256) void attention_split(const float *__restrict__ q, const float *__restrict__ k,
+                                                        const float *__restrict__ v, const float *__restrict__ wq,
+                                                        const float *__restrict__ wk, float eps,
+                                                        const float2 *__restrict__ cs, float *kc, float *vc,
+                                                        float *__restrict__ part, int n_head, int n_kv,
+                                                        const int *__restrict__ pos_ptr, int n_ctx, float sqrt_d,
+                                                        int n_chunks) {
     constexpr int d = D, QI = D / 64;          // float4 of q (and of a key) per lane
     constexpr int NG = D / 4, KP = 256 / NG;   // column groups of four, key parts
     constexpr int VI = ATT_CHUNK / KP;         // keys per thread in the value sum
     __shared__ float sc[ATT_CHUNK];
     __shared__ float4 accs[256];               // [key part][column group]
     const int chunk = blockIdx.x % n_chunks, hq = (blockIdx.x / n_chunks) % n_head, t = blockIdx.x / (n_chunks * n_head);
-    const int kvh = hq / (n_head / n_kv), n_keys = *pos_ptr + t + 1;
+    const int group = n_head / n_kv, kvh = hq / group, pos0 = *pos_ptr, n_keys = pos0 + t + 1;
     const int j0 = chunk * ATT_CHUNK, nj = min(ATT_CHUNK, n_keys - j0);
     float *po = part + ((size_t)(t * n_head + hq) * n_chunks + chunk) * (d + 2);
     if (nj <= 0) {
         if (threadIdx.x == 0) po[0] = -INFINITY, po[1] = 0.0f;
         return;
     }
+    const bool keeper = hq % group == 0;  // stores this token's new key and value rows
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15, kq = lane >> 4;
     const float *qp = q + ((size_t)t * n_head + hq) * d;
-    const float *kb = kc + ((size_t)kvh * n_ctx + j0) * d;
     const int cg = threadIdx.x % NG, kp = threadIdx.x / NG;
-    const float *vb = vc + ((size_t)kvh * n_ctx + j0) * d + 4 * cg;
     // every global read of this workgroup is issued here, before any of them is needed: the query slice,
     // this lane's slices of its four keys, this thread's VI value rows (rows past the chunk's end are
-    // read from its last valid row and not used)
+    // read from its last valid row and not used); rows of this step's tokens come from k and v
     float4 qv[QI], kv[4][QI], vv[VI];
 #pragma unroll
     for (int i = 0; i < QI; i++) qv[i] = *(const float4 *)(qp + 4 * sub + 64 * i);
 #pragma unroll
     for (int s = 0; s < 4; s++) {
-        const int j = min(wave * 4 + kq + 16 * s, nj - 1);
+        const int jg = j0 + min(wave * 4 + kq + 16 * s, nj - 1);
+        const float *row = jg >= pos0 ? k + ((size_t)(jg - pos0) * n_kv + kvh) * d : kc + ((size_t)kvh * n_ctx + jg) * d;
 #pragma unroll
-        for (int i = 0; i < QI; i++) kv[s][i] = *(const float4 *)(kb + (size_t)j * d + 4 * sub + 64 * i);
+        for (int i = 0; i < QI; i++) kv[s][i] = *(const float4 *)(row + 4 * sub + 64 * i);
     }
 #pragma unroll
-    for (int s = 0; s < VI; s++) vv[s] = *(const float4 *)(vb + (size_t)min(kp + KP * s, nj - 1) * d);
+    for (int s = 0; s < VI; s++) {
+        const int jg = j0 + min(kp + KP * s, nj - 1);
+        const float *row = jg >= pos0 ? v + ((size_t)(jg - pos0) * n_kv + kvh) * d : vc + ((size_t)kvh * n_ctx + jg) * d;
+        vv[s] = *(const float4 *)(row + 4 * cg);
+    }
+    head_norm_rope<D>(qv, wq, eps, cs + (size_t)t * (d / 2), sub);
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int jg = j0 + min(wave * 4 + kq + 16 * s, nj - 1);
+        if (jg >= pos0) {  // a key of this step: the same for the 16 lanes that hold it
+            head_norm_rope<D>(kv[s], wk, eps, cs + (size_t)(jg - pos0) * (d / 2), sub);
+            if (keeper && jg == pos0 + t) {
+                float *dst = kc + ((size_t)kvh * n_ctx + jg) * d;
+#pragma unroll
+                for (int i = 0; i < QI; i++) *(float4 *)(dst + 4 * sub + 64 * i) = kv[s][i];
+            }
+        }
+    }
 
 #pragma unroll
     for (int s = 0; s < 4; s++) {
@@ -232,6 +314,13 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
         po[2 + 4 * threadIdx.x + 2] = a.z, po[2 + 4 * threadIdx.x + 3] = a.w;
     }
     if (threadIdx.x == 0) po[0] = mx, po[1] = l;
+    if (keeper) {  // this token's value row into the cache (its key row went in above)
+#pragma unroll
+        for (int s = 0; s < VI; s++) {
+            const int jg = j0 + min(kp + KP * s, nj - 1);
+            if (jg == pos0 + t) *(float4 *)(vc + ((size_t)kvh * n_ctx + jg) * d + 4 * cg) = vv[s];
+        }
+    }
 }
 
 // out[(t, head), :] = sum_ch exp(m_ch - m) acc_ch / sum_ch exp(m_ch - m) l_ch over the chunks with keys.
