@@ -194,3 +194,33 @@ def test_tied_embeddings_when_no_output_head():
     o = oq.Qwen3Oracle(CFG, tensors, avx2=oracle.have_avx2())
     ok, e = close(m.forward([9, 8, 7], 0), o.forward([9, 8, 7], 0))
     assert ok, e
+
+
+FALLBACK_CHILD = r"""
+import sys, numpy as np
+sys.path.insert(0, %r)
+from tests.test_gpu_qwen3 import CFG, make, close
+cfg = dict(CFG, n_layer=2, hidden=4096, n_head=4, n_kv_head=2, head_dim=128, ffn=512, vocab=512, n_ctx=32)
+m, o = make(cfg, 33, "q4_k")
+pos = 0
+for chunk in ([3, 500, 41], [7], [9], [256, 12]):
+    ok, e = close(m.forward(chunk, pos), o.forward(chunk, pos))
+    assert ok, (pos, e)
+    pos += len(chunk)
+print("fallback ok")
+"""
+
+
+@pytest.mark.parametrize("env", [{"JQ_Q4K_DOT4": "0"}, {"JQ_NO_FUSED_NORM": "1"}, {"JQ_NO_PAIRED_GATE_UP": "1"}])
+def test_single_token_steps_without_the_fused_launches(env):
+    """The switches are read when the library first dispatches, so each runs in a child process: without
+    the v_dot4 kernel the row-paired gate|up matrix goes through the plain product and a pairwise
+    SwiGLU; without the fused norm the pieces run as launches of their own; without pairing gate and up
+    are laid one after the other."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", FALLBACK_CHILD % root], env=dict(os.environ, **env), capture_output=True,
+                         text=True, timeout=110)
+    assert res.returncode == 0 and "fallback ok" in res.stdout, res.stdout + res.stderr
