@@ -15,6 +15,17 @@
 
 namespace jq {
 
+// |x|, or +inf when x is not finite (a NaN fails the comparison): the fixed-point quantisers take the
+// block maximum of these and give a block with a non-finite activation the scale NaN (fixed_scale), so
+// that the results say so instead of reading the block as zeros.
+__device__ __forceinline__ float mag_or_inf(float x) {
+    const float a = fabsf(x);
+    return a <= 3.402823466e38f ? a : INFINITY;
+}
+__device__ __forceinline__ float fixed_scale(float amax, float range) {
+    return amax > 0.0f ? (amax < INFINITY ? amax / range : NAN) : 0.0f;
+}
+
 // Sums over the aligned 16 (8) lanes around a lane, in every lane of the group, on the data-parallel
 // primitives (row rotations, half-row mirror, quad permutes): four (three) instructions with no trip
 // through LDS, where __shfl_xor costs a ds_bpermute each.

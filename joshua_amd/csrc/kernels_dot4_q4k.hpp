@@ -67,10 +67,10 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
     // ---- activation of this wave's super-block: lane i quantises elements 4i .. 4i+3 ----
     {
         const float4 v = *(const float4 *)(X + 256 * wave + 4 * lane);
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
         amax = max_row8(amax);  // the 8 lanes of a sub-block
         const bool live = amax > 0.0f && amax < INFINITY;
-        const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
+        const float inv = live ? QD_RANGE / amax : 0.0f, s = fixed_scale(amax, QD_RANGE);
         const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
                            __float2int_rn(v.w * inv)};
         uint32_t wl = 0, wh = 0;
@@ -230,10 +230,10 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
             v = float4{v.x * inv * g.x, v.y * inv * g.y, v.z * inv * g.z, v.w * inv * g.w};
             if (blockIdx.x == 0 && nm.hn_out) *(float4 *)(nm.hn_out + 256 * wave + 4 * lane) = v;
         }
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
         amax = max_row8(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
-        const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
+        const float inv = live ? QD_RANGE / amax : 0.0f, s = fixed_scale(amax, QD_RANGE);
         const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
                            __float2int_rn(v.w * inv)};
         uint32_t wl = 0, wh = 0;

@@ -49,10 +49,10 @@ __global__ __launch_bounds__(1024) void q6k_gemv_dot4_lds(const uint8_t *__restr
 #pragma unroll
     for (int g = 0; g < NG; g++) {
         const float4 v = *(const float4 *)(X + (size_t)(16 * g + wave) * 256 + 4 * lane);
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
         amax = max_row8(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
-        const float inv = live ? QD_RANGE / amax : 0.0f, s = live ? amax / QD_RANGE : 0.0f;
+        const float inv = live ? QD_RANGE / amax : 0.0f, s = fixed_scale(amax, QD_RANGE);
         const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
                            __float2int_rn(v.w * inv)};
         uint32_t wl = 0, wh = 0;

@@ -140,7 +140,7 @@ __global__ __launch_bounds__(64 * Q4K_MAX_WAVES) void q4k_gemv_mfma(const uint8_
     if (threadIdx.x < Q4K_ZERO_BYTES / 4) ((uint32_t *)(lds + L.zeros))[threadIdx.x] = 0u;
     auto stage = [&](int mi, int fi, float4 v) {
         const bool live = m0 + mi < m;
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
         float sum = (v.x + v.y) + (v.z + v.w);
         // lanes 4j..4j+3 hold 16 consecutive elements: one quantization group
         amax = fmaxf(amax, __shfl_xor(amax, 1, 64));

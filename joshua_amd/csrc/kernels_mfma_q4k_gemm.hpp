@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void q4k_gemm_prep(const float *__restrict__ x
     const int row = (int)(unit / nb), b = (int)(unit % nb), lane = threadIdx.x & 63;
     float4 v = float4{0.0f, 0.0f, 0.0f, 0.0f};
     if (row < m) v = *(const float4 *)(x + (size_t)row * k + 256 * b + 4 * lane);
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
     const bool live = amax > 0.0f && amax < INFINITY;
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256) void q4k_gemm_prep(const float *__restrict__ x
     }
     if (lane == 0) {  // lane 48 + m%16 of the block: the scale in its first dword, zeros behind it
         uint32_t *o = (uint32_t *)(a.mins + (((size_t)mt * nb + b) * 64 + 48 + (row & 15)) * 8);
-        o[0] = __float_as_uint(live ? amax / QG_RANGE : 0.0f);
+        o[0] = __float_as_uint(fixed_scale(amax, QG_RANGE));
         o[1] = o[2] = o[3] = 0;
     }
 }

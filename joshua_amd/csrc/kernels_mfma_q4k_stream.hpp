@@ -54,13 +54,13 @@ __device__ __forceinline__ void qs_quantise_acts(const float *xrow, int wave, in
             xv[ks][0] = a.x, xv[ks][1] = a.y, xv[ks][2] = a.z, xv[ks][3] = a.w;
             xv[ks][4] = c.x, xv[ks][5] = c.y, xv[ks][6] = c.z, xv[ks][7] = c.w;
 #pragma unroll
-            for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xv[ks][i]));
+            for (int i = 0; i < 8; i++) amax = fmaxf(amax, mag_or_inf(xv[ks][i]));
         }
         amax = max_xor16(amax);
         amax = max_xor32(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
         const float inv = live ? QG_RANGE / amax : 0.0f;
-        A.sx[j] = live ? amax / QG_RANGE : 0.0f;
+        A.sx[j] = fixed_scale(amax, QG_RANGE);
         int xs[8];
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
@@ -115,11 +115,11 @@ __global__ __launch_bounds__(256) void q4k_acts_prep(const float *__restrict__ X
     const float xv[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
     float amax = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xv[i]));
+    for (int i = 0; i < 8; i++) amax = fmaxf(amax, mag_or_inf(xv[i]));
 #pragma unroll
     for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
     const bool live = amax > 0.0f && amax < INFINITY;
-    const float inv = live ? QG_RANGE / amax : 0.0f, sx = live ? amax / QG_RANGE : 0.0f;
+    const float inv = live ? QG_RANGE / amax : 0.0f, sx = fixed_scale(amax, QG_RANGE);
     int lo[8], hi[8], sum = 0;
 #pragma unroll
     for (int i = 0; i < 8; i++) {

@@ -414,7 +414,7 @@ __global__ __launch_bounds__(256) void acts_i8_prep(const float *__restrict__ X,
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // four elements a thread, eight threads a block
     if (i >= rows * (size_t)(k / 4)) return;  // whole groups of 8 lanes leave together (k % 32 == 0)
     const float4 v = *(const float4 *)(X + 4 * i);
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
     amax = max_row8(amax);
     const bool live = amax > 0.0f && amax < INFINITY;
     const float inv = live ? 32639.0f / amax : 0.0f;
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(256) void acts_i8_prep(const float *__restrict__ X,
     out.xh[i] = wh;
     sum = isum_row8(sum);
     if ((i & 7) == 0) {
-        const float s = live ? amax / 32639.0f : 0.0f;
+        const float s = fixed_scale(amax, 32639.0f);
         out.sx[i >> 3] = s;
         out.sxs[i >> 3] = s * (float)sum;
     }
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
         const float *xrow = X + xr * k;
         for (int i = threadIdx.x; i < k / 4; i += 64 * ROWS_PER_WG) {
             const float4 v = *(const float4 *)(xrow + 4 * i);
-            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+            float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
             amax = max_row8(amax);
             const bool live = amax > 0.0f && amax < INFINITY;
             const float inv = live ? 32639.0f / amax : 0.0f;
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
             xh_lds[i] = wh;
             sum = isum_row8(sum);
             if ((i & 7) == 0) {
-                const float s = live ? amax / 32639.0f : 0.0f;
+                const float s = fixed_scale(amax, 32639.0f);
                 sx_lds[i >> 3] = s;
                 sxs_lds[i >> 3] = s * (float)sum;
             }

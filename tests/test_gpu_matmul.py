@@ -262,6 +262,27 @@ def test_q8_0_dot4_integer_dot_products_are_bit_exact():
     assert np.array_equal(got[0], want.astype(np.float32))
 
 
+@pytest.mark.parametrize("qtype,m,k,n", [
+    (capi.Q4_K, 1, 4096, 4096), (capi.Q4_K, 1, 2048, 512), (capi.Q4_K, 5, 4096, 512), (capi.Q4_K, 40, 1024, 256),
+    (capi.Q6_K, 1, 4096, 4096), (capi.Q8_0, 1, 4096, 4096), (capi.Q4_K, 6, 512, 32768),
+])
+def test_non_finite_activations_show_in_the_result(qtype, m, k, n):
+    """The fixed-point kernels scale every block of activations by its maximum; an inf or a NaN in a
+    block must not be read as zeros: every output of that activation row comes out non-finite (as f32
+    arithmetic would have it wherever the weights are not zero), the other rows are untouched."""
+    blocks = make_blocks(qtype, n, k, 51)
+    lhs = synth.normal(52, (m, k))
+    want = oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    for bad in (np.inf, np.nan):
+        x = lhs.copy()
+        x[m - 1, k // 2 + 3] = bad
+        got = w.matmul_t(m, x)
+        assert not np.isfinite(got[m - 1]).any()
+        if m > 1:
+            assert close(got[:m - 1], want[:m - 1])
+
+
 def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
     """4096-wide rows, one activation row: the v_dot4 kernel, activation range 32639 per 32-element
     sub-block."""
