@@ -25,6 +25,7 @@
 #include "kernels_moe.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
 #include "kernels_valu.hpp"
+#include "kernels_mfma_decoded.hpp"
 
 namespace {
 
@@ -395,6 +396,43 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
+// Any format, more than 16 activation rows, k a multiple of 256: activations as two f16 planes in a
+// stream-ordered scratch allocation, then the MFMA GEMM over decoded weights.  Returns -1 when the
+// shape is outside its reach.
+template <class Q>
+int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                        hipStream_t s) {
+    static const char *off = getenv("JQ_NO_DECODED_GEMM");
+    if (off || k % jq::GD_KC != 0 || ((uintptr_t)X & 15) != 0) return -1;
+    const size_t m_pad = (m + jq::GD_MT - 1) / jq::GD_MT * jq::GD_MT, nc = k / jq::GD_KC;
+    auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t plane = up(m_pad * k * sizeof(_Float16)), sbytes = up(m_pad * nc * sizeof(float));
+    uint8_t *buf = nullptr;
+    HIP_TRY(hipMallocAsync((void **)&buf, 2 * plane + sbytes, s));
+    jq::ActsF16 a{(_Float16 *)buf, (_Float16 *)(buf + plane), (float *)(buf + 2 * plane)};
+    hipLaunchKernelGGL(jq::acts_f16_prep, dim3((unsigned)((m_pad * nc * 64 + 255) / 256)), dim3(256), 0, s, X, (int)m,
+                       (int)m_pad, (int)k, a);
+    hipLaunchKernelGGL(jq::gemm_decoded_mfma<Q>, dim3((unsigned)((n + jq::GD_NT - 1) / jq::GD_NT), (unsigned)(m_pad / jq::GD_MT)),
+                       dim3(256), 0, s, W, row_bytes, a, Y, (int)m, (int)k, (int)n);
+    hipError_t launched = hipGetLastError();
+    HIP_TRY(hipFreeAsync(buf, s));
+    HIP_TRY(launched);
+    return 0;
+}
+
+int dispatch_gemm_decoded(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
+                          size_t k, size_t n, hipStream_t s) {
+    switch (type) {
+    case JQ_TYPE_Q8_0: return launch_gemm_decoded<jq::Q8_0>(W, row_bytes, X, Y, m, k, n, s);
+    case JQ_TYPE_Q2_K: return launch_gemm_decoded<jq::Q2_K>(W, row_bytes, X, Y, m, k, n, s);
+    case JQ_TYPE_Q4_K: return launch_gemm_decoded<jq::Q4_K>(W, row_bytes, X, Y, m, k, n, s);
+    case JQ_TYPE_Q6_K: return launch_gemm_decoded<jq::Q6_K>(W, row_bytes, X, Y, m, k, n, s);
+    case JQ_TYPE_IQ2_XXS: return launch_gemm_decoded<jq::IQ2_XXS>(W, row_bytes, X, Y, m, k, n, s);
+    case JQ_TYPE_MXFP4: return launch_gemm_decoded<jq::MXFP4>(W, row_bytes, X, Y, m, k, n, s);
+    default: return -1;
+    }
+}
+
 // All pointers are device pointers; shapes already validated; m, n > 0.
 int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
                     size_t k, size_t n, hipStream_t s) {
@@ -427,6 +465,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&
         !getenv("JQ_Q4K_NO_GEMM"))
         return dispatch_q4k_gemm(W, row_bytes, X, Y, m, k, n, s);
+    if (m > Q4K_MFMA_MAX_M && type != JQ_TYPE_Q4_K) {
+        const int rc = dispatch_gemm_decoded(type, W, row_bytes, X, Y, m, k, n, s);
+        if (rc >= 0) return rc;
+    }
     switch (type) {
     case JQ_TYPE_Q8_0: launch_rows<jq::Q8_0>(W, row_bytes, X, Y, m, k, n, s); break;
     case JQ_TYPE_Q2_K: launch_rows<jq::Q2_K>(W, row_bytes, X, Y, m, k, n, s); break;

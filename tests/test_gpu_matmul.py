@@ -283,6 +283,49 @@ def test_non_finite_activations_show_in_the_result(qtype, m, k, n):
             assert close(got[:m - 1], want[:m - 1])
 
 
+@pytest.mark.parametrize("qtype", [capi.Q8_0, capi.Q2_K, capi.Q6_K, capi.IQ2_XXS, capi.MXFP4])
+@pytest.mark.parametrize("m,k,n", [(17, 256, 64), (40, 768, 100), (130, 1024, 77), (64, 2048, 256)])
+def test_many_rows_on_the_decoded_weights_gemm(qtype, m, k, n):
+    """More than 16 activation rows of a format other than Q4_K: weights decoded to f16 in LDS, f16
+    MFMA over two activation planes; ragged tiles in both directions."""
+    blocks = make_blocks(qtype, n, k, 61)
+    lhs = synth.normal(62 + m, (m, k))
+    got = capi.Weight.upload(qtype, blocks, n, k).matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+@pytest.mark.parametrize("qtype", [capi.Q6_K, capi.MXFP4, capi.Q8_0])
+def test_decoded_weights_gemm_on_views_at_odd_byte_offsets(qtype):
+    """Experts of a stacked tensor start at any multiple of the block size (210, 17, 34 bytes): the
+    kernel reads whole words from the word at or below each row chunk's first byte."""
+    n, k, experts, m = 24, 512, 3, 33
+    stacked_blocks = make_blocks(qtype, experts * n, k, 63)
+    stacked = capi.Weight.upload(qtype, stacked_blocks, experts * n, k)
+    lhs = synth.normal(64, (m, k))
+    per = stacked_blocks.size // experts
+    for e in range(experts):
+        want = oracle.matmul_t(qtype, (m, k, n), lhs, stacked_blocks[e * per:(e + 1) * per], avx2=oracle.have_avx2())
+        assert close(stacked.view(e * per, n, k).matmul_t(m, lhs), want)
+
+
+def test_decoded_weights_gemm_activation_scales_span_many_orders():
+    """256-element chunks of a row of very different magnitude, rows that are zero but for one value or
+    for a stretch, and a row with a non-finite value."""
+    n, k, m = 96, 2048, 48
+    blocks = make_blocks(capi.Q6_K, n, k, 65)
+    rng = np.random.default_rng(7)
+    lhs = synth.normal(66, (m, k))
+    lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 256)).repeat(256).astype(np.float32)
+    lhs[1, :] = 0.0
+    lhs[1, 777] = -2.5
+    lhs[2, 512:1024] = 0.0
+    w = capi.Weight.upload(capi.Q6_K, blocks, n, k)
+    assert close(w.matmul_t(m, lhs), oracle.matmul_t(capi.Q6_K, (m, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+    lhs[7, 300] = np.inf
+    got = w.matmul_t(m, lhs)
+    assert not np.isfinite(got[7]).any() and np.isfinite(got[8]).all()
+
+
 def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
     """4096-wide rows, one activation row: the v_dot4 kernel, activation range 32639 per 32-element
     sub-block."""
