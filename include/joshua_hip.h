@@ -168,6 +168,9 @@ typedef struct {
 int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out);
 void jq_qwen3_free(jq_model *model);
 
+/* The configuration the model was created with (for models built by jq_qwen3_load_gguf). */
+int jq_qwen3_get_config(const jq_model *model, jq_qwen3_config *out);
+
 /* Installs one tensor under its GGUF name ("token_embd.weight",
  * "blk.3.attn_q.weight", "blk.3.attn_q_norm.weight", "output_norm.weight",
  * "output.weight", ...).  ggml_type 0 is F32 (norm weights); the others are the
@@ -189,6 +192,85 @@ int jq_qwen3_greedy(jq_model *model, uint32_t *token, void *stream);
 
 /* Forgets the KV cache (reference: clear_kv_cache, src/quantized_qwen3_moe.rs:822-826). */
 int jq_qwen3_reset(jq_model *model);
+
+/* ---- GGUF files -------------------------------------------------------------------
+ * A tolerant reader of the container: header, metadata and tensor directory of a
+ * file mapped read-only, tensor types kept as raw ids so that MXFP4 (39) and
+ * IQ2_XXS (16) survive parsing (reference: src/gguf_ext.rs:400-480 read_header with
+ * the limits of :33-59; the mapping and its bounds check src/mmap_tensor.rs:105-123).
+ * Host only: none of the jq_gguf_* calls except jq_gguf_upload touches the GPU. */
+typedef struct jq_gguf jq_gguf;
+
+/* Bytes of `elems` elements of a raw type id, for every id the reference sizes
+ * (F32, F16, BF16, Q4_0..Q8_1, Q2_K..Q8_K, I32, IQ2_XXS, MXFP4); fails for an
+ * unknown id or a count that is not whole blocks
+ * (reference: src/gguf_ext.rs:483-512 type_size_bytes). */
+int jq_type_size_bytes(uint32_t ggml_type, size_t elems, size_t *bytes);
+
+/* Maps `path` and parses its header. */
+int jq_gguf_open(const char *path, jq_gguf **out);
+/* Parses a header held in memory (the bytes are copied); tensor data may be absent. */
+int jq_gguf_parse(const void *bytes, size_t len, jq_gguf **out);
+void jq_gguf_close(jq_gguf *g);
+
+uint32_t jq_gguf_version(const jq_gguf *g);
+uint64_t jq_gguf_tensor_data_offset(const jq_gguf *g);
+size_t jq_gguf_tensor_count(const jq_gguf *g);
+size_t jq_gguf_metadata_count(const jq_gguf *g);
+
+/* Directory entry `index` (file order).  dims has room for 8 values and receives them
+ * in row-major order, slowest first (the file stores them fastest first); offset counts
+ * from jq_gguf_tensor_data_offset.  Any output pointer may be NULL.  `*name` stays
+ * valid until jq_gguf_close (reference: src/gguf_ext.rs:117-135 RawTensorInfo). */
+int jq_gguf_tensor_at(const jq_gguf *g, size_t index, const char **name, uint32_t *ggml_type, uint32_t *n_dims,
+                      uint64_t *dims, uint64_t *offset);
+int jq_gguf_find_tensor(const jq_gguf *g, const char *name, size_t *index);
+/* The tensor's bytes inside the mapping; fails when its type has no known size or the
+ * range runs past the end of the file. */
+int jq_gguf_tensor_bytes(const jq_gguf *g, size_t index, const void **data, size_t *nbytes);
+
+/* Metadata scalars: nonzero when the key is missing or holds another type.  u32 accepts
+ * every integer type up to 32 bits that is not negative
+ * (reference: src/quantized_qwen3_moe.rs:64-88 Meta helpers). */
+int jq_gguf_meta_u32(const jq_gguf *g, const char *key, uint32_t *out);
+int jq_gguf_meta_f32(const jq_gguf *g, const char *key, float *out);
+int jq_gguf_meta_bool(const jq_gguf *g, const char *key, int *out);
+int jq_gguf_meta_str(const jq_gguf *g, const char *key, const char **out, size_t *len);
+int jq_gguf_meta_array_len(const jq_gguf *g, const char *key, size_t *len);
+
+/* Uploads one tensor once, in its native block layout, straight from the mapping: a
+ * matrix [n, k], or a stack [E, n, k] as one weight of E*n rows whose expert slices
+ * jq_view addresses (reference: src/mmap_tensor.rs:520-565 borrowed_qtensor_raw,
+ * src/quantized_qwen3_moe.rs:596-631 split_experts). */
+int jq_gguf_upload(const jq_gguf *g, const char *name, jq_weight **out);
+
+/* Builds the dense Qwen3 decoder from a GGUF file: configuration from the `qwen3.*`
+ * metadata with the reference loader's rules (attention.key_length wins over
+ * embedding_length / head_count, rope.freq_base defaults to 10000; reference:
+ * src/quantized_qwen3_moe.rs:90-147), every tensor uploaded once; a file without
+ * output.weight uses token_embd.weight as the output head
+ * (reference: src/quantized_qwen3_moe.rs:737-743).  n_ctx == 0 takes the file's
+ * context_length. */
+int jq_qwen3_load_gguf(const char *path, uint32_t n_ctx, jq_model **out);
+
+/* ---- Model-level plugin boundary ----------------------------------------------------
+ * The four symbols the reference engine looks up when it is started with a backend
+ * library (reference: src/npu/mod.rs:32-50 contract; src/npu/vendor.rs:17-20
+ * signatures, :49-56 symbol check, :95-121 init; src/main.rs:166-172 the switch).
+ * init loads the GGUF at model_path as a dense Qwen3 decoder with a KV cache of
+ * n_ctx tokens and reports the vocabulary size; forward appends n_tokens tokens at
+ * absolute position pos, which must equal the number of tokens fed so far, and
+ * writes vocab logits for the last one; reset forgets the fed tokens.  0 is success;
+ * the codes are those of the reference's model plugin
+ * (crates/joshua-mock-npu/src/lib.rs:41-131): -1 null argument or empty batch,
+ * -2 the model did not load, -3 pos is not the number of tokens fed so far,
+ * -4 the context is full, -5 the device call failed (jq_last_error has the text).
+ * A handle is used by one thread at a time but may move between threads. */
+int32_t joshua_npu_init(const char *model_path, uint32_t n_ctx, uint32_t *out_vocab, void **out_handle);
+int32_t joshua_npu_forward(void *handle, const uint32_t *tokens, uint32_t n_tokens, uint32_t pos,
+                           float *out_logits);
+int32_t joshua_npu_reset(void *handle);
+void joshua_npu_free(void *handle);
 
 /* Blocks until everything enqueued on `stream` has finished. */
 int jq_stream_synchronize(void *stream);

@@ -24,6 +24,11 @@ EXPORTS = (
     "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_try_matmul_fused", "jq_dequantize",
     "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
     "jq_qwen3_create", "jq_qwen3_free", "jq_qwen3_set_tensor", "jq_qwen3_forward", "jq_qwen3_greedy", "jq_qwen3_reset",
+    "jq_qwen3_get_config", "jq_qwen3_load_gguf", "jq_type_size_bytes", "jq_gguf_open", "jq_gguf_parse", "jq_gguf_close",
+    "jq_gguf_version", "jq_gguf_tensor_data_offset", "jq_gguf_tensor_count", "jq_gguf_metadata_count",
+    "jq_gguf_tensor_at", "jq_gguf_find_tensor", "jq_gguf_tensor_bytes", "jq_gguf_meta_u32", "jq_gguf_meta_f32",
+    "jq_gguf_meta_bool", "jq_gguf_meta_str", "jq_gguf_meta_array_len", "jq_gguf_upload",
+    "joshua_npu_init", "joshua_npu_forward", "joshua_npu_reset", "joshua_npu_free",
 )
 
 
@@ -96,6 +101,39 @@ def lib() -> ctypes.CDLL:
         L.jq_qwen3_forward.argtypes = [vp, vp, u32, u32, vp, i32, vp]
         L.jq_qwen3_greedy.argtypes = [vp, ctypes.POINTER(u32), vp]
         L.jq_qwen3_reset.argtypes = [vp]
+        L.jq_qwen3_get_config.argtypes = [vp, ctypes.POINTER(Qwen3Config)]
+        L.jq_qwen3_load_gguf.argtypes = [ctypes.c_char_p, u32, ctypes.POINTER(vp)]
+        u64 = ctypes.c_uint64
+        L.jq_type_size_bytes.argtypes = [u32, sz, ctypes.POINTER(sz)]
+        L.jq_gguf_open.argtypes = [ctypes.c_char_p, ctypes.POINTER(vp)]
+        L.jq_gguf_parse.argtypes = [vp, sz, ctypes.POINTER(vp)]
+        L.jq_gguf_close.argtypes = [vp]
+        L.jq_gguf_close.restype = None
+        L.jq_gguf_version.argtypes = [vp]
+        L.jq_gguf_version.restype = u32
+        L.jq_gguf_tensor_data_offset.argtypes = [vp]
+        L.jq_gguf_tensor_data_offset.restype = u64
+        for f in (L.jq_gguf_tensor_count, L.jq_gguf_metadata_count):
+            f.argtypes = [vp]
+            f.restype = sz
+        L.jq_gguf_tensor_at.argtypes = [vp, sz, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(u32), ctypes.POINTER(u32),
+                                        ctypes.POINTER(u64), ctypes.POINTER(u64)]
+        L.jq_gguf_find_tensor.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(sz)]
+        L.jq_gguf_tensor_bytes.argtypes = [vp, sz, ctypes.POINTER(vp), ctypes.POINTER(sz)]
+        L.jq_gguf_meta_u32.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(u32)]
+        L.jq_gguf_meta_f32.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(ctypes.c_float)]
+        L.jq_gguf_meta_bool.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(i32)]
+        L.jq_gguf_meta_str.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(vp), ctypes.POINTER(sz)]
+        L.jq_gguf_meta_array_len.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(sz)]
+        L.jq_gguf_upload.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(vp)]
+        L.joshua_npu_init.argtypes = [ctypes.c_char_p, u32, ctypes.POINTER(u32), ctypes.POINTER(vp)]
+        L.joshua_npu_init.restype = ctypes.c_int32
+        L.joshua_npu_forward.argtypes = [vp, vp, u32, u32, vp]
+        L.joshua_npu_forward.restype = ctypes.c_int32
+        L.joshua_npu_reset.argtypes = [vp]
+        L.joshua_npu_reset.restype = ctypes.c_int32
+        L.joshua_npu_free.argtypes = [vp]
+        L.joshua_npu_free.restype = None
         _lib = L
     return _lib
 
@@ -280,6 +318,18 @@ class Qwen3:
         _check(lib().jq_qwen3_create(ctypes.byref(cfg), ctypes.byref(out)))
         self._h = out
 
+    @classmethod
+    def from_gguf(cls, path: str, n_ctx: int = 0) -> "Qwen3":
+        """Loads a dense qwen3 GGUF file: configuration from its metadata, every tensor
+        uploaded once in native layout (reference: src/quantized_qwen3_moe.rs:90-147,725-775)."""
+        out = ctypes.c_void_p()
+        _check(lib().jq_qwen3_load_gguf(os.fsencode(path), n_ctx, ctypes.byref(out)))
+        self = cls.__new__(cls)
+        self._h = out
+        self.cfg = Qwen3Config()
+        _check(lib().jq_qwen3_get_config(out, ctypes.byref(self.cfg)))
+        return self
+
     def close(self) -> None:
         if self._h:
             lib().jq_qwen3_free(self._h)
@@ -314,3 +364,132 @@ class Qwen3:
 
     def reset(self) -> None:
         _check(lib().jq_qwen3_reset(self._h))
+
+
+def type_size_bytes(qtype: int, elems: int) -> "int | None":
+    """Bytes of `elems` elements of a raw GGUF type id, or None
+    (reference: src/gguf_ext.rs:483-512)."""
+    out = ctypes.c_size_t()
+    return out.value if lib().jq_type_size_bytes(qtype, elems, ctypes.byref(out)) == 0 else None
+
+
+class Gguf:
+    """A GGUF file mapped read-only, or a header parsed from bytes: the tensor directory with
+    raw type ids, metadata scalars, and uploads straight from the mapping
+    (reference: src/gguf_ext.rs:117-146 RawTensorInfo / GgufHeader, :400-480 read_header)."""
+
+    def __init__(self, handle: ctypes.c_void_p):
+        self._h = handle
+
+    @classmethod
+    def open(cls, path: str) -> "Gguf":
+        out = ctypes.c_void_p()
+        _check(lib().jq_gguf_open(os.fsencode(path), ctypes.byref(out)))
+        return cls(out)
+
+    @classmethod
+    def parse(cls, data: bytes) -> "Gguf":
+        out = ctypes.c_void_p()
+        buf = (ctypes.c_char * max(len(data), 1)).from_buffer_copy(data or b"\0")
+        _check(lib().jq_gguf_parse(ctypes.addressof(buf), len(data), ctypes.byref(out)))
+        return cls(out)
+
+    def close(self) -> None:
+        if self._h:
+            lib().jq_gguf_close(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def version(self) -> int:
+        return lib().jq_gguf_version(self._h)
+
+    @property
+    def tensor_data_offset(self) -> int:
+        return lib().jq_gguf_tensor_data_offset(self._h)
+
+    @property
+    def metadata_count(self) -> int:
+        return lib().jq_gguf_metadata_count(self._h)
+
+    def tensors(self) -> dict:
+        """name -> (raw type id, dims in row-major order, offset from tensor_data_offset)."""
+        out = {}
+        for i in range(lib().jq_gguf_tensor_count(self._h)):
+            name, ty, nd, off = ctypes.c_char_p(), ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64()
+            dims = (ctypes.c_uint64 * 8)()
+            _check(lib().jq_gguf_tensor_at(self._h, i, ctypes.byref(name), ctypes.byref(ty), ctypes.byref(nd), dims,
+                                           ctypes.byref(off)))
+            out[name.value.decode(errors="replace")] = (ty.value, list(dims[:nd.value]), off.value)
+        return out
+
+    def tensor_bytes(self, name: str) -> np.ndarray:
+        """A copy of the tensor's bytes out of the mapping."""
+        idx, p, n = ctypes.c_size_t(), ctypes.c_void_p(), ctypes.c_size_t()
+        _check(lib().jq_gguf_find_tensor(self._h, name.encode(), ctypes.byref(idx)))
+        _check(lib().jq_gguf_tensor_bytes(self._h, idx.value, ctypes.byref(p), ctypes.byref(n)))
+        return np.frombuffer(ctypes.string_at(p.value, n.value), dtype=np.uint8).copy()
+
+    def meta_u32(self, key: str) -> "int | None":
+        v = ctypes.c_uint32()
+        return v.value if lib().jq_gguf_meta_u32(self._h, key.encode(), ctypes.byref(v)) == 0 else None
+
+    def meta_f32(self, key: str) -> "float | None":
+        v = ctypes.c_float()
+        return v.value if lib().jq_gguf_meta_f32(self._h, key.encode(), ctypes.byref(v)) == 0 else None
+
+    def meta_bool(self, key: str) -> "bool | None":
+        v = ctypes.c_int()
+        return bool(v.value) if lib().jq_gguf_meta_bool(self._h, key.encode(), ctypes.byref(v)) == 0 else None
+
+    def meta_str(self, key: str) -> "bytes | None":
+        """The string's bytes with trailing NULs dropped (decode with errors="replace" for text)."""
+        p, n = ctypes.c_void_p(), ctypes.c_size_t()
+        if lib().jq_gguf_meta_str(self._h, key.encode(), ctypes.byref(p), ctypes.byref(n)) != 0:
+            return None
+        return ctypes.string_at(p.value, n.value)
+
+    def meta_array_len(self, key: str) -> "int | None":
+        n = ctypes.c_size_t()
+        return n.value if lib().jq_gguf_meta_array_len(self._h, key.encode(), ctypes.byref(n)) == 0 else None
+
+    def upload(self, name: str) -> Weight:
+        out = ctypes.c_void_p()
+        _check(lib().jq_gguf_upload(self._h, name.encode(), ctypes.byref(out)))
+        return Weight(out.value)
+
+
+class NpuPlugin:
+    """The library driven through the four joshua_npu_* symbols, the way the reference engine
+    drives a backend plugin (reference: src/npu/vendor.rs:95-121 init, :150-185 forward_into,
+    :244-251 free on drop).  Failures surface as the plugin's return codes."""
+
+    def __init__(self, model_path: str, n_ctx: int):
+        vocab, h = ctypes.c_uint32(), ctypes.c_void_p()
+        self.rc = lib().joshua_npu_init(os.fsencode(model_path), n_ctx, ctypes.byref(vocab), ctypes.byref(h))
+        self.vocab, self._h = vocab.value, h
+
+    def forward(self, tokens, pos: int) -> "tuple[int, np.ndarray]":
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        logits = np.zeros(self.vocab, np.float32)
+        rc = lib().joshua_npu_forward(self._h, t.ctypes.data, t.size, pos, logits.ctypes.data)
+        return rc, logits
+
+    def reset(self) -> int:
+        return lib().joshua_npu_reset(self._h)
+
+    def close(self) -> None:
+        if self._h:
+            lib().joshua_npu_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1598,11 +1598,299 @@ int jq_qwen3_greedy(jq_model *m, uint32_t *token, void *stream) {
     return 0;
 }
 
+int jq_qwen3_get_config(const jq_model *m, jq_qwen3_config *out) {
+    if (!m || !out) return fail("jq_qwen3_get_config: null argument");
+    *out = m->cfg;
+    return 0;
+}
+
 int jq_qwen3_reset(jq_model *m) {
     if (!m) return fail("jq_qwen3_reset: model is null");
     std::lock_guard<std::mutex> lock(m->mu);
     m->n_past = 0;
     return 0;
+}
+
+}  // extern "C"
+
+// ---- GGUF files and the model-level plugin boundary ------------------------------------------
+
+#include "gguf.hpp"
+
+struct jq_gguf {
+    std::unique_ptr<jq::Gguf> g;
+};
+
+namespace {
+
+int gguf_wrap(std::unique_ptr<jq::Gguf> g, const std::string &err, jq_gguf **out) {
+    if (!g) return fail("%s", err.c_str());
+    *out = new jq_gguf{std::move(g)};
+    return 0;
+}
+
+// Every tensor the graph reads is installed, or the name of the first one that is not.
+int model_check_complete(jq_model *m) {
+    std::vector<std::string> names = {"token_embd.weight", "output_norm.weight", "output.weight"};
+    for (uint32_t l = 0; l < m->cfg.n_layer; l++)
+        for (const char *role : {"attn_norm", "attn_q", "attn_k", "attn_v", "attn_q_norm", "attn_k_norm", "attn_output",
+                                 "ffn_norm", "ffn_gate", "ffn_up", "ffn_down"})
+            names.push_back("blk." + std::to_string(l) + "." + role + ".weight");
+    for (const auto &nm : names)
+        if (!m->q.count(nm) && !m->f.count(nm)) return fail("qwen3: missing tensor `%s`", nm.c_str());
+    return 0;
+}
+
+// Configuration of a dense qwen3 file from its metadata, with the reference loader's rules
+// (reference: src/quantized_qwen3_moe.rs:90-147): attention.key_length wins over
+// embedding_length / head_count, rope.freq_base defaults to 10000, head_count must be a multiple
+// of head_count_kv, head_dim must be positive and even.
+int qwen3_config_from_gguf(const jq::Gguf &g, uint32_t n_ctx, jq_qwen3_config *c) {
+    const std::string *arch = g.meta_str("general.architecture");
+    if (!arch || *arch != "qwen3")
+        return fail("qwen3: general.architecture is `%s`, expected `qwen3`", arch ? arch->c_str() : "(missing)");
+    auto need_u32 = [&](const char *key, uint32_t *v) {
+        if (g.meta_u32(std::string("qwen3.") + key, v)) return 0;
+        return fail("qwen3: missing GGUF metadata key `qwen3.%s`", key);
+    };
+    uint32_t context_length = 0, key_length = 0;
+    if (need_u32("attention.head_count", &c->n_head) || need_u32("attention.head_count_kv", &c->n_kv_head) ||
+        need_u32("block_count", &c->n_layer) || need_u32("embedding_length", &c->hidden) ||
+        need_u32("context_length", &context_length))
+        return 1;
+    if (!g.meta_f32("qwen3.attention.layer_norm_rms_epsilon", &c->rms_eps))
+        return fail("qwen3: missing GGUF metadata key `qwen3.attention.layer_norm_rms_epsilon`");
+    if (c->n_head == 0) return fail("qwen3: head_count is zero");
+    c->head_dim = g.meta_u32("qwen3.attention.key_length", &key_length) ? key_length : c->hidden / c->n_head;
+    if (c->head_dim == 0 || c->head_dim % 2 != 0)
+        return fail("qwen3: invalid head_dim %u (must be a positive even number)", c->head_dim);
+    if (c->n_kv_head == 0 || c->n_head % c->n_kv_head != 0)
+        return fail("qwen3: head_count %u must be a multiple of head_count_kv %u", c->n_head, c->n_kv_head);
+    if (!g.meta_f32("qwen3.rope.freq_base", &c->rope_theta)) c->rope_theta = 10000.0f;
+    // the two sizes the metadata may leave out are read off the tensors
+    const jq::GgufTensor *emb = g.tensor("token_embd.weight");
+    if (!emb || emb->dims.size() != 2) return fail("qwen3: missing tensor `token_embd.weight`");
+    c->vocab = (uint32_t)emb->dims[0];
+    if (!g.meta_u32("qwen3.feed_forward_length", &c->ffn)) {
+        const jq::GgufTensor *gate = g.tensor("blk.0.ffn_gate.weight");
+        if (!gate || gate->dims.size() != 2) return fail("qwen3: missing GGUF metadata key `qwen3.feed_forward_length`");
+        c->ffn = (uint32_t)gate->dims[0];
+    }
+    c->n_ctx = n_ctx ? n_ctx : context_length;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int jq_type_size_bytes(uint32_t ggml_type, size_t elems, size_t *bytes) {
+    uint64_t b;
+    if (!bytes) return fail("jq_type_size_bytes: bytes is null");
+    if (!jq::gguf_type_size_bytes(ggml_type, elems, &b))
+        return fail("type id %u with %zu elements has no known size", ggml_type, elems);
+    *bytes = (size_t)b;
+    return 0;
+}
+
+int jq_gguf_open(const char *path, jq_gguf **out) {
+    if (!path || !out) return fail("jq_gguf_open: null argument");
+    *out = nullptr;
+    std::string err;
+    auto g = jq::gguf_open(path, &err);
+    return gguf_wrap(std::move(g), err, out);
+}
+
+int jq_gguf_parse(const void *bytes, size_t len, jq_gguf **out) {
+    if (!bytes || !out) return fail("jq_gguf_parse: null argument");
+    *out = nullptr;
+    std::vector<uint8_t> copy((const uint8_t *)bytes, (const uint8_t *)bytes + len);
+    std::string err;
+    auto g = jq::gguf_parse(copy.data(), copy.size(), &err);
+    if (g) {
+        g->owned = std::move(copy);  // moving a vector keeps its storage, so g->base stays valid
+        g->base = g->owned.data();
+    }
+    return gguf_wrap(std::move(g), err, out);
+}
+
+void jq_gguf_close(jq_gguf *g) { delete g; }
+
+uint32_t jq_gguf_version(const jq_gguf *g) { return g ? g->g->version : 0; }
+uint64_t jq_gguf_tensor_data_offset(const jq_gguf *g) { return g ? g->g->tensor_data_offset : 0; }
+size_t jq_gguf_tensor_count(const jq_gguf *g) { return g ? g->g->tensors.size() : 0; }
+size_t jq_gguf_metadata_count(const jq_gguf *g) { return g ? g->g->metadata.size() : 0; }
+
+int jq_gguf_tensor_at(const jq_gguf *g, size_t index, const char **name, uint32_t *ggml_type, uint32_t *n_dims,
+                      uint64_t *dims, uint64_t *offset) {
+    if (!g) return fail("jq_gguf_tensor_at: file is null");
+    if (index >= g->g->tensors.size()) return fail("GGUF: tensor index %zu of %zu", index, g->g->tensors.size());
+    const jq::GgufTensor &t = g->g->tensors[index];
+    if (name) *name = t.name.c_str();
+    if (ggml_type) *ggml_type = t.dtype;
+    if (n_dims) *n_dims = (uint32_t)t.dims.size();
+    if (dims)
+        for (size_t d = 0; d < t.dims.size(); d++) dims[d] = t.dims[d];
+    if (offset) *offset = t.offset;
+    return 0;
+}
+
+int jq_gguf_find_tensor(const jq_gguf *g, const char *name, size_t *index) {
+    if (!g || !name || !index) return fail("jq_gguf_find_tensor: null argument");
+    auto it = g->g->by_name.find(name);
+    if (it == g->g->by_name.end()) return fail("GGUF: no tensor `%s`", name);
+    *index = it->second;
+    return 0;
+}
+
+int jq_gguf_tensor_bytes(const jq_gguf *g, size_t index, const void **data, size_t *nbytes) {
+    if (!g || !data || !nbytes) return fail("jq_gguf_tensor_bytes: null argument");
+    if (index >= g->g->tensors.size()) return fail("GGUF: tensor index %zu of %zu", index, g->g->tensors.size());
+    const uint8_t *p;
+    uint64_t n;
+    std::string err;
+    if (!g->g->tensor_bytes(g->g->tensors[index], &p, &n, &err)) return fail("GGUF: %s", err.c_str());
+    *data = p;
+    *nbytes = (size_t)n;
+    return 0;
+}
+
+int jq_gguf_meta_u32(const jq_gguf *g, const char *key, uint32_t *out) {
+    if (!g || !key || !out) return fail("jq_gguf_meta_u32: null argument");
+    return g->g->meta_u32(key, out) ? 0 : fail("GGUF: no unsigned 32-bit value under `%s`", key);
+}
+
+int jq_gguf_meta_f32(const jq_gguf *g, const char *key, float *out) {
+    if (!g || !key || !out) return fail("jq_gguf_meta_f32: null argument");
+    return g->g->meta_f32(key, out) ? 0 : fail("GGUF: no f32 value under `%s`", key);
+}
+
+int jq_gguf_meta_bool(const jq_gguf *g, const char *key, int *out) {
+    if (!g || !key || !out) return fail("jq_gguf_meta_bool: null argument");
+    bool b;
+    if (!g->g->meta_bool(key, &b)) return fail("GGUF: no bool value under `%s`", key);
+    *out = b;
+    return 0;
+}
+
+int jq_gguf_meta_str(const jq_gguf *g, const char *key, const char **out, size_t *len) {
+    if (!g || !key || !out) return fail("jq_gguf_meta_str: null argument");
+    const std::string *s = g->g->meta_str(key);
+    if (!s) return fail("GGUF: no string value under `%s`", key);
+    *out = s->c_str();
+    if (len) *len = s->size();
+    return 0;
+}
+
+int jq_gguf_meta_array_len(const jq_gguf *g, const char *key, size_t *len) {
+    if (!g || !key || !len) return fail("jq_gguf_meta_array_len: null argument");
+    const jq::GgufValue *v = g->g->find(key);
+    if (!v || v->type != 9) return fail("GGUF: no array under `%s`", key);
+    *len = v->items.size();
+    return 0;
+}
+
+int jq_gguf_upload(const jq_gguf *g, const char *name, jq_weight **out) {
+    if (!g || !name || !out) return fail("jq_gguf_upload: null argument");
+    *out = nullptr;
+    const jq::GgufTensor *t = g->g->tensor(name);
+    if (!t) return fail("GGUF: no tensor `%s`", name);
+    if (t->dims.size() < 2) return fail("GGUF: tensor `%s` has %zu dimensions, a matrix needs 2", name, t->dims.size());
+    const uint8_t *p;
+    uint64_t nbytes;
+    std::string err;
+    if (!g->g->tensor_bytes(*t, &p, &nbytes, &err)) return fail("GGUF: %s", err.c_str());
+    size_t k = (size_t)t->dims.back(), n = (size_t)(t->elem_count() / (k ? k : 1));
+    return jq_upload(t->dtype, p, (size_t)nbytes, n, k, 0, out);
+}
+
+int jq_qwen3_load_gguf(const char *path, uint32_t n_ctx, jq_model **out) {
+    if (!path || !out) return fail("jq_qwen3_load_gguf: null argument");
+    *out = nullptr;
+    std::string err;
+    auto g = jq::gguf_open(path, &err);
+    if (!g) return fail("%s", err.c_str());
+    jq_qwen3_config cfg{};
+    if (qwen3_config_from_gguf(*g, n_ctx, &cfg)) return 1;
+    jq_model *m = nullptr;
+    if (jq_qwen3_create(&cfg, &m)) return 1;
+    bool have_output = false;
+    for (const jq::GgufTensor &t : g->tensors) {
+        size_t n, k;
+        if (!qwen3_shape(cfg, t.name, &n, &k)) continue;  // rope tables and the like
+        const uint8_t *p;
+        uint64_t nbytes;
+        if (!g->tensor_bytes(t, &p, &nbytes, &err)) {
+            jq_qwen3_free(m);
+            return fail("GGUF: %s", err.c_str());
+        }
+        const bool shape_ok = k == 0 ? (t.dims.size() == 1 && t.dims[0] == n)
+                                     : (t.dims.size() == 2 && t.dims[0] == n && t.dims[1] == k);
+        if (!shape_ok) {
+            jq_qwen3_free(m);
+            return fail("qwen3: tensor `%s` does not have the shape the metadata implies", t.name.c_str());
+        }
+        if (jq_qwen3_set_tensor(m, t.name.c_str(), t.dtype, p, (size_t)nbytes)) {
+            jq_qwen3_free(m);
+            return 1;
+        }
+        have_output |= t.name == "output.weight";
+    }
+    if (!have_output) {
+        // conversions with tied embeddings ship no output head
+        // (reference: src/quantized_qwen3_moe.rs:739-743)
+        const jq::GgufTensor *emb = g->tensor("token_embd.weight");
+        const uint8_t *p;
+        uint64_t nbytes;
+        if (!emb || !g->tensor_bytes(*emb, &p, &nbytes, &err) ||
+            jq_qwen3_set_tensor(m, "output.weight", emb->dtype, p, (size_t)nbytes)) {
+            jq_qwen3_free(m);
+            return emb ? 1 : fail("qwen3: missing tensor `token_embd.weight`");
+        }
+    }
+    if (model_check_complete(m)) {
+        jq_qwen3_free(m);
+        return 1;
+    }
+    *out = m;
+    return 0;
+}
+
+// The four symbols the reference engine binds when it loads a backend as a shared library
+// (reference: src/npu/mod.rs:32-50 contract, src/npu/vendor.rs:17-20 signatures, :49-56 symbol
+// check, :95-121 init; crates/joshua-mock-npu/src/lib.rs:41-131 return codes of the model plugin).
+int32_t joshua_npu_init(const char *model_path, uint32_t n_ctx, uint32_t *out_vocab, void **out_handle) {
+    if (!model_path || !out_vocab || !out_handle) return -1;
+    *out_handle = nullptr;
+    jq_model *m = nullptr;
+    if (jq_qwen3_load_gguf(model_path, n_ctx, &m)) return -2;
+    *out_vocab = m->cfg.vocab;
+    *out_handle = m;
+    return 0;
+}
+
+int32_t joshua_npu_forward(void *handle, const uint32_t *tokens, uint32_t n_tokens, uint32_t pos, float *out_logits) {
+    if (!handle || !tokens || !out_logits || n_tokens == 0) return -1;
+    jq_model *m = (jq_model *)handle;
+    // the handle may arrive on another thread than the one that made it; the device is per thread
+    if (hipSetDevice(g_device) != hipSuccess) return -5;
+    {
+        std::lock_guard<std::mutex> lock(m->mu);
+        if (pos != m->n_past) return -3;
+        if ((uint64_t)pos + n_tokens > m->cfg.n_ctx) return -4;
+    }
+    return jq_qwen3_forward(m, tokens, n_tokens, pos, out_logits, 0, nullptr) ? -5 : 0;
+}
+
+int32_t joshua_npu_reset(void *handle) {
+    if (!handle) return -1;
+    return jq_qwen3_reset((jq_model *)handle) ? -5 : 0;
+}
+
+void joshua_npu_free(void *handle) {
+    if (!handle) return;
+    (void)hipSetDevice(g_device);
+    jq_qwen3_free((jq_model *)handle);
 }
 
 }  // extern "C"

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_symbols():
     text = open(os.path.join(ROOT, "include", "joshua_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(jq_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b((?:jq|joshua_npu)_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_and_binding_list_the_same_symbols():

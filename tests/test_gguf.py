@@ -1,0 +1,283 @@
+"""GGUF container reader: the C++ reader behind the C ABI and the oracle's restatement, both
+against the cases the reference's own parser tests hold (src/gguf_ext.rs:515-949, rebuilt here
+from their byte-level descriptions) and against each other on files our writer makes.
+Host only: nothing here touches a GPU."""
+import struct
+
+import numpy as np
+import pytest
+
+from joshua_amd import capi
+from joshua_amd.synth import gguf as gw
+from oracle import gguf as og
+
+MAGIC = struct.pack("<I", 0x46554747)
+
+
+def s64(b: bytes) -> bytes:
+    return struct.pack("<Q", len(b)) + b
+
+
+def tensor_w(dtype: int) -> bytes:
+    """Directory entry of the tensor every reference case carries: "w", dims [64, 8], offset 0."""
+    return s64(b"w") + struct.pack("<IQQIQ", 2, 64, 8, dtype, 0)
+
+
+def header_one_tensor(dtype: int) -> bytes:
+    """src/gguf_ext.rs:519-545: version 3, one tensor, general.architecture = "kimi-k3"."""
+    return (MAGIC + struct.pack("<IQQ", 3, 1, 1) + s64(b"general.architecture") + struct.pack("<I", 8) + s64(b"kimi-k3")
+            + tensor_w(dtype))
+
+
+def one_kv(key: bytes, payload: bytes) -> bytes:
+    return MAGIC + struct.pack("<IQQ", 3, 1, 1) + s64(key) + payload + tensor_w(0)
+
+
+def both(data: bytes):
+    """(oracle view, C++ view) of one header, reduced to comparable dictionaries."""
+    o = og.read_header(data)
+    g = capi.Gguf.parse(data)
+    c = {"version": g.version, "tensors": {k: tuple(v) for k, v in g.tensors().items()},
+         "tensor_data_offset": g.tensor_data_offset, "metadata_count": g.metadata_count}
+    o2 = {"version": o["version"], "tensors": {k: (v[0], v[1], v[2]) for k, v in o["tensors"].items()},
+          "tensor_data_offset": o["tensor_data_offset"], "metadata_count": len(o["metadata"])}
+    assert c == o2
+    return o, g
+
+
+def both_fail(data: bytes, phrase: str):
+    with pytest.raises(og.GgufError, match=phrase):
+        og.read_header(data)
+    with pytest.raises(capi.JoshuaHipError, match=phrase):
+        capi.Gguf.parse(data)
+
+
+def test_parses_a_header_whose_type_the_common_table_lacks():
+    # src/gguf_ext.rs:547-566: MXFP4 (39) survives; dims come back row-major
+    o, g = both(header_one_tensor(39))
+    assert og.architecture(o) == "kimi-k3" and g.meta_str("general.architecture") == b"kimi-k3"
+    assert o["tensors"]["w"] == (39, [8, 64], 0) and g.tensors()["w"] == (39, [8, 64], 0)
+
+
+@pytest.mark.parametrize("dtype", [0, 4, 5, 12, 16])
+def test_any_type_id_survives_the_header(dtype):
+    # src/gguf_ext.rs:617-643: ids are not judged while parsing
+    o, g = both(header_one_tensor(dtype))
+    assert g.tensors()["w"][0] == dtype
+
+
+def test_rejects_bad_magic():
+    data = bytearray(header_one_tensor(0))      # src/gguf_ext.rs:654-659
+    data[0] ^= 0xFF
+    both_fail(bytes(data), "bad magic")
+
+
+@pytest.mark.parametrize("version", [0, 4, 0xFFFFFFFF])
+def test_rejects_unknown_versions(version):
+    data = bytearray(header_one_tensor(0))
+    data[4:8] = struct.pack("<I", version)
+    both_fail(bytes(data), "unsupported GGUF version")
+
+
+def test_version_one_lengths_are_32_bit():
+    def s32(b):
+        return struct.pack("<I", len(b)) + b
+    data = (MAGIC + struct.pack("<III", 1, 1, 1) + s32(b"general.architecture") + struct.pack("<I", 8) + s32(b"v1")
+            + s32(b"w") + struct.pack("<IIIIQ", 2, 64, 8, 12, 96))
+    o, g = both(data)
+    assert g.version == 1 and g.tensors()["w"] == (12, [8, 64], 96)
+    assert gw.header_bytes({"general.architecture": gw.string("v1")}, [("w", [8, 64], 12, 96)], version=1) == data
+
+
+def test_implausible_counts_are_refused():
+    # src/gguf_ext.rs:415-417: counts above 2^24 end the parse before anything is stored
+    for tc, kc in (((1 << 24) + 1, 0), (0, 1 << 40)):
+        both_fail(MAGIC + struct.pack("<IQQ", 3, tc, kc), "implausible")
+    # a count at the limit with nothing behind it is a short read, not an allocation
+    both_fail(MAGIC + struct.pack("<IQQ", 3, 1 << 24, 0), "GGUF header")
+
+
+def test_lenient_strings_nul_terminated_and_invalid_utf8():
+    # src/gguf_ext.rs:661-714
+    data = (MAGIC + struct.pack("<IQQ", 3, 1, 2) + s64(b"general.name") + struct.pack("<I", 8) + s64(b"DeepSeek-V4\0")
+            + s64(b"general.architecture") + struct.pack("<I", 8) + s64(b"kimi-k3\xff") + tensor_w(0))
+    o, g = both(data)
+    assert o["metadata"]["general.name"] == (8, "DeepSeek-V4") and g.meta_str("general.name") == b"DeepSeek-V4"
+    assert og.architecture(o) == "kimi-k3�"
+    assert g.meta_str("general.architecture").decode(errors="replace") == "kimi-k3�"
+    assert g.tensors()["w"][0] == 0
+
+
+def test_string_claim_beyond_cap_is_rejected():
+    # src/gguf_ext.rs:716-750: 32 MiB claimed
+    both_fail(one_kv(b"general.name", struct.pack("<IQ", 8, 32 << 20)), "exceeds max")
+
+
+def test_string_claim_beyond_stream_is_rejected():
+    # src/gguf_ext.rs:752-783: 8 MiB claimed, within the cap, beyond the bytes left
+    both_fail(one_kv(b"general.name", struct.pack("<IQ", 8, 8 << 20)), "bytes remaining")
+
+
+def test_array_element_count_beyond_cap_is_rejected():
+    # src/gguf_ext.rs:785-818
+    both_fail(one_kv(b"tokenizer.ggml.tokens", struct.pack("<IIQ", 9, 8, 32 << 20)), "exceeds max")
+
+
+def test_nested_arrays_parse():
+    # src/gguf_ext.rs:820-878: [[1, 2], [3]]
+    payload = struct.pack("<IIQ", 9, 9, 2) + struct.pack("<IQII", 4, 2, 1, 2) + struct.pack("<IQI", 4, 1, 3)
+    data = one_kv(b"general.special", payload)
+    o, g = both(data)
+    assert o["metadata"]["general.special"] == (9, [(9, [(4, 1), (4, 2)]), (9, [(4, 3)])])
+    assert g.meta_array_len("general.special") == 2
+    special = gw.array(gw.ARRAY, [gw.array(gw.U32, [1, 2]), gw.array(gw.U32, [3])])
+    assert gw.header_bytes({"general.special": special}, [("w", [8, 64], 0, 0)]) == data
+
+
+def test_value_nesting_depth_is_capped():
+    # src/gguf_ext.rs:880-919: 66 nested arrays
+    payload = struct.pack("<I", 9) + struct.pack("<IQ", 9, 1) * 66 + struct.pack("<IQI", 0, 1, 42)
+    both_fail(one_kv(b"general.deep", payload), "nesting depth")
+    # 60 levels are fine (an innermost array of one u32)
+    payload = struct.pack("<I", 9) + struct.pack("<IQ", 9, 1) * 60 + struct.pack("<IQI", 4, 1, 42)
+    both(one_kv(b"general.deep", payload))
+
+
+def test_unknown_value_type_and_too_many_dimensions():
+    both_fail(one_kv(b"k", struct.pack("<II", 13, 0)), "unknown metadata value type 13")
+    data = MAGIC + struct.pack("<IQQ", 3, 1, 0) + s64(b"w") + struct.pack("<I", 9)
+    both_fail(data, "claims 9 dimensions")
+
+
+@pytest.mark.parametrize("vtype,fmt,value,ok", [
+    (gw.U8, "<B", 64, True), (gw.U16, "<H", 4096, True), (gw.U32, "<I", 128, True), (gw.I8, "<b", 16, True),
+    (gw.I16, "<h", 256, True), (gw.I32, "<i", 1, True), (gw.U32, "<I", 48, False), (gw.U32, "<I", 0, False),
+    (gw.I32, "<i", -64, None), (gw.U64, "<Q", 64, None), (gw.F32, "<f", 64.0, None),
+])
+def test_alignment_rules(vtype, fmt, value, ok):
+    """src/gguf_ext.rs:456-473: integer types up to 32 bits that are not negative set the alignment, anything
+    else leaves 32; zero and non-powers of two are refused."""
+    data = one_kv(b"general.alignment", struct.pack("<I", vtype) + struct.pack(fmt, value))
+    if ok is False:
+        both_fail(data, "invalid general.alignment")
+        return
+    o, g = both(data)
+    align = value if ok else 32
+    assert g.tensor_data_offset == (len(data) + align - 1) // align * align
+    assert g.tensor_data_offset % align == 0
+
+
+def test_type_sizes():
+    # src/gguf_ext.rs:921-948
+    for f in (og.type_size_bytes, capi.type_size_bytes):
+        assert f(39, 64) == 34 and f(39, 40) is None and f(0, 10) == 40
+        for dtype, nbytes in ((10, 84), (11, 110), (12, 144), (13, 176), (14, 210), (15, 292)):
+            assert f(dtype, 256) == nbytes and f(dtype, 512) == 2 * nbytes and f(dtype, 128) is None
+        for dtype, nbytes in ((2, 18), (3, 20), (6, 22), (7, 24), (8, 34), (9, 36)):
+            assert f(dtype, 32) == nbytes and f(dtype, 33) is None
+        assert f(1, 3) == 6 and f(30, 3) == 6 and f(26, 3) == 12 and f(16, 256) == 66
+        assert f(4, 32) is None and f(5, 32) is None and f(40, 32) is None
+
+
+def test_metadata_scalars():
+    md = {"a.u32": gw.u32(7), "a.u8": gw.Value(gw.U8, 200), "a.i32": gw.Value(gw.I32, -3), "a.i16": gw.Value(gw.I16, 12),
+          "a.f32": gw.f32(1e-6), "a.bool": gw.boolean(True), "a.str": gw.string("x"), "a.u64": gw.Value(gw.U64, 1 << 40),
+          "a.f64": gw.Value(gw.F64, 2.5), "a.arr": gw.array(gw.STRING, ["p", "q", "r"])}
+    data = gw.header_bytes(md, [])
+    o, g = both(data)
+    assert g.meta_u32("a.u32") == 7 and g.meta_u32("a.u8") == 200 and g.meta_u32("a.i16") == 12
+    assert g.meta_u32("a.i32") is None and g.meta_u32("a.u64") is None and g.meta_u32("a.f32") is None
+    assert g.meta_u32("missing") is None
+    assert g.meta_f32("a.f32") == np.float32(1e-6) and g.meta_f32("a.f64") is None and g.meta_f32("a.u32") is None
+    assert g.meta_bool("a.bool") is True and g.meta_bool("a.u32") is None
+    assert g.meta_str("a.str") == b"x" and g.meta_str("a.u32") is None
+    assert g.meta_array_len("a.arr") == 3 and g.meta_array_len("a.str") is None
+    assert o["metadata"]["a.arr"] == (9, [(8, "p"), (8, "q"), (8, "r")]) and o["metadata"]["a.u64"] == (10, 1 << 40)
+
+
+def test_truncated_headers_fail_cleanly():
+    data = gw.header_bytes({"general.architecture": gw.string("qwen3"), "x": gw.array(gw.U32, [1, 2, 3])},
+                           [("a", [4, 256], 12, 0), ("b", [2, 3, 256], 14, 1024)])
+    both(data)
+    for cut in range(len(data)):
+        with pytest.raises(og.GgufError):
+            og.read_header(data[:cut])
+        with pytest.raises(capi.JoshuaHipError):
+            capi.Gguf.parse(data[:cut])
+
+
+def test_written_file_reads_back(tmp_path):
+    rng = np.random.default_rng(3)
+    tensors = [("token_embd.weight", 12, [8, 256], rng.integers(0, 256, 8 * 144, dtype=np.uint8)),
+               ("blk.0.attn_norm.weight", 0, [256], rng.standard_normal(256).astype(np.float32)),
+               ("blk.0.ffn_gate_exps.weight", 39, [4, 6, 64], rng.integers(0, 256, 4 * 6 * 2 * 17, dtype=np.uint8)),
+               ("odd", 8, [1, 32], rng.integers(0, 256, 34, dtype=np.uint8))]
+    for align in (None, 64, 8):
+        path = str(tmp_path / f"a{align}.gguf")
+        where = gw.write_gguf(path, {"general.architecture": gw.string("t")}, tensors, alignment=align)
+        o = og.read_header(open(path, "rb").read())
+        g = capi.Gguf.open(path)
+        a = align or 32
+        assert g.tensor_data_offset == o["tensor_data_offset"] and g.tensor_data_offset % a == 0
+        for name, dtype, dims, data in tensors:
+            assert g.tensors()[name][:2] == (dtype, dims) == o["tensors"][name][:2]
+            assert g.tensors()[name][2] % a == 0 and g.tensor_data_offset + g.tensors()[name][2] == where[name]
+            assert np.array_equal(g.tensor_bytes(name), np.ascontiguousarray(data).view(np.uint8).reshape(-1))
+        g.close()
+
+
+def test_tensor_ranges_are_checked(tmp_path):
+    """The borrow check of the mapping (src/mmap_tensor.rs:105-123): a range past the end of the file, an
+    offset that wraps, and a type without a size are refused; nothing is read."""
+    path = str(tmp_path / "short.gguf")
+    directory = [("ok", [1, 256], 12, 0), ("past", [1, 256], 12, 32), ("wrap", [1, 256], 12, (1 << 64) - 16),
+                 ("nosize", [1, 256], 4, 0), ("ragged", [1, 100], 12, 0)]
+    head = gw.header_bytes({}, directory)
+    start = (len(head) + 31) // 32 * 32
+    with open(path, "wb") as f:
+        f.write(head + b"\0" * (start - len(head)) + bytes(range(144)))
+    g = capi.Gguf.open(path)
+    assert g.tensor_bytes("ok").tolist() == list(range(144))
+    for name, phrase in (("past", "run past"), ("wrap", "run past"), ("nosize", "no known size"),
+                         ("ragged", "no known size")):
+        with pytest.raises(capi.JoshuaHipError, match=phrase):
+            g.tensor_bytes(name)
+    with pytest.raises(capi.JoshuaHipError, match="no tensor"):
+        g.tensor_bytes("absent")
+
+
+def test_open_failures(tmp_path):
+    with pytest.raises(capi.JoshuaHipError, match="cannot open"):
+        capi.Gguf.open(str(tmp_path / "nope.gguf"))
+    empty = tmp_path / "empty.gguf"
+    empty.write_bytes(b"")
+    with pytest.raises(capi.JoshuaHipError):
+        capi.Gguf.open(str(empty))
+    junk = tmp_path / "junk.gguf"
+    junk.write_bytes(b"not a model file at all")
+    with pytest.raises(capi.JoshuaHipError, match="bad magic"):
+        capi.Gguf.open(str(junk))
+
+
+def test_plugin_entry_points_reject_null_and_unloadable_models(tmp_path):
+    """Return codes of the model plugin's argument checks (crates/joshua-mock-npu/src/lib.rs:49-51,77-79,
+    121-123); a file that is not a qwen3 GGUF fails to load with -2 before any device call."""
+    import ctypes
+    L = capi.lib()
+    vocab, h = ctypes.c_uint32(), ctypes.c_void_p()
+    assert L.joshua_npu_init(None, 16, ctypes.byref(vocab), ctypes.byref(h)) == -1
+    assert L.joshua_npu_forward(None, None, 0, 0, None) == -1
+    assert L.joshua_npu_reset(None) == -1
+    L.joshua_npu_free(None)
+    junk = tmp_path / "junk.gguf"
+    junk.write_bytes(b"GGUF")
+    p = capi.NpuPlugin(str(junk), 16)
+    assert p.rc == -2 and not p._h
+    other = tmp_path / "other.gguf"
+    other.write_bytes(gw.header_bytes({"general.architecture": gw.string("llama")}, []))
+    p = capi.NpuPlugin(str(other), 16)
+    assert p.rc == -2 and "expected `qwen3`" in capi.last_error()
+    missing = tmp_path / "missing_keys.gguf"
+    missing.write_bytes(gw.header_bytes({"general.architecture": gw.string("qwen3")}, []))
+    p = capi.NpuPlugin(str(missing), 16)
+    assert p.rc == -2 and "missing GGUF metadata key `qwen3.attention.head_count`" in capi.last_error()
