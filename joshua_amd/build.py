@@ -13,6 +13,9 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
     # keep the compiler from forming packed-f32 instructions out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the leading kernel arguments arrive in scalar registers with the wave instead of by a scalar load
+    # from memory at its entry (0.4 us sooner to the first global load of a kernel that starts cold)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 

@@ -247,7 +247,7 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
         const size_t rounds = (tiles + 255) / 256;
         const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)atoi(genv) : (tiles + rounds - 1) / rounds);
 #define JQ_DOT4_LDS(NORM, SWIGLU, NM) \
-    hipLaunchKernelGGL((jq::q4k_gemv_dot4_lds<NORM, SWIGLU>), dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, NM)
+    hipLaunchKernelGGL((jq::q4k_gemv_dot4_lds<NORM, SWIGLU>), dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid, NM)
         if (norm && swiglu) JQ_DOT4_LDS(true, true, *norm);
         else if (norm) JQ_DOT4_LDS(true, false, *norm);
         else if (swiglu) JQ_DOT4_LDS(false, true, jq::QdNorm{});
@@ -278,9 +278,9 @@ int dispatch_q6k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     if (tiles * ng < 512) return -1;  // under two steps a workgroup the staged f32 kernel is as fast (5.9 vs 4.5 us at 1024 x 4096)
     static const char *genv = getenv("JQ_Q6K_DOT4_GRID");
     const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)std::max(atoi(genv), 1) : (tiles + rounds - 1) / rounds);
-    if (ng == 1) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
-    else if (ng == 2) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
-    else hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    if (ng == 1) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
+    else if (ng == 2) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
+    else hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -296,9 +296,9 @@ int dispatch_q8_0_dot4(const uint8_t *W, size_t row_bytes, const float *X, float
     const size_t tiles = (n + jq::Q8D_ROWS - 1) / jq::Q8D_ROWS, rounds = (tiles + 255) / 256;
     if (tiles * ng < 512) return -1;  // under two steps a workgroup the staged f32 kernel is as fast
     const unsigned grid = (unsigned)std::min<size_t>(tiles, (tiles + rounds - 1) / rounds);
-    if (ng == 1) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
-    else if (ng == 2) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
-    else hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n);
+    if (ng == 1) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
+    else if (ng == 2) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
+    else hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
     HIP_TRY(hipGetLastError());
     return 0;
 }

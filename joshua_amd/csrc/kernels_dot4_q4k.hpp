@@ -171,7 +171,7 @@ struct QdNorm {
 // (reference: src/quantized_qwen3_moe.rs:397-401).
 template <bool NORM, bool SWIGLU>
 __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                          float *__restrict__ Y, int n, QdNorm nm) {
+                                                          float *__restrict__ Y, int n, int G, QdNorm nm) {
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][QD_TILE_LDS];
     __shared__ float ss_lds[16];
     __shared__ uint32_t xl_lds[16][64], xh_lds[16][64];
@@ -181,8 +181,9 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, c = lane >> 4;
     // tiles blockIdx.x, blockIdx.x + G, ...: at any moment the chip reads one contiguous stretch of the
-    // matrix (measured 5.4 TB/s against 5.1 TB/s for one contiguous range per workgroup)
-    const int G = (int)gridDim.x;
+    // matrix (measured 5.4 TB/s against 5.1 TB/s for one contiguous range per workgroup).  G, the number of
+    // workgroups, is an argument: with the leading arguments preloaded into scalar registers the first
+    // loads go out 0.4 us after the wave starts, where gridDim.x costs a scalar load from memory first.
     const int n_tiles = (((n + 15) >> 4) - (int)blockIdx.x + G - 1) / G;
     if (n_tiles <= 0) return;
 
@@ -205,8 +206,15 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         if (nm.res) async_load16(nm.res + 256 * wave + 4 * lane, lds_offset_of(r_raw));
     }
     fetch(0, 0);
-    fetch(1, 1);  // (a clamped copy of tile 0 when the workgroup has one tile only)
-    asm volatile("s_waitcnt vmcnt(6)" ::: "memory");  // the activation landed (own wave's data: no barrier needed)
+    // a workgroup with one tile only (4096 rows over 256 workgroups) fetches nothing more; the wait
+    // counts below are for the loads issued after the awaited ones, so they differ by a tile's three
+    const bool two = n_tiles > 1;
+    if (two) {
+        fetch(1, 1);
+        asm volatile("s_waitcnt vmcnt(6)" ::: "memory");  // the activation landed (own wave's data: no barrier needed)
+    } else {
+        asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    }
 
     {
         float4 v = *(const float4 *)&x_raw[wave][4 * lane];
@@ -253,7 +261,9 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
             xs_lds[wave][lane >> 3] = s * (float)sum;
         }
     }
-    asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");  // tile 0 landed (tile 1 may be in flight), planes written
+    // tile 0 landed (tile 1 may be in flight), planes written
+    if (two) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     uint32_t xl_lo[8], xh_lo[8], xl_hi[8], xh_hi[8];

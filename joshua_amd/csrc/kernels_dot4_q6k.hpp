@@ -20,14 +20,13 @@ constexpr int Q6D_SLICE = 16 * 210, Q6D_SLICE_LDS = Q6D_SLICE + 16, Q6D_ROWS = 8
 
 template <int NG>
 __global__ __launch_bounds__(1024) void q6k_gemv_dot4_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                          float *__restrict__ Y, int n) {
+                                                          float *__restrict__ Y, int n, int G) {
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][Q6D_STEP_LDS];
     __shared__ uint32_t xl_lds[NG][16][64], xh_lds[NG][16][64];
     __shared__ float s_lds[NG][16][8];
     __shared__ float red[2][16][Q6D_ROWS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane >> 3, h = (lane >> 2) & 1, e = lane & 3;  // row of the step, half of the super-block, eighth
-    const int G = (int)gridDim.x;
     const int n_tiles = (((n + Q6D_ROWS - 1) / Q6D_ROWS) - (int)blockIdx.x + G - 1) / G;  // row tiles blockIdx.x, + G, ...
     if (n_tiles <= 0) return;
     const int n_steps = NG * n_tiles;

@@ -331,7 +331,7 @@ __global__ __launch_bounds__(128) void attention_merge(const float *__restrict__
     extern __shared__ float wch[];  // [n_chunks] maxima, then rescaling weights; [n_chunks] l
     float *lch = wch + n_chunks;
     const float *pp = part + (size_t)blockIdx.x * n_chunks * (d + 2);
-    for (int ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {
+    for (int ch = threadIdx.x; ch < n_chunks; ch += 128) {
         const float2 ml = *(const float2 *)(pp + (size_t)ch * (d + 2));
         wch[ch] = ml.x, lch[ch] = ml.y;
     }
@@ -339,11 +339,11 @@ __global__ __launch_bounds__(128) void attention_merge(const float *__restrict__
     float mx = -INFINITY;
     for (int ch = 0; ch < n_chunks; ch++) mx = fmaxf(mx, wch[ch]);
     __syncthreads();
-    for (int ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) wch[ch] = lch[ch] > 0.0f ? expf(wch[ch] - mx) : 0.0f;
+    for (int ch = threadIdx.x; ch < n_chunks; ch += 128) wch[ch] = lch[ch] > 0.0f ? expf(wch[ch] - mx) : 0.0f;
     __syncthreads();
     float tot = 0.0f;
     for (int ch = 0; ch < n_chunks; ch++) tot = fmaf(lch[ch], wch[ch], tot);
-    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    for (int c = threadIdx.x; c < d; c += 128) {
         float a = 0.0f;
         for (int ch0 = 0; ch0 < n_chunks; ch0 += 16) {
             float v[16];
