@@ -32,7 +32,7 @@ __device__ __forceinline__ float fixed_scale(float amax, float range) {
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
     const int u = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(u, u, CTRL, 0xF, 0xF, false));
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, u, CTRL, 0xF, 0xF, true));
 }
 __device__ __forceinline__ float sum_row16(float v) {
     v += dpp_f<0x128>(v);  // row_ror:8
@@ -62,7 +62,7 @@ __device__ __forceinline__ float max_row8(float v) {
     return v;
 }
 template <int CTRL>
-__device__ __forceinline__ int dpp_i(int u) { return __builtin_amdgcn_update_dpp(u, u, CTRL, 0xF, 0xF, false); }
+__device__ __forceinline__ int dpp_i(int u) { return __builtin_amdgcn_update_dpp(0, u, CTRL, 0xF, 0xF, true); }
 __device__ __forceinline__ int isum_row8(int v) {
     v += dpp_i<0x141>(v);
     v += dpp_i<0xB1>(v);
@@ -144,6 +144,20 @@ __device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t
     }
 }
 
+// The (scale, min) pairs of sub-blocks 2c and 2c + 1 of a Q4_K block at once and without a branch, for
+// lanes whose c differs: sc and mn hold the two 6-bit values as bytes 0 and 1 (the bits above are junk
+// when c is even), so that `(float)(sc & 0xFF)` and `(float)((sc >> 8) & 0xFF)` are one byte-to-float
+// conversion each.  Same values as q4k_scale_min(.., 2c, ..) and (.., 2c + 1, ..).
+__device__ __forceinline__ void q4k_scale_min_pair(uint32_t s0, uint32_t s1, uint32_t s2, int c, uint32_t &sc,
+                                                   uint32_t &mn) {
+    const int sh = 16 * (c & 1);
+    const uint32_t a = s0 >> sh, b = s1 >> sh, h = s2 >> sh;  // bytes (2c', 2c'+1) of each word, c' = c & 1
+    const uint32_t sc_lo = a & 0x3F3Fu, mn_lo = b & 0x3F3Fu;
+    const uint32_t sc_hi = (h & 0x0F0Fu) | ((a >> 2) & 0x3030u), mn_hi = ((h >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);
+    sc = c < 2 ? sc_lo : sc_hi;
+    mn = c < 2 ? mn_lo : mn_hi;
+}
+
 // IQ2_XXS codebook expanded at compile time to 256 x 8 bytes (value j of entry
 // c in byte j), from the base-3 packed form in iq2xxs_grid_codes.h.
 struct Tables {
@@ -219,9 +233,9 @@ struct Q4_K {  // d | dmin | scales[12] | qs[128]   (reference: src/kquant_dot.r
     __device__ static float dot8(const uint64_t *, const uint8_t *blk, int c, const uint32_t *xl, const uint32_t *xh,
                                  const float *sx, const float *sxs) {
         const uint4 hdr = ld<uint4>(blk);
-        uint32_t sc0, mn0, sc1, mn1;
-        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc0, mn0);
-        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc1, mn1);
+        uint32_t scp, mnp;
+        q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, scp, mnp);
+        const uint32_t sc0 = scp & 0xFFu, sc1 = (scp >> 8) & 0xFFu, mn0 = mnp & 0xFFu, mn1 = (mnp >> 8) & 0xFFu;
         const uint4 qa = ld<uint4>(blk + 16 + 32 * c), qb = ld<uint4>(blk + 32 + 32 * c);
         const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
         int l0 = 0, h0 = 0, l1 = 0, h1 = 0;

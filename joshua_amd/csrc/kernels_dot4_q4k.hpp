@@ -104,9 +104,9 @@ __global__ __launch_bounds__(64 * QD_MAX_WAVES) void q4k_gemv_dot4(const uint8_t
     auto step = [&](QdTile &cur, QdTile &fill) __attribute__((always_inline)) {
         load_tile(t + 2, fill);
 
-        uint32_t sc_lo, mn_lo, sc_hi, mn_hi;
-        q4k_scale_min(cur.hdr.y, cur.hdr.z, cur.hdr.w, 2 * c, sc_lo, mn_lo);
-        q4k_scale_min(cur.hdr.y, cur.hdr.z, cur.hdr.w, 2 * c + 1, sc_hi, mn_hi);
+        uint32_t scp, mnp;
+        q4k_scale_min_pair(cur.hdr.y, cur.hdr.z, cur.hdr.w, c, scp, mnp);
+        const uint32_t sc_lo = scp & 0xFFu, sc_hi = (scp >> 8) & 0xFFu, mn_lo = mnp & 0xFFu, mn_hi = (mnp >> 8) & 0xFFu;
         const uint32_t q[8] = {cur.qa.x, cur.qa.y, cur.qa.z, cur.qa.w, cur.qb.x, cur.qb.y, cur.qb.z, cur.qb.w};
         int sl_lo = 0, sh_lo = 0, sl_hi = 0, sh_hi = 0;
 #pragma unroll
@@ -206,15 +206,12 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         if (nm.res) async_load16(nm.res + 256 * wave + 4 * lane, lds_offset_of(r_raw));
     }
     fetch(0, 0);
-    // a workgroup with one tile only (4096 rows over 256 workgroups) fetches nothing more; the wait
-    // counts below are for the loads issued after the awaited ones, so they differ by a tile's three
+    // Tile 1 is asked for only after the activation has been prepared: every workgroup's tile 0 then has
+    // the memory system to itself and lands sooner, and the arithmetic, which is what the kernel waits
+    // for in the end, starts sooner.  A workgroup with one tile (4096 rows over 256 workgroups) fetches
+    // nothing more.
     const bool two = n_tiles > 1;
-    if (two) {
-        fetch(1, 1);
-        asm volatile("s_waitcnt vmcnt(6)" ::: "memory");  // the activation landed (own wave's data: no barrier needed)
-    } else {
-        asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-    }
+    asm volatile("s_waitcnt vmcnt(3)" ::: "memory");  // the activation landed (own wave's data: no barrier needed)
 
     {
         float4 v = *(const float4 *)&x_raw[wave][4 * lane];
@@ -262,8 +259,12 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         }
     }
     // tile 0 landed (tile 1 may be in flight), planes written
-    if (two) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    if (two) {
+        fetch(1, 1);
+        asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     uint32_t xl_lo[8], xh_lo[8], xl_hi[8], xh_hi[8];
@@ -284,9 +285,9 @@ __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restr
         const uint8_t *blk = &ring[slot][r * QD_ROW_LDS + wave * 144];
         const uint4 hdr = *(const uint4 *)blk;
         const uint4 qa = *(const uint4 *)(blk + 16 + 32 * c), qb = *(const uint4 *)(blk + 32 + 32 * c);
-        uint32_t sc_lo, mn_lo, sc_hi, mn_hi;
-        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc_lo, mn_lo);
-        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc_hi, mn_hi);
+        uint32_t scp, mnp;
+        q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, c, scp, mnp);
+        const uint32_t sc_lo = scp & 0xFFu, sc_hi = (scp >> 8) & 0xFFu, mn_lo = mnp & 0xFFu, mn_hi = (mnp >> 8) & 0xFFu;
         const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
         int sl_lo = 0, sh_lo = 0, sl_hi = 0, sh_hi = 0;
 #pragma unroll
