@@ -25,6 +25,7 @@ __global__ __launch_bounds__(1024) void q6k_gemv_dot4_lds(const uint8_t *__restr
     __shared__ uint32_t xl_lds[NG][16][64], xh_lds[NG][16][64];
     __shared__ float s_lds[NG][16][8];
     __shared__ float red[2][16][Q6D_ROWS];
+    __shared__ __attribute__((aligned(16))) float x_raw[NG][16][256];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane >> 3, h = (lane >> 2) & 1, e = lane & 3;  // row of the step, half of the super-block, eighth
     const int n_tiles = (((n + Q6D_ROWS - 1) / Q6D_ROWS) - (int)blockIdx.x + G - 1) / G;  // row tiles blockIdx.x, + G, ...
@@ -41,13 +42,19 @@ __global__ __launch_bounds__(1024) void q6k_gemv_dot4_lds(const uint8_t *__restr
         async_load16(src, dst);
         if (lane < 41) async_load16(src + 1024, dst + 1024);  // 105 pieces of 16 bytes per half slice
     };
+    // every global read of this kernel is an asynchronous load counted by hand: the activation columns
+    // first, then step 0; step 1 is asked for once the activations are prepared, so that every
+    // workgroup's step 0 has the memory system to itself and the arithmetic starts sooner
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+        async_load16(X + (size_t)(16 * g + wave) * 256 + 4 * lane, lds_offset_of(&x_raw[g][wave][0]));
     fetch(0, 0);
-    fetch(1, 1);  // (a clamped copy of step 0 when there is one step only)
+    asm volatile("s_waitcnt vmcnt(2)" ::: "memory");  // the activations landed (own wave's data: no barrier needed)
 
     // activations of super-block 16 g + wave: 4 elements a lane, one scale per 32
 #pragma unroll
     for (int g = 0; g < NG; g++) {
-        const float4 v = *(const float4 *)(X + (size_t)(16 * g + wave) * 256 + 4 * lane);
+        const float4 v = *(const float4 *)&x_raw[g][wave][4 * lane];
         float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
         amax = max_row8(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
@@ -65,7 +72,13 @@ __global__ __launch_bounds__(1024) void q6k_gemv_dot4_lds(const uint8_t *__restr
         xh_lds[g][wave][lane] = wh;
         if ((lane & 7) == 0) s_lds[g][wave][lane >> 3] = s;
     }
-    asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");  // step 0 landed (step 1 may be in flight), planes written
+    // step 0 landed (step 1 may be in flight), planes written
+    if (n_steps > 1) {
+        fetch(1, 1);
+        asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     // this lane's share: quarter t of half h covers elements 128 h + 32 t + 8 e .. + 7 (two registers a plane)
