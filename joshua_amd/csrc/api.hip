@@ -20,6 +20,7 @@
 #include "kernels_mfma_q4k_gemm.hpp"
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
+#include "kernels_dot4_q4k_r8.hpp"
 #include "kernels_dot4_q6k.hpp"
 #include "kernels_dot4_q8.hpp"
 #include "kernels_moe.hpp"
@@ -236,9 +237,18 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     const size_t nb = k / 256;
     static const char *mode_env = getenv("JQ_Q4K_DOT4");
     static const std::string mode = mode_env ? mode_env : "auto";
-    if (mode == "0" || nb == 0 || nb > jq::QD_MAX_WAVES || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 ||
-        ((uintptr_t)X & 15) != 0)
-        return -1;
+    if (mode == "0" || nb == 0 || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0) return -1;
+    // rows of 8192 or 12288 (a feed-forward down projection): steps of 8 rows x 4096 columns
+    // (4096 x 12288: 9.2 us against 11.1 us for the MFMA GEMV)
+    if (mode == "auto" && !norm && !swiglu && (nb == 32 || nb == 48) && row_bytes == nb / 16 * jq::QD_ROW && n >= 1024) {
+        const size_t tiles8 = (n + 7) / 8, rounds = (tiles8 + 255) / 256;
+        const unsigned grid = (unsigned)((tiles8 + rounds - 1) / rounds);
+        if (nb == 32) hipLaunchKernelGGL(jq::q4k_gemv_dot4_r8<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
+        else hipLaunchKernelGGL(jq::q4k_gemv_dot4_r8<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
+    if (nb > jq::QD_MAX_WAVES) return -1;
     static const char *genv = getenv("JQ_Q4K_DOT4_GRID");
     const size_t tiles = (n + 15) / 16;
     if (mode != "regs") {

@@ -335,6 +335,30 @@ def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
     assert np.array_equal(got[0], (x @ q.T).astype(np.float32))
 
 
+@pytest.mark.parametrize("k,n", [(8192, 1024), (12288, 1029), (12288, 4096), (8192, 2043)])
+def test_q4k_dot4_gemv_long_rows(k, n):
+    """Rows of 8192 and 12288, one activation row, 1024 weight rows or more: the v_dot4 kernel in steps
+    of 8 rows x 4096 columns; row counts that leave a partial last step; wide-ranging activations."""
+    blocks = make_blocks(capi.Q4_K, n, k, 51 + n)
+    rng = np.random.default_rng(n)
+    lhs = synth.normal(52 + n, (1, k))
+    lhs[0] *= (10.0 ** rng.integers(-5, 1, size=k // 32)).repeat(32).astype(np.float32)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    assert close(w.matmul_t(1, lhs), oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks, avx2=True))
+    lhs[0, 5000] = np.nan
+    assert np.isnan(w.matmul_t(1, lhs)).all()
+
+
+@pytest.mark.parametrize("k", [8192, 12288])
+def test_q4k_dot4_gemv_long_rows_integer_dot_products_are_bit_exact(k):
+    n = 1040
+    blocks, q, x = q4k_integer_case(n, k, 9, group=32, big_value=32639, small=1000)
+    want = x @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+    assert np.array_equal(got[0], want.astype(np.float32))
+
+
 @pytest.mark.parametrize("m", [17, 64, 200])
 def test_q4k_gemm_integer_dot_products_are_bit_exact(m):
     """The same construction for the MFMA GEMM (m > 16): its activation range is 4193279
