@@ -222,14 +222,21 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
                                                         const float2 *__restrict__ cs, float *kc, float *vc,
                                                         float *__restrict__ part, int n_head, int n_kv,
                                                         const int *__restrict__ pos_ptr, int n_ctx, float sqrt_d,
-                                                        int n_chunks) {
+                                                        int n_chunks, int n_tri) {
     constexpr int d = D, QI = D / 64;          // float4 of q (and of a key) per lane
     constexpr int NG = D / 4, KP = 256 / NG;   // column groups of four, key parts
     constexpr int VI = ATT_CHUNK / KP;         // keys per thread in the value sum
     __shared__ float sc[ATT_CHUNK];
     __shared__ float4 accs[256];               // [key part][column group]
-    const int chunk = blockIdx.x % n_chunks, hq = (blockIdx.x / n_chunks) % n_head, t = blockIdx.x / (n_chunks * n_head);
-    const int group = n_head / n_kv, kvh = hq / group, pos0 = *pos_ptr, n_keys = pos0 + t + 1;
+    // Workgroup ids 8 apart run on the same XCD (ids go round the 8 XCDs in turn) and share its L2: the
+    // query heads of one KV head and chunk read the same key and value rows, so they get ids 8 apart and
+    // the rows come from HBM once.  id = x + 8 (g + group y): g the query head within its group, 8 y + x
+    // the (token, KV head, chunk) triple; ids past the last triple have nothing to do.
+    const int group = n_head / n_kv;
+    const int tri = 8 * ((int)(blockIdx.x >> 3) / group) + (int)(blockIdx.x & 7);
+    if (tri >= n_tri) return;
+    const int chunk = tri % n_chunks, kvh = (tri / n_chunks) % n_kv, t = tri / (n_chunks * n_kv);
+    const int hq = kvh * group + (int)(blockIdx.x >> 3) % group, pos0 = *pos_ptr, n_keys = pos0 + t + 1;
     const int j0 = chunk * ATT_CHUNK, nj = min(ATT_CHUNK, n_keys - j0);
     float *po = part + ((size_t)(t * n_head + hq) * n_chunks + chunk) * (d + 2);
     if (nj <= 0) {
