@@ -44,6 +44,14 @@ extern "C" {
 #define JQ_TYPE_Q6_K 14u
 #define JQ_TYPE_IQ2_XXS 16u
 #define JQ_TYPE_MXFP4 39u
+/* Formats the reference serves through the canonical decode plus the 8-lane dot
+ * (reference: src/quant_matmul.rs:228-248; sizes src/gguf_ext.rs:487-500). */
+#define JQ_TYPE_Q4_0 2u
+#define JQ_TYPE_Q4_1 3u
+#define JQ_TYPE_Q5_0 6u
+#define JQ_TYPE_Q5_1 7u
+#define JQ_TYPE_Q3_K 11u
+#define JQ_TYPE_Q5_K 13u
 
 typedef struct jq_weight jq_weight;
 

@@ -16,7 +16,12 @@ LIB_PATH = os.path.join(_HERE, "libjoshua_hip.so")
 
 Q8_0, Q2_K, Q4_K, Q6_K, IQ2_XXS, MXFP4 = 8, 10, 12, 14, 16, 39
 ALL_TYPES = (Q8_0, Q2_K, Q4_K, Q6_K, IQ2_XXS, MXFP4)
-TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "IQ2_XXS", MXFP4: "MXFP4"}
+# formats the reference serves through the canonical decode plus its 8-lane dot
+# (reference: src/quant_matmul.rs:228-248; sizes src/gguf_ext.rs:487-500)
+Q4_0, Q4_1, Q5_0, Q5_1, Q3_K, Q5_K = 2, 3, 6, 7, 11, 13
+GENERIC_TYPES = (Q4_0, Q4_1, Q5_0, Q5_1, Q3_K, Q5_K)
+TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "IQ2_XXS", MXFP4: "MXFP4", Q4_0: "Q4_0",
+              Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q3_K: "Q3_K", Q5_K: "Q5_K"}
 
 # Every symbol include/joshua_hip.h declares.
 EXPORTS = (

@@ -58,6 +58,12 @@ bool geometry(uint32_t t, Geometry *g) {
     case JQ_TYPE_Q6_K: *g = {256, 210}; return true;
     case JQ_TYPE_IQ2_XXS: *g = {256, 66}; return true;
     case JQ_TYPE_MXFP4: *g = {32, 17}; return true;
+    case JQ_TYPE_Q4_0: *g = {32, 18}; return true;
+    case JQ_TYPE_Q4_1: *g = {32, 20}; return true;
+    case JQ_TYPE_Q5_0: *g = {32, 22}; return true;
+    case JQ_TYPE_Q5_1: *g = {32, 24}; return true;
+    case JQ_TYPE_Q3_K: *g = {256, 110}; return true;
+    case JQ_TYPE_Q5_K: *g = {256, 176}; return true;
     default: return false;
     }
 }
@@ -68,11 +74,19 @@ const char *type_name(uint32_t t) {
     case JQ_TYPE_Q2_K: return "quantized";
     case JQ_TYPE_Q4_K: return "quantized";
     case JQ_TYPE_Q6_K: return "quantized";
+    case JQ_TYPE_Q4_0: case JQ_TYPE_Q4_1: case JQ_TYPE_Q5_0: case JQ_TYPE_Q5_1: case JQ_TYPE_Q3_K: case JQ_TYPE_Q5_K:
+        return "quantized";
     case JQ_TYPE_IQ2_XXS: return "iq2_xxs";
     case JQ_TYPE_MXFP4: return "mxfp4";
     default: return "unknown";
     }
 }
+
+// Every block format the library decodes: X(type id, trait).
+#define JQ_FOR_EACH_FORMAT(X) \
+    X(JQ_TYPE_Q8_0, Q8_0) X(JQ_TYPE_Q2_K, Q2_K) X(JQ_TYPE_Q4_K, Q4_K) X(JQ_TYPE_Q6_K, Q6_K) X(JQ_TYPE_IQ2_XXS, IQ2_XXS) \
+    X(JQ_TYPE_MXFP4, MXFP4) X(JQ_TYPE_Q4_0, Q4_0) X(JQ_TYPE_Q4_1, Q4_1) X(JQ_TYPE_Q5_0, Q5_0) X(JQ_TYPE_Q5_1, Q5_1)  \
+    X(JQ_TYPE_Q3_K, Q3_K) X(JQ_TYPE_Q5_K, Q5_K)
 
 std::once_flag g_init_once;
 int g_init_rc = 0;
@@ -433,12 +447,10 @@ int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, floa
 int dispatch_gemm_decoded(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m,
                           size_t k, size_t n, hipStream_t s) {
     switch (type) {
-    case JQ_TYPE_Q8_0: return launch_gemm_decoded<jq::Q8_0>(W, row_bytes, X, Y, m, k, n, s);
-    case JQ_TYPE_Q2_K: return launch_gemm_decoded<jq::Q2_K>(W, row_bytes, X, Y, m, k, n, s);
-    case JQ_TYPE_Q4_K: return launch_gemm_decoded<jq::Q4_K>(W, row_bytes, X, Y, m, k, n, s);
-    case JQ_TYPE_Q6_K: return launch_gemm_decoded<jq::Q6_K>(W, row_bytes, X, Y, m, k, n, s);
-    case JQ_TYPE_IQ2_XXS: return launch_gemm_decoded<jq::IQ2_XXS>(W, row_bytes, X, Y, m, k, n, s);
-    case JQ_TYPE_MXFP4: return launch_gemm_decoded<jq::MXFP4>(W, row_bytes, X, Y, m, k, n, s);
+#define JQ_CASE(ID, Q) \
+    case ID: return launch_gemm_decoded<jq::Q>(W, row_bytes, X, Y, m, k, n, s);
+        JQ_FOR_EACH_FORMAT(JQ_CASE)
+#undef JQ_CASE
     default: return -1;
     }
 }
@@ -480,12 +492,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         if (rc >= 0) return rc;
     }
     switch (type) {
-    case JQ_TYPE_Q8_0: launch_rows<jq::Q8_0>(W, row_bytes, X, Y, m, k, n, s); break;
-    case JQ_TYPE_Q2_K: launch_rows<jq::Q2_K>(W, row_bytes, X, Y, m, k, n, s); break;
-    case JQ_TYPE_Q4_K: launch_rows<jq::Q4_K>(W, row_bytes, X, Y, m, k, n, s); break;
-    case JQ_TYPE_Q6_K: launch_rows<jq::Q6_K>(W, row_bytes, X, Y, m, k, n, s); break;
-    case JQ_TYPE_IQ2_XXS: launch_rows<jq::IQ2_XXS>(W, row_bytes, X, Y, m, k, n, s); break;
-    case JQ_TYPE_MXFP4: launch_rows<jq::MXFP4>(W, row_bytes, X, Y, m, k, n, s); break;
+#define JQ_CASE(ID, Q) \
+    case ID: launch_rows<jq::Q>(W, row_bytes, X, Y, m, k, n, s); break;
+        JQ_FOR_EACH_FORMAT(JQ_CASE)
+#undef JQ_CASE
     default: return fail("unsupported tensor type id %u", type);
     }
     HIP_TRY(hipGetLastError());
@@ -503,12 +513,10 @@ void launch_decode(const jq_weight *w, const uint32_t *ids, float *out, size_t r
 
 int dispatch_decode(const jq_weight *w, const uint32_t *ids, float *out, size_t rows, hipStream_t s) {
     switch (w->type) {
-    case JQ_TYPE_Q8_0: launch_decode<jq::Q8_0>(w, ids, out, rows, s); break;
-    case JQ_TYPE_Q2_K: launch_decode<jq::Q2_K>(w, ids, out, rows, s); break;
-    case JQ_TYPE_Q4_K: launch_decode<jq::Q4_K>(w, ids, out, rows, s); break;
-    case JQ_TYPE_Q6_K: launch_decode<jq::Q6_K>(w, ids, out, rows, s); break;
-    case JQ_TYPE_IQ2_XXS: launch_decode<jq::IQ2_XXS>(w, ids, out, rows, s); break;
-    case JQ_TYPE_MXFP4: launch_decode<jq::MXFP4>(w, ids, out, rows, s); break;
+#define JQ_CASE(ID, Q) \
+    case ID: launch_decode<jq::Q>(w, ids, out, rows, s); break;
+        JQ_FOR_EACH_FORMAT(JQ_CASE)
+#undef JQ_CASE
     default: return fail("unsupported tensor type id %u", w->type);
     }
     HIP_TRY(hipGetLastError());
@@ -827,12 +835,7 @@ int dispatch_moe_staged(uint32_t type, const uint8_t *const *Wa, const uint8_t *
         rc = launch_moe_staged<jq::Q, DUAL>(Wa, Wb, row_bytes, aligned16, X, gexp, offsets, xsel, yrow, Y, k, n,     \
                                             groups, max_group, s);                                                  \
         break;
-        JQ_MOE_CASE(JQ_TYPE_Q8_0, Q8_0)
-        JQ_MOE_CASE(JQ_TYPE_Q2_K, Q2_K)
-        JQ_MOE_CASE(JQ_TYPE_Q4_K, Q4_K)
-        JQ_MOE_CASE(JQ_TYPE_Q6_K, Q6_K)
-        JQ_MOE_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
-        JQ_MOE_CASE(JQ_TYPE_MXFP4, MXFP4)
+        JQ_FOR_EACH_FORMAT(JQ_MOE_CASE)
 #undef JQ_MOE_CASE
     default: return fail("unsupported tensor type id %u", type);
     }
@@ -929,12 +932,7 @@ int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_byte
         launch_moe_rows<jq::Q, SWIGLU>(Wptr, row_bytes, X, X2, gexp, offsets, xsel, yrow, Y, k, n, groups, max_group, \
                                        s);                                                                          \
         break;
-        JQ_MOE_CASE(JQ_TYPE_Q8_0, Q8_0)
-        JQ_MOE_CASE(JQ_TYPE_Q2_K, Q2_K)
-        JQ_MOE_CASE(JQ_TYPE_Q4_K, Q4_K)
-        JQ_MOE_CASE(JQ_TYPE_Q6_K, Q6_K)
-        JQ_MOE_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
-        JQ_MOE_CASE(JQ_TYPE_MXFP4, MXFP4)
+        JQ_FOR_EACH_FORMAT(JQ_MOE_CASE)
 #undef JQ_MOE_CASE
     default: return fail("unsupported tensor type id %u", type);
     }

@@ -203,6 +203,75 @@ struct Q8_0 {  // d:f16 | qs[32] i8   (reference: src/kquant_dot.rs:53-61,287-30
     }
 };
 
+// The 32-element formats with 4 or 5 bits a weight.  The reference has no kernel of its own for them:
+// they run through the canonical decode plus the 8-lane dot (reference: src/quant_matmul.rs:228-248);
+// the layouts are those of vendor/candle-metal-kernels/src/metal_src/quantized.metal:21-61 and the
+// element maps those of its dequantize_q4_0 .. dequantize_q5_1 (:6482-6567): byte j of qs holds
+// element j in its low and element j + 16 in its high nibble, bit e of qh is the fifth bit of element e.
+// Every product below is exact in f32 and each weight has at most one rounding, so the order of the
+// operations does not matter.
+struct Q4_0 {  // d:f16 | qs[16]        w = d (q - 8)
+    static constexpr int BLOCK_ELEMS = 32, BLOCK_BYTES = 18, UNITS = 1;
+    static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
+    __device__ static int elem_base(int) { return 0; }
+    __device__ static void decode(const uint8_t *blk, int, float *w) {
+        const float d = f16_bits(ld<uint16_t>(blk));
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int b = blk[2 + j];
+            w[j] = d * (float)((b & 0xF) - 8);
+            w[j + 16] = d * (float)((b >> 4) - 8);
+        }
+    }
+};
+
+struct Q4_1 {  // d:f16 | m:f16 | qs[16]        w = d q + m
+    static constexpr int BLOCK_ELEMS = 32, BLOCK_BYTES = 20, UNITS = 1;
+    static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
+    __device__ static int elem_base(int) { return 0; }
+    __device__ static void decode(const uint8_t *blk, int, float *w) {
+        const float d = f16_bits(ld<uint16_t>(blk)), m = f16_bits(ld<uint16_t>(blk + 2));
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int b = blk[4 + j];
+            w[j] = fmaf(d, (float)(b & 0xF), m);
+            w[j + 16] = fmaf(d, (float)(b >> 4), m);
+        }
+    }
+};
+
+struct Q5_0 {  // d:f16 | qh:u32 | qs[16]        w = d (q - 16)
+    static constexpr int BLOCK_ELEMS = 32, BLOCK_BYTES = 22, UNITS = 1;
+    static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
+    __device__ static int elem_base(int) { return 0; }
+    __device__ static void decode(const uint8_t *blk, int, float *w) {
+        const float d = f16_bits(ld<uint16_t>(blk));
+        const uint32_t qh = ld<uint32_t>(blk + 2);
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int b = blk[6 + j];
+            w[j] = d * (float)(((b & 0xF) | (int)(((qh >> j) & 1u) << 4)) - 16);
+            w[j + 16] = d * (float)(((b >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4)) - 16);
+        }
+    }
+};
+
+struct Q5_1 {  // d:f16 | m:f16 | qh:u32 | qs[16]        w = d q + m
+    static constexpr int BLOCK_ELEMS = 32, BLOCK_BYTES = 24, UNITS = 1;
+    static constexpr int SEGS = 1, SEGLEN = 32, SEG_STRIDE = 0;
+    __device__ static int elem_base(int) { return 0; }
+    __device__ static void decode(const uint8_t *blk, int, float *w) {
+        const float d = f16_bits(ld<uint16_t>(blk)), m = f16_bits(ld<uint16_t>(blk + 2));
+        const uint32_t qh = ld<uint32_t>(blk + 4);
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int b = blk[8 + j];
+            w[j] = fmaf(d, (float)((b & 0xF) | (int)(((qh >> j) & 1u) << 4)), m);
+            w[j + 16] = fmaf(d, (float)((b >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4)), m);
+        }
+    }
+};
+
 struct Q4_K {  // d | dmin | scales[12] | qs[128]   (reference: src/kquant_dot.rs:78-93,426-466)
     static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 144, UNITS = 4;
     static constexpr int SEGS = 1, SEGLEN = 64, SEG_STRIDE = 0;
@@ -277,6 +346,57 @@ struct Q2_K {  // scales[16] | qs[64] | d | dmin   (reference: src/kquant_dot.rs
 #pragma unroll
                 for (int b = 0; b < 4; b++) w[16 * f + 4 * i + b] = fmaf((float)((v >> (8 * b)) & 0xFFu), d1, -m1);
             }
+        }
+    }
+};
+
+struct Q3_K {  // hmask[32] | qs[64] | scales[12] | d        w = d (sc - 32) (q - (hbit ? 0 : 4))
+    // (layout and element map: vendor/candle-metal-kernels/src/metal_src/quantized.metal:151-156,6597-6623)
+    // unit u = (half h = u/2, byte half hf = u%2): 16 bytes of qs, four 2-bit fields t -> elements
+    // 128 h + 32 t + 16 hf + [0,16); their third bit is bit 4 h + t of hmask[16 hf + i]; the 6-bit scale
+    // of the 16 elements is number 8 h + 2 t + hf: low four bits in scales[0..7] (a nibble each, the
+    // first eight scales low, the next eight high), high two bits in scales[8..11].
+    static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 110, UNITS = 4;
+    static constexpr int SEGS = 4, SEGLEN = 16, SEG_STRIDE = 32;
+    __device__ static int elem_base(int u) { return 128 * (u >> 1) + 16 * (u & 1); }
+    __device__ static void decode(const uint8_t *blk, int u, float *w) {
+        const int h = u >> 1, hf = u & 1;
+        const float d = f16_bits(ld<uint16_t>(blk + 108));
+        const uint8_t *q = blk + 32 + 32 * h + 16 * hf, *hm = blk + 16 * hf, *sc = blk + 96;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int is = 8 * h + 2 * t + hf;
+            const int low4 = is < 8 ? (sc[is] & 0xF) : (sc[is - 8] >> 4);
+            const int high2 = (sc[8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+            const float dl = d * (float)((low4 | (high2 << 4)) - 32);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int v = ((q[i] >> (2 * t)) & 3) - (((hm[i] >> (4 * h + t)) & 1) ? 0 : 4);
+                w[16 * t + i] = dl * (float)v;
+            }
+        }
+    }
+};
+
+struct Q5_K {  // d | dmin | scales[12] | qh[32] | qs[128]        w = d sc q - dmin m
+    // (layout and element map: vendor/candle-metal-kernels/src/metal_src/quantized.metal:176-189,6649-6670)
+    // unit c: 64 elements, sub-blocks 2c (low nibbles of qs[32c + l]) and 2c + 1 (high nibbles); the
+    // fifth bit of element l of sub-block j is bit j of qh[l]; scales and mins are packed as in Q4_K.
+    static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 176, UNITS = 4;
+    static constexpr int SEGS = 1, SEGLEN = 64, SEG_STRIDE = 0;
+    __device__ static int elem_base(int u) { return 64 * u; }
+    __device__ static void decode(const uint8_t *blk, int c, float *w) {
+        const uint4 hdr = ld<uint4>(blk);
+        const float d = f16_bits(hdr.x), dmin = f16_bits(hdr.x >> 16);
+        uint32_t sc0, mn0, sc1, mn1;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c, sc0, mn0);
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, 2 * c + 1, sc1, mn1);
+        const float d0 = d * (float)sc0, m0 = dmin * (float)mn0, d1 = d * (float)sc1, m1 = dmin * (float)mn1;
+#pragma unroll
+        for (int l = 0; l < 32; l++) {
+            const int b = blk[48 + 32 * c + l], hb = blk[16 + l];
+            w[l] = fmaf((float)((b & 0xF) | (((hb >> (2 * c)) & 1) << 4)), d0, -m0);
+            w[32 + l] = fmaf((float)((b >> 4) | (((hb >> (2 * c + 1)) & 1) << 4)), d1, -m1);
         }
     }
 };

@@ -84,3 +84,28 @@ def normal_quantized(qtype: int, seed: int, n_elems: int, sigma: float, mean: fl
     if _L().jsyn_normal_quantized(qtype, seed, start, n_elems, mean, sigma, out.ctypes.data, threads) != 0:
         raise ValueError(f"cannot quantize {n_elems} elements as type {qtype}")
     return out
+
+
+# (block elements, block bytes, [(byte offset of an f16 scale, its magnitude)]) of the formats that have no
+# quantizer here: every byte pattern is a valid block, so seeded random bytes with sane scales stand in
+# for quantized weights of roughly N(0, 0.02).
+_RANDOM_LAYOUT = {
+    2: (32, 18, [(0, 2.0 ** -8)]), 3: (32, 20, [(0, 2.0 ** -8), (2, -7.5 * 2.0 ** -8)]),
+    6: (32, 22, [(0, 2.0 ** -9)]), 7: (32, 24, [(0, 2.0 ** -9), (2, -15.5 * 2.0 ** -9)]),
+    11: (256, 110, [(108, 2.0 ** -12)]), 13: (256, 176, [(0, 2.0 ** -14), (2, 2.0 ** -13)]),
+}
+
+
+def random_blocks(qtype: int, seed: int, n_elems: int) -> np.ndarray:
+    """Packed blocks of Q4_0, Q4_1, Q5_0, Q5_1, Q3_K or Q5_K (ids 2, 3, 6, 7, 11, 13) holding seeded random
+    quants and scales within a factor of two of a per-format magnitude (negative for the offsets of Q4_1
+    and Q5_1, which centres their weights)."""
+    elems, nbytes, scales = _RANDOM_LAYOUT[qtype]
+    if n_elems % elems:
+        raise ValueError(f"type {qtype}: {n_elems} elements is not a whole number of blocks")
+    rng = np.random.default_rng(seed * 1000 + qtype)
+    blk = rng.integers(0, 256, size=(n_elems // elems, nbytes), dtype=np.uint8)
+    for off, mag in scales:
+        v = mag * rng.uniform(0.5, 1.0, size=blk.shape[0])
+        blk[:, off:off + 2] = v.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    return blk.reshape(-1)

@@ -19,7 +19,10 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 Q8_0, Q2_K, Q4_K, Q6_K, IQ2_XXS, MXFP4 = 8, 10, 12, 14, 16, 39
 ALL_TYPES = (Q8_0, Q2_K, Q4_K, Q6_K, IQ2_XXS, MXFP4)
-TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "IQ2_XXS", MXFP4: "MXFP4"}
+Q4_0, Q4_1, Q5_0, Q5_1, Q3_K, Q5_K = 2, 3, 6, 7, 11, 13
+GENERIC_TYPES = (Q4_0, Q4_1, Q5_0, Q5_1, Q3_K, Q5_K)   # decoded by to_float, multiplied by the 8-lane dot
+TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "IQ2_XXS", MXFP4: "MXFP4", 2: "Q4_0",
+              3: "Q4_1", 6: "Q5_0", 7: "Q5_1", 11: "Q3_K", 13: "Q5_K"}
 
 
 def build(force: bool = False) -> str:

@@ -62,6 +62,12 @@ int orc_block_geometry(uint32_t type, size_t *elems, size_t *bytes) {
     case ORC_TYPE_Q6_K: e = 256; b = 210; break;
     case ORC_TYPE_IQ2_XXS: e = 256; b = 66; break;
     case ORC_TYPE_MXFP4: e = 32; b = 17; break;
+    case ORC_TYPE_Q4_0: e = 32; b = 18; break;
+    case ORC_TYPE_Q4_1: e = 32; b = 20; break;
+    case ORC_TYPE_Q5_0: e = 32; b = 22; break;
+    case ORC_TYPE_Q5_1: e = 32; b = 24; break;
+    case ORC_TYPE_Q3_K: e = 256; b = 110; break;
+    case ORC_TYPE_Q5_K: e = 256; b = 176; break;
     default: return -1;
     }
     if (elems) *elems = e;
@@ -178,6 +184,85 @@ static void deq_q6_k(const uint8_t *b, float *y) {
     }
 }
 
+/* The formats below have no kernel in the reference: candle's to_float (third party, not in the
+ * container) decodes them and dot_row_avx2 multiplies (src/quant_matmul.rs:228-248).  Layouts and
+ * element maps are restated from the vendored Metal source, the one statement of them under
+ * /root/reference: vendor/candle-metal-kernels/src/metal_src/quantized.metal:21-61 (structs of the
+ * 32-element formats), :151-156 and :176-189 (Q3_K, Q5_K), :6482-6567 and :6597-6670 (element maps).
+ * Every product is exact in f32 and each weight is rounded at most once, so the values do not depend
+ * on the order of the operations; pinned by tests/np_decode.py on arbitrary bytes and by exhaustive
+ * field sweeps. */
+static void deq_q4_0(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b));
+    for (int j = 0; j < 16; j++) {
+        y[j] = (float)((b[2 + j] & 0xF) - 8) * d;
+        y[j + 16] = (float)((b[2 + j] >> 4) - 8) * d;
+    }
+}
+
+static void deq_q4_1(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b)), m = orc_f16_to_f32(rd16(b + 2));
+    for (int j = 0; j < 16; j++) {
+        y[j] = (float)(b[4 + j] & 0xF) * d + m;
+        y[j + 16] = (float)(b[4 + j] >> 4) * d + m;
+    }
+}
+
+static void deq_q5_0(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b));
+    uint32_t qh = rd32(b + 2);
+    for (int j = 0; j < 16; j++) {
+        int lo = (b[6 + j] & 0xF) | (int)(((qh >> j) & 1u) << 4);
+        int hi = (b[6 + j] >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4);
+        y[j] = (float)(lo - 16) * d;
+        y[j + 16] = (float)(hi - 16) * d;
+    }
+}
+
+static void deq_q5_1(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b)), m = orc_f16_to_f32(rd16(b + 2));
+    uint32_t qh = rd32(b + 4);
+    for (int j = 0; j < 16; j++) {
+        int lo = (b[8 + j] & 0xF) | (int)(((qh >> j) & 1u) << 4);
+        int hi = (b[8 + j] >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4);
+        y[j] = (float)lo * d + m;
+        y[j + 16] = (float)hi * d + m;
+    }
+}
+
+/* hmask[32] | qs[64] | scales[12] | d.  Element e = 128 h + 32 t + l: two low bits from field t of
+ * qs[32 h + l], third bit = bit 4 h + t of hmask[l] (set: nothing subtracted, clear: 4); sixteen 6-bit
+ * scales, one per 16 elements. */
+static void deq_q3_k(const uint8_t *b, float *y) {
+    const uint8_t *hm = b, *qs = b + 32, *sc = b + 96;
+    float d = orc_f16_to_f32(rd16(b + 108));
+    for (int e = 0; e < 256; e++) {
+        int h = e / 128, t = (e % 128) / 32, l = e % 32, is = e / 16;
+        int low4 = is < 8 ? (sc[is] & 0xF) : (sc[is - 8] >> 4);
+        int high2 = (sc[8 + is % 4] >> (2 * (is / 4))) & 3;
+        int scale = (low4 | (high2 << 4)) - 32;
+        int q = ((qs[32 * h + l] >> (2 * t)) & 3) - (((hm[l] >> (4 * h + t)) & 1) ? 0 : 4);
+        y[e] = (d * (float)scale) * (float)q;
+    }
+}
+
+/* d | dmin | scales[12] | qh[32] | qs[128].  Sub-block j (32 elements): nibble (j & 1) of
+ * qs[32 (j / 2) + l], fifth bit = bit j of qh[l]; scales and mins packed as in Q4_K. */
+static void deq_q5_k(const uint8_t *b, float *y) {
+    float d = orc_f16_to_f32(rd16(b)), dmin = orc_f16_to_f32(rd16(b + 2));
+    const uint8_t *qh = b + 16, *qs = b + 48;
+    for (int j = 0; j < 8; j++) {
+        uint8_t sc, mn;
+        orc_q4k_scale_min(b + 4, j, &sc, &mn);
+        float d1 = d * (float)sc, m1 = dmin * (float)mn;
+        for (int l = 0; l < 32; l++) {
+            int nib = (j & 1) ? (qs[32 * (j / 2) + l] >> 4) : (qs[32 * (j / 2) + l] & 0xF);
+            int q = nib | (((qh[l] >> j) & 1) << 4);
+            y[32 * j + l] = d1 * (float)q - m1;
+        }
+    }
+}
+
 /* (reference: src/iq2xxs.rs:44-71). */
 static void deq_iq2_xxs(const uint8_t *b, float *y) {
     float d = orc_f16_to_f32(rd16(b));
@@ -222,6 +307,12 @@ static deq_fn deq_for(uint32_t type) {
     case ORC_TYPE_Q6_K: return deq_q6_k;
     case ORC_TYPE_IQ2_XXS: return deq_iq2_xxs;
     case ORC_TYPE_MXFP4: return deq_mxfp4;
+    case ORC_TYPE_Q4_0: return deq_q4_0;
+    case ORC_TYPE_Q4_1: return deq_q4_1;
+    case ORC_TYPE_Q5_0: return deq_q5_0;
+    case ORC_TYPE_Q5_1: return deq_q5_1;
+    case ORC_TYPE_Q3_K: return deq_q3_k;
+    case ORC_TYPE_Q5_K: return deq_q5_k;
     default: return NULL;
     }
 }
@@ -377,6 +468,12 @@ int orc_matmul_t(uint32_t type, size_t m, size_t k, size_t n, const float *lhs, 
     /* No fused kernel: to_float into a k-float scratch, then the 8-lane dot
      * (reference: src/quant_matmul.rs:228-248,292-325). */
     case ORC_TYPE_Q6_K: rowdec = deq_q6_k; break;
+    case ORC_TYPE_Q4_0: rowdec = deq_q4_0; break;
+    case ORC_TYPE_Q4_1: rowdec = deq_q4_1; break;
+    case ORC_TYPE_Q5_0: rowdec = deq_q5_0; break;
+    case ORC_TYPE_Q5_1: rowdec = deq_q5_1; break;
+    case ORC_TYPE_Q3_K: rowdec = deq_q3_k; break;
+    case ORC_TYPE_Q5_K: rowdec = deq_q5_k; break;
     default: return orc_fail("unknown tensor type %u", type);
     }
     float *w = (float *)malloc(k * sizeof(float));

@@ -30,6 +30,15 @@
  *                            to_float) whose source is not available, so the
  *                            ulp-level operation order ((d*sc)*q) is
  *                            PARITY UNPINNED.
+ *   orc_dequantize Q4_0/Q4_1/Q5_0/Q5_1/Q3_K/Q5_K  pinned on layout by an
+ *                            independent numpy decode written from the block
+ *                            definitions and by exhaustive sweeps of every
+ *                            field; the values do not depend on the operation
+ *                            order (every product is exact in f32, one rounding
+ *                            at most per weight), so nothing is left open at
+ *                            ulp level.  The reference decodes them through
+ *                            candle-core ^0.11 k_quants (not in the container);
+ *                            the layouts come from the vendored Metal source.
  *   orc_matmul_t (all)       pinned: equals a float64 GEMM over the decoded
  *                            weights within the reference's own tolerances,
  *                            assign semantics, shape rejection, scalar build
@@ -54,7 +63,15 @@ enum {
     ORC_TYPE_Q4_K = 12,
     ORC_TYPE_Q6_K = 14,
     ORC_TYPE_IQ2_XXS = 16,
-    ORC_TYPE_MXFP4 = 39
+    ORC_TYPE_MXFP4 = 39,
+    /* served by the reference through candle's to_float plus the 8-lane dot
+     * (src/quant_matmul.rs:228-248); sizes src/gguf_ext.rs:487-500 */
+    ORC_TYPE_Q4_0 = 2,
+    ORC_TYPE_Q4_1 = 3,
+    ORC_TYPE_Q5_0 = 6,
+    ORC_TYPE_Q5_1 = 7,
+    ORC_TYPE_Q3_K = 11,
+    ORC_TYPE_Q5_K = 13
 };
 
 /* Elements and bytes per block of `type`; returns 0, or -1 for an unknown id. */

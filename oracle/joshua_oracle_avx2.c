@@ -380,12 +380,20 @@ static void rows_worker(void *ctx, size_t rb, size_t re) {
     case ORC_TYPE_MXFP4:
         for (size_t r = rb; r < re; r++) row_mxfp4(j, r);
         break;
-    case ORC_TYPE_Q6_K: {
-        /* One scratch per task, reused across its rows
-         * (reference: src/quant_matmul.rs:229-241). */
+    case ORC_TYPE_Q6_K:
+    case ORC_TYPE_Q4_0:
+    case ORC_TYPE_Q4_1:
+    case ORC_TYPE_Q5_0:
+    case ORC_TYPE_Q5_1:
+    case ORC_TYPE_Q3_K:
+    case ORC_TYPE_Q5_K: {
+        /* The generic path: to_float into one scratch per task, reused across its rows, then the
+         * 8-lane dot (reference: src/quant_matmul.rs:229-248). */
+        size_t elems, bytes;
+        orc_block_geometry(j->type, &elems, &bytes);
         float *wrow = (float *)malloc(j->k * sizeof(float));
         for (size_t r = rb; r < re; r++) {
-            orc_dequantize(ORC_TYPE_Q6_K, j->blocks + r * j->bpr * 210, j->bpr, wrow);
+            orc_dequantize(j->type, j->blocks + r * j->bpr * bytes, j->bpr, wrow);
             dot_row_avx2(j, wrow, r);
         }
         free(wrow);

@@ -92,3 +92,74 @@ def iq2_xxs(raw, grid):
         sign = np.where((s8[:, :, None] >> np.arange(8)) & 1, np.float32(-1), np.float32(1))
         out[:, :, l, :] = (db[:, :, None] * g).astype(np.float32) * sign
     return out.reshape(-1)
+
+
+def _nibbles16(qs):  # (blk, 16) bytes -> (blk, 32): element j low nibble of byte j, element j + 16 its high nibble
+    return np.concatenate([qs & 0xF, qs >> 4], axis=1).astype(np.int32)
+
+
+def _fifth_bits(qh4):  # (blk, 4) bytes, little-endian u32 -> (blk, 32): bit e of the word
+    word = np.ascontiguousarray(qh4).view("<u4")[:, 0]
+    return ((word[:, None] >> np.arange(32, dtype=np.uint32)) & 1).astype(np.int32)
+
+
+def q4_0(raw):
+    b = raw.reshape(-1, 18)
+    d = _f16(b[:, 0:2])
+    return ((_nibbles16(b[:, 2:]) - 8).astype(np.float32) * d[:, None]).reshape(-1)
+
+
+def q4_1(raw):
+    b = raw.reshape(-1, 20)
+    d, m = _f16(b[:, 0:2]), _f16(b[:, 2:4])
+    return ((_nibbles16(b[:, 4:]).astype(np.float32) * d[:, None]).astype(np.float32) + m[:, None]).astype(np.float32).reshape(-1)
+
+
+def q5_0(raw):
+    b = raw.reshape(-1, 22)
+    d = _f16(b[:, 0:2])
+    q = _nibbles16(b[:, 6:]) + 16 * _fifth_bits(b[:, 2:6])
+    return ((q - 16).astype(np.float32) * d[:, None]).reshape(-1)
+
+
+def q5_1(raw):
+    b = raw.reshape(-1, 24)
+    d, m = _f16(b[:, 0:2]), _f16(b[:, 2:4])
+    q = _nibbles16(b[:, 8:]) + 16 * _fifth_bits(b[:, 4:8])
+    return ((q.astype(np.float32) * d[:, None]).astype(np.float32) + m[:, None]).astype(np.float32).reshape(-1)
+
+
+def q3_k(raw):
+    b = raw.reshape(-1, 110)
+    hm, qs, sc = b[:, 0:32].astype(np.int32), b[:, 32:96].reshape(-1, 2, 32).astype(np.int32), b[:, 96:108].astype(np.int32)
+    d = _f16(b[:, 108:110])
+    low4 = np.concatenate([sc[:, 0:8] & 0xF, sc[:, 0:8] >> 4], axis=1)                      # scale i: nibble of byte i % 8
+    high2 = np.stack([(sc[:, 8 + i % 4] >> (2 * (i // 4))) & 3 for i in range(16)], axis=1)  # two bits of byte 8 + i % 4
+    scale = (low4 | (high2 << 4)) - 32                                                        # [blk, 16]
+    out = np.empty((b.shape[0], 2, 4, 32), np.int32)
+    for h in range(2):
+        for t in range(4):
+            third = (hm >> (4 * h + t)) & 1
+            out[:, h, t, :] = ((qs[:, h, :] >> (2 * t)) & 3) - 4 * (1 - third)
+    q = out.reshape(-1, 16, 16).astype(np.float32)
+    dl = (d[:, None] * scale.astype(np.float32)).astype(np.float32)
+    return (dl[:, :, None] * q).astype(np.float32).reshape(-1)
+
+
+def q5_k(raw):
+    b = raw.reshape(-1, 176)
+    d, dmin = _f16(b[:, 0:2]), _f16(b[:, 2:4])
+    s = b[:, 4:16].astype(np.int32)
+    sc = np.empty((b.shape[0], 8), np.int32)
+    mn = np.empty_like(sc)
+    sc[:, :4] = s[:, 0:4] & 63
+    mn[:, :4] = s[:, 4:8] & 63
+    sc[:, 4:] = (s[:, 8:12] & 0xF) | ((s[:, 0:4] >> 6) << 4)
+    mn[:, 4:] = (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)
+    qh = b[:, 16:48].astype(np.int32)
+    qs = b[:, 48:].reshape(-1, 4, 32).astype(np.int32)
+    q = np.stack([qs & 0xF, qs >> 4], axis=2).reshape(-1, 8, 32)                      # [blk, sub-block, 32]
+    q = q + 16 * ((qh[:, None, :] >> np.arange(8)[None, :, None]) & 1)
+    d1 = (d[:, None] * sc.astype(np.float32)).astype(np.float32)
+    m1 = (dmin[:, None] * mn.astype(np.float32)).astype(np.float32)
+    return ((d1[:, :, None] * q.astype(np.float32)).astype(np.float32) - m1[:, :, None]).astype(np.float32).reshape(-1)

@@ -128,3 +128,31 @@ def test_upload_from_the_mapping(tmp_path):
         g.upload("absent")
     g.close()
     assert close(w.matmul_t(3, x), oracle.matmul_t(capi.Q6_K, (3, k, n), x, mat))     # the copy in HBM outlives the file
+
+
+def test_model_file_with_the_other_block_formats(tmp_path):
+    """A model whose matrices use Q5_K, Q5_0, Q5_1, Q4_0, Q4_1 and Q3_K beside Q4_K and Q6_K, as the
+    K-quant mixes other than Q4_K_M hold."""
+    plan = qwen3_tensor_plan(CFG)
+    shapes = {n: (r, k) for n, _, r, k in plan}
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(CFG, 47)}
+    swap = {"attn_q": capi.Q5_K, "attn_k": capi.Q5_0, "attn_output": capi.Q5_1, "ffn_gate": capi.Q4_1, "ffn_up": capi.Q3_K,
+            "ffn_down": capi.Q5_K}
+    for name in list(tensors):
+        role = name.split(".")[2] if name.startswith("blk.") else name.split(".")[0]
+        qt = swap.get(role, capi.Q4_0 if role == "token_embd" else None)
+        if qt is not None:
+            r, k = shapes[name]
+            tensors[name] = (qt, synth.random_blocks(qt, 48 + len(name), r * k))
+    path = str(tmp_path / "mixed.gguf")
+    gw.write_qwen3(path, CFG, [(n, qt, d) for n, (qt, d) in tensors.items()], plan)
+    o = oq.Qwen3Oracle(CFG, tensors, avx2=oracle.have_avx2())
+    p = capi.NpuPlugin(path, CFG["n_ctx"])
+    assert p.rc == 0, capi.last_error()
+    prompt = [3, 700, 41, 41, 256, 9, 88]
+    rc, got = p.forward(prompt, 0)
+    assert rc == 0 and close(got, o.forward(prompt, 0))
+    for i, t in enumerate([5, 123]):
+        rc, got = p.forward([t], len(prompt) + i)
+        assert rc == 0 and close(got, o.forward([t], len(prompt) + i))
+    p.close()
