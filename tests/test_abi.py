@@ -37,5 +37,8 @@ def test_block_geometry_needs_no_gpu():
     assert capi.block_geometry(capi.Q6_K) == (256, 210)
     assert capi.block_geometry(capi.IQ2_XXS) == (256, 66)
     assert capi.block_geometry(capi.MXFP4) == (32, 17)
-    with pytest.raises(capi.JoshuaHipError):
-        capi.block_geometry(11)
+    assert [capi.block_geometry(t) for t in capi.GENERIC_TYPES] == [(32, 18), (32, 20), (32, 22), (32, 24), (256, 110),
+                                                                     (256, 176)]
+    for unknown in (0, 1, 4, 5, 9, 15, 30, 40):      # no decode kernel: floats, removed ids, Q8_1, Q8_K
+        with pytest.raises(capi.JoshuaHipError):
+            capi.block_geometry(unknown)
