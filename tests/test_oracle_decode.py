@@ -24,7 +24,7 @@ def test_block_geometry_matches_gguf_table():
     assert oracle.block_geometry(oracle.IQ2_XXS) == (256, 66)
     assert oracle.block_geometry(oracle.MXFP4) == (32, 17)
     with pytest.raises(oracle.OracleError):
-        oracle.block_geometry(11)
+        oracle.block_geometry(15)
 
 
 def test_f16_conversion_every_code():
