@@ -271,11 +271,13 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
         const size_t rounds = (tiles + 255) / 256;
         const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)atoi(genv) : (tiles + rounds - 1) / rounds);
 #define JQ_DOT4_LDS(NORM, SWIGLU, NM) \
-    hipLaunchKernelGGL((jq::q4k_gemv_dot4_lds<NORM, SWIGLU>), dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid, NM)
-        if (norm && swiglu) JQ_DOT4_LDS(true, true, *norm);
-        else if (norm) JQ_DOT4_LDS(true, false, *norm);
-        else if (swiglu) JQ_DOT4_LDS(false, true, jq::QdNorm{});
-        else JQ_DOT4_LDS(false, false, jq::QdNorm{});
+    hipLaunchKernelGGL((jq::q4k_gemv_dot4_lds<NORM, SWIGLU>), dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid, \
+                       NM.res, NM.w, NM.eps, NM.x_out, NM.hn_out)
+        const jq::QdNorm none{};
+        if (norm && swiglu) JQ_DOT4_LDS(true, true, (*norm));
+        else if (norm) JQ_DOT4_LDS(true, false, (*norm));
+        else if (swiglu) JQ_DOT4_LDS(false, true, none);
+        else JQ_DOT4_LDS(false, false, none);
 #undef JQ_DOT4_LDS
         HIP_TRY(hipGetLastError());
         return 0;

@@ -171,7 +171,12 @@ struct QdNorm {
 // (reference: src/quantized_qwen3_moe.rs:397-401).
 template <bool NORM, bool SWIGLU>
 __global__ __launch_bounds__(1024) void q4k_gemv_dot4_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                          float *__restrict__ Y, int n, int G, QdNorm nm) {
+                                                          float *__restrict__ Y, int n, int G, const float *nm_res,
+                                                          const float *nm_w, float nm_eps, float *nm_x_out,
+                                                          float *nm_hn_out) {
+    // the norm's operands are arguments of their own, not a struct: scalars and pointers at the head of
+    // the argument list arrive preloaded in registers, a struct is fetched by a scalar load first
+    const QdNorm nm{nm_res, nm_w, nm_eps, nm_x_out, nm_hn_out};
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][QD_TILE_LDS];
     __shared__ float ss_lds[16];
     __shared__ uint32_t xl_lds[16][64], xh_lds[16][64];
