@@ -1408,9 +1408,9 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         if (split) {  // head norm, rotation and cache writes happen inside the attention kernel
             const int n_tri = (int)(T * nkv * n_chunks);
 #define JQ_ATT_SPLIT(D)                                                                                          \
-    hipLaunchKernelGGL(jq::attention_split<D>, dim3(8 * (nh / nkv) * ((n_tri + 7) / 8)), dim3(256), 0, s, qp, kp, \
-                       vp, w_qn, w_kn, c.rms_eps, m->rope_cs, m->kc[l], m->vc[l], m->part, nh, nkv, m->pos,        \
-                       (int)c.n_ctx, sqrt_d, n_chunks, n_tri)
+    hipLaunchKernelGGL(jq::attention_split<D>, dim3(8 * (nh / nkv) * ((n_tri + 7) / 8)), dim3(256), 0, s, nh, nkv, \
+                       n_chunks, n_tri, (int)pos, (int)c.n_ctx, qp, kp, vp, m->kc[l], m->vc[l], w_qn, w_kn,         \
+                       m->rope_cs, m->part, c.rms_eps, sqrt_d)
             if (d == 64) JQ_ATT_SPLIT(64);
             else if (d == 128) JQ_ATT_SPLIT(128);
             else JQ_ATT_SPLIT(256);

@@ -210,19 +210,20 @@ __device__ __forceinline__ void head_norm_rope(float4 (&x)[D / 64], const float 
 // 16 lanes per key (4 keys per wave step), head_dim 64, 128 or 256.  Chunks past the causal
 // limit write l = 0 and are skipped by the merge.
 // q, k, v are the step's raw projections: the kernel applies the per-head RMSNorm and the rotation to
-// its query row and to the keys of the step's own tokens (positions *pos_ptr and up, not in the cache
+// its query row and to the keys of the step's own tokens (positions pos0 and up, not in the cache
 // yet) itself, and the workgroups of a kv head's first query head store the new key and value rows
 // into the cache for the steps to come.
 constexpr int ATT_CHUNK = 64;
 
 template <int D>  // head_dim: 64, 128 or 256
-__global__ __launch_bounds__(256) void attention_split(const float *__restrict__ q, const float *__restrict__ k,
-                                                        const float *__restrict__ v, const float *__restrict__ wq,
-                                                        const float *__restrict__ wk, float eps,
-                                                        const float2 *__restrict__ cs, float *kc, float *vc,
-                                                        float *__restrict__ part, int n_head, int n_kv,
-                                                        const int *__restrict__ pos_ptr, int n_ctx, float sqrt_d,
-                                                        int n_chunks, int n_tri) {
+__global__ __launch_bounds__(256) void attention_split(int n_head, int n_kv, int n_chunks, int n_tri, int pos0, int n_ctx,
+                                                        const float *__restrict__ q, const float *__restrict__ k,
+                                                        const float *__restrict__ v, float *kc, float *vc,
+                                                        const float *__restrict__ wq, const float *__restrict__ wk,
+                                                        const float2 *__restrict__ cs, float *__restrict__ part,
+                                                        float eps, float sqrt_d) {
+    // (what the first loads need comes first in the argument list: the leading 16 words of arguments
+    // arrive in scalar registers with the wave, the rest by a scalar load)
     constexpr int d = D, QI = D / 64;          // float4 of q (and of a key) per lane
     constexpr int NG = D / 4, KP = 256 / NG;   // column groups of four, key parts
     constexpr int VI = ATT_CHUNK / KP;         // keys per thread in the value sum
@@ -236,7 +237,7 @@ __global__ __launch_bounds__(256) void attention_split(const float *__restrict__
     const int tri = 8 * ((int)(blockIdx.x >> 3) / group) + (int)(blockIdx.x & 7);
     if (tri >= n_tri) return;
     const int chunk = tri % n_chunks, kvh = (tri / n_chunks) % n_kv, t = tri / (n_chunks * n_kv);
-    const int hq = kvh * group + (int)(blockIdx.x >> 3) % group, pos0 = *pos_ptr, n_keys = pos0 + t + 1;
+    const int hq = kvh * group + (int)(blockIdx.x >> 3) % group, n_keys = pos0 + t + 1;
     const int j0 = chunk * ATT_CHUNK, nj = min(ATT_CHUNK, n_keys - j0);
     float *po = part + ((size_t)(t * n_head + hq) * n_chunks + chunk) * (d + 2);
     if (nj <= 0) {
