@@ -121,6 +121,29 @@ __device__ __forceinline__ T ld(const uint8_t *p) {
     return v;
 }
 
+// 4, 8 or 16 bytes at any address, taken from the aligned 32-bit words that hold them and shifted into
+// place.  For blocks whose size is not a multiple of four (Q8_0 34, Q6_K 210, IQ2_XXS 66, MXFP4 17,
+// Q5_0 22 bytes) a plain wide read lands on odd addresses, and in LDS a read that is not naturally aligned
+// runs at a fraction of the aligned rate (the Q6_K output head: 130 us with 8-byte reads at 2-byte
+// aligned LDS addresses, 88 us through aligned words).  The word past the field is only read when the
+// field reaches into it, so nothing is touched beyond the bytes asked for.
+template <class T>
+__device__ __forceinline__ T ldw(const uint8_t *p) {
+    constexpr int N = sizeof(T) / 4;
+    static_assert(sizeof(T) % 4 == 0 && N >= 1 && N <= 4, "ldw reads 4, 8 or 16 bytes");
+    const uint32_t mis = (uint32_t)(uintptr_t)p & 3u;
+    const uint32_t *q = (const uint32_t *)(p - mis);
+    uint32_t w[N + 1], o[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) w[i] = q[i];
+    w[N] = q[mis ? N : N - 1];
+#pragma unroll
+    for (int i = 0; i < N; i++) o[i] = __builtin_amdgcn_alignbyte(w[i + 1], w[i], mis);
+    T v;
+    __builtin_memcpy(&v, o, sizeof(T));
+    return v;
+}
+
 __device__ __forceinline__ float f16_bits(uint32_t h) {
     return __half2float(__ushort_as_half((unsigned short)(h & 0xFFFFu)));
 }
@@ -194,11 +217,12 @@ struct Q8_0 {  // d:f16 | qs[32] i8   (reference: src/kquant_dot.rs:53-61,287-30
     __device__ static int elem_base(int) { return 0; }
     __device__ static void decode(const uint8_t *blk, int, float *w) {
         float d = f16_bits(ld<uint16_t>(blk));
+        const uint4 qa = ldw<uint4>(blk + 2), qb = ldw<uint4>(blk + 18);
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            uint32_t v = ld<uint32_t>(blk + 2 + 4 * i);
 #pragma unroll
-            for (int b = 0; b < 4; b++) w[4 * i + b] = (float)(int8_t)(v >> (8 * b)) * d;
+            for (int b = 0; b < 4; b++) w[4 * i + b] = (float)(int8_t)(q[i] >> (8 * b)) * d;
         }
     }
 };
@@ -246,7 +270,7 @@ struct Q5_0 {  // d:f16 | qh:u32 | qs[16]        w = d (q - 16)
     __device__ static int elem_base(int) { return 0; }
     __device__ static void decode(const uint8_t *blk, int, float *w) {
         const float d = f16_bits(ld<uint16_t>(blk));
-        const uint32_t qh = ld<uint32_t>(blk + 2);
+        const uint32_t qh = ldw<uint32_t>(blk + 2);
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             const int b = blk[6 + j];
@@ -412,9 +436,9 @@ struct Q6_K {  // ql[128] | qh[64] | scales[16] i8 | d
     __device__ static void decode(const uint8_t *blk, int u, float *w) {
         int h = u >> 1, lq = u & 1;
         float d = f16_bits(ld<uint16_t>(blk + 208));
-        uint4 la = ld<uint4>(blk + 64 * h + 16 * lq);        // ql[64h + l]
-        uint4 lb = ld<uint4>(blk + 64 * h + 32 + 16 * lq);   // ql[64h + 32 + l]
-        uint4 hv = ld<uint4>(blk + 128 + 32 * h + 16 * lq);  // qh[32h + l]
+        uint4 la = ldw<uint4>(blk + 64 * h + 16 * lq);        // ql[64h + l]
+        uint4 lb = ldw<uint4>(blk + 64 * h + 32 + 16 * lq);   // ql[64h + 32 + l]
+        uint4 hv = ldw<uint4>(blk + 128 + 32 * h + 16 * lq);  // qh[32h + l]
         uint32_t a[4] = {la.x, la.y, la.z, la.w}, b[4] = {lb.x, lb.y, lb.z, lb.w}, hh[4] = {hv.x, hv.y, hv.z, hv.w};
 #pragma unroll
         for (int t = 0; t < 4; t++) {
@@ -442,7 +466,7 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
     __device__ static const uint64_t *table() { return g_tables.iq2xxs_grid; }
     __device__ static void decode_with(const uint64_t *grid_table, const uint8_t *blk, int u, float *w) {
         float d = f16_bits(ld<uint16_t>(blk));
-        uint2 g = ld<uint2>(blk + 2 + 8 * u);
+        uint2 g = ldw<uint2>(blk + 2 + 8 * u);
         uint32_t lo = g.x, hi = g.y;
         float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
 #pragma unroll
@@ -465,7 +489,7 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
     __device__ static float dot8(const uint64_t *grid_table, const uint8_t *blk, int u, const uint32_t *xl,
                                  const uint32_t *xh, const float *sx, const float *) {
         const float d = f16_bits(ld<uint16_t>(blk));
-        const uint2 g = ld<uint2>(blk + 2 + 8 * u);
+        const uint2 g = ldw<uint2>(blk + 2 + 8 * u);
         const uint32_t lo = g.x, hi = g.y;
         int pl = 0, ph = 0, nl = 0, nh = 0;
 #pragma unroll
@@ -512,9 +536,11 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
         if (e == 0xFFu) return 0.0f;
         const float d = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
         int pl = 0, ph = 0, nl = 0, nh = 0;
+        const uint4 qv = ldw<uint4>(blk + 1);
+        const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t w = ld<uint32_t>(blk + 1 + 4 * i);
+            const uint32_t w = qw[i];
 #pragma unroll
             for (int hi = 0; hi < 2; hi++) {  // low nibbles: elements 4i .. 4i+3; high nibbles: 16 + 4i ..
                 const uint32_t v = hi ? w >> 4 : w;
@@ -534,9 +560,11 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
         // 2^(e-127); e == 0 is the f32 denormal 2^-127; 0xFF (reserved) decodes the block to zeros
         float d = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
         const bool dead = e == 0xFFu;
+        const uint4 qv = ldw<uint4>(blk + 1);
+        const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            uint32_t v = ld<uint32_t>(blk + 1 + 4 * i);
+            uint32_t v = qw[i];
 #pragma unroll
             for (int b = 0; b < 4; b++) {
                 uint32_t byte = (v >> (8 * b)) & 0xFFu;

@@ -109,10 +109,22 @@ __global__ __launch_bounds__(1024) void q6k_gemv_dot4_lds(const uint8_t *__restr
             const bool more = st + 2 < n_steps;
             if (more) fetch(st + 2, (st + 2) % 3);  // the slot of step st-1, which every wave finished reading before that barrier
 
+            // Block `wave` of a row starts 210 * wave bytes into the slice: a multiple of four for even
+            // waves, two bytes past one for odd waves.  LDS reads that are not naturally aligned run at
+            // a fraction of the aligned rate (the 151936 x 4096 output head: 130 us with 8-byte reads
+            // at these addresses, 82 us with every read on a word boundary), so each 8-byte field is
+            // read as the three aligned words that hold it and shifted into place; the shift is the
+            // same for the whole wave.
             const uint8_t *blk = &ring[st % 3][r * Q6D_SLICE_LDS + wave * 210];
-            const uint2 qa = ld<uint2>(blk + 64 * h + 8 * e);         // ql[64h + l]
-            const uint2 qb = ld<uint2>(blk + 64 * h + 32 + 8 * e);    // ql[64h + 32 + l]
-            const uint2 qh = ld<uint2>(blk + 128 + 32 * h + 8 * e);   // qh[32h + l]
+            const uint32_t *blk4 = (const uint32_t *)(blk - 2 * (wave & 1));
+            const uint32_t mis = 16 * (wave & 1);
+            auto field = [&](int off) __attribute__((always_inline)) {   // off: a multiple of 4
+                const uint32_t d0 = blk4[off / 4], d1 = blk4[off / 4 + 1], d2 = blk4[off / 4 + 2];
+                return uint2{__builtin_amdgcn_alignbit(d1, d0, mis), __builtin_amdgcn_alignbit(d2, d1, mis)};
+            };
+            const uint2 qa = field(64 * h + 8 * e);         // ql[64h + l]
+            const uint2 qb = field(64 * h + 32 + 8 * e);    // ql[64h + 32 + l]
+            const uint2 qh = field(128 + 32 * h + 8 * e);   // qh[32h + l]
             const float d = f16_bits(ld<uint16_t>(blk + 208));
             const uint32_t a[2] = {qa.x, qa.y}, b[2] = {qb.x, qb.y}, hh[2] = {qh.x, qh.y};
             float f = 0.0f;

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
 
             const uint8_t *blk = &ring[st % 3][r * Q8D_SLICE_LDS + (8 * wave + j) * 34];
             const float d = f16_bits(ld<uint16_t>(blk));
-            const uint4 qa = ld<uint4>(blk + 2), qb = ld<uint4>(blk + 18);
+            const uint4 qa = ldw<uint4>(blk + 2), qb = ldw<uint4>(blk + 18);  // 34-byte blocks: odd word offsets
             const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
             int sl = 0, sh = 0;
 #pragma unroll
