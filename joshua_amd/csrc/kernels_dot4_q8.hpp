@@ -40,13 +40,30 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
         async_load16(src + 1024, dst + 1024);
         if (lane < 8) async_load16(src + 2048, dst + 2048);  // 136 pieces of 16 bytes per half slice
     };
-    fetch(0, 0);
-    fetch(1, 1);  // (a clamped copy of step 0 when there is one step only)
+    // Up to two column groups (LDS has room for their raw activations): every global read is an
+    // asynchronous load counted by hand, the activation columns first, then step 0, and step 1 once the
+    // activations are prepared, so that every workgroup's step 0 has the memory system to itself.  With
+    // three groups the activations are plain loads behind both steps (the compiler's wait for them then
+    // covers the steps as well).
+    constexpr bool STAGED_X = NG <= 2;
+    __shared__ __attribute__((aligned(16))) float x_raw[STAGED_X ? NG : 1][16][256];
+    if constexpr (STAGED_X) {
+#pragma unroll
+        for (int g = 0; g < NG; g++)
+            async_load16(X + (size_t)(16 * g + wave) * 256 + 4 * lane, lds_offset_of(&x_raw[g][wave][0]));
+        fetch(0, 0);
+        asm volatile("s_waitcnt vmcnt(3)" ::: "memory");  // the activations landed (own wave's data: no barrier needed)
+    } else {
+        fetch(0, 0);
+        fetch(1, 1);  // (a clamped copy of step 0 when there is one step only)
+    }
 
     // activations of blocks 128 g + 8 wave .. + 7: 4 elements a lane, one scale per block of 32
 #pragma unroll
     for (int g = 0; g < NG; g++) {
-        const float4 v = *(const float4 *)(X + (size_t)(16 * g + wave) * 256 + 4 * lane);
+        float4 v;
+        if constexpr (STAGED_X) v = *(const float4 *)&x_raw[g][wave][4 * lane];
+        else v = *(const float4 *)(X + (size_t)(16 * g + wave) * 256 + 4 * lane);
         float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
         amax = max_row8(amax);
         const bool live = amax > 0.0f && amax < INFINITY;
@@ -64,7 +81,13 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
         xh_lds[g][wave][lane] = wh;
         if ((lane & 7) == 0) s_lds[g][wave][lane >> 3] = s;
     }
-    asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");  // step 0 landed (step 1 may be in flight), planes written
+    // step 0 landed (step 1 may be in flight), planes written
+    if (STAGED_X && n_steps == 1) {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    } else {
+        if constexpr (STAGED_X) fetch(1, 1);
+        asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+    }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     uint32_t xl[NG][8], xh[NG][8];  // this lane's block: elements 32 j .. 32 j + 31 of the wave's 256
