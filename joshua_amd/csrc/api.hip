@@ -477,7 +477,9 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     // whose time hardly depends on the row count
     // 3 to 16 rows against a very long matrix (a vocabulary projection): the LDS-ring kernel, whose
     // two launches and scratch allocation only pay off from some 100 us of streaming on
-    if (type == JQ_TYPE_Q4_K && m > 2 && m <= Q4K_MFMA_MAX_M && n >= 32768) {
+    static const char *ring_min_env = getenv("JQ_Q4K_RING_MIN_N");
+    static const size_t ring_min_n = ring_min_env ? (size_t)atoll(ring_min_env) : 32768;
+    if (type == JQ_TYPE_Q4_K && m > 2 && m <= Q4K_MFMA_MAX_M && n >= ring_min_n) {
         const int rc = dispatch_q4k_ring(W, row_bytes, X, Y, m, k, n, s);
         if (rc >= 0) return rc;
     }
