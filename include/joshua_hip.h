@@ -136,6 +136,10 @@ typedef struct {
     float weights_scale;     /* 0 or 1: none (src/quantized_deepseek2.rs:549-551) */
     uint32_t n_group;        /* <= 1: no group limit (src/quantized_deepseek2.rs:563-566) */
     uint32_t topk_group;
+    /* Clamp in front of the experts' SwiGLU: gate to (-inf, c], up to [-c, c]; <= 0: none.  The shared
+     * expert has a limit of its own (src/quantized_deepseek4.rs:445-462, :2419-2448). */
+    float swiglu_clamp;
+    float swiglu_clamp_shared;
 } jq_moe_config;
 
 /* router_w is [E, h] row-major f32 on the host (ffn_gate_inp), router_bias [E]

@@ -45,7 +45,8 @@ class MoeConfig(ctypes.Structure):
     """jq_moe_config of include/joshua_hip.h."""
     _fields_ = [("n_expert", ctypes.c_uint32), ("n_expert_used", ctypes.c_uint32), ("hidden", ctypes.c_uint32),
                 ("inter", ctypes.c_uint32), ("gating", ctypes.c_uint32), ("norm_topk", ctypes.c_uint32),
-                ("weights_scale", ctypes.c_float), ("n_group", ctypes.c_uint32), ("topk_group", ctypes.c_uint32)]
+                ("weights_scale", ctypes.c_float), ("n_group", ctypes.c_uint32), ("topk_group", ctypes.c_uint32),
+                ("swiglu_clamp", ctypes.c_float), ("swiglu_clamp_shared", ctypes.c_float)]
 
 
 class Qwen3Config(ctypes.Structure):

@@ -380,7 +380,7 @@ int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float 
     launch_q4k_acts_prep(X, m, k, acts, s);
 #define JQ_RING(MAXNB)                                                                                              \
     hipLaunchKernelGGL((jq::q4k_ring_mfma<MAXNB, false, false>), dim3(grid), dim3(64 * (unsigned)nb), 0, s, W, nullptr, \
-                       nullptr, acts, nullptr, nullptr, nullptr, nullptr, Y, (int)m, (int)n)
+                       nullptr, acts, nullptr, nullptr, nullptr, nullptr, Y, (int)m, (int)n, jq::MoeClamp{})
     if (maxnb == 16) JQ_RING(16);
     else if (maxnb == 8) JQ_RING(8);
     else JQ_RING(4);
@@ -791,14 +791,14 @@ int moe_reserve(jq_moe *m, size_t T) {
 template <class Q, bool SWIGLU>
 void launch_moe_rows(const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2, const int *gexp,
                      const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n, int groups,
-                     int max_group, hipStream_t s) {
+                     int max_group, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     dim3 grid((unsigned)((n + jq::ROWS_PER_WG - 1) / jq::ROWS_PER_WG), (unsigned)groups), block(64 * jq::ROWS_PER_WG);
     if (max_group <= 1)
         hipLaunchKernelGGL((jq::moe_rows_valu<Q, 1, SWIGLU>), grid, block, 0, s, Wptr, row_bytes, X, X2, gexp, offsets,
-                           xsel, yrow, Y, k, n);
+                           xsel, yrow, Y, k, n, cl);
     else
         hipLaunchKernelGGL((jq::moe_rows_valu<Q, 4, SWIGLU>), grid, block, 0, s, Wptr, row_bytes, X, X2, gexp, offsets,
-                           xsel, yrow, Y, k, n);
+                           xsel, yrow, Y, k, n, cl);
 }
 
 // The LDS-staged grouped kernel when the rows allow it (aligned row starts, four waves' rows within
@@ -806,7 +806,7 @@ void launch_moe_rows(const uint8_t *const *Wptr, size_t row_bytes, const float *
 template <class Q, bool DUAL>
 int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
                       const float *X, const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y,
-                      int k, int n, int groups, int max_group, hipStream_t s) {
+                      int k, int n, int groups, int max_group, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
     const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
@@ -816,7 +816,7 @@ int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t
     const size_t lds = wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>();
 #define JQ_MOE_STAGED(MT, GG)                                                                                      \
     hipLaunchKernelGGL((jq::moe_rows_staged<Q, MT, DUAL, GG>), grid, block, lds, s, Wa, Wb, row_bytes, X, gexp,     \
-                       offsets, xsel, yrow, Y, k, n, L, (int)wave_lds)
+                       offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, cl)
     if (max_group <= 1) {
         if (G == 16) JQ_MOE_STAGED(1, 16);
         else JQ_MOE_STAGED(1, 4);
@@ -831,13 +831,13 @@ int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t
 template <bool DUAL>
 int dispatch_moe_staged(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes,
                         bool aligned16, const float *X, const int *gexp, const int *offsets, const int *xsel,
-                        const int *yrow, float *Y, int k, int n, int groups, int max_group, hipStream_t s) {
+                        const int *yrow, float *Y, int k, int n, int groups, int max_group, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     int rc;
     switch (type) {
 #define JQ_MOE_CASE(ID, Q)                                                                                          \
     case ID:                                                                                                        \
         rc = launch_moe_staged<jq::Q, DUAL>(Wa, Wb, row_bytes, aligned16, X, gexp, offsets, xsel, yrow, Y, k, n,     \
-                                            groups, max_group, s);                                                  \
+                                            groups, max_group, s, cl);                                              \
         break;
         JQ_FOR_EACH_FORMAT(JQ_MOE_CASE)
 #undef JQ_MOE_CASE
@@ -852,7 +852,7 @@ int dispatch_moe_staged(uint32_t type, const uint8_t *const *Wa, const uint8_t *
 template <bool DUAL>
 int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
                           const float *X, size_t x_rows, uint8_t *acts, const int *gexp, const int *offsets,
-                          const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s) {
+                          const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     const int nb = k / 256;
     static const char *off = getenv("JQ_MOE_NO_RING");
     if (off || !acts || k % 256 != 0 || nb == 0 || nb > 16 || row_bytes != (size_t)nb * 144 || !aligned16 ||
@@ -865,7 +865,7 @@ int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, si
     dim3 grid((unsigned)std::min(n_tiles, std::max(per_group, 1)), (unsigned)groups), block(64 * nb);
 #define JQ_RING(MAXNB)                                                                                             \
     hipLaunchKernelGGL((jq::q4k_ring_mfma<MAXNB, true, DUAL>), grid, block, 0, s, nullptr, Wa, Wb, acts, gexp,     \
-                       offsets, xsel, yrow, Y, 0, n)
+                       offsets, xsel, yrow, Y, 0, n, cl)
     if (maxnb == 16) JQ_RING(16);
     else if (maxnb == 8) JQ_RING(8);
     else JQ_RING(4);
@@ -880,7 +880,7 @@ int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, si
 template <class Q, bool DUAL>
 int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16, const float *X,
                     size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets, const int *xsel, const int *yrow,
-                    float *Y, int k, int n, int groups, hipStream_t s) {
+                    float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
     const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
@@ -898,7 +898,7 @@ int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t r
     dim3 grid((unsigned)wgs, (unsigned)groups), block(64 * jq::ROWS_PER_WG);
 #define JQ_DOT8(GG, OWN)                                                                                          \
     hipLaunchKernelGGL((jq::moe_rows_dot8<Q, DUAL, GG, OWN>), grid, block, lds, s, Wa, Wb, row_bytes, X, xq, gexp,  \
-                       offsets, xsel, yrow, Y, k, n, L, (int)wave_lds)
+                       offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, cl)
     if (G == 16 && own) JQ_DOT8(16, true);
     else if (G == 16) JQ_DOT8(16, false);
     else if (own) JQ_DOT8(4, true);
@@ -911,13 +911,13 @@ int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t r
 template <bool DUAL>
 int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
                       const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets,
-                      const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s) {
+                      const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     if (!moe_has_dot8(type) || k % 32 != 0 || ((uintptr_t)X & 15) != 0) return -1;
     switch (type) {
 #define JQ_DOT8_CASE(ID, Q)                                                                                         \
     case ID:                                                                                                        \
         return launch_moe_dot8<jq::Q, DUAL>(Wa, Wb, row_bytes, aligned16, X, x_rows, xq, gexp, offsets, xsel, yrow, Y, k, n, \
-                                            groups, s);
+                                            groups, s, cl);
         JQ_DOT8_CASE(JQ_TYPE_MXFP4, MXFP4)
         JQ_DOT8_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
         JQ_DOT8_CASE(JQ_TYPE_Q4_K, Q4_K)
@@ -929,12 +929,12 @@ int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *co
 template <bool SWIGLU>
 int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2,
                       const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
-                      int groups, int max_group, hipStream_t s) {
+                      int groups, int max_group, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     switch (type) {
 #define JQ_MOE_CASE(ID, Q)                                                                                          \
     case ID:                                                                                                        \
         launch_moe_rows<jq::Q, SWIGLU>(Wptr, row_bytes, X, X2, gexp, offsets, xsel, yrow, Y, k, n, groups, max_group, \
-                                       s);                                                                          \
+                                       s, cl);                                                                      \
         break;
         JQ_FOR_EACH_FORMAT(JQ_MOE_CASE)
 #undef JQ_MOE_CASE
@@ -961,6 +961,8 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
 int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s) {
     const jq_moe_config &c = m->cfg;
     const int P = (int)(T * c.n_expert_used), extra = m->fold_shared ? 1 : 0;
+    // the experts' SwiGLU clamp; a folded shared expert is expert number n_expert and has its own
+    const jq::MoeClamp clamp{c.swiglu_clamp, c.swiglu_clamp_shared, (int)c.n_expert};
     int groups, max_group;
     if ((size_t)P <= c.n_expert) {  // decode-sized: one group per pair, written by the gating kernel itself
         if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra})) return 1;
@@ -983,15 +985,15 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     const bool same_gu = m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes;
     if (same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K)
         rc = dispatch_moe_q4k_ring<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qacts, m->gexp, m->offsets,
-                                         m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s);
+                                         m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
     if (rc > 0) return 1;
     if (rc < 0 && same_gu && max_group <= 1)
         rc = dispatch_moe_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
-                                     m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s);
+                                     m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
     if (rc > 0) return 1;
     if (rc < 0 && same_gu)
         rc = dispatch_moe_staged<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, m->gexp, m->offsets,
-                                       m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s);
+                                       m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, max_group, s, clamp);
     if (rc > 0) return 1;
     const bool fused_act = rc == 0;
     if (!fused_act) {
@@ -1025,7 +1027,8 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
                                          m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups, max_group, s))
                 return 1;
         } else if (dispatch_moe_rows<true>(m->down->type, m->pdown, m->down->row_bytes, m->G, m->U, m->gexp, m->offsets,
-                                           m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups, max_group, s)) {
+                                           m->yrow, m->yrow, m->out, (int)c.inter, (int)c.hidden, groups, max_group, s,
+                                           clamp)) {
             return 1;
         }
     }
@@ -1038,7 +1041,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         if (dispatch_matmul(m->sup->type, m->sup->dev, m->sup->row_bytes, x, m->sU, T, c.hidden, si, s)) return 1;
         size_t total = T * si;
         hipLaunchKernelGGL(jq::swiglu_rows, dim3((unsigned)std::min<size_t>((total + 255) / 256, 4096)), dim3(256), 0, s,
-                           m->sG, m->sU, m->sH, total);
+                           m->sG, m->sU, m->sH, total, c.swiglu_clamp_shared);
         if (dispatch_matmul(m->sdown->type, m->sdown->dev, m->sdown->row_bytes, m->sH, m->sOut, T, si, c.hidden, s))
             return 1;
         shared_out = m->sOut;
@@ -1448,7 +1451,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             hipLaunchKernelGGL(jq::swiglu_pairs, dim3(grid_for((size_t)c.ffn)), dim3(256), 0, s, m->cat, m->mid, (size_t)c.ffn);
         } else {
             hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, gp, up, m->mid,
-                               (size_t)T * c.ffn);
+                               (size_t)T * c.ffn, 0.0f);
         }
         if (model_mm(m, p + ".ffn_down.weight", m->mid, m->proj, T, s)) return 1;
         pending = m->proj;

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(1024) void q4k_ring_mfma(const uint8_t *__restrict_
                                                       const uint8_t *__restrict__ acts, const int *__restrict__ gexp,
                                                       const int *__restrict__ offsets,
                                                       const int *__restrict__ xsel, const int *__restrict__ yrow,
-                                                      float *__restrict__ Y, int m, int n) {
+                                                      float *__restrict__ Y, int m, int n, MoeClamp cl) {
     static_assert(!DUAL || GROUPED, "two tables only in the grouped form");
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][16 * qr_row_lds(MAXNB)];
     // the waves' partial tiles; 264 floats a wave (256 + 8) so that lanes summing different waves'
@@ -63,12 +63,14 @@ __global__ __launch_bounds__(1024) void q4k_ring_mfma(const uint8_t *__restrict_
 
     int beg = 0, cnt = m;
     const uint8_t *wa = W, *wb = W;
+    float limit = 0.0f;  // the expert's SwiGLU clamp
     if (GROUPED) {
         const int grp = blockIdx.y;
         beg = offsets[grp], cnt = offsets[grp + 1] - beg;
         if (cnt == 0) return;  // the whole workgroup leaves together
         const int e = gexp[grp];
         wa = Wa[e], wb = DUAL ? Wb[e] : wa;
+        limit = e >= cl.n_routed ? cl.shared : cl.routed;
     }
 
     // a row is 9 * waves pieces of 16 bytes: `full` whole instructions and one of `rem` lanes; every
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(1024) void q4k_ring_mfma(const uint8_t *__restrict_
                         gate_keep[q] = s;  // the same rows of the second table are the next step
                     } else if (p == 0 && mm < mc && nn < n) {
                         const size_t yr = GROUPED ? (size_t)yrow[beg + m0 + mm] : (size_t)mm;
-                        Y[yr * n + nn] = DUAL ? silu(gate_keep[q]) * s : s;
+                        Y[yr * n + nn] = DUAL ? swiglu(gate_keep[q], s, limit) : s;
                     }
                 }
             }

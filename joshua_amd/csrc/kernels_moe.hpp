@@ -245,7 +245,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_valu(const uint8_t 
                                                                    const int *__restrict__ offsets,
                                                                    const int *__restrict__ xsel,
                                                                    const int *__restrict__ yrow,
-                                                                   float *__restrict__ Y, int k, int n) {
+                                                                   float *__restrict__ Y, int k, int n, MoeClamp cl) {
     const int grp = blockIdx.y;
     const int beg = offsets[grp], cnt = offsets[grp + 1] - beg;
     if (cnt == 0) return;
@@ -281,7 +281,8 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_valu(const uint8_t 
                             float4 xv = ld<float4>((const uint8_t *)(xp + s * Q::SEG_STRIDE + el));
                             if (SWIGLU) {
                                 const float4 uv = ld<float4>((const uint8_t *)(xp2 + s * Q::SEG_STRIDE + el));
-                                xv = float4{silu(xv.x) * uv.x, silu(xv.y) * uv.y, silu(xv.z) * uv.z, silu(xv.w) * uv.w};
+                                xv = float4{swiglu(xv.x, uv.x, cl, e), swiglu(xv.y, uv.y, cl, e), swiglu(xv.z, uv.z, cl, e),
+                                            swiglu(xv.w, uv.w, cl, e)};
                             }
                             acc[i] = fmaf(xv.x, w[s * Q::SEGLEN + el + 0], acc[i]);
                             acc[i] = fmaf(xv.y, w[s * Q::SEGLEN + el + 1], acc[i]);
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
                                                                      const int *__restrict__ xsel,
                                                                      const int *__restrict__ yrow,
                                                                      float *__restrict__ Y, int k, int n, int L,
-                                                                     int wave_lds) {
+                                                                     int wave_lds, MoeClamp cl) {
     extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
     const auto *table = stage_table<Q>(staged_moe);  // before any wave leaves: it holds a barrier
     const int grp = blockIdx.y;
@@ -398,7 +399,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
                 if (DUAL) s2 += __shfl_xor(s2, off, 64);
             }
             if (sub == 0 && active && m0 + i < cnt)
-                Y[(size_t)yrow[beg + m0 + i] * n + row] = DUAL ? silu(s) * s2 : s;
+                Y[(size_t)yrow[beg + m0 + i] * n + row] = DUAL ? swiglu(s, s2, cl, e) : s;
         }
     }
 }
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
                                                                    const int *__restrict__ xsel,
                                                                    const int *__restrict__ yrow,
                                                                    float *__restrict__ Y, int k, int n, int L,
-                                                                   int wave_lds) {
+                                                                   int wave_lds, MoeClamp cl) {
     static_assert(Q::SEGS == 1 && Q::SEGLEN % 32 == 0, "units of 32 or 64 consecutive elements");
     constexpr int XW = Q::SEGLEN / 4, NS = Q::SEGLEN / 32;  // activation words a plane, scales a unit
     extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
@@ -551,7 +552,7 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
         acc += __shfl_xor(acc, off, 64);
         if (DUAL) acc2 += __shfl_xor(acc2, off, 64);
     }
-    if (sub == 0 && active) Y[(size_t)yrow[beg] * n + row] = DUAL ? silu(acc) * acc2 : acc;
+    if (sub == 0 && active) Y[(size_t)yrow[beg] * n + row] = DUAL ? swiglu(acc, acc2, cl, e) : acc;
 }
 
 // y[t, :] = sum_s w[t, s] * out[t*k + s, :]  (+ shared_out[t, :] of the shared expert),
@@ -574,11 +575,11 @@ __global__ __launch_bounds__(256) void moe_combine(const float *__restrict__ out
 
 namespace jq {
 
-// h[i] = silu(g[i]) * u[i]  (the shared expert's activation)
+// h[i] = silu(g[i]) * u[i], both clamped first when limit > 0  (the shared expert's activation; the decoder's)
 __global__ __launch_bounds__(256) void swiglu_rows(const float *__restrict__ g, const float *__restrict__ u,
-                                                    float *__restrict__ h, size_t total) {
+                                                    float *__restrict__ h, size_t total, float limit) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
-        h[i] = silu(g[i]) * u[i];
+        h[i] = swiglu(g[i], u[i], limit);
 }
 
 }  // namespace jq

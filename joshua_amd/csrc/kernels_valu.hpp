@@ -17,6 +17,24 @@ namespace jq {
 
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 
+// The optional clamp in front of an expert's SwiGLU: gate from above, up on both sides
+// (reference: src/quantized_deepseek4.rs:445-462; limit <= 0: none).  An expert whose id is at or past
+// `n_routed` is a shared expert and has a limit of its own (:2419-2448).  A NaN stays a NaN.
+struct MoeClamp {
+    float routed, shared;
+    int n_routed;
+};
+__device__ __forceinline__ float swiglu(float g, float u, float limit) {
+    if (limit > 0.0f) {
+        g = g > limit ? limit : g;
+        u = u > limit ? limit : (u < -limit ? -limit : u);
+    }
+    return silu(g) * u;
+}
+__device__ __forceinline__ float swiglu(float g, float u, const MoeClamp &cl, int expert) {
+    return swiglu(g, u, expert >= cl.n_routed ? cl.shared : cl.routed);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
     v = sum_xor32(v);
     v = sum_xor16(v);

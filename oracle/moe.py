@@ -30,7 +30,7 @@ def topk_indices(v: np.ndarray, k: int) -> np.ndarray:
 class MoeOracle:
     def __init__(self, qtype, h, inter, n_expert, k_used, router_w, gate, up, down, *, gating="softmax",
                  norm_topk=True, weights_scale=0.0, n_group=1, topk_group=1, router_bias=None, shared=None,
-                 avx2=False):
+                 avx2=False, swiglu_clamp=0.0, swiglu_clamp_shared=0.0):
         self.qtype, self.h, self.inter, self.E, self.k = qtype, h, inter, n_expert, k_used
         self.router_w = np.asarray(router_w, np.float32)          # [E, h]
         self.gate, self.up, self.down = gate, up, down            # stacked block bytes
@@ -39,6 +39,14 @@ class MoeOracle:
         self.bias = None if router_bias is None else np.asarray(router_bias, np.float32)
         self.shared = shared                                      # (qtype, inter_s, gate, up, down) or None
         self.avx2 = avx2
+        self.clamp, self.clamp_shared = np.float32(swiglu_clamp), np.float32(swiglu_clamp_shared)
+
+    @staticmethod
+    def clamped(g, u, c):
+        """src/quantized_deepseek4.rs:445-462: gate to (-inf, c], up to [-c, c] when c > 0."""
+        if c > 0:
+            g, u = np.minimum(g, c), np.clip(u, -c, c)
+        return g, u
 
     # -- routing (src/quantized_qwen3_moe.rs:424-436, src/quantized_deepseek2.rs:527-551) ----
     def route(self, x2: np.ndarray):
@@ -86,6 +94,7 @@ class MoeOracle:
         m = x.shape[0]
         g = matmul_t(self.qtype, (m, self.h, self.inter), x, self._slice(self.gate, e), avx2=self.avx2)
         u = matmul_t(self.qtype, (m, self.h, self.inter), x, self._slice(self.up, e), avx2=self.avx2)
+        g, u = self.clamped(g, u, self.clamp)
         hid = (silu(g) * u).astype(np.float32)
         return matmul_t(self.qtype, (m, self.inter, self.h), hid, self._slice(self.down, e), avx2=self.avx2).copy()
 
@@ -94,6 +103,7 @@ class MoeOracle:
         m = x.shape[0]
         gg = matmul_t(qt, (m, self.h, si), x, g, avx2=self.avx2)
         uu = matmul_t(qt, (m, self.h, si), x, u, avx2=self.avx2)
+        gg, uu = self.clamped(gg, uu, self.clamp_shared)
         hid = (silu(gg) * uu).astype(np.float32)
         return matmul_t(qt, (m, si, self.h), hid, d, avx2=self.avx2).copy()
 

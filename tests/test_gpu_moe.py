@@ -25,7 +25,8 @@ def build(qtype, h, inter, E, k, seed, sigma=0.02, shared_inter=0, **kw):
                     capi.Weight.upload(qtype, sd, h, shared_inter))
     ora = MoeOracle(qtype, h, inter, E, k, rw, gate, up, down, shared=shared_o, avx2=oracle.have_avx2(), **kw)
     cfg = capi.MoeConfig(E, k, h, inter, 1 if kw.get("gating") == "sigmoid" else 0, 1 if kw.get("norm_topk", True) else 0,
-                         float(kw.get("weights_scale", 0.0)), kw.get("n_group", 1), kw.get("topk_group", 1))
+                         float(kw.get("weights_scale", 0.0)), kw.get("n_group", 1), kw.get("topk_group", 1),
+                         float(kw.get("swiglu_clamp", 0.0)), float(kw.get("swiglu_clamp_shared", 0.0)))
     dev = capi.Moe(cfg, rw, capi.Weight.upload(qtype, gate, E * inter, h), capi.Weight.upload(qtype, up, E * inter, h),
                    capi.Weight.upload(qtype, down, E * h, inter), router_bias=kw.get("router_bias"), shared=shared_w)
     return ora, dev
@@ -140,3 +141,23 @@ def test_moe_rejects_mismatched_shapes():
         capi.Moe(capi.MoeConfig(4, 5, 256, 32, 0, 1, 0.0, 1, 1), rw, gate, gate, down)      # k > E
     with pytest.raises(capi.JoshuaHipError):
         capi.Moe(capi.MoeConfig(4, 2, 256, 64, 0, 1, 0.0, 1, 1), rw, gate, gate, down)      # wrong inter
+
+
+@pytest.mark.parametrize("qtype,h,inter,tokens,shared_inter", [
+    (capi.Q4_K, 512, 256, 1, 0),       # decode-sized call, integer-dot kernel
+    (capi.MXFP4, 512, 256, 2, 256),    # the same with a shared expert riding along as a group
+    (capi.Q8_0, 512, 256, 1, 0),       # decode-sized call, f32 staged kernel
+    (capi.Q4_K, 1024, 256, 40, 256),   # many tokens a group: the MFMA ring kernel, shared expert folded in
+    (capi.Q6_K, 512, 256, 24, 0),      # many tokens a group, f32 staged kernel
+    (capi.Q4_K, 512, 256, 3, 512),     # a shared expert of another width: launches of its own
+])
+def test_swiglu_clamp(qtype, h, inter, tokens, shared_inter):
+    """Gate clamped from above and up on both sides before the activation, with a limit of its own for
+    the shared expert (reference: src/quantized_deepseek4.rs:445-462, :2419-2448); limits low enough to bite."""
+    kw = dict(swiglu_clamp=0.02, swiglu_clamp_shared=0.01)
+    ora, dev = build(qtype, h, inter, 16, 4, 70, shared_inter=shared_inter, **kw)
+    plain, _ = build(qtype, h, inter, 16, 4, 70, shared_inter=shared_inter)
+    x = synth.normal(71, (tokens, h))
+    want = ora.forward(x)
+    assert not close(want, plain.forward(x))          # the limits change the result
+    assert close(dev.forward(x), want)
