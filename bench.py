@@ -252,6 +252,50 @@ def decode_leg(prompt_len: int, n_decode: int, cpu_seconds: float, share_layers:
     return res
 
 
+def plugin_leg(prompt_len: int, n_decode: int, share_layers: bool) -> dict:
+    """The same model written to a GGUF file, loaded and driven through the four joshua_npu_* symbols as
+    the reference engine drives a backend plugin (reference: src/npu/vendor.rs:95-185): the load (header,
+    mapping, one upload per tensor), a prefill and greedy steps whose logits come back to the host."""
+    import tempfile
+
+    from joshua_amd import capi
+    from joshua_amd.synth import gguf as gw
+    from joshua_amd.synth import uniform_u32
+    from joshua_amd.synth.model import qwen3_tensor_plan, qwen3_tensors
+
+    cfg = dict(QWEN3_8B, n_ctx=prompt_len + n_decode)
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "qwen3-8b-shaped-q4_k_m.gguf")
+        t0 = time.perf_counter()
+        gw.write_qwen3(path, cfg, qwen3_tensors(cfg, 7, "q4_k_m", share_layers=share_layers), qwen3_tensor_plan(cfg))
+        t_write = time.perf_counter() - t0
+        size = os.path.getsize(path)
+        t0 = time.perf_counter()
+        plug = capi.NpuPlugin(path, cfg["n_ctx"])
+        t_load = time.perf_counter() - t0
+        if plug.rc != 0:
+            raise RuntimeError(f"joshua_npu_init failed ({plug.rc}): {capi.last_error()}")
+        prompt = uniform_u32(31, prompt_len, cfg["vocab"])
+        rc, logits = plug.forward(prompt[:16], 0)       # warm-up, then start over
+        assert rc == 0 and plug.reset() == 0
+        t0 = time.perf_counter()
+        rc, logits = plug.forward(prompt, 0)
+        t_prefill = time.perf_counter() - t0
+        assert rc == 0
+        t0 = time.perf_counter()
+        for i in range(n_decode - 1):
+            # greedy on the host, as the engine's sampler does: the last index holding the maximum
+            tok = int(logits.size - 1 - np.argmax(logits[::-1]))
+            rc, logits = plug.forward([tok], prompt_len + i)
+            assert rc == 0
+        t_dec = time.perf_counter() - t0
+        plug.close()
+    return {"gguf_bytes": size, "write_s": round(t_write, 1), "load_s": round(t_load, 2),
+            "load_gbs": round(size / t_load / 1e9, 2), "prefill_tokens_per_s": round(prompt_len / t_prefill, 1),
+            "tokens_per_s": round((n_decode - 1) / t_dec, 2),
+            "note": "logits of every step copied to the host (608 KB) and the arg-max taken there"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -266,6 +310,8 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--share-layers", type=int, default=0, help="1: draw each layer role's bytes once (faster set-up)")
     ap.add_argument("--no-graph", action="store_true", help="enqueue launches one by one instead of a HIP graph")
+    ap.add_argument("--plugin", type=int, default=0,
+                    help="1: also write the model to a GGUF file and run it through the joshua_npu_* symbols")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -373,6 +419,8 @@ def main() -> int:
     if args.decode:
         out["decode"] = decode_leg(args.prompt, args.new_tokens, args.cpu_seconds, bool(args.share_layers))
         parity_ok = parity_ok and out["decode"].get("parity_ok", True)
+    if args.plugin:
+        out["plugin"] = plugin_leg(args.prompt, args.new_tokens, bool(args.share_layers))
     print(json.dumps(out))
     return 0 if parity_ok else 1
 
