@@ -255,6 +255,15 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     // rows of 8192 or 12288 (a feed-forward down projection): steps of 8 rows x 4096 columns
     // (4096 x 12288: 9.2 us against 11.1 us for the MFMA GEMV)
     if (mode == "auto" && !norm && !swiglu && (nb == 32 || nb == 48) && row_bytes == nb / 16 * jq::QD_ROW && n >= 1024) {
+        // one 16-row tile for (nearly) every compute unit: the 16-row steps are 3 to 6 % ahead there
+        // (4096 x 12288: 8.8 us; 4096 x 8192: 6.4 us against 6.8 us)
+        const size_t tiles16 = (n + 15) / 16;
+        if (tiles16 > 224 && tiles16 <= 256) {
+            if (nb == 32) hipLaunchKernelGGL(jq::q4k_gemv_dot4_cols<2>, dim3(tiles16), dim3(1024), 0, s, W, X, Y, (int)n, (int)tiles16);
+            else hipLaunchKernelGGL(jq::q4k_gemv_dot4_cols<3>, dim3(tiles16), dim3(1024), 0, s, W, X, Y, (int)n, (int)tiles16);
+            HIP_TRY(hipGetLastError());
+            return 0;
+        }
         const size_t tiles8 = (n + 7) / 8, rounds = (tiles8 + 255) / 256;
         const unsigned grid = (unsigned)((tiles8 + rounds - 1) / rounds);
         if (nb == 32) hipLaunchKernelGGL(jq::q4k_gemv_dot4_r8<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);

@@ -335,10 +335,11 @@ def test_q4k_dot4_gemv_integer_dot_products_are_bit_exact():
     assert np.array_equal(got[0], (x @ q.T).astype(np.float32))
 
 
-@pytest.mark.parametrize("k,n", [(8192, 1024), (12288, 1029), (12288, 4096), (8192, 2043)])
+@pytest.mark.parametrize("k,n", [(8192, 1024), (12288, 1029), (12288, 4096), (8192, 2043), (8192, 4090), (12288, 3600)])
 def test_q4k_dot4_gemv_long_rows(k, n):
     """Rows of 8192 and 12288, one activation row, 1024 weight rows or more: the v_dot4 kernel in steps
-    of 8 rows x 4096 columns; row counts that leave a partial last step; wide-ranging activations."""
+    of 8 rows x 4096 columns, or of 16 rows when that gives one tile per compute unit (3585 to 4096
+    rows); row counts that leave a partial last step; wide-ranging activations."""
     blocks = make_blocks(capi.Q4_K, n, k, 51 + n)
     rng = np.random.default_rng(n)
     lhs = synth.normal(52 + n, (1, k))
@@ -349,9 +350,8 @@ def test_q4k_dot4_gemv_long_rows(k, n):
     assert np.isnan(w.matmul_t(1, lhs)).all()
 
 
-@pytest.mark.parametrize("k", [8192, 12288])
-def test_q4k_dot4_gemv_long_rows_integer_dot_products_are_bit_exact(k):
-    n = 1040
+@pytest.mark.parametrize("k,n", [(8192, 1040), (12288, 1040), (8192, 4000), (12288, 4096)])
+def test_q4k_dot4_gemv_long_rows_integer_dot_products_are_bit_exact(k, n):
     blocks, q, x = q4k_integer_case(n, k, 9, group=32, big_value=32639, small=1000)
     want = x @ q.T
     assert np.abs(want).max() < 2 ** 24
