@@ -162,6 +162,51 @@ int jq_moe_route(jq_moe *moe, size_t n_tokens, const float *x, uint32_t *ids, fl
  * its scratch buffers). */
 int jq_moe_forward(jq_moe *moe, size_t n_tokens, const float *x, float *y, int ptrs_are_device, void *stream);
 
+/* ---- Multi-head latent attention (DeepSeek-V2 / V3 / Kimi-K2) -----------------------
+ * The attention block of the reference's `deepseek2` graph: Q projection (plain or
+ * low-rank a -> RMSNorm -> b), compressed KV projection, interleaved RoPE (YaRN-aware) on
+ * the rope slices, KV up-projection, causal softmax attention over the cache, output
+ * projection (reference: src/quantized_deepseek2.rs:357-499 Attention::forward,
+ * :240-311 RotaryEmbedding, :875-889 the causal mask).  Results match the reference's
+ * unabsorbed computation within f32 tolerance; the cache holds the normed latent and
+ * the rotated shared key of every token instead of per-head keys and values. */
+typedef struct jq_mla jq_mla;
+
+typedef struct {
+    uint32_t n_embd, n_head;
+    uint32_t q_lora_rank;            /* 0: plain Q projection (src/quantized_deepseek2.rs:357-371) */
+    uint32_t kv_lora_rank, qk_nope_head_dim, qk_rope_head_dim, v_head_dim;
+    uint32_t n_ctx;                  /* positions of the cache and of the rotary tables */
+    float rms_eps, rope_theta;
+    /* YaRN (src/quantized_deepseek2.rs:161-192, :246-301): factor 0 = none.  The softmax
+     * scale is 1/sqrt(qk_nope + qk_rope), times mscale^2 under YaRN. */
+    float yarn_factor, yarn_mscale_all_dim;
+    uint32_t yarn_orig_context_length;
+} jq_mla_config;
+
+/* q_or_q_a: attn_q [n_head*(nope+rope), n_embd], or attn_q_a [q_lora_rank, n_embd] with
+ * q_a_norm [q_lora_rank] (host f32) and q_b = attn_q_b [n_head*(nope+rope), q_lora_rank].
+ * kv_a_mqa [kv_lora_rank + rope, n_embd]; kv_a_norm [kv_lora_rank] (host f32).  The KV
+ * up-projection [n_head*(nope+v), kv_lora_rank] comes as a quantized weight (kv_b) or as
+ * dense row-major f32 on the host (kv_b_dense; what the reference rebuilds from the
+ * pre-split attn_k_b / attn_v_b tensors, src/quantized_deepseek2.rs:931-958): exactly one
+ * of the two.  o_proj [n_embd, n_head*v].  The weights must outlive the object. */
+int jq_mla_create(const jq_mla_config *cfg, const jq_weight *q_or_q_a, const float *q_a_norm,
+                  const jq_weight *q_b, const jq_weight *kv_a_mqa, const float *kv_a_norm,
+                  const jq_weight *kv_b, const float *kv_b_dense, const jq_weight *o_proj, jq_mla **out);
+void jq_mla_free(jq_mla *mla);
+
+/* out[n_tokens, n_embd] = attention(x[n_tokens, n_embd]) for tokens at cache positions
+ * pos .. pos + n_tokens - 1; `pos` must equal the number of tokens cached so far (the
+ * reference appends to its cache on every call, src/quantized_deepseek2.rs:479-486).
+ * Token i attends to positions 0 .. pos + i.  One call at a time per object. */
+int jq_mla_forward(jq_mla *mla, size_t n_tokens, size_t pos, const float *x, float *out,
+                   int ptrs_are_device, void *stream);
+/* Empties the cache (reference: src/quantized_deepseek2.rs:501-503 clear_kv_cache). */
+int jq_mla_reset(jq_mla *mla);
+/* Tokens in the cache. */
+size_t jq_mla_cached_tokens(const jq_mla *mla);
+
 /* ---- Dense Qwen3 decoder (end-to-end decode harness) -----------------------------
  * The graph the reference runs for a qwen3 GGUF: embedding gather, per layer
  * RMSNorm -> q/k/v -> per-head q/k RMSNorm -> half-split RoPE -> KV append ->

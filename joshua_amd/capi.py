@@ -28,6 +28,7 @@ EXPORTS = (
     "jq_last_error", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
     "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_try_matmul_fused", "jq_dequantize",
     "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
+    "jq_mla_create", "jq_mla_free", "jq_mla_forward", "jq_mla_reset", "jq_mla_cached_tokens",
     "jq_qwen3_create", "jq_qwen3_free", "jq_qwen3_set_tensor", "jq_qwen3_forward", "jq_qwen3_greedy", "jq_qwen3_reset",
     "jq_qwen3_get_config", "jq_qwen3_load_gguf", "jq_type_size_bytes", "jq_gguf_open", "jq_gguf_parse", "jq_gguf_close",
     "jq_gguf_version", "jq_gguf_tensor_data_offset", "jq_gguf_tensor_count", "jq_gguf_metadata_count",
@@ -47,6 +48,15 @@ class MoeConfig(ctypes.Structure):
                 ("inter", ctypes.c_uint32), ("gating", ctypes.c_uint32), ("norm_topk", ctypes.c_uint32),
                 ("weights_scale", ctypes.c_float), ("n_group", ctypes.c_uint32), ("topk_group", ctypes.c_uint32),
                 ("swiglu_clamp", ctypes.c_float), ("swiglu_clamp_shared", ctypes.c_float)]
+
+
+class MlaConfig(ctypes.Structure):
+    """jq_mla_config of include/joshua_hip.h."""
+    _fields_ = [("n_embd", ctypes.c_uint32), ("n_head", ctypes.c_uint32), ("q_lora_rank", ctypes.c_uint32),
+                ("kv_lora_rank", ctypes.c_uint32), ("qk_nope_head_dim", ctypes.c_uint32),
+                ("qk_rope_head_dim", ctypes.c_uint32), ("v_head_dim", ctypes.c_uint32), ("n_ctx", ctypes.c_uint32),
+                ("rms_eps", ctypes.c_float), ("rope_theta", ctypes.c_float), ("yarn_factor", ctypes.c_float),
+                ("yarn_mscale_all_dim", ctypes.c_float), ("yarn_orig_context_length", ctypes.c_uint32)]
 
 
 class Qwen3Config(ctypes.Structure):
@@ -100,6 +110,13 @@ def lib() -> ctypes.CDLL:
         L.jq_moe_free.restype = None
         L.jq_moe_route.argtypes = [vp, sz, vp, vp, vp, i32, vp]
         L.jq_moe_forward.argtypes = [vp, sz, vp, vp, i32, vp]
+        L.jq_mla_create.argtypes = [ctypes.POINTER(MlaConfig), vp, vp, vp, vp, vp, vp, vp, vp, ctypes.POINTER(vp)]
+        L.jq_mla_free.argtypes = [vp]
+        L.jq_mla_free.restype = None
+        L.jq_mla_forward.argtypes = [vp, sz, sz, vp, vp, i32, vp]
+        L.jq_mla_reset.argtypes = [vp]
+        L.jq_mla_cached_tokens.argtypes = [vp]
+        L.jq_mla_cached_tokens.restype = sz
         L.jq_qwen3_create.argtypes = [ctypes.POINTER(Qwen3Config), ctypes.POINTER(vp)]
         L.jq_qwen3_free.argtypes = [vp]
         L.jq_qwen3_free.restype = None
@@ -311,6 +328,57 @@ class Moe:
 
     def forward_dev(self, n_tokens: int, x_ptr: int, y_ptr: int, stream: int = 0) -> None:
         _check(lib().jq_moe_forward(self._h, n_tokens, x_ptr, y_ptr, 1, stream or None))
+
+
+class Mla:
+    """The multi-head latent attention block of the reference's deepseek2 graph on the device
+    (reference: src/quantized_deepseek2.rs:374-503 Attention).  `q` is attn_q, or with a low-rank Q
+    projection the triple (attn_q_a, attn_q_a_norm, attn_q_b); `kv_b` is a Weight or a dense f32
+    [n_head * (qk_nope + v_head_dim), kv_lora_rank] array."""
+
+    def __init__(self, cfg: MlaConfig, q, kv_a_mqa: Weight, kv_a_norm: np.ndarray, kv_b, o_proj: Weight):
+        self.cfg = cfg
+        q_a, q_norm, q_b = q if isinstance(q, tuple) else (q, None, None)
+        qn = None if q_norm is None else np.ascontiguousarray(q_norm, dtype=np.float32)
+        kn = np.ascontiguousarray(kv_a_norm, dtype=np.float32)
+        dense = None if isinstance(kv_b, Weight) else np.ascontiguousarray(kv_b, dtype=np.float32)
+        if dense is not None:
+            assert dense.size == cfg.n_head * (cfg.qk_nope_head_dim + cfg.v_head_dim) * cfg.kv_lora_rank
+        assert kn.size == cfg.kv_lora_rank and (qn is None or qn.size == cfg.q_lora_rank)
+        self._keep = (q_a, q_b, kv_a_mqa, kv_b, o_proj)
+        out = ctypes.c_void_p()
+        _check(lib().jq_mla_create(ctypes.byref(cfg), q_a.handle, None if qn is None else qn.ctypes.data,
+                                   None if q_b is None else q_b.handle, kv_a_mqa.handle, kn.ctypes.data,
+                                   kv_b.handle if dense is None else None, None if dense is None else dense.ctypes.data,
+                                   o_proj.handle, ctypes.byref(out)))
+        self._h = out
+
+    def close(self) -> None:
+        if self._h:
+            lib().jq_mla_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def forward(self, x: np.ndarray, pos: int) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        y = np.empty_like(x)
+        _check(lib().jq_mla_forward(self._h, x.shape[0], pos, x.ctypes.data, y.ctypes.data, 0, None))
+        return y
+
+    def forward_dev(self, n_tokens: int, pos: int, x_ptr: int, y_ptr: int, stream: int = 0) -> None:
+        _check(lib().jq_mla_forward(self._h, n_tokens, pos, x_ptr, y_ptr, 1, stream or None))
+
+    def reset(self) -> None:
+        _check(lib().jq_mla_reset(self._h))
+
+    @property
+    def cached_tokens(self) -> int:
+        return int(lib().jq_mla_cached_tokens(self._h))
 
 
 class Qwen3:

@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <set>
 #include <mutex>
 #include <string>
@@ -17,6 +18,7 @@
 #include "../../include/joshua_hip.h"
 #include "kernels_mfma_q4k.hpp"
 #include "kernels_graph.hpp"
+#include "kernels_mla.hpp"
 #include "kernels_mfma_q4k_gemm.hpp"
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
@@ -1190,6 +1192,259 @@ int jq_moe_forward(jq_moe *m, size_t n_tokens, const float *x, float *y, int ptr
     HIP_TRY(hipStreamSynchronize(s));
     return 0;
 }
+
+}  // extern "C"
+
+// ---- multi-head latent attention -----------------------------------------------------
+
+struct jq_mla {
+    jq_mla_config cfg;
+    const jq_weight *q, *q_b, *kv_a, *kv_b, *o;
+    float *q_a_norm = nullptr, *kv_a_norm = nullptr;
+    float *wkv = nullptr;   // the KV up-projection as dense f32 [n_head * (nope + vh), lkv]
+    float2 *cs = nullptr;   // [n_ctx][rope / 2] (cos, sin), scaled by the YaRN mscale
+    float *lat = nullptr, *kpe = nullptr;  // the cache: [n_ctx][lkv] normed latents, [n_ctx][rope] rotated keys
+    float scale = 0.0f;
+    size_t n_past = 0;
+    // scratch, grown to the largest token count seen
+    size_t cap_tokens = 0;
+    float *t1 = nullptr, *t1n = nullptr, *qv = nullptr, *comp = nullptr, *qabs = nullptr, *part = nullptr, *ctx = nullptr;
+    std::mutex mu;
+};
+
+namespace {
+
+constexpr size_t MLA_PART_SLOTS = 64;  // partial results kept per head: tokens of a call x context splits
+
+void mla_free_scratch(jq_mla *m) {
+    for (void *p : {(void *)m->t1, (void *)m->t1n, (void *)m->qv, (void *)m->comp, (void *)m->qabs, (void *)m->part, (void *)m->ctx})
+        if (p) (void)hipFree(p);
+    m->t1 = m->t1n = m->qv = m->comp = m->qabs = m->part = m->ctx = nullptr;
+    m->cap_tokens = 0;
+}
+
+int mla_reserve(jq_mla *m, size_t T) {
+    if (T <= m->cap_tokens) return 0;
+    mla_free_scratch(m);
+    const jq_mla_config &c = m->cfg;
+    const size_t qd = c.qk_nope_head_dim + c.qk_rope_head_dim;
+    if (c.q_lora_rank) {
+        HIP_TRY(hipMalloc((void **)&m->t1, T * c.q_lora_rank * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&m->t1n, T * c.q_lora_rank * sizeof(float)));
+    }
+    HIP_TRY(hipMalloc((void **)&m->qv, T * c.n_head * qd * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->comp, T * (c.kv_lora_rank + c.qk_rope_head_dim) * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->qabs, T * c.n_head * c.kv_lora_rank * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->part, std::max(T, MLA_PART_SLOTS) * c.n_head * (c.kv_lora_rank + 2) * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->ctx, T * c.n_head * c.v_head_dim * sizeof(float)));
+    m->cap_tokens = T;
+    return 0;
+}
+
+// YaRN helpers in f32, as the reference computes them (src/quantized_deepseek2.rs:230-236, :314-339).
+float yarn_get_mscale(float scale, float mscale) { return scale <= 1.0f ? 1.0f : 0.1f * mscale * logf(scale) + 1.0f; }
+float yarn_find_correction_dim(float num_rot, size_t dim, float base, size_t max_pos) {
+    return ((float)dim * logf((float)max_pos / (num_rot * 2.0f * 3.14159265358979323846f))) / (2.0f * logf(base));
+}
+
+// (cos, sin) of every position and rotary pair, scaled by mscale (src/quantized_deepseek2.rs:246-301).
+std::vector<float2> mla_rope_table(const jq_mla_config &c) {
+    const size_t dim = c.qk_rope_head_dim, half = dim / 2;
+    std::vector<float> inv(half);
+    float mscale = 1.0f;
+    for (size_t i = 0; i < half; i++) inv[i] = 1.0f / powf(c.rope_theta, (float)(2 * i) / (float)dim);
+    if (c.yarn_factor > 0.0f) {
+        float lo = floorf(yarn_find_correction_dim(32.0f, dim, c.rope_theta, c.yarn_orig_context_length));
+        float hi = ceilf(yarn_find_correction_dim(1.0f, dim, c.rope_theta, c.yarn_orig_context_length));
+        lo = std::max(lo, 0.0f), hi = std::min(hi, (float)dim - 1.0f);
+        if (fabsf(lo - hi) < 1.1920929e-7f) hi += 0.001f;
+        for (size_t i = 0; i < half; i++) {
+            const float extra = inv[i], inter = 1.0f / (c.yarn_factor * powf(c.rope_theta, (float)(2 * i) / (float)dim));
+            const float ramp = std::min(std::max(((float)i - lo) / (hi - lo), 0.0f), 1.0f), mask = 1.0f - ramp;
+            inv[i] = inter * (1.0f - mask) + extra * mask;
+        }
+        mscale = yarn_get_mscale(c.yarn_factor, c.yarn_mscale_all_dim);
+    }
+    std::vector<float2> cs((size_t)c.n_ctx * half);
+    for (size_t t = 0; t < c.n_ctx; t++)
+        for (size_t i = 0; i < half; i++) {
+            const float f = (float)t * inv[i];
+            cs[t * half + i] = float2{cosf(f) * mscale, sinf(f) * mscale};
+        }
+    return cs;
+}
+
+int mla_check_weight(const char *what, const jq_weight *w, size_t n, size_t k) {
+    if (!w) return fail("jq_mla_create: %s is null", what);
+    if (w->n != n || w->k != k) return fail("jq_mla_create: %s is [%zu, %zu], expected [%zu, %zu]", what, w->n, w->k, n, k);
+    return 0;
+}
+
+template <int G>
+int mla_launch_attention(const jq_mla *m, size_t S, size_t pos, unsigned n_split, hipStream_t s) {
+    const jq_mla_config &c = m->cfg;
+    const dim3 grid(c.n_head / G, n_split, (unsigned)S);
+    const int lpl = (int)((c.kv_lora_rank + 63) / 64);
+#define JQ_MLA_ATT(LPL)                                                                                              \
+    hipLaunchKernelGGL((jq::mla_attention<G, LPL>), grid, dim3(256), 0, s, m->qabs, m->qv, m->lat, m->kpe, m->part, \
+                       (int)c.n_head, (int)c.qk_nope_head_dim, (int)c.qk_rope_head_dim, (int)c.kv_lora_rank, (int)pos, \
+                       (int)n_split, m->scale)
+    if (lpl <= 1) JQ_MLA_ATT(1);
+    else if (lpl <= 2) JQ_MLA_ATT(2);
+    else if (lpl <= 4) JQ_MLA_ATT(4);
+    else JQ_MLA_ATT(8);
+#undef JQ_MLA_ATT
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// x, out: device pointers; S tokens at positions pos .. pos + S - 1; scratch reserved for S.
+int mla_forward_dev(jq_mla *m, size_t S, size_t pos, const float *x, float *out, hipStream_t s) {
+    const jq_mla_config &c = m->cfg;
+    const size_t nh = c.n_head, nope = c.qk_nope_head_dim, rope = c.qk_rope_head_dim, vh = c.v_head_dim,
+                 lkv = c.kv_lora_rank, qd = nope + rope;
+    if (c.q_lora_rank) {
+        if (dispatch_matmul(m->q->type, m->q->dev, m->q->row_bytes, x, m->t1, S, c.n_embd, c.q_lora_rank, s)) return 1;
+        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3((unsigned)S), dim3(1024), 0, s, m->t1, (const float *)nullptr,
+                           (const float *)m->q_a_norm, c.rms_eps, m->t1n, (int)c.q_lora_rank);
+        HIP_TRY(hipGetLastError());
+        if (dispatch_matmul(m->q_b->type, m->q_b->dev, m->q_b->row_bytes, m->t1n, m->qv, S, c.q_lora_rank, nh * qd, s)) return 1;
+    } else if (dispatch_matmul(m->q->type, m->q->dev, m->q->row_bytes, x, m->qv, S, c.n_embd, nh * qd, s)) {
+        return 1;
+    }
+    if (dispatch_matmul(m->kv_a->type, m->kv_a->dev, m->kv_a->row_bytes, x, m->comp, S, c.n_embd, lkv + rope, s)) return 1;
+    hipLaunchKernelGGL(jq::mla_rope_latent, dim3((unsigned)nh + 1, (unsigned)S), dim3(64), 0, s, m->qv, (const float *)m->comp,
+                       (const float *)m->kv_a_norm, (const float2 *)m->cs, m->lat, m->kpe, (int)nh, (int)nope, (int)rope,
+                       (int)lkv, (int)pos, c.rms_eps);
+    HIP_TRY(hipGetLastError());
+    constexpr int ST = 4;
+    hipLaunchKernelGGL(jq::mla_absorb_q<ST>, dim3((unsigned)nh, (unsigned)((S + ST - 1) / ST)), dim3(256), 0, s,
+                       (const float *)m->qv, (const float *)m->wkv, m->qabs, (int)S, (int)nh, (int)nope, (int)rope, (int)vh,
+                       (int)lkv);
+    HIP_TRY(hipGetLastError());
+    // heads per workgroup, then enough context splits to fill the chip when the call has few tokens
+    const int G = nh % 8 == 0 ? 8 : nh % 4 == 0 ? 4 : nh % 2 == 0 ? 2 : 1;
+    const size_t wgs = S * (nh / G), total = pos + S;
+    size_t n_split = std::min<size_t>({(1024 + wgs - 1) / wgs, (total + 31) / 32, (size_t)jq::MLA_SPLIT_MAX,
+                                       std::max<size_t>(MLA_PART_SLOTS / S, 1)});
+    n_split = std::max<size_t>(n_split, 1);
+    int rc = G == 8 ? mla_launch_attention<8>(m, S, pos, (unsigned)n_split, s)
+             : G == 4 ? mla_launch_attention<4>(m, S, pos, (unsigned)n_split, s)
+             : G == 2 ? mla_launch_attention<2>(m, S, pos, (unsigned)n_split, s)
+                      : mla_launch_attention<1>(m, S, pos, (unsigned)n_split, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(jq::mla_merge_vproj, dim3((unsigned)nh, (unsigned)S), dim3(256), 0, s, (const float *)m->part,
+                       (const float *)m->wkv, m->ctx, (int)nh, (int)nope, (int)vh, (int)lkv, (int)n_split);
+    HIP_TRY(hipGetLastError());
+    return dispatch_matmul(m->o->type, m->o->dev, m->o->row_bytes, m->ctx, out, S, nh * vh, c.n_embd, s);
+}
+
+}  // namespace
+
+extern "C" {
+
+int jq_mla_create(const jq_mla_config *cfg, const jq_weight *q_or_q_a, const float *q_a_norm, const jq_weight *q_b,
+                  const jq_weight *kv_a_mqa, const float *kv_a_norm, const jq_weight *kv_b, const float *kv_b_dense,
+                  const jq_weight *o_proj, jq_mla **out) {
+    if (!cfg || !out) return fail("jq_mla_create: null argument");
+    if (ensure_init()) return 1;
+    const jq_mla_config &c = *cfg;
+    const size_t nh = c.n_head, nope = c.qk_nope_head_dim, rope = c.qk_rope_head_dim, vh = c.v_head_dim,
+                 lkv = c.kv_lora_rank, qd = nope + rope;
+    if (!c.n_embd || !nh || !lkv || !rope || !vh || !c.n_ctx) return fail("jq_mla_create: a dimension is zero");
+    if (rope % 2 != 0 || rope > 64) return fail("jq_mla_create: qk_rope_head_dim %zu must be even and at most 64", rope);
+    if (lkv > (size_t)jq::MLA_MAX_LKV) return fail("jq_mla_create: kv_lora_rank %zu exceeds %d", lkv, jq::MLA_MAX_LKV);
+    if (nope > (size_t)jq::MLA_MAX_NOPE) return fail("jq_mla_create: qk_nope_head_dim %zu exceeds %d", nope, jq::MLA_MAX_NOPE);
+    if (c.q_lora_rank && (c.q_lora_rank % 4 != 0 || c.q_lora_rank > 8192))
+        return fail("jq_mla_create: q_lora_rank %u must be a multiple of 4, at most 8192", c.q_lora_rank);
+    if (c.yarn_factor > 0.0f && c.yarn_orig_context_length == 0) return fail("jq_mla_create: YaRN without an original context length");
+    if (c.q_lora_rank) {
+        if (mla_check_weight("attn_q_a", q_or_q_a, c.q_lora_rank, c.n_embd)) return 1;
+        if (mla_check_weight("attn_q_b", q_b, nh * qd, c.q_lora_rank)) return 1;
+        if (!q_a_norm) return fail("jq_mla_create: attn_q_a_norm is null");
+    } else if (mla_check_weight("attn_q", q_or_q_a, nh * qd, c.n_embd)) {
+        return 1;
+    }
+    if (mla_check_weight("attn_kv_a_mqa", kv_a_mqa, lkv + rope, c.n_embd)) return 1;
+    if (!kv_a_norm) return fail("jq_mla_create: attn_kv_a_norm is null");
+    if ((kv_b != nullptr) == (kv_b_dense != nullptr)) return fail("jq_mla_create: give attn_kv_b either quantized or dense");
+    if (kv_b && mla_check_weight("attn_kv_b", kv_b, nh * (nope + vh), lkv)) return 1;
+    if (mla_check_weight("attn_output", o_proj, c.n_embd, nh * vh)) return 1;
+
+    std::unique_ptr<jq_mla, void (*)(jq_mla *)> m(new jq_mla, jq_mla_free);
+    m->cfg = c;
+    m->q = q_or_q_a, m->q_b = q_b, m->kv_a = kv_a_mqa, m->kv_b = kv_b, m->o = o_proj;
+    double scale = 1.0 / sqrt((double)qd);  // f64 as in the reference (src/quantized_deepseek2.rs:186-192)
+    if (c.yarn_factor > 0.0f) {
+        const double ms = (double)yarn_get_mscale(c.yarn_factor, c.yarn_mscale_all_dim);
+        scale *= ms * ms;
+    }
+    m->scale = (float)scale;
+    const size_t wkv_elems = nh * (nope + vh) * lkv;
+    HIP_TRY(hipMalloc((void **)&m->wkv, wkv_elems * sizeof(float)));
+    if (kv_b) {
+        if (dispatch_decode(kv_b, nullptr, m->wkv, kv_b->n, nullptr)) return 1;
+    } else {
+        HIP_TRY(hipMemcpy(m->wkv, kv_b_dense, wkv_elems * sizeof(float), hipMemcpyHostToDevice));
+    }
+    if (c.q_lora_rank) {
+        HIP_TRY(hipMalloc((void **)&m->q_a_norm, c.q_lora_rank * sizeof(float)));
+        HIP_TRY(hipMemcpy(m->q_a_norm, q_a_norm, c.q_lora_rank * sizeof(float), hipMemcpyHostToDevice));
+    }
+    HIP_TRY(hipMalloc((void **)&m->kv_a_norm, lkv * sizeof(float)));
+    HIP_TRY(hipMemcpy(m->kv_a_norm, kv_a_norm, lkv * sizeof(float), hipMemcpyHostToDevice));
+    const std::vector<float2> cs = mla_rope_table(c);
+    HIP_TRY(hipMalloc((void **)&m->cs, cs.size() * sizeof(float2)));
+    HIP_TRY(hipMemcpy(m->cs, cs.data(), cs.size() * sizeof(float2), hipMemcpyHostToDevice));
+    HIP_TRY(hipMalloc((void **)&m->lat, (size_t)c.n_ctx * lkv * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->kpe, (size_t)c.n_ctx * rope * sizeof(float)));
+    HIP_TRY(hipDeviceSynchronize());
+    *out = m.release();
+    return 0;
+}
+
+void jq_mla_free(jq_mla *m) {
+    if (!m) return;
+    mla_free_scratch(m);
+    for (void *p : {(void *)m->q_a_norm, (void *)m->kv_a_norm, (void *)m->wkv, (void *)m->cs, (void *)m->lat, (void *)m->kpe})
+        if (p) (void)hipFree(p);
+    delete m;
+}
+
+int jq_mla_forward(jq_mla *m, size_t n_tokens, size_t pos, const float *x, float *out, int ptrs_are_device, void *stream) {
+    if (!m) return fail("jq_mla_forward: object is null");
+    if (n_tokens == 0) return 0;
+    if (!x || !out) return fail("jq_mla_forward: null pointer");
+    std::lock_guard<std::mutex> lock(m->mu);
+    if (pos != m->n_past) return fail("jq_mla_forward: pos %zu, but %zu tokens are cached", pos, m->n_past);
+    if (pos + n_tokens > m->cfg.n_ctx) return fail("jq_mla_forward: %zu + %zu tokens exceed the context of %u", pos, n_tokens, m->cfg.n_ctx);
+    if (n_tokens > 0x7FFF) return fail("jq_mla_forward: at most 32767 tokens a call");
+    hipStream_t s = (hipStream_t)stream;
+    if (mla_reserve(m, n_tokens)) return 1;
+    const size_t bytes = n_tokens * m->cfg.n_embd * sizeof(float);
+    if (ptrs_are_device) {
+        if (mla_forward_dev(m, n_tokens, pos, x, out, s)) return 1;
+    } else {
+        DevBuf xd, yd;
+        HIP_TRY(xd.alloc(bytes));
+        HIP_TRY(yd.alloc(bytes));
+        HIP_TRY(hipMemcpyAsync(xd.p, x, bytes, hipMemcpyHostToDevice, s));
+        if (mla_forward_dev(m, n_tokens, pos, (const float *)xd.p, (float *)yd.p, s)) return 1;
+        HIP_TRY(hipMemcpyAsync(out, yd.p, bytes, hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+    }
+    m->n_past += n_tokens;
+    return 0;
+}
+
+int jq_mla_reset(jq_mla *m) {
+    if (!m) return fail("jq_mla_reset: object is null");
+    std::lock_guard<std::mutex> lock(m->mu);
+    m->n_past = 0;
+    return 0;
+}
+
+size_t jq_mla_cached_tokens(const jq_mla *m) { return m ? m->n_past : 0; }
 
 }  // extern "C"
 

@@ -1,0 +1,211 @@
+// Multi-head latent attention (DeepSeek-V2 / V3 / Kimi-K2) in its absorbed form, f32 throughout.
+//
+// The reference (src/quantized_deepseek2.rs:422-499) expands every new token's latent through the KV
+// up-projection into per-head keys and values and caches those: n_head * (qk_nope + qk_rope +
+// v_head_dim) floats a token (160 KB at V3 size), all of which a decode step reads back.  The same
+// numbers come out of the latent itself: with W_k[h] (qk_nope x kv_lora_rank) and W_v[h] (v_head_dim x
+// kv_lora_rank) the rows of the up-projection for head h,
+//     q_nope[h] . (W_k[h] c_t)  =  (W_k[h]^T q_nope[h]) . c_t
+//     sum_t p_t (W_v[h] c_t)    =  W_v[h] (sum_t p_t c_t)
+// so the cache holds, per token, the normed latent c_t (kv_lora_rank) and the rotated shared key k_pe
+// (qk_rope): 2.3 KB at V3 size, shared by all heads.  A step is
+//   mla_rope_latent   rotate q_pe in place; norm the latent, rotate k_pe, append both to the cache
+//   mla_absorb_q      q_abs[h] = W_k[h]^T q_nope[h]
+//   mla_attention     scores over the cached latents, running softmax, o_lat[h] = sum p_t c_t, the
+//                     context split over workgroups (partial maximum, sum and vector per split)
+//   mla_merge_vproj   merge the splits, ctx[h] = W_v[h] o_lat[h]
+// around the quantized projections (q, kv_a, o), which run on the matmul kernels.
+#pragma once
+#include "kernels_graph.hpp"
+
+namespace jq {
+
+// grid (n_head + 1, S), one wave.  Workgroups x < n_head rotate the rope slice of q[s, x] in place
+// (neighbouring pairs (2i, 2i+1), candle's rope_i; cs[p][i] = (cos, sin) of position p, pair i, already
+// scaled by the YaRN mscale; reference :302-311).  Workgroup x == n_head norms the latent
+// comp[s, 0:lkv] (RMSNorm, weight w) into lat[pos0 + s] and rotates comp[s, lkv:] into kpe[pos0 + s].
+__global__ __launch_bounds__(64) void mla_rope_latent(float *__restrict__ q, const float *__restrict__ comp,
+                                                       const float *__restrict__ w, const float2 *__restrict__ cs,
+                                                       float *__restrict__ lat, float *__restrict__ kpe, int n_head,
+                                                       int nope, int rope, int lkv, int pos0, float eps) {
+    const int s = blockIdx.y, lane = threadIdx.x, half = rope >> 1;
+    const float2 *c = cs + (size_t)(pos0 + s) * half;
+    if ((int)blockIdx.x < n_head) {
+        float *v = q + ((size_t)s * n_head + blockIdx.x) * (nope + rope) + nope;
+        for (int i = lane; i < half; i += 64) {
+            const float a = v[2 * i], b = v[2 * i + 1];
+            v[2 * i] = a * c[i].x - b * c[i].y;
+            v[2 * i + 1] = a * c[i].y + b * c[i].x;
+        }
+        return;
+    }
+    const float *x = comp + (size_t)s * (lkv + rope);
+    float ss = 0.0f;
+    for (int i = lane; i < lkv; i += 64) ss = fmaf(x[i], x[i], ss);
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)lkv + eps);
+    float *l = lat + (size_t)(pos0 + s) * lkv, *k = kpe + (size_t)(pos0 + s) * rope;
+    for (int i = lane; i < lkv; i += 64) l[i] = x[i] * inv * w[i];
+    for (int i = lane; i < half; i += 64) {
+        const float a = x[lkv + 2 * i], b = x[lkv + 2 * i + 1];
+        k[2 * i] = a * c[i].x - b * c[i].y;
+        k[2 * i + 1] = a * c[i].y + b * c[i].x;
+    }
+}
+
+// q_abs[s, h, c] = sum_r q[s, h, r] * Wkv[h * (nope + vh) + r, c], r < nope.  grid (n_head, ceil(S / ST)),
+// 256 threads: a thread owns columns c, c + 256, ... and walks the nope rows of its head, whose values
+// for the ST tokens wait in LDS; the rows are read coalesced, once per ST tokens.
+constexpr int MLA_MAX_NOPE = 256;
+template <int ST>
+__global__ __launch_bounds__(256) void mla_absorb_q(const float *__restrict__ q, const float *__restrict__ Wkv,
+                                                     float *__restrict__ qabs, int S, int n_head, int nope, int rope,
+                                                     int vh, int lkv) {
+    __shared__ float qs[MLA_MAX_NOPE][ST];
+    const int h = blockIdx.x, s0 = blockIdx.y * ST, qd = nope + rope;
+    for (int e = threadIdx.x; e < nope * ST; e += 256) {
+        const int r = e / ST, j = e % ST;
+        qs[r][j] = s0 + j < S ? q[((size_t)(s0 + j) * n_head + h) * qd + r] : 0.0f;
+    }
+    __syncthreads();
+    const float *W = Wkv + (size_t)h * (nope + vh) * lkv;
+    for (int c = threadIdx.x; c < lkv; c += 256) {
+        float acc[ST];
+#pragma unroll
+        for (int j = 0; j < ST; j++) acc[j] = 0.0f;
+#pragma unroll 8
+        for (int r = 0; r < nope; r++) {
+            const float wv = W[(size_t)r * lkv + c];
+#pragma unroll
+            for (int j = 0; j < ST; j++) acc[j] = fmaf(qs[r][j], wv, acc[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < ST; j++)
+            if (s0 + j < S) qabs[((size_t)(s0 + j) * n_head + h) * lkv + c] = acc[j];
+    }
+}
+
+// Scores, running softmax and the weighted latent sum for G heads of one query token over one split of
+// its context.  grid (n_head / G, n_split, S), four waves; wave w takes tokens t0 + w, t0 + w + 4, ... of
+// the split: a lane holds LPL consecutive latent elements (and one rope element) of the token, loaded
+// once for the G heads, and the same elements of every head's absorbed query; a score is the wave sum
+// of the products.  The four waves' (maximum, sum, vector) merge through LDS into
+// part[s, h, split] = {m, l, o[lkv]}, unnormalised.  lkv <= 64 LPL, rope <= 64.  Query token s sees
+// cache tokens 0 .. pos0 + s (the causal mask of the reference, :875-889).
+constexpr int MLA_SPLIT_MAX = 64;
+template <int G, int LPL>
+__global__ __launch_bounds__(256) void mla_attention(const float *__restrict__ qabs, const float *__restrict__ q,
+                                                      const float *__restrict__ lat, const float *__restrict__ kpe,
+                                                      float *__restrict__ part, int n_head, int nope, int rope, int lkv,
+                                                      int pos0, int n_split, float scale) {
+    __shared__ float wm[4][G], wl[4][G];
+    __shared__ float wo[4][G][64 * LPL];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h0 = blockIdx.x * G, split = blockIdx.y, s = blockIdx.z;
+    const int T = pos0 + s + 1, chunk = (T + n_split - 1) / n_split;
+    const int t0 = split * chunk, t1 = min(T, t0 + chunk);
+    const bool vec = lkv == 64 * LPL && LPL % 4 == 0;  // whole float4 loads
+    const int e0 = lane * LPL;
+
+    float qa[G][LPL], qp[G], m[G], l[G], o[G][LPL];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const float *qv = qabs + ((size_t)s * n_head + h0 + g) * lkv;
+#pragma unroll
+        for (int i = 0; i < LPL; i++) qa[g][i] = e0 + i < lkv ? qv[e0 + i] : 0.0f, o[g][i] = 0.0f;
+        qp[g] = lane < rope ? q[((size_t)s * n_head + h0 + g) * (nope + rope) + nope + lane] : 0.0f;
+        m[g] = -INFINITY, l[g] = 0.0f;
+    }
+    for (int t = t0 + wave; t < t1; t += 4) {
+        float c[LPL];
+        const float *cv = lat + (size_t)t * lkv;
+        bool loaded = false;
+        if constexpr (LPL % 4 == 0) {
+            if (vec) {
+#pragma unroll
+                for (int i = 0; i < LPL; i += 4) {
+                    const float4 v = *(const float4 *)(cv + e0 + i);
+                    c[i] = v.x, c[i + 1] = v.y, c[i + 2] = v.z, c[i + 3] = v.w;
+                }
+                loaded = true;
+            }
+        }
+        if (!loaded) {
+#pragma unroll
+            for (int i = 0; i < LPL; i++) c[i] = e0 + i < lkv ? cv[e0 + i] : 0.0f;
+        }
+        const float kp = lane < rope ? kpe[(size_t)t * rope + lane] : 0.0f;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float sc = qp[g] * kp;
+#pragma unroll
+            for (int i = 0; i < LPL; i++) sc = fmaf(qa[g][i], c[i], sc);
+            sc = wave_sum(sc) * scale;
+            const float mn = fmaxf(m[g], sc);
+            const float a = __expf(m[g] - mn), p = __expf(sc - mn);  // the first token: a = exp(-inf) = 0
+            l[g] = fmaf(l[g], a, p);
+#pragma unroll
+            for (int i = 0; i < LPL; i++) o[g][i] = fmaf(o[g][i], a, p * c[i]);
+            m[g] = mn;
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        if (lane == 0) wm[wave][g] = m[g], wl[wave][g] = l[g];
+#pragma unroll
+        for (int i = 0; i < LPL; i++) wo[wave][g][e0 + i] = o[g][i];
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < G * 64 * LPL; e += 256) {
+        const int g = e / (64 * LPL), i = e % (64 * LPL);
+        const float M = fmaxf(fmaxf(wm[0][g], wm[1][g]), fmaxf(wm[2][g], wm[3][g]));
+        float ov = 0.0f, lv = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float f = wm[w][g] == -INFINITY ? 0.0f : __expf(wm[w][g] - M);  // a wave without tokens
+            ov = fmaf(wo[w][g][i], f, ov);
+            lv = fmaf(wl[w][g], f, lv);
+        }
+        float *p = part + (((size_t)s * n_head + h0 + g) * n_split + split) * (lkv + 2);
+        if (i < lkv) p[2 + i] = ov;
+        if (i == 0) p[0] = M, p[1] = lv;
+    }
+}
+
+// grid (n_head, S), 256 threads: merges the splits of (s, h) into the normalised latent sum (in LDS)
+// and multiplies by the head's value rows: ctx[s, h * vh + j] = Wkv[h * (nope + vh) + nope + j, :] .
+// o_lat, one wave per row, rows j = wave, wave + 4, ...
+constexpr int MLA_MAX_LKV = 512;
+__global__ __launch_bounds__(256) void mla_merge_vproj(const float *__restrict__ part, const float *__restrict__ Wkv,
+                                                        float *__restrict__ ctx, int n_head, int nope, int vh, int lkv,
+                                                        int n_split) {
+    __shared__ float ol[MLA_MAX_LKV];
+    __shared__ float f[MLA_SPLIT_MAX];
+    __shared__ float Linv;
+    const int h = blockIdx.x, s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float *p = part + ((size_t)s * n_head + h) * n_split * (lkv + 2);
+    if (wave == 0) {  // n_split <= 64
+        const float mi = lane < n_split ? p[(size_t)lane * (lkv + 2)] : -INFINITY;
+        const float M = wave_max(mi);
+        const float fi = mi == -INFINITY ? 0.0f : __expf(mi - M);  // an empty split
+        const float L = wave_sum(lane < n_split ? p[(size_t)lane * (lkv + 2) + 1] * fi : 0.0f);
+        f[lane] = fi;
+        if (lane == 0) Linv = 1.0f / L;
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < lkv; c += 256) {
+        float v = 0.0f;
+        for (int i = 0; i < n_split; i++) v = fmaf(p[(size_t)i * (lkv + 2) + 2 + c], f[i], v);
+        ol[c] = v * Linv;
+    }
+    __syncthreads();
+    const float *W = Wkv + ((size_t)h * (nope + vh) + nope) * lkv;
+    for (int j = wave; j < vh; j += 4) {
+        float acc = 0.0f;
+        for (int c = lane; c < lkv; c += 64) acc = fmaf(W[(size_t)j * lkv + c], ol[c], acc);
+        acc = wave_sum(acc);
+        if (lane == 0) ctx[((size_t)s * n_head + h) * vh + j] = acc;
+    }
+}
+
+}  // namespace jq
