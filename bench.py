@@ -151,11 +151,69 @@ def moe_workload(torch, capi, synth, qtype: int, h: int, inter: int, n_expert: i
     return res
 
 
-def extra_workloads(steps: int) -> dict:
+DEEPSEEK_V3_MLA = dict(n_embd=7168, n_head=128, q_lora_rank=1536, kv_lora_rank=512, qk_nope_head_dim=128,
+                       qk_rope_head_dim=64, v_head_dim=128, rms_eps=1e-6, rope_theta=10000.0, yarn_factor=40.0,
+                       yarn_mscale_all_dim=1.0, yarn_orig_context_length=4096)
+
+
+def mla_workload(torch, capi, synth, qtype: int, context: int, steps: int, seed: int) -> dict:
+    """One multi-head latent attention block of DeepSeek-V3 size: a prompt of `context` tokens in chunks of
+    512, then `steps` single-token calls (the cache grows by one token a call)."""
+    c = DEEPSEEK_V3_MLA
+    be, bb = BLOCK[qtype]
+    dev = torch.device("cuda:0")
+    nh, qd = c["n_head"], c["qk_nope_head_dim"] + c["qk_rope_head_dim"]
+    shapes = {"q_a": (c["q_lora_rank"], c["n_embd"]), "q_b": (nh * qd, c["q_lora_rank"]),
+              "kv_a": (c["kv_lora_rank"] + c["qk_rope_head_dim"], c["n_embd"]),
+              "kv_b": (nh * (c["qk_nope_head_dim"] + c["v_head_dim"]), c["kv_lora_rank"]),
+              "o": (c["n_embd"], nh * c["v_head_dim"])}
+    w = {name: capi.Weight.upload(qtype, synth.normal_quantized(qtype, seed + i, n * k, 0.02), n, k)
+         for i, (name, (n, k)) in enumerate(shapes.items())}
+    cfg = capi.MlaConfig(n_ctx=context + 2 * steps + 64, **c)
+    mla = capi.Mla(cfg, (w["q_a"], np.ones(c["q_lora_rank"], np.float32), w["q_b"]), w["kv_a"],
+                   np.ones(c["kv_lora_rank"], np.float32), w["kv_b"], w["o"])
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+    chunk = 512
+    xs = torch.from_numpy(synth.normal(seed + 10, (chunk, c["n_embd"]))).to(dev)
+    y = torch.zeros((chunk, c["n_embd"]), device=dev)
+    pos, prefill_ms = 0, 0.0
+    while pos < context:
+        t = min(chunk, context - pos)
+        p0 = pos
+        prefill_ms += _time_calls(torch, stream, lambda i: mla.forward_dev(t, p0, xs.data_ptr(), y.data_ptr(), sh), 1)
+        pos += t
+    state = {"pos": pos}
+
+    def call(i):
+        mla.forward_dev(1, state["pos"], xs.data_ptr() + 4 * c["n_embd"] * (i % chunk), y.data_ptr(), sh)
+        state["pos"] += 1
+
+    _time_calls(torch, stream, call, max(steps // 10, 3))
+    ms = _time_calls(torch, stream, call, steps)
+    quantized = sum(n * (k // be) * bb for name, (n, k) in shapes.items() if name != "kv_b")
+    kv_b_f32 = 4 * shapes["kv_b"][0] * shapes["kv_b"][1]  # the up-projection is held decoded
+    cache = 4 * (c["kv_lora_rank"] + c["qk_rope_head_dim"]) * (context + steps // 2)
+    abytes = quantized + kv_b_f32 + cache + 8 * c["n_embd"]
+    res = {"us": round(ms * 1e3, 2), "context": context, "algorithmic_bytes": abytes, "gbs": round(abytes / ms / 1e6, 1),
+           "hbm_frac": round(abytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+           "prefill_tokens_per_s": round(context / prefill_ms * 1e3, 1),
+           "cache_bytes_per_token": 4 * (c["kv_lora_rank"] + c["qk_rope_head_dim"]),
+           "reference_cache_bytes_per_token": 4 * nh * (qd + c["v_head_dim"])}
+    mla.close()
+    return res
+
+
+def extra_workloads(steps: int, only: str = "") -> dict:
     """The other configurations of the path, one figure each (cold HBM unless noted)."""
     import torch
     from joshua_amd import capi, synth
     out = {}
+    if only:  # a single workload, for profiling
+        if "mla" in only:
+            out["mla_deepseek_v3_q4_k_ctx%s_b1" % only.split(":")[-1]] = mla_workload(
+                torch, capi, synth, 12, int(only.split(":")[-1]), steps, 107)
+        return out
     out["q8_0_gemv_4096x4096_m1"] = matmul_workload(torch, capi, synth, 8, 4096, 4096, 1, 101, steps, 24)
     out["q4_k_14336x4096_m16"] = matmul_workload(torch, capi, synth, 12, N, K, 16, 102, steps, 24)
     out["q4_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 12, N, K, 512, 102, max(steps // 10, 10), 4)
@@ -171,6 +229,9 @@ def extra_workloads(steps: int) -> dict:
     out["moe_deepseek_v3_mxfp4_b1"] = moe_workload(torch, capi, synth, 39, 7168, 2048, 256, 8, 1, 105, max(steps // 4, 10),
                                                    True, 1)
     torch.cuda.empty_cache()
+    for context in (1024, 8192):
+        out[f"mla_deepseek_v3_q4_k_ctx{context}_b1"] = mla_workload(torch, capi, synth, 12, context, min(steps, 100), 107)
+        torch.cuda.empty_cache()
     return out
 
 
@@ -305,6 +366,7 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=24, help="distinct weight copies rotated through (cold HBM)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline (0 = skip)")
     ap.add_argument("--extras", type=int, default=1, help="1: also time the other configurations of the path")
+    ap.add_argument("--only", default="", help="with --extras 1: a single extra workload, e.g. mla:1024")
     ap.add_argument("--decode", type=int, default=1, help="1: also run the Qwen3-8B-shaped end-to-end decode leg")
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -415,7 +477,7 @@ def main() -> int:
     del weights, base
     torch.cuda.empty_cache()
     if args.extras:
-        out["workloads"] = extra_workloads(min(steps, 200))
+        out["workloads"] = extra_workloads(min(steps, 200), args.only)
     if args.decode:
         out["decode"] = decode_leg(args.prompt, args.new_tokens, args.cpu_seconds, bool(args.share_layers))
         parity_ok = parity_ok and out["decode"].get("parity_ok", True)

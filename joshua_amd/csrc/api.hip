@@ -1317,11 +1317,21 @@ int mla_forward_dev(jq_mla *m, size_t S, size_t pos, const float *x, float *out,
                        (const float *)m->kv_a_norm, (const float2 *)m->cs, m->lat, m->kpe, (int)nh, (int)nope, (int)rope,
                        (int)lkv, (int)pos, c.rms_eps);
     HIP_TRY(hipGetLastError());
-    constexpr int ST = 4;
-    hipLaunchKernelGGL(jq::mla_absorb_q<ST>, dim3((unsigned)nh, (unsigned)((S + ST - 1) / ST)), dim3(256), 0, s,
-                       (const float *)m->qv, (const float *)m->wkv, m->qabs, (int)S, (int)nh, (int)nope, (int)rope, (int)vh,
-                       (int)lkv);
-    HIP_TRY(hipGetLastError());
+    // one token a workgroup in a decode step, four in a prefill; 16-byte loads when the latent width allows
+    const bool vec4 = lkv % 4 == 0;
+    const unsigned st = S == 1 ? 1 : 4;
+    {
+        const dim3 grid((unsigned)nh, (unsigned)((S + st - 1) / st));
+#define JQ_MLA_ABSORB(ST, CW)                                                                                          \
+    hipLaunchKernelGGL((jq::mla_absorb_q<ST, CW>), grid, dim3(512), 0, s, (const float *)m->qv, (const float *)m->wkv, \
+                       m->qabs, (int)S, (int)nh, (int)nope, (int)rope, (int)vh, (int)lkv)
+        if (vec4 && st == 1) JQ_MLA_ABSORB(1, 4);
+        else if (vec4) JQ_MLA_ABSORB(4, 4);
+        else if (st == 1) JQ_MLA_ABSORB(1, 1);
+        else JQ_MLA_ABSORB(4, 1);
+#undef JQ_MLA_ABSORB
+        HIP_TRY(hipGetLastError());
+    }
     // heads per workgroup, then enough context splits to fill the chip when the call has few tokens
     const int G = nh % 8 == 0 ? 8 : nh % 4 == 0 ? 4 : nh % 2 == 0 ? 2 : 1;
     const size_t wgs = S * (nh / G), total = pos + S;
@@ -1333,9 +1343,22 @@ int mla_forward_dev(jq_mla *m, size_t S, size_t pos, const float *x, float *out,
              : G == 2 ? mla_launch_attention<2>(m, S, pos, (unsigned)n_split, s)
                       : mla_launch_attention<1>(m, S, pos, (unsigned)n_split, s);
     if (rc) return rc;
-    hipLaunchKernelGGL(jq::mla_merge_vproj, dim3((unsigned)nh, (unsigned)S), dim3(256), 0, s, (const float *)m->part,
-                       (const float *)m->wkv, m->ctx, (int)nh, (int)nope, (int)vh, (int)lkv, (int)n_split);
+    // the absorbed queries are spent: their buffer takes the merged latent sums
+    hipLaunchKernelGGL(jq::mla_merge, dim3((unsigned)nh, (unsigned)S), dim3(256), 0, s, (const float *)m->part, m->qabs, (int)nh,
+                       (int)lkv, (int)n_split);
     HIP_TRY(hipGetLastError());
+    {
+        const dim3 grid((unsigned)nh, (unsigned)((vh + 15) / 16), (unsigned)((S + st - 1) / st));
+#define JQ_MLA_VPROJ(ST, VEC)                                                                                          \
+    hipLaunchKernelGGL((jq::mla_vproj<ST, VEC>), grid, dim3(256), 0, s, (const float *)m->qabs, (const float *)m->wkv, \
+                       m->ctx, (int)S, (int)nh, (int)nope, (int)vh, (int)lkv)
+        if (vec4 && st == 1) JQ_MLA_VPROJ(1, true);
+        else if (vec4) JQ_MLA_VPROJ(4, true);
+        else if (st == 1) JQ_MLA_VPROJ(1, false);
+        else JQ_MLA_VPROJ(4, false);
+#undef JQ_MLA_VPROJ
+        HIP_TRY(hipGetLastError());
+    }
     return dispatch_matmul(m->o->type, m->o->dev, m->o->row_bytes, m->ctx, out, S, nh * vh, c.n_embd, s);
 }
 
@@ -1354,6 +1377,7 @@ int jq_mla_create(const jq_mla_config *cfg, const jq_weight *q_or_q_a, const flo
     if (!c.n_embd || !nh || !lkv || !rope || !vh || !c.n_ctx) return fail("jq_mla_create: a dimension is zero");
     if (rope % 2 != 0 || rope > 64) return fail("jq_mla_create: qk_rope_head_dim %zu must be even and at most 64", rope);
     if (lkv > (size_t)jq::MLA_MAX_LKV) return fail("jq_mla_create: kv_lora_rank %zu exceeds %d", lkv, jq::MLA_MAX_LKV);
+    if (lkv % 4 != 0 && lkv > 128) return fail("jq_mla_create: kv_lora_rank %zu above 128 must be a multiple of 4", lkv);
     if (nope > (size_t)jq::MLA_MAX_NOPE) return fail("jq_mla_create: qk_nope_head_dim %zu exceeds %d", nope, jq::MLA_MAX_NOPE);
     if (c.q_lora_rank && (c.q_lora_rank % 4 != 0 || c.q_lora_rank > 8192))
         return fail("jq_mla_create: q_lora_rank %u must be a multiple of 4, at most 8192", c.q_lora_rank);

@@ -13,7 +13,8 @@
 //   mla_absorb_q      q_abs[h] = W_k[h]^T q_nope[h]
 //   mla_attention     scores over the cached latents, running softmax, o_lat[h] = sum p_t c_t, the
 //                     context split over workgroups (partial maximum, sum and vector per split)
-//   mla_merge_vproj   merge the splits, ctx[h] = W_v[h] o_lat[h]
+//   mla_merge         merge the splits into o_lat[h]
+//   mla_vproj         ctx[h] = W_v[h] o_lat[h]
 // around the quantized projections (q, kv_a, o), which run on the matmul kernels.
 #pragma once
 #include "kernels_graph.hpp"
@@ -54,34 +55,61 @@ __global__ __launch_bounds__(64) void mla_rope_latent(float *__restrict__ q, con
 }
 
 // q_abs[s, h, c] = sum_r q[s, h, r] * Wkv[h * (nope + vh) + r, c], r < nope.  grid (n_head, ceil(S / ST)),
-// 256 threads: a thread owns columns c, c + 256, ... and walks the nope rows of its head, whose values
-// for the ST tokens wait in LDS; the rows are read coalesced, once per ST tokens.
-constexpr int MLA_MAX_NOPE = 256;
-template <int ST>
-__global__ __launch_bounds__(256) void mla_absorb_q(const float *__restrict__ q, const float *__restrict__ Wkv,
+// 512 threads: thread (row quarter, column group of CW) walks a quarter of the head's nope rows (the
+// rows are read coalesced, once per ST tokens, whose query values wait in LDS); the four quarters sum
+// through LDS.  CW = 4 (16-byte loads) needs lkv % 4 == 0 and lkv <= 512; CW = 1 any lkv <= 128.
+constexpr int MLA_MAX_NOPE = 256, MLA_MAX_LKV = 512;
+template <int ST, int CW>
+__global__ __launch_bounds__(512) void mla_absorb_q(const float *__restrict__ q, const float *__restrict__ Wkv,
                                                      float *__restrict__ qabs, int S, int n_head, int nope, int rope,
                                                      int vh, int lkv) {
     __shared__ float qs[MLA_MAX_NOPE][ST];
+    __shared__ float red[3][ST][128 * CW];
     const int h = blockIdx.x, s0 = blockIdx.y * ST, qd = nope + rope;
-    for (int e = threadIdx.x; e < nope * ST; e += 256) {
+    for (int e = threadIdx.x; e < nope * ST; e += 512) {
         const int r = e / ST, j = e % ST;
         qs[r][j] = s0 + j < S ? q[((size_t)(s0 + j) * n_head + h) * qd + r] : 0.0f;
     }
     __syncthreads();
     const float *W = Wkv + (size_t)h * (nope + vh) * lkv;
-    for (int c = threadIdx.x; c < lkv; c += 256) {
-        float acc[ST];
+    const int part = threadIdx.x >> 7, c = (threadIdx.x & 127) * CW;
+    const int r0 = part * ((nope + 3) >> 2), r1 = min(nope, r0 + ((nope + 3) >> 2));
+    float acc[ST][CW];
 #pragma unroll
-        for (int j = 0; j < ST; j++) acc[j] = 0.0f;
+    for (int j = 0; j < ST; j++)
+#pragma unroll
+        for (int i = 0; i < CW; i++) acc[j][i] = 0.0f;
+    if (c < lkv) {
 #pragma unroll 8
-        for (int r = 0; r < nope; r++) {
-            const float wv = W[(size_t)r * lkv + c];
+        for (int r = r0; r < r1; r++) {
+            float wv[CW];
+            if constexpr (CW == 4) {
+                const float4 v = *(const float4 *)(W + (size_t)r * lkv + c);
+                wv[0] = v.x, wv[1] = v.y, wv[2] = v.z, wv[3] = v.w;
+            } else {
+                wv[0] = W[(size_t)r * lkv + c];
+            }
 #pragma unroll
-            for (int j = 0; j < ST; j++) acc[j] = fmaf(qs[r][j], wv, acc[j]);
+            for (int j = 0; j < ST; j++)
+#pragma unroll
+                for (int i = 0; i < CW; i++) acc[j][i] = fmaf(qs[r][j], wv[i], acc[j][i]);
         }
+    }
+    if (part > 0) {
 #pragma unroll
         for (int j = 0; j < ST; j++)
-            if (s0 + j < S) qabs[((size_t)(s0 + j) * n_head + h) * lkv + c] = acc[j];
+#pragma unroll
+            for (int i = 0; i < CW; i++) red[part - 1][j][c + i] = acc[j][i];
+    }
+    __syncthreads();
+    if (part == 0 && c < lkv) {
+#pragma unroll
+        for (int j = 0; j < ST; j++)
+#pragma unroll
+            for (int i = 0; i < CW; i++) {
+                const float v = acc[j][i] + red[0][j][c + i] + red[1][j][c + i] + red[2][j][c + i];
+                if (s0 + j < S) qabs[((size_t)(s0 + j) * n_head + h) * lkv + c + i] = v;
+            }
     }
 }
 
@@ -172,14 +200,10 @@ __global__ __launch_bounds__(256) void mla_attention(const float *__restrict__ q
     }
 }
 
-// grid (n_head, S), 256 threads: merges the splits of (s, h) into the normalised latent sum (in LDS)
-// and multiplies by the head's value rows: ctx[s, h * vh + j] = Wkv[h * (nope + vh) + nope + j, :] .
-// o_lat, one wave per row, rows j = wave, wave + 4, ...
-constexpr int MLA_MAX_LKV = 512;
-__global__ __launch_bounds__(256) void mla_merge_vproj(const float *__restrict__ part, const float *__restrict__ Wkv,
-                                                        float *__restrict__ ctx, int n_head, int nope, int vh, int lkv,
-                                                        int n_split) {
-    __shared__ float ol[MLA_MAX_LKV];
+// grid (n_head, S), 256 threads: merges the splits of (s, h) into the normalised latent sum
+// olat[s, h, :] = sum_i f_i o_i / sum_i f_i l_i, f_i = exp(m_i - max m).
+__global__ __launch_bounds__(256) void mla_merge(const float *__restrict__ part, float *__restrict__ olat, int n_head,
+                                                  int lkv, int n_split) {
     __shared__ float f[MLA_SPLIT_MAX];
     __shared__ float Linv;
     const int h = blockIdx.x, s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -196,15 +220,52 @@ __global__ __launch_bounds__(256) void mla_merge_vproj(const float *__restrict__
     for (int c = threadIdx.x; c < lkv; c += 256) {
         float v = 0.0f;
         for (int i = 0; i < n_split; i++) v = fmaf(p[(size_t)i * (lkv + 2) + 2 + c], f[i], v);
-        ol[c] = v * Linv;
+        olat[((size_t)s * n_head + h) * lkv + c] = v * Linv;
+    }
+}
+
+// ctx[s, h * vh + j] = Wkv[h * (nope + vh) + nope + j, :] . olat[s, h, :].  grid (n_head, ceil(vh / 16),
+// ceil(S / ST)), four waves: a wave takes four value rows, read coalesced (16-byte loads when VEC:
+// lkv % 4 == 0) once for the ST tokens whose latent sums wait in LDS.
+template <int ST, bool VEC>
+__global__ __launch_bounds__(256) void mla_vproj(const float *__restrict__ olat, const float *__restrict__ Wkv,
+                                                  float *__restrict__ ctx, int S, int n_head, int nope, int vh, int lkv) {
+    __shared__ __attribute__((aligned(16))) float ol[ST][MLA_MAX_LKV];
+    const int h = blockIdx.x, s0 = blockIdx.z * ST, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int e = threadIdx.x; e < ST * lkv; e += 256) {
+        const int j = e / lkv, c = e % lkv;
+        ol[j][c] = s0 + j < S ? olat[((size_t)(s0 + j) * n_head + h) * lkv + c] : 0.0f;
     }
     __syncthreads();
     const float *W = Wkv + ((size_t)h * (nope + vh) + nope) * lkv;
-    for (int j = wave; j < vh; j += 4) {
-        float acc = 0.0f;
-        for (int c = lane; c < lkv; c += 64) acc = fmaf(W[(size_t)j * lkv + c], ol[c], acc);
-        acc = wave_sum(acc);
-        if (lane == 0) ctx[((size_t)s * n_head + h) * vh + j] = acc;
+#pragma unroll
+    for (int rr = 0; rr < 4; rr++) {
+        const int j = blockIdx.y * 16 + wave * 4 + rr;
+        if (j >= vh) break;  // the whole wave
+        float acc[ST];
+#pragma unroll
+        for (int t = 0; t < ST; t++) acc[t] = 0.0f;
+        if constexpr (VEC) {
+            for (int c = 4 * lane; c < lkv; c += 256) {
+                const float4 wv = *(const float4 *)(W + (size_t)j * lkv + c);
+#pragma unroll
+                for (int t = 0; t < ST; t++) {
+                    const float4 o = *(const float4 *)&ol[t][c];
+                    acc[t] = fmaf(wv.x, o.x, fmaf(wv.y, o.y, fmaf(wv.z, o.z, fmaf(wv.w, o.w, acc[t]))));
+                }
+            }
+        } else {
+            for (int c = lane; c < lkv; c += 64) {
+                const float wv = W[(size_t)j * lkv + c];
+#pragma unroll
+                for (int t = 0; t < ST; t++) acc[t] = fmaf(wv, ol[t][c], acc[t]);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < ST; t++) {
+            const float v = wave_sum(acc[t]);
+            if (lane == 0 && s0 + t < S) ctx[((size_t)(s0 + t) * n_head + h) * vh + j] = v;
+        }
     }
 }
 

@@ -115,6 +115,12 @@ def test_dense_kv_b_and_other_formats():
     ref, dev = build(cfg(), dense_kv_b=True, seed=500)
     x = normal(11, (6, 256))
     assert close(dev.forward(x, 0), ref.forward(x, 0))
+    # the latent width of the reference's own tiny attention (src/quantized_deepseek2.rs:1102-1125)
+    c = cfg(n_embd=32, n_head=2, kv_lora_rank=6, qk_nope=4, qk_rope=4, v_head_dim=16)
+    ref, dev = build(c, dense_kv_b=True, seed=600)
+    x = normal(12, (4, 32))
+    assert close(dev.forward(x[:3], 0), ref.forward(x[:3], 0))
+    assert close(dev.forward(x[3:], 3), ref.forward(x[3:], 3))
 
 
 def test_reset_and_position_checks():
