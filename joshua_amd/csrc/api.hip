@@ -1332,19 +1332,37 @@ int mla_forward_dev(jq_mla *m, size_t S, size_t pos, const float *x, float *out,
 #undef JQ_MLA_ABSORB
         HIP_TRY(hipGetLastError());
     }
-    // heads per workgroup, then enough context splits to fill the chip when the call has few tokens
-    const int G = nh % 8 == 0 ? 8 : nh % 4 == 0 ? 4 : nh % 2 == 0 ? 2 : 1;
-    const size_t wgs = S * (nh / G), total = pos + S;
-    size_t n_split = std::min<size_t>({(1024 + wgs - 1) / wgs, (total + 31) / 32, (size_t)jq::MLA_SPLIT_MAX,
-                                       std::max<size_t>(MLA_PART_SLOTS / S, 1)});
-    n_split = std::max<size_t>(n_split, 1);
-    int rc = G == 8 ? mla_launch_attention<8>(m, S, pos, (unsigned)n_split, s)
-             : G == 4 ? mla_launch_attention<4>(m, S, pos, (unsigned)n_split, s)
-             : G == 2 ? mla_launch_attention<2>(m, S, pos, (unsigned)n_split, s)
-                      : mla_launch_attention<1>(m, S, pos, (unsigned)n_split, s);
-    if (rc) return rc;
+    const size_t total = pos + S;
+    size_t n_split;
+    static const char *mla_env = getenv("JQ_MLA_ATTENTION");  // "valu": never the matrix-core kernel
+    const bool mfma = lkv == jq::MLA_M_LKV && rope == jq::MLA_M_ROPE && nh % 32 == 0 && nope % 4 == 0 && !(mla_env && !strcmp(mla_env, "valu"));
+    if (mfma) {
+        // one workgroup a compute unit when the call has few tokens, tiles of 32 tokens
+        const size_t wgs = S * (nh / 32);
+        n_split = std::min<size_t>({(256 + wgs - 1) / wgs, (total + 31) / 32, (size_t)jq::MLA_SPLIT_MAX,
+                                    std::max<size_t>(MLA_PART_SLOTS / S, 1)});
+        static const char *split_env = getenv("JQ_MLA_SPLIT");
+        if (split_env) n_split = std::min<size_t>(n_split, (size_t)atoi(split_env));
+        n_split = std::max<size_t>(n_split, 1);
+        hipLaunchKernelGGL(jq::mla_attention_mfma, dim3((unsigned)(nh / 32), (unsigned)n_split, (unsigned)S), dim3(512), 0, s,
+                           (const float *)m->qabs, (const float *)m->qv, (const float *)m->lat, (const float *)m->kpe, m->part,
+                           (int)nh, (int)nope, (int)pos, (int)n_split, m->scale);
+        HIP_TRY(hipGetLastError());
+    } else {
+        // heads per workgroup, then enough context splits to fill the chip when the call has few tokens
+        const int G = nh % 8 == 0 ? 8 : nh % 4 == 0 ? 4 : nh % 2 == 0 ? 2 : 1;
+        const size_t wgs = S * (nh / G);
+        n_split = std::min<size_t>({(1024 + wgs - 1) / wgs, (total + 31) / 32, (size_t)jq::MLA_SPLIT_MAX,
+                                    std::max<size_t>(MLA_PART_SLOTS / S, 1)});
+        n_split = std::max<size_t>(n_split, 1);
+        int rc = G == 8 ? mla_launch_attention<8>(m, S, pos, (unsigned)n_split, s)
+                 : G == 4 ? mla_launch_attention<4>(m, S, pos, (unsigned)n_split, s)
+                 : G == 2 ? mla_launch_attention<2>(m, S, pos, (unsigned)n_split, s)
+                          : mla_launch_attention<1>(m, S, pos, (unsigned)n_split, s);
+        if (rc) return rc;
+    }
     // the absorbed queries are spent: their buffer takes the merged latent sums
-    hipLaunchKernelGGL(jq::mla_merge, dim3((unsigned)nh, (unsigned)S), dim3(256), 0, s, (const float *)m->part, m->qabs, (int)nh,
+    hipLaunchKernelGGL(jq::mla_merge, dim3((unsigned)nh, (unsigned)S, (unsigned)((lkv + 127) / 128)), dim3(128), 0, s, (const float *)m->part, m->qabs, (int)nh,
                        (int)lkv, (int)n_split);
     HIP_TRY(hipGetLastError());
     {

@@ -200,9 +200,131 @@ __global__ __launch_bounds__(256) void mla_attention(const float *__restrict__ q
     }
 }
 
-// grid (n_head, S), 256 threads: merges the splits of (s, h) into the normalised latent sum
-// olat[s, h, :] = sum_i f_i o_i / sum_i f_i l_i, f_i = exp(m_i - max m).
-__global__ __launch_bounds__(256) void mla_merge(const float *__restrict__ part, float *__restrict__ olat, int n_head,
+// The same scores and latent sums on the f32 matrix cores (v_mfma_f32_32x32x2_f32: exact f32 products,
+// f32 sums), for the geometry every DeepSeek MLA model has: 512 latent + 64 rope elements, heads in
+// groups of 32.  grid (n_head / 32, n_split, S), eight waves.  A tile is 32 heads x 32 tokens; the
+// tokens' rows [latent | rope key] (576 floats) wait in LDS.
+//   scores  = Q[32 x 576] . C^T[576 x 32]: wave w multiplies columns 72 w .. 72 w + 71 (36 steps of 2;
+//             its slice of Q stays in 36 registers), the eight partial tiles sum through LDS;
+//   softmax: 16 threads a head, two tokens each, running maximum and sum in registers;
+//   o_lat  += P[32 x 32] . C[32 x 512]: wave w owns latent columns 64 w .. 64 w + 63 (two tiles of 32,
+//             32 accumulator registers), 16 steps of 2 tokens.
+// The next tile's rows are fetched into registers while a tile is worked on.  Output as mla_attention.
+constexpr int MLA_M_LKV = 512, MLA_M_ROPE = 64, MLA_M_KT = MLA_M_LKV + MLA_M_ROPE, MLA_M_STRIDE = MLA_M_KT + 4;
+typedef float mla_f16v __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(512) void mla_attention_mfma(const float *__restrict__ qabs, const float *__restrict__ q,
+                                                           const float *__restrict__ lat, const float *__restrict__ kpe,
+                                                           float *__restrict__ part, int n_head, int nope, int pos0,
+                                                           int n_split, float scale) {
+    __shared__ __attribute__((aligned(16))) float ct[32][MLA_M_STRIDE];
+    __shared__ float sp[8][32][33];
+    __shared__ float ps[32][33];
+    __shared__ __attribute__((aligned(16))) float al[32];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, lk = lane >> 5;
+    const int h0 = blockIdx.x * 32, split = blockIdx.y, s = blockIdx.z;
+    const int T = pos0 + s + 1, chunk = (T + n_split - 1) / n_split;
+    const int t0 = split * chunk, t1 = min(T, t0 + chunk);
+
+    // 32 rows (tokens of a tile, or the heads' queries) x 144 pieces of 16 bytes (128 latent, 16 rope) = 9 a thread
+    float4 pre[9];
+    auto load_tile = [&](int tb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 9; u++) {
+            const int idx = tid + 512 * u, tok = idx / 144, f = idx % 144, t = tb + tok;
+            if (t < t1) pre[u] = f < 128 ? *(const float4 *)(lat + (size_t)t * MLA_M_LKV + 4 * f)
+                                         : *(const float4 *)(kpe + (size_t)t * MLA_M_ROPE + 4 * (f - 128));
+            else pre[u] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    };
+    if (t0 < t1) load_tile(t0);
+    // this wave's slice of the 32 heads' queries, element 72 wave + 2 ks + lk of head li, by way of LDS
+    // (rows [absorbed query | rotated rope query] read whole, then picked apart)
+    float qreg[36];
+    {
+#pragma unroll
+        for (int u = 0; u < 9; u++) {
+            const int idx = tid + 512 * u, i = idx / 144, f = idx % 144;
+            const size_t row = (size_t)s * n_head + h0 + i;
+            *(float4 *)&ct[i][4 * f] = f < 128 ? *(const float4 *)(qabs + row * MLA_M_LKV + 4 * f)
+                                               : *(const float4 *)(q + row * (nope + MLA_M_ROPE) + nope + 4 * (f - 128));
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < 36; ks++) qreg[ks] = ct[li][72 * wave + 2 * ks + lk];
+        __syncthreads();
+    }
+    mla_f16v o[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[nt][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;  // of head tid / 16, the same in its 16 threads
+
+    for (int tb = t0; tb < t1; tb += 32) {
+        if (tb > t0) __syncthreads();  // every wave is done with the rows of the tile before
+#pragma unroll
+        for (int u = 0; u < 9; u++) {
+            const int idx = tid + 512 * u, tok = idx / 144, f = idx % 144;
+            *(float4 *)&ct[tok][4 * f] = pre[u];
+        }
+        __syncthreads();
+        if (tb + 32 < t1) load_tile(tb + 32);
+
+        mla_f16v sc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sc[r] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 36; ks++)
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[ks], ct[li][72 * wave + 2 * ks + lk], sc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; r++) sp[wave][8 * (r >> 2) + 4 * lk + (r & 3)][li] = sc[r];  // row = head, column = token
+        __syncthreads();
+        {
+            const int i = tid >> 4, j = 2 * (tid & 15);
+            float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 8; w++) s0 += sp[w][i][j], s1 += sp[w][i][j + 1];
+            s0 = tb + j < t1 ? s0 * scale : -INFINITY;
+            s1 = tb + j + 1 < t1 ? s1 * scale : -INFINITY;
+            const float mn = fmaxf(m_run, max_row16(fmaxf(s0, s1)));  // finite: token tb is inside the split
+            const float p0 = __expf(s0 - mn), p1 = __expf(s1 - mn), a = __expf(m_run - mn);
+            l_run = fmaf(l_run, a, sum_row16(p0 + p1));
+            m_run = mn;
+            ps[i][j] = p0, ps[i][j + 1] = p1;
+            if ((tid & 15) == 0) al[i] = a;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const float4 a = *(const float4 *)&al[8 * b + 4 * lk];
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++) o[nt][4 * b] *= a.x, o[nt][4 * b + 1] *= a.y, o[nt][4 * b + 2] *= a.z, o[nt][4 * b + 3] *= a.w;
+        }
+#pragma unroll
+        for (int kk = 0; kk < 16; kk++) {
+            const float pa = ps[li][2 * kk + lk];
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+                o[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa, ct[2 * kk + lk][64 * wave + 32 * nt + li], o[nt], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int i = 8 * (r >> 2) + 4 * lk + (r & 3);
+            part[(((size_t)s * n_head + h0 + i) * n_split + split) * (MLA_M_LKV + 2) + 2 + 64 * wave + 32 * nt + li] = o[nt][r];
+        }
+    if ((tid & 15) == 0) {
+        float *p = part + (((size_t)s * n_head + h0 + (tid >> 4)) * n_split + split) * (MLA_M_LKV + 2);
+        p[0] = m_run, p[1] = l_run;
+    }
+}
+
+// grid (n_head, S, ceil(lkv / 128)), 128 threads, one latent column each: merges the splits of (s, h)
+// into the normalised latent sum olat[s, h, :] = sum_i f_i o_i / sum_i f_i l_i, f_i = exp(m_i - max m).
+__global__ __launch_bounds__(128) void mla_merge(const float *__restrict__ part, float *__restrict__ olat, int n_head,
                                                   int lkv, int n_split) {
     __shared__ float f[MLA_SPLIT_MAX];
     __shared__ float Linv;
@@ -217,11 +339,12 @@ __global__ __launch_bounds__(256) void mla_merge(const float *__restrict__ part,
         if (lane == 0) Linv = 1.0f / L;
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < lkv; c += 256) {
-        float v = 0.0f;
-        for (int i = 0; i < n_split; i++) v = fmaf(p[(size_t)i * (lkv + 2) + 2 + c], f[i], v);
-        olat[((size_t)s * n_head + h) * lkv + c] = v * Linv;
-    }
+    const int c = blockIdx.z * 128 + threadIdx.x;
+    if (c >= lkv) return;
+    float v = 0.0f;
+#pragma unroll 8
+    for (int i = 0; i < n_split; i++) v = fmaf(p[(size_t)i * (lkv + 2) + 2 + c], f[i], v);
+    olat[((size_t)s * n_head + h) * lkv + c] = v * Linv;
 }
 
 // ctx[s, h * vh + j] = Wkv[h * (nope + vh) + nope + j, :] . olat[s, h, :].  grid (n_head, ceil(vh / 16),

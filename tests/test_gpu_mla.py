@@ -106,6 +106,19 @@ def test_long_context_is_split_over_workgroups():
     assert close(dev.forward(x[602:650], 602), ref.forward(x[602:650], 602))  # a second prefill chunk at an offset
 
 
+def test_matrix_core_attention_for_the_deepseek_geometry():
+    """512 latent + 64 rope elements and heads in groups of 32 run on the f32 matrix cores: tiles of 32
+    tokens, several tiles a workgroup in the prefill, several context splits in the decode steps, a
+    ragged last tile."""
+    c = cfg(n_embd=256, n_head=64, kv_lora_rank=512, qk_nope=32, qk_rope=64, v_head_dim=32, context_length=260)
+    ref, dev = build(c, seed=700)
+    x = normal(14, (250, c["n_embd"])) * np.float32(2.0)
+    assert close(dev.forward(x[:150], 0), ref.forward(x[:150], 0))
+    for p in (150, 151, 152):
+        assert close(dev.forward(x[p:p + 1], p), ref.forward(x[p:p + 1], p))
+    assert close(dev.forward(x[153:250], 153), ref.forward(x[153:250], 153))
+
+
 def test_dense_kv_b_and_other_formats():
     c = cfg(kv_lora_rank=256, n_embd=256, v_head_dim=64)
     for qtype in (capi.Q4_K, capi.Q6_K):
