@@ -27,6 +27,7 @@
 #include "kernels_dot4_q8.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
+#include "kernels_mfma_q4k_rows16.hpp"
 #include "kernels_valu.hpp"
 #include "kernels_mfma_decoded.hpp"
 
@@ -368,6 +369,71 @@ void launch_q4k_acts_prep(const float *X, size_t rows, size_t k, uint8_t *out, h
     hipLaunchKernelGGL(jq::q4k_acts_prep, dim3((unsigned)((units + 7) / 8)), dim3(256), 0, s, X, (int)rows, (int)k, out);
 }
 
+// Device memory for what one call's launches hand to each other (prepared activation operands), on
+// stream s.  Requests up to SCRATCH_KEEP bytes are served from one allocation per (device, stream), made
+// at first use, grown when a call needs more and kept until the process ends: the launches of a stream
+// run in order, so consecutive calls can share it, and a call pays no allocator round trip
+// (hipMallocAsync with hipFreeAsync takes some 18 us of host time a call, more than the kernels of a
+// small matmul take on the device).  The holder keeps that allocation's lock until it goes out of
+// scope, after the call's last launch is enqueued, so host threads that share a stream enqueue their
+// calls one after the other.  Larger requests are stream-ordered allocations, freed behind the call's
+// launches.  First use on a stream allocates, and growing waits for the stream: neither is possible
+// while the stream is being captured, so a caller warms a stream up before capturing it.
+constexpr size_t SCRATCH_KEEP = 64u << 20;
+
+struct StreamBuffer {
+    std::mutex mu;
+    uint8_t *ptr = nullptr;
+    size_t bytes = 0;
+};
+
+class CallScratch {
+    std::unique_lock<std::mutex> lock_;
+    hipStream_t stream_ = nullptr;
+    uint8_t *transient_ = nullptr;
+
+public:
+    CallScratch() = default;
+    CallScratch(const CallScratch &) = delete;
+    CallScratch &operator=(const CallScratch &) = delete;
+    ~CallScratch() {
+        if (transient_) (void)hipFreeAsync(transient_, stream_);
+    }
+    hipError_t get(size_t bytes, hipStream_t s, uint8_t **out) {
+        stream_ = s;
+        if (bytes > SCRATCH_KEEP) {
+            hipError_t e = hipMallocAsync((void **)&transient_, bytes, s);
+            *out = transient_;
+            return e;
+        }
+        static std::mutex table_mu;
+        static std::map<std::pair<int, hipStream_t>, std::unique_ptr<StreamBuffer>> table;
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        StreamBuffer *b;
+        {
+            std::lock_guard<std::mutex> g(table_mu);
+            auto &slot = table[{dev, s}];
+            if (!slot) slot.reset(new StreamBuffer);
+            b = slot.get();
+        }
+        lock_ = std::unique_lock<std::mutex>(b->mu);
+        if (b->bytes < bytes) {
+            if (b->ptr) {
+                if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
+                if ((e = hipFree(b->ptr)) != hipSuccess) return e;
+                b->ptr = nullptr, b->bytes = 0;
+            }
+            const size_t want = std::max<size_t>((bytes + 0xFFFFF) & ~(size_t)0xFFFFF, 1u << 20);
+            if ((e = hipMalloc((void **)&b->ptr, want)) != hipSuccess) return e;
+            b->bytes = want;
+        }
+        *out = b->ptr;
+        return hipSuccess;
+    }
+};
+
 // Workgroups of the LDS-ring MFMA kernel that fit a compute unit (LDS and the 16 waves of a SIMD group).
 constexpr int ring_wgs_per_cu(int maxnb) { return maxnb == 16 ? 1 : maxnb == 8 ? 2 : 4; }
 
@@ -385,9 +451,10 @@ int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float 
     static const char *genv = getenv("JQ_Q4K_RING_GRID");
     const size_t per = (tiles + slots - 1) / slots;
     const unsigned grid = genv ? (unsigned)std::max(atoi(genv), 1) : (unsigned)((tiles + per - 1) / per);
-    // the activations as MFMA operand records, in a stream-ordered scratch allocation
+    // the activations as MFMA operand records, in the call scratch of the stream
+    CallScratch scratch;
     uint8_t *acts = nullptr;
-    HIP_TRY(hipMallocAsync((void **)&acts, m * nb * jq::QS_REC, s));
+    HIP_TRY(scratch.get(m * nb * jq::QS_REC, s, &acts));
     launch_q4k_acts_prep(X, m, k, acts, s);
 #define JQ_RING(MAXNB)                                                                                              \
     hipLaunchKernelGGL((jq::q4k_ring_mfma<MAXNB, false, false>), dim3(grid), dim3(64 * (unsigned)nb), 0, s, W, nullptr, \
@@ -396,14 +463,35 @@ int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float 
     else if (maxnb == 8) JQ_RING(8);
     else JQ_RING(4);
 #undef JQ_RING
-    hipError_t launched = hipGetLastError();
-    HIP_TRY(hipFreeAsync(acts, s));
-    HIP_TRY(launched);
+    HIP_TRY(hipGetLastError());
     return 0;
 }
 
-// Q4_K with more than 16 activation rows: prepare the fixed-point activation planes in a
-// stream-ordered scratch allocation, then the MFMA GEMM.
+// Q4_K, 2..16 activation rows, contiguous rows of exactly 16 super-blocks: the int8 matrix-core kernel on the
+// one-row GEMV's weight stream, its operands prepared by one small launch into the call scratch of the stream.
+// Returns -1 when the shape is outside its reach.
+int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                        hipStream_t s) {
+    static const char *off = getenv("JQ_Q4K_NO_ROWS16");
+    static const char *min_env = getenv("JQ_Q4K_ROWS16_MIN_N");
+    static const size_t min_n = min_env ? (size_t)atoll(min_env) : 1024;
+    if (off || m < 2 || m > 16 || k != 4096 || row_bytes != (size_t)jq::QD_ROW || n < min_n || n > 0x7FFFFFF0ull ||
+        ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
+        return -1;
+    const size_t tiles = (n + 15) / 16, rounds = (tiles + 255) / 256;
+    static const char *genv = getenv("JQ_Q4K_ROWS16_GRID");
+    const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)std::max(atoi(genv), 1) : (tiles + rounds - 1) / rounds);
+    CallScratch scratch;
+    uint8_t *acts = nullptr;
+    HIP_TRY(scratch.get(16 * (size_t)jq::QM_REC, s, &acts));
+    hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, 16), dim3(64), 0, s, X, (int)m, (int)k, acts);
+    hipLaunchKernelGGL(jq::q4k_rows16_mfma, dim3(grid), dim3(1024), 0, s, W, (const uint8_t *)acts, Y, (int)m, (int)n, (int)grid);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// Q4_K with more than 16 activation rows: prepare the fixed-point activation planes in the
+// call scratch of the stream, then the MFMA GEMM.
 int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
                       hipStream_t s) {
     constexpr size_t MT = jq::QG_MT;
@@ -412,8 +500,9 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
     const size_t plane_bytes = up(m_pad * k * 2 * sizeof(uint16_t)), min_bytes = up(m_pad * nb * 64);
     const size_t m_tiles = m_pad / MT, n_tiles = (n + jq::QG_NT - 1) / jq::QG_NT, total = m_tiles * n_tiles;
     if (total > 0x0FFFFFFFull) return fail("q4k gemm: %zu x %zu tiles exceed the grid limit", m_tiles, n_tiles);
+    CallScratch scratch;
     uint8_t *buf = nullptr;
-    HIP_TRY(hipMallocAsync((void **)&buf, plane_bytes + min_bytes, s));
+    HIP_TRY(scratch.get(plane_bytes + min_bytes, s, &buf));
     jq::Q4kGemmActs a;
     a.planes = (_Float16 *)buf;
     a.mins = (_Float16 *)(buf + plane_bytes);
@@ -428,13 +517,12 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
     hipLaunchKernelGGL(jq::q4k_gemm_mfma, dim3(grid), dim3(512), 0, s, W, row_bytes, a, Y, (int)m, (int)m_pad, (int)k, (int)n,
                        (int)m_tiles, (int)total);
     hipError_t e = hipGetLastError();
-    HIP_TRY(hipFreeAsync(buf, s));
     if (e != hipSuccess) return fail("q4k gemm launch: %s", hipGetErrorString(e));
     return 0;
 }
 
-// Any format, more than 16 activation rows, k a multiple of 256: activations as two f16 planes in a
-// stream-ordered scratch allocation, then the MFMA GEMM over decoded weights.  Returns -1 when the
+// Any format, more than 16 activation rows, k a multiple of 256: activations as two f16 planes in the
+// call scratch of the stream, then the MFMA GEMM over decoded weights.  Returns -1 when the
 // shape is outside its reach.
 template <class Q>
 int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
@@ -444,16 +532,15 @@ int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, floa
     const size_t m_pad = (m + jq::GD_MT - 1) / jq::GD_MT * jq::GD_MT, nc = k / jq::GD_KC;
     auto up = [](size_t v) { return (v + 255) / 256 * 256; };
     const size_t plane = up(m_pad * k * sizeof(_Float16)), sbytes = up(m_pad * nc * sizeof(float));
+    CallScratch scratch;
     uint8_t *buf = nullptr;
-    HIP_TRY(hipMallocAsync((void **)&buf, 2 * plane + sbytes, s));
+    HIP_TRY(scratch.get(2 * plane + sbytes, s, &buf));
     jq::ActsF16 a{(_Float16 *)buf, (_Float16 *)(buf + plane), (float *)(buf + 2 * plane)};
     hipLaunchKernelGGL(jq::acts_f16_prep, dim3((unsigned)((m_pad * nc * 64 + 255) / 256)), dim3(256), 0, s, X, (int)m,
                        (int)m_pad, (int)k, a);
     hipLaunchKernelGGL(jq::gemm_decoded_mfma<Q>, dim3((unsigned)((n + jq::GD_NT - 1) / jq::GD_NT), (unsigned)(m_pad / jq::GD_MT)),
                        dim3(256), 0, s, W, row_bytes, a, Y, (int)m, (int)k, (int)n);
-    hipError_t launched = hipGetLastError();
-    HIP_TRY(hipFreeAsync(buf, s));
-    HIP_TRY(launched);
+    HIP_TRY(hipGetLastError());
     return 0;
 }
 
@@ -488,6 +575,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     // whose time hardly depends on the row count
     // 3 to 16 rows against a very long matrix (a vocabulary projection): the LDS-ring kernel, whose
     // two launches and scratch allocation only pay off from some 100 us of streaming on
+    if (type == JQ_TYPE_Q4_K && m >= 2 && m <= 16) {
+        const int rc = dispatch_q4k_rows16(W, row_bytes, X, Y, m, k, n, s);
+        if (rc >= 0) return rc;
+    }
     static const char *ring_min_env = getenv("JQ_Q4K_RING_MIN_N");
     static const size_t ring_min_n = ring_min_env ? (size_t)atoll(ring_min_env) : 32768;
     if (type == JQ_TYPE_Q4_K && m > 2 && m <= Q4K_MFMA_MAX_M && n >= ring_min_n) {

@@ -359,6 +359,38 @@ def test_q4k_dot4_gemv_long_rows_integer_dot_products_are_bit_exact(k, n):
     assert np.array_equal(got[0], want.astype(np.float32))
 
 
+@pytest.mark.parametrize("m,n", [(2, 1024), (5, 1030), (16, 14336), (16, 4097), (3, 5000), (8, 8190), (16, 4112)])
+def test_q4k_few_rows_over_4096_wide_rows(m, n):
+    """2..16 activation rows over rows of 4096, 1024 weight rows or more: the int8 matrix-core kernel on
+    the one-row kernel's weight stream; row counts with a partial last tile, one and several tiles a
+    workgroup; wide-ranging activations, a zero row, a non-finite activation."""
+    k = 4096
+    blocks = make_blocks(capi.Q4_K, n, k, 61 + n)
+    rng = np.random.default_rng(n + m)
+    lhs = synth.normal(62 + n, (m, k))
+    lhs[0] *= (10.0 ** rng.integers(-5, 2, size=k // 32)).repeat(32).astype(np.float32)
+    lhs[m - 1, 1000:3000] = 0.0
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    got = w.matmul_t(m, lhs, np.full(m * n, 55.5, np.float32))
+    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True))
+    one = w.matmul_t(1, lhs[1:2])
+    assert close(one, got[1:2])
+    lhs[1, 4000] = np.inf
+    bad = w.matmul_t(m, lhs)
+    assert np.isnan(bad[1]).all() and np.array_equal(bad[0], got[0])
+
+
+@pytest.mark.parametrize("m,n", [(2, 1024), (16, 1040), (7, 4500)])
+def test_q4k_few_rows_over_4096_wide_rows_integer_dot_products_are_bit_exact(m, n):
+    k = 4096
+    blocks, q, x = q4k_integer_case(n, k, 13 + m, group=32, big_value=32639, small=1000)
+    xs = np.stack([np.roll(x, 32 * i) * (1 if i % 2 == 0 else -1) for i in range(m)])
+    want = xs @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, xs.astype(np.float32))
+    assert np.array_equal(got, want.astype(np.float32))
+
+
 @pytest.mark.parametrize("m", [17, 64, 200])
 def test_q4k_gemm_integer_dot_products_are_bit_exact(m):
     """The same construction for the MFMA GEMM (m > 16): its activation range is 4193279
