@@ -467,31 +467,72 @@ int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
-// Q4_K, 2..16 activation rows, contiguous rows of exactly 16 super-blocks: the int8 matrix-core kernel on the
-// one-row GEMV's weight stream, its operands prepared by one small launch into the call scratch of the stream.
-// Returns -1 when the shape is outside its reach.
+// How many runs of super-blocks a GEMM of `total` workgroup tiles splits its k dimension into.  One tile
+// list fills the 256 compute units only from 256 tiles on; a list of 32 tiles split eight ways does, at the
+// price of writing and re-reading the partial sums.  Estimated per candidate from the measured step time of
+// a workgroup (us per super-block, plus its start and end) and ~3 TB/s for the partial sums; the choice
+// depends on the shape only, so a shape always gets the same order of additions.
+int gemm_k_splits(size_t total, size_t nb, size_t m, size_t n, double us_per_block, const char *env,
+                  double *estimate_us = nullptr) {
+    if (env && !estimate_us) return (int)std::min<size_t>(std::max(atoi(env), 1), nb);
+    int best = 1;
+    double best_us = 0.0;
+    for (size_t sp = 1; sp <= std::min<size_t>(nb, 16); sp++) {
+        const double rounds = (double)((total * sp + 255) / 256);
+        const double wg_us = 3.0 + us_per_block * (double)((nb + sp - 1) / sp);
+        const double sum_us = sp == 1 ? 0.0 : 3.0 + (double)(2 * sp + 1) * (double)(m * n) * 4.0 / 3.0e6;
+        const double us = rounds * wg_us + sum_us;
+        if (sp == 1 || us < best_us * 0.95) best = (int)sp, best_us = us;
+    }
+    if (estimate_us) *estimate_us = best_us;
+    return best;
+}
+
+// Estimated time of the Q4_K MFMA GEMM (dispatch_q4k_gemm) on an m x k by n x k product, in us.
+double q4k_gemm_estimate_us(size_t m, size_t k, size_t n) {
+    const size_t m_tiles = (m + jq::QG_MT - 1) / jq::QG_MT, n_tiles = (n + jq::QG_NT - 1) / jq::QG_NT;
+    double us = 0.0;
+    gemm_k_splits(m_tiles * n_tiles, k / 256, m, n, 6.0, nullptr, &us);
+    return us;
+}
+
+// Q4_K, two activation rows or more, contiguous rows of exactly 16 super-blocks: the int8 matrix-core kernel
+// on the one-row GEMV's weight stream, once per group of 16 activation rows (a matrix of this size stays
+// in the last-level cache between the passes), its operands prepared by one small launch into the call
+// scratch of the stream.  Beyond 16 rows it runs while its estimated time (a pass costs ~4.3 us plus
+// 0.53 us per 1024 weight rows) stays below the MFMA GEMM's.  Returns -1 when the shape is outside its reach.
+constexpr size_t Q4K_ROWS16_MAX_M = 256;
+
 int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
                         hipStream_t s) {
     static const char *off = getenv("JQ_Q4K_NO_ROWS16");
     static const char *min_env = getenv("JQ_Q4K_ROWS16_MIN_N");
     static const size_t min_n = min_env ? (size_t)atoll(min_env) : 1024;
-    if (off || m < 2 || m > 16 || k != 4096 || row_bytes != (size_t)jq::QD_ROW || n < min_n || n > 0x7FFFFFF0ull ||
+    static const char *max_env = getenv("JQ_Q4K_ROWS16_MAX_M");
+    static const size_t max_m = max_env ? std::min<size_t>((size_t)atoll(max_env), 1024) : Q4K_ROWS16_MAX_M;
+    if (off || m < 2 || m > max_m || k != 4096 || row_bytes != (size_t)jq::QD_ROW || n < min_n || n > 0x7FFFFFF0ull ||
         ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
         return -1;
-    const size_t tiles = (n + 15) / 16, rounds = (tiles + 255) / 256;
+    const size_t tiles = (n + 15) / 16, rounds = (tiles + 255) / 256, groups = (m + 15) / 16;
+    if (groups > 1 && !max_env && 3.0 + (double)groups * (4.3 + 0.527 * (double)n / 1024.0) >= q4k_gemm_estimate_us(m, k, n))
+        return -1;
     static const char *genv = getenv("JQ_Q4K_ROWS16_GRID");
     const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)std::max(atoi(genv), 1) : (tiles + rounds - 1) / rounds);
     CallScratch scratch;
     uint8_t *acts = nullptr;
-    HIP_TRY(scratch.get(16 * (size_t)jq::QM_REC, s, &acts));
-    hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, 16), dim3(64), 0, s, X, (int)m, (int)k, acts);
-    hipLaunchKernelGGL(jq::q4k_rows16_mfma, dim3(grid), dim3(1024), 0, s, W, (const uint8_t *)acts, Y, (int)m, (int)n, (int)grid);
+    const size_t group_bytes = 16 * (size_t)jq::QM_REC;
+    HIP_TRY(scratch.get(groups * group_bytes, s, &acts));
+    hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, 16, (unsigned)groups), dim3(64), 0, s, X, (int)m, (int)k, acts);
+    for (size_t g = 0; g < groups; g++)
+        hipLaunchKernelGGL(jq::q4k_rows16_mfma, dim3(grid), dim3(1024), 0, s, W, (const uint8_t *)(acts + g * group_bytes),
+                           Y + 16 * g * n, (int)std::min<size_t>(16, m - 16 * g), (int)n, (int)grid);
     HIP_TRY(hipGetLastError());
     return 0;
 }
 
 // Q4_K with more than 16 activation rows: prepare the fixed-point activation planes in the
-// call scratch of the stream, then the MFMA GEMM.
+// call scratch of the stream, then the MFMA GEMM, split over k when its tiles alone would leave
+// compute units idle.
 int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
                       hipStream_t s) {
     constexpr size_t MT = jq::QG_MT;
@@ -499,23 +540,30 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
     auto up = [](size_t v) { return (v + 255) / 256 * 256; };
     const size_t plane_bytes = up(m_pad * k * 2 * sizeof(uint16_t)), min_bytes = up(m_pad * nb * 64);
     const size_t m_tiles = m_pad / MT, n_tiles = (n + jq::QG_NT - 1) / jq::QG_NT, total = m_tiles * n_tiles;
-    if (total > 0x0FFFFFFFull) return fail("q4k gemm: %zu x %zu tiles exceed the grid limit", m_tiles, n_tiles);
-    CallScratch scratch;
-    uint8_t *buf = nullptr;
-    HIP_TRY(scratch.get(plane_bytes + min_bytes, s, &buf));
-    jq::Q4kGemmActs a;
-    a.planes = (_Float16 *)buf;
-    a.mins = (_Float16 *)(buf + plane_bytes);
-    const size_t units = m_pad * nb;
-    hipLaunchKernelGGL(jq::q4k_gemm_prep, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, X, (int)m, (int)m_pad, (int)k, a);
     // 8 XCDs x the longest per-XCD work list (see the tile order at the top of the kernel)
     size_t per_xcd;
     if (m_tiles >= 8) per_xcd = (m_tiles + 7) / 8 * n_tiles;
     else if (8 % m_tiles != 0) per_xcd = (total + 7) / 8;
     else per_xcd = (n_tiles + 8 / m_tiles - 1) / (8 / m_tiles);
-    const unsigned grid = (unsigned)(8 * per_xcd);
-    hipLaunchKernelGGL(jq::q4k_gemm_mfma, dim3(grid), dim3(512), 0, s, W, row_bytes, a, Y, (int)m, (int)m_pad, (int)k, (int)n,
-                       (int)m_tiles, (int)total);
+    const size_t base_grid = 8 * per_xcd;
+    static const char *split_env = getenv("JQ_Q4K_GEMM_SPLITS");
+    const size_t splits = m * n / 1024 < 0x7FFFFFFFull ? (size_t)gemm_k_splits(total, nb, m, n, 6.0, split_env) : 1;
+    if (base_grid * splits > 0x0FFFFFFFull) return fail("q4k gemm: %zu x %zu tiles exceed the grid limit", m_tiles, n_tiles);
+    const size_t part_bytes = splits > 1 ? splits * m * n * sizeof(float) : 0;
+    CallScratch scratch;
+    uint8_t *buf = nullptr;
+    HIP_TRY(scratch.get(plane_bytes + min_bytes + part_bytes, s, &buf));
+    jq::Q4kGemmActs a;
+    a.planes = (_Float16 *)buf;
+    a.mins = (_Float16 *)(buf + plane_bytes);
+    float *parts = (float *)(buf + plane_bytes + min_bytes);
+    const size_t units = m_pad * nb;
+    hipLaunchKernelGGL(jq::q4k_gemm_prep, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, X, (int)m, (int)m_pad, (int)k, a);
+    hipLaunchKernelGGL(jq::q4k_gemm_mfma, dim3((unsigned)(base_grid * splits)), dim3(512), 0, s, W, row_bytes, a,
+                       splits > 1 ? parts : Y, (int)m, (int)m_pad, (int)k, (int)n, (int)m_tiles, (int)total, (int)splits,
+                       (int)base_grid, splits > 1 ? m * n : (size_t)0);
+    if (splits > 1)
+        hipLaunchKernelGGL(jq::splitk_sum, dim3((unsigned)((m * n + 1023) / 1024)), dim3(256), 0, s, parts, Y, m * n, (int)splits);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("q4k gemm launch: %s", hipGetErrorString(e));
     return 0;
@@ -571,11 +619,12 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         const int rc = dispatch_q8_0_dot4(W, row_bytes, X, Y, k, n, s);
         if (rc >= 0) return rc;
     }
-    // one or two activation rows: the int8 GEMV below is faster; from three on the streaming kernel,
-    // whose time hardly depends on the row count
-    // 3 to 16 rows against a very long matrix (a vocabulary projection): the LDS-ring kernel, whose
-    // two launches and scratch allocation only pay off from some 100 us of streaming on
-    if (type == JQ_TYPE_Q4_K && m >= 2 && m <= 16) {
+    // Q4_K with a few activation rows.  Rows of 4096, 1024 weight rows or more: the int8 matrix-core kernel
+    // on the one-row kernel's weight stream, in passes of 16 activation rows.  Other row lengths: one or two
+    // rows on the int8 GEMV further down; from three on the streaming kernel, whose time hardly depends on
+    // the row count, or, against a very long matrix (a vocabulary projection), the LDS-ring kernel, whose
+    // second launch only pays off from some 100 us of streaming on.
+    if (type == JQ_TYPE_Q4_K && m >= 2) {
         const int rc = dispatch_q4k_rows16(W, row_bytes, X, Y, m, k, n, s);
         if (rc >= 0) return rc;
     }

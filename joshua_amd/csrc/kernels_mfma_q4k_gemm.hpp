@@ -174,9 +174,15 @@ constexpr int QG_B_U4 = 2 * 2 * QG_MT16 * 64;  // of a B chunk: [kstep][plane][m
 // Every global read of the main loop is an asynchronous global->LDS load (no register in
 // between), ordered and awaited by hand: the vmcnt arithmetic in step() relies on each
 // wave issuing exactly the operations listed there, youngest last.
+//
+// Split over k: the grid is `splits` copies of the tile list (base_grid workgroups each, a multiple of 8
+// so that the XCD of a workgroup does not change); copy i takes the i-th of `splits` contiguous runs of
+// super-blocks and stores its m x n partial sums at Y + i * split_stride (splitk_sum adds them up in a
+// fixed order).  With splits == 1 and split_stride == 0, Y is the result.
 __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__ W, size_t row_bytes, Q4kGemmActs acts,
                                                       float *__restrict__ Y, int m, int m_pad, int k, int n,
-                                                      int m_tiles, int total_tiles) {
+                                                      int m_tiles, int total_tiles, int splits, int base_grid,
+                                                      size_t split_stride) {
     constexpr int MI = QG_MI, MT = QG_MT, MT16 = QG_MT16;
     static_assert(MT16 == 8, "one activation tile of mins per wave");
     // Rings of 64-k chunks.  The slots are separate arrays so that the compiler can tell a
@@ -193,7 +199,8 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
     // L2.  The activation planes are the heavy operand (4 bytes per element against 0.5 for the
     // weights), so an XCD works on as few activation tiles as possible and keeps them in its L2,
     // while a weight tile is fetched by the XCDs that share it.
-    const int xcd = (int)(blockIdx.x & 7), slot = (int)(blockIdx.x >> 3);
+    const int split = (int)blockIdx.x / base_grid, bid = (int)blockIdx.x - split * base_grid;
+    const int xcd = bid & 7, slot = bid >> 3;
     int mt, nt;
     if (m_tiles >= 8 || (8 % m_tiles) != 0) {
         // activation tiles xcd, xcd + 8, ... (or plain round-robin when the counts do not divide)
@@ -216,20 +223,22 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wn = wave & 1, wm = wave >> 1;
-    const int nb = k >> 8, nch = k >> 6;
+    const int nb_all = k >> 8, nch_all = k >> 6;
+    const int b_begin = (int)((long)split * nb_all / splits), b_end = (int)((long)(split + 1) * nb_all / splits);
+    const int nb = b_end - b_begin, nch = 4 * nb;   // this workgroup's super-blocks and 64-k chunks, numbered from 0
     const int col = lane & 15, kg = lane >> 4;
     const int m0 = mt * MT + wm * 16 * MI;       // first activation row of this wave
     const bool wave_live = m0 < m;
 
     const int ar = tid >> 2, aq = tid & 3;        // unpack role: weight row of the tile, 8-byte piece of its 32 nibble bytes
-    const qg_u4 *bsrc = (const qg_u4 *)acts.planes + (size_t)(mt * MT16) * nch * 256;
+    const qg_u4 *bsrc = (const qg_u4 *)acts.planes + ((size_t)(mt * MT16) * nch_all + 4 * b_begin) * 256;
     // asynchronous-load roles: nibble rows 16 wave + 8 j + lane/8 (dword lane%8), header row 16 wave + lane/4
     const uint8_t *nib_src[2];
 #pragma unroll
     for (int j = 0; j < 2; j++)
-        nib_src[j] = W + (size_t)min(nt * QG_NT + 16 * wave + 8 * j + (lane >> 3), n - 1) * row_bytes + 16 + 4 * (lane & 7);
-    const uint8_t *hdr_src = W + (size_t)min(nt * QG_NT + 16 * wave + (lane >> 2), n - 1) * row_bytes + 4 * (lane & 3);
-    const qg_u4 *xs_src = (const qg_u4 *)acts.mins + (size_t)(mt * MT16 + wave) * nb * 64 + lane;
+        nib_src[j] = W + (size_t)min(nt * QG_NT + 16 * wave + 8 * j + (lane >> 3), n - 1) * row_bytes + (size_t)b_begin * 144 + 16 + 4 * (lane & 7);
+    const uint8_t *hdr_src = W + (size_t)min(nt * QG_NT + 16 * wave + (lane >> 2), n - 1) * row_bytes + (size_t)b_begin * 144 + 4 * (lane & 3);
+    const qg_u4 *xs_src = (const qg_u4 *)acts.mins + ((size_t)(mt * MT16 + wave) * nb_all + b_begin) * 64 + lane;
 
     auto b_slot = [&](auto S) __attribute__((always_inline)) -> qg_u4 * {
         if constexpr (decltype(S)::value == 0) return b_s0;
@@ -270,7 +279,7 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
         for (int i = 0; i < 4; i++) {
             const int blk = wave * 4 + i;                       // LDS block = ksp * MT16 + mtile
             const int ksp = blk / MT16, mtile = blk % MT16;
-            const qg_u4 *src = bsrc + ((size_t)mtile * nch + c) * 256 + ksp * 64 + lane;
+            const qg_u4 *src = bsrc + ((size_t)mtile * nch_all + c) * 256 + ksp * 64 + lane;
             qg_async_load16(src, qg_lds_offset(bb + blk * 64));
         }
     };
@@ -418,7 +427,7 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
 #pragma unroll
         for (int ni = 0; ni < 4; ni++) {
             const int nn = nt * QG_NT + wn * 64 + 16 * ni + 4 * kg;
-            float *yp = Y + (size_t)row * n + nn;
+            float *yp = Y + (size_t)split * split_stride + (size_t)row * n + nn;
             if (nn + 3 < n && (n & 3) == 0) {
                 *(float4 *)yp = float4{acc[ni][mi][0], acc[ni][mi][1], acc[ni][mi][2], acc[ni][mi][3]};
             } else {
@@ -426,6 +435,27 @@ __global__ __launch_bounds__(512) void q4k_gemm_mfma(const uint8_t *__restrict__
                 for (int j = 0; j < 4; j++)
                     if (nn + j < n) yp[j] = acc[ni][mi][j];
             }
+        }
+    }
+}
+
+// Y[i] = P[0][i] + P[1][i] + ... + P[splits - 1][i], in that order, four elements a thread.
+__global__ __launch_bounds__(256) void splitk_sum(const float *__restrict__ P, float *__restrict__ Y, size_t count,
+                                                   int splits) {
+    const size_t i = 4 * ((size_t)blockIdx.x * 256 + threadIdx.x);
+    if (i >= count) return;
+    if (i + 3 < count && (count & 3) == 0) {
+        float4 a = *(const float4 *)(P + i);
+        for (int sp = 1; sp < splits; sp++) {
+            const float4 b = *(const float4 *)(P + (size_t)sp * count + i);
+            a.x += b.x, a.y += b.y, a.z += b.z, a.w += b.w;
+        }
+        *(float4 *)(Y + i) = a;
+    } else {
+        for (size_t j = i; j < count && j < i + 4; j++) {
+            float a = P[j];
+            for (int sp = 1; sp < splits; sp++) a += P[(size_t)sp * count + j];
+            Y[j] = a;
         }
     }
 }

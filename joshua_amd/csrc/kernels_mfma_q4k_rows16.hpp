@@ -27,15 +27,17 @@ constexpr int QM_RED_STRIDE = 260;  // floats a wave in the reduction buffer: th
 typedef int qm_i4 __attribute__((ext_vector_type(4)));
 typedef float qm_f4 __attribute__((ext_vector_type(4)));
 
-// grid (8 sub-blocks, k / 256 columns), one wave.  Rows m_rows .. 15 are zero operands.
+// grid (8 sub-blocks, k / 256 columns, groups of 16 activation rows), one wave.  Rows from m_rows on
+// are zero operands.
 __global__ __launch_bounds__(64) void q4k_acts16_prep(const float *__restrict__ X, int m_rows, int k,
                                                        uint8_t *__restrict__ out) {
     const int lane = threadIdx.x, i = lane & 15, g = lane >> 4, j = blockIdx.x, col = blockIdx.y;
-    uint8_t *rec = out + (size_t)col * QM_REC;
+    const int row = 16 * (int)blockIdx.z + i;
+    uint8_t *rec = out + ((size_t)blockIdx.z * gridDim.y + col) * QM_REC;
     float v[8];
-    if (i < m_rows) {
-        const float4 a = *(const float4 *)(X + (size_t)i * k + 256 * col + 32 * j + 8 * g);
-        const float4 b = *(const float4 *)(X + (size_t)i * k + 256 * col + 32 * j + 8 * g + 4);
+    if (row < m_rows) {
+        const float4 a = *(const float4 *)(X + (size_t)row * k + 256 * col + 32 * j + 8 * g);
+        const float4 b = *(const float4 *)(X + (size_t)row * k + 256 * col + 32 * j + 8 * g + 4);
         v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
     } else {
 #pragma unroll

@@ -359,11 +359,13 @@ def test_q4k_dot4_gemv_long_rows_integer_dot_products_are_bit_exact(k, n):
     assert np.array_equal(got[0], want.astype(np.float32))
 
 
-@pytest.mark.parametrize("m,n", [(2, 1024), (5, 1030), (16, 14336), (16, 4097), (3, 5000), (8, 8190), (16, 4112)])
+@pytest.mark.parametrize("m,n", [(2, 1024), (5, 1030), (16, 14336), (16, 4097), (3, 5000), (8, 8190), (16, 4112),
+                                 (17, 1024), (33, 4100), (64, 14336), (48, 1031), (130, 4096)])
 def test_q4k_few_rows_over_4096_wide_rows(m, n):
-    """2..16 activation rows over rows of 4096, 1024 weight rows or more: the int8 matrix-core kernel on
-    the one-row kernel's weight stream; row counts with a partial last tile, one and several tiles a
-    workgroup; wide-ranging activations, a zero row, a non-finite activation."""
+    """2..64 activation rows over rows of 4096, 1024 weight rows or more: the int8 matrix-core kernel on
+    the one-row kernel's weight stream, a pass per 16 activation rows; row counts with a partial last
+    tile, one and several tiles a workgroup; wide-ranging activations, a zero row, a non-finite
+    activation."""
     k = 4096
     blocks = make_blocks(capi.Q4_K, n, k, 61 + n)
     rng = np.random.default_rng(n + m)
@@ -380,7 +382,7 @@ def test_q4k_few_rows_over_4096_wide_rows(m, n):
     assert np.isnan(bad[1]).all() and np.array_equal(bad[0], got[0])
 
 
-@pytest.mark.parametrize("m,n", [(2, 1024), (16, 1040), (7, 4500)])
+@pytest.mark.parametrize("m,n", [(2, 1024), (16, 1040), (7, 4500), (37, 14336)])
 def test_q4k_few_rows_over_4096_wide_rows_integer_dot_products_are_bit_exact(m, n):
     k = 4096
     blocks, q, x = q4k_integer_case(n, k, 13 + m, group=32, big_value=32639, small=1000)
