@@ -1077,6 +1077,66 @@ int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *co
     }
 }
 
+// The decode-sized down projection and the weighted combine in one launch (moe_down_combine_dot8): T
+// tokens, k_used routed pairs each plus n_extra for a folded shared expert, activations the rows of X
+// in pair order.  Returns -1 when the shape is outside its reach.
+template <class Q>
+int launch_moe_down_combine(const uint8_t *const *Wa, size_t row_bytes, bool aligned16, const float *X, size_t x_rows,
+                            jq::ActsI8 xq, const int *gexp, const float *wts, float *y, int k, int n, int T, int k_used,
+                            int n_extra, hipStream_t s) {
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS, S = k_used + n_extra;
+    const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
+    const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
+    const size_t wgs = (n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R);
+    const bool own = wgs * (size_t)k <= 512 * 1024 || !xq.xl;  // as in launch_moe_dot8
+    const size_t slot_lds = ((size_t)R * row_bytes + 15) / 16 * 16;
+    const size_t lds = slot_lds * S * jq::ROWS_PER_WG + jq::table_bytes<Q>() + (own ? (size_t)S * ((size_t)k * 2 + (size_t)k / 4) : 0);
+    // worth it from two workgroups a compute unit on: each one works through its S pairs in turn
+    if (G == 0 || S > 64 || lds > 96 * 1024 || T > 65535 || k % 16 != 0 || wgs * (size_t)T < 512) return -1;
+    if (!own) {
+        const size_t words = x_rows * (size_t)(k / 4);
+        hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
+    }
+    dim3 grid((unsigned)wgs, (unsigned)T), block(64 * jq::ROWS_PER_WG);
+#define JQ_DC(GG, OWN)                                                                                              \
+    do {                                                                                                            \
+        auto kern = jq::moe_down_combine_dot8<Q, GG, OWN>;                                                          \
+        static std::once_flag big_lds;                                                                              \
+        static hipError_t attr_rc = hipSuccess;                                                                     \
+        std::call_once(big_lds, [&] {                                                                               \
+            attr_rc = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); \
+        });                                                                                                         \
+        HIP_TRY(attr_rc);                                                                                           \
+        hipLaunchKernelGGL(kern, grid, block, lds, s, Wa, row_bytes, X, xq, gexp, wts, y, k, n, L, (int)slot_lds,  \
+                           k_used, n_extra, T * k_used);                                                            \
+    } while (0)
+    if (G == 16 && own) JQ_DC(16, true);
+    else if (G == 16) JQ_DC(16, false);
+    else if (own) JQ_DC(4, true);
+    else JQ_DC(4, false);
+#undef JQ_DC
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int dispatch_moe_down_combine(uint32_t type, const uint8_t *const *Wa, size_t row_bytes, bool aligned16, const float *X,
+                              size_t x_rows, jq::ActsI8 xq, const int *gexp, const float *wts, float *y, int k, int n,
+                              int T, int k_used, int n_extra, hipStream_t s) {
+    static const char *off = getenv("JQ_MOE_NO_DOWN_COMBINE");
+    if (off || !moe_has_dot8(type) || k % 32 != 0 || ((uintptr_t)X & 15) != 0) return -1;
+    switch (type) {
+#define JQ_DC_CASE(ID, Q)                                                                                           \
+    case ID:                                                                                                        \
+        return launch_moe_down_combine<jq::Q>(Wa, row_bytes, aligned16, X, x_rows, xq, gexp, wts, y, k, n, T, k_used, \
+                                              n_extra, s);
+        JQ_DC_CASE(JQ_TYPE_MXFP4, MXFP4)
+        JQ_DC_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
+        JQ_DC_CASE(JQ_TYPE_Q4_K, Q4_K)
+#undef JQ_DC_CASE
+    default: return -1;
+    }
+}
+
 template <bool SWIGLU>
 int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2,
                       const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
@@ -1161,6 +1221,13 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);
+    if (rc > 0) return 1;
+    // decode-sized, and no shared expert outside the pair list: down projection and combine in one launch
+    if (rc < 0 && fused_act && max_group <= 1 && (m->fold_shared || !m->sgate)) {
+        rc = dispatch_moe_down_combine(m->down->type, m->pdown, m->down->row_bytes, d16, m->G, (size_t)P + extra * T, m->qi8,
+                                       m->gexp, m->wts, y, (int)c.inter, (int)c.hidden, (int)T, (int)c.n_expert_used, extra, s);
+        if (rc == 0) return 0;
+    }
     if (rc > 0) return 1;
     if (rc < 0 && fused_act && max_group <= 1)
         rc = dispatch_moe_dot8<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,

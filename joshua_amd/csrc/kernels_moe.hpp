@@ -71,7 +71,7 @@ struct MoePairGroups {
 __global__ __launch_bounds__(256) void moe_gate_topk(const float *__restrict__ logits, const float *__restrict__ bias,
                                                       MoeGateParams p, uint32_t *__restrict__ ids,
                                                       float *__restrict__ wts, MoePairGroups pg) {
-    extern __shared__ float sm[];  // probs[E], sel[E], gscore[n_group], selw[k_used], red[4]
+    extern __shared__ __attribute__((aligned(16))) float sm[];  // probs[E], sel[E], gscore[n_group], selw[k_used], red[4]
     float *probs = sm, *sel = sm + p.E, *gscore = sm + 2 * p.E, *selw = gscore + (p.n_group > 1 ? p.n_group : 1);
     float *red = selw + p.k_used;
     const int t = blockIdx.x, lane = threadIdx.x, wv = threadIdx.x >> 6;  // `lane` strides the experts by 256
@@ -130,7 +130,19 @@ __global__ __launch_bounds__(256) void moe_gate_topk(const float *__restrict__ l
     for (int e = lane; e < p.E; e += NT) {
         const float v = sel[e];
         int rank = 0;
-        for (int o = 0; o < p.E; o++) rank += sel[o] > v || (sel[o] == v && o < e);
+        // how many experts come before e: four scores a read, sixteen reads in flight (one score a read,
+        // each waited for in turn, made this loop two thirds of the kernel's time)
+        int o = 0;
+        if ((p.E & 3) == 0) {
+            const float4 *sel4 = (const float4 *)sel;  // sm is 16-byte aligned and E a multiple of 4
+#pragma unroll 4
+            for (; o < p.E; o += 4) {
+                const float4 q = sel4[o >> 2];
+                rank += (q.x > v || (q.x == v && o < e)) + (q.y > v || (q.y == v && o + 1 < e)) +
+                        (q.z > v || (q.z == v && o + 2 < e)) + (q.w > v || (q.w == v && o + 3 < e));
+            }
+        }
+        for (; o < p.E; o++) rank += sel[o] > v || (sel[o] == v && o < e);
         if (rank < p.k_used) {
             ids[(size_t)t * p.k_used + rank] = (uint32_t)e;
             selw[rank] = probs[e];
@@ -553,6 +565,121 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
         if (DUAL) acc2 += __shfl_xor(acc2, off, 64);
     }
     if (sub == 0 && active) Y[(size_t)yrow[beg] * n + row] = DUAL ? swiglu(acc, acc2, cl, e) : acc;
+}
+
+// The decode-sized down projection with the weighted combine in the same kernel.  Workgroup (tile of
+// output rows, token t) walks the token's pairs: its k_used routed experts in slot order (pair
+// t * k_used + s, weight wts[pair]) and then, with n_extra, the shared expert (pair P + t, weight 1).  Pair p
+// multiplies row p of X (the activations silu(gate) * up of that pair) by expert gexp[p]'s rows.  All
+// pairs' rows of a wave are asked for at once (S times the bytes in flight of moe_rows_dot8, and a ninth
+// of its workgroups at DeepSeek-V3's sizes), and
+//   y[t, row] = sum_s w_s * (W[e_s] x_s)[row]  (+ the shared expert's)
+// is formed in the order moe_combine adds in, without the trip of the per-pair results through memory
+// or the launch of moe_combine.  The S activation rows are fixed-point planes: quantised into LDS by the
+// workgroup itself with OWN_PREP, else read from acts_i8_prep's output (copying those into LDS as well
+// leaves room for one workgroup a compute unit at DeepSeek-V3's sizes and measured a quarter slower).
+// Dynamic LDS: the format's table, ROWS_PER_WG * S * slot_lds of staged rows, with OWN_PREP S * 2.25 k more.
+template <class Q, int G, bool OWN_PREP>
+__global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_down_combine_dot8(const uint8_t *const *__restrict__ Wa,
+                                                                           size_t row_bytes, const float *__restrict__ X,
+                                                                           ActsI8 xq, const int *__restrict__ gexp,
+                                                                           const float *__restrict__ wts,
+                                                                           float *__restrict__ y, int k, int n, int L,
+                                                                           int slot_lds, int k_used, int n_extra, int P) {
+    static_assert(Q::SEGS == 1 && Q::SEGLEN % 32 == 0, "units of 32 or 64 consecutive elements");
+    constexpr int XW = Q::SEGLEN / 4, NS = Q::SEGLEN / 32;
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
+    const auto *table = stage_table<Q>(staged_moe);  // holds a barrier
+    const int t = blockIdx.y, S = k_used + n_extra;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int R = 64 / L;
+    const int row0 = (blockIdx.x * ROWS_PER_WG + wave) * R;
+    const int nrows = min(R, n - row0);  // <= 0: this wave has no rows and only helps with the activations
+    uint8_t *ra = staged_moe + table_bytes<Q>() + (size_t)wave * S * slot_lds;
+    if (nrows > 0) {
+        const int pieces = (int)((size_t)nrows * row_bytes / G);
+        for (int sl = 0; sl < S; sl++) {
+            const int pair = sl < k_used ? t * k_used + sl : P + t;
+            const uint8_t *sa = Wa[gexp[pair]] + (size_t)row0 * row_bytes;
+            uint8_t *dst = ra + (size_t)sl * slot_lds;
+            for (int p0 = 0; p0 < pieces; p0 += 64) {
+                if (p0 + lane < pieces) {
+                    if (G == 16) async_load16(sa + (size_t)(p0 + lane) * 16, lds_offset_of(dst + (size_t)p0 * 16));
+                    else async_load4(sa + (size_t)(p0 + lane) * 4, lds_offset_of(dst + (size_t)p0 * 4));
+                }
+            }
+        }
+    }
+    const int kw = k / 4, kb = k / 32;
+    uint32_t *xl_lds = (uint32_t *)(staged_moe + table_bytes<Q>() + (size_t)ROWS_PER_WG * S * slot_lds);
+    uint32_t *xh_lds = xl_lds + (size_t)S * kw;
+    float *sx_lds = (float *)(xh_lds + (size_t)S * kw), *sxs_lds = sx_lds + (size_t)S * kb;
+    if (OWN_PREP) {  // four elements a thread, eight threads a 32-element block (k % 32 == 0)
+        for (int i = threadIdx.x; i < S * kw; i += 64 * ROWS_PER_WG) {
+            const int sl = i / kw, j = i - sl * kw;
+            const int pair = sl < k_used ? t * k_used + sl : P + t;
+            const float4 v = *(const float4 *)(X + (size_t)pair * k + 4 * j);
+            float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
+            amax = max_row8(amax);
+            const bool live = amax > 0.0f && amax < INFINITY;
+            const float inv = live ? 32639.0f / amax : 0.0f;
+            const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                               __float2int_rn(v.w * inv)};
+            uint32_t wl = 0, wh = 0;
+            int sum = 0;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const int lo = ((Xq[c] + 128) & 255) - 128, hi = (Xq[c] - lo) >> 8;
+                wl |= (uint32_t)(lo & 255) << (8 * c);
+                wh |= (uint32_t)(hi & 255) << (8 * c);
+                sum += Xq[c];
+            }
+            xl_lds[i] = wl;
+            xh_lds[i] = wh;
+            sum = isum_row8(sum);
+            if ((i & 7) == 0) {
+                const float sc = fixed_scale(amax, 32639.0f);
+                sx_lds[i >> 3] = sc;
+                sxs_lds[i >> 3] = sc * (float)sum;
+            }
+        }
+        __syncthreads();
+    }
+    if (nrows <= 0) return;
+    const int sub = lane % L, rl = lane / L, row = row0 + rl;
+    const bool active = rl < nrows;
+    const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows landed (this wave's own data)
+    float total = 0.0f;
+    for (int sl = 0; sl < S; sl++) {
+        const size_t pair = sl < k_used ? (size_t)t * k_used + sl : (size_t)P + t;
+        const uint32_t *xlp = OWN_PREP ? xl_lds + (size_t)sl * kw : xq.xl + pair * kw;
+        const uint32_t *xhp = OWN_PREP ? xh_lds + (size_t)sl * kw : xq.xh + pair * kw;
+        const float *sxp = OWN_PREP ? sx_lds + (size_t)sl * kb : xq.sx + pair * kb;
+        const float *sxsp = OWN_PREP ? sxs_lds + (size_t)sl * kb : xq.sxs + pair * kb;
+        const uint8_t *rpa = ra + (size_t)sl * slot_lds + (size_t)rl * row_bytes;
+        float acc = 0.0f;
+        if (active) {
+            for (int u = sub; u < units; u += L) {
+                const int b = u / Q::UNITS, ub = u % Q::UNITS;
+                const int el = b * Q::BLOCK_ELEMS + Q::elem_base(ub);  // a multiple of 32
+                uint32_t xl[XW], xh[XW];
+                float sx[NS], sxs[NS];
+#pragma unroll
+                for (int i = 0; i < XW; i += 4) {
+                    const uint4 lw = *(const uint4 *)(xlp + el / 4 + i), hw = *(const uint4 *)(xhp + el / 4 + i);
+                    xl[i] = lw.x, xl[i + 1] = lw.y, xl[i + 2] = lw.z, xl[i + 3] = lw.w;
+                    xh[i] = hw.x, xh[i + 1] = hw.y, xh[i + 2] = hw.z, xh[i + 3] = hw.w;
+                }
+#pragma unroll
+                for (int i = 0; i < NS; i++) sx[i] = sxp[el / 32 + i], sxs[i] = sxsp[el / 32 + i];
+                acc += Q::dot8(table, rpa + (size_t)b * Q::BLOCK_BYTES, ub, xl, xh, sx, sxs);
+            }
+        }
+        for (int off = L >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        total = sl < k_used ? fmaf(acc, wts[t * k_used + sl], total) : total + acc;
+    }
+    if (sub == 0 && active) y[(size_t)t * n + row] = total;
 }
 
 // y[t, :] = sum_s w[t, s] * out[t*k + s, :]  (+ shared_out[t, :] of the shared expert),

@@ -124,6 +124,23 @@ def test_decode_sized_call_over_large_expert_matrices(qtype):
     assert close(dev.forward(x), ora.forward(x))
 
 
+@pytest.mark.parametrize("qtype,h,inter,E,k,shared_inter,tokens", [
+    (capi.Q4_K, 2048, 768, 16, 4, 0, 4),          # 16 rows a workgroup, planes quantised by the workgroup
+    (capi.MXFP4, 4096, 512, 16, 4, 512, 2),       # shared expert as a fifth pair
+    (capi.IQ2_XXS, 4096, 2048, 8, 4, 2048, 1),    # planes copied from the quantisation launch, shared expert
+    (capi.MXFP4, 4128, 2048, 8, 3, 0, 2),         # three pairs a token, two tokens
+])
+def test_decode_sized_down_projection_with_the_combine_fused(qtype, h, inter, E, k, shared_inter, tokens):
+    """Decode-sized calls with 512 workgroups or more in the down projection: one launch walks each
+    token's pairs and forms the weighted sum itself."""
+    kw = dict(gating="sigmoid", weights_scale=2.5) if shared_inter else {}
+    ora, dev = build(qtype, h, inter, E, k, 130 + h, shared_inter=shared_inter, **kw)
+    x = synth.normal(131 + tokens, (tokens, h))
+    want = ora.forward(x)
+    assert close(dev.forward(x), want)
+    assert close(dev.forward(x), want)
+
+
 def test_many_tokens_group_beyond_the_lds_pair_list():
     ora, dev = build(capi.Q8_0, 64, 32, 4, 2, 110)
     x = synth.normal(111, (6200, 64))          # 12400 pairs
