@@ -1729,7 +1729,7 @@ namespace {
 
 void model_free_scratch(jq_model *m) {
     for (void *p : {(void *)m->ids, (void *)m->x, (void *)m->x2, (void *)m->hn, (void *)m->qb, (void *)m->kb, (void *)m->vb,
-                    (void *)m->att, (void *)m->proj, (void *)m->g, (void *)m->u, (void *)m->mid})
+                    (void *)m->att, (void *)m->proj, (void *)m->g, (void *)m->mid})  // u is the second half of g
         if (p) (void)hipFree(p);
     m->ids = nullptr;
     m->x2 = nullptr;
@@ -1751,8 +1751,10 @@ int model_reserve(jq_model *m, size_t T) {
     HIP_TRY(hipMalloc((void **)&m->vb, T * kd * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->att, T * qd * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->proj, T * c.hidden * sizeof(float)));
-    HIP_TRY(hipMalloc((void **)&m->g, T * c.ffn * sizeof(float)));
-    HIP_TRY(hipMalloc((void **)&m->u, T * c.ffn * sizeof(float)));
+    // gate and up results in one allocation: a many-token step over a paired gate|up matrix writes its
+    // T x 2 ffn result (gate_j, up_j alternating) across both
+    HIP_TRY(hipMalloc((void **)&m->g, 2 * T * c.ffn * sizeof(float)));
+    m->u = m->g + T * c.ffn;
     HIP_TRY(hipMalloc((void **)&m->mid, T * c.ffn * sizeof(float)));
     m->cap_tokens = T;
     return 0;
@@ -1951,10 +1953,21 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
                                                                    paired ? m->mid : m->cat, paired, s);
         if (normed2) std::swap(xc, xo), activated = paired;
         else hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, m->proj, w_fn, c.rms_eps, m->hn, h);
+        // many tokens over a paired gate|up matrix: one product with twice the rows (768 GEMM tiles at Qwen3-8B's
+        // sizes fill the 256 compute units three times over; two products of 384 tiles leave half of them idle
+        // in their second rounds), then SwiGLU over the alternating results
+        static const char *no_pair_gemm = getenv("JQ_NO_PAIRED_PREFILL");
+        auto fgm = T > 1 && !no_pair_gemm ? m->fused.find(p + ".gate_up") : m->fused.end();
+        if (fgm != m->fused.end() && !m->paired.count(fgm->first)) fgm = m->fused.end();
         if (fg != m->fused.end()) {
             const jq_weight *w = fg->second;
             if (!normed2 && dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
             gp = m->cat, up = m->cat + c.ffn;
+        } else if (fgm != m->fused.end()) {
+            const jq_weight *w = fgm->second;
+            if (dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->g, T, w->k, w->n, s)) return 1;
+            hipLaunchKernelGGL(jq::swiglu_pairs, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, m->g, m->mid, (size_t)T * c.ffn);
+            activated = true;
         } else if (model_mm(m, p + ".ffn_gate.weight", m->hn, m->g, T, s) ||
                    model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s)) {
             return 1;
@@ -2103,7 +2116,7 @@ int jq_qwen3_forward(jq_model *m, const uint32_t *tokens, uint32_t n_tokens, uin
         if (tokens[i] >= m->cfg.vocab) return fail("embedding id %u is out of range for %u rows", tokens[i], m->cfg.vocab);
     hipStream_t s = (hipStream_t)stream;
     if (model_reserve(m, n_tokens)) return 1;
-    if (n_tokens == 1 && model_prepare_fused(m)) return 1;
+    if (model_prepare_fused(m)) return 1;  // first step only: q|k(|v) and gate|up as single matrices
     HIP_TRY(hipMemcpyAsync(m->ids, tokens, n_tokens * sizeof(uint32_t), hipMemcpyHostToDevice, s));
     if (model_forward_dev(m, n_tokens, pos, s)) return 1;
     m->n_past = pos + n_tokens;
