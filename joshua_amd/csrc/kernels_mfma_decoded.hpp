@@ -10,8 +10,9 @@
 // Workgroup: 64 weight rows x 64 activation rows, 4 waves (16 weight rows each), chunks of 256
 // elements: the raw block bytes of the chunk (4-byte loads from the word at or below each row's
 // unaligned start) and the activation planes go to LDS, 256 threads decode one or two units each,
-// then 8 k-steps x 4 column tiles x 2 planes of MFMA per wave.  No pipelining between the stages: the
-// kernel replaces f32 row kernels that run at 5 to 9 TFLOP/s.
+// then 8 k-steps x 4 column tiles x 2 planes of MFMA per wave.  The next chunk's global data travels into
+// registers while the current chunk is decoded and multiplied; the stages themselves run one after the
+// other (the kernel replaces f32 row kernels that run at 5 to 9 TFLOP/s).
 #pragma once
 #include "kernels_mfma_q4k_gemm.hpp"
 #include "kernels_valu.hpp"
@@ -78,24 +79,55 @@ __global__ __launch_bounds__(256) void gemm_decoded_mfma(const uint8_t *__restri
     for (int ct = 0; ct < 4; ct++) acc[ct] = qg_f4{0.f, 0.f, 0.f, 0.f};
 
     const int nc = k >> 8;
-    for (int c = 0; c < nc; c++) {
-        // ---- the chunk's raw bytes: row r's words from the word at or below its first byte ----
-        for (int idx = tid; idx < GD_NT * NDW; idx += 256) {
+    // The next chunk's global data (raw block bytes, activation planes, activation scales) is asked for
+    // into registers before the decode and MFMA stages of the current one and stored into LDS at the top
+    // of the next iteration, so the trip to memory runs beside the arithmetic.
+    constexpr int RAW_IT = (GD_NT * NDW + 255) / 256, B_IT = GD_MT * (GD_KC / 8) / 256;
+    uint32_t raw_r[RAW_IT];
+    qg_u4 bh_r[B_IT], bl_r[B_IT];
+    float s_r = 0.0f;
+    auto fetch = [&](int c) __attribute__((always_inline)) {
+        // row r's words from the word at or below its first byte
+#pragma unroll
+        for (int it = 0; it < RAW_IT; it++) {
+            const int idx = tid + 256 * it;
             const int r = idx / NDW, dw = idx % NDW;
-            const uintptr_t src = (uintptr_t)(W + (size_t)min(n0 + r, n - 1) * row_bytes + (size_t)c * CB);
-            const uint32_t *wp = (const uint32_t *)(src & ~(uintptr_t)3) + dw;
-            // the last word may lie past the chunk: it is read only when it still holds bytes of it
-            raw[r][dw] = (uintptr_t)wp < src + CB ? *wp : 0u;
+            raw_r[it] = 0u;
+            if (idx < GD_NT * NDW) {
+                const uintptr_t src = (uintptr_t)(W + (size_t)min(n0 + r, n - 1) * row_bytes + (size_t)c * CB);
+                const uint32_t *wp = (const uint32_t *)(src & ~(uintptr_t)3) + dw;
+                // the last word may lie past the chunk: it is read only when it still holds bytes of it
+                if ((uintptr_t)wp < src + CB) raw_r[it] = *wp;
+            }
         }
-        // ---- the activation planes of the 64 rows m0 .. m0 + 63 (prepared, zero beyond m) ----
-        for (int idx = tid; idx < GD_MT * (GD_KC / 8); idx += 256) {
+        // the activation planes of the 64 rows m0 .. m0 + 63 (prepared, zero beyond m)
+#pragma unroll
+        for (int it = 0; it < B_IT; it++) {
+            const int idx = tid + 256 * it;
             const int col = idx / (GD_KC / 8), part = idx % (GD_KC / 8);
             const size_t at = (size_t)(m0 + col) * k + (size_t)c * GD_KC + 8 * part;
-            *(qg_u4 *)&b_lds[0][col][8 * part] = *(const qg_u4 *)(acts.hi + at);
-            *(qg_u4 *)&b_lds[1][col][8 * part] = *(const qg_u4 *)(acts.lo + at);
+            bh_r[it] = *(const qg_u4 *)(acts.hi + at);
+            bl_r[it] = *(const qg_u4 *)(acts.lo + at);
         }
-        if (tid < GD_MT) s_lds[tid] = acts.s[(size_t)(m0 + tid) * nc + c];
+        if (tid < GD_MT) s_r = acts.s[(size_t)(m0 + tid) * nc + c];
+    };
+    fetch(0);
+    for (int c = 0; c < nc; c++) {
+#pragma unroll
+        for (int it = 0; it < RAW_IT; it++) {
+            const int idx = tid + 256 * it;
+            if (idx < GD_NT * NDW) raw[idx / NDW][idx % NDW] = raw_r[it];
+        }
+#pragma unroll
+        for (int it = 0; it < B_IT; it++) {
+            const int idx = tid + 256 * it;
+            const int col = idx / (GD_KC / 8), part = idx % (GD_KC / 8);
+            *(qg_u4 *)&b_lds[0][col][8 * part] = bh_r[it];
+            *(qg_u4 *)&b_lds[1][col][8 * part] = bl_r[it];
+        }
+        if (tid < GD_MT) s_lds[tid] = s_r;
         __syncthreads();
+        if (c + 1 < nc) fetch(c + 1);
         // ---- decode: unit u of row r -> f16 in operand order ----
         for (int id = tid; id < GD_NT * UPR; id += 256) {
             const int r = id / UPR, u = id % UPR, b = u / Q::UNITS, ub = u % Q::UNITS;
