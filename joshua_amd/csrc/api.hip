@@ -1940,9 +1940,22 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         } else {
             hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, qp, kp, vp, w_qn, w_kn,
                                c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
-            size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
-            hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, qp, m->kc[l], m->vc[l], m->att, nh,
-                               nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
+            // head dimension 128 and 1, 2, 4 or 8 query heads a KV head: tiles of 16 tokens on the f32 matrix cores
+            static const char *no_tiles = getenv("JQ_NO_ATTENTION_TILES");
+            const int gq = nh / nkv;
+            const dim3 tgrid((unsigned)((T + 15) / 16), (unsigned)nkv);
+#define JQ_ATT_TILES(GQ)                                                                                            \
+    hipLaunchKernelGGL((jq::attention_tiles<128, GQ>), tgrid, dim3(64 * GQ), 0, s, qp, m->kc[l], m->vc[l], m->att, (int)T, \
+                       nh, m->pos, (int)c.n_ctx, sqrt_d)
+            if (no_tiles || d != 128 || (gq != 1 && gq != 2 && gq != 4 && gq != 8)) {
+                size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
+                hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, qp, m->kc[l], m->vc[l], m->att, nh,
+                                   nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
+            } else if (gq == 1) JQ_ATT_TILES(1);
+            else if (gq == 2) JQ_ATT_TILES(2);
+            else if (gq == 4) JQ_ATT_TILES(4);
+            else JQ_ATT_TILES(8);
+#undef JQ_ATT_TILES
         }
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
         const float *gp = m->g, *up = m->u;

@@ -144,6 +144,119 @@ __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ 
     }
 }
 
+// The same attention for a step of many tokens, on the f32 matrix cores.  One workgroup per (tile of 16
+// tokens, KV head), one wave per query head of that KV head (G = n_head / n_kv waves), so the G heads
+// share every K and V row the workgroup stages.  Keys go by in tiles of 16 through LDS (the next tile's
+// rows travel into registers while the current one is multiplied); per tile and wave
+//   S^T = K Q^T   (16 keys x 16 tokens; 32 v_mfma_f32_16x16x4_f32 over the D = 128 head dimensions),
+//   running maximum and sum per token, p = exp(s - max)   (online softmax, keys after a token masked),
+//   O += P V      (32 more, 8 tiles of 16 dimensions)
+// Lane (n = lane % 16, g = lane / 16) holds S^T[key 4 g + j][token n], j < 4, which is the A operand of
+// P V as it stands when the product's inner index g stands for key 4 g + j in step j on both sides; the
+// outputs come out as O[token 4 g + j][dimension], so a token's rescaling factor is fetched from the lane
+// that holds its statistics.  Scores are divided by sqrt(d) as the reference does (src/embedding.rs:386).
+constexpr int AT_PAD = 4;  // floats a staged row is longer than D: 16 rows then fall into different banks
+
+template <int D, int G>
+__global__ __launch_bounds__(64 * G) void attention_tiles(const float *__restrict__ q, const float *__restrict__ kc,
+                                                          const float *__restrict__ vc, float *__restrict__ out,
+                                                          int T, int n_head, const int *__restrict__ pos_ptr,
+                                                          int n_ctx, float sqrt_d) {
+    constexpr int NT = 64 * G, STRIDE = D + AT_PAD, PIECES = 16 * (D / 4), PER = (PIECES + NT - 1) / NT;
+    __shared__ __attribute__((aligned(16))) float ks[16 * STRIDE], vs[16 * STRIDE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
+    const int t0 = 16 * (int)blockIdx.x, kvh = blockIdx.y, hq = kvh * G + wave, pos0 = *pos_ptr;
+    const int last_key = pos0 + min(t0 + 15, T - 1);        // the last key any token of the tile may see
+    const int n_tiles = last_key / 16 + 1;
+    const float *kb = kc + (size_t)kvh * n_ctx * D, *vb = vc + (size_t)kvh * n_ctx * D;
+
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    // this lane's share of Q^T as B operands: token n, dimensions 4 s + g
+    float qr[D / 4];
+    {
+        const float *qp = q + ((size_t)min(t0 + n, T - 1) * n_head + hq) * D + g;
+#pragma unroll
+        for (int s_ = 0; s_ < D / 4; s_++) qr[s_] = qp[4 * s_];
+    }
+    f4 o[D / 16];
+#pragma unroll
+    for (int dt = 0; dt < D / 16; dt++) o[dt] = f4{0.f, 0.f, 0.f, 0.f};
+    float mx = -INFINITY, sum = 0.0f;                       // of token n (the same in the four lanes that hold it)
+
+    float4 kpre[PER], vpre[PER];
+    auto fetch = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int piece = tid + NT * i, row = piece / (D / 4), c4 = piece % (D / 4), key = 16 * tile + row;
+            kpre[i] = vpre[i] = float4{0.f, 0.f, 0.f, 0.f};  // rows after the last key: the cache holds nothing there
+            if (piece < PIECES && key <= last_key) {
+                kpre[i] = *(const float4 *)(kb + (size_t)key * D + 4 * c4);
+                vpre[i] = *(const float4 *)(vb + (size_t)key * D + 4 * c4);
+            }
+        }
+    };
+    fetch(0);
+    for (int tile = 0; tile < n_tiles; tile++) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int piece = tid + NT * i, row = piece / (D / 4), c4 = piece % (D / 4);
+            if (piece < PIECES) {
+                *(float4 *)(ks + row * STRIDE + 4 * c4) = kpre[i];
+                *(float4 *)(vs + row * STRIDE + 4 * c4) = vpre[i];
+            }
+        }
+        __syncthreads();
+        if (tile + 1 < n_tiles) fetch(tile + 1);
+        // S^T: keys 16 tile + (4 g + j) x token n
+        f4 st = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s_ = 0; s_ < D / 4; s_++)
+            st = __builtin_amdgcn_mfma_f32_16x16x4f32(ks[n * STRIDE + 4 * s_ + g], qr[s_], st, 0, 0, 0);
+        float p[4], tmax = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int key = 16 * tile + 4 * g + j;
+            p[j] = key <= pos0 + t0 + n ? st[j] / sqrt_d : -INFINITY;
+            tmax = fmaxf(tmax, p[j]);
+        }
+        tmax = max_xor32(max_xor16(tmax));
+        const float mnew = fmaxf(mx, tmax), rescale = expf(mx - mnew);
+        float tsum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            p[j] = expf(p[j] - mnew);
+            tsum += p[j];
+        }
+        tsum = sum_xor32(sum_xor16(tsum));
+        sum = fmaf(sum, rescale, tsum);
+        mx = mnew;
+        // O rows are tokens 4 g + j: their factors live in the lanes of those tokens
+        float rs[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) rs[j] = __shfl(rescale, 4 * g + j, 64);
+#pragma unroll
+        for (int dt = 0; dt < D / 16; dt++) {
+            f4 acc = f4{o[dt][0] * rs[0], o[dt][1] * rs[1], o[dt][2] * rs[2], o[dt][3] * rs[3]};
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(p[j], vs[(4 * g + j) * STRIDE + 16 * dt + n], acc, 0, 0, 0);
+            o[dt] = acc;
+        }
+        __syncthreads();
+    }
+    float inv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) inv[j] = 1.0f / __shfl(sum, 4 * g + j, 64);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int t = t0 + 4 * g + j;
+        if (t >= T) continue;
+        float *op = out + ((size_t)t * n_head + hq) * D + n;
+#pragma unroll
+        for (int dt = 0; dt < D / 16; dt++) op[16 * dt] = o[dt][j] * inv[j];
+    }
+}
+
 // *pos = p, and the rotary angles of the T positions p .. p + T - 1 of a step: cs[t][i] = (cos, sin) of
 // (p + t) * theta^(-2i/d), i < d/2 — the arithmetic of qkv_norm_rope_cache, done once a step for the
 // attention kernel that applies head norm and rotation itself.

@@ -108,10 +108,13 @@ def test_prefill_in_two_chunks_matches_one():
     assert ok, e
 
 
-@pytest.mark.parametrize("head_dim,n_head,n_kv", [(64, 4, 2), (128, 4, 1), (256, 2, 2), (192, 4, 2)])
+@pytest.mark.parametrize("head_dim,n_head,n_kv", [(64, 4, 2), (128, 4, 1), (256, 2, 2), (192, 4, 2), (128, 8, 1),
+                                                  (128, 2, 2), (128, 4, 2)])
 def test_decode_over_several_key_chunks(head_dim, n_head, n_kv):
     """A cache longer than one 64-key chunk of the split attention kernel, entered both by a
-    long prefill and by short multi-token steps; head sizes with and without a split kernel."""
+    long prefill and by short multi-token steps; head sizes with and without a split kernel.  The
+    multi-token steps with head size 128 run the tiled matrix-core attention, with 8, 4, 2 and 1 query
+    heads a KV head, token counts that do not fill a tile and keys already in the cache."""
     cfg = dict(CFG, n_ctx=224, n_layer=2, head_dim=head_dim, n_head=n_head, n_kv_head=n_kv)
     m, o = make(cfg, 26)
     rng = np.random.default_rng(3)
