@@ -580,14 +580,22 @@ int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, floa
     const size_t m_pad = (m + jq::GD_MT - 1) / jq::GD_MT * jq::GD_MT, nc = k / jq::GD_KC;
     auto up = [](size_t v) { return (v + 255) / 256 * 256; };
     const size_t plane = up(m_pad * k * sizeof(_Float16)), sbytes = up(m_pad * nc * sizeof(float));
+    // split over k when the 64 x 64 tiles alone leave compute units idle (a workgroup takes ~5 us a chunk)
+    const size_t n_tiles = (n + jq::GD_NT - 1) / jq::GD_NT, m_tiles = m_pad / jq::GD_MT;
+    static const char *split_env = getenv("JQ_DECODED_GEMM_SPLITS");
+    const size_t splits = m * n / 1024 < 0x7FFFFFFFull ? (size_t)gemm_k_splits(n_tiles * m_tiles, nc, m, n, 5.0, split_env) : 1;
+    const size_t part_bytes = splits > 1 ? splits * m * n * sizeof(float) : 0;
     CallScratch scratch;
     uint8_t *buf = nullptr;
-    HIP_TRY(scratch.get(2 * plane + sbytes, s, &buf));
+    HIP_TRY(scratch.get(2 * plane + sbytes + part_bytes, s, &buf));
     jq::ActsF16 a{(_Float16 *)buf, (_Float16 *)(buf + plane), (float *)(buf + 2 * plane)};
+    float *parts = (float *)(buf + 2 * plane + sbytes);
     hipLaunchKernelGGL(jq::acts_f16_prep, dim3((unsigned)((m_pad * nc * 64 + 255) / 256)), dim3(256), 0, s, X, (int)m,
                        (int)m_pad, (int)k, a);
-    hipLaunchKernelGGL(jq::gemm_decoded_mfma<Q>, dim3((unsigned)((n + jq::GD_NT - 1) / jq::GD_NT), (unsigned)(m_pad / jq::GD_MT)),
-                       dim3(256), 0, s, W, row_bytes, a, Y, (int)m, (int)k, (int)n);
+    hipLaunchKernelGGL(jq::gemm_decoded_mfma<Q>, dim3((unsigned)n_tiles, (unsigned)m_tiles, (unsigned)splits), dim3(256), 0, s, W,
+                       row_bytes, a, splits > 1 ? parts : Y, (int)m, (int)k, (int)n, splits > 1 ? m * n : (size_t)0);
+    if (splits > 1)
+        hipLaunchKernelGGL(jq::splitk_sum, dim3((unsigned)((m * n + 1023) / 1024)), dim3(256), 0, s, parts, Y, m * n, (int)splits);
     HIP_TRY(hipGetLastError());
     return 0;
 }

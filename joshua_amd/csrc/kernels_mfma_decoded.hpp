@@ -59,8 +59,10 @@ __global__ __launch_bounds__(256) void acts_f16_prep(const float *__restrict__ X
 }
 
 template <class Q>
+// Split over k: blockIdx.z takes the z-th of gridDim.z contiguous runs of chunks and stores its partial
+// sums at Y + z * split_stride (splitk_sum adds them in order); one run and stride 0 give the result.
 __global__ __launch_bounds__(256) void gemm_decoded_mfma(const uint8_t *__restrict__ W, size_t row_bytes, ActsF16 acts,
-                                                         float *__restrict__ Y, int m, int k, int n) {
+                                                         float *__restrict__ Y, int m, int k, int n, size_t split_stride) {
     constexpr int CB = Q::BLOCK_BYTES * (GD_KC / Q::BLOCK_ELEMS);  // bytes of a row's chunk
     constexpr int NDW = (CB + 3 + 3) / 4;                          // words that cover it from any byte offset
     constexpr int UE = Q::SEGS * Q::SEGLEN, UPR = GD_KC / UE;      // elements a unit, units a row chunk
@@ -111,8 +113,10 @@ __global__ __launch_bounds__(256) void gemm_decoded_mfma(const uint8_t *__restri
         }
         if (tid < GD_MT) s_r = acts.s[(size_t)(m0 + tid) * nc + c];
     };
-    fetch(0);
-    for (int c = 0; c < nc; c++) {
+    const int c_begin = (int)((long)blockIdx.z * nc / gridDim.z), c_end = (int)((long)(blockIdx.z + 1) * nc / gridDim.z);
+    Y += (size_t)blockIdx.z * split_stride;
+    fetch(c_begin);
+    for (int c = c_begin; c < c_end; c++) {
 #pragma unroll
         for (int it = 0; it < RAW_IT; it++) {
             const int idx = tid + 256 * it;
@@ -127,7 +131,7 @@ __global__ __launch_bounds__(256) void gemm_decoded_mfma(const uint8_t *__restri
         }
         if (tid < GD_MT) s_lds[tid] = s_r;
         __syncthreads();
-        if (c + 1 < nc) fetch(c + 1);
+        if (c + 1 < c_end) fetch(c + 1);
         // ---- decode: unit u of row r -> f16 in operand order ----
         for (int id = tid; id < GD_NT * UPR; id += 256) {
             const int r = id / UPR, u = id % UPR, b = u / Q::UNITS, ub = u % Q::UNITS;
