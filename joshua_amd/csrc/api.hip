@@ -650,7 +650,13 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&
         !getenv("JQ_Q4K_NO_GEMM"))
         return dispatch_q4k_gemm(W, row_bytes, X, Y, m, k, n, s);
-    if (m > Q4K_MFMA_MAX_M && type != JQ_TYPE_Q4_K) {
+    // the other formats: the MFMA GEMM over decoded weights from 17 rows on, and (split over k, its 64-row
+    // activation tile part empty) from JQ_DECODED_GEMM_MIN_M rows (default 8) on against matrices of 8M
+    // elements or more, where the f32 staged kernel takes a pass over the matrix per four rows (Q6_K
+    // 4096 x 12288: 77 us at any row count against 92 us at 8 rows and 178 us at 16)
+    static const char *min_m_env = getenv("JQ_DECODED_GEMM_MIN_M");
+    static const size_t gemm_min_m = min_m_env ? (size_t)std::max(atoi(min_m_env), 2) : 8;
+    if ((m > Q4K_MFMA_MAX_M || (m >= gemm_min_m && n * k >= ((size_t)8 << 20))) && type != JQ_TYPE_Q4_K) {
         const int rc = dispatch_gemm_decoded(type, W, row_bytes, X, Y, m, k, n, s);
         if (rc >= 0) return rc;
     }

@@ -283,6 +283,20 @@ def test_non_finite_activations_show_in_the_result(qtype, m, k, n):
             assert close(got[:m - 1], want[:m - 1])
 
 
+@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q6_K, 8, 12288, 1024), (capi.Q8_0, 16, 4096, 2100), (capi.MXFP4, 11, 7168, 1200),
+                                         (capi.Q6_K, 512, 4096, 1024), (capi.IQ2_XXS, 70, 5120, 300)])
+def test_decoded_weights_gemm_split_over_k(qtype, m, k, n):
+    """8..16 rows against matrices of 8M elements or more, and many rows against few weight rows: the GEMM's
+    tiles alone leave compute units idle, so runs of chunks go to workgroups of their own and the partial
+    sums are added in a fixed order (the same result on every call)."""
+    blocks = make_blocks(qtype, n, k, 300 + m)
+    lhs = synth.normal(301 + m, (m, k))
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    got = w.matmul_t(m, lhs)
+    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
+    assert np.array_equal(got, w.matmul_t(m, lhs))
+
+
 @pytest.mark.parametrize("qtype", [capi.Q8_0, capi.Q2_K, capi.Q6_K, capi.IQ2_XXS, capi.MXFP4])
 @pytest.mark.parametrize("m,k,n", [(17, 256, 64), (40, 768, 100), (130, 1024, 77), (64, 2048, 256)])
 def test_many_rows_on_the_decoded_weights_gemm(qtype, m, k, n):
