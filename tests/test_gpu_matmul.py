@@ -493,6 +493,48 @@ def test_results_do_not_depend_on_how_rows_are_batched():
         assert np.array_equal(full, again)
 
 
+def test_threads_sharing_the_default_stream_get_their_own_results():
+    """Calls that prepare operands keep one scratch allocation per stream; host threads that share the
+    stream enqueue their calls in turn, so every thread's result is the one it gets alone, bit for bit.
+    The shapes take the 16-row int8 kernel, the Q4_K GEMM split over k and the decoded-weights GEMM, in
+    sizes that make the scratch grow between calls."""
+    import threading
+    cases = []
+    for i, (qtype, m, k, n) in enumerate([(capi.Q4_K, 16, 4096, 1024), (capi.Q4_K, 100, 2048, 300), (capi.Q6_K, 40, 1024, 200),
+                                          (capi.Q4_K, 5, 4096, 2048)]):
+        w = capi.Weight.upload(qtype, make_blocks(qtype, n, k, 500 + i), n, k)
+        lhs = synth.normal(510 + i, (m, k))
+        cases.append((w, m, lhs, w.matmul_t(m, lhs).copy()))
+    failures = []
+
+    def worker(tid):
+        for it in range(6):
+            w, m, lhs, want = cases[(tid + it) % len(cases)]
+            got = w.matmul_t(m, lhs)
+            if not np.array_equal(got, want):
+                failures.append((tid, it))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
+
+
+def test_q4k_few_rows_over_a_view_of_the_stacked_tensor():
+    """The 16-row kernel over a view that starts some rows into the allocation (an expert slice)."""
+    n, k, m = 3000, 4096, 9
+    blocks = make_blocks(capi.Q4_K, n, k, 520)
+    lhs = synth.normal(521, (m, k))
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    full = w.matmul_t(m, lhs)
+    row_bytes = 144 * k // 256
+    part = w.view(700 * row_bytes, 1500, k).matmul_t(m, lhs)
+    assert np.array_equal(part, full[:, 700:2200])
+    assert close(full, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True))
+
+
 def test_rejects_bad_shapes_and_leaves_dst_alone():
     # reference: src/quant_matmul.rs:597-608
     blocks = synth.quantize(capi.Q8_0, ref_weights(2, 256))
