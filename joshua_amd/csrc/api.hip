@@ -646,6 +646,13 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         const int rc = dispatch_q4k_stream(W, row_bytes, X, Y, m, k, n, s);
         if (rc >= 0) return rc;
     }
+    // rows longer than 4096 with 3..16 activation rows: the int8 GEMV below walks the matrix once per two
+    // rows (6.5 us a row at 4096 x 12288); from where that exceeds the estimate of the GEMM split over k
+    // (48 us there at any of these row counts), the GEMM
+    const bool gemm_ok = type == JQ_TYPE_Q4_K && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 && !getenv("JQ_Q4K_NO_GEMM");
+    if (gemm_ok && m > 2 && m <= Q4K_MFMA_MAX_M && k > 4096 &&
+        q4k_gemm_estimate_us(m, k, n) < (double)m * (2.0 + (double)n * (double)row_bytes / 4.0e6))
+        return dispatch_q4k_gemm(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k, n)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&
         !getenv("JQ_Q4K_NO_GEMM"))
