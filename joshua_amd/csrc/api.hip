@@ -496,9 +496,9 @@ double q4k_gemm_estimate_us(size_t m, size_t k, size_t n) {
     return us;
 }
 
-// Q4_K, two activation rows or more, contiguous rows of exactly 16 super-blocks: the int8 matrix-core kernel
-// on the one-row GEMV's weight stream, once per group of 16 activation rows (a matrix of this size stays
-// in the last-level cache between the passes), its operands prepared by one small launch into the call
+// Q4_K, two activation rows or more, rows of 4096, 8192, 12288 or 16384 columns: the int8 matrix-core kernel
+// on the one-row GEMV's weight stream, once per group of 16 activation rows and of 4096 columns (a matrix
+// of this size stays in the last-level cache between the passes; later column groups add to the result), its operands prepared by one small launch into the call
 // scratch of the stream.  Beyond 16 rows it runs while its estimated time (a pass costs ~4.3 us plus
 // 0.53 us per 1024 weight rows) stays below the MFMA GEMM's.  Returns -1 when the shape is outside its reach.
 constexpr size_t Q4K_ROWS16_MAX_M = 256;
@@ -510,22 +510,26 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
     static const size_t min_n = min_env ? (size_t)atoll(min_env) : 1024;
     static const char *max_env = getenv("JQ_Q4K_ROWS16_MAX_M");
     static const size_t max_m = max_env ? std::min<size_t>((size_t)atoll(max_env), 1024) : Q4K_ROWS16_MAX_M;
-    if (off || m < 2 || m > max_m || k != 4096 || row_bytes != (size_t)jq::QD_ROW || n < min_n || n > 0x7FFFFFF0ull ||
-        ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
+    if (off || m < 2 || m > max_m || k == 0 || k % 4096 != 0 || k > 4 * 4096 || row_bytes % 16 != 0 ||
+        row_bytes < k / 256 * 144 || n < min_n || n > 0x7FFFFFF0ull || ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
         return -1;
-    const size_t tiles = (n + 15) / 16, rounds = (tiles + 255) / 256, groups = (m + 15) / 16;
-    if (groups > 1 && !max_env && 3.0 + (double)groups * (4.3 + 0.527 * (double)n / 1024.0) >= q4k_gemm_estimate_us(m, k, n))
-        return -1;
+    const size_t tiles = (n + 15) / 16, rounds = (tiles + 255) / 256, groups = (m + 15) / 16, col_groups = k / 4096;
+    // a pass = 16 activation rows x 4096 columns over all weight rows
+    const double passes_us = 3.0 + (double)(groups * col_groups) * (4.3 + 0.527 * (double)n / 1024.0);
+    if ((groups > 1 || col_groups > 1) && !max_env && passes_us >= q4k_gemm_estimate_us(m, k, n)) return -1;
+    if (col_groups > 1 && m < 3) return -1;  // two rows: the two-row GEMV walks the matrix once
     static const char *genv = getenv("JQ_Q4K_ROWS16_GRID");
     const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)std::max(atoi(genv), 1) : (tiles + rounds - 1) / rounds);
     CallScratch scratch;
     uint8_t *acts = nullptr;
-    const size_t group_bytes = 16 * (size_t)jq::QM_REC;
+    const size_t cols = k / 256, group_bytes = cols * (size_t)jq::QM_REC;
     HIP_TRY(scratch.get(groups * group_bytes, s, &acts));
-    hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, 16, (unsigned)groups), dim3(64), 0, s, X, (int)m, (int)k, acts);
+    hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, (unsigned)cols, (unsigned)groups), dim3(64), 0, s, X, (int)m, (int)k, acts);
     for (size_t g = 0; g < groups; g++)
-        hipLaunchKernelGGL(jq::q4k_rows16_mfma, dim3(grid), dim3(1024), 0, s, W, (const uint8_t *)(acts + g * group_bytes),
-                           Y + 16 * g * n, (int)std::min<size_t>(16, m - 16 * g), (int)n, (int)grid);
+        for (size_t cg = 0; cg < col_groups; cg++)
+            hipLaunchKernelGGL(jq::q4k_rows16_mfma, dim3(grid), dim3(1024), 0, s, W + cg * (size_t)jq::QD_ROW,
+                               (const uint8_t *)(acts + g * group_bytes + 16 * cg * (size_t)jq::QM_REC), Y + 16 * g * n,
+                               (int)std::min<size_t>(16, m - 16 * g), (int)n, (int)grid, row_bytes, (int)(cg > 0));
     HIP_TRY(hipGetLastError());
     return 0;
 }

@@ -1,4 +1,5 @@
-// Q4_K matmul for 2..16 activation rows over 4096-wide weight rows: the weight stream of the one-row
+// Q4_K matmul for 2..16 activation rows over weight rows of 4096 columns (longer rows: one launch per
+// group of 4096 columns, the later ones adding to the result): the weight stream of the one-row
 // GEMV (q4k_gemv_dot4_lds: asynchronous loads into a ring of three 16-row tiles in LDS, one wave per
 // super-block column) with the integer dot products on the int8 matrix cores.
 //
@@ -71,8 +72,12 @@ __global__ __launch_bounds__(64) void q4k_acts16_prep(const float *__restrict__ 
 // super-block column w.  In the MFMAs the activations are the A operand and the weights the B operand, so
 // a lane ends up with weight row lane % 16 (whose eight sub-block scales it decodes for itself, four
 // bytes at a time) and activation rows 4 (lane / 16) .. + 3.  Y is m_rows x n.
+// W points at the first of the 16 super-blocks this launch covers in row 0, rows are row_bytes apart; with
+// `accumulate` the sums are added to what Y holds (rows longer than 4096: one launch per group of 4096
+// columns, in column order).
 __global__ __launch_bounds__(1024) void q4k_rows16_mfma(const uint8_t *__restrict__ W, const uint8_t *__restrict__ acts,
-                                                        float *__restrict__ Y, int m_rows, int n, int G) {
+                                                        float *__restrict__ Y, int m_rows, int n, int G,
+                                                        size_t row_bytes, int accumulate) {
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][QD_TILE_LDS];
     __shared__ float red[2][16 * QM_RED_STRIDE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -82,7 +87,7 @@ __global__ __launch_bounds__(1024) void q4k_rows16_mfma(const uint8_t *__restric
 
     auto fetch = [&](int i, int slot) __attribute__((always_inline)) {
         const int row = min(16 * ((int)blockIdx.x + min(i, n_tiles - 1) * G) + wave, n - 1);
-        const uint8_t *src = W + (size_t)row * QD_ROW + 16 * lane;
+        const uint8_t *src = W + (size_t)row * row_bytes + 16 * lane;
         const uint32_t dst = lds_offset_of(&ring[slot][wave * QD_ROW_LDS]);
         async_load16(src, dst);
         async_load16(src + 1024, dst + 1024);
@@ -183,7 +188,10 @@ __global__ __launch_bounds__(1024) void q4k_rows16_mfma(const uint8_t *__restric
             v = sum_xor16(v);
             v = sum_xor32(v);
             const int row = 16 * ((int)blockIdx.x + t * G) + r;
-            if (lane < 16 && wave < m_rows && row < n) Y[(size_t)wave * n + row] = v;
+            if (lane < 16 && wave < m_rows && row < n) {
+                float *yp = Y + (size_t)wave * n + row;
+                *yp = accumulate ? *yp + v : v;
+            }
         }
     }
 }

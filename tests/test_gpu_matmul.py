@@ -522,6 +522,32 @@ def test_threads_sharing_the_default_stream_get_their_own_results():
     assert not failures, failures
 
 
+@pytest.mark.parametrize("m,k,n", [(16, 12288, 4096), (3, 8192, 1030), (9, 16384, 1024), (40, 12288, 2050)])
+def test_q4k_few_rows_over_rows_of_several_4096_column_groups(m, k, n):
+    """Rows of 8192, 12288 and 16384: the 16-row kernel once per group of 4096 columns, the later launches
+    adding to the result; a dirty destination, wide-ranging activations, a non-finite one."""
+    blocks = make_blocks(capi.Q4_K, n, k, 71 + n)
+    rng = np.random.default_rng(n + m)
+    lhs = synth.normal(72 + n, (m, k))
+    lhs[0] *= (10.0 ** rng.integers(-5, 2, size=k // 32)).repeat(32).astype(np.float32)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    got = w.matmul_t(m, lhs, np.full(m * n, -7.25, np.float32))
+    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=True))
+    lhs[1, k - 5] = np.nan
+    bad = w.matmul_t(m, lhs)
+    assert np.isnan(bad[1]).all() and np.array_equal(bad[0], got[0])
+
+
+def test_q4k_few_rows_over_long_rows_integer_dot_products_are_bit_exact():
+    n, k, m = 1040, 12288, 7
+    blocks, q, x = q4k_integer_case(n, k, 17, group=32, big_value=32639, small=300)
+    xs = np.stack([np.roll(x, 32 * i) * (1 if i % 2 == 0 else -1) for i in range(m)])
+    want = xs @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, xs.astype(np.float32))
+    assert np.array_equal(got, want.astype(np.float32))
+
+
 def test_q4k_few_rows_over_a_view_of_the_stacked_tensor():
     """The 16-row kernel over a view that starts some rows into the allocation (an expert slice)."""
     n, k, m = 3000, 4096, 9
