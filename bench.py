@@ -455,10 +455,11 @@ def main() -> int:
         "metric": "Q4_K GEMV HBM GB/s (% of peak); decode tokens/s, 1 MI355X",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        # one row: 4-bit weights x two int8 activation planes on v_dot4 (int32 sums), f32 scales and result
-        "dtype": "int8" if m == 1 else "f16", "dtype_note": "integer dot products per 32-element sub-block "
+        # up to 64 rows: 4-bit weights x two int8 activation planes (v_dot4 for one row, int8 MFMA from two
+        # on; int32 sums), f32 scales and result; beyond: f16 MFMA GEMM
+        "dtype": "int8" if m <= 64 else "f16", "dtype_note": "integer dot products per 32-element sub-block "
         "(int4 weights x 15-bit fixed-point activations in two int8 planes), f32 scales and accumulation across sub-blocks"
-        if m == 1 else "f16 MFMA on exact integers (scale x nibble, 23-bit fixed-point activations in two planes), f32 result",
+        if m <= 64 else "f16 MFMA on exact integers (scale x nibble, 23-bit fixed-point activations in two planes), f32 result",
         "data": "synthetic",
         "config": {"workload": f"Q4_K matmul_t {N}x{K} (Llama-3-8B FFN-up), M={m}, f32 activations N(0,1), "
                                f"weights N(0,0.02) quantized to Q4_K, {len(weights)} weight copies rotated (cold HBM)",
