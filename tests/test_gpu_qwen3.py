@@ -108,6 +108,22 @@ def test_prefill_in_two_chunks_matches_one():
     assert ok, e
 
 
+@pytest.mark.parametrize("n_head,n_kv", [(4, 1), (4, 2), (2, 2)])
+def test_prefill_in_chunks_with_head_size_128(n_head, n_kv):
+    """Chunks of more than 8 tokens at a position past 0: the tiled attention with keys already in the
+    cache, token counts that leave the last tile part empty, and a chunk that starts inside a key tile."""
+    cfg = dict(CFG, n_ctx=96, n_layer=2, head_dim=128, n_head=n_head, n_kv_head=n_kv)
+    m, o = make(cfg, 27)
+    rng = np.random.default_rng(4)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=90)]
+    pos = 0
+    for step in (21, 16, 37, 9):
+        chunk = toks[pos:pos + step]
+        ok, e = close(m.forward(chunk, pos), o.forward(chunk, pos))
+        assert ok, f"pos {pos} +{step}: {e}"
+        pos += step
+
+
 @pytest.mark.parametrize("head_dim,n_head,n_kv", [(64, 4, 2), (128, 4, 1), (256, 2, 2), (192, 4, 2), (128, 8, 1),
                                                   (128, 2, 2), (128, 4, 2)])
 def test_decode_over_several_key_chunks(head_dim, n_head, n_kv):
