@@ -38,6 +38,25 @@ def rope_half_split(v: np.ndarray, pos0: int, theta: float) -> np.ndarray:
     return np.concatenate([a * c - b * s, a * s + b * c], axis=-1).astype(f32)
 
 
+def gqa_attention(q: np.ndarray, K: np.ndarray, V: np.ndarray, pos: int) -> np.ndarray:
+    """softmax(q K^T / sqrt(d) + causal mask) V per query head; q: [T, n_head, d] for the tokens at
+    positions pos .. pos + T - 1, K and V: [pos + T, n_kv_head, d], the whole cache.  Query head h reads
+    KV head h // (n_head / n_kv_head): repeat_kv lays the copies of a KV head side by side
+    (src/quantized_qwen3_moe.rs:267-278, :366-381); token t sees keys 0 .. pos + t (mask :776-789)."""
+    T, nh, d = q.shape
+    rep = nh // K.shape[1]
+    att = np.empty((T, nh, d), f32)
+    for hq in range(nh):
+        kv = hq // rep
+        sc = (q[:, hq, :] @ K[:, kv, :].T).astype(f32) / f32(np.sqrt(f32(d)))
+        mask = np.arange(K.shape[0])[None, :] > (pos + np.arange(T))[:, None]
+        sc = np.where(mask, f32(-np.inf), sc)
+        e = np.exp(sc - sc.max(axis=-1, keepdims=True), dtype=f32)
+        pr = (e / e.sum(axis=-1, keepdims=True, dtype=f32)).astype(f32)
+        att[:, hq, :] = pr @ V[:, kv, :]
+    return att
+
+
 class Qwen3Oracle:
     """cfg: dict with n_layer, hidden, n_head, n_kv_head, head_dim, ffn, vocab, rms_eps,
     rope_theta.  tensors: name -> (qtype, data) with qtype 0 for f32 vectors."""
@@ -83,17 +102,7 @@ class Qwen3Oracle:
             k = rope_half_split(rmsnorm(k, self.vec(p + ".attn_k_norm.weight"), c["rms_eps"]), pos, c["rope_theta"])
             self.k[l] = k if self.k[l] is None else np.concatenate([self.k[l], k], axis=0)
             self.v[l] = v if self.v[l] is None else np.concatenate([self.v[l], v], axis=0)
-            K, V = self.k[l], self.v[l]                      # [pos + T, nkv, d]
-            rep = nh // nkv
-            att = np.empty((T, nh, d), f32)
-            for hq in range(nh):
-                kv = hq // rep
-                sc = (q[:, hq, :] @ K[:, kv, :].T).astype(f32) / f32(np.sqrt(f32(d)))
-                mask = np.arange(K.shape[0])[None, :] > (pos + np.arange(T))[:, None]
-                sc = np.where(mask, f32(-np.inf), sc)
-                e = np.exp(sc - sc.max(axis=-1, keepdims=True), dtype=f32)
-                pr = (e / e.sum(axis=-1, keepdims=True, dtype=f32)).astype(f32)
-                att[:, hq, :] = pr @ V[:, kv, :]
+            att = gqa_attention(q, self.k[l], self.v[l], pos)
             x = (x + self.mm(p + ".attn_output.weight", att.reshape(T, nh * d), h)).astype(f32)
             hn = rmsnorm(x, self.vec(p + ".ffn_norm.weight"), c["rms_eps"])
             g = self.mm(p + ".ffn_gate.weight", hn, c["ffn"])

@@ -70,3 +70,43 @@ def test_shared_expert_is_added_for_every_token():
     x = synth.normal(13, (2, 256))
     diff = withs.forward(x) - base.forward(x)
     assert np.allclose(diff, withs.shared_mlp(x), atol=1e-5)
+
+
+def test_silu_by_value():
+    """x / (1 + exp(-x)) at points whose values are known: fails for sigmoid alone, for x * sigmoid(-x),
+    for gelu."""
+    from oracle.moe import silu
+    got = silu(np.array([0.0, 1.0, -1.0, 20.0, -20.0], np.float32))
+    assert got[0] == 0.0
+    assert got[1] == pytest.approx(0.7310585786, rel=1e-6)
+    assert got[2] == pytest.approx(-0.2689414214, rel=1e-6)
+    assert got[3] == pytest.approx(20.0, rel=1e-6) and abs(got[4]) < 1e-7
+
+
+def test_expert_mlp_is_down_of_silu_gate_times_up():
+    """One expert's MLP against float64 over the decoded weights, down (silu(gate x) * (up x))
+    (src/quantized_qwen3_moe.rs:397-401).  gate and up hold different bytes, so applying the activation to
+    up instead of gate, or dropping it, fails; so does reading another expert's slice."""
+    from scipy.special import expit
+    h, inter, E = 256, 64, 4
+    moe = tiny(h=h, inter=inter, E=E, seed=21)
+    x = synth.normal(22, (3, h))
+    for e in (0, 3):
+        def dec(blocks, n, k):
+            per = blocks.size // E
+            return oracle.dequantize(moe.qtype, blocks[e * per:(e + 1) * per]).reshape(n, k).astype(np.float64)
+        g, u = x.astype(np.float64) @ dec(moe.gate, inter, h).T, x.astype(np.float64) @ dec(moe.up, inter, h).T
+        want = (g * expit(g) * u) @ dec(moe.down, h, inter).T
+        got = moe.mlp(e, x)
+        assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1.0)
+        swapped = (u * expit(u) * g) @ dec(moe.down, h, inter).T
+        assert np.abs(swapped - want).max() > 1e-2 * np.abs(want).max()      # the check can tell them apart
+
+
+def test_decode_dispatch_is_the_weighted_sum_of_the_selected_experts():
+    """y = sum_s w_s mlp(e_s, x) over the router's k picks (src/quantized_qwen3_moe.rs:504-520)."""
+    moe = tiny(E=8, k=3, seed=31)
+    x = synth.normal(32, (1, 256))
+    idx, w = moe.route(x)
+    want = sum(float(w[0, s]) * moe.mlp(int(idx[0, s]), x).astype(np.float64) for s in range(3))
+    assert np.allclose(moe.forward(x), want, rtol=1e-5, atol=1e-6)

@@ -75,3 +75,134 @@ def test_prefill_equals_token_by_token():
         l3b = d.forward([t], i)
     assert np.allclose(l3, l3b, rtol=1e-4, atol=1e-4)
     assert not np.allclose(l3, la, atol=1e-3)
+
+
+# ---- attention: closed forms that fix the scale, the causal mask and the KV-head map ----------------
+# reference: src/quantized_qwen3_moe.rs:267-278 (repeat_kv), :366-381 (scores, mask, softmax, context),
+# :776-789 (mask).  Each case is a closed form, not the oracle's formula typed again, and each fails under
+# one of the plausible mistakes named in its docstring (checked by editing the oracle while writing them).
+
+def test_attention_with_equal_scores_averages_exactly_the_visible_values():
+    """All keys zero -> every visible key gets the same probability, whatever the scale: token t at
+    position pos + t must return the mean of value rows 0 .. pos + t.  Fails when the mask is off by one
+    (`>=` for `>`), ignores `pos`, or is missing."""
+    T, pos, nh, nkv, d = 3, 2, 4, 2, 8
+    q = normal(1, (T, nh, d)).astype(np.float32)
+    K = np.zeros((pos + T, nkv, d), np.float32)
+    V = normal(2, (pos + T, nkv, d)).astype(np.float32)
+    out = oq.gqa_attention(q, K, V, pos)
+    for t in range(T):
+        for h in range(nh):
+            want = V[:pos + t + 1, h // 2, :].astype(np.float64).mean(axis=0)
+            assert np.allclose(out[t, h], want, rtol=1e-6, atol=1e-6), (t, h)
+
+
+def test_attention_reads_kv_head_h_div_rep():
+    """Values of KV head 0 are all +1, of KV head 1 all -1: query heads 0, 1 must return +1 and heads 2, 3
+    -1 (copies of a KV head sit side by side).  Fails for `h % n_kv_head`, which would give +1 -1 +1 -1."""
+    T, pos, nh, nkv, d = 2, 1, 4, 2, 8
+    q = normal(3, (T, nh, d)).astype(np.float32)
+    K = normal(4, (pos + T, nkv, d)).astype(np.float32)
+    V = np.ones((pos + T, nkv, d), np.float32)
+    V[:, 1, :] = -1.0
+    out = oq.gqa_attention(q, K, V, pos)
+    assert np.allclose(out[:, :2, :], 1.0, atol=1e-6) and np.allclose(out[:, 2:, :], -1.0, atol=1e-6)
+    # and the keys come from the same KV head: make head 1's keys decide which value row wins
+    K2 = np.zeros((2, nkv, d), np.float32)
+    K2[1, 1, 0] = 50.0                       # only KV head 1 prefers key 1, strongly
+    V2 = np.zeros((2, nkv, d), np.float32)
+    V2[1, :, :] = 1.0                        # key 1's value row is all ones, key 0's all zeros
+    q2 = np.zeros((1, nh, d), np.float32)
+    q2[0, :, 0] = 1.0
+    o2 = oq.gqa_attention(q2, K2, V2, 1)
+    assert np.allclose(o2[0, :2], 0.5, atol=1e-6)        # KV head 0: equal scores
+    assert np.allclose(o2[0, 2:], 1.0, atol=1e-6)        # KV head 1: key 1 takes everything
+
+
+def test_attention_scale_is_one_over_sqrt_head_dim():
+    """One query against two keys with scores (a b, 0) before scaling: the weight of key 0 must be
+    1 / (1 + exp(-a b / sqrt(d))).  Fails without the scale (0.982 instead of 0.731 here), with 1 / d, or
+    with sqrt(d) multiplied instead of divided."""
+    d, a, b = 16, 2.0, 2.0
+    q = np.zeros((1, 1, d), np.float32)
+    q[0, 0, 0] = a
+    K = np.zeros((2, 1, d), np.float32)
+    K[0, 0, 0] = b
+    V = np.zeros((2, 1, d), np.float32)
+    V[0, 0, 0] = 1.0                                      # output[0] = weight of key 0
+    V[1, 0, 1] = 1.0                                      # output[1] = weight of key 1
+    out = oq.gqa_attention(q, K, V, 1)
+    p0 = 1.0 / (1.0 + np.exp(-a * b / np.sqrt(d)))
+    assert out[0, 0, 0] == pytest.approx(p0, rel=1e-6) and out[0, 0, 1] == pytest.approx(1.0 - p0, rel=1e-6)
+    assert p0 == pytest.approx(0.7310585786, rel=1e-9)    # a b / sqrt(d) = 1
+
+
+def test_attention_equals_an_f64_loop_over_heads_tokens_and_keys():
+    """Plain triple loop in float64 with distinguishable KV heads, 4 query heads on 2 KV heads, 3 tokens
+    behind 2 cached ones."""
+    T, pos, nh, nkv, d = 3, 2, 4, 2, 16
+    q = normal(5, (T, nh, d)).astype(np.float32)
+    K = normal(6, (pos + T, nkv, d)).astype(np.float32)
+    V = normal(7, (pos + T, nkv, d)).astype(np.float32)
+    out = oq.gqa_attention(q, K, V, pos)
+    for t in range(T):
+        for h in range(nh):
+            g = h // (nh // nkv)
+            s = [float(np.dot(q[t, h].astype(np.float64), K[j, g].astype(np.float64))) / np.sqrt(d) for j in range(pos + t + 1)]
+            w = np.exp(np.array(s) - max(s))
+            w /= w.sum()
+            want = sum(w[j] * V[j, g].astype(np.float64) for j in range(pos + t + 1))
+            assert np.allclose(out[t, h], want, rtol=1e-5, atol=1e-6), (t, h)
+
+
+def test_forward_equals_an_independent_f64_graph_over_decoded_weights():
+    """The whole decoder (1 layer) against a float64 graph written from the architecture's definition over
+    the decoded weights: pre-norm residual blocks, per-head q/k RMSNorm in front of the half-split rotation,
+    grouped-query attention, down(silu(gate) * up), last-token logits
+    (src/embedding.rs:297-396, src/quantized_qwen3_moe.rs:231-386,776-819).  Fails when gate and up are
+    swapped, a residual is dropped, the q/k norms come after the rotation, or the head norm weights swap."""
+    from scipy.special import expit, softmax
+    cfg = dict(CFG, n_layer=1)
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(cfg, 23)}
+    toks = [7, 301, 44, 12]
+    got = oq.Qwen3Oracle(cfg, tensors, avx2=oracle.have_avx2()).forward(toks, 0)
+
+    h, nh, nkv, d, ffn = cfg["hidden"], cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"], cfg["ffn"]
+
+    def W(name, n, k):
+        qt, blocks = tensors[name]
+        return oracle.dequantize(qt, blocks).reshape(n, k).astype(np.float64)
+
+    def vec(name):
+        return np.asarray(tensors[name][1], np.float64)
+
+    def norm(x, w):
+        return x / np.sqrt((x * x).mean(axis=-1, keepdims=True) + cfg["rms_eps"]) * w
+
+    def rot(v):                                            # [T, heads, d], positions 0 .. T-1
+        half = d // 2
+        out = v.copy()
+        for t in range(v.shape[0]):
+            for i in range(half):
+                ang = t * cfg["rope_theta"] ** (-2.0 * i / d)
+                a, b = v[t, :, i], v[t, :, i + half]
+                out[t, :, i], out[t, :, i + half] = a * np.cos(ang) - b * np.sin(ang), a * np.sin(ang) + b * np.cos(ang)
+        return out
+
+    T = len(toks)
+    x = W("token_embd.weight", cfg["vocab"], h)[toks]
+    hn = norm(x, vec("blk.0.attn_norm.weight"))
+    q = (hn @ W("blk.0.attn_q.weight", nh * d, h).T).reshape(T, nh, d)
+    k = (hn @ W("blk.0.attn_k.weight", nkv * d, h).T).reshape(T, nkv, d)
+    v = (hn @ W("blk.0.attn_v.weight", nkv * d, h).T).reshape(T, nkv, d)
+    q, k = rot(norm(q, vec("blk.0.attn_q_norm.weight"))), rot(norm(k, vec("blk.0.attn_k_norm.weight")))
+    kk, vv = np.repeat(k, nh // nkv, axis=1), np.repeat(v, nh // nkv, axis=1)      # side-by-side copies
+    sc = np.einsum("thd,shd->hts", q, kk) / np.sqrt(d) + np.triu(np.full((T, T), -np.inf), 1)[None]
+    ctx = np.einsum("hts,shd->thd", softmax(sc, axis=-1), vv).reshape(T, nh * d)
+    x = x + ctx @ W("blk.0.attn_output.weight", h, nh * d).T
+    hn = norm(x, vec("blk.0.ffn_norm.weight"))
+    g, u = hn @ W("blk.0.ffn_gate.weight", ffn, h).T, hn @ W("blk.0.ffn_up.weight", ffn, h).T
+    x = x + (g * expit(g) * u) @ W("blk.0.ffn_down.weight", h, ffn).T
+    want = norm(x[-1:], vec("output_norm.weight")) @ W("output.weight", cfg["vocab"], h).T
+    scale = np.abs(want).max()
+    assert np.abs(got - want[0]).max() <= 1e-3 * scale
