@@ -1973,7 +1973,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
     hipLaunchKernelGGL((jq::attention_tiles<128, GQ>), tgrid, dim3(64 * GQ), 0, s, qp, m->kc[l], m->vc[l], m->att, (int)T, \
                        nh, m->pos, (int)c.n_ctx, sqrt_d)
             if (no_tiles || d != 128 || (gq != 1 && gq != 2 && gq != 4 && gq != 8)) {
-                size_t sm = ((size_t)d + pos + T + 16) * sizeof(float);
+                size_t sm = ((size_t)d + jq::AR_CHUNK + 16) * sizeof(float);
                 hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, qp, m->kc[l], m->vc[l], m->att, nh,
                                    nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
             } else if (gq == 1) JQ_ATT_TILES(1);
@@ -2046,6 +2046,7 @@ int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out) {
         return fail("qwen3: zero in configuration");
     if (c.n_head % c.n_kv_head != 0) return fail("qwen3: %u query heads over %u kv heads", c.n_head, c.n_kv_head);
     if (c.head_dim % 8 != 0 || c.hidden % 4 != 0 || c.ffn % 4 != 0) return fail("qwen3: dimensions must be multiples of 4/8");
+    if (c.head_dim > (uint32_t)jq::AR_MAX_D) return fail("qwen3: head_dim %u exceeds %d", c.head_dim, jq::AR_MAX_D);
     if (ensure_init()) return 1;
     jq_model *m = new jq_model;
     m->cfg = c;

@@ -94,53 +94,71 @@ __global__ __launch_bounds__(64) void qkv_norm_rope_cache(float *__restrict__ q,
 
 // One workgroup per (token, query head): softmax(q . K^T / sqrt(d)) . V over the
 // keys 0 .. pos0 + t (causal), K/V of head hq / (n_head / n_kv)
-// (reference: src/quantized_qwen3_moe.rs:366-379; mask :776-789).
+// (reference: src/quantized_qwen3_moe.rs:366-379; mask :776-789).  The keys go by in chunks of
+// AR_CHUNK with a running maximum and sum (each chunk's scores wait in LDS, the value sums are rescaled
+// when the maximum moves), so the LDS a launch needs does not grow with the context.  d <= 4 * 256.
+constexpr int AR_CHUNK = 1024, AR_MAX_D = 1024;
+
 __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ q, const float *__restrict__ kc,
                                                        const float *__restrict__ vc, float *__restrict__ out,
                                                        int n_head, int n_kv, int d, const int *__restrict__ pos_ptr,
                                                        int n_ctx, float sqrt_d) {
-    extern __shared__ float sm[];  // q[d], scores[n_keys], red[16]
+    extern __shared__ float sm[];  // q[d], scores[AR_CHUNK], red[16]
     const int t = blockIdx.x / n_head, hq = blockIdx.x % n_head;
     const int kvh = hq / (n_head / n_kv), n_keys = *pos_ptr + t + 1;
-    float *qs = sm, *sc = sm + d, *red = sm + d + n_keys;
+    float *qs = sm, *sc = sm + d, *red = sm + d + AR_CHUNK;
     const float *qp = q + ((size_t)t * n_head + hq) * d;
     for (int c = threadIdx.x; c < d; c += blockDim.x) qs[c] = qp[c];
     __syncthreads();
-    const float *kb = kc + (size_t)kvh * n_ctx * d;
-    float mx = -INFINITY;
-    for (int j = threadIdx.x; j < n_keys; j += blockDim.x) {
-        const float *kr = kb + (size_t)j * d;
-        float acc = 0.0f;
-        for (int c = 0; c < d; c += 4) {
-            const float4 kv = ld<float4>((const uint8_t *)(kr + c));
-            acc = fmaf(qs[c], kv.x, acc);
-            acc = fmaf(qs[c + 1], kv.y, acc);
-            acc = fmaf(qs[c + 2], kv.z, acc);
-            acc = fmaf(qs[c + 3], kv.w, acc);
+    const float *kb = kc + (size_t)kvh * n_ctx * d, *vb = vc + (size_t)kvh * n_ctx * d;
+    float m_run = -INFINITY, l_run = 0.0f, acc[AR_MAX_D / 256] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j0 = 0; j0 < n_keys; j0 += AR_CHUNK) {
+        const int nj = min(AR_CHUNK, n_keys - j0);
+        float mx = -INFINITY;
+        for (int j = threadIdx.x; j < nj; j += blockDim.x) {
+            const float *kr = kb + (size_t)(j0 + j) * d;
+            float a = 0.0f;
+            for (int c = 0; c < d; c += 4) {
+                const float4 kv = ld<float4>((const uint8_t *)(kr + c));
+                a = fmaf(qs[c], kv.x, a);
+                a = fmaf(qs[c + 1], kv.y, a);
+                a = fmaf(qs[c + 2], kv.z, a);
+                a = fmaf(qs[c + 3], kv.w, a);
+            }
+            a = a / sqrt_d;  // the reference divides by sqrt(head_dim) (src/embedding.rs:386)
+            sc[j] = a;
+            mx = fmaxf(mx, a);
         }
-        acc = acc / sqrt_d;  // the reference divides by sqrt(head_dim) (src/embedding.rs:386)
-        sc[j] = acc;
-        mx = fmaxf(mx, acc);
+        mx = wave_max(mx);
+        __syncthreads();  // the previous chunk's readers of red are done
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+        __syncthreads();
+        for (int i = 0; i < (int)(blockDim.x >> 6); i++) mx = fmaxf(mx, red[i]);
+        const float m_new = fmaxf(m_run, mx), rescale = expf(m_run - m_new);  // exp(-inf) = 0 in front of the first chunk
+        float sum = 0.0f;
+        for (int j = threadIdx.x; j < nj; j += blockDim.x) {
+            const float e = expf(sc[j] - m_new);
+            sc[j] = e;
+            sum += e;
+        }
+        sum = block_sum(sum, red);
+        l_run = fmaf(l_run, rescale, sum);
+        m_run = m_new;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < AR_MAX_D / 256; i++) {
+            const int c = threadIdx.x + 256 * i;
+            if (c >= d) break;
+            float a = acc[i] * rescale;
+            for (int j = 0; j < nj; j++) a = fmaf(sc[j], vb[(size_t)(j0 + j) * d + c], a);
+            acc[i] = a;
+        }
+        __syncthreads();  // sc is rewritten by the next chunk
     }
-    mx = wave_max(mx);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
-    __syncthreads();
-    for (int i = 0; i < (int)(blockDim.x >> 6); i++) mx = fmaxf(mx, red[i]);
-    float sum = 0.0f;
-    for (int j = threadIdx.x; j < n_keys; j += blockDim.x) {
-        const float e = expf(sc[j] - mx);
-        sc[j] = e;
-        sum += e;
-    }
-    sum = block_sum(sum, red);
-    for (int j = threadIdx.x; j < n_keys; j += blockDim.x) sc[j] = sc[j] / sum;
-    __syncthreads();
-    const float *vb = vc + (size_t)kvh * n_ctx * d;
-    for (int c = threadIdx.x; c < d; c += blockDim.x) {
-        float acc = 0.0f;
-        for (int j = 0; j < n_keys; j++) acc = fmaf(sc[j], vb[(size_t)j * d + c], acc);
-        out[((size_t)t * n_head + hq) * d + c] = acc;
+#pragma unroll
+    for (int i = 0; i < AR_MAX_D / 256; i++) {
+        const int c = threadIdx.x + 256 * i;
+        if (c < d) out[((size_t)t * n_head + hq) * d + c] = acc[i] / l_run;
     }
 }
 
@@ -471,7 +489,12 @@ __global__ __launch_bounds__(128) void attention_merge(const float *__restrict__
 #pragma unroll
             for (int j = 0; j < 16; j++) v[j] = pp[(size_t)min(ch0 + j, n_chunks - 1) * (d + 2) + 2 + c];
 #pragma unroll
-            for (int j = 0; j < 16; j++) a = fmaf(ch0 + j < n_chunks ? wch[ch0 + j] : 0.0f, v[j], a);
+            for (int j = 0; j < 16; j++) {
+                // a chunk past a token's last key holds no sums, only whatever the buffer held before: its
+                // slots may be inf or NaN, and 0 * NaN is NaN, so such a chunk is left out, not weighted by 0
+                const float wgt = ch0 + j < n_chunks ? wch[ch0 + j] : 0.0f;
+                a = wgt > 0.0f ? fmaf(wgt, v[j], a) : a;
+            }
         }
         out[(size_t)blockIdx.x * d + c] = a / tot;
     }

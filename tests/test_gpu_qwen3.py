@@ -243,3 +243,47 @@ def test_single_token_steps_without_the_fused_launches(env):
     res = subprocess.run([sys.executable, "-c", FALLBACK_CHILD % root], env=dict(os.environ, **env), capture_output=True,
                          text=True, timeout=110)
     assert res.returncode == 0 and "fallback ok" in res.stdout, res.stdout + res.stderr
+
+
+def test_short_step_across_a_key_chunk_boundary_after_a_longer_context():
+    """A step of 2..8 tokens whose first tokens end before a 64-key chunk that its last tokens reach:
+    those tokens have no sums for that chunk, and the buffer of partial sums still holds an earlier,
+    longer context's values (laid out for more chunks, so its -inf markers sit where sums are read now).
+    The merge must leave such chunks out; weighting them by zero turns inf into NaN."""
+    cfg = dict(CFG, n_ctx=224, n_layer=2)
+    m, o = make(cfg, 35)
+    rng = np.random.default_rng(6)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=200)]
+    m.forward(toks[:124], 0)
+    m.forward(toks[124:132], 124)           # 3 chunks; tokens 0..3 stop at key 127 and skip the third
+    m.forward(toks[132:196], 132)
+    m.forward(toks[196:198], 196)           # 4 chunks: 196 keys for token 0 ... stride of the buffer changes
+    m.reset()
+    got, ref = m.forward(toks[:60], 0), o.forward(toks[:60], 0)
+    ok, e = close(got, ref)
+    assert ok, f"prefill: {e}"
+    for pos, step in ((60, 8), (68, 1), (69, 3)):     # 60 + 8 crosses key 64; tokens 0..3 skip chunk 1
+        chunk = toks[pos:pos + step]
+        got, ref = m.forward(chunk, pos), o.forward(chunk, pos)
+        assert np.all(np.isfinite(got)), f"pos {pos} +{step}: non-finite logits"
+        ok, e = close(got, ref)
+        assert ok, f"pos {pos} +{step}: {e}"
+
+
+def test_long_context_with_five_query_heads_a_kv_head():
+    """5 query heads a KV head take the one-row-per-workgroup attention for steps of more than 8 tokens;
+    its scores go by in chunks, so a context of more than 16384 keys (64 KB of scores a row) works.
+    Prefill in chunks of 2048 up to 16384 tokens, then a 16-token step whose rows see up to 16400 keys."""
+    cfg = dict(n_layer=1, hidden=256, n_head=5, n_kv_head=1, head_dim=64, ffn=256, vocab=256, n_ctx=16400 + 16,
+               rms_eps=1e-6, rope_theta=1e6)
+    m, o = make(cfg, 36, "8")            # Q8_0: blocks of 32 fit the 320-wide attention output
+    rng = np.random.default_rng(7)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=16400)]
+    pos = 0
+    while pos < 16384:
+        m.forward_only(toks[pos:pos + 2048], pos)
+        o.forward(toks[pos:pos + 2048], pos)
+        pos += 2048
+    got, ref = m.forward(toks[pos:pos + 16], pos), o.forward(toks[pos:pos + 16], pos)
+    ok, e = close(got, ref)
+    assert ok, e
