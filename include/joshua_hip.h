@@ -100,6 +100,22 @@ const void *jq_device_ptr(const jq_weight *w);
 int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, float *dst,
                 size_t dst_len, int ptrs_are_device, void *stream);
 
+/* jq_matmul_t for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+ * in the reference.  Same product, same kernels, device pointers only; what jq_matmul_t
+ * keeps in an allocation per stream (prepared activation operands, partial sums of a
+ * product split over k) lives in one fixed array of JQ_NOALLOC_SCRATCH_BYTES in each
+ * device's memory, held from library load until the process ends.  The call makes no
+ * hipMalloc / hipFree and fails, dst untouched, when the product needs more scratch than
+ * the array holds (one activation row never needs any; Q4_K needs about 9 KB per 16
+ * activation rows and 256 columns up to 256 rows and 4 m k bytes beyond; the other
+ * formats 4 m k bytes from 8 rows on; a product split over k adds 4 m n bytes a split).
+ * Every call on a device shares that device's array: calls whose kernels overlap on
+ * one device (two streams, two threads) race; calls on one stream are safe. */
+#define JQ_NOALLOC_SCRATCH_BYTES (32u << 20)
+int jq_matmul_t_noalloc(const jq_weight *w, size_t m, const float *lhs_dev, size_t lhs_len,
+                        float *dst_dev, size_t dst_len, void *stream);
+
 /* The free-function form over raw device-resident block bytes: runs the fused
  * kernel for `ggml_type` or declines (returns 1, dst untouched) when the type
  * has no kernel or nbytes is not a whole number of blocks

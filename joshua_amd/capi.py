@@ -26,7 +26,7 @@ TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "
 # Every symbol include/joshua_hip.h declares.
 EXPORTS = (
     "jq_last_error", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
-    "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_try_matmul_fused", "jq_dequantize",
+    "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_matmul_t_noalloc", "jq_try_matmul_fused", "jq_dequantize",
     "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
     "jq_mla_create", "jq_mla_free", "jq_mla_forward", "jq_mla_reset", "jq_mla_cached_tokens",
     "jq_qwen3_create", "jq_qwen3_free", "jq_qwen3_set_tensor", "jq_qwen3_forward", "jq_qwen3_greedy", "jq_qwen3_reset",
@@ -101,6 +101,7 @@ def lib() -> ctypes.CDLL:
         L.jq_device_ptr.argtypes = [vp]
         L.jq_device_ptr.restype = vp
         L.jq_matmul_t.argtypes = [vp, sz, vp, sz, vp, sz, i32, vp]
+        L.jq_matmul_t_noalloc.argtypes = [vp, sz, vp, sz, vp, sz, vp]
         L.jq_try_matmul_fused.argtypes = [u32, sz, sz, sz, vp, vp, sz, vp, vp]
         L.jq_dequantize.argtypes = [vp, vp, sz, i32, vp]
         L.jq_embedding.argtypes = [vp, vp, sz, vp, sz, i32, vp]
@@ -270,6 +271,10 @@ class Weight:
     # -- device-pointer calls (raw addresses; inputs already in HBM) -------------
     def matmul_t_dev(self, m: int, lhs_ptr: int, lhs_len: int, dst_ptr: int, dst_len: int, stream: int = 0) -> None:
         _check(lib().jq_matmul_t(self._h, m, lhs_ptr, lhs_len, dst_ptr, dst_len, 1, stream or None))
+
+    def matmul_t_noalloc(self, m: int, lhs_ptr: int, lhs_len: int, dst_ptr: int, dst_len: int, stream: int = 0) -> None:
+        """The same product through the entry point that allocates no device memory."""
+        _check(lib().jq_matmul_t_noalloc(self._h, m, lhs_ptr, lhs_len, dst_ptr, dst_len, stream or None))
 
 
 def try_matmul_fused(qtype: int, mkn, lhs_ptr: int, blocks_ptr: int, nbytes: int, dst_ptr: int, stream: int = 0) -> bool:

@@ -95,13 +95,43 @@ std::once_flag g_init_once;
 int g_init_rc = 0;
 int g_device = 0;
 
+}  // namespace
+
+// Scratch memory of jq_matmul_t_noalloc: a fixed array in every device's memory, held from the moment the
+// library is loaded on that device until the process ends.  Host code never uses the array's name as an
+// address (on the host it is a stand-in, not device memory): noalloc_scratch_on() asks the runtime for the
+// array's address on a device, once, with that device current, and every launch gets that pointer.
+static __device__ __align__(256) uint8_t scratch[JQ_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+uint8_t *g_scratch_ptr[MAX_DEVICES] = {};
+std::mutex g_scratch_mu[MAX_DEVICES];  // one call at a time enqueues launches that use a device's array
+std::mutex g_scratch_table_mu;
+
+// The address of `scratch` on `device`, which must be the current device.
+int noalloc_scratch_on(int device, uint8_t **out) {
+    if (device < 0 || device >= MAX_DEVICES) return fail("device %d is beyond the %d this library keeps scratch for", device, MAX_DEVICES);
+    std::lock_guard<std::mutex> g(g_scratch_table_mu);
+    if (!g_scratch_ptr[device]) {
+        void *p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail("hipGetSymbolAddress returned no address for the scratch array on device %d", device);
+        g_scratch_ptr[device] = (uint8_t *)p;
+    }
+    *out = g_scratch_ptr[device];
+    return 0;
+}
+
 int do_init(int device) {
     int count = 0;
     HIP_TRY(hipGetDeviceCount(&count));
     if (device < 0 || device >= count) return fail("jq_init: device %d out of range (%d visible)", device, count);
     HIP_TRY(hipSetDevice(device));
     g_device = device;
-    return 0;
+    uint8_t *p = nullptr;
+    return noalloc_scratch_on(device, &p);
 }
 
 int ensure_init() {
@@ -369,22 +399,42 @@ void launch_q4k_acts_prep(const float *X, size_t rows, size_t k, uint8_t *out, h
     hipLaunchKernelGGL(jq::q4k_acts_prep, dim3((unsigned)((units + 7) / 8)), dim3(256), 0, s, X, (int)rows, (int)k, out);
 }
 
-// Device memory for what one call's launches hand to each other (prepared activation operands), on
-// stream s.  Requests up to SCRATCH_KEEP bytes are served from one allocation per (device, stream), made
-// at first use, grown when a call needs more and kept until the process ends: the launches of a stream
-// run in order, so consecutive calls can share it, and a call pays no allocator round trip
+// Device memory for what one call's launches hand to each other (prepared activation operands, partial
+// sums of a product split over k), on stream s.  Requests up to SCRATCH_KEEP bytes are served from one
+// allocation per (device, stream), made at first use and kept until the process ends: the launches of a
+// stream run in order, so consecutive calls can share it, and a call pays no allocator round trip
 // (hipMallocAsync with hipFreeAsync takes some 18 us of host time a call, more than the kernels of a
-// small matmul take on the device).  The holder keeps that allocation's lock until it goes out of
-// scope, after the call's last launch is enqueued, so host threads that share a stream enqueue their
-// calls one after the other.  Larger requests are stream-ordered allocations, freed behind the call's
-// launches.  First use on a stream allocates, and growing waits for the stream: neither is possible
-// while the stream is being captured, so a caller warms a stream up before capturing it.
+// small matmul take on the device).  A call that needs more than the stream's buffer holds gets a new,
+// larger one; the old one is retired, not freed, because a HIP graph captured earlier on the stream
+// still names it (sizes at least double, so a stream retires at most a handful of buffers).  The holder
+// keeps that allocation's lock until it goes out of scope, after the call's last launch is enqueued, so
+// host threads that share a stream enqueue their calls one after the other.  Larger requests are
+// stream-ordered allocations, freed behind the call's launches.  First use and growth allocate: neither
+// is possible while the stream is being captured, so a caller warms a stream up with its largest call
+// before capturing it.
+//
+// jq_matmul_t_noalloc serves the same requests from a fixed array in device memory instead (below): it
+// installs the array for the calling thread with FixedScratchScope, and get() then hands out that
+// array, or fails when the request exceeds it, and never reaches an allocator.
 constexpr size_t SCRATCH_KEEP = 64u << 20;
 
 struct StreamBuffer {
     std::mutex mu;
     uint8_t *ptr = nullptr;
     size_t bytes = 0;
+    std::vector<uint8_t *> retired;
+};
+
+struct FixedScratch {
+    uint8_t *ptr = nullptr;
+    size_t bytes = 0;
+    std::mutex *mu = nullptr;
+};
+thread_local const FixedScratch *tl_fixed_scratch = nullptr;
+
+struct FixedScratchScope {
+    explicit FixedScratchScope(const FixedScratch *f) { tl_fixed_scratch = f; }
+    ~FixedScratchScope() { tl_fixed_scratch = nullptr; }
 };
 
 class CallScratch {
@@ -399,18 +449,26 @@ public:
     ~CallScratch() {
         if (transient_) (void)hipFreeAsync(transient_, stream_);
     }
-    hipError_t get(size_t bytes, hipStream_t s, uint8_t **out) {
+    // 0 on success; on failure the message is set
+    int get(size_t bytes, hipStream_t s, uint8_t **out) {
         stream_ = s;
+        if (const FixedScratch *f = tl_fixed_scratch) {
+            if (bytes > f->bytes)
+                return fail("this product needs %zu bytes of scratch memory; the entry point that allocates nothing "
+                            "holds %zu", bytes, f->bytes);
+            lock_ = std::unique_lock<std::mutex>(*f->mu);
+            *out = f->ptr;
+            return 0;
+        }
         if (bytes > SCRATCH_KEEP) {
-            hipError_t e = hipMallocAsync((void **)&transient_, bytes, s);
+            HIP_TRY(hipMallocAsync((void **)&transient_, bytes, s));
             *out = transient_;
-            return e;
+            return 0;
         }
         static std::mutex table_mu;
         static std::map<std::pair<int, hipStream_t>, std::unique_ptr<StreamBuffer>> table;
         int dev = 0;
-        hipError_t e = hipGetDevice(&dev);
-        if (e != hipSuccess) return e;
+        HIP_TRY(hipGetDevice(&dev));
         StreamBuffer *b;
         {
             std::lock_guard<std::mutex> g(table_mu);
@@ -420,17 +478,15 @@ public:
         }
         lock_ = std::unique_lock<std::mutex>(b->mu);
         if (b->bytes < bytes) {
-            if (b->ptr) {
-                if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
-                if ((e = hipFree(b->ptr)) != hipSuccess) return e;
-                b->ptr = nullptr, b->bytes = 0;
-            }
-            const size_t want = std::max<size_t>((bytes + 0xFFFFF) & ~(size_t)0xFFFFF, 1u << 20);
-            if ((e = hipMalloc((void **)&b->ptr, want)) != hipSuccess) return e;
-            b->bytes = want;
+            const size_t want = std::min(SCRATCH_KEEP, std::max<size_t>({(bytes + 0xFFFFF) & ~(size_t)0xFFFFF, 2 * b->bytes,
+                                                                          (size_t)1 << 20}));
+            uint8_t *fresh = nullptr;
+            HIP_TRY(hipMalloc((void **)&fresh, want));
+            if (b->ptr) b->retired.push_back(b->ptr);
+            b->ptr = fresh, b->bytes = want;
         }
         *out = b->ptr;
-        return hipSuccess;
+        return 0;
     }
 };
 
@@ -454,7 +510,7 @@ int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float 
     // the activations as MFMA operand records, in the call scratch of the stream
     CallScratch scratch;
     uint8_t *acts = nullptr;
-    HIP_TRY(scratch.get(m * nb * jq::QS_REC, s, &acts));
+    if (scratch.get(m * nb * jq::QS_REC, s, &acts)) return 1;
     launch_q4k_acts_prep(X, m, k, acts, s);
 #define JQ_RING(MAXNB)                                                                                              \
     hipLaunchKernelGGL((jq::q4k_ring_mfma<MAXNB, false, false>), dim3(grid), dim3(64 * (unsigned)nb), 0, s, W, nullptr, \
@@ -523,7 +579,7 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
     CallScratch scratch;
     uint8_t *acts = nullptr;
     const size_t cols = k / 256, group_bytes = cols * (size_t)jq::QM_REC;
-    HIP_TRY(scratch.get(groups * group_bytes, s, &acts));
+    if (scratch.get(groups * group_bytes, s, &acts)) return 1;
     hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, (unsigned)cols, (unsigned)groups), dim3(64), 0, s, X, (int)m, (int)k, acts);
     for (size_t g = 0; g < groups; g++)
         for (size_t cg = 0; cg < col_groups; cg++)
@@ -556,7 +612,7 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
     const size_t part_bytes = splits > 1 ? splits * m * n * sizeof(float) : 0;
     CallScratch scratch;
     uint8_t *buf = nullptr;
-    HIP_TRY(scratch.get(plane_bytes + min_bytes + part_bytes, s, &buf));
+    if (scratch.get(plane_bytes + min_bytes + part_bytes, s, &buf)) return 1;
     jq::Q4kGemmActs a;
     a.planes = (_Float16 *)buf;
     a.mins = (_Float16 *)(buf + plane_bytes);
@@ -591,7 +647,7 @@ int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, floa
     const size_t part_bytes = splits > 1 ? splits * m * n * sizeof(float) : 0;
     CallScratch scratch;
     uint8_t *buf = nullptr;
-    HIP_TRY(scratch.get(2 * plane + sbytes + part_bytes, s, &buf));
+    if (scratch.get(2 * plane + sbytes + part_bytes, s, &buf)) return 1;
     jq::ActsF16 a{(_Float16 *)buf, (_Float16 *)(buf + plane), (float *)(buf + 2 * plane)};
     float *parts = (float *)(buf + 2 * plane + sbytes);
     hipLaunchKernelGGL(jq::acts_f16_prep, dim3((unsigned)((m_pad * nc * 64 + 255) / 256)), dim3(256), 0, s, X, (int)m,
@@ -810,6 +866,22 @@ int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, 
     HIP_TRY(hipMemcpyAsync(dst, y.p, dst_len * sizeof(float), hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
     return 0;
+}
+
+int jq_matmul_t_noalloc(const jq_weight *w, size_t m, const float *lhs_dev, size_t lhs_len, float *dst_dev,
+                        size_t dst_len, void *stream) {
+    if (!w) return fail("jq_matmul_t_noalloc: weight is null");
+    if (validate(w->type, m, w->k, w->n, lhs_len, w->nbytes, dst_len)) return 1;
+    if (m == 0 || w->n == 0) return 0;
+    if (!lhs_dev || !dst_dev) return fail("jq_matmul_t_noalloc: lhs/dst is null");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    FixedScratch f;
+    if (noalloc_scratch_on(dev, &f.ptr)) return 1;  // resolved by jq_init; the first call on another device resolves it there
+    f.bytes = JQ_NOALLOC_SCRATCH_BYTES;
+    f.mu = &g_scratch_mu[dev];
+    FixedScratchScope scope(&f);
+    return dispatch_matmul(w->type, w->dev, w->row_bytes, lhs_dev, dst_dev, m, w->k, w->n, (hipStream_t)stream);
 }
 
 int jq_try_matmul_fused(uint32_t ggml_type, size_t m, size_t k, size_t n, const float *lhs_dev,

@@ -1,0 +1,62 @@
+"""jq_matmul_t_noalloc, the entry point that allocates no device memory, against jq_matmul_t on the
+same device-resident inputs.  Both run the same kernels, so the results are compared bit for bit
+(which is inside the 1e-3 bound of the other parity tests) and the first one of every pair also
+against the CPU oracle.  Each case makes two calls in a row, the second with fewer activation rows:
+the fixed scratch array keeps the first call's contents, and the second must not see them."""
+import numpy as np
+import pytest
+
+import oracle
+from joshua_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+
+
+def run_both(w, m, lhs):
+    import torch
+    x = torch.from_numpy(np.ascontiguousarray(lhs, dtype=np.float32)).cuda()
+    stream = torch.cuda.current_stream().cuda_stream
+    y_ref = torch.full((m, w.n), float("nan"), device="cuda")
+    y_new = torch.full((m, w.n), float("nan"), device="cuda")
+    w.matmul_t_dev(m, x.data_ptr(), x.numel(), y_ref.data_ptr(), y_ref.numel(), stream)
+    w.matmul_t_noalloc(m, x.data_ptr(), x.numel(), y_new.data_ptr(), y_new.numel(), stream)
+    torch.cuda.synchronize()
+    return y_ref.cpu().numpy(), y_new.cpu().numpy()
+
+
+CASES = [  # (format, k, n, first m, second m): shapes whose kernels keep operands or partial sums in scratch
+    (capi.Q4_K, 4096, 2048, 16, 5),      # 16-row int8 kernel: prepared activation operands
+    (capi.Q4_K, 4096, 1024, 96, 40),     # GEMM split over k: activation planes and partial sums
+    (capi.Q4_K, 1024, 512, 12, 3),       # streaming kernel (no scratch) and one row
+    (capi.Q6_K, 2048, 4096, 48, 9),      # GEMM over decoded weights, split over k
+    (capi.Q8_0, 4096, 4096, 1, 1),       # one row: no scratch at all
+]
+
+
+@pytest.mark.parametrize("qtype,k,n,m1,m2", CASES)
+def test_noalloc_matches_matmul_t_twice(qtype, k, n, m1, m2):
+    blocks = synth.normal_quantized(qtype, 31, n * k, 0.02)
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    for i, m in enumerate((m1, m2)):
+        lhs = synth.normal(40 + i, (m, k))
+        ref, new = run_both(w, m, lhs)
+        assert np.array_equal(ref.view(np.uint32), new.view(np.uint32)), (capi.TYPE_NAMES[qtype], m)
+        want = oracle.matmul_t(qtype, (m, k, n), lhs, blocks)
+        assert np.all(np.abs(new - want) <= TOL * np.maximum(np.abs(want), 1.0)), (capi.TYPE_NAMES[qtype], m)
+
+
+def test_noalloc_rejects_a_product_beyond_its_scratch():
+    import torch
+    k, n, m = 4096, 256, 4096            # the Q4_K GEMM wants 4 m k = 64 MiB of activation planes
+    w = capi.Weight.upload(capi.Q4_K, synth.normal_quantized(capi.Q4_K, 5, n * k, 0.02), n, k)
+    x = torch.zeros(m * k, device="cuda")
+    y = torch.full((m * n,), 7.0, device="cuda")
+    with pytest.raises(capi.JoshuaHipError, match="scratch"):
+        w.matmul_t_noalloc(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.all(y == 7.0)           # nothing written
+    # shape errors read like jq_matmul_t's
+    with pytest.raises(capi.JoshuaHipError, match="lhs/dst sized"):
+        w.matmul_t_noalloc(2, x.data_ptr(), k, y.data_ptr(), 2 * n, 0)
