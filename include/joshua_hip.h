@@ -59,6 +59,12 @@ typedef struct jq_weight jq_weight;
  * (replaces candle's Error::Msg strings). */
 const char *jq_last_error(void);
 
+/* Name of the kernel that the calling thread's last jq_matmul_t / jq_matmul_t_noalloc /
+ * jq_try_matmul_fused call chose ("" before the first one): which kernel serves a shape
+ * depends on measured crossover points, and tests pin the choice with this
+ * (no counterpart in the reference, which has one kernel per format). */
+const char *jq_last_kernel(void);
+
 /* Elements and bytes per block of a type id; nonzero for an unknown id
  * (reference: src/gguf_ext.rs:483-512 type_size_bytes). */
 int jq_block_geometry(uint32_t ggml_type, size_t *elems, size_t *bytes);

@@ -25,7 +25,7 @@ TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "
 
 # Every symbol include/joshua_hip.h declares.
 EXPORTS = (
-    "jq_last_error", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
+    "jq_last_error", "jq_last_kernel", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
     "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_matmul_t_noalloc", "jq_try_matmul_fused", "jq_dequantize",
     "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
     "jq_mla_create", "jq_mla_free", "jq_mla_forward", "jq_mla_reset", "jq_mla_cached_tokens",
@@ -87,6 +87,7 @@ def lib() -> ctypes.CDLL:
         L = ctypes.CDLL(LIB_PATH)
         sz, u32, vp, i32 = ctypes.c_size_t, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_int
         L.jq_last_error.restype = ctypes.c_char_p
+        L.jq_last_kernel.restype = ctypes.c_char_p
         L.jq_block_geometry.argtypes = [u32, ctypes.POINTER(sz), ctypes.POINTER(sz)]
         L.jq_init.argtypes = [i32]
         L.jq_upload.argtypes = [u32, vp, sz, sz, sz, i32, ctypes.POINTER(vp)]
@@ -164,6 +165,11 @@ def lib() -> ctypes.CDLL:
 
 def last_error() -> str:
     return lib().jq_last_error().decode()
+
+
+def last_kernel() -> str:
+    """The kernel the calling thread's last matmul call chose."""
+    return lib().jq_last_kernel().decode()
 
 
 def _check(rc: int) -> None:

@@ -22,6 +22,7 @@
 #include "kernels_mfma_q4k_gemm.hpp"
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
+#include "kernels_q4k_gemv_mfma.hpp"
 #include "kernels_dot4_q4k_r8.hpp"
 #include "kernels_dot4_q6k.hpp"
 #include "kernels_dot4_q8.hpp"
@@ -34,6 +35,9 @@
 namespace {
 
 thread_local char g_err[512] = "";
+// Name of the kernel the calling thread's last matmul dispatch chose (jq_last_kernel).
+thread_local const char *g_last_kernel = "";
+void note_kernel(const char *name) { g_last_kernel = name; }
 
 int fail(const char *fmt, ...) {
     va_list ap;
@@ -189,6 +193,7 @@ void launch_rows(const uint8_t *W, size_t row_bytes, const float *X, float *Y, s
             hipLaunchKernelGGL((jq::matmul_rows_valu<Q, MT>), grid, block, 0, s, W, row_bytes, X, Y, (int)m, (int)k,     \
                                (int)n);                                                                                  \
     } while (0)
+    note_kernel(gran ? "matmul_rows_staged" : "matmul_rows_valu");
     if (m == 1) JQ_LAUNCH_ROWS(1);
     else if (m == 2) JQ_LAUNCH_ROWS(2);
     else JQ_LAUNCH_ROWS(4);
@@ -248,6 +253,7 @@ int launch_q4k_mfma(const Q4kPlan &p, const uint8_t *W, size_t row_bytes, const 
     if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
     int tiles = (n + 15) / 16, tpw = p.waves / p.units_per_tile;
     size_t lds = (size_t)jq::q4k_lds_layout(k, MT, p.waves).total;
+    note_kernel("q4k_gemv_mfma");
     hipLaunchKernelGGL((jq::q4k_gemv_mfma<MT>), dim3((unsigned)((tiles + tpw - 1) / tpw)), dim3(64 * p.waves), lds, s, W,
                        row_bytes, X, Y, m0, m, k, n, p.units_per_tile);
     return 0;
@@ -292,6 +298,7 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
         // (4096 x 12288: 8.8 us; 4096 x 8192: 6.4 us against 6.8 us)
         const size_t tiles16 = (n + 15) / 16;
         if (tiles16 > 224 && tiles16 <= 256) {
+            note_kernel("q4k_gemv_dot4_cols");
             if (nb == 32) hipLaunchKernelGGL(jq::q4k_gemv_dot4_cols<2>, dim3(tiles16), dim3(1024), 0, s, W, X, Y, (int)n, (int)tiles16);
             else hipLaunchKernelGGL(jq::q4k_gemv_dot4_cols<3>, dim3(tiles16), dim3(1024), 0, s, W, X, Y, (int)n, (int)tiles16);
             HIP_TRY(hipGetLastError());
@@ -299,6 +306,7 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
         }
         const size_t tiles8 = (n + 7) / 8, rounds = (tiles8 + 255) / 256;
         const unsigned grid = (unsigned)((tiles8 + rounds - 1) / rounds);
+        note_kernel("q4k_gemv_dot4_r8");
         if (nb == 32) hipLaunchKernelGGL(jq::q4k_gemv_dot4_r8<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
         else hipLaunchKernelGGL(jq::q4k_gemv_dot4_r8<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
         HIP_TRY(hipGetLastError());
@@ -309,6 +317,18 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     const size_t tiles = (n + 15) / 16;
     if (mode != "regs") {
         if (nb != 16 || row_bytes != jq::QD_ROW) return -1;
+        // from 8192 rows on, the plain product runs its dot products on the int8 matrix cores (14336 rows:
+        // 7.35 against 7.9 us; 12288: 6.95 against 7.2; 65536: 25.2 against 26.3; 4096: 4.5 against 4.3 us)
+        static const char *mfma_env = getenv("JQ_Q4K_GEMV_MFMA");
+        static const size_t mfma_min_n = mfma_env ? (size_t)atoll(mfma_env) : 8192;
+        if (!norm && !swiglu && !genv && mfma_min_n > 0 && n >= mfma_min_n && n <= 0x7FFFFFF0ull) {
+            const size_t rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
+            const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
+            note_kernel("q4k_gemv_mfma_lds");
+            hipLaunchKernelGGL(jq::q4k_gemv_mfma_lds, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
+            HIP_TRY(hipGetLastError());
+            return 0;
+        }
         // a whole number of tiles per workgroup when the chip allows it (224 x 4 at 14336 rows)
         const size_t rounds = (tiles + 255) / 256;
         const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)atoi(genv) : (tiles + rounds - 1) / rounds);
@@ -316,6 +336,7 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     hipLaunchKernelGGL((jq::q4k_gemv_dot4_lds<NORM, SWIGLU>), dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid, \
                        NM.res, NM.w, NM.eps, NM.x_out, NM.hn_out)
         const jq::QdNorm none{};
+        note_kernel("q4k_gemv_dot4_lds");
         if (norm && swiglu) JQ_DOT4_LDS(true, true, (*norm));
         else if (norm) JQ_DOT4_LDS(true, false, (*norm));
         else if (swiglu) JQ_DOT4_LDS(false, true, none);
@@ -329,6 +350,7 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     // with an equal share of the rows
     const size_t cap = genv ? (size_t)atoi(genv) : 256 * std::max<size_t>(1, jq::QD_MAX_WAVES / nb);
     const unsigned grid = (unsigned)std::min<size_t>(tiles, std::max<size_t>(cap, 1));
+    note_kernel("q4k_gemv_dot4");
     hipLaunchKernelGGL(jq::q4k_gemv_dot4, dim3(grid), dim3((unsigned)(64 * nb)), 0, s, W, row_bytes, X, Y, (int)k, (int)n);
     HIP_TRY(hipGetLastError());
     return 0;
@@ -346,6 +368,7 @@ int dispatch_q6k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     if (tiles * ng < 512) return -1;  // under two steps a workgroup the staged f32 kernel is as fast (5.9 vs 4.5 us at 1024 x 4096)
     static const char *genv = getenv("JQ_Q6K_DOT4_GRID");
     const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)std::max(atoi(genv), 1) : (tiles + rounds - 1) / rounds);
+    note_kernel("q6k_gemv_dot4_lds");
     if (ng == 1) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
     else if (ng == 2) hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
     else hipLaunchKernelGGL(jq::q6k_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
@@ -364,6 +387,7 @@ int dispatch_q8_0_dot4(const uint8_t *W, size_t row_bytes, const float *X, float
     const size_t tiles = (n + jq::Q8D_ROWS - 1) / jq::Q8D_ROWS, rounds = (tiles + 255) / 256;
     if (tiles * ng < 512) return -1;  // under two steps a workgroup the staged f32 kernel is as fast
     const unsigned grid = (unsigned)std::min<size_t>(tiles, (tiles + rounds - 1) / rounds);
+    note_kernel("q8_0_gemv_dot4_lds");
     if (ng == 1) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<1>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
     else if (ng == 2) hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
     else hipLaunchKernelGGL(jq::q8_0_gemv_dot4_lds<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
@@ -385,6 +409,7 @@ int dispatch_q4k_stream(const uint8_t *W, size_t row_bytes, const float *X, floa
     static const char *genv = getenv("JQ_Q4K_STREAM_GRID");
     const size_t cap = genv ? (size_t)atoi(genv) : (cpw == 2 ? 256 : 512);
     const unsigned grid = (unsigned)std::min<size_t>(n_tiles, std::max<size_t>(cap, 1));
+    note_kernel("q4k_stream_mfma");
     if (cpw == 2)
         hipLaunchKernelGGL(jq::q4k_stream_mfma<2>, dim3(grid), dim3(64 * waves), 0, s, W, row_bytes, X, Y, (int)m, (int)k, (int)n);
     else
@@ -515,6 +540,7 @@ int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float 
 #define JQ_RING(MAXNB)                                                                                              \
     hipLaunchKernelGGL((jq::q4k_ring_mfma<MAXNB, false, false>), dim3(grid), dim3(64 * (unsigned)nb), 0, s, W, nullptr, \
                        nullptr, acts, nullptr, nullptr, nullptr, nullptr, Y, (int)m, (int)n, jq::MoeClamp{})
+    note_kernel("q4k_ring_mfma");
     if (maxnb == 16) JQ_RING(16);
     else if (maxnb == 8) JQ_RING(8);
     else JQ_RING(4);
@@ -580,6 +606,7 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
     uint8_t *acts = nullptr;
     const size_t cols = k / 256, group_bytes = cols * (size_t)jq::QM_REC;
     if (scratch.get(groups * group_bytes, s, &acts)) return 1;
+    note_kernel("q4k_rows16_mfma");
     hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, (unsigned)cols, (unsigned)groups), dim3(64), 0, s, X, (int)m, (int)k, acts);
     for (size_t g = 0; g < groups; g++)
         for (size_t cg = 0; cg < col_groups; cg++)
@@ -618,6 +645,7 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
     a.mins = (_Float16 *)(buf + plane_bytes);
     float *parts = (float *)(buf + plane_bytes + min_bytes);
     const size_t units = m_pad * nb;
+    note_kernel(splits > 1 ? "q4k_gemm_mfma+splitk" : "q4k_gemm_mfma");
     hipLaunchKernelGGL(jq::q4k_gemm_prep, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, X, (int)m, (int)m_pad, (int)k, a);
     hipLaunchKernelGGL(jq::q4k_gemm_mfma, dim3((unsigned)(base_grid * splits)), dim3(512), 0, s, W, row_bytes, a,
                        splits > 1 ? parts : Y, (int)m, (int)m_pad, (int)k, (int)n, (int)m_tiles, (int)total, (int)splits,
@@ -650,6 +678,7 @@ int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, floa
     if (scratch.get(2 * plane + sbytes + part_bytes, s, &buf)) return 1;
     jq::ActsF16 a{(_Float16 *)buf, (_Float16 *)(buf + plane), (float *)(buf + 2 * plane)};
     float *parts = (float *)(buf + 2 * plane + sbytes);
+    note_kernel(splits > 1 ? "gemm_decoded_mfma+splitk" : "gemm_decoded_mfma");
     hipLaunchKernelGGL(jq::acts_f16_prep, dim3((unsigned)((m_pad * nc * 64 + 255) / 256)), dim3(256), 0, s, X, (int)m,
                        (int)m_pad, (int)k, a);
     hipLaunchKernelGGL(jq::gemm_decoded_mfma<Q>, dim3((unsigned)n_tiles, (unsigned)m_tiles, (unsigned)splits), dim3(256), 0, s, W,
@@ -773,6 +802,7 @@ struct DevBuf {
 extern "C" {
 
 const char *jq_last_error(void) { return g_err; }
+const char *jq_last_kernel(void) { return g_last_kernel; }
 
 int jq_block_geometry(uint32_t ggml_type, size_t *elems, size_t *bytes) {
     Geometry g;

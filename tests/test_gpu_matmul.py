@@ -680,3 +680,115 @@ def test_q4k_gemv_kernels_selected_by_environment(mode):
     env = dict(os.environ, JQ_Q4K_DOT4=mode)
     res = subprocess.run([sys.executable, "-c", DOT4_CHILD % root], env=env, capture_output=True, text=True, timeout=110)
     assert res.returncode == 0 and "dot4 ok" in res.stdout, res.stdout + res.stderr
+
+
+# ---- the int8 matrix-core GEMV for one activation row (4096-wide rows, 8192 weight rows and more) ----
+
+@pytest.mark.parametrize("n", [8192, 8192 + 5, 14336, 16 * 256 * 5 + 16 * 3 + 7, 65536 + 31])
+def test_q4k_mfma_gemv_row_counts(n):
+    """Row counts that give the workgroups equal and unequal numbers of tiles, more than four tiles a
+    workgroup (the ring and the partial sums wrap) and a ragged last tile."""
+    k = 4096
+    blocks = make_blocks(capi.Q4_K, n, k, 300 + n % 97)
+    lhs = synth.normal(301, (1, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, lhs)
+    assert capi.last_kernel() == "q4k_gemv_mfma_lds"
+    assert close(got, oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+def test_q4k_mfma_gemv_integer_dot_products_are_bit_exact():
+    """Activation range 32639 per 32-element sub-block, as in the v_dot4 kernel: the sums of the low-nibble
+    sub-blocks come straight from the matrix cores, those of the high-nibble sub-blocks as
+    (16 sum h X - 128 XS + 128 XS) / 16, all in integers."""
+    n, k = 8192 + 48, 4096
+    blocks, q, x = q4k_integer_case(n, k, 17, group=32, big_value=32639, small=4000)
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+    assert capi.last_kernel() == "q4k_gemv_mfma_lds"
+    assert np.array_equal(got[0], (x @ q.T).astype(np.float32))
+    # every nibble value at every position of a chunk, negative and positive activations: random bytes
+    rng = np.random.default_rng(3)
+    raw = rng.integers(0, 256, size=n * 16 * 144, dtype=np.uint8).reshape(-1, 144)
+    raw[:, 0:4] = np.frombuffer(np.float16([1.0, 1.0]).tobytes(), np.uint8)          # d = dmin = 1
+    xi = rng.integers(-32639, 32640, size=k).astype(np.int64)
+    xi[::32] = 32639                                                                 # scale exactly 1 per sub-block
+    w = oracle.dequantize(capi.Q4_K, raw.reshape(-1)).reshape(n, k).astype(np.int64)  # integers: sc q - m
+    want = w @ xi
+    got = capi.Weight.upload(capi.Q4_K, raw.reshape(-1), n, k).matmul_t(1, xi[None, :].astype(np.float32))
+    # sums reach 2^31: compare in f64 at f32 resolution of the per-block terms instead of bit for bit
+    assert np.all(np.abs(got[0].astype(np.float64) - want) <= 2.0 ** -20 * np.abs(w).astype(np.float64) @ np.abs(xi))
+
+
+def test_q4k_mfma_gemv_non_finite_and_wide_range_activations():
+    n, k = 8192, 4096
+    blocks = make_blocks(capi.Q4_K, n, k, 311)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    rng = np.random.default_rng(9)
+    lhs = synth.normal(312, (1, k))
+    lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 16)).repeat(16).astype(np.float32)
+    # Magnitudes from 1e-6 to 1e6 inside one row: among 8192 rows some results cancel to a thousandth of
+    # their terms, where no f32 summation order agrees with another to 1e-3 of the result.  The bound is
+    # taken against the sum of the terms' magnitudes instead: 16-bit fixed point per 32 elements stays
+    # below 2^-16 of it, and so must the kernel.
+    wd = oracle.dequantize(capi.Q4_K, blocks).reshape(n, k).astype(np.float64)
+    want, mag = wd @ lhs[0].astype(np.float64), np.abs(wd) @ np.abs(lhs[0].astype(np.float64))
+    got = w.matmul_t(1, lhs)[0].astype(np.float64)
+    assert np.all(np.abs(got - want) <= 2.0 ** -16 * mag)
+    big = np.abs(want) >= 0.05 * mag          # rows without much cancellation: the usual bound
+    assert big.sum() > n // 4 and np.all(np.abs(got - want)[big] <= TOL * np.abs(want)[big])
+    for bad in (np.inf, -np.inf, np.nan):
+        lhs = synth.normal(313, (1, k))
+        lhs[0, 777] = bad
+        got = w.matmul_t(1, lhs)
+        assert capi.last_kernel() == "q4k_gemv_mfma_lds"
+        assert np.all(np.isnan(got))            # every row has weights in that sub-block
+
+
+def test_q4k_mfma_gemv_switched_off_by_environment():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    child = ("import sys; sys.path.insert(0, %r)\n"
+             "import numpy as np, oracle\nfrom joshua_amd import capi, synth\n"
+             "n, k = 8192, 4096\nb = synth.normal_quantized(capi.Q4_K, 5, n * k, 0.02)\nx = synth.normal(6, (1, k))\n"
+             "got = capi.Weight.upload(capi.Q4_K, b, n, k).matmul_t(1, x)\n"
+             "assert capi.last_kernel() == 'q4k_gemv_dot4_lds', capi.last_kernel()\n"
+             "want = oracle.matmul_t(capi.Q4_K, (1, k, n), x, b, avx2=oracle.have_avx2())\n"
+             "assert np.all(np.abs(got - want) <= 1e-3 * np.maximum(np.abs(want), 1.0))\nprint('ok')\n") % root
+    res = subprocess.run([sys.executable, "-c", child], env=dict(os.environ, JQ_Q4K_GEMV_MFMA="0"), capture_output=True,
+                         text=True, timeout=110)
+    assert res.returncode == 0 and "ok" in res.stdout, res.stdout + res.stderr
+
+
+KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (format, m, k, n) -> jq_last_kernel()
+    (capi.Q4_K, 1, 4096, 14336, "q4k_gemv_mfma_lds"),        # headline
+    (capi.Q4_K, 1, 4096, 4096, "q4k_gemv_dot4_lds"),
+    (capi.Q4_K, 1, 12288, 4096, "q4k_gemv_dot4_cols"),       # a feed-forward down projection
+    (capi.Q4_K, 1, 8192, 2048, "q4k_gemv_dot4_r8"),
+    (capi.Q4_K, 1, 2048, 768, "q4k_gemv_mfma"),              # an expert's gate projection
+    (capi.Q4_K, 2, 2048, 768, "q4k_gemv_mfma"),
+    (capi.Q4_K, 16, 4096, 14336, "q4k_rows16_mfma"),
+    (capi.Q4_K, 16, 2048, 768, "q4k_stream_mfma"),
+    (capi.Q4_K, 512, 4096, 14336, "q4k_gemm_mfma"),
+    (capi.Q4_K, 512, 4096, 1024, "q4k_gemm_mfma+splitk"),
+    (capi.Q8_0, 1, 4096, 4096, "q8_0_gemv_dot4_lds"),
+    (capi.Q6_K, 1, 12288, 4096, "q6k_gemv_dot4_lds"),
+    (capi.Q6_K, 1, 1024, 4096, "matmul_rows_staged"),
+    (capi.Q6_K, 64, 4096, 1024, "gemm_decoded_mfma+splitk"),
+    (capi.Q2_K, 1, 7680, 2048, "matmul_rows_staged"),
+    (capi.MXFP4, 1, 7168, 2048, "matmul_rows_staged"),
+    (capi.IQ2_XXS, 1, 7168, 2048, "matmul_rows_staged"),
+]
+
+
+@pytest.mark.parametrize("qtype,m,k,n,kernel", KERNEL_OF_SHAPE)
+def test_kernel_chosen_for_a_shape(qtype, m, k, n, kernel):
+    """The dispatcher's crossover points are measured constants; this pins what they select, so that a
+    parity test named after a kernel keeps covering that kernel."""
+    import torch
+    blocks = make_blocks(qtype, n, k, 400)
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    x = torch.zeros(m * k, device="cuda")
+    y = torch.zeros(m * n, device="cuda")
+    w.matmul_t_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert capi.last_kernel() == kernel
