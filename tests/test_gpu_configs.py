@@ -132,3 +132,42 @@ def test_single_token_steps_at_qwen3_8b_layer_sizes():
             assert m.greedy() == oq.greedy(ref)
         pos += 1
     m.close()
+
+
+def test_mla_at_deepseek_v3_size():
+    """Multi-head latent attention with DeepSeek-V3's dimensions (7168 wide, 128 heads, query rank 1536,
+    latent 512 + 64 rope, YaRN factor 40; src/quantized_deepseek2.rs:357-499): a 200-token prefill in two
+    chunks, then single-token steps, absorbed device form against the reference's unabsorbed form."""
+    from tests.test_gpu_mla import build, cfg, close as mla_close
+    c = cfg(n_embd=7168, n_head=128, q_lora_rank=1536, kv_lora_rank=512, qk_nope=128, qk_rope=64, v_head_dim=128,
+            context_length=256, yarn=dict(factor=40.0, orig_context_length=4096, mscale_all_dim=1.0))
+    ref, dev = build(c, qtype=capi.Q4_K, seed=900)
+    x = synth.normal(901, (204, c["n_embd"]))
+    assert mla_close(dev.forward(x[:128], 0), ref.forward(x[:128], 0))
+    assert mla_close(dev.forward(x[128:200], 128), ref.forward(x[128:200], 128))
+    for p in range(200, 204):
+        assert mla_close(dev.forward(x[p:p + 1], p), ref.forward(x[p:p + 1], p))
+
+
+def test_group_limited_routing_at_deepseek_v3_size():
+    """256 experts in 8 groups, 4 groups kept, top-8, sigmoid scores with a selection bias, weights scaled
+    by 2.5 (src/quantized_deepseek2.rs:527-597): ids and weights of 33 tokens against the oracle."""
+    h, E = 7168, 256
+    router = synth.normal(910, (E, h), 0.02)
+    bias = synth.normal(911, (E,), 0.01)
+    tiny = synth.normal_quantized(capi.Q8_0, 912, E * 32 * h, 0.02)      # experts are not exercised here
+    down = synth.normal_quantized(capi.Q8_0, 913, E * h * 32, 0.02)
+    ora = MoeOracle(capi.Q8_0, h, 32, E, 8, router, tiny, tiny, down, gating="sigmoid", norm_topk=True,
+                    weights_scale=2.5, n_group=8, topk_group=4, router_bias=bias)
+    cfg_ = capi.MoeConfig(E, 8, h, 32, 1, 1, 2.5, 8, 4, 0.0, 0.0)
+    g = capi.Weight.upload(capi.Q8_0, tiny, E * 32, h)
+    d = capi.Weight.upload(capi.Q8_0, down, E * h, 32)
+    layer = capi.Moe(cfg_, router, g, g, d, router_bias=bias)
+    x = synth.normal(914, (33, h))
+    ids, w = layer.route(x)
+    oid, ow = ora.route(x)
+    assert np.array_equal(ids, oid)
+    assert np.allclose(w, ow, rtol=2e-5, atol=1e-7)
+    for t in range(33):                      # the picks really sit in 4 of the 8 groups
+        assert len({int(e) // 32 for e in ids[t]}) <= 4
+    layer.close()
