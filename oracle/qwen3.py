@@ -12,6 +12,8 @@ and exact agreement of the greedy token only where the top-2 margin exceeds it.
 """
 from __future__ import annotations
 
+import time
+
 import numpy as np
 
 from . import dequantize, matmul_t
@@ -69,11 +71,15 @@ class Qwen3Oracle:
         self.k = [None] * self.c["n_layer"]
         self.v = [None] * self.c["n_layer"]
         self.n_past = 0
+        self.mm_seconds = 0.0   # time spent inside the C matmul kernels (the rest is this numpy graph)
 
     def mm(self, name: str, x: np.ndarray, n: int) -> np.ndarray:
         qt, blocks = self.t[name]
         m, k = x.shape
-        return matmul_t(qt, (m, k, n), np.ascontiguousarray(x, f32), blocks, avx2=self.avx2, threads=self.threads)
+        t0 = time.perf_counter()
+        y = matmul_t(qt, (m, k, n), np.ascontiguousarray(x, f32), blocks, avx2=self.avx2, threads=self.threads)
+        self.mm_seconds += time.perf_counter() - t0
+        return y
 
     def vec(self, name: str) -> np.ndarray:
         return np.asarray(self.t[name][1], f32)
