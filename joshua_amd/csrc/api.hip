@@ -22,7 +22,7 @@
 #include "kernels_mfma_q4k_gemm.hpp"
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
-#include "kernels_q4k_gemv_mfma.hpp"
+#include "kernels_gemv_mfma.hpp"
 #include "kernels_dot4_q4k_r8.hpp"
 #include "kernels_dot4_q6k.hpp"
 #include "kernels_dot4_q8.hpp"
@@ -325,7 +325,7 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
             const size_t rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
             const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
             note_kernel("q4k_gemv_mfma_lds");
-            hipLaunchKernelGGL(jq::q4k_gemv_mfma_lds, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
+            hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ4K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
             HIP_TRY(hipGetLastError());
             return 0;
         }
@@ -352,6 +352,21 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     const unsigned grid = (unsigned)std::min<size_t>(tiles, std::max<size_t>(cap, 1));
     note_kernel("q4k_gemv_dot4");
     hipLaunchKernelGGL(jq::q4k_gemv_dot4, dim3(grid), dim3((unsigned)(64 * nb)), 0, s, W, row_bytes, X, Y, (int)k, (int)n);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// Q2_K, one activation row, rows of 4096: the int8 matrix-core GEMV.  Returns -1 when the shape is outside
+// its reach.  JQ_Q2K_GEMV_MFMA = 0 switches it off.
+int dispatch_q2k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
+    static const char *mode = getenv("JQ_Q2K_GEMV_MFMA");
+    if ((mode && mode[0] == '0') || k != 4096 || row_bytes != (size_t)jq::QvQ2K::ROW || ((uintptr_t)W & 15) != 0 ||
+        ((uintptr_t)X & 15) != 0 || n < 256 || n > 0x7FFFFFF0ull)
+        return -1;
+    const size_t tiles = (n + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
+    const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
+    note_kernel("q2k_gemv_mfma_lds");
+    hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ2K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -710,6 +725,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     }
     if (type == JQ_TYPE_Q6_K && m == 1) {
         const int rc = dispatch_q6k_dot4(W, row_bytes, X, Y, k, n, s);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q2_K && m == 1) {
+        const int rc = dispatch_q2k_mfma(W, row_bytes, X, Y, k, n, s);
         if (rc >= 0) return rc;
     }
     if (type == JQ_TYPE_Q8_0 && m == 1) {

@@ -1,5 +1,9 @@
-// Q4_K GEMV for one activation row over weight rows of 4096 columns with the integer dot products on the
-// int8 matrix cores.
+// GEMV for one activation row over weight rows of 4096 columns (16 super-blocks of 256) with the integer
+// dot products on the int8 matrix cores: one kernel (gemv_mfma_lds<F>, at the end of the file) over a
+// per-format policy F that says how a row's bytes are laid out, how a lane's operands are made from the
+// wave's 256 activations and how a super-block is multiplied.  Policies: QvQ4K and QvQ2K.
+//
+// ---- Q4_K ----
 //
 // Per 32-element sub-block j of a weight row (reference arithmetic w = d sc q - dmin m,
 // src/kquant_dot.rs:440-465):
@@ -118,23 +122,132 @@ __device__ __forceinline__ float qv_block_dot(const uint8_t *blk, const QvActs &
     return sum_xor32(acc);
 }
 
+// The Q4_K policy.
+struct QvQ4K {
+    static constexpr int BLOCK = 144, ROW = 16 * BLOCK, ROW_LDS = QD_ROW_LDS;  // rows 16 bytes apart in banks
+    static constexpr int STAGE_BYTES = 1152;  // what prepare() uses of `stage`
+    typedef QvActs Acts;
+    __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) { return qv_prepare(v, stage, lane); }
+    __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) { return qv_block_dot(blk, a, c); }
+};
+
+// ---- Q2_K ----
+//
+// Block of 84 bytes: scales[16] | qs[64] | d | dmin; element 128 sg + 32 f + l (l < 32) is the two-bit
+// field f of byte qs[32 sg + l], and the 16 elements 128 sg + 32 f + 16 hf + [0, 16) share the scale byte
+// scales[8 sg + 2 f + hf]: w = d (sc & 15) q - dmin (sc >> 4)  (reference: src/kquant_dot.rs:326-400).
+// Lane (r, c) takes bytes 16c .. 16c+15 of the block's qs, i.e. super-group c / 2, byte half c % 2: one
+// 16-element scale group per field.  Four MFMAs a block, one per field, with B = the field where it sits
+// (q & 0x03, q & 0x0C = 4 f1, q & 0x30 = 16 f2; the top field shifted down) and the powers of four taken
+// back through the activation scale; A row 4c + plane is non-zero in lane group c only, so a lane receives
+// the two plane sums of its own group.  The activations are 16-bit fixed point per 32 elements, as for Q4_K;
+// the min term needs their sums per 16.
+struct Q2Acts {
+    qv_i4 a[4];         // A operand per field
+    float s[4], xs[4];  // per field: activation scale of its 32 elements (over 1, 4, 16, 1), scale x sum of the lane's 16
+};
+
+struct QvQ2K {
+    static constexpr int BLOCK = 84, ROW = 16 * BLOCK, ROW_LDS = ROW + 16;  // 340 words: 16 rows x 4 words fill the 64 banks
+    static constexpr int STAGE_BYTES = 640;
+    typedef Q2Acts Acts;
+    __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) {
+        const int r = lane & 15, c = lane >> 4;
+        float *stage_f = (float *)(stage + 128);  // [0,8) scales of the 32-element sub-blocks, [8,24) scale x sum per 16
+        {
+            float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
+            amax = max_row8(amax);
+            const bool live = amax > 0.0f && amax < INFINITY;
+            const float inv = live ? QD_RANGE / amax : 0.0f, s = fixed_scale(amax, QD_RANGE);
+            const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                               __float2int_rn(v.w * inv)};
+            uint32_t wl = 0, wh = 0;
+            int sum = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                wl |= (uint32_t)(Xq[i] & 255) << (8 * i);
+                wh |= (uint32_t)(((Xq[i] + 128) >> 8) & 255) << (8 * i);
+                sum += Xq[i];
+            }
+            stage[lane] = wl, stage[64 + lane] = wh;
+            sum += dpp_i<0xB1>(sum);  // the four lanes of a 16-element group
+            sum += dpp_i<0x4E>(sum);
+            if ((lane & 7) == 0) stage_f[lane >> 3] = s;
+            if ((lane & 3) == 0) stage_f[8 + (lane >> 2)] = s * (float)sum;
+        }
+        Acts a;
+        const int cm = r >> 2, pl = r & 3;  // A row m = 4 cm + plane
+        const bool mine = cm == c && pl < 2;
+        const uint4 z = uint4{0, 0, 0, 0};
+#pragma unroll
+        for (int f = 0; f < 4; f++) {
+            // elements 128 (c / 2) + 32 f + 16 (c % 2) + [0, 16): words 32 (c / 2) + 8 f + 4 (c % 2) of the plane
+            const uint4 w = mine ? *(const uint4 *)(stage + 64 * (pl & 1) + 32 * (c >> 1) + 8 * f + 4 * (c & 1)) : z;
+            a.a[f] = qv_i4{(int)w.x, (int)w.y, (int)w.z, (int)w.w};
+            const float pw = f == 1 ? 0.25f : (f == 2 ? 0.0625f : 1.0f);
+            a.s[f] = stage_f[4 * (c >> 1) + f] * pw;
+            a.xs[f] = stage_f[8 + 8 * (c >> 1) + 2 * f + (c & 1)];
+        }
+        return a;
+    }
+    __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) {
+        // blocks sit at multiples of 84 bytes: everything is read as aligned 32-bit words
+        const uint32_t *w32 = (const uint32_t *)blk;
+        const uint32_t sc0 = w32[2 * (c >> 1)] >> (8 * (c & 1)), sc1 = w32[2 * (c >> 1) + 1] >> (8 * (c & 1));
+        const uint32_t q[4] = {w32[4 + 4 * c], w32[5 + 4 * c], w32[6 + 4 * c], w32[7 + 4 * c]};
+        const uint32_t dd = w32[20];
+        const qv_i4 zero = qv_i4{0, 0, 0, 0};
+        const qv_i4 b0 = qv_i4{(int)(q[0] & 0x03030303u), (int)(q[1] & 0x03030303u), (int)(q[2] & 0x03030303u), (int)(q[3] & 0x03030303u)};
+        const qv_i4 b1 = qv_i4{(int)(q[0] & 0x0C0C0C0Cu), (int)(q[1] & 0x0C0C0C0Cu), (int)(q[2] & 0x0C0C0C0Cu), (int)(q[3] & 0x0C0C0C0Cu)};
+        const qv_i4 b2 = qv_i4{(int)(q[0] & 0x30303030u), (int)(q[1] & 0x30303030u), (int)(q[2] & 0x30303030u), (int)(q[3] & 0x30303030u)};
+        const qv_i4 b3 = qv_i4{(int)((q[0] >> 6) & 0x03030303u), (int)((q[1] >> 6) & 0x03030303u), (int)((q[2] >> 6) & 0x03030303u),
+                               (int)((q[3] >> 6) & 0x03030303u)};
+        const qv_i4 C0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[0], b0, zero, 0, 0, 0);
+        const qv_i4 C1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[1], b1, zero, 0, 0, 0);
+        const qv_i4 C2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[2], b2, zero, 0, 0, 0);
+        const qv_i4 C3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[3], b3, zero, 0, 0, 0);
+        // scale bytes of the lane's four groups: bytes 0 and 2 of sc0 (fields 0, 1) and of sc1 (fields 2, 3)
+        const float t0 = (float)((C0[1] << 8) + C0[0]) * a.s[0], t1 = (float)((C1[1] << 8) + C1[0]) * a.s[1];
+        const float t2 = (float)((C2[1] << 8) + C2[0]) * a.s[2], t3 = (float)((C3[1] << 8) + C3[0]) * a.s[3];
+        float sd = (float)(sc0 & 0xFu) * t0;
+        sd = fmaf((float)((sc0 >> 16) & 0xFu), t1, sd);
+        sd = fmaf((float)(sc1 & 0xFu), t2, sd);
+        sd = fmaf((float)((sc1 >> 16) & 0xFu), t3, sd);
+        float sm = (float)((sc0 >> 4) & 0xFu) * a.xs[0];
+        sm = fmaf((float)((sc0 >> 20) & 0xFu), a.xs[1], sm);
+        sm = fmaf((float)((sc1 >> 4) & 0xFu), a.xs[2], sm);
+        sm = fmaf((float)((sc1 >> 20) & 0xFu), a.xs[3], sm);
+        float acc = fmaf(-f16_bits(dd >> 16), sm, f16_bits(dd) * sd);
+        acc = sum_xor16(acc);
+        return sum_xor32(acc);
+    }
+};
+
 // Work of workgroup b (of G): tiles b, b + G, b + 2 G, ... of 16 rows each; there are rounds G + extra tiles,
 // so the first `extra` workgroups take one more than the others.  (Tiles of 14 rows, which give each of 256
 // workgroups four tiles of a 14336-row matrix where tiles of 16 rows leave 32 compute units idle, measured
-// 1.5 % slower: 7.49 against 7.39 us.)
+// 1.5 % slower for Q4_K: 7.49 against 7.39 us.)
 struct QvWork {
     int n, G, rounds, extra;
 };
 
-// Wave w copies row w of a tile into a ring of four tiles in LDS (three contiguous asynchronous loads, two
-// tiles ahead of the arithmetic) and multiplies column w of all 16 rows, so a tile is published by a
-// barrier.  The waves' partial sums of up to four tiles wait in LDS and are added, stored and forgotten
-// behind one more barrier.
-__global__ __launch_bounds__(1024) void q4k_gemv_mfma_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                          float *__restrict__ Y, QvWork wk) {
+// Wave w copies row w of a tile into a ring of four tiles in LDS (contiguous asynchronous loads, two tiles
+// ahead of the arithmetic) and multiplies column w of all 16 rows, so a tile is published by a barrier.
+// The waves' partial sums of up to four tiles wait in LDS and are added, stored and forgotten behind one
+// more barrier.
+template <class F>
+__global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
+                                                      float *__restrict__ Y, QvWork wk) {
     constexpr int D = 2;  // tiles asked for ahead of the one being multiplied (3 measured slower)
-    __shared__ __attribute__((aligned(16))) uint8_t ring[QV_SLOTS][QD_TILE_LDS];
+    constexpr int LOADS = (F::ROW + 1023) / 1024;  // asynchronous loads a wave and tile
+    __shared__ __attribute__((aligned(16))) uint8_t ring[QV_SLOTS][16 * F::ROW_LDS];
     __shared__ float part[QV_SLOTS][16][16];  // [tile % 4][wave][row]
+    // a wave's staging area (what prepare() needs, then its 256 raw activations): its own row of ring slot 3
+    // when that is long enough, which no load targets before tile 3 is asked for in the main loop; else
+    // memory of its own
+    constexpr int STAGE = F::STAGE_BYTES + 1024;
+    constexpr bool STAGE_IN_RING = STAGE <= F::ROW_LDS;
+    __shared__ __attribute__((aligned(16))) uint8_t stage_mem[STAGE_IN_RING ? 16 : 16 * STAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, c = lane >> 4, b = (int)blockIdx.x;
     const int n = wk.n, G = wk.G;
@@ -146,17 +259,19 @@ __global__ __launch_bounds__(1024) void q4k_gemv_mfma_lds(const uint8_t *__restr
     auto fetch = [&](int slot_i) __attribute__((always_inline)) {
         const int i = min(slot_i, nt - 1);
         const int row = min(tile_row0(i) + wave, n - 1);
-        const uint8_t *src = W + (size_t)row * QD_ROW + 16 * lane;
-        const uint32_t dst = lds_offset_of(&ring[slot_i & (QV_SLOTS - 1)][wave * QD_ROW_LDS]);
-        async_load16(src, dst);
-        async_load16(src + 1024, dst + 1024);
-        if (lane < 16) async_load16(src + 2048, dst + 2048);
+        const uint8_t *src = W + (size_t)row * F::ROW + 16 * lane;
+        const uint32_t dst = lds_offset_of(&ring[slot_i & (QV_SLOTS - 1)][wave * F::ROW_LDS]);
+#pragma unroll
+        for (int j = 0; j < LOADS; j++) {
+            constexpr int full = F::ROW / 1024;
+            if (j < full) async_load16(src + 1024 * j, dst + 1024 * j);
+            else if (lane < (F::ROW - 1024 * full) / 16) async_load16(src + 1024 * j, dst + 1024 * j);
+        }
     };
-    // staging area of this wave: its own row of ring slot 3, which no load targets before tile 3 is asked
-    // for in the main loop; from byte 1152 the wave's 256 raw activations, which travel like the tiles
-    // (every global read of this kernel is an asynchronous load counted by hand)
-    uint32_t *stage = (uint32_t *)&ring[QV_SLOTS - 1][wave * QD_ROW_LDS];
-    float *x_raw = (float *)(stage + 288);
+    // the raw activations travel like the tiles (every global read of this kernel is an asynchronous load
+    // counted by hand)
+    uint32_t *stage = (uint32_t *)(STAGE_IN_RING ? &ring[QV_SLOTS - 1][wave * F::ROW_LDS] : &stage_mem[wave * STAGE]);
+    float *x_raw = (float *)((uint8_t *)stage + F::STAGE_BYTES);
     async_load16(X + 256 * wave + 4 * lane, lds_offset_of(x_raw));
     // every wave's activations are asked for before anybody's tile: the memory pipeline takes a compute
     // unit's requests in the order they were issued, and a wave whose activations queue behind the other
@@ -165,9 +280,10 @@ __global__ __launch_bounds__(1024) void q4k_gemv_mfma_lds(const uint8_t *__restr
     // tile 0 is asked for alone: it has the memory system to itself and lands while the activations are
     // prepared; the next D - 1 tiles follow the preparation
     fetch(0);
-    asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    if (LOADS == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
     const float4 v = *(const float4 *)&x_raw[4 * lane];
-    const QvActs acts = qv_prepare(v, stage, lane);
+    const typename F::Acts acts = F::prepare(v, stage, lane);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     fetch(1);
     if (D == 3) fetch(2);
@@ -179,14 +295,20 @@ __global__ __launch_bounds__(1024) void q4k_gemv_mfma_lds(const uint8_t *__restr
             // tile t has landed; tiles up to max(D - 1, min(nt - 1, t + D - 1)) have been asked for and may be
             // in flight, nothing behind the last tile
             const int ahead = t == nt - 1 ? 0 : max(D - 1, min(nt - 1, t + D - 1)) - t;
-            if (ahead >= 2) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-            else if (ahead == 1) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (LOADS == 3) {
+                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            } else {
+                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             // every wave is done with tile t - 1, so the slot of tile t + D - 4 is free
             if (t + D < nt) fetch(t + D);
-            const float acc = qv_block_dot(&ring[t & (QV_SLOTS - 1)][r * QD_ROW_LDS + wave * 144], acts, c);
+            const float acc = F::block_dot(&ring[t & (QV_SLOTS - 1)][r * F::ROW_LDS + wave * F::BLOCK], acts, c);
             if (lane < 16) part[t & (QV_SLOTS - 1)][wave][lane] = acc;
         }
         // the waves' partial sums of this group's tiles are written: lane (tt = lane / 16, ww = lane % 16)

@@ -775,6 +775,7 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q6_K, 1, 1024, 4096, "matmul_rows_staged"),
     (capi.Q6_K, 64, 4096, 1024, "gemm_decoded_mfma+splitk"),
     (capi.Q2_K, 1, 7680, 2048, "matmul_rows_staged"),
+    (capi.Q2_K, 1, 4096, 14336, "q2k_gemv_mfma_lds"),
     (capi.MXFP4, 1, 7168, 2048, "matmul_rows_staged"),
     (capi.IQ2_XXS, 1, 7168, 2048, "matmul_rows_staged"),
 ]
@@ -792,3 +793,50 @@ def test_kernel_chosen_for_a_shape(qtype, m, k, n, kernel):
     w.matmul_t_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert capi.last_kernel() == kernel
+
+
+# ---- Q2_K, one activation row over 4096-wide rows: the int8 matrix-core GEMV ----
+
+@pytest.mark.parametrize("n", [256, 1000, 4096, 14336, 16 * 256 * 5 + 16 * 3 + 7])
+def test_q2k_mfma_gemv_row_counts(n):
+    k = 4096
+    blocks = make_blocks(capi.Q2_K, n, k, 500 + n % 89)
+    lhs = synth.normal(501, (1, k))
+    got = capi.Weight.upload(capi.Q2_K, blocks, n, k).matmul_t(1, lhs)
+    assert capi.last_kernel() == "q2k_gemv_mfma_lds"
+    assert close(got, oracle.matmul_t(capi.Q2_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+def test_q2k_mfma_gemv_integer_dot_products_are_exact():
+    """Random block bytes with d = dmin = 1 (integer weights sc q - m, every two-bit value at every position,
+    every scale nibble) against integer activations whose 32-element groups have maximum magnitude 32639,
+    so that their fixed-point scale is exactly 1: every per-group sum is an integer the kernel must get
+    exactly; the f32 sum over a row's 256 groups is checked at 2^-20 of the terms' magnitudes."""
+    n, k = 1024 + 48, 4096
+    rng = np.random.default_rng(11)
+    raw = rng.integers(0, 256, size=n * 16 * 84, dtype=np.uint8).reshape(-1, 84)
+    raw[:, 80:84] = np.frombuffer(np.float16([1.0, 1.0]).tobytes(), np.uint8)
+    xi = rng.integers(-32639, 32640, size=k).astype(np.int64)
+    xi[::32] = 32639
+    w = oracle.dequantize(capi.Q2_K, raw.reshape(-1)).reshape(n, k).astype(np.int64)
+    want = w @ xi
+    got = capi.Weight.upload(capi.Q2_K, raw.reshape(-1), n, k).matmul_t(1, xi[None, :].astype(np.float32))
+    assert capi.last_kernel() == "q2k_gemv_mfma_lds"
+    assert np.all(np.abs(got[0].astype(np.float64) - want) <= 2.0 ** -20 * (np.abs(w).astype(np.float64) @ np.abs(xi)))
+    # one group at a time: a single non-zero activation group isolates its scale byte, field and plane sums
+    for g in (0, 1, 7, 8, 9, 15, 100, 255):
+        x1 = np.zeros(k, np.int64)
+        x1[16 * g:16 * g + 16] = rng.integers(-32639, 32640, size=16)
+        x1[16 * g] = 32639
+        got = capi.Weight.upload(capi.Q2_K, raw.reshape(-1), n, k).matmul_t(1, x1[None, :].astype(np.float32))
+        assert np.array_equal(got[0], (w @ x1).astype(np.float32)), g
+
+
+def test_q2k_mfma_gemv_non_finite_activations():
+    n, k = 512, 4096
+    blocks = make_blocks(capi.Q2_K, n, k, 511)
+    w = capi.Weight.upload(capi.Q2_K, blocks, n, k)
+    for bad in (np.inf, np.nan):
+        lhs = synth.normal(513, (1, k))
+        lhs[0, 2000] = bad
+        assert np.all(np.isnan(w.matmul_t(1, lhs)))
