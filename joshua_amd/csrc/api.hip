@@ -29,6 +29,7 @@
 #include "kernels_moe.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
 #include "kernels_mfma_q4k_rows16.hpp"
+#include "kernels_mfma_q4k_gemm_i8.hpp"
 #include "kernels_valu.hpp"
 #include "kernels_mfma_decoded.hpp"
 
@@ -632,6 +633,78 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
     return 0;
 }
 
+// Q4_K with many activation rows on the int8 matrix cores: the activations as two int8 planes per
+// 32-element sub-block in the call scratch of the stream, then q4k_gemm_i8 with a workgroup shape chosen for
+// the row count (8 waves as WM x 8 / WM) and NG weight-row groups of 16 a wave chosen so that the tiles
+// fill the 256 compute units as evenly as possible.  Returns -1 when the shape is outside its reach or has
+// too few tiles to occupy the chip (the f16 GEMM splits those over k).  JQ_Q4K_GEMM_I8 = 0 switches it off.
+struct GemmI8Shape {
+    int nw, ng;
+};
+
+int dispatch_q4k_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                         hipStream_t s) {
+    static const char *mode = getenv("JQ_Q4K_GEMM_I8");
+    static const char *min_tiles_env = getenv("JQ_Q4K_GEMM_I8_MIN_TILES");
+    static const char *shape_env = getenv("JQ_Q4K_GEMM_I8_SHAPE");  // "waves,groups": one of the shapes below
+    static const size_t min_tiles = min_tiles_env ? (size_t)atoll(min_tiles_env) : 160;
+    if ((mode && mode[0] == '0') || m < 17 || k % 256 != 0 || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 ||
+        ((uintptr_t)X & 15) != 0 || m > 0x7FFFFFF0ull || n > 0x7FFFFFF0ull)
+        return -1;
+    // Two workgroup shapes: 256 x 112 outputs (eight waves, one workgroup a compute unit) and 128 x 64 (four
+    // waves, two a compute unit).  Measured at k = 4096, in us: the large one 17 + 105 per round of 256 tiles;
+    // the small one 52 up to 256 tiles, 30 + 0.137 a tile beyond.  There is no split over k here, so below
+    // about 160 small tiles the f16 kernel with its split wins (512 x 4096 x 1024: 34 us against 51) and the
+    // call is declined.
+    static const GemmI8Shape shapes[] = {{8, 7}, {4, 4}};
+    auto tiles_of = [&](const GemmI8Shape &sh) {
+        const size_t mt = 32 * (size_t)sh.nw, nt = 16 * (size_t)sh.ng;
+        return ((m + mt - 1) / mt) * ((n + nt - 1) / nt);
+    };
+    const size_t tiles_large = tiles_of(shapes[0]), tiles_small = tiles_of(shapes[1]);
+    const double t_large = 17.0 + 105.0 * (double)((tiles_large + 255) / 256);
+    const double t_small = tiles_small <= 256 ? 52.0 : 30.0 + 0.137 * (double)tiles_small;
+    const GemmI8Shape *best = t_large < t_small ? &shapes[0] : &shapes[1];
+    int want_nw = 0, want_ng = 0;
+    if (shape_env && sscanf(shape_env, "%d,%d", &want_nw, &want_ng) == 2)
+        for (const GemmI8Shape &sh : shapes)
+            if (sh.nw == want_nw && sh.ng == want_ng) best = &sh;
+    if (tiles_small < min_tiles) return -1;
+    const size_t nb = k / 256, groups = (m + 15) / 16;
+    CallScratch scratch;
+    uint8_t *acts = nullptr;
+    if (scratch.get(groups * nb * (size_t)jq::QI_REC, s, &acts)) return 1;
+    const size_t mt = 32 * (size_t)best->nw, nt = 16 * (size_t)best->ng;
+    const size_t tx = (n + nt - 1) / nt, ty = (m + mt - 1) / mt;
+    const size_t grid = 8 % ty == 0 ? (tx * ty + 7) / 8 * 8 : tx * ty;
+    if (grid > 0x7FFFFFFFull) return -1;
+    hipError_t attr_rc = hipSuccess;
+#define JQ_GEMM_I8(NW_, NG_)                                                                                          \
+    if (best->nw == NW_ && best->ng == NG_) {                                                                         \
+        auto kern = jq::q4k_gemm_i8<NW_, NG_>;                                                                        \
+        constexpr int lds = jq::qi_lds_bytes<NG_>();                                                                  \
+        static std::once_flag big_lds;                                                                                \
+        static hipError_t rc_once = hipSuccess;                                                                       \
+        std::call_once(big_lds, [&] {                                                                                 \
+            rc_once = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);       \
+        });                                                                                                           \
+        attr_rc = rc_once;                                                                                            \
+        if (attr_rc == hipSuccess) {                                                                                  \
+            hipLaunchKernelGGL(jq::q4k_gemm_i8_prep, dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, X, (int)m, \
+                               (int)k, acts);                                                                         \
+            hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NW_), lds, s, W, row_bytes, (const uint8_t *)acts, \
+                               Y, (int)m, (int)n, (int)nb, (int)groups, (int)tx, (int)ty);                            \
+        }                                                                                                             \
+    }
+    JQ_GEMM_I8(8, 7)
+    JQ_GEMM_I8(4, 4)
+#undef JQ_GEMM_I8
+    if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
+    note_kernel("q4k_gemm_i8");
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // Q4_K with more than 16 activation rows: prepare the fixed-point activation planes in the
 // call scratch of the stream, then the MFMA GEMM, split over k when its tiles alone would leave
 // compute units idle.
@@ -762,6 +835,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         q4k_gemm_estimate_us(m, k, n) < (double)m * (2.0 + (double)n * (double)row_bytes / 4.0e6))
         return dispatch_q4k_gemm(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k, n)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
+    if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M) {
+        const int rc = dispatch_q4k_gemm_i8(W, row_bytes, X, Y, m, k, n, s);
+        if (rc >= 0) return rc;
+    }
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&
         !getenv("JQ_Q4K_NO_GEMM"))
         return dispatch_q4k_gemm(W, row_bytes, X, Y, m, k, n, s);

@@ -1,0 +1,336 @@
+// Q4_K matmul for many activation rows on the int8 matrix cores.
+//
+// Per 256-element super-block B of weight row n and activation row m (reference arithmetic
+// w = d sc q - dmin m, src/kquant_dot.rs:440-465):
+//
+//   sum_k x_k w_k = s (d I1 - dmin I2),   I1 = sum_k (sc_j(k) q_k) X_k,   I2 = sum_j m_j XS_j
+//
+// with the activations in 16-bit fixed point per (row, super-block), X = round(x / s), s = amax_B |x| / 32639,
+// and XS_j the sum of X over sub-block j.  Both factors of I1 are split into two signed bytes,
+//
+//   X = 256 Xh + Xl          p = sc q = 256 Ph + Pl   (p <= 945: Ph = (p + 128) >> 8 in 0..4, Pl in -128..127)
+//   I1 = 65536 HH + 256 MID + LL,   HH = sum Xh Ph,  MID = sum Xh Pl + Xl Ph,  LL = sum Xl Pl
+//
+// so that the 6-bit sub-block scales are part of the integer operand and every super-block costs four
+// v_mfma_i32_16x16x64_i8 per 64 k and 16 x 16 outputs, with int32 sums that are exact, and one conversion
+// to f32 per super-block (seven vector instructions an output) instead of one per sub-block.  I2 is one
+// v_mfma_f32_16x16x32_f16 per super-block over exact f16 integers (XS = 1024 a1 + a0 against m and 1024 m).
+// A single scale per 256 activations leaves an error of at most 2^-16 of the super-block's largest
+// magnitude per element: rows whose values span many orders of magnitude inside one super-block are
+// resolved relative to the largest of them, like the reference's own 8-bit Q8_K activations
+// (src/kquant_dot.rs:407-483) but with 256 times the resolution.
+//
+// Workgroup: NW waves, tile 32 NW activation rows x 16 NG weight rows; a wave owns 32 activation rows (two
+// groups of 16) against all 16 NG weight rows.  Each thread takes the packed bytes of (weight row, 64-k
+// chunk) units from global memory an iteration ahead, multiplies the nibbles by their scales (two elements an
+// instruction), splits the products and stores them into LDS as MFMA B operands: two buffers, one barrier a
+// super-block, an eighth of the work in every eighth of the iteration.  The activation operands come
+// prepared in operand order (q4k_gemm_i8_prep) straight from global memory (L2) into registers, one chunk of
+// one row group at a time, three quarters of a half iteration before the MFMAs want them.
+//
+// What bounds it (counters at 512 x 4096 x 14336): the matrix cores are busy 59 % of the cycles and the
+// vector ALU most of the rest: on this part an MFMA and a vector instruction of the same SIMD hardly
+// overlap (a loop of independent MFMAs slows by about 2.7 cycles for every vector instruction put between
+// them, with two waves a SIMD), so the seven instructions an output and super-block of the conversion and the
+// ~150 of the unpack add to the MFMA time instead of hiding under it.
+#pragma once
+#include "kernels_mfma_q4k_rows16.hpp"
+
+namespace jq {
+
+typedef _Float16 qi_h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 qi_h8 __attribute__((ext_vector_type(8)));
+
+// Prepared activations, per (group of 16 activation rows, super-block): 4 chunks x 2 planes (Xh, Xl) x 64
+// lanes x 16 bytes (lane (i = lane % 16, g = lane / 16): elements 64 c + 16 g .. + 15 of row i), then the I2
+// operand (64 lanes x 8 halves: g = 0 holds a0 of the 8 sub-blocks, g = 1 a1, g = 2, 3 zero), then s of the
+// 16 rows.
+constexpr int QI_PLANES = 4 * 2 * 64 * 16, QI_MIN = QI_PLANES, QI_SCALE = QI_PLANES + 1024, QI_REC = QI_SCALE + 64;
+
+// grid (k / 256 super-blocks, groups of 16 activation rows), 256 threads: wave c, lane (i, g) quantises the
+// 16 elements 64 c + 16 g .. of row i.  Rows from m_rows on are zero operands.
+__global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict__ X, int m_rows, int k,
+                                                         uint8_t *__restrict__ out) {
+    __shared__ float amax_sh[4][16];
+    __shared__ int xs_sh[16][8];
+    const int tid = threadIdx.x, lane = tid & 63, c = tid >> 6, i = lane & 15, g = lane >> 4;
+    const int b = blockIdx.x, row = 16 * (int)blockIdx.y + i;
+    uint8_t *rec = out + ((size_t)blockIdx.y * gridDim.x + b) * QI_REC;
+    float v[16];
+    if (row < m_rows) {
+        const float4 *src = (const float4 *)(X + (size_t)row * k + 256 * b + 64 * c + 16 * g);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const float4 a = src[q];
+            v[4 * q] = a.x, v[4 * q + 1] = a.y, v[4 * q + 2] = a.z, v[4 * q + 3] = a.w;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; e++) v[e] = 0.0f;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) amax = fmaxf(amax, mag_or_inf(v[e]));
+    amax = max_xor32(max_xor16(amax));  // the four lane groups of this wave
+    if (g == 0) amax_sh[c][i] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(amax_sh[0][i], amax_sh[1][i]), fmaxf(amax_sh[2][i], amax_sh[3][i]));
+    const bool live = amax > 0.0f && amax < INFINITY;
+    const float inv = live ? QD_RANGE / amax : 0.0f, s = fixed_scale(amax, QD_RANGE);
+    uint32_t h[4] = {0, 0, 0, 0}, l[4] = {0, 0, 0, 0};
+    int sum = 0;
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+        const int Xq = __float2int_rn(v[e] * inv);
+        l[e >> 2] |= (uint32_t)(Xq & 255) << (8 * (e & 3));
+        h[e >> 2] |= (uint32_t)(((Xq + 128) >> 8) & 255) << (8 * (e & 3));
+        sum += Xq;
+    }
+    sum = isum_xor16(sum);  // the two lane groups of a sub-block
+    if ((g & 1) == 0) xs_sh[i][2 * c + (g >> 1)] = sum;
+    *(uint4 *)(rec + ((size_t)(2 * c) * 64 + lane) * 16) = uint4{h[0], h[1], h[2], h[3]};
+    *(uint4 *)(rec + ((size_t)(2 * c + 1) * 64 + lane) * 16) = uint4{l[0], l[1], l[2], l[3]};
+    __syncthreads();
+    if (tid < 64) {
+        uint32_t w[4] = {0, 0, 0, 0};
+        if (g < 2) {
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                qi_h2 pair;
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const int xs = xs_sh[i][j + e], a1 = (xs + 512) >> 10, a0 = xs - 1024 * a1;
+                    pair[e] = (_Float16)(float)(g == 0 ? a0 : a1);
+                }
+                w[j >> 1] = __builtin_bit_cast(uint32_t, pair);
+            }
+        }
+        *(uint4 *)(rec + QI_MIN + lane * 16) = uint4{w[0], w[1], w[2], w[3]};
+    }
+    if (tid < 16) ((float *)(rec + QI_SCALE))[tid] = s;
+}
+
+// LDS per buffer: NG tiles of 16 weight rows x [chunk 4][plane 2 (Ph, Pl)][lane 64] x 16 bytes, then per
+// weight row 48 bytes: m_0..7 as halves, 1024 m_0..7 as halves, d, dmin as floats, 8 unused.
+constexpr int QI_TILE = 4 * 2 * 64 * 16, QI_META = 48;
+template <int NG>
+constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * QI_META); }
+
+struct QiRaw {  // one unit: the header of a weight row's block and the 32 bytes of one chunk
+    uint4 hdr, q0, q1;
+};
+
+// The products p = sc q of the four bytes of `word` (nibble `hi`), plus 128, as halfwords: elements 0, 2 in
+// `even`, 1, 3 in `odd`.
+__device__ __forceinline__ void qi_products(uint32_t word, bool hi, uint32_t sc, uint32_t &even, uint32_t &odd) {
+    const uint32_t w = hi ? word >> 4 : word;
+    even = __umul24(w & 0x000F000Fu, sc) + 0x00800080u;  // one v_mad_u32_u24
+    odd = __umul24((w >> 8) & 0x000F000Fu, sc) + 0x00800080u;
+}
+
+// grid: 1-D; workgroup L takes tile (x, y) of tx x ty (weight-row tiles x activation-row tiles).  When ty
+// divides 8 the eight XCDs (L % 8) each work on one activation-row tile, whose operands then stay in that
+// XCD's L2; the grid is padded to a multiple of 8 and workgroups past the last tile leave at once.
+template <int NW, int NG>
+__global__ __launch_bounds__(64 * NW) void q4k_gemm_i8(const uint8_t *__restrict__ W, size_t row_bytes,
+                                                       const uint8_t *__restrict__ acts, float *__restrict__ Y,
+                                                       int m_rows, int n, int nb, int groups, int tx, int ty) {
+    constexpr int NT = 16 * NG, THREADS = 64 * NW, UNITS = 4 * NT, PER = (UNITS + THREADS - 1) / THREADS;
+    constexpr int BUF = NG * QI_TILE + NT * QI_META;
+    extern __shared__ __attribute__((aligned(16))) uint8_t qi_lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+    int bx, by;
+    if (8 % ty == 0) {
+        const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
+        by = xcd % ty, bx = slot * (8 / ty) + xcd / ty;
+    } else {
+        by = (int)blockIdx.x / tx, bx = (int)blockIdx.x % tx;
+    }
+    if (bx >= tx || by >= ty) return;
+    const int n0 = bx * NT, m0 = by * 32 * NW;
+
+    // activation operands of this wave: row groups 2 wave, 2 wave + 1 of the tile (clamped: rows past m_rows
+    // are computed and not stored)
+    const uint8_t *arec[2];
+#pragma unroll
+    for (int mg = 0; mg < 2; mg++) arec[mg] = acts + (size_t)min(m0 / 16 + 2 * wave + mg, groups - 1) * nb * QI_REC;
+
+    // unpack units of this thread: chunk c = tid % 4 of weight rows tid / 4 + (THREADS / 4) p
+    const int uc = tid & 3;
+    const uint8_t *wsrc[PER];
+#pragma unroll
+    for (int p = 0; p < PER; p++) {
+        const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);
+        wsrc[p] = W + (size_t)min(n0 + row, n - 1) * row_bytes;
+    }
+    QiRaw raw[PER];
+    uint4 hdr_next[PER];
+    auto fetch_part = [&](int b, int part) __attribute__((always_inline)) {  // 0: header into hdr_next, 1, 2: the two halves of the chunk
+#pragma unroll
+        for (int p = 0; p < PER; p++) {
+            const uint8_t *src = wsrc[p] + (size_t)b * 144;
+            if (part == 0) hdr_next[p] = *(const uint4 *)src;
+            if (part == 1) raw[p].q0 = *(const uint4 *)(src + 16 + 32 * uc);
+            if (part == 2) raw[p].q1 = *(const uint4 *)(src + 32 + 32 * uc);
+        }
+    };
+    // Piece j of 8: the four bytes j of this thread's chunk become two operand words of either plane (low
+    // nibbles: sub-block 2 uc, high nibbles: sub-block 2 uc + 1).
+    auto unpack_piece = [&](uint8_t *buf, int j) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < PER; p++) {
+            const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);  // threads past the last unit repeat it
+            const uint4 hdr = raw[p].hdr;
+            const uint32_t scl = hdr.y & 0x3F3F3F3Fu, sch = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+            const uint32_t s4 = (uc < 2 ? scl : sch) >> (16 * (uc & 1));
+            const uint32_t sc[2] = {s4 & 0xFFu, (s4 >> 8) & 0xFFu};
+            uint8_t *tile = buf + (row >> 4) * QI_TILE + uc * 2048 + (row & 15) * 16;
+            const uint4 qv = j < 4 ? raw[p].q0 : raw[p].q1;
+            const uint32_t word = (j & 3) == 0 ? qv.x : (j & 3) == 1 ? qv.y : (j & 3) == 2 ? qv.z : qv.w;
+#pragma unroll
+            for (int nib = 0; nib < 2; nib++) {
+                uint32_t even, odd;
+                qi_products(word, nib != 0, sc[nib], even, odd);
+                const int gg = 2 * nib + (j >> 2);
+                *(uint32_t *)(tile + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+                *(uint32_t *)(tile + 1024 + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+            }
+        }
+    };
+    auto unpack_meta = [&](uint8_t *buf) __attribute__((always_inline)) {  // the row's scales of the min term, d and dmin
+#pragma unroll
+        for (int p = 0; p < PER; p++) {
+            const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);
+            const uint4 hdr = raw[p].hdr;
+            const uint32_t mnl = hdr.z & 0x3F3F3F3Fu, mnh = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+            const uint32_t m4 = (uc < 2 ? mnl : mnh) >> (16 * (uc & 1));
+            const float mn[2] = {(float)(m4 & 0xFFu), (float)((m4 >> 8) & 0xFFu)};
+            uint8_t *meta = buf + NG * QI_TILE + row * QI_META;
+            const qi_h2 m1 = {(_Float16)mn[0], (_Float16)mn[1]}, m1k = {(_Float16)(1024.0f * mn[0]), (_Float16)(1024.0f * mn[1])};
+            *(uint32_t *)(meta + 4 * uc) = __builtin_bit_cast(uint32_t, m1);
+            *(uint32_t *)(meta + 16 + 4 * uc) = __builtin_bit_cast(uint32_t, m1k);
+            *(float2 *)(meta + 32) = float2{f16_bits(hdr.x), f16_bits(hdr.x >> 16)};  // the same from all four
+        }
+    };
+    auto take_header = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < PER; p++) raw[p].hdr = hdr_next[p];
+    };
+
+    fetch_part(0, 0), fetch_part(0, 1), fetch_part(0, 2);
+    take_header();
+#pragma unroll
+    for (int j = 0; j < 8; j++) unpack_piece(qi_lds, j);
+    unpack_meta(qi_lds);
+    fetch_part(min(1, nb - 1), 0), fetch_part(min(1, nb - 1), 1), fetch_part(min(1, nb - 1), 2);
+
+    // The loop walks through quarters: (activation row group mg of this wave, 64-k chunk c) against all NG
+    // groups of weight rows.  A[c] holds the operands of chunk c for the row group at work; once the quarter is
+    // through with them, the same chunk of the other row group is asked for (of the next super-block when mg is
+    // 1), three quarters before its turn.
+    qm_i4 A[4][2];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int P = 0; P < 2; P++) A[c][P] = *(const qm_i4 *)(arec[0] + ((size_t)(2 * c + P) * 64 + lane) * 16);
+
+    qm_f4 acc[2][NG];
+#pragma unroll
+    for (int mg = 0; mg < 2; mg++)
+#pragma unroll
+        for (int cg = 0; cg < NG; cg++) acc[mg][cg] = qm_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const qm_i4 zero_i = {0, 0, 0, 0};
+    const qm_f4 zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
+    __syncthreads();
+
+    for (int b = 0; b < nb; b++) {
+        const uint8_t *buf = qi_lds + (b & 1) * BUF;
+        const int b_next = min(b + 1, nb - 1), b_next2 = min(b + 2, nb - 1);
+#pragma unroll
+        for (int mg = 0; mg < 2; mg++) {
+            // scales and I2 operand of this row group: wanted in the last quarter
+            const qm_f4 sx = *(const qm_f4 *)(arec[mg] + (size_t)b * QI_REC + QI_SCALE + 16 * g);
+            const qi_h8 minA = *(const qi_h8 *)(arec[mg] + (size_t)b * QI_REC + QI_MIN + lane * 16);
+            // The weight-row groups in two sets (T0 and NG - T0 of them), each taken through the four chunks: the
+            // integer sums of one set are alive at a time.  Step s of a half = (set, chunk, group within the set).
+            constexpr int T0 = (NG + 1) / 2, STEPS = 4 * NG;
+            auto step_cg = [](int s) { return s < 4 * T0 ? s % T0 : T0 + (s - 4 * T0) % (NG - T0); };
+            auto step_c = [](int s) { return s < 4 * T0 ? s / T0 : (s - 4 * T0) / (NG - T0); };
+            qm_i4 HH[NG], MID[NG], LL[NG];
+            // the weight operands travel one step ahead of the MFMAs that use them, through two register sets
+            qm_i4 Bh[2], Bl[2];
+            Bh[0] = *(const qm_i4 *)(buf + lane * 16), Bl[0] = *(const qm_i4 *)(buf + 1024 + lane * 16);
+            auto finish = [&](int cg) __attribute__((always_inline)) {  // the 16 x 16 results of weight-row group cg
+                const uint8_t *meta = buf + NG * QI_TILE + (16 * cg + r) * QI_META;
+                const float2 dd = *(const float2 *)(meta + 32);
+                // lane groups 2, 3 meet zeros in the activation operand: any finite halves will do for them
+                const qi_h8 mB = *(const qi_h8 *)(meta + 16 * (g & 1));
+                const qm_f4 I2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(minA, mB, zero_f, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float I1 = fmaf((float)(HH[cg][i] * 256 + MID[cg][i]), 256.0f, (float)LL[cg][i]);
+                    acc[mg][cg][i] = fmaf(sx[i], dd.x * I1 - dd.y * I2[i], acc[mg][cg][i]);
+                }
+            };
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                const int cg = step_cg(s), c = step_c(s), cur = s & 1, nxt = cur ^ 1;
+                const bool first_of_pass = s < 4 * T0 ? s % T0 == 0 : (s - 4 * T0) % (NG - T0) == 0;
+                const bool last_of_pass = s < 4 * T0 ? s % T0 == T0 - 1 : (s - 4 * T0) % (NG - T0) == NG - T0 - 1;
+                const int pass = s < 4 * T0 ? c : 4 + c;  // 0..7 within the half
+                if (first_of_pass) {
+                    // An eighth of the next super-block's weights becomes operands in every pass, thinly spread
+                    // among the MFMAs (its bytes were asked for half an iteration or more ago); the registers of
+                    // a part are refilled with the super-block after that as soon as the part is used up.
+                    const int piece = 4 * mg + (pass >> 1);
+                    if (mg == 0 && pass == 0) take_header();
+                    if ((pass & 1) == 0) unpack_piece(qi_lds + ((b + 1) & 1) * BUF, piece);
+                    if (mg == 1 && pass == 0) fetch_part(b_next2, 1), fetch_part(b_next2, 0);
+                    if (mg == 1 && pass == 7) unpack_meta(qi_lds + ((b + 1) & 1) * BUF);
+                }
+                if (c == 0) HH[cg] = zero_i, MID[cg] = zero_i, LL[cg] = zero_i;
+                if (s + 1 < STEPS) {
+                    const int cg1 = step_cg(s + 1), c1 = step_c(s + 1);
+                    Bh[nxt] = *(const qm_i4 *)(buf + (4 * cg1 + c1) * 2048 + lane * 16);
+                    Bl[nxt] = *(const qm_i4 *)(buf + (4 * cg1 + c1) * 2048 + 1024 + lane * 16);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                MID[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][0], Bl[cur], MID[cg], 0, 0, 0);
+                HH[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][0], Bh[cur], HH[cg], 0, 0, 0);
+                LL[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][1], Bl[cur], LL[cg], 0, 0, 0);
+                MID[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][1], Bh[cur], MID[cg], 0, 0, 0);
+                // one group behind the MFMAs, whose results it would otherwise wait for
+                if (c == 3 && !first_of_pass) finish(cg - 1);
+                if (last_of_pass && pass >= 4) {
+                    // this chunk's operands have done their work in this half: the other row group's take their place
+#pragma unroll
+                    for (int P = 0; P < 2; P++)
+                        A[c][P] = *(const qm_i4 *)(arec[mg ^ 1] + (size_t)(mg == 0 ? b : b_next) * QI_REC + ((size_t)(2 * c + P) * 64 + lane) * 16);
+                }
+                if (c == 3 && last_of_pass && pass < 4) finish(cg);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            finish(NG - 1);
+            if (mg == 1) fetch_part(b_next2, 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // every wave is done with the buffer the next super-block went into: it was read one iteration ago, in
+        // front of the barrier that ended that iteration
+        __syncthreads();
+    }
+#pragma unroll
+    for (int mg = 0; mg < 2; mg++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = m0 + 32 * wave + 16 * mg + 4 * g + i;
+            if (row >= m_rows) continue;
+#pragma unroll
+            for (int cg = 0; cg < NG; cg++) {
+                const int col = n0 + 16 * cg + r;
+                if (col < n) Y[(size_t)row * n + col] = acc[mg][cg][i];
+            }
+        }
+    }
+}
+
+}  // namespace jq

@@ -83,7 +83,7 @@ def test_qwen3_30b_a3b_shaped_layer_with_all_128_experts(tokens):
 
 
 def test_q4k_prefill_gemm_at_the_headline_shape():
-    """Q4_K 14336 x 4096 with 512 activation rows: 448 tiles, no split over k.  The oracle multiplies a
+    """Q4_K 14336 x 4096 with 512 activation rows: 256 tiles of 256 x 112 on the int8 matrix cores.  The oracle multiplies a
     sample of 1536 weight rows (the first and last 128-row tiles, and rows spread over the rest) by all 512
     activation rows; the device result is checked at those columns."""
     import torch
@@ -95,7 +95,7 @@ def test_q4k_prefill_gemm_at_the_headline_shape():
     y = torch.full((m, n), float("nan"), device="cuda")
     w.matmul_t_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert capi.last_kernel() == "q4k_gemm_mfma"
+    assert capi.last_kernel() == "q4k_gemm_i8"
     got = y.cpu().numpy()
     assert np.all(np.isfinite(got))
     rows = np.unique(np.concatenate([np.arange(128), np.arange(n - 128, n), np.arange(128, n - 128, 11)[:1280]]))

@@ -768,7 +768,9 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 2, 2048, 768, "q4k_gemv_mfma"),
     (capi.Q4_K, 16, 4096, 14336, "q4k_rows16_mfma"),
     (capi.Q4_K, 16, 2048, 768, "q4k_stream_mfma"),
-    (capi.Q4_K, 512, 4096, 14336, "q4k_gemm_mfma"),
+    (capi.Q4_K, 512, 4096, 14336, "q4k_gemm_i8"),           # 256 tiles of 256 x 112
+    (capi.Q4_K, 128, 4096, 14336, "q4k_gemm_i8"),           # 224 tiles of 128 x 64
+    (capi.Q4_K, 128, 4096, 4096, "q4k_gemm_mfma+splitk"),   # 64 tiles: the f16 kernel with its split over k
     (capi.Q4_K, 512, 4096, 1024, "q4k_gemm_mfma+splitk"),
     (capi.Q8_0, 1, 4096, 4096, "q8_0_gemv_dot4_lds"),
     (capi.Q6_K, 1, 12288, 4096, "q6k_gemv_dot4_lds"),
@@ -840,3 +842,77 @@ def test_q2k_mfma_gemv_non_finite_activations():
         lhs = synth.normal(513, (1, k))
         lhs[0, 2000] = bad
         assert np.all(np.isnan(w.matmul_t(1, lhs)))
+
+
+# ---- Q4_K with many activation rows on the int8 matrix cores ----
+
+GEMM_I8_CHILD = r"""
+import sys, numpy as np
+sys.path.insert(0, %r)
+import oracle
+from joshua_amd import capi, synth
+from tests.test_gpu_matmul import q4k_integer_case, close
+# one to three tiles in either direction, ragged row and column counts
+for (m, k, n) in [(17, 256, 64), (33, 512, 100), (64, 1024, 300), (100, 1024, 257), (130, 1024, 70), (200, 768, 1000),
+                  (257, 512, 113), (300, 4096, 450), (512, 2048, 2048)]:
+    blocks = synth.normal_quantized(capi.Q4_K, 5 + n, n * k, 0.02)
+    lhs = synth.normal(6 + k, (m, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
+    assert capi.last_kernel() == "q4k_gemm_i8", (capi.last_kernel(), m, k, n)
+    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())), (m, k, n)
+# exact integers: activation range 32639 per 32-element sub-block
+n, k, m = 160, 2048, 40
+blocks, q, x = q4k_integer_case(n, k, 23, group=32, big_value=32639, small=4000)
+lhs = np.stack([np.roll(x, 32 * i) for i in range(m)])
+got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs.astype(np.float32))
+assert capi.last_kernel() == "q4k_gemm_i8"
+assert np.array_equal(got, (lhs @ q.T).astype(np.float32)), "integer case"
+# a row whose 16-element groups span twelve orders of magnitude, a row with a single non-zero element, a
+# row with an empty stretch.  One 16-bit scale per 256 activations resolves each super-block relative to its
+# largest magnitude: the wide row is held to 2^-12 of the sum of its terms' magnitudes on every output, and to
+# the usual bound where the terms do not cancel below a twentieth of that sum.
+n, k = 64, 4096
+blocks = synth.normal_quantized(capi.Q4_K, 77, n * k, 0.02)
+rng = np.random.default_rng(5)
+lhs = synth.normal(78, (40, k))
+lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 16)).repeat(16).astype(np.float32)
+lhs[1, :] = 0.0
+lhs[1, 1234] = 3.5
+lhs[2, 512:1024] = 0.0
+got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(40, lhs)
+assert capi.last_kernel() == "q4k_gemm_i8"
+want = oracle.matmul_t(capi.Q4_K, (40, k, n), lhs, blocks, avx2=oracle.have_avx2())
+assert close(got[1:], want[1:]), "rows of ordinary range"
+wd = oracle.dequantize(capi.Q4_K, blocks).reshape(n, k).astype(np.float64)
+x0 = lhs[0].astype(np.float64)
+w0, mag = wd @ x0, np.abs(wd) @ np.abs(x0)
+err = np.abs(got[0] - w0)
+print("wide row: max err / mag = 2^%.1f" % np.log2((err / mag).max()))
+assert np.all(err <= 2.0 ** -12 * mag), "wide range"
+big = np.abs(w0) >= 0.05 * mag
+assert big.sum() > n // 4 and np.all(err[big] <= 1e-3 * np.abs(w0[big])), "wide range, rows without cancellation"
+# non-finite activations poison their own row only
+lhs = synth.normal(79, (20, k))
+lhs[3, 100] = np.inf
+lhs[7, 4000] = np.nan
+got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(20, lhs)
+want = oracle.matmul_t(capi.Q4_K, (20, k, n), lhs, blocks, avx2=oracle.have_avx2())
+assert np.all(np.isnan(got[3])) and np.all(np.isnan(got[7]))
+ok = np.ones(20, bool); ok[[3, 7]] = False
+assert close(got[ok], want[ok])
+print("gemm i8 ok")
+"""
+
+
+@pytest.mark.parametrize("shape", ["8,7", "4,4"])
+def test_q4k_int8_gemm_small_shapes_in_a_child_process(shape):
+    """The int8 GEMM serves a product only from about 160 tiles on; with the threshold lowered and the workgroup
+    shape forced through the environment (read when the library first dispatches, hence the child process) both
+    shapes run on small products: parity, ragged edges, exact integer sums, wide-range and non-finite
+    activation rows."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, JQ_Q4K_GEMM_I8_MIN_TILES="1", JQ_Q4K_GEMM_I8_SHAPE=shape)
+    res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1)], env=env, capture_output=True, text=True, timeout=170)
+    assert res.returncode == 0 and "gemm i8 ok" in res.stdout, res.stdout + res.stderr
