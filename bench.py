@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # (a plain copy of 33 030 144 bytes).  A counter run cannot happen inside this process, so the figure is
 # quoted only while the dispatcher still chooses the kernel it was measured on (jq_last_kernel); any other
 # kernel reports null until its own counter runs are in.
-MEASURED_TRAFFIC = {"kernel": "q4k_gemv_mfma_lds", "m": 1, "bytes": None}
+MEASURED_TRAFFIC = {"kernel": "q4k_gemv_mfma_lds", "m": 1, "bytes": 33_258_394}
 SEED_W, SEED_X = 102, 202
 
 
@@ -303,6 +303,8 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
             out["q4_k_14336x4096_m16"] = matmul_workload(torch, capi, synth, 12, N, K, 16, 102, steps, 24, 0.0)
         elif only == "m512":
             out["q4_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 12, N, K, 512, 102, max(steps // 10, 10), 4, 0.0)
+        elif only == "q2k":
+            out["q2_k_gemv_14336x4096_m1"] = matmul_workload(torch, capi, synth, 10, N, K, 1, 108, steps, 24, 0.0)
         elif only == "moe_b1":
             out["moe_qwen3_30b_a3b_q4_k_b1"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 1, 104, steps, False, 0, 0.0)
         elif only == "moe_v3":
