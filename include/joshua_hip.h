@@ -134,6 +134,20 @@ int jq_try_matmul_fused(uint32_t ggml_type, size_t m, size_t k, size_t n, const 
  * src/quant_matmul.rs:36-103 decode_raw_to_f32). */
 int jq_dequantize(const jq_weight *w, float *out, size_t out_len, int out_is_device, void *stream);
 
+/* Frees the scratch memory the library keeps for `stream` on the current device (the buffer the products
+ * with prepared activations share, and every smaller one it outgrew), after waiting for the stream.  For
+ * teardown: a HIP graph captured on the stream names those buffers and must not be replayed afterwards.  No
+ * counterpart in the reference (its scratch is host memory owned by each call). */
+int jq_stream_release(void *stream);
+
+/* Raw tensor bytes of ggml type `ggml_type` to `elems` f32 values: every block format of this library, F16
+ * (1), Q8_1 (9) and Q8_K (15).  Returns 0 with `out` filled; 2 where the reference answers Ok(None) -- F32 (0),
+ * whose bytes the caller's own reader keeps exact, and every type without a decoder there; 1 with a message
+ * when nbytes does not hold elems elements (the reference's wording)
+ * (reference: src/quant_matmul.rs:36-103 decode_raw_to_f32). */
+int jq_decode_raw_to_f32(uint32_t ggml_type, const void *bytes, size_t nbytes, size_t elems, float *out,
+                         int ptrs_are_device, void *stream);
+
 /* Row gather with decode: out[i, :] = decode(W[ids[i], :]); an id >= n fails
  * (reference: src/mmap_tensor.rs:140-167 embedding). */
 int jq_embedding(const jq_weight *w, const uint32_t *ids, size_t n_ids, float *out, size_t out_len,

@@ -49,12 +49,17 @@ def build_calibration() -> str:
 
 
 def build_all(verbose: bool = False) -> None:
+    """The library and the synthetic-data helper: what tests, smoke and the benchmark load.  The counter
+    calibration program is a profiling aid, built on request (`python -m joshua_amd.build --calibration`)."""
     from . import synth
     build_hip(verbose)
-    build_calibration()
     synth.build()
 
 
 if __name__ == "__main__":
-    build_all(verbose=True)
-    print("built", HIP_LIB)
+    import sys
+    if "--calibration" in sys.argv[1:]:
+        print("built", build_calibration())
+    else:
+        build_all(verbose=True)
+        print("built", HIP_LIB)

@@ -26,7 +26,7 @@ TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "
 # Every symbol include/joshua_hip.h declares.
 EXPORTS = (
     "jq_last_error", "jq_last_kernel", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
-    "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_matmul_t_noalloc", "jq_try_matmul_fused", "jq_dequantize",
+    "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_matmul_t_noalloc", "jq_try_matmul_fused", "jq_dequantize", "jq_decode_raw_to_f32", "jq_stream_release",
     "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
     "jq_mla_create", "jq_mla_free", "jq_mla_forward", "jq_mla_reset", "jq_mla_cached_tokens",
     "jq_qwen3_create", "jq_qwen3_free", "jq_qwen3_set_tensor", "jq_qwen3_forward", "jq_qwen3_greedy", "jq_qwen3_reset",
@@ -105,6 +105,8 @@ def lib() -> ctypes.CDLL:
         L.jq_matmul_t_noalloc.argtypes = [vp, sz, vp, sz, vp, sz, vp]
         L.jq_try_matmul_fused.argtypes = [u32, sz, sz, sz, vp, vp, sz, vp, vp]
         L.jq_dequantize.argtypes = [vp, vp, sz, i32, vp]
+        L.jq_decode_raw_to_f32.argtypes = [u32, vp, sz, sz, vp, i32, vp]
+        L.jq_stream_release.argtypes = [vp]
         L.jq_embedding.argtypes = [vp, vp, sz, vp, sz, i32, vp]
         L.jq_stream_synchronize.argtypes = [vp]
         L.jq_moe_create.argtypes = [ctypes.POINTER(MoeConfig), vp, vp, vp, vp, vp, vp, vp, vp, ctypes.POINTER(vp)]
@@ -170,6 +172,24 @@ def last_error() -> str:
 def last_kernel() -> str:
     """The kernel the calling thread's last matmul call chose."""
     return lib().jq_last_kernel().decode()
+
+
+def stream_release(stream: int = 0) -> None:
+    """Frees the scratch memory the library keeps for a stream (graphs captured on it become invalid)."""
+    _check(lib().jq_stream_release(stream or None))
+
+
+def decode_raw_to_f32(dtype: int, raw, elems: int):
+    """f32 values of raw tensor bytes, or None where the reference's decode_raw_to_f32 answers None
+    (src/quant_matmul.rs:36-103); a size mismatch raises with the reference's wording."""
+    raw = np.ascontiguousarray(np.frombuffer(raw, dtype=np.uint8) if not isinstance(raw, np.ndarray) else raw.view(np.uint8).reshape(-1))
+    out = np.empty(elems, dtype=np.float32)
+    rc = lib().jq_decode_raw_to_f32(dtype, raw.ctypes.data if raw.size else None, raw.size, elems,
+                                    out.ctypes.data if elems else None, 0, None)
+    if rc == 2:
+        return None
+    _check(rc)
+    return out
 
 
 def _check(rc: int) -> None:

@@ -466,6 +466,28 @@ struct StreamBuffer {
     std::vector<uint8_t *> retired;
 };
 
+std::mutex g_stream_table_mu;
+std::map<std::pair<int, hipStream_t>, std::unique_ptr<StreamBuffer>> g_stream_table;
+
+// jq_stream_release: waits for the stream, then frees its buffer and the retired ones.
+int release_stream_scratch(hipStream_t s) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    std::unique_ptr<StreamBuffer> b;
+    {
+        std::lock_guard<std::mutex> g(g_stream_table_mu);
+        auto it = g_stream_table.find({dev, s});
+        if (it == g_stream_table.end()) return 0;
+        b = std::move(it->second);
+        g_stream_table.erase(it);
+    }
+    { std::lock_guard<std::mutex> wait_for_the_last_holder(b->mu); }
+    HIP_TRY(hipStreamSynchronize(s));
+    if (b->ptr) (void)hipFree(b->ptr);
+    for (uint8_t *p : b->retired) (void)hipFree(p);
+    return 0;
+}
+
 struct FixedScratch {
     uint8_t *ptr = nullptr;
     size_t bytes = 0;
@@ -506,14 +528,12 @@ public:
             *out = transient_;
             return 0;
         }
-        static std::mutex table_mu;
-        static std::map<std::pair<int, hipStream_t>, std::unique_ptr<StreamBuffer>> table;
         int dev = 0;
         HIP_TRY(hipGetDevice(&dev));
         StreamBuffer *b;
         {
-            std::lock_guard<std::mutex> g(table_mu);
-            auto &slot = table[{dev, s}];
+            std::lock_guard<std::mutex> g(g_stream_table_mu);
+            auto &slot = g_stream_table[{dev, s}];
             if (!slot) slot.reset(new StreamBuffer);
             b = slot.get();
         }
@@ -1027,6 +1047,11 @@ int jq_try_matmul_fused(uint32_t ggml_type, size_t m, size_t k, size_t n, const 
                            (hipStream_t)stream);
 }
 
+int jq_stream_release(void *stream) {
+    if (ensure_init()) return 1;
+    return release_stream_scratch((hipStream_t)stream);
+}
+
 int jq_dequantize(const jq_weight *w, float *out, size_t out_len, int out_is_device, void *stream) {
     if (!w) return fail("jq_dequantize: weight is null");
     if (out_len != w->n * w->k)
@@ -1040,6 +1065,53 @@ int jq_dequantize(const jq_weight *w, float *out, size_t out_len, int out_is_dev
     if (dispatch_decode(w, nullptr, (float *)y.p, w->n, s)) return 1;
     HIP_TRY(hipMemcpyAsync(out, y.p, out_len * sizeof(float), hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int jq_decode_raw_to_f32(uint32_t ggml_type, const void *bytes, size_t nbytes, size_t elems, float *out,
+                         int ptrs_are_device, void *stream) {
+    if (ggml_type == 0) return 2;  // F32: the caller's own reader keeps it exact
+    const bool plain = ggml_type == 1 || ggml_type == 9 || ggml_type == 15;
+    size_t blck = 1, bb = 2;
+    if (ggml_type == 9) blck = 32, bb = 36;
+    else if (ggml_type == 15) blck = 256, bb = 292;
+    else if (!plain) {
+        Geometry g;
+        if (!geometry(ggml_type, &g)) return 2;  // no decoder in the reference either: Ok(None)
+        blck = g.elems, bb = g.bytes;
+    }
+    if (elems % blck != 0 || nbytes != elems / blck * bb) {
+        if (ggml_type == 1) return fail("dtype F16: %zu bytes for %zu elements", nbytes, elems);
+        return fail("dtype %u: %zu bytes for %zu elements (%zu per %zu-block)", ggml_type, nbytes, elems, bb, blck);
+    }
+    if (elems == 0) return 0;
+    if (!bytes || !out) return fail("jq_decode_raw_to_f32: null pointer");
+    if (ensure_init()) return 1;
+    hipStream_t s = (hipStream_t)stream;
+    DevBuf in, y;
+    const uint8_t *src = (const uint8_t *)bytes;
+    float *dst = out;
+    if (!ptrs_are_device) {
+        HIP_TRY(in.alloc(nbytes));
+        HIP_TRY(y.alloc(elems * sizeof(float)));
+        HIP_TRY(hipMemcpyAsync(in.p, bytes, nbytes, hipMemcpyHostToDevice, s));
+        src = (const uint8_t *)in.p, dst = (float *)y.p;
+    }
+    if (plain) {
+        const unsigned blocks = (unsigned)std::min<size_t>((elems + 255) / 256, 65535u * 16u);
+        if (ggml_type == 1) hipLaunchKernelGGL((jq::decode_plain<1>), dim3(blocks), dim3(256), 0, s, src, dst, elems);
+        else if (ggml_type == 9) hipLaunchKernelGGL((jq::decode_plain<9>), dim3(blocks), dim3(256), 0, s, src, dst, elems);
+        else hipLaunchKernelGGL((jq::decode_plain<15>), dim3(blocks), dim3(256), 0, s, src, dst, elems);
+        HIP_TRY(hipGetLastError());
+    } else {
+        jq_weight view{};  // one row of `elems` columns over the caller's bytes
+        view.type = ggml_type, view.dev = const_cast<uint8_t *>(src), view.n = 1, view.k = elems, view.row_bytes = nbytes;
+        if (dispatch_decode(&view, nullptr, dst, 1, s)) return 1;
+    }
+    if (!ptrs_are_device) {
+        HIP_TRY(hipMemcpyAsync(out, y.p, elems * sizeof(float), hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+    }
     return 0;
 }
 
@@ -1178,12 +1250,12 @@ void launch_moe_rows(const uint8_t *const *Wptr, size_t row_bytes, const float *
 // The LDS-staged grouped kernel when the rows allow it (aligned row starts, four waves' rows within
 // 64 KB); returns -1 when they do not and the caller takes the plain kernels.
 template <class Q, bool DUAL>
-int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
+int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align,
                       const float *X, const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y,
                       int k, int n, int groups, int max_group, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
-    const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
+    const int G = (row_bytes % 16 == 0 && base_align >= 16) ? 16 : (row_bytes % 4 == 0 && base_align >= 4) ? 4 : 0;
     const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
     if (G == 0 || wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>() > 64 * 1024 || getenv("JQ_NO_STAGED_ROWS")) return -1;
     dim3 grid((unsigned)((n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R)), (unsigned)groups), block(64 * jq::ROWS_PER_WG);
@@ -1204,13 +1276,13 @@ int launch_moe_staged(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t
 
 template <bool DUAL>
 int dispatch_moe_staged(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes,
-                        bool aligned16, const float *X, const int *gexp, const int *offsets, const int *xsel,
+                        int base_align, const float *X, const int *gexp, const int *offsets, const int *xsel,
                         const int *yrow, float *Y, int k, int n, int groups, int max_group, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     int rc;
     switch (type) {
 #define JQ_MOE_CASE(ID, Q)                                                                                          \
     case ID:                                                                                                        \
-        rc = launch_moe_staged<jq::Q, DUAL>(Wa, Wb, row_bytes, aligned16, X, gexp, offsets, xsel, yrow, Y, k, n,     \
+        rc = launch_moe_staged<jq::Q, DUAL>(Wa, Wb, row_bytes, base_align, X, gexp, offsets, xsel, yrow, Y, k, n,     \
                                             groups, max_group, s, cl);                                              \
         break;
         JQ_FOR_EACH_FORMAT(JQ_MOE_CASE)
@@ -1224,12 +1296,12 @@ int dispatch_moe_staged(uint32_t type, const uint8_t *const *Wa, const uint8_t *
 // Q4_K experts with several tokens per group: the LDS-ring MFMA kernel per group.
 // Returns -1 when the shape is outside its reach.
 template <bool DUAL>
-int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
+int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align,
                           const float *X, size_t x_rows, uint8_t *acts, const int *gexp, const int *offsets,
                           const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     const int nb = k / 256;
     static const char *off = getenv("JQ_MOE_NO_RING");
-    if (off || !acts || k % 256 != 0 || nb == 0 || nb > 16 || row_bytes != (size_t)nb * 144 || !aligned16 ||
+    if (off || !acts || k % 256 != 0 || nb == 0 || nb > 16 || row_bytes != (size_t)nb * 144 || base_align < 16 ||
         ((uintptr_t)X & 15) != 0)
         return -1;
     launch_q4k_acts_prep(X, x_rows, (size_t)k, acts, s);
@@ -1252,12 +1324,12 @@ int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, si
 // v_dot4 against the activation row as int8 planes, quantised by every workgroup itself (small
 // matrices) or once by acts_i8_prep (x_rows rows of X).  Returns -1 when the shape is outside its reach.
 template <class Q, bool DUAL>
-int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16, const float *X,
+int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align, const float *X,
                     size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets, const int *xsel, const int *yrow,
                     float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
-    const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
+    const int G = (row_bytes % 16 == 0 && base_align >= 16) ? 16 : (row_bytes % 4 == 0 && base_align >= 4) ? 4 : 0;
     // every workgroup of a group redoing the row's quantisation is cheaper than a launch up to about
     // half a million elements a group
     const size_t wgs = (n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R);
@@ -1283,14 +1355,14 @@ int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t r
 }
 
 template <bool DUAL>
-int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, bool aligned16,
+int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align,
                       const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets,
                       const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
     if (!moe_has_dot8(type) || k % 32 != 0 || ((uintptr_t)X & 15) != 0) return -1;
     switch (type) {
 #define JQ_DOT8_CASE(ID, Q)                                                                                         \
     case ID:                                                                                                        \
-        return launch_moe_dot8<jq::Q, DUAL>(Wa, Wb, row_bytes, aligned16, X, x_rows, xq, gexp, offsets, xsel, yrow, Y, k, n, \
+        return launch_moe_dot8<jq::Q, DUAL>(Wa, Wb, row_bytes, base_align, X, x_rows, xq, gexp, offsets, xsel, yrow, Y, k, n, \
                                             groups, s, cl);
         JQ_DOT8_CASE(JQ_TYPE_MXFP4, MXFP4)
         JQ_DOT8_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
@@ -1304,12 +1376,12 @@ int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *co
 // tokens, k_used routed pairs each plus n_extra for a folded shared expert, activations the rows of X
 // in pair order.  Returns -1 when the shape is outside its reach.
 template <class Q>
-int launch_moe_down_combine(const uint8_t *const *Wa, size_t row_bytes, bool aligned16, const float *X, size_t x_rows,
+int launch_moe_down_combine(const uint8_t *const *Wa, size_t row_bytes, int base_align, const float *X, size_t x_rows,
                             jq::ActsI8 xq, const int *gexp, const float *wts, float *y, int k, int n, int T, int k_used,
                             int n_extra, hipStream_t s) {
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS, S = k_used + n_extra;
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
-    const int G = (row_bytes % 16 == 0 && aligned16) ? 16 : (row_bytes % 4 == 0) ? 4 : 0;
+    const int G = (row_bytes % 16 == 0 && base_align >= 16) ? 16 : (row_bytes % 4 == 0 && base_align >= 4) ? 4 : 0;
     const size_t wgs = (n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R);
     const bool own = wgs * (size_t)k <= 512 * 1024 || !xq.xl;  // as in launch_moe_dot8
     const size_t slot_lds = ((size_t)R * row_bytes + 15) / 16 * 16;
@@ -1342,7 +1414,7 @@ int launch_moe_down_combine(const uint8_t *const *Wa, size_t row_bytes, bool ali
     return 0;
 }
 
-int dispatch_moe_down_combine(uint32_t type, const uint8_t *const *Wa, size_t row_bytes, bool aligned16, const float *X,
+int dispatch_moe_down_combine(uint32_t type, const uint8_t *const *Wa, size_t row_bytes, int base_align, const float *X,
                               size_t x_rows, jq::ActsI8 xq, const int *gexp, const float *wts, float *y, int k, int n,
                               int T, int k_used, int n_extra, hipStream_t s) {
     static const char *off = getenv("JQ_MOE_NO_DOWN_COMBINE");
@@ -1350,7 +1422,7 @@ int dispatch_moe_down_combine(uint32_t type, const uint8_t *const *Wa, size_t ro
     switch (type) {
 #define JQ_DC_CASE(ID, Q)                                                                                           \
     case ID:                                                                                                        \
-        return launch_moe_down_combine<jq::Q>(Wa, row_bytes, aligned16, X, x_rows, xq, gexp, wts, y, k, n, T, k_used, \
+        return launch_moe_down_combine<jq::Q>(Wa, row_bytes, base_align, X, x_rows, xq, gexp, wts, y, k, n, T, k_used, \
                                               n_extra, s);
         JQ_DC_CASE(JQ_TYPE_MXFP4, MXFP4)
         JQ_DC_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
@@ -1413,8 +1485,16 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     }
     HIP_TRY(hipGetLastError());
     // silu(gate x) * (up x) of every pair into G, then down over it
-    const bool a16 = ((uintptr_t)m->gate->dev & 15) == 0 && ((uintptr_t)m->up->dev & 15) == 0 &&
-                     (!m->fold_shared || (((uintptr_t)m->sgate->dev & 15) == 0 && ((uintptr_t)m->sup->dev & 15) == 0));
+    // What every expert's first byte is a multiple of (a view may start at any whole block, and blocks of 17,
+    // 34, 66, 210 bytes put that anywhere): 16-byte and 4-byte loads into LDS want it, the kernels that read
+    // through registers do not.
+    auto align_of = [](std::initializer_list<const jq_weight *> ws) {
+        uintptr_t bits = 0;
+        for (const jq_weight *w : ws)
+            if (w) bits |= (uintptr_t)w->dev;
+        return (bits & 15) == 0 ? 16 : (bits & 3) == 0 ? 4 : 1;
+    };
+    const int a16 = align_of({m->gate, m->up, m->fold_shared ? m->sgate : nullptr, m->fold_shared ? m->sup : nullptr});
     int rc = -1;
     const bool same_gu = m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes;
     if (same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K)
@@ -1438,7 +1518,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
                                      m->yrow, m->U, (int)c.hidden, (int)c.inter, groups, max_group, s))
             return 1;
     }
-    const bool d16 = ((uintptr_t)m->down->dev & 15) == 0 && (!m->fold_shared || ((uintptr_t)m->sdown->dev & 15) == 0);
+    const int d16 = align_of({m->down, m->fold_shared ? m->sdown : nullptr});
     rc = -1;
     if (fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K)
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,

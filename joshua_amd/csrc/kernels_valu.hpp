@@ -262,4 +262,23 @@ __global__ __launch_bounds__(256) void decode_rows(const uint8_t *__restrict__ W
     }
 }
 
+// Raw tensor bytes that are no weight format of the matmuls, to f32 (reference: src/quant_matmul.rs:36-103
+// decode_raw_to_f32): KIND 1 = F16 elements, 9 = Q8_1 blocks (f16 d, f16 s, 32 int8: d * q, the published ggml
+// layout), 15 = Q8_K blocks (f32 d, 256 int8, 16 int16 sums: d * q).  One element a thread.
+template <int KIND>
+__global__ __launch_bounds__(256) void decode_plain(const uint8_t *__restrict__ raw, float *__restrict__ out, size_t elems) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < elems; i += (size_t)gridDim.x * blockDim.x) {
+        if (KIND == 1) {
+            out[i] = f16_bits((uint32_t)raw[2 * i] | ((uint32_t)raw[2 * i + 1] << 8));
+        } else {
+            constexpr size_t BLCK = KIND == 9 ? 32 : 256, BB = KIND == 9 ? 36 : 292;
+            const uint8_t *blk = raw + (i / BLCK) * BB;
+            float d;
+            if (KIND == 9) d = f16_bits((uint32_t)blk[0] | ((uint32_t)blk[1] << 8));
+            else d = __builtin_bit_cast(float, (uint32_t)blk[0] | ((uint32_t)blk[1] << 8) | ((uint32_t)blk[2] << 16) | ((uint32_t)blk[3] << 24));
+            out[i] = d * (float)(int8_t)blk[4 + i % BLCK];
+        }
+    }
+}
+
 }  // namespace jq

@@ -49,6 +49,7 @@ def lib() -> ctypes.CDLL:
         sz, u32, vp, fp = ctypes.c_size_t, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p
         L.orc_block_geometry.argtypes = [u32, ctypes.POINTER(sz), ctypes.POINTER(sz)]
         L.orc_dequantize.argtypes = [u32, vp, sz, fp]
+        L.orc_decode_raw_to_f32.argtypes = [u32, vp, sz, sz, fp]
         L.orc_matmul_t.argtypes = [u32, sz, sz, sz, fp, sz, vp, sz, fp, sz]
         L.orc_matmul_t_avx2.argtypes = [u32, sz, sz, sz, fp, sz, vp, sz, fp, sz, ctypes.c_int]
         L.orc_iq2xxs_matmul_scalar.argtypes = [sz, sz, sz, fp, sz, vp, sz, fp, sz]
@@ -91,6 +92,18 @@ def dequantize(qtype: int, blocks) -> np.ndarray:
     nblocks = raw.size // nbytes
     out = np.empty(nblocks * elems, dtype=np.float32)
     _check(lib().orc_dequantize(qtype, raw.ctypes.data, nblocks, out.ctypes.data))
+    return out
+
+
+def decode_raw_to_f32(dtype: int, raw, elems: int):
+    """The reference's decode_raw_to_f32 (src/quant_matmul.rs:36-103): f32 values, or None where the reference
+    answers None (F32 and types without a decoder there)."""
+    raw = _bytes_arr(raw)
+    out = np.empty(elems, dtype=np.float32)
+    rc = lib().orc_decode_raw_to_f32(dtype, raw.ctypes.data, raw.size, elems, out.ctypes.data)
+    if rc == 2:
+        return None
+    _check(rc)
     return out
 
 

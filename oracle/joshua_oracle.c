@@ -326,6 +326,42 @@ int orc_dequantize(uint32_t type, const void *blocks, size_t nblocks, float *out
     return 0;
 }
 
+
+/* decode_raw_to_f32 (reference: src/quant_matmul.rs:36-103): raw tensor bytes of ggml type `dtype` to f32.
+ * Returns 0 with `out` filled, 2 where the reference answers None (F32, and every type without a decoder
+ * there: the caller keeps its own reader), 1 with a message on a size mismatch.  F16 is converted per
+ * element (:71-80); Q8_K is d * q with an f32 d (4 + 256 + 32 bytes a block); Q8_1 is d * q with an f16 d
+ * (2 + 2 + 32 bytes a block) by the published ggml layout -- parity unpinned for Q8_1: the reference hands it
+ * to candle-core 0.11's BlockQ8_1::to_float, which is not in the tree. */
+int orc_decode_raw_to_f32(uint32_t dtype, const void *bytes, size_t nbytes, size_t elems, float *out) {
+    const uint8_t *p = (const uint8_t *)bytes;
+    if (dtype == 0) return 2;
+    if (dtype == 1) {
+        if (nbytes != elems * 2) return orc_fail("dtype F16: %zu bytes for %zu elements", nbytes, elems);
+        for (size_t i = 0; i < elems; i++) out[i] = orc_f16_to_f32((uint16_t)(p[2 * i] | (p[2 * i + 1] << 8)));
+        return 0;
+    }
+    if (dtype == 9 || dtype == 15) {
+        const size_t blck = dtype == 9 ? 32 : 256, bb = dtype == 9 ? 36 : 292;
+        if (elems % blck != 0 || nbytes != elems / blck * bb)
+            return orc_fail("dtype %u: %zu bytes for %zu elements (%zu per %zu-block)", dtype, nbytes, elems, bb, blck);
+        for (size_t b = 0; b < elems / blck; b++) {
+            const uint8_t *blk = p + b * bb;
+            float d;
+            if (dtype == 9) d = orc_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+            else memcpy(&d, blk, 4);
+            const int8_t *q = (const int8_t *)(blk + 4);
+            for (size_t e = 0; e < blck; e++) out[b * blck + e] = d * (float)q[e];
+        }
+        return 0;
+    }
+    size_t be, bb;
+    if (!deq_for(dtype) || orc_block_geometry(dtype, &be, &bb)) return 2;
+    if (elems % be != 0 || nbytes != elems / be * bb)
+        return orc_fail("dtype %u: %zu bytes for %zu elements (%zu per %zu-block)", dtype, nbytes, elems, bb, be);
+    return orc_dequantize(dtype, bytes, elems / be, out);
+}
+
 /* ---- matmul in the reference's x86_64 operation order ------------------ */
 
 /* Shared shape check (reference: src/quant_matmul.rs:133-165,

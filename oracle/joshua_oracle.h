@@ -30,6 +30,9 @@
  *                            to_float) whose source is not available, so the
  *                            ulp-level operation order ((d*sc)*q) is
  *                            PARITY UNPINNED.
+ *   orc_decode_raw_to_f32 F16, Q8_K  pinned: numpy's own float16 conversion and d * q written in numpy
+ *                             (tests/test_decode_raw.py); Q8_1: parity unpinned (candle-core 0.11's
+ *                             BlockQ8_1::to_float is not in the tree; ggml's published layout is used)
  *   orc_dequantize Q4_0/Q4_1/Q5_0/Q5_1/Q3_K/Q5_K  pinned on layout by an
  *                            independent numpy decode written from the block
  *                            definitions and by exhaustive sweeps of every
@@ -79,6 +82,8 @@ int orc_block_geometry(uint32_t type, size_t *elems, size_t *bytes);
 
 /* Canonical decode ("to_float") of `nblocks` blocks into out[nblocks*elems]. */
 int orc_dequantize(uint32_t type, const void *blocks, size_t nblocks, float *out);
+/* 0: decoded; 2: the reference answers None for this type; 1: error (reference: src/quant_matmul.rs:36-103) */
+int orc_decode_raw_to_f32(uint32_t dtype, const void *bytes, size_t nbytes, size_t elems, float *out);
 
 /* dst[m,n] = lhs[m,k] . W[n,k]^T in the reference's x86_64 operation order.
  * `lhs_len`/`dst_len` are element counts, `nbytes` the byte length of

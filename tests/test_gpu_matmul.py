@@ -916,3 +916,44 @@ def test_q4k_int8_gemm_small_shapes_in_a_child_process(shape):
     env = dict(os.environ, JQ_Q4K_GEMM_I8_MIN_TILES="1", JQ_Q4K_GEMM_I8_SHAPE=shape)
     res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1)], env=env, capture_output=True, text=True, timeout=170)
     assert res.returncode == 0 and "gemm i8 ok" in res.stdout, res.stdout + res.stderr
+
+
+def test_graph_captured_before_the_stream_scratch_grows_still_replays():
+    """A 16-row Q4_K product (prepared activations in the stream's scratch buffer) is captured in a HIP graph;
+    then a 512-row product on the same stream makes that buffer grow.  The old buffer is retired, not freed,
+    so the graph, which names it, replays to the eager result every time, with eager work in between."""
+    import torch
+    n, k = 2048, 4096
+    blocks = make_blocks(capi.Q4_K, n, k, 411)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    big = capi.Weight.upload(capi.Q4_K, make_blocks(capi.Q4_K, 14336, k, 412), 14336, k)
+    stream = torch.cuda.Stream()
+    x16 = torch.from_numpy(synth.normal(413, (16, k))).cuda()
+    y16 = torch.zeros(16 * n, device="cuda")
+    xb = torch.from_numpy(synth.normal(414, (512, k))).cuda()
+    yb = torch.zeros(512 * 14336, device="cuda")
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        w.matmul_t_dev(16, x16.data_ptr(), x16.numel(), y16.data_ptr(), y16.numel(), stream.cuda_stream)  # first use allocates
+        stream.synchronize()
+        want = y16.clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            w.matmul_t_dev(16, x16.data_ptr(), x16.numel(), y16.data_ptr(), y16.numel(), torch.cuda.current_stream().cuda_stream)
+        cap_stream = stream.cuda_stream
+        for rep in range(3):
+            # a larger product on the stream the first call warmed up: its scratch buffer grows on the first pass
+            big.matmul_t_dev(512, xb.data_ptr(), xb.numel(), yb.data_ptr(), yb.numel(), cap_stream)
+            y16.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y16, want), rep
+    assert np.all(np.isfinite(yb[:14336].cpu().numpy()))
+    del graph
+    torch.cuda.synchronize()
+    capi.stream_release(stream.cuda_stream)
+    capi.stream_release(stream.cuda_stream)      # nothing left to free: not an error
+    with torch.cuda.stream(stream):              # the stream serves calls again after a release
+        w.matmul_t_dev(16, x16.data_ptr(), x16.numel(), y16.data_ptr(), y16.numel(), stream.cuda_stream)
+        stream.synchronize()
+    assert torch.equal(y16, want)

@@ -178,3 +178,32 @@ def test_swiglu_clamp(qtype, h, inter, tokens, shared_inter):
     want = ora.forward(x)
     assert not close(want, plain.forward(x))          # the limits change the result
     assert close(dev.forward(x), want)
+
+
+@pytest.mark.parametrize("qtype,lead_blocks", [(capi.Q8_0, 1), (capi.MXFP4, 3), (capi.IQ2_XXS, 1), (capi.Q6_K, 1)])
+def test_experts_that_are_views_at_odd_block_offsets(qtype, lead_blocks):
+    """Expert stacks that start mid-buffer, a whole number of 34-, 17-, 66- or 210-byte blocks in: their
+    first byte is 1- or 2-byte aligned while every row is a multiple of 4 bytes long, so the kernels that load
+    rows into LDS four or sixteen bytes at a time must stand aside (one and five tokens: the decode-sized and
+    the grouped dispatch)."""
+    h, inter, E, k_used, seed = 1024, 512, 8, 2, 300 + qtype
+    bb = oracle.block_geometry(qtype)[1]
+    lead = lead_blocks * bb
+    assert lead % 4 != 0
+    parts, views = [], []
+    for i, (rows, cols) in enumerate(((inter, h), (inter, h), (h, inter))):
+        blocks = synth.normal_quantized(qtype, seed + i, E * rows * cols, 0.02)
+        parts.append(blocks)
+        buf = np.concatenate([np.zeros(lead, np.uint8), blocks])
+        # the parent: one row of whole blocks that spans the buffer; the view: the stack behind the lead
+        per_block = oracle.block_geometry(qtype)[0]
+        parent = capi.Weight.upload(qtype, buf, 1, buf.size // bb * per_block)
+        views.append(parent.view(lead, E * rows, cols))
+    rw = synth.normal(seed + 9, (E, h), 0.02)
+    ora = MoeOracle(qtype, h, inter, E, k_used, rw, parts[0], parts[1], parts[2], avx2=oracle.have_avx2())
+    cfg = capi.MoeConfig(E, k_used, h, inter, 0, 1, 0.0, 1, 1, 0.0, 0.0)
+    dev = capi.Moe(cfg, rw, views[0], views[1], views[2])
+    for tokens in (1, 5):
+        x = synth.normal(seed + 20 + tokens, (tokens, h))
+        assert close(dev.forward(x), ora.forward(x)), (capi.TYPE_NAMES[qtype], tokens)
+    dev.close()
