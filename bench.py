@@ -224,7 +224,7 @@ DEEPSEEK_V3_MLA = dict(n_embd=7168, n_head=128, q_lora_rank=1536, kv_lora_rank=5
                        yarn_mscale_all_dim=1.0, yarn_orig_context_length=4096)
 
 
-def mla_workload(torch, capi, synth, qtype: int, context: int, steps: int, seed: int) -> dict:
+def mla_workload(torch, capi, synth, qtype: int, context: int, steps: int, seed: int, cpu_seconds: float = 0.0) -> dict:
     """One multi-head latent attention block of DeepSeek-V3 size: a prompt of `context` tokens in chunks of
     512, then `steps` single-token calls (the cache grows by one token a call)."""
     c = DEEPSEEK_V3_MLA
@@ -257,6 +257,17 @@ def mla_workload(torch, capi, synth, qtype: int, context: int, steps: int, seed:
     ref = om.MlaOracle(oc, ot)
     parity_ok = _close(mla.forward(xs_host[:64], 0), ref.forward(xs_host[:64], 0))
     parity_ok = parity_ok and _close(mla.forward(xs_host[64:65], 64), ref.forward(xs_host[64:65], 64))
+    cpu = None
+    if cpu_seconds > 0:  # the oracle's single-token step, at the short context it can afford
+        import time
+        t_cpu = []
+        for p in range(65, 68):
+            t0 = time.perf_counter()
+            ref.forward(xs_host[p:p + 1], p)
+            t_cpu.append(time.perf_counter() - t0)
+        cpu = {"us": round(sorted(t_cpu)[1] * 1e6, 1), "cores": os.cpu_count(), "kind": "port",
+               "sample": "median of 3 single-token steps of oracle/mla.py (numpy, the reference's unabsorbed form over "
+                         "decoded weights) at a 65-67 token context; the device figure is at the full context"}
     mla.reset()
     xs = torch.from_numpy(xs_host).to(dev)
     y = torch.zeros((chunk, c["n_embd"]), device=dev)
@@ -284,6 +295,8 @@ def mla_workload(torch, capi, synth, qtype: int, context: int, steps: int, seed:
            "parity_ok": parity_ok, "parity_note": "64-token prefill and one step against the reference's unabsorbed form",
            "cache_bytes_per_token": 4 * (c["kv_lora_rank"] + c["qk_rope_head_dim"]),
            "reference_cache_bytes_per_token": 4 * nh * (qd + c["v_head_dim"])}
+    if cpu:
+        res["cpu_baseline"] = cpu
     mla.close()
     return res
 
@@ -307,6 +320,9 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
             out["q2_k_gemv_14336x4096_m1"] = matmul_workload(torch, capi, synth, 10, N, K, 1, 108, steps, 24, 0.0)
         elif only == "moe_b1":
             out["moe_qwen3_30b_a3b_q4_k_b1"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 1, 104, steps, False, 0, 0.0)
+        elif only == "moe_b64":
+            out["moe_qwen3_30b_a3b_q4_k_b64"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 64, 104, max(steps // 10, 10),
+                                                             False, 0, 0.0)
         elif only == "moe_v3":
             out["moe_deepseek_v3_iq2_xxs_b1"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 1, 105, steps, True, 1, 0.0)
         return out
@@ -327,7 +343,7 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
                                                    True, 1, cs)
     torch.cuda.empty_cache()
     for context in (1024, 8192):
-        out[f"mla_deepseek_v3_q4_k_ctx{context}_b1"] = mla_workload(torch, capi, synth, 12, context, min(steps, 100), 107)
+        out[f"mla_deepseek_v3_q4_k_ctx{context}_b1"] = mla_workload(torch, capi, synth, 12, context, min(steps, 100), 107, cs)
         torch.cuda.empty_cache()
     return out
 

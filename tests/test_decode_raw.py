@@ -50,6 +50,7 @@ def test_oracle_plain_types_against_numpy():
 def test_oracle_none_and_errors():
     assert oracle.decode_raw_to_f32(0, np.zeros(16, np.uint8), 4) is None          # F32: the caller's reader
     assert oracle.decode_raw_to_f32(26, np.zeros(16, np.uint8), 4) is None         # an I32 table: no decoder
+    assert oracle.decode_raw_to_f32(30, np.zeros(8, np.uint8), 4) is None          # BF16: no arm in the reference's match
     with pytest.raises(oracle.OracleError, match="dtype F16: 7 bytes for 4 elements"):
         oracle.decode_raw_to_f32(1, np.zeros(7, np.uint8), 4)
     with pytest.raises(oracle.OracleError, match="144-byte|per 256-block"):
@@ -77,6 +78,7 @@ def test_device_decode_raw_against_the_oracle():
         assert np.array_equal(capi.decode_raw_to_f32(qt, blocks, 2048), oracle.decode_raw_to_f32(qt, blocks, 2048)), qt
     assert capi.decode_raw_to_f32(0, np.zeros(16, np.uint8), 4) is None
     assert capi.decode_raw_to_f32(26, np.zeros(16, np.uint8), 4) is None
+    assert capi.decode_raw_to_f32(30, np.zeros(8, np.uint8), 4) is None
     with pytest.raises(capi.JoshuaHipError, match="dtype F16: 7 bytes for 4 elements"):
         capi.decode_raw_to_f32(1, np.zeros(7, np.uint8), 4)
     with pytest.raises(capi.JoshuaHipError, match="per 256-block"):
