@@ -28,6 +28,7 @@
 #include "kernels_dot4_q8.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
+#include "kernels_moe_q4k_quads.hpp"
 #include "kernels_mfma_q4k_rows16.hpp"
 #include "kernels_mfma_q4k_gemm_i8.hpp"
 #include "kernels_valu.hpp"
@@ -1320,6 +1321,37 @@ int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, si
     return 0;
 }
 
+// Q4_K experts with a few tokens per group (four on average at batch 64 over 128 experts): the int8 kernel
+// that multiplies four activation rows an MFMA.  Returns -1 when the shape is outside its reach.
+template <bool DUAL>
+int dispatch_moe_q4k_quads(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align,
+                           const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets,
+                           const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s,
+                           const jq::MoeClamp &cl = jq::MoeClamp{}) {
+    const int nb = k / 256;
+    static const char *off = getenv("JQ_MOE_NO_QUADS");
+    if (off || !xq.xl || k % 256 != 0 || nb < 2 || nb > 16 || row_bytes != (size_t)nb * 144 || base_align < 16 ||
+        ((uintptr_t)X & 15) != 0)
+        return -1;
+    const size_t words = x_rows * (size_t)(k / 4);
+    hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
+    const int maxnb = nb > 8 ? 16 : nb > 4 ? 8 : 4, n_tiles = (n + 15) / 16;
+    // 2048 workgroups a launch (measured at 128 groups of 768 x 2048: 8 a group 184 us a layer call, 16: 173,
+    // 24: 177, 48: 202; the f16 ring kernel: 204 at 8 and more above)
+    static const char *genv = getenv("JQ_MOE_QUADS_GRID");
+    const int per_group = genv ? atoi(genv) : 2048 / std::max(groups, 1);
+    dim3 grid((unsigned)std::min(n_tiles, std::max(per_group, 1)), (unsigned)groups), block(64 * nb);
+#define JQ_QUADS(MAXNB)                                                                                            \
+    hipLaunchKernelGGL((jq::moe_q4k_quads_mfma<MAXNB, DUAL>), grid, block, 0, s, Wa, Wb, xq, gexp, offsets, xsel,  \
+                       yrow, Y, k, n, cl)
+    if (maxnb == 16) JQ_QUADS(16);
+    else if (maxnb == 8) JQ_QUADS(8);
+    else JQ_QUADS(4);
+#undef JQ_QUADS
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // One activation row a group, a format with Q::dot8: expert rows staged through LDS and multiplied on
 // v_dot4 against the activation row as int8 planes, quantised by every workgroup itself (small
 // matrices) or once by acts_i8_prep (x_rows rows of X).  Returns -1 when the shape is outside its reach.
@@ -1497,7 +1529,14 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     const int a16 = align_of({m->gate, m->up, m->fold_shared ? m->sgate : nullptr, m->fold_shared ? m->sup : nullptr});
     int rc = -1;
     const bool same_gu = m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes;
-    if (same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K)
+    // few tokens an expert (at most six on average): the int8 kernel that takes four rows an MFMA; more: the
+    // f16 ring kernel, which reads a group's weights once for up to 16 rows
+    const bool few = (size_t)P <= 6 * (size_t)c.n_expert;
+    if (same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K && few)
+        rc = dispatch_moe_q4k_quads<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp, m->offsets,
+                                          m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
+    if (rc > 0) return 1;
+    if (rc < 0 && same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K)
         rc = dispatch_moe_q4k_ring<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qacts, m->gexp, m->offsets,
                                          m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
     if (rc > 0) return 1;
@@ -1520,7 +1559,12 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     }
     const int d16 = align_of({m->down, m->fold_shared ? m->sdown : nullptr});
     rc = -1;
-    if (fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K)
+    if (fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && few)
+        rc = dispatch_moe_q4k_quads<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
+                                           m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
+                                           (int)c.hidden, groups, s);
+    if (rc > 0) return 1;
+    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K)
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);

@@ -207,3 +207,20 @@ def test_experts_that_are_views_at_odd_block_offsets(qtype, lead_blocks):
         x = synth.normal(seed + 20 + tokens, (tokens, h))
         assert close(dev.forward(x), ora.forward(x)), (capi.TYPE_NAMES[qtype], tokens)
     dev.close()
+
+
+@pytest.mark.parametrize("tokens", [9, 20, 40])
+def test_few_tokens_an_expert_take_the_int8_quads_kernel(tokens):
+    """16 experts, top-2: 18 to 80 pairs over 16 experts is at most five a group on average, the range of the
+    int8 kernel that multiplies four activation rows an MFMA (one quad, two quads, and groups of more than
+    eight rows, which take a second pass over the weights); inter 768 gives its down projection three waves a
+    workgroup, hidden 2048 its gate and up eight."""
+    ora, dev = build(capi.Q4_K, 2048, 768, 16, 2, 90)
+    x = synth.normal(91 + tokens, (tokens, 2048))
+    if tokens == 40:
+        x[:12] = x[0] + 0.01 * x[:12]                # a dozen tokens that route alike
+    ids, _ = dev.route(x)
+    counts = np.bincount(ids.reshape(-1), minlength=16)
+    if tokens == 40:
+        assert counts.max() > 8                      # at least one group needs two passes
+    assert close(dev.forward(x), ora.forward(x))
