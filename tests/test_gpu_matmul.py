@@ -957,3 +957,39 @@ def test_graph_captured_before_the_stream_scratch_grows_still_replays():
         w.matmul_t_dev(16, x16.data_ptr(), x16.numel(), y16.data_ptr(), y16.numel(), stream.cuda_stream)
         stream.synchronize()
     assert torch.equal(y16, want)
+
+
+def _random_shapes(seed, count):
+    rng = np.random.default_rng(seed)
+    ms = [1, 2, 3, 4, 7, 8, 15, 16, 17, 24, 33, 64, 65, 100, 128, 200, 300]
+    ks = [256, 512, 768, 1024, 2048, 4096, 8192, 12288]
+    out = []
+    while len(out) < count:
+        m, k = int(rng.choice(ms)), int(rng.choice(ks))
+        n = int(rng.integers(1, 20000)) if rng.random() < 0.3 else int(rng.integers(1, 3000))
+        if m * k * n <= 1.2e9:
+            out.append((m, k, n))
+    return out
+
+
+@pytest.mark.parametrize("m,k,n", _random_shapes(2024, 48))
+def test_q4k_random_shapes_across_the_dispatcher(m, k, n):
+    """Seeded random (rows, row length, weight rows) triples: whatever kernel the dispatcher picks for a shape
+    (one-row kernels, 16-row passes, streaming, ring, int8 and f16 GEMMs, their ragged edges), the result
+    holds the reference's bound against the oracle."""
+    blocks = make_blocks(capi.Q4_K, n, k, 500 + (m * 31 + k * 7 + n) % 1000)
+    lhs = synth.normal(600 + n % 97, (m, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
+    want = oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())
+    assert close(got, want), (m, k, n, capi.last_kernel())
+
+
+@pytest.mark.parametrize("qtype", [capi.Q8_0, capi.Q2_K, capi.Q6_K, capi.IQ2_XXS, capi.MXFP4])
+@pytest.mark.parametrize("m,k,n", _random_shapes(77, 6))
+def test_other_formats_random_shapes(qtype, m, k, n):
+    n = min(n, 2500)
+    blocks = make_blocks(qtype, n, k, 700 + qtype)
+    lhs = synth.normal(800 + n % 89, (m, k))
+    got = capi.Weight.upload(qtype, blocks, n, k).matmul_t(m, lhs)
+    want = oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())
+    assert close(got, want), (capi.TYPE_NAMES[qtype], m, k, n, capi.last_kernel())
