@@ -1490,6 +1490,19 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
     jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
                          (int)c.n_group, (int)c.topk_group};
     size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);
+    // no expert groups and at most 256 experts: one wave a token, reductions in registers
+    static const char *no_wave = getenv("JQ_MOE_NO_WAVE_GATE");
+    if (!no_wave && c.n_group <= 1 && c.n_expert <= 256 && c.n_expert_used <= 64) {
+        const int ne = (int)(c.n_expert + 63) / 64;
+#define JQ_GATE(NE) hipLaunchKernelGGL(jq::moe_gate_topk_wave<NE>, dim3((unsigned)T), dim3(64), 0, s, m->logits, m->router_bias, gp, m->ids, m->wts, pg)
+        if (ne == 1) JQ_GATE(1);
+        else if (ne == 2) JQ_GATE(2);
+        else if (ne == 3) JQ_GATE(3);
+        else JQ_GATE(4);
+#undef JQ_GATE
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
     hipLaunchKernelGGL(jq::moe_gate_topk, dim3((unsigned)T), dim3(256), sm, s, m->logits, m->router_bias, gp, m->ids,
                        m->wts, pg);
     HIP_TRY(hipGetLastError());

@@ -173,6 +173,90 @@ __global__ __launch_bounds__(256) void moe_gate_topk(const float *__restrict__ l
     }
 }
 
+// The same gating by ONE wave per token, for layers without expert groups and with at most 256 experts: lane l
+// holds experts l, l + 64, ..., the softmax and each of the k_used arg-max rounds are register-to-register
+// reductions (no LDS, no barrier), where moe_gate_topk's 256 threads meet at eight barriers and rank every
+// expert against every other through LDS: 3 us a launch instead of 7.  Equal scores go to the lower expert
+// index, as there.
+template <int NE>
+__global__ __launch_bounds__(64) void moe_gate_topk_wave(const float *__restrict__ logits, const float *__restrict__ bias,
+                                                          MoeGateParams p, uint32_t *__restrict__ ids,
+                                                          float *__restrict__ wts, MoePairGroups pg) {
+    const int t = blockIdx.x, T = gridDim.x, lane = threadIdx.x;
+    const float *lg = logits + (size_t)t * p.E;
+    float prob[NE], sel[NE];
+    {
+        float v[NE];
+#pragma unroll
+        for (int i = 0; i < NE; i++) v[i] = lane + 64 * i < p.E ? lg[lane + 64 * i] : -INFINITY;
+        if (p.sigmoid) {
+#pragma unroll
+            for (int i = 0; i < NE; i++) prob[i] = 1.0f / (1.0f + expf(-v[i]));
+        } else {
+            float mx = v[0];
+#pragma unroll
+            for (int i = 1; i < NE; i++) mx = fmaxf(mx, v[i]);
+            mx = wave_max(mx);
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NE; i++) {
+                prob[i] = lane + 64 * i < p.E ? expf(v[i] - mx) : 0.0f;
+                sum += prob[i];
+            }
+            sum = wave_sum(sum);
+#pragma unroll
+            for (int i = 0; i < NE; i++) prob[i] = prob[i] / sum;
+        }
+#pragma unroll
+        for (int i = 0; i < NE; i++)
+            sel[i] = lane + 64 * i < p.E ? prob[i] + (bias ? bias[lane + 64 * i] : 0.0f) : -INFINITY;
+    }
+    int my_e = 0;
+    float my_p = 0.0f;  // lane r keeps slot r
+    for (int r = 0; r < p.k_used; r++) {
+        float best = sel[0];
+        int bi = 0;
+#pragma unroll
+        for (int i = 1; i < NE; i++)
+            if (sel[i] > best) best = sel[i], bi = i;  // the lower index stays on a tie
+        const float top = wave_max(best);
+        const float cand = best == top ? (float)(lane + 64 * bi) : 1e9f;
+        const int e = __builtin_amdgcn_readfirstlane((int)(-wave_max(-cand)));  // the lowest expert index among the ties
+        const int owner = e & 63, slot = e >> 6;
+        float pw = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NE; i++) {
+            if (i == slot) {
+                pw = prob[i];
+                if (lane == owner) sel[i] = -INFINITY;
+            }
+        }
+        pw = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pw), owner));
+        if (lane == r) my_e = e, my_p = pw;
+    }
+    float w = my_p;
+    if (p.norm_topk) {
+        float s = 0.0f;
+        for (int j = 0; j < p.k_used; j++) s += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_p), j));
+        w = w / fmaxf(s, 6.103515625e-5f);
+    }
+    if (p.scale != 0.0f && p.scale != 1.0f) w = w * p.scale;
+    if (lane < p.k_used) {
+        const int pidx = t * p.k_used + lane;
+        ids[pidx] = (uint32_t)my_e;
+        wts[pidx] = w;
+        if (pg.gexp) pg.gexp[pidx] = my_e, pg.offsets[pidx] = pidx, pg.xrow[pidx] = t, pg.yrow[pidx] = pidx;
+    }
+    if (pg.gexp && lane == 0) {
+        const int P = T * p.k_used, total = P + pg.n_extra * T;
+        if (t == 0) pg.offsets[total] = total;
+        if (pg.n_extra) {  // the shared expert as one more pair of this token
+            const int pidx = P + t;
+            pg.gexp[pidx] = p.E, pg.offsets[pidx] = pidx, pg.xrow[pidx] = t, pg.yrow[pidx] = pidx;
+        }
+    }
+}
+
 // Groups the T*k routed (token, slot) pairs by expert, keeping pair order inside
 // a group (the reference buckets the same way on the host,
 // src/quantized_qwen3_moe.rs:459-480).  Group e is expert e:
