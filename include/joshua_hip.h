@@ -136,7 +136,8 @@ int jq_dequantize(const jq_weight *w, float *out, size_t out_len, int out_is_dev
 
 /* Frees the scratch memory the library keeps for `stream` on the current device (the buffer the products
  * with prepared activations share, and every smaller one it outgrew), after waiting for the stream.  For
- * teardown: a HIP graph captured on the stream names those buffers and must not be replayed afterwards.  No
+ * teardown: a HIP graph captured on the stream names those buffers and must not be replayed afterwards, and no
+ * other thread may have a call in progress on that stream.  No
  * counterpart in the reference (its scratch is host memory owned by each call). */
 int jq_stream_release(void *stream);
 
