@@ -663,13 +663,15 @@ struct GemmI8Shape {
     int nw, ng;
 };
 
-int dispatch_q4k_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
-                         hipStream_t s) {
+template <class F>
+int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
+                     hipStream_t s, const char *name) {
+    constexpr size_t ALIGN = F::BLOCK % 16 == 0 ? 16 : 2;
     static const char *mode = getenv("JQ_Q4K_GEMM_I8");
     static const char *min_tiles_env = getenv("JQ_Q4K_GEMM_I8_MIN_TILES");
     static const char *shape_env = getenv("JQ_Q4K_GEMM_I8_SHAPE");  // "waves,groups": one of the shapes below
     static const size_t min_tiles = min_tiles_env ? (size_t)atoll(min_tiles_env) : 160;
-    if ((mode && mode[0] == '0') || m < 17 || k % 256 != 0 || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 ||
+    if ((mode && mode[0] == '0') || m < 17 || k % 256 != 0 || row_bytes % ALIGN != 0 || ((uintptr_t)W & (ALIGN - 1)) != 0 ||
         ((uintptr_t)X & 15) != 0 || m > 0x7FFFFFF0ull || n > 0x7FFFFFF0ull)
         return -1;
     // Two workgroup shapes: 256 x 112 outputs (eight waves, one workgroup a compute unit) and 128 x 64 (four
@@ -702,7 +704,7 @@ int dispatch_q4k_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, flo
     hipError_t attr_rc = hipSuccess;
 #define JQ_GEMM_I8(NW_, NG_)                                                                                          \
     if (best->nw == NW_ && best->ng == NG_) {                                                                         \
-        auto kern = jq::q4k_gemm_i8<NW_, NG_>;                                                                        \
+        auto kern = jq::kq_gemm_i8<F, NW_, NG_>;                                                                       \
         constexpr int lds = jq::qi_lds_bytes<NG_>();                                                                  \
         static std::once_flag big_lds;                                                                                \
         static hipError_t rc_once = hipSuccess;                                                                       \
@@ -721,7 +723,7 @@ int dispatch_q4k_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, flo
     JQ_GEMM_I8(4, 4)
 #undef JQ_GEMM_I8
     if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
-    note_kernel("q4k_gemm_i8");
+    note_kernel(name);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -857,7 +859,11 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         return dispatch_q4k_gemm(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k, n)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M) {
-        const int rc = dispatch_q4k_gemm_i8(W, row_bytes, X, Y, m, k, n, s);
+        const int rc = dispatch_gemm_i8<jq::QiQ4K>(W, row_bytes, X, Y, m, k, n, s, "q4k_gemm_i8");
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q6_K && m > Q4K_MFMA_MAX_M) {
+        const int rc = dispatch_gemm_i8<jq::QiQ6K>(W, row_bytes, X, Y, m, k, n, s, "q6k_gemm_i8");
         if (rc >= 0) return rc;
     }
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&

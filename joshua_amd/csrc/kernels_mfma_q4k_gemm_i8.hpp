@@ -1,4 +1,5 @@
-// Q4_K matmul for many activation rows on the int8 matrix cores.
+// Q4_K and Q6_K matmul for many activation rows on the int8 matrix cores.  The arithmetic is written out
+// for Q4_K; Q6_K (w = d sc (q - 32), signed 8-bit sc, no min term) takes the same path with p = sc (q - 32).
 //
 // Per 256-element super-block B of weight row n and activation row m (reference arithmetic
 // w = d sc q - dmin m, src/kquant_dot.rs:440-465):
@@ -116,25 +117,120 @@ constexpr int QI_TILE = 4 * 2 * 64 * 16, QI_META = 48;
 template <int NG>
 constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * QI_META); }
 
-struct QiRaw {  // one unit: the header of a weight row's block and the 32 bytes of one chunk
-    uint4 hdr, q0, q1;
+typedef short qi_s2 __attribute__((ext_vector_type(2)));
+
+// A format's side of the GEMM.  A thread's unit is (weight row, 64-k chunk uc) of a super-block at `blk`:
+// fetch() takes its bytes in three parts (0: the scales, into `next`, 1, 2: the halves of the chunk's
+// packed bytes), take() makes the scales fetched ahead current, piece(j) turns the bytes of elements
+// 16 g + 4 (j % 4) .. + 3 of slices g = j / 4 and 2 + j / 4 into operand words (p + 128 = 256 Ph + L,
+// Pl = L - 128; slice g of the chunk at tile + 256 g, plane Pl 1024 bytes further), meta() writes the
+// row's 48 bytes.
+struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 0..945
+    static constexpr int BLOCK = 144;
+    static constexpr bool HAS_MIN = true;
+    struct Hdr {
+        uint4 h;
+    };
+    struct Raw {
+        Hdr hdr;
+        uint4 q0, q1;
+    };
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        if (part == 0) next.h = *(const uint4 *)blk;
+        if (part == 1) raw.q0 = *(const uint4 *)(blk + 16 + 32 * uc);
+        if (part == 2) raw.q1 = *(const uint4 *)(blk + 32 + 32 * uc);
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) { raw.hdr = next; }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+        const uint4 hdr = raw.hdr.h;
+        const uint32_t scl = hdr.y & 0x3F3F3F3Fu, sch = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+        const uint32_t s4 = (uc < 2 ? scl : sch) >> (16 * (uc & 1));
+        const uint32_t sc[2] = {s4 & 0xFFu, (s4 >> 8) & 0xFFu};
+        const uint4 qv = j < 4 ? raw.q0 : raw.q1;
+        const uint32_t word = (j & 3) == 0 ? qv.x : (j & 3) == 1 ? qv.y : (j & 3) == 2 ? qv.z : qv.w;
+#pragma unroll
+        for (int nib = 0; nib < 2; nib++) {  // low nibbles: sub-block 2 uc, high nibbles: sub-block 2 uc + 1
+            // two elements an instruction (v_mad_u32_u24): elements 0, 2 of the word in `even`, 1, 3 in `odd`
+            const uint32_t w = nib ? word >> 4 : word;
+            const uint32_t even = __umul24(w & 0x000F000Fu, sc[nib]) + 0x00800080u;
+            const uint32_t odd = __umul24((w >> 8) & 0x000F000Fu, sc[nib]) + 0x00800080u;
+            const int gg = 2 * nib + (j >> 2);
+            *(uint32_t *)(tile + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {  // the min scales, d and dmin
+        const uint4 hdr = raw.hdr.h;
+        const uint32_t mnl = hdr.z & 0x3F3F3F3Fu, mnh = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+        const uint32_t m4 = (uc < 2 ? mnl : mnh) >> (16 * (uc & 1));
+        const float mn[2] = {(float)(m4 & 0xFFu), (float)((m4 >> 8) & 0xFFu)};
+        const qi_h2 m1 = {(_Float16)mn[0], (_Float16)mn[1]}, m1k = {(_Float16)(1024.0f * mn[0]), (_Float16)(1024.0f * mn[1])};
+        *(uint32_t *)(meta + 4 * uc) = __builtin_bit_cast(uint32_t, m1);
+        *(uint32_t *)(meta + 16 + 4 * uc) = __builtin_bit_cast(uint32_t, m1k);
+        *(float2 *)(meta + 32) = float2{f16_bits(hdr.x), f16_bits(hdr.x >> 16)};  // the same from all four
+    }
 };
 
-// The products p = sc q of the four bytes of `word` (nibble `hi`), plus 128, as halfwords: elements 0, 2 in
-// `even`, 1, 3 in `odd`.
-__device__ __forceinline__ void qi_products(uint32_t word, bool hi, uint32_t sc, uint32_t &even, uint32_t &odd) {
-    const uint32_t w = hi ? word >> 4 : word;
-    even = __umul24(w & 0x000F000Fu, sc) + 0x00800080u;  // one v_mad_u32_u24
-    odd = __umul24((w >> 8) & 0x000F000Fu, sc) + 0x00800080u;
-}
+// Q6_K: ql[128] | qh[64] | scales[16] i8 | d, w = d sc (q - 32) with q in 0..63 (layout:
+// vendor/candle-metal-kernels/src/metal_src/quantized.metal:198-203, 6673-6694): p = sc (q - 32) in
+// -4096..3968, Ph in -16..15, no min term.  Chunk uc = 2 h + jj of the super-block is elements
+// 128 h + 64 jj + e: e < 32 from ql[64 h + e] and qh[32 h + e] >> 4 jj, e >= 32 from ql[64 h + e] and
+// qh[32 h + e - 32] >> (4 jj + 2), nibble jj of ql, scales[8 h + 4 jj + e / 16].  Blocks of 210 bytes sit at
+// even addresses only: everything is read through aligned words.
+struct QiQ6K {
+    static constexpr int BLOCK = 210;
+    static constexpr bool HAS_MIN = false;
+    struct Hdr {
+        uint32_t sc4, d;
+    };
+    struct Raw {
+        Hdr hdr;
+        uint4 la[2], lb[2], hv[2];  // halves of ql[64 h ..+31], ql[64 h + 32 ..+31], qh[32 h ..+31]
+    };
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        const int h = uc >> 1;
+        if (part == 0) next.sc4 = ldw<uint32_t>(blk + 192 + 4 * uc), next.d = ld<uint16_t>(blk + 208);
+        if (part == 1 || part == 2) {
+            const int o = 16 * (part - 1);
+            raw.la[part - 1] = ldw<uint4>(blk + 64 * h + o);
+            raw.lb[part - 1] = ldw<uint4>(blk + 64 * h + 32 + o);
+            raw.hv[part - 1] = ldw<uint4>(blk + 128 + 32 * h + o);
+        }
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) { raw.hdr = next; }
+    __device__ __forceinline__ static uint32_t word_of(const uint4 &v, int i) {
+        return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
+    }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+        const int sh = 4 * (uc & 1), half = j >> 2, wi = j & 3;
+        const uint32_t qh = word_of(raw.hv[half], wi) >> sh;
+        const uint32_t lo[2] = {word_of(raw.la[half], wi) >> sh, word_of(raw.lb[half], wi) >> sh};
+#pragma unroll
+        for (int e32 = 0; e32 < 2; e32++) {  // elements 16 half + 4 wi .. of the first and second 32 of the chunk
+            const uint32_t q = (lo[e32] & 0x0F0F0F0Fu) | (((qh >> (2 * e32)) & 0x03030303u) << 4);
+            const int gg = 2 * e32 + half;
+            const short sc = (short)(int8_t)(raw.hdr.sc4 >> (8 * gg));
+            const short bias = (short)(128 - 32 * sc);
+            // two elements an instruction (v_pk_mad_i16): sc q + 128 - 32 sc in -3968..4096 as signed halfwords
+            const qi_s2 even = __builtin_bit_cast(qi_s2, q & 0x00FF00FFu) * qi_s2{sc, sc} + qi_s2{bias, bias};
+            const qi_s2 odd = __builtin_bit_cast(qi_s2, (q >> 8) & 0x00FF00FFu) * qi_s2{sc, sc} + qi_s2{bias, bias};
+            const uint32_t ev = __builtin_bit_cast(uint32_t, even), od = __builtin_bit_cast(uint32_t, odd);
+            *(uint32_t *)(tile + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(od, ev, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(od, ev, 0x06020400u) ^ 0x80808080u;
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        *(float2 *)(meta + 32) = float2{f16_bits(raw.hdr.d), 0.0f};  // the same from all four
+    }
+};
 
 // grid: 1-D; workgroup L takes tile (x, y) of tx x ty (weight-row tiles x activation-row tiles).  When ty
 // divides 8 the eight XCDs (L % 8) each work on one activation-row tile, whose operands then stay in that
 // XCD's L2; the grid is padded to a multiple of 8 and workgroups past the last tile leave at once.
-template <int NW, int NG>
-__global__ __launch_bounds__(64 * NW) void q4k_gemm_i8(const uint8_t *__restrict__ W, size_t row_bytes,
-                                                       const uint8_t *__restrict__ acts, float *__restrict__ Y,
-                                                       int m_rows, int n, int nb, int groups, int tx, int ty) {
+template <class F, int NW, int NG>
+__global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict__ W, size_t row_bytes,
+                                                      const uint8_t *__restrict__ acts, float *__restrict__ Y,
+                                                      int m_rows, int n, int nb, int groups, int tx, int ty) {
     constexpr int NT = 16 * NG, THREADS = 64 * NW, UNITS = 4 * NT, PER = (UNITS + THREADS - 1) / THREADS;
     constexpr int BUF = NG * QI_TILE + NT * QI_META;
     extern __shared__ __attribute__((aligned(16))) uint8_t qi_lds[];
@@ -163,58 +259,30 @@ __global__ __launch_bounds__(64 * NW) void q4k_gemm_i8(const uint8_t *__restrict
         const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);
         wsrc[p] = W + (size_t)min(n0 + row, n - 1) * row_bytes;
     }
-    QiRaw raw[PER];
-    uint4 hdr_next[PER];
-    auto fetch_part = [&](int b, int part) __attribute__((always_inline)) {  // 0: header into hdr_next, 1, 2: the two halves of the chunk
+    typename F::Raw raw[PER];
+    typename F::Hdr hdr_next[PER];
+    auto fetch_part = [&](int b, int part) __attribute__((always_inline)) {  // 0: scales into hdr_next, 1, 2: the two halves of the chunk
 #pragma unroll
-        for (int p = 0; p < PER; p++) {
-            const uint8_t *src = wsrc[p] + (size_t)b * 144;
-            if (part == 0) hdr_next[p] = *(const uint4 *)src;
-            if (part == 1) raw[p].q0 = *(const uint4 *)(src + 16 + 32 * uc);
-            if (part == 2) raw[p].q1 = *(const uint4 *)(src + 32 + 32 * uc);
-        }
+        for (int p = 0; p < PER; p++) F::fetch(wsrc[p] + (size_t)b * F::BLOCK, uc, part, raw[p], hdr_next[p]);
     };
-    // Piece j of 8: the four bytes j of this thread's chunk become two operand words of either plane (low
-    // nibbles: sub-block 2 uc, high nibbles: sub-block 2 uc + 1).
+    // Piece j of 8: an eighth of this thread's chunk becomes two operand words of either plane.
     auto unpack_piece = [&](uint8_t *buf, int j) __attribute__((always_inline)) {
 #pragma unroll
         for (int p = 0; p < PER; p++) {
             const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);  // threads past the last unit repeat it
-            const uint4 hdr = raw[p].hdr;
-            const uint32_t scl = hdr.y & 0x3F3F3F3Fu, sch = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
-            const uint32_t s4 = (uc < 2 ? scl : sch) >> (16 * (uc & 1));
-            const uint32_t sc[2] = {s4 & 0xFFu, (s4 >> 8) & 0xFFu};
-            uint8_t *tile = buf + (row >> 4) * QI_TILE + uc * 2048 + (row & 15) * 16;
-            const uint4 qv = j < 4 ? raw[p].q0 : raw[p].q1;
-            const uint32_t word = (j & 3) == 0 ? qv.x : (j & 3) == 1 ? qv.y : (j & 3) == 2 ? qv.z : qv.w;
-#pragma unroll
-            for (int nib = 0; nib < 2; nib++) {
-                uint32_t even, odd;
-                qi_products(word, nib != 0, sc[nib], even, odd);
-                const int gg = 2 * nib + (j >> 2);
-                *(uint32_t *)(tile + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
-                *(uint32_t *)(tile + 1024 + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
-            }
+            F::piece(raw[p], uc, j, buf + (row >> 4) * QI_TILE + uc * 2048 + (row & 15) * 16);
         }
     };
     auto unpack_meta = [&](uint8_t *buf) __attribute__((always_inline)) {  // the row's scales of the min term, d and dmin
 #pragma unroll
         for (int p = 0; p < PER; p++) {
             const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);
-            const uint4 hdr = raw[p].hdr;
-            const uint32_t mnl = hdr.z & 0x3F3F3F3Fu, mnh = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
-            const uint32_t m4 = (uc < 2 ? mnl : mnh) >> (16 * (uc & 1));
-            const float mn[2] = {(float)(m4 & 0xFFu), (float)((m4 >> 8) & 0xFFu)};
-            uint8_t *meta = buf + NG * QI_TILE + row * QI_META;
-            const qi_h2 m1 = {(_Float16)mn[0], (_Float16)mn[1]}, m1k = {(_Float16)(1024.0f * mn[0]), (_Float16)(1024.0f * mn[1])};
-            *(uint32_t *)(meta + 4 * uc) = __builtin_bit_cast(uint32_t, m1);
-            *(uint32_t *)(meta + 16 + 4 * uc) = __builtin_bit_cast(uint32_t, m1k);
-            *(float2 *)(meta + 32) = float2{f16_bits(hdr.x), f16_bits(hdr.x >> 16)};  // the same from all four
+            F::meta(raw[p], uc, buf + NG * QI_TILE + row * QI_META);
         }
     };
     auto take_header = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int p = 0; p < PER; p++) raw[p].hdr = hdr_next[p];
+        for (int p = 0; p < PER; p++) F::take(raw[p], hdr_next[p]);
     };
 
     fetch_part(0, 0), fetch_part(0, 1), fetch_part(0, 2);
@@ -263,13 +331,17 @@ __global__ __launch_bounds__(64 * NW) void q4k_gemm_i8(const uint8_t *__restrict
             auto finish = [&](int cg) __attribute__((always_inline)) {  // the 16 x 16 results of weight-row group cg
                 const uint8_t *meta = buf + NG * QI_TILE + (16 * cg + r) * QI_META;
                 const float2 dd = *(const float2 *)(meta + 32);
-                // lane groups 2, 3 meet zeros in the activation operand: any finite halves will do for them
-                const qi_h8 mB = *(const qi_h8 *)(meta + 16 * (g & 1));
-                const qm_f4 I2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(minA, mB, zero_f, 0, 0, 0);
+                qm_f4 I2 = zero_f;
+                if constexpr (F::HAS_MIN) {
+                    // lane groups 2, 3 meet zeros in the activation operand: any finite halves will do for them
+                    const qi_h8 mB = *(const qi_h8 *)(meta + 16 * (g & 1));
+                    I2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(minA, mB, zero_f, 0, 0, 0);
+                }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float I1 = fmaf((float)(HH[cg][i] * 256 + MID[cg][i]), 256.0f, (float)LL[cg][i]);
-                    acc[mg][cg][i] = fmaf(sx[i], dd.x * I1 - dd.y * I2[i], acc[mg][cg][i]);
+                    if constexpr (F::HAS_MIN) acc[mg][cg][i] = fmaf(sx[i], dd.x * I1 - dd.y * I2[i], acc[mg][cg][i]);
+                    else acc[mg][cg][i] = fmaf(sx[i], dd.x * I1, acc[mg][cg][i]);
                 }
             };
 #pragma unroll

@@ -198,19 +198,21 @@ def test_q6k_one_row_over_4096_wide_row_groups(k, n):
     assert close(got, oracle.matmul_t(capi.Q6_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
 
 
-def test_q6k_dot4_integer_dot_products_are_bit_exact():
-    """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
-    scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
-    n, k = 4096 + 3, 4096
-    rng = np.random.default_rng(5)
+def q6k_integer_case(n, k, seed, nonzero=24, random_scales=False, small=3000):
+    """Q6_K blocks with d = 1 and `nonzero` weights q - 32 in -32..31 a row (times the 16-element group's
+    scale: 1, or any int8 value), and integer activations whose 32-element blocks peak at 32639 (activation
+    scale exactly 1 per 32 and per 256 elements) where the weights are zero.  Returns (blocks, integer
+    weights, activations)."""
+    rng = np.random.default_rng(seed)
     q = np.zeros((n, k), np.int64)
     for r in range(n):
-        idx = rng.choice(k, size=24, replace=False)
-        q[r, idx] = rng.integers(-32, 32, size=24)
-    x = rng.integers(-3000, 3001, size=k).astype(np.int64)
+        idx = rng.choice(k, size=nonzero, replace=False)
+        q[r, idx] = rng.integers(-32, 32, size=nonzero)
+    x = rng.integers(-small, small + 1, size=k).astype(np.int64)
     peak = np.arange(0, k, 32) + int(rng.integers(0, 32))
     x[peak] = 32639 * rng.choice([-1, 1], size=k // 32)
     q[:, peak] = 0
+    sc = rng.integers(-128, 128, size=(n, k // 16)) if random_scales else np.ones((n, k // 16), np.int64)
     qq = (q + 32).reshape(n, k // 256, 2, 4, 32)                   # [half][quarter][l]
     ql = np.zeros((n, k // 256, 2, 64), np.uint8)
     ql[..., :32] = (qq[:, :, :, 0, :] & 15) | ((qq[:, :, :, 2, :] & 15) << 4)
@@ -220,10 +222,19 @@ def test_q6k_dot4_integer_dot_products_are_bit_exact():
     blocks = np.zeros((n, k // 256, 210), np.uint8)
     blocks[:, :, 0:128] = ql.reshape(n, k // 256, 128)
     blocks[:, :, 128:192] = qh.reshape(n, k // 256, 64)
-    blocks[:, :, 192:208] = 1
+    blocks[:, :, 192:208] = sc.reshape(n, k // 256, 16).astype(np.int8).view(np.uint8)
     blocks[:, :, 208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
     blocks = blocks.reshape(-1)
-    assert np.array_equal(oracle.dequantize(capi.Q6_K, blocks).reshape(n, k), q.astype(np.float32))
+    w = q * sc.repeat(16, axis=1)
+    assert np.array_equal(oracle.dequantize(capi.Q6_K, blocks).reshape(n, k), w.astype(np.float32))
+    return blocks, w, x
+
+
+def test_q6k_dot4_integer_dot_products_are_bit_exact():
+    """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
+    scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
+    n, k = 4096 + 3, 4096
+    blocks, q, x = q6k_integer_case(n, k, 5)
     want = x @ q.T
     assert np.abs(want).max() < 2 ** 24
     got = capi.Weight.upload(capi.Q6_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
@@ -776,6 +787,7 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q6_K, 1, 12288, 4096, "q6k_gemv_dot4_lds"),
     (capi.Q6_K, 1, 1024, 4096, "matmul_rows_staged"),
     (capi.Q6_K, 64, 4096, 1024, "gemm_decoded_mfma+splitk"),
+    (capi.Q6_K, 512, 12288, 4096, "q6k_gemm_i8"),           # a feed-forward down projection in prefill
     (capi.Q2_K, 1, 7680, 2048, "matmul_rows_staged"),
     (capi.Q2_K, 1, 4096, 14336, "q2k_gemv_mfma_lds"),
     (capi.MXFP4, 1, 7168, 2048, "matmul_rows_staged"),
@@ -844,46 +856,51 @@ def test_q2k_mfma_gemv_non_finite_activations():
         assert np.all(np.isnan(w.matmul_t(1, lhs)))
 
 
-# ---- Q4_K with many activation rows on the int8 matrix cores ----
+# ---- Q4_K and Q6_K with many activation rows on the int8 matrix cores ----
 
 GEMM_I8_CHILD = r"""
 import sys, numpy as np
 sys.path.insert(0, %r)
 import oracle
 from joshua_amd import capi, synth
-from tests.test_gpu_matmul import q4k_integer_case, close
+from tests.test_gpu_matmul import q4k_integer_case, q6k_integer_case, close
+FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8")}[sys.argv[1]]
 # one to three tiles in either direction, ragged row and column counts
 for (m, k, n) in [(17, 256, 64), (33, 512, 100), (64, 1024, 300), (100, 1024, 257), (130, 1024, 70), (200, 768, 1000),
                   (257, 512, 113), (300, 4096, 450), (512, 2048, 2048)]:
-    blocks = synth.normal_quantized(capi.Q4_K, 5 + n, n * k, 0.02)
+    blocks = synth.normal_quantized(FMT, 5 + n, n * k, 0.02)
     lhs = synth.normal(6 + k, (m, k))
-    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs)
-    assert capi.last_kernel() == "q4k_gemm_i8", (capi.last_kernel(), m, k, n)
-    assert close(got, oracle.matmul_t(capi.Q4_K, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())), (m, k, n)
+    got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(m, lhs)
+    assert capi.last_kernel() == KERNEL, (capi.last_kernel(), m, k, n)
+    assert close(got, oracle.matmul_t(FMT, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())), (m, k, n)
 # exact integers: activation range 32639 per 32-element sub-block
 n, k, m = 160, 2048, 40
-blocks, q, x = q4k_integer_case(n, k, 23, group=32, big_value=32639, small=4000)
+if FMT == capi.Q4_K:
+    blocks, q, x = q4k_integer_case(n, k, 23, group=32, big_value=32639, small=4000)
+else:  # every int8 scale value times q - 32, eight weights a row: sums below 2^24
+    blocks, q, x = q6k_integer_case(n, k, 23, nonzero=8, random_scales=True, small=400)
 lhs = np.stack([np.roll(x, 32 * i) for i in range(m)])
-got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(m, lhs.astype(np.float32))
-assert capi.last_kernel() == "q4k_gemm_i8"
+assert np.abs(lhs @ q.T).max() < 2 ** 24
+got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(m, lhs.astype(np.float32))
+assert capi.last_kernel() == KERNEL
 assert np.array_equal(got, (lhs @ q.T).astype(np.float32)), "integer case"
 # a row whose 16-element groups span twelve orders of magnitude, a row with a single non-zero element, a
 # row with an empty stretch.  One 16-bit scale per 256 activations resolves each super-block relative to its
 # largest magnitude: the wide row is held to 2^-12 of the sum of its terms' magnitudes on every output, and to
 # the usual bound where the terms do not cancel below a twentieth of that sum.
 n, k = 64, 4096
-blocks = synth.normal_quantized(capi.Q4_K, 77, n * k, 0.02)
+blocks = synth.normal_quantized(FMT, 77, n * k, 0.02)
 rng = np.random.default_rng(5)
 lhs = synth.normal(78, (40, k))
 lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 16)).repeat(16).astype(np.float32)
 lhs[1, :] = 0.0
 lhs[1, 1234] = 3.5
 lhs[2, 512:1024] = 0.0
-got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(40, lhs)
-assert capi.last_kernel() == "q4k_gemm_i8"
-want = oracle.matmul_t(capi.Q4_K, (40, k, n), lhs, blocks, avx2=oracle.have_avx2())
+got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(40, lhs)
+assert capi.last_kernel() == KERNEL
+want = oracle.matmul_t(FMT, (40, k, n), lhs, blocks, avx2=oracle.have_avx2())
 assert close(got[1:], want[1:]), "rows of ordinary range"
-wd = oracle.dequantize(capi.Q4_K, blocks).reshape(n, k).astype(np.float64)
+wd = oracle.dequantize(FMT, blocks).reshape(n, k).astype(np.float64)
 x0 = lhs[0].astype(np.float64)
 w0, mag = wd @ x0, np.abs(wd) @ np.abs(x0)
 err = np.abs(got[0] - w0)
@@ -895,8 +912,8 @@ assert big.sum() > n // 4 and np.all(err[big] <= 1e-3 * np.abs(w0[big])), "wide 
 lhs = synth.normal(79, (20, k))
 lhs[3, 100] = np.inf
 lhs[7, 4000] = np.nan
-got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(20, lhs)
-want = oracle.matmul_t(capi.Q4_K, (20, k, n), lhs, blocks, avx2=oracle.have_avx2())
+got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(20, lhs)
+want = oracle.matmul_t(FMT, (20, k, n), lhs, blocks, avx2=oracle.have_avx2())
 assert np.all(np.isnan(got[3])) and np.all(np.isnan(got[7]))
 ok = np.ones(20, bool); ok[[3, 7]] = False
 assert close(got[ok], want[ok])
@@ -904,8 +921,9 @@ print("gemm i8 ok")
 """
 
 
+@pytest.mark.parametrize("fmt", ["q4k", "q6k"])
 @pytest.mark.parametrize("shape", ["8,7", "4,4"])
-def test_q4k_int8_gemm_small_shapes_in_a_child_process(shape):
+def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves a product only from about 160 tiles on; with the threshold lowered and the workgroup
     shape forced through the environment (read when the library first dispatches, hence the child process) both
     shapes run on small products: parity, ragged edges, exact integer sums, wide-range and non-finite
@@ -914,7 +932,7 @@ def test_q4k_int8_gemm_small_shapes_in_a_child_process(shape):
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     env = dict(os.environ, JQ_Q4K_GEMM_I8_MIN_TILES="1", JQ_Q4K_GEMM_I8_SHAPE=shape)
-    res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1)], env=env, capture_output=True, text=True, timeout=170)
+    res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1), fmt], env=env, capture_output=True, text=True, timeout=170)
     assert res.returncode == 0 and "gemm i8 ok" in res.stdout, res.stdout + res.stderr
 
 
