@@ -106,6 +106,16 @@ const void *jq_device_ptr(const jq_weight *w);
 int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, float *dst,
                 size_t dst_len, int ptrs_are_device, void *stream);
 
+/* The same product over f16 activations into f16 results, elements as IEEE binary16 bit
+ * patterns: lhs is widened to f32, multiplied as jq_matmul_t does, and the f32 result is
+ * rounded to f16 (nearest even, overflow to infinity) (reference:
+ * src/mmap_tensor.rs:136-138, :378-380, :451-453 matmul_t_f16; the wrappers
+ * src/mxfp4.rs:242-258, src/iq2xxs.rs:396-412).  Same validation and empty case.  The
+ * f32 operands live in stream-ordered allocations, freed in stream order: the call
+ * cannot be captured into a HIP graph. */
+int jq_matmul_t_f16(const jq_weight *w, size_t m, const uint16_t *lhs, size_t lhs_len, uint16_t *dst,
+                    size_t dst_len, int ptrs_are_device, void *stream);
+
 /* jq_matmul_t for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
  * in the reference.  Same product, same kernels, device pointers only; what jq_matmul_t

@@ -26,7 +26,7 @@ TYPE_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ2_XXS: "
 # Every symbol include/joshua_hip.h declares.
 EXPORTS = (
     "jq_last_error", "jq_last_kernel", "jq_block_geometry", "jq_init", "jq_upload", "jq_view", "jq_free", "jq_dtype", "jq_rows",
-    "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_matmul_t_noalloc", "jq_try_matmul_fused", "jq_dequantize", "jq_decode_raw_to_f32", "jq_stream_release",
+    "jq_cols", "jq_storage_size_in_bytes", "jq_device_ptr", "jq_matmul_t", "jq_matmul_t_f16", "jq_matmul_t_noalloc", "jq_try_matmul_fused", "jq_dequantize", "jq_decode_raw_to_f32", "jq_stream_release",
     "jq_embedding", "jq_stream_synchronize", "jq_moe_create", "jq_moe_free", "jq_moe_route", "jq_moe_forward",
     "jq_mla_create", "jq_mla_free", "jq_mla_forward", "jq_mla_reset", "jq_mla_cached_tokens",
     "jq_qwen3_create", "jq_qwen3_free", "jq_qwen3_set_tensor", "jq_qwen3_forward", "jq_qwen3_greedy", "jq_qwen3_reset",
@@ -102,6 +102,7 @@ def lib() -> ctypes.CDLL:
         L.jq_device_ptr.argtypes = [vp]
         L.jq_device_ptr.restype = vp
         L.jq_matmul_t.argtypes = [vp, sz, vp, sz, vp, sz, i32, vp]
+        L.jq_matmul_t_f16.argtypes = [vp, sz, vp, sz, vp, sz, i32, vp]
         L.jq_matmul_t_noalloc.argtypes = [vp, sz, vp, sz, vp, sz, vp]
         L.jq_try_matmul_fused.argtypes = [u32, sz, sz, sz, vp, vp, sz, vp, vp]
         L.jq_dequantize.argtypes = [vp, vp, sz, i32, vp]
@@ -283,6 +284,13 @@ class Weight:
         _check(lib().jq_matmul_t(self._h, m, x.ctypes.data, x.size, dst.ctypes.data, dst.size, 0, None))
         return dst.reshape(m, self.n) if dst.size == m * self.n else dst
 
+    def matmul_t_f16(self, m: int, lhs: np.ndarray) -> np.ndarray:
+        """f16 activations in, f16 results out (reference: src/mmap_tensor.rs:136-138 matmul_t_f16)."""
+        x = np.ascontiguousarray(np.asarray(lhs, dtype=np.float16).reshape(-1))
+        dst = np.empty(m * self.n, dtype=np.float16)
+        _check(lib().jq_matmul_t_f16(self._h, m, x.ctypes.data, x.size, dst.ctypes.data, dst.size, 0, None))
+        return dst.reshape(m, self.n)
+
     def dequantize(self) -> np.ndarray:
         out = np.empty(self.n * self.k, dtype=np.float32)
         _check(lib().jq_dequantize(self._h, out.ctypes.data, out.size, 0, None))
@@ -297,6 +305,9 @@ class Weight:
     # -- device-pointer calls (raw addresses; inputs already in HBM) -------------
     def matmul_t_dev(self, m: int, lhs_ptr: int, lhs_len: int, dst_ptr: int, dst_len: int, stream: int = 0) -> None:
         _check(lib().jq_matmul_t(self._h, m, lhs_ptr, lhs_len, dst_ptr, dst_len, 1, stream or None))
+
+    def matmul_t_f16_dev(self, m: int, lhs_ptr: int, lhs_len: int, dst_ptr: int, dst_len: int, stream: int = 0) -> None:
+        _check(lib().jq_matmul_t_f16(self._h, m, lhs_ptr, lhs_len, dst_ptr, dst_len, 1, stream or None))
 
     def matmul_t_noalloc(self, m: int, lhs_ptr: int, lhs_len: int, dst_ptr: int, dst_len: int, stream: int = 0) -> None:
         """The same product through the entry point that allocates no device memory."""

@@ -1021,6 +1021,46 @@ int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, 
     return 0;
 }
 
+int jq_matmul_t_f16(const jq_weight *w, size_t m, const uint16_t *lhs, size_t lhs_len, uint16_t *dst, size_t dst_len,
+                    int ptrs_are_device, void *stream) {
+    if (!w) return fail("jq_matmul_t_f16: weight is null");
+    if (validate(w->type, m, w->k, w->n, lhs_len, w->nbytes, dst_len)) return 1;
+    if (m == 0 || w->n == 0) return 0;
+    if (!lhs || !dst) return fail("jq_matmul_t_f16: lhs/dst is null");
+    hipStream_t s = (hipStream_t)stream;
+    // f16 -> f32, the f32 product, f32 -> f16 (reference: src/mxfp4.rs:242-258, src/iq2xxs.rs:396-412): the
+    // f32 operands live in stream-ordered allocations, so device callers are not synchronised
+    void *x32 = nullptr, *y32 = nullptr, *h16 = nullptr;
+    const size_t h16_bytes = ptrs_are_device ? 0 : std::max(lhs_len, dst_len) * sizeof(uint16_t);
+    auto release = [&] {
+        if (x32) (void)hipFreeAsync(x32, s);
+        if (y32) (void)hipFreeAsync(y32, s);
+        if (h16) (void)hipFreeAsync(h16, s);
+    };
+    hipError_t e = hipMallocAsync(&x32, lhs_len * sizeof(float), s);
+    if (e == hipSuccess) e = hipMallocAsync(&y32, dst_len * sizeof(float), s);
+    if (e == hipSuccess && h16_bytes) e = hipMallocAsync(&h16, h16_bytes, s);
+    if (e == hipSuccess && !ptrs_are_device) e = hipMemcpyAsync(h16, lhs, lhs_len * sizeof(uint16_t), hipMemcpyHostToDevice, s);
+    if (e != hipSuccess) {
+        release();
+        return fail("jq_matmul_t_f16: %s", hipGetErrorString(e));
+    }
+    const uint16_t *x16 = ptrs_are_device ? lhs : (const uint16_t *)h16;
+    uint16_t *y16 = ptrs_are_device ? dst : (uint16_t *)h16;
+    auto grid_of = [](size_t elems) { return (unsigned)std::min<size_t>((elems + 255) / 256, 65536); };
+    hipLaunchKernelGGL((jq::decode_plain<1>), dim3(grid_of(lhs_len)), dim3(256), 0, s, (const uint8_t *)x16, (float *)x32, lhs_len);
+    int rc = dispatch_matmul(w->type, w->dev, w->row_bytes, (const float *)x32, (float *)y32, m, w->k, w->n, s);
+    if (rc == 0) {
+        hipLaunchKernelGGL(jq::f32_to_f16, dim3(grid_of(dst_len)), dim3(256), 0, s, (const float *)y32, y16, dst_len);
+        e = hipGetLastError();
+        if (e == hipSuccess && !ptrs_are_device) e = hipMemcpyAsync(dst, h16, dst_len * sizeof(uint16_t), hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess && !ptrs_are_device) e = hipStreamSynchronize(s);
+        if (e != hipSuccess) rc = fail("jq_matmul_t_f16: %s", hipGetErrorString(e));
+    }
+    release();
+    return rc;
+}
+
 int jq_matmul_t_noalloc(const jq_weight *w, size_t m, const float *lhs_dev, size_t lhs_len, float *dst_dev,
                         size_t dst_len, void *stream) {
     if (!w) return fail("jq_matmul_t_noalloc: weight is null");

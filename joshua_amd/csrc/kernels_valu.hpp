@@ -281,4 +281,10 @@ __global__ __launch_bounds__(256) void decode_plain(const uint8_t *__restrict__ 
     }
 }
 
+// f32 -> f16 (round to nearest even, overflow to infinity: half::f16::from_f32), one element a thread.
+__global__ __launch_bounds__(256) void f32_to_f16(const float *__restrict__ in, uint16_t *__restrict__ out, size_t elems) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < elems; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = __builtin_bit_cast(uint16_t, (_Float16)in[i]);
+}
+
 }  // namespace jq

@@ -129,6 +129,16 @@ def matmul_t(qtype: int, mkn, lhs, blocks, *, avx2: bool = False, threads: int =
     return dst.reshape(m, n) if dst.size == m * n else dst
 
 
+def matmul_t_f16(qtype: int, mkn, lhs, blocks, *, avx2: bool = False) -> np.ndarray:
+    """f16 activations in, f16 results out: widen to f32 (exact), the f32 product, round to f16 (nearest even,
+    overflow to infinity), as the reference's wrappers do (src/mxfp4.rs:242-258, src/iq2xxs.rs:396-412;
+    the k-quant types go through candle's matmul_f16, src/mmap_tensor.rs:136-138, whose f16 result is the
+    same rounding of an f32 sum)."""
+    m, k, n = mkn
+    x16 = np.asarray(lhs, dtype=np.float16)
+    return matmul_t(qtype, mkn, x16.astype(np.float32), blocks, avx2=avx2).astype(np.float16)
+
+
 def iq2xxs_matmul_scalar(mkn, lhs, blocks) -> np.ndarray:
     m, k, n = mkn
     x = np.ascontiguousarray(np.asarray(lhs, dtype=np.float32).reshape(-1))
