@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <algorithm>
@@ -654,49 +655,80 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
     return 0;
 }
 
-// Q4_K with many activation rows on the int8 matrix cores: the activations as two int8 planes per
-// 32-element sub-block in the call scratch of the stream, then q4k_gemm_i8 with a workgroup shape chosen for
-// the row count (8 waves as WM x 8 / WM) and NG weight-row groups of 16 a wave chosen so that the tiles
-// fill the 256 compute units as evenly as possible.  Returns -1 when the shape is outside its reach or has
-// too few tiles to occupy the chip (the f16 GEMM splits those over k).  JQ_Q4K_GEMM_I8 = 0 switches it off.
+// Q4_K and Q6_K with many activation rows on the int8 matrix cores: the activations as two int8 planes per
+// 256-element super-block in the call scratch of the stream, then kq_gemm_i8 with the workgroup shape and the
+// split over k that an estimate fitted to measurements prefers.  Returns -1 when the shape is outside its
+// reach or the product is tiny.  JQ_Q4K_GEMM_I8 = 0 switches it off; JQ_Q4K_GEMM_I8_SHAPE and _SPLITS force the
+// choice, _MIN_TILES moves the floor (small tiles times the splits that k allows; default 64), _MIN_M the
+// fewest activation rows (default 64, at least 17).
 struct GemmI8Shape {
     int nw, ng;
 };
 
 template <class F>
 int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
-                     hipStream_t s, const char *name) {
+                     hipStream_t s, const char *name, const char *name_split) {
     constexpr size_t ALIGN = F::BLOCK % 16 == 0 ? 16 : 2;
     static const char *mode = getenv("JQ_Q4K_GEMM_I8");
     static const char *min_tiles_env = getenv("JQ_Q4K_GEMM_I8_MIN_TILES");
     static const char *shape_env = getenv("JQ_Q4K_GEMM_I8_SHAPE");  // "waves,groups": one of the shapes below
-    static const size_t min_tiles = min_tiles_env ? (size_t)atoll(min_tiles_env) : 160;
-    if ((mode && mode[0] == '0') || m < 17 || k % 256 != 0 || row_bytes % ALIGN != 0 || ((uintptr_t)W & (ALIGN - 1)) != 0 ||
+    static const size_t min_tiles = min_tiles_env ? (size_t)atoll(min_tiles_env) : 64;
+    // One activation scale per 256 elements resolves a row relative to its super-blocks' largest magnitudes:
+    // that is the contract from 64 rows on (prefill); fewer rows keep the kernels with a scale per 32.
+    static const char *min_m_env = getenv("JQ_Q4K_GEMM_I8_MIN_M");
+    static const size_t min_m = min_m_env ? std::max<size_t>((size_t)atoll(min_m_env), 17) : 64;
+    if ((mode && mode[0] == '0') || m < min_m || k % 256 != 0 || row_bytes % ALIGN != 0 || ((uintptr_t)W & (ALIGN - 1)) != 0 ||
         ((uintptr_t)X & 15) != 0 || m > 0x7FFFFFF0ull || n > 0x7FFFFFF0ull)
         return -1;
     // Two workgroup shapes: 256 x 112 outputs (eight waves, one workgroup a compute unit) and 128 x 64 (four
-    // waves, two a compute unit).  Measured at k = 4096, in us: the large one 17 + 105 per round of 256 tiles;
-    // the small one 52 up to 256 tiles, 30 + 0.137 a tile beyond.  There is no split over k here, so below
-    // about 160 small tiles the f16 kernel with its split wins (512 x 4096 x 1024: 34 us against 51) and the
-    // call is declined.
+    // waves, two a compute unit), and a split over k (the parts summed by splitk_sum) when the tiles alone leave
+    // compute units idle: every workgroup then walks nb / splits super-blocks.
     static const GemmI8Shape shapes[] = {{8, 7}, {4, 4}};
+    const size_t nb = k / 256, groups = (m + 15) / 16;
     auto tiles_of = [&](const GemmI8Shape &sh) {
         const size_t mt = 32 * (size_t)sh.nw, nt = 16 * (size_t)sh.ng;
         return ((m + mt - 1) / mt) * ((n + nt - 1) / nt);
     };
-    const size_t tiles_large = tiles_of(shapes[0]), tiles_small = tiles_of(shapes[1]);
-    const double t_large = 17.0 + 105.0 * (double)((tiles_large + 255) / 256);
-    const double t_small = tiles_small <= 256 ? 52.0 : 30.0 + 0.137 * (double)tiles_small;
-    const GemmI8Shape *best = t_large < t_small ? &shapes[0] : &shapes[1];
+    if (tiles_of(shapes[1]) * std::max<size_t>(1, std::min<size_t>(nb / 4, 8)) < min_tiles) return -1;
+    // Estimate per (shape, splits), in us, fitted to whole-call times of Q4_K products of 32 to 2048 rows
+    // against 1024 to 24576 weight rows of 4096 and 12288 columns (the picks are within 5 % of the best
+    // measured choice there; Q6_K runs ~10 % longer with the same ordering): the preparation, a fixed part,
+    // the super-blocks a workgroup walks at a cost that grows with the workgroups at work (a large workgroup:
+    // 5.0 us a super-block with 74 at work, 6.6 with 256; a small one: 2.5 with 64, 3.0 with 256, 4.7 when two
+    // share every compute unit), and the sum's launch and its (splits + 1) m n floats, which the last-level
+    // cache holds.
+    const size_t acts_bytes = (groups * nb * (size_t)jq::QI_REC + 255) & ~(size_t)255;
+    const size_t scratch_cap = tl_fixed_scratch ? tl_fixed_scratch->bytes : (size_t)1 << 40;
+    auto estimate = [&](const GemmI8Shape &sh, size_t sp) {
+        const double wgs = (double)(tiles_of(sh) * sp), nbl = (double)(nb / sp);
+        double us = 3.0 + 0.0035 * (double)(nb * groups);
+        if (sh.nw == 8) us += 10.0 + nbl * (4.3 + 0.009 * std::min(wgs, 256.0)) * std::ceil(wgs / 256.0);
+        else if (wgs <= 256.0) us += 3.9 + nbl * (2.3 + 0.0027 * wgs);
+        else us += 3.9 + nbl * (3.1 + 0.0032 * std::min(wgs, 512.0)) * std::max(1.0, wgs / 512.0);
+        if (sp > 1) us += 1.0 + 0.8 * (double)sp + (double)(sp + 1) * (double)(m * n) * 4.0 / 8.0e6;
+        return us;
+    };
+    const GemmI8Shape *best = nullptr;
+    size_t splits = 1;
+    double best_us = 0.0;
+    static const char *splits_env = getenv("JQ_Q4K_GEMM_I8_SPLITS");
     int want_nw = 0, want_ng = 0;
-    if (shape_env && sscanf(shape_env, "%d,%d", &want_nw, &want_ng) == 2)
-        for (const GemmI8Shape &sh : shapes)
-            if (sh.nw == want_nw && sh.ng == want_ng) best = &sh;
-    if (tiles_small < min_tiles) return -1;
-    const size_t nb = k / 256, groups = (m + 15) / 16;
+    const bool forced = shape_env && sscanf(shape_env, "%d,%d", &want_nw, &want_ng) == 2;
+    for (const GemmI8Shape &sh : shapes) {
+        if (forced && (sh.nw != want_nw || sh.ng != want_ng)) continue;
+        for (size_t sp = 1; sp <= 8; sp++) {
+            if (nb % sp != 0 || (sp > 1 && nb / sp < 4)) continue;
+            if (splits_env && sp != (size_t)atoi(splits_env)) continue;
+            if (sp > 1 && (m * n > 0x3FFFFFFFull || acts_bytes + sp * m * n * sizeof(float) > scratch_cap)) continue;
+            const double us = estimate(sh, sp);
+            if (!best || us < best_us) best = &sh, splits = sp, best_us = us;
+        }
+    }
+    if (!best) return -1;
     CallScratch scratch;
     uint8_t *acts = nullptr;
-    if (scratch.get(groups * nb * (size_t)jq::QI_REC, s, &acts)) return 1;
+    if (scratch.get(acts_bytes + (splits > 1 ? splits * m * n * sizeof(float) : 0), s, &acts)) return 1;
+    float *parts = (float *)(acts + acts_bytes);
     const size_t mt = 32 * (size_t)best->nw, nt = 16 * (size_t)best->ng;
     const size_t tx = (n + nt - 1) / nt, ty = (m + mt - 1) / mt;
     const size_t grid = 8 % ty == 0 ? (tx * ty + 7) / 8 * 8 : tx * ty;
@@ -704,7 +736,7 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
     hipError_t attr_rc = hipSuccess;
 #define JQ_GEMM_I8(NW_, NG_)                                                                                          \
     if (best->nw == NW_ && best->ng == NG_) {                                                                         \
-        auto kern = jq::kq_gemm_i8<F, NW_, NG_>;                                                                       \
+        auto kern = jq::kq_gemm_i8<F, NW_, NG_>;                                                                      \
         constexpr int lds = jq::qi_lds_bytes<NG_>();                                                                  \
         static std::once_flag big_lds;                                                                                \
         static hipError_t rc_once = hipSuccess;                                                                       \
@@ -715,15 +747,19 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
         if (attr_rc == hipSuccess) {                                                                                  \
             hipLaunchKernelGGL(jq::q4k_gemm_i8_prep, dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, X, (int)m, \
                                (int)k, acts);                                                                         \
-            hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NW_), lds, s, W, row_bytes, (const uint8_t *)acts, \
-                               Y, (int)m, (int)n, (int)nb, (int)groups, (int)tx, (int)ty);                            \
+            hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)splits), dim3(64 * NW_), lds, s, W, row_bytes,    \
+                               (const uint8_t *)acts, splits > 1 ? parts : Y, (int)m, (int)n, (int)(nb / splits),     \
+                               (int)groups, (int)tx, (int)ty, (int)nb, splits > 1 ? m * n : (size_t)0);               \
+            if (splits > 1)                                                                                           \
+                hipLaunchKernelGGL(jq::splitk_sum, dim3((unsigned)((m * n + 1023) / 1024)), dim3(256), 0, s, parts, Y, \
+                                   m * n, (int)splits);                                                               \
         }                                                                                                             \
     }
     JQ_GEMM_I8(8, 7)
     JQ_GEMM_I8(4, 4)
 #undef JQ_GEMM_I8
     if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
-    note_kernel(name);
+    note_kernel(splits > 1 ? name_split : name);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -859,11 +895,11 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         return dispatch_q4k_gemm(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && q4k_mfma_applies(m, k, n)) return dispatch_q4k_mfma(W, row_bytes, X, Y, m, k, n, s);
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M) {
-        const int rc = dispatch_gemm_i8<jq::QiQ4K>(W, row_bytes, X, Y, m, k, n, s, "q4k_gemm_i8");
+        const int rc = dispatch_gemm_i8<jq::QiQ4K>(W, row_bytes, X, Y, m, k, n, s, "q4k_gemm_i8", "q4k_gemm_i8+splitk");
         if (rc >= 0) return rc;
     }
     if (type == JQ_TYPE_Q6_K && m > Q4K_MFMA_MAX_M) {
-        const int rc = dispatch_gemm_i8<jq::QiQ6K>(W, row_bytes, X, Y, m, k, n, s, "q6k_gemm_i8");
+        const int rc = dispatch_gemm_i8<jq::QiQ6K>(W, row_bytes, X, Y, m, k, n, s, "q6k_gemm_i8", "q6k_gemm_i8+splitk");
         if (rc >= 0) return rc;
     }
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&

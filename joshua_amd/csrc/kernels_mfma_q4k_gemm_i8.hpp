@@ -227,10 +227,12 @@ struct QiQ6K {
 // grid: 1-D; workgroup L takes tile (x, y) of tx x ty (weight-row tiles x activation-row tiles).  When ty
 // divides 8 the eight XCDs (L % 8) each work on one activation-row tile, whose operands then stay in that
 // XCD's L2; the grid is padded to a multiple of 8 and workgroups past the last tile leave at once.
+// gridDim.y > 1 splits the product over k.
 template <class F, int NW, int NG>
 __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict__ W, size_t row_bytes,
                                                       const uint8_t *__restrict__ acts, float *__restrict__ Y,
-                                                      int m_rows, int n, int nb, int groups, int tx, int ty) {
+                                                      int m_rows, int n, int nb, int groups, int tx, int ty,
+                                                      int nb_total, size_t split_stride) {
     constexpr int NT = 16 * NG, THREADS = 64 * NW, UNITS = 4 * NT, PER = (UNITS + THREADS - 1) / THREADS;
     constexpr int BUF = NG * QI_TILE + NT * QI_META;
     extern __shared__ __attribute__((aligned(16))) uint8_t qi_lds[];
@@ -244,12 +246,17 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
     }
     if (bx >= tx || by >= ty) return;
     const int n0 = bx * NT, m0 = by * 32 * NW;
+    // split over k: workgroups blockIdx.y = i take super-blocks i nb .. (i + 1) nb - 1 of the nb_total and store
+    // their sums at Y + i split_stride (splitk_sum adds the parts in a fixed order)
+    const int b_first = (int)blockIdx.y * nb;
+    Y += (size_t)blockIdx.y * split_stride;
 
     // activation operands of this wave: row groups 2 wave, 2 wave + 1 of the tile (clamped: rows past m_rows
     // are computed and not stored)
     const uint8_t *arec[2];
 #pragma unroll
-    for (int mg = 0; mg < 2; mg++) arec[mg] = acts + (size_t)min(m0 / 16 + 2 * wave + mg, groups - 1) * nb * QI_REC;
+    for (int mg = 0; mg < 2; mg++)
+        arec[mg] = acts + ((size_t)min(m0 / 16 + 2 * wave + mg, groups - 1) * nb_total + b_first) * QI_REC;
 
     // unpack units of this thread: chunk c = tid % 4 of weight rows tid / 4 + (THREADS / 4) p
     const int uc = tid & 3;
@@ -257,7 +264,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
 #pragma unroll
     for (int p = 0; p < PER; p++) {
         const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);
-        wsrc[p] = W + (size_t)min(n0 + row, n - 1) * row_bytes;
+        wsrc[p] = W + (size_t)min(n0 + row, n - 1) * row_bytes + (size_t)b_first * F::BLOCK;
     }
     typename F::Raw raw[PER];
     typename F::Hdr hdr_next[PER];

@@ -780,14 +780,16 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 16, 4096, 14336, "q4k_rows16_mfma"),
     (capi.Q4_K, 16, 2048, 768, "q4k_stream_mfma"),
     (capi.Q4_K, 512, 4096, 14336, "q4k_gemm_i8"),           # 256 tiles of 256 x 112
-    (capi.Q4_K, 128, 4096, 14336, "q4k_gemm_i8"),           # 224 tiles of 128 x 64
-    (capi.Q4_K, 128, 4096, 4096, "q4k_gemm_mfma+splitk"),   # 64 tiles: the f16 kernel with its split over k
-    (capi.Q4_K, 512, 4096, 1024, "q4k_gemm_mfma+splitk"),
+    (capi.Q4_K, 128, 4096, 14336, "q4k_gemm_i8+splitk"),    # 224 tiles of 128 x 64, two splits
+    (capi.Q4_K, 128, 4096, 4096, "q4k_gemm_i8+splitk"),     # 64 tiles of 128 x 64: split over k
+    (capi.Q4_K, 512, 4096, 1024, "q4k_gemm_i8+splitk"),
+    (capi.Q4_K, 128, 4096, 256, "q4k_gemm_mfma+splitk"),    # a small product: the f16 kernel
     (capi.Q8_0, 1, 4096, 4096, "q8_0_gemv_dot4_lds"),
     (capi.Q6_K, 1, 12288, 4096, "q6k_gemv_dot4_lds"),
     (capi.Q6_K, 1, 1024, 4096, "matmul_rows_staged"),
-    (capi.Q6_K, 64, 4096, 1024, "gemm_decoded_mfma+splitk"),
-    (capi.Q6_K, 512, 12288, 4096, "q6k_gemm_i8"),           # a feed-forward down projection in prefill
+    (capi.Q6_K, 64, 4096, 1024, "q6k_gemm_i8+splitk"),
+    (capi.Q6_K, 64, 2048, 256, "gemm_decoded_mfma+splitk"), # a small product: weights decoded in the workgroup
+    (capi.Q6_K, 512, 12288, 4096, "q6k_gemm_i8+splitk"),    # a feed-forward down projection in prefill: 74 tiles of 256 x 112, three splits
     (capi.Q2_K, 1, 7680, 2048, "matmul_rows_staged"),
     (capi.Q2_K, 1, 4096, 14336, "q2k_gemv_mfma_lds"),
     (capi.MXFP4, 1, 7168, 2048, "matmul_rows_staged"),
@@ -865,6 +867,18 @@ import oracle
 from joshua_amd import capi, synth
 from tests.test_gpu_matmul import q4k_integer_case, q6k_integer_case, close
 FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8")}[sys.argv[1]]
+# the same products split over k: the parts are summed in a fixed order
+if __import__("os").environ.get("JQ_Q4K_GEMM_I8_SPLITS", "1") != "1":
+    for (m, k, n) in [(40, 4096, 100), (300, 4096, 130), (64, 12288, 70)]:
+        blocks = synth.normal_quantized(FMT, 15 + n, n * k, 0.02)
+        lhs = synth.normal(16 + k, (m, k))
+        w = capi.Weight.upload(FMT, blocks, n, k)
+        got = w.matmul_t(m, lhs)
+        assert capi.last_kernel() == KERNEL + "+splitk", (capi.last_kernel(), m, k, n)
+        assert close(got, oracle.matmul_t(FMT, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())), (m, k, n)
+        assert np.array_equal(got, w.matmul_t(m, lhs))
+    print("gemm i8 ok")
+    sys.exit(0)
 # one to three tiles in either direction, ragged row and column counts
 for (m, k, n) in [(17, 256, 64), (33, 512, 100), (64, 1024, 300), (100, 1024, 257), (130, 1024, 70), (200, 768, 1000),
                   (257, 512, 113), (300, 4096, 450), (512, 2048, 2048)]:
@@ -931,9 +945,14 @@ def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     import subprocess
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, JQ_Q4K_GEMM_I8_MIN_TILES="1", JQ_Q4K_GEMM_I8_SHAPE=shape)
+    env = dict(os.environ, JQ_Q4K_GEMM_I8_MIN_TILES="1", JQ_Q4K_GEMM_I8_MIN_M="17", JQ_Q4K_GEMM_I8_SHAPE=shape, JQ_Q4K_GEMM_I8_SPLITS="1")
     res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1), fmt], env=env, capture_output=True, text=True, timeout=170)
     assert res.returncode == 0 and "gemm i8 ok" in res.stdout, res.stdout + res.stderr
+    # forced splits of 2 and 4 (k of 4096 and 12288: 16 and 48 super-blocks)
+    for splits in ("2", "4"):
+        env["JQ_Q4K_GEMM_I8_SPLITS"] = splits
+        res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1), fmt], env=env, capture_output=True, text=True, timeout=170)
+        assert res.returncode == 0 and "gemm i8 ok" in res.stdout, splits + res.stdout + res.stderr
 
 
 def test_graph_captured_before_the_stream_scratch_grows_still_replays():
