@@ -2188,7 +2188,7 @@ int model_reserve(jq_model *m, size_t T) {
     HIP_TRY(hipMalloc((void **)&m->x, T * c.hidden * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->x2, c.hidden * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->hn, T * c.hidden * sizeof(float)));
-    HIP_TRY(hipMalloc((void **)&m->qb, T * qd * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&m->qb, T * (qd + 2 * kd) * sizeof(float)));  // q, or the rows of one q|k|v product
     HIP_TRY(hipMalloc((void **)&m->kb, T * kd * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->vb, T * kd * sizeof(float)));
     HIP_TRY(hipMalloc((void **)&m->att, T * qd * sizeof(float)));
@@ -2349,7 +2349,11 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             model_vec(m, p + ".attn_q_norm.weight", &w_qn) || model_vec(m, p + ".attn_k_norm.weight", &w_kn))
             return 1;
         float *qp = m->qb, *kp = m->kb, *vp = m->vb;
+        int q_stride = (int)(nh * d), k_stride = (int)(nkv * d), v_stride = (int)(nkv * d);  // floats from a token to the next
         auto fq = T == 1 ? m->fused.find(p + ".qkv") : m->fused.end();
+        static const char *no_fused_prefill = getenv("JQ_NO_FUSED_QKV_PREFILL");
+        // (the split attention kernel of steps up to 8 tokens reads q, k and v of a token as rows of their own)
+        auto fqm = T > 1 && !split && !no_fused_prefill ? m->fused.find(p + ".qkv") : m->fused.end();
         const bool v_fused = fq != m->fused.end() && fq->second->n == (size_t)(nh + 2 * nkv) * d;
         // single token: residual add, norm and q|k(|v) as one launch when the kernel has that form
         const bool normed = fq != m->fused.end() &&
@@ -2361,6 +2365,14 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             if (!normed && dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->cat, 1, w->k, w->n, s)) return 1;
             qp = m->cat, kp = m->cat + (size_t)nh * d;
             if (v_fused) vp = kp + (size_t)nkv * d;
+            else if (model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s)) return 1;
+        } else if (fqm != m->fused.end()) {
+            // several tokens: q|k(|v) as one product, whose rows hold a token's q, k (and v) heads side by side
+            const jq_weight *w = fqm->second;
+            if (dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->qb, T, w->k, w->n, s)) return 1;
+            q_stride = k_stride = (int)w->n;
+            kp = m->qb + (size_t)nh * d;
+            if (w->n == (size_t)(nh + 2 * nkv) * d) vp = kp + (size_t)nkv * d, v_stride = (int)w->n;
             else if (model_mm(m, p + ".attn_v.weight", m->hn, m->vb, T, s)) return 1;
         } else if (model_mm(m, p + ".attn_q.weight", m->hn, m->qb, T, s) ||
                    model_mm(m, p + ".attn_k.weight", m->hn, m->kb, T, s) ||
@@ -2381,18 +2393,19 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
                                n_chunks);
         } else {
             hipLaunchKernelGGL(jq::qkv_norm_rope_cache, dim3(T * (nh + 2 * nkv)), dim3(64), 0, s, qp, kp, vp, w_qn, w_kn,
-                               c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx);
+                               c.rms_eps, nh, nkv, d, m->pos, c.rope_theta, m->kc[l], m->vc[l], (int)c.n_ctx, q_stride,
+                               k_stride, v_stride);
             // head dimension 128 and 1, 2, 4 or 8 query heads a KV head: tiles of 16 tokens on the f32 matrix cores
             static const char *no_tiles = getenv("JQ_NO_ATTENTION_TILES");
             const int gq = nh / nkv;
             const dim3 tgrid((unsigned)((T + 15) / 16), (unsigned)nkv);
 #define JQ_ATT_TILES(GQ)                                                                                            \
     hipLaunchKernelGGL((jq::attention_tiles<128, GQ>), tgrid, dim3(64 * GQ), 0, s, qp, m->kc[l], m->vc[l], m->att, (int)T, \
-                       nh, m->pos, (int)c.n_ctx, sqrt_d)
+                       nh, m->pos, (int)c.n_ctx, sqrt_d, q_stride)
             if (no_tiles || d != 128 || (gq != 1 && gq != 2 && gq != 4 && gq != 8)) {
                 size_t sm = ((size_t)d + jq::AR_CHUNK + 16) * sizeof(float);
                 hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, qp, m->kc[l], m->vc[l], m->att, nh,
-                                   nkv, d, m->pos, (int)c.n_ctx, sqrt_d);
+                                   nkv, d, m->pos, (int)c.n_ctx, sqrt_d, q_stride);
             } else if (gq == 1) JQ_ATT_TILES(1);
             else if (gq == 2) JQ_ATT_TILES(2);
             else if (gq == 4) JQ_ATT_TILES(4);

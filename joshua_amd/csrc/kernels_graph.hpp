@@ -57,26 +57,28 @@ __global__ __launch_bounds__(1024) void rmsnorm_rows(float *__restrict__ x, cons
 // a token: q is rewritten in place, k goes normed and rotated straight into the K
 // cache, v is copied into the V cache.  inv_freq_i = theta^(-2i/d); pairs (i, i + d/2)
 // (reference: src/quantized_qwen3_moe.rs:237-262,345-364; closed form in its test :867-895).
-// cache layout [kv_head, n_ctx, d]; *pos_ptr is the number of tokens already cached.
+// cache layout [kv_head, n_ctx, d]; *pos_ptr is the number of tokens already cached.  A token's q, k and v
+// heads start qs, ks and vs floats after the previous token's (the three may be parts of one product's rows).
 __global__ __launch_bounds__(64) void qkv_norm_rope_cache(float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ wq,
                                                            const float *__restrict__ wk, float eps, int n_head, int n_kv,
                                                            int d, const int *__restrict__ pos_ptr, float theta,
-                                                           float *__restrict__ kc, float *__restrict__ vc, int n_ctx) {
+                                                           float *__restrict__ kc, float *__restrict__ vc, int n_ctx,
+                                                           int qs, int ks, int vs) {
     const int per = n_head + 2 * n_kv;
     const int t = blockIdx.x / per, j = blockIdx.x % per, lane = threadIdx.x;
     const int pos = *pos_ptr + t;
     if (j >= n_head + n_kv) {  // v head: plain copy
         const int hd = j - n_head - n_kv;
-        const float *src = v + ((size_t)t * n_kv + hd) * d;
+        const float *src = v + (size_t)t * vs + (size_t)hd * d;
         float *dst = vc + ((size_t)hd * n_ctx + pos) * d;
         for (int c = lane; c < d; c += 64) dst[c] = src[c];
         return;
     }
     const bool is_q = j < n_head;
     const int hd = is_q ? j : j - n_head;
-    const float *src = is_q ? q + ((size_t)t * n_head + hd) * d : k + ((size_t)t * n_kv + hd) * d;
-    float *dst = is_q ? q + ((size_t)t * n_head + hd) * d : kc + ((size_t)hd * n_ctx + pos) * d;
+    const float *src = is_q ? q + (size_t)t * qs + (size_t)hd * d : k + (size_t)t * ks + (size_t)hd * d;
+    float *dst = is_q ? q + (size_t)t * qs + (size_t)hd * d : kc + ((size_t)hd * n_ctx + pos) * d;
     const float *w = is_q ? wq : wk;
     float ss = 0.0f;
     for (int c = lane; c < d; c += 64) ss = fmaf(src[c], src[c], ss);
@@ -102,12 +104,12 @@ constexpr int AR_CHUNK = 1024, AR_MAX_D = 1024;
 __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ q, const float *__restrict__ kc,
                                                        const float *__restrict__ vc, float *__restrict__ out,
                                                        int n_head, int n_kv, int d, const int *__restrict__ pos_ptr,
-                                                       int n_ctx, float sqrt_d) {
+                                                       int n_ctx, float sqrt_d, int q_stride) {
     extern __shared__ float sm[];  // q[d], scores[AR_CHUNK], red[16]
     const int t = blockIdx.x / n_head, hq = blockIdx.x % n_head;
     const int kvh = hq / (n_head / n_kv), n_keys = *pos_ptr + t + 1;
     float *qs = sm, *sc = sm + d, *red = sm + d + AR_CHUNK;
-    const float *qp = q + ((size_t)t * n_head + hq) * d;
+    const float *qp = q + (size_t)t * q_stride + (size_t)hq * d;  // a token's heads start q_stride floats apart
     for (int c = threadIdx.x; c < d; c += blockDim.x) qs[c] = qp[c];
     __syncthreads();
     const float *kb = kc + (size_t)kvh * n_ctx * d, *vb = vc + (size_t)kvh * n_ctx * d;
@@ -179,7 +181,7 @@ template <int D, int G>
 __global__ __launch_bounds__(64 * G) void attention_tiles(const float *__restrict__ q, const float *__restrict__ kc,
                                                           const float *__restrict__ vc, float *__restrict__ out,
                                                           int T, int n_head, const int *__restrict__ pos_ptr,
-                                                          int n_ctx, float sqrt_d) {
+                                                          int n_ctx, float sqrt_d, int q_stride) {
     constexpr int NT = 64 * G, STRIDE = D + AT_PAD, PIECES = 16 * (D / 4), PER = (PIECES + NT - 1) / NT;
     __shared__ __attribute__((aligned(16))) float ks[16 * STRIDE], vs[16 * STRIDE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(64 * G) void attention_tiles(const float *__restric
     // this lane's share of Q^T as B operands: token n, dimensions 4 s + g
     float qr[D / 4];
     {
-        const float *qp = q + ((size_t)min(t0 + n, T - 1) * n_head + hq) * D + g;
+        const float *qp = q + (size_t)min(t0 + n, T - 1) * q_stride + (size_t)hq * D + g;  // tokens q_stride floats apart
 #pragma unroll
         for (int s_ = 0; s_ < D / 4; s_++) qr[s_] = qp[4 * s_];
     }
