@@ -102,7 +102,15 @@ const void *jq_device_ptr(const jq_weight *w);
  * (reference: src/mmap_tensor.rs:132-134 matmul_t,
  * src/quant_matmul.rs:133-178 validate + empty case).  With
  * ptrs_are_device == 0 the call stages lhs/dst through HBM and returns after
- * the result has landed in dst. */
+ * the result has landed in dst.
+ * Accuracy: |dst - ref| <= 1e-3 * max(|ref|, 1) against the reference's f32 arithmetic
+ * (its own bound, src/kquant_dot.rs:853).  The integer kernels hold the activations in
+ * 16-bit fixed point: one scale per 32 elements of a row up to 63 activation rows, so a
+ * row whose groups span many orders of magnitude keeps the bound; from 64 rows on Q4_K
+ * and Q6_K use one scale per 256 elements, which resolves each super-block to 2^-16 of
+ * its largest magnitude (2^-12 of the sum of the terms' magnitudes on such rows; the
+ * reference's integer path quantises activations to 8 bits per 256,
+ * src/quant_matmul.rs:184).  A row holding an inf or a NaN comes out all NaN. */
 int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, float *dst,
                 size_t dst_len, int ptrs_are_device, void *stream);
 
