@@ -2399,17 +2399,24 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             static const char *no_tiles = getenv("JQ_NO_ATTENTION_TILES");
             const int gq = nh / nkv;
             const dim3 tgrid((unsigned)((T + 15) / 16), (unsigned)nkv);
-#define JQ_ATT_TILES(GQ)                                                                                            \
-    hipLaunchKernelGGL((jq::attention_tiles<128, GQ>), tgrid, dim3(64 * GQ), 0, s, qp, m->kc[l], m->vc[l], m->att, (int)T, \
-                       nh, m->pos, (int)c.n_ctx, sqrt_d, q_stride)
+#define JQ_ATT_TILES(GQ, KS)                                                                                        \
+    hipLaunchKernelGGL((jq::attention_tiles<128, GQ, KS>), tgrid, dim3(64 * GQ * KS), 0, s, qp, m->kc[l], m->vc[l],   \
+                       m->att, (int)T, nh, m->pos, (int)c.n_ctx, sqrt_d, q_stride)
+            // two key splits a workgroup once the last tokens walk 8 key tiles or more (up to 4 query heads a KV
+            // head: the merge of 8 would not fit the static LDS)
+            static const char *no_split_env = getenv("JQ_ATTENTION_TILES_NO_KEY_SPLIT");
+            const bool ksplit = !no_split_env && pos + T >= 128;
             if (no_tiles || d != 128 || (gq != 1 && gq != 2 && gq != 4 && gq != 8)) {
                 size_t sm = ((size_t)d + jq::AR_CHUNK + 16) * sizeof(float);
                 hipLaunchKernelGGL(jq::attention_rows, dim3(T * nh), dim3(256), sm, s, qp, m->kc[l], m->vc[l], m->att, nh,
                                    nkv, d, m->pos, (int)c.n_ctx, sqrt_d, q_stride);
-            } else if (gq == 1) JQ_ATT_TILES(1);
-            else if (gq == 2) JQ_ATT_TILES(2);
-            else if (gq == 4) JQ_ATT_TILES(4);
-            else JQ_ATT_TILES(8);
+            } else if (gq == 1 && ksplit) JQ_ATT_TILES(1, 2);
+            else if (gq == 1) JQ_ATT_TILES(1, 1);
+            else if (gq == 2 && ksplit) JQ_ATT_TILES(2, 2);
+            else if (gq == 2) JQ_ATT_TILES(2, 1);
+            else if (gq == 4 && ksplit) JQ_ATT_TILES(4, 2);
+            else if (gq == 4) JQ_ATT_TILES(4, 1);
+            else JQ_ATT_TILES(8, 1);
 #undef JQ_ATT_TILES
         }
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;

@@ -177,17 +177,28 @@ __global__ __launch_bounds__(256) void attention_rows(const float *__restrict__ 
 // that holds its statistics.  Scores are divided by sqrt(d) as the reference does (src/embedding.rs:386).
 constexpr int AT_PAD = 4;  // floats a staged row is longer than D: 16 rows then fall into different banks
 
-template <int D, int G>
-__global__ __launch_bounds__(64 * G) void attention_tiles(const float *__restrict__ q, const float *__restrict__ kc,
-                                                          const float *__restrict__ vc, float *__restrict__ out,
-                                                          int T, int n_head, const int *__restrict__ pos_ptr,
-                                                          int n_ctx, float sqrt_d, int q_stride) {
+// KS = 2 splits a tile's keys between two sets of G waves (key tiles of even and odd number), each with a
+// running maximum, sum and output of its own, merged through LDS at the end: the workgroups of the last
+// tokens, which walk the most key tiles and set the time of a causal prefill, take half as many steps.
+template <int D, int G, int KS>
+__global__ __launch_bounds__(64 * G * KS) void attention_tiles(const float *__restrict__ q, const float *__restrict__ kc,
+                                                               const float *__restrict__ vc, float *__restrict__ out,
+                                                               int T, int n_head, const int *__restrict__ pos_ptr,
+                                                               int n_ctx, float sqrt_d, int q_stride) {
+    static_assert(KS == 1 || KS == 2, "one or two key splits");
     constexpr int NT = 64 * G, STRIDE = D + AT_PAD, PIECES = 16 * (D / 4), PER = (PIECES + NT - 1) / NT;
-    __shared__ __attribute__((aligned(16))) float ks[16 * STRIDE], vs[16 * STRIDE];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
+    constexpr int MERGE = KS == 2 ? G * 64 * (D / 4 + 2) : 0;  // floats: a split's outputs, maximum and sum per lane
+    constexpr int STAGE = 2 * KS * 16 * STRIDE;                 // the key and value tile of each split
+    // the merge reuses the tiles' memory: every wave has left the loop by then
+    __shared__ __attribute__((aligned(16))) float lds[STAGE > MERGE ? STAGE : MERGE];
+    static_assert(sizeof(float) * (STAGE > MERGE ? STAGE : MERGE) <= 65536, "static LDS");
+    const int lane = threadIdx.x & 63, wave_all = threadIdx.x >> 6, wave = wave_all % G, sp = wave_all / G;
+    const int tid = threadIdx.x - NT * sp;  // within the split's G waves, which stage the split's tiles
+    const int n = lane & 15, g = lane >> 4;
+    float *ks = lds + sp * 16 * STRIDE, *vs = lds + (KS + sp) * 16 * STRIDE, *merge = lds;
     const int t0 = 16 * (int)blockIdx.x, kvh = blockIdx.y, hq = kvh * G + wave, pos0 = *pos_ptr;
     const int last_key = pos0 + min(t0 + 15, T - 1);        // the last key any token of the tile may see
-    const int n_tiles = last_key / 16 + 1;
+    const int n_tiles = last_key / 16 + 1, n_steps = (n_tiles + KS - 1) / KS;
     const float *kb = kc + (size_t)kvh * n_ctx * D, *vb = vc + (size_t)kvh * n_ctx * D;
 
     typedef float f4 __attribute__((ext_vector_type(4)));
@@ -215,8 +226,9 @@ __global__ __launch_bounds__(64 * G) void attention_tiles(const float *__restric
             }
         }
     };
-    fetch(0);
-    for (int tile = 0; tile < n_tiles; tile++) {
+    fetch(sp);
+    for (int step = 0; step < n_steps; step++) {
+        const int tile = KS * step + sp;  // past the last tile (the odd split, in the last step): all keys masked
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int piece = tid + NT * i, row = piece / (D / 4), c4 = piece % (D / 4);
@@ -226,43 +238,71 @@ __global__ __launch_bounds__(64 * G) void attention_tiles(const float *__restric
             }
         }
         __syncthreads();
-        if (tile + 1 < n_tiles) fetch(tile + 1);
-        // S^T: keys 16 tile + (4 g + j) x token n
-        f4 st = f4{0.f, 0.f, 0.f, 0.f};
+        if (step + 1 < n_steps) fetch(tile + KS);
+        if (tile < n_tiles) {
+            // S^T: keys 16 tile + (4 g + j) x token n
+            f4 st = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s_ = 0; s_ < D / 4; s_++)
-            st = __builtin_amdgcn_mfma_f32_16x16x4f32(ks[n * STRIDE + 4 * s_ + g], qr[s_], st, 0, 0, 0);
-        float p[4], tmax = -INFINITY;
+            for (int s_ = 0; s_ < D / 4; s_++)
+                st = __builtin_amdgcn_mfma_f32_16x16x4f32(ks[n * STRIDE + 4 * s_ + g], qr[s_], st, 0, 0, 0);
+            float p[4], tmax = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int key = 16 * tile + 4 * g + j;
-            p[j] = key <= pos0 + t0 + n ? st[j] / sqrt_d : -INFINITY;
-            tmax = fmaxf(tmax, p[j]);
-        }
-        tmax = max_xor32(max_xor16(tmax));
-        const float mnew = fmaxf(mx, tmax), rescale = expf(mx - mnew);
-        float tsum = 0.0f;
+            for (int j = 0; j < 4; j++) {
+                const int key = 16 * tile + 4 * g + j;
+                p[j] = key <= pos0 + t0 + n ? st[j] / sqrt_d : -INFINITY;
+                tmax = fmaxf(tmax, p[j]);
+            }
+            tmax = max_xor32(max_xor16(tmax));
+            // a token that sees none of this tile's keys (the odd split's first tile may lie past a token's
+            // last key) keeps its state: exp(-inf - -inf) would be NaN
+            const float mnew = fmaxf(mx, tmax), rescale = mnew == -INFINITY ? 1.0f : expf(mx - mnew);
+            float tsum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            p[j] = expf(p[j] - mnew);
-            tsum += p[j];
-        }
-        tsum = sum_xor32(sum_xor16(tsum));
-        sum = fmaf(sum, rescale, tsum);
-        mx = mnew;
-        // O rows are tokens 4 g + j: their factors live in the lanes of those tokens
-        float rs[4];
+            for (int j = 0; j < 4; j++) {
+                p[j] = mnew == -INFINITY ? 0.0f : expf(p[j] - mnew);
+                tsum += p[j];
+            }
+            tsum = sum_xor32(sum_xor16(tsum));
+            sum = fmaf(sum, rescale, tsum);
+            mx = mnew;
+            // O rows are tokens 4 g + j: their factors live in the lanes of those tokens
+            float rs[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) rs[j] = __shfl(rescale, 4 * g + j, 64);
+            for (int j = 0; j < 4; j++) rs[j] = __shfl(rescale, 4 * g + j, 64);
 #pragma unroll
-        for (int dt = 0; dt < D / 16; dt++) {
-            f4 acc = f4{o[dt][0] * rs[0], o[dt][1] * rs[1], o[dt][2] * rs[2], o[dt][3] * rs[3]};
+            for (int dt = 0; dt < D / 16; dt++) {
+                f4 acc = f4{o[dt][0] * rs[0], o[dt][1] * rs[1], o[dt][2] * rs[2], o[dt][3] * rs[3]};
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(p[j], vs[(4 * g + j) * STRIDE + 16 * dt + n], acc, 0, 0, 0);
-            o[dt] = acc;
+                for (int j = 0; j < 4; j++)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(p[j], vs[(4 * g + j) * STRIDE + 16 * dt + n], acc, 0, 0, 0);
+                o[dt] = acc;
+            }
         }
         __syncthreads();
+    }
+    if constexpr (KS == 2) {
+        // the odd split hands its state over; the even split (which always holds key 0) rescales both to the
+        // common maximum
+        float *mine = merge + (size_t)(wave * 64 + lane) * (D / 4 + 2);
+        if (sp == 1) {
+#pragma unroll
+            for (int dt = 0; dt < D / 16; dt++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) mine[4 * dt + j] = o[dt][j];
+            mine[D / 4] = mx, mine[D / 4 + 1] = sum;
+        }
+        __syncthreads();
+        if (sp == 1) return;
+        const float m1 = mine[D / 4], s1 = mine[D / 4 + 1];
+        const float mnew = fmaxf(mx, m1), f0 = expf(mx - mnew), f1 = m1 == -INFINITY ? 0.0f : expf(m1 - mnew);
+        sum = sum * f0 + s1 * f1;
+        float F0[4], F1[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) F0[j] = __shfl(f0, 4 * g + j, 64), F1[j] = __shfl(f1, 4 * g + j, 64);
+#pragma unroll
+        for (int dt = 0; dt < D / 16; dt++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[dt][j] = o[dt][j] * F0[j] + mine[4 * dt + j] * F1[j];
     }
     float inv[4];
 #pragma unroll

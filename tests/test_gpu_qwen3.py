@@ -124,6 +124,23 @@ def test_prefill_in_chunks_with_head_size_128(n_head, n_kv):
         pos += step
 
 
+@pytest.mark.parametrize("n_head,n_kv", [(4, 1), (4, 2), (2, 2), (8, 1)])
+def test_long_prefill_chunks_split_their_keys_between_two_sets_of_waves(n_head, n_kv):
+    """From 128 keys on the tiled attention gives the key tiles of even and odd number to two sets of waves
+    and merges their running softmax states (up to four query heads a KV head; eight keep one set): a chunk
+    from position 0, chunks that start inside a key tile, an odd number of key tiles, a last tile part empty."""
+    cfg = dict(CFG, n_ctx=400, n_layer=2, head_dim=128, n_head=n_head, n_kv_head=n_kv)
+    m, o = make(cfg, 33)
+    rng = np.random.default_rng(14)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=390)]
+    pos = 0
+    for step in (137, 150, 9, 94):
+        chunk = toks[pos:pos + step]
+        ok, e = close(m.forward(chunk, pos), o.forward(chunk, pos))
+        assert ok, f"pos {pos} +{step}: {e}"
+        pos += step
+
+
 @pytest.mark.parametrize("head_dim,n_head,n_kv", [(64, 4, 2), (128, 4, 1), (256, 2, 2), (192, 4, 2), (128, 8, 1),
                                                   (128, 2, 2), (128, 4, 2)])
 def test_decode_over_several_key_chunks(head_dim, n_head, n_kv):
