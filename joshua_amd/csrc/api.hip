@@ -667,7 +667,7 @@ struct GemmI8Shape {
 
 template <class F>
 int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
-                     hipStream_t s, const char *name, const char *name_split) {
+                     hipStream_t s, const char *name, const char *name_split, bool swiglu_pairs = false) {
     constexpr size_t ALIGN = F::BLOCK % 16 == 0 ? 16 : 2;
     static const char *mode = getenv("JQ_Q4K_GEMM_I8");
     static const char *min_tiles_env = getenv("JQ_Q4K_GEMM_I8_MIN_TILES");
@@ -745,8 +745,12 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
         });                                                                                                           \
         attr_rc = rc_once;                                                                                            \
         if (attr_rc == hipSuccess) {                                                                                  \
-            hipLaunchKernelGGL(jq::q4k_gemm_i8_prep, dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, X, (int)m, \
-                               (int)k, acts);                                                                         \
+            if (swiglu_pairs)                                                                                         \
+                hipLaunchKernelGGL(jq::q4k_gemm_i8_prep<true>, dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, \
+                                   X, (int)m, (int)k, acts);                                                          \
+            else                                                                                                      \
+                hipLaunchKernelGGL(jq::q4k_gemm_i8_prep<false>, dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, \
+                                   X, (int)m, (int)k, acts);                                                          \
             hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)splits), dim3(64 * NW_), lds, s, W, row_bytes,    \
                                (const uint8_t *)acts, splits > 1 ? parts : Y, (int)m, (int)n, (int)(nb / splits),     \
                                (int)groups, (int)tx, (int)ty, (int)nb, splits > 1 ? m * n : (size_t)0);               \
@@ -2424,6 +2428,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         auto fg = T == 1 ? m->fused.find(p + ".gate_up") : m->fused.end();
         const bool paired = fg != m->fused.end() && m->paired.count(fg->first);  // gate and up rows alternate
         bool activated = false;  // m->mid already holds silu(gate) * up
+        bool down_done = false;  // m->proj already holds the down projection
         const bool normed2 = fg != m->fused.end() && model_norm_mm(fg->second, xc, m->proj, w_fn, c.rms_eps, xo, nullptr,
                                                                    paired ? m->mid : m->cat, paired, s);
         if (normed2) std::swap(xc, xo), activated = paired;
@@ -2441,7 +2446,24 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         } else if (fgm != m->fused.end()) {
             const jq_weight *w = fgm->second;
             if (dispatch_matmul(w->type, w->dev, w->row_bytes, m->hn, m->g, T, w->k, w->n, s)) return 1;
-            hipLaunchKernelGGL(jq::swiglu_pairs, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, m->g, m->mid, (size_t)T * c.ffn);
+            // many rows into a Q4_K or Q6_K down projection: the int8 GEMM's activation preparation applies
+            // SwiGLU to the pairs as it reads them
+            auto dn = m->q.find(p + ".ffn_down.weight");
+            static const char *no_fused_swiglu = getenv("JQ_NO_SWIGLU_IN_PREP");
+            if (dn != m->q.end() && !no_fused_swiglu && dn->second->k == c.ffn) {
+                const jq_weight *wd = dn->second;
+                int rc = -1;
+                if (wd->type == JQ_TYPE_Q4_K)
+                    rc = dispatch_gemm_i8<jq::QiQ4K>(wd->dev, wd->row_bytes, m->g, m->proj, T, wd->k, wd->n, s, "q4k_gemm_i8",
+                                                     "q4k_gemm_i8+splitk", true);
+                else if (wd->type == JQ_TYPE_Q6_K)
+                    rc = dispatch_gemm_i8<jq::QiQ6K>(wd->dev, wd->row_bytes, m->g, m->proj, T, wd->k, wd->n, s, "q6k_gemm_i8",
+                                                     "q6k_gemm_i8+splitk", true);
+                if (rc > 0) return 1;
+                down_done = rc == 0;
+            }
+            if (!down_done)
+                hipLaunchKernelGGL(jq::swiglu_pairs, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, m->g, m->mid, (size_t)T * c.ffn);
             activated = true;
         } else if (model_mm(m, p + ".ffn_gate.weight", m->hn, m->g, T, s) ||
                    model_mm(m, p + ".ffn_up.weight", m->hn, m->u, T, s)) {
@@ -2454,7 +2476,7 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
             hipLaunchKernelGGL(jq::swiglu_rows, dim3(grid_for((size_t)T * c.ffn)), dim3(256), 0, s, gp, up, m->mid,
                                (size_t)T * c.ffn, 0.0f);
         }
-        if (model_mm(m, p + ".ffn_down.weight", m->mid, m->proj, T, s)) return 1;
+        if (!down_done && model_mm(m, p + ".ffn_down.weight", m->mid, m->proj, T, s)) return 1;
         pending = m->proj;
     }
     const float *w_on;

@@ -50,6 +50,10 @@ constexpr int QI_PLANES = 4 * 2 * 64 * 16, QI_MIN = QI_PLANES, QI_SCALE = QI_PLA
 
 // grid (k / 256 super-blocks, groups of 16 activation rows), 256 threads: wave c, lane (i, g) quantises the
 // 16 elements 64 c + 16 g .. of row i.  Rows from m_rows on are zero operands.
+// With PAIRS the activations are silu(gate) * up over rows of 2 k floats in which gate_j and up_j alternate
+// (the result of a product with a row-paired gate|up matrix): the SwiGLU of a feed-forward block happens on the
+// way into the down projection.
+template <bool PAIRS>
 __global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict__ X, int m_rows, int k,
                                                          uint8_t *__restrict__ out) {
     __shared__ float amax_sh[4][16];
@@ -58,7 +62,14 @@ __global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict_
     const int b = blockIdx.x, row = 16 * (int)blockIdx.y + i;
     uint8_t *rec = out + ((size_t)blockIdx.y * gridDim.x + b) * QI_REC;
     float v[16];
-    if (row < m_rows) {
+    if (row < m_rows && PAIRS) {
+        const float4 *src = (const float4 *)(X + 2 * ((size_t)row * k + 256 * b + 64 * c + 16 * g));
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const float4 a = src[q];
+            v[2 * q] = silu(a.x) * a.y, v[2 * q + 1] = silu(a.z) * a.w;
+        }
+    } else if (row < m_rows) {
         const float4 *src = (const float4 *)(X + (size_t)row * k + 256 * b + 64 * c + 16 * g);
 #pragma unroll
         for (int q = 0; q < 4; q++) {

@@ -124,6 +124,23 @@ def test_prefill_in_chunks_with_head_size_128(n_head, n_kv):
         pos += step
 
 
+@pytest.mark.parametrize("mix", ["q4_k_m", "q4_k"])
+def test_prefill_of_many_tokens_with_4096_wide_rows(mix):
+    """80 and 70 tokens a step at hidden = 4096: q|k(|v) as one product read through row strides, gate|up as
+    one product over the paired matrix, SwiGLU applied by the down projection's activation preparation
+    (Q4_K and, in the q4_k_m mix, Q6_K down projections on the int8 GEMM), then single-token steps."""
+    cfg = dict(CFG, n_layer=2, hidden=4096, n_head=4, n_kv_head=2, head_dim=128, ffn=1024, vocab=512, n_ctx=192)
+    m, o = make(cfg, 35, mix)
+    rng = np.random.default_rng(15)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=153)]
+    pos = 0
+    for step in (80, 70, 1, 1, 1):
+        chunk = toks[pos:pos + step]
+        ok, e = close(m.forward(chunk, pos), o.forward(chunk, pos))
+        assert ok, f"pos {pos} +{step}: {e}"
+        pos += step
+
+
 @pytest.mark.parametrize("n_head,n_kv", [(4, 1), (4, 2), (2, 2), (8, 1)])
 def test_long_prefill_chunks_split_their_keys_between_two_sets_of_waves(n_head, n_kv):
     """From 128 keys on the tiled attention gives the key tiles of even and odd number to two sets of waves
