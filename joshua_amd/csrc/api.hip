@@ -1610,9 +1610,16 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         groups = (int)c.n_expert + extra;
         max_group = (int)T;
         const int in_lds = (size_t)P <= 12288;
-        hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(jq::GROUP_PAIRS_THREADS), (c.n_expert + 1 + (in_lds ? P : 0)) * sizeof(int), s,
-                           m->ids, (int)T, (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow,
-                           extra, in_lds);
+        const size_t chunks = ((size_t)P + 63) / 64, rank_ints = chunks * c.n_expert + c.n_expert + 1;
+        static const char *no_ranked = getenv("JQ_MOE_NO_RANKED_GROUPING");
+        if (!no_ranked && chunks <= (size_t)jq::GROUP_RANK_CHUNKS && rank_ints <= 12288)
+            hipLaunchKernelGGL(jq::moe_group_pairs_ranked, dim3(1), dim3(jq::GROUP_PAIRS_THREADS), rank_ints * sizeof(int), s,
+                               m->ids, (int)T, (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow,
+                               extra);
+        else
+            hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(jq::GROUP_PAIRS_THREADS), (c.n_expert + 1 + (in_lds ? P : 0)) * sizeof(int), s,
+                               m->ids, (int)T, (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow,
+                               extra, in_lds);
     }
     HIP_TRY(hipGetLastError());
     // silu(gate x) * (up x) of every pair into G, then down over it

@@ -328,6 +328,95 @@ __global__ __launch_bounds__(GROUP_PAIRS_THREADS) void moe_group_pairs(const uin
     }
 }
 
+// The same grouping for pair lists of up to GROUP_RANK_CHUNKS * 64 pairs, by ranks instead of one pass over
+// the list per expert: a wave takes 64 consecutive pairs, every lane counts the lanes before it that name its
+// expert (its rank within the chunk), the last lane of an expert in the chunk records the chunk's count of
+// that expert in hist[chunk][expert]; prefix sums over the chunks and then over the experts turn the counts
+// into start positions, and a pair's place is its expert's start + the earlier chunks' count + its rank.
+// LDS: chunks * E + E + 1 ints.
+constexpr int GROUP_RANK_CHUNKS = 64, GROUP_RANK_PER_WAVE = GROUP_RANK_CHUNKS * 64 / GROUP_PAIRS_THREADS;
+
+__global__ __launch_bounds__(GROUP_PAIRS_THREADS) void moe_group_pairs_ranked(const uint32_t *__restrict__ ids, int T,
+                                                                              int k_used, int E, int *__restrict__ gexp,
+                                                                              int *__restrict__ offsets,
+                                                                              int *__restrict__ xrow, int *__restrict__ yrow,
+                                                                              int shared_group) {
+    extern __shared__ int hist[];  // [chunks][E], then start[E + 1]
+    const int P = T * k_used, chunks = (P + 63) / 64;
+    int *start = hist + chunks * E;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int WAVES = GROUP_PAIRS_THREADS / 64;
+    for (int i = threadIdx.x; i < chunks * E; i += GROUP_PAIRS_THREADS) hist[i] = 0;
+    __syncthreads();
+    uint32_t mine[GROUP_RANK_PER_WAVE];
+    int rank[GROUP_RANK_PER_WAVE];
+#pragma unroll
+    for (int c = 0; c < GROUP_RANK_PER_WAVE; c++) {
+        const int chunk = wave + WAVES * c, pidx = 64 * chunk + lane;
+        mine[c] = 0xFFFFFFFFu, rank[c] = 0;
+        if (chunk >= chunks) continue;  // the same for the whole wave
+        const uint32_t e = pidx < P ? ids[pidx] : 0xFFFFFFFFu;
+        int before = 0, after = 0;
+        for (int j = 0; j < 64; j++) {
+            const bool same = (uint32_t)__shfl((int)e, j, 64) == e;
+            before += same && j < lane;
+            after += same && j > lane;
+        }
+        mine[c] = e, rank[c] = before;
+        if (e < (uint32_t)E && after == 0) hist[chunk * E + (int)e] = before + 1;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += GROUP_PAIRS_THREADS) {  // counts -> counts in earlier chunks; the expert's total
+        int run = 0;
+        for (int ch = 0; ch < chunks; ch++) {
+            const int c = hist[ch * E + e];
+            hist[ch * E + e] = run;
+            run += c;
+        }
+        start[e] = run;
+    }
+    __syncthreads();
+    if (wave == 0) {  // totals -> start positions: each lane a run of experts, a wave scan between the runs
+        const int per = (E + 63) / 64, b = lane * per;
+        int local = 0;
+        for (int i = 0; i < per; i++)
+            if (b + i < E) local += start[b + i];
+        int incl = local;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
+        }
+        int run = incl - local;
+        for (int i = 0; i < per; i++) {
+            if (b + i < E) {
+                const int c = start[b + i];
+                start[b + i] = run;
+                run += c;
+            }
+        }
+        if (lane == 63) start[E] = incl;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e <= E; e += GROUP_PAIRS_THREADS) {
+        offsets[e] = start[e];
+        if (e < E) gexp[e] = e;
+    }
+    if (shared_group) {  // group E: the shared expert over every token, output rows P .. P + T - 1
+        if (threadIdx.x == 0) gexp[E] = E, offsets[E + 1] = P + T;
+        for (int t = threadIdx.x; t < T; t += GROUP_PAIRS_THREADS) xrow[P + t] = t, yrow[P + t] = P + t;
+    }
+#pragma unroll
+    for (int c = 0; c < GROUP_RANK_PER_WAVE; c++) {
+        const int chunk = wave + WAVES * c, pidx = 64 * chunk + lane;
+        if (mine[c] < (uint32_t)E) {
+            const int at = start[mine[c]] + hist[chunk * E + (int)mine[c]] + rank[c];
+            xrow[at] = pidx / k_used;
+            yrow[at] = pidx;
+        }
+    }
+}
+
 
 // Expert matmuls over the grouped pairs: blockIdx.y = group (its expert is
 // gexp[group]), rows of the expert's weight over blockIdx.x.  The activation row of the pair at sorted

@@ -115,6 +115,19 @@ def test_row_lengths_that_change_the_staging(qtype, h, inter):
         assert close(dev.forward(x), ora.forward(x))
 
 
+@pytest.mark.parametrize("tokens,E,k", [(300, 16, 4), (1000, 16, 4), (1024, 24, 4), (1100, 16, 4), (150, 160, 6)])
+def test_many_tokens_are_grouped_by_expert_in_pair_order(tokens, E, k):
+    """Pair lists of up to 4096 pairs are grouped by ranks within chunks of 64 pairs (one to four chunks a
+    wave, a last chunk part empty, experts nobody picked); longer lists, or more chunks x experts than the
+    LDS table holds, by one pass per expert.  A pair out of place would multiply a token by another expert
+    or add it to another token's sum."""
+    ora, dev = build(capi.Q8_0, 128, 64, E, k, 140 + tokens)
+    x = synth.normal(141 + tokens, (tokens, 128))
+    ids, _ = dev.route(x)
+    assert np.array_equal(ids, ora.route(x)[0])
+    assert close(dev.forward(x), ora.forward(x))
+
+
 @pytest.mark.parametrize("qtype", [capi.Q4_K, capi.MXFP4, capi.IQ2_XXS])
 def test_decode_sized_call_over_large_expert_matrices(qtype):
     """One token, expert matrices large enough that the integer-dot kernels take their activations
