@@ -126,9 +126,33 @@ __device__ __forceinline__ float qv_block_dot(const uint8_t *blk, const QvActs &
 struct QvQ4K {
     static constexpr int BLOCK = 144, ROW = 16 * BLOCK, ROW_LDS = QD_ROW_LDS;  // rows 16 bytes apart in banks
     static constexpr int STAGE_BYTES = 1152;  // what prepare() uses of `stage`
+    static constexpr bool SIDE_LDS = false;
     typedef QvActs Acts;
     __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) { return qv_prepare(v, stage, lane); }
     __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) { return qv_block_dot(blk, a, c); }
+};
+
+// The same for the kernel that keeps the operands of four columns: the accumulator start as the one word
+// that is not zero, and the four scale factors of a lane group in LDS (16 bytes a wave, column and lane group,
+// read back once a tile), 18 registers a column instead of 24.
+struct QvQ4KCompact {
+    static constexpr int BLOCK = QvQ4K::BLOCK, ROW = QvQ4K::ROW, ROW_LDS = QvQ4K::ROW_LDS, STAGE_BYTES = QvQ4K::STAGE_BYTES;
+    static constexpr bool SIDE_LDS = true;
+    struct Acts {
+        qv_i4 a_even[2], a_odd[2];
+        int c_init2;
+        const float4 *side;  // s_e, s_o16, xs_e, xs_o
+    };
+    __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane, float4 *side) {
+        const QvActs a = qv_prepare(v, stage, lane);
+        *side = float4{a.s_e, a.s_o16, a.xs_e, a.xs_o};  // the same from the 16 lanes of a group
+        return Acts{{a.a_even[0], a.a_even[1]}, {a.a_odd[0], a.a_odd[1]}, a.c_init[2], side};
+    }
+    __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) {
+        const float4 f = *a.side;
+        const QvActs full{{a.a_even[0], a.a_even[1]}, {a.a_odd[0], a.a_odd[1]}, qv_i4{0, 0, a.c_init2, 0}, f.x, f.y, f.z, f.w};
+        return qv_block_dot(blk, full, c);
+    }
 };
 
 // ---- Q2_K ----
@@ -321,6 +345,110 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
         sum = sum_row16(sum);
         if (r == 0 && t < t_end) {
             const int row = tile_row0(t) + wave;
+            if (row < n) Y[row] = sum;
+        }
+    }
+}
+
+// The same kernel for rows of more than 16 super-blocks (up to 16 NG): a tile is 16 rows x one pass of 16
+// columns (the last pass may hold fewer), tile i of a workgroup = (row tile i / NG, pass i % NG), and wave w
+// keeps the operands of its column of every pass.  The partial sums of a row tile's passes are added when the
+// tile is flushed.  nb = super-blocks a row (contiguous rows of nb blocks); rounds / extra count row tiles.
+struct QvColsWork {
+    int n, G, rounds, extra, nb;
+};
+
+template <class F, int NG>
+__global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict__ W, const float *__restrict__ X,
+                                                       float *__restrict__ Y, QvColsWork wk) {
+    static_assert(NG >= 2 && NG <= 4, "two to four passes a row");
+    constexpr int D = 2, LOADS = (F::ROW + 1023) / 1024, TG = NG == 3 ? 3 : 4;  // tiles a flush: whole row tiles
+    // the raw activations of the passes wait in the wave's own rows of ring slots 3 (behind what prepare()
+    // uses), 2 and 1, which no load targets before the wave itself asks for tiles 1, 2 and 3
+    static_assert(F::STAGE_BYTES + 1024 <= F::ROW_LDS && 2048 <= F::ROW_LDS, "staging in the ring");
+    __shared__ __attribute__((aligned(16))) uint8_t ring[QV_SLOTS][16 * F::ROW_LDS];
+    __shared__ float part[TG][16][16];  // [tile of the flush group][wave][row]
+    __shared__ float4 side[F::SIDE_LDS ? 16 * NG * 4 : 1];  // [wave][pass][lane group], for the policies that want it
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, c = lane >> 4, b = (int)blockIdx.x;
+    const int n = wk.n, G = wk.G, nb = wk.nb;
+    const size_t row_bytes = (size_t)nb * F::BLOCK;
+    const int nt = NG * (wk.rounds + (b < wk.extra ? 1 : 0));
+    if (nt <= 0) return;
+    // every fetch is LOADS instructions with at least one lane at work, so that every wave counts the same
+    // loads; a short last pass repeats its last 16 bytes into LDS bytes nobody reads
+    auto fetch = [&](int slot_i) __attribute__((always_inline)) {
+        const int i = min(slot_i, nt - 1), rt = i / NG, cg = i - rt * NG;
+        const int row = min(16 * (b + rt * G) + wave, n - 1);
+        const int len = min(16, nb - 16 * cg) * F::BLOCK;
+        const uint8_t *src = W + (size_t)row * row_bytes + (size_t)cg * F::ROW;
+        const uint32_t dst = lds_offset_of(&ring[slot_i & (QV_SLOTS - 1)][wave * F::ROW_LDS]);
+#pragma unroll
+        for (int j = 0; j < LOADS; j++) {
+            const int lanes = max(1, min(64, (min(len, F::ROW) - 1024 * j) / 16));
+            if (lane < lanes) async_load16(src + min(1024 * j + 16 * lane, len - 16), dst + 1024 * j);
+        }
+    };
+    uint32_t *stage = (uint32_t *)&ring[3][wave * F::ROW_LDS];
+    auto x_raw = [&](int cg) __attribute__((always_inline)) {
+        return cg == 0   ? (float *)((uint8_t *)stage + F::STAGE_BYTES)
+               : cg == 3 ? (float *)&ring[1][wave * F::ROW_LDS]
+                         : (float *)&ring[2][wave * F::ROW_LDS + 1024 * (cg - 1)];
+    };
+#pragma unroll
+    for (int cg = 0; cg < NG; cg++)  // a column past the row's last block reads the last one's and is not used
+        async_load16(X + 256 * min(16 * cg + wave, nb - 1) + 4 * lane, lds_offset_of(x_raw(cg)));
+    __builtin_amdgcn_s_barrier();
+    fetch(0);
+    if (LOADS == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    typename F::Acts acts[NG];
+#pragma unroll
+    for (int cg = 0; cg < NG; cg++) {
+        const float4 v = *(const float4 *)&x_raw(cg)[4 * lane];
+        if constexpr (F::SIDE_LDS) acts[cg] = F::prepare(v, stage, lane, &side[(wave * NG + cg) * 4 + c]);
+        else acts[cg] = F::prepare(v, stage, lane);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    fetch(1);
+
+    const int n_groups = (nt + TG - 1) / TG;
+    for (int grp = 0; grp < n_groups; grp++) {
+        const int t0 = TG * grp, t_end = min(nt, t0 + TG);
+#pragma unroll
+        for (int u = 0; u < TG; u++) {
+            const int t = t0 + u;
+            if (t >= t_end) break;  // the same for the whole workgroup
+            const int ahead = t == nt - 1 ? 0 : max(D - 1, min(nt - 1, t + D - 1)) - t;
+            if (LOADS == 3) {
+                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            } else {
+                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (t + D < nt) fetch(t + D);
+            const int cg = u % NG;  // t0 is a multiple of NG
+            float acc = 0.0f;
+            if (16 * cg + wave < nb)
+                acc = F::block_dot(&ring[t & (QV_SLOTS - 1)][r * F::ROW_LDS + wave * F::BLOCK], acts[cg], c);
+            if (lane < 16) part[u][wave][lane] = acc;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // lane (tt = lane / 16, ww = lane % 16) takes wave ww's sum of row `wave` in tile tt of the group, the
+        // 16 lanes of a tile add up, then the tiles that are passes of one row tile
+        float sum = t0 + c < t_end ? part[c < TG ? c : 0][r][wave] : 0.0f;
+        sum = sum_row16(sum);
+        if (NG == 2) sum = sum_xor16(sum);
+        else sum = sum_xor32(sum_xor16(sum));
+        if (r == 0 && c % NG == 0 && t0 + c < t_end) {
+            const int row = 16 * (b + ((t0 + c) / NG) * G) + wave;
             if (row < n) Y[row] = sum;
         }
     }

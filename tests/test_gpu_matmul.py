@@ -775,7 +775,10 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 1, 4096, 4096, "q4k_gemv_dot4_lds"),
     (capi.Q4_K, 1, 12288, 4096, "q4k_gemv_dot4_cols"),       # a feed-forward down projection
     (capi.Q4_K, 1, 8192, 2048, "q4k_gemv_dot4_r8"),
+    (capi.Q4_K, 1, 8192, 8192, "q4k_gemv_mfma_cols"),        # more than one row tile a workgroup
     (capi.Q4_K, 1, 2048, 768, "q4k_gemv_mfma"),              # an expert's gate projection
+    (capi.Q4_K, 1, 7168, 1536, "q4k_gemv_mfma_cols"),        # DeepSeek-V3's query down-projection
+    (capi.Q4_K, 1, 16384, 7168, "q4k_gemv_mfma_cols"),       # its attention output projection
     (capi.Q4_K, 2, 2048, 768, "q4k_gemv_mfma"),
     (capi.Q4_K, 16, 4096, 14336, "q4k_rows16_mfma"),
     (capi.Q4_K, 16, 2048, 768, "q4k_stream_mfma"),
@@ -809,6 +812,49 @@ def test_kernel_chosen_for_a_shape(qtype, m, k, n, kernel):
     w.matmul_t_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert capi.last_kernel() == kernel
+
+
+# ---- Q4_K, one activation row over rows of 17 to 64 super-blocks: the matrix-core GEMV in passes of 16 columns ----
+
+@pytest.mark.parametrize("k,n", [(4352, 600), (5120, 512), (7168, 1536), (7168, 576 + 7), (8192 + 256, 1000), (12288 + 512, 4200),
+                                 (13056, 4096 + 3), (16384, 7168), (16384, 4100), (16128, 4229)])
+def test_q4k_mfma_gemv_in_passes_of_16_columns(k, n):
+    """Two, three and four passes, a last pass of 1 to 16 columns, row counts that leave workgroups one tile
+    more than others and a last tile part empty."""
+    blocks = make_blocks(capi.Q4_K, n, k, 600 + n % 97)
+    lhs = synth.normal(601 + k % 13, (1, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, lhs)
+    assert capi.last_kernel() == "q4k_gemv_mfma_cols"
+    assert close(got, oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+@pytest.mark.parametrize("k,n", [(5120, 530), (12032, 530), (16384, 4130)])
+def test_q4k_mfma_gemv_in_passes_integer_sums_and_odd_activations(k, n):
+    """Exact integer products (activation scale 1 in every 32-element group), then a row that spans many
+    orders of magnitude and a non-finite value."""
+    blocks, q, x = q4k_integer_case(n, k, 33 + k % 7, group=32, big_value=32639, small=300)
+    want = x @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    got = w.matmul_t(1, x[None, :].astype(np.float32))
+    assert capi.last_kernel() == "q4k_gemv_mfma_cols"
+    assert np.array_equal(got[0], want.astype(np.float32))
+    blocks = make_blocks(capi.Q4_K, n, k, 610)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    rng = np.random.default_rng(k)
+    lhs = synth.normal(611, (1, k))
+    lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 32)).repeat(32).astype(np.float32)
+    # 16-bit fixed point per 32 elements: 2^-15 of a group's largest magnitude an element; held to 2^-14 of the
+    # sum of the terms' magnitudes everywhere and to the usual bound where the terms do not cancel below a
+    # twentieth of it
+    wd = oracle.dequantize(capi.Q4_K, blocks).reshape(n, k).astype(np.float64)
+    ref, mag = wd @ lhs[0].astype(np.float64), np.abs(wd) @ np.abs(lhs[0].astype(np.float64))
+    err = np.abs(w.matmul_t(1, lhs)[0] - ref)
+    assert np.all(err <= 2.0 ** -14 * mag)
+    big = np.abs(ref) >= 0.05 * mag
+    assert big.sum() > n // 8 and np.all(err[big] <= 1e-3 * np.abs(ref[big]))
+    lhs[0, k - 5] = np.inf
+    assert np.all(np.isnan(w.matmul_t(1, lhs)))
 
 
 # ---- Q2_K, one activation row over 4096-wide rows: the int8 matrix-core GEMV ----
