@@ -1883,6 +1883,8 @@ struct jq_mla {
     const jq_weight *q, *q_b, *kv_a, *kv_b, *o;
     float *q_a_norm = nullptr, *kv_a_norm = nullptr;
     float *wkv = nullptr;   // the KV up-projection as dense f32 [n_head * (nope + vh), lkv]
+    uint8_t *qa_kva = nullptr;  // q_a's rows followed by kv_a's in one allocation (same format and width): one product a single-token step
+    float *qa_kva_out = nullptr;  // its result, q_lora_rank + lkv + rope floats
     float2 *cs = nullptr;   // [n_ctx][rope / 2] (cos, sin), scaled by the YaRN mscale
     float *lat = nullptr, *kpe = nullptr;  // the cache: [n_ctx][lkv] normed latents, [n_ctx][rope] rotated keys
     float scale = 0.0f;
@@ -1984,17 +1986,25 @@ int mla_forward_dev(jq_mla *m, size_t S, size_t pos, const float *x, float *out,
     const jq_mla_config &c = m->cfg;
     const size_t nh = c.n_head, nope = c.qk_nope_head_dim, rope = c.qk_rope_head_dim, vh = c.v_head_dim,
                  lkv = c.kv_lora_rank, qd = nope + rope;
+    const float *comp = m->comp;
     if (c.q_lora_rank) {
-        if (dispatch_matmul(m->q->type, m->q->dev, m->q->row_bytes, x, m->t1, S, c.n_embd, c.q_lora_rank, s)) return 1;
-        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3((unsigned)S), dim3(1024), 0, s, m->t1, (const float *)nullptr,
+        float *t1 = m->t1;
+        if (S == 1 && m->qa_kva) {  // one token: q_a and kv_a as one product over the rows laid end to end
+            if (dispatch_matmul(m->q->type, m->qa_kva, m->q->row_bytes, x, m->qa_kva_out, 1, c.n_embd, m->q->n + m->kv_a->n, s)) return 1;
+            t1 = m->qa_kva_out, comp = m->qa_kva_out + m->q->n;
+        } else if (dispatch_matmul(m->q->type, m->q->dev, m->q->row_bytes, x, m->t1, S, c.n_embd, c.q_lora_rank, s)) {
+            return 1;
+        }
+        hipLaunchKernelGGL(jq::rmsnorm_rows, dim3((unsigned)S), dim3(1024), 0, s, t1, (const float *)nullptr,
                            (const float *)m->q_a_norm, c.rms_eps, m->t1n, (int)c.q_lora_rank);
         HIP_TRY(hipGetLastError());
         if (dispatch_matmul(m->q_b->type, m->q_b->dev, m->q_b->row_bytes, m->t1n, m->qv, S, c.q_lora_rank, nh * qd, s)) return 1;
     } else if (dispatch_matmul(m->q->type, m->q->dev, m->q->row_bytes, x, m->qv, S, c.n_embd, nh * qd, s)) {
         return 1;
     }
-    if (dispatch_matmul(m->kv_a->type, m->kv_a->dev, m->kv_a->row_bytes, x, m->comp, S, c.n_embd, lkv + rope, s)) return 1;
-    hipLaunchKernelGGL(jq::mla_rope_latent, dim3((unsigned)nh + 1, (unsigned)S), dim3(64), 0, s, m->qv, (const float *)m->comp,
+    if (comp == m->comp && dispatch_matmul(m->kv_a->type, m->kv_a->dev, m->kv_a->row_bytes, x, m->comp, S, c.n_embd, lkv + rope, s))
+        return 1;
+    hipLaunchKernelGGL(jq::mla_rope_latent, dim3((unsigned)nh + 1, (unsigned)S), dim3(64), 0, s, m->qv, comp,
                        (const float *)m->kv_a_norm, (const float2 *)m->cs, m->lat, m->kpe, (int)nh, (int)nope, (int)rope,
                        (int)lkv, (int)pos, c.rms_eps);
     HIP_TRY(hipGetLastError());
@@ -2116,6 +2126,13 @@ int jq_mla_create(const jq_mla_config *cfg, const jq_weight *q_or_q_a, const flo
     }
     HIP_TRY(hipMalloc((void **)&m->kv_a_norm, lkv * sizeof(float)));
     HIP_TRY(hipMemcpy(m->kv_a_norm, kv_a_norm, lkv * sizeof(float), hipMemcpyHostToDevice));
+    if (c.q_lora_rank && m->q->type == m->kv_a->type && m->q->row_bytes == m->kv_a->row_bytes && !getenv("JQ_MLA_NO_FUSED_QA_KVA")) {
+        const size_t qa_bytes = m->q->n * m->q->row_bytes, kva_bytes = m->kv_a->n * m->kv_a->row_bytes;
+        HIP_TRY(hipMalloc((void **)&m->qa_kva, qa_bytes + kva_bytes));
+        HIP_TRY(hipMemcpy(m->qa_kva, m->q->dev, qa_bytes, hipMemcpyDeviceToDevice));
+        HIP_TRY(hipMemcpy(m->qa_kva + qa_bytes, m->kv_a->dev, kva_bytes, hipMemcpyDeviceToDevice));
+        HIP_TRY(hipMalloc((void **)&m->qa_kva_out, (m->q->n + m->kv_a->n) * sizeof(float)));
+    }
     const std::vector<float2> cs = mla_rope_table(c);
     HIP_TRY(hipMalloc((void **)&m->cs, cs.size() * sizeof(float2)));
     HIP_TRY(hipMemcpy(m->cs, cs.data(), cs.size() * sizeof(float2), hipMemcpyHostToDevice));
@@ -2129,7 +2146,8 @@ int jq_mla_create(const jq_mla_config *cfg, const jq_weight *q_or_q_a, const flo
 void jq_mla_free(jq_mla *m) {
     if (!m) return;
     mla_free_scratch(m);
-    for (void *p : {(void *)m->q_a_norm, (void *)m->kv_a_norm, (void *)m->wkv, (void *)m->cs, (void *)m->lat, (void *)m->kpe})
+    for (void *p : {(void *)m->q_a_norm, (void *)m->kv_a_norm, (void *)m->wkv, (void *)m->cs, (void *)m->lat, (void *)m->kpe,
+                    (void *)m->qa_kva, (void *)m->qa_kva_out})
         if (p) (void)hipFree(p);
     delete m;
 }
