@@ -135,7 +135,10 @@ int jq_matmul_t_f16(const jq_weight *w, size_t m, const uint16_t *lhs, size_t lh
  * activation rows and 256 columns up to 256 rows and 4 m k bytes beyond; the other
  * formats 4 m k bytes from 8 rows on; a product split over k adds 4 m n bytes a split).
  * Every call on a device shares that device's array: calls whose kernels overlap on
- * one device (two streams, two threads) race; calls on one stream are safe. */
+ * one device (two streams, two threads) race; calls on one stream are safe.
+ * Where jq_matmul_t would split a product over k into more partial results than the
+ * array holds, this call takes fewer splits: the result then differs from jq_matmul_t's
+ * in the order of its f32 additions (within the accuracy bound, not bit for bit). */
 #define JQ_NOALLOC_SCRATCH_BYTES (32u << 20)
 int jq_matmul_t_noalloc(const jq_weight *w, size_t m, const float *lhs_dev, size_t lhs_len,
                         float *dst_dev, size_t dst_len, void *stream);

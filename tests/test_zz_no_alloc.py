@@ -28,7 +28,8 @@ def run_both(w, m, lhs):
 
 CASES = [  # (format, k, n, first m, second m): shapes whose kernels keep operands or partial sums in scratch
     (capi.Q4_K, 4096, 2048, 16, 5),      # 16-row int8 kernel: prepared activation operands
-    (capi.Q4_K, 4096, 1024, 96, 40),     # GEMM split over k: activation planes and partial sums
+    (capi.Q4_K, 4096, 1024, 96, 40),     # int8 and f16 GEMMs split over k: activation planes and partial sums
+    (capi.Q6_K, 4096, 1024, 128, 64),    # Q6_K int8 GEMM split over k
     (capi.Q4_K, 1024, 512, 12, 3),       # streaming kernel (no scratch) and one row
     (capi.Q6_K, 2048, 4096, 48, 9),      # GEMM over decoded weights, split over k
     (capi.Q8_0, 4096, 4096, 1, 1),       # one row: no scratch at all
