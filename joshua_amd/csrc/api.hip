@@ -2004,24 +2004,38 @@ int mla_forward_dev(jq_mla *m, size_t S, size_t pos, const float *x, float *out,
     }
     if (comp == m->comp && dispatch_matmul(m->kv_a->type, m->kv_a->dev, m->kv_a->row_bytes, x, m->comp, S, c.n_embd, lkv + rope, s))
         return 1;
-    hipLaunchKernelGGL(jq::mla_rope_latent, dim3((unsigned)nh + 1, (unsigned)S), dim3(64), 0, s, m->qv, comp,
-                       (const float *)m->kv_a_norm, (const float2 *)m->cs, m->lat, m->kpe, (int)nh, (int)nope, (int)rope,
-                       (int)lkv, (int)pos, c.rms_eps);
-    HIP_TRY(hipGetLastError());
-    // one token a workgroup in a decode step, four in a prefill; 16-byte loads when the latent width allows
     const bool vec4 = lkv % 4 == 0;
     const unsigned st = S == 1 ? 1 : 4;
-    {
-        const dim3 grid((unsigned)nh, (unsigned)((S + st - 1) / st));
-#define JQ_MLA_ABSORB(ST, CW)                                                                                          \
-    hipLaunchKernelGGL((jq::mla_absorb_q<ST, CW>), grid, dim3(512), 0, s, (const float *)m->qv, (const float *)m->wkv, \
-                       m->qabs, (int)S, (int)nh, (int)nope, (int)rope, (int)vh, (int)lkv)
-        if (vec4 && st == 1) JQ_MLA_ABSORB(1, 4);
-        else if (vec4) JQ_MLA_ABSORB(4, 4);
-        else if (st == 1) JQ_MLA_ABSORB(1, 1);
-        else JQ_MLA_ABSORB(4, 1);
-#undef JQ_MLA_ABSORB
+    static const char *no_absorb_rope = getenv("JQ_MLA_NO_ABSORB_ROPE");
+    if (S == 1 && !no_absorb_rope) {
+        // one token: the rotation / latent kernel's work rides in the first wave of the absorption's workgroups
+        if (vec4)
+            hipLaunchKernelGGL(jq::mla_absorb_rope<4>, dim3((unsigned)nh + 1), dim3(512), 0, s, m->qv, (const float *)m->wkv, m->qabs,
+                               (int)nh, (int)nope, (int)rope, (int)vh, (int)lkv, comp, (const float *)m->kv_a_norm,
+                               (const float2 *)m->cs, m->lat, m->kpe, (int)pos, c.rms_eps);
+        else
+            hipLaunchKernelGGL(jq::mla_absorb_rope<1>, dim3((unsigned)nh + 1), dim3(512), 0, s, m->qv, (const float *)m->wkv, m->qabs,
+                               (int)nh, (int)nope, (int)rope, (int)vh, (int)lkv, comp, (const float *)m->kv_a_norm,
+                               (const float2 *)m->cs, m->lat, m->kpe, (int)pos, c.rms_eps);
         HIP_TRY(hipGetLastError());
+    } else {
+        hipLaunchKernelGGL(jq::mla_rope_latent, dim3((unsigned)nh + 1, (unsigned)S), dim3(64), 0, s, m->qv, comp,
+                           (const float *)m->kv_a_norm, (const float2 *)m->cs, m->lat, m->kpe, (int)nh, (int)nope, (int)rope,
+                           (int)lkv, (int)pos, c.rms_eps);
+        HIP_TRY(hipGetLastError());
+        // one token a workgroup in a decode step, four in a prefill; 16-byte loads when the latent width allows
+        {
+            const dim3 grid((unsigned)nh, (unsigned)((S + st - 1) / st));
+#define JQ_MLA_ABSORB(ST, CW)                                                                                          \
+        hipLaunchKernelGGL((jq::mla_absorb_q<ST, CW>), grid, dim3(512), 0, s, (const float *)m->qv, (const float *)m->wkv, \
+                           m->qabs, (int)S, (int)nh, (int)nope, (int)rope, (int)vh, (int)lkv)
+            if (vec4 && st == 1) JQ_MLA_ABSORB(1, 4);
+            else if (vec4) JQ_MLA_ABSORB(4, 4);
+            else if (st == 1) JQ_MLA_ABSORB(1, 1);
+            else JQ_MLA_ABSORB(4, 1);
+#undef JQ_MLA_ABSORB
+            HIP_TRY(hipGetLastError());
+        }
     }
     const size_t total = pos + S;
     size_t n_split;

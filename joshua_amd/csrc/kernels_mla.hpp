@@ -25,14 +25,15 @@ namespace jq {
 // (neighbouring pairs (2i, 2i+1), candle's rope_i; cs[p][i] = (cos, sin) of position p, pair i, already
 // scaled by the YaRN mscale; reference :302-311).  Workgroup x == n_head norms the latent
 // comp[s, 0:lkv] (RMSNorm, weight w) into lat[pos0 + s] and rotates comp[s, lkv:] into kpe[pos0 + s].
-__global__ __launch_bounds__(64) void mla_rope_latent(float *__restrict__ q, const float *__restrict__ comp,
-                                                       const float *__restrict__ w, const float2 *__restrict__ cs,
-                                                       float *__restrict__ lat, float *__restrict__ kpe, int n_head,
-                                                       int nope, int rope, int lkv, int pos0, float eps) {
-    const int s = blockIdx.y, lane = threadIdx.x, half = rope >> 1;
+__device__ __forceinline__ void mla_rope_latent_wave(float *__restrict__ q, const float *__restrict__ comp,
+                                                     const float *__restrict__ w, const float2 *__restrict__ cs,
+                                                     float *__restrict__ lat, float *__restrict__ kpe, int n_head,
+                                                     int nope, int rope, int lkv, int pos0, float eps, int bx, int s,
+                                                     int lane) {
+    const int half = rope >> 1;
     const float2 *c = cs + (size_t)(pos0 + s) * half;
-    if ((int)blockIdx.x < n_head) {
-        float *v = q + ((size_t)s * n_head + blockIdx.x) * (nope + rope) + nope;
+    if (bx < n_head) {
+        float *v = q + ((size_t)s * n_head + bx) * (nope + rope) + nope;
         for (int i = lane; i < half; i += 64) {
             const float a = v[2 * i], b = v[2 * i + 1];
             v[2 * i] = a * c[i].x - b * c[i].y;
@@ -54,18 +55,26 @@ __global__ __launch_bounds__(64) void mla_rope_latent(float *__restrict__ q, con
     }
 }
 
+__global__ __launch_bounds__(64) void mla_rope_latent(float *__restrict__ q, const float *__restrict__ comp,
+                                                       const float *__restrict__ w, const float2 *__restrict__ cs,
+                                                       float *__restrict__ lat, float *__restrict__ kpe, int n_head,
+                                                       int nope, int rope, int lkv, int pos0, float eps) {
+    mla_rope_latent_wave(q, comp, w, cs, lat, kpe, n_head, nope, rope, lkv, pos0, eps, (int)blockIdx.x, (int)blockIdx.y,
+                         (int)threadIdx.x);
+}
+
 // q_abs[s, h, c] = sum_r q[s, h, r] * Wkv[h * (nope + vh) + r, c], r < nope.  grid (n_head, ceil(S / ST)),
 // 512 threads: thread (row quarter, column group of CW) walks a quarter of the head's nope rows (the
 // rows are read coalesced, once per ST tokens, whose query values wait in LDS); the four quarters sum
 // through LDS.  CW = 4 (16-byte loads) needs lkv % 4 == 0 and lkv <= 512; CW = 1 any lkv <= 128.
 constexpr int MLA_MAX_NOPE = 256, MLA_MAX_LKV = 512;
 template <int ST, int CW>
-__global__ __launch_bounds__(512) void mla_absorb_q(const float *__restrict__ q, const float *__restrict__ Wkv,
-                                                     float *__restrict__ qabs, int S, int n_head, int nope, int rope,
-                                                     int vh, int lkv) {
+__device__ __forceinline__ void mla_absorb_q_workgroup(const float *__restrict__ q, const float *__restrict__ Wkv,
+                                                       float *__restrict__ qabs, int S, int n_head, int nope, int rope,
+                                                       int vh, int lkv, int h, int s0) {
     __shared__ float qs[MLA_MAX_NOPE][ST];
     __shared__ float red[3][ST][128 * CW];
-    const int h = blockIdx.x, s0 = blockIdx.y * ST, qd = nope + rope;
+    const int qd = nope + rope;
     for (int e = threadIdx.x; e < nope * ST; e += 512) {
         const int r = e / ST, j = e % ST;
         qs[r][j] = s0 + j < S ? q[((size_t)(s0 + j) * n_head + h) * qd + r] : 0.0f;
@@ -111,6 +120,28 @@ __global__ __launch_bounds__(512) void mla_absorb_q(const float *__restrict__ q,
                 if (s0 + j < S) qabs[((size_t)(s0 + j) * n_head + h) * lkv + c + i] = v;
             }
     }
+}
+
+template <int ST, int CW>
+__global__ __launch_bounds__(512) void mla_absorb_q(const float *__restrict__ q, const float *__restrict__ Wkv,
+                                                     float *__restrict__ qabs, int S, int n_head, int nope, int rope,
+                                                     int vh, int lkv) {
+    mla_absorb_q_workgroup<ST, CW>(q, Wkv, qabs, S, n_head, nope, rope, vh, lkv, (int)blockIdx.x, (int)blockIdx.y * ST);
+}
+
+// mla_rope_latent and mla_absorb_q of a single-token step as one launch: grid n_head + 1, 512 threads.  The
+// first wave of workgroup x does what workgroup x of mla_rope_latent does (it touches the rope slice of
+// q[x], the absorption reads the other slice); workgroup n_head has nothing else to do.
+template <int CW>
+__global__ __launch_bounds__(512) void mla_absorb_rope(float *__restrict__ q, const float *__restrict__ Wkv,
+                                                        float *__restrict__ qabs, int n_head, int nope, int rope, int vh,
+                                                        int lkv, const float *__restrict__ comp, const float *__restrict__ w,
+                                                        const float2 *__restrict__ cs, float *__restrict__ lat,
+                                                        float *__restrict__ kpe, int pos0, float eps) {
+    if (threadIdx.x < 64)
+        mla_rope_latent_wave(q, comp, w, cs, lat, kpe, n_head, nope, rope, lkv, pos0, eps, (int)blockIdx.x, 0, (int)threadIdx.x);
+    if ((int)blockIdx.x == n_head) return;
+    mla_absorb_q_workgroup<1, CW>(q, Wkv, qabs, 1, n_head, nope, rope, vh, lkv, (int)blockIdx.x, 0);
 }
 
 // Scores, running softmax and the weighted latent sum for G heads of one query token over one split of
