@@ -327,6 +327,8 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
                                                              False, 0, 0.0)
         elif only == "moe_v3":
             out["moe_deepseek_v3_iq2_xxs_b1"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 1, 105, steps, True, 1, 0.0)
+        elif only == "moe_v3_mxfp4":
+            out["moe_deepseek_v3_mxfp4_b1"] = moe_workload(torch, capi, synth, 39, 7168, 2048, 256, 8, 1, 105, steps, True, 1, 0.0)
         return out
     out["q8_0_gemv_4096x4096_m1"] = matmul_workload(torch, capi, synth, 8, 4096, 4096, 1, 101, steps, 24, cs)
     out["q4_k_14336x4096_m16"] = matmul_workload(torch, capi, synth, 12, N, K, 16, 102, steps, 24, cs)

@@ -676,20 +676,21 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
     return 0;
 }
 
-// Q4_K and Q6_K with many activation rows on the int8 matrix cores: the activations as two int8 planes per
+// Q4_K, Q6_K, Q2_K and Q8_0 with many activation rows on the int8 matrix cores: the activations as two int8 planes per
 // 256-element super-block in the call scratch of the stream, then kq_gemm_i8 with the workgroup shape and the
 // split over k that an estimate fitted to measurements prefers.  Returns -1 when the shape is outside its
 // reach or the product is tiny.  JQ_Q4K_GEMM_I8 = 0 switches it off; JQ_Q4K_GEMM_I8_SHAPE and _SPLITS force the
 // choice, _MIN_TILES moves the floor (small tiles times the splits that k allows; default 64), _MIN_M the
-// fewest activation rows (default 64, at least 17).
+// fewest activation rows (default: min_m_default, 64 for Q4_K, which has kernels of its own below that).
 struct GemmI8Shape {
     int nw, ng;
 };
 
 template <class F>
 int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t m, size_t k, size_t n,
-                     hipStream_t s, const char *name, const char *name_split, bool swiglu_pairs = false) {
-    constexpr size_t ALIGN = F::BLOCK % 16 == 0 ? 16 : 2;
+                     hipStream_t s, const char *name, const char *name_split, bool swiglu_pairs = false,
+                     size_t min_m_default = 64) {
+    constexpr size_t ALIGN = F::ALIGN;
     static const char *mode = getenv("JQ_Q4K_GEMM_I8");
     static const char *min_tiles_env = getenv("JQ_Q4K_GEMM_I8_MIN_TILES");
     static const char *shape_env = getenv("JQ_Q4K_GEMM_I8_SHAPE");  // "waves,groups": one of the shapes below
@@ -697,7 +698,10 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
     // One activation scale per 256 elements resolves a row relative to its super-blocks' largest magnitudes:
     // that is the contract from 64 rows on (prefill); fewer rows keep the kernels with a scale per 32.
     static const char *min_m_env = getenv("JQ_Q4K_GEMM_I8_MIN_M");
-    static const size_t min_m = min_m_env ? std::max<size_t>((size_t)atoll(min_m_env), 17) : 64;
+    const size_t min_m = min_m_env ? std::max<size_t>((size_t)atoll(min_m_env), 2) : min_m_default;
+    // fewer than 64 rows (the formats without a kernel of their own for them): against 8M weights or more; below
+    // that the GEMM over decoded weights is as fast or faster (32 x 2048 x 2048: 16 us against 22)
+    if (!min_m_env && m < 64 && n * k < ((size_t)8 << 20)) return -1;
     if ((mode && mode[0] == '0') || m < min_m || k % 256 != 0 || row_bytes % ALIGN != 0 || ((uintptr_t)W & (ALIGN - 1)) != 0 ||
         ((uintptr_t)X & 15) != 0 || m > 0x7FFFFFF0ull || n > 0x7FFFFFF0ull)
         return -1;
@@ -758,7 +762,7 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
 #define JQ_GEMM_I8(NW_, NG_)                                                                                          \
     if (best->nw == NW_ && best->ng == NG_) {                                                                         \
         auto kern = jq::kq_gemm_i8<F, NW_, NG_>;                                                                      \
-        constexpr int lds = jq::qi_lds_bytes<NG_>();                                                                  \
+        constexpr int lds = jq::qi_lds_bytes<F, NG_>();                                                                  \
         static std::once_flag big_lds;                                                                                \
         static hipError_t rc_once = hipSuccess;                                                                       \
         std::call_once(big_lds, [&] {                                                                                 \
@@ -767,10 +771,10 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
         attr_rc = rc_once;                                                                                            \
         if (attr_rc == hipSuccess) {                                                                                  \
             if (swiglu_pairs)                                                                                         \
-                hipLaunchKernelGGL(jq::q4k_gemm_i8_prep<true>, dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, \
+                hipLaunchKernelGGL((jq::q4k_gemm_i8_prep<true, F::SUB16>), dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, \
                                    X, (int)m, (int)k, acts);                                                          \
             else                                                                                                      \
-                hipLaunchKernelGGL(jq::q4k_gemm_i8_prep<false>, dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, \
+                hipLaunchKernelGGL((jq::q4k_gemm_i8_prep<false, F::SUB16>), dim3((unsigned)nb, (unsigned)groups), dim3(256), 0, s, \
                                    X, (int)m, (int)k, acts);                                                          \
             hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)splits), dim3(64 * NW_), lds, s, W, row_bytes,    \
                                (const uint8_t *)acts, splits > 1 ? parts : Y, (int)m, (int)n, (int)(nb / splits),     \
@@ -923,8 +927,21 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         const int rc = dispatch_gemm_i8<jq::QiQ4K>(W, row_bytes, X, Y, m, k, n, s, "q4k_gemm_i8", "q4k_gemm_i8+splitk");
         if (rc >= 0) return rc;
     }
-    if (type == JQ_TYPE_Q6_K && m > Q4K_MFMA_MAX_M) {
-        const int rc = dispatch_gemm_i8<jq::QiQ6K>(W, row_bytes, X, Y, m, k, n, s, "q6k_gemm_i8", "q6k_gemm_i8+splitk");
+    // Q6_K, Q2_K, Q8_0: the same GEMM wherever the MFMA GEMM over decoded weights would run otherwise (from 17
+    // rows on, and from JQ_DECODED_GEMM_MIN_M rows on against matrices of 8M elements or more)
+    static const char *dec_min_m_env = getenv("JQ_DECODED_GEMM_MIN_M");
+    static const size_t gemm_min_m = dec_min_m_env ? (size_t)std::max(atoi(dec_min_m_env), 2) : 8;
+    const bool many_rows = m > Q4K_MFMA_MAX_M || (m >= gemm_min_m && n * k >= ((size_t)8 << 20));
+    if (type == JQ_TYPE_Q6_K && many_rows) {
+        const int rc = dispatch_gemm_i8<jq::QiQ6K>(W, row_bytes, X, Y, m, k, n, s, "q6k_gemm_i8", "q6k_gemm_i8+splitk", false, 2);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q2_K && many_rows) {
+        const int rc = dispatch_gemm_i8<jq::QiQ2K>(W, row_bytes, X, Y, m, k, n, s, "q2k_gemm_i8", "q2k_gemm_i8+splitk", false, 2);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q8_0 && many_rows) {
+        const int rc = dispatch_gemm_i8<jq::QiQ8_0>(W, row_bytes, X, Y, m, k, n, s, "q8_0_gemm_i8", "q8_0_gemm_i8+splitk", false, 2);
         if (rc >= 0) return rc;
     }
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&
@@ -934,9 +951,7 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     // activation tile part empty) from JQ_DECODED_GEMM_MIN_M rows (default 8) on against matrices of 8M
     // elements or more, where the f32 staged kernel takes a pass over the matrix per four rows (Q6_K
     // 4096 x 12288: 77 us at any row count against 92 us at 8 rows and 178 us at 16)
-    static const char *min_m_env = getenv("JQ_DECODED_GEMM_MIN_M");
-    static const size_t gemm_min_m = min_m_env ? (size_t)std::max(atoi(min_m_env), 2) : 8;
-    if ((m > Q4K_MFMA_MAX_M || (m >= gemm_min_m && n * k >= ((size_t)8 << 20))) && type != JQ_TYPE_Q4_K) {
+    if (many_rows && type != JQ_TYPE_Q4_K) {
         const int rc = dispatch_gemm_decoded(type, W, row_bytes, X, Y, m, k, n, s);
         if (rc >= 0) return rc;
     }

@@ -1,5 +1,7 @@
-// Q4_K and Q6_K matmul for many activation rows on the int8 matrix cores.  The arithmetic is written out
-// for Q4_K; Q6_K (w = d sc (q - 32), signed 8-bit sc, no min term) takes the same path with p = sc (q - 32).
+// Q4_K, Q6_K, Q2_K and Q8_0 matmul for many activation rows on the int8 matrix cores.  The arithmetic is
+// written out for Q4_K; Q6_K (w = d sc (q - 32), signed 8-bit sc, no min term) takes the same path with
+// p = sc (q - 32), Q2_K with a one-byte p = sc q and sixteen sub-blocks in I2, Q8_0 with eight blocks put on
+// a common scale (QiQ2K, QiQ8_0 below).
 //
 // Per 256-element super-block B of weight row n and activation row m (reference arithmetic
 // w = d sc q - dmin m, src/kquant_dot.rs:440-465):
@@ -53,11 +55,13 @@ constexpr int QI_PLANES = 4 * 2 * 64 * 16, QI_MIN = QI_PLANES, QI_SCALE = QI_PLA
 // With PAIRS the activations are silu(gate) * up over rows of 2 k floats in which gate_j and up_j alternate
 // (the result of a product with a row-paired gate|up matrix): the SwiGLU of a feed-forward block happens on the
 // way into the down projection.
-template <bool PAIRS>
+// With SUB16 the I2 operand is over the 16 sub-blocks of 16 elements (Q2_K): g = 0 holds a0 of sub-blocks
+// 0..7, g = 1 a0 of 8..15, g = 2 and 3 a1 of the same.
+template <bool PAIRS, bool SUB16 = false>
 __global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict__ X, int m_rows, int k,
                                                          uint8_t *__restrict__ out) {
     __shared__ float amax_sh[4][16];
-    __shared__ int xs_sh[16][8];
+    __shared__ int xs_sh[16][SUB16 ? 16 : 8];
     const int tid = threadIdx.x, lane = tid & 63, c = tid >> 6, i = lane & 15, g = lane >> 4;
     const int b = blockIdx.x, row = 16 * (int)blockIdx.y + i;
     uint8_t *rec = out + ((size_t)blockIdx.y * gridDim.x + b) * QI_REC;
@@ -98,21 +102,25 @@ __global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict_
         h[e >> 2] |= (uint32_t)(((Xq + 128) >> 8) & 255) << (8 * (e & 3));
         sum += Xq;
     }
-    sum = isum_xor16(sum);  // the two lane groups of a sub-block
-    if ((g & 1) == 0) xs_sh[i][2 * c + (g >> 1)] = sum;
+    if (SUB16) {
+        xs_sh[i][4 * c + g] = sum;  // a lane's 16 elements are a sub-block
+    } else {
+        sum = isum_xor16(sum);  // the two lane groups of a sub-block
+        if ((g & 1) == 0) xs_sh[i][2 * c + (g >> 1)] = sum;
+    }
     *(uint4 *)(rec + ((size_t)(2 * c) * 64 + lane) * 16) = uint4{h[0], h[1], h[2], h[3]};
     *(uint4 *)(rec + ((size_t)(2 * c + 1) * 64 + lane) * 16) = uint4{l[0], l[1], l[2], l[3]};
     __syncthreads();
     if (tid < 64) {
         uint32_t w[4] = {0, 0, 0, 0};
-        if (g < 2) {
+        if (SUB16 || g < 2) {
 #pragma unroll
             for (int j = 0; j < 8; j += 2) {
                 qi_h2 pair;
 #pragma unroll
                 for (int e = 0; e < 2; e++) {
-                    const int xs = xs_sh[i][j + e], a1 = (xs + 512) >> 10, a0 = xs - 1024 * a1;
-                    pair[e] = (_Float16)(float)(g == 0 ? a0 : a1);
+                    const int xs = xs_sh[i][(SUB16 ? 8 * (g & 1) : 0) + j + e], a1 = (xs + 512) >> 10, a0 = xs - 1024 * a1;
+                    pair[e] = (_Float16)(float)((SUB16 ? g < 2 : g == 0) ? a0 : a1);
                 }
                 w[j >> 1] = __builtin_bit_cast(uint32_t, pair);
             }
@@ -123,10 +131,12 @@ __global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict_
 }
 
 // LDS per buffer: NG tiles of 16 weight rows x [chunk 4][plane 2 (Ph, Pl)][lane 64] x 16 bytes, then per
-// weight row 48 bytes: m_0..7 as halves, 1024 m_0..7 as halves, d, dmin as floats, 8 unused.
-constexpr int QI_TILE = 4 * 2 * 64 * 16, QI_META = 48;
-template <int NG>
-constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * QI_META); }
+// weight row F::META bytes: the I2 operands of the lane groups (16 bytes each), d and dmin as floats in the
+// last 16.  With eight sub-blocks (48 bytes): m_0..7 as halves, 1024 m_0..7 as halves; with sixteen (80
+// bytes): m_0..7, m_8..15, 1024 m_0..7, 1024 m_8..15.
+constexpr int QI_TILE = 4 * 2 * 64 * 16;
+template <class F, int NG>
+constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * F::META); }
 
 typedef short qi_s2 __attribute__((ext_vector_type(2)));
 
@@ -137,8 +147,8 @@ typedef short qi_s2 __attribute__((ext_vector_type(2)));
 // Pl = L - 128; slice g of the chunk at tile + 256 g, plane Pl 1024 bytes further), meta() writes the
 // row's 48 bytes.
 struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 0..945
-    static constexpr int BLOCK = 144;
-    static constexpr bool HAS_MIN = true;
+    static constexpr int BLOCK = 144, META = 48, ALIGN = 16;
+    static constexpr bool HAS_MIN = true, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
         uint4 h;
     };
@@ -189,8 +199,8 @@ struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 
 // qh[32 h + e - 32] >> (4 jj + 2), nibble jj of ql, scales[8 h + 4 jj + e / 16].  Blocks of 210 bytes sit at
 // even addresses only: everything is read through aligned words.
 struct QiQ6K {
-    static constexpr int BLOCK = 210;
-    static constexpr bool HAS_MIN = false;
+    static constexpr int BLOCK = 210, META = 48, ALIGN = 2;
+    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
         uint32_t sc4, d;
     };
@@ -235,6 +245,117 @@ struct QiQ6K {
     }
 };
 
+// Q2_K: scales[16] (scale | min << 4) | qs[64] | d | dmin, w = d sc q - dmin m with q in 0..3 and 4-bit sc and m
+// over sub-blocks of 16 elements (src/kquant_dot.rs:63-76, 345-385): element 128 sg + 32 f + 16 hf + i is
+// field f of qs[32 sg + 16 hf + i] with the scale byte 8 sg + 2 f + hf.  p = sc q in 0..45 is a single signed
+// byte: Ph = 0, so HH and half of MID vanish and a chunk costs two MFMAs instead of four.  Chunk uc is
+// elements 64 uc ..: slice gg of 16 is sub-block 4 uc + gg, fields 2 (uc % 2) + gg / 2 of the 16 bytes
+// qs[32 (uc / 2) + 16 (gg % 2) ..].  The four products of a byte come out of a register table (0, sc, 2 sc,
+// 3 sc) with one v_perm_b32 per four elements.
+struct QiQ2K {
+    static constexpr int BLOCK = 84, META = 80, ALIGN = 4;
+    static constexpr bool HAS_MIN = true, ONE_PLANE = true, SUB16 = true;
+    struct Hdr {
+        uint32_t sc4, dd;
+    };
+    struct Raw {
+        Hdr hdr;
+        uint32_t table[4];  // per slice: sc * (0, 1, 2, 3) as bytes
+        uint4 q0, q1;
+    };
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        if (part == 0) next.sc4 = ld<uint32_t>(blk + 4 * uc), next.dd = ld<uint32_t>(blk + 80);
+        if (part == 1) raw.q0 = ld<uint4>(blk + 16 + 32 * (uc >> 1));
+        if (part == 2) raw.q1 = ld<uint4>(blk + 32 + 32 * (uc >> 1));
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) {
+        raw.hdr = next;
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) {
+            const uint32_t sc = (next.sc4 >> (8 * gg)) & 0xFu;
+            raw.table[gg] = (sc << 8) + (sc << 17) + ((sc + 2 * sc) << 24);
+        }
+    }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+        const int half = j >> 2, wi = j & 3;
+        const uint4 qv = half ? raw.q1 : raw.q0;
+        const uint32_t word = (wi == 0 ? qv.x : wi == 1 ? qv.y : wi == 2 ? qv.z : qv.w) >> (4 * (uc & 1));
+#pragma unroll
+        for (int e = 0; e < 2; e++) {  // slices half and 2 + half: the same bytes, the next field
+            const int gg = 2 * e + half;
+            const uint32_t q = (word >> (2 * e)) & 0x03030303u;
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(0u, raw.table[gg], q);
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        float mn[4];
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) mn[gg] = (float)((raw.hdr.sc4 >> (8 * gg + 4)) & 0xFu);
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const qi_h2 m1 = {(_Float16)mn[2 * e], (_Float16)mn[2 * e + 1]};
+            const qi_h2 m1k = {(_Float16)(1024.0f * mn[2 * e]), (_Float16)(1024.0f * mn[2 * e + 1])};
+            *(uint32_t *)(meta + 8 * uc + 4 * e) = __builtin_bit_cast(uint32_t, m1);
+            *(uint32_t *)(meta + 32 + 8 * uc + 4 * e) = __builtin_bit_cast(uint32_t, m1k);
+        }
+        *(float2 *)(meta + 64) = float2{f16_bits(raw.hdr.dd), f16_bits(raw.hdr.dd >> 16)};  // the same from all four
+    }
+};
+
+// Q8_0: blocks of d (f16) | 32 signed bytes, w = d q (src/kquant_dot.rs:37-46); a "super-block" here is eight
+// blocks, 272 bytes.  The scale of a block of 32 cannot ride in an integer operand exactly, so the eight
+// blocks are put on one scale D / 256, D the largest |d| among them: p = round(256 q d / D) in
+// -32512..32512, w ~ (D / 256) p.  That resolves every weight to 2^-16 of the largest magnitude its 256-run
+// can hold -- what the activations' fixed point does on their side -- and is exact where the eight scales are
+// equal.  Chunk uc is blocks 2 uc and 2 uc + 1; the four threads of a weight row are neighbouring lanes and
+// agree on D with two quad permutes.  Blocks sit at even addresses only: read through aligned words.
+struct QiQ8_0 {
+    static constexpr int BLOCK = 272, META = 48, ALIGN = 2;
+    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
+    struct Hdr {
+        float d0, d1;
+    };
+    struct Raw {
+        float r0, r1, unit;  // 256 d / D of the chunk's two blocks, and D / 256
+        uint4 qa[2], qb[2];  // halves of the quants of block 2 uc and of block 2 uc + 1
+    };
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        if (part == 0) next.d0 = f16_bits(ld<uint16_t>(blk + 68 * uc)), next.d1 = f16_bits(ld<uint16_t>(blk + 68 * uc + 34));
+        if (part == 1 || part == 2) {
+            raw.qa[part - 1] = ldw<uint4>(blk + 68 * uc + 2 + 16 * (part - 1));
+            raw.qb[part - 1] = ldw<uint4>(blk + 68 * uc + 36 + 16 * (part - 1));
+        }
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) {
+        float D = fmaxf(mag_or_inf(next.d0), mag_or_inf(next.d1));
+        D = fmaxf(D, dpp_f<0xB1>(D));  // quad_perm [1,0,3,2]
+        D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
+        const float inv = D > 0.0f ? 256.0f / D : 0.0f;
+        raw.r0 = next.d0 * inv, raw.r1 = next.d1 * inv, raw.unit = D * (1.0f / 256.0f);
+    }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+        const int half = j >> 2, wi = j & 3;
+#pragma unroll
+        for (int e32 = 0; e32 < 2; e32++) {
+            const uint4 qv = e32 ? raw.qb[half] : raw.qa[half];
+            const uint32_t word = wi == 0 ? qv.x : wi == 1 ? qv.y : wi == 2 ? qv.z : qv.w;
+            const float ratio = e32 ? raw.r1 : raw.r0;
+            // round(q ratio) + 128 in the low 16 bits of 1.5 * 2^23 + 128 + q ratio
+            uint32_t t[4];
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                t[b] = __builtin_bit_cast(uint32_t, fmaf((float)(int)(int8_t)(word >> (8 * b)), ratio, 12583040.0f));
+            const uint32_t even = __builtin_amdgcn_perm(t[2], t[0], 0x05040100u), odd = __builtin_amdgcn_perm(t[3], t[1], 0x05040100u);
+            const int gg = 2 * e32 + half;
+            *(uint32_t *)(tile + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+    }
+};
+
 // grid: 1-D; workgroup L takes tile (x, y) of tx x ty (weight-row tiles x activation-row tiles).  When ty
 // divides 8 the eight XCDs (L % 8) each work on one activation-row tile, whose operands then stay in that
 // XCD's L2; the grid is padded to a multiple of 8 and workgroups past the last tile leave at once.
@@ -245,7 +366,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                                                       int m_rows, int n, int nb, int groups, int tx, int ty,
                                                       int nb_total, size_t split_stride) {
     constexpr int NT = 16 * NG, THREADS = 64 * NW, UNITS = 4 * NT, PER = (UNITS + THREADS - 1) / THREADS;
-    constexpr int BUF = NG * QI_TILE + NT * QI_META;
+    constexpr int BUF = NG * QI_TILE + NT * F::META;
     extern __shared__ __attribute__((aligned(16))) uint8_t qi_lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
     int bx, by;
@@ -295,7 +416,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
 #pragma unroll
         for (int p = 0; p < PER; p++) {
             const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);
-            F::meta(raw[p], uc, buf + NG * QI_TILE + row * QI_META);
+            F::meta(raw[p], uc, buf + NG * QI_TILE + row * F::META);
         }
     };
     auto take_header = [&]() __attribute__((always_inline)) {
@@ -345,19 +466,22 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
             qm_i4 HH[NG], MID[NG], LL[NG];
             // the weight operands travel one step ahead of the MFMAs that use them, through two register sets
             qm_i4 Bh[2], Bl[2];
-            Bh[0] = *(const qm_i4 *)(buf + lane * 16), Bl[0] = *(const qm_i4 *)(buf + 1024 + lane * 16);
+            if constexpr (!F::ONE_PLANE) Bh[0] = *(const qm_i4 *)(buf + lane * 16);
+            Bl[0] = *(const qm_i4 *)(buf + 1024 + lane * 16);
             auto finish = [&](int cg) __attribute__((always_inline)) {  // the 16 x 16 results of weight-row group cg
-                const uint8_t *meta = buf + NG * QI_TILE + (16 * cg + r) * QI_META;
-                const float2 dd = *(const float2 *)(meta + 32);
+                const uint8_t *meta = buf + NG * QI_TILE + (16 * cg + r) * F::META;
+                const float2 dd = *(const float2 *)(meta + F::META - 16);
                 qm_f4 I2 = zero_f;
                 if constexpr (F::HAS_MIN) {
-                    // lane groups 2, 3 meet zeros in the activation operand: any finite halves will do for them
-                    const qi_h8 mB = *(const qi_h8 *)(meta + 16 * (g & 1));
+                    // eight sub-blocks: lane groups 2, 3 meet zeros in the activation operand, any finite halves
+                    // will do for them
+                    const qi_h8 mB = *(const qi_h8 *)(meta + 16 * (F::SUB16 ? g : g & 1));
                     I2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(minA, mB, zero_f, 0, 0, 0);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const float I1 = fmaf((float)(HH[cg][i] * 256 + MID[cg][i]), 256.0f, (float)LL[cg][i]);
+                    const float I1 = F::ONE_PLANE ? (float)(MID[cg][i] * 256 + LL[cg][i])
+                                                  : fmaf((float)(HH[cg][i] * 256 + MID[cg][i]), 256.0f, (float)LL[cg][i]);
                     if constexpr (F::HAS_MIN) acc[mg][cg][i] = fmaf(sx[i], dd.x * I1 - dd.y * I2[i], acc[mg][cg][i]);
                     else acc[mg][cg][i] = fmaf(sx[i], dd.x * I1, acc[mg][cg][i]);
                 }
@@ -381,14 +505,14 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                 if (c == 0) HH[cg] = zero_i, MID[cg] = zero_i, LL[cg] = zero_i;
                 if (s + 1 < STEPS) {
                     const int cg1 = step_cg(s + 1), c1 = step_c(s + 1);
-                    Bh[nxt] = *(const qm_i4 *)(buf + (4 * cg1 + c1) * 2048 + lane * 16);
+                    if constexpr (!F::ONE_PLANE) Bh[nxt] = *(const qm_i4 *)(buf + (4 * cg1 + c1) * 2048 + lane * 16);
                     Bl[nxt] = *(const qm_i4 *)(buf + (4 * cg1 + c1) * 2048 + 1024 + lane * 16);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 MID[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][0], Bl[cur], MID[cg], 0, 0, 0);
-                HH[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][0], Bh[cur], HH[cg], 0, 0, 0);
+                if constexpr (!F::ONE_PLANE) HH[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][0], Bh[cur], HH[cg], 0, 0, 0);
                 LL[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][1], Bl[cur], LL[cg], 0, 0, 0);
-                MID[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][1], Bh[cur], MID[cg], 0, 0, 0);
+                if constexpr (!F::ONE_PLANE) MID[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][1], Bh[cur], MID[cg], 0, 0, 0);
                 // one group behind the MFMAs, whose results it would otherwise wait for
                 if (c == 3 && !first_of_pass) finish(cg - 1);
                 if (last_of_pass && pass >= 4) {

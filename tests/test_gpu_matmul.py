@@ -230,6 +230,60 @@ def q6k_integer_case(n, k, seed, nonzero=24, random_scales=False, small=3000):
     return blocks, w, x
 
 
+def q2k_integer_case(n, k, seed, nonzero=16, min_blocks=3, small=400):
+    """Q2_K blocks with d = dmin = 1: `nonzero` 2-bit weights a row under random 4-bit scales of their
+    16-element sub-blocks, and `min_blocks` sub-blocks a row with a min of 1..15, so w = sc q - m in integers;
+    integer activations that peak at 32639 once per 256 elements (activation scale exactly 1 per super-block).
+    Returns (blocks, integer weights, activations)."""
+    rng = np.random.default_rng(seed)
+    q = np.zeros((n, k), np.int64)
+    for r in range(n):
+        q[r, rng.choice(k, size=nonzero, replace=False)] = rng.integers(1, 4, size=nonzero)
+    sc = rng.integers(0, 16, size=(n, k // 16))
+    mn = np.zeros((n, k // 16), np.int64)
+    for r in range(n):
+        mn[r, rng.choice(k // 16, size=min_blocks, replace=False)] = rng.integers(1, 16, size=min_blocks)
+    x = rng.integers(-small, small + 1, size=k).astype(np.int64)
+    peak = np.arange(0, k, 256) + int(rng.integers(0, 256))      # same slot in every super-block
+    x[peak] = 32639 * rng.choice([-1, 1], size=k // 256)
+    # element 128 sg + 32 f + 16 hf + i: field f of qs[32 sg + 16 hf + i], scale byte 8 sg + 2 f + hf
+    qq = q.reshape(n, k // 256, 2, 4, 2, 16)                    # [sg][f][hf][i]
+    qs = np.zeros((n, k // 256, 2, 2, 16), np.int64)             # [sg][hf][i]
+    for f in range(4):
+        qs |= qq[:, :, :, f, :, :] << (2 * f)
+    blocks = np.zeros((n, k // 256, 84), np.uint8)
+    blocks[:, :, 0:16] = (sc | (mn << 4)).reshape(n, k // 256, 16).astype(np.uint8)
+    blocks[:, :, 16:80] = qs.reshape(n, k // 256, 64).astype(np.uint8)
+    blocks[:, :, 80:82] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks[:, :, 82:84] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks = blocks.reshape(-1)
+    w = q * sc.repeat(16, axis=1) - mn.repeat(16, axis=1)
+    assert np.array_equal(oracle.dequantize(capi.Q2_K, blocks).reshape(n, k), w.astype(np.float32))
+    return blocks, w, x
+
+
+def q8_0_integer_case(n, k, seed, nonzero=16, small=400):
+    """Q8_0 blocks whose scales are powers of two between 1/4 and 2 and `nonzero` weights q in -127..127 a
+    row; integer activations that peak at 32639 once per 256 elements, where the weights are zero.  Returns
+    (blocks, the weights d q as float64, activations)."""
+    rng = np.random.default_rng(seed)
+    q = np.zeros((n, k), np.int64)
+    for r in range(n):
+        q[r, rng.choice(k, size=nonzero, replace=False)] = rng.integers(-127, 128, size=nonzero)
+    x = rng.integers(-small, small + 1, size=k).astype(np.int64)
+    peak = np.arange(0, k, 256) + int(rng.integers(0, 256))      # same slot in every super-block
+    x[peak] = 32639 * rng.choice([-1, 1], size=k // 256)
+    q[:, peak] = 0
+    d = rng.choice(np.array([0.25, 0.5, 1.0, 2.0]), size=(n, k // 32))
+    blocks = np.zeros((n, k // 32, 34), np.uint8)
+    blocks[:, :, 0:2] = d.astype(np.float16)[..., None].view(np.uint8)
+    blocks[:, :, 2:] = q.reshape(n, k // 32, 32).astype(np.int8).view(np.uint8)
+    blocks = blocks.reshape(-1)
+    w = q * d.repeat(32, axis=1)
+    assert np.array_equal(oracle.dequantize(capi.Q8_0, blocks).reshape(n, k), w.astype(np.float32))
+    return blocks, w, x
+
+
 def test_q6k_dot4_integer_dot_products_are_bit_exact():
     """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
     scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
@@ -294,8 +348,23 @@ def test_non_finite_activations_show_in_the_result(qtype, m, k, n):
             assert close(got[:m - 1], want[:m - 1])
 
 
-@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q6_K, 8, 12288, 1024), (capi.Q8_0, 16, 4096, 2100), (capi.MXFP4, 11, 7168, 1200),
-                                         (capi.Q6_K, 512, 4096, 1024), (capi.IQ2_XXS, 70, 5120, 300)])
+@pytest.mark.parametrize("qtype", [capi.Q6_K, capi.Q8_0, capi.Q2_K])
+@pytest.mark.parametrize("m,k,n", [(8, 12288, 1024), (16, 4096, 2100), (33, 4096, 2048 + 5), (48, 8192, 1100)])
+def test_few_rows_of_q6k_q8_0_q2k_against_a_large_matrix_take_the_int8_gemm(qtype, m, k, n):
+    """8 to 63 activation rows against 8M weights or more: the int8 GEMM split over k, most of its
+    activation-row tile empty; the partial sums are added in a fixed order (the same result on every call)."""
+    blocks = make_blocks(qtype, n, k, 310 + m)
+    lhs = synth.normal(311 + m, (m, k))
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    got = w.matmul_t(m, lhs)
+    name = {capi.Q6_K: "q6k", capi.Q8_0: "q8_0", capi.Q2_K: "q2k"}[qtype]
+    assert capi.last_kernel() == name + "_gemm_i8+splitk"
+    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
+    assert np.array_equal(got, w.matmul_t(m, lhs))
+
+
+@pytest.mark.parametrize("qtype,m,k,n", [(capi.IQ2_XXS, 8, 12288, 1024), (capi.MXFP4, 16, 4096, 2100), (capi.MXFP4, 11, 7168, 1200),
+                                         (capi.Q6_K, 512, 2048, 100), (capi.IQ2_XXS, 70, 5120, 300)])
 def test_decoded_weights_gemm_split_over_k(qtype, m, k, n):
     """8..16 rows against matrices of 8M elements or more, and many rows against few weight rows: the GEMM's
     tiles alone leave compute units idle, so runs of chunks go to workgroups of their own and the partial
@@ -305,6 +374,7 @@ def test_decoded_weights_gemm_split_over_k(qtype, m, k, n):
     w = capi.Weight.upload(qtype, blocks, n, k)
     got = w.matmul_t(m, lhs)
     assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
+    assert capi.last_kernel().startswith("gemm_decoded_mfma")
     assert np.array_equal(got, w.matmul_t(m, lhs))
 
 
@@ -793,6 +863,12 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q6_K, 64, 4096, 1024, "q6k_gemm_i8+splitk"),
     (capi.Q6_K, 64, 2048, 256, "gemm_decoded_mfma+splitk"), # a small product: weights decoded in the workgroup
     (capi.Q6_K, 512, 12288, 4096, "q6k_gemm_i8+splitk"),    # a feed-forward down projection in prefill: 74 tiles of 256 x 112, three splits
+    (capi.Q6_K, 32, 4096, 14336, "q6k_gemm_i8+splitk"),     # few rows against a large matrix
+    (capi.Q8_0, 512, 4096, 14336, "q8_0_gemm_i8"),
+    (capi.Q8_0, 16, 4096, 4096, "q8_0_gemm_i8+splitk"),
+    (capi.Q8_0, 32, 2048, 2048, "gemm_decoded_mfma+splitk"),# few rows against a small matrix
+    (capi.Q2_K, 512, 4096, 14336, "q2k_gemm_i8"),
+    (capi.Q2_K, 64, 12288, 4096, "q2k_gemm_i8+splitk"),
     (capi.Q2_K, 1, 7680, 2048, "matmul_rows_staged"),
     (capi.Q2_K, 1, 4096, 14336, "q2k_gemv_mfma_lds"),
     (capi.MXFP4, 1, 7168, 2048, "matmul_rows_staged"),
@@ -911,8 +987,9 @@ import sys, numpy as np
 sys.path.insert(0, %r)
 import oracle
 from joshua_amd import capi, synth
-from tests.test_gpu_matmul import q4k_integer_case, q6k_integer_case, close
-FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8")}[sys.argv[1]]
+from tests.test_gpu_matmul import q4k_integer_case, q6k_integer_case, q2k_integer_case, q8_0_integer_case, close
+FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8"), "q2k": (capi.Q2_K, "q2k_gemm_i8"),
+               "q8_0": (capi.Q8_0, "q8_0_gemm_i8")}[sys.argv[1]]
 # the same products split over k: the parts are summed in a fixed order
 if __import__("os").environ.get("JQ_Q4K_GEMM_I8_SPLITS", "1") != "1":
     for (m, k, n) in [(40, 4096, 100), (300, 4096, 130), (64, 12288, 70)]:
@@ -937,10 +1014,18 @@ for (m, k, n) in [(17, 256, 64), (33, 512, 100), (64, 1024, 300), (100, 1024, 25
 n, k, m = 160, 2048, 40
 if FMT == capi.Q4_K:
     blocks, q, x = q4k_integer_case(n, k, 23, group=32, big_value=32639, small=4000)
-else:  # every int8 scale value times q - 32, eight weights a row: sums below 2^24
+elif FMT == capi.Q6_K:  # every int8 scale value times q - 32, eight weights a row: sums below 2^24
     blocks, q, x = q6k_integer_case(n, k, 23, nonzero=8, random_scales=True, small=400)
-lhs = np.stack([np.roll(x, 32 * i) for i in range(m)])
+elif FMT == capi.Q2_K:  # 4-bit scales and mins over sub-blocks of 16
+    blocks, q, x = q2k_integer_case(n, k, 23)
+else:  # scales of 1/4 to 2 inside a run of 256: the common scale holds every weight exactly, the sum 256 q d / D
+    # against the activations stays below 2^24
+    blocks, q, x = q8_0_integer_case(n, k, 23)
+lhs = np.stack([np.roll(x, (256 if FMT in (capi.Q2_K, capi.Q8_0) else 32) * i) for i in range(m)])
 assert np.abs(lhs @ q.T).max() < 2 ** 24
+if FMT == capi.Q8_0:  # per run of 256, 1024 times the sum is still an integer that f32 holds
+    runs = np.einsum("mbe,nbe->mnb", lhs.reshape(m, -1, 256).astype(np.float64), q.reshape(n, -1, 256))
+    assert np.abs(runs).max() < 2 ** 19
 got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(m, lhs.astype(np.float32))
 assert capi.last_kernel() == KERNEL
 assert np.array_equal(got, (lhs @ q.T).astype(np.float32)), "integer case"
@@ -981,7 +1066,7 @@ print("gemm i8 ok")
 """
 
 
-@pytest.mark.parametrize("fmt", ["q4k", "q6k"])
+@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0"])
 @pytest.mark.parametrize("shape", ["8,7", "4,4"])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup

@@ -31,7 +31,9 @@ CASES = [  # (format, k, n, first m, second m): shapes whose kernels keep operan
     (capi.Q4_K, 4096, 1024, 96, 40),     # int8 and f16 GEMMs split over k: activation planes and partial sums
     (capi.Q6_K, 4096, 1024, 128, 64),    # Q6_K int8 GEMM split over k
     (capi.Q4_K, 1024, 512, 12, 3),       # streaming kernel (no scratch) and one row
-    (capi.Q6_K, 2048, 4096, 48, 9),      # GEMM over decoded weights, split over k
+    (capi.MXFP4, 2048, 4096, 48, 9),     # GEMM over decoded weights, split over k
+    (capi.Q8_0, 4096, 4096, 40, 9),      # Q8_0 int8 GEMM on few rows, split over k
+    (capi.Q2_K, 4096, 2048, 128, 20),    # Q2_K int8 GEMM
     (capi.Q8_0, 4096, 4096, 1, 1),       # one row: no scratch at all
 ]
 
