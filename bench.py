@@ -318,6 +318,10 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
             out["q4_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 12, N, K, 512, 102, max(steps // 10, 10), 4, 0.0)
         elif only == "q6k_m512":
             out["q6_k_4096x12288_m512"] = matmul_workload(torch, capi, synth, 14, 4096, 12288, 512, 109, max(steps // 10, 10), 4, 0.0)
+        elif only == "q8_0_m512":
+            out["q8_0_4096x4096_m512"] = matmul_workload(torch, capi, synth, 8, 4096, 4096, 512, 110, max(steps // 10, 10), 8, 0.0)
+        elif only == "q2k_m512":
+            out["q2_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 10, N, K, 512, 111, max(steps // 10, 10), 4, 0.0)
         elif only == "q2k":
             out["q2_k_gemv_14336x4096_m1"] = matmul_workload(torch, capi, synth, 10, N, K, 1, 108, steps, 24, 0.0)
         elif only == "moe_b1":
@@ -336,6 +340,8 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
     out["q6_k_gemv_4096x12288_m1"] = matmul_workload(torch, capi, synth, 14, 4096, 12288, 1, 106, steps, 12, cs)
     out["q6_k_4096x12288_m512"] = matmul_workload(torch, capi, synth, 14, 4096, 12288, 512, 109, max(steps // 10, 10), 4, cs)
     out["q2_k_gemv_14336x4096_m1"] = matmul_workload(torch, capi, synth, 10, N, K, 1, 108, steps, 24, cs)
+    out["q2_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 10, N, K, 512, 111, max(steps // 10, 10), 4, cs)
+    out["q8_0_4096x4096_m512"] = matmul_workload(torch, capi, synth, 8, 4096, 4096, 512, 110, max(steps // 10, 10), 8, cs)
     torch.cuda.empty_cache()
     out["moe_qwen3_30b_a3b_q4_k_b1"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 1, 104, steps, False, 0, cs)
     out["moe_qwen3_30b_a3b_q4_k_b64"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 64, 104, max(steps // 10, 10),
