@@ -778,7 +778,7 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
                                    X, (int)m, (int)k, acts);                                                          \
             hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)splits), dim3(64 * NW_), lds, s, W, row_bytes,    \
                                (const uint8_t *)acts, splits > 1 ? parts : Y, (int)m, (int)n, (int)(nb / splits),     \
-                               (int)groups, (int)tx, (int)ty, (int)nb, splits > 1 ? m * n : (size_t)0);               \
+                               (int)groups, (int)tx, (int)ty, (int)nb, splits > 1 ? m * n : (size_t)0, jq::QiGrouped{}); \
             if (splits > 1)                                                                                           \
                 hipLaunchKernelGGL(jq::splitk_sum, dim3((unsigned)((m * n + 1023) / 1024)), dim3(256), 0, s, parts, Y, \
                                    m * n, (int)splits);                                                               \
@@ -927,7 +927,7 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         const int rc = dispatch_gemm_i8<jq::QiQ4K>(W, row_bytes, X, Y, m, k, n, s, "q4k_gemm_i8", "q4k_gemm_i8+splitk");
         if (rc >= 0) return rc;
     }
-    // Q6_K, Q2_K, Q8_0: the same GEMM wherever the MFMA GEMM over decoded weights would run otherwise (from 17
+    // Q6_K, Q2_K, Q8_0, IQ2_XXS, MXFP4: the same GEMM wherever the MFMA GEMM over decoded weights would run otherwise (from 17
     // rows on, and from JQ_DECODED_GEMM_MIN_M rows on against matrices of 8M elements or more)
     static const char *dec_min_m_env = getenv("JQ_DECODED_GEMM_MIN_M");
     static const size_t gemm_min_m = dec_min_m_env ? (size_t)std::max(atoi(dec_min_m_env), 2) : 8;
@@ -942,6 +942,14 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     }
     if (type == JQ_TYPE_Q8_0 && many_rows) {
         const int rc = dispatch_gemm_i8<jq::QiQ8_0>(W, row_bytes, X, Y, m, k, n, s, "q8_0_gemm_i8", "q8_0_gemm_i8+splitk", false, 2);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_IQ2_XXS && many_rows) {
+        const int rc = dispatch_gemm_i8<jq::QiIQ2XXS>(W, row_bytes, X, Y, m, k, n, s, "iq2xxs_gemm_i8", "iq2xxs_gemm_i8+splitk", false, 2);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_MXFP4 && many_rows) {
+        const int rc = dispatch_gemm_i8<jq::QiMXFP4>(W, row_bytes, X, Y, m, k, n, s, "mxfp4_gemm_i8", "mxfp4_gemm_i8+splitk", false, 2);
         if (rc >= 0) return rc;
     }
     if (type == JQ_TYPE_Q4_K && m > Q4K_MFMA_MAX_M && row_bytes % 16 == 0 && ((uintptr_t)W & 15) == 0 &&
@@ -1292,6 +1300,9 @@ struct jq_moe {
     uint32_t *ids = nullptr;
     int *gexp = nullptr, *offsets = nullptr, *xrow = nullptr, *yrow = nullptr;
     uint8_t *qacts = nullptr;  // activations as MFMA operand records (Q4_K experts, grouped path)
+    uint8_t *gacts = nullptr;  // activations of the grouped int8 GEMM, and its tables
+    int *gtab = nullptr;
+    size_t gtab_rows = 0;      // row groups (and tiles) the tables hold
     jq::ActsI8 qi8{nullptr, nullptr, nullptr, nullptr};  // activations as int8 planes (decode path, long rows)
     std::mutex mu;
 };
@@ -1302,9 +1313,10 @@ void moe_free_scratch(jq_moe *m) {
     for (void *p : {(void *)m->logits, (void *)m->wts, (void *)m->G, (void *)m->U, (void *)m->out, (void *)m->sG,
                     (void *)m->sU, (void *)m->sH, (void *)m->sOut, (void *)m->ids, (void *)m->gexp,
                     (void *)m->offsets, (void *)m->xrow, (void *)m->yrow, (void *)m->qacts, (void *)m->qi8.xl,
-                    (void *)m->qi8.xh, (void *)m->qi8.sx, (void *)m->qi8.sxs})
+                    (void *)m->qi8.xh, (void *)m->qi8.sx, (void *)m->qi8.sxs, (void *)m->gacts, (void *)m->gtab})
         if (p) (void)hipFree(p);
     m->qacts = nullptr;
+    m->gacts = nullptr, m->gtab = nullptr, m->gtab_rows = 0;
     m->qi8 = jq::ActsI8{nullptr, nullptr, nullptr, nullptr};
     m->logits = m->wts = m->G = m->U = m->out = m->sG = m->sU = m->sH = m->sOut = nullptr;
     m->ids = nullptr;
@@ -1319,6 +1331,14 @@ bool moe_has_dot8(uint32_t type) {
     if (!env) return true;
     const std::string list = std::string(",") + env + ",";
     return list.find("," + std::to_string(type) + ",") != std::string::npos;
+}
+
+// Formats with a side of the int8 GEMM (kq_gemm_i8): their grouped expert matmuls run on it.
+bool moe_has_gemm_i8(uint32_t type) {
+    static const char *off = getenv("JQ_MOE_NO_GEMM_I8");
+    if (off) return false;
+    return type == JQ_TYPE_Q4_K || type == JQ_TYPE_Q6_K || type == JQ_TYPE_Q2_K || type == JQ_TYPE_Q8_0 ||
+           type == JQ_TYPE_IQ2_XXS || type == JQ_TYPE_MXFP4;
 }
 
 int moe_reserve(jq_moe *m, size_t T) {
@@ -1346,6 +1366,12 @@ int moe_reserve(jq_moe *m, size_t T) {
     }
     if (m->gate->type == JQ_TYPE_Q4_K || m->down->type == JQ_TYPE_Q4_K)
         HIP_TRY(hipMalloc((void **)&m->qacts, std::max(T * (c.hidden / 256), PR * (c.inter / 256)) * jq::QS_REC + 16));
+    if (P > c.n_expert && (moe_has_gemm_i8(m->gate->type) || moe_has_gemm_i8(m->down->type))) {
+        // row groups of 16 pairs that never mix two experts: at most PR / 16 + one part-filled group an expert
+        m->gtab_rows = PR / 16 + c.n_expert + 2;
+        HIP_TRY(hipMalloc((void **)&m->gacts, m->gtab_rows * (std::max<size_t>(c.hidden, c.inter) / 256 + 1) * jq::QI_REC));
+        HIP_TRY(hipMalloc((void **)&m->gtab, (5 * m->gtab_rows + 2) * sizeof(int)));
+    }
     if (m->sgate) {
         size_t si = m->sgate->n;
         HIP_TRY(hipMalloc((void **)&m->sG, T * si * sizeof(float)));
@@ -1604,6 +1630,59 @@ int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_byte
     return 0;
 }
 
+// One grouped expert matmul on the int8 GEMM: activation rows X[xsel[pair]] prepared into m->gacts (unless
+// `prepared`: the previous call left the same ones there) by the tables in m->gtab, results to Y[m->yrow[pair]].
+// Returns -1 when the matrix is outside its reach.
+jq::QiGroupTables moe_gemm_tables(const jq_moe *m) {
+    const size_t R = m->gtab_rows;
+    return jq::QiGroupTables{m->gtab, m->gtab + R, m->gtab + 2 * R, m->gtab + 3 * R, m->gtab + 4 * R, m->gtab + 5 * R};
+}
+
+template <class F>
+int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, int base_align, const float *X,
+                       const int *xsel, bool prepared, float *Y, int k, int n, hipStream_t s) {
+    if (!m->gacts || k % 256 != 0 || row_bytes % F::ALIGN != 0 || base_align < F::ALIGN) return -1;
+    constexpr int NW = 4, NG = 4;
+    const size_t nb = (size_t)k / 256, tx = ((size_t)n + 16 * NG - 1) / (16 * NG);
+    const size_t max_rg = m->gtab_rows, max_mt = m->gtab_rows;
+    if (tx * max_mt > 0x7FFFFFFFull) return -1;
+    const jq::QiGroupTables t = moe_gemm_tables(m);
+    if (!prepared)
+        hipLaunchKernelGGL((jq::moe_gemm_i8_prep<F::SUB16>), dim3((unsigned)nb, (unsigned)max_rg), dim3(256), 0, s, X, xsel, t, k,
+                           m->gacts);
+    auto kern = jq::kq_gemm_i8<F, NW, NG, true>;
+    constexpr int lds = jq::qi_lds_bytes<F, NG>();
+    static std::once_flag big_lds;
+    static hipError_t attr_rc = hipSuccess;
+    std::call_once(big_lds, [&] {
+        attr_rc = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    });
+    HIP_TRY(attr_rc);
+    note_kernel("moe_gemm_i8");
+    const jq::QiGrouped gp{wptr, m->gexp, m->yrow, t};
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tx * max_mt)), dim3(64 * NW), lds, s, (const uint8_t *)nullptr, row_bytes,
+                       (const uint8_t *)m->gacts, Y, 0, n, (int)nb, 0, (int)tx, 0, (int)nb, (size_t)0, gp);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, size_t row_bytes, int base_align,
+                         const float *X, const int *xsel, bool prepared, float *Y, int k, int n, hipStream_t s) {
+    if (!moe_has_gemm_i8(type)) return -1;
+    switch (type) {
+#define JQ_QI_CASE(ID, F) \
+    case ID: return launch_moe_gemm_i8<jq::F>(m, wptr, row_bytes, base_align, X, xsel, prepared, Y, k, n, s);
+        JQ_QI_CASE(JQ_TYPE_Q4_K, QiQ4K)
+        JQ_QI_CASE(JQ_TYPE_Q6_K, QiQ6K)
+        JQ_QI_CASE(JQ_TYPE_Q2_K, QiQ2K)
+        JQ_QI_CASE(JQ_TYPE_Q8_0, QiQ8_0)
+        JQ_QI_CASE(JQ_TYPE_IQ2_XXS, QiIQ2XXS)
+        JQ_QI_CASE(JQ_TYPE_MXFP4, QiMXFP4)
+#undef JQ_QI_CASE
+    default: return -1;
+    }
+}
+
 int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg) {
     const jq_moe_config &c = m->cfg;
     const unsigned token_runs = (unsigned)((T + jq::ROUTER_TOKENS_PER_WG - 1) / jq::ROUTER_TOKENS_PER_WG);
@@ -1682,6 +1761,27 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         rc = dispatch_moe_q4k_ring<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qacts, m->gexp, m->offsets,
                                          m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
     if (rc > 0) return 1;
+    // bucketed, any format with a side of the int8 GEMM: gate -> G and up -> U from one preparation of x, then
+    // the activation in place
+    bool planned = false;
+    if (rc < 0 && same_gu && max_group > 1 && m->gacts) {
+        hipLaunchKernelGGL(jq::moe_gemm_i8_plan, dim3(1), dim3(256), 0, s, m->offsets, groups, 8, moe_gemm_tables(m));
+        planned = true;
+        rc = dispatch_moe_gemm_i8(m, m->gate->type, m->pgate, m->gate->row_bytes, a16, x, m->xrow, false, m->G, (int)c.hidden,
+                                  (int)c.inter, s);
+        if (rc == 0) {
+            if (dispatch_moe_gemm_i8(m, m->up->type, m->pup, m->up->row_bytes, a16, x, m->xrow, true, m->U, (int)c.hidden,
+                                     (int)c.inter, s) != 0)
+                return fail("moe: the grouped GEMM took the gate projection and not the up projection");
+            const size_t routed = (size_t)P * c.inter, folded = (size_t)extra * T * c.inter;
+            hipLaunchKernelGGL(jq::swiglu_in_place, dim3((unsigned)std::min<size_t>((routed + 255) / 256, 4096)), dim3(256), 0,
+                               s, m->G, m->U, routed, c.swiglu_clamp);
+            if (folded)
+                hipLaunchKernelGGL(jq::swiglu_in_place, dim3((unsigned)std::min<size_t>((folded + 255) / 256, 4096)), dim3(256),
+                                   0, s, m->G + routed, m->U + routed, folded, c.swiglu_clamp_shared);
+        }
+    }
+    if (rc > 0) return 1;
     if (rc < 0 && same_gu && max_group <= 1)
         rc = dispatch_moe_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
                                      m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
@@ -1710,6 +1810,13 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);
+    if (rc > 0) return 1;
+    if (rc < 0 && fused_act && max_group > 1 && m->gacts) {
+        if (!planned)
+            hipLaunchKernelGGL(jq::moe_gemm_i8_plan, dim3(1), dim3(256), 0, s, m->offsets, groups, 8, moe_gemm_tables(m));
+        rc = dispatch_moe_gemm_i8(m, m->down->type, m->pdown, m->down->row_bytes, d16, m->G, m->yrow, false, m->out,
+                                  (int)c.inter, (int)c.hidden, s);
+    }
     if (rc > 0) return 1;
     // decode-sized, and no shared expert outside the pair list: down projection and combine in one launch
     if (rc < 0 && fused_act && max_group <= 1 && (m->fold_shared || !m->sgate)) {

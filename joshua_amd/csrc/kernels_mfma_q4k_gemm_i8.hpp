@@ -50,40 +50,15 @@ typedef _Float16 qi_h8 __attribute__((ext_vector_type(8)));
 // 16 rows.
 constexpr int QI_PLANES = 4 * 2 * 64 * 16, QI_MIN = QI_PLANES, QI_SCALE = QI_PLANES + 1024, QI_REC = QI_SCALE + 64;
 
-// grid (k / 256 super-blocks, groups of 16 activation rows), 256 threads: wave c, lane (i, g) quantises the
-// 16 elements 64 c + 16 g .. of row i.  Rows from m_rows on are zero operands.
-// With PAIRS the activations are silu(gate) * up over rows of 2 k floats in which gate_j and up_j alternate
-// (the result of a product with a row-paired gate|up matrix): the SwiGLU of a feed-forward block happens on the
-// way into the down projection.
+// The 16 elements v[] of a thread (wave c, lane (i, g): elements 64 c + 16 g .. of row i of the row group)
+// become the record `rec` of (row group, super-block).  256 threads.
 // With SUB16 the I2 operand is over the 16 sub-blocks of 16 elements (Q2_K): g = 0 holds a0 of sub-blocks
 // 0..7, g = 1 a0 of 8..15, g = 2 and 3 a1 of the same.
-template <bool PAIRS, bool SUB16 = false>
-__global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict__ X, int m_rows, int k,
-                                                         uint8_t *__restrict__ out) {
+template <bool SUB16>
+__device__ __forceinline__ void qi_prep_record(const float (&v)[16], uint8_t *__restrict__ rec) {
     __shared__ float amax_sh[4][16];
     __shared__ int xs_sh[16][SUB16 ? 16 : 8];
     const int tid = threadIdx.x, lane = tid & 63, c = tid >> 6, i = lane & 15, g = lane >> 4;
-    const int b = blockIdx.x, row = 16 * (int)blockIdx.y + i;
-    uint8_t *rec = out + ((size_t)blockIdx.y * gridDim.x + b) * QI_REC;
-    float v[16];
-    if (row < m_rows && PAIRS) {
-        const float4 *src = (const float4 *)(X + 2 * ((size_t)row * k + 256 * b + 64 * c + 16 * g));
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            const float4 a = src[q];
-            v[2 * q] = silu(a.x) * a.y, v[2 * q + 1] = silu(a.z) * a.w;
-        }
-    } else if (row < m_rows) {
-        const float4 *src = (const float4 *)(X + (size_t)row * k + 256 * b + 64 * c + 16 * g);
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const float4 a = src[q];
-            v[4 * q] = a.x, v[4 * q + 1] = a.y, v[4 * q + 2] = a.z, v[4 * q + 3] = a.w;
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < 16; e++) v[e] = 0.0f;
-    }
     float amax = 0.0f;
 #pragma unroll
     for (int e = 0; e < 16; e++) amax = fmaxf(amax, mag_or_inf(v[e]));
@@ -130,13 +105,122 @@ __global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict_
     if (tid < 16) ((float *)(rec + QI_SCALE))[tid] = s;
 }
 
+// grid (k / 256 super-blocks, groups of 16 activation rows), 256 threads.  Rows from m_rows on are zero
+// operands.
+// With PAIRS the activations are silu(gate) * up over rows of 2 k floats in which gate_j and up_j alternate
+// (the result of a product with a row-paired gate|up matrix): the SwiGLU of a feed-forward block happens on the
+// way into the down projection.
+template <bool PAIRS, bool SUB16 = false>
+__global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict__ X, int m_rows, int k,
+                                                         uint8_t *__restrict__ out) {
+    const int tid = threadIdx.x, lane = tid & 63, c = tid >> 6, i = lane & 15, g = lane >> 4;
+    const int b = blockIdx.x, row = 16 * (int)blockIdx.y + i;
+    uint8_t *rec = out + ((size_t)blockIdx.y * gridDim.x + b) * QI_REC;
+    float v[16];
+    if (row < m_rows && PAIRS) {
+        const float4 *src = (const float4 *)(X + 2 * ((size_t)row * k + 256 * b + 64 * c + 16 * g));
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const float4 a = src[q];
+            v[2 * q] = silu(a.x) * a.y, v[2 * q + 1] = silu(a.z) * a.w;
+        }
+    } else if (row < m_rows) {
+        const float4 *src = (const float4 *)(X + (size_t)row * k + 256 * b + 64 * c + 16 * g);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const float4 a = src[q];
+            v[4 * q] = a.x, v[4 * q + 1] = a.y, v[4 * q + 2] = a.z, v[4 * q + 3] = a.w;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; e++) v[e] = 0.0f;
+    }
+    qi_prep_record<SUB16>(v, rec);
+}
+
+// The grouped product (expert matmuls over (token, slot) pairs sorted by expert): pairs offsets[g] ..
+// offsets[g + 1] - 1 of group g are laid out in row groups of 16 that never mix two experts, and the row
+// groups of an expert in tiles of up to `tile_rgs` of them.  One workgroup of 256 threads writes the tables:
+//   rg_pair[r], rg_cnt[r]   first pair and number of pairs (1..16) of row group r
+//   mt_group[t], mt_rg0[t], mt_nrg[t]   group, first row group and number of row groups of tile t
+//   counts[0], counts[1]    row groups and tiles in all
+// for at most max_rg row groups and max_mt tiles (callers size them as pairs / 16 + groups and
+// pairs / (16 tile_rgs) + groups, which always suffice).
+struct QiGroupTables {
+    int *rg_pair, *rg_cnt, *mt_group, *mt_rg0, *mt_nrg, *counts;
+};
+__global__ __launch_bounds__(256) void moe_gemm_i8_plan(const int *__restrict__ offsets, int groups, int tile_rgs,
+                                                         QiGroupTables t) {
+    __shared__ int rg_base[257], mt_base[257];
+    // serial prefix over the groups in chunks of 256 (a few hundred groups at most)
+    __shared__ int carry[2];
+    if (threadIdx.x == 0) carry[0] = carry[1] = 0;
+    __syncthreads();
+    for (int g0 = 0; g0 < groups; g0 += 256) {
+        const int g = g0 + (int)threadIdx.x;
+        const int cnt = g < groups ? offsets[g + 1] - offsets[g] : 0;
+        const int nrg = (cnt + 15) >> 4, nmt = (nrg + tile_rgs - 1) / tile_rgs;
+        rg_base[threadIdx.x] = nrg, mt_base[threadIdx.x] = nmt;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int a = carry[0], b = carry[1];
+            for (int i = 0; i < 256; i++) {
+                const int x = rg_base[i], y = mt_base[i];
+                rg_base[i] = a, mt_base[i] = b;
+                a += x, b += y;
+            }
+            carry[0] = a, carry[1] = b;
+        }
+        __syncthreads();
+        if (g < groups) {
+            const int first = offsets[g];
+            for (int r = 0; r < nrg; r++) {
+                t.rg_pair[rg_base[threadIdx.x] + r] = first + 16 * r;
+                t.rg_cnt[rg_base[threadIdx.x] + r] = min(16, cnt - 16 * r);
+            }
+            for (int q = 0; q < nmt; q++) {
+                t.mt_group[mt_base[threadIdx.x] + q] = g;
+                t.mt_rg0[mt_base[threadIdx.x] + q] = rg_base[threadIdx.x] + tile_rgs * q;
+                t.mt_nrg[mt_base[threadIdx.x] + q] = min(tile_rgs, nrg - tile_rgs * q);
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) t.counts[0] = carry[0], t.counts[1] = carry[1];
+}
+
+// Prepared activations of the grouped product: grid (k / 256, max row groups); row i of row group r is
+// X[xsel[rg_pair[r] + i]] (rows past rg_cnt[r] are zero operands; workgroups past counts[0] leave).
+template <bool SUB16>
+__global__ __launch_bounds__(256) void moe_gemm_i8_prep(const float *__restrict__ X, const int *__restrict__ xsel,
+                                                         QiGroupTables t, int k, uint8_t *__restrict__ out) {
+    const int r = (int)blockIdx.y;
+    if (r >= t.counts[0]) return;
+    const int tid = threadIdx.x, lane = tid & 63, c = tid >> 6, i = lane & 15, g = lane >> 4;
+    const int b = blockIdx.x;
+    uint8_t *rec = out + ((size_t)r * gridDim.x + b) * QI_REC;
+    float v[16];
+    if (i < t.rg_cnt[r]) {
+        const float4 *src = (const float4 *)(X + (size_t)xsel[t.rg_pair[r] + i] * k + 256 * b + 64 * c + 16 * g);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const float4 a = src[q];
+            v[4 * q] = a.x, v[4 * q + 1] = a.y, v[4 * q + 2] = a.z, v[4 * q + 3] = a.w;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; e++) v[e] = 0.0f;
+    }
+    qi_prep_record<SUB16>(v, rec);
+}
+
 // LDS per buffer: NG tiles of 16 weight rows x [chunk 4][plane 2 (Ph, Pl)][lane 64] x 16 bytes, then per
 // weight row F::META bytes: the I2 operands of the lane groups (16 bytes each), d and dmin as floats in the
 // last 16.  With eight sub-blocks (48 bytes): m_0..7 as halves, 1024 m_0..7 as halves; with sixteen (80
 // bytes): m_0..7, m_8..15, 1024 m_0..7, 1024 m_8..15.
 constexpr int QI_TILE = 4 * 2 * 64 * 16;
 template <class F, int NG>
-constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * F::META); }
+constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * F::META) + F::TABLE; }
 
 typedef short qi_s2 __attribute__((ext_vector_type(2)));
 
@@ -147,7 +231,7 @@ typedef short qi_s2 __attribute__((ext_vector_type(2)));
 // Pl = L - 128; slice g of the chunk at tile + 256 g, plane Pl 1024 bytes further), meta() writes the
 // row's 48 bytes.
 struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 0..945
-    static constexpr int BLOCK = 144, META = 48, ALIGN = 16;
+    static constexpr int BLOCK = 144, META = 48, ALIGN = 16, TABLE = 0;
     static constexpr bool HAS_MIN = true, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
         uint4 h;
@@ -161,8 +245,8 @@ struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 
         if (part == 1) raw.q0 = *(const uint4 *)(blk + 16 + 32 * uc);
         if (part == 2) raw.q1 = *(const uint4 *)(blk + 32 + 32 * uc);
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) { raw.hdr = next; }
-    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) { raw.hdr = next; }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
         const uint4 hdr = raw.hdr.h;
         const uint32_t scl = hdr.y & 0x3F3F3F3Fu, sch = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
         const uint32_t s4 = (uc < 2 ? scl : sch) >> (16 * (uc & 1));
@@ -199,7 +283,7 @@ struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 
 // qh[32 h + e - 32] >> (4 jj + 2), nibble jj of ql, scales[8 h + 4 jj + e / 16].  Blocks of 210 bytes sit at
 // even addresses only: everything is read through aligned words.
 struct QiQ6K {
-    static constexpr int BLOCK = 210, META = 48, ALIGN = 2;
+    static constexpr int BLOCK = 210, META = 48, ALIGN = 2, TABLE = 0;
     static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
         uint32_t sc4, d;
@@ -218,11 +302,11 @@ struct QiQ6K {
             raw.hv[part - 1] = ldw<uint4>(blk + 128 + 32 * h + o);
         }
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) { raw.hdr = next; }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) { raw.hdr = next; }
     __device__ __forceinline__ static uint32_t word_of(const uint4 &v, int i) {
         return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
     }
-    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
         const int sh = 4 * (uc & 1), half = j >> 2, wi = j & 3;
         const uint32_t qh = word_of(raw.hv[half], wi) >> sh;
         const uint32_t lo[2] = {word_of(raw.la[half], wi) >> sh, word_of(raw.lb[half], wi) >> sh};
@@ -253,7 +337,7 @@ struct QiQ6K {
 // qs[32 (uc / 2) + 16 (gg % 2) ..].  The four products of a byte come out of a register table (0, sc, 2 sc,
 // 3 sc) with one v_perm_b32 per four elements.
 struct QiQ2K {
-    static constexpr int BLOCK = 84, META = 80, ALIGN = 4;
+    static constexpr int BLOCK = 84, META = 80, ALIGN = 4, TABLE = 0;
     static constexpr bool HAS_MIN = true, ONE_PLANE = true, SUB16 = true;
     struct Hdr {
         uint32_t sc4, dd;
@@ -268,7 +352,7 @@ struct QiQ2K {
         if (part == 1) raw.q0 = ld<uint4>(blk + 16 + 32 * (uc >> 1));
         if (part == 2) raw.q1 = ld<uint4>(blk + 32 + 32 * (uc >> 1));
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) {
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
         raw.hdr = next;
 #pragma unroll
         for (int gg = 0; gg < 4; gg++) {
@@ -276,7 +360,7 @@ struct QiQ2K {
             raw.table[gg] = (sc << 8) + (sc << 17) + ((sc + 2 * sc) << 24);
         }
     }
-    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
         const int half = j >> 2, wi = j & 3;
         const uint4 qv = half ? raw.q1 : raw.q0;
         const uint32_t word = (wi == 0 ? qv.x : wi == 1 ? qv.y : wi == 2 ? qv.z : qv.w) >> (4 * (uc & 1));
@@ -310,7 +394,7 @@ struct QiQ2K {
 // equal.  Chunk uc is blocks 2 uc and 2 uc + 1; the four threads of a weight row are neighbouring lanes and
 // agree on D with two quad permutes.  Blocks sit at even addresses only: read through aligned words.
 struct QiQ8_0 {
-    static constexpr int BLOCK = 272, META = 48, ALIGN = 2;
+    static constexpr int BLOCK = 272, META = 48, ALIGN = 2, TABLE = 0;
     static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
         float d0, d1;
@@ -326,14 +410,14 @@ struct QiQ8_0 {
             raw.qb[part - 1] = ldw<uint4>(blk + 68 * uc + 36 + 16 * (part - 1));
         }
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next) {
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
         float D = fmaxf(mag_or_inf(next.d0), mag_or_inf(next.d1));
         D = fmaxf(D, dpp_f<0xB1>(D));  // quad_perm [1,0,3,2]
         D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
         const float inv = D > 0.0f ? 256.0f / D : 0.0f;
         raw.r0 = next.d0 * inv, raw.r1 = next.d1 * inv, raw.unit = D * (1.0f / 256.0f);
     }
-    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile) {
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
         const int half = j >> 2, wi = j & 3;
 #pragma unroll
         for (int e32 = 0; e32 < 2; e32++) {
@@ -356,39 +440,209 @@ struct QiQ8_0 {
     }
 };
 
+// IQ2_XXS: d (f16) | 8 groups of (4 codebook indices, 4 x 7 sign bits + a 4-bit scale), w = d (2 s + 1) / 8 *
+// (+-grid value), grid values 8, 25 and 43 (src/iq2xxs.rs:34-71, 349-380): p = +-(2 s + 1) grid in
+// -1333..1333 is exact in two bytes, the scale of a super-block is d / 8 and there is no min term.  Chunk uc is
+// groups 2 uc and 2 uc + 1.  The codebook sits in LDS behind the operand buffers (a read from global memory
+// in the unpacking would wait for the weight bytes asked for ahead of it); grid value v is number v >> 4 of
+// the three, so per group six products (three magnitudes, two signs) make two 8-byte tables a plane and one
+// v_perm_b32 a plane looks four elements up with the selector (v >> 4) | sign << 2.  Blocks of 66 bytes sit
+// at even addresses only: read through aligned words.
+struct QiIQ2XXS {
+    static constexpr int BLOCK = 66, META = 48, ALIGN = 2, TABLE = 2048;
+    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
+    struct Hdr {
+        uint32_t d;
+    };
+    struct Raw {
+        float unit;
+        uint32_t lo[2], signs[2];        // per group: the four codes; the four sign bytes (parity bit restored)
+        uint32_t th[2][2], tl[2][2];     // per group: Ph and Pl of +p_0..2 (word 0) and -p_0..2 (word 1)
+        uint4 q;                         // the bytes of the next super-block's chunk
+    };
+    __device__ __forceinline__ static void stage(uint8_t *lds) {
+        for (int i = threadIdx.x; i < 256; i += blockDim.x) ((uint64_t *)lds)[i] = g_tables.iq2xxs_grid[i];
+    }
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        if (part == 0) next.d = ld<uint16_t>(blk);
+        if (part == 2) raw.q = ldw<uint4>(blk + 2 + 16 * uc);
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
+        raw.unit = f16_bits(next.d) * 0.125f;
+        const uint32_t w[4] = {raw.q.x, raw.q.y, raw.q.z, raw.q.w};
+#pragma unroll
+        for (int grp = 0; grp < 2; grp++) {
+            const uint32_t hi = w[2 * grp + 1];
+            raw.lo[grp] = w[2 * grp];
+            uint32_t signs = 0;
+#pragma unroll
+            for (int l = 0; l < 4; l++) {
+                const uint32_t s7 = (hi >> (7 * l)) & 127u;
+                signs |= (s7 | ((__popc(s7) & 1u) << 7)) << (8 * l);
+            }
+            raw.signs[grp] = signs;
+            const int sc = 2 * (int)(hi >> 28) + 1;
+            uint32_t th[2] = {0, 0}, tl[2] = {0, 0};
+#pragma unroll
+            for (int i = 0; i < 3; i++) {
+                const int p = sc * (i == 0 ? 8 : i == 1 ? 25 : 43);
+#pragma unroll
+                for (int neg = 0; neg < 2; neg++) {
+                    const int v = (neg ? -p : p) + 128;  // 256 Ph + L
+                    th[neg] |= (uint32_t)((v >> 8) & 255) << (8 * i);
+                    tl[neg] |= (uint32_t)((v & 255) ^ 128) << (8 * i);
+                }
+            }
+            raw.th[grp][0] = th[0], raw.th[grp][1] = th[1], raw.tl[grp][0] = tl[0], raw.tl[grp][1] = tl[1];
+        }
+    }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *tab) {
+        const int half = j >> 2, wi = j & 3, l = 2 * half + (wi >> 1), hf = wi & 1;
+#pragma unroll
+        for (int grp = 0; grp < 2; grp++) {  // elements 16 half + 4 wi .. + 3 of both groups
+            const uint32_t code = (raw.lo[grp] >> (8 * l)) & 0xFFu;
+            const uint32_t mag = *(const uint32_t *)(tab + 8 * code + 4 * hf);
+            const uint32_t nib = (raw.signs[grp] >> (8 * l + 4 * hf)) & 15u;
+            const uint32_t sel = ((mag >> 4) & 0x03030303u) | (((nib * 0x00204081u) & 0x01010101u) << 2);
+            const int gg = 2 * grp + half;
+            *(uint32_t *)(tile + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(raw.th[grp][1], raw.th[grp][0], sel);
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(raw.tl[grp][1], raw.tl[grp][0], sel);
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+    }
+};
+
+// MXFP4: blocks of e (E8M0) | 16 bytes of E2M1 codes, w = 2^(e - 127) * +-{0, .5, 1, 1.5, 2, 3, 4, 6}, low
+// nibbles elements 0..15, high nibbles 16..31, e = 255 a block of zeros (src/mxfp4.rs:45-94); a "super-block"
+// here is eight blocks, 136 bytes.  As for Q8_0 the eight blocks are put on one scale: with D the largest
+// 2^(e - 127) among them, p = round(4096 w / D) in -24576..24576 -- exact for every block within eleven
+// octaves of the largest, rounded to 2^-12 of the largest element below that.  Per block the eight
+// magnitudes times two signs make two 8-byte tables a plane and sign: four v_perm_b32 and two bit selects
+// for four elements.  Blocks sit at any byte: read through aligned words.  Runs whose largest scale is below
+// 2^-100 count as zeros.
+struct QiMXFP4 {
+    static constexpr int BLOCK = 136, META = 48, ALIGN = 1, TABLE = 0;
+    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
+    struct Hdr {
+        float d0, d1;
+    };
+    struct Raw {
+        float unit;
+        uint32_t th[2][4], tl[2][4];  // per block: Ph / Pl of +p_0..7 (words 0, 1) and of -p_0..7 (words 2, 3)
+        uint4 qa, qb;                 // the codes of block 2 uc and of block 2 uc + 1
+        uint4 na, nb;                 // the same of the next super-block
+    };
+    __device__ __forceinline__ static float scale_of(uint32_t e) {
+        return e == 0xFFu ? 0.0f : __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
+    }
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        if (part == 0) next.d0 = scale_of(blk[34 * uc]), next.d1 = scale_of(blk[34 * uc + 17]);
+        if (part == 1) raw.na = ldw<uint4>(blk + 34 * uc + 1);
+        if (part == 2) raw.nb = ldw<uint4>(blk + 34 * uc + 18);
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
+        float D = fmaxf(next.d0, next.d1);
+        D = fmaxf(D, dpp_f<0xB1>(D));  // quad_perm [1,0,3,2]
+        D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
+        const bool live = D >= 7.888609052210118e-31f;  // 2^-100
+        const float inv = live ? 2048.0f / D : 0.0f;    // doubled magnitudes: 4096 w / D = (2 |w| / d) * 2048 d / D
+        raw.unit = live ? D * (1.0f / 4096.0f) : 0.0f;
+        raw.qa = raw.na, raw.qb = raw.nb;
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {
+            const float ratio = (blk ? next.d1 : next.d0) * inv;
+            uint32_t t[2][8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {  // round(+-v ratio) + 128 in the low 16 bits of 1.5 * 2^23 + 128 +- v ratio
+                const float v = (float)(i < 5 ? i : i == 5 ? 6 : i == 6 ? 8 : 12);
+                t[0][i] = __builtin_bit_cast(uint32_t, fmaf(v, ratio, 12583040.0f));
+                t[1][i] = __builtin_bit_cast(uint32_t, fmaf(-v, ratio, 12583040.0f));
+            }
+#pragma unroll
+            for (int sgn = 0; sgn < 2; sgn++)
+#pragma unroll
+                for (int h4 = 0; h4 < 2; h4++) {
+                    const uint32_t *q = &t[sgn][4 * h4];
+                    const uint32_t a = __builtin_amdgcn_perm(q[1], q[0], 0x05010400u);  // L0 L1 H0 H1
+                    const uint32_t b = __builtin_amdgcn_perm(q[3], q[2], 0x05010400u);  // L2 L3 H2 H3
+                    raw.tl[blk][2 * sgn + h4] = __builtin_amdgcn_perm(b, a, 0x05040100u) ^ 0x80808080u;
+                    raw.th[blk][2 * sgn + h4] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+                }
+        }
+    }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
+        const int half = j >> 2, wi = j & 3;
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {  // elements 16 half + 4 wi .. + 3 of both blocks
+            const uint4 qv = blk ? raw.qb : raw.qa;
+            const uint32_t word = (wi == 0 ? qv.x : wi == 1 ? qv.y : wi == 2 ? qv.z : qv.w) >> (4 * half);
+            const uint32_t sel = word & 0x07070707u, neg = ((word >> 3) & 0x01010101u) * 0xFFu;
+            const uint32_t ph = __builtin_amdgcn_perm(raw.th[blk][1], raw.th[blk][0], sel);
+            const uint32_t nh = __builtin_amdgcn_perm(raw.th[blk][3], raw.th[blk][2], sel);
+            const uint32_t pl = __builtin_amdgcn_perm(raw.tl[blk][1], raw.tl[blk][0], sel);
+            const uint32_t nl = __builtin_amdgcn_perm(raw.tl[blk][3], raw.tl[blk][2], sel);
+            const int gg = 2 * blk + half;
+            *(uint32_t *)(tile + gg * 256 + 4 * wi) = (nh & neg) | (ph & ~neg);
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = (nl & neg) | (pl & ~neg);
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+    }
+};
+
 // grid: 1-D; workgroup L takes tile (x, y) of tx x ty (weight-row tiles x activation-row tiles).  When ty
 // divides 8 the eight XCDs (L % 8) each work on one activation-row tile, whose operands then stay in that
 // XCD's L2; the grid is padded to a multiple of 8 and workgroups past the last tile leave at once.
 // gridDim.y > 1 splits the product over k.
-template <class F, int NW, int NG>
+// GROUPED: the expert matmuls of a mixture-of-experts layer over pairs sorted by expert (tables of
+// moe_gemm_i8_plan, activations of moe_gemm_i8_prep).  Workgroup L takes weight-row tile L % tx of activation
+// tile L / tx (workgroups past the last tile leave at once): the weights are those of the tile's expert,
+// gp.wptr[gp.gexp[group]], row i of the tile's row group j is pair rg_pair + i, stored at Y[gp.yrow[pair]].
+// W, m_rows, groups, ty and the split arguments are unused.
+struct QiGrouped {
+    const uint8_t *const *wptr;
+    const int *gexp, *yrow;
+    QiGroupTables t;
+};
+template <class F, int NW, int NG, bool GROUPED = false>
 __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict__ W, size_t row_bytes,
                                                       const uint8_t *__restrict__ acts, float *__restrict__ Y,
                                                       int m_rows, int n, int nb, int groups, int tx, int ty,
-                                                      int nb_total, size_t split_stride) {
+                                                      int nb_total, size_t split_stride, QiGrouped gp = QiGrouped{}) {
     constexpr int NT = 16 * NG, THREADS = 64 * NW, UNITS = 4 * NT, PER = (UNITS + THREADS - 1) / THREADS;
     constexpr int BUF = NG * QI_TILE + NT * F::META;
     extern __shared__ __attribute__((aligned(16))) uint8_t qi_lds[];
+    const uint8_t *tab = qi_lds + 2 * BUF;  // the format's lookup table, behind the two buffers
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
     int bx, by;
-    if (8 % ty == 0) {
+    int rg0 = 0, nrg = 0;  // GROUPED: the tile's first row group and how many it has
+    if (GROUPED) {
+        by = (int)blockIdx.x / tx, bx = (int)blockIdx.x % tx;
+        if (by >= gp.t.counts[1]) return;
+        rg0 = gp.t.mt_rg0[by], nrg = gp.t.mt_nrg[by];
+        W = gp.wptr[gp.gexp[gp.t.mt_group[by]]];
+    } else if (8 % ty == 0) {
         const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
         by = xcd % ty, bx = slot * (8 / ty) + xcd / ty;
     } else {
         by = (int)blockIdx.x / tx, bx = (int)blockIdx.x % tx;
     }
-    if (bx >= tx || by >= ty) return;
+    if (bx >= tx || (!GROUPED && by >= ty)) return;
     const int n0 = bx * NT, m0 = by * 32 * NW;
     // split over k: workgroups blockIdx.y = i take super-blocks i nb .. (i + 1) nb - 1 of the nb_total and store
     // their sums at Y + i split_stride (splitk_sum adds the parts in a fixed order)
-    const int b_first = (int)blockIdx.y * nb;
-    Y += (size_t)blockIdx.y * split_stride;
+    const int b_first = GROUPED ? 0 : (int)blockIdx.y * nb;
+    if (!GROUPED) Y += (size_t)blockIdx.y * split_stride;
 
     // activation operands of this wave: row groups 2 wave, 2 wave + 1 of the tile (clamped: rows past m_rows
     // are computed and not stored)
     const uint8_t *arec[2];
 #pragma unroll
     for (int mg = 0; mg < 2; mg++)
-        arec[mg] = acts + ((size_t)min(m0 / 16 + 2 * wave + mg, groups - 1) * nb_total + b_first) * QI_REC;
+        arec[mg] = acts + ((size_t)(GROUPED ? rg0 + min(2 * wave + mg, nrg - 1) : min(m0 / 16 + 2 * wave + mg, groups - 1)) * nb_total + b_first) * QI_REC;
 
     // unpack units of this thread: chunk c = tid % 4 of weight rows tid / 4 + (THREADS / 4) p
     const int uc = tid & 3;
@@ -409,7 +663,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
 #pragma unroll
         for (int p = 0; p < PER; p++) {
             const int row = min((tid >> 2) + (THREADS / 4) * p, NT - 1);  // threads past the last unit repeat it
-            F::piece(raw[p], uc, j, buf + (row >> 4) * QI_TILE + uc * 2048 + (row & 15) * 16);
+            F::piece(raw[p], uc, j, buf + (row >> 4) * QI_TILE + uc * 2048 + (row & 15) * 16, tab);
         }
     };
     auto unpack_meta = [&](uint8_t *buf) __attribute__((always_inline)) {  // the row's scales of the min term, d and dmin
@@ -421,10 +675,14 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
     };
     auto take_header = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int p = 0; p < PER; p++) F::take(raw[p], hdr_next[p]);
+        for (int p = 0; p < PER; p++) F::take(raw[p], hdr_next[p], tab);
     };
 
     fetch_part(0, 0), fetch_part(0, 1), fetch_part(0, 2);
+    if constexpr (F::TABLE > 0) {  // every workgroup that got this far: no wave has left
+        F::stage(qi_lds + 2 * BUF);
+        __syncthreads();
+    }
     take_header();
 #pragma unroll
     for (int j = 0; j < 8; j++) unpack_piece(qi_lds, j);
@@ -534,10 +792,17 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
     }
 #pragma unroll
     for (int mg = 0; mg < 2; mg++) {
+        int first_pair = 0, pairs = 0;
+        if (GROUPED && 2 * wave + mg < nrg) first_pair = gp.t.rg_pair[rg0 + 2 * wave + mg], pairs = gp.t.rg_cnt[rg0 + 2 * wave + mg];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int row = m0 + 32 * wave + 16 * mg + 4 * g + i;
-            if (row >= m_rows) continue;
+            int row = m0 + 32 * wave + 16 * mg + 4 * g + i;
+            if (GROUPED) {
+                if (4 * g + i >= pairs) continue;
+                row = gp.yrow[first_pair + 4 * g + i];
+            } else if (row >= m_rows) {
+                continue;
+            }
 #pragma unroll
             for (int cg = 0; cg < NG; cg++) {
                 const int col = n0 + 16 * cg + r;

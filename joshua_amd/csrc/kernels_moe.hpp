@@ -882,4 +882,11 @@ __global__ __launch_bounds__(256) void swiglu_rows(const float *__restrict__ g, 
         h[i] = swiglu(g[i], u[i], limit);
 }
 
+// g[i] = silu(g[i]) * u[i] in place (gate and up results of the grouped GEMM, in front of the down projection)
+__global__ __launch_bounds__(256) void swiglu_in_place(float *__restrict__ g, const float *__restrict__ u, size_t total,
+                                                        float limit) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+        g[i] = swiglu(g[i], u[i], limit);
+}
+
 }  // namespace jq

@@ -284,6 +284,39 @@ def q8_0_integer_case(n, k, seed, nonzero=16, small=400):
     return blocks, w, x
 
 
+def iq2xxs_integer_case(n, k, seed):
+    """IQ2_XXS blocks of random codes, signs and scales with d = 8, so w = +-(2 s + 1) grid in integers (scale 0
+    in the group that holds the activations' peak); activations in multiples of 2^-8: -1, 0 or 1 of them, and
+    32639 of them at one slot of every 256 (activation scale exactly 2^-8 per super-block).  Returns (blocks,
+    weights, activations as float64)."""
+    rng = np.random.default_rng(seed)
+    slot = int(rng.integers(0, 256))
+    blocks = rng.integers(0, 256, size=(n, k // 256, 66), dtype=np.uint8)
+    blocks[:, :, 0:2] = np.frombuffer(np.float16(8.0).tobytes(), np.uint8)
+    blocks[:, :, 2 + 8 * (slot // 32) + 7] &= 0x0F           # the top nibble of the group's second word is its scale
+    blocks = blocks.reshape(-1)
+    w = oracle.dequantize(capi.IQ2_XXS, blocks).reshape(n, k).astype(np.float64)
+    assert np.array_equal(w, np.round(w)) and np.abs(w).max() <= 1333 and np.abs(w[:, slot::256]).max() <= 43
+    x = rng.integers(-1, 2, size=k).astype(np.float64)
+    x[slot::256] = 32639 * rng.choice([-1, 1], size=k // 256)
+    return blocks, w, x / 256.0
+
+
+def mxfp4_integer_case(n, k, seed):
+    """MXFP4 blocks of random codes with scales 1/4 to 1; activations in multiples of 2^-8: -2..2 of them, and
+    32639 of them at one slot of every 256.  Returns (blocks, weights, activations as float64)."""
+    rng = np.random.default_rng(seed)
+    slot = int(rng.integers(0, 256))
+    blocks = rng.integers(0, 256, size=(n, k // 32, 17), dtype=np.uint8)
+    blocks[:, :, 0] = rng.integers(125, 128, size=(n, k // 32))
+    blocks = blocks.reshape(-1)
+    w = oracle.dequantize(capi.MXFP4, blocks).reshape(n, k).astype(np.float64)
+    assert np.array_equal(8 * w, np.round(8 * w)) and np.abs(w).max() <= 6
+    x = rng.integers(-2, 3, size=k).astype(np.float64)
+    x[slot::256] = 32639 * rng.choice([-1, 1], size=k // 256)
+    return blocks, w, x / 256.0
+
+
 def test_q6k_dot4_integer_dot_products_are_bit_exact():
     """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
     scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
@@ -348,32 +381,32 @@ def test_non_finite_activations_show_in_the_result(qtype, m, k, n):
             assert close(got[:m - 1], want[:m - 1])
 
 
-@pytest.mark.parametrize("qtype", [capi.Q6_K, capi.Q8_0, capi.Q2_K])
+@pytest.mark.parametrize("qtype", [capi.Q6_K, capi.Q8_0, capi.Q2_K, capi.IQ2_XXS, capi.MXFP4])
 @pytest.mark.parametrize("m,k,n", [(8, 12288, 1024), (16, 4096, 2100), (33, 4096, 2048 + 5), (48, 8192, 1100)])
-def test_few_rows_of_q6k_q8_0_q2k_against_a_large_matrix_take_the_int8_gemm(qtype, m, k, n):
+def test_few_rows_against_a_large_matrix_take_the_int8_gemm(qtype, m, k, n):
     """8 to 63 activation rows against 8M weights or more: the int8 GEMM split over k, most of its
     activation-row tile empty; the partial sums are added in a fixed order (the same result on every call)."""
     blocks = make_blocks(qtype, n, k, 310 + m)
     lhs = synth.normal(311 + m, (m, k))
     w = capi.Weight.upload(qtype, blocks, n, k)
     got = w.matmul_t(m, lhs)
-    name = {capi.Q6_K: "q6k", capi.Q8_0: "q8_0", capi.Q2_K: "q2k"}[qtype]
+    name = {capi.Q6_K: "q6k", capi.Q8_0: "q8_0", capi.Q2_K: "q2k", capi.IQ2_XXS: "iq2xxs", capi.MXFP4: "mxfp4"}[qtype]
     assert capi.last_kernel() == name + "_gemm_i8+splitk"
     assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
     assert np.array_equal(got, w.matmul_t(m, lhs))
 
 
-@pytest.mark.parametrize("qtype,m,k,n", [(capi.IQ2_XXS, 8, 12288, 1024), (capi.MXFP4, 16, 4096, 2100), (capi.MXFP4, 11, 7168, 1200),
-                                         (capi.Q6_K, 512, 2048, 100), (capi.IQ2_XXS, 70, 5120, 300)])
+@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q5_K, 8, 12288, 1024), (capi.Q4_0, 16, 4096, 2100), (capi.Q3_K, 11, 7168, 1200),
+                                         (capi.Q6_K, 512, 2048, 100), (capi.IQ2_XXS, 40, 5120, 300)])
 def test_decoded_weights_gemm_split_over_k(qtype, m, k, n):
     """8..16 rows against matrices of 8M elements or more, and many rows against few weight rows: the GEMM's
     tiles alone leave compute units idle, so runs of chunks go to workgroups of their own and the partial
     sums are added in a fixed order (the same result on every call)."""
-    blocks = make_blocks(qtype, n, k, 300 + m)
+    blocks = synth.random_blocks(qtype, 300 + m, n * k) if qtype in capi.GENERIC_TYPES else make_blocks(qtype, n, k, 300 + m)
     lhs = synth.normal(301 + m, (m, k))
     w = capi.Weight.upload(qtype, blocks, n, k)
     got = w.matmul_t(m, lhs)
-    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=True))
+    assert close(got, oracle.matmul_t(qtype, (m, k, n), lhs, blocks))
     assert capi.last_kernel().startswith("gemm_decoded_mfma")
     assert np.array_equal(got, w.matmul_t(m, lhs))
 
@@ -987,9 +1020,11 @@ import sys, numpy as np
 sys.path.insert(0, %r)
 import oracle
 from joshua_amd import capi, synth
-from tests.test_gpu_matmul import q4k_integer_case, q6k_integer_case, q2k_integer_case, q8_0_integer_case, close
+from tests.test_gpu_matmul import (q4k_integer_case, q6k_integer_case, q2k_integer_case, q8_0_integer_case,
+                                   iq2xxs_integer_case, mxfp4_integer_case, close)
 FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8"), "q2k": (capi.Q2_K, "q2k_gemm_i8"),
-               "q8_0": (capi.Q8_0, "q8_0_gemm_i8")}[sys.argv[1]]
+               "q8_0": (capi.Q8_0, "q8_0_gemm_i8"), "iq2xxs": (capi.IQ2_XXS, "iq2xxs_gemm_i8"),
+               "mxfp4": (capi.MXFP4, "mxfp4_gemm_i8")}[sys.argv[1]]
 # the same products split over k: the parts are summed in a fixed order
 if __import__("os").environ.get("JQ_Q4K_GEMM_I8_SPLITS", "1") != "1":
     for (m, k, n) in [(40, 4096, 100), (300, 4096, 130), (64, 12288, 70)]:
@@ -1018,11 +1053,15 @@ elif FMT == capi.Q6_K:  # every int8 scale value times q - 32, eight weights a r
     blocks, q, x = q6k_integer_case(n, k, 23, nonzero=8, random_scales=True, small=400)
 elif FMT == capi.Q2_K:  # 4-bit scales and mins over sub-blocks of 16
     blocks, q, x = q2k_integer_case(n, k, 23)
-else:  # scales of 1/4 to 2 inside a run of 256: the common scale holds every weight exactly, the sum 256 q d / D
-    # against the activations stays below 2^24
+elif FMT == capi.Q8_0:  # scales of 1/4 to 2 inside a run of 256: the common scale holds every weight exactly, the
+    # sum 256 q d / D against the activations stays below 2^24
     blocks, q, x = q8_0_integer_case(n, k, 23)
-lhs = np.stack([np.roll(x, (256 if FMT in (capi.Q2_K, capi.Q8_0) else 32) * i) for i in range(m)])
-assert np.abs(lhs @ q.T).max() < 2 ** 24
+elif FMT == capi.IQ2_XXS:  # dense integer weights up to 1333 against activations in multiples of 2^-8
+    blocks, q, x = iq2xxs_integer_case(n, k, 23)
+else:  # dense weights in multiples of 1/8 under scales of 1/4 to 1 against activations in multiples of 2^-8
+    blocks, q, x = mxfp4_integer_case(n, k, 23)
+lhs = np.stack([np.roll(x, (32 if FMT in (capi.Q4_K, capi.Q6_K) else 256) * i) for i in range(m)])
+assert np.abs(lhs @ q.T).max() < {capi.IQ2_XXS: 2 ** 16, capi.MXFP4: 2 ** 13}.get(FMT, 2 ** 24)
 if FMT == capi.Q8_0:  # per run of 256, 1024 times the sum is still an integer that f32 holds
     runs = np.einsum("mbe,nbe->mnb", lhs.reshape(m, -1, 256).astype(np.float64), q.reshape(n, -1, 256))
     assert np.abs(runs).max() < 2 ** 19
@@ -1066,7 +1105,7 @@ print("gemm i8 ok")
 """
 
 
-@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0"])
+@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4"])
 @pytest.mark.parametrize("shape", ["8,7", "4,4"])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup
