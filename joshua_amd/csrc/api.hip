@@ -1303,6 +1303,7 @@ struct jq_moe {
     uint8_t *gacts = nullptr;  // activations of the grouped int8 GEMM, and its tables
     int *gtab = nullptr;
     size_t gtab_rows = 0;      // row groups (and tiles) the tables hold
+    int gtile_rgs = 8;         // row groups a tile of the current plan: 8 (waves share the rows) or 2 (the weight rows)
     jq::ActsI8 qi8{nullptr, nullptr, nullptr, nullptr};  // activations as int8 planes (decode path, long rows)
     std::mutex mu;
 };
@@ -1642,7 +1643,7 @@ template <class F>
 int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, int base_align, const float *X,
                        const int *xsel, bool prepared, float *Y, int k, int n, hipStream_t s) {
     if (!m->gacts || k % 256 != 0 || row_bytes % F::ALIGN != 0 || base_align < F::ALIGN) return -1;
-    constexpr int NW = 4, NG = 4;
+    constexpr int NG = 4;
     const size_t nb = (size_t)k / 256, tx = ((size_t)n + 16 * NG - 1) / (16 * NG);
     const size_t max_rg = m->gtab_rows, max_mt = m->gtab_rows;
     if (tx * max_mt > 0x7FFFFFFFull) return -1;
@@ -1650,20 +1651,38 @@ int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, 
     if (!prepared)
         hipLaunchKernelGGL((jq::moe_gemm_i8_prep<F::SUB16>), dim3((unsigned)nb, (unsigned)max_rg), dim3(256), 0, s, X, xsel, t, k,
                            m->gacts);
-    auto kern = jq::kq_gemm_i8<F, NW, NG, true>;
     constexpr int lds = jq::qi_lds_bytes<F, NG>();
-    static std::once_flag big_lds;
-    static hipError_t attr_rc = hipSuccess;
-    std::call_once(big_lds, [&] {
-        attr_rc = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    });
-    HIP_TRY(attr_rc);
-    note_kernel("moe_gemm_i8");
     const jq::QiGrouped gp{wptr, m->gexp, m->yrow, t};
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tx * max_mt)), dim3(64 * NW), lds, s, (const uint8_t *)nullptr, row_bytes,
-                       (const uint8_t *)m->gacts, Y, 0, n, (int)nb, 0, (int)tx, 0, (int)nb, (size_t)0, gp);
+    hipError_t attr_rc = hipSuccess;
+#define JQ_MOE_GEMM(NW_, NSPLIT_)                                                                                     \
+    do {                                                                                                              \
+        auto kern = jq::kq_gemm_i8<F, NW_, NG, true, NSPLIT_>;                                                        \
+        static std::once_flag big_lds;                                                                                \
+        static hipError_t rc_once = hipSuccess;                                                                       \
+        std::call_once(big_lds, [&] {                                                                                 \
+            rc_once = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);       \
+        });                                                                                                           \
+        attr_rc = rc_once;                                                                                            \
+        if (attr_rc == hipSuccess)                                                                                    \
+            hipLaunchKernelGGL(kern, dim3((unsigned)(tx * max_mt)), dim3(64 * NW_), lds, s, (const uint8_t *)nullptr, \
+                               row_bytes, (const uint8_t *)m->gacts, Y, 0, n, (int)nb, 0, (int)tx, 0, (int)nb,       \
+                               (size_t)0, gp);                                                                        \
+    } while (0)
+    if (m->gtile_rgs == 2) JQ_MOE_GEMM(2, true);
+    else JQ_MOE_GEMM(4, false);
+#undef JQ_MOE_GEMM
+    HIP_TRY(attr_rc);
+    note_kernel(m->gtile_rgs == 2 ? "moe_gemm_i8_few" : "moe_gemm_i8");
     HIP_TRY(hipGetLastError());
     return 0;
+}
+
+// The tile plan of a bucketed call: few pairs an expert (32 on average or fewer) -> tiles of two row groups whose
+// waves share the weight rows; more -> tiles of eight row groups whose waves share the rows.
+void moe_gemm_plan(jq_moe *m, int groups, size_t pairs, hipStream_t s) {
+    static const char *env = getenv("JQ_MOE_GEMM_TILE_ROWS");  // 32 or 128: the tile for every call
+    m->gtile_rgs = env ? (atoi(env) == 32 ? 2 : 8) : (pairs <= 32 * (size_t)groups ? 2 : 8);
+    hipLaunchKernelGGL(jq::moe_gemm_i8_plan, dim3(1), dim3(256), 0, s, m->offsets, groups, m->gtile_rgs, moe_gemm_tables(m));
 }
 
 int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, size_t row_bytes, int base_align,
@@ -1765,7 +1784,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     // the activation in place
     bool planned = false;
     if (rc < 0 && same_gu && max_group > 1 && m->gacts) {
-        hipLaunchKernelGGL(jq::moe_gemm_i8_plan, dim3(1), dim3(256), 0, s, m->offsets, groups, 8, moe_gemm_tables(m));
+        moe_gemm_plan(m, groups, (size_t)P + (size_t)extra * T, s);
         planned = true;
         rc = dispatch_moe_gemm_i8(m, m->gate->type, m->pgate, m->gate->row_bytes, a16, x, m->xrow, false, m->G, (int)c.hidden,
                                   (int)c.inter, s);
@@ -1812,8 +1831,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
                                           (int)c.hidden, groups, s);
     if (rc > 0) return 1;
     if (rc < 0 && fused_act && max_group > 1 && m->gacts) {
-        if (!planned)
-            hipLaunchKernelGGL(jq::moe_gemm_i8_plan, dim3(1), dim3(256), 0, s, m->offsets, groups, 8, moe_gemm_tables(m));
+        if (!planned) moe_gemm_plan(m, groups, (size_t)P + (size_t)extra * T, s);
         rc = dispatch_moe_gemm_i8(m, m->down->type, m->pdown, m->down->row_bytes, d16, m->G, m->yrow, false, m->out,
                                   (int)c.inter, (int)c.hidden, s);
     }

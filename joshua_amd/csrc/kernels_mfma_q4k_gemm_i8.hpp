@@ -607,13 +607,20 @@ struct QiGrouped {
     const int *gexp, *yrow;
     QiGroupTables t;
 };
-template <class F, int NW, int NG, bool GROUPED = false>
+// NSPLIT: few activation rows.  The tile is 32 activation rows (two row groups) against 16 NG weight rows, and
+// the waves share the weight-row groups instead of the activation rows: wave w takes groups w NG / NW ..
+// of them against both row groups, so that every wave has matrix work whatever the row count (with the rows
+// split, a tile of one row group leaves all waves but one only the unpacking).
+template <class F, int NW, int NG, bool GROUPED = false, bool NSPLIT = false>
 __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict__ W, size_t row_bytes,
                                                       const uint8_t *__restrict__ acts, float *__restrict__ Y,
                                                       int m_rows, int n, int nb, int groups, int tx, int ty,
                                                       int nb_total, size_t split_stride, QiGrouped gp = QiGrouped{}) {
     constexpr int NT = 16 * NG, THREADS = 64 * NW, UNITS = 4 * NT, PER = (UNITS + THREADS - 1) / THREADS;
     constexpr int BUF = NG * QI_TILE + NT * F::META;
+    constexpr int NGW = NSPLIT ? NG / NW : NG;  // weight-row groups a wave multiplies
+    constexpr int MT = NSPLIT ? 32 : 32 * NW;   // activation rows a tile
+    static_assert(!NSPLIT || (NG % NW == 0 && NGW >= 2), "two weight-row groups a wave or more");
     extern __shared__ __attribute__((aligned(16))) uint8_t qi_lds[];
     const uint8_t *tab = qi_lds + 2 * BUF;  // the format's lookup table, behind the two buffers
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
@@ -631,7 +638,9 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
         by = (int)blockIdx.x / tx, bx = (int)blockIdx.x % tx;
     }
     if (bx >= tx || (!GROUPED && by >= ty)) return;
-    const int n0 = bx * NT, m0 = by * 32 * NW;
+    const int n0 = bx * NT, m0 = by * MT;
+    const int cg0 = NSPLIT ? (tid >> 6) * NGW : 0;   // this wave's first weight-row group
+    const int wrow = NSPLIT ? 0 : 2 * (tid >> 6);    // this wave's first row group within the tile
     // split over k: workgroups blockIdx.y = i take super-blocks i nb .. (i + 1) nb - 1 of the nb_total and store
     // their sums at Y + i split_stride (splitk_sum adds the parts in a fixed order)
     const int b_first = GROUPED ? 0 : (int)blockIdx.y * nb;
@@ -642,7 +651,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
     const uint8_t *arec[2];
 #pragma unroll
     for (int mg = 0; mg < 2; mg++)
-        arec[mg] = acts + ((size_t)(GROUPED ? rg0 + min(2 * wave + mg, nrg - 1) : min(m0 / 16 + 2 * wave + mg, groups - 1)) * nb_total + b_first) * QI_REC;
+        arec[mg] = acts + ((size_t)(GROUPED ? rg0 + min(wrow + mg, nrg - 1) : min(m0 / 16 + wrow + mg, groups - 1)) * nb_total + b_first) * QI_REC;
 
     // unpack units of this thread: chunk c = tid % 4 of weight rows tid / 4 + (THREADS / 4) p
     const int uc = tid & 3;
@@ -699,11 +708,11 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
 #pragma unroll
         for (int P = 0; P < 2; P++) A[c][P] = *(const qm_i4 *)(arec[0] + ((size_t)(2 * c + P) * 64 + lane) * 16);
 
-    qm_f4 acc[2][NG];
+    qm_f4 acc[2][NGW];
 #pragma unroll
     for (int mg = 0; mg < 2; mg++)
 #pragma unroll
-        for (int cg = 0; cg < NG; cg++) acc[mg][cg] = qm_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int cg = 0; cg < NGW; cg++) acc[mg][cg] = qm_f4{0.0f, 0.0f, 0.0f, 0.0f};
     const qm_i4 zero_i = {0, 0, 0, 0};
     const qm_f4 zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
     __syncthreads();
@@ -716,18 +725,18 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
             // scales and I2 operand of this row group: wanted in the last quarter
             const qm_f4 sx = *(const qm_f4 *)(arec[mg] + (size_t)b * QI_REC + QI_SCALE + 16 * g);
             const qi_h8 minA = *(const qi_h8 *)(arec[mg] + (size_t)b * QI_REC + QI_MIN + lane * 16);
-            // The weight-row groups in two sets (T0 and NG - T0 of them), each taken through the four chunks: the
+            // The wave's weight-row groups in two sets (T0 and NGW - T0 of them), each taken through the four chunks: the
             // integer sums of one set are alive at a time.  Step s of a half = (set, chunk, group within the set).
-            constexpr int T0 = (NG + 1) / 2, STEPS = 4 * NG;
-            auto step_cg = [](int s) { return s < 4 * T0 ? s % T0 : T0 + (s - 4 * T0) % (NG - T0); };
-            auto step_c = [](int s) { return s < 4 * T0 ? s / T0 : (s - 4 * T0) / (NG - T0); };
-            qm_i4 HH[NG], MID[NG], LL[NG];
+            constexpr int T0 = (NGW + 1) / 2, STEPS = 4 * NGW;
+            auto step_cg = [](int s) { return s < 4 * T0 ? s % T0 : T0 + (s - 4 * T0) % (NGW - T0); };
+            auto step_c = [](int s) { return s < 4 * T0 ? s / T0 : (s - 4 * T0) / (NGW - T0); };
+            qm_i4 HH[NGW], MID[NGW], LL[NGW];
             // the weight operands travel one step ahead of the MFMAs that use them, through two register sets
             qm_i4 Bh[2], Bl[2];
-            if constexpr (!F::ONE_PLANE) Bh[0] = *(const qm_i4 *)(buf + lane * 16);
-            Bl[0] = *(const qm_i4 *)(buf + 1024 + lane * 16);
+            if constexpr (!F::ONE_PLANE) Bh[0] = *(const qm_i4 *)(buf + 4 * cg0 * 2048 + lane * 16);
+            Bl[0] = *(const qm_i4 *)(buf + 4 * cg0 * 2048 + 1024 + lane * 16);
             auto finish = [&](int cg) __attribute__((always_inline)) {  // the 16 x 16 results of weight-row group cg
-                const uint8_t *meta = buf + NG * QI_TILE + (16 * cg + r) * F::META;
+                const uint8_t *meta = buf + NG * QI_TILE + (16 * (cg0 + cg) + r) * F::META;
                 const float2 dd = *(const float2 *)(meta + F::META - 16);
                 qm_f4 I2 = zero_f;
                 if constexpr (F::HAS_MIN) {
@@ -747,8 +756,8 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
                 const int cg = step_cg(s), c = step_c(s), cur = s & 1, nxt = cur ^ 1;
-                const bool first_of_pass = s < 4 * T0 ? s % T0 == 0 : (s - 4 * T0) % (NG - T0) == 0;
-                const bool last_of_pass = s < 4 * T0 ? s % T0 == T0 - 1 : (s - 4 * T0) % (NG - T0) == NG - T0 - 1;
+                const bool first_of_pass = s < 4 * T0 ? s % T0 == 0 : (s - 4 * T0) % (NGW - T0) == 0;
+                const bool last_of_pass = s < 4 * T0 ? s % T0 == T0 - 1 : (s - 4 * T0) % (NGW - T0) == NGW - T0 - 1;
                 const int pass = s < 4 * T0 ? c : 4 + c;  // 0..7 within the half
                 if (first_of_pass) {
                     // An eighth of the next super-block's weights becomes operands in every pass, thinly spread
@@ -763,8 +772,8 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                 if (c == 0) HH[cg] = zero_i, MID[cg] = zero_i, LL[cg] = zero_i;
                 if (s + 1 < STEPS) {
                     const int cg1 = step_cg(s + 1), c1 = step_c(s + 1);
-                    if constexpr (!F::ONE_PLANE) Bh[nxt] = *(const qm_i4 *)(buf + (4 * cg1 + c1) * 2048 + lane * 16);
-                    Bl[nxt] = *(const qm_i4 *)(buf + (4 * cg1 + c1) * 2048 + 1024 + lane * 16);
+                    if constexpr (!F::ONE_PLANE) Bh[nxt] = *(const qm_i4 *)(buf + (4 * (cg0 + cg1) + c1) * 2048 + lane * 16);
+                    Bl[nxt] = *(const qm_i4 *)(buf + (4 * (cg0 + cg1) + c1) * 2048 + 1024 + lane * 16);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 MID[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[c][0], Bl[cur], MID[cg], 0, 0, 0);
@@ -782,7 +791,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                 if (c == 3 && last_of_pass && pass < 4) finish(cg);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            finish(NG - 1);
+            finish(NGW - 1);
             if (mg == 1) fetch_part(b_next2, 2);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -793,10 +802,10 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
 #pragma unroll
     for (int mg = 0; mg < 2; mg++) {
         int first_pair = 0, pairs = 0;
-        if (GROUPED && 2 * wave + mg < nrg) first_pair = gp.t.rg_pair[rg0 + 2 * wave + mg], pairs = gp.t.rg_cnt[rg0 + 2 * wave + mg];
+        if (GROUPED && wrow + mg < nrg) first_pair = gp.t.rg_pair[rg0 + wrow + mg], pairs = gp.t.rg_cnt[rg0 + wrow + mg];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            int row = m0 + 32 * wave + 16 * mg + 4 * g + i;
+            int row = m0 + 16 * (wrow + mg) + 4 * g + i;
             if (GROUPED) {
                 if (4 * g + i >= pairs) continue;
                 row = gp.yrow[first_pair + 4 * g + i];
@@ -804,8 +813,8 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                 continue;
             }
 #pragma unroll
-            for (int cg = 0; cg < NG; cg++) {
-                const int col = n0 + 16 * cg + r;
+            for (int cg = 0; cg < NGW; cg++) {
+                const int col = n0 + 16 * (cg0 + cg) + r;
                 if (col < n) Y[(size_t)row * n + col] = acc[mg][cg][i];
             }
         }

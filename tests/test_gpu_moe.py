@@ -239,24 +239,28 @@ def test_few_tokens_an_expert_take_the_int8_quads_kernel(tokens):
     assert close(dev.forward(x), ora.forward(x))
 
 
-@pytest.mark.parametrize("qtype,h,inter,E,k,tokens,shared_inter,kw", [
-    (capi.Q4_K, 5120, 256, 8, 2, 40, 0, {}),                         # rows too long for the Q4_K grouped kernels
-    (capi.IQ2_XXS, 1024, 512, 8, 2, 70, 512, dict(gating="sigmoid", swiglu_clamp=0.02, swiglu_clamp_shared=0.01)),
-    (capi.MXFP4, 512, 768, 16, 4, 33, 0, {}),
-    (capi.Q6_K, 768, 256, 4, 2, 300, 0, {}),                         # about 150 pairs an expert: two tiles of 128
-    (capi.Q2_K, 512, 256, 4, 2, 300, 0, dict(swiglu_clamp=0.02)),
-    (capi.Q8_0, 256, 512, 16, 4, 64, 512, dict(gating="sigmoid", weights_scale=2.5)),
-    (capi.MXFP4, 256, 256, 160, 6, 150, 0, {}),                      # more experts than one pass of the tile plan
+@pytest.mark.parametrize("qtype,h,inter,E,k,tokens,shared_inter,kw,kernel", [
+    (capi.Q4_K, 5120, 256, 8, 2, 40, 0, {}, "moe_gemm_i8_few"),      # rows too long for the Q4_K grouped kernels
+    (capi.IQ2_XXS, 1024, 512, 8, 2, 70, 512, dict(gating="sigmoid", swiglu_clamp=0.02, swiglu_clamp_shared=0.01),
+     "moe_gemm_i8_few"),                                             # the shared expert's 70 pairs: three tiles of 32
+    (capi.MXFP4, 512, 768, 16, 4, 33, 0, {}, "moe_gemm_i8_few"),
+    (capi.Q6_K, 768, 256, 4, 2, 300, 0, {}, "moe_gemm_i8"),          # about 150 pairs an expert: two tiles of 128
+    (capi.Q2_K, 512, 256, 4, 2, 300, 0, dict(swiglu_clamp=0.02), "moe_gemm_i8"),
+    (capi.Q8_0, 256, 512, 16, 4, 64, 512, dict(gating="sigmoid", weights_scale=2.5), "moe_gemm_i8_few"),
+    (capi.MXFP4, 256, 256, 160, 6, 150, 0, {}, "moe_gemm_i8_few"),   # more experts than one pass of the tile plan
+    (capi.IQ2_XXS, 512, 512, 4, 2, 200, 0, {}, "moe_gemm_i8"),
 ])
-def test_many_tokens_take_the_grouped_int8_gemm(qtype, h, inter, E, k, tokens, shared_inter, kw):
+def test_many_tokens_take_the_grouped_int8_gemm(qtype, h, inter, E, k, tokens, shared_inter, kw, kernel):
     """Bucketed calls of the formats with a side of the int8 GEMM: pairs sorted by expert are laid out in row
     groups of 16 that never mix two experts, gate and up run from one preparation of the tokens, the activation
-    is applied in place (with the shared expert's own clamp on its rows) and the down projection reads it."""
+    is applied in place (with the shared expert's own clamp on its rows) and the down projection reads it.  Up
+    to 32 pairs an expert on average: tiles of 32 rows whose waves share the weight rows; more: tiles of 128
+    rows whose waves share the rows."""
     ora, dev = build(qtype, h, inter, E, k, 150 + h, shared_inter=shared_inter, **kw)
     x = synth.normal(151 + tokens, (tokens, h))
     want = ora.forward(x)
     got = dev.forward(x)
-    assert capi.last_kernel() == "moe_gemm_i8"
+    assert capi.last_kernel() == kernel
     assert close(got, want)
     assert np.array_equal(got, dev.forward(x))
     few = synth.normal(152, (3, h))                                   # then a decode-sized call on the same layer
