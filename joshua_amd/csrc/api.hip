@@ -1772,11 +1772,18 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     // few tokens an expert (at most six on average): the int8 kernel that takes four rows an MFMA; more: the
     // f16 ring kernel, which reads a group's weights once for up to 16 rows
     const bool few = (size_t)P <= 6 * (size_t)c.n_expert;
+    // many tokens an expert (48 on average or more): the grouped int8 GEMM, which unpacks a weight tile once for
+    // 128 rows (Qwen3-30B-A3B sizes, 2048 tokens: 1.34 ms a call against the ring kernel's 2.03; equal at 512)
+    static const char *gemm_from_env = getenv("JQ_MOE_GEMM_FROM_PAIRS_PER_EXPERT");
+    const size_t gemm_from = gemm_from_env ? (size_t)atoll(gemm_from_env) : 48;
+    const bool prefer_gemm = m->gacts && max_group > 1 && (size_t)P >= gemm_from * (size_t)c.n_expert &&
+                             c.hidden % 256 == 0 && c.inter % 256 == 0 && a16 >= 16 &&
+                             align_of({m->down, m->fold_shared ? m->sdown : nullptr}) >= 16;
     if (same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K && few)
         rc = dispatch_moe_q4k_quads<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp, m->offsets,
                                           m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
     if (rc > 0) return 1;
-    if (rc < 0 && same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K)
+    if (rc < 0 && same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K && !prefer_gemm)
         rc = dispatch_moe_q4k_ring<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qacts, m->gexp, m->offsets,
                                          m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
     if (rc > 0) return 1;
@@ -1825,7 +1832,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
                                            m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                            (int)c.hidden, groups, s);
     if (rc > 0) return 1;
-    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K)
+    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && !prefer_gemm)
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);

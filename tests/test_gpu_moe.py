@@ -249,6 +249,7 @@ def test_few_tokens_an_expert_take_the_int8_quads_kernel(tokens):
     (capi.Q8_0, 256, 512, 16, 4, 64, 512, dict(gating="sigmoid", weights_scale=2.5), "moe_gemm_i8_few"),
     (capi.MXFP4, 256, 256, 160, 6, 150, 0, {}, "moe_gemm_i8_few"),   # more experts than one pass of the tile plan
     (capi.IQ2_XXS, 512, 512, 4, 2, 200, 0, {}, "moe_gemm_i8"),
+    (capi.Q4_K, 512, 256, 4, 2, 300, 256, dict(gating="sigmoid"), "moe_gemm_i8"),  # 48 pairs an expert or more: ahead of the ring kernel
 ])
 def test_many_tokens_take_the_grouped_int8_gemm(qtype, h, inter, E, k, tokens, shared_inter, kw, kernel):
     """Bucketed calls of the formats with a side of the int8 GEMM: pairs sorted by expert are laid out in row
