@@ -514,61 +514,80 @@ struct QiIQ2XXS {
     }
 };
 
-// MXFP4: blocks of e (E8M0) | 16 bytes of E2M1 codes, w = 2^(e - 127) * +-{0, .5, 1, 1.5, 2, 3, 4, 6}, low
-// nibbles elements 0..15, high nibbles 16..31, e = 255 a block of zeros (src/mxfp4.rs:45-94); a "super-block"
-// here is eight blocks, 136 bytes.  As for Q8_0 the eight blocks are put on one scale: with D the largest
-// 2^(e - 127) among them, p = round(4096 w / D) in -24576..24576 -- exact for every block within eleven
-// octaves of the largest, rounded to 2^-12 of the largest element below that.  Per block the eight
-// magnitudes times two signs make two 8-byte tables a plane and sign: four v_perm_b32 and two bit selects
-// for four elements.  Blocks sit at any byte: read through aligned words.  Runs whose largest scale is below
-// 2^-100 count as zeros.
-struct QiMXFP4 {
-    static constexpr int BLOCK = 136, META = 48, ALIGN = 1, TABLE = 0;
+// Blocks of 32 elements as a scale and sixteen bytes of 4-bit codes, low nibbles elements 0..15, high nibbles
+// 16..31, w = scale * value(code); a "super-block" here is eight blocks.  As for Q8_0 the eight blocks are put
+// on one scale: with D the largest |scale| among them, p = round(2048 value scale / D), within +-24576 --
+// exact for every block within seven octaves or more of the largest (eleven for MXFP4), rounded to 2^-12 of
+// the run's largest element below that.  Per block the sixteen products make two 8-byte tables a plane (codes
+// 0..7 and 8..15): four v_perm_b32 and two bit selects for four elements.  Runs whose largest scale is below
+// 2^-100 count as zeros.  T gives the block: BYTES, HEAD (bytes in front of the codes), ALIGN, scale_of(block),
+// value(code) and UNIT (the value of one unit of p over D).
+//   MXFP4: e (E8M0) | codes, w = 2^(e - 127) * +-{0, .5, 1, 1.5, 2, 3, 4, 6}, e = 255 a block of zeros
+//   (src/mxfp4.rs:45-94); value() is the doubled E2M1 value.  Blocks of 17 bytes sit at any byte.
+//   Q4_0: d (f16) | codes, w = d (code - 8) (vendor/candle-metal-kernels/src/metal_src/quantized.metal:86-89).
+struct QtMXFP4 {
+    static constexpr int BYTES = 17, HEAD = 1, ALIGN = 1;
+    static constexpr float UNIT = 1.0f / 4096.0f;
+    __device__ __forceinline__ static float scale_of(const uint8_t *blk) {
+        const uint32_t e = blk[0];
+        return e == 0xFFu ? 0.0f : __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
+    }
+    __device__ __forceinline__ static constexpr float value(int code) {
+        const int i = code & 7, v = i < 5 ? i : i == 5 ? 6 : i == 6 ? 8 : 12;
+        return (float)(code & 8 ? -v : v);
+    }
+};
+struct QtQ4_0 {
+    static constexpr int BYTES = 18, HEAD = 2, ALIGN = 2;
+    static constexpr float UNIT = 1.0f / 2048.0f;
+    __device__ __forceinline__ static float scale_of(const uint8_t *blk) { return f16_bits(ld<uint16_t>(blk)); }
+    __device__ __forceinline__ static constexpr float value(int code) { return (float)(code - 8); }
+};
+template <class T>
+struct QiNibbles32 {
+    static constexpr int BLOCK = 8 * T::BYTES, META = 48, ALIGN = T::ALIGN, TABLE = 0;
     static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
         float d0, d1;
     };
     struct Raw {
         float unit;
-        uint32_t th[2][4], tl[2][4];  // per block: Ph / Pl of +p_0..7 (words 0, 1) and of -p_0..7 (words 2, 3)
+        uint32_t th[2][4], tl[2][4];  // per block: Ph / Pl of codes 0..7 (words 0, 1) and of codes 8..15 (words 2, 3)
         uint4 qa, qb;                 // the codes of block 2 uc and of block 2 uc + 1
         uint4 na, nb;                 // the same of the next super-block
     };
-    __device__ __forceinline__ static float scale_of(uint32_t e) {
-        return e == 0xFFu ? 0.0f : __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
-    }
     __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
-        if (part == 0) next.d0 = scale_of(blk[34 * uc]), next.d1 = scale_of(blk[34 * uc + 17]);
-        if (part == 1) raw.na = ldw<uint4>(blk + 34 * uc + 1);
-        if (part == 2) raw.nb = ldw<uint4>(blk + 34 * uc + 18);
+        const uint8_t *pair = blk + 2 * T::BYTES * uc;
+        if (part == 0) next.d0 = T::scale_of(pair), next.d1 = T::scale_of(pair + T::BYTES);
+        if (part == 1) raw.na = ldw<uint4>(pair + T::HEAD);
+        if (part == 2) raw.nb = ldw<uint4>(pair + T::BYTES + T::HEAD);
     }
     __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
-        float D = fmaxf(next.d0, next.d1);
+        float D = fmaxf(mag_or_inf(next.d0), mag_or_inf(next.d1));
         D = fmaxf(D, dpp_f<0xB1>(D));  // quad_perm [1,0,3,2]
         D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
         const bool live = D >= 7.888609052210118e-31f;  // 2^-100
-        const float inv = live ? 2048.0f / D : 0.0f;    // doubled magnitudes: 4096 w / D = (2 |w| / d) * 2048 d / D
-        raw.unit = live ? D * (1.0f / 4096.0f) : 0.0f;
+        const float inv = live ? 2048.0f / D : 0.0f;
+        raw.unit = live ? D * T::UNIT : 0.0f;
         raw.qa = raw.na, raw.qb = raw.nb;
 #pragma unroll
         for (int blk = 0; blk < 2; blk++) {
             const float ratio = (blk ? next.d1 : next.d0) * inv;
             uint32_t t[2][8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) {  // round(+-v ratio) + 128 in the low 16 bits of 1.5 * 2^23 + 128 +- v ratio
-                const float v = (float)(i < 5 ? i : i == 5 ? 6 : i == 6 ? 8 : 12);
-                t[0][i] = __builtin_bit_cast(uint32_t, fmaf(v, ratio, 12583040.0f));
-                t[1][i] = __builtin_bit_cast(uint32_t, fmaf(-v, ratio, 12583040.0f));
+            for (int i = 0; i < 8; i++) {  // round(value ratio) + 128 in the low 16 bits of 1.5 * 2^23 + 128 + value ratio
+                t[0][i] = __builtin_bit_cast(uint32_t, fmaf(T::value(i), ratio, 12583040.0f));
+                t[1][i] = __builtin_bit_cast(uint32_t, fmaf(T::value(8 + i), ratio, 12583040.0f));
             }
 #pragma unroll
-            for (int sgn = 0; sgn < 2; sgn++)
+            for (int top = 0; top < 2; top++)
 #pragma unroll
                 for (int h4 = 0; h4 < 2; h4++) {
-                    const uint32_t *q = &t[sgn][4 * h4];
+                    const uint32_t *q = &t[top][4 * h4];
                     const uint32_t a = __builtin_amdgcn_perm(q[1], q[0], 0x05010400u);  // L0 L1 H0 H1
                     const uint32_t b = __builtin_amdgcn_perm(q[3], q[2], 0x05010400u);  // L2 L3 H2 H3
-                    raw.tl[blk][2 * sgn + h4] = __builtin_amdgcn_perm(b, a, 0x05040100u) ^ 0x80808080u;
-                    raw.th[blk][2 * sgn + h4] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+                    raw.tl[blk][2 * top + h4] = __builtin_amdgcn_perm(b, a, 0x05040100u) ^ 0x80808080u;
+                    raw.th[blk][2 * top + h4] = __builtin_amdgcn_perm(b, a, 0x07060302u);
                 }
         }
     }
@@ -578,18 +597,63 @@ struct QiMXFP4 {
         for (int blk = 0; blk < 2; blk++) {  // elements 16 half + 4 wi .. + 3 of both blocks
             const uint4 qv = blk ? raw.qb : raw.qa;
             const uint32_t word = (wi == 0 ? qv.x : wi == 1 ? qv.y : wi == 2 ? qv.z : qv.w) >> (4 * half);
-            const uint32_t sel = word & 0x07070707u, neg = ((word >> 3) & 0x01010101u) * 0xFFu;
-            const uint32_t ph = __builtin_amdgcn_perm(raw.th[blk][1], raw.th[blk][0], sel);
-            const uint32_t nh = __builtin_amdgcn_perm(raw.th[blk][3], raw.th[blk][2], sel);
-            const uint32_t pl = __builtin_amdgcn_perm(raw.tl[blk][1], raw.tl[blk][0], sel);
-            const uint32_t nl = __builtin_amdgcn_perm(raw.tl[blk][3], raw.tl[blk][2], sel);
+            const uint32_t sel = word & 0x07070707u, top = ((word >> 3) & 0x01010101u) * 0xFFu;
+            const uint32_t h0 = __builtin_amdgcn_perm(raw.th[blk][1], raw.th[blk][0], sel);
+            const uint32_t h1 = __builtin_amdgcn_perm(raw.th[blk][3], raw.th[blk][2], sel);
+            const uint32_t l0 = __builtin_amdgcn_perm(raw.tl[blk][1], raw.tl[blk][0], sel);
+            const uint32_t l1 = __builtin_amdgcn_perm(raw.tl[blk][3], raw.tl[blk][2], sel);
             const int gg = 2 * blk + half;
-            *(uint32_t *)(tile + gg * 256 + 4 * wi) = (nh & neg) | (ph & ~neg);
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = (nl & neg) | (pl & ~neg);
+            *(uint32_t *)(tile + gg * 256 + 4 * wi) = (h1 & top) | (h0 & ~top);
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = (l1 & top) | (l0 & ~top);
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
         *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+    }
+};
+using QiMXFP4 = QiNibbles32<QtMXFP4>;
+using QiQ4_0 = QiNibbles32<QtQ4_0>;
+
+// Q5_K: d | dmin | scales[12] | qh[32] | qs[128], w = d sc q - dmin m with q in 0..31: the nibble of Q4_K's
+// layout and, for element l of sub-block j, bit j of qh[l] as the fifth bit
+// (vendor/candle-metal-kernels/src/metal_src/quantized.metal:176-189, 6649-6670); scales and mins as in Q4_K.
+// p = sc q in 0..1953.
+struct QiQ5K {
+    static constexpr int BLOCK = 176, META = 48, ALIGN = 16, TABLE = 0;
+    static constexpr bool HAS_MIN = true, ONE_PLANE = false, SUB16 = false;
+    using Hdr = QiQ4K::Hdr;
+    struct Raw {
+        Hdr hdr;
+        uint4 q0, q1, h0, h1;
+    };
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        if (part == 0) next.h = *(const uint4 *)blk;
+        if (part == 1) raw.q0 = *(const uint4 *)(blk + 48 + 32 * uc), raw.h0 = *(const uint4 *)(blk + 16);
+        if (part == 2) raw.q1 = *(const uint4 *)(blk + 64 + 32 * uc), raw.h1 = *(const uint4 *)(blk + 32);
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) { raw.hdr = next; }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
+        const uint4 hdr = raw.hdr.h;
+        const uint32_t scl = hdr.y & 0x3F3F3F3Fu, sch = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+        const uint32_t s4 = (uc < 2 ? scl : sch) >> (16 * (uc & 1));
+        const uint32_t sc[2] = {s4 & 0xFFu, (s4 >> 8) & 0xFFu};
+        const uint4 qv = j < 4 ? raw.q0 : raw.q1, hv = j < 4 ? raw.h0 : raw.h1;
+        const uint32_t word = (j & 3) == 0 ? qv.x : (j & 3) == 1 ? qv.y : (j & 3) == 2 ? qv.z : qv.w;
+        const uint32_t high = ((j & 3) == 0 ? hv.x : (j & 3) == 1 ? hv.y : (j & 3) == 2 ? hv.z : hv.w) >> (2 * uc);
+#pragma unroll
+        for (int nib = 0; nib < 2; nib++) {  // low nibbles: sub-block 2 uc, high nibbles: sub-block 2 uc + 1
+            const uint32_t q = ((nib ? word >> 4 : word) & 0x0F0F0F0Fu) | (((high >> nib) & 0x01010101u) << 4);
+            const uint32_t even = __umul24(q & 0x00FF00FFu, sc[nib]) + 0x00800080u;
+            const uint32_t odd = __umul24((q >> 8) & 0x00FF00FFu, sc[nib]) + 0x00800080u;
+            const int gg = 2 * nib + (j >> 2);
+            *(uint32_t *)(tile + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        QiQ4K::Raw as_q4k;
+        as_q4k.hdr = raw.hdr;
+        QiQ4K::meta(as_q4k, uc, meta);
     }
 };
 

@@ -317,6 +317,57 @@ def mxfp4_integer_case(n, k, seed):
     return blocks, w, x / 256.0
 
 
+def q5k_integer_case(n, k, seed, nonzero=16, small=4000):
+    """Q5_K blocks with d = 1, dmin = 0, every sub-block scale 1 and `nonzero` weights in 1..31 a row (the
+    fifth bit of element l of sub-block j is bit j of qh[l]); integer activations that peak at 32639 at one
+    slot of every 32, where the weights are zero.  Returns (blocks, integer weights, activations)."""
+    rng = np.random.default_rng(seed)
+    q = np.zeros((n, k), np.int64)
+    x = rng.integers(-small, small + 1, size=k).astype(np.int64)
+    peak = np.arange(0, k, 32) + int(rng.integers(0, 32))
+    x[peak] = 32639 * rng.choice([-1, 1], size=k // 32)
+    free = np.setdiff1d(np.arange(k), peak)
+    for r in range(n):
+        q[r, rng.choice(free, size=nonzero, replace=False)] = rng.integers(1, 32, size=nonzero)
+    qb = q.reshape(n, k // 256, 4, 2, 32)                      # chunk c: sub-block 2c (low nibbles), 2c + 1 (high)
+    packed = ((qb[:, :, :, 0, :] & 15) | ((qb[:, :, :, 1, :] & 15) << 4)).astype(np.uint8).reshape(n, k // 256, 128)
+    qh = np.zeros((n, k // 256, 32), np.int64)
+    for j in range(8):
+        qh |= (q.reshape(n, k // 256, 8, 32)[:, :, j, :] >> 4) << j
+    blocks = np.zeros((n, k // 256, 176), np.uint8)
+    blocks[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks[:, :, 4:8] = 1                                       # sc_0..3 = 1, m = 0
+    blocks[:, :, 12:16] = 1                                     # sc_4..7 = 1 (low 4 bits), m = 0
+    blocks[:, :, 16:48] = qh.astype(np.uint8)
+    blocks[:, :, 48:] = packed
+    blocks = blocks.reshape(-1)
+    assert np.array_equal(oracle.dequantize(capi.Q5_K, blocks).reshape(n, k), q.astype(np.float32))
+    return blocks, q, x
+
+
+def q4_0_integer_case(n, k, seed, nonzero=16, small=400):
+    """Q4_0 blocks whose scales are powers of two between 1/2 and 4 and `nonzero` weights code - 8 in -8..7 a
+    row; integer activations that peak at 32639 at one slot of every 256, where the weights are zero.
+    Returns (blocks, the weights d (code - 8) as float64, activations)."""
+    rng = np.random.default_rng(seed)
+    q = np.zeros((n, k), np.int64)
+    for r in range(n):
+        q[r, rng.choice(k, size=nonzero, replace=False)] = rng.integers(-8, 8, size=nonzero)
+    x = rng.integers(-small, small + 1, size=k).astype(np.int64)
+    peak = np.arange(0, k, 256) + int(rng.integers(0, 256))
+    x[peak] = 32639 * rng.choice([-1, 1], size=k // 256)
+    q[:, peak] = 0
+    d = rng.choice(np.array([0.5, 1.0, 2.0, 4.0]), size=(n, k // 32))
+    codes = (q + 8).reshape(n, k // 32, 2, 16)                   # low nibbles: elements 0..15, high: 16..31
+    blocks = np.zeros((n, k // 32, 18), np.uint8)
+    blocks[:, :, 0:2] = d.astype(np.float16)[..., None].view(np.uint8)
+    blocks[:, :, 2:] = (codes[:, :, 0, :] | (codes[:, :, 1, :] << 4)).astype(np.uint8)
+    blocks = blocks.reshape(-1)
+    w = q * d.repeat(32, axis=1)
+    assert np.array_equal(oracle.dequantize(capi.Q4_0, blocks).reshape(n, k), w.astype(np.float32))
+    return blocks, w, x
+
+
 def test_q6k_dot4_integer_dot_products_are_bit_exact():
     """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
     scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
@@ -396,7 +447,7 @@ def test_few_rows_against_a_large_matrix_take_the_int8_gemm(qtype, m, k, n):
     assert np.array_equal(got, w.matmul_t(m, lhs))
 
 
-@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q5_K, 8, 12288, 1024), (capi.Q4_0, 16, 4096, 2100), (capi.Q3_K, 11, 7168, 1200),
+@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q5_0, 8, 12288, 1024), (capi.Q4_1, 16, 4096, 2100), (capi.Q3_K, 11, 7168, 1200),
                                          (capi.Q6_K, 512, 2048, 100), (capi.IQ2_XXS, 40, 5120, 300)])
 def test_decoded_weights_gemm_split_over_k(qtype, m, k, n):
     """8..16 rows against matrices of 8M elements or more, and many rows against few weight rows: the GEMM's
@@ -1021,10 +1072,19 @@ sys.path.insert(0, %r)
 import oracle
 from joshua_amd import capi, synth
 from tests.test_gpu_matmul import (q4k_integer_case, q6k_integer_case, q2k_integer_case, q8_0_integer_case,
-                                   iq2xxs_integer_case, mxfp4_integer_case, close)
+                                   iq2xxs_integer_case, mxfp4_integer_case, q5k_integer_case, q4_0_integer_case, close)
 FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8"), "q2k": (capi.Q2_K, "q2k_gemm_i8"),
                "q8_0": (capi.Q8_0, "q8_0_gemm_i8"), "iq2xxs": (capi.IQ2_XXS, "iq2xxs_gemm_i8"),
-               "mxfp4": (capi.MXFP4, "mxfp4_gemm_i8")}[sys.argv[1]]
+               "mxfp4": (capi.MXFP4, "mxfp4_gemm_i8"), "q5k": (capi.Q5_K, "q5k_gemm_i8"),
+               "q4_0": (capi.Q4_0, "q4_0_gemm_i8")}[sys.argv[1]]
+_synth = synth
+class _Synth:  # the formats without a quantiser of normal weights get random blocks
+    normal = staticmethod(_synth.normal)
+    @staticmethod
+    def normal_quantized(fmt, seed, count, sigma):
+        return _synth.random_blocks(fmt, seed, count) if fmt in capi.GENERIC_TYPES else _synth.normal_quantized(fmt, seed, count, sigma)
+synth = _Synth
+AVX2 = oracle.have_avx2() and FMT not in capi.GENERIC_TYPES
 # the same products split over k: the parts are summed in a fixed order
 if __import__("os").environ.get("JQ_Q4K_GEMM_I8_SPLITS", "1") != "1":
     for (m, k, n) in [(40, 4096, 100), (300, 4096, 130), (64, 12288, 70)]:
@@ -1033,7 +1093,7 @@ if __import__("os").environ.get("JQ_Q4K_GEMM_I8_SPLITS", "1") != "1":
         w = capi.Weight.upload(FMT, blocks, n, k)
         got = w.matmul_t(m, lhs)
         assert capi.last_kernel() == KERNEL + "+splitk", (capi.last_kernel(), m, k, n)
-        assert close(got, oracle.matmul_t(FMT, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())), (m, k, n)
+        assert close(got, oracle.matmul_t(FMT, (m, k, n), lhs, blocks, avx2=AVX2)), (m, k, n)
         assert np.array_equal(got, w.matmul_t(m, lhs))
     print("gemm i8 ok")
     sys.exit(0)
@@ -1044,7 +1104,7 @@ for (m, k, n) in [(17, 256, 64), (33, 512, 100), (64, 1024, 300), (100, 1024, 25
     lhs = synth.normal(6 + k, (m, k))
     got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(m, lhs)
     assert capi.last_kernel() == KERNEL, (capi.last_kernel(), m, k, n)
-    assert close(got, oracle.matmul_t(FMT, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())), (m, k, n)
+    assert close(got, oracle.matmul_t(FMT, (m, k, n), lhs, blocks, avx2=AVX2)), (m, k, n)
 # exact integers: activation range 32639 per 32-element sub-block
 n, k, m = 160, 2048, 40
 if FMT == capi.Q4_K:
@@ -1058,11 +1118,15 @@ elif FMT == capi.Q8_0:  # scales of 1/4 to 2 inside a run of 256: the common sca
     blocks, q, x = q8_0_integer_case(n, k, 23)
 elif FMT == capi.IQ2_XXS:  # dense integer weights up to 1333 against activations in multiples of 2^-8
     blocks, q, x = iq2xxs_integer_case(n, k, 23)
-else:  # dense weights in multiples of 1/8 under scales of 1/4 to 1 against activations in multiples of 2^-8
+elif FMT == capi.MXFP4:  # dense weights in multiples of 1/8 under scales of 1/4 to 1 against activations in multiples of 2^-8
     blocks, q, x = mxfp4_integer_case(n, k, 23)
-lhs = np.stack([np.roll(x, (32 if FMT in (capi.Q4_K, capi.Q6_K) else 256) * i) for i in range(m)])
+elif FMT == capi.Q5_K:  # the fifth bits
+    blocks, q, x = q5k_integer_case(n, k, 23)
+else:  # scales of 1/2 to 4 inside a run of 256
+    blocks, q, x = q4_0_integer_case(n, k, 23)
+lhs = np.stack([np.roll(x, (32 if FMT in (capi.Q4_K, capi.Q6_K, capi.Q5_K) else 256) * i) for i in range(m)])
 assert np.abs(lhs @ q.T).max() < {capi.IQ2_XXS: 2 ** 16, capi.MXFP4: 2 ** 13}.get(FMT, 2 ** 24)
-if FMT == capi.Q8_0:  # per run of 256, 1024 times the sum is still an integer that f32 holds
+if FMT in (capi.Q8_0, capi.Q4_0):  # per run of 256, 1024 times the sum is still an integer that f32 holds
     runs = np.einsum("mbe,nbe->mnb", lhs.reshape(m, -1, 256).astype(np.float64), q.reshape(n, -1, 256))
     assert np.abs(runs).max() < 2 ** 19
 got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(m, lhs.astype(np.float32))
@@ -1082,7 +1146,7 @@ lhs[1, 1234] = 3.5
 lhs[2, 512:1024] = 0.0
 got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(40, lhs)
 assert capi.last_kernel() == KERNEL
-want = oracle.matmul_t(FMT, (40, k, n), lhs, blocks, avx2=oracle.have_avx2())
+want = oracle.matmul_t(FMT, (40, k, n), lhs, blocks, avx2=AVX2)
 assert close(got[1:], want[1:]), "rows of ordinary range"
 wd = oracle.dequantize(FMT, blocks).reshape(n, k).astype(np.float64)
 x0 = lhs[0].astype(np.float64)
@@ -1097,7 +1161,7 @@ lhs = synth.normal(79, (20, k))
 lhs[3, 100] = np.inf
 lhs[7, 4000] = np.nan
 got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(20, lhs)
-want = oracle.matmul_t(FMT, (20, k, n), lhs, blocks, avx2=oracle.have_avx2())
+want = oracle.matmul_t(FMT, (20, k, n), lhs, blocks, avx2=AVX2)
 assert np.all(np.isnan(got[3])) and np.all(np.isnan(got[7]))
 ok = np.ones(20, bool); ok[[3, 7]] = False
 assert close(got[ok], want[ok])
@@ -1105,7 +1169,7 @@ print("gemm i8 ok")
 """
 
 
-@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4"])
+@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0"])
 @pytest.mark.parametrize("shape", ["8,7", "4,4"])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup
