@@ -684,6 +684,7 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
 // fewest activation rows (default: min_m_default, 64 for Q4_K, which has kernels of its own below that).
 struct GemmI8Shape {
     int nw, ng;
+    bool nsplit;  // tiles of 32 activation rows whose waves share the weight rows
 };
 
 template <class F>
@@ -708,10 +709,11 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
     // Two workgroup shapes: 256 x 112 outputs (eight waves, one workgroup a compute unit) and 128 x 64 (four
     // waves, two a compute unit), and a split over k (the parts summed by splitk_sum) when the tiles alone leave
     // compute units idle: every workgroup then walks nb / splits super-blocks.
-    static const GemmI8Shape shapes[] = {{8, 7}, {4, 4}};
+    // Up to 32 rows also: 32 x 64 (two waves that share the weight rows, two workgroups a compute unit).
+    static const GemmI8Shape shapes[] = {{8, 7, false}, {4, 4, false}, {2, 4, true}};
     const size_t nb = k / 256, groups = (m + 15) / 16;
     auto tiles_of = [&](const GemmI8Shape &sh) {
-        const size_t mt = 32 * (size_t)sh.nw, nt = 16 * (size_t)sh.ng;
+        const size_t mt = sh.nsplit ? 32 : 32 * (size_t)sh.nw, nt = 16 * (size_t)sh.ng;
         return ((m + mt - 1) / mt) * ((n + nt - 1) / nt);
     };
     if (tiles_of(shapes[1]) * std::max<size_t>(1, std::min<size_t>(nb / 4, 8)) < min_tiles) return -1;
@@ -727,7 +729,10 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
     auto estimate = [&](const GemmI8Shape &sh, size_t sp) {
         const double wgs = (double)(tiles_of(sh) * sp), nbl = (double)(nb / sp);
         double us = 3.0 + 0.0035 * (double)(nb * groups);
-        if (sh.nw == 8) us += 10.0 + nbl * (4.3 + 0.009 * std::min(wgs, 256.0)) * std::ceil(wgs / 256.0);
+        if (sh.nsplit)  // 3.1 us a super-block with 64 at work, 3.4 with 256, 4.4 with 512 (two a compute unit), in whole rounds
+            us += 3.9 + nbl * (2.95 + 0.0029 * std::min(wgs, 512.0)) *
+                            (wgs <= 512.0 ? 1.0 : wgs < 2048.0 ? std::ceil(wgs / 512.0) : wgs / 512.0);
+        else if (sh.nw == 8) us += 10.0 + nbl * (4.3 + 0.009 * std::min(wgs, 256.0)) * std::ceil(wgs / 256.0);
         else if (wgs <= 256.0) us += 3.9 + nbl * (2.3 + 0.0027 * wgs);
         else us += 3.9 + nbl * (3.1 + 0.0032 * std::min(wgs, 512.0)) * std::max(1.0, wgs / 512.0);
         if (sp > 1) us += 1.0 + 0.8 * (double)sp + (double)(sp + 1) * (double)(m * n) * 4.0 / 8.0e6;
@@ -741,6 +746,7 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
     const bool forced = shape_env && sscanf(shape_env, "%d,%d", &want_nw, &want_ng) == 2;
     for (const GemmI8Shape &sh : shapes) {
         if (forced && (sh.nw != want_nw || sh.ng != want_ng)) continue;
+        if (sh.nsplit && !forced && m > 32) continue;
         for (size_t sp = 1; sp <= 8; sp++) {
             if (nb % sp != 0 || (sp > 1 && nb / sp < 4)) continue;
             if (splits_env && sp != (size_t)atoi(splits_env)) continue;
@@ -754,14 +760,14 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
     uint8_t *acts = nullptr;
     if (scratch.get(acts_bytes + (splits > 1 ? splits * m * n * sizeof(float) : 0), s, &acts)) return 1;
     float *parts = (float *)(acts + acts_bytes);
-    const size_t mt = 32 * (size_t)best->nw, nt = 16 * (size_t)best->ng;
+    const size_t mt = best->nsplit ? 32 : 32 * (size_t)best->nw, nt = 16 * (size_t)best->ng;
     const size_t tx = (n + nt - 1) / nt, ty = (m + mt - 1) / mt;
     const size_t grid = 8 % ty == 0 ? (tx * ty + 7) / 8 * 8 : tx * ty;
     if (grid > 0x7FFFFFFFull) return -1;
     hipError_t attr_rc = hipSuccess;
-#define JQ_GEMM_I8(NW_, NG_)                                                                                          \
+#define JQ_GEMM_I8(NW_, NG_, NSPLIT_)                                                                                 \
     if (best->nw == NW_ && best->ng == NG_) {                                                                         \
-        auto kern = jq::kq_gemm_i8<F, NW_, NG_>;                                                                      \
+        auto kern = jq::kq_gemm_i8<F, NW_, NG_, false, NSPLIT_>;                                                      \
         constexpr int lds = jq::qi_lds_bytes<F, NG_>();                                                                  \
         static std::once_flag big_lds;                                                                                \
         static hipError_t rc_once = hipSuccess;                                                                       \
@@ -784,8 +790,9 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
                                    m * n, (int)splits);                                                               \
         }                                                                                                             \
     }
-    JQ_GEMM_I8(8, 7)
-    JQ_GEMM_I8(4, 4)
+    JQ_GEMM_I8(8, 7, false)
+    JQ_GEMM_I8(4, 4, false)
+    JQ_GEMM_I8(2, 4, true)
 #undef JQ_GEMM_I8
     if (attr_rc != hipSuccess) return fail("hipFuncSetAttribute: %s", hipGetErrorString(attr_rc));
     note_kernel(splits > 1 ? name_split : name);

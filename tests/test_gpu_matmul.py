@@ -1170,10 +1170,10 @@ print("gemm i8 ok")
 
 
 @pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0"])
-@pytest.mark.parametrize("shape", ["8,7", "4,4"])
+@pytest.mark.parametrize("shape", ["8,7", "4,4", "2,4"])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup
-    shape forced through the environment (read when the library first dispatches, hence the child process) both
+    shape forced through the environment (read when the library first dispatches, hence the child process) all three
     shapes run on small products: parity, ragged edges, exact integer sums, wide-range and non-finite
     activation rows."""
     import subprocess
