@@ -83,8 +83,21 @@ __device__ __forceinline__ void qi_prep_record(const float (&v)[16], uint8_t *__
         sum = isum_xor16(sum);  // the two lane groups of a sub-block
         if ((g & 1) == 0) xs_sh[i][2 * c + (g >> 1)] = sum;
     }
-    *(uint4 *)(rec + ((size_t)(2 * c) * 64 + lane) * 16) = uint4{h[0], h[1], h[2], h[3]};
-    *(uint4 *)(rec + ((size_t)(2 * c + 1) * 64 + lane) * 16) = uint4{l[0], l[1], l[2], l[3]};
+    // word w of chunk c at position (w + c) % 4, as in the weight tiles (qi_word)
+    auto rotated = [&](const uint32_t (&v)[4]) {
+        uint32_t a0 = v[0], a1 = v[1], a2 = v[2], a3 = v[3];
+        if (c & 1) {
+            const uint32_t t = a3;
+            a3 = a2, a2 = a1, a1 = a0, a0 = t;
+        }
+        if (c & 2) {
+            const uint32_t t0 = a0, t1 = a1;
+            a0 = a2, a1 = a3, a2 = t0, a3 = t1;
+        }
+        return uint4{a0, a1, a2, a3};
+    };
+    *(uint4 *)(rec + ((size_t)(2 * c) * 64 + lane) * 16) = rotated(h);
+    *(uint4 *)(rec + ((size_t)(2 * c + 1) * 64 + lane) * 16) = rotated(l);
     __syncthreads();
     if (tid < 64) {
         uint32_t w[4] = {0, 0, 0, 0};
@@ -224,6 +237,12 @@ constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * F::META) + F
 
 typedef short qi_s2 __attribute__((ext_vector_type(2)));
 
+// Where word wi (elements 4 wi .. + 3) of a lane's 16 operand bytes of chunk uc goes: rotated by the chunk
+// number, in the weight tiles and in the activation records alike (the MFMA sums over a lane's 16 elements, so
+// their order is free as long as both operands agree).  The four threads of a weight row unpack its four chunks
+// at once, and unrotated their stores fall on the same LDS bank (the chunks are 2048 bytes apart).
+__device__ __forceinline__ int qi_word(int uc, int wi) { return 4 * ((wi + uc) & 3); }
+
 // A format's side of the GEMM.  A thread's unit is (weight row, 64-k chunk uc) of a super-block at `blk`:
 // fetch() takes its bytes in three parts (0: the scales, into `next`, 1, 2: the halves of the chunk's
 // packed bytes), take() makes the scales fetched ahead current, piece(j) turns the bytes of elements
@@ -260,8 +279,8 @@ struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 
             const uint32_t even = __umul24(w & 0x000F000Fu, sc[nib]) + 0x00800080u;
             const uint32_t odd = __umul24((w >> 8) & 0x000F000Fu, sc[nib]) + 0x00800080u;
             const int gg = 2 * nib + (j >> 2);
-            *(uint32_t *)(tile + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {  // the min scales, d and dmin
@@ -320,8 +339,8 @@ struct QiQ6K {
             const qi_s2 even = __builtin_bit_cast(qi_s2, q & 0x00FF00FFu) * qi_s2{sc, sc} + qi_s2{bias, bias};
             const qi_s2 odd = __builtin_bit_cast(qi_s2, (q >> 8) & 0x00FF00FFu) * qi_s2{sc, sc} + qi_s2{bias, bias};
             const uint32_t ev = __builtin_bit_cast(uint32_t, even), od = __builtin_bit_cast(uint32_t, odd);
-            *(uint32_t *)(tile + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(od, ev, 0x07030501u);
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(od, ev, 0x06020400u) ^ 0x80808080u;
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(od, ev, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(od, ev, 0x06020400u) ^ 0x80808080u;
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
@@ -368,7 +387,7 @@ struct QiQ2K {
         for (int e = 0; e < 2; e++) {  // slices half and 2 + half: the same bytes, the next field
             const int gg = 2 * e + half;
             const uint32_t q = (word >> (2 * e)) & 0x03030303u;
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(0u, raw.table[gg], q);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(0u, raw.table[gg], q);
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
@@ -431,8 +450,8 @@ struct QiQ8_0 {
                 t[b] = __builtin_bit_cast(uint32_t, fmaf((float)(int)(int8_t)(word >> (8 * b)), ratio, 12583040.0f));
             const uint32_t even = __builtin_amdgcn_perm(t[2], t[0], 0x05040100u), odd = __builtin_amdgcn_perm(t[3], t[1], 0x05040100u);
             const int gg = 2 * e32 + half;
-            *(uint32_t *)(tile + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
@@ -505,8 +524,8 @@ struct QiIQ2XXS {
             const uint32_t nib = (raw.signs[grp] >> (8 * l + 4 * hf)) & 15u;
             const uint32_t sel = ((mag >> 4) & 0x03030303u) | (((nib * 0x00204081u) & 0x01010101u) << 2);
             const int gg = 2 * grp + half;
-            *(uint32_t *)(tile + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(raw.th[grp][1], raw.th[grp][0], sel);
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = __builtin_amdgcn_perm(raw.tl[grp][1], raw.tl[grp][0], sel);
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(raw.th[grp][1], raw.th[grp][0], sel);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(raw.tl[grp][1], raw.tl[grp][0], sel);
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
@@ -603,8 +622,8 @@ struct QiNibbles32 {
             const uint32_t l0 = __builtin_amdgcn_perm(raw.tl[blk][1], raw.tl[blk][0], sel);
             const uint32_t l1 = __builtin_amdgcn_perm(raw.tl[blk][3], raw.tl[blk][2], sel);
             const int gg = 2 * blk + half;
-            *(uint32_t *)(tile + gg * 256 + 4 * wi) = (h1 & top) | (h0 & ~top);
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * wi) = (l1 & top) | (l0 & ~top);
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, wi)) = (h1 & top) | (h0 & ~top);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, wi)) = (l1 & top) | (l0 & ~top);
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
@@ -646,8 +665,8 @@ struct QiQ5K {
             const uint32_t even = __umul24(q & 0x00FF00FFu, sc[nib]) + 0x00800080u;
             const uint32_t odd = __umul24((q >> 8) & 0x00FF00FFu, sc[nib]) + 0x00800080u;
             const int gg = 2 * nib + (j >> 2);
-            *(uint32_t *)(tile + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
-            *(uint32_t *)(tile + 1024 + gg * 256 + 4 * (j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, j & 3)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, j & 3)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
