@@ -331,6 +331,9 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
                                                              False, 0, 0.0)
         elif only == "moe_v3":
             out["moe_deepseek_v3_iq2_xxs_b1"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 1, 105, steps, True, 1, 0.0)
+        elif only == "moe_v3_b512":  # a 512-token call of the same layer: the grouped int8 GEMM
+            out["moe_deepseek_v3_iq2_xxs_b512"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 512, 105, max(steps // 10, 5),
+                                                               True, 1, 0.0)
         elif only == "moe_v3_mxfp4":
             out["moe_deepseek_v3_mxfp4_b1"] = moe_workload(torch, capi, synth, 39, 7168, 2048, 256, 8, 1, 105, steps, True, 1, 0.0)
         return out
