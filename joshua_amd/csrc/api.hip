@@ -1763,10 +1763,19 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         const int in_lds = (size_t)P <= 12288;
         const size_t chunks = ((size_t)P + 63) / 64, rank_ints = chunks * c.n_expert + c.n_expert + 1;
         static const char *no_ranked = getenv("JQ_MOE_NO_RANKED_GROUPING");
-        if (!no_ranked && chunks <= (size_t)jq::GROUP_RANK_CHUNKS && rank_ints <= 12288)
+        // (its rank table: chunks x experts ints of LDS, up to 144 KB)
+        if (!no_ranked && chunks <= (size_t)jq::GROUP_RANK_CHUNKS && rank_ints <= 36864) {
+            static std::once_flag big_lds;
+            static hipError_t attr_rc = hipSuccess;
+            std::call_once(big_lds, [&] {
+                attr_rc = hipFuncSetAttribute((const void *)jq::moe_group_pairs_ranked, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              36864 * (int)sizeof(int));
+            });
+            HIP_TRY(attr_rc);
             hipLaunchKernelGGL(jq::moe_group_pairs_ranked, dim3(1), dim3(jq::GROUP_PAIRS_THREADS), rank_ints * sizeof(int), s,
                                m->ids, (int)T, (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow,
                                extra);
+        }
         else
             hipLaunchKernelGGL(jq::moe_group_pairs, dim3(1), dim3(jq::GROUP_PAIRS_THREADS), (c.n_expert + 1 + (in_lds ? P : 0)) * sizeof(int), s,
                                m->ids, (int)T, (int)c.n_expert_used, (int)c.n_expert, m->gexp, m->offsets, m->xrow, m->yrow,

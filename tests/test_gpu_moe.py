@@ -115,7 +115,8 @@ def test_row_lengths_that_change_the_staging(qtype, h, inter):
         assert close(dev.forward(x), ora.forward(x))
 
 
-@pytest.mark.parametrize("tokens,E,k", [(300, 16, 4), (1000, 16, 4), (1024, 24, 4), (1100, 16, 4), (150, 160, 6)])
+@pytest.mark.parametrize("tokens,E,k", [(300, 16, 4), (1000, 16, 4), (1024, 24, 4), (1100, 16, 4), (150, 160, 6),
+                                        (500, 200, 8)])   # the last: a rank table of more than 64 KB
 def test_many_tokens_are_grouped_by_expert_in_pair_order(tokens, E, k):
     """Pair lists of up to 4096 pairs are grouped by ranks within chunks of 64 pairs (one to four chunks a
     wave, a last chunk part empty, experts nobody picked); longer lists, or more chunks x experts than the
