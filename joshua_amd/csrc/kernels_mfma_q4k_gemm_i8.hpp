@@ -245,7 +245,8 @@ __device__ __forceinline__ int qi_word(int uc, int wi) { return 4 * ((wi + uc) &
 
 // A format's side of the GEMM.  A thread's unit is (weight row, 64-k chunk uc) of a super-block at `blk`:
 // fetch() takes its bytes in three parts (0: the scales, into `next`, 1, 2: the halves of the chunk's
-// packed bytes), take() makes the scales fetched ahead current, piece(j) turns the bytes of elements
+// packed bytes), take() makes the scales fetched ahead current (and builds what depends on them alone),
+// piece(j) turns the bytes of elements
 // 16 g + 4 (j % 4) .. + 3 of slices g = j / 4 and 2 + j / 4 into operand words (p + 128 = 256 Ph + L,
 // Pl = L - 128; slice g of the chunk at tile + 256 g, plane Pl 1024 bytes further), meta() writes the
 // row's 48 bytes.
@@ -264,7 +265,7 @@ struct QiQ4K {  // w = d sc q - dmin m, 6-bit sc and m, q in 0..15: p = sc q in 
         if (part == 1) raw.q0 = *(const uint4 *)(blk + 16 + 32 * uc);
         if (part == 2) raw.q1 = *(const uint4 *)(blk + 32 + 32 * uc);
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) { raw.hdr = next; }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) { raw.hdr = next; }
     __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
         const uint4 hdr = raw.hdr.h;
         const uint32_t scl = hdr.y & 0x3F3F3F3Fu, sch = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
@@ -321,7 +322,7 @@ struct QiQ6K {
             raw.hv[part - 1] = ldw<uint4>(blk + 128 + 32 * h + o);
         }
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) { raw.hdr = next; }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) { raw.hdr = next; }
     __device__ __forceinline__ static uint32_t word_of(const uint4 &v, int i) {
         return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
     }
@@ -371,7 +372,7 @@ struct QiQ2K {
         if (part == 1) raw.q0 = ld<uint4>(blk + 16 + 32 * (uc >> 1));
         if (part == 2) raw.q1 = ld<uint4>(blk + 32 + 32 * (uc >> 1));
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) {
         raw.hdr = next;
 #pragma unroll
         for (int gg = 0; gg < 4; gg++) {
@@ -429,7 +430,7 @@ struct QiQ8_0 {
             raw.qb[part - 1] = ldw<uint4>(blk + 68 * uc + 36 + 16 * (part - 1));
         }
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) {
         float D = fmaxf(mag_or_inf(next.d0), mag_or_inf(next.d1));
         D = fmaxf(D, dpp_f<0xB1>(D));  // quad_perm [1,0,3,2]
         D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
@@ -486,7 +487,7 @@ struct QiIQ2XXS {
         if (part == 0) next.d = ld<uint16_t>(blk);
         if (part == 2) raw.q = ldw<uint4>(blk + 2 + 16 * uc);
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) {
         raw.unit = f16_bits(next.d) * 0.125f;
         const uint32_t w[4] = {raw.q.x, raw.q.y, raw.q.z, raw.q.w};
 #pragma unroll
@@ -581,7 +582,7 @@ struct QiNibbles32 {
         if (part == 1) raw.na = ldw<uint4>(pair + T::HEAD);
         if (part == 2) raw.nb = ldw<uint4>(pair + T::BYTES + T::HEAD);
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) {
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) {
         float D = fmaxf(mag_or_inf(next.d0), mag_or_inf(next.d1));
         D = fmaxf(D, dpp_f<0xB1>(D));  // quad_perm [1,0,3,2]
         D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
@@ -650,7 +651,7 @@ struct QiQ5K {
         if (part == 1) raw.q0 = *(const uint4 *)(blk + 48 + 32 * uc), raw.h0 = *(const uint4 *)(blk + 16);
         if (part == 2) raw.q1 = *(const uint4 *)(blk + 64 + 32 * uc), raw.h1 = *(const uint4 *)(blk + 32);
     }
-    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, const uint8_t *) { raw.hdr = next; }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) { raw.hdr = next; }
     __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
         const uint4 hdr = raw.hdr.h;
         const uint32_t scl = hdr.y & 0x3F3F3F3Fu, sch = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
@@ -673,6 +674,76 @@ struct QiQ5K {
         QiQ4K::Raw as_q4k;
         as_q4k.hdr = raw.hdr;
         QiQ4K::meta(as_q4k, uc, meta);
+    }
+};
+
+// Q3_K: hmask[32] | qs[64] | scales[12] | d, w = d (sc - 32) (q - (hbit ? 0 : 4)) over sub-blocks of 16: element
+// 128 h + 32 t + 16 hf + i is field t of qs[32 h + 16 hf + i] with bit 4 h + t of hmask[16 hf + i] as its
+// third bit and the 6-bit scale number 8 h + 2 t + hf, low four bits in scales[0..7] (a nibble each, the first
+// eight scales low, the next eight high), high two bits in scales[8..11]
+// (vendor/candle-metal-kernels/src/metal_src/quantized.metal:151-156, 6597-6623).  With v = q + 4 hbit in
+// 0..7 the weight is d s (v - 4), s = sc - 32 in -32..31: p = s (v - 4) in -124..128, two bytes (Ph is 0 or 1),
+// no min term.  Chunk uc is half h = uc / 2, fields 2 (uc % 2) and 2 (uc % 2) + 1: slice gg of 16 is field
+// 2 (uc % 2) + gg / 2 of bytes 16 (gg % 2) .., scale number 4 uc + gg.  Per slice the eight products make one
+// 8-byte table a plane; one v_perm_b32 a plane looks four elements up with selector v.  Blocks of 110 bytes
+// sit at even addresses only: read through aligned words.
+struct QiQ3K {
+    static constexpr int BLOCK = 110, META = 48, ALIGN = 2, TABLE = 0;
+    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
+    struct Hdr {
+        uint32_t s0, s1, s2, d;
+    };
+    struct Raw {
+        float d;
+        uint32_t th[4][2], tl[4][2];  // per slice: Ph and Pl of s (v - 4), v = 0..3 and 4..7
+        uint4 q[2], m[2];             // qs[32 h + 16 hf ..] and hmask[16 hf ..], hf = 0, 1
+    };
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        if (part == 0) {
+            next.s0 = ldw<uint32_t>(blk + 96), next.s1 = ldw<uint32_t>(blk + 100), next.s2 = ldw<uint32_t>(blk + 104);
+            next.d = ld<uint16_t>(blk + 108);
+        }
+        if (part == 1 || part == 2) {
+            raw.q[part - 1] = ldw<uint4>(blk + 32 + 32 * (uc >> 1) + 16 * (part - 1));
+            raw.m[part - 1] = ldw<uint4>(blk + 16 * (part - 1));
+        }
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &hdr, int uc, const uint8_t *) {
+        raw.d = f16_bits(hdr.d);
+        const uint32_t lw = (uc & 1) ? hdr.s1 : hdr.s0;
+        const uint32_t sc6 = ((uc < 2 ? lw : lw >> 4) & 0x0F0F0F0Fu) | (((hdr.s2 >> (2 * uc)) & 0x03030303u) << 4);
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) {
+            const short sc = (short)((int)((sc6 >> (8 * gg)) & 0xFFu) - 32);
+            // s (v - 4) + 128 for v = 0..7 as signed halfwords, two an instruction
+            const qi_s2 step2 = {(short)(2 * sc), (short)(2 * sc)};
+            const qi_s2 v01 = {(short)(128 - 4 * sc), (short)(128 - 3 * sc)};
+            const qi_s2 v23 = v01 + step2, v45 = v23 + step2, v67 = v45 + step2;
+            const uint32_t a = __builtin_bit_cast(uint32_t, v01), b = __builtin_bit_cast(uint32_t, v23);
+            const uint32_t c = __builtin_bit_cast(uint32_t, v45), e = __builtin_bit_cast(uint32_t, v67);
+            raw.tl[gg][0] = __builtin_amdgcn_perm(b, a, 0x06040200u) ^ 0x80808080u;
+            raw.th[gg][0] = __builtin_amdgcn_perm(b, a, 0x07050301u);
+            raw.tl[gg][1] = __builtin_amdgcn_perm(e, c, 0x06040200u) ^ 0x80808080u;
+            raw.th[gg][1] = __builtin_amdgcn_perm(e, c, 0x07050301u);
+        }
+    }
+    __device__ __forceinline__ static uint32_t word_of(const uint4 &v, int i) {
+        return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
+    }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
+        const int hf = j >> 2, wi = j & 3;
+        const uint32_t word = word_of(raw.q[hf], wi) >> (4 * (uc & 1));
+        const uint32_t high = word_of(raw.m[hf], wi) >> (4 * (uc >> 1) + 2 * (uc & 1));
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {  // slices hf and 2 + hf: the same bytes, the next field
+            const int gg = 2 * tt + hf;
+            const uint32_t v = ((word >> (2 * tt)) & 0x03030303u) | (((high >> tt) & 0x01010101u) << 2);
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(raw.th[gg][1], raw.th[gg][0], v);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(raw.tl[gg][1], raw.tl[gg][0], v);
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        *(float2 *)(meta + 32) = float2{raw.d, 0.0f};  // the same from all four
     }
 };
 
@@ -767,7 +838,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
     };
     auto take_header = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int p = 0; p < PER; p++) F::take(raw[p], hdr_next[p], tab);
+        for (int p = 0; p < PER; p++) F::take(raw[p], hdr_next[p], uc, tab);
     };
 
     fetch_part(0, 0), fetch_part(0, 1), fetch_part(0, 2);

@@ -368,6 +368,42 @@ def q4_0_integer_case(n, k, seed, nonzero=16, small=400):
     return blocks, w, x
 
 
+def q3k_integer_case(n, k, seed):
+    """Q3_K blocks with d = 1: random 2-bit fields, third bits and 6-bit scales, so w = (sc - 32) (q - (hbit ? 0 :
+    4)) in integers up to 128 in magnitude (scale 33 in the sub-block that holds the activations' peak);
+    activations in multiples of 2^-8: -1, 0 or 1 of them, and 32639 of them at one slot of every 256.  Returns
+    (blocks, weights, activations as float64)."""
+    rng = np.random.default_rng(seed)
+    slot = int(rng.integers(0, 256))
+    nb = k // 256
+    q2 = rng.integers(0, 4, size=(n, nb, 2, 4, 2, 16))            # [h][t][hf][i]: element 128 h + 32 t + 16 hf + i
+    hb = rng.integers(0, 2, size=(n, nb, 2, 4, 2, 16))
+    sc = rng.integers(0, 64, size=(n, nb, 16))                    # scale number 8 h + 2 t + hf
+    h, t, hf = slot // 128, (slot % 128) // 32, (slot % 32) // 16
+    sc[:, :, 8 * h + 2 * t + hf] = 33
+    blocks = np.zeros((n, nb, 110), np.uint8)
+    qs = np.zeros((n, nb, 2, 2, 16), np.int64)                    # [h][hf][i]
+    hm = np.zeros((n, nb, 2, 16), np.int64)                       # [hf][i]
+    for hh in range(2):
+        for tt in range(4):
+            qs[:, :, hh] |= q2[:, :, hh, tt] << (2 * tt)
+            hm |= hb[:, :, hh, tt] << (4 * hh + tt)
+    blocks[:, :, 0:32] = hm.reshape(n, nb, 32)
+    blocks[:, :, 32:96] = qs.reshape(n, nb, 64)
+    low, high = sc & 15, sc >> 4
+    blocks[:, :, 96:104] = low[:, :, :8] | (low[:, :, 8:] << 4)
+    for b in range(4):
+        blocks[:, :, 104 + b] = high[:, :, b] | (high[:, :, 4 + b] << 2) | (high[:, :, 8 + b] << 4) | (high[:, :, 12 + b] << 6)
+    blocks[:, :, 108:110] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks = blocks.reshape(-1)
+    scale = sc.reshape(n, nb, 2, 4, 2)[..., None] - 32            # [h][t][hf] broadcast over i
+    w = (scale * (q2 - 4 * (1 - hb))).reshape(n, k).astype(np.float64)
+    assert np.array_equal(oracle.dequantize(capi.Q3_K, blocks).reshape(n, k), w.astype(np.float32))
+    x = rng.integers(-1, 2, size=k).astype(np.float64)
+    x[slot::256] = 32639 * rng.choice([-1, 1], size=k // 256)
+    return blocks, w, x / 256.0
+
+
 def test_q6k_dot4_integer_dot_products_are_bit_exact():
     """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
     scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
@@ -447,7 +483,7 @@ def test_few_rows_against_a_large_matrix_take_the_int8_gemm(qtype, m, k, n):
     assert np.array_equal(got, w.matmul_t(m, lhs))
 
 
-@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q5_0, 8, 12288, 1024), (capi.Q4_1, 16, 4096, 2100), (capi.Q3_K, 11, 7168, 1200),
+@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q5_0, 8, 12288, 1024), (capi.Q4_1, 16, 4096, 2100), (capi.Q5_1, 11, 7168, 1200),
                                          (capi.Q6_K, 512, 2048, 100), (capi.IQ2_XXS, 40, 5120, 300)])
 def test_decoded_weights_gemm_split_over_k(qtype, m, k, n):
     """8..16 rows against matrices of 8M elements or more, and many rows against few weight rows: the GEMM's
@@ -1072,11 +1108,12 @@ sys.path.insert(0, %r)
 import oracle
 from joshua_amd import capi, synth
 from tests.test_gpu_matmul import (q4k_integer_case, q6k_integer_case, q2k_integer_case, q8_0_integer_case,
-                                   iq2xxs_integer_case, mxfp4_integer_case, q5k_integer_case, q4_0_integer_case, close)
+                                   iq2xxs_integer_case, mxfp4_integer_case, q5k_integer_case, q4_0_integer_case,
+                                   q3k_integer_case, close)
 FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8"), "q2k": (capi.Q2_K, "q2k_gemm_i8"),
                "q8_0": (capi.Q8_0, "q8_0_gemm_i8"), "iq2xxs": (capi.IQ2_XXS, "iq2xxs_gemm_i8"),
                "mxfp4": (capi.MXFP4, "mxfp4_gemm_i8"), "q5k": (capi.Q5_K, "q5k_gemm_i8"),
-               "q4_0": (capi.Q4_0, "q4_0_gemm_i8")}[sys.argv[1]]
+               "q4_0": (capi.Q4_0, "q4_0_gemm_i8"), "q3k": (capi.Q3_K, "q3k_gemm_i8")}[sys.argv[1]]
 _synth = synth
 class _Synth:  # the formats without a quantiser of normal weights get random blocks
     normal = staticmethod(_synth.normal)
@@ -1122,10 +1159,12 @@ elif FMT == capi.MXFP4:  # dense weights in multiples of 1/8 under scales of 1/4
     blocks, q, x = mxfp4_integer_case(n, k, 23)
 elif FMT == capi.Q5_K:  # the fifth bits
     blocks, q, x = q5k_integer_case(n, k, 23)
-else:  # scales of 1/2 to 4 inside a run of 256
+elif FMT == capi.Q4_0:  # scales of 1/2 to 4 inside a run of 256
     blocks, q, x = q4_0_integer_case(n, k, 23)
+else:  # every scale, field and third bit: dense integer weights up to 128
+    blocks, q, x = q3k_integer_case(n, k, 23)
 lhs = np.stack([np.roll(x, (32 if FMT in (capi.Q4_K, capi.Q6_K, capi.Q5_K) else 256) * i) for i in range(m)])
-assert np.abs(lhs @ q.T).max() < {capi.IQ2_XXS: 2 ** 16, capi.MXFP4: 2 ** 13}.get(FMT, 2 ** 24)
+assert np.abs(lhs @ q.T).max() < {capi.IQ2_XXS: 2 ** 16, capi.Q3_K: 2 ** 16, capi.MXFP4: 2 ** 13}.get(FMT, 2 ** 24)
 if FMT in (capi.Q8_0, capi.Q4_0):  # per run of 256, 1024 times the sum is still an integer that f32 holds
     runs = np.einsum("mbe,nbe->mnb", lhs.reshape(m, -1, 256).astype(np.float64), q.reshape(n, -1, 256))
     assert np.abs(runs).max() < 2 ** 19
@@ -1169,7 +1208,7 @@ print("gemm i8 ok")
 """
 
 
-@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0"])
+@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0", "q3k"])
 @pytest.mark.parametrize("shape", ["8,7", "4,4", "2,4"])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup
