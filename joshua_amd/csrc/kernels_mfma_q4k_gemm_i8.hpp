@@ -677,6 +677,65 @@ struct QiQ5K {
     }
 };
 
+// Q5_0: blocks of d (f16) | qh (32 fifth bits) | 16 code bytes, w = d (q - 16) with q the nibble and bit j (low
+// nibbles, elements 0..15) or 16 + j (high nibbles, elements 16..31) of qh as its fifth bit
+// (vendor/candle-metal-kernels/src/metal_src/quantized.metal:98-102); a "super-block" here is eight blocks, 176
+// bytes, put on one scale as for Q8_0: p = round(1024 (q - 16) d / D), within +-16384 whatever the sign of d.
+// The four fifth bits of a word are spread to bytes with a multiply, q - 16 becomes a signed byte without
+// carries between bytes ((q | 0x80) - 0x10, then the top bit flipped back), and the product goes the way of
+// Q8_0's.  Blocks sit at even addresses only: read through aligned words.
+struct QiQ5_0 {
+    static constexpr int BLOCK = 176, META = 48, ALIGN = 2, TABLE = 0;
+    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
+    struct Hdr {
+        float d0, d1;
+    };
+    struct Raw {
+        float r0, r1, unit;  // 1024 d / D of the chunk's two blocks, and D / 1024
+        uint32_t ha, hb;     // the fifth bits of block 2 uc and of block 2 uc + 1
+        uint4 qa, qb;        // their code bytes
+        uint32_t hna, hnb;   // the same of the next super-block (every piece reads all 16 bytes of a block, so the
+        uint4 na, nb;        // bytes fetched ahead wait here until take())
+    };
+    __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
+        const uint8_t *pair = blk + 44 * uc;
+        if (part == 0) next.d0 = f16_bits(ld<uint16_t>(pair)), next.d1 = f16_bits(ld<uint16_t>(pair + 22));
+        if (part == 1) raw.hna = ldw<uint32_t>(pair + 2), raw.na = ldw<uint4>(pair + 6);
+        if (part == 2) raw.hnb = ldw<uint32_t>(pair + 24), raw.nb = ldw<uint4>(pair + 28);
+    }
+    __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) {
+        float D = fmaxf(mag_or_inf(next.d0), mag_or_inf(next.d1));
+        D = fmaxf(D, dpp_f<0xB1>(D));  // quad_perm [1,0,3,2]
+        D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
+        const float inv = D > 0.0f ? 1024.0f / D : 0.0f;
+        raw.r0 = next.d0 * inv, raw.r1 = next.d1 * inv, raw.unit = D * (1.0f / 1024.0f);
+        raw.ha = raw.hna, raw.hb = raw.hnb, raw.qa = raw.na, raw.qb = raw.nb;
+    }
+    __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
+        const int half = j >> 2, wi = j & 3;
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {  // elements 16 half + 4 wi .. + 3 of both blocks
+            const uint4 qv = blk ? raw.qb : raw.qa;
+            const uint32_t word = (wi == 0 ? qv.x : wi == 1 ? qv.y : wi == 2 ? qv.z : qv.w) >> (4 * half);
+            const uint32_t fifth = (((blk ? raw.hb : raw.ha) >> (16 * half + 4 * wi)) & 15u) * 0x00204081u & 0x01010101u;
+            const uint32_t q = (word & 0x0F0F0F0Fu) | (fifth << 4);
+            const uint32_t sb = ((q | 0x80808080u) - 0x10101010u) ^ 0x80808080u;  // q - 16 as signed bytes
+            const float ratio = blk ? raw.r1 : raw.r0;
+            uint32_t t[4];
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                t[b] = __builtin_bit_cast(uint32_t, fmaf((float)(int)(int8_t)(sb >> (8 * b)), ratio, 12583040.0f));
+            const uint32_t even = __builtin_amdgcn_perm(t[2], t[0], 0x05040100u), odd = __builtin_amdgcn_perm(t[3], t[1], 0x05040100u);
+            const int gg = 2 * blk + half;
+            *(uint32_t *)(tile + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(odd, even, 0x07030501u);
+            *(uint32_t *)(tile + 1024 + gg * 256 + qi_word(uc, wi)) = __builtin_amdgcn_perm(odd, even, 0x06020400u) ^ 0x80808080u;
+        }
+    }
+    __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
+        *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+    }
+};
+
 // Q3_K: hmask[32] | qs[64] | scales[12] | d, w = d (sc - 32) (q - (hbit ? 0 : 4)) over sub-blocks of 16: element
 // 128 h + 32 t + 16 hf + i is field t of qs[32 h + 16 hf + i] with bit 4 h + t of hmask[16 hf + i] as its
 // third bit and the 6-bit scale number 8 h + 2 t + hf, low four bits in scales[0..7] (a nibble each, the first
