@@ -934,7 +934,7 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         const int rc = dispatch_gemm_i8<jq::QiQ4K>(W, row_bytes, X, Y, m, k, n, s, "q4k_gemm_i8", "q4k_gemm_i8+splitk");
         if (rc >= 0) return rc;
     }
-    // Q6_K, Q2_K, Q8_0, IQ2_XXS, MXFP4, Q5_K, Q4_0, Q3_K, Q5_0: the same GEMM wherever the MFMA GEMM over decoded weights would run otherwise (from 17
+    // every other format (Q6_K, Q2_K, Q8_0, IQ2_XXS, MXFP4, Q5_K, Q4_0, Q3_K, Q5_0, Q4_1, Q5_1): the same GEMM wherever the MFMA GEMM over decoded weights would run otherwise (from 17
     // rows on, and from JQ_DECODED_GEMM_MIN_M rows on against matrices of 8M elements or more)
     static const char *dec_min_m_env = getenv("JQ_DECODED_GEMM_MIN_M");
     static const size_t gemm_min_m = dec_min_m_env ? (size_t)std::max(atoi(dec_min_m_env), 2) : 8;
@@ -965,6 +965,14 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     }
     if (type == JQ_TYPE_Q5_0 && many_rows) {
         const int rc = dispatch_gemm_i8<jq::QiQ5_0>(W, row_bytes, X, Y, m, k, n, s, "q5_0_gemm_i8", "q5_0_gemm_i8+splitk", false, 2);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q4_1 && many_rows) {
+        const int rc = dispatch_gemm_i8<jq::QiQ4_1>(W, row_bytes, X, Y, m, k, n, s, "q4_1_gemm_i8", "q4_1_gemm_i8+splitk", false, 2);
+        if (rc >= 0) return rc;
+    }
+    if (type == JQ_TYPE_Q5_1 && many_rows) {
+        const int rc = dispatch_gemm_i8<jq::QiQ5_1>(W, row_bytes, X, Y, m, k, n, s, "q5_1_gemm_i8", "q5_1_gemm_i8+splitk", false, 2);
         if (rc >= 0) return rc;
     }
     if (type == JQ_TYPE_Q4_0 && many_rows) {
@@ -1362,7 +1370,8 @@ bool moe_has_gemm_i8(uint32_t type) {
     static const char *off = getenv("JQ_MOE_NO_GEMM_I8");
     if (off) return false;
     return type == JQ_TYPE_Q4_K || type == JQ_TYPE_Q6_K || type == JQ_TYPE_Q2_K || type == JQ_TYPE_Q8_0 ||
-           type == JQ_TYPE_IQ2_XXS || type == JQ_TYPE_MXFP4 || type == JQ_TYPE_Q5_K || type == JQ_TYPE_Q4_0 || type == JQ_TYPE_Q3_K || type == JQ_TYPE_Q5_0;
+           type == JQ_TYPE_IQ2_XXS || type == JQ_TYPE_MXFP4 || type == JQ_TYPE_Q5_K || type == JQ_TYPE_Q4_0 || type == JQ_TYPE_Q3_K || type == JQ_TYPE_Q5_0 || type == JQ_TYPE_Q4_1 ||
+           type == JQ_TYPE_Q5_1;
 }
 
 int moe_reserve(jq_moe *m, size_t T) {
@@ -1724,6 +1733,8 @@ int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, s
         JQ_QI_CASE(JQ_TYPE_Q4_0, QiQ4_0)
         JQ_QI_CASE(JQ_TYPE_Q3_K, QiQ3K)
         JQ_QI_CASE(JQ_TYPE_Q5_0, QiQ5_0)
+        JQ_QI_CASE(JQ_TYPE_Q4_1, QiQ4_1)
+        JQ_QI_CASE(JQ_TYPE_Q5_1, QiQ5_1)
 #undef JQ_QI_CASE
     default: return -1;
     }

@@ -547,7 +547,9 @@ struct QiIQ2XXS {
 //   Q4_0: d (f16) | codes, w = d (code - 8) (vendor/candle-metal-kernels/src/metal_src/quantized.metal:86-89).
 struct QtMXFP4 {
     static constexpr int BYTES = 17, HEAD = 1, ALIGN = 1;
+    static constexpr bool HAS_OFFSET = false;
     static constexpr float UNIT = 1.0f / 4096.0f;
+    __device__ __forceinline__ static float offset_of(const uint8_t *) { return 0.0f; }
     __device__ __forceinline__ static float scale_of(const uint8_t *blk) {
         const uint32_t e = blk[0];
         return e == 0xFFu ? 0.0f : __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
@@ -559,26 +561,40 @@ struct QtMXFP4 {
 };
 struct QtQ4_0 {
     static constexpr int BYTES = 18, HEAD = 2, ALIGN = 2;
+    static constexpr bool HAS_OFFSET = false;
     static constexpr float UNIT = 1.0f / 2048.0f;
     __device__ __forceinline__ static float scale_of(const uint8_t *blk) { return f16_bits(ld<uint16_t>(blk)); }
+    __device__ __forceinline__ static float offset_of(const uint8_t *) { return 0.0f; }
     __device__ __forceinline__ static constexpr float value(int code) { return (float)(code - 8); }
+};
+//   Q4_1: d (f16) | m (f16) | codes, w = d code + m (quantized.metal:91-95): the offsets are the min term.
+struct QtQ4_1 {
+    static constexpr int BYTES = 20, HEAD = 4, ALIGN = 2;
+    static constexpr bool HAS_OFFSET = true;
+    static constexpr float UNIT = 1.0f / 2048.0f;
+    __device__ __forceinline__ static float scale_of(const uint8_t *blk) { return f16_bits(ld<uint16_t>(blk)); }
+    __device__ __forceinline__ static float offset_of(const uint8_t *blk) { return f16_bits(ld<uint16_t>(blk + 2)); }
+    __device__ __forceinline__ static constexpr float value(int code) { return (float)code; }
 };
 template <class T>
 struct QiNibbles32 {
     static constexpr int BLOCK = 8 * T::BYTES, META = 48, ALIGN = T::ALIGN, TABLE = 0;
-    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
+    static constexpr bool HAS_MIN = T::HAS_OFFSET, MIN_F16 = T::HAS_OFFSET, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
-        float d0, d1;
+        float d0, d1, m0, m1;
     };
     struct Raw {
-        float unit;
+        float unit, m0, m1;
         uint32_t th[2][4], tl[2][4];  // per block: Ph / Pl of codes 0..7 (words 0, 1) and of codes 8..15 (words 2, 3)
         uint4 qa, qb;                 // the codes of block 2 uc and of block 2 uc + 1
         uint4 na, nb;                 // the same of the next super-block
     };
     __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
         const uint8_t *pair = blk + 2 * T::BYTES * uc;
-        if (part == 0) next.d0 = T::scale_of(pair), next.d1 = T::scale_of(pair + T::BYTES);
+        if (part == 0) {
+            next.d0 = T::scale_of(pair), next.d1 = T::scale_of(pair + T::BYTES);
+            next.m0 = T::offset_of(pair), next.m1 = T::offset_of(pair + T::BYTES);
+        }
         if (part == 1) raw.na = ldw<uint4>(pair + T::HEAD);
         if (part == 2) raw.nb = ldw<uint4>(pair + T::BYTES + T::HEAD);
     }
@@ -589,6 +605,7 @@ struct QiNibbles32 {
         const bool live = D >= 7.888609052210118e-31f;  // 2^-100
         const float inv = live ? 2048.0f / D : 0.0f;
         raw.unit = live ? D * T::UNIT : 0.0f;
+        raw.m0 = next.m0, raw.m1 = next.m1;
         raw.qa = raw.na, raw.qb = raw.nb;
 #pragma unroll
         for (int blk = 0; blk < 2; blk++) {
@@ -628,11 +645,19 @@ struct QiNibbles32 {
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
-        *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+        if constexpr (T::HAS_OFFSET) {  // the chunk's two offsets among m_0..7, zeros in the second sixteen bytes
+            const qi_h2 m = {(_Float16)raw.m0, (_Float16)raw.m1};
+            *(uint32_t *)(meta + 4 * uc) = __builtin_bit_cast(uint32_t, m);
+            *(uint32_t *)(meta + 16 + 4 * uc) = 0u;
+            *(float2 *)(meta + 32) = float2{raw.unit, -1.0f};  // + sum m XS
+        } else {
+            *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+        }
     }
 };
 using QiMXFP4 = QiNibbles32<QtMXFP4>;
 using QiQ4_0 = QiNibbles32<QtQ4_0>;
+using QiQ4_1 = QiNibbles32<QtQ4_1>;
 
 // Q5_K: d | dmin | scales[12] | qh[32] | qs[128], w = d sc q - dmin m with q in 0..31: the nibble of Q4_K's
 // layout and, for element l of sub-block j, bit j of qh[l] as the fifth bit
@@ -678,30 +703,38 @@ struct QiQ5K {
 };
 
 // Q5_0: blocks of d (f16) | qh (32 fifth bits) | 16 code bytes, w = d (q - 16) with q the nibble and bit j (low
-// nibbles, elements 0..15) or 16 + j (high nibbles, elements 16..31) of qh as its fifth bit
-// (vendor/candle-metal-kernels/src/metal_src/quantized.metal:98-102); a "super-block" here is eight blocks, 176
-// bytes, put on one scale as for Q8_0: p = round(1024 (q - 16) d / D), within +-16384 whatever the sign of d.
-// The four fifth bits of a word are spread to bytes with a multiply, q - 16 becomes a signed byte without
-// carries between bytes ((q | 0x80) - 0x10, then the top bit flipped back), and the product goes the way of
-// Q8_0's.  Blocks sit at even addresses only: read through aligned words.
-struct QiQ5_0 {
-    static constexpr int BLOCK = 176, META = 48, ALIGN = 2, TABLE = 0;
-    static constexpr bool HAS_MIN = false, ONE_PLANE = false, SUB16 = false;
+// nibbles, elements 0..15) or 16 + j (high nibbles, elements 16..31) of qh as its fifth bit; Q5_1: d | m (f16) |
+// qh | codes, w = d q + m (vendor/candle-metal-kernels/src/metal_src/quantized.metal:98-110).  A "super-block"
+// here is eight blocks, put on one scale as for Q8_0: p = round(1024 (q - 16) d / D) or round(1024 q d / D),
+// within +-31744 whatever the sign of d; Q5_1's offsets are the min term (MIN_F16).  The four fifth bits of a
+// word are spread to bytes with a multiply, q - 16 becomes a signed byte without carries between bytes
+// ((q | 0x80) - 0x10, then the top bit flipped back), and the product goes the way of Q8_0's.  Blocks sit at
+// even addresses only: read through aligned words.
+template <bool OFFSET>
+struct QiQ5x {
+    static constexpr int BYTES = OFFSET ? 24 : 22, HIGH = OFFSET ? 4 : 2, CODES = OFFSET ? 8 : 6;
+    static constexpr int BLOCK = 8 * BYTES, META = 48, ALIGN = 2, TABLE = 0;
+    static constexpr bool HAS_MIN = OFFSET, MIN_F16 = OFFSET, ONE_PLANE = false, SUB16 = false;
     struct Hdr {
-        float d0, d1;
+        float d0, d1, m0, m1;
     };
     struct Raw {
         float r0, r1, unit;  // 1024 d / D of the chunk's two blocks, and D / 1024
+        float m0, m1;
         uint32_t ha, hb;     // the fifth bits of block 2 uc and of block 2 uc + 1
         uint4 qa, qb;        // their code bytes
         uint32_t hna, hnb;   // the same of the next super-block (every piece reads all 16 bytes of a block, so the
         uint4 na, nb;        // bytes fetched ahead wait here until take())
     };
     __device__ __forceinline__ static void fetch(const uint8_t *blk, int uc, int part, Raw &raw, Hdr &next) {
-        const uint8_t *pair = blk + 44 * uc;
-        if (part == 0) next.d0 = f16_bits(ld<uint16_t>(pair)), next.d1 = f16_bits(ld<uint16_t>(pair + 22));
-        if (part == 1) raw.hna = ldw<uint32_t>(pair + 2), raw.na = ldw<uint4>(pair + 6);
-        if (part == 2) raw.hnb = ldw<uint32_t>(pair + 24), raw.nb = ldw<uint4>(pair + 28);
+        const uint8_t *pair = blk + 2 * BYTES * uc;
+        if (part == 0) {
+            next.d0 = f16_bits(ld<uint16_t>(pair)), next.d1 = f16_bits(ld<uint16_t>(pair + BYTES));
+            next.m0 = OFFSET ? f16_bits(ld<uint16_t>(pair + 2)) : 0.0f;
+            next.m1 = OFFSET ? f16_bits(ld<uint16_t>(pair + BYTES + 2)) : 0.0f;
+        }
+        if (part == 1) raw.hna = ldw<uint32_t>(pair + HIGH), raw.na = ldw<uint4>(pair + CODES);
+        if (part == 2) raw.hnb = ldw<uint32_t>(pair + BYTES + HIGH), raw.nb = ldw<uint4>(pair + BYTES + CODES);
     }
     __device__ __forceinline__ static void take(Raw &raw, const Hdr &next, int uc, const uint8_t *) {
         float D = fmaxf(mag_or_inf(next.d0), mag_or_inf(next.d1));
@@ -709,6 +742,7 @@ struct QiQ5_0 {
         D = fmaxf(D, dpp_f<0x4E>(D));  // quad_perm [2,3,0,1]
         const float inv = D > 0.0f ? 1024.0f / D : 0.0f;
         raw.r0 = next.d0 * inv, raw.r1 = next.d1 * inv, raw.unit = D * (1.0f / 1024.0f);
+        raw.m0 = next.m0, raw.m1 = next.m1;
         raw.ha = raw.hna, raw.hb = raw.hnb, raw.qa = raw.na, raw.qb = raw.nb;
     }
     __device__ __forceinline__ static void piece(const Raw &raw, int uc, int j, uint8_t *tile, const uint8_t *) {
@@ -719,7 +753,8 @@ struct QiQ5_0 {
             const uint32_t word = (wi == 0 ? qv.x : wi == 1 ? qv.y : wi == 2 ? qv.z : qv.w) >> (4 * half);
             const uint32_t fifth = (((blk ? raw.hb : raw.ha) >> (16 * half + 4 * wi)) & 15u) * 0x00204081u & 0x01010101u;
             const uint32_t q = (word & 0x0F0F0F0Fu) | (fifth << 4);
-            const uint32_t sb = ((q | 0x80808080u) - 0x10101010u) ^ 0x80808080u;  // q - 16 as signed bytes
+            // Q5_0: q - 16 as signed bytes; Q5_1: q as it is (0..31)
+            const uint32_t sb = OFFSET ? q : ((q | 0x80808080u) - 0x10101010u) ^ 0x80808080u;
             const float ratio = blk ? raw.r1 : raw.r0;
             uint32_t t[4];
 #pragma unroll
@@ -732,9 +767,18 @@ struct QiQ5_0 {
         }
     }
     __device__ __forceinline__ static void meta(const Raw &raw, int uc, uint8_t *meta) {
-        *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+        if constexpr (OFFSET) {  // the chunk's two offsets among m_0..7, zeros in the second sixteen bytes
+            const qi_h2 m = {(_Float16)raw.m0, (_Float16)raw.m1};
+            *(uint32_t *)(meta + 4 * uc) = __builtin_bit_cast(uint32_t, m);
+            *(uint32_t *)(meta + 16 + 4 * uc) = 0u;
+            *(float2 *)(meta + 32) = float2{raw.unit, -1.0f};  // + sum m XS
+        } else {
+            *(float2 *)(meta + 32) = float2{raw.unit, 0.0f};  // the same from all four
+        }
     }
 };
+using QiQ5_0 = QiQ5x<false>;
+using QiQ5_1 = QiQ5x<true>;
 
 // Q3_K: hmask[32] | qs[64] | scales[12] | d, w = d (sc - 32) (q - (hbit ? 0 : 4)) over sub-blocks of 16: element
 // 128 h + 32 t + 16 hf + i is field t of qs[32 h + 16 hf + i] with bit 4 h + t of hmask[16 hf + i] as its
@@ -805,6 +849,14 @@ struct QiQ3K {
         *(float2 *)(meta + 32) = float2{raw.d, 0.0f};  // the same from all four
     }
 };
+
+// Sides whose min term has an f16 factor per block of 32 (Q4_1, Q5_1: w = d q + m) say MIN_F16: the row meta
+// holds m_0..7 as halves and sixteen bytes of zeros, and the term takes two f16 MFMAs, sum m a0 and sum m a1
+// (1024 m, which the integer mins carry as a second operand, may not be an f16 value).
+template <class F, class = void>
+struct QiMinF16 : std::false_type {};
+template <class F>
+struct QiMinF16<F, std::void_t<decltype(F::MIN_F16)>> : std::bool_constant<F::MIN_F16> {};
 
 // grid: 1-D; workgroup L takes tile (x, y) of tx x ty (weight-row tiles x activation-row tiles).  When ty
 // divides 8 the eight XCDs (L % 8) each work on one activation-row tile, whose operands then stay in that
@@ -952,7 +1004,14 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                 const uint8_t *meta = buf + NG * QI_TILE + (16 * (cg0 + cg) + r) * F::META;
                 const float2 dd = *(const float2 *)(meta + F::META - 16);
                 qm_f4 I2 = zero_f;
-                if constexpr (F::HAS_MIN) {
+                if constexpr (QiMinF16<F>::value) {
+                    // lane group 0 carries a0, group 1 a1: m against the one, zeros against the other
+                    const qi_h8 m0 = *(const qi_h8 *)(meta + 16 * (g & 1)), m1 = *(const qi_h8 *)(meta + 16 * (~g & 1));
+                    I2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(minA, m0, zero_f, 0, 0, 0);
+                    const qm_f4 high = __builtin_amdgcn_mfma_f32_16x16x32_f16(minA, m1, zero_f, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) I2[i] = fmaf(1024.0f, high[i], I2[i]);
+                } else if constexpr (F::HAS_MIN) {
                     // eight sub-blocks: lane groups 2, 3 meet zeros in the activation operand, any finite halves
                     // will do for them
                     const qi_h8 mB = *(const qi_h8 *)(meta + 16 * (F::SUB16 ? g : g & 1));

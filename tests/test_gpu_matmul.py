@@ -432,6 +432,41 @@ def q5_0_integer_case(n, k, seed, nonzero=16, small=400):
     return blocks, w, x
 
 
+def q4_1_q5_1_integer_case(qtype, n, k, seed, nonzero=16, offset_blocks=3, small=400):
+    """Q4_1 or Q5_1 blocks, w = d q + m: scales of 1/2 to 4, `nonzero` codes q in 1..15 (1..31) a row, and
+    `offset_blocks` blocks a row with an offset m in multiples of 1/4 up to 4 in magnitude; integer activations
+    that peak at 32639 at one slot of every 256, where the codes are zero.  Returns (blocks, weights as float64,
+    activations)."""
+    rng = np.random.default_rng(seed)
+    five = qtype == capi.Q5_1
+    q = np.zeros((n, k), np.int64)
+    for r in range(n):
+        q[r, rng.choice(k, size=nonzero, replace=False)] = rng.integers(1, 32 if five else 16, size=nonzero)
+    x = rng.integers(-small, small + 1, size=k).astype(np.int64)
+    peak = np.arange(0, k, 256) + int(rng.integers(0, 256))
+    x[peak] = 32639 * rng.choice([-1, 1], size=k // 256)
+    q[:, peak] = 0
+    d = rng.choice(np.array([0.5, 1.0, 2.0, 4.0]), size=(n, k // 32))
+    m = np.zeros((n, k // 32))
+    for r in range(n):
+        m[r, rng.choice(k // 32, size=offset_blocks, replace=False)] = rng.integers(-16, 17, size=offset_blocks) / 4.0
+    codes = q.reshape(n, k // 32, 2, 16)                         # low nibbles: elements 0..15, high: 16..31
+    nbytes = 24 if five else 20
+    blocks = np.zeros((n, k // 32, nbytes), np.uint8)
+    blocks[:, :, 0:2] = d.astype(np.float16)[..., None].view(np.uint8)
+    blocks[:, :, 2:4] = m.astype(np.float16)[..., None].view(np.uint8)
+    if five:
+        qh = np.zeros((n, k // 32), np.int64)
+        for j in range(16):
+            qh |= ((codes[:, :, 0, j] >> 4) << j) | ((codes[:, :, 1, j] >> 4) << (16 + j))
+        blocks[:, :, 4:8] = qh.astype(np.uint32)[..., None].view(np.uint8)
+    blocks[:, :, nbytes - 16:] = ((codes[:, :, 0, :] & 15) | ((codes[:, :, 1, :] & 15) << 4)).astype(np.uint8)
+    blocks = blocks.reshape(-1)
+    w = q * d.repeat(32, axis=1) + m.repeat(32, axis=1)
+    assert np.array_equal(oracle.dequantize(qtype, blocks).reshape(n, k), w.astype(np.float32))
+    return blocks, w, x
+
+
 def test_q6k_dot4_integer_dot_products_are_bit_exact():
     """d = 1, every scale 1, integer activations whose 32-element blocks peak at 32639 (activation
     scale exactly 1): the kernel's integer sums, f32 FMA and int64 arithmetic agree exactly."""
@@ -511,12 +546,13 @@ def test_few_rows_against_a_large_matrix_take_the_int8_gemm(qtype, m, k, n):
     assert np.array_equal(got, w.matmul_t(m, lhs))
 
 
-@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q5_1, 8, 12288, 1024), (capi.Q4_1, 16, 4096, 2100), (capi.Q5_1, 11, 7168, 1200),
+@pytest.mark.parametrize("qtype,m,k,n", [(capi.Q5_1, 40, 2048, 1024), (capi.Q4_1, 33, 4096, 500), (capi.MXFP4, 20, 7168, 600),
                                          (capi.Q6_K, 512, 2048, 100), (capi.IQ2_XXS, 40, 5120, 300)])
 def test_decoded_weights_gemm_split_over_k(qtype, m, k, n):
-    """8..16 rows against matrices of 8M elements or more, and many rows against few weight rows: the GEMM's
-    tiles alone leave compute units idle, so runs of chunks go to workgroups of their own and the partial
-    sums are added in a fixed order (the same result on every call)."""
+    """Products the int8 GEMM leaves to the GEMM over decoded weights: fewer than 64 rows against fewer than 8M
+    weights, and many rows against few weight rows.  Its tiles alone leave compute units idle, so runs of
+    chunks go to workgroups of their own and the partial sums are added in a fixed order (the same result on
+    every call)."""
     blocks = synth.random_blocks(qtype, 300 + m, n * k) if qtype in capi.GENERIC_TYPES else make_blocks(qtype, n, k, 300 + m)
     lhs = synth.normal(301 + m, (m, k))
     w = capi.Weight.upload(qtype, blocks, n, k)
@@ -1137,12 +1173,13 @@ import oracle
 from joshua_amd import capi, synth
 from tests.test_gpu_matmul import (q4k_integer_case, q6k_integer_case, q2k_integer_case, q8_0_integer_case,
                                    iq2xxs_integer_case, mxfp4_integer_case, q5k_integer_case, q4_0_integer_case,
-                                   q3k_integer_case, q5_0_integer_case, close)
+                                   q3k_integer_case, q5_0_integer_case, q4_1_q5_1_integer_case, close)
 FMT, KERNEL = {"q4k": (capi.Q4_K, "q4k_gemm_i8"), "q6k": (capi.Q6_K, "q6k_gemm_i8"), "q2k": (capi.Q2_K, "q2k_gemm_i8"),
                "q8_0": (capi.Q8_0, "q8_0_gemm_i8"), "iq2xxs": (capi.IQ2_XXS, "iq2xxs_gemm_i8"),
                "mxfp4": (capi.MXFP4, "mxfp4_gemm_i8"), "q5k": (capi.Q5_K, "q5k_gemm_i8"),
                "q4_0": (capi.Q4_0, "q4_0_gemm_i8"), "q3k": (capi.Q3_K, "q3k_gemm_i8"),
-               "q5_0": (capi.Q5_0, "q5_0_gemm_i8")}[sys.argv[1]]
+               "q5_0": (capi.Q5_0, "q5_0_gemm_i8"), "q4_1": (capi.Q4_1, "q4_1_gemm_i8"),
+               "q5_1": (capi.Q5_1, "q5_1_gemm_i8")}[sys.argv[1]]
 _synth = synth
 class _Synth:  # the formats without a quantiser of normal weights get random blocks
     normal = staticmethod(_synth.normal)
@@ -1192,11 +1229,13 @@ elif FMT == capi.Q4_0:  # scales of 1/2 to 4 inside a run of 256
     blocks, q, x = q4_0_integer_case(n, k, 23)
 elif FMT == capi.Q3_K:  # every scale, field and third bit: dense integer weights up to 128
     blocks, q, x = q3k_integer_case(n, k, 23)
-else:  # fifth bits; scales of 1/2 to 4, some negative, inside a run of 256
+elif FMT == capi.Q5_0:  # fifth bits; scales of 1/2 to 4, some negative, inside a run of 256
     blocks, q, x = q5_0_integer_case(n, k, 23)
+else:  # an f16 offset per block of 32
+    blocks, q, x = q4_1_q5_1_integer_case(FMT, n, k, 23)
 lhs = np.stack([np.roll(x, (32 if FMT in (capi.Q4_K, capi.Q6_K, capi.Q5_K) else 256) * i) for i in range(m)])
 assert np.abs(lhs @ q.T).max() < {capi.IQ2_XXS: 2 ** 16, capi.Q3_K: 2 ** 16, capi.MXFP4: 2 ** 13}.get(FMT, 2 ** 24)
-if FMT in (capi.Q8_0, capi.Q4_0, capi.Q5_0):  # per run of 256, 1024 times the sum is still an integer that f32 holds
+if FMT in (capi.Q8_0, capi.Q4_0, capi.Q5_0, capi.Q4_1, capi.Q5_1):  # per run of 256, 1024 times the sum is still an integer that f32 holds
     runs = np.einsum("mbe,nbe->mnb", lhs.reshape(m, -1, 256).astype(np.float64), q.reshape(n, -1, 256))
     assert np.abs(runs).max() < 2 ** 19
 got = capi.Weight.upload(FMT, blocks, n, k).matmul_t(m, lhs.astype(np.float32))
@@ -1239,7 +1278,7 @@ print("gemm i8 ok")
 """
 
 
-@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0", "q3k", "q5_0"])
+@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0", "q3k", "q5_0", "q4_1", "q5_1"])
 @pytest.mark.parametrize("shape", ["8,7", "4,4", "2,4"])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup
