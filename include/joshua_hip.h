@@ -107,15 +107,15 @@ const void *jq_device_ptr(const jq_weight *w);
  * (its own bound, src/kquant_dot.rs:853).  The integer kernels hold the activations in
  * 16-bit fixed point: one scale per 32 elements of a row for Q4_K up to 63 activation rows
  * and for every one-row product, so a row whose groups span many orders of magnitude keeps
- * the bound; the matrix-core GEMM (Q4_K from 64 rows on; every other format from 17 rows on,
- * and from 8 against 8M weights or more) uses one scale per 256
- * elements, which resolves each super-block to 2^-16 of its largest magnitude (2^-12 of the
- * sum of the terms' magnitudes on such rows; the reference's integer path quantises
- * activations to 8 bits per 256, src/quant_matmul.rs:184).  In that GEMM the formats with a
- * scale per 32 elements (Q8_0, MXFP4, Q4_0, Q4_1, Q5_0, Q5_1) have the eight blocks of a 256-run put on the
- * run's largest scale at 16 bits: exact where the scales are equal or a few powers of two
- * apart, else each weight to 2^-16 of the run's largest magnitude.  A row holding an inf or
- * a NaN comes out all NaN. */
+ * the bound; the matrix-core GEMM (Q4_K from 64 rows on; every other format from 17 rows
+ * on, and from 8 against 8M weights or more) uses one scale per 256 elements, which
+ * resolves each super-block to 2^-16 of its largest magnitude (2^-12 of the sum of the
+ * terms' magnitudes on such rows; the reference's integer path quantises activations to 8
+ * bits per 256, src/quant_matmul.rs:184).  In that GEMM the formats with a scale per 32
+ * elements (Q8_0, MXFP4, Q4_0, Q4_1, Q5_0, Q5_1) have the eight blocks of a 256-run put on
+ * the run's largest scale at 15 or 16 bits: exact where the scales are equal or a few powers
+ * of two apart, else each weight to 2^-15 of the run's largest magnitude or better.  A row
+ * holding an inf or a NaN comes out all NaN. */
 int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, float *dst,
                 size_t dst_len, int ptrs_are_device, void *stream);
 
