@@ -710,13 +710,13 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
     // waves, two a compute unit), and a split over k (the parts summed by splitk_sum) when the tiles alone leave
     // compute units idle: every workgroup then walks nb / splits super-blocks.
     // Up to 32 rows also: 32 x 64 (two waves that share the weight rows, two workgroups a compute unit).
-    static const GemmI8Shape shapes[] = {{8, 7, false}, {4, 4, false}, {2, 4, true}};
+    static const GemmI8Shape shapes[] = {{8, 7, false}, {8, 6, false}, {4, 4, false}, {2, 4, true}};
     const size_t nb = k / 256, groups = (m + 15) / 16;
     auto tiles_of = [&](const GemmI8Shape &sh) {
         const size_t mt = sh.nsplit ? 32 : 32 * (size_t)sh.nw, nt = 16 * (size_t)sh.ng;
         return ((m + mt - 1) / mt) * ((n + nt - 1) / nt);
     };
-    if (tiles_of(shapes[1]) * std::max<size_t>(1, std::min<size_t>(nb / 4, 8)) < min_tiles) return -1;
+    if (tiles_of(shapes[2]) * std::max<size_t>(1, std::min<size_t>(nb / 4, 8)) < min_tiles) return -1;
     // Estimate per (shape, splits), in us, fitted to whole-call times of Q4_K products of 32 to 2048 rows
     // against 1024 to 24576 weight rows of 4096 and 12288 columns (the picks are within 5 % of the best
     // measured choice there; Q6_K runs ~10 % longer with the same ordering): the preparation, a fixed part,
@@ -732,7 +732,8 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
         if (sh.nsplit)  // 3.1 us a super-block with 64 at work, 3.4 with 256, 4.4 with 512 (two a compute unit), in whole rounds
             us += 3.9 + nbl * (2.95 + 0.0029 * std::min(wgs, 512.0)) *
                             (wgs <= 512.0 ? 1.0 : wgs < 2048.0 ? std::ceil(wgs / 512.0) : wgs / 512.0);
-        else if (sh.nw == 8) us += 10.0 + nbl * (4.3 + 0.009 * std::min(wgs, 256.0)) * std::ceil(wgs / 256.0);
+        else if (sh.nw == 8)  // (six groups of weight rows instead of seven: six sevenths of the work a super-block)
+            us += 10.0 + nbl * (4.3 + 0.009 * std::min(wgs, 256.0)) * std::ceil(wgs / 256.0) * (sh.ng == 7 ? 1.0 : 0.88);
         else if (wgs <= 256.0) us += 3.9 + nbl * (2.3 + 0.0027 * wgs);
         else us += 3.9 + nbl * (3.1 + 0.0032 * std::min(wgs, 512.0)) * std::max(1.0, wgs / 512.0);
         if (sp > 1) us += 1.0 + 0.8 * (double)sp + (double)(sp + 1) * (double)(m * n) * 4.0 / 8.0e6;
@@ -791,6 +792,7 @@ int dispatch_gemm_i8(const uint8_t *W, size_t row_bytes, const float *X, float *
         }                                                                                                             \
     }
     JQ_GEMM_I8(8, 7, false)
+    JQ_GEMM_I8(8, 6, false)
     JQ_GEMM_I8(4, 4, false)
     JQ_GEMM_I8(2, 4, true)
 #undef JQ_GEMM_I8

@@ -1278,12 +1278,15 @@ print("gemm i8 ok")
 """
 
 
-@pytest.mark.parametrize("fmt", ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0", "q3k", "q5_0", "q4_1", "q5_1"])
-@pytest.mark.parametrize("shape", ["8,7", "4,4", "2,4"])
+GEMM_I8_FORMATS = ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0", "q3k", "q5_0", "q4_1", "q5_1"]
+
+
+@pytest.mark.parametrize("shape,fmt", [(s, f) for s in ("8,7", "4,4", "2,4") for f in GEMM_I8_FORMATS] +
+                         [("8,6", f) for f in ("q4k", "q6k", "q2k")])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup
-    shape forced through the environment (read when the library first dispatches, hence the child process) all three
-    shapes run on small products: parity, ragged edges, exact integer sums, wide-range and non-finite
+    shape forced through the environment (read when the library first dispatches, hence the child process) every
+    shape runs on small products: parity, ragged edges, exact integer sums, wide-range and non-finite
     activation rows."""
     import subprocess
     import sys
