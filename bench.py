@@ -353,6 +353,10 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
     out["moe_deepseek_v3_iq2_xxs_b1"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 1, 105, max(steps // 4, 10),
                                                      True, 1, cs)
     torch.cuda.empty_cache()
+    # the same layer over 512 tokens (a prompt): the grouped int8 GEMM; no CPU timing (the oracle's parity run is
+    # the bounded sample here)
+    out["moe_deepseek_v3_iq2_xxs_b512"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 512, 105, 8, True, 1, 0.0)
+    torch.cuda.empty_cache()
     out["moe_deepseek_v3_mxfp4_b1"] = moe_workload(torch, capi, synth, 39, 7168, 2048, 256, 8, 1, 105, max(steps // 4, 10),
                                                    True, 1, cs)
     torch.cuda.empty_cache()
