@@ -1376,3 +1376,31 @@ def test_other_formats_random_shapes(qtype, m, k, n):
     got = capi.Weight.upload(qtype, blocks, n, k).matmul_t(m, lhs)
     want = oracle.matmul_t(qtype, (m, k, n), lhs, blocks, avx2=oracle.have_avx2())
     assert close(got, want), (capi.TYPE_NAMES[qtype], m, k, n, capi.last_kernel())
+
+
+def _large_random_shapes(seed, count):
+    """Shapes of 8M weights or more, where every format's products of 8 rows and more take the int8 GEMM."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        m = int(rng.choice([8, 11, 16, 17, 31, 32, 33, 63, 64, 100, 130, 257, 300]))
+        k = int(rng.choice([2048, 4096, 5120, 7168, 8192]))
+        n = int(rng.integers((8 << 20) // k + 1, 3 * (8 << 20) // k))
+        out.append((m, k, n))
+    return out
+
+
+@pytest.mark.parametrize("qtype", [t for t in capi.ALL_TYPES + capi.GENERIC_TYPES if t != capi.Q4_K])
+@pytest.mark.parametrize("m,k,n", _large_random_shapes(78, 4))
+def test_every_format_on_the_int8_gemm_at_random_large_shapes(qtype, m, k, n):
+    """Seeded random shapes against large matrices: whatever tile shape and split over k the estimate picks
+    (32 x 64 tiles up to 32 rows, 128 x 64, 256 x 96 or 256 x 112 beyond), ragged in both directions, the result
+    holds the reference's bound against the oracle on a sample of the weight rows."""
+    blocks = synth.random_blocks(qtype, 710 + qtype, n * k) if qtype in capi.GENERIC_TYPES else make_blocks(qtype, n, k, 710 + qtype)
+    lhs = synth.normal(810 + n % 89, (m, k))
+    got = capi.Weight.upload(qtype, blocks, n, k).matmul_t(m, lhs)
+    assert "gemm_i8" in capi.last_kernel(), capi.last_kernel()
+    rows = np.unique(np.concatenate([np.arange(130), np.arange(n - 130, n), np.arange(130, n - 130, 7)[:240]]))
+    sub = blocks.reshape(n, -1)[rows].reshape(-1)
+    want = oracle.matmul_t(qtype, (m, k, rows.size), lhs, sub, avx2=oracle.have_avx2() and qtype not in capi.GENERIC_TYPES)
+    assert close(got[:, rows], want), (capi.TYPE_NAMES[qtype], m, k, n, capi.last_kernel())
