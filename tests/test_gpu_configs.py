@@ -67,6 +67,20 @@ def test_deepseek_v3_shaped_expert_layer(qtype):
     layer.close()
 
 
+@pytest.mark.parametrize("qtype,tokens", [(capi.IQ2_XXS, 48), (capi.MXFP4, 40)])
+def test_deepseek_v3_shaped_expert_layer_over_a_prompt(qtype, tokens):
+    """The same layer over more pairs than experts (48 tokens: 384 routed pairs over 256 experts and the shared
+    expert's 48): the grouped int8 GEMM at the layer's own row lengths, gate and up of 7168 columns (28
+    super-blocks), down of 2048."""
+    layer, ora = moe_layer(qtype, 7168, 2048, 256, 8, 500 + qtype, shared=True, gating="sigmoid")
+    x = synth.normal(530 + tokens, (tokens, 7168))
+    got = layer.forward(x)
+    assert capi.last_kernel() == "moe_gemm_i8_few"
+    ok, e = close(got, ora.forward(x))
+    assert ok, f"{capi.TYPE_NAMES[qtype]} tokens={tokens}: {e}"
+    layer.close()
+
+
 @pytest.mark.parametrize("tokens", [1, 64])
 def test_qwen3_30b_a3b_shaped_layer_with_all_128_experts(tokens):
     """h 2048, 128 experts of 768, top-8, Q4_K (src/quantized_qwen3_moe.rs:404-520): batch 1 takes the
