@@ -1565,6 +1565,7 @@ int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t r
     else if (own) JQ_DOT8(4, true);
     else JQ_DOT8(4, false);
 #undef JQ_DOT8
+    note_kernel("moe_rows_dot8");
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -1625,6 +1626,7 @@ int launch_moe_down_combine(const uint8_t *const *Wa, size_t row_bytes, int base
     else if (own) JQ_DC(4, true);
     else JQ_DC(4, false);
 #undef JQ_DC
+    note_kernel("moe_down_combine_dot8");
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -1775,7 +1777,26 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     // the experts' SwiGLU clamp; a folded shared expert is expert number n_expert and has its own
     const jq::MoeClamp clamp{c.swiglu_clamp, c.swiglu_clamp_shared, (int)c.n_expert};
     int groups, max_group;
-    if ((size_t)P <= c.n_expert) {  // decode-sized: one group per pair, written by the gating kernel itself
+    // Decode-sized (one group a pair, every pair reading its expert's rows) or bucketed by expert (every expert hit
+    // read once)?  A pair costs about a = 0.10 + 0.17 bytes-per-weight ns a weight on the integer-dot kernels;
+    // a bucketed expert costs g = 0.45 ns a weight on the grouped int8 GEMM (bound by the unpacking) and 0.28 on the
+    // Q4_K kernels for short rows.  With d(P) = E (1 - (1 - 1/E)^P) experts hit by P pairs, pairs win while
+    // P a <= d(P) g (Qwen3-30B-A3B sizes: up to ~100 pairs over 128 experts; DeepSeek-V3 sizes, IQ2_XXS: ~750 over
+    // 256).  Formats without integer-dot kernels keep pairs up to the number of experts.
+    // JQ_MOE_DECODE_PAIRS_PCT: pairs, in percent of the experts, up to which a call is decode-sized.
+    static const char *pct_env = getenv("JQ_MOE_DECODE_PAIRS_PCT");
+    bool decode_sized = (size_t)P <= c.n_expert;
+    if (pct_env) {
+        decode_sized = (size_t)P * 100 <= c.n_expert * (size_t)atoll(pct_env);
+    } else if (moe_has_dot8(m->gate->type) && moe_has_dot8(m->up->type) && moe_has_dot8(m->down->type) &&
+               c.hidden % 256 == 0 && c.inter % 256 == 0) {
+        const double bpw = (double)m->gate->row_bytes / (double)c.hidden;
+        const bool short_q4k = m->gate->type == JQ_TYPE_Q4_K && c.hidden <= 2048 && c.inter <= 2048;
+        const double a = 0.10 + 0.17 * bpw, g = short_q4k ? 0.28 : 0.45;
+        const double hit = (double)c.n_expert * (1.0 - std::pow(1.0 - 1.0 / (double)c.n_expert, (double)P));
+        decode_sized = (double)P * a <= hit * g && P <= 16384;
+    }
+    if (decode_sized) {  // one group per pair, written by the gating kernel itself
         if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra})) return 1;
         groups = P + extra * (int)T;
         max_group = 1;

@@ -67,15 +67,16 @@ def test_deepseek_v3_shaped_expert_layer(qtype):
     layer.close()
 
 
-@pytest.mark.parametrize("qtype,tokens", [(capi.IQ2_XXS, 48), (capi.MXFP4, 40)])
-def test_deepseek_v3_shaped_expert_layer_over_a_prompt(qtype, tokens):
-    """The same layer over more pairs than experts (48 tokens: 384 routed pairs over 256 experts and the shared
-    expert's 48): the grouped int8 GEMM at the layer's own row lengths, gate and up of 7168 columns (28
-    super-blocks), down of 2048."""
+@pytest.mark.parametrize("qtype,tokens,bucketed", [(capi.IQ2_XXS, 150, True), (capi.MXFP4, 90, True), (capi.IQ2_XXS, 48, False)])
+def test_deepseek_v3_shaped_expert_layer_over_a_prompt(qtype, tokens, bucketed):
+    """The same layer over more pairs than experts.  150 tokens of IQ2_XXS (1200 routed pairs over 256 experts and
+    the shared expert's 150) and 90 of MXFP4: bucketed by expert on the grouped int8 GEMM at the layer's own row
+    lengths, gate and up of 7168 columns (28 super-blocks), down of 2048.  48 tokens: still one group a pair (a
+    pair's rows cost less to read again than an expert's to unpack for a tile of 32 rows)."""
     layer, ora = moe_layer(qtype, 7168, 2048, 256, 8, 500 + qtype, shared=True, gating="sigmoid")
     x = synth.normal(530 + tokens, (tokens, 7168))
     got = layer.forward(x)
-    assert capi.last_kernel() == "moe_gemm_i8_few"
+    assert capi.last_kernel() == ("moe_gemm_i8_few" if bucketed else "moe_down_combine_dot8")
     ok, e = close(got, ora.forward(x))
     assert ok, f"{capi.TYPE_NAMES[qtype]} tokens={tokens}: {e}"
     layer.close()
