@@ -1281,7 +1281,10 @@ print("gemm i8 ok")
 GEMM_I8_FORMATS = ["q4k", "q6k", "q2k", "q8_0", "iq2xxs", "mxfp4", "q5k", "q4_0", "q3k", "q5_0", "q4_1", "q5_1"]
 
 
-@pytest.mark.parametrize("shape,fmt", [(s, f) for s in ("8,7", "4,4", "2,4") for f in GEMM_I8_FORMATS] +
+# every format under the largest and the smallest workgroup shape; the two in between for the formats that differ
+# in what the kernel holds in LDS (row meta of 48 or 80 bytes, a lookup table) or in how many planes it multiplies
+@pytest.mark.parametrize("shape,fmt", [(s, f) for s in ("8,7", "2,4") for f in GEMM_I8_FORMATS] +
+                         [("4,4", f) for f in ("q4k", "q6k", "q2k", "iq2xxs", "q4_1")] +
                          [("8,6", f) for f in ("q4k", "q6k", "q2k")])
 def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     """The int8 GEMM serves products of 64 activation rows or more; with the thresholds lowered and the workgroup
@@ -1295,7 +1298,7 @@ def test_int8_gemm_small_shapes_in_a_child_process(shape, fmt):
     res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1), fmt], env=env, capture_output=True, text=True, timeout=170)
     assert res.returncode == 0 and "gemm i8 ok" in res.stdout, res.stdout + res.stderr
     # forced splits of 2 and 4 (k of 4096 and 12288: 16 and 48 super-blocks)
-    for splits in ("2", "4"):
+    for splits in ("2", "4") if shape in ("8,7", "4,4") else ():
         env["JQ_Q4K_GEMM_I8_SPLITS"] = splits
         res = subprocess.run([sys.executable, "-c", GEMM_I8_CHILD.replace("%r", repr(root), 1), fmt], env=env, capture_output=True, text=True, timeout=170)
         assert res.returncode == 0 and "gemm i8 ok" in res.stdout, splits + res.stdout + res.stderr
