@@ -1747,8 +1747,13 @@ int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, s
 int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg) {
     const jq_moe_config &c = m->cfg;
     const unsigned token_runs = (unsigned)((T + jq::ROUTER_TOKENS_PER_WG - 1) / jq::ROUTER_TOKENS_PER_WG);
-    hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert, token_runs), dim3(256), 0, s, m->router_w, x, m->logits,
-                       (int)T, (int)c.hidden, (int)c.n_expert);
+    static const char *no_tile = getenv("JQ_MOE_NO_ROUTER_TILE");
+    if (T >= 32 && !no_tile)  // many tokens: a token's activations read once per eight experts (the same bits)
+        hipLaunchKernelGGL(jq::moe_router_logits_tile, dim3((c.n_expert + 7) / 8, (unsigned)((T + 7) / 8)), dim3(256), 0, s,
+                           m->router_w, x, m->logits, (int)T, (int)c.hidden, (int)c.n_expert);
+    else
+        hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert, token_runs), dim3(256), 0, s, m->router_w, x, m->logits,
+                           (int)T, (int)c.hidden, (int)c.n_expert);
     jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
                          (int)c.n_group, (int)c.topk_group};
     size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);

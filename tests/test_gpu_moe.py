@@ -51,6 +51,20 @@ def test_route_matches_oracle(kw):
     assert np.allclose(w, ow, rtol=2e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize("h,E,tokens", [(544, 30, 45), (2080, 9, 33), (1024, 64, 128)])
+def test_router_logits_of_many_tokens_are_those_of_few(h, E, tokens):
+    """From 32 tokens on the logits come from a kernel that works on 8 experts x 8 tokens a workgroup (an expert
+    count and a token count that are not multiples of 8, a row that ends inside a step of 1024 columns); it adds
+    the same products in the same order, so ids and weights equal those of calls of 8 tokens bit for bit."""
+    ora, dev = build(capi.Q8_0, h, 32, E, 4, 50 + E)
+    x = synth.normal(51 + E, (tokens, h))
+    ids, w = dev.route(x)
+    assert np.array_equal(ids, ora.route(x)[0])
+    for t0 in range(0, tokens, 8):
+        i8, w8 = dev.route(x[t0:t0 + 8])
+        assert np.array_equal(ids[t0:t0 + 8], i8) and np.array_equal(w[t0:t0 + 8], w8)
+
+
 @pytest.mark.parametrize("tokens", [1, 2, 7, 64])
 def test_qwen3moe_shaped_layer_q4k(tokens):
     """Qwen3-30B-A3B layer shape (h 2048, inter 768, top-8) with 16 experts."""
