@@ -1367,6 +1367,12 @@ bool moe_has_dot8(uint32_t type) {
     return list.find("," + std::to_string(type) + ",") != std::string::npos;
 }
 
+// Formats whose units decode to signed int8 words (Q::decode_i8): bucketed calls of few pairs an expert can
+// run on moe_expert_dot8.
+bool moe_has_decode_i8(uint32_t type) {
+    return (type == JQ_TYPE_MXFP4 || type == JQ_TYPE_IQ2_XXS) && moe_has_dot8(type);
+}
+
 // Formats with a side of the int8 GEMM (kq_gemm_i8): their grouped expert matmuls run on it.
 bool moe_has_gemm_i8(uint32_t type) {
     static const char *off = getenv("JQ_MOE_NO_GEMM_I8");
@@ -1568,6 +1574,61 @@ int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t r
     note_kernel("moe_rows_dot8");
     HIP_TRY(hipGetLastError());
     return 0;
+}
+
+// Several pairs a group (bucketed by expert), a format with Q::decode_i8: moe_expert_dot8 over acts_i8_prep's
+// planes of the x_rows rows of X.  Returns -1 when the shape is outside its reach.
+template <class Q, bool DUAL>
+int launch_moe_expert_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align,
+                           const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets, const int *xsel,
+                           const int *yrow, float *Y, int k, int n, int groups, hipStream_t s,
+                           const jq::MoeClamp &cl = jq::MoeClamp{}) {
+    const int units = k / 32;
+    // lanes a row: the fewest of 16, 32, 64 that leave a lane at most eight units
+    const int L = units <= 128 ? 16 : units <= 256 ? 32 : 64, R = 64 / L, ul = (units + L - 1) / L;
+    const size_t wgs = (n + jq::EXPERT_DOT8_WAVES * R - 1) / (jq::EXPERT_DOT8_WAVES * R);
+    const int G = (row_bytes % 16 == 0 && base_align >= 16) ? 16 : (row_bytes % 4 == 0 && base_align >= 4) ? 4 : 0;
+    const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
+    const size_t lds = std::max(jq::EXPERT_DOT8_WAVES * wave_lds, (size_t)2 * 68 * units) + jq::table_bytes<Q>() +
+                       8 * Q::I8_EXTRA_ENTRIES;
+    if (k % 128 != 0 || ul > 8 || G == 0 || lds > 64 * 1024 || !xq.xl) return -1;
+    const size_t words = x_rows * (size_t)(k / 4);
+    hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
+    dim3 grid((unsigned)wgs, (unsigned)groups), block(64 * jq::EXPERT_DOT8_WAVES);
+#define JQ_EXPERT_DOT8(UL_)                                                                                         \
+    case UL_:                                                                                                       \
+        if (G == 16)                                                                                                \
+            hipLaunchKernelGGL((jq::moe_expert_dot8<Q, DUAL, 16, UL_>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp,  \
+                               offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, cl);                                 \
+        else                                                                                                        \
+            hipLaunchKernelGGL((jq::moe_expert_dot8<Q, DUAL, 4, UL_>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp,   \
+                               offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, cl);                                 \
+        break;
+    switch (ul) {
+        JQ_EXPERT_DOT8(1) JQ_EXPERT_DOT8(2) JQ_EXPERT_DOT8(3) JQ_EXPERT_DOT8(4)
+        JQ_EXPERT_DOT8(5) JQ_EXPERT_DOT8(6) JQ_EXPERT_DOT8(7) JQ_EXPERT_DOT8(8)
+    }
+#undef JQ_EXPERT_DOT8
+    note_kernel("moe_expert_dot8");
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+template <bool DUAL>
+int dispatch_moe_expert_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes,
+                             int base_align, const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp,
+                             const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n, int groups,
+                             hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
+    if (((uintptr_t)X & 15) != 0) return -1;
+    switch (type) {
+    case JQ_TYPE_MXFP4:
+        return launch_moe_expert_dot8<jq::MXFP4, DUAL>(Wa, Wb, row_bytes, base_align, X, x_rows, xq, gexp, offsets, xsel, yrow,
+                                                       Y, k, n, groups, s, cl);
+    case JQ_TYPE_IQ2_XXS:
+        return launch_moe_expert_dot8<jq::IQ2_XXS, DUAL>(Wa, Wb, row_bytes, base_align, X, x_rows, xq, gexp, offsets, xsel,
+                                                         yrow, Y, k, n, groups, s, cl);
+    default: return -1;
+    }
 }
 
 template <bool DUAL>
@@ -1789,17 +1850,36 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     // P a <= d(P) g (Qwen3-30B-A3B sizes: up to ~100 pairs over 128 experts; DeepSeek-V3 sizes, IQ2_XXS: ~750 over
     // 256).  Formats without integer-dot kernels keep pairs up to the number of experts.
     // JQ_MOE_DECODE_PAIRS_PCT: pairs, in percent of the experts, up to which a call is decode-sized.
+    // MXFP4 and IQ2_XXS have a third way, bucketed with the expert's rows decoded once into registers and the pairs
+    // streamed past them (moe_expert_dot8): x = 0.10 ns a weight and expert hit plus 0.032 a pair, and about 90 us a
+    // call for its launches over every (expert, row tile), most of them empty when few experts are hit.  At
+    // DeepSeek-V3's sizes it is the cheapest from ~10 tokens (16 tokens of IQ2_XXS: 0.76 ms against 0.89 by pairs;
+    // 64: 1.90 against 3.15; 256: 4.50 against the GEMM's 5.09) to ~350, where the GEMM takes over.
+    // JQ_MOE_DECODE_PAIRS_PCT: pairs, in percent of the experts, up to which a call is decode-sized.
+    // JQ_MOE_EXPERT_DOT8_UPTO_PAIRS_PER_EXPERT: bucketed calls take moe_expert_dot8 up to this many pairs an expert
+    // on average (0: never).
     static const char *pct_env = getenv("JQ_MOE_DECODE_PAIRS_PCT");
+    const char *expert_env = getenv("JQ_MOE_EXPERT_DOT8_UPTO_PAIRS_PER_EXPERT");  // read at every call
+    const bool has_expert_dot8 = moe_has_decode_i8(m->gate->type) && m->gate->type == m->up->type &&
+                                 moe_has_decode_i8(m->down->type) && c.hidden % 128 == 0 && c.inter % 128 == 0 && m->qi8.xl;
     bool decode_sized = (size_t)P <= c.n_expert;
+    bool expert_dot8 = expert_env && has_expert_dot8 && (size_t)P <= (size_t)atoll(expert_env) * c.n_expert;
     if (pct_env) {
         decode_sized = (size_t)P * 100 <= c.n_expert * (size_t)atoll(pct_env);
+    } else if (expert_dot8) {
+        // asked for: every call of more pairs than experts, up to the given number an expert
     } else if (moe_has_dot8(m->gate->type) && moe_has_dot8(m->up->type) && moe_has_dot8(m->down->type) &&
                c.hidden % 256 == 0 && c.inter % 256 == 0) {
         const double bpw = (double)m->gate->row_bytes / (double)c.hidden;
         const bool short_q4k = m->gate->type == JQ_TYPE_Q4_K && c.hidden <= 2048 && c.inter <= 2048;
         const double a = 0.10 + 0.17 * bpw, g = short_q4k ? 0.28 : 0.45;
         const double hit = (double)c.n_expert * (1.0 - std::pow(1.0 - 1.0 / (double)c.n_expert, (double)P));
-        decode_sized = (double)P * a <= hit * g && P <= 16384;
+        const double by_pairs = (double)P * a, by_gemm = hit * g;
+        double by_expert = INFINITY;
+        if (has_expert_dot8 && !expert_env)
+            by_expert = 0.10 * (hit + extra) + 0.032 * (double)(P + extra * (int)T) + 90e6 / (3.0 * c.hidden * (double)c.inter);
+        decode_sized = by_pairs <= std::min(by_gemm, by_expert) && P <= 16384;
+        if (!expert_env) expert_dot8 = by_expert < by_gemm;
     }
     if (decode_sized) {  // one group per pair, written by the gating kernel itself
         if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra})) return 1;
@@ -1864,6 +1944,11 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     if (rc > 0) return 1;
     // bucketed, any format with a side of the int8 GEMM: gate -> G and up -> U from one preparation of x, then
     // the activation in place
+    const bool multi = max_group > 1 && expert_dot8;
+    if (rc < 0 && same_gu && multi)
+        rc = dispatch_moe_expert_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
+                                           m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
+    if (rc > 0) return 1;
     bool planned = false;
     if (rc < 0 && same_gu && max_group > 1 && m->gacts) {
         moe_gemm_plan(m, groups, (size_t)P + (size_t)extra * T, s);
@@ -1911,6 +1996,11 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);
+    if (rc > 0) return 1;
+    if (rc < 0 && fused_act && multi)
+        rc = dispatch_moe_expert_dot8<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G,
+                                            (size_t)P + extra * T, m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out,
+                                            (int)c.inter, (int)c.hidden, groups, s);
     if (rc > 0) return 1;
     if (rc < 0 && fused_act && max_group > 1 && m->gacts) {
         if (!planned) moe_gemm_plan(m, groups, (size_t)P + (size_t)extra * T, s);

@@ -511,6 +511,36 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
         const float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
         return sx[0] * db * (float)(((ph - 2 * nh) << 8) + (pl - 2 * nl));
     }
+    // Unit u as eight words of signed int8 (elements 4i .. 4i+3 in word i) and its scale: the codebook's
+    // magnitudes 8, 25, 43 negated byte by byte where the sign bit is set ((m ^ 0xFF) + 1 = 256 - m never
+    // carries for m >= 8).
+    // The table is the codebook (entries 0..255) followed by the 128 sign patterns as byte masks (entry 256 + s:
+    // byte j is 0xFF where element j of a group with the seven sign bits s is negative), which the caller
+    // fills with i8_extra_entry.
+    static constexpr bool HAS_DECODE_I8 = true;
+    static constexpr int I8_EXTRA_ENTRIES = 128;
+    __device__ static uint64_t i8_extra_entry(int s7) {
+        const uint32_t signs = (uint32_t)s7 | ((__popc((uint32_t)s7) & 1u) << 7);
+        const uint32_t lo = ((signs & 15u) * 0x00204081u & 0x01010101u) * 0xFFu;
+        const uint32_t hi = ((signs >> 4) * 0x00204081u & 0x01010101u) * 0xFFu;
+        return ((uint64_t)hi << 32) | lo;
+    }
+    __device__ static void decode_i8(const uint64_t *grid_table, const uint8_t *blk, int u, int *w, float &scale) {
+        const float d = f16_bits(ld<uint16_t>(blk));
+        const uint2 g = ldw<uint2>(blk + 2 + 8 * u);
+        const uint32_t lo = g.x, hi = g.y;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint64_t grid = grid_table[(lo >> (8 * l)) & 0xFFu];
+            const uint64_t neg = grid_table[256 + ((hi >> (7 * l)) & 127u)];
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                const uint32_t mag = (uint32_t)(grid >> (32 * hf)), mask = (uint32_t)(neg >> (32 * hf));
+                w[2 * l + hf] = (int)((mag ^ mask) + (mask & 0x01010101u));
+            }
+        }
+        scale = d * (0.5f + (float)(hi >> 28)) * 0.25f;
+    }
 };
 
 struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
@@ -554,6 +584,31 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
         }
         const int s2 = ((ph - 2 * nh) << 8) + (pl - 2 * nl);  // twice the sum: the table holds doubled values
         return sx[0] * d * (0.5f * (float)s2);
+    }
+    // The block as eight words of signed int8, twice the E2M1 values (elements 4i .. 4i+3 in word i, the low
+    // nibbles first), and the scale that goes with them (half the block's): two lookups, of the doubled
+    // magnitudes and of their negatives, and the sign bit picks between them byte by byte.
+    static constexpr bool HAS_DECODE_I8 = true;
+    static constexpr int I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale) {
+        const uint32_t e = blk[0];
+        const uint4 qv = ldw<uint4>(blk + 1);
+        const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int hi = 0; hi < 2; hi++) {
+                const uint32_t v = hi ? qw[i] >> 4 : qw[i];
+                const uint32_t sel = v & 0x07070707u;
+                const uint32_t pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
+                const uint32_t neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
+                const uint32_t mask = ((v >> 3) & 0x01010101u) * 0xFFu;
+                w[4 * hi + i] = (int)((pos & ~mask) | (neg & mask));
+            }
+        }
+        // 2^(e-127) / 2; e == 0 is the f32 denormal 2^-127; 0xFF (reserved) decodes the block to zeros
+        scale = e == 0xFFu ? 0.0f : 0.5f * __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
     }
     __device__ static void decode(const uint8_t *blk, int, float *w) {
         uint32_t e = blk[0];

@@ -786,6 +786,163 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
     if (sub == 0 && active) Y[(size_t)yrow[beg] * n + row] = DUAL ? swiglu(acc, acc2, cl, e) : acc;
 }
 
+// Groups of several pairs (bucketed by expert), formats with Q::decode_i8: the expert's rows are decoded ONCE, to
+// signed int8 words held in registers (a lane keeps UL units of 32 elements of its row, or of gate's and up's row
+// with DUAL; the rows come through LDS, 16 or 4 bytes a lane and load), and the group's pairs stream past them: a
+// pair's activation planes (acts_i8_prep's, row xsel[pair]) are copied into LDS once for the workgroup's four
+// waves, two pairs in flight, and every unit costs sixteen v_dot4 a matrix.  Per-pair kernels re-read a pair's
+// planes in every wave (2.1 bytes an element and wave, from L2: at DeepSeek-V3's sizes that traffic, not the
+// weights, bounds calls of 64 tokens and more) and decode the weights again for every pair.  The rows' staging
+// area becomes the activation buffers once every wave has decoded.  Groups are taken from the last down: a
+// folded shared expert, the one group with a pair per token, is the last group and starts first.  A pair's
+// buffer holds, for units = k / 32: the first four words of every unit of the low plane, the last four, the
+// same of the high plane, and the units' scales.
+// Dynamic LDS: the format's table and its I8_EXTRA_ENTRIES words of 8 bytes, then
+// max(4 * wave_lds, 2 * 68 * units) bytes.
+constexpr int EXPERT_DOT8_WAVES = 4;
+template <class Q, bool DUAL, int G, int UL>
+__global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
+    const uint8_t *const *__restrict__ Wa, const uint8_t *const *__restrict__ Wb, size_t row_bytes, ActsI8 xq,
+    const int *__restrict__ gexp, const int *__restrict__ offsets, const int *__restrict__ xsel,
+    const int *__restrict__ yrow, float *__restrict__ Y, int k, int n, int L, int wave_lds, MoeClamp cl) {
+    static_assert(Q::SEGS == 1 && Q::SEGLEN == 32 && Q::HAS_DECODE_I8, "units of 32 consecutive elements");
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
+    const int grp = (int)gridDim.y - 1 - (int)blockIdx.y;
+    const int beg = offsets[grp], cnt = offsets[grp + 1] - beg;
+    if (cnt == 0) return;  // the whole workgroup
+    const int e = gexp[grp];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int units = k / 32, x_lds = 68 * units, chunks = 4 * units + units / 4;  // 16-byte pieces of a pair's planes and scales
+    uint8_t *base = staged_moe + table_bytes<Q>() + 8 * Q::I8_EXTRA_ENTRIES;
+    auto copy = [&](int p, int buf) {
+        const size_t xr = (size_t)xsel[beg + p];
+        const uint8_t *xl = (const uint8_t *)(xq.xl + xr * (size_t)(k / 4)), *xh = (const uint8_t *)(xq.xh + xr * (size_t)(k / 4));
+        const uint8_t *sx = (const uint8_t *)(xq.sx + xr * (size_t)(k / 32));
+        uint8_t *dst = base + (size_t)buf * x_lds;
+        for (int c0 = 64 * wave; c0 < chunks; c0 += 64 * EXPERT_DOT8_WAVES) {
+            const int c = c0 + lane;
+            if (c < chunks) {
+                const uint8_t *src;
+                if (c < 4 * units) {
+                    const int q = c / units, u = c - q * units;  // q: low plane first half, second half, high plane ...
+                    src = ((q & 2) ? xh : xl) + 32 * u + 16 * (q & 1);
+                } else {
+                    src = sx + 16 * (c - 4 * units);
+                }
+                async_load16(src, lds_offset_of(dst + (size_t)c0 * 16));
+            }
+        }
+    };
+    const int R = 64 / L;
+    const int row0 = (blockIdx.x * EXPERT_DOT8_WAVES + wave) * R;
+    const int nrows = min(R, n - row0);  // <= 0: this wave has no rows; it still copies activations and meets the barriers
+    uint8_t *ra = base + (size_t)wave * wave_lds, *rb = ra + (DUAL ? wave_lds / 2 : 0);
+    if (nrows > 0) {
+        const int pieces = (int)((size_t)nrows * row_bytes / G);
+        const uint8_t *sa = Wa[e] + (size_t)row0 * row_bytes;
+        const uint8_t *sb = DUAL ? Wb[e] + (size_t)row0 * row_bytes : nullptr;
+        for (int p0 = 0; p0 < pieces; p0 += 64) {
+            if (p0 + lane < pieces) {
+                if (G == 16) {
+                    async_load16(sa + (size_t)(p0 + lane) * 16, lds_offset_of(ra + (size_t)p0 * 16));
+                    if (DUAL) async_load16(sb + (size_t)(p0 + lane) * 16, lds_offset_of(rb + (size_t)p0 * 16));
+                } else {
+                    async_load4(sa + (size_t)(p0 + lane) * 4, lds_offset_of(ra + (size_t)p0 * 4));
+                    if (DUAL) async_load4(sb + (size_t)(p0 + lane) * 4, lds_offset_of(rb + (size_t)p0 * 4));
+                }
+            }
+        }
+    }
+    if ((int)threadIdx.x < Q::I8_EXTRA_ENTRIES)
+        ((uint64_t *)(staged_moe + table_bytes<Q>()))[threadIdx.x] = Q::i8_extra_entry((int)threadIdx.x);
+    const auto *table = stage_table<Q>(staged_moe);  // holds a barrier when the format has a table
+    const int sub = lane % L, rl = lane / L, row = row0 + rl;
+    const bool active = rl < nrows;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows landed (this wave's own data)
+    int wa[UL][8], wb[DUAL ? UL : 1][8];
+    float da[UL], db[DUAL ? UL : 1];
+#pragma unroll
+    for (int j = 0; j < UL; j++) {
+        const int u = sub + L * j;
+        if (active && u < units) {
+            const size_t at = (size_t)rl * row_bytes + (size_t)(u / Q::UNITS) * Q::BLOCK_BYTES;
+            Q::decode_i8(table, ra + at, u % Q::UNITS, wa[j], da[j]);
+            if (DUAL) Q::decode_i8(table, rb + at, u % Q::UNITS, wb[j], db[j]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                wa[j][i] = 0;
+                if (DUAL) wb[j][i] = 0;
+            }
+            da[j] = 0.0f;
+            if (DUAL) db[j] = 0.0f;
+        }
+    }
+    __syncthreads();  // every wave holds its weights: the rows' LDS now takes the activations
+    copy(0, 0);
+    for (int p = 0; p < cnt; p++) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // pair p's planes are in; every wave is done with pair p - 1's buffer
+        if (p + 1 < cnt) copy(p + 1, (p + 1) & 1);
+        const uint8_t *xb = base + (size_t)(p & 1) * x_lds;
+        float acc = 0.0f, acc2 = 0.0f;
+        // a unit's activations: eight words of each plane and the scale.  The next unit's are asked for before
+        // this unit's products; the fences keep the compiler from asking for every unit's at once (17 registers
+        // a unit, which with the weights would not fit).
+        struct UnitX {
+            uint4 l0, l1, h0, h1;
+            float sx;
+        };
+        auto unit_x = [&](int j) {
+            const int u = min(sub + L * j, units - 1);  // past the row's end: zero weights against the last unit
+            UnitX x;
+            x.l0 = *(const uint4 *)(xb + 16 * u), x.l1 = *(const uint4 *)(xb + 16 * (units + u));
+            x.h0 = *(const uint4 *)(xb + 16 * (2 * units + u)), x.h1 = *(const uint4 *)(xb + 16 * (3 * units + u));
+            x.sx = *(const float *)(xb + 64 * units + 4 * u);
+            return x;
+        };
+        UnitX cur = unit_x(0);
+#pragma unroll
+        for (int j = 0; j < UL; j++) {
+            UnitX nxt = cur;
+            if (j + 1 < UL) nxt = unit_x(j + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            const int xl[8] = {(int)cur.l0.x, (int)cur.l0.y, (int)cur.l0.z, (int)cur.l0.w,
+                               (int)cur.l1.x, (int)cur.l1.y, (int)cur.l1.z, (int)cur.l1.w};
+            const int xh[8] = {(int)cur.h0.x, (int)cur.h0.y, (int)cur.h0.z, (int)cur.h0.w,
+                               (int)cur.h1.x, (int)cur.h1.y, (int)cur.h1.z, (int)cur.h1.w};
+            int pl = 0, ph = 0, pl2 = 0, ph2 = 0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                pl = __builtin_amdgcn_sdot4(wa[j][i], xl[i], pl, false);
+                ph = __builtin_amdgcn_sdot4(wa[j][i], xh[i], ph, false);
+                if (DUAL) {
+                    pl2 = __builtin_amdgcn_sdot4(wb[j][i], xl[i], pl2, false);
+                    ph2 = __builtin_amdgcn_sdot4(wb[j][i], xh[i], ph2, false);
+                }
+            }
+            acc = fmaf(cur.sx * da[j], (float)((ph << 8) + pl), acc);
+            if (DUAL) {
+                acc2 = fmaf(cur.sx * db[j], (float)((ph2 << 8) + pl2), acc2);
+                // both sums are due here: left alone, the second matrix's products of every unit are put after
+                // the first's, with every unit's activations held until then
+                asm volatile("" : "+v"(acc), "+v"(acc2));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt;
+        }
+        if (L >= 64) acc = sum_xor32(acc);  // L is 16, 32 or 64: whole rows of 16 lanes
+        if (L >= 32) acc = sum_xor16(acc);
+        acc = sum_row16(acc);
+        if (DUAL) {
+            if (L >= 64) acc2 = sum_xor32(acc2);
+            if (L >= 32) acc2 = sum_xor16(acc2);
+            acc2 = sum_row16(acc2);
+        }
+        if (sub == 0 && active) Y[(size_t)yrow[beg + p] * n + row] = DUAL ? swiglu(acc, acc2, cl, e) : acc;
+    }
+}
+
 // The decode-sized down projection with the weighted combine in the same kernel.  Workgroup (tile of
 // output rows, token t) walks the token's pairs: its k_used routed experts in slot order (pair
 // t * k_used + s, weight wts[pair]) and then, with n_extra, the shared expert (pair P + t, weight 1).  Pair p

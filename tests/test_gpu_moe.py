@@ -281,3 +281,24 @@ def test_many_tokens_take_the_grouped_int8_gemm(qtype, h, inter, E, k, tokens, s
     assert np.array_equal(got, dev.forward(x))
     few = synth.normal(152, (3, h))                                   # then a decode-sized call on the same layer
     assert close(dev.forward(few), ora.forward(few))
+
+
+@pytest.mark.parametrize("qtype,h,inter,E,k,tokens,shared_inter,kw", [
+    (capi.IQ2_XXS, 512, 512, 8, 2, 9, 0, {}),                       # 16 units a row: one a lane; 2 pairs an expert
+    (capi.MXFP4, 1280, 384, 8, 3, 12, 384, {}),                     # 40 units over 16 lanes: a ragged third unit
+    (capi.MXFP4, 4352, 128, 4, 2, 7, 128, dict(swiglu_clamp=0.5, swiglu_clamp_shared=0.25)),  # 136 units: 32 lanes, 5 a lane
+    (capi.IQ2_XXS, 8704, 512, 4, 2, 5, 0, {}),                      # 272 units: 64 lanes, 5 a lane, rows of 2244 bytes
+    (capi.IQ2_XXS, 1024, 4608, 6, 2, 40, 0, dict(gating="sigmoid")),  # down rows of 144 units; 13 pairs an expert
+    (capi.MXFP4, 256, 2944, 5, 1, 30, 0, {}),                       # 2944 rows: 23 units (not a multiple of 4 x 16) in gate
+])
+def test_few_pairs_an_expert_stream_past_weights_decoded_once(monkeypatch, qtype, h, inter, E, k, tokens, shared_inter, kw):
+    """Bucketed calls of MXFP4 and IQ2_XXS experts with few pairs an expert: moe_expert_dot8 keeps an expert's rows as
+    int8 words in registers and streams the pairs' activation planes through LDS.  Row lengths that give one to
+    eight units a lane on 16, 32 and 64 lanes a row, a last unit past the row's end, groups of one pair and of
+    many, the folded shared expert (a group with a pair per token) and the clamped activation."""
+    monkeypatch.setenv("JQ_MOE_EXPERT_DOT8_UPTO_PAIRS_PER_EXPERT", "1000")
+    ora, dev = build(qtype, h, inter, E, k, 900 + h, shared_inter=shared_inter, **kw)
+    x = synth.normal(901 + h, (tokens, h))
+    got = dev.forward(x)
+    assert capi.last_kernel() == "moe_expert_dot8"
+    assert close(got, ora.forward(x))
