@@ -331,6 +331,9 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
                                                              False, 0, 0.0)
         elif only == "moe_v3":
             out["moe_deepseek_v3_iq2_xxs_b1"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 1, 105, steps, True, 1, 0.0)
+        elif only == "moe_v3_b64":  # a 64-token call of the same layer: experts decoded once, their pairs streamed past
+            out["moe_deepseek_v3_iq2_xxs_b64"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 64, 105, max(steps // 10, 5),
+                                                              True, 1, 0.0)
         elif only == "moe_v3_b512":  # a 512-token call of the same layer: the grouped int8 GEMM
             out["moe_deepseek_v3_iq2_xxs_b512"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 512, 105, max(steps // 10, 5),
                                                                True, 1, 0.0)
@@ -353,8 +356,10 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
     out["moe_deepseek_v3_iq2_xxs_b1"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 1, 105, max(steps // 4, 10),
                                                      True, 1, cs)
     torch.cuda.empty_cache()
-    # the same layer over 512 tokens (a prompt): the grouped int8 GEMM; no CPU timing (the oracle's parity run is
-    # the bounded sample here)
+    # the same layer over 64 tokens (experts decoded once into registers, their pairs streamed past) and over 512
+    # (a prompt: the grouped int8 GEMM); no CPU timing (the oracle's parity run is the bounded sample here)
+    out["moe_deepseek_v3_iq2_xxs_b64"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 64, 105, 10, True, 1, 0.0)
+    torch.cuda.empty_cache()
     out["moe_deepseek_v3_iq2_xxs_b512"] = moe_workload(torch, capi, synth, 16, 7168, 2048, 256, 8, 512, 105, 8, True, 1, 0.0)
     torch.cuda.empty_cache()
     out["moe_deepseek_v3_mxfp4_b1"] = moe_workload(torch, capi, synth, 39, 7168, 2048, 256, 8, 1, 105, max(steps // 4, 10),

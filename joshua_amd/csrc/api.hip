@@ -1587,7 +1587,11 @@ int launch_moe_expert_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, s
     // lanes a row: the fewest of 16, 32, 64 that leave a lane at most eight units
     const int L = units <= 128 ? 16 : units <= 256 ? 32 : 64, R = 64 / L, ul = (units + L - 1) / L;
     const size_t wgs = (n + jq::EXPERT_DOT8_WAVES * R - 1) / (jq::EXPERT_DOT8_WAVES * R);
-    const int G = (row_bytes % 16 == 0 && base_align >= 16) ? 16 : (row_bytes % 4 == 0 && base_align >= 4) ? 4 : 0;
+    // a wave copies its R rows as one run of bytes: 16 bytes a lane when the run is whole pieces of 16 (IQ2_XXS rows
+    // of 7168: 1848 bytes, two of them 231 pieces), else 4
+    const int G = (((size_t)R * row_bytes) % 16 == 0 && n % R == 0 && base_align >= 16) ? 16
+                  : (row_bytes % 4 == 0 && base_align >= 4)                              ? 4
+                                                                                         : 0;
     const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
     const size_t lds = std::max(jq::EXPERT_DOT8_WAVES * wave_lds, (size_t)2 * 68 * units) + jq::table_bytes<Q>() +
                        8 * Q::I8_EXTRA_ENTRIES;
