@@ -1593,8 +1593,10 @@ int launch_moe_expert_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, s
                   : (row_bytes % 4 == 0 && base_align >= 4)                              ? 4
                                                                                          : 0;
     const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
-    const size_t lds = std::max(jq::EXPERT_DOT8_WAVES * wave_lds, (size_t)2 * 68 * units) + jq::table_bytes<Q>() +
-                       8 * Q::I8_EXTRA_ENTRIES;
+    const size_t tables = jq::table_bytes<Q>() + 8 * Q::I8_EXTRA_ENTRIES, rows_lds = jq::EXPERT_DOT8_WAVES * wave_lds;
+    // the activation buffers behind the rows when both fit, else in their place once the rows are decoded
+    const size_t x_at = rows_lds + (size_t)2 * 68 * units + tables <= 64 * 1024 ? rows_lds : 0;
+    const size_t lds = std::max(rows_lds, x_at + (size_t)2 * 68 * units) + tables;
     if (k % 128 != 0 || ul > 8 || G == 0 || lds > 64 * 1024 || !xq.xl) return -1;
     const size_t words = x_rows * (size_t)(k / 4);
     hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
@@ -1603,10 +1605,10 @@ int launch_moe_expert_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, s
     case UL_:                                                                                                       \
         if (G == 16)                                                                                                \
             hipLaunchKernelGGL((jq::moe_expert_dot8<Q, DUAL, 16, UL_>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp,  \
-                               offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, cl);                                 \
+                               offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, (int)x_at, cl);                      \
         else                                                                                                        \
             hipLaunchKernelGGL((jq::moe_expert_dot8<Q, DUAL, 4, UL_>), grid, block, lds, s, Wa, Wb, row_bytes, xq, gexp,   \
-                               offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, cl);                                 \
+                               offsets, xsel, yrow, Y, k, n, L, (int)wave_lds, (int)x_at, cl);                      \
         break;
     switch (ul) {
         JQ_EXPERT_DOT8(1) JQ_EXPERT_DOT8(2) JQ_EXPERT_DOT8(3) JQ_EXPERT_DOT8(4)

@@ -798,13 +798,13 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
 // buffer holds, for units = k / 32: the first four words of every unit of the low plane, the last four, the
 // same of the high plane, and the units' scales.
 // Dynamic LDS: the format's table and its I8_EXTRA_ENTRIES words of 8 bytes, then
-// max(4 * wave_lds, 2 * 68 * units) bytes.
+// max(4 * wave_lds, x_at + 2 * 68 * units) bytes.
 constexpr int EXPERT_DOT8_WAVES = 4;
 template <class Q, bool DUAL, int G, int UL>
 __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
     const uint8_t *const *__restrict__ Wa, const uint8_t *const *__restrict__ Wb, size_t row_bytes, ActsI8 xq,
     const int *__restrict__ gexp, const int *__restrict__ offsets, const int *__restrict__ xsel,
-    const int *__restrict__ yrow, float *__restrict__ Y, int k, int n, int L, int wave_lds, MoeClamp cl) {
+    const int *__restrict__ yrow, float *__restrict__ Y, int k, int n, int L, int wave_lds, int x_at, MoeClamp cl) {
     static_assert(Q::SEGS == 1 && Q::SEGLEN == 32 && Q::HAS_DECODE_I8, "units of 32 consecutive elements");
     extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
     const int grp = (int)gridDim.y - 1 - (int)blockIdx.y;
@@ -818,7 +818,7 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
         const size_t xr = (size_t)xsel[beg + p];
         const uint8_t *xl = (const uint8_t *)(xq.xl + xr * (size_t)(k / 4)), *xh = (const uint8_t *)(xq.xh + xr * (size_t)(k / 4));
         const uint8_t *sx = (const uint8_t *)(xq.sx + xr * (size_t)(k / 32));
-        uint8_t *dst = base + (size_t)buf * x_lds;
+        uint8_t *dst = base + x_at + (size_t)buf * x_lds;
         for (int c0 = 64 * wave; c0 < chunks; c0 += 64 * EXPERT_DOT8_WAVES) {
             const int c = c0 + lane;
             if (c < chunks) {
@@ -853,6 +853,7 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
             }
         }
     }
+    if (x_at) copy(0, 0);  // the activations have room of their own: the first pair comes in beside the rows
     if ((int)threadIdx.x < Q::I8_EXTRA_ENTRIES)
         ((uint64_t *)(staged_moe + table_bytes<Q>()))[threadIdx.x] = Q::i8_extra_entry((int)threadIdx.x);
     const auto *table = stage_table<Q>(staged_moe);  // holds a barrier when the format has a table
@@ -878,13 +879,15 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
             if (DUAL) db[j] = 0.0f;
         }
     }
-    __syncthreads();  // every wave holds its weights: the rows' LDS now takes the activations
-    copy(0, 0);
+    if (!x_at) {
+        __syncthreads();  // every wave holds its weights: the rows' LDS now takes the activations
+        copy(0, 0);
+    }
     for (int p = 0; p < cnt; p++) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();  // pair p's planes are in; every wave is done with pair p - 1's buffer
         if (p + 1 < cnt) copy(p + 1, (p + 1) & 1);
-        const uint8_t *xb = base + (size_t)(p & 1) * x_lds;
+        const uint8_t *xb = base + x_at + (size_t)(p & 1) * x_lds;
         float acc = 0.0f, acc2 = 0.0f;
         // a unit's activations: eight words of each plane and the scale.  The next unit's are asked for before
         // this unit's products; the fences keep the compiler from asking for every unit's at once (17 registers
