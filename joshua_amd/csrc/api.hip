@@ -1370,7 +1370,7 @@ bool moe_has_dot8(uint32_t type) {
 // Formats whose units decode to signed int8 words (Q::decode_i8): bucketed calls of few pairs an expert can
 // run on moe_expert_dot8.
 bool moe_has_decode_i8(uint32_t type) {
-    return (type == JQ_TYPE_MXFP4 || type == JQ_TYPE_IQ2_XXS) && moe_has_dot8(type);
+    return (type == JQ_TYPE_MXFP4 || type == JQ_TYPE_IQ2_XXS || type == JQ_TYPE_Q4_K) && moe_has_dot8(type);
 }
 
 // Formats with a side of the int8 GEMM (kq_gemm_i8): their grouped expert matmuls run on it.
@@ -1584,8 +1584,9 @@ int launch_moe_expert_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, s
                            const int *yrow, float *Y, int k, int n, int groups, hipStream_t s,
                            const jq::MoeClamp &cl = jq::MoeClamp{}) {
     const int units = k / 32;
-    // lanes a row: the fewest of 16, 32, 64 that leave a lane at most eight units
-    const int L = units <= 128 ? 16 : units <= 256 ? 32 : 64, R = 64 / L, ul = (units + L - 1) / L;
+    // lanes a row: the fewest of 16, 32, 64 that leave a lane at most seven units (eight for the longest rows)
+    const int L = units <= 112 ? 16 : units <= 224 ? 32 : 64, R = 64 / L, ul = (units + L - 1) / L;
+    constexpr size_t XB = 68 + (Q::I8_HAS_MIN ? 4 : 0);
     const size_t wgs = (n + jq::EXPERT_DOT8_WAVES * R - 1) / (jq::EXPERT_DOT8_WAVES * R);
     // a wave copies its R rows as one run of bytes: 16 bytes a lane when the run is whole pieces of 16 (IQ2_XXS rows
     // of 7168: 1848 bytes, two of them 231 pieces), else 4
@@ -1595,8 +1596,8 @@ int launch_moe_expert_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, s
     const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
     const size_t tables = jq::table_bytes<Q>() + 8 * Q::I8_EXTRA_ENTRIES, rows_lds = jq::EXPERT_DOT8_WAVES * wave_lds;
     // the activation buffers behind the rows when both fit, else in their place once the rows are decoded
-    const size_t x_at = rows_lds + (size_t)2 * 68 * units + tables <= 64 * 1024 ? rows_lds : 0;
-    const size_t lds = std::max(rows_lds, x_at + (size_t)2 * 68 * units) + tables;
+    const size_t x_at = rows_lds + 2 * XB * units + tables <= 64 * 1024 ? rows_lds : 0;
+    const size_t lds = std::max(rows_lds, x_at + 2 * XB * units) + tables;
     if (k % 128 != 0 || ul > 8 || G == 0 || lds > 64 * 1024 || !xq.xl) return -1;
     const size_t words = x_rows * (size_t)(k / 4);
     hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
@@ -1633,6 +1634,9 @@ int dispatch_moe_expert_dot8(uint32_t type, const uint8_t *const *Wa, const uint
     case JQ_TYPE_IQ2_XXS:
         return launch_moe_expert_dot8<jq::IQ2_XXS, DUAL>(Wa, Wb, row_bytes, base_align, X, x_rows, xq, gexp, offsets, xsel,
                                                          yrow, Y, k, n, groups, s, cl);
+    case JQ_TYPE_Q4_K:
+        return launch_moe_expert_dot8<jq::Q4_K, DUAL>(Wa, Wb, row_bytes, base_align, X, x_rows, xq, gexp, offsets, xsel, yrow,
+                                                      Y, k, n, groups, s, cl);
     default: return -1;
     }
 }
@@ -1851,16 +1855,15 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     int groups, max_group;
     // Decode-sized (one group a pair, every pair reading its expert's rows) or bucketed by expert (every expert hit
     // read once)?  A pair costs about a = 0.10 + 0.17 bytes-per-weight ns a weight on the integer-dot kernels;
-    // a bucketed expert costs g = 0.45 ns a weight on the grouped int8 GEMM (bound by the unpacking) and 0.28 on the
-    // Q4_K kernels for short rows.  With d(P) = E (1 - (1 - 1/E)^P) experts hit by P pairs, pairs win while
-    // P a <= d(P) g (Qwen3-30B-A3B sizes: up to ~100 pairs over 128 experts; DeepSeek-V3 sizes, IQ2_XXS: ~750 over
-    // 256).  Formats without integer-dot kernels keep pairs up to the number of experts.
-    // JQ_MOE_DECODE_PAIRS_PCT: pairs, in percent of the experts, up to which a call is decode-sized.
-    // MXFP4 and IQ2_XXS have a third way, bucketed with the expert's rows decoded once into registers and the pairs
+    // a bucketed expert costs g = 0.45 ns a weight on the grouped int8 GEMM (bound by the unpacking; 0.36 for Q4_K)
+    // and 0.28 on the Q4_K kernels for short rows.  With d(P) = E (1 - (1 - 1/E)^P) experts hit by P pairs, pairs win
+    // while P a <= d(P) g (Qwen3-30B-A3B sizes: up to ~100 pairs over 128 experts).  Formats without integer-dot
+    // kernels keep pairs up to the number of experts.
+    // MXFP4, IQ2_XXS and Q4_K have a third way, bucketed with the expert's rows decoded once into registers and the pairs
     // streamed past them (moe_expert_dot8): x = 0.10 ns a weight and expert hit plus 0.032 a pair, and about 90 us a
     // call for its launches over every (expert, row tile), most of them empty when few experts are hit.  At
-    // DeepSeek-V3's sizes it is the cheapest from ~10 tokens (16 tokens of IQ2_XXS: 0.76 ms against 0.89 by pairs;
-    // 64: 1.90 against 3.15; 256: 4.50 against the GEMM's 5.09) to ~350, where the GEMM takes over.
+    // DeepSeek-V3's sizes it is the cheapest from ~10 tokens (16 tokens of IQ2_XXS: 0.73 ms against 0.89 by pairs;
+    // 64: 1.76 against 3.15; 256: 4.33 against the GEMM's 5.09) to ~350 (Q4_K: ~250), where the GEMM takes over.
     // JQ_MOE_DECODE_PAIRS_PCT: pairs, in percent of the experts, up to which a call is decode-sized.
     // JQ_MOE_EXPERT_DOT8_UPTO_PAIRS_PER_EXPERT: bucketed calls take moe_expert_dot8 up to this many pairs an expert
     // on average (0: never).
@@ -1878,7 +1881,8 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
                c.hidden % 256 == 0 && c.inter % 256 == 0) {
         const double bpw = (double)m->gate->row_bytes / (double)c.hidden;
         const bool short_q4k = m->gate->type == JQ_TYPE_Q4_K && c.hidden <= 2048 && c.inter <= 2048;
-        const double a = 0.10 + 0.17 * bpw, g = short_q4k ? 0.28 : 0.45;
+        // (Q4_K unpacks for less: a 256-token call of DeepSeek-V3-sized Q4_K experts, 3.8 ms, is 0.34 an expert)
+        const double a = 0.10 + 0.17 * bpw, g = short_q4k ? 0.28 : m->gate->type == JQ_TYPE_Q4_K ? 0.36 : 0.45;
         const double hit = (double)c.n_expert * (1.0 - std::pow(1.0 - 1.0 / (double)c.n_expert, (double)P));
         const double by_pairs = (double)P * a, by_gemm = hit * g;
         double by_expert = INFINITY;
@@ -1940,7 +1944,13 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     const bool prefer_gemm = m->gacts && max_group > 1 && (size_t)P >= gemm_from * (size_t)c.n_expert &&
                              c.hidden % 256 == 0 && c.inter % 256 == 0 && a16 >= 16 &&
                              align_of({m->down, m->fold_shared ? m->sdown : nullptr}) >= 16;
-    if (same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K && few)
+    // few pairs an expert, by the cost estimate above: the expert's rows decoded once, its pairs streamed past
+    const bool multi = max_group > 1 && expert_dot8;
+    if (same_gu && multi)
+        rc = dispatch_moe_expert_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
+                                            m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
+    if (rc > 0) return 1;
+    if (rc < 0 && same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K && few)
         rc = dispatch_moe_q4k_quads<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp, m->offsets,
                                           m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
     if (rc > 0) return 1;
@@ -1950,11 +1960,6 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     if (rc > 0) return 1;
     // bucketed, any format with a side of the int8 GEMM: gate -> G and up -> U from one preparation of x, then
     // the activation in place
-    const bool multi = max_group > 1 && expert_dot8;
-    if (rc < 0 && same_gu && multi)
-        rc = dispatch_moe_expert_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
-                                           m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
-    if (rc > 0) return 1;
     bool planned = false;
     if (rc < 0 && same_gu && max_group > 1 && m->gacts) {
         moe_gemm_plan(m, groups, (size_t)P + (size_t)extra * T, s);
@@ -1993,7 +1998,12 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     }
     const int d16 = align_of({m->down, m->fold_shared ? m->sdown : nullptr});
     rc = -1;
-    if (fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && few)
+    if (fused_act && multi)
+        rc = dispatch_moe_expert_dot8<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G,
+                                             (size_t)P + extra * T, m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out,
+                                             (int)c.inter, (int)c.hidden, groups, s);
+    if (rc > 0) return 1;
+    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && few)
         rc = dispatch_moe_q4k_quads<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                            m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                            (int)c.hidden, groups, s);
@@ -2002,11 +2012,6 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);
-    if (rc > 0) return 1;
-    if (rc < 0 && fused_act && multi)
-        rc = dispatch_moe_expert_dot8<false>(m->down->type, m->pdown, nullptr, m->down->row_bytes, d16, m->G,
-                                            (size_t)P + extra * T, m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out,
-                                            (int)c.inter, (int)c.hidden, groups, s);
     if (rc > 0) return 1;
     if (rc < 0 && fused_act && max_group > 1 && m->gacts) {
         if (!planned) moe_gemm_plan(m, groups, (size_t)P + (size_t)extra * T, s);

@@ -345,6 +345,22 @@ struct Q4_K {  // d | dmin | scales[12] | qs[128]   (reference: src/kquant_dot.r
         const float acc = d * fmaf((float)sc0, f0, (float)sc1 * f1);
         return fmaf(-dmin, fmaf((float)mn0, sxs[0], (float)mn1 * sxs[1]), acc);
     }
+    // Sub-block u (32 elements, eight a block) as eight words of int8: its nibbles 0..15 as they are, the
+    // scale d * sc_u that goes with their sum and the offset dmin * m_u that goes with the activations' sum.
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = true;
+    static constexpr int I8_UNITS = 8, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int u, int *w, float &scale, float &offset) {
+        const uint4 hdr = ld<uint4>(blk);
+        uint32_t sc, mn;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, u, sc, mn);
+        const uint4 qa = ld<uint4>(blk + 16 + 32 * (u >> 1)), qb = ld<uint4>(blk + 32 + 32 * (u >> 1));
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) w[i] = (int)((q[i] >> (4 * (u & 1))) & 0x0F0F0F0Fu);
+        scale = f16_bits(hdr.x) * (float)sc;
+        offset = f16_bits(hdr.x >> 16) * (float)mn;
+    }
 };
 
 struct Q2_K {  // scales[16] | qs[64] | d | dmin   (reference: src/kquant_dot.rs:63-76,345-385)
@@ -517,15 +533,16 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
     // The table is the codebook (entries 0..255) followed by the 128 sign patterns as byte masks (entry 256 + s:
     // byte j is 0xFF where element j of a group with the seven sign bits s is negative), which the caller
     // fills with i8_extra_entry.
-    static constexpr bool HAS_DECODE_I8 = true;
-    static constexpr int I8_EXTRA_ENTRIES = 128;
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = false;
+    static constexpr int I8_UNITS = 8, I8_EXTRA_ENTRIES = 128;
     __device__ static uint64_t i8_extra_entry(int s7) {
         const uint32_t signs = (uint32_t)s7 | ((__popc((uint32_t)s7) & 1u) << 7);
         const uint32_t lo = ((signs & 15u) * 0x00204081u & 0x01010101u) * 0xFFu;
         const uint32_t hi = ((signs >> 4) * 0x00204081u & 0x01010101u) * 0xFFu;
         return ((uint64_t)hi << 32) | lo;
     }
-    __device__ static void decode_i8(const uint64_t *grid_table, const uint8_t *blk, int u, int *w, float &scale) {
+    __device__ static void decode_i8(const uint64_t *grid_table, const uint8_t *blk, int u, int *w, float &scale, float &offset) {
+        offset = 0.0f;
         const float d = f16_bits(ld<uint16_t>(blk));
         const uint2 g = ldw<uint2>(blk + 2 + 8 * u);
         const uint32_t lo = g.x, hi = g.y;
@@ -588,10 +605,11 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
     // The block as eight words of signed int8, twice the E2M1 values (elements 4i .. 4i+3 in word i, the low
     // nibbles first), and the scale that goes with them (half the block's): two lookups, of the doubled
     // magnitudes and of their negatives, and the sign bit picks between them byte by byte.
-    static constexpr bool HAS_DECODE_I8 = true;
-    static constexpr int I8_EXTRA_ENTRIES = 0;
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = false;
+    static constexpr int I8_UNITS = 1, I8_EXTRA_ENTRIES = 0;
     __device__ static uint64_t i8_extra_entry(int) { return 0; }
-    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale) {
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale, float &offset) {
+        offset = 0.0f;
         const uint32_t e = blk[0];
         const uint4 qv = ldw<uint4>(blk + 1);
         const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};

@@ -796,28 +796,31 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_dot8(const uint8_t 
 // area becomes the activation buffers once every wave has decoded.  Groups are taken from the last down: a
 // folded shared expert, the one group with a pair per token, is the last group and starts first.  A pair's
 // buffer holds, for units = k / 32: the first four words of every unit of the low plane, the last four, the
-// same of the high plane, and the units' scales.
+// same of the high plane, the units' scales and, for formats with an offset a sub-block (Q4_K), the units' scaled
+// sums.
 // Dynamic LDS: the format's table and its I8_EXTRA_ENTRIES words of 8 bytes, then
-// max(4 * wave_lds, x_at + 2 * 68 * units) bytes.
+// max(4 * wave_lds, x_at + 2 * (68 or 72) * units) bytes.
 constexpr int EXPERT_DOT8_WAVES = 4;
 template <class Q, bool DUAL, int G, int UL>
 __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
     const uint8_t *const *__restrict__ Wa, const uint8_t *const *__restrict__ Wb, size_t row_bytes, ActsI8 xq,
     const int *__restrict__ gexp, const int *__restrict__ offsets, const int *__restrict__ xsel,
     const int *__restrict__ yrow, float *__restrict__ Y, int k, int n, int L, int wave_lds, int x_at, MoeClamp cl) {
-    static_assert(Q::SEGS == 1 && Q::SEGLEN == 32 && Q::HAS_DECODE_I8, "units of 32 consecutive elements");
+    static_assert(Q::HAS_DECODE_I8 && Q::BLOCK_ELEMS == 32 * Q::I8_UNITS, "units of 32 consecutive elements");
+    constexpr int XB = 68 + (Q::I8_HAS_MIN ? 4 : 0);  // bytes of a pair's buffer a unit
     extern __shared__ __attribute__((aligned(16))) uint8_t staged_moe[];
     const int grp = (int)gridDim.y - 1 - (int)blockIdx.y;
     const int beg = offsets[grp], cnt = offsets[grp + 1] - beg;
     if (cnt == 0) return;  // the whole workgroup
     const int e = gexp[grp];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int units = k / 32, x_lds = 68 * units, chunks = 4 * units + units / 4;  // 16-byte pieces of a pair's planes and scales
+    const int units = k / 32, x_lds = XB * units;
+    const int chunks = 4 * units + (Q::I8_HAS_MIN ? 2 : 1) * (units / 4);  // 16-byte pieces of a pair's planes and scales
     uint8_t *base = staged_moe + table_bytes<Q>() + 8 * Q::I8_EXTRA_ENTRIES;
     auto copy = [&](int p, int buf) {
         const size_t xr = (size_t)xsel[beg + p];
         const uint8_t *xl = (const uint8_t *)(xq.xl + xr * (size_t)(k / 4)), *xh = (const uint8_t *)(xq.xh + xr * (size_t)(k / 4));
-        const uint8_t *sx = (const uint8_t *)(xq.sx + xr * (size_t)(k / 32));
+        const uint8_t *sx = (const uint8_t *)(xq.sx + xr * (size_t)(k / 32)), *sxs = (const uint8_t *)(xq.sxs + xr * (size_t)(k / 32));
         uint8_t *dst = base + x_at + (size_t)buf * x_lds;
         for (int c0 = 64 * wave; c0 < chunks; c0 += 64 * EXPERT_DOT8_WAVES) {
             const int c = c0 + lane;
@@ -826,8 +829,10 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
                 if (c < 4 * units) {
                     const int q = c / units, u = c - q * units;  // q: low plane first half, second half, high plane ...
                     src = ((q & 2) ? xh : xl) + 32 * u + 16 * (q & 1);
-                } else {
+                } else if (!Q::I8_HAS_MIN || c < 4 * units + units / 4) {
                     src = sx + 16 * (c - 4 * units);
+                } else {
+                    src = sxs + 16 * (c - 4 * units - units / 4);
                 }
                 async_load16(src, lds_offset_of(dst + (size_t)c0 * 16));
             }
@@ -861,15 +866,24 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
     const bool active = rl < nrows;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows landed (this wave's own data)
     int wa[UL][8], wb[DUAL ? UL : 1][8];
-    float da[UL], db[DUAL ? UL : 1];
+    float da[UL], db[DUAL ? UL : 1], oa[Q::I8_HAS_MIN ? UL : 1], ob[Q::I8_HAS_MIN && DUAL ? UL : 1];
 #pragma unroll
     for (int j = 0; j < UL; j++) {
         const int u = sub + L * j;
         if (active && u < units) {
-            const size_t at = (size_t)rl * row_bytes + (size_t)(u / Q::UNITS) * Q::BLOCK_BYTES;
-            Q::decode_i8(table, ra + at, u % Q::UNITS, wa[j], da[j]);
-            if (DUAL) Q::decode_i8(table, rb + at, u % Q::UNITS, wb[j], db[j]);
+            const size_t at = (size_t)rl * row_bytes + (size_t)(u / Q::I8_UNITS) * Q::BLOCK_BYTES;
+            float o, o2 = 0.0f;
+            Q::decode_i8(table, ra + at, u % Q::I8_UNITS, wa[j], da[j], o);
+            if (DUAL) Q::decode_i8(table, rb + at, u % Q::I8_UNITS, wb[j], db[j], o2);
+            if (Q::I8_HAS_MIN) {
+                oa[j] = o;
+                if (DUAL) ob[j] = o2;
+            }
         } else {
+            if (Q::I8_HAS_MIN) {
+                oa[j] = 0.0f;
+                if (DUAL) ob[j] = 0.0f;
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 wa[j][i] = 0;
@@ -894,7 +908,7 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
         // a unit, which with the weights would not fit).
         struct UnitX {
             uint4 l0, l1, h0, h1;
-            float sx;
+            float sx, sxs;
         };
         auto unit_x = [&](int j) {
             const int u = min(sub + L * j, units - 1);  // past the row's end: zero weights against the last unit
@@ -902,6 +916,7 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
             x.l0 = *(const uint4 *)(xb + 16 * u), x.l1 = *(const uint4 *)(xb + 16 * (units + u));
             x.h0 = *(const uint4 *)(xb + 16 * (2 * units + u)), x.h1 = *(const uint4 *)(xb + 16 * (3 * units + u));
             x.sx = *(const float *)(xb + 64 * units + 4 * u);
+            x.sxs = Q::I8_HAS_MIN ? *(const float *)(xb + 68 * units + 4 * u) : 0.0f;
             return x;
         };
         UnitX cur = unit_x(0);
@@ -925,8 +940,10 @@ __global__ __launch_bounds__(64 * EXPERT_DOT8_WAVES) void moe_expert_dot8(
                 }
             }
             acc = fmaf(cur.sx * da[j], (float)((ph << 8) + pl), acc);
+            if (Q::I8_HAS_MIN) acc = fmaf(-oa[j], cur.sxs, acc);
             if (DUAL) {
                 acc2 = fmaf(cur.sx * db[j], (float)((ph2 << 8) + pl2), acc2);
+                if (Q::I8_HAS_MIN) acc2 = fmaf(-ob[j], cur.sxs, acc2);
                 // both sums are due here: left alone, the second matrix's products of every unit are put after
                 // the first's, with every unit's activations held until then
                 asm volatile("" : "+v"(acc), "+v"(acc2));

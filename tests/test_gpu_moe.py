@@ -290,9 +290,12 @@ def test_many_tokens_take_the_grouped_int8_gemm(qtype, h, inter, E, k, tokens, s
     (capi.IQ2_XXS, 8704, 512, 4, 2, 5, 0, {}),                      # 272 units: 64 lanes, 5 a lane, rows of 2244 bytes
     (capi.IQ2_XXS, 1024, 4608, 6, 2, 40, 0, dict(gating="sigmoid")),  # down rows of 144 units; 13 pairs an expert
     (capi.MXFP4, 256, 2944, 5, 1, 30, 0, {}),                       # 2944 rows: 23 units (not a multiple of 4 x 16) in gate
+    (capi.Q4_K, 512, 256, 8, 2, 9, 0, {}),                          # Q4_K: an offset a sub-block against the activations' sums
+    (capi.Q4_K, 4096, 1536, 8, 2, 24, 1536, dict(swiglu_clamp=0.75, swiglu_clamp_shared=0.5)),  # Qwen3-235B-A22B row lengths
+    (capi.Q4_K, 7168, 256, 4, 2, 6, 0, dict(gating="sigmoid")),     # rows of 28 super-blocks: seven units a lane
 ])
 def test_few_pairs_an_expert_stream_past_weights_decoded_once(monkeypatch, qtype, h, inter, E, k, tokens, shared_inter, kw):
-    """Bucketed calls of MXFP4 and IQ2_XXS experts with few pairs an expert: moe_expert_dot8 keeps an expert's rows as
+    """Bucketed calls of MXFP4, IQ2_XXS and Q4_K experts with few pairs an expert: moe_expert_dot8 keeps an expert's rows as
     int8 words in registers and streams the pairs' activation planes through LDS.  Row lengths that give one to
     eight units a lane on 16, 32 and 64 lanes a row, a last unit past the row's end, groups of one pair and of
     many, the folded shared expert (a group with a pair per token) and the clamped activation."""
