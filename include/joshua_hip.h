@@ -222,7 +222,14 @@ int jq_moe_route(jq_moe *moe, size_t n_tokens, const float *x, uint32_t *ids, fl
                  int ptrs_are_device, void *stream);
 
 /* y[n_tokens, h] = MoE(x[n_tokens, h]).  One call at a time per jq_moe (it owns
- * its scratch buffers). */
+ * its scratch buffers).  Accuracy as for jq_matmul_t, with the expert matmuls' inputs
+ * (x, and silu(gate) * up for the down projection) in 16-bit fixed point: one scale
+ * per 32 elements on the integer-dot kernels, per 256 on the grouped GEMM.  The error
+ * grows with a row's largest magnitude: measured at 8192 columns with gate and up
+ * results of standard deviation 1.8 (activations up to 50, outputs up to 40), the
+ * mean error is 6e-5 of max(|ref|, 1) on the integer-dot kernels and 1.4e-4 on the
+ * grouped GEMM, which then passes 1e-3 on 0.3 % of the elements (largest 2.7e-3);
+ * with inputs of the magnitude a normed layer gives the bound holds on every path. */
 int jq_moe_forward(jq_moe *moe, size_t n_tokens, const float *x, float *y, int ptrs_are_device, void *stream);
 
 /* ---- Multi-head latent attention (DeepSeek-V2 / V3 / Kimi-K2) -----------------------

@@ -305,3 +305,38 @@ def test_few_pairs_an_expert_stream_past_weights_decoded_once(monkeypatch, qtype
     got = dev.forward(x)
     assert capi.last_kernel() == "moe_expert_dot8"
     assert close(got, ora.forward(x))
+
+
+def _random_expert_layers():
+    rng = np.random.default_rng(20251125)
+    cases = []
+    for seed in range(10):
+        qtype = [capi.MXFP4, capi.IQ2_XXS, capi.Q4_K][seed % 3]
+        step = 512 if qtype == capi.IQ2_XXS else 256     # IQ2_XXS rows a multiple of 4 bytes: 512 columns
+        for _ in range(100):
+            h, inter = step * int(rng.integers(1, 17)), step * int(rng.integers(1, 7))
+            E = int(rng.integers(2, 13))
+            if h * inter * E <= 12 << 20:
+                break
+        k = int(rng.integers(1, min(E, 4) + 1))
+        tokens = int(rng.integers(E // k + 1, 70))       # more pairs than experts
+        shared = inter if rng.integers(0, 2) else 0
+        cases.append((qtype, h, inter, E, k, tokens, shared, 950 + seed))
+    return cases
+
+
+@pytest.mark.parametrize("qtype,h,inter,E,k,tokens,shared_inter,seed", _random_expert_layers())
+def test_expert_kernel_at_seeded_random_layers(monkeypatch, qtype, h, inter, E, k, tokens, shared_inter, seed):
+    """moe_expert_dot8 at layer shapes drawn from a fixed seed: row lengths of 8 to 256 units (every lanes-a-row
+    and units-a-lane combination comes up), 2 to 12 experts, top-1 to top-4, with and without the folded shared
+    expert, against the oracle's layer.  The inputs are scaled so that gate and up results keep a standard
+    deviation of about one at every row length, as a layer's normed activations give: unit-variance inputs
+    against 8192 columns of weights of 0.02 make them 1.8 and the activations reach 50, where the fixed-point
+    planes' error (in proportion to a row's largest magnitude) sits at the tolerance itself (one element of
+    253952 at 1.06e-3)."""
+    monkeypatch.setenv("JQ_MOE_EXPERT_DOT8_UPTO_PAIRS_PER_EXPERT", "1000")
+    ora, dev = build(qtype, h, inter, E, k, seed, shared_inter=shared_inter)
+    x = synth.normal(seed + 1, (tokens, h)) * np.float32(min(1.0, 1.0 / (0.02 * np.sqrt(h))))
+    got = dev.forward(x)
+    assert capi.last_kernel() == "moe_expert_dot8", (h, inter, E, k, tokens)
+    assert close(got, ora.forward(x))
