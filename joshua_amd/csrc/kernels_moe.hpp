@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict
     }
 }
 
-// The same logits for many tokens: one workgroup per (8 router rows, 8 tokens), so a token's activations are read
+// The same logits for several tokens: one workgroup per (8 router rows, 8 tokens), so a token's activations are read
 // once per eight experts instead of once per expert (512 tokens x 256 experts of 7168: 228 -> 60 us).  Every
 // logit is accumulated by the same thread over the same columns in the same order as in moe_router_logits and
 // reduced the same way, so the two kernels give the same bits.
