@@ -182,9 +182,12 @@ __device__ __forceinline__ void q4k_scale_min_pair(uint32_t s0, uint32_t s1, uin
 }
 
 // IQ2_XXS codebook expanded at compile time to 256 x 8 bytes (value j of entry
-// c in byte j), from the base-3 packed form in iq2xxs_grid_codes.h.
+// c in byte j), from the base-3 packed form in iq2xxs_grid_codes.h, followed by the
+// 128 sign patterns of a group of eight as byte masks: entry 256 + s holds 0xFF in
+// byte j where element j is negative, for the seven stored sign bits s and the
+// eighth that makes their number even (reference: src/iq2xxs.rs:349-380).
 struct Tables {
-    uint64_t iq2xxs_grid[256];
+    uint64_t iq2xxs_grid[384];
     constexpr Tables() : iq2xxs_grid{} {
         for (int i = 0; i < 256; i++) {
             unsigned c = JQ_IQ2XXS_GRID_TRITS[i];
@@ -195,6 +198,15 @@ struct Tables {
                 v |= (uint64_t)(8 + 17 * t + (t >> 1)) << (8 * j);
             }
             iq2xxs_grid[i] = v;
+        }
+        for (unsigned s = 0; s < 128; s++) {
+            unsigned ones = 0;
+            for (int j = 0; j < 7; j++) ones += (s >> j) & 1u;
+            const unsigned signs = s | ((ones & 1u) << 7);
+            uint64_t v = 0;
+            for (int j = 0; j < 8; j++)
+                if ((signs >> j) & 1u) v |= (uint64_t)0xFF << (8 * j);
+            iq2xxs_grid[256 + s] = v;
         }
     }
 };
@@ -478,7 +490,7 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
     __device__ static int elem_base(int u) { return 32 * u; }
     // `grid` is the 256-entry codebook: the constant table, or a workgroup's copy of it in LDS
     // (TABLE_BYTES), where the four lookups of a group cost LDS instead of vector-memory latency.
-    static constexpr int TABLE_BYTES = 2048;
+    static constexpr int TABLE_BYTES = 3072;  // the codebook and the sign masks behind it
     __device__ static const uint64_t *table() { return g_tables.iq2xxs_grid; }
     __device__ static void decode_with(const uint64_t *grid_table, const uint8_t *blk, int u, float *w) {
         float d = f16_bits(ld<uint16_t>(blk));
@@ -498,49 +510,35 @@ struct IQ2_XXS {  // d | 8 x (lo:u32 codes, hi:u32 signs+scale)   (reference: sr
         }
     }
     __device__ static void decode(const uint8_t *blk, int u, float *w) { decode_with(g_tables.iq2xxs_grid, blk, u, w); }
-    // Unit u (32 elements) against its activations as two int8 planes: the codebook's magnitude bytes go
-    // to v_dot4 as they are; the 8 sign bits of a group are spread to byte masks (a multiply moves bit j
-    // of a nibble to bit 8j) and a negative element counts twice in a second sum instead of being negated.
+    // Unit u (32 elements) against its activations as two int8 planes: the codebook's magnitudes 8, 25, 43 are
+    // negated byte by byte where the group's sign mask (table entry 256 + s) says so ((m ^ 0xFF) + 1 = 256 - m
+    // never carries for m >= 8) and go to v_dot4 as signed bytes, so the integer arithmetic is exact.
     static constexpr bool HAS_DOT8 = true;
     __device__ static float dot8(const uint64_t *grid_table, const uint8_t *blk, int u, const uint32_t *xl,
                                  const uint32_t *xh, const float *sx, const float *) {
         const float d = f16_bits(ld<uint16_t>(blk));
         const uint2 g = ldw<uint2>(blk + 2 + 8 * u);
         const uint32_t lo = g.x, hi = g.y;
-        int pl = 0, ph = 0, nl = 0, nh = 0;
+        int pl = 0, ph = 0;
 #pragma unroll
         for (int l = 0; l < 4; l++) {
             const uint64_t grid = grid_table[(lo >> (8 * l)) & 0xFFu];
-            const uint32_t s7 = (hi >> (7 * l)) & 127u;
-            const uint32_t signs = s7 | ((__popc(s7) & 1u) << 7);
+            const uint64_t neg = grid_table[256 + ((hi >> (7 * l)) & 127u)];
 #pragma unroll
             for (int hf = 0; hf < 2; hf++) {  // elements 8l + 4hf .. + 3
-                const int mag = (int)(uint32_t)(grid >> (32 * hf));
-                const uint32_t bits = ((signs >> (4 * hf)) & 15u) * 0x00204081u & 0x01010101u;
-                const int neg = mag & (int)(bits * 0xFFu);
-                pl = __builtin_amdgcn_sdot4(mag, (int)xl[2 * l + hf], pl, false);
-                ph = __builtin_amdgcn_sdot4(mag, (int)xh[2 * l + hf], ph, false);
-                nl = __builtin_amdgcn_sdot4(neg, (int)xl[2 * l + hf], nl, false);
-                nh = __builtin_amdgcn_sdot4(neg, (int)xh[2 * l + hf], nh, false);
+                const uint32_t mag = (uint32_t)(grid >> (32 * hf)), mask = (uint32_t)(neg >> (32 * hf));
+                const int w = (int)((mag ^ mask) + (mask & 0x01010101u));
+                pl = __builtin_amdgcn_sdot4(w, (int)xl[2 * l + hf], pl, false);
+                ph = __builtin_amdgcn_sdot4(w, (int)xh[2 * l + hf], ph, false);
             }
         }
         const float db = d * (0.5f + (float)(hi >> 28)) * 0.25f;
-        return sx[0] * db * (float)(((ph - 2 * nh) << 8) + (pl - 2 * nl));
+        return sx[0] * db * (float)((ph << 8) + pl);
     }
-    // Unit u as eight words of signed int8 (elements 4i .. 4i+3 in word i) and its scale: the codebook's
-    // magnitudes 8, 25, 43 negated byte by byte where the sign bit is set ((m ^ 0xFF) + 1 = 256 - m never
-    // carries for m >= 8).
-    // The table is the codebook (entries 0..255) followed by the 128 sign patterns as byte masks (entry 256 + s:
-    // byte j is 0xFF where element j of a group with the seven sign bits s is negative), which the caller
-    // fills with i8_extra_entry.
+    // Unit u as eight words of signed int8 (elements 4i .. 4i+3 in word i) and its scale, the same way.
     static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = false;
-    static constexpr int I8_UNITS = 8, I8_EXTRA_ENTRIES = 128;
-    __device__ static uint64_t i8_extra_entry(int s7) {
-        const uint32_t signs = (uint32_t)s7 | ((__popc((uint32_t)s7) & 1u) << 7);
-        const uint32_t lo = ((signs & 15u) * 0x00204081u & 0x01010101u) * 0xFFu;
-        const uint32_t hi = ((signs >> 4) * 0x00204081u & 0x01010101u) * 0xFFu;
-        return ((uint64_t)hi << 32) | lo;
-    }
+    static constexpr int I8_UNITS = 8, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
     __device__ static void decode_i8(const uint64_t *grid_table, const uint8_t *blk, int u, int *w, float &scale, float &offset) {
         offset = 0.0f;
         const float d = f16_bits(ld<uint16_t>(blk));
@@ -573,8 +571,8 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
     }
     // The block against its 32 activations given as 15-bit fixed point in two int8 planes (X = 256 hi +
     // lo, eight registers a plane): v_perm_b32 looks four magnitude codes up at once in the table of
-    // doubled E2M1 values {0,1,2,3,4,6,8,12}; a negative element counts twice in a second sum instead of
-    // being negated (sum w X = sum |w| X - 2 sum_{w<0} |w| X), so the integer arithmetic is exact.
+    // doubled E2M1 values {0,1,2,3,4,6,8,12} and once more in the table of their negatives, the sign bits
+    // pick between the two byte by byte, and the signed bytes go to v_dot4, so the integer arithmetic is exact.
     // Returns sum w_i x_i over the block: sx is the activations' scale, x = sx X.
     static constexpr bool HAS_DOT8 = true;
     __device__ static float dot8(const uint64_t *, const uint8_t *blk, int, const uint32_t *xl, const uint32_t *xh,
@@ -582,24 +580,24 @@ struct MXFP4 {  // e:u8 | qs[16]   (reference: src/mxfp4.rs:45-94)
         const uint32_t e = blk[0];
         if (e == 0xFFu) return 0.0f;
         const float d = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
-        int pl = 0, ph = 0, nl = 0, nh = 0;
+        int pl = 0, ph = 0;
         const uint4 qv = ldw<uint4>(blk + 1);
         const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t w = qw[i];
 #pragma unroll
             for (int hi = 0; hi < 2; hi++) {  // low nibbles: elements 4i .. 4i+3; high nibbles: 16 + 4i ..
-                const uint32_t v = hi ? w >> 4 : w;
-                const int mag = (int)__builtin_amdgcn_perm(0x0C080604u, 0x03020100u, v & 0x07070707u);
-                const int neg = mag & (int)(((v >> 3) & 0x01010101u) * 0xFFu);
-                pl = __builtin_amdgcn_sdot4(mag, (int)xl[4 * hi + i], pl, false);
-                ph = __builtin_amdgcn_sdot4(mag, (int)xh[4 * hi + i], ph, false);
-                nl = __builtin_amdgcn_sdot4(neg, (int)xl[4 * hi + i], nl, false);
-                nh = __builtin_amdgcn_sdot4(neg, (int)xh[4 * hi + i], nh, false);
+                const uint32_t v = hi ? qw[i] >> 4 : qw[i];
+                const uint32_t sel = v & 0x07070707u;
+                const uint32_t pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
+                const uint32_t neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
+                const uint32_t mask = ((v >> 3) & 0x01010101u) * 0xFFu;
+                const int w = (int)((pos & ~mask) | (neg & mask));
+                pl = __builtin_amdgcn_sdot4(w, (int)xl[4 * hi + i], pl, false);
+                ph = __builtin_amdgcn_sdot4(w, (int)xh[4 * hi + i], ph, false);
             }
         }
-        const int s2 = ((ph - 2 * nh) << 8) + (pl - 2 * nl);  // twice the sum: the table holds doubled values
+        const int s2 = (ph << 8) + pl;  // twice the sum: the table holds doubled values
         return sx[0] * d * (0.5f * (float)s2);
     }
     // The block as eight words of signed int8, twice the E2M1 values (elements 4i .. 4i+3 in word i, the low
