@@ -1547,18 +1547,19 @@ int dispatch_moe_q4k_quads(const uint8_t *const *Wa, const uint8_t *const *Wb, s
 template <class Q, bool DUAL>
 int launch_moe_dot8(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align, const float *X,
                     size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets, const int *xsel, const int *yrow,
-                    float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
+                    float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{},
+                    bool planes_ready = false) {
     const int units = (k / Q::BLOCK_ELEMS) * Q::UNITS;
     const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
     const int G = (row_bytes % 16 == 0 && base_align >= 16) ? 16 : (row_bytes % 4 == 0 && base_align >= 4) ? 4 : 0;
     // every workgroup of a group redoing the row's quantisation is cheaper than a launch up to about
-    // half a million elements a group
+    // half a million elements a group (moe_dot8_takes_planes says the same)
     const size_t wgs = (n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R);
     const bool own = wgs * (size_t)k <= 512 * 1024 || !xq.xl;
     const size_t one = ((size_t)R * row_bytes + 15) / 16 * 16, wave_lds = one * (DUAL ? 2 : 1);
     const size_t lds = wave_lds * jq::ROWS_PER_WG + jq::table_bytes<Q>() + (own ? (size_t)k * 2 + (size_t)k / 4 : 0);
     if (G == 0 || lds > 64 * 1024) return -1;
-    if (!own) {
+    if (!own && !planes_ready) {
         const size_t words = x_rows * (size_t)(k / 4);
         hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
     }
@@ -1641,16 +1642,27 @@ int dispatch_moe_expert_dot8(uint32_t type, const uint8_t *const *Wa, const uint
     }
 }
 
+// Whether launch_moe_dot8 reads the activation planes acts_i8_prep makes (long rows) instead of quantising the row
+// in every workgroup.
+bool moe_dot8_takes_planes(uint32_t type, int k, int n, const jq::ActsI8 &xq) {
+    if (!moe_has_dot8(type) || k % 32 != 0 || !xq.xl) return false;
+    const int units = type == JQ_TYPE_Q4_K ? k / 64 : k / 32;
+    const int L = units >= 48 ? 64 : units >= 24 ? 32 : 16, R = 64 / L;
+    const size_t wgs = (n + jq::ROWS_PER_WG * R - 1) / (jq::ROWS_PER_WG * R);
+    return wgs * (size_t)k > 512 * 1024;
+}
+
 template <bool DUAL>
 int dispatch_moe_dot8(uint32_t type, const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align,
                       const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets,
-                      const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s, const jq::MoeClamp &cl = jq::MoeClamp{}) {
+                      const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s,
+                      const jq::MoeClamp &cl = jq::MoeClamp{}, bool planes_ready = false) {
     if (!moe_has_dot8(type) || k % 32 != 0 || ((uintptr_t)X & 15) != 0) return -1;
     switch (type) {
 #define JQ_DOT8_CASE(ID, Q)                                                                                         \
     case ID:                                                                                                        \
         return launch_moe_dot8<jq::Q, DUAL>(Wa, Wb, row_bytes, base_align, X, x_rows, xq, gexp, offsets, xsel, yrow, Y, k, n, \
-                                            groups, s, cl);
+                                            groups, s, cl, planes_ready);
         JQ_DOT8_CASE(JQ_TYPE_MXFP4, MXFP4)
         JQ_DOT8_CASE(JQ_TYPE_IQ2_XXS, IQ2_XXS)
         JQ_DOT8_CASE(JQ_TYPE_Q4_K, Q4_K)
@@ -1815,7 +1827,10 @@ int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, s
     }
 }
 
-int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg) {
+// `planes`: also leave x as fixed-point planes there (the one-expert-a-workgroup router kernel does; *planes_made
+// says whether it ran)
+int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg,
+                  jq::ActsI8 planes = jq::ActsI8{nullptr, nullptr, nullptr, nullptr}, bool *planes_made = nullptr) {
     const jq_moe_config &c = m->cfg;
     const unsigned token_runs = (unsigned)((T + jq::ROUTER_TOKENS_PER_WG - 1) / jq::ROUTER_TOKENS_PER_WG);
     static const char *no_tile = getenv("JQ_MOE_NO_ROUTER_TILE");
@@ -1826,7 +1841,8 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
                            m->router_w, x, m->logits, (int)T, (int)c.hidden, (int)c.n_expert);
     else
         hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert, token_runs), dim3(256), 0, s, m->router_w, x, m->logits,
-                           (int)T, (int)c.hidden, (int)c.n_expert);
+                           (int)T, (int)c.hidden, (int)c.n_expert, planes);
+    if (planes_made) *planes_made = planes.xl && !(T >= tile_from && !no_tile);
     jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
                          (int)c.n_group, (int)c.topk_group};
     size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);
@@ -1893,8 +1909,16 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         decode_sized = by_pairs <= std::min(by_gemm, by_expert) && P <= 16384;
         if (!expert_env) expert_dot8 = by_expert < by_gemm;
     }
+    bool planes_ready = false;
     if (decode_sized) {  // one group per pair, written by the gating kernel itself
-        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra})) return 1;
+        // long rows: the gate and up kernel reads x as fixed-point planes, which the router kernel can leave behind
+        jq::ActsI8 planes{nullptr, nullptr, nullptr, nullptr};
+        static const char *no_router_planes = getenv("JQ_MOE_NO_ROUTER_PLANES");
+        if (!no_router_planes && m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes &&
+            ((uintptr_t)x & 15) == 0 && moe_dot8_takes_planes(m->gate->type, (int)c.hidden, (int)c.inter, m->qi8))
+            planes = m->qi8;
+        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra}, planes, &planes_ready))
+            return 1;
         groups = P + extra * (int)T;
         max_group = 1;
     } else {
@@ -1983,7 +2007,8 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     if (rc > 0) return 1;
     if (rc < 0 && same_gu && max_group <= 1)
         rc = dispatch_moe_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
-                                     m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
+                                     m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp,
+                                     planes_ready);
     if (rc > 0) return 1;
     if (rc < 0 && same_gu)
         rc = dispatch_moe_staged<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, m->gexp, m->offsets,

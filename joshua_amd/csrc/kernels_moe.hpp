@@ -8,18 +8,59 @@
 
 namespace jq {
 
+// Activations as 15-bit fixed point per 32-element block, two int8 planes (X = 256 hi + lo) and the
+// block's scale: what the formats with an integer dot product (Q::dot8) multiply against.
+struct ActsI8 {
+    uint32_t *xl, *xh;  // [rows][k / 4]: four elements a word
+    float *sx, *sxs;    // [rows][k / 32]: the block's scale, and scale * sum of its fixed-point values
+};
+
+// Elements 4 i .. 4 i + 3 of X: eight consecutive lanes (i a multiple of 8 in the first) make one block of 32.
+__device__ __forceinline__ void acts_i8_quantize(const float *__restrict__ X, size_t i, const ActsI8 &out) {
+    const float4 v = *(const float4 *)(X + 4 * i);
+    float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
+    amax = max_row8(amax);
+    const bool live = amax > 0.0f && amax < INFINITY;
+    const float inv = live ? 32639.0f / amax : 0.0f;
+    const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
+                       __float2int_rn(v.w * inv)};
+    uint32_t wl = 0, wh = 0;
+    int sum = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int lo = ((Xq[e] + 128) & 255) - 128, hi = (Xq[e] - lo) >> 8;
+        wl |= (uint32_t)(lo & 255) << (8 * e);
+        wh |= (uint32_t)(hi & 255) << (8 * e);
+        sum += Xq[e];
+    }
+    out.xl[i] = wl;
+    out.xh[i] = wh;
+    sum = isum_row8(sum);
+    if ((i & 7) == 0) {
+        const float s = fixed_scale(amax, 32639.0f);
+        out.sx[i >> 3] = s;
+        out.sxs[i >> 3] = s * (float)sum;
+    }
+}
+
 // logits[t, e] = x[t, :] . router[e, :]   (reference: src/quantized_qwen3_moe.rs:425,
 // src/quantized_deepseek2.rs:528; an f32 matmul there too)
 constexpr int ROUTER_TOKENS_PER_WG = 8;
 
 __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict__ Wr, const float *__restrict__ X,
-                                                          float *__restrict__ logits, int T, int h, int E) {
+                                                          float *__restrict__ logits, int T, int h, int E, ActsI8 planes) {
     // one workgroup per (expert row of the router, run of 8 tokens): every load of the row in
     // flight at once; a logit's arithmetic does not depend on how the tokens are split
     __shared__ float red[4][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, e = blockIdx.x;
     const float *wr = Wr + (size_t)e * h;
     const int t_begin = blockIdx.y * ROUTER_TOKENS_PER_WG, t_end = min(T, t_begin + ROUTER_TOKENS_PER_WG);
+    // With `planes` (h a multiple of 32): the tokens' activations as fixed-point planes for the expert kernels
+    // that follow, one launch less.  Workgroup e makes blocks e, e + E, .. of its tokens: eight lanes a block.
+    if (planes.xl && (int)threadIdx.x < 8 * (t_end - t_begin)) {
+        const size_t t = (size_t)t_begin + (threadIdx.x >> 3);
+        for (int b = e; b < h / 32; b += E) acts_i8_quantize(X, t * (size_t)(h / 4) + 8 * b + (threadIdx.x & 7), planes);
+    }
     for (int t0 = t_begin; t0 < t_end; t0 += 4) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
         for (int c = threadIdx.x * 4; c < h; c += 1024) {
@@ -635,40 +676,10 @@ __global__ __launch_bounds__(64 * ROWS_PER_WG) void moe_rows_staged(const uint8_
     }
 }
 
-// Activations as 15-bit fixed point per 32-element block, two int8 planes (X = 256 hi + lo) and the
-// block's scale: what the formats with an integer dot product (Q::dot8) multiply against.
-struct ActsI8 {
-    uint32_t *xl, *xh;  // [rows][k / 4]: four elements a word
-    float *sx, *sxs;    // [rows][k / 32]: the block's scale, and scale * sum of its fixed-point values
-};
-
 __global__ __launch_bounds__(256) void acts_i8_prep(const float *__restrict__ X, size_t rows, int k, ActsI8 out) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // four elements a thread, eight threads a block
     if (i >= rows * (size_t)(k / 4)) return;  // whole groups of 8 lanes leave together (k % 32 == 0)
-    const float4 v = *(const float4 *)(X + 4 * i);
-    float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
-    amax = max_row8(amax);
-    const bool live = amax > 0.0f && amax < INFINITY;
-    const float inv = live ? 32639.0f / amax : 0.0f;
-    const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
-                       __float2int_rn(v.w * inv)};
-    uint32_t wl = 0, wh = 0;
-    int sum = 0;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        const int lo = ((Xq[e] + 128) & 255) - 128, hi = (Xq[e] - lo) >> 8;
-        wl |= (uint32_t)(lo & 255) << (8 * e);
-        wh |= (uint32_t)(hi & 255) << (8 * e);
-        sum += Xq[e];
-    }
-    out.xl[i] = wl;
-    out.xh[i] = wh;
-    sum = isum_row8(sum);
-    if ((i & 7) == 0) {
-        const float s = fixed_scale(amax, 32639.0f);
-        out.sx[i >> 3] = s;
-        out.sxs[i >> 3] = s * (float)sum;
-    }
+    acts_i8_quantize(X, i, out);
 }
 
 // The decode-shaped grouped expert matmul (one activation row a group) on integer dot products: rows
