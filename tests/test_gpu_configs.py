@@ -69,13 +69,13 @@ def test_deepseek_v3_shaped_expert_layer(qtype):
 
 @pytest.mark.parametrize("qtype,tokens,expert_dot8,kernel", [
     (capi.IQ2_XXS, 150, True, "moe_expert_dot8"), (capi.MXFP4, 90, True, "moe_expert_dot8"),
-    (capi.IQ2_XXS, 20, True, "moe_expert_dot8"), (capi.IQ2_XXS, 5, True, "moe_down_combine_dot8"),
+    (capi.IQ2_XXS, 30, True, "moe_expert_dot8"), (capi.IQ2_XXS, 5, True, "moe_down_combine_dot8"),
     (capi.IQ2_XXS, 150, False, "moe_gemm_i8_few"), (capi.MXFP4, 90, False, "moe_gemm_i8_few"),
     (capi.IQ2_XXS, 48, False, "moe_down_combine_dot8")])
 def test_deepseek_v3_shaped_expert_layer_over_a_prompt(monkeypatch, qtype, tokens, expert_dot8, kernel):
     """The same layer over a prompt, at the layer's own row lengths: gate and up of 7168 columns (28 super-blocks,
     224 units of 32: seven a lane), down of 2048.  150 tokens of IQ2_XXS (1200 routed pairs over 256 experts and the
-    shared expert's 150), 90 of MXFP4 and 20 of IQ2_XXS (160 pairs, fewer than experts): bucketed by expert, an
+    shared expert's 150), 90 of MXFP4 and 30 of IQ2_XXS (240 pairs, fewer than experts): bucketed by expert, an
     expert's rows decoded once into registers and its pairs streamed past them.  5 tokens: one group a pair.
     With that kernel switched off: the grouped int8 GEMM, and at 48 tokens still one group a pair (a pair's rows cost
     less to read again than an expert's to unpack for a tile of 32 rows)."""
