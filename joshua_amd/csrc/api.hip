@@ -330,9 +330,9 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
         const size_t tiles = (n + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
         const jq::QvColsWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G), (int)nb};
         note_kernel("q4k_gemv_mfma_cols");
-        if (nb <= 32) hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ4K, 2>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
-        else if (nb <= 48) hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ4K, 3>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
-        else hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ4KCompact, 4>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
+        if (nb <= 32) hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ4K, 2>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra, wk.nb);
+        else if (nb <= 48) hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ4K, 3>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra, wk.nb);
+        else hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ4KCompact, 4>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra, wk.nb);
         HIP_TRY(hipGetLastError());
         return 0;
     }
@@ -349,7 +349,7 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
             const size_t rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
             const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
             note_kernel("q4k_gemv_mfma_lds");
-            hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ4K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
+            hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ4K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra);
             HIP_TRY(hipGetLastError());
             return 0;
         }
@@ -390,7 +390,7 @@ int dispatch_q2k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
     const size_t tiles = (n + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
     const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
     note_kernel("q2k_gemv_mfma_lds");
-    hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ2K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk);
+    hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ2K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra);
     HIP_TRY(hipGetLastError());
     return 0;
 }

@@ -41,66 +41,93 @@ struct QvActs {
     float s_e, s_o16, xs_e, xs_o;
 };
 
+// A lane's four activations (elements 4i .. 4i+3 of a 32-element sub-block held by 8 lanes) as 16-bit fixed
+// point against the sub-block's maximum, in as few vector instructions as the arithmetic allows: every
+// workgroup repeats this for the whole activation row in front of its first product, four waves a SIMD, so
+// an instruction here costs sixteen cycles of the launch's start.
+//   * the maximum is taken over the magnitudes' bit patterns as unsigned integers: NaN > inf > finite, so a
+//     non-finite element needs no test of its own;
+//   * the scale amax / 32639 by a multiplication with one correction step, which is exact whenever the
+//     quotient is a float; its inverse by the hardware reciprocal (a relative error of 2^-22 moves X by less
+//     than 0.02, so an activation that is an integer multiple of the scale still quantises to that integer);
+//   * X = round(x inv) as the mantissa of fma(x, inv, 1.5 * 2^23 + 128): bits 0..15 of the result are X + 128,
+//     byte 1 the high plane, byte 0 the low plane with its top bit flipped; four v_perm_b32 gather the planes.
+// Returns the plane words of X (wl, wh) and of -X (nl, nh), the scale (NaN for a sub-block with a non-finite
+// element, 0 for one of zeros) and the sum of the sub-block's X in every lane of the sub-block.
+struct QvQuant {
+    uint32_t wl, wh, nl, nh;
+    float s;
+    int sum;
+};
+__device__ __forceinline__ QvQuant qv_quantise4(const float4 v) {
+    const uint32_t b0 = __builtin_bit_cast(uint32_t, v.x) & 0x7FFFFFFFu, b1 = __builtin_bit_cast(uint32_t, v.y) & 0x7FFFFFFFu;
+    const uint32_t b2 = __builtin_bit_cast(uint32_t, v.z) & 0x7FFFFFFFu, b3 = __builtin_bit_cast(uint32_t, v.w) & 0x7FFFFFFFu;
+    uint32_t m = max(max(b0, b1), max(b2, b3));
+    m = max(m, (uint32_t)dpp_i<0x141>((int)m));
+    m = max(m, (uint32_t)dpp_i<0xB1>((int)m));
+    m = max(m, (uint32_t)dpp_i<0x4E>((int)m));
+    const float amax = __builtin_bit_cast(float, m);
+    constexpr float RC = 1.0f / QD_RANGE;
+    float s = amax * RC;
+    s = fmaf(fmaf(-s, QD_RANGE, amax), RC, s);
+    const float inv = __builtin_amdgcn_rcpf(fmaxf(s, 1e-35f));  // of the scale: a normal number for every finite amax
+    s = m >= 0x7F800000u ? NAN : s;
+    constexpr float MAGIC = 12582912.0f + 128.0f;
+    const float ninv = -inv;
+    const uint32_t t0 = __builtin_bit_cast(uint32_t, fmaf(v.x, inv, MAGIC)), t1 = __builtin_bit_cast(uint32_t, fmaf(v.y, inv, MAGIC));
+    const uint32_t t2 = __builtin_bit_cast(uint32_t, fmaf(v.z, inv, MAGIC)), t3 = __builtin_bit_cast(uint32_t, fmaf(v.w, inv, MAGIC));
+    const uint32_t u0 = __builtin_bit_cast(uint32_t, fmaf(v.x, ninv, MAGIC)), u1 = __builtin_bit_cast(uint32_t, fmaf(v.y, ninv, MAGIC));
+    const uint32_t u2 = __builtin_bit_cast(uint32_t, fmaf(v.z, ninv, MAGIC)), u3 = __builtin_bit_cast(uint32_t, fmaf(v.w, ninv, MAGIC));
+    // v_perm_b32(a, b, sel): selector 0..3 takes byte 0..3 of b, 4..7 of a
+    const uint32_t p01 = __builtin_amdgcn_perm(t1, t0, 0x05010400u), p23 = __builtin_amdgcn_perm(t3, t2, 0x05010400u);
+    const uint32_t n01 = __builtin_amdgcn_perm(u1, u0, 0x05010400u), n23 = __builtin_amdgcn_perm(u3, u2, 0x05010400u);
+    QvQuant q;
+    q.wl = __builtin_amdgcn_perm(p23, p01, 0x05040100u) ^ 0x80808080u, q.wh = __builtin_amdgcn_perm(p23, p01, 0x07060302u);
+    q.nl = __builtin_amdgcn_perm(n23, n01, 0x05040100u) ^ 0x80808080u, q.nh = __builtin_amdgcn_perm(n23, n01, 0x07060302u);
+    q.s = s;
+    constexpr uint32_t BASE4 = 4u * 0x4B400080u;  // four times the bit pattern of MAGIC, modulo 2^32
+    q.sum = isum_row8((int)(t0 + t1 + t2 + t3 - BASE4));
+    return q;
+}
+
 // Quantises the wave's activation column (lane i holds elements 4i .. 4i+3, sub-block i / 8) and builds
-// the lane's operands through `stage`, 1152 bytes of LDS that only this wave touches:
-// words [0,64) Xl, [64,128) Xh, [128,192) and [192,256) the planes of -X, then 8 scales, 8 scaled sums, 8
-// integer sums.
+// the lane's operands through `stage`, 1184 bytes of LDS that only this wave touches:
+// words [0,64) Xl, [64,128) Xh, [128,192) and [192,256) the planes of -X, 8 words of zeros, then per
+// sub-block {scale, scale x sum, 128 x sum (integer), scale / 16}.
 __device__ __forceinline__ QvActs qv_prepare(const float4 v, uint32_t *stage, int lane) {
     const int r = lane & 15, c = lane >> 4;
-    float *stage_f = (float *)(stage + 256);
+    float4 *side = (float4 *)(stage + 264);
     {
-        float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
-        amax = max_row8(amax);
-        const bool live = amax > 0.0f && amax < INFINITY;
-        const float inv = live ? QD_RANGE / amax : 0.0f, s = fixed_scale(amax, QD_RANGE);
-        const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
-                           __float2int_rn(v.w * inv)};
-        uint32_t wl = 0, wh = 0, nl = 0, nh = 0;
-        int sum = 0;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            // balanced planes: the low byte read as signed, the rest above it
-            wl |= (uint32_t)(Xq[i] & 255) << (8 * i);
-            wh |= (uint32_t)(((Xq[i] + 128) >> 8) & 255) << (8 * i);
-            nl |= (uint32_t)(-Xq[i] & 255) << (8 * i);
-            nh |= (uint32_t)(((-Xq[i] + 128) >> 8) & 255) << (8 * i);
-            sum += Xq[i];
-        }
-        stage[lane] = wl, stage[64 + lane] = wh, stage[128 + lane] = nl, stage[192 + lane] = nh;
-        sum = isum_row8(sum);
-        if ((lane & 7) == 0) {
-            stage_f[lane >> 3] = s;
-            stage_f[8 + (lane >> 3)] = s * (float)sum;
-            ((int *)stage_f)[16 + (lane >> 3)] = sum;
-        }
+        const QvQuant q = qv_quantise4(v);
+        stage[lane] = q.wl, stage[64 + lane] = q.wh, stage[128 + lane] = q.nl, stage[192 + lane] = q.nh;
+        if (lane < 8) stage[256 + lane] = 0;
+        if ((lane & 7) == 0) side[lane >> 3] = float4{q.s, q.s * (float)q.sum, __builtin_bit_cast(float, 128 * q.sum), q.s * 0.0625f};
     }
     QvActs a;
     {
-        // A operands of lane (m = r, g = c): sub-block jm = m / 2, plane m % 2; non-zero when jm is 2g or 2g + 1
-        const int jm = r >> 1, pl = r & 1, p = jm - 2 * c;  // p: 0 low-nibble sub-block, 1 high-nibble sub-block
-        const bool mine = p == 0 || p == 1;
-        const uint32_t *pos = stage + 64 * pl + 16 * c + 8 * (p & 1);  // plane words of the sub-block's 32 elements
-        const uint32_t *neg = pos + 128;
-        const uint4 z = uint4{0, 0, 0, 0};
-        const uint4 p0 = mine ? *(const uint4 *)pos : z, p1 = mine ? *(const uint4 *)(pos + 4) : z;
-        const uint4 n0 = mine ? *(const uint4 *)neg : z, n1 = mine ? *(const uint4 *)(neg + 4) : z;
-        const bool odd = p == 1;
-        const uint4 e0 = odd ? n0 : p0, e1 = odd ? n1 : p1, o0 = odd ? p0 : z, o1 = odd ? p1 : z;
+        // A operands of lane (m = r, g = c): row m is sub-block m / 2, plane m % 2, and non-zero in lane group
+        // (m / 2) / 2 only; p = 0: the low-nibble sub-block 2g, 1: the high-nibble sub-block 2g + 1.  The lanes
+        // that hold zeros read them from the staging area's zero words, so no register is selected afterwards.
+        const bool mine = (r >> 2) == c, odd = (r & 2) != 0;
+        const uint32_t *pos = stage + 64 * (r & 1) + 16 * c + (odd ? 8 : 0);  // plane words of the sub-block's 32 elements
+        const uint32_t *zero = stage + 256;
+        const uint32_t *ev = mine ? (odd ? pos + 128 : pos) : zero, *od = mine && odd ? pos : zero;
+        const uint4 e0 = *(const uint4 *)ev, e1 = *(const uint4 *)(ev + 4), o0 = *(const uint4 *)od, o1 = *(const uint4 *)(od + 4);
         a.a_even[0] = qv_i4{(int)e0.x, (int)e0.y, (int)e0.z, (int)e0.w};
         a.a_even[1] = qv_i4{(int)e1.x, (int)e1.y, (int)e1.z, (int)e1.w};
         a.a_odd[0] = qv_i4{(int)o0.x, (int)o0.y, (int)o0.z, (int)o0.w};
         a.a_odd[1] = qv_i4{(int)o1.x, (int)o1.y, (int)o1.z, (int)o1.w};
     }
     // what lane (r, c) needs of sub-blocks 2c and 2c + 1 after the MFMAs
-    a.s_e = stage_f[2 * c], a.s_o16 = stage_f[2 * c + 1] * 0.0625f;
-    a.xs_e = stage_f[8 + 2 * c], a.xs_o = stage_f[8 + 2 * c + 1];
-    a.c_init = qv_i4{0, 0, 128 * ((const int *)stage_f)[16 + 2 * c + 1], 0};
+    const float4 fe = side[2 * c], fo = side[2 * c + 1];
+    a.s_e = fe.x, a.xs_e = fe.y, a.s_o16 = fo.w, a.xs_o = fo.y;
+    a.c_init = qv_i4{0, 0, __builtin_bit_cast(int, fo.z), 0};
     return a;
 }
 
-// The sum of a super-block of weight row r against the wave's column, over chunk c, reduced over the four
-// chunks: every lane of a row ends up with the block's sum.  blk: the row's 144-byte block in LDS.
-__device__ __forceinline__ float qv_block_dot(const uint8_t *blk, const QvActs &a, int c) {
+// The sum of chunk c of a super-block of weight row r against the wave's column.  blk: the row's 144-byte
+// block in LDS.
+__device__ __forceinline__ float qv_block_dot_lane(const uint8_t *blk, const QvActs &a, int c) {
     const uint4 hdr = *(const uint4 *)blk;
     const uint4 qa = *(const uint4 *)(blk + 16 + 32 * c), qb = *(const uint4 *)(blk + 32 + 32 * c);
     const qv_i4 la = qv_i4{(int)(qa.x & 0x0F0F0F0Fu), (int)(qa.y & 0x0F0F0F0Fu), (int)(qa.z & 0x0F0F0F0Fu), (int)(qa.w & 0x0F0F0F0Fu)};
@@ -117,19 +144,22 @@ __device__ __forceinline__ float qv_block_dot(const uint8_t *blk, const QvActs &
     const float d = f16_bits(hdr.x), dmin = f16_bits(hdr.x >> 16);
     const float f_e = (float)((C[1] << 8) + C[0]) * a.s_e, f_o = (float)((C[3] << 8) + C[2]) * a.s_o16;
     float acc = d * fmaf((float)sc_lo, f_e, (float)sc_hi * f_o);
-    acc = fmaf(-dmin, fmaf((float)mn_lo, a.xs_e, (float)mn_hi * a.xs_o), acc);
-    acc = sum_xor16(acc);
-    return sum_xor32(acc);
+    return fmaf(-dmin, fmaf((float)mn_lo, a.xs_e, (float)mn_hi * a.xs_o), acc);
+}
+// The same reduced over the four chunks: every lane of a row ends up with the block's sum.
+__device__ __forceinline__ float qv_block_dot(const uint8_t *blk, const QvActs &a, int c) {
+    return sum_xor32(sum_xor16(qv_block_dot_lane(blk, a, c)));
 }
 
 // The Q4_K policy.
 struct QvQ4K {
     static constexpr int BLOCK = 144, ROW = 16 * BLOCK, ROW_LDS = QD_ROW_LDS;  // rows 16 bytes apart in banks
-    static constexpr int STAGE_BYTES = 1152;  // what prepare() uses of `stage`
+    static constexpr int STAGE_BYTES = 1184;  // what prepare() uses of `stage`
     static constexpr bool SIDE_LDS = false;
     typedef QvActs Acts;
     __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) { return qv_prepare(v, stage, lane); }
     __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) { return qv_block_dot(blk, a, c); }
+    __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) { return qv_block_dot_lane(blk, a, c); }
 };
 
 // The same for the kernel that keeps the operands of four columns: the accumulator start as the one word
@@ -215,6 +245,9 @@ struct QvQ2K {
         return a;
     }
     __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) {
+        return sum_xor32(sum_xor16(block_dot_lane(blk, a, c)));
+    }
+    __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) {
         // blocks sit at multiples of 84 bytes: everything is read as aligned 32-bit words
         const uint32_t *w32 = (const uint32_t *)blk;
         const uint32_t sc0 = w32[2 * (c >> 1)] >> (8 * (c & 1)), sc1 = w32[2 * (c >> 1) + 1] >> (8 * (c & 1));
@@ -241,111 +274,107 @@ struct QvQ2K {
         sm = fmaf((float)((sc0 >> 20) & 0xFu), a.xs[1], sm);
         sm = fmaf((float)((sc1 >> 4) & 0xFu), a.xs[2], sm);
         sm = fmaf((float)((sc1 >> 20) & 0xFu), a.xs[3], sm);
-        float acc = fmaf(-f16_bits(dd >> 16), sm, f16_bits(dd) * sd);
-        acc = sum_xor16(acc);
-        return sum_xor32(acc);
+        return fmaf(-f16_bits(dd >> 16), sm, f16_bits(dd) * sd);
     }
 };
 
 // Work of workgroup b (of G): tiles b, b + G, b + 2 G, ... of 16 rows each; there are rounds G + extra tiles,
-// so the first `extra` workgroups take one more than the others.  (Tiles of 14 rows, which give each of 256
+// so the first `extra` workgroups take one more than the others.  The kernels take the four numbers as
+// arguments of their own: scalars among the leading arguments arrive preloaded in registers, a struct is
+// fetched by a scalar load in front of the first global load.  (Tiles of 14 rows, which give each of 256
 // workgroups four tiles of a 14336-row matrix where tiles of 16 rows leave 32 compute units idle, measured
 // 1.5 % slower for Q4_K: 7.49 against 7.39 us.)
 struct QvWork {
     int n, G, rounds, extra;
 };
 
-// Wave w copies row w of a tile into a ring of four tiles in LDS (contiguous asynchronous loads, two tiles
+// An asynchronous 16-byte load a lane whose global address is a scalar base (the wave's row) plus the lane's own
+// byte offset: no vector instruction goes into the address.
+__device__ __forceinline__ void async_load16_s(const uint8_t *sbase, uint32_t voff, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory");
+}
+
+// Wave w copies row w of a tile into a ring of three tiles in LDS (contiguous asynchronous loads, two tiles
 // ahead of the arithmetic) and multiplies column w of all 16 rows, so a tile is published by a barrier.
-// The waves' partial sums of up to four tiles wait in LDS and are added, stored and forgotten behind one
-// more barrier.
+//   * A tile's arithmetic comes first, the request for the tile after next behind it: a load instruction holds its
+//     wave until the compute unit's memory pipeline accepts it, which with a tile in flight takes until most of
+//     that tile has landed, and a wave that waits there multiplies late.
+//   * A lane keeps its chunk's sum; the four chunk sums of a (row, wave) pair and the 16 waves' sums of a row are
+//     added when the rows are stored, once per four tiles and behind one more barrier.  The partial sums sit in
+//     LDS as [tile][row][4 wave + chunk] with rows 16 bytes longer than their 64 words: the writes of a wave
+//     (lane (r, c) -> row r) and the 16-byte reads of the flush (lane (tile, wave) of row w) both touch every
+//     bank once.  (As [tile][wave][row] the flush's reads fell on two banks: 0.5 us of the launch's end.)
+//   * Stores go out only behind the last tile of four: a store between the tiles' loads costs 0.15 us each.
 template <class F>
 __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                      float *__restrict__ Y, QvWork wk) {
-    constexpr int D = 2;  // tiles asked for ahead of the one being multiplied (3 measured slower)
-    constexpr int LOADS = (F::ROW + 1023) / 1024;  // asynchronous loads a wave and tile
-    __shared__ __attribute__((aligned(16))) uint8_t ring[QV_SLOTS][16 * F::ROW_LDS];
-    __shared__ float part[QV_SLOTS][16][16];  // [tile % 4][wave][row]
-    // a wave's staging area (what prepare() needs, then its 256 raw activations): its own row of ring slot 3
-    // when that is long enough, which no load targets before tile 3 is asked for in the main loop; else
+                                                      float *__restrict__ Y, int n, int G, int rounds, int extra) {
+    constexpr int SLOTS = 3, FL = 4;                 // ring slots (two tiles in flight); tiles a flush
+    constexpr int FULL = F::ROW / 1024, REST = (F::ROW - 1024 * FULL) / 16, LOADS = FULL + (REST ? 1 : 0);
+    __shared__ __attribute__((aligned(16))) uint8_t ring[SLOTS][16 * F::ROW_LDS];
+    __shared__ __attribute__((aligned(16))) float part[FL][16][68];
+    // a wave's staging area (what prepare() needs, then its 256 raw activations): its own row of the last ring
+    // slot when that is long enough, which no load targets before tile 2 is asked for in the main loop; else
     // memory of its own
     constexpr int STAGE = F::STAGE_BYTES + 1024;
     constexpr bool STAGE_IN_RING = STAGE <= F::ROW_LDS;
     __shared__ __attribute__((aligned(16))) uint8_t stage_mem[STAGE_IN_RING ? 16 : 16 * STAGE];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, c = lane >> 4, b = (int)blockIdx.x;
-    const int n = wk.n, G = wk.G;
-    const int nt = wk.rounds + (b < wk.extra ? 1 : 0);  // tiles of this workgroup (no division in front of the first loads)
+    const int nt = rounds + (b < extra ? 1 : 0);  // tiles of this workgroup (no division in front of the first loads)
     if (nt <= 0) return;
     auto tile_row0 = [&](int i) __attribute__((always_inline)) { return 16 * (b + i * G); };
-    // fetch(i) asks for tile min(i, nt - 1) into slot i % 4 (the fetches in front of the main loop are
-    // unconditional, so that every wave counts the same loads)
+    const uint32_t voff = 16 * lane, ring0 = lds_offset_of(&ring[0][0]);
+    // fetch(i) asks for tile min(i, nt - 1) into slot i % 3 (the fetches in front of the main loop are
+    // unconditional, so that every wave counts the same loads); the row's address is scalar arithmetic
     auto fetch = [&](int slot_i) __attribute__((always_inline)) {
         const int i = min(slot_i, nt - 1);
         const int row = min(tile_row0(i) + wave, n - 1);
-        const uint8_t *src = W + (size_t)row * F::ROW + 16 * lane;
-        const uint32_t dst = lds_offset_of(&ring[slot_i & (QV_SLOTS - 1)][wave * F::ROW_LDS]);
+        const uint8_t *src = W + (size_t)row * F::ROW;
+        const uint32_t dst = ring0 + (uint32_t)(slot_i % SLOTS) * (16 * F::ROW_LDS) + (uint32_t)wave * F::ROW_LDS;
 #pragma unroll
-        for (int j = 0; j < LOADS; j++) {
-            constexpr int full = F::ROW / 1024;
-            if (j < full) async_load16(src + 1024 * j, dst + 1024 * j);
-            else if (lane < (F::ROW - 1024 * full) / 16) async_load16(src + 1024 * j, dst + 1024 * j);
-        }
+        for (int j = 0; j < FULL; j++) async_load16_s(src + 1024 * j, voff, dst + 1024 * j);
+        if (REST && lane < REST) async_load16_s(src + 1024 * FULL, voff, dst + 1024 * FULL);
     };
     // the raw activations travel like the tiles (every global read of this kernel is an asynchronous load
     // counted by hand)
-    uint32_t *stage = (uint32_t *)(STAGE_IN_RING ? &ring[QV_SLOTS - 1][wave * F::ROW_LDS] : &stage_mem[wave * STAGE]);
+    uint32_t *stage = (uint32_t *)(STAGE_IN_RING ? &ring[SLOTS - 1][wave * F::ROW_LDS] : &stage_mem[wave * STAGE]);
     float *x_raw = (float *)((uint8_t *)stage + F::STAGE_BYTES);
     async_load16(X + 256 * wave + 4 * lane, lds_offset_of(x_raw));
     // every wave's activations are asked for before anybody's tile: the memory pipeline takes a compute
     // unit's requests in the order they were issued, and a wave whose activations queue behind the other
-    // waves' tile loads starts its preparation a microsecond late
+    // waves' tile loads starts its preparation late
     __builtin_amdgcn_s_barrier();
-    // tile 0 is asked for alone: it has the memory system to itself and lands while the activations are
-    // prepared; the next D - 1 tiles follow the preparation
+    // tile 0 is asked for alone and lands while the activations are prepared; tile 1 follows the preparation
     fetch(0);
-    if (LOADS == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
     const float4 v = *(const float4 *)&x_raw[4 * lane];
     const typename F::Acts acts = F::prepare(v, stage, lane);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     fetch(1);
-    if (D == 3) fetch(2);
 
-    const int n_groups = (nt + QV_SLOTS - 1) / QV_SLOTS;
-    for (int grp = 0; grp < n_groups; grp++) {
-        const int t_end = min(nt, QV_SLOTS * (grp + 1));
-        for (int t = QV_SLOTS * grp; t < t_end; t++) {
-            // tile t has landed; tiles up to max(D - 1, min(nt - 1, t + D - 1)) have been asked for and may be
-            // in flight, nothing behind the last tile
-            const int ahead = t == nt - 1 ? 0 : max(D - 1, min(nt - 1, t + D - 1)) - t;
-            if (LOADS == 3) {
-                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            } else {
-                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            }
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            // every wave is done with tile t - 1, so the slot of tile t + D - 4 is free
-            if (t + D < nt) fetch(t + D);
-            const float acc = F::block_dot(&ring[t & (QV_SLOTS - 1)][r * F::ROW_LDS + wave * F::BLOCK], acts, c);
-            if (lane < 16) part[t & (QV_SLOTS - 1)][wave][lane] = acc;
-        }
-        // the waves' partial sums of this group's tiles are written: lane (tt = lane / 16, ww = lane % 16)
-        // takes wave ww's sum of row `wave` in tile tt of the group
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    for (int t = 0; t < nt; t++) {
+        // tile t has landed when only tile t + 1's loads are out (nothing behind the last tile)
+        if (t + 1 < nt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        const int t = QV_SLOTS * grp + c;
-        float sum = part[c][r][wave];
-        sum = sum_row16(sum);
-        if (r == 0 && t < t_end) {
-            const int row = tile_row0(t) + wave;
-            if (row < n) Y[row] = sum;
+        part[t & (FL - 1)][r][4 * wave + c] = F::block_dot_lane(&ring[t % SLOTS][r * F::ROW_LDS + wave * F::BLOCK], acts, c);
+        // every wave is done with tile t - 1, whose slot tile t + 2 takes
+        if (t + 2 < nt) fetch(t + 2);
+        if ((t & (FL - 1)) == FL - 1 || t == nt - 1) {
+            // the partial sums of this group's tiles are written: lane (tt = lane / 16, ww = lane % 16) takes wave
+            // ww's four chunk sums of row `wave` in tile tt of the group
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            const int tt = (t & ~(FL - 1)) + c;
+            const float4 p = *(const float4 *)&part[c][wave][4 * r];
+            float sum = (p.x + p.y) + (p.z + p.w);
+            sum = sum_row16(sum);
+            if (r == 0 && tt <= t) {
+                const int row = tile_row0(tt) + wave;
+                if (row < n) Y[row] = sum;
+            }
         }
     }
 }
@@ -360,7 +389,7 @@ struct QvColsWork {
 
 template <class F, int NG>
 __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                       float *__restrict__ Y, QvColsWork wk) {
+                                                       float *__restrict__ Y, int n, int G, int rounds, int extra, int nb) {
     static_assert(NG >= 2 && NG <= 4, "two to four passes a row");
     constexpr int D = 2, LOADS = (F::ROW + 1023) / 1024, TG = NG == 3 ? 3 : 4;  // tiles a flush: whole row tiles
     // the raw activations of the passes wait in the wave's own rows of ring slots 3 (behind what prepare()
@@ -371,9 +400,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict
     __shared__ float4 side[F::SIDE_LDS ? 16 * NG * 4 : 1];  // [wave][pass][lane group], for the policies that want it
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, c = lane >> 4, b = (int)blockIdx.x;
-    const int n = wk.n, G = wk.G, nb = wk.nb;
     const size_t row_bytes = (size_t)nb * F::BLOCK;
-    const int nt = NG * (wk.rounds + (b < wk.extra ? 1 : 0));
+    const int nt = NG * (rounds + (b < extra ? 1 : 0));
     if (nt <= 0) return;
     // every fetch is LOADS instructions with at least one lane at work, so that every wave counts the same
     // loads; a short last pass repeats its last 16 bytes into LDS bytes nobody reads
