@@ -341,15 +341,25 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     const size_t tiles = (n + 15) / 16;
     if (mode != "regs") {
         if (nb != 16 || row_bytes != jq::QD_ROW) return -1;
-        // from 8192 rows on, the plain product runs its dot products on the int8 matrix cores (14336 rows:
-        // 7.35 against 7.9 us; 12288: 6.95 against 7.2; 65536: 25.2 against 26.3; 4096: 4.5 against 4.3 us)
+        // from 2048 rows on, the product runs its dot products on the int8 matrix cores, with the norm and SwiGLU
+        // forms of the decoder's fused launches (14336 rows: 7.1 against 7.9 us; 24576 rows with norm and SwiGLU:
+        // 11.5 against 11.9; 4096: 3.8 against 4.3 us; a decoded token of the Qwen3-8B-shaped model 1.67 against
+        // 1.74 ms)
         static const char *mfma_env = getenv("JQ_Q4K_GEMV_MFMA");
-        static const size_t mfma_min_n = mfma_env ? (size_t)atoll(mfma_env) : 8192;
-        if (!norm && !swiglu && !genv && mfma_min_n > 0 && n >= mfma_min_n && n <= 0x7FFFFFF0ull) {
+        static const size_t mfma_min_n = mfma_env ? (size_t)atoll(mfma_env) : 2048;
+        if (!genv && mfma_min_n > 0 && n >= mfma_min_n && n <= 0x7FFFFFF0ull && (!swiglu || n % 2 == 0)) {
             const size_t rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
             const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
+            const jq::QdNorm nm = norm ? *norm : jq::QdNorm{};
             note_kernel("q4k_gemv_mfma_lds");
-            hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ4K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra);
+#define JQ_MFMA_LDS(NORM, SWIGLU) \
+    hipLaunchKernelGGL((jq::gemv_mfma_lds<jq::QvQ4K, NORM, SWIGLU>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, \
+                       wk.rounds, wk.extra, nm.res, nm.w, nm.eps, nm.x_out, nm.hn_out)
+            if (norm && swiglu) JQ_MFMA_LDS(true, true);
+            else if (norm) JQ_MFMA_LDS(true, false);
+            else if (swiglu) JQ_MFMA_LDS(false, true);
+            else JQ_MFMA_LDS(false, false);
+#undef JQ_MFMA_LDS
             HIP_TRY(hipGetLastError());
             return 0;
         }
@@ -390,7 +400,7 @@ int dispatch_q2k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
     const size_t tiles = (n + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
     const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
     note_kernel("q2k_gemv_mfma_lds");
-    hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ2K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra);
+    hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ2K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra, nullptr, nullptr, 0.0f, nullptr, nullptr);
     HIP_TRY(hipGetLastError());
     return 0;
 }

@@ -156,7 +156,10 @@ struct QvQ4K {
     static constexpr int BLOCK = 144, ROW = 16 * BLOCK, ROW_LDS = QD_ROW_LDS;  // rows 16 bytes apart in banks
     static constexpr int STAGE_BYTES = 1184;  // what prepare() uses of `stage`
     static constexpr bool SIDE_LDS = false;
+    static constexpr int COLS = 4096;
     typedef QvActs Acts;
+    // the activations times f: one factor onto everything that carries the activation scale
+    __device__ static __forceinline__ void scale(Acts &a, float f) { a.s_e *= f, a.s_o16 *= f, a.xs_e *= f, a.xs_o *= f; }
     __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) { return qv_prepare(v, stage, lane); }
     __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) { return qv_block_dot(blk, a, c); }
     __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) { return qv_block_dot_lane(blk, a, c); }
@@ -204,7 +207,12 @@ struct Q2Acts {
 struct QvQ2K {
     static constexpr int BLOCK = 84, ROW = 16 * BLOCK, ROW_LDS = ROW + 16;  // 340 words: 16 rows x 4 words fill the 64 banks
     static constexpr int STAGE_BYTES = 640;
+    static constexpr int COLS = 4096;
     typedef Q2Acts Acts;
+    __device__ static __forceinline__ void scale(Acts &a, float f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) a.s[i] *= f, a.xs[i] *= f;
+    }
     __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) {
         const int r = lane & 15, c = lane >> 4;
         float *stage_f = (float *)(stage + 128);  // [0,8) scales of the 32-element sub-blocks, [8,24) scale x sum per 16
@@ -305,10 +313,22 @@ __device__ __forceinline__ void async_load16_s(const uint8_t *sbase, uint32_t vo
 //     (lane (r, c) -> row r) and the 16-byte reads of the flush (lane (tile, wave) of row w) both touch every
 //     bank once.  (As [tile][wave][row] the flush's reads fell on two banks: 0.5 us of the launch's end.)
 //   * Stores go out only behind the last tile of four: a store between the tiles' loads costs 0.15 us each.
-template <class F>
+//   * NORM puts a residual add and an RMSNorm in front of the product (QdNorm: x += res; hn = x / rms(x) * w;
+//     y = W hn as one launch): every workgroup normalises the row for itself and quantises (x + res) w; the
+//     1 / rms, one factor for the whole row, goes onto the sub-block scales behind the barrier that publishes
+//     tile 0, where the waves' sums of squares have met anyway.  Workgroup 0 stores x + res (into a buffer other
+//     than X: the others are still reading X) and, when asked, the normalised row.  The norm's operands are
+//     arguments of their own so that the leading ones arrive preloaded.
+//   * SWIGLU: the matrix holds gate and up rows alternately (row 2j gate_j, row 2j + 1 up_j) and
+//     Y[j] = silu(gate_j . x) * (up_j . x), n / 2 values (reference: src/quantized_qwen3_moe.rs:397-401).
+template <class F, bool NORM = false, bool SWIGLU = false>
 __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                      float *__restrict__ Y, int n, int G, int rounds, int extra) {
+                                                      float *__restrict__ Y, int n, int G, int rounds, int extra,
+                                                      const float *nm_res, const float *nm_w, float nm_eps,
+                                                      float *nm_x_out, float *nm_hn_out) {
     constexpr int SLOTS = 3, FL = 4;                 // ring slots (two tiles in flight); tiles a flush
+    static_assert(!NORM || 2048 <= F::ROW_LDS, "the norm's operands wait in a wave's row of ring slot 1");
+    __shared__ float ss_lds[16];
     constexpr int FULL = F::ROW / 1024, REST = (F::ROW - 1024 * FULL) / 16, LOADS = FULL + (REST ? 1 : 0);
     __shared__ __attribute__((aligned(16))) uint8_t ring[SLOTS][16 * F::ROW_LDS];
     __shared__ __attribute__((aligned(16))) float part[FL][16][68];
@@ -340,16 +360,39 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
     uint32_t *stage = (uint32_t *)(STAGE_IN_RING ? &ring[SLOTS - 1][wave * F::ROW_LDS] : &stage_mem[wave * STAGE]);
     float *x_raw = (float *)((uint8_t *)stage + F::STAGE_BYTES);
     async_load16(X + 256 * wave + 4 * lane, lds_offset_of(x_raw));
+    // norm weight and residual columns wait in the wave's row of ring slot 1, which no tile enters before the
+    // activations are prepared
+    float *w_raw = (float *)&ring[1][wave * F::ROW_LDS], *r_raw = w_raw + 256;
+    if (NORM) {
+        async_load16(nm_w + 256 * wave + 4 * lane, lds_offset_of(w_raw));
+        if (nm_res) async_load16(nm_res + 256 * wave + 4 * lane, lds_offset_of(r_raw));
+    }
     // every wave's activations are asked for before anybody's tile: the memory pipeline takes a compute
     // unit's requests in the order they were issued, and a wave whose activations queue behind the other
     // waves' tile loads starts its preparation late
     __builtin_amdgcn_s_barrier();
     // tile 0 is asked for alone and lands while the activations are prepared; tile 1 follows the preparation
+    // (asked for in front of it, tile 1 delays the preparation: a wave stands at a load until the memory
+    // pipeline accepts it; measured slower both on a resident activation row and behind another kernel)
     fetch(0);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
-    const float4 v = *(const float4 *)&x_raw[4 * lane];
-    const typename F::Acts acts = F::prepare(v, stage, lane);
+    float4 v = *(const float4 *)&x_raw[4 * lane];
+    if (NORM) {
+        if (nm_res) {
+            const float4 rr = *(const float4 *)&r_raw[4 * lane];
+            v.x += rr.x, v.y += rr.y, v.z += rr.z, v.w += rr.w;
+        }
+        float ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w)));
+        ss = wave_sum(ss);
+        if (lane == 0) ss_lds[wave] = ss;
+        const float4 g = *(const float4 *)&w_raw[4 * lane];
+        if (b == 0) *(float4 *)(nm_x_out + 256 * wave + 4 * lane) = v;
+        v = float4{v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w};
+    }
+    typename F::Acts acts = F::prepare(v, stage, lane);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // (the store of x + res counts among the wave's memory operations until it is acknowledged: the waits
+    // below then hold a little longer in workgroup 0, never too short)
     fetch(1);
 
     for (int t = 0; t < nt; t++) {
@@ -358,6 +401,14 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        if (NORM && t == 0) {  // the waves' sums of squares are all written
+            float tot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) tot += ss_lds[i];
+            const float inv = 1.0f / sqrtf(tot / (float)F::COLS + nm_eps);
+            F::scale(acts, inv);
+            if (b == 0 && nm_hn_out) *(float4 *)(nm_hn_out + 256 * wave + 4 * lane) = float4{v.x * inv, v.y * inv, v.z * inv, v.w * inv};
+        }
         part[t & (FL - 1)][r][4 * wave + c] = F::block_dot_lane(&ring[t % SLOTS][r * F::ROW_LDS + wave * F::BLOCK], acts, c);
         // every wave is done with tile t - 1, whose slot tile t + 2 takes
         if (t + 2 < nt) fetch(t + 2);
@@ -371,9 +422,19 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
             const float4 p = *(const float4 *)&part[c][wave][4 * r];
             float sum = (p.x + p.y) + (p.z + p.w);
             sum = sum_row16(sum);
-            if (r == 0 && tt <= t) {
-                const int row = tile_row0(tt) + wave;
-                if (row < n) Y[row] = sum;
+            if (!SWIGLU) {
+                if (r == 0 && tt <= t) {
+                    const int row = tile_row0(tt) + wave;
+                    if (row < n) Y[row] = sum;
+                }
+            } else if ((wave & 1) == 0) {  // an even wave takes its gate row and the up row behind it
+                const float4 q = *(const float4 *)&part[c][wave + 1][4 * r];
+                float up = (q.x + q.y) + (q.z + q.w);
+                up = sum_row16(up);
+                if (r == 0 && tt <= t) {
+                    const int row = tile_row0(tt) + wave;
+                    if (row + 1 < n) Y[row >> 1] = silu(sum) * up;
+                }
             }
         }
     }
