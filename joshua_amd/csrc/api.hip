@@ -24,7 +24,6 @@
 #include "kernels_mfma_q4k_stream.hpp"
 #include "kernels_dot4_q4k.hpp"
 #include "kernels_gemv_mfma.hpp"
-#include "kernels_dot4_q4k_r8.hpp"
 #include "kernels_dot4_q6k.hpp"
 #include "kernels_dot4_q8.hpp"
 #include "kernels_moe.hpp"
@@ -294,39 +293,13 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     static const char *mode_env = getenv("JQ_Q4K_DOT4");
     static const std::string mode = mode_env ? mode_env : "auto";
     if (mode == "0" || nb == 0 || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0) return -1;
-    // rows of 8192 or 12288 (a feed-forward down projection): steps of 8 rows x 4096 columns
-    // (4096 x 12288: 9.2 us against 11.1 us for the MFMA GEMV)
-    static const char *cols_all_env = getenv("JQ_Q4K_GEMV_COLS");  // "all": rows of 8192 and 12288 too on the matrix-core kernel in passes
-    const bool cols_all = cols_all_env && !strcmp(cols_all_env, "all");
-    // (up to 4096 weight rows, one row tile a workgroup: 4096 x 12288 8.1 us against 9.1 on the matrix-core kernel
-    // in passes; beyond, that kernel: 8192 x 8192 8.6 against 10.3, 28672 x 8192 22.6 against 25.4)
-    if (mode == "auto" && !norm && !swiglu && !cols_all && (nb == 32 || nb == 48) && row_bytes == nb / 16 * jq::QD_ROW && n >= 1024 &&
-        n <= 4096) {
-        // one 16-row tile for (nearly) every compute unit: the 16-row steps are 3 to 6 % ahead there
-        // (4096 x 12288: 8.8 us; 4096 x 8192: 6.4 us against 6.8 us)
-        const size_t tiles16 = (n + 15) / 16;
-        if (tiles16 > 224 && tiles16 <= 256) {
-            note_kernel("q4k_gemv_dot4_cols");
-            if (nb == 32) hipLaunchKernelGGL(jq::q4k_gemv_dot4_cols<2>, dim3(tiles16), dim3(1024), 0, s, W, X, Y, (int)n, (int)tiles16);
-            else hipLaunchKernelGGL(jq::q4k_gemv_dot4_cols<3>, dim3(tiles16), dim3(1024), 0, s, W, X, Y, (int)n, (int)tiles16);
-            HIP_TRY(hipGetLastError());
-            return 0;
-        }
-        const size_t tiles8 = (n + 7) / 8, rounds = (tiles8 + 255) / 256;
-        const unsigned grid = (unsigned)((tiles8 + rounds - 1) / rounds);
-        note_kernel("q4k_gemv_dot4_r8");
-        if (nb == 32) hipLaunchKernelGGL(jq::q4k_gemv_dot4_r8<2>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
-        else hipLaunchKernelGGL(jq::q4k_gemv_dot4_r8<3>, dim3(grid), dim3(1024), 0, s, W, X, Y, (int)n, (int)grid);
-        HIP_TRY(hipGetLastError());
-        return 0;
-    }
-    // other rows of more than 16 super-blocks (up to 64: rows of 4352 to 16384 columns, contiguous), 512 weight
-    // rows or more: the matrix-core kernel over two to four passes of 16 columns
+    // rows of more than 16 super-blocks (up to 64: rows of 4352 to 16384 columns, contiguous), 512 weight rows or
+    // more: the matrix-core kernel over two to four passes of 16 columns (4096 x 12288, a feed-forward down
+    // projection: 7.2 us, where v_dot4 kernels in steps of 8 and 16 rows took 8.9; 4096 x 8192 5.6 against 6.5;
+    // 7168 x 16384 15.7 us against 22.7 for the one-shot kernel).  JQ_Q4K_GEMV_COLS = 0 switches it off.
     static const char *cols_env = getenv("JQ_Q4K_GEMV_COLS");
-    // (four passes keep 16 spilled registers: ahead of the one-shot kernel from two row tiles a workgroup on,
-    // 7168 x 16384 21.1 against 22.7 us, behind it at one, 4096 x 16384 14.9 against 12.0)
     if (mode == "auto" && !norm && !swiglu && !(cols_env && cols_env[0] == '0') && nb > 16 && nb <= 64 &&
-        row_bytes == nb * 144 && n >= 512 && n <= 0x7FFFFFF0ull && (nb <= 48 || n > 4096)) {
+        row_bytes == nb * 144 && n >= 512 && n <= 0x7FFFFFF0ull) {
         const size_t tiles = (n + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
         const jq::QvColsWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G), (int)nb};
         note_kernel("q4k_gemv_mfma_cols");

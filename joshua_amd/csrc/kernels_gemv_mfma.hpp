@@ -30,8 +30,6 @@
 
 namespace jq {
 
-constexpr int QV_SLOTS = 4;  // ring slots
-
 typedef int qv_i4 __attribute__((ext_vector_type(4)));
 
 // What a lane keeps of its wave's 256 activations for the whole kernel.
@@ -181,10 +179,10 @@ struct QvQ4KCompact {
         *side = float4{a.s_e, a.s_o16, a.xs_e, a.xs_o};  // the same from the 16 lanes of a group
         return Acts{{a.a_even[0], a.a_even[1]}, {a.a_odd[0], a.a_odd[1]}, a.c_init[2], side};
     }
-    __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) {
+    __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) {
         const float4 f = *a.side;
         const QvActs full{{a.a_even[0], a.a_even[1]}, {a.a_odd[0], a.a_odd[1]}, qv_i4{0, 0, a.c_init2, 0}, f.x, f.y, f.z, f.w};
-        return qv_block_dot(blk, full, c);
+        return qv_block_dot_lane(blk, full, c);
     }
 };
 
@@ -299,7 +297,9 @@ struct QvWork {
 // An asynchronous 16-byte load a lane whose global address is a scalar base (the wave's row) plus the lane's own
 // byte offset: no vector instruction goes into the address.
 __device__ __forceinline__ void async_load16_s(const uint8_t *sbase, uint32_t voff, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory");
 }
 
 // Wave w copies row w of a tile into a ring of three tiles in LDS (contiguous asynchronous loads, two tiles
@@ -442,8 +442,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
 
 // The same kernel for rows of more than 16 super-blocks (up to 16 NG): a tile is 16 rows x one pass of 16
 // columns (the last pass may hold fewer), tile i of a workgroup = (row tile i / NG, pass i % NG), and wave w
-// keeps the operands of its column of every pass.  The partial sums of a row tile's passes are added when the
-// tile is flushed.  nb = super-blocks a row (contiguous rows of nb blocks); rounds / extra count row tiles.
+// keeps the operands of its column of every pass.  A lane adds its chunk sums of a row tile's passes in a
+// register.  nb = super-blocks a row (contiguous rows of nb blocks); rounds / extra count row tiles.
 struct QvColsWork {
     int n, G, rounds, extra, nb;
 };
@@ -452,18 +452,23 @@ template <class F, int NG>
 __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict__ W, const float *__restrict__ X,
                                                        float *__restrict__ Y, int n, int G, int rounds, int extra, int nb) {
     static_assert(NG >= 2 && NG <= 4, "two to four passes a row");
-    constexpr int D = 2, LOADS = (F::ROW + 1023) / 1024, TG = NG == 3 ? 3 : 4;  // tiles a flush: whole row tiles
-    // the raw activations of the passes wait in the wave's own rows of ring slots 3 (behind what prepare()
-    // uses), 2 and 1, which no load targets before the wave itself asks for tiles 1, 2 and 3
+    // ring slots (two tiles in flight; a fourth slot only where the staging of four passes needs it) and row
+    // tiles a flush
+    constexpr int SLOTS = NG == 4 ? 4 : 3, FL = NG == 4 ? 2 : 4;
+    constexpr int LOADS = (F::ROW + 1023) / 1024;
+    // the raw activations of the passes wait in the wave's own rows of the last ring slot (behind what prepare()
+    // uses), of the one in front of it and of slot 1, which no load targets before the wave itself has prepared
+    // its activations and asks for tile 1
     static_assert(F::STAGE_BYTES + 1024 <= F::ROW_LDS && 2048 <= F::ROW_LDS, "staging in the ring");
-    __shared__ __attribute__((aligned(16))) uint8_t ring[QV_SLOTS][16 * F::ROW_LDS];
-    __shared__ float part[TG][16][16];  // [tile of the flush group][wave][row]
+    __shared__ __attribute__((aligned(16))) uint8_t ring[SLOTS][16 * F::ROW_LDS];
+    __shared__ __attribute__((aligned(16))) float part[FL][16][68];  // [row tile][row][4 wave + chunk], as in gemv_mfma_lds
     __shared__ float4 side[F::SIDE_LDS ? 16 * NG * 4 : 1];  // [wave][pass][lane group], for the policies that want it
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, c = lane >> 4, b = (int)blockIdx.x;
     const size_t row_bytes = (size_t)nb * F::BLOCK;
-    const int nt = NG * (rounds + (b < extra ? 1 : 0));
+    const int nrt = rounds + (b < extra ? 1 : 0), nt = NG * nrt;  // row tiles, tiles (row tile, pass) of this workgroup
     if (nt <= 0) return;
+    const uint32_t ring0 = lds_offset_of(&ring[0][0]);
     // every fetch is LOADS instructions with at least one lane at work, so that every wave counts the same
     // loads; a short last pass repeats its last 16 bytes into LDS bytes nobody reads
     auto fetch = [&](int slot_i) __attribute__((always_inline)) {
@@ -471,26 +476,25 @@ __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict
         const int row = min(16 * (b + rt * G) + wave, n - 1);
         const int len = min(16, nb - 16 * cg) * F::BLOCK;
         const uint8_t *src = W + (size_t)row * row_bytes + (size_t)cg * F::ROW;
-        const uint32_t dst = lds_offset_of(&ring[slot_i & (QV_SLOTS - 1)][wave * F::ROW_LDS]);
+        const uint32_t dst = ring0 + (uint32_t)(slot_i % SLOTS) * (16 * F::ROW_LDS) + (uint32_t)wave * F::ROW_LDS;
 #pragma unroll
         for (int j = 0; j < LOADS; j++) {
             const int lanes = max(1, min(64, (min(len, F::ROW) - 1024 * j) / 16));
-            if (lane < lanes) async_load16(src + min(1024 * j + 16 * lane, len - 16), dst + 1024 * j);
+            if (lane < lanes) async_load16_s(src, (uint32_t)min(1024 * j + 16 * lane, len - 16), dst + 1024 * j);
         }
     };
-    uint32_t *stage = (uint32_t *)&ring[3][wave * F::ROW_LDS];
+    uint32_t *stage = (uint32_t *)&ring[SLOTS - 1][wave * F::ROW_LDS];
     auto x_raw = [&](int cg) __attribute__((always_inline)) {
         return cg == 0   ? (float *)((uint8_t *)stage + F::STAGE_BYTES)
                : cg == 3 ? (float *)&ring[1][wave * F::ROW_LDS]
-                         : (float *)&ring[2][wave * F::ROW_LDS + 1024 * (cg - 1)];
+                         : (float *)&ring[SLOTS - 2][wave * F::ROW_LDS + 1024 * (cg - 1)];
     };
 #pragma unroll
     for (int cg = 0; cg < NG; cg++)  // a column past the row's last block reads the last one's and is not used
         async_load16(X + 256 * min(16 * cg + wave, nb - 1) + 4 * lane, lds_offset_of(x_raw(cg)));
     __builtin_amdgcn_s_barrier();
     fetch(0);
-    if (LOADS == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
     typename F::Acts acts[NG];
 #pragma unroll
     for (int cg = 0; cg < NG; cg++) {
@@ -501,44 +505,35 @@ __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     fetch(1);
 
-    const int n_groups = (nt + TG - 1) / TG;
-    for (int grp = 0; grp < n_groups; grp++) {
-        const int t0 = TG * grp, t_end = min(nt, t0 + TG);
+    for (int rt = 0; rt < nrt; rt++) {
+        float acc = 0.0f;  // a lane's chunk sums of the row tile's passes
 #pragma unroll
-        for (int u = 0; u < TG; u++) {
-            const int t = t0 + u;
-            if (t >= t_end) break;  // the same for the whole workgroup
-            const int ahead = t == nt - 1 ? 0 : max(D - 1, min(nt - 1, t + D - 1)) - t;
-            if (LOADS == 3) {
-                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            } else {
-                if (ahead >= 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-                else if (ahead == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            }
+        for (int cg = 0; cg < NG; cg++) {
+            const int t = NG * rt + cg;
+            if (t + 1 < nt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (t + D < nt) fetch(t + D);
-            const int cg = u % NG;  // t0 is a multiple of NG
-            float acc = 0.0f;
             if (16 * cg + wave < nb)
-                acc = F::block_dot(&ring[t & (QV_SLOTS - 1)][r * F::ROW_LDS + wave * F::BLOCK], acts[cg], c);
-            if (lane < 16) part[u][wave][lane] = acc;
+                acc += F::block_dot_lane(&ring[t % SLOTS][r * F::ROW_LDS + wave * F::BLOCK], acts[cg], c);
+            // every wave is done with tile t - 1, whose slot tile t + 2 takes (with four slots: tile t - 2's)
+            if (t + 2 < nt) fetch(t + 2);
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        // lane (tt = lane / 16, ww = lane % 16) takes wave ww's sum of row `wave` in tile tt of the group, the
-        // 16 lanes of a tile add up, then the tiles that are passes of one row tile
-        float sum = t0 + c < t_end ? part[c < TG ? c : 0][r][wave] : 0.0f;
-        sum = sum_row16(sum);
-        if (NG == 2) sum = sum_xor16(sum);
-        else sum = sum_xor32(sum_xor16(sum));
-        if (r == 0 && c % NG == 0 && t0 + c < t_end) {
-            const int row = 16 * (b + ((t0 + c) / NG) * G) + wave;
-            if (row < n) Y[row] = sum;
+        part[rt & (FL - 1)][r][4 * wave + c] = acc;
+        if ((rt & (FL - 1)) == FL - 1 || rt == nrt - 1) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            // lane (tt = lane / 16, ww = lane % 16) takes wave ww's four chunk sums of row `wave` in row tile tt of
+            // the group
+            const int tt = (rt & ~(FL - 1)) + c;
+            const float4 p = *(const float4 *)&part[c & (FL - 1)][wave][4 * r];
+            float sum = (p.x + p.y) + (p.z + p.w);
+            sum = sum_row16(sum);
+            if (r == 0 && c < FL && tt <= rt) {
+                const int row = 16 * (b + tt * G) + wave;
+                if (row < n) Y[row] = sum;
+            }
         }
     }
 }

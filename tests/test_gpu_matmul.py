@@ -1026,9 +1026,10 @@ def test_q4k_mfma_gemv_switched_off_by_environment():
 
 KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (format, m, k, n) -> jq_last_kernel()
     (capi.Q4_K, 1, 4096, 14336, "q4k_gemv_mfma_lds"),        # headline
-    (capi.Q4_K, 1, 4096, 4096, "q4k_gemv_dot4_lds"),
-    (capi.Q4_K, 1, 12288, 4096, "q4k_gemv_dot4_cols"),       # a feed-forward down projection
-    (capi.Q4_K, 1, 8192, 2048, "q4k_gemv_dot4_r8"),
+    (capi.Q4_K, 1, 4096, 4096, "q4k_gemv_mfma_lds"),
+    (capi.Q4_K, 1, 4096, 1024, "q4k_gemv_dot4_lds"),         # fewer than 2048 weight rows
+    (capi.Q4_K, 1, 12288, 4096, "q4k_gemv_mfma_cols"),       # a feed-forward down projection
+    (capi.Q4_K, 1, 8192, 2048, "q4k_gemv_mfma_cols"),
     (capi.Q4_K, 1, 8192, 8192, "q4k_gemv_mfma_cols"),        # more than one row tile a workgroup
     (capi.Q4_K, 1, 2048, 768, "q4k_gemv_mfma"),              # an expert's gate projection
     (capi.Q4_K, 1, 7168, 1536, "q4k_gemv_mfma_cols"),        # DeepSeek-V3's query down-projection
