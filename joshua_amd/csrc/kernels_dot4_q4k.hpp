@@ -28,6 +28,56 @@ namespace jq {
 constexpr int QD_MAX_WAVES = 16;
 constexpr float QD_RANGE = 32639.0f;  // 127 * 256 + 127
 
+// A lane's four activations (elements 4i .. 4i+3 of a 32-element sub-block held by 8 lanes) as 16-bit fixed
+// point against the sub-block's maximum, in as few vector instructions as the arithmetic allows: every
+// workgroup repeats this for the whole activation row in front of its first product, four waves a SIMD, so
+// an instruction here costs sixteen cycles of the launch's start.  (The one-row kernels of every format use it.)
+//   * the maximum is taken over the magnitudes' bit patterns as unsigned integers: NaN > inf > finite, so a
+//     non-finite element needs no test of its own;
+//   * the scale amax / 32639 by a multiplication with one correction step, which is exact whenever the
+//     quotient is a float; its inverse by the hardware reciprocal (a relative error of 2^-22 moves X by less
+//     than 0.02, so an activation that is an integer multiple of the scale still quantises to that integer);
+//   * X = round(x inv) as the mantissa of fma(x, inv, 1.5 * 2^23 + 128): bits 0..15 of the result are X + 128,
+//     byte 1 the high plane, byte 0 the low plane with its top bit flipped; four v_perm_b32 gather the planes.
+// Returns the plane words of X (wl, wh) and of -X (nl, nh), the scale (NaN for a sub-block with a non-finite
+// element, 0 for one of zeros) and the sum of the sub-block's X in every lane of the sub-block.
+struct QvQuant {
+    uint32_t wl, wh, nl, nh;
+    float s;
+    int sum;
+};
+__device__ __forceinline__ QvQuant qv_quantise4(const float4 v) {
+    const uint32_t b0 = __builtin_bit_cast(uint32_t, v.x) & 0x7FFFFFFFu, b1 = __builtin_bit_cast(uint32_t, v.y) & 0x7FFFFFFFu;
+    const uint32_t b2 = __builtin_bit_cast(uint32_t, v.z) & 0x7FFFFFFFu, b3 = __builtin_bit_cast(uint32_t, v.w) & 0x7FFFFFFFu;
+    uint32_t m = max(max(b0, b1), max(b2, b3));
+    m = max(m, (uint32_t)dpp_i<0x141>((int)m));
+    m = max(m, (uint32_t)dpp_i<0xB1>((int)m));
+    m = max(m, (uint32_t)dpp_i<0x4E>((int)m));
+    const float amax = __builtin_bit_cast(float, m);
+    constexpr float RC = 1.0f / QD_RANGE;
+    float s = amax * RC;
+    s = fmaf(fmaf(-s, QD_RANGE, amax), RC, s);
+    const float inv = __builtin_amdgcn_rcpf(fmaxf(s, 1e-35f));  // of the scale: a normal number for every finite amax
+    s = m >= 0x7F800000u ? NAN : s;
+    constexpr float MAGIC = 12582912.0f + 128.0f;
+    const float ninv = -inv;
+    const uint32_t t0 = __builtin_bit_cast(uint32_t, fmaf(v.x, inv, MAGIC)), t1 = __builtin_bit_cast(uint32_t, fmaf(v.y, inv, MAGIC));
+    const uint32_t t2 = __builtin_bit_cast(uint32_t, fmaf(v.z, inv, MAGIC)), t3 = __builtin_bit_cast(uint32_t, fmaf(v.w, inv, MAGIC));
+    const uint32_t u0 = __builtin_bit_cast(uint32_t, fmaf(v.x, ninv, MAGIC)), u1 = __builtin_bit_cast(uint32_t, fmaf(v.y, ninv, MAGIC));
+    const uint32_t u2 = __builtin_bit_cast(uint32_t, fmaf(v.z, ninv, MAGIC)), u3 = __builtin_bit_cast(uint32_t, fmaf(v.w, ninv, MAGIC));
+    // v_perm_b32(a, b, sel): selector 0..3 takes byte 0..3 of b, 4..7 of a
+    const uint32_t p01 = __builtin_amdgcn_perm(t1, t0, 0x05010400u), p23 = __builtin_amdgcn_perm(t3, t2, 0x05010400u);
+    const uint32_t n01 = __builtin_amdgcn_perm(u1, u0, 0x05010400u), n23 = __builtin_amdgcn_perm(u3, u2, 0x05010400u);
+    QvQuant q;
+    q.wl = __builtin_amdgcn_perm(p23, p01, 0x05040100u) ^ 0x80808080u, q.wh = __builtin_amdgcn_perm(p23, p01, 0x07060302u);
+    q.nl = __builtin_amdgcn_perm(n23, n01, 0x05040100u) ^ 0x80808080u, q.nh = __builtin_amdgcn_perm(n23, n01, 0x07060302u);
+    q.s = s;
+    constexpr uint32_t BASE4 = 4u * 0x4B400080u;  // four times the bit pattern of MAGIC, modulo 2^32
+    q.sum = isum_row8((int)(t0 + t1 + t2 + t3 - BASE4));
+    return q;
+}
+
+
 struct QdTile {  // what a lane holds of one 16-row tile
     uint4 hdr, qa, qb;
 };

@@ -22,7 +22,8 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
     __shared__ __attribute__((aligned(16))) uint8_t ring[3][Q8D_STEP_LDS];
     __shared__ uint32_t xl_lds[NG][16][64], xh_lds[NG][16][64];
     __shared__ float s_lds[NG][16][8];
-    __shared__ float red[2][16][Q8D_ROWS];
+    __shared__ float red[2][Q8D_ROWS][17];   // [tile % 2][row][wave]: a wave's writes and a row's reads each touch a bank once
+    __shared__ float out_lds[8][Q8D_ROWS];  // the rows of up to eight tiles wait here: a store between the steps' loads costs 0.15 us
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane >> 3, j = lane & 7;  // row of the step, block of the wave's eight
     const int n_tiles = (((n + Q8D_ROWS - 1) / Q8D_ROWS) - (int)blockIdx.x + G - 1) / G;  // row tiles blockIdx.x, + G, ...
@@ -64,21 +65,10 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
         float4 v;
         if constexpr (STAGED_X) v = *(const float4 *)&x_raw[g][wave][4 * lane];
         else v = *(const float4 *)(X + (size_t)(16 * g + wave) * 256 + 4 * lane);
-        float amax = fmaxf(fmaxf(mag_or_inf(v.x), mag_or_inf(v.y)), fmaxf(mag_or_inf(v.z), mag_or_inf(v.w)));
-        amax = max_row8(amax);
-        const bool live = amax > 0.0f && amax < INFINITY;
-        const float inv = live ? QD_RANGE / amax : 0.0f, s = fixed_scale(amax, QD_RANGE);
-        const int Xq[4] = {__float2int_rn(v.x * inv), __float2int_rn(v.y * inv), __float2int_rn(v.z * inv),
-                           __float2int_rn(v.w * inv)};
-        uint32_t wl = 0, wh = 0;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int lo = ((Xq[i] + 128) & 255) - 128, hi = (Xq[i] - lo) >> 8;
-            wl |= (uint32_t)(lo & 255) << (8 * i);
-            wh |= (uint32_t)(hi & 255) << (8 * i);
-        }
-        xl_lds[g][wave][lane] = wl;
-        xh_lds[g][wave][lane] = wh;
+        const QvQuant qx = qv_quantise4(v);
+        xl_lds[g][wave][lane] = qx.wl;
+        xh_lds[g][wave][lane] = qx.wh;
+        const float s = qx.s;
         if ((lane & 7) == 0) s_lds[g][wave][lane >> 3] = s;
     }
     // step 0 landed (step 1 may be in flight), planes written
@@ -123,7 +113,7 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
             const int buf = tile & 1;
             if (g == NG - 1) {  // the row tile is complete: the lanes of a row, then the waves through LDS
                 acc = sum_row8(acc);
-                if (j == 0) red[buf][wave][r] = acc;
+                if (j == 0) red[buf][r][wave] = acc;
                 acc = 0.0f;
             }
             // step st+1 has landed (and the partial sums are written): at most this step's 3 loads stay in flight
@@ -131,11 +121,19 @@ __global__ __launch_bounds__(1024) void q8_0_gemv_dot4_lds(const uint8_t *__rest
             else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (g == NG - 1 && wave < Q8D_ROWS) {  // wave w sums row w of the tile over the 16 waves
-                float v = (lane < 16) ? red[buf][lane][wave] : 0.0f;
-                v = sum_row16(v);
-                const int row = Q8D_ROWS * ((int)blockIdx.x + tile * G) + wave;
-                if (lane == 0 && row < n) Y[row] = v;
+            if (g == NG - 1) {
+                if (wave < Q8D_ROWS) {  // wave w sums row w of the tile over the 16 waves
+                    float v = (lane < 16) ? red[buf][wave][lane] : 0.0f;
+                    v = sum_row16(v);
+                    if (lane == 0) out_lds[tile & 7][wave] = v;
+                }
+                if ((tile & 7) == 7 || tile == n_tiles - 1) {  // wave 0 stores the rows of the last (up to) eight tiles
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    const int tt = (tile & ~7) + (lane >> 3), row = Q8D_ROWS * ((int)blockIdx.x + tt * G) + (lane & 7);
+                    if (wave == 0 && tt <= tile && row < n) Y[row] = out_lds[lane >> 3][lane & 7];
+                }
             }
         }
     }
