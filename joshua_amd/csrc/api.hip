@@ -596,12 +596,16 @@ int dispatch_q4k_ring(const uint8_t *W, size_t row_bytes, const float *X, float 
 // price of writing and re-reading the partial sums.  Estimated per candidate from the measured step time of
 // a workgroup (us per super-block, plus its start and end) and ~3 TB/s for the partial sums; the choice
 // depends on the shape only, so a shape always gets the same order of additions.
+// `other_bytes`: what the call keeps in its scratch beside the partial sums; with a scratch of fixed size (the
+// entry point that allocates nothing) a split count whose partial sums would not fit is passed over.
 int gemm_k_splits(size_t total, size_t nb, size_t m, size_t n, double us_per_block, const char *env,
-                  double *estimate_us = nullptr) {
+                  double *estimate_us = nullptr, size_t other_bytes = 0) {
     if (env && !estimate_us) return (int)std::min<size_t>(std::max(atoi(env), 1), nb);
+    const size_t cap = tl_fixed_scratch && !estimate_us ? tl_fixed_scratch->bytes : (size_t)1 << 60;
     int best = 1;
     double best_us = 0.0;
     for (size_t sp = 1; sp <= std::min<size_t>(nb, 16); sp++) {
+        if (sp > 1 && other_bytes + sp * m * n * sizeof(float) > cap) continue;
         const double rounds = (double)((total * sp + 255) / 256);
         const double wg_us = 3.0 + us_per_block * (double)((nb + sp - 1) / sp);
         const double sum_us = sp == 1 ? 0.0 : 3.0 + (double)(2 * sp + 1) * (double)(m * n) * 4.0 / 3.0e6;
@@ -802,7 +806,7 @@ int dispatch_q4k_gemm(const uint8_t *W, size_t row_bytes, const float *X, float 
     else per_xcd = (n_tiles + 8 / m_tiles - 1) / (8 / m_tiles);
     const size_t base_grid = 8 * per_xcd;
     static const char *split_env = getenv("JQ_Q4K_GEMM_SPLITS");
-    const size_t splits = m * n / 1024 < 0x7FFFFFFFull ? (size_t)gemm_k_splits(total, nb, m, n, 6.0, split_env) : 1;
+    const size_t splits = m * n / 1024 < 0x7FFFFFFFull ? (size_t)gemm_k_splits(total, nb, m, n, 6.0, split_env, nullptr, plane_bytes + min_bytes) : 1;
     if (base_grid * splits > 0x0FFFFFFFull) return fail("q4k gemm: %zu x %zu tiles exceed the grid limit", m_tiles, n_tiles);
     const size_t part_bytes = splits > 1 ? splits * m * n * sizeof(float) : 0;
     CallScratch scratch;
@@ -839,7 +843,7 @@ int launch_gemm_decoded(const uint8_t *W, size_t row_bytes, const float *X, floa
     // split over k when the 64 x 64 tiles alone leave compute units idle (a workgroup takes ~5 us a chunk)
     const size_t n_tiles = (n + jq::GD_NT - 1) / jq::GD_NT, m_tiles = m_pad / jq::GD_MT;
     static const char *split_env = getenv("JQ_DECODED_GEMM_SPLITS");
-    const size_t splits = m * n / 1024 < 0x7FFFFFFFull ? (size_t)gemm_k_splits(n_tiles * m_tiles, nc, m, n, 5.0, split_env) : 1;
+    const size_t splits = m * n / 1024 < 0x7FFFFFFFull ? (size_t)gemm_k_splits(n_tiles * m_tiles, nc, m, n, 5.0, split_env, nullptr, 2 * plane + sbytes) : 1;
     const size_t part_bytes = splits > 1 ? splits * m * n * sizeof(float) : 0;
     CallScratch scratch;
     uint8_t *buf = nullptr;
@@ -1227,6 +1231,14 @@ int jq_decode_raw_to_f32(uint32_t ggml_type, const void *bytes, size_t nbytes, s
         if (!geometry(ggml_type, &g)) return 2;  // no decoder in the reference either: Ok(None)
         blck = g.elems, bb = g.bytes;
     }
+    if (ggml_type == 16 || ggml_type == 39) {
+        // the in-mapping formats fail in their own block readers, with their own words
+        // (src/iq2xxs.rs:75-82,422-429, src/mxfp4.rs:99-106,265-272; the output there is sized by `elems`)
+        const char *nm = ggml_type == 16 ? "iq2_xxs" : "mxfp4";
+        if (nbytes % bb != 0)
+            return fail(ggml_type == 16 ? "%s: %zu bytes is not a whole number of %zu byte blocks" : "%s: %zu bytes is not a whole number of %zu-byte blocks", nm, nbytes, bb);
+        if (elems != nbytes / bb * blck) return fail("%s: output holds %zu values, expected %zu", nm, elems, nbytes / bb * blck);
+    }
     if (elems % blck != 0 || nbytes != elems / blck * bb) {
         if (ggml_type == 1) return fail("dtype F16: %zu bytes for %zu elements", nbytes, elems);
         return fail("dtype %u: %zu bytes for %zu elements (%zu per %zu-block)", ggml_type, nbytes, elems, bb, blck);
@@ -1251,9 +1263,20 @@ int jq_decode_raw_to_f32(uint32_t ggml_type, const void *bytes, size_t nbytes, s
         else hipLaunchKernelGGL((jq::decode_plain<15>), dim3(blocks), dim3(256), 0, s, src, dst, elems);
         HIP_TRY(hipGetLastError());
     } else {
-        jq_weight view{};  // one row of `elems` columns over the caller's bytes
-        view.type = ggml_type, view.dev = const_cast<uint8_t *>(src), view.n = 1, view.k = elems, view.row_bytes = nbytes;
-        if (dispatch_decode(&view, nullptr, dst, 1, s)) return 1;
+        // The block decoders index a row's columns with an int, so the caller's bytes are decoded as rows of at
+        // most 2^20 blocks (a tensor of 2^31 elements or more, a stacked expert tensor, is many such rows and a
+        // shorter last one).  JQ_DECODE_CHUNK_BLOCKS, read at every call, sets another row length (for tests).
+        size_t chunk_max = (size_t)1 << 20;
+        if (const char *env = getenv("JQ_DECODE_CHUNK_BLOCKS")) chunk_max = std::max<size_t>(1, (size_t)atoll(env));
+        const size_t blocks_total = elems / blck;
+        for (size_t b0 = 0; b0 < blocks_total;) {
+            const size_t left = blocks_total - b0;
+            const size_t rows = left >= chunk_max ? left / chunk_max : 1, per = left >= chunk_max ? chunk_max : left;
+            jq_weight view{};
+            view.type = ggml_type, view.dev = const_cast<uint8_t *>(src) + b0 * bb, view.n = rows, view.k = per * blck, view.row_bytes = per * bb;
+            if (dispatch_decode(&view, nullptr, dst + b0 * blck, rows, s)) return 1;
+            b0 += rows * per;
+        }
     }
     if (!ptrs_are_device) {
         HIP_TRY(hipMemcpyAsync(out, y.p, elems * sizeof(float), hipMemcpyDeviceToHost, s));
@@ -2236,6 +2259,7 @@ struct jq_mla {
     // scratch, grown to the largest token count seen
     size_t cap_tokens = 0;
     float *t1 = nullptr, *t1n = nullptr, *qv = nullptr, *comp = nullptr, *qabs = nullptr, *part = nullptr, *ctx = nullptr;
+    std::vector<void *> retired;  // outgrown scratch, kept until the object goes
     std::mutex mu;
 };
 
@@ -2246,13 +2270,20 @@ constexpr size_t MLA_PART_SLOTS = 64;  // partial results kept per head: tokens 
 void mla_free_scratch(jq_mla *m) {
     for (void *p : {(void *)m->t1, (void *)m->t1n, (void *)m->qv, (void *)m->comp, (void *)m->qabs, (void *)m->part, (void *)m->ctx})
         if (p) (void)hipFree(p);
+    for (void *p : m->retired) (void)hipFree(p);
+    m->retired.clear();
     m->t1 = m->t1n = m->qv = m->comp = m->qabs = m->part = m->ctx = nullptr;
     m->cap_tokens = 0;
 }
 
+// Scratch for calls of up to T tokens.  Buffers that are outgrown are retired, not freed: a HIP graph captured
+// over an earlier, smaller call still names them, and they go with the object (jq_mla_free).
 int mla_reserve(jq_mla *m, size_t T) {
     if (T <= m->cap_tokens) return 0;
-    mla_free_scratch(m);
+    for (void *p : {(void *)m->t1, (void *)m->t1n, (void *)m->qv, (void *)m->comp, (void *)m->qabs, (void *)m->part, (void *)m->ctx})
+        if (p) m->retired.push_back(p);
+    m->t1 = m->t1n = m->qv = m->comp = m->qabs = m->part = m->ctx = nullptr;
+    m->cap_tokens = 0;
     const jq_mla_config &c = m->cfg;
     const size_t qd = c.qk_nope_head_dim + c.qk_rope_head_dim;
     if (c.q_lora_rank) {

@@ -2,6 +2,8 @@
 formats' definitions, then the device entry point against the oracle.  F16 is pinned by numpy's own
 float16 conversion, Q8_K by d * q in numpy; Q8_1 follows ggml's published layout (parity unpinned: the
 reference hands it to candle-core 0.11, which is not in the tree)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -76,6 +78,16 @@ def test_device_decode_raw_against_the_oracle():
     for qt in (8, 10, 12, 14, 16, 39):
         blocks = synth.normal_quantized(qt, 60 + qt, 2048, 0.02)
         assert np.array_equal(capi.decode_raw_to_f32(qt, blocks, 2048), oracle.decode_raw_to_f32(qt, blocks, 2048)), qt
+    # a tensor beyond the decoders' int column index goes through as rows of 2^20 blocks and a shorter last one:
+    # the same walk with rows of 3 blocks (7 blocks: two whole rows and a rest, for every block format)
+    os.environ["JQ_DECODE_CHUNK_BLOCKS"] = "3"
+    try:
+        for qt in (8, 10, 12, 14, 16, 39):
+            elems = 7 * (32 if qt in (8, 39) else 256)
+            blocks = synth.normal_quantized(qt, 70 + qt, elems, 0.02)
+            assert np.array_equal(capi.decode_raw_to_f32(qt, blocks, elems), oracle.decode_raw_to_f32(qt, blocks, elems)), qt
+    finally:
+        del os.environ["JQ_DECODE_CHUNK_BLOCKS"]
     assert capi.decode_raw_to_f32(0, np.zeros(16, np.uint8), 4) is None
     assert capi.decode_raw_to_f32(26, np.zeros(16, np.uint8), 4) is None
     assert capi.decode_raw_to_f32(30, np.zeros(8, np.uint8), 4) is None
@@ -83,3 +95,12 @@ def test_device_decode_raw_against_the_oracle():
         capi.decode_raw_to_f32(1, np.zeros(7, np.uint8), 4)
     with pytest.raises(capi.JoshuaHipError, match="per 256-block"):
         capi.decode_raw_to_f32(12, np.zeros(143, np.uint8), 256)
+    # the in-mapping formats answer in their block readers' words (src/iq2xxs.rs:75-82,422-429, src/mxfp4.rs:99-106,265-272)
+    with pytest.raises(capi.JoshuaHipError, match="iq2_xxs: 65 bytes is not a whole number of 66 byte blocks"):
+        capi.decode_raw_to_f32(16, np.zeros(65, np.uint8), 256)
+    with pytest.raises(capi.JoshuaHipError, match="iq2_xxs: output holds 512 values, expected 256"):
+        capi.decode_raw_to_f32(16, np.zeros(66, np.uint8), 512)
+    with pytest.raises(capi.JoshuaHipError, match="mxfp4: 18 bytes is not a whole number of 17-byte blocks"):
+        capi.decode_raw_to_f32(39, np.zeros(18, np.uint8), 32)
+    with pytest.raises(capi.JoshuaHipError, match="mxfp4: output holds 64 values, expected 32"):
+        capi.decode_raw_to_f32(39, np.zeros(17, np.uint8), 64)

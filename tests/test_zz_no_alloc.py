@@ -63,3 +63,30 @@ def test_noalloc_rejects_a_product_beyond_its_scratch():
     # shape errors read like jq_matmul_t's
     with pytest.raises(capi.JoshuaHipError, match="lhs/dst sized"):
         w.matmul_t_noalloc(2, x.data_ptr(), k, y.data_ptr(), 2 * n, 0)
+
+
+def test_noalloc_leaves_device_memory_alone_on_a_stream_never_used_before():
+    """jq_matmul_t keeps a scratch allocation per stream, made at a stream's first call; the entry point that
+    allocates nothing must not.  On a fresh stream (no allocation of its own yet) the free device memory reads
+    the same before and after a product that needs prepared operands and partial sums, and the result still
+    equals jq_matmul_t's (which runs afterwards, on the default stream)."""
+    import torch
+    k, n, m = 4096, 1024, 96
+    blocks = synth.normal_quantized(capi.Q4_K, 77, n * k, 0.02)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    lhs = synth.normal(78, (m, k))
+    x = torch.from_numpy(lhs).cuda()
+    y_new = torch.full((m, n), float("nan"), device="cuda")
+    y_ref = torch.full((m, n), float("nan"), device="cuda")
+    fresh = torch.cuda.Stream()
+    with torch.cuda.stream(fresh):   # the runtime's own first-use allocations of a stream (2 MiB of queue memory),
+        y_new.fill_(float("nan"))    # by a launch that is not this library's
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    w.matmul_t_noalloc(m, x.data_ptr(), x.numel(), y_new.data_ptr(), y_new.numel(), fresh.cuda_stream)
+    fresh.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    w.matmul_t_dev(m, x.data_ptr(), x.numel(), y_ref.data_ptr(), y_ref.numel(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert np.array_equal(y_ref.cpu().numpy().view(np.uint32), y_new.cpu().numpy().view(np.uint32))
