@@ -386,6 +386,28 @@ int dispatch_q6k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     if ((mode && mode[0] == '0') || k % 4096 != 0 || ng < 1 || ng > 3 || row_bytes != ng * jq::Q6D_SLICE ||
         ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0)
         return -1;
+    // The int8 matrix-core GEMV over the Q6_K policy, for rows of 8192 and 12288 columns and up to 8192 weight
+    // rows (4096 x 12288, a feed-forward down projection: 11.4 us against 12.0 on v_dot4).  A tile of 16 rows is
+    // 54 KB, so its ring has two slots and one tile in flight while a tile is multiplied: with more tiles a
+    // workgroup, and at rows of 4096, the v_dot4 kernel's ring of three 8-row steps streams faster (151936 x 4096:
+    // 87 against 92 us; 4096 x 4096: 6.1 us either way).  JQ_Q6K_GEMV_MFMA = 0 switches it off, = all takes
+    // every shape it can.
+    static const char *mfma_env = getenv("JQ_Q6K_GEMV_MFMA");
+    const bool mfma_all = mfma_env && !strcmp(mfma_env, "all"), mfma_off = mfma_env && mfma_env[0] == '0';
+    if (!mfma_off && n >= 256 && n <= 0x7FFFFFF0ull && (mfma_all || (ng >= 2 && n <= 8192))) {
+        const size_t tiles16 = (n + 15) / 16, rounds_up = (tiles16 + 255) / 256, G = (tiles16 + rounds_up - 1) / rounds_up;
+        const jq::QvColsWork wk{(int)n, (int)G, (int)(tiles16 / G), (int)(tiles16 % G), (int)(16 * ng)};
+        note_kernel(ng == 1 ? "q6k_gemv_mfma_lds" : "q6k_gemv_mfma_cols");
+        if (ng == 1)
+            hipLaunchKernelGGL(jq::gemv_mfma_lds<jq::QvQ6K>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra,
+                               nullptr, nullptr, 0.0f, nullptr, nullptr);
+        else if (ng == 2)
+            hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ6K, 2>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra, wk.nb);
+        else
+            hipLaunchKernelGGL((jq::gemv_mfma_cols<jq::QvQ6K, 3>), dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra, wk.nb);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
     const size_t tiles = (n + jq::Q6D_ROWS - 1) / jq::Q6D_ROWS, rounds = (tiles + 255) / 256;
     if (tiles * ng < 512) return -1;  // under two steps a workgroup the staged f32 kernel is as fast (5.9 vs 4.5 us at 1024 x 4096)
     static const char *genv = getenv("JQ_Q6K_DOT4_GRID");

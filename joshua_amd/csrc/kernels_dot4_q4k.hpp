@@ -44,7 +44,8 @@ constexpr float QD_RANGE = 32639.0f;  // 127 * 256 + 127
 struct QvQuant {
     uint32_t wl, wh, nl, nh;
     float s;
-    int sum;
+    int sum;   // of the sub-block's 32 values
+    int sum4;  // of the lane's own four
 };
 __device__ __forceinline__ QvQuant qv_quantise4(const float4 v) {
     const uint32_t b0 = __builtin_bit_cast(uint32_t, v.x) & 0x7FFFFFFFu, b1 = __builtin_bit_cast(uint32_t, v.y) & 0x7FFFFFFFu;
@@ -73,7 +74,8 @@ __device__ __forceinline__ QvQuant qv_quantise4(const float4 v) {
     q.nl = __builtin_amdgcn_perm(n23, n01, 0x05040100u) ^ 0x80808080u, q.nh = __builtin_amdgcn_perm(n23, n01, 0x07060302u);
     q.s = s;
     constexpr uint32_t BASE4 = 4u * 0x4B400080u;  // four times the bit pattern of MAGIC, modulo 2^32
-    q.sum = isum_row8((int)(t0 + t1 + t2 + t3 - BASE4));
+    q.sum4 = (int)(t0 + t1 + t2 + t3 - BASE4);
+    q.sum = isum_row8(q.sum4);
     return q;
 }
 

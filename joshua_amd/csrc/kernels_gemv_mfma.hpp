@@ -105,7 +105,7 @@ struct QvQ4K {
     static constexpr int BLOCK = 144, ROW = 16 * BLOCK, ROW_LDS = QD_ROW_LDS;  // rows 16 bytes apart in banks
     static constexpr int STAGE_BYTES = 1184;  // what prepare() uses of `stage`
     static constexpr bool SIDE_LDS = false;
-    static constexpr int COLS = 4096;
+    static constexpr int COLS = 4096, SLOTS = 3;
     typedef QvActs Acts;
     // the activations times f: one factor onto everything that carries the activation scale
     __device__ static __forceinline__ void scale(Acts &a, float f) { a.s_e *= f, a.s_o16 *= f, a.xs_e *= f, a.xs_o *= f; }
@@ -120,6 +120,7 @@ struct QvQ4K {
 struct QvQ4KCompact {
     static constexpr int BLOCK = QvQ4K::BLOCK, ROW = QvQ4K::ROW, ROW_LDS = QvQ4K::ROW_LDS, STAGE_BYTES = QvQ4K::STAGE_BYTES;
     static constexpr bool SIDE_LDS = true;
+    static constexpr int SLOTS = 3;
     struct Acts {
         qv_i4 a_even[2], a_odd[2];
         int c_init2;
@@ -156,7 +157,8 @@ struct Q2Acts {
 struct QvQ2K {
     static constexpr int BLOCK = 84, ROW = 16 * BLOCK, ROW_LDS = ROW + 16;  // 340 words: 16 rows x 4 words fill the 64 banks
     static constexpr int STAGE_BYTES = 640;
-    static constexpr int COLS = 4096;
+    static constexpr int COLS = 4096, SLOTS = 3;
+    static constexpr bool SIDE_LDS = false;
     typedef Q2Acts Acts;
     __device__ static __forceinline__ void scale(Acts &a, float f) {
 #pragma unroll
@@ -235,6 +237,95 @@ struct QvQ2K {
     }
 };
 
+// ---- Q6_K ----
+//
+// Block of 210 bytes: ql[128] | qh[64] | scales[16] (int8) | d; element 128 h + 32 t + l (l < 32) is the low (t < 2) or
+// high nibble of ql[64 h + 32 (t & 1) + l] with bits 2t, 2t + 1 of qh[32 h + l] above it, and the 16 elements
+// 128 h + 32 t + 16 lh + [0, 16) share scales[8 h + 2 t + lh]: w = d sc (q - 32)  (the reference decodes the
+// format through candle's to_float, src/quant_matmul.rs:228-248; layout as in
+// vendor/candle-metal-kernels/src/metal_src/quantized.metal:198-203,6673-6694).
+// Lane (r, c = 2 h + lh) takes the 16 values of l in [16 lh, 16 lh + 16) of half h in all four quarters t: 16
+// bytes of each of ql's two runs and of qh, four MFMAs (one a quarter: B = the sixteen 6-bit values q, 0..63, of
+// one scale group; A row 4c + 2 (t & 1) + plane non-zero in lane group c only, so the quarters (0, 1) share one
+// accumulator and (2, 3) another), and the accumulators start at -32 sum X of the group, which turns sum q X
+// into sum (q - 32) X.  The blocks sit at multiples of 210 bytes: every field is read as aligned words and
+// shifted into place (ldw).
+struct Q6Acts {
+    qv_i4 a[4];     // A operand per quarter
+    qv_i4 init[2];  // accumulator starts of quarters (0, 1) and (2, 3): -32 sum X in the low-plane rows
+    float s[4];     // activation scale of the quarter's 32-element block
+};
+
+struct QvQ6K {
+    static constexpr int BLOCK = 210, ROW = 16 * BLOCK, ROW_LDS = ROW + 16;  // rows 48 bytes apart in a bank row: 8 rows, 8 slots
+    static constexpr int STAGE_BYTES = 640;
+    static constexpr int COLS = 4096, SLOTS = 2;  // a tile is 54 KB: two of them, and one more barrier a tile
+    static constexpr bool SIDE_LDS = false;
+    typedef Q6Acts Acts;
+    __device__ static __forceinline__ void scale(Acts &a, float f) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) a.s[t] *= f;
+    }
+    // stage: words [0,64) Xl, [64,128) Xh, 8 words of zeros, 8 block scales, 16 sums of X per 16 elements
+    __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) {
+        const int r = lane & 15, c = lane >> 4, h = c >> 1, lh = c & 1;
+        float *sf = (float *)(stage + 136);
+        int *xs16 = (int *)(stage + 144);
+        {
+            const QvQuant q = qv_quantise4(v);
+            stage[lane] = q.wl, stage[64 + lane] = q.wh;
+            if (lane < 8) stage[128 + lane] = 0;
+            int s4 = q.sum4;
+            s4 += dpp_i<0xB1>(s4);  // the four lanes of a 16-element group
+            s4 += dpp_i<0x4E>(s4);
+            if ((lane & 7) == 0) sf[lane >> 3] = q.s;
+            if ((lane & 3) == 0) xs16[lane >> 2] = s4;
+        }
+        Acts a;
+        const bool mine = (r >> 2) == c;
+        const int p = (r >> 1) & 1, pl = r & 1;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint32_t *src = mine && p == (t & 1) ? stage + 64 * pl + 32 * h + 8 * t + 4 * lh : stage + 128;
+            const uint4 w = *(const uint4 *)src;
+            a.a[t] = qv_i4{(int)w.x, (int)w.y, (int)w.z, (int)w.w};
+            a.s[t] = sf[4 * h + t];
+        }
+        a.init[0] = qv_i4{-32 * xs16[8 * h + lh], 0, -32 * xs16[8 * h + 2 + lh], 0};
+        a.init[1] = qv_i4{-32 * xs16[8 * h + 4 + lh], 0, -32 * xs16[8 * h + 6 + lh], 0};
+        return a;
+    }
+    __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) {
+        const int h = c >> 1, lh = c & 1;
+        const uint4 qa = ldw<uint4>(blk + 64 * h + 16 * lh), qb = ldw<uint4>(blk + 64 * h + 32 + 16 * lh);
+        const uint4 qh = ldw<uint4>(blk + 128 + 32 * h + 16 * lh);
+        const uint2 sc8 = ldw<uint2>(blk + 192 + 8 * h);
+        const float d = f16_bits(ld<uint16_t>(blk + 208));
+        const uint32_t A[4] = {qa.x, qa.y, qa.z, qa.w}, B[4] = {qb.x, qb.y, qb.z, qb.w}, H[4] = {qh.x, qh.y, qh.z, qh.w};
+        qv_i4 b0, b1, b2, b3;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            b0[j] = (int)((A[j] & 0x0F0F0F0Fu) | ((H[j] << 4) & 0x30303030u));
+            b1[j] = (int)((B[j] & 0x0F0F0F0Fu) | ((H[j] << 2) & 0x30303030u));
+            b2[j] = (int)(((A[j] >> 4) & 0x0F0F0F0Fu) | (H[j] & 0x30303030u));
+            b3[j] = (int)(((B[j] >> 4) & 0x0F0F0F0Fu) | ((H[j] >> 2) & 0x30303030u));
+        }
+        qv_i4 C1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[0], b0, a.init[0], 0, 0, 0);
+        qv_i4 C2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[2], b2, a.init[1], 0, 0, 0);
+        C1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[1], b1, C1, 0, 0, 0);
+        C2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a[3], b3, C2, 0, 0, 0);
+        // the lane's four scale bytes: scales[8 h + 2 t + lh], bytes lh and 2 + lh of each word
+        const int o = 8 * lh;
+        const float s0 = (float)(int8_t)(sc8.x >> o), s1 = (float)(int8_t)(sc8.x >> (16 + o));
+        const float s2 = (float)(int8_t)(sc8.y >> o), s3 = (float)(int8_t)(sc8.y >> (16 + o));
+        float f = s0 * ((float)((C1[1] << 8) + C1[0]) * a.s[0]);
+        f = fmaf(s1, (float)((C1[3] << 8) + C1[2]) * a.s[1], f);
+        f = fmaf(s2, (float)((C2[1] << 8) + C2[0]) * a.s[2], f);
+        f = fmaf(s3, (float)((C2[3] << 8) + C2[2]) * a.s[3], f);
+        return d * f;
+    }
+};
+
 // Work of workgroup b (of G): tiles b, b + G, b + 2 G, ... of 16 rows each; there are rounds G + extra tiles,
 // so the first `extra` workgroups take one more than the others.  The kernels take the four numbers as
 // arguments of their own: scalars among the leading arguments arrive preloaded in registers, a struct is
@@ -277,8 +368,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
                                                       float *__restrict__ Y, int n, int G, int rounds, int extra,
                                                       const float *nm_res, const float *nm_w, float nm_eps,
                                                       float *nm_x_out, float *nm_hn_out) {
-    constexpr int SLOTS = 3, FL = 4;                 // ring slots (two tiles in flight); tiles a flush
-    static_assert(!NORM || 2048 <= F::ROW_LDS, "the norm's operands wait in a wave's row of ring slot 1");
+    constexpr int SLOTS = F::SLOTS, FL = 4;          // ring slots (three: two tiles in flight); tiles a flush
+    static_assert(!NORM || (2048 <= F::ROW_LDS && F::SLOTS == 3), "the norm's operands wait in a wave's row of ring slot 1");
     __shared__ float ss_lds[16];
     constexpr int FULL = F::ROW / 1024, REST = (F::ROW - 1024 * FULL) / 16, LOADS = FULL + (REST ? 1 : 0);
     __shared__ __attribute__((aligned(16))) uint8_t ring[SLOTS][16 * F::ROW_LDS];
@@ -361,8 +452,12 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
             if (b == 0 && nm_hn_out) *(float4 *)(nm_hn_out + 256 * wave + 4 * lane) = float4{v.x * inv, v.y * inv, v.z * inv, v.w * inv};
         }
         part[t & (FL - 1)][r][4 * wave + c] = F::block_dot_lane(&ring[t % SLOTS][r * F::ROW_LDS + wave * F::BLOCK], acts, c);
-        // every wave is done with tile t - 1, whose slot tile t + 2 takes
-        if (t + 2 < nt) fetch(t + 2);
+        // every wave is done with tile t - 1, whose slot tile t + 2 takes; with two slots it takes tile t's own,
+        // once every wave has read it
+        if (t + 2 < nt) {
+            if (SLOTS == 2) __builtin_amdgcn_s_barrier();
+            fetch(t + 2);
+        }
         if ((t & (FL - 1)) == FL - 1 || t == nt - 1) {
             // the partial sums of this group's tiles are written: lane (tt = lane / 16, ww = lane % 16) takes wave
             // ww's four chunk sums of row `wave` in tile tt of the group
@@ -405,12 +500,13 @@ __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict
     static_assert(NG >= 2 && NG <= 4, "two to four passes a row");
     // ring slots (two tiles in flight; a fourth slot only where the staging of four passes needs it) and row
     // tiles a flush
-    constexpr int SLOTS = NG == 4 ? 4 : 3, FL = NG == 4 ? 2 : 4;
+    constexpr int SLOTS = F::SLOTS == 2 ? 2 : (NG == 4 ? 4 : 3), FL = NG == 4 ? 2 : 4;
+    static_assert(SLOTS > 2 || NG <= 3, "two slots: the staging below holds three passes");
     constexpr int LOADS = (F::ROW + 1023) / 1024;
     // the raw activations of the passes wait in the wave's own rows of the last ring slot (behind what prepare()
     // uses), of the one in front of it and of slot 1, which no load targets before the wave itself has prepared
     // its activations and asks for tile 1
-    static_assert(F::STAGE_BYTES + 1024 <= F::ROW_LDS && 2048 <= F::ROW_LDS, "staging in the ring");
+    static_assert(F::STAGE_BYTES + 1024 <= F::ROW_LDS && 2048 <= F::ROW_LDS && (F::SLOTS > 2 || F::STAGE_BYTES + 2048 <= F::ROW_LDS), "staging in the ring");
     __shared__ __attribute__((aligned(16))) uint8_t ring[SLOTS][16 * F::ROW_LDS];
     __shared__ __attribute__((aligned(16))) float part[FL][16][68];  // [row tile][row][4 wave + chunk], as in gemv_mfma_lds
     __shared__ float4 side[F::SIDE_LDS ? 16 * NG * 4 : 1];  // [wave][pass][lane group], for the policies that want it
@@ -436,9 +532,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict
     };
     uint32_t *stage = (uint32_t *)&ring[SLOTS - 1][wave * F::ROW_LDS];
     auto x_raw = [&](int cg) __attribute__((always_inline)) {
+        if (SLOTS == 2)  // two passes behind the staging area in the wave's row of slot 1, a third in the partial sums' memory
+            return cg < 2 ? (float *)((uint8_t *)stage + F::STAGE_BYTES + 1024 * cg) : (float *)&part[0][0][0] + 256 * wave;
         return cg == 0   ? (float *)((uint8_t *)stage + F::STAGE_BYTES)
                : cg == 3 ? (float *)&ring[1][wave * F::ROW_LDS]
-                         : (float *)&ring[SLOTS - 2][wave * F::ROW_LDS + 1024 * (cg - 1)];
+                         : (float *)&ring[SLOTS > 2 ? SLOTS - 2 : 0][wave * F::ROW_LDS + 1024 * (cg - 1)];
     };
 #pragma unroll
     for (int cg = 0; cg < NG; cg++)  // a column past the row's last block reads the last one's and is not used
@@ -467,8 +565,12 @@ __global__ __launch_bounds__(1024) void gemv_mfma_cols(const uint8_t *__restrict
             asm volatile("" ::: "memory");
             if (16 * cg + wave < nb)
                 acc += F::block_dot_lane(&ring[t % SLOTS][r * F::ROW_LDS + wave * F::BLOCK], acts[cg], c);
-            // every wave is done with tile t - 1, whose slot tile t + 2 takes (with four slots: tile t - 2's)
-            if (t + 2 < nt) fetch(t + 2);
+            // every wave is done with tile t - 1, whose slot tile t + 2 takes (with four slots: tile t - 2's; with
+            // two: tile t's own, once every wave has read it)
+            if (t + 2 < nt) {
+                if (SLOTS == 2) __builtin_amdgcn_s_barrier();
+                fetch(t + 2);
+            }
         }
         part[rt & (FL - 1)][r][4 * wave + c] = acc;
         if ((rt & (FL - 1)) == FL - 1 || rt == nrt - 1) {

@@ -478,6 +478,50 @@ def test_q6k_dot4_integer_dot_products_are_bit_exact():
     assert np.array_equal(got[0], want.astype(np.float32))
 
 
+Q6K_MFMA_CHILD = """
+import sys
+import numpy as np
+sys.path.insert(0, %r)
+import oracle
+from joshua_amd import capi, synth
+from tests.test_gpu_matmul import q6k_integer_case, close, make_blocks
+# exact integers: d = 1, random int8 scales per 16 elements, activation scale 1 per 32 elements
+for (n, k, name) in [(300, 4096, "q6k_gemv_mfma_lds"), (1030, 12288, "q6k_gemv_mfma_cols")]:
+    blocks, q, x = q6k_integer_case(n, k, 5, random_scales=True, small=40)
+    want = x @ q.T
+    assert np.abs(want).max() < 2 ** 24
+    got = capi.Weight.upload(capi.Q6_K, blocks, n, k).matmul_t(1, x[None, :].astype(np.float32))
+    assert capi.last_kernel() == name, capi.last_kernel()
+    assert np.array_equal(got[0], want.astype(np.float32)), (n, k)
+# ragged tiles, several tiles a workgroup (the ring of two slots wraps), one to three passes a row
+for (n, k) in [(4096, 4096), (16 * 256 * 3 + 16 * 5 + 7, 4096), (2048 + 77, 8192), (4096, 12288), (1368 + 3, 12288), (257, 12288)]:
+    blocks = make_blocks(capi.Q6_K, n, k, 31)
+    lhs = synth.normal(32 + n %% 7, (1, k))
+    got = capi.Weight.upload(capi.Q6_K, blocks, n, k).matmul_t(1, lhs)
+    assert capi.last_kernel().startswith("q6k_gemv_mfma"), capi.last_kernel()
+    assert close(got, oracle.matmul_t(capi.Q6_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2())), (n, k)
+# a non-finite activation poisons the row, zeros stay zeros
+lhs = synth.normal(9, (1, 4096)); lhs[0, 777] = np.inf
+blocks = make_blocks(capi.Q6_K, 512, 4096, 33)
+assert np.isnan(capi.Weight.upload(capi.Q6_K, blocks, 512, 4096).matmul_t(1, lhs)).all()
+assert np.all(capi.Weight.upload(capi.Q6_K, blocks, 512, 4096).matmul_t(1, np.zeros((1, 4096), np.float32)) == 0.0)
+print("q6k mfma ok")
+"""
+
+
+def test_q6k_matrix_core_gemv_at_every_shape_it_takes():
+    """The Q6_K policy of the int8 matrix-core GEMV serves rows of 8192 and 12288 columns by default;
+    JQ_Q6K_GEMV_MFMA=all sends it every shape it can take (rows of 4096 too, many tiles a workgroup), in a
+    child process because the choice is read once: exact integer sums with random int8 group scales, ragged
+    row counts, non-finite and zero activation rows."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", Q6K_MFMA_CHILD % root], env=dict(os.environ, JQ_Q6K_GEMV_MFMA="all"),
+                         capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0 and "q6k mfma ok" in res.stdout, res.stdout + res.stderr
+
+
 @pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 8 * 600 + 5), (8192, 2048 + 77), (12288, 1368 + 3)])
 def test_q8_0_one_row_over_4096_wide_row_groups(k, n):
     """Q8_0 rows of 4096, 8192 and 12288 with one activation row take the v_dot4 kernel (8-row steps,
@@ -1043,7 +1087,8 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 512, 4096, 1024, "q4k_gemm_i8+splitk"),
     (capi.Q4_K, 128, 4096, 256, "q4k_gemm_mfma+splitk"),    # a small product: the f16 kernel
     (capi.Q8_0, 1, 4096, 4096, "q8_0_gemv_dot4_lds"),
-    (capi.Q6_K, 1, 12288, 4096, "q6k_gemv_dot4_lds"),
+    (capi.Q6_K, 1, 12288, 4096, "q6k_gemv_mfma_cols"),      # a feed-forward down projection
+    (capi.Q6_K, 1, 4096, 4096, "q6k_gemv_dot4_lds"),
     (capi.Q6_K, 1, 1024, 4096, "matmul_rows_staged"),
     (capi.Q6_K, 64, 4096, 1024, "q6k_gemm_i8+splitk"),
     (capi.Q6_K, 64, 2048, 256, "gemm_decoded_mfma+splitk"), # a small product: weights decoded in the workgroup
