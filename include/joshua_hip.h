@@ -290,6 +290,11 @@ typedef struct jq_model jq_model;
 typedef struct {
     uint32_t n_layer, hidden, n_head, n_kv_head, head_dim, ffn, vocab, n_ctx;
     float rms_eps, rope_theta;
+    /* Qwen3-MoE (general.architecture = qwen3moe; reference: src/quantized_qwen3_moe.rs:100-147):
+     * n_expert > 0 makes every layer's feed-forward block a mixture of experts (softmax over all
+     * experts, top n_expert_used, weights divided by their sum when norm_topk_prob), ffn is then
+     * unused and may be 0.  All four zero: the dense model. */
+    uint32_t n_expert, n_expert_used, expert_ffn, norm_topk_prob;
 } jq_qwen3_config;
 
 int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out);
@@ -302,7 +307,11 @@ int jq_qwen3_get_config(const jq_model *model, jq_qwen3_config *out);
  * "blk.3.attn_q.weight", "blk.3.attn_q_norm.weight", "output_norm.weight",
  * "output.weight", ...).  ggml_type 0 is F32 (norm weights); the others are the
  * JQ_TYPE_* ids, uploaded in native block layout.  The expected shape comes
- * from the configuration; a wrong byte count fails. */
+ * from the configuration; a wrong byte count fails.  A mixture-of-experts model
+ * takes "blk.N.ffn_gate_inp.weight" (F32 or F16, [n_expert, hidden]) and the stacked
+ * "blk.N.ffn_{gate,up,down}_exps.weight" ([n_expert, out, in], expert e the e-th
+ * slice; reference: src/quantized_qwen3_moe.rs:556-571, :653-675) in place of the
+ * dense ffn_gate / ffn_up / ffn_down. */
 int jq_qwen3_set_tensor(jq_model *model, const char *name, uint32_t ggml_type, const void *data,
                         size_t nbytes);
 
@@ -371,7 +380,10 @@ int jq_gguf_meta_array_len(const jq_gguf *g, const char *key, size_t *len);
  * src/quantized_qwen3_moe.rs:596-631 split_experts). */
 int jq_gguf_upload(const jq_gguf *g, const char *name, jq_weight **out);
 
-/* Builds the dense Qwen3 decoder from a GGUF file: configuration from the `qwen3.*`
+/* Builds a Qwen3 decoder from a GGUF file, dense (general.architecture = qwen3) or
+ * mixture-of-experts (qwen3moe: expert_count, expert_used_count and
+ * expert_feed_forward_length required, attention.norm_topk_prob defaulting to true,
+ * expert tensors shaped [n_expert, out, in]): configuration from the `<arch>.*`
  * metadata with the reference loader's rules (attention.key_length wins over
  * embedding_length / head_count, rope.freq_base defaults to 10000; reference:
  * src/quantized_qwen3_moe.rs:90-147), every tensor uploaded once; a file without

@@ -64,7 +64,8 @@ class Qwen3Config(ctypes.Structure):
     _fields_ = [("n_layer", ctypes.c_uint32), ("hidden", ctypes.c_uint32), ("n_head", ctypes.c_uint32),
                 ("n_kv_head", ctypes.c_uint32), ("head_dim", ctypes.c_uint32), ("ffn", ctypes.c_uint32),
                 ("vocab", ctypes.c_uint32), ("n_ctx", ctypes.c_uint32), ("rms_eps", ctypes.c_float),
-                ("rope_theta", ctypes.c_float)]
+                ("rope_theta", ctypes.c_float), ("n_expert", ctypes.c_uint32), ("n_expert_used", ctypes.c_uint32),
+                ("expert_ffn", ctypes.c_uint32), ("norm_topk_prob", ctypes.c_uint32)]
 
 
 _lib = None

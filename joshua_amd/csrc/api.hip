@@ -2625,10 +2625,29 @@ struct jq_model {
     float *x2 = nullptr;      // second residual row of a single-token step (the fused norm + matmul launches alternate)
     float *x = nullptr, *hn = nullptr, *qb = nullptr, *kb = nullptr, *vb = nullptr, *att = nullptr, *proj = nullptr,
           *g = nullptr, *u = nullptr, *mid = nullptr, *logits = nullptr;
+    // Mixture-of-experts feed-forward blocks (cfg.n_expert > 0): the routers as they arrived from the host,
+    // one layer object each (built at the first step, rebuilt when a tensor of the layer is replaced), and
+    // the index of the one that currently holds the scratch buffers all of them take turns with.
+    std::map<std::string, std::vector<float>> router_host;
+    std::vector<jq_moe *> moe;
+    int moe_scratch_at = -1;
     std::mutex mu;
 };
 
 namespace {
+
+// Hands the scratch buffers of one layer object to another of the same configuration.  Work on a stream
+// runs in launch order and every kernel got its pointers when it was launched, so the layers of a model
+// can take turns with one set.
+void moe_swap_scratch(jq_moe *a, jq_moe *b) {
+    std::swap(a->cap_tokens, b->cap_tokens);
+    std::swap(a->logits, b->logits), std::swap(a->wts, b->wts), std::swap(a->G, b->G), std::swap(a->U, b->U);
+    std::swap(a->out, b->out), std::swap(a->sG, b->sG), std::swap(a->sU, b->sU), std::swap(a->sH, b->sH);
+    std::swap(a->sOut, b->sOut), std::swap(a->ids, b->ids), std::swap(a->gexp, b->gexp);
+    std::swap(a->offsets, b->offsets), std::swap(a->xrow, b->xrow), std::swap(a->yrow, b->yrow);
+    std::swap(a->qacts, b->qacts), std::swap(a->gacts, b->gacts), std::swap(a->gtab, b->gtab);
+    std::swap(a->gtab_rows, b->gtab_rows), std::swap(a->gtile_rgs, b->gtile_rgs), std::swap(a->qi8, b->qi8);
+}
 
 void model_free_scratch(jq_model *m) {
     for (void *p : {(void *)m->ids, (void *)m->x, (void *)m->x2, (void *)m->hn, (void *)m->qb, (void *)m->kb, (void *)m->vb,
@@ -2680,6 +2699,11 @@ bool qwen3_shape(const jq_qwen3_config &c, const std::string &name, size_t *n, s
     if (ends(".attn_output.weight")) { *n = c.hidden; *k = qd; return true; }
     if (ends(".ffn_gate.weight") || ends(".ffn_up.weight")) { *n = c.ffn; *k = c.hidden; return true; }
     if (ends(".ffn_down.weight")) { *n = c.hidden; *k = c.ffn; return true; }
+    if (c.n_expert) {  // stacked experts, [n_expert, out, in] in the file (reference: src/quantized_qwen3_moe.rs:556-571)
+        if (ends(".ffn_gate_inp.weight")) { *n = (size_t)c.n_expert * c.hidden; *k = 0; return true; }
+        if (ends(".ffn_gate_exps.weight") || ends(".ffn_up_exps.weight")) { *n = (size_t)c.n_expert * c.expert_ffn; *k = c.hidden; return true; }
+        if (ends(".ffn_down_exps.weight")) { *n = (size_t)c.n_expert * c.hidden; *k = c.expert_ffn; return true; }
+    }
     return false;
 }
 
@@ -2746,7 +2770,33 @@ int model_fuse(jq_model *m, const std::string &key, const std::vector<std::strin
     return 0;
 }
 
+// The layer objects of a mixture-of-experts model that are not built yet (all of them at the first step).
+int model_prepare_moe(jq_model *m) {
+    const jq_qwen3_config &c = m->cfg;
+    if (!c.n_expert) return 0;
+    m->moe.resize(c.n_layer, nullptr);
+    for (uint32_t l = 0; l < c.n_layer; l++) {
+        if (m->moe[l]) continue;
+        const std::string p = "blk." + std::to_string(l);
+        auto r = m->router_host.find(p + ".ffn_gate_inp.weight");
+        auto g = m->q.find(p + ".ffn_gate_exps.weight"), u = m->q.find(p + ".ffn_up_exps.weight"),
+             d = m->q.find(p + ".ffn_down_exps.weight");
+        if (r == m->router_host.end()) return fail("qwen3moe: missing tensor `%s.ffn_gate_inp.weight`", p.c_str());
+        for (auto *it : {&g, &u, &d})
+            if (*it == m->q.end()) return fail("qwen3moe: missing an expert tensor of `%s`", p.c_str());
+        // softmax over all experts, top k, weights divided by their sum when norm_topk_prob
+        // (reference: src/quantized_qwen3_moe.rs:424-436)
+        jq_moe_config mc{};
+        mc.n_expert = c.n_expert, mc.n_expert_used = c.n_expert_used, mc.hidden = c.hidden, mc.inter = c.expert_ffn;
+        mc.gating = 0, mc.norm_topk = c.norm_topk_prob ? 1 : 0;
+        if (jq_moe_create(&mc, r->second.data(), nullptr, g->second, u->second, d->second, nullptr, nullptr, nullptr, &m->moe[l]))
+            return 1;
+    }
+    return 0;
+}
+
 int model_prepare_fused(jq_model *m) {
+    if (model_prepare_moe(m)) return 1;
     if (m->fused_ready) return 0;
     const jq_qwen3_config &c = m->cfg;
     for (uint32_t l = 0; l < c.n_layer; l++) {
@@ -2760,7 +2810,7 @@ int model_prepare_fused(jq_model *m) {
                                   : std::vector<std::string>{p + ".attn_q.weight", p + ".attn_k.weight"}))
                 return 1;
         }
-        if (!m->fused.count(p + ".gate_up")) {
+        if (!c.n_expert && !m->fused.count(p + ".gate_up")) {
             // 4096-wide Q4_K rows: paired, for the launch that also applies SwiGLU
             auto g = m->q.find(p + ".ffn_gate.weight");
             const bool pair = g != m->q.end() && g->second->type == JQ_TYPE_Q4_K && g->second->k == 4096 &&
@@ -2881,6 +2931,17 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
 #undef JQ_ATT_TILES
         }
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
+        if (c.n_expert) {
+            // x + moe(norm(x)) (reference: src/quantized_qwen3_moe.rs:806-812)
+            hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, m->proj, w_fn, c.rms_eps, m->hn, h);
+            jq_moe *moe = m->moe[l];
+            if (m->moe_scratch_at >= 0 && m->moe_scratch_at != (int)l && m->moe[m->moe_scratch_at])
+                moe_swap_scratch(moe, m->moe[m->moe_scratch_at]);
+            m->moe_scratch_at = (int)l;
+            if (jq_moe_forward(moe, T, m->hn, m->proj, 1, s)) return 1;
+            pending = m->proj;
+            continue;
+        }
         const float *gp = m->g, *up = m->u;
         auto fg = T == 1 ? m->fused.find(p + ".gate_up") : m->fused.end();
         const bool paired = fg != m->fused.end() && m->paired.count(fg->first);  // gate and up rows alternate
@@ -2958,8 +3019,13 @@ int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out) {
     *out = nullptr;
     if (!cfg) return fail("jq_qwen3_create: cfg is null");
     const jq_qwen3_config &c = *cfg;
-    if (!c.n_layer || !c.hidden || !c.n_head || !c.n_kv_head || !c.head_dim || !c.ffn || !c.vocab || !c.n_ctx)
+    if (!c.n_layer || !c.hidden || !c.n_head || !c.n_kv_head || !c.head_dim || !c.vocab || !c.n_ctx ||
+        (!c.ffn && !c.n_expert))
         return fail("qwen3: zero in configuration");
+    // reference: src/quantized_qwen3_moe.rs:122-129
+    if (c.n_expert && (c.n_expert_used == 0 || c.n_expert_used > c.n_expert))
+        return fail("qwen3moe: expert_used_count %u must be in 1..=expert_count %u", c.n_expert_used, c.n_expert);
+    if (c.n_expert && c.expert_ffn == 0) return fail("qwen3moe: expert_feed_forward_length must be positive");
     if (c.n_head % c.n_kv_head != 0) return fail("qwen3: %u query heads over %u kv heads", c.n_head, c.n_kv_head);
     if (c.head_dim % 8 != 0 || c.hidden % 4 != 0 || c.ffn % 4 != 0) return fail("qwen3: dimensions must be multiples of 4/8");
     if (c.head_dim > (uint32_t)jq::AR_MAX_D) return fail("qwen3: head_dim %u exceeds %d", c.head_dim, jq::AR_MAX_D);
@@ -2995,6 +3061,7 @@ int jq_qwen3_create(const jq_qwen3_config *cfg, jq_model **out) {
 void jq_qwen3_free(jq_model *m) {
     if (!m) return;
     model_free_scratch(m);
+    for (jq_moe *e : m->moe) jq_moe_free(e);
     for (auto &kv : m->q) jq_free(kv.second);
     for (auto &kv : m->fused) jq_free(kv.second);
     for (auto *w : m->retired) jq_free(w);
@@ -3017,6 +3084,38 @@ int jq_qwen3_set_tensor(jq_model *m, const char *name, uint32_t ggml_type, const
     size_t n, k;
     if (!qwen3_shape(m->cfg, name, &n, &k)) return fail("qwen3: unknown tensor `%s`", name);
     std::lock_guard<std::mutex> lock(m->mu);
+    const std::string nm = name;
+    const size_t dot = nm.find('.', 4);
+    const bool in_layer = nm.rfind("blk.", 0) == 0 && dot != std::string::npos;
+    const std::string role = in_layer ? nm.substr(dot) : std::string();
+    if (role == ".ffn_gate_inp.weight" || role == ".ffn_gate_exps.weight" || role == ".ffn_up_exps.weight" ||
+        role == ".ffn_down_exps.weight") {
+        // the layer object is rebuilt from the new tensors at the next step
+        const size_t l = (size_t)atoll(nm.c_str() + 4);
+        if (l < m->moe.size() && m->moe[l]) {
+            if (m->moe_scratch_at == (int)l) m->moe_scratch_at = -1;  // its scratch goes with it
+            jq_moe_free(m->moe[l]);
+            m->moe[l] = nullptr;
+        }
+    }
+    if (role == ".ffn_gate_inp.weight") {
+        // the router is read as f32 whatever the file holds (reference: src/quantized_qwen3_moe.rs:197-199, :654-657)
+        std::vector<float> host(n);
+        if (ggml_type == 0 && nbytes == n * sizeof(float)) {
+            memcpy(host.data(), data, nbytes);
+        } else if (ggml_type == 1 && nbytes == n * sizeof(uint16_t)) {
+            const uint16_t *hsrc = (const uint16_t *)data;
+            for (size_t i = 0; i < n; i++) {
+                _Float16 hv;
+                memcpy(&hv, hsrc + i, sizeof hv);
+                host[i] = (float)hv;
+            }
+        } else {
+            return fail("qwen3moe: `%s` must be F32 or F16 with %zu values (type %u, %zu bytes)", name, n, ggml_type, nbytes);
+        }
+        m->router_host[nm] = std::move(host);
+        return 0;
+    }
     if (k == 0) {
         if (ggml_type != 0) return fail("qwen3: `%s` must be F32", name);
         if (nbytes != n * sizeof(float)) return fail("qwen3: `%s` holds %zu bytes, expected %zu", name, nbytes, n * sizeof(float));
@@ -3039,10 +3138,8 @@ int jq_qwen3_set_tensor(jq_model *m, const char *name, uint32_t ggml_type, const
     m->q[name] = w;
     // a replaced part: the fused copy it belonged to is retired (the other parts' views keep pointing
     // into it) and that group runs as separate launches from now on
-    const std::string nm = name;
-    const size_t dot = nm.find('.', 4);
-    if (nm.rfind("blk.", 0) == 0 && dot != std::string::npos) {
-        const std::string layer = nm.substr(0, dot), role = nm.substr(dot);
+    if (in_layer) {
+        const std::string layer = nm.substr(0, dot);
         const char *key = (role == ".attn_q.weight" || role == ".attn_k.weight" || role == ".attn_v.weight") ? ".qkv"
                           : (role == ".ffn_gate.weight" || role == ".ffn_up.weight")                         ? ".gate_up"
                                                                                                              : nullptr;
@@ -3129,12 +3226,17 @@ int gguf_wrap(std::unique_ptr<jq::Gguf> g, const std::string &err, jq_gguf **out
 // Every tensor the graph reads is installed, or the name of the first one that is not.
 int model_check_complete(jq_model *m) {
     std::vector<std::string> names = {"token_embd.weight", "output_norm.weight", "output.weight"};
-    for (uint32_t l = 0; l < m->cfg.n_layer; l++)
-        for (const char *role : {"attn_norm", "attn_q", "attn_k", "attn_v", "attn_q_norm", "attn_k_norm", "attn_output",
-                                 "ffn_norm", "ffn_gate", "ffn_up", "ffn_down"})
+    const bool moe = m->cfg.n_expert != 0;
+    for (uint32_t l = 0; l < m->cfg.n_layer; l++) {
+        for (const char *role : {"attn_norm", "attn_q", "attn_k", "attn_v", "attn_q_norm", "attn_k_norm", "attn_output", "ffn_norm"})
             names.push_back("blk." + std::to_string(l) + "." + role + ".weight");
+        for (const char *role : {moe ? "ffn_gate_inp" : "ffn_gate", moe ? "ffn_gate_exps" : "ffn_up", moe ? "ffn_up_exps" : "ffn_down"})
+            names.push_back("blk." + std::to_string(l) + "." + role + ".weight");
+        if (moe) names.push_back("blk." + std::to_string(l) + ".ffn_down_exps.weight");
+    }
     for (const auto &nm : names)
-        if (!m->q.count(nm) && !m->f.count(nm)) return fail("qwen3: missing tensor `%s`", nm.c_str());
+        if (!m->q.count(nm) && !m->f.count(nm) && !m->router_host.count(nm))
+            return fail("%s: missing tensor `%s`", moe ? "qwen3moe" : "qwen3", nm.c_str());
     return 0;
 }
 
@@ -3144,31 +3246,46 @@ int model_check_complete(jq_model *m) {
 // of head_count_kv, head_dim must be positive and even.
 int qwen3_config_from_gguf(const jq::Gguf &g, uint32_t n_ctx, jq_qwen3_config *c) {
     const std::string *arch = g.meta_str("general.architecture");
-    if (!arch || *arch != "qwen3")
-        return fail("qwen3: general.architecture is `%s`, expected `qwen3`", arch ? arch->c_str() : "(missing)");
+    if (!arch || (*arch != "qwen3" && *arch != "qwen3moe"))
+        return fail("qwen3: general.architecture is `%s`, expected `qwen3` or `qwen3moe`", arch ? arch->c_str() : "(missing)");
+    const std::string a = *arch;
+    const bool moe = a == "qwen3moe";
     auto need_u32 = [&](const char *key, uint32_t *v) {
-        if (g.meta_u32(std::string("qwen3.") + key, v)) return 0;
-        return fail("qwen3: missing GGUF metadata key `qwen3.%s`", key);
+        if (g.meta_u32(a + "." + key, v)) return 0;
+        return fail("%s: missing GGUF metadata key `%s.%s`", a.c_str(), a.c_str(), key);
     };
     uint32_t context_length = 0, key_length = 0;
     if (need_u32("attention.head_count", &c->n_head) || need_u32("attention.head_count_kv", &c->n_kv_head) ||
         need_u32("block_count", &c->n_layer) || need_u32("embedding_length", &c->hidden) ||
         need_u32("context_length", &context_length))
         return 1;
-    if (!g.meta_f32("qwen3.attention.layer_norm_rms_epsilon", &c->rms_eps))
-        return fail("qwen3: missing GGUF metadata key `qwen3.attention.layer_norm_rms_epsilon`");
-    if (c->n_head == 0) return fail("qwen3: head_count is zero");
-    c->head_dim = g.meta_u32("qwen3.attention.key_length", &key_length) ? key_length : c->hidden / c->n_head;
+    if (!g.meta_f32(a + ".attention.layer_norm_rms_epsilon", &c->rms_eps))
+        return fail("%s: missing GGUF metadata key `%s.attention.layer_norm_rms_epsilon`", a.c_str(), a.c_str());
+    if (c->n_head == 0) return fail("%s: head_count is zero", a.c_str());
+    c->head_dim = g.meta_u32(a + ".attention.key_length", &key_length) ? key_length : c->hidden / c->n_head;
     if (c->head_dim == 0 || c->head_dim % 2 != 0)
-        return fail("qwen3: invalid head_dim %u (must be a positive even number)", c->head_dim);
+        return fail("%s: invalid head_dim %u (must be a positive even number)", a.c_str(), c->head_dim);
     if (c->n_kv_head == 0 || c->n_head % c->n_kv_head != 0)
-        return fail("qwen3: head_count %u must be a multiple of head_count_kv %u", c->n_head, c->n_kv_head);
-    if (!g.meta_f32("qwen3.rope.freq_base", &c->rope_theta)) c->rope_theta = 10000.0f;
+        return fail("%s: head_count %u must be a multiple of head_count_kv %u", a.c_str(), c->n_head, c->n_kv_head);
+    if (!g.meta_f32(a + ".rope.freq_base", &c->rope_theta)) c->rope_theta = 10000.0f;
+    if (moe) {
+        // reference: src/quantized_qwen3_moe.rs:119-134 (every layer's feed-forward block is a mixture of experts)
+        if (need_u32("expert_count", &c->n_expert) || need_u32("expert_used_count", &c->n_expert_used) ||
+            need_u32("expert_feed_forward_length", &c->expert_ffn))
+            return 1;
+        if (c->n_expert_used == 0 || c->n_expert_used > c->n_expert)
+            return fail("qwen3moe: expert_used_count %u must be in 1..=expert_count %u", c->n_expert_used, c->n_expert);
+        if (c->expert_ffn == 0) return fail("qwen3moe: expert_feed_forward_length must be positive");
+        bool norm = true;
+        if (!g.meta_bool("qwen3moe.attention.norm_topk_prob", &norm)) norm = true;
+        c->norm_topk_prob = norm ? 1 : 0;
+        c->ffn = 0;
+    }
     // the two sizes the metadata may leave out are read off the tensors
     const jq::GgufTensor *emb = g.tensor("token_embd.weight");
     if (!emb || emb->dims.size() != 2) return fail("qwen3: missing tensor `token_embd.weight`");
     c->vocab = (uint32_t)emb->dims[0];
-    if (!g.meta_u32("qwen3.feed_forward_length", &c->ffn)) {
+    if (!moe && !g.meta_u32("qwen3.feed_forward_length", &c->ffn)) {
         const jq::GgufTensor *gate = g.tensor("blk.0.ffn_gate.weight");
         if (!gate || gate->dims.size() != 2) return fail("qwen3: missing GGUF metadata key `qwen3.feed_forward_length`");
         c->ffn = (uint32_t)gate->dims[0];
@@ -3321,8 +3438,18 @@ int jq_qwen3_load_gguf(const char *path, uint32_t n_ctx, jq_model **out) {
             jq_qwen3_free(m);
             return fail("GGUF: %s", err.c_str());
         }
-        const bool shape_ok = k == 0 ? (t.dims.size() == 1 && t.dims[0] == n)
-                                     : (t.dims.size() == 2 && t.dims[0] == n && t.dims[1] == k);
+        bool shape_ok = k == 0 ? (t.dims.size() == 1 && t.dims[0] == n)
+                               : (t.dims.size() == 2 && t.dims[0] == n && t.dims[1] == k);
+        const bool router = t.name.size() > 20 && t.name.compare(t.name.size() - 20, 20, ".ffn_gate_inp.weight") == 0;
+        const bool stacked = t.name.find("_exps.weight") != std::string::npos;
+        if (router) shape_ok = t.dims.size() == 2 && t.dims[0] == cfg.n_expert && t.dims[1] == cfg.hidden;
+        if (stacked) {
+            if (t.dims.size() != 3 || t.dims[0] != cfg.n_expert) {
+                jq_qwen3_free(m);
+                return fail("qwen3moe: expected expert tensor `%s` shaped [n_expert, out, in]", t.name.c_str());
+            }
+            shape_ok = t.dims[0] * t.dims[1] == n && t.dims[2] == k;
+        }
         if (!shape_ok) {
             jq_qwen3_free(m);
             return fail("qwen3: tensor `%s` does not have the shape the metadata implies", t.name.c_str());

@@ -99,26 +99,36 @@ def write_gguf(path: str, metadata: dict, tensors: list, alignment: "int | None"
     return where
 
 
-def qwen3_metadata(cfg: dict, with_key_length: bool = True, with_ffn: bool = True) -> dict:
-    """The `qwen3.*` keys a dense Qwen3 file carries (read by the loader at
-    reference: src/quantized_qwen3_moe.rs:90-147, there under the `qwen3moe.` prefix)."""
-    md = {"general.architecture": string("qwen3"), "general.name": string("synthetic-qwen3"),
-          "qwen3.block_count": u32(cfg["n_layer"]), "qwen3.embedding_length": u32(cfg["hidden"]),
-          "qwen3.attention.head_count": u32(cfg["n_head"]), "qwen3.attention.head_count_kv": u32(cfg["n_kv_head"]),
-          "qwen3.context_length": u32(cfg.get("context_length", cfg["n_ctx"])),
-          "qwen3.attention.layer_norm_rms_epsilon": f32(cfg["rms_eps"]), "qwen3.rope.freq_base": f32(cfg["rope_theta"])}
+def qwen3_metadata(cfg: dict, with_key_length: bool = True, with_ffn: bool = True, with_norm_topk=None) -> dict:
+    """The `qwen3.*` keys a dense Qwen3 file carries, or with n_expert in the configuration the
+    `qwen3moe.*` keys of a mixture-of-experts one (read by the loader at
+    reference: src/quantized_qwen3_moe.rs:90-147).  with_norm_topk: True / False writes
+    attention.norm_topk_prob, None leaves it out (the loader then takes true)."""
+    a = "qwen3moe" if cfg.get("n_expert") else "qwen3"
+    md = {"general.architecture": string(a), "general.name": string("synthetic-" + a),
+          a + ".block_count": u32(cfg["n_layer"]), a + ".embedding_length": u32(cfg["hidden"]),
+          a + ".attention.head_count": u32(cfg["n_head"]), a + ".attention.head_count_kv": u32(cfg["n_kv_head"]),
+          a + ".context_length": u32(cfg.get("context_length", cfg["n_ctx"])),
+          a + ".attention.layer_norm_rms_epsilon": f32(cfg["rms_eps"]), a + ".rope.freq_base": f32(cfg["rope_theta"])}
     if with_key_length:
-        md["qwen3.attention.key_length"] = u32(cfg["head_dim"])
-        md["qwen3.attention.value_length"] = u32(cfg["head_dim"])
-    if with_ffn:
-        md["qwen3.feed_forward_length"] = u32(cfg["ffn"])
+        md[a + ".attention.key_length"] = u32(cfg["head_dim"])
+        md[a + ".attention.value_length"] = u32(cfg["head_dim"])
+    if cfg.get("n_expert"):
+        md[a + ".expert_count"] = u32(cfg["n_expert"])
+        md[a + ".expert_used_count"] = u32(cfg["n_expert_used"])
+        md[a + ".expert_feed_forward_length"] = u32(cfg["expert_ffn"])
+        if with_norm_topk is not None:
+            md[a + ".attention.norm_topk_prob"] = boolean(bool(with_norm_topk))
+    elif with_ffn:
+        md[a + ".feed_forward_length"] = u32(cfg["ffn"])
     return md
 
 
 def write_qwen3(path: str, cfg: dict, tensors, plan, **kw) -> dict:
     """tensors: iterable of (name, qtype, data) as qwen3_tensors yields; plan: qwen3_tensor_plan
     of the same configuration (for the shapes)."""
-    shapes = {name: ([n] if k == 0 else [n, k]) for name, _, n, k in plan}
+    from .model import gguf_dims
+    shapes = {name: gguf_dims(cfg, name, n, k) for name, _, n, k in plan}
     items = [(name, qt, shapes[name], data) for name, qt, data in tensors]
-    md_kw = {k: kw.pop(k) for k in ("with_key_length", "with_ffn") if k in kw}
+    md_kw = {k: kw.pop(k) for k in ("with_key_length", "with_ffn", "with_norm_topk") if k in kw}
     return write_gguf(path, qwen3_metadata(cfg, **md_kw), items, **kw)

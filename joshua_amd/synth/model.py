@@ -22,8 +22,11 @@ def more_bits(layer: int, n_layer: int) -> bool:
 
 
 def qwen3_tensor_plan(cfg: dict, mix: str = "q4_k_m"):
-    """[(name, qtype, n, k)] for every tensor of the model; k == 0 marks an f32 vector."""
-    h, d, ffn = cfg["hidden"], cfg["head_dim"], cfg["ffn"]
+    """[(name, qtype, n, k)] for every tensor of the model; k == 0 marks an f32 vector.  With n_expert in
+    the configuration the feed-forward tensors are those of a qwen3moe file: the f32 router
+    ffn_gate_inp of n_expert * hidden values and the stacked ffn_{gate,up,down}_exps, expert after expert."""
+    h, d, ffn = cfg["hidden"], cfg["head_dim"], cfg.get("ffn", 0)
+    E, eff = cfg.get("n_expert", 0), cfg.get("expert_ffn", 0)
     qd, kd, L = cfg["n_head"] * d, cfg["n_kv_head"] * d, cfg["n_layer"]
     base = Q4_K if mix in ("q4_k_m", "q4_k") else int(mix)
     plan = [("token_embd.weight", base, cfg["vocab"], h), ("output_norm.weight", F32, h, 0),
@@ -34,10 +37,25 @@ def qwen3_tensor_plan(cfg: dict, mix: str = "q4_k_m"):
         plan += [(p + "attn_norm.weight", F32, h, 0), (p + "attn_q.weight", base, qd, h),
                  (p + "attn_k.weight", base, kd, h), (p + "attn_v.weight", hi, kd, h),
                  (p + "attn_q_norm.weight", F32, d, 0), (p + "attn_k_norm.weight", F32, d, 0),
-                 (p + "attn_output.weight", base, h, qd), (p + "ffn_norm.weight", F32, h, 0),
-                 (p + "ffn_gate.weight", base, ffn, h), (p + "ffn_up.weight", base, ffn, h),
-                 (p + "ffn_down.weight", hi, h, ffn)]
+                 (p + "attn_output.weight", base, h, qd), (p + "ffn_norm.weight", F32, h, 0)]
+        if E:
+            plan += [(p + "ffn_gate_inp.weight", F32, E * h, 0), (p + "ffn_gate_exps.weight", base, E * eff, h),
+                     (p + "ffn_up_exps.weight", base, E * eff, h), (p + "ffn_down_exps.weight", hi, E * h, eff)]
+        else:
+            plan += [(p + "ffn_gate.weight", base, ffn, h), (p + "ffn_up.weight", base, ffn, h),
+                     (p + "ffn_down.weight", hi, h, ffn)]
     return plan
+
+
+def gguf_dims(cfg: dict, name: str, n: int, k: int) -> list:
+    """The shape a GGUF directory gives the tensor, slowest dimension first: [n] for vectors, [n, k] for
+    matrices, [n_expert, hidden] for the router and [n_expert, out, in] for stacked experts."""
+    E = cfg.get("n_expert", 0)
+    if name.endswith(".ffn_gate_inp.weight"):
+        return [E, n // E]
+    if name.endswith("_exps.weight"):
+        return [E, n // E, k]
+    return [n] if k == 0 else [n, k]
 
 
 def qwen3_tensors(cfg: dict, seed: int, mix: str = "q4_k_m", share_layers: bool = False):
@@ -50,7 +68,9 @@ def qwen3_tensors(cfg: dict, seed: int, mix: str = "q4_k_m", share_layers: bool 
         key = (role, qt, n, k) if share_layers else (name,)
         if key not in cache:
             s = seed * 1000003 + (zlib.crc32(role.encode()) % 1000 if share_layers else i)
-            if k == 0:
+            if name.endswith(".ffn_gate_inp.weight"):   # router rows: logits of standard deviation ~1 on a normed row
+                cache[key] = normal(s, (n,), float(1.0 / np.sqrt(cfg["hidden"])), 0.0)
+            elif k == 0:
                 cache[key] = normal(s, (n,), 0.1, 1.0)
             else:
                 cache[key] = normal_quantized(qt, s, n * k, float(1.0 / np.sqrt(k)))

@@ -30,8 +30,9 @@ def topk_indices(v: np.ndarray, k: int) -> np.ndarray:
 class MoeOracle:
     def __init__(self, qtype, h, inter, n_expert, k_used, router_w, gate, up, down, *, gating="softmax",
                  norm_topk=True, weights_scale=0.0, n_group=1, topk_group=1, router_bias=None, shared=None,
-                 avx2=False, swiglu_clamp=0.0, swiglu_clamp_shared=0.0):
+                 avx2=False, swiglu_clamp=0.0, swiglu_clamp_shared=0.0, qtype_down=None):
         self.qtype, self.h, self.inter, self.E, self.k = qtype, h, inter, n_expert, k_used
+        self.qtype_down = qtype if qtype_down is None else qtype_down   # ffn_down_exps may hold more bits
         self.router_w = np.asarray(router_w, np.float32)          # [E, h]
         self.gate, self.up, self.down = gate, up, down            # stacked block bytes
         self.gating, self.norm_topk, self.scale = gating, norm_topk, np.float32(weights_scale)
@@ -96,7 +97,7 @@ class MoeOracle:
         u = matmul_t(self.qtype, (m, self.h, self.inter), x, self._slice(self.up, e), avx2=self.avx2)
         g, u = self.clamped(g, u, self.clamp)
         hid = (silu(g) * u).astype(np.float32)
-        return matmul_t(self.qtype, (m, self.inter, self.h), hid, self._slice(self.down, e), avx2=self.avx2).copy()
+        return matmul_t(self.qtype_down, (m, self.inter, self.h), hid, self._slice(self.down, e), avx2=self.avx2).copy()
 
     def shared_mlp(self, x: np.ndarray) -> np.ndarray:
         qt, si, g, u, d = self.shared

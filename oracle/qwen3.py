@@ -1,10 +1,12 @@
-"""CPU restatement of the reference's dense Qwen3 decoder graph on top of the
-oracle matmul.  TEST INFRASTRUCTURE (see oracle/__init__.py).
+"""CPU restatement of the reference's Qwen3 decoder graph, dense or with
+mixture-of-experts feed-forward blocks, on top of the oracle matmul.  TEST INFRASTRUCTURE (see oracle/__init__.py).
 
 Layer structure follows src/embedding.rs:297-396 (pre-norm residual blocks,
 per-head Q/K RMSNorm before RoPE, half-split rotary pairs, grouped-query
 attention, SwiGLU MLP); KV cache, causal mask and last-token logits follow
-src/quantized_qwen3_moe.rs:366-386,776-826.  RMSNorm, softmax, silu, the f32
+src/quantized_qwen3_moe.rs:366-386,776-826; with n_expert in the configuration
+every layer's feed-forward block is the mixture of experts of :404-528, 806-812
+(oracle/moe.py).  RMSNorm, softmax, silu, the f32
 attention matmuls and cos/sin are third-party candle ops: their formulas are
 public, their ulp-level rounding order is not pinned by anything in the
 reference, so comparisons against this file use a relative bound on the logits
@@ -17,7 +19,7 @@ import time
 import numpy as np
 
 from . import dequantize, matmul_t
-from .moe import silu
+from .moe import MoeOracle, silu
 
 f32 = np.float32
 
@@ -61,10 +63,13 @@ def gqa_attention(q: np.ndarray, K: np.ndarray, V: np.ndarray, pos: int) -> np.n
 
 class Qwen3Oracle:
     """cfg: dict with n_layer, hidden, n_head, n_kv_head, head_dim, ffn, vocab, rms_eps,
-    rope_theta.  tensors: name -> (qtype, data) with qtype 0 for f32 vectors."""
+    rope_theta; a mixture-of-experts model adds n_expert, n_expert_used, expert_ffn and
+    norm_topk_prob (default True).  tensors: name -> (qtype, data) with qtype 0 for f32
+    vectors and the router."""
 
     def __init__(self, cfg: dict, tensors: dict, *, avx2: bool = True, threads: int = 0):
         self.c, self.t, self.avx2, self.threads = cfg, tensors, avx2, threads
+        self._moe: dict = {}
         self.reset()
 
     def reset(self) -> None:
@@ -80,6 +85,21 @@ class Qwen3Oracle:
         y = matmul_t(qt, (m, k, n), np.ascontiguousarray(x, f32), blocks, avx2=self.avx2, threads=self.threads)
         self.mm_seconds += time.perf_counter() - t0
         return y
+
+    def moe(self, l: int) -> MoeOracle:
+        """The layer's expert block from its four tensors (src/quantized_qwen3_moe.rs:653-675)."""
+        if l not in self._moe:
+            c, p = self.c, f"blk.{l}."
+            as_bytes = lambda name: np.frombuffer(bytes(self.t[name][1]), np.uint8) if not isinstance(
+                self.t[name][1], np.ndarray) else self.t[name][1].view(np.uint8).ravel()
+            qg, qu, qd = (self.t[p + f"ffn_{r}_exps.weight"][0] for r in ("gate", "up", "down"))
+            assert qg == qu
+            router = np.asarray(self.t[p + "ffn_gate_inp.weight"][1], f32).reshape(c["n_expert"], c["hidden"])
+            self._moe[l] = MoeOracle(qg, c["hidden"], c["expert_ffn"], c["n_expert"], c["n_expert_used"], router,
+                                     as_bytes(p + "ffn_gate_exps.weight"), as_bytes(p + "ffn_up_exps.weight"),
+                                     as_bytes(p + "ffn_down_exps.weight"), gating="softmax",
+                                     norm_topk=bool(c.get("norm_topk_prob", True)), avx2=self.avx2, qtype_down=qd)
+        return self._moe[l]
 
     def vec(self, name: str) -> np.ndarray:
         return np.asarray(self.t[name][1], f32)
@@ -111,6 +131,9 @@ class Qwen3Oracle:
             att = gqa_attention(q, self.k[l], self.v[l], pos)
             x = (x + self.mm(p + ".attn_output.weight", att.reshape(T, nh * d), h)).astype(f32)
             hn = rmsnorm(x, self.vec(p + ".ffn_norm.weight"), c["rms_eps"])
+            if c.get("n_expert"):
+                x = (x + self.moe(l).forward(hn)).astype(f32)
+                continue
             g = self.mm(p + ".ffn_gate.weight", hn, c["ffn"])
             u = self.mm(p + ".ffn_up.weight", hn, c["ffn"])
             x = (x + self.mm(p + ".ffn_down.weight", (silu(g) * u).astype(f32), h)).astype(f32)

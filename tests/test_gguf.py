@@ -281,3 +281,26 @@ def test_plugin_entry_points_reject_null_and_unloadable_models(tmp_path):
     missing.write_bytes(gw.header_bytes({"general.architecture": gw.string("qwen3")}, []))
     p = capi.NpuPlugin(str(missing), 16)
     assert p.rc == -2 and "missing GGUF metadata key `qwen3.attention.head_count`" in capi.last_error()
+
+
+def test_qwen3moe_metadata_is_checked_before_any_device_call(tmp_path):
+    """The expert keys of a qwen3moe file and their ranges (reference: src/quantized_qwen3_moe.rs:119-129)."""
+    cfg = dict(n_layer=1, hidden=256, n_head=2, n_kv_head=1, head_dim=64, vocab=64, n_ctx=8, rms_eps=1e-6, rope_theta=1e4,
+               n_expert=4, n_expert_used=2, expert_ffn=128)
+    emb = []
+
+    def attempt(name, md, expect):
+        f = tmp_path / name
+        f.write_bytes(gw.header_bytes(md, emb))
+        p = capi.NpuPlugin(str(f), 8)
+        assert p.rc == -2 and expect in capi.last_error(), capi.last_error()
+
+    md = gw.qwen3_metadata(cfg)
+    assert md["general.architecture"].value == "qwen3moe" and "qwen3moe.attention.norm_topk_prob" not in md
+    for key in ("expert_count", "expert_used_count", "expert_feed_forward_length"):
+        attempt(key + ".gguf", {k: v for k, v in md.items() if k != "qwen3moe." + key},
+                f"missing GGUF metadata key `qwen3moe.{key}`")
+    attempt("used0.gguf", gw.qwen3_metadata(dict(cfg, n_expert_used=0)), "expert_used_count 0 must be in 1..=expert_count 4")
+    attempt("used5.gguf", gw.qwen3_metadata(dict(cfg, n_expert_used=5)), "expert_used_count 5 must be in 1..=expert_count 4")
+    attempt("ff0.gguf", gw.qwen3_metadata(dict(cfg, expert_ffn=0)), "expert_feed_forward_length must be positive")
+    attempt("heads.gguf", gw.qwen3_metadata(dict(cfg, n_kv_head=3)), "must be a multiple of head_count_kv")

@@ -206,3 +206,74 @@ def test_forward_equals_an_independent_f64_graph_over_decoded_weights():
     want = norm(x[-1:], vec("output_norm.weight")) @ W("output.weight", cfg["vocab"], h).T
     scale = np.abs(want).max()
     assert np.abs(got - want[0]).max() <= 1e-3 * scale
+
+
+MOE = dict(CFG, ffn=0, n_expert=4, n_expert_used=2, expert_ffn=256)
+
+
+def test_moe_plan_and_gguf_shapes():
+    from joshua_amd.synth.model import gguf_dims
+    plan = {n: (qt, a, b) for n, qt, a, b in qwen3_tensor_plan(MOE)}
+    assert "blk.0.ffn_gate.weight" not in plan
+    assert plan["blk.0.ffn_gate_inp.weight"] == (0, 4 * 256, 0)
+    assert plan["blk.1.ffn_up_exps.weight"] == (12, 4 * 256, 256) and plan["blk.1.ffn_down_exps.weight"][1:] == (4 * 256, 256)
+    assert gguf_dims(MOE, "blk.0.ffn_gate_inp.weight", 1024, 0) == [4, 256]
+    assert gguf_dims(MOE, "blk.0.ffn_down_exps.weight", 1024, 256) == [4, 256, 256]
+    assert gguf_dims(MOE, "blk.0.attn_q.weight", 256, 256) == [256, 256] and gguf_dims(MOE, "output_norm.weight", 256, 0) == [256]
+
+
+def test_a_single_expert_model_is_the_dense_model():
+    """With one expert, used always and its weight normalised to 1, x + moe(norm(x)) is the dense block on
+    the same three matrices: the expert wiring of the graph against the dense graph pinned above."""
+    one = dict(CFG, ffn=0, n_expert=1, n_expert_used=1, expert_ffn=CFG["ffn"])
+    dense = {n: (qt, d) for n, qt, d in qwen3_tensors(CFG, 21)}
+    moe = {}
+    for name, v in dense.items():
+        for role in ("gate", "up", "down"):
+            if name.endswith(f".ffn_{role}.weight"):
+                name = name.replace(f".ffn_{role}.weight", f".ffn_{role}_exps.weight")
+        moe[name] = v
+    for l in range(CFG["n_layer"]):
+        moe[f"blk.{l}.ffn_gate_inp.weight"] = (0, normal(30 + l, (CFG["hidden"],)))
+    toks = [7, 300, 12, 12, 5]
+    a, b = oq.Qwen3Oracle(CFG, dense), oq.Qwen3Oracle(one, moe)
+    assert np.allclose(a.forward(toks, 0), b.forward(toks, 0), rtol=1e-5, atol=1e-5)
+    assert np.allclose(a.forward([9], 5), b.forward([9], 5), rtol=1e-5, atol=1e-5)
+
+
+def test_moe_prefill_equals_token_by_token():
+    """The bucketed dispatch of a many-token step and the single-row dispatch of decode steps agree
+    (reference: src/quantized_qwen3_moe.rs:444-520), as do cache and mask, through the expert layers."""
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(MOE, 22)}
+    toks = [3, 17, 255, 9, 100, 64]
+    whole = oq.Qwen3Oracle(MOE, tensors).forward(toks, 0)
+    step = oq.Qwen3Oracle(MOE, tensors)
+    for i, t in enumerate(toks):
+        last = step.forward([t], i)
+    assert np.allclose(whole, last, rtol=1e-4, atol=1e-4)
+
+
+def test_moe_layer_equals_an_f64_loop_over_tokens_and_experts():
+    """One expert layer of the model against a plain float64 restatement over decoded weights:
+    softmax over all experts, the two largest, their weights divided by their sum, and
+    sum_e w_e down_e(silu(gate_e x) * up_e x)."""
+    cfg = dict(MOE, n_layer=1)
+    tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(cfg, 23, "q4_k")}
+    o = oq.Qwen3Oracle(cfg, tensors)
+    h, eff, E = cfg["hidden"], cfg["expert_ffn"], cfg["n_expert"]
+    dec = lambda name, n, k: oracle.dequantize(tensors[name][0], np.asarray(tensors[name][1]).view(np.uint8).ravel()).reshape(n, k).astype(np.float64)
+    R = np.asarray(tensors["blk.0.ffn_gate_inp.weight"][1], np.float64).reshape(E, h)
+    G, U, D = dec("blk.0.ffn_gate_exps.weight", E * eff, h), dec("blk.0.ffn_up_exps.weight", E * eff, h), dec("blk.0.ffn_down_exps.weight", E * h, eff)
+    x = normal(24, (3, h)).astype(np.float32)
+    got = o.moe(0).forward(x)
+    for t in range(3):
+        xt = x[t].astype(np.float64)
+        lg = R @ xt
+        pr = np.exp(lg - lg.max()); pr /= pr.sum()
+        top = np.argsort(-pr)[:2]
+        w = pr[top] / pr[top].sum()
+        y = np.zeros(h)
+        for e, we in zip(top, w):
+            g, u = G[e * eff:(e + 1) * eff] @ xt, U[e * eff:(e + 1) * eff] @ xt
+            y += we * (D[e * h:(e + 1) * h] @ (g / (1 + np.exp(-g)) * u))
+        assert np.allclose(got[t], y, rtol=2e-2, atol=2e-2)   # the oracle matmul quantises activations to Q8_K
