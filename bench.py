@@ -511,6 +511,82 @@ def plugin_leg(prompt_len: int, n_decode: int, share_layers: bool) -> dict:
             "note": "logits of every step copied to the host (608 KB) and the arg-max taken there"}
 
 
+QWEN3_30B_A3B = dict(n_layer=48, hidden=2048, n_head=32, n_kv_head=4, head_dim=128, ffn=0, vocab=151936,
+                     rms_eps=1e-6, rope_theta=1e6, n_expert=128, n_expert_used=8, expert_ffn=768)
+
+
+def plugin_moe_leg(prompt_len: int, n_decode: int, share_layers: bool, n_layer: int, cpu_seconds: float) -> dict:
+    """A Qwen3-30B-A3B-shaped random-init qwen3moe file (Q4_K_M mix) through the joshua_npu_* symbols, in the
+    shape of the reference's own model benchmark (reference: examples/bench_qwen3moe.rs:147-174): load, one
+    prefill of prompt_len copies of token 42, then n_decode single-token steps that each feed token 42 and
+    take the arg-max of the returned logits on the host."""
+    import tempfile
+
+    from joshua_amd import capi
+    from joshua_amd.synth import gguf as gw
+    from joshua_amd.synth.model import qwen3_tensor_plan, qwen3_tensors
+
+    cfg = dict(QWEN3_30B_A3B, n_layer=n_layer, n_ctx=prompt_len + n_decode)
+    res = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "qwen3-30b-a3b-shaped-q4_k_m.gguf")
+        t0 = time.perf_counter()
+        gw.write_qwen3(path, cfg, qwen3_tensors(cfg, 9, "q4_k_m", share_layers=share_layers), qwen3_tensor_plan(cfg))
+        t_write = time.perf_counter() - t0
+        size = os.path.getsize(path)
+        t0 = time.perf_counter()
+        plug = capi.NpuPlugin(path, cfg["n_ctx"])
+        t_load = time.perf_counter() - t0
+        if plug.rc != 0:
+            raise RuntimeError(f"joshua_npu_init failed ({plug.rc}): {capi.last_error()}")
+        rc, logits = plug.forward([42] * 16, 0)       # warm-up (builds the layer objects), then start over
+        assert rc == 0 and plug.forward([42], 16)[0] == 0 and plug.reset() == 0
+        t0 = time.perf_counter()
+        rc, logits = plug.forward([42] * prompt_len, 0)
+        t_prefill = time.perf_counter() - t0
+        assert rc == 0
+        prefill_top = int(logits.size - 1 - np.argmax(logits[::-1]))
+        t0 = time.perf_counter()
+        last_top = prefill_top
+        for i in range(n_decode):
+            rc, logits = plug.forward([42], prompt_len + i)
+            assert rc == 0
+            last_top = int(logits.size - 1 - np.argmax(logits[::-1]))
+        t_dec = time.perf_counter() - t0
+        if cpu_seconds > 0:
+            # parity at these sizes: a 6-token prompt and three single-token steps against the numpy graph over
+            # the oracle matmul on the same tensors
+            import oracle
+            from oracle import qwen3 as oq
+            tensors = {n: (qt, d) for n, qt, d in qwen3_tensors(cfg, 9, "q4_k_m", share_layers=share_layers)}
+            o = oq.Qwen3Oracle(cfg, tensors, avx2=oracle.have_avx2(), threads=min(oracle.default_threads(), len(os.sched_getaffinity(0))))
+            assert plug.reset() == 0
+            toks, ok, steps = [42, 7, 1000, 42, 99999, 5], True, 0
+            t0 = time.perf_counter()
+            ref = o.forward(toks, 0)
+            ok = ok and _close(plug.forward(toks, 0)[1], ref)
+            cpu_times = []
+            for i in range(3):
+                t1 = time.perf_counter()
+                ref = o.forward([42], len(toks) + i)
+                cpu_times.append(time.perf_counter() - t1)
+                ok = ok and _close(plug.forward([42], len(toks) + i)[1], ref)
+                steps += 1
+            res["parity_ok"] = bool(ok)
+            res["parity"] = {"prefill_tokens": len(toks), "single_token_steps": steps}
+            res["cpu_tokens_per_s"] = round(1.0 / float(np.median(cpu_times)), 3)
+        plug.close()
+    res.update({"gguf_bytes": size, "write_s": round(t_write, 1), "load_s": round(t_load, 2),
+                "load_gbs": round(size / t_load / 1e9, 2), "prefill_tokens_per_s": round(prompt_len / t_prefill, 1),
+                "tokens_per_s": round(n_decode / t_dec, 2), "ms_per_token": round(1e3 * t_dec / n_decode, 4),
+                "top_token_after_prefill": prefill_top, "top_token_after_decode": last_top,
+                "workload": f"Qwen3-30B-A3B-shaped random-init qwen3moe model, {n_layer} of 48 layers, Q4_K_M mix, 128 experts "
+                            f"(8 used) of 768 rows, prefill of {prompt_len} x token 42 then {n_decode} steps feeding token 42",
+                "layers_share_bytes": share_layers,
+                "note": "logits of every step copied to the host (608 KB) and the arg-max taken there"})
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -530,6 +606,9 @@ def main() -> int:
                     help="repetitions of the K timed steps whose median is reported (0: enough for ~30 ms, 5..400)")
     ap.add_argument("--plugin", type=int, default=0,
                     help="1: also write the model to a GGUF file and run it through the joshua_npu_* symbols")
+    ap.add_argument("--plugin-moe", type=int, default=0,
+                    help="N > 0: also write a Qwen3-30B-A3B-shaped qwen3moe GGUF of N layers (48 = the whole model) and run "
+                         "it through the joshua_npu_* symbols")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -645,6 +724,9 @@ def main() -> int:
         parity_ok = parity_ok and out["decode"].get("parity_ok", True)
     if args.plugin:
         out["plugin"] = plugin_leg(args.prompt, args.new_tokens, bool(args.share_layers))
+    if args.plugin_moe:
+        out["plugin_moe"] = plugin_moe_leg(args.prompt, args.new_tokens, bool(args.share_layers), args.plugin_moe, args.cpu_seconds)
+        parity_ok = parity_ok and out["plugin_moe"].get("parity_ok", True)
     print(json.dumps(out))
     return 0 if parity_ok else 1
 
