@@ -27,6 +27,7 @@
 #include "kernels_dot4_q6k.hpp"
 #include "kernels_dot4_q8.hpp"
 #include "kernels_moe.hpp"
+#include "kernels_moe_mfma.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
 #include "kernels_moe_q4k_quads.hpp"
 #include "kernels_mfma_q4k_rows16.hpp"
@@ -1768,6 +1769,112 @@ int dispatch_moe_down_combine(uint32_t type, const uint8_t *const *Wa, size_t ro
     }
 }
 
+// The decode-sized expert matmuls on the int8 matrix cores (kernels_moe_mfma.hpp).  -1: outside their reach
+// (format without a policy, rows that are not 1, 2, 4 or 8 super-blocks for gate and up or more than 16 for down,
+// rows that do not start on 16 bytes).
+template <class K>
+int moe_mfma_big_lds(K kern, int lds) {
+    if (lds <= 64 * 1024) return 0;
+    HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    return 0;
+}
+
+jq::MoeStack moe_stack(const jq_weight *w, size_t rows_per_expert, size_t n_expert, const jq_weight *extra) {
+    return jq::MoeStack{w->dev, rows_per_expert * w->row_bytes, extra ? extra->dev : w->dev, (int)n_expert};
+}
+
+// Does moe_gate_up_mfma take this layer's gate and up projections?
+bool moe_gate_up_mfma_takes(const jq_moe *m, const float *X) {
+    static const char *off = getenv("JQ_MOE_NO_MFMA");
+    const jq_moe_config &c = m->cfg;
+    const int nb = (int)(c.hidden / 256);
+    if (off || m->gate->type != JQ_TYPE_Q4_K || m->up->type != JQ_TYPE_Q4_K || c.hidden % 256 != 0 || ((uintptr_t)X & 15) != 0)
+        return false;
+    if (nb != 1 && nb != 2 && nb != 4 && nb != 8) return false;
+    if (m->gate->row_bytes != (size_t)nb * jq::QvQ4K::BLOCK || m->up->row_bytes != m->gate->row_bytes) return false;
+    uintptr_t bits = (uintptr_t)m->gate->dev | (uintptr_t)m->up->dev;
+    if (m->fold_shared) bits |= (uintptr_t)m->sgate->dev | (uintptr_t)m->sup->dev;
+    return (bits & 15) == 0;
+}
+
+// `gate`: the launch runs the gating of the T tokens too (the router's logits are in m->logits).
+int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStream_t s, const jq::MoeClamp &cl, float *zero,
+                              int zero_n, const jq::MoeGateIn *gate) {
+    const jq_moe_config &c = m->cfg;
+    if (!moe_gate_up_mfma_takes(m, X) || pairs <= 0 || pairs > 65535) return -1;
+    const int nb = (int)(c.hidden / 256), n = (int)c.inter;
+    const jq::MoeStack wa = moe_stack(m->gate, c.inter, c.n_expert, m->fold_shared ? m->sgate : nullptr),
+                       wb = moe_stack(m->up, c.inter, c.n_expert, m->fold_shared ? m->sup : nullptr);
+    const jq::MoeGateIn gi = gate ? *gate : jq::MoeGateIn{};
+#define JQ_GU(NB, GATE)                                                                                               \
+    do {                                                                                                              \
+        auto kern = jq::moe_gate_up_mfma<jq::QvQ4K, NB, GATE>;                                                        \
+        constexpr int lds = jq::moe_gate_up_mfma_lds<jq::QvQ4K, NB>();                                                \
+        static const int attr_rc = moe_mfma_big_lds(kern, lds);                                                       \
+        if (attr_rc) return 1;                                                                                        \
+        hipLaunchKernelGGL(kern, dim3((unsigned)((n + 7) / 8), (unsigned)pairs), dim3(64 * NB), lds, s, wa, wb, X, m->gexp, \
+                           m->xrow, m->yrow, m->G, n, cl, zero, zero_n, gi);                                          \
+    } while (0)
+    if (nb == 8 && gate) JQ_GU(8, true);
+    else if (nb == 8) JQ_GU(8, false);
+    else if (nb == 4 && gate) JQ_GU(4, true);
+    else if (nb == 4) JQ_GU(4, false);
+    else if (nb == 2 && gate) JQ_GU(2, true);
+    else if (nb == 2) JQ_GU(2, false);
+    else if (gate) JQ_GU(1, true);
+    else JQ_GU(1, false);
+#undef JQ_GU
+    note_kernel(gate ? "moe_gate_up_mfma+gating" : "moe_gate_up_mfma");
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// `split`: the caller has cleared y and two workgroups may share a row tile.
+int dispatch_moe_down_mfma(const jq_moe *m, const float *A, float *y, int T, int n_extra, bool split, hipStream_t s) {
+    static const char *off = getenv("JQ_MOE_NO_MFMA");
+    const jq_moe_config &c = m->cfg;
+    const int k = (int)c.inter, n = (int)c.hidden, k_used = (int)c.n_expert_used, S = k_used + n_extra;
+    uintptr_t bits = (uintptr_t)m->down->dev | (uintptr_t)A;
+    if (m->fold_shared) bits |= (uintptr_t)m->sdown->dev;
+    if (off || m->down->type != JQ_TYPE_Q4_K || k % 256 != 0 || (bits & 15) != 0 || S > 64 || T <= 0 || T > 65535) return -1;
+    const int nb = k / 256;
+    if (m->down->row_bytes != (size_t)nb * jq::QvQ4K::BLOCK || nb > 16) return -1;
+    const jq::MoeStack wd = moe_stack(m->down, c.hidden, c.n_expert, m->fold_shared ? m->sdown : nullptr);
+#define JQ_DN(NB, SPP, SL)                                                                                            \
+    do {                                                                                                              \
+        auto kern = jq::moe_down_mfma<jq::QvQ4K, NB, SPP, SL>;                                                        \
+        constexpr int lds = jq::moe_down_mfma_lds<jq::QvQ4K, NB, SPP, SL>();                                          \
+        static_assert(lds <= 158 * 1024, "the ring fits a compute unit");                                             \
+        static const int attr_rc = moe_mfma_big_lds(kern, lds);                                                       \
+        if (attr_rc) return 1;                                                                                        \
+        const unsigned z = split && (S + SPP - 1) / SPP == 2 ? 2 : 1;                                                 \
+        if (split && z == 1) return -1;                                                                               \
+        hipLaunchKernelGGL(kern, dim3((unsigned)((n + 15) / 16), (unsigned)T, z), dim3(1024), lds, s, wd, A, m->gexp, m->wts, \
+                           y, n, k_used, n_extra, T * k_used);                                                        \
+    } while (0)
+    // segments a pass: as many as fill the 16 waves, or fewer when the passes then come out even
+    if (nb == 3 && (S + 3) / 4 == (S + 4) / 5) JQ_DN(3, 4, 3);
+    else if (nb == 3) JQ_DN(3, 5, 2);
+    else if (nb == 8) JQ_DN(8, 2, 2);
+    else if (nb == 4) JQ_DN(4, 4, 2);
+    else if (nb == 2) JQ_DN(2, 8, 2);
+    else if (nb == 1) JQ_DN(1, 16, 2);
+    else return -1;
+#undef JQ_DN
+    note_kernel("moe_down_mfma");
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// Would dispatch_moe_down_mfma run this call with two workgroups a row tile (into a cleared y)?
+bool moe_down_mfma_splits(const jq_moe *m, int T, int n_extra) {
+    const jq_moe_config &c = m->cfg;
+    const int S = (int)c.n_expert_used + n_extra, nb = (int)(c.inter / 256);
+    if (c.inter % 256 != 0 || nb < 1 || nb > 16 || (nb > 4 && nb != 8)) return false;
+    const int spp = nb == 3 ? ((S + 3) / 4 == (S + 4) / 5 ? 4 : 5) : 16 / nb;
+    return (S + spp - 1) / spp == 2 && (size_t)T * ((c.hidden + 15) / 16) <= 128;
+}
+
 template <bool SWIGLU>
 int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_bytes, const float *X, const float *X2,
                       const int *gexp, const int *offsets, const int *xsel, const int *yrow, float *Y, int k, int n,
@@ -1865,13 +1972,20 @@ int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, s
 
 // `planes`: also leave x as fixed-point planes there (the one-expert-a-workgroup router kernel does; *planes_made
 // says whether it ran)
+// `gate_later`: when the gating can run by one wave a token, it is left to the caller's next kernel (the logits are
+// in m->logits) and *gate_later holds its operands; else it is cleared.
 int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg,
-                  jq::ActsI8 planes = jq::ActsI8{nullptr, nullptr, nullptr, nullptr}, bool *planes_made = nullptr) {
+                  jq::ActsI8 planes = jq::ActsI8{nullptr, nullptr, nullptr, nullptr}, bool *planes_made = nullptr,
+                  jq::MoeGateIn *gate_later = nullptr) {
     const jq_moe_config &c = m->cfg;
     const unsigned token_runs = (unsigned)((T + jq::ROUTER_TOKENS_PER_WG - 1) / jq::ROUTER_TOKENS_PER_WG);
     static const char *no_tile = getenv("JQ_MOE_NO_ROUTER_TILE");
     // (a router of a million weights or more, 256 experts of 7168: from 8 tokens, 16 us against 27)
     const size_t tile_from = (size_t)c.hidden * c.n_expert >= (1u << 20) ? 8 : 32;
+    jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
+                         (int)c.n_group, (int)c.topk_group};
+    static const char *no_wave = getenv("JQ_MOE_NO_WAVE_GATE");
+    const bool wave_gate = !no_wave && c.n_group <= 1 && c.n_expert <= 256 && c.n_expert_used <= 64;
     if (T >= tile_from && !no_tile)  // many tokens: a token's activations read once per eight experts (the same bits)
         hipLaunchKernelGGL(jq::moe_router_logits_tile, dim3((c.n_expert + 7) / 8, (unsigned)((T + 7) / 8)), dim3(256), 0, s,
                            m->router_w, x, m->logits, (int)T, (int)c.hidden, (int)c.n_expert);
@@ -1879,12 +1993,17 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
         hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert, token_runs), dim3(256), 0, s, m->router_w, x, m->logits,
                            (int)T, (int)c.hidden, (int)c.n_expert, planes);
     if (planes_made) *planes_made = planes.xl && !(T >= tile_from && !no_tile);
-    jq::MoeGateParams gp{(int)c.n_expert, (int)c.n_expert_used, (int)c.gating, (int)c.norm_topk, c.weights_scale,
-                         (int)c.n_group, (int)c.topk_group};
     size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);
+    if (gate_later) {
+        if (wave_gate) {
+            *gate_later = jq::MoeGateIn{m->logits, m->router_bias, gp, m->ids, m->wts, pg, (int)T};
+            HIP_TRY(hipGetLastError());
+            return 0;
+        }
+        gate_later->logits = nullptr;
+    }
     // no expert groups and at most 256 experts: one wave a token, reductions in registers
-    static const char *no_wave = getenv("JQ_MOE_NO_WAVE_GATE");
-    if (!no_wave && c.n_group <= 1 && c.n_expert <= 256 && c.n_expert_used <= 64) {
+    if (wave_gate) {
         const int ne = (int)(c.n_expert + 63) / 64;
 #define JQ_GATE(NE) hipLaunchKernelGGL(jq::moe_gate_topk_wave<NE>, dim3((unsigned)T), dim3(64), 0, s, m->logits, m->router_bias, gp, m->ids, m->wts, pg)
         if (ne == 1) JQ_GATE(1);
@@ -1947,16 +2066,21 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         if (!expert_env) expert_dot8 = by_expert < by_gemm;
     }
     bool planes_ready = false;
+    jq::MoeGateIn gate_later{};
     if (decode_sized) {  // one group per pair, written by the gating kernel itself
         // long rows: the gate and up kernel reads x as fixed-point planes, which the router kernel can leave behind
         jq::ActsI8 planes{nullptr, nullptr, nullptr, nullptr};
         static const char *no_router_planes = getenv("JQ_MOE_NO_ROUTER_PLANES");
         if (!no_router_planes && m->gate->type == m->up->type && m->gate->row_bytes == m->up->row_bytes &&
-            ((uintptr_t)x & 15) == 0 &&
+            ((uintptr_t)x & 15) == 0 && !moe_gate_up_mfma_takes(m, x) &&
             moe_dot8_takes_planes(m->gate->type, m->gate->row_bytes, (((uintptr_t)m->gate->dev | (uintptr_t)m->up->dev) & 15) ? 4 : 16,
                                   (int)c.hidden, (int)c.inter, m->qi8))
             planes = m->qi8;
-        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra}, planes, &planes_ready))
+        // the matrix-core gate and up kernel can run the gating itself
+        static const char *no_late_gate = getenv("JQ_MOE_NO_GATING_IN_GATE_UP");
+        const bool late = !no_late_gate && m->gate->type == m->up->type && moe_gate_up_mfma_takes(m, x);
+        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra}, planes, &planes_ready,
+                          late ? &gate_later : nullptr))
             return 1;
         groups = P + extra * (int)T;
         max_group = 1;
@@ -2044,6 +2168,17 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         }
     }
     if (rc > 0) return 1;
+    // decode-sized Q4_K: the matrix-core kernels; a call of few row tiles clears y here and lets two workgroups a
+    // tile add into it in the down projection
+    bool y_cleared = false;
+    if (rc < 0 && same_gu && max_group <= 1) {
+        const bool will_split = (m->fold_shared || !m->sgate) && m->down->type == JQ_TYPE_Q4_K && moe_down_mfma_splits(m, (int)T, extra);
+        rc = dispatch_moe_gate_up_mfma(m, x, groups, s, clamp, will_split ? y : nullptr, will_split ? (int)(T * c.hidden) : 0,
+                                       gate_later.logits ? &gate_later : nullptr);
+        if (rc < 0 && gate_later.logits) return fail("moe: the gating was left to a kernel that declined the call");
+        y_cleared = rc == 0 && will_split;
+    }
+    if (rc > 0) return 1;
     if (rc < 0 && same_gu && max_group <= 1)
         rc = dispatch_moe_dot8<true>(m->gate->type, m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp,
                                      m->offsets, m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp,
@@ -2087,6 +2222,9 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     if (rc > 0) return 1;
     // decode-sized, and no shared expert outside the pair list: down projection and combine in one launch
     if (rc < 0 && fused_act && max_group <= 1 && (m->fold_shared || !m->sgate)) {
+        rc = dispatch_moe_down_mfma(m, m->G, y, (int)T, extra, y_cleared, s);
+        if (rc == 0) return 0;
+        if (rc > 0) return 1;
         rc = dispatch_moe_down_combine(m->down->type, m->pdown, m->down->row_bytes, d16, m->G, (size_t)P + extra * T, m->qi8,
                                        m->gexp, m->wts, y, (int)c.inter, (int)c.hidden, (int)T, (int)c.n_expert_used, extra, s);
         if (rc == 0) return 0;

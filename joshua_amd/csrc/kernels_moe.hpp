@@ -47,8 +47,8 @@ __device__ __forceinline__ void acts_i8_quantize(const float *__restrict__ X, si
 // src/quantized_deepseek2.rs:528; an f32 matmul there too)
 constexpr int ROUTER_TOKENS_PER_WG = 8;
 
-__global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict__ Wr, const float *__restrict__ X,
-                                                          float *__restrict__ logits, int T, int h, int E, ActsI8 planes) {
+__device__ __forceinline__ void moe_router_logits_body(const float *__restrict__ Wr, const float *__restrict__ X,
+                                                       float *__restrict__ logits, int T, int h, int E, ActsI8 planes) {
     // one workgroup per (expert row of the router, run of 8 tokens): every load of the row in
     // flight at once; a logit's arithmetic does not depend on how the tokens are split
     __shared__ float red[4][4];
@@ -87,6 +87,11 @@ __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict
                 (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
         __syncthreads();
     }
+}
+
+__global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict__ Wr, const float *__restrict__ X,
+                                                          float *__restrict__ logits, int T, int h, int E, ActsI8 planes) {
+    moe_router_logits_body(Wr, X, logits, T, h, E, planes);
 }
 
 // The same logits for several tokens: one workgroup per (8 router rows, 8 tokens), so a token's activations are read
@@ -265,11 +270,13 @@ __global__ __launch_bounds__(256) void moe_gate_topk(const float *__restrict__ l
 // reductions (no LDS, no barrier), where moe_gate_topk's 256 threads meet at eight barriers and rank every
 // expert against every other through LDS: 3 us a launch instead of 7.  Equal scores go to the lower expert
 // index, as there.
+// The gating of token t by one wave.  Lane r < k_used ends with slot r's expert in *slot_e; `write`: the slots go
+// to ids / wts and the pair groups as well (a kernel that runs the gating in every workgroup writes them once).
 template <int NE>
-__global__ __launch_bounds__(64) void moe_gate_topk_wave(const float *__restrict__ logits, const float *__restrict__ bias,
-                                                          MoeGateParams p, uint32_t *__restrict__ ids,
-                                                          float *__restrict__ wts, MoePairGroups pg) {
-    const int t = blockIdx.x, T = gridDim.x, lane = threadIdx.x;
+__device__ __forceinline__ void moe_gate_topk_wave_body(int t, int T, int lane, const float *__restrict__ logits,
+                                                        const float *__restrict__ bias, const MoeGateParams &p,
+                                                        uint32_t *__restrict__ ids, float *__restrict__ wts,
+                                                        const MoePairGroups &pg, bool write, int *slot_e) {
     const float *lg = logits + (size_t)t * p.E;
     float prob[NE], sel[NE];
     {
@@ -302,14 +309,19 @@ __global__ __launch_bounds__(64) void moe_gate_topk_wave(const float *__restrict
     float my_p = 0.0f;  // lane r keeps slot r
     for (int r = 0; r < p.k_used; r++) {
         float best = sel[0];
-        int bi = 0;
 #pragma unroll
-        for (int i = 1; i < NE; i++)
-            if (sel[i] > best) best = sel[i], bi = i;  // the lower index stays on a tie
+        for (int i = 1; i < NE; i++) best = fmaxf(best, sel[i]);
         const float top = wave_max(best);
-        const float cand = best == top ? (float)(lane + 64 * bi) : 1e9f;
-        const int e = __builtin_amdgcn_readfirstlane((int)(-wave_max(-cand)));  // the lowest expert index among the ties
-        const int owner = e & 63, slot = e >> 6;
+        // the lowest expert index holding the maximum: the first slot any lane holds it in, and there the first
+        // lane (scalar work on the lanes' votes; scores that compare with nothing, from activations that are not
+        // numbers, leave slot r to expert r)
+        int slot = 0, owner = r & 63;
+#pragma unroll
+        for (int i = NE - 1; i >= 0; i--) {
+            const unsigned long long votes = __ballot(sel[i] == top);
+            if (votes) slot = i, owner = __builtin_ctzll(votes);
+        }
+        const int e = min(owner + 64 * slot, p.E - 1);  // (in range whatever the scores were)
         float pw = 0.0f;
 #pragma unroll
         for (int i = 0; i < NE; i++) {
@@ -328,6 +340,8 @@ __global__ __launch_bounds__(64) void moe_gate_topk_wave(const float *__restrict
         w = w / fmaxf(s, 6.103515625e-5f);
     }
     if (p.scale != 0.0f && p.scale != 1.0f) w = w * p.scale;
+    *slot_e = my_e;
+    if (!write) return;
     if (lane < p.k_used) {
         const int pidx = t * p.k_used + lane;
         ids[pidx] = (uint32_t)my_e;
@@ -342,6 +356,14 @@ __global__ __launch_bounds__(64) void moe_gate_topk_wave(const float *__restrict
             pg.gexp[pidx] = p.E, pg.offsets[pidx] = pidx, pg.xrow[pidx] = t, pg.yrow[pidx] = pidx;
         }
     }
+}
+
+template <int NE>
+__global__ __launch_bounds__(64) void moe_gate_topk_wave(const float *__restrict__ logits, const float *__restrict__ bias,
+                                                          MoeGateParams p, uint32_t *__restrict__ ids,
+                                                          float *__restrict__ wts, MoePairGroups pg) {
+    int slot_e;
+    moe_gate_topk_wave_body<NE>((int)blockIdx.x, (int)gridDim.x, (int)threadIdx.x, logits, bias, p, ids, wts, pg, true, &slot_e);
 }
 
 // Groups the T*k routed (token, slot) pairs by expert, keeping pair order inside

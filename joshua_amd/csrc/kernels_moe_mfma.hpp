@@ -1,0 +1,255 @@
+// The expert matmuls of a decode-sized mixture-of-experts call (every routed (token, expert) pair reads its
+// expert's rows once) on the int8 matrix cores, over the per-format policies of the one-row GEMV
+// (kernels_gemv_mfma.hpp): a wave quantises 256 activations once into registers as the block-diagonal A operand
+// and multiplies them with one super-block column of 16 weight rows an instruction group, so no activation
+// is read a second time and the integer dot products cost four MFMAs a wave and 16 rows.
+//
+//   moe_gate_up_mfma    G[pair, j] = silu(gate_e[j] . x_t) * (up_e[j] . x_t)    (reference: src/quantized_qwen3_moe.rs:397-401)
+//   moe_down_mfma       y[t, r]    = sum_s w[t, s] (down_e(s)[r] . G[pair(t, s)])  (:504-520, src/quantized_deepseek2.rs:553-557)
+//
+// Both take rows of at most 8 (gate, up) or 16 (down) super-blocks: the waves of a workgroup then cover whole tiles
+// of 16 rows at once and every weight byte of the call is asked for in the launch's first microsecond.
+#pragma once
+#include "kernels_gemv_mfma.hpp"
+#include "kernels_valu.hpp"
+#include "kernels_moe.hpp"
+
+namespace jq {
+
+// LDS rows 16 bytes past a multiple of 256: the 16 rows a wave's lanes read side by side fall on all banks.
+constexpr int moe_mfma_row_lds(int bytes) { return (bytes + 255) / 256 * 256 + 16; }
+// a wave's staging area: what the policy's prepare() uses, and in front of that the wave's 256 raw activations
+template <class F>
+constexpr int moe_mfma_stage() { return ((F::STAGE_BYTES > 1024 ? F::STAGE_BYTES : 1024) + 15) / 16 * 16; }
+
+// Where the experts of a stacked tensor start: expert e < n_routed at base + e stride, the folded shared expert
+// (number n_routed) at `extra`.
+struct MoeStack {
+    const uint8_t *base;
+    size_t stride;
+    const uint8_t *extra;
+    int n_routed;
+};
+__device__ __forceinline__ const uint8_t *moe_expert_base(const MoeStack &st, int e) {
+    return e < st.n_routed ? st.base + (size_t)e * st.stride : st.extra;
+}
+
+template <class F, int NB>
+constexpr int moe_gate_up_mfma_lds() {
+    return 16 * moe_mfma_row_lds(NB * F::BLOCK) + NB * moe_mfma_stage<F>() + 16 * 68 * 4;
+}
+
+// One workgroup of NB waves per (pair, 8 rows of gate and the same 8 rows of up): gate and up multiply the same
+// activations, so the 16 weight rows of a matrix-core tile are 8 of each, wave w takes super-block column w of all
+// 16, and SwiGLU meets both halves where the rows are stored.  With rows of 8 super-blocks a tile is 18 KB and a
+// call's tiles (96 a pair at 768 rows) spread evenly over the chip, four workgroups a compute unit, all asked
+// for in the launch's first microsecond behind the waves' activations, which are quantised while they land.
+// `zero`: zero_n floats the launch also clears, for the kernel behind it that adds into them.
+// GATE: the launch runs the gating too.  Every workgroup's first wave picks the token's experts from the router's
+// logits (moe_gate_topk_wave's arithmetic, the same bits) while the activations travel, and takes its pair's
+// expert from there; the first workgroup of a token's first pair writes ids, weights and pair groups for the down
+// projection.  A launch less than gating on its own, which costs 4 us of which 3 are the launch and its wait for
+// the router.
+struct MoeGateIn {
+    const float *logits, *bias;
+    MoeGateParams p;
+    uint32_t *ids;
+    float *wts;
+    MoePairGroups pg;
+    int T;
+};
+
+template <class F, int NB, bool GATE>
+__global__ __launch_bounds__(64 * NB) void moe_gate_up_mfma(MoeStack Wa, MoeStack Wb, const float *__restrict__ X,
+                                                            const int *__restrict__ gexp, const int *__restrict__ xrow,
+                                                            const int *__restrict__ yrow, float *__restrict__ G, int inter,
+                                                            MoeClamp cl, float *__restrict__ zero, int zero_n, MoeGateIn gi) {
+    static_assert(NB == 1 || NB == 2 || NB == 4 || NB == 8, "a row of 1, 2, 4 or 8 super-blocks");
+    constexpr int RB = NB * F::BLOCK, ROW_LDS = moe_mfma_row_lds(RB), LOADS = (RB + 1023) / 1024, STG = moe_mfma_stage<F>();
+    constexpr int RPW = 16 / NB;  // tile rows a wave copies
+    static_assert(RB % 16 == 0, "rows are copied 16 bytes a lane");
+    extern __shared__ __attribute__((aligned(16))) uint8_t moe_mfma_lds[];
+    __shared__ int picked;
+    uint8_t *tile = moe_mfma_lds;                                               // [16][ROW_LDS]: 8 gate rows, 8 up rows
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    uint32_t *stage = (uint32_t *)(moe_mfma_lds + 16 * ROW_LDS + wave * STG);
+    float *part = (float *)(moe_mfma_lds + 16 * ROW_LDS + NB * STG);            // [16][68]
+    const int p = blockIdx.y;
+    int e, t, out_row;
+    if (GATE) {  // pair p is slot p % k_used of token p / k_used, or behind the routed pairs the token's shared expert
+        const int P = gi.T * gi.p.k_used;
+        t = p < P ? p / gi.p.k_used : p - P;
+        out_row = p;
+    } else {
+        e = gexp[p], t = xrow[p], out_row = yrow[p];
+    }
+    async_load16(X + (size_t)t * (256 * NB) + 256 * wave + 4 * lane, lds_offset_of(stage));
+    typename F::Acts acts;
+    // the activations are quantised while the tile lands; with the gating in the launch, by the waves that do not
+    // run it while it runs (wave 0 follows behind its tile loads)
+    auto prepare = [&]() __attribute__((always_inline)) {
+        const float4 v = *(const float4 *)((const float *)stage + 4 * lane);
+        acts = F::prepare(v, stage, lane);
+    };
+    if (GATE) {
+        const int P = gi.T * gi.p.k_used;
+        if (wave == 0) {
+            int slot_e;
+            moe_gate_topk_wave_body<4>(t, gi.T, lane, gi.logits, gi.bias, gi.p, gi.ids, gi.wts, gi.pg,
+                                       blockIdx.x == 0 && p < P && p % gi.p.k_used == 0, &slot_e);
+            const int mine = p < P ? __builtin_amdgcn_readlane(slot_e, p % gi.p.k_used) : gi.p.E;
+            if (lane == 0) picked = mine;
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            prepare();
+        }
+        __syncthreads();
+        e = __builtin_amdgcn_readfirstlane(picked);
+    }
+    const uint8_t *wa = moe_expert_base(Wa, e), *wb = moe_expert_base(Wb, e);
+    const int j0 = blockIdx.x * 8;
+    const uint32_t tile0 = lds_offset_of(tile);
+#pragma unroll
+    for (int i = 0; i < RPW; i++) {
+        const int rr = wave + NB * i, j = min(j0 + (rr & 7), inter - 1);
+        const uint8_t *src = (rr < 8 ? wa : wb) + (size_t)j * RB;
+        const uint32_t dst = tile0 + (uint32_t)rr * ROW_LDS;
+#pragma unroll
+        for (int l = 0; l < LOADS; l++) {
+            constexpr int full = 64;
+            const int lanes = (RB - 1024 * l) / 16 < full ? (RB - 1024 * l) / 16 : full;
+            if (lane < lanes) async_load16_s(src + 1024 * l, 16 * lane, dst + 1024 * l);
+        }
+    }
+    if (!GATE || wave == 0) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPW * LOADS) : "memory");  // the activations are in
+        prepare();
+    }
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
+    if (NB > 1) __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    part[r * 68 + 4 * wave + c] = F::block_dot_lane(tile + r * ROW_LDS + wave * F::BLOCK, acts, c);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (NB > 1) __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // wave w adds the 4 NB chunk sums of gate row w (w + NB, ..) and of the up row beside it
+#pragma unroll
+    for (int q = 0; q < 8 / NB; q++) {
+        const int jj = wave + NB * q;
+        float g = lane < 4 * NB ? part[jj * 68 + lane] : 0.0f;
+        float u = lane < 4 * NB ? part[(jj + 8) * 68 + lane] : 0.0f;
+        g = wave_sum(g), u = wave_sum(u);
+        if (lane == 0 && j0 + jj < inter) G[(size_t)out_row * inter + j0 + jj] = swiglu(g, u, cl, e);
+    }
+    if (zero) {
+        const int wg = blockIdx.y * gridDim.x + blockIdx.x, n_wg = gridDim.x * gridDim.y;
+        for (int i = wg * (64 * NB) + tid; i < zero_n; i += n_wg * 64 * NB) zero[i] = 0.0f;
+    }
+}
+
+// A pointer every lane of the wave holds, moved to scalar registers.
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+}
+
+template <class F, int NB, int SPP, int SLOTS>
+constexpr int moe_down_mfma_lds() {
+    return SLOTS * 16 * moe_mfma_row_lds(SPP * NB * F::BLOCK) + 2 * 16 * 1024 + 16 * moe_mfma_stage<F>() + 16 * 68 * 4;
+}
+
+// One workgroup per (token, 16 rows of the result).  The token's S = k_used + n_extra pairs are the segments of
+// one long row, [down_e(0)[r] | down_e(1)[r] | ..] against [w_0 a_0 | w_1 a_1 | ..] with a_s the pair's activation
+// row of NB super-blocks: the combine weights ride on the activations and the sum over the pairs is the sum over
+// the row.  A pass is SPP segments (NB SPP <= 16 waves at work: wave w takes block w % NB of segment w / NB),
+// its 16 rows x SPP segments travel through a ring of SLOTS slots (three: two passes in flight; two where three
+// do not fit) with the waves' activations beside them, and a lane adds its chunk sums of all passes in a register.
+template <class F, int NB, int SPP, int SLOTS>
+__global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *__restrict__ A,
+                                                      const int *__restrict__ gexp, const float *__restrict__ wts,
+                                                      float *__restrict__ Y, int n, int k_used, int n_extra, int P) {
+    static_assert(NB * SPP <= 16, "a pass is at most 16 super-block columns");
+    static_assert(SLOTS == 2 || SLOTS == 3, "one or two passes ahead of the arithmetic");
+    constexpr int RB = NB * F::BLOCK, ROW_LDS = moe_mfma_row_lds(SPP * RB), LOADS = (RB + 1023) / 1024, STG = moe_mfma_stage<F>();
+    constexpr int LPF = SPP * LOADS + 1;  // loads a wave and pass: its row's segments and its activations
+    static_assert(RB % 16 == 0, "rows are copied 16 bytes a lane");
+    constexpr int MAX_S = 64;
+    extern __shared__ __attribute__((aligned(16))) uint8_t moe_mfma_lds[];
+    __shared__ const uint8_t *seg_base[MAX_S];
+    __shared__ float seg_wt[MAX_S];
+    __shared__ int seg_pair[MAX_S];
+    uint8_t *ring = moe_mfma_lds;                                  // [SLOTS][16][ROW_LDS]
+    float *xbuf = (float *)(moe_mfma_lds + SLOTS * 16 * ROW_LDS);      // [2][16][256]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    uint32_t *stage = (uint32_t *)(moe_mfma_lds + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + wave * STG);
+    float *part = (float *)(moe_mfma_lds + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + 16 * STG);  // [16][68]
+    // gridDim.z workgroups share a (token, row tile): number z takes passes z, z + gridDim.z, ..
+    const int t = blockIdx.y, S = k_used + n_extra, Z = gridDim.z, z = blockIdx.z;
+    const int NP = ((S + SPP - 1) / SPP - z + Z - 1) / Z;
+    if (tid < S) {
+        const int pair = tid < k_used ? t * k_used + tid : P + t;
+        seg_base[tid] = moe_expert_base(Wd, gexp[pair]);
+        seg_wt[tid] = tid < k_used ? wts[pair] : 1.0f;
+        seg_pair[tid] = pair;
+    }
+    __syncthreads();
+    const int row = min(16 * (int)blockIdx.x + wave, n - 1);
+    const int q = wave / NB, blk = wave % NB;       // this wave's segment of a pass and block of the segment
+    const bool worker = q < SPP;
+    const uint32_t ring0 = lds_offset_of(ring), xbuf0 = lds_offset_of(xbuf);
+    const int inter = 256 * NB;
+    auto fetch = [&](int i) __attribute__((always_inline)) {
+        const uint32_t dst = ring0 + (uint32_t)((i % SLOTS) * 16 + wave) * ROW_LDS;
+        const int first = (z + Z * i) * SPP;  // the pass's first segment
+#pragma unroll
+        for (int qq = 0; qq < SPP; qq++) {
+            const int s = min(first + qq, S - 1);
+            const uint8_t *src = uniform_ptr(seg_base[s]) + (size_t)row * RB;
+#pragma unroll
+            for (int j = 0; j < LOADS; j++) {
+                constexpr int full = 64;
+                const int lanes = (RB - 1024 * j) / 16 < full ? (RB - 1024 * j) / 16 : full;
+                if (lane < lanes) async_load16_s(src + 1024 * j, 16 * lane, dst + qq * RB + 1024 * j);
+            }
+        }
+        const int s = min(first + min(q, SPP - 1), S - 1);
+        async_load16(A + (size_t)seg_pair[s] * inter + 256 * blk + 4 * lane, xbuf0 + (uint32_t)(((i & 1) * 16 + wave) * 1024));
+    };
+    fetch(0);
+    if (SLOTS == 3 && NP > 1) fetch(1);
+    float acc = 0.0f;
+    for (int i = 0; i < NP; i++) {
+        if (SLOTS == 3 && i + 1 < NP) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPF) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const int s = (z + Z * i) * SPP + q;
+        const bool live = worker && s < S;
+        float4 v = *(const float4 *)(xbuf + ((i & 1) * 16 + wave) * 256 + 4 * lane);
+        const float w = seg_wt[min(s, S - 1)];
+        v = float4{v.x * w, v.y * w, v.z * w, v.w * w};
+        const typename F::Acts acts = F::prepare(v, stage, lane);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (live) acc += F::block_dot_lane(ring + ((i % SLOTS) * 16 + r) * ROW_LDS + q * RB + blk * F::BLOCK, acts, c);
+        // every wave has passed this pass's barrier, so all are done with pass i - 1, whose slot the next pass to
+        // ask for takes; this wave's activations of pass i are in registers and make room as well
+        if (i + SLOTS - 1 < NP) fetch(i + SLOTS - 1);
+    }
+    part[r * 68 + 4 * wave + c] = acc;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const float sum = wave_sum(part[wave * 68 + lane]);
+    const int out_row = 16 * (int)blockIdx.x + wave;
+    if (lane == 0 && out_row < n) {
+        // two workgroups a row tile add into a result the launch before cleared: 0 + a + b in either order
+        if (Z > 1) atomicAdd(Y + (size_t)t * n + out_row, sum);
+        else Y[(size_t)t * n + out_row] = sum;
+    }
+}
+
+}  // namespace jq
