@@ -1783,18 +1783,40 @@ jq::MoeStack moe_stack(const jq_weight *w, size_t rows_per_expert, size_t n_expe
     return jq::MoeStack{w->dev, rows_per_expert * w->row_bytes, extra ? extra->dev : w->dev, (int)n_expert};
 }
 
-// Does moe_gate_up_mfma take this layer's gate and up projections?
+// Bytes of a 256-element super-block in the formats the matrix-core expert kernels have a policy for; 0: none.
+int moe_mfma_block_bytes(uint32_t type) {
+    switch (type) {
+    case JQ_TYPE_Q4_K: return jq::QvQ4K::BLOCK;
+    case JQ_TYPE_IQ2_XXS: return jq::QvI8<jq::IQ2_XXS>::BLOCK;
+    case JQ_TYPE_MXFP4: return jq::QvI8<jq::MXFP4>::BLOCK;
+    default: return 0;
+    }
+}
+
+// Does a matrix-core kernel take this layer's gate and up projections?  Rows of 1, 2, 4 or 8 super-blocks (Q4_K;
+// 8 for the others): moe_gate_up_mfma; of 9 to 32: moe_gate_up_rows_mfma.
 bool moe_gate_up_mfma_takes(const jq_moe *m, const float *X) {
     static const char *off = getenv("JQ_MOE_NO_MFMA");
     const jq_moe_config &c = m->cfg;
-    const int nb = (int)(c.hidden / 256);
-    if (off || m->gate->type != JQ_TYPE_Q4_K || m->up->type != JQ_TYPE_Q4_K || c.hidden % 256 != 0 || ((uintptr_t)X & 15) != 0)
-        return false;
-    if (nb != 1 && nb != 2 && nb != 4 && nb != 8) return false;
-    if (m->gate->row_bytes != (size_t)nb * jq::QvQ4K::BLOCK || m->up->row_bytes != m->gate->row_bytes) return false;
+    const int nb = (int)(c.hidden / 256), bb = moe_mfma_block_bytes(m->gate->type);
+    if (off || !bb || m->up->type != m->gate->type || c.hidden % 256 != 0 || ((uintptr_t)X & 15) != 0) return false;
+    if (m->gate->row_bytes != (size_t)nb * bb || m->up->row_bytes != m->gate->row_bytes) return false;
     uintptr_t bits = (uintptr_t)m->gate->dev | (uintptr_t)m->up->dev;
     if (m->fold_shared) bits |= (uintptr_t)m->sgate->dev | (uintptr_t)m->sup->dev;
-    return (bits & 15) == 0;
+    if ((bits & 15) != 0) return false;
+    // JQ_MOE_MFMA_ONLY=gate_up / down: only that projection takes the matrix-core kernels (for measurements)
+    static const char *only = getenv("JQ_MOE_MFMA_ONLY");
+    const char only_part = only ? only[0] : 0;
+    if (only_part == 'd') return false;
+    if (nb <= 8) return nb == 8 || (m->gate->type == JQ_TYPE_Q4_K && (nb == 1 || nb == 2 || nb == 4));
+    // whole rows of a tile as two spans of 8 rows, copied by 1024 lanes in one instruction (IQ2_XXS) or two; a ring of
+    // three slots (IQ2_XXS) or two whose slots behind the first hold the waves' 32 KB of raw activations at the start
+    const bool iq2 = m->gate->type == JQ_TYPE_IQ2_XXS;
+    const size_t pieces = (size_t)nb * bb / 2, slot = (size_t)16 * nb * bb, slots = iq2 ? 3 : 2;
+    const size_t lds = iq2 ? jq::moe_gate_up_rows_mfma_lds<jq::QvI8<jq::IQ2_XXS>, 2, 3, 1>(nb)
+                           : m->gate->type == JQ_TYPE_MXFP4 ? jq::moe_gate_up_rows_mfma_lds<jq::QvI8<jq::MXFP4>, 2, 2, 2>(nb)
+                                                            : jq::moe_gate_up_rows_mfma_lds<jq::QvQ4K, 2, 2, 2>(nb);
+    return nb <= 32 && c.inter % 8 == 0 && pieces <= (iq2 ? 1024u : 2048u) && (slots - 1) * slot >= 32 * 1024 && lds <= 158 * 1024;
 }
 
 // `gate`: the launch runs the gating of the T tokens too (the router's logits are in m->logits).
@@ -1806,24 +1828,54 @@ int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStr
     const jq::MoeStack wa = moe_stack(m->gate, c.inter, c.n_expert, m->fold_shared ? m->sgate : nullptr),
                        wb = moe_stack(m->up, c.inter, c.n_expert, m->fold_shared ? m->sup : nullptr);
     const jq::MoeGateIn gi = gate ? *gate : jq::MoeGateIn{};
-#define JQ_GU(NB, GATE)                                                                                               \
+#define JQ_GU(F, NB, GATE)                                                                                            \
     do {                                                                                                              \
-        auto kern = jq::moe_gate_up_mfma<jq::QvQ4K, NB, GATE>;                                                        \
-        constexpr int lds = jq::moe_gate_up_mfma_lds<jq::QvQ4K, NB>();                                                \
+        auto kern = jq::moe_gate_up_mfma<F, NB, GATE>;                                                                \
+        constexpr int lds = jq::moe_gate_up_mfma_lds<F, NB>();                                                        \
         static const int attr_rc = moe_mfma_big_lds(kern, lds);                                                       \
         if (attr_rc) return 1;                                                                                        \
         hipLaunchKernelGGL(kern, dim3((unsigned)((n + 7) / 8), (unsigned)pairs), dim3(64 * NB), lds, s, wa, wb, X, m->gexp, \
                            m->xrow, m->yrow, m->G, n, cl, zero, zero_n, gi);                                          \
     } while (0)
-    if (nb == 8 && gate) JQ_GU(8, true);
-    else if (nb == 8) JQ_GU(8, false);
-    else if (nb == 4 && gate) JQ_GU(4, true);
-    else if (nb == 4) JQ_GU(4, false);
-    else if (nb == 2 && gate) JQ_GU(2, true);
-    else if (nb == 2) JQ_GU(2, false);
-    else if (gate) JQ_GU(1, true);
-    else JQ_GU(1, false);
+    // rows of more than 8 super-blocks: 16 waves a pair and tile sequence, two columns a wave
+#define JQ_GUR(F, SL, J, GATE)                                                                                        \
+    do {                                                                                                              \
+        auto kern = jq::moe_gate_up_rows_mfma<F, 2, SL, J, GATE>;                                                     \
+        const int lds = jq::moe_gate_up_rows_mfma_lds<F, 2, SL, J>(nb);                                               \
+        const int slot = (16 * nb * F::BLOCK + 15) / 16 * 16;                                                         \
+        if (lds > 158 * 1024 || (SL - 1) * slot < 2 * 16 * 1024 || zero) return -1;                                   \
+        static const int attr_rc = moe_mfma_big_lds(kern, 158 * 1024);                                                \
+        if (attr_rc) return 1;                                                                                        \
+        const int per_pair = std::max(1, std::min(n / 8, (lds > 79 * 1024 ? 256 : 512) / pairs));                     \
+        hipLaunchKernelGGL(kern, dim3((unsigned)per_pair, (unsigned)pairs), dim3(1024), lds, s, wa, wb, X, m->gexp, m->xrow, \
+                           m->yrow, m->G, n, nb, cl, gi);                                                             \
+    } while (0)
+    const uint32_t type = m->gate->type;
+    if (nb > 8) {
+        if (type == JQ_TYPE_IQ2_XXS && gate) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 3, 1, true);
+        else if (type == JQ_TYPE_IQ2_XXS) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 3, 1, false);
+        else if (type == JQ_TYPE_MXFP4 && gate) JQ_GUR(jq::QvI8<jq::MXFP4>, 2, 2, true);
+        else if (type == JQ_TYPE_MXFP4) JQ_GUR(jq::QvI8<jq::MXFP4>, 2, 2, false);
+        else if (gate) JQ_GUR(jq::QvQ4K, 2, 2, true);
+        else JQ_GUR(jq::QvQ4K, 2, 2, false);
+        note_kernel(gate ? "moe_gate_up_rows_mfma+gating" : "moe_gate_up_rows_mfma");
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
+    if (type == JQ_TYPE_IQ2_XXS && gate) JQ_GU(jq::QvI8<jq::IQ2_XXS>, 8, true);
+    else if (type == JQ_TYPE_IQ2_XXS) JQ_GU(jq::QvI8<jq::IQ2_XXS>, 8, false);
+    else if (type == JQ_TYPE_MXFP4 && gate) JQ_GU(jq::QvI8<jq::MXFP4>, 8, true);
+    else if (type == JQ_TYPE_MXFP4) JQ_GU(jq::QvI8<jq::MXFP4>, 8, false);
+    else if (nb == 8 && gate) JQ_GU(jq::QvQ4K, 8, true);
+    else if (nb == 8) JQ_GU(jq::QvQ4K, 8, false);
+    else if (nb == 4 && gate) JQ_GU(jq::QvQ4K, 4, true);
+    else if (nb == 4) JQ_GU(jq::QvQ4K, 4, false);
+    else if (nb == 2 && gate) JQ_GU(jq::QvQ4K, 2, true);
+    else if (nb == 2) JQ_GU(jq::QvQ4K, 2, false);
+    else if (gate) JQ_GU(jq::QvQ4K, 1, true);
+    else JQ_GU(jq::QvQ4K, 1, false);
 #undef JQ_GU
+#undef JQ_GUR
     note_kernel(gate ? "moe_gate_up_mfma+gating" : "moe_gate_up_mfma");
     HIP_TRY(hipGetLastError());
     return 0;
@@ -1834,16 +1886,19 @@ int dispatch_moe_down_mfma(const jq_moe *m, const float *A, float *y, int T, int
     static const char *off = getenv("JQ_MOE_NO_MFMA");
     const jq_moe_config &c = m->cfg;
     const int k = (int)c.inter, n = (int)c.hidden, k_used = (int)c.n_expert_used, S = k_used + n_extra;
+    const uint32_t type = m->down->type;
+    const int bb = moe_mfma_block_bytes(type);
     uintptr_t bits = (uintptr_t)m->down->dev | (uintptr_t)A;
     if (m->fold_shared) bits |= (uintptr_t)m->sdown->dev;
-    if (off || m->down->type != JQ_TYPE_Q4_K || k % 256 != 0 || (bits & 15) != 0 || S > 64 || T <= 0 || T > 65535) return -1;
+    static const char *only = getenv("JQ_MOE_MFMA_ONLY");
+    if (off || (only && only[0] == 'g') || !bb || k % 256 != 0 || (bits & 15) != 0 || S > 64 || T <= 0 || T > 65535) return -1;
     const int nb = k / 256;
-    if (m->down->row_bytes != (size_t)nb * jq::QvQ4K::BLOCK || nb > 16) return -1;
+    if (m->down->row_bytes != (size_t)nb * bb || nb > 16 || (type != JQ_TYPE_Q4_K && nb != 8)) return -1;
     const jq::MoeStack wd = moe_stack(m->down, c.hidden, c.n_expert, m->fold_shared ? m->sdown : nullptr);
-#define JQ_DN(NB, SPP, SL)                                                                                            \
+#define JQ_DN(F, NB, SPP, SL)                                                                                         \
     do {                                                                                                              \
-        auto kern = jq::moe_down_mfma<jq::QvQ4K, NB, SPP, SL>;                                                        \
-        constexpr int lds = jq::moe_down_mfma_lds<jq::QvQ4K, NB, SPP, SL>();                                          \
+        auto kern = jq::moe_down_mfma<F, NB, SPP, SL>;                                                                \
+        constexpr int lds = jq::moe_down_mfma_lds<F, NB, SPP, SL>();                                                  \
         static_assert(lds <= 158 * 1024, "the ring fits a compute unit");                                             \
         static const int attr_rc = moe_mfma_big_lds(kern, lds);                                                       \
         if (attr_rc) return 1;                                                                                        \
@@ -1853,12 +1908,14 @@ int dispatch_moe_down_mfma(const jq_moe *m, const float *A, float *y, int T, int
                            y, n, k_used, n_extra, T * k_used);                                                        \
     } while (0)
     // segments a pass: as many as fill the 16 waves, or fewer when the passes then come out even
-    if (nb == 3 && (S + 3) / 4 == (S + 4) / 5) JQ_DN(3, 4, 3);
-    else if (nb == 3) JQ_DN(3, 5, 2);
-    else if (nb == 8) JQ_DN(8, 2, 2);
-    else if (nb == 4) JQ_DN(4, 4, 2);
-    else if (nb == 2) JQ_DN(2, 8, 2);
-    else if (nb == 1) JQ_DN(1, 16, 2);
+    if (type == JQ_TYPE_IQ2_XXS) JQ_DN(jq::QvI8<jq::IQ2_XXS>, 8, 2, 3);
+    else if (type == JQ_TYPE_MXFP4) JQ_DN(jq::QvI8<jq::MXFP4>, 8, 2, 2);
+    else if (nb == 3 && (S + 3) / 4 == (S + 4) / 5) JQ_DN(jq::QvQ4K, 3, 4, 3);
+    else if (nb == 3) JQ_DN(jq::QvQ4K, 3, 5, 2);
+    else if (nb == 8) JQ_DN(jq::QvQ4K, 8, 2, 2);
+    else if (nb == 4) JQ_DN(jq::QvQ4K, 4, 4, 2);
+    else if (nb == 2) JQ_DN(jq::QvQ4K, 2, 8, 2);
+    else if (nb == 1) JQ_DN(jq::QvQ4K, 1, 16, 2);
     else return -1;
 #undef JQ_DN
     note_kernel("moe_down_mfma");
@@ -2172,7 +2229,8 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     // tile add into it in the down projection
     bool y_cleared = false;
     if (rc < 0 && same_gu && max_group <= 1) {
-        const bool will_split = (m->fold_shared || !m->sgate) && m->down->type == JQ_TYPE_Q4_K && moe_down_mfma_splits(m, (int)T, extra);
+        const bool will_split = (m->fold_shared || !m->sgate) && m->down->type == JQ_TYPE_Q4_K && c.hidden <= 2048 &&
+                                moe_down_mfma_splits(m, (int)T, extra);
         rc = dispatch_moe_gate_up_mfma(m, x, groups, s, clamp, will_split ? y : nullptr, will_split ? (int)(T * c.hidden) : 0,
                                        gate_later.logits ? &gate_later : nullptr);
         if (rc < 0 && gate_later.logits) return fail("moe: the gating was left to a kernel that declined the call");

@@ -52,6 +52,7 @@ __device__ __forceinline__ QvActs qv_prepare(const float4 v, uint32_t *stage, in
         if (lane < 8) stage[256 + lane] = 0;
         if ((lane & 7) == 0) side[lane >> 3] = float4{q.s, q.s * (float)q.sum, __builtin_bit_cast(float, 128 * q.sum), q.s * 0.0625f};
     }
+    asm volatile("" ::: "memory");  // (written as scalars, read back as vectors: the compiler keeps the order only when told)
     QvActs a;
     {
         // A operands of lane (m = r, g = c): row m is sub-block m / 2, plane m % 2, and non-zero in lane group
@@ -71,6 +72,7 @@ __device__ __forceinline__ QvActs qv_prepare(const float4 v, uint32_t *stage, in
     const float4 fe = side[2 * c], fo = side[2 * c + 1];
     a.s_e = fe.x, a.xs_e = fe.y, a.s_o16 = fo.w, a.xs_o = fo.y;
     a.c_init = qv_i4{0, 0, __builtin_bit_cast(int, fo.z), 0};
+    asm volatile("" ::: "memory");  // (the next column's preparation writes the same words as another type)
     return a;
 }
 
@@ -188,6 +190,7 @@ struct QvQ2K {
             if ((lane & 7) == 0) stage_f[lane >> 3] = s;
             if ((lane & 3) == 0) stage_f[8 + (lane >> 2)] = s * (float)sum;
         }
+        asm volatile("" ::: "memory");  // (written as scalars, read back as vectors: the compiler keeps the order only when told)
         Acts a;
         const int cm = r >> 2, pl = r & 3;  // A row m = 4 cm + plane
         const bool mine = cm == c && pl < 2;
@@ -201,6 +204,7 @@ struct QvQ2K {
             a.s[f] = stage_f[4 * (c >> 1) + f] * pw;
             a.xs[f] = stage_f[8 + 8 * (c >> 1) + 2 * f + (c & 1)];
         }
+        asm volatile("" ::: "memory");  // (the next column's preparation writes the same words as another type)
         return a;
     }
     __device__ static __forceinline__ float block_dot(const uint8_t *blk, const Acts &a, int c) {
@@ -281,6 +285,7 @@ struct QvQ6K {
             if ((lane & 7) == 0) sf[lane >> 3] = q.s;
             if ((lane & 3) == 0) xs16[lane >> 2] = s4;
         }
+        asm volatile("" ::: "memory");  // (written as scalars, read back as vectors: the compiler keeps the order only when told)
         Acts a;
         const bool mine = (r >> 2) == c;
         const int p = (r >> 1) & 1, pl = r & 1;
@@ -293,6 +298,7 @@ struct QvQ6K {
         }
         a.init[0] = qv_i4{-32 * xs16[8 * h + lh], 0, -32 * xs16[8 * h + 2 + lh], 0};
         a.init[1] = qv_i4{-32 * xs16[8 * h + 4 + lh], 0, -32 * xs16[8 * h + 6 + lh], 0};
+        asm volatile("" ::: "memory");  // (the next column's preparation writes the same words as another type)
         return a;
     }
     __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) {

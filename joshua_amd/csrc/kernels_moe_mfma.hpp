@@ -16,6 +16,88 @@
 
 namespace jq {
 
+// The policy of the formats whose 32-element units decode to signed int8 words (Q::decode_i8: IQ2_XXS through its
+// codebook, MXFP4 through two byte permutes): a super-block is 256 consecutive elements, 8 units (one IQ2_XXS block,
+// eight MXFP4 blocks).  Lane (r, c) decodes units 2c and 2c + 1 of weight row r into the B operands of four MFMAs;
+// the activations are 15-bit fixed point a 32-element sub-block in two int8 planes, block-diagonal in A as for
+// Q4_K (row 4c + 2p + plane is non-zero in lane group c only), so the lane receives the two planes' sums of both
+// its units and   sum = scale(2c) s(2c) (256 Sh + Sl) + scale(2c + 1) s(2c + 1) (256 Sh' + Sl').
+// Every integer sum is exact (|w| <= 43, |X| <= 128, 32 terms).
+template <class Q>
+struct QvI8 {
+    static_assert(Q::HAS_DECODE_I8 && !Q::I8_HAS_MIN, "units that decode to int8 words and a scale");
+    static constexpr int SUB = 256 / Q::BLOCK_ELEMS;   // format blocks a super-block
+    static_assert(SUB * Q::I8_UNITS == 8, "eight units of 32 elements a super-block");
+    static constexpr int BLOCK = SUB * Q::BLOCK_BYTES;
+    static constexpr int STAGE_BYTES = 4 * (128 + 8 + 8);  // the two planes, eight zero words, the sub-blocks' scales
+    static constexpr bool TAKES_TABLE = true;
+    typedef Q Format;
+    struct Acts {
+        qv_i4 a_even[2], a_odd[2];
+        float s_e, s_o;
+    };
+    __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) {
+        const int r = lane & 15, c = lane >> 4;
+        const QvQuant q = qv_quantise4(v);
+        stage[lane] = q.wl, stage[64 + lane] = q.wh;
+        if (lane < 8) stage[128 + lane] = 0;
+        float *scales = (float *)(stage + 136);
+        if ((lane & 7) == 0) scales[lane >> 3] = q.s;
+        // (the words are written as scalars and read back as vectors: the compiler keeps the order only when told)
+        asm volatile("" ::: "memory");
+        // row m = r of A: lane group (r / 4) only, unit parity (r / 2) % 2, plane r % 2; the others read zeros
+        const bool mine = (r >> 2) == c, odd = (r & 2) != 0;
+        const uint32_t *pos = stage + 64 * (r & 1) + 16 * c + (odd ? 8 : 0), *zero = stage + 128;
+        const uint32_t *ev = mine && !odd ? pos : zero, *od = mine && odd ? pos : zero;
+        const uint4 e0 = *(const uint4 *)ev, e1 = *(const uint4 *)(ev + 4), o0 = *(const uint4 *)od, o1 = *(const uint4 *)(od + 4);
+        Acts a;
+        a.a_even[0] = qv_i4{(int)e0.x, (int)e0.y, (int)e0.z, (int)e0.w};
+        a.a_even[1] = qv_i4{(int)e1.x, (int)e1.y, (int)e1.z, (int)e1.w};
+        a.a_odd[0] = qv_i4{(int)o0.x, (int)o0.y, (int)o0.z, (int)o0.w};
+        a.a_odd[1] = qv_i4{(int)o1.x, (int)o1.y, (int)o1.z, (int)o1.w};
+        a.s_e = scales[2 * c], a.s_o = scales[2 * c + 1];
+        asm volatile("" ::: "memory");
+        return a;
+    }
+    __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c, const uint64_t *table) {
+        int we[8], wo[8];
+        float se, so, off;
+        if (SUB == 1) {
+            Q::decode_i8(table, blk, 2 * c, we, se, off);
+            Q::decode_i8(table, blk, 2 * c + 1, wo, so, off);
+        } else {
+            Q::decode_i8(table, blk + (2 * c) * Q::BLOCK_BYTES, 0, we, se, off);
+            Q::decode_i8(table, blk + (2 * c + 1) * Q::BLOCK_BYTES, 0, wo, so, off);
+        }
+        qv_i4 C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_even[0], qv_i4{we[0], we[1], we[2], we[3]}, qv_i4{0, 0, 0, 0}, 0, 0, 0);
+        C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_even[1], qv_i4{we[4], we[5], we[6], we[7]}, C, 0, 0, 0);
+        C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_odd[0], qv_i4{wo[0], wo[1], wo[2], wo[3]}, C, 0, 0, 0);
+        C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_odd[1], qv_i4{wo[4], wo[5], wo[6], wo[7]}, C, 0, 0, 0);
+        return fmaf(se * a.s_e, (float)((C[1] << 8) + C[0]), so * a.s_o * (float)((C[3] << 8) + C[2]));
+    }
+};
+
+// Policies whose block_dot_lane wants the format's lookup table (a copy in LDS) as a fourth argument.
+template <class F, class = void>
+struct QvTakesTable : std::false_type {};
+template <class F>
+struct QvTakesTable<F, std::void_t<decltype(F::TAKES_TABLE)>> : std::true_type {};
+template <class F>
+__host__ __device__ constexpr int qv_table_bytes() {
+    if constexpr (QvTakesTable<F>::value) return (table_bytes<typename F::Format>() + 15) / 16 * 16;
+    else return 0;
+}
+template <class F>
+__device__ __forceinline__ const uint64_t *qv_stage_table(uint8_t *lds) {  // holds a barrier when there is a table
+    if constexpr (QvTakesTable<F>::value) return stage_table<typename F::Format>(lds);
+    else return nullptr;
+}
+template <class F>
+__device__ __forceinline__ float qv_dot(const uint8_t *blk, const typename F::Acts &a, int c, const uint64_t *table) {
+    if constexpr (QvTakesTable<F>::value) return F::block_dot_lane(blk, a, c, table);
+    else return F::block_dot_lane(blk, a, c);
+}
+
 // LDS rows 16 bytes past a multiple of 256: the 16 rows a wave's lanes read side by side fall on all banks.
 constexpr int moe_mfma_row_lds(int bytes) { return (bytes + 255) / 256 * 256 + 16; }
 // a wave's staging area: what the policy's prepare() uses, and in front of that the wave's 256 raw activations
@@ -36,7 +118,7 @@ __device__ __forceinline__ const uint8_t *moe_expert_base(const MoeStack &st, in
 
 template <class F, int NB>
 constexpr int moe_gate_up_mfma_lds() {
-    return 16 * moe_mfma_row_lds(NB * F::BLOCK) + NB * moe_mfma_stage<F>() + 16 * 68 * 4;
+    return qv_table_bytes<F>() + 16 * moe_mfma_row_lds(NB * F::BLOCK) + NB * moe_mfma_stage<F>() + 16 * 68 * 4;
 }
 
 // One workgroup of NB waves per (pair, 8 rows of gate and the same 8 rows of up): gate and up multiply the same
@@ -70,11 +152,12 @@ __global__ __launch_bounds__(64 * NB) void moe_gate_up_mfma(MoeStack Wa, MoeStac
     static_assert(RB % 16 == 0, "rows are copied 16 bytes a lane");
     extern __shared__ __attribute__((aligned(16))) uint8_t moe_mfma_lds[];
     __shared__ int picked;
-    uint8_t *tile = moe_mfma_lds;                                               // [16][ROW_LDS]: 8 gate rows, 8 up rows
+    const uint64_t *table = qv_stage_table<F>(moe_mfma_lds);
+    uint8_t *tile = moe_mfma_lds + qv_table_bytes<F>();                         // [16][ROW_LDS]: 8 gate rows, 8 up rows
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, c = lane >> 4;
-    uint32_t *stage = (uint32_t *)(moe_mfma_lds + 16 * ROW_LDS + wave * STG);
-    float *part = (float *)(moe_mfma_lds + 16 * ROW_LDS + NB * STG);            // [16][68]
+    uint32_t *stage = (uint32_t *)(tile + 16 * ROW_LDS + wave * STG);
+    float *part = (float *)(tile + 16 * ROW_LDS + NB * STG);                    // [16][68]
     const int p = blockIdx.y;
     int e, t, out_row;
     if (GATE) {  // pair p is slot p % k_used of token p / k_used, or behind the routed pairs the token's shared expert
@@ -129,7 +212,7 @@ __global__ __launch_bounds__(64 * NB) void moe_gate_up_mfma(MoeStack Wa, MoeStac
     asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
     if (NB > 1) __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    part[r * 68 + 4 * wave + c] = F::block_dot_lane(tile + r * ROW_LDS + wave * F::BLOCK, acts, c);
+    part[r * 68 + 4 * wave + c] = qv_dot<F>(tile + r * ROW_LDS + wave * F::BLOCK, acts, c, table);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if (NB > 1) __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -148,6 +231,121 @@ __global__ __launch_bounds__(64 * NB) void moe_gate_up_mfma(MoeStack Wa, MoeStac
     }
 }
 
+// Gate and up for rows of more than 8 super-blocks (nb <= 16 NG).  A workgroup of 16 waves stays with one pair
+// and walks tiles b, b + gridDim.x, .. of it, a tile again 8 rows of gate and the same 8 rows of up: wave w keeps the
+// operands of columns w, w + 16, .. for the whole launch, the tiles travel through a ring of SLOTS slots as whole
+// rows (8 consecutive rows of a matrix are one span of memory, copied 16 bytes a lane by all 1024 lanes: J
+// instructions a span and wave), and a lane adds its chunk sums of its columns in a register.
+// The raw activations wait in the ring's slots behind the first until they are prepared.
+template <class F, int NG, int SLOTS, int J>
+constexpr int moe_gate_up_rows_mfma_lds(int nb) {
+    return qv_table_bytes<F>() + SLOTS * ((16 * nb * F::BLOCK + 15) / 16 * 16) + 1024 + 16 * moe_mfma_stage<F>() + 16 * 68 * 4;
+}
+
+template <class F, int NG, int SLOTS, int J, bool GATE>
+__global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeStack Wb, const float *__restrict__ X,
+                                                              const int *__restrict__ gexp, const int *__restrict__ xrow,
+                                                              const int *__restrict__ yrow, float *__restrict__ G, int inter,
+                                                              int nb, MoeClamp cl, MoeGateIn gi) {
+    static_assert(NG >= 1 && NG <= 2 && (SLOTS == 2 || SLOTS == 3) && (J == 1 || J == 2), "two columns a wave at most");
+    constexpr int STG = moe_mfma_stage<F>(), LPF = 2 * J;  // loads a wave and tile: J a span
+    extern __shared__ __attribute__((aligned(16))) uint8_t moe_mfma_lds[];
+    __shared__ int picked;
+    const uint64_t *table = qv_stage_table<F>(moe_mfma_lds);
+    const int RB = nb * F::BLOCK, span = 8 * RB, slot_bytes = (2 * span + 15) / 16 * 16;  // 8 RB is a multiple of 16
+    uint8_t *ring = moe_mfma_lds + qv_table_bytes<F>();
+    uint8_t *dump = ring + SLOTS * slot_bytes;                       // where a wave without a piece of a span points its load
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    uint32_t *stage = (uint32_t *)(dump + 1024 + wave * STG);
+    float *part = (float *)(dump + 1024 + 16 * STG);                 // [16][68]
+    float *xraw = (float *)(ring + slot_bytes);                      // [NG][16][256], in the slots behind the first
+    const int p = blockIdx.y;
+    int e, t, out_row;
+    if (GATE) {
+        const int P = gi.T * gi.p.k_used;
+        t = p < P ? p / gi.p.k_used : p - P;
+        out_row = p;
+    } else {
+        e = gexp[p], t = xrow[p], out_row = yrow[p];
+    }
+    const int ntiles = inter / 8, b = blockIdx.x, G_ = gridDim.x;
+    const int nt = (ntiles - b + G_ - 1) / G_;
+    if (nt <= 0) return;  // (whole workgroups: the barriers below see either all waves or none)
+#pragma unroll
+    for (int cg = 0; cg < NG; cg++)
+        async_load16(X + (size_t)t * (256 * nb) + 256 * min(16 * cg + wave, nb - 1) + 4 * lane,
+                     lds_offset_of(xraw + (cg * 16 + wave) * 256));
+    if (GATE) {
+        const int P = gi.T * gi.p.k_used;
+        if (wave == 0) {
+            int slot_e;
+            moe_gate_topk_wave_body<4>(t, gi.T, lane, gi.logits, gi.bias, gi.p, gi.ids, gi.wts, gi.pg,
+                                       b == 0 && p < P && p % gi.p.k_used == 0, &slot_e);
+            const int mine = p < P ? __builtin_amdgcn_readlane(slot_e, p % gi.p.k_used) : gi.p.E;
+            if (lane == 0) picked = mine;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    typename F::Acts acts[NG];
+#pragma unroll
+    for (int cg = 0; cg < NG; cg++) {
+        const float4 v = *(const float4 *)(xraw + (cg * 16 + wave) * 256 + 4 * lane);
+        acts[cg] = F::prepare(v, stage, lane);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();  // the raw activations are read: the slots they waited in are free; the gating's pick is written
+    if (GATE) e = __builtin_amdgcn_readfirstlane(picked);
+    const uint8_t *wa = moe_expert_base(Wa, e), *wb = moe_expert_base(Wb, e);
+    const uint32_t ring0 = lds_offset_of(ring), dump0 = lds_offset_of(dump);
+    const int pieces = span / 16;
+    auto fetch = [&](int i) __attribute__((always_inline)) {
+        const size_t row0 = (size_t)8 * (b + (size_t)min(i, nt - 1) * G_);
+        const uint32_t slot0 = ring0 + (uint32_t)(i % SLOTS) * slot_bytes;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint8_t *src = (half ? wb : wa) + row0 * RB;
+#pragma unroll
+            for (int j = 0; j < J; j++) {
+                const int first = 64 * (wave + 16 * j), left = pieces - first;  // this wave's pieces of the span
+                if (left > 0) {
+                    if (lane < left) async_load16_s(src + 16 * (size_t)first, 16 * lane, slot0 + half * span + 16 * first);
+                } else if (lane == 0) {
+                    async_load16_s(src, 0, dump0 + 16 * wave);  // so that every wave counts the same loads
+                }
+            }
+        }
+    };
+    fetch(0);
+    if (nt > 1) fetch(1);
+    if (SLOTS == 3 && nt > 2) fetch(2);
+    for (int i = 0; i < nt; i++) {
+        // tile i is in when only the tiles asked for behind it are out
+        const int behind = min(SLOTS - 1, nt - 1 - i);
+        if (behind >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPF) : "memory");
+        else if (behind == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPF) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const uint8_t *slot = ring + (i % SLOTS) * slot_bytes;
+        float acc = 0.0f;
+#pragma unroll
+        for (int cg = 0; cg < NG; cg++)
+            if (16 * cg + wave < nb) acc += qv_dot<F>(slot + r * RB + (16 * cg + wave) * F::BLOCK, acts[cg], c, table);
+        part[r * 68 + 4 * wave + c] = acc;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // every wave is done with tile i: its slot takes tile i + SLOTS
+        if (i + SLOTS < nt) fetch(i + SLOTS);
+        if (wave < 8) {
+            float g = wave_sum(part[wave * 68 + lane]), u = wave_sum(part[(wave + 8) * 68 + lane]);
+            const int j = 8 * (b + i * G_) + wave;
+            if (lane == 0) G[(size_t)out_row * inter + j] = swiglu(g, u, cl, e);
+        }
+    }
+}
+
 // A pointer every lane of the wave holds, moved to scalar registers.
 __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     const uint64_t v = (uint64_t)p;
@@ -158,7 +356,8 @@ __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
 
 template <class F, int NB, int SPP, int SLOTS>
 constexpr int moe_down_mfma_lds() {
-    return SLOTS * 16 * moe_mfma_row_lds(SPP * NB * F::BLOCK) + 2 * 16 * 1024 + 16 * moe_mfma_stage<F>() + 16 * 68 * 4;
+    return qv_table_bytes<F>() + SLOTS * 16 * moe_mfma_row_lds(SPP * NB * F::BLOCK) + 2 * 16 * 1024 + 16 * moe_mfma_stage<F>() +
+           16 * 68 * 4;
 }
 
 // One workgroup per (token, 16 rows of the result).  The token's S = k_used + n_extra pairs are the segments of
@@ -181,12 +380,13 @@ __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *
     __shared__ const uint8_t *seg_base[MAX_S];
     __shared__ float seg_wt[MAX_S];
     __shared__ int seg_pair[MAX_S];
-    uint8_t *ring = moe_mfma_lds;                                  // [SLOTS][16][ROW_LDS]
-    float *xbuf = (float *)(moe_mfma_lds + SLOTS * 16 * ROW_LDS);      // [2][16][256]
+    const uint64_t *table = qv_stage_table<F>(moe_mfma_lds);
+    uint8_t *ring = moe_mfma_lds + qv_table_bytes<F>();            // [SLOTS][16][ROW_LDS]
+    float *xbuf = (float *)(ring + SLOTS * 16 * ROW_LDS);          // [2][16][256]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, c = lane >> 4;
-    uint32_t *stage = (uint32_t *)(moe_mfma_lds + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + wave * STG);
-    float *part = (float *)(moe_mfma_lds + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + 16 * STG);  // [16][68]
+    uint32_t *stage = (uint32_t *)(ring + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + wave * STG);
+    float *part = (float *)(ring + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + 16 * STG);  // [16][68]
     // gridDim.z workgroups share a (token, row tile): number z takes passes z, z + gridDim.z, ..
     const int t = blockIdx.y, S = k_used + n_extra, Z = gridDim.z, z = blockIdx.z;
     const int NP = ((S + SPP - 1) / SPP - z + Z - 1) / Z;
@@ -234,7 +434,7 @@ __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *
         v = float4{v.x * w, v.y * w, v.z * w, v.w * w};
         const typename F::Acts acts = F::prepare(v, stage, lane);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (live) acc += F::block_dot_lane(ring + ((i % SLOTS) * 16 + r) * ROW_LDS + q * RB + blk * F::BLOCK, acts, c);
+        if (live) acc += qv_dot<F>(ring + ((i % SLOTS) * 16 + r) * ROW_LDS + q * RB + blk * F::BLOCK, acts, c, table);
         // every wave has passed this pass's barrier, so all are done with pass i - 1, whose slot the next pass to
         // ask for takes; this wave's activations of pass i are in registers and make room as well
         if (i + SLOTS - 1 < NP) fetch(i + SLOTS - 1);
