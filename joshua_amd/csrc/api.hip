@@ -1809,14 +1809,14 @@ bool moe_gate_up_mfma_takes(const jq_moe *m, const float *X) {
     const char only_part = only ? only[0] : 0;
     if (only_part == 'd') return false;
     if (nb <= 8) return nb == 8 || (m->gate->type == JQ_TYPE_Q4_K && (nb == 1 || nb == 2 || nb == 4));
-    // whole rows of a tile as two spans of 8 rows, copied by 1024 lanes in one instruction (IQ2_XXS) or two; a ring of
-    // three slots (IQ2_XXS) or two whose slots behind the first hold the waves' 32 KB of raw activations at the start
+    // whole rows of a tile as two spans of 8 rows, copied by 1024 lanes in one instruction (IQ2_XXS) or two, through a
+    // ring of two slots; the slot behind the first holds the waves' raw activations (1 KB a column) at the start
     const bool iq2 = m->gate->type == JQ_TYPE_IQ2_XXS;
-    const size_t pieces = (size_t)nb * bb / 2, slot = (size_t)16 * nb * bb, slots = iq2 ? 3 : 2;
-    const size_t lds = iq2 ? jq::moe_gate_up_rows_mfma_lds<jq::QvI8<jq::IQ2_XXS>, 2, 3, 1>(nb)
+    const size_t pieces = (size_t)nb * bb / 2, slot = (size_t)16 * nb * bb;
+    const size_t lds = iq2 ? jq::moe_gate_up_rows_mfma_lds<jq::QvI8<jq::IQ2_XXS>, 2, 2, 1>(nb)
                            : m->gate->type == JQ_TYPE_MXFP4 ? jq::moe_gate_up_rows_mfma_lds<jq::QvI8<jq::MXFP4>, 2, 2, 2>(nb)
                                                             : jq::moe_gate_up_rows_mfma_lds<jq::QvQ4K, 2, 2, 2>(nb);
-    return nb <= 32 && c.inter % 8 == 0 && pieces <= (iq2 ? 1024u : 2048u) && (slots - 1) * slot >= 32 * 1024 && lds <= 158 * 1024;
+    return nb <= 32 && c.inter % 8 == 0 && pieces <= (iq2 ? 1024u : 2048u) && slot >= (size_t)nb * 1024 && lds <= 158 * 1024;
 }
 
 // `gate`: the launch runs the gating of the T tokens too (the router's logits are in m->logits).
@@ -1843,7 +1843,7 @@ int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStr
         auto kern = jq::moe_gate_up_rows_mfma<F, 2, SL, J, GATE>;                                                     \
         const int lds = jq::moe_gate_up_rows_mfma_lds<F, 2, SL, J>(nb);                                               \
         const int slot = (16 * nb * F::BLOCK + 15) / 16 * 16;                                                         \
-        if (lds > 158 * 1024 || (SL - 1) * slot < 2 * 16 * 1024 || zero) return -1;                                   \
+        if (lds > 158 * 1024 || (SL - 1) * slot < nb * 1024 || zero) return -1;                                   \
         static const int attr_rc = moe_mfma_big_lds(kern, 158 * 1024);                                                \
         if (attr_rc) return 1;                                                                                        \
         const int per_pair = std::max(1, std::min(n / 8, (lds > 79 * 1024 ? 256 : 512) / pairs));                     \
@@ -1852,8 +1852,8 @@ int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStr
     } while (0)
     const uint32_t type = m->gate->type;
     if (nb > 8) {
-        if (type == JQ_TYPE_IQ2_XXS && gate) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 3, 1, true);
-        else if (type == JQ_TYPE_IQ2_XXS) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 3, 1, false);
+        if (type == JQ_TYPE_IQ2_XXS && gate) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 2, 1, true);
+        else if (type == JQ_TYPE_IQ2_XXS) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 2, 1, false);
         else if (type == JQ_TYPE_MXFP4 && gate) JQ_GUR(jq::QvI8<jq::MXFP4>, 2, 2, true);
         else if (type == JQ_TYPE_MXFP4) JQ_GUR(jq::QvI8<jq::MXFP4>, 2, 2, false);
         else if (gate) JQ_GUR(jq::QvQ4K, 2, 2, true);
@@ -1895,10 +1895,10 @@ int dispatch_moe_down_mfma(const jq_moe *m, const float *A, float *y, int T, int
     const int nb = k / 256;
     if (m->down->row_bytes != (size_t)nb * bb || nb > 16 || (type != JQ_TYPE_Q4_K && nb != 8)) return -1;
     const jq::MoeStack wd = moe_stack(m->down, c.hidden, c.n_expert, m->fold_shared ? m->sdown : nullptr);
-#define JQ_DN(F, NB, SPP, SL)                                                                                         \
+#define JQ_DN(F, NB, SPP, SL, XB)                                                                                       \
     do {                                                                                                              \
-        auto kern = jq::moe_down_mfma<F, NB, SPP, SL>;                                                                \
-        constexpr int lds = jq::moe_down_mfma_lds<F, NB, SPP, SL>();                                                  \
+        auto kern = jq::moe_down_mfma<F, NB, SPP, SL, XB>;                                                            \
+        constexpr int lds = jq::moe_down_mfma_lds<F, NB, SPP, SL, XB>();                                              \
         static_assert(lds <= 158 * 1024, "the ring fits a compute unit");                                             \
         static const int attr_rc = moe_mfma_big_lds(kern, lds);                                                       \
         if (attr_rc) return 1;                                                                                        \
@@ -1908,14 +1908,15 @@ int dispatch_moe_down_mfma(const jq_moe *m, const float *A, float *y, int T, int
                            y, n, k_used, n_extra, T * k_used);                                                        \
     } while (0)
     // segments a pass: as many as fill the 16 waves, or fewer when the passes then come out even
-    if (type == JQ_TYPE_IQ2_XXS) JQ_DN(jq::QvI8<jq::IQ2_XXS>, 8, 2, 3);
-    else if (type == JQ_TYPE_MXFP4) JQ_DN(jq::QvI8<jq::MXFP4>, 8, 2, 2);
-    else if (nb == 3 && (S + 3) / 4 == (S + 4) / 5) JQ_DN(jq::QvQ4K, 3, 4, 3);
-    else if (nb == 3) JQ_DN(jq::QvQ4K, 3, 5, 2);
-    else if (nb == 8) JQ_DN(jq::QvQ4K, 8, 2, 2);
-    else if (nb == 4) JQ_DN(jq::QvQ4K, 4, 4, 2);
-    else if (nb == 2) JQ_DN(jq::QvQ4K, 2, 8, 2);
-    else if (nb == 1) JQ_DN(jq::QvQ4K, 1, 16, 2);
+    // (IQ2_XXS: two slots and one activation buffer, 74 KB, two workgroups a compute unit)
+    if (type == JQ_TYPE_IQ2_XXS) JQ_DN(jq::QvI8<jq::IQ2_XXS>, 8, 2, 2, 1);
+    else if (type == JQ_TYPE_MXFP4) JQ_DN(jq::QvI8<jq::MXFP4>, 8, 2, 2, 2);
+    else if (nb == 3 && (S + 3) / 4 == (S + 4) / 5) JQ_DN(jq::QvQ4K, 3, 4, 3, 2);
+    else if (nb == 3) JQ_DN(jq::QvQ4K, 3, 5, 2, 2);
+    else if (nb == 8) JQ_DN(jq::QvQ4K, 8, 2, 2, 2);
+    else if (nb == 4) JQ_DN(jq::QvQ4K, 4, 4, 2, 2);
+    else if (nb == 2) JQ_DN(jq::QvQ4K, 2, 8, 2, 2);
+    else if (nb == 1) JQ_DN(jq::QvQ4K, 1, 16, 2, 2);
     else return -1;
 #undef JQ_DN
     note_kernel("moe_down_mfma");

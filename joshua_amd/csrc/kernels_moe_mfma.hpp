@@ -116,6 +116,10 @@ __device__ __forceinline__ const uint8_t *moe_expert_base(const MoeStack &st, in
     return e < st.n_routed ? st.base + (size_t)e * st.stride : st.extra;
 }
 
+// (where the raw activations have a place of their own)
+template <class F>
+constexpr int moe_mfma_stage_only() { return (F::STAGE_BYTES + 15) / 16 * 16; }
+
 template <class F, int NB>
 constexpr int moe_gate_up_mfma_lds() {
     return qv_table_bytes<F>() + 16 * moe_mfma_row_lds(NB * F::BLOCK) + NB * moe_mfma_stage<F>() + 16 * 68 * 4;
@@ -236,10 +240,10 @@ __global__ __launch_bounds__(64 * NB) void moe_gate_up_mfma(MoeStack Wa, MoeStac
 // operands of columns w, w + 16, .. for the whole launch, the tiles travel through a ring of SLOTS slots as whole
 // rows (8 consecutive rows of a matrix are one span of memory, copied 16 bytes a lane by all 1024 lanes: J
 // instructions a span and wave), and a lane adds its chunk sums of its columns in a register.
-// The raw activations wait in the ring's slots behind the first until they are prepared.
+// The raw activations (1 KB a column) wait in the ring's slots behind the first until they are prepared.
 template <class F, int NG, int SLOTS, int J>
 constexpr int moe_gate_up_rows_mfma_lds(int nb) {
-    return qv_table_bytes<F>() + SLOTS * ((16 * nb * F::BLOCK + 15) / 16 * 16) + 1024 + 16 * moe_mfma_stage<F>() + 16 * 68 * 4;
+    return qv_table_bytes<F>() + SLOTS * ((16 * nb * F::BLOCK + 15) / 16 * 16) + 1024 + 16 * moe_mfma_stage_only<F>() + 16 * 68 * 4;
 }
 
 template <class F, int NG, int SLOTS, int J, bool GATE>
@@ -248,7 +252,7 @@ __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeSt
                                                               const int *__restrict__ yrow, float *__restrict__ G, int inter,
                                                               int nb, MoeClamp cl, MoeGateIn gi) {
     static_assert(NG >= 1 && NG <= 2 && (SLOTS == 2 || SLOTS == 3) && (J == 1 || J == 2), "two columns a wave at most");
-    constexpr int STG = moe_mfma_stage<F>(), LPF = 2 * J;  // loads a wave and tile: J a span
+    constexpr int STG = moe_mfma_stage_only<F>(), LPF = 2 * J;  // loads a wave and tile: J a span
     extern __shared__ __attribute__((aligned(16))) uint8_t moe_mfma_lds[];
     __shared__ int picked;
     const uint64_t *table = qv_stage_table<F>(moe_mfma_lds);
@@ -259,7 +263,7 @@ __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeSt
     const int r = lane & 15, c = lane >> 4;
     uint32_t *stage = (uint32_t *)(dump + 1024 + wave * STG);
     float *part = (float *)(dump + 1024 + 16 * STG);                 // [16][68]
-    float *xraw = (float *)(ring + slot_bytes);                      // [NG][16][256], in the slots behind the first
+    float *xraw = (float *)(ring + slot_bytes);                      // [nb][256], in the slots behind the first
     const int p = blockIdx.y;
     int e, t, out_row;
     if (GATE) {
@@ -275,7 +279,7 @@ __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeSt
 #pragma unroll
     for (int cg = 0; cg < NG; cg++)
         async_load16(X + (size_t)t * (256 * nb) + 256 * min(16 * cg + wave, nb - 1) + 4 * lane,
-                     lds_offset_of(xraw + (cg * 16 + wave) * 256));
+                     lds_offset_of(xraw + min(16 * cg + wave, nb - 1) * 256));
     if (GATE) {
         const int P = gi.T * gi.p.k_used;
         if (wave == 0) {
@@ -290,7 +294,7 @@ __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeSt
     typename F::Acts acts[NG];
 #pragma unroll
     for (int cg = 0; cg < NG; cg++) {
-        const float4 v = *(const float4 *)(xraw + (cg * 16 + wave) * 256 + 4 * lane);
+        const float4 v = *(const float4 *)(xraw + min(16 * cg + wave, nb - 1) * 256 + 4 * lane);
         acts[cg] = F::prepare(v, stage, lane);
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -354,9 +358,9 @@ __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     return (const uint8_t *)(((uint64_t)hi << 32) | lo);
 }
 
-template <class F, int NB, int SPP, int SLOTS>
+template <class F, int NB, int SPP, int SLOTS, int XB>
 constexpr int moe_down_mfma_lds() {
-    return qv_table_bytes<F>() + SLOTS * 16 * moe_mfma_row_lds(SPP * NB * F::BLOCK) + 2 * 16 * 1024 + 16 * moe_mfma_stage<F>() +
+    return qv_table_bytes<F>() + SLOTS * 16 * moe_mfma_row_lds(SPP * NB * F::BLOCK) + XB * 16 * 1024 + 16 * moe_mfma_stage_only<F>() +
            16 * 68 * 4;
 }
 
@@ -366,13 +370,16 @@ constexpr int moe_down_mfma_lds() {
 // the row.  A pass is SPP segments (NB SPP <= 16 waves at work: wave w takes block w % NB of segment w / NB),
 // its 16 rows x SPP segments travel through a ring of SLOTS slots (three: two passes in flight; two where three
 // do not fit) with the waves' activations beside them, and a lane adds its chunk sums of all passes in a register.
-template <class F, int NB, int SPP, int SLOTS>
+// XB: buffers of the waves' raw activations (two with three slots; one is enough with two, where the next pass is
+// asked for once this one's activations are in registers).
+template <class F, int NB, int SPP, int SLOTS, int XB>
 __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *__restrict__ A,
                                                       const int *__restrict__ gexp, const float *__restrict__ wts,
                                                       float *__restrict__ Y, int n, int k_used, int n_extra, int P) {
     static_assert(NB * SPP <= 16, "a pass is at most 16 super-block columns");
     static_assert(SLOTS == 2 || SLOTS == 3, "one or two passes ahead of the arithmetic");
-    constexpr int RB = NB * F::BLOCK, ROW_LDS = moe_mfma_row_lds(SPP * RB), LOADS = (RB + 1023) / 1024, STG = moe_mfma_stage<F>();
+    static_assert(XB == 2 || (XB == 1 && SLOTS == 2), "two passes in flight keep two activation buffers");
+    constexpr int RB = NB * F::BLOCK, ROW_LDS = moe_mfma_row_lds(SPP * RB), LOADS = (RB + 1023) / 1024, STG = moe_mfma_stage_only<F>();
     constexpr int LPF = SPP * LOADS + 1;  // loads a wave and pass: its row's segments and its activations
     static_assert(RB % 16 == 0, "rows are copied 16 bytes a lane");
     constexpr int MAX_S = 64;
@@ -382,11 +389,11 @@ __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *
     __shared__ int seg_pair[MAX_S];
     const uint64_t *table = qv_stage_table<F>(moe_mfma_lds);
     uint8_t *ring = moe_mfma_lds + qv_table_bytes<F>();            // [SLOTS][16][ROW_LDS]
-    float *xbuf = (float *)(ring + SLOTS * 16 * ROW_LDS);          // [2][16][256]
+    float *xbuf = (float *)(ring + SLOTS * 16 * ROW_LDS);          // [XB][16][256]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, c = lane >> 4;
-    uint32_t *stage = (uint32_t *)(ring + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + wave * STG);
-    float *part = (float *)(ring + SLOTS * 16 * ROW_LDS + 2 * 16 * 1024 + 16 * STG);  // [16][68]
+    uint32_t *stage = (uint32_t *)(ring + SLOTS * 16 * ROW_LDS + XB * 16 * 1024 + wave * STG);
+    float *part = (float *)(ring + SLOTS * 16 * ROW_LDS + XB * 16 * 1024 + 16 * STG);  // [16][68]
     // gridDim.z workgroups share a (token, row tile): number z takes passes z, z + gridDim.z, ..
     const int t = blockIdx.y, S = k_used + n_extra, Z = gridDim.z, z = blockIdx.z;
     const int NP = ((S + SPP - 1) / SPP - z + Z - 1) / Z;
@@ -417,7 +424,7 @@ __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *
             }
         }
         const int s = min(first + min(q, SPP - 1), S - 1);
-        async_load16(A + (size_t)seg_pair[s] * inter + 256 * blk + 4 * lane, xbuf0 + (uint32_t)(((i & 1) * 16 + wave) * 1024));
+        async_load16(A + (size_t)seg_pair[s] * inter + 256 * blk + 4 * lane, xbuf0 + (uint32_t)(((i % XB) * 16 + wave) * 1024));
     };
     fetch(0);
     if (SLOTS == 3 && NP > 1) fetch(1);
@@ -429,15 +436,15 @@ __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *
         asm volatile("" ::: "memory");
         const int s = (z + Z * i) * SPP + q;
         const bool live = worker && s < S;
-        float4 v = *(const float4 *)(xbuf + ((i & 1) * 16 + wave) * 256 + 4 * lane);
+        float4 v = *(const float4 *)(xbuf + ((i % XB) * 16 + wave) * 256 + 4 * lane);
         const float w = seg_wt[min(s, S - 1)];
-        v = float4{v.x * w, v.y * w, v.z * w, v.w * w};
-        const typename F::Acts acts = F::prepare(v, stage, lane);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (live) acc += qv_dot<F>(ring + ((i % SLOTS) * 16 + r) * ROW_LDS + q * RB + blk * F::BLOCK, acts, c, table);
         // every wave has passed this pass's barrier, so all are done with pass i - 1, whose slot the next pass to
         // ask for takes; this wave's activations of pass i are in registers and make room as well
         if (i + SLOTS - 1 < NP) fetch(i + SLOTS - 1);
+        v = float4{v.x * w, v.y * w, v.z * w, v.w * w};
+        const typename F::Acts acts = F::prepare(v, stage, lane);
+        if (live) acc += qv_dot<F>(ring + ((i % SLOTS) * 16 + r) * ROW_LDS + q * RB + blk * F::BLOCK, acts, c, table);
     }
     part[r * 68 + 4 * wave + c] = acc;
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
