@@ -39,12 +39,17 @@ CALIB_SRC = os.path.join(HERE, "calib", "copy_kernel.hip")
 CALIB_BIN = os.path.join(HERE, "calib", "copy_kernel")
 
 
+PROBE_SRC = os.path.join(HERE, "calib", "read_probe.hip")
+PROBE_BIN = os.path.join(HERE, "calib", "read_probe")
+
+
 def build_calibration() -> str:
-    """The copy kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
-    res = subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-o", CALIB_BIN, CALIB_SRC], capture_output=True,
-                         text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed:\n{res.stderr}")
+    """The copy kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters, and the plain-read probe that gives
+    the floor of one launch over a matrix of the benchmark's size."""
+    for src, out in ((CALIB_SRC, CALIB_BIN), (PROBE_SRC, PROBE_BIN)):
+        res = subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-o", out, src], capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed:\n{res.stderr}")
     return CALIB_BIN
 
 
