@@ -65,8 +65,12 @@ def cpu_baseline(blocks: np.ndarray, lhs: np.ndarray, budget_s: float) -> dict:
                       f"{threads} threads, 3 warm-up runs", "ms_per_step": round(med * 1e3, 4)}
 
 
-BLOCK = {8: (32, 34), 10: (256, 84), 12: (256, 144), 14: (256, 210), 16: (256, 66), 39: (32, 17)}
+BLOCK = {8: (32, 34), 10: (256, 84), 12: (256, 144), 14: (256, 210), 16: (256, 66), 39: (32, 17),
+         2: (32, 18), 3: (32, 20), 6: (32, 22), 7: (32, 24), 11: (256, 110), 13: (256, 176)}
+# the formats the reference serves through its canonical decode plus the 8-lane dot (src/quant_matmul.rs:228-248)
+F2_FORMATS = {2: "q4_0", 3: "q4_1", 6: "q5_0", 7: "q5_1", 11: "q3_k", 13: "q5_k"}
 F16_MFMA_PEAK_TFLOPS = 2500.0
+INT8_MFMA_PEAK_TOPS = 5000.0
 
 
 def _time_calls(torch, stream, fn, count: int) -> float:
@@ -117,7 +121,8 @@ def matmul_workload(torch, capi, synth, qtype: int, n: int, k: int, m: int, seed
     weight rows), and the oracle's AVX2 build is timed on the same product."""
     import oracle
     be, bb = BLOCK[qtype]
-    blocks = synth.normal_quantized(qtype, seed, n * k, 0.02)
+    # (formats without a quantiser here: seeded random blocks with scales of a N(0, 0.02) tensor's size)
+    blocks = synth.random_blocks(qtype, seed, n * k) if qtype in F2_FORMATS else synth.normal_quantized(qtype, seed, n * k, 0.02)
     lhs = synth.normal(seed + 100, (m, k))
     dev = torch.device("cuda:0")
     x = torch.from_numpy(lhs).to(dev)
@@ -140,6 +145,10 @@ def matmul_workload(torch, capi, synth, qtype: int, n: int, k: int, m: int, seed
         tflops = 2.0 * m * n * k / ms / 1e9
         res["useful_tflops"] = round(tflops, 1)
         res["mfma_frac_of_f16_peak"] = round(tflops / F16_MFMA_PEAK_TFLOPS, 4)
+        if "gemm_i8" in kernel:
+            # the many-row GEMM multiplies on the int8 matrix cores (two int8 planes of activations: two integer MACs a
+            # useful one); against that unit's dense peak, counting useful operations only
+            res["mfma_frac_of_int8_peak"] = round(tflops / INT8_MFMA_PEAK_TOPS, 4)
     got = y.cpu().numpy()
     avx2 = oracle.have_avx2()
     if m * n * k <= (1 << 32):
@@ -255,19 +264,28 @@ def mla_workload(torch, capi, synth, qtype: int, context: int, steps: int, seed:
           "kv_b": (qtype, blocks["kv_b"]), "o": (qtype, blocks["o"]),
           "kv_a_norm": np.ones(c["kv_lora_rank"], np.float32), "q_a_norm": np.ones(c["q_lora_rank"], np.float32)}
     ref = om.MlaOracle(oc, ot)
-    parity_ok = _close(mla.forward(xs_host[:64], 0), ref.forward(xs_host[:64], 0))
-    parity_ok = parity_ok and _close(mla.forward(xs_host[64:65], 64), ref.forward(xs_host[64:65], 64))
+    # parity at the order of the timed context: a prefill of min(context, 1024) tokens in chunks of 512 on both sides
+    # (the oracle's unabsorbed form takes ~15 s of host time for 1024 tokens), then single-token steps at that
+    # context, which also give the CPU figure; without a CPU budget a 64-token prefill and one step
+    pc = min(context, 1024) if cpu_seconds > 0 else 64
+    xp = synth.normal(seed + 11, (pc + 4, c["n_embd"]))
+    parity_ok, pos = True, 0
+    while pos < pc:
+        t = min(chunk, pc - pos)
+        parity_ok = _close(mla.forward(xp[pos:pos + t], pos), ref.forward(xp[pos:pos + t], pos)) and parity_ok
+        pos += t
     cpu = None
-    if cpu_seconds > 0:  # the oracle's single-token step, at the short context it can afford
-        import time
-        t_cpu = []
-        for p in range(65, 68):
-            t0 = time.perf_counter()
-            ref.forward(xs_host[p:p + 1], p)
-            t_cpu.append(time.perf_counter() - t0)
-        cpu = {"us": round(sorted(t_cpu)[1] * 1e6, 1), "cores": os.cpu_count(), "kind": "port",
-               "sample": "median of 3 single-token steps of oracle/mla.py (numpy, the reference's unabsorbed form over "
-                         "decoded weights) at a 65-67 token context; the device figure is at the full context"}
+    import time
+    t_cpu = []
+    for p in range(pc, pc + (3 if cpu_seconds > 0 else 1)):
+        t0 = time.perf_counter()
+        want = ref.forward(xp[p:p + 1], p)
+        t_cpu.append(time.perf_counter() - t0)
+        parity_ok = _close(mla.forward(xp[p:p + 1], p), want) and parity_ok
+    if cpu_seconds > 0:
+        cpu = {"us": round(sorted(t_cpu)[1] * 1e6, 1), "cores": os.cpu_count(), "kind": "port", "context": pc,
+               "sample": f"median of 3 single-token steps of oracle/mla.py (numpy, the reference's unabsorbed form over "
+                         f"decoded weights) at a context of {pc} tokens"}
     mla.reset()
     xs = torch.from_numpy(xs_host).to(dev)
     y = torch.zeros((chunk, c["n_embd"]), device=dev)
@@ -292,7 +310,9 @@ def mla_workload(torch, capi, synth, qtype: int, context: int, steps: int, seed:
     res = {"us": round(ms * 1e3, 2), "context": context, "algorithmic_bytes": abytes, "gbs": round(abytes / ms / 1e6, 1),
            "hbm_frac": round(abytes / ms / 1e6 / HBM_PEAK_GBS, 4),
            "prefill_tokens_per_s": round(context / prefill_ms * 1e3, 1),
-           "parity_ok": parity_ok, "parity_note": "64-token prefill and one step against the reference's unabsorbed form",
+           "parity_ok": parity_ok,
+           "parity_note": f"{pc}-token prefill in chunks of 512 and single-token steps at that context against the "
+                          "reference's unabsorbed form",
            "cache_bytes_per_token": 4 * (c["kv_lora_rank"] + c["qk_rope_head_dim"]),
            "reference_cache_bytes_per_token": 4 * nh * (qd + c["v_head_dim"])}
     if cpu:
@@ -324,6 +344,11 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
             out["q2_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 10, N, K, 512, 111, max(steps // 10, 10), 4, 0.0)
         elif only == "q2k":
             out["q2_k_gemv_14336x4096_m1"] = matmul_workload(torch, capi, synth, 10, N, K, 1, 108, steps, 24, 0.0)
+        elif only == "f2":
+            for qt, name in F2_FORMATS.items():
+                out[f"{name}_gemv_4096x4096_m1"] = matmul_workload(torch, capi, synth, qt, 4096, 4096, 1, 120 + qt, steps, 24, 0.0)
+                out[f"{name}_4096x4096_m512"] = matmul_workload(torch, capi, synth, qt, 4096, 4096, 512, 140 + qt,
+                                                                max(steps // 10, 10), 8, 0.0)
         elif only == "moe_b1":
             out["moe_qwen3_30b_a3b_q4_k_b1"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 1, 104, steps, False, 0, 0.0)
         elif only == "moe_b64":
@@ -348,6 +373,9 @@ def extra_workloads(steps: int, only: str = "", cpu_seconds: float = 0.0) -> dic
     out["q2_k_gemv_14336x4096_m1"] = matmul_workload(torch, capi, synth, 10, N, K, 1, 108, steps, 24, cs)
     out["q2_k_14336x4096_m512"] = matmul_workload(torch, capi, synth, 10, N, K, 512, 111, max(steps // 10, 10), 4, cs)
     out["q8_0_4096x4096_m512"] = matmul_workload(torch, capi, synth, 8, 4096, 4096, 512, 110, max(steps // 10, 10), 8, cs)
+    for qt, name in F2_FORMATS.items():   # (no CPU timing: the parity run is the oracle's sample here)
+        out[f"{name}_gemv_4096x4096_m1"] = matmul_workload(torch, capi, synth, qt, 4096, 4096, 1, 120 + qt, steps, 24, 0.0)
+        out[f"{name}_4096x4096_m512"] = matmul_workload(torch, capi, synth, qt, 4096, 4096, 512, 140 + qt, max(steps // 10, 10), 8, 0.0)
     torch.cuda.empty_cache()
     out["moe_qwen3_30b_a3b_q4_k_b1"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 1, 104, steps, False, 0, cs)
     out["moe_qwen3_30b_a3b_q4_k_b64"] = moe_workload(torch, capi, synth, 12, 2048, 768, 128, 8, 64, 104, max(steps // 10, 10),
@@ -375,7 +403,7 @@ QWEN3_8B = dict(n_layer=36, hidden=4096, n_head=32, n_kv_head=8, head_dim=128, f
                 rms_eps=1e-6, rope_theta=1e6)
 
 
-def decode_leg(prompt_len: int, n_decode: int, cpu_seconds: float, share_layers: bool) -> dict:
+def decode_leg(prompt_len: int, n_decode: int, cpu_seconds: float, share_layers: bool, prefill_parity: int = 0) -> dict:
     """End-to-end greedy decode of a random-init Qwen3-8B-shaped Q4_K_M model: prefill of
     prompt_len uniform-random ids, then n_decode greedy tokens, one host round trip per
     token (the engine's loop, reference: src/engine.rs:1149-1294).  The CPU leg runs the
@@ -417,7 +445,7 @@ def decode_leg(prompt_len: int, n_decode: int, cpu_seconds: float, share_layers:
     tps = (n_decode - 1) / t_dec
     res = {"tokens_per_s": round(tps, 2), "ms_per_token": round(1e3 / tps, 4),
            "prefill_tokens_per_s": round(prompt_len / t_prefill, 1),
-           "workload": f"Qwen3-8B-shaped random-init model, Q4_K_M mix (Q4_K + Q6_K), {prompt_len} uniform-random "
+           "workload": f"Qwen3-8B-shaped random-init model, weights N(0, 0.02), Q4_K_M mix (Q4_K + Q6_K + Q8_0), {prompt_len} uniform-random "
                        f"prompt ids then {n_decode} greedy tokens, batch 1, f32 activations and KV cache",
            "weight_bytes_per_token": wbytes, "weights_gbs": round(wbytes * tps / 1e9, 1),
            "hbm_frac": round(wbytes * tps / 1e9 / HBM_PEAK_GBS, 4),
@@ -461,6 +489,22 @@ def decode_leg(prompt_len: int, n_decode: int, cpu_seconds: float, share_layers:
                                              f"{n_pre}-token prefill, AVX2 row kernels, {threads} threads",
                                    "share_of_time_in_c_kernels": round(share, 3),
                                    "tokens_per_s_counting_kernel_time_only": round(cpu_tps / max(share, 1e-6), 3)}
+            if prefill_parity > 0:
+                # the many-row path at full size: the first `prefill_parity` prompt tokens in one step through all
+                # layers (int8 GEMMs, tiled attention) against the same graph over the oracle's kernels: the last
+                # token's logits over the whole vocabulary.  Minutes of host time at 512 tokens, so on request only.
+                n_pp = min(prefill_parity, prompt_len)
+                model.reset()
+                o.reset()
+                t0 = time.perf_counter()
+                ref_pp = o.forward(list(prompt[:n_pp]), 0)
+                t_ref = time.perf_counter() - t0
+                got_pp = model.forward(prompt[:n_pp], 0)
+                err = np.abs(got_pp - ref_pp) / np.maximum(np.abs(ref_pp), 1.0)
+                res["prefill_parity"] = {"tokens": n_pp, "logits_compared": int(ref_pp.size), "within_1e-3": bool(err.max() <= 1e-3),
+                                         "largest_error": float(err.max()), "greedy_equal": bool(oq.greedy(got_pp) == oq.greedy(ref_pp)),
+                                         "oracle_seconds": round(t_ref, 1)}
+                res["parity_ok"] = bool(res["parity_ok"] and err.max() <= 1e-3)
             res["speedup_vs_cpu"] = round(tps / cpu_tps, 2)
             res["speedup_vs_cpu_kernel_time_only"] = round(tps / (cpu_tps / max(share, 1e-6)), 2)
     model.close()
@@ -606,6 +650,9 @@ def main() -> int:
                     help="repetitions of the K timed steps whose median is reported (0: enough for ~30 ms, 5..400)")
     ap.add_argument("--plugin", type=int, default=0,
                     help="1: also write the model to a GGUF file and run it through the joshua_npu_* symbols")
+    ap.add_argument("--prefill-parity", type=int, default=0,
+                    help="N > 0: the decode leg also checks a one-step prefill of N prompt tokens of the 36-layer model against "
+                         "the oracle (minutes of host time at 512)")
     ap.add_argument("--plugin-moe", type=int, default=0,
                     help="N > 0: also write a Qwen3-30B-A3B-shaped qwen3moe GGUF of N layers (48 = the whole model) and run "
                          "it through the joshua_npu_* symbols")
@@ -689,11 +736,11 @@ def main() -> int:
         "metric": "Q4_K GEMV HBM GB/s (% of peak); decode tokens/s, 1 MI355X",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        # up to 64 rows: 4-bit weights x two int8 activation planes (v_dot4 for one row, int8 MFMA from two
-        # on; int32 sums), f32 scales and result; beyond: f16 MFMA GEMM
-        "dtype": "int8" if m <= 64 else "f16", "dtype_note": "integer dot products per 32-element sub-block "
-        "(int4 weights x 15-bit fixed-point activations in two int8 planes), f32 scales and accumulation across sub-blocks"
-        if m <= 64 else "f16 MFMA on exact integers (scale x nibble, 23-bit fixed-point activations in two planes), f32 result",
+        # 4-bit weights x two int8 activation planes on every path (v_dot4 or int8 MFMA, int32 sums), f32 scales and result
+        "dtype": "int8", "dtype_note": "integer dot products per 32-element sub-block (int4 weights x 15-bit fixed-point "
+        "activations in two int8 planes), f32 scales and accumulation across sub-blocks" if m < 64 else
+        "int8 MFMA GEMM (int4 weights unpacked to int8 x 15-bit fixed-point activations in two int8 planes, one scale per "
+        "256-element run), int32 sums per 32-element sub-block, f32 scales and accumulation across sub-blocks",
         "data": "synthetic",
         "config": {"workload": f"Q4_K matmul_t {N}x{K} (Llama-3-8B FFN-up), M={m}, f32 activations N(0,1), "
                                f"weights N(0,0.02) quantized to Q4_K, {len(weights)} weight copies rotated (cold HBM)",
@@ -720,7 +767,7 @@ def main() -> int:
         out["workloads"] = extra_workloads(min(max(steps, 100), 200), args.only, args.cpu_seconds)
         parity_ok = parity_ok and all(wl.get("parity_ok", True) for wl in out["workloads"].values())
     if args.decode:
-        out["decode"] = decode_leg(args.prompt, args.new_tokens, args.cpu_seconds, bool(args.share_layers))
+        out["decode"] = decode_leg(args.prompt, args.new_tokens, args.cpu_seconds, bool(args.share_layers), args.prefill_parity)
         parity_ok = parity_ok and out["decode"].get("parity_ok", True)
     if args.plugin:
         out["plugin"] = plugin_leg(args.prompt, args.new_tokens, bool(args.share_layers))

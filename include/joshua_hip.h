@@ -124,8 +124,10 @@ int jq_matmul_t(const jq_weight *w, size_t m, const float *lhs, size_t lhs_len, 
  * rounded to f16 (nearest even, overflow to infinity) (reference:
  * src/mmap_tensor.rs:136-138, :378-380, :451-453 matmul_t_f16; the wrappers
  * src/mxfp4.rs:242-258, src/iq2xxs.rs:396-412).  Same validation and empty case.  The
- * f32 operands live in stream-ordered allocations, freed in stream order: the call
- * cannot be captured into a HIP graph. */
+ * f32 operands live in a buffer the library keeps per stream (grown at first use, up
+ * to 64 MB; larger calls take a stream-ordered allocation): with device pointers, a
+ * call on a stream that has run one of its size before allocates nothing and can be
+ * captured into a HIP graph, as jq_matmul_t can. */
 int jq_matmul_t_f16(const jq_weight *w, size_t m, const uint16_t *lhs, size_t lhs_len, uint16_t *dst,
                     size_t dst_len, int ptrs_are_device, void *stream);
 

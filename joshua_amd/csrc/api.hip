@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <cstring>
 #include <map>
+#include <tuple>
 #include <memory>
 #include <set>
 #include <mutex>
@@ -496,24 +497,31 @@ struct StreamBuffer {
 };
 
 std::mutex g_stream_table_mu;
-std::map<std::pair<int, hipStream_t>, std::unique_ptr<StreamBuffer>> g_stream_table;
+// keyed by (device, stream, kind): kind 0 is what a product's launches hand to each other, kind 1 the f32 copies of
+// jq_matmul_t_f16's operands around such a product (which takes buffer 0 itself)
+std::map<std::tuple<int, hipStream_t, int>, std::unique_ptr<StreamBuffer>> g_stream_table;
 
 // jq_stream_release: waits for the stream, then frees its buffer and the retired ones.
 int release_stream_scratch(hipStream_t s) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
-    std::unique_ptr<StreamBuffer> b;
+    std::vector<std::unique_ptr<StreamBuffer>> bufs;
     {
         std::lock_guard<std::mutex> g(g_stream_table_mu);
-        auto it = g_stream_table.find({dev, s});
-        if (it == g_stream_table.end()) return 0;
-        b = std::move(it->second);
-        g_stream_table.erase(it);
+        for (int kind = 0; kind < 2; kind++) {
+            auto it = g_stream_table.find({dev, s, kind});
+            if (it == g_stream_table.end()) continue;
+            bufs.push_back(std::move(it->second));
+            g_stream_table.erase(it);
+        }
     }
-    { std::lock_guard<std::mutex> wait_for_the_last_holder(b->mu); }
+    if (bufs.empty()) return 0;
+    for (auto &b : bufs) { std::lock_guard<std::mutex> wait_for_the_last_holder(b->mu); }
     HIP_TRY(hipStreamSynchronize(s));
-    if (b->ptr) (void)hipFree(b->ptr);
-    for (uint8_t *p : b->retired) (void)hipFree(p);
+    for (auto &b : bufs) {
+        if (b->ptr) (void)hipFree(b->ptr);
+        for (uint8_t *p : b->retired) (void)hipFree(p);
+    }
     return 0;
 }
 
@@ -533,9 +541,11 @@ class CallScratch {
     std::unique_lock<std::mutex> lock_;
     hipStream_t stream_ = nullptr;
     uint8_t *transient_ = nullptr;
+    int kind_ = 0;
 
 public:
     CallScratch() = default;
+    explicit CallScratch(int kind) : kind_(kind) {}
     CallScratch(const CallScratch &) = delete;
     CallScratch &operator=(const CallScratch &) = delete;
     ~CallScratch() {
@@ -544,7 +554,7 @@ public:
     // 0 on success; on failure the message is set
     int get(size_t bytes, hipStream_t s, uint8_t **out) {
         stream_ = s;
-        if (const FixedScratch *f = tl_fixed_scratch) {
+        if (const FixedScratch *f = kind_ == 0 ? tl_fixed_scratch : nullptr) {
             if (bytes > f->bytes)
                 return fail("this product needs %zu bytes of scratch memory; the entry point that allocates nothing "
                             "holds %zu", bytes, f->bytes);
@@ -562,7 +572,7 @@ public:
         StreamBuffer *b;
         {
             std::lock_guard<std::mutex> g(g_stream_table_mu);
-            auto &slot = g_stream_table[{dev, s}];
+            auto &slot = g_stream_table[{dev, s, kind_}];
             if (!slot) slot.reset(new StreamBuffer);
             b = slot.get();
         }
@@ -1155,37 +1165,29 @@ int jq_matmul_t_f16(const jq_weight *w, size_t m, const uint16_t *lhs, size_t lh
     if (m == 0 || w->n == 0) return 0;
     if (!lhs || !dst) return fail("jq_matmul_t_f16: lhs/dst is null");
     hipStream_t s = (hipStream_t)stream;
-    // f16 -> f32, the f32 product, f32 -> f16 (reference: src/mxfp4.rs:242-258, src/iq2xxs.rs:396-412): the
-    // f32 operands live in stream-ordered allocations, so device callers are not synchronised
-    void *x32 = nullptr, *y32 = nullptr, *h16 = nullptr;
+    // f16 -> f32, the f32 product, f32 -> f16 (reference: src/mxfp4.rs:242-258, src/iq2xxs.rs:396-412): the f32
+    // operands live in the stream's second kept buffer (up to 64 MB; a stream-ordered allocation beyond), so
+    // device callers are not synchronised and a call on a warmed-up stream allocates nothing
     const size_t h16_bytes = ptrs_are_device ? 0 : std::max(lhs_len, dst_len) * sizeof(uint16_t);
-    auto release = [&] {
-        if (x32) (void)hipFreeAsync(x32, s);
-        if (y32) (void)hipFreeAsync(y32, s);
-        if (h16) (void)hipFreeAsync(h16, s);
-    };
-    hipError_t e = hipMallocAsync(&x32, lhs_len * sizeof(float), s);
-    if (e == hipSuccess) e = hipMallocAsync(&y32, dst_len * sizeof(float), s);
-    if (e == hipSuccess && h16_bytes) e = hipMallocAsync(&h16, h16_bytes, s);
-    if (e == hipSuccess && !ptrs_are_device) e = hipMemcpyAsync(h16, lhs, lhs_len * sizeof(uint16_t), hipMemcpyHostToDevice, s);
-    if (e != hipSuccess) {
-        release();
-        return fail("jq_matmul_t_f16: %s", hipGetErrorString(e));
-    }
+    const size_t x_bytes = (lhs_len * sizeof(float) + 255) & ~(size_t)255, y_bytes = (dst_len * sizeof(float) + 255) & ~(size_t)255;
+    CallScratch stage(1);
+    uint8_t *base = nullptr;
+    if (stage.get(x_bytes + y_bytes + h16_bytes, s, &base)) return 1;
+    float *x32 = (float *)base, *y32 = (float *)(base + x_bytes);
+    uint16_t *h16 = (uint16_t *)(base + x_bytes + y_bytes);
+    if (!ptrs_are_device) HIP_TRY(hipMemcpyAsync(h16, lhs, lhs_len * sizeof(uint16_t), hipMemcpyHostToDevice, s));
     const uint16_t *x16 = ptrs_are_device ? lhs : (const uint16_t *)h16;
-    uint16_t *y16 = ptrs_are_device ? dst : (uint16_t *)h16;
+    uint16_t *y16 = ptrs_are_device ? dst : h16;
     auto grid_of = [](size_t elems) { return (unsigned)std::min<size_t>((elems + 255) / 256, 65536); };
-    hipLaunchKernelGGL((jq::decode_plain<1>), dim3(grid_of(lhs_len)), dim3(256), 0, s, (const uint8_t *)x16, (float *)x32, lhs_len);
-    int rc = dispatch_matmul(w->type, w->dev, w->row_bytes, (const float *)x32, (float *)y32, m, w->k, w->n, s);
-    if (rc == 0) {
-        hipLaunchKernelGGL(jq::f32_to_f16, dim3(grid_of(dst_len)), dim3(256), 0, s, (const float *)y32, y16, dst_len);
-        e = hipGetLastError();
-        if (e == hipSuccess && !ptrs_are_device) e = hipMemcpyAsync(dst, h16, dst_len * sizeof(uint16_t), hipMemcpyDeviceToHost, s);
-        if (e == hipSuccess && !ptrs_are_device) e = hipStreamSynchronize(s);
-        if (e != hipSuccess) rc = fail("jq_matmul_t_f16: %s", hipGetErrorString(e));
+    hipLaunchKernelGGL((jq::decode_plain<1>), dim3(grid_of(lhs_len)), dim3(256), 0, s, (const uint8_t *)x16, x32, lhs_len);
+    if (dispatch_matmul(w->type, w->dev, w->row_bytes, x32, y32, m, w->k, w->n, s)) return 1;
+    hipLaunchKernelGGL(jq::f32_to_f16, dim3(grid_of(dst_len)), dim3(256), 0, s, (const float *)y32, y16, dst_len);
+    HIP_TRY(hipGetLastError());
+    if (!ptrs_are_device) {
+        HIP_TRY(hipMemcpyAsync(dst, h16, dst_len * sizeof(uint16_t), hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
     }
-    release();
-    return rc;
+    return 0;
 }
 
 int jq_matmul_t_noalloc(const jq_weight *w, size_t m, const float *lhs_dev, size_t lhs_len, float *dst_dev,

@@ -1,10 +1,11 @@
 """Random-weight Qwen3 decoder tensors in the block types a Q4_K_M GGUF holds.
 
 There is no network for checkpoints, so the end-to-end harness runs on seeded
-normal weights of the real architecture and tensor-type mix: everything Q4_K
-except the output head and, on the layers llama.cpp's Q4_K_M recipe gives more
-bits (first and last eighth, and every third in between), attn_v and ffn_down
-in Q6_K.  Norm weights are f32 around 1.
+normal weights N(0, 0.02) of the real architecture and tensor-type mix: everything
+Q4_K except the output head (Q6_K) and, on the layers llama.cpp's Q4_K_M recipe
+gives more bits (first and last eighth, and every third in between), ffn_down in
+Q6_K and attn_v in Q6_K or, on every other of those layers, Q8_0 (the three block
+types a Q4_K / Q6_K / Q8_0 file mixes).  Norm weights are f32 around 1.
 """
 from __future__ import annotations
 
@@ -14,7 +15,8 @@ import numpy as np
 
 from . import normal, normal_quantized
 
-Q4_K, Q6_K, F32 = 12, 14, 0
+Q4_K, Q6_K, Q8_0, F32 = 12, 14, 8, 0
+WEIGHT_SIGMA = 0.02
 
 
 def more_bits(layer: int, n_layer: int) -> bool:
@@ -33,9 +35,10 @@ def qwen3_tensor_plan(cfg: dict, mix: str = "q4_k_m"):
             ("output.weight", Q6_K if mix == "q4_k_m" else base, cfg["vocab"], h)]
     for l in range(L):
         hi = Q6_K if (mix == "q4_k_m" and more_bits(l, L)) else base
+        hi_v = Q8_0 if (hi == Q6_K and l % 2 == 1) else hi
         p = f"blk.{l}."
         plan += [(p + "attn_norm.weight", F32, h, 0), (p + "attn_q.weight", base, qd, h),
-                 (p + "attn_k.weight", base, kd, h), (p + "attn_v.weight", hi, kd, h),
+                 (p + "attn_k.weight", base, kd, h), (p + "attn_v.weight", hi_v, kd, h),
                  (p + "attn_q_norm.weight", F32, d, 0), (p + "attn_k_norm.weight", F32, d, 0),
                  (p + "attn_output.weight", base, h, qd), (p + "ffn_norm.weight", F32, h, 0)]
         if E:
@@ -73,5 +76,5 @@ def qwen3_tensors(cfg: dict, seed: int, mix: str = "q4_k_m", share_layers: bool 
             elif k == 0:
                 cache[key] = normal(s, (n,), 0.1, 1.0)
             else:
-                cache[key] = normal_quantized(qt, s, n * k, float(1.0 / np.sqrt(k)))
+                cache[key] = normal_quantized(qt, s, n * k, WEIGHT_SIGMA)
         yield name, qt, cache[key]

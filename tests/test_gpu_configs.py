@@ -55,7 +55,7 @@ def moe_layer(qtype, h, inter, n_expert, k_used, seed, shared, gating):
 def test_deepseek_v3_shaped_expert_layer(qtype):
     """h = 7168: IQ2_XXS rows of 1848 bytes (8-byte aligned only) and MXFP4 rows of 3808 bytes, 2048-wide
     experts, 256 routed experts + 1 shared, top-8, sigmoid gating (src/quantized_deepseek2.rs:520-559; expert
-    slices src/quantized_deepseek4.rs:2306-2331).  One token (the decode path with the fused down + combine)
+    slices src/quantized_deepseek4.rs:2306-2331).  One token (the decode path: the matrix-core expert kernels)
     and three tokens (27 pairs, still one group a pair)."""
     layer, ora = moe_layer(qtype, 7168, 2048, 256, 8, 500 + qtype, shared=True, gating="sigmoid")
     for tokens in (1, 3):
@@ -69,9 +69,9 @@ def test_deepseek_v3_shaped_expert_layer(qtype):
 
 @pytest.mark.parametrize("qtype,tokens,expert_dot8,kernel", [
     (capi.IQ2_XXS, 150, True, "moe_expert_dot8"), (capi.MXFP4, 90, True, "moe_expert_dot8"),
-    (capi.IQ2_XXS, 30, True, "moe_expert_dot8"), (capi.IQ2_XXS, 5, True, "moe_down_combine_dot8"),
+    (capi.IQ2_XXS, 30, True, "moe_expert_dot8"), (capi.IQ2_XXS, 5, True, "moe_down_mfma"),
     (capi.IQ2_XXS, 150, False, "moe_gemm_i8_few"), (capi.MXFP4, 90, False, "moe_gemm_i8_few"),
-    (capi.IQ2_XXS, 48, False, "moe_down_combine_dot8")])
+    (capi.IQ2_XXS, 48, False, "moe_down_mfma")])
 def test_deepseek_v3_shaped_expert_layer_over_a_prompt(monkeypatch, qtype, tokens, expert_dot8, kernel):
     """The same layer over a prompt, at the layer's own row lengths: gate and up of 7168 columns (28 super-blocks,
     224 units of 32: seven a lane), down of 2048.  150 tokens of IQ2_XXS (1200 routed pairs over 256 experts and the

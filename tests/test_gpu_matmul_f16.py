@@ -89,6 +89,37 @@ def test_device_pointers_give_the_host_result():
     assert np.array_equal(y.cpu().numpy(), host)
 
 
+def test_f16_product_on_a_warmed_up_stream_is_captured_into_a_graph():
+    """The f32 copies of the operands live in a buffer kept per stream: after one call of the size, the next
+    allocates nothing and goes into a HIP graph, which replays to the eager result with eager calls in between."""
+    import torch
+    n, k, m = 1536, 4096, 16
+    w = capi.Weight.upload(capi.Q6_K, synth.normal_quantized(capi.Q6_K, 41, n * k, 0.02), n, k)
+    x = torch.from_numpy(synth.normal(42, (m, k)).astype(np.float16)).cuda()
+    x2 = torch.from_numpy(synth.normal(43, (m, k)).astype(np.float16)).cuda()
+    y = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    y2 = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        w.matmul_t_f16_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), stream.cuda_stream)   # first use allocates
+        stream.synchronize()
+        want = y.clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            w.matmul_t_f16_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
+        for rep in range(3):
+            w.matmul_t_f16_dev(m, x2.data_ptr(), x2.numel(), y2.data_ptr(), y2.numel(), stream.cuda_stream)  # eager, same buffer
+            y.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, want), rep
+    assert not torch.equal(y2, want)
+    del graph
+    torch.cuda.synchronize()
+    capi.stream_release(stream.cuda_stream)
+
+
 def test_bad_lengths_are_refused_and_empty_products_succeed():
     n, k = 32, 256
     blocks = synth.normal_quantized(capi.Q4_K, 31, n * k, 0.02)

@@ -56,6 +56,10 @@ def test_q4_k_m_plan():
     assert plan["blk.0.attn_k.weight"] == (12, 128, 256)
     assert plan["blk.1.ffn_down.weight"][1:] == (256, 512)
     assert [more_bits(i, 36) for i in (0, 3, 4, 5, 6, 32, 35)] == [True, True, False, False, True, True, True]
+    # the layers with more bits: ffn_down Q6_K, attn_v Q6_K on the even ones and Q8_0 on the odd ones
+    big = {n: qt for n, qt, _, _ in qwen3_tensor_plan(dict(CFG, n_layer=36))}
+    assert (big["blk.0.attn_v.weight"], big["blk.1.attn_v.weight"], big["blk.4.attn_v.weight"]) == (14, 8, 12)
+    assert big["blk.1.ffn_down.weight"] == 14 and big["blk.1.attn_q.weight"] == 12
 
 
 def test_prefill_equals_token_by_token():
