@@ -1,7 +1,12 @@
 """Random-weight Qwen3 decoder tensors in the block types a Q4_K_M GGUF holds.
 
 There is no network for checkpoints, so the end-to-end harness runs on seeded
-normal weights N(0, 0.02) of the real architecture and tensor-type mix: everything
+normal weights of the real architecture and tensor-type mix, drawn N(0, 1/sqrt(k))
+for a matrix of k columns so that every product keeps its input's scale through
+all layers (at N(0, 0.02), 1.3 to 2.2 times that, the 36-layer model's logits
+differ from the CPU restatement's by up to 1.7e-3 of max(|ref|, 1): the 15-bit
+fixed point of the activations compounds past the 1e-3 a single product is held
+to; the bytes read are the same either way): everything
 Q4_K except the output head (Q6_K) and, on the layers llama.cpp's Q4_K_M recipe
 gives more bits (first and last eighth, and every third in between), ffn_down in
 Q6_K and attn_v in Q6_K or, on every other of those layers, Q8_0 (the three block
@@ -16,7 +21,6 @@ import numpy as np
 from . import normal, normal_quantized
 
 Q4_K, Q6_K, Q8_0, F32 = 12, 14, 8, 0
-WEIGHT_SIGMA = 0.02
 
 
 def more_bits(layer: int, n_layer: int) -> bool:
@@ -76,5 +80,5 @@ def qwen3_tensors(cfg: dict, seed: int, mix: str = "q4_k_m", share_layers: bool 
             elif k == 0:
                 cache[key] = normal(s, (n,), 0.1, 1.0)
             else:
-                cache[key] = normal_quantized(qt, s, n * k, WEIGHT_SIGMA)
+                cache[key] = normal_quantized(qt, s, n * k, float(1.0 / np.sqrt(k)))
         yield name, qt, cache[key]
