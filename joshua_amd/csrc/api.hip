@@ -380,6 +380,38 @@ int dispatch_q2k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
+// Q4_0, Q4_1, Q5_0, Q5_1 and Q5_K, one activation row, rows of 4096: the int8 matrix-core GEMV over the policy of
+// the formats whose units decode to int8 codes with a scale and an offset.  Returns -1 when the shape is outside its
+// reach (then the f32 row kernel runs).
+template <class Q>
+int launch_i8_gemv(const char *name, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n,
+                   hipStream_t s) {
+    typedef jq::QvI8<Q> F;
+    static const char *off = getenv("JQ_NO_I8_GEMV");
+    if (off || k != 4096 || row_bytes != (size_t)F::ROW || ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0 || n < 256 ||
+        n > 0x7FFFFFF0ull)
+        return -1;
+    const size_t tiles = (n + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
+    const jq::QvWork wk{(int)n, (int)G, (int)(tiles / G), (int)(tiles % G)};
+    note_kernel(name);
+    hipLaunchKernelGGL(jq::gemv_mfma_lds<F>, dim3((unsigned)G), dim3(1024), 0, s, W, X, Y, wk.n, wk.G, wk.rounds, wk.extra, nullptr,
+                       nullptr, 0.0f, nullptr, nullptr);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int dispatch_i8_gemv(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n,
+                     hipStream_t s) {
+    switch (type) {
+    case JQ_TYPE_Q4_0: return launch_i8_gemv<jq::Q4_0>("q4_0_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q4_1: return launch_i8_gemv<jq::Q4_1>("q4_1_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q5_0: return launch_i8_gemv<jq::Q5_0>("q5_0_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q5_1: return launch_i8_gemv<jq::Q5_1>("q5_1_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q5_K: return launch_i8_gemv<jq::Q5_K>("q5k_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    default: return -1;
+    }
+}
+
 // Q6_K, one activation row, rows of 4096, 8192 or 12288: the v_dot4 LDS-ring kernel.
 // Returns -1 when the shape is outside its reach.
 int dispatch_q6k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
@@ -925,6 +957,22 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         const int rc = dispatch_q8_0_dot4(W, row_bytes, X, Y, k, n, s);
         if (rc >= 0) return rc;
     }
+    if (m == 1) {
+        const int rc = dispatch_i8_gemv(type, W, row_bytes, X, Y, k, n, s);
+        if (rc >= 0) return rc;
+    }
+    // Q6_K and Q8_0 with two or three activation rows against a matrix of 16M weights or more: the one-row kernel
+    // once a row (4096 x 12288 of Q6_K, two rows: 23 us against 28 for the f32 row kernel; the int8 GEMM's 38 us
+    // are the same for 2 to 16 rows)
+    if ((type == JQ_TYPE_Q6_K || type == JQ_TYPE_Q8_0) && (m == 2 || m == 3) && n * k >= ((size_t)16 << 20)) {
+        static const char *no_loop = getenv("JQ_NO_ONE_ROW_LOOP");
+        int rc = no_loop ? -1 : 0;
+        for (size_t r = 0; r < m && rc == 0; r++)
+            rc = type == JQ_TYPE_Q6_K ? dispatch_q6k_dot4(W, row_bytes, X + r * k, Y + r * n, k, n, s)
+                                      : dispatch_q8_0_dot4(W, row_bytes, X + r * k, Y + r * n, k, n, s);
+        if (rc == 0) return 0;
+        if (rc > 0) return rc;  // (a kernel that declines does so at the first row, before anything is launched)
+    }
     // Q4_K with a few activation rows.  Rows of 4096, 1024 weight rows or more: the int8 matrix-core kernel
     // on the one-row kernel's weight stream, in passes of 16 activation rows.  Other row lengths: one or two
     // rows on the int8 GEMV further down; from three on the streaming kernel, whose time hardly depends on
@@ -960,7 +1008,10 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     // rows on, and from JQ_DECODED_GEMM_MIN_M rows on against matrices of 8M elements or more)
     static const char *dec_min_m_env = getenv("JQ_DECODED_GEMM_MIN_M");
     static const size_t gemm_min_m = dec_min_m_env ? (size_t)std::max(atoi(dec_min_m_env), 2) : 8;
-    const bool many_rows = m > Q4K_MFMA_MAX_M || (m >= gemm_min_m && n * k >= ((size_t)8 << 20));
+    // (the f32 row kernel's time grows with the row count, 12 us a row against 50M weights of Q6_K, the GEMM's does
+    // not: 38 us there, 22 us against 16M; it takes over from 4 rows against 32M weights or more, from 6 against 8M)
+    const size_t min_m = dec_min_m_env ? gemm_min_m : n * k >= ((size_t)32 << 20) ? 4 : 6;
+    const bool many_rows = m > Q4K_MFMA_MAX_M || (m >= min_m && n * k >= ((size_t)8 << 20));
     if (type == JQ_TYPE_Q6_K && many_rows) {
         const int rc = dispatch_gemm_i8<jq::QiQ6K>(W, row_bytes, X, Y, m, k, n, s, "q6k_gemm_i8", "q6k_gemm_i8+splitk", false, 2);
         if (rc >= 0) return rc;

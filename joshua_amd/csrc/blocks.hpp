@@ -239,6 +239,9 @@ struct Q8_0 {  // d:f16 | qs[32] i8   (reference: src/kquant_dot.rs:53-61,287-30
     }
 };
 
+// Bits 0..3 of b as bit 4 of bytes 0..3: the fifth bits of four 5-bit codes beside their nibbles.
+__device__ __forceinline__ uint32_t fifth_bits(uint32_t b) { return (((b & 0xFu) * 0x00204081u) & 0x01010101u) << 4; }
+
 // The 32-element formats with 4 or 5 bits a weight.  The reference has no kernel of its own for them:
 // they run through the canonical decode plus the 8-lane dot (reference: src/quant_matmul.rs:228-248);
 // the layouts are those of vendor/candle-metal-kernels/src/metal_src/quantized.metal:21-61 and the
@@ -259,6 +262,19 @@ struct Q4_0 {  // d:f16 | qs[16]        w = d (q - 8)
             w[j + 16] = d * (float)((b >> 4) - 8);
         }
     }
+    // The block as eight words of int8 (elements 4i .. 4i+3 in word i: the low nibbles' sixteen first), the codes as they
+    // are; w = scale code - offset.
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = true;
+    static constexpr int I8_UNITS = 1, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale, float &offset) {
+        const uint4 qv = ldw<uint4>(blk + 2);
+        const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (int)(q[i] & 0x0F0F0F0Fu), w[4 + i] = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+        scale = f16_bits(ld<uint16_t>(blk));
+        offset = 8.0f * scale;
+    }
 };
 
 struct Q4_1 {  // d:f16 | m:f16 | qs[16]        w = d q + m
@@ -273,6 +289,19 @@ struct Q4_1 {  // d:f16 | m:f16 | qs[16]        w = d q + m
             w[j] = fmaf(d, (float)(b & 0xF), m);
             w[j + 16] = fmaf(d, (float)(b >> 4), m);
         }
+    }
+    // The block as eight words of int8 (elements 4i .. 4i+3 in word i: the low nibbles' sixteen first), the codes as they
+    // are; w = scale code - offset.
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = true;
+    static constexpr int I8_UNITS = 1, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale, float &offset) {
+        const uint4 qv = ldw<uint4>(blk + 4);
+        const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (int)(q[i] & 0x0F0F0F0Fu), w[4 + i] = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+        scale = f16_bits(ld<uint16_t>(blk));
+        offset = -f16_bits(ld<uint16_t>(blk + 2));
     }
 };
 
@@ -290,6 +319,23 @@ struct Q5_0 {  // d:f16 | qh:u32 | qs[16]        w = d (q - 16)
             w[j + 16] = d * (float)(((b >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4)) - 16);
         }
     }
+    // The block as eight words of int8 (elements 4i .. 4i+3 in word i: the low nibbles' sixteen first), the codes as they
+    // are; w = scale code - offset.
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = true;
+    static constexpr int I8_UNITS = 1, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale, float &offset) {
+        const uint32_t qh = ldw<uint32_t>(blk + 2);
+        const uint4 qv = ldw<uint4>(blk + 6);
+        const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (int)((q[i] & 0x0F0F0F0Fu) | fifth_bits(qh >> (4 * i)));
+            w[4 + i] = (int)(((q[i] >> 4) & 0x0F0F0F0Fu) | fifth_bits(qh >> (16 + 4 * i)));
+        }
+        scale = f16_bits(ld<uint16_t>(blk));
+        offset = 16.0f * scale;
+    }
 };
 
 struct Q5_1 {  // d:f16 | m:f16 | qh:u32 | qs[16]        w = d q + m
@@ -305,6 +351,23 @@ struct Q5_1 {  // d:f16 | m:f16 | qh:u32 | qs[16]        w = d q + m
             w[j] = fmaf(d, (float)((b & 0xF) | (int)(((qh >> j) & 1u) << 4)), m);
             w[j + 16] = fmaf(d, (float)((b >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4)), m);
         }
+    }
+    // The block as eight words of int8 (elements 4i .. 4i+3 in word i: the low nibbles' sixteen first), the codes as they
+    // are; w = scale code - offset.
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = true;
+    static constexpr int I8_UNITS = 1, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale, float &offset) {
+        const uint32_t qh = ldw<uint32_t>(blk + 4);
+        const uint4 qv = ldw<uint4>(blk + 8);
+        const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (int)((q[i] & 0x0F0F0F0Fu) | fifth_bits(qh >> (4 * i)));
+            w[4 + i] = (int)(((q[i] >> 4) & 0x0F0F0F0Fu) | fifth_bits(qh >> (16 + 4 * i)));
+        }
+        scale = f16_bits(ld<uint16_t>(blk));
+        offset = -f16_bits(ld<uint16_t>(blk + 2));
     }
 };
 
@@ -450,6 +513,24 @@ struct Q5_K {  // d | dmin | scales[12] | qh[32] | qs[128]        w = d sc q - d
             w[l] = fmaf((float)((b & 0xF) | (((hb >> (2 * c)) & 1) << 4)), d0, -m0);
             w[32 + l] = fmaf((float)((b >> 4) | (((hb >> (2 * c + 1)) & 1) << 4)), d1, -m1);
         }
+    }
+    // Sub-block u (32 elements, eight a block) as eight words of int8: its 5-bit codes as they are, the scale d sc_u that
+    // goes with their sum and the offset dmin m_u that goes with the activations' sum.
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = true;
+    static constexpr int I8_UNITS = 8, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int u, int *w, float &scale, float &offset) {
+        const uint4 hdr = ld<uint4>(blk);
+        uint32_t sc, mn;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, u, sc, mn);
+        const uint4 qa = ld<uint4>(blk + 48 + 32 * (u >> 1)), qb = ld<uint4>(blk + 64 + 32 * (u >> 1));
+        const uint4 ha = ld<uint4>(blk + 16), hb = ld<uint4>(blk + 32);
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        const uint32_t h[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) w[i] = (int)(((q[i] >> (4 * (u & 1))) & 0x0F0F0F0Fu) | (((h[i] >> u) & 0x01010101u) << 4));
+        scale = f16_bits(hdr.x) * (float)sc;
+        offset = f16_bits(hdr.x >> 16) * (float)mn;
     }
 };
 

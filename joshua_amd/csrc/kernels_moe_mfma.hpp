@@ -16,6 +16,9 @@
 
 namespace jq {
 
+// LDS rows 16 bytes past a multiple of 256: the 16 rows a wave's lanes read side by side fall on all banks.
+constexpr int moe_mfma_row_lds(int bytes) { return (bytes + 255) / 256 * 256 + 16; }
+
 // The policy of the formats whose 32-element units decode to signed int8 words (Q::decode_i8: IQ2_XXS through its
 // codebook, MXFP4 through two byte permutes): a super-block is 256 consecutive elements, 8 units (one IQ2_XXS block,
 // eight MXFP4 blocks).  Lane (r, c) decodes units 2c and 2c + 1 of weight row r into the B operands of four MFMAs;
@@ -23,26 +26,32 @@ namespace jq {
 // Q4_K (row 4c + 2p + plane is non-zero in lane group c only), so the lane receives the two planes' sums of both
 // its units and   sum = scale(2c) s(2c) (256 Sh + Sl) + scale(2c + 1) s(2c + 1) (256 Sh' + Sl').
 // Every integer sum is exact (|w| <= 43, |X| <= 128, 32 terms).
+// Formats whose codes are unsigned with an offset (Q4_0 .. Q5_1, Q5_K: w = scale code - offset) add
+// - offset(2c) s(2c) sum X - offset(2c + 1) s(2c + 1) sum X'.  Also a policy of the one-row GEMV (gemv_mfma_lds,
+// gemv_mfma_cols) for the formats without a lookup table.
 template <class Q>
 struct QvI8 {
-    static_assert(Q::HAS_DECODE_I8 && !Q::I8_HAS_MIN, "units that decode to int8 words and a scale");
+    static_assert(Q::HAS_DECODE_I8, "units that decode to int8 words, a scale and an offset");
     static constexpr int SUB = 256 / Q::BLOCK_ELEMS;   // format blocks a super-block
     static_assert(SUB * Q::I8_UNITS == 8, "eight units of 32 elements a super-block");
-    static constexpr int BLOCK = SUB * Q::BLOCK_BYTES;
-    static constexpr int STAGE_BYTES = 4 * (128 + 8 + 8);  // the two planes, eight zero words, the sub-blocks' scales
-    static constexpr bool TAKES_TABLE = true;
+    static constexpr int BLOCK = SUB * Q::BLOCK_BYTES, ROW = 16 * BLOCK, ROW_LDS = moe_mfma_row_lds(ROW);
+    static constexpr int STAGE_BYTES = 4 * (128 + 8 + 16);  // the two planes, eight zero words, the sub-blocks' scales and scale x sum
+    static constexpr bool TAKES_TABLE = true, SIDE_LDS = false;
+    // the one-row GEMV's ring: three tiles of 16 rows where they fit beside its partial sums, else two
+    static constexpr int COLS = 4096, SLOTS = 3 * 16 * ROW_LDS + 20 * 1024 <= 160 * 1024 ? 3 : 2;
     typedef Q Format;
     struct Acts {
         qv_i4 a_even[2], a_odd[2];
-        float s_e, s_o;
+        float s_e, s_o, xs_e, xs_o;
     };
+    __device__ static __forceinline__ void scale(Acts &a, float f) { a.s_e *= f, a.s_o *= f, a.xs_e *= f, a.xs_o *= f; }
     __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) {
         const int r = lane & 15, c = lane >> 4;
         const QvQuant q = qv_quantise4(v);
         stage[lane] = q.wl, stage[64 + lane] = q.wh;
         if (lane < 8) stage[128 + lane] = 0;
         float *scales = (float *)(stage + 136);
-        if ((lane & 7) == 0) scales[lane >> 3] = q.s;
+        if ((lane & 7) == 0) scales[lane >> 3] = q.s, scales[8 + (lane >> 3)] = q.s * (float)q.sum;
         // (the words are written as scalars and read back as vectors: the compiler keeps the order only when told)
         asm volatile("" ::: "memory");
         // row m = r of A: lane group (r / 4) only, unit parity (r / 2) % 2, plane r % 2; the others read zeros
@@ -55,25 +64,30 @@ struct QvI8 {
         a.a_even[1] = qv_i4{(int)e1.x, (int)e1.y, (int)e1.z, (int)e1.w};
         a.a_odd[0] = qv_i4{(int)o0.x, (int)o0.y, (int)o0.z, (int)o0.w};
         a.a_odd[1] = qv_i4{(int)o1.x, (int)o1.y, (int)o1.z, (int)o1.w};
-        a.s_e = scales[2 * c], a.s_o = scales[2 * c + 1];
+        a.s_e = scales[2 * c], a.s_o = scales[2 * c + 1], a.xs_e = scales[8 + 2 * c], a.xs_o = scales[9 + 2 * c];
         asm volatile("" ::: "memory");
         return a;
     }
     __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c, const uint64_t *table) {
         int we[8], wo[8];
-        float se, so, off;
+        float se, so, oe, oo;
         if (SUB == 1) {
-            Q::decode_i8(table, blk, 2 * c, we, se, off);
-            Q::decode_i8(table, blk, 2 * c + 1, wo, so, off);
+            Q::decode_i8(table, blk, 2 * c, we, se, oe);
+            Q::decode_i8(table, blk, 2 * c + 1, wo, so, oo);
         } else {
-            Q::decode_i8(table, blk + (2 * c) * Q::BLOCK_BYTES, 0, we, se, off);
-            Q::decode_i8(table, blk + (2 * c + 1) * Q::BLOCK_BYTES, 0, wo, so, off);
+            Q::decode_i8(table, blk + (2 * c) * Q::BLOCK_BYTES, 0, we, se, oe);
+            Q::decode_i8(table, blk + (2 * c + 1) * Q::BLOCK_BYTES, 0, wo, so, oo);
         }
         qv_i4 C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_even[0], qv_i4{we[0], we[1], we[2], we[3]}, qv_i4{0, 0, 0, 0}, 0, 0, 0);
         C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_even[1], qv_i4{we[4], we[5], we[6], we[7]}, C, 0, 0, 0);
         C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_odd[0], qv_i4{wo[0], wo[1], wo[2], wo[3]}, C, 0, 0, 0);
         C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_odd[1], qv_i4{wo[4], wo[5], wo[6], wo[7]}, C, 0, 0, 0);
-        return fmaf(se * a.s_e, (float)((C[1] << 8) + C[0]), so * a.s_o * (float)((C[3] << 8) + C[2]));
+        float sum = fmaf(se * a.s_e, (float)((C[1] << 8) + C[0]), so * a.s_o * (float)((C[3] << 8) + C[2]));
+        if (Q::I8_HAS_MIN) sum -= fmaf(oe, a.xs_e, oo * a.xs_o);
+        return sum;
+    }
+    __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) {
+        return block_dot_lane(blk, a, c, nullptr);  // (the formats without a table)
     }
 };
 
@@ -98,8 +112,6 @@ __device__ __forceinline__ float qv_dot(const uint8_t *blk, const typename F::Ac
     else return F::block_dot_lane(blk, a, c);
 }
 
-// LDS rows 16 bytes past a multiple of 256: the 16 rows a wave's lanes read side by side fall on all banks.
-constexpr int moe_mfma_row_lds(int bytes) { return (bytes + 255) / 256 * 256 + 16; }
 // a wave's staging area: what the policy's prepare() uses, and in front of that the wave's 256 raw activations
 template <class F>
 constexpr int moe_mfma_stage() { return ((F::STAGE_BYTES > 1024 ? F::STAGE_BYTES : 1024) + 15) / 16 * 16; }

@@ -98,3 +98,39 @@ def test_mixture_of_experts_layer(qtype, tokens):
                    capi.Weight.upload(qtype, up, E * inter, h), capi.Weight.upload(qtype, down, E * h, inter))
     x = synth.normal(64, (tokens, h))
     assert close(dev.forward(x), ora.forward(x))
+
+
+I8_GEMV_KERNEL = {2: "q4_0_gemv_mfma_lds", 3: "q4_1_gemv_mfma_lds", 6: "q5_0_gemv_mfma_lds", 7: "q5_1_gemv_mfma_lds",
+                  13: "q5k_gemv_mfma_lds"}
+
+
+@pytest.mark.parametrize("qtype", sorted(I8_GEMV_KERNEL))
+def test_one_row_against_rows_of_4096_runs_on_the_int8_matrix_cores(qtype):
+    """One activation row against 256 weight rows or more of 4096 columns: the int8 matrix-core GEMV over the codes
+    as they are in the file, with the format's offset (-8 d, m, -16 d, dmin m) on the activations' sums.  A row
+    count that ends inside a tile of 16 and inside a workgroup's round; activations whose 32-element sub-blocks
+    differ by orders of magnitude (each has its own 15-bit fixed-point scale: tiny sub-blocks keep their digits, and
+    with a sub-block 10^4 times the others the error stays below 10^-4 of the sum of the terms' magnitudes; the
+    element-wise bound cannot hold there for the rows whose large terms cancel); a row of zeros; an
+    infinity (the whole result is NaN, as for every integer kernel)."""
+    k = 4096
+    for n in (256, 1000, 4099):
+        blocks = synth.random_blocks(qtype, 60 + qtype + n, n * k)
+        x = synth.normal(61 + n, (1, k))
+        x[0, 1024:1056] *= 1e-5
+        x[0, 2048:2080] *= 1e-2
+        w = capi.Weight.upload(qtype, blocks, n, k)
+        got = w.matmul_t(1, x)
+        assert capi.last_kernel() == I8_GEMV_KERNEL[qtype]
+        assert close(got, oracle.matmul_t(qtype, (1, k, n), x, blocks, avx2=oracle.have_avx2()))
+    dense = oracle.dequantize(qtype, blocks).reshape(n, k).astype(np.float64)
+    xb = x.copy()
+    xb[0, 96:128] *= 1e4
+    exact, terms = dense @ xb[0].astype(np.float64), np.abs(dense) @ np.abs(xb[0]).astype(np.float64)
+    assert np.all(np.abs(w.matmul_t(1, xb)[0] - exact) <= 1e-4 * terms)
+    only = np.zeros((1, k), np.float32)
+    only[0, 1024:1056] = x[0, 1024:1056]                                      # the tiny sub-block alone: its own digits
+    assert close(w.matmul_t(1, only) * 1e5, (dense @ only[0].astype(np.float64))[None, :] * 1e5, 1e-4)
+    assert np.array_equal(w.matmul_t(1, np.zeros((1, k), np.float32)), np.zeros((1, n), np.float32))
+    x[0, 7] = np.inf
+    assert np.all(np.isnan(w.matmul_t(1, x)))
