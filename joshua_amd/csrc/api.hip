@@ -380,13 +380,12 @@ int dispatch_q2k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
-// Q4_0, Q4_1, Q5_0, Q5_1 and Q5_K, one activation row, rows of 4096: the int8 matrix-core GEMV over the policy of
-// the formats whose units decode to int8 codes with a scale and an offset.  Returns -1 when the shape is outside its
+// Q4_0, Q4_1, Q5_0, Q5_1, Q5_K and Q3_K, one activation row, rows of 4096: the int8 matrix-core GEMV over the policy of
+// the formats whose units decode to int8 codes with a scale and an offset (Q3_K: two scales a unit, signed codes).  Returns -1 when the shape is outside its
 // reach (then the f32 row kernel runs).
-template <class Q>
+template <class F>
 int launch_i8_gemv(const char *name, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n,
                    hipStream_t s) {
-    typedef jq::QvI8<Q> F;
     static const char *off = getenv("JQ_NO_I8_GEMV");
     if (off || k != 4096 || row_bytes != (size_t)F::ROW || ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0 || n < 256 ||
         n > 0x7FFFFFF0ull)
@@ -403,11 +402,12 @@ int launch_i8_gemv(const char *name, const uint8_t *W, size_t row_bytes, const f
 int dispatch_i8_gemv(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n,
                      hipStream_t s) {
     switch (type) {
-    case JQ_TYPE_Q4_0: return launch_i8_gemv<jq::Q4_0>("q4_0_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
-    case JQ_TYPE_Q4_1: return launch_i8_gemv<jq::Q4_1>("q4_1_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
-    case JQ_TYPE_Q5_0: return launch_i8_gemv<jq::Q5_0>("q5_0_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
-    case JQ_TYPE_Q5_1: return launch_i8_gemv<jq::Q5_1>("q5_1_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
-    case JQ_TYPE_Q5_K: return launch_i8_gemv<jq::Q5_K>("q5k_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q4_0: return launch_i8_gemv<jq::QvI8<jq::Q4_0>>("q4_0_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q4_1: return launch_i8_gemv<jq::QvI8<jq::Q4_1>>("q4_1_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q5_0: return launch_i8_gemv<jq::QvI8<jq::Q5_0>>("q5_0_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q5_1: return launch_i8_gemv<jq::QvI8<jq::Q5_1>>("q5_1_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q5_K: return launch_i8_gemv<jq::QvI8<jq::Q5_K>>("q5k_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
+    case JQ_TYPE_Q3_K: return launch_i8_gemv<jq::QvQ3K>("q3k_gemv_mfma_lds", W, row_bytes, X, Y, k, n, s);
     default: return -1;
     }
 }

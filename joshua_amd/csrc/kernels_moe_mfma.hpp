@@ -91,6 +91,58 @@ struct QvI8 {
     }
 };
 
+// Q3_K on the same activation operands: w = d (sc - 32) (code - 4) with a 6-bit scale per 16 elements, so the four
+// MFMAs of a lane's chunk (16 elements each) keep accumulators of their own and each sum meets its scale in f32.
+// The 3-bit codes (two bits of qs, the third from hmask) go through one byte permute to the signed values -4 .. 3.
+// (layout: vendor/candle-metal-kernels/src/metal_src/quantized.metal:151-156, 6597-6623)
+struct QvQ3K {
+    typedef QvI8<Q5_K> Side;  // the activation side does not depend on the weights' format
+    static constexpr int BLOCK = 110, ROW = 16 * BLOCK, ROW_LDS = moe_mfma_row_lds(ROW), STAGE_BYTES = Side::STAGE_BYTES;
+    static constexpr bool SIDE_LDS = false;
+    static constexpr int COLS = 4096, SLOTS = 3;
+    typedef Side::Acts Acts;
+    __device__ static __forceinline__ void scale(Acts &a, float f) { Side::scale(a, f); }
+    __device__ static __forceinline__ Acts prepare(const float4 v, uint32_t *stage, int lane) { return Side::prepare(v, stage, lane); }
+    __device__ static __forceinline__ float block_dot_lane(const uint8_t *blk, const Acts &a, int c) {
+        // sub-blocks j = 2c (h = j / 4, field t = j % 4) and j + 1: the same half h and the field behind
+        const int h = c >> 1, t = 2 * (c & 1);
+        const uint4 qa = ldw<uint4>(blk + 32 + 32 * h), qb = ldw<uint4>(blk + 48 + 32 * h);   // elements i and 16 + i of a field
+        const uint4 ha = ldw<uint4>(blk), hb = ldw<uint4>(blk + 16);
+        const uint2 s8 = ldw<uint2>(blk + 96);
+        const uint32_t s4 = ldw<uint32_t>(blk + 104);
+        const float d = f16_bits(ld<uint16_t>(blk + 108));
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        const uint32_t hm[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+        const uint64_t lo8 = ((uint64_t)s8.y << 32) | s8.x;
+        int w[2][8];
+        float sc[2][2];
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            const int tt = t + p;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint32_t code = ((q[i] >> (2 * tt)) & 0x03030303u) | (((hm[i] >> (4 * h + tt)) & 0x01010101u) << 2);
+                w[p][i] = (int)__builtin_amdgcn_perm(0x03020100u, 0xFFFEFDFCu, code);
+            }
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                const int is = 8 * h + 2 * tt + hf;
+                const uint32_t low4 = (uint32_t)(lo8 >> (8 * (is & 7) + (is < 8 ? 0 : 4))) & 0xFu;
+                const uint32_t high2 = (s4 >> (8 * (is & 3) + 2 * (is >> 2))) & 3u;
+                sc[p][hf] = (float)((int)(low4 | (high2 << 4)) - 32);
+            }
+        }
+        const qv_i4 z = qv_i4{0, 0, 0, 0};
+        const qv_i4 C1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_even[0], qv_i4{w[0][0], w[0][1], w[0][2], w[0][3]}, z, 0, 0, 0);
+        const qv_i4 C2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_even[1], qv_i4{w[0][4], w[0][5], w[0][6], w[0][7]}, z, 0, 0, 0);
+        const qv_i4 C3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_odd[0], qv_i4{w[1][0], w[1][1], w[1][2], w[1][3]}, z, 0, 0, 0);
+        const qv_i4 C4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a.a_odd[1], qv_i4{w[1][4], w[1][5], w[1][6], w[1][7]}, z, 0, 0, 0);
+        const float even = fmaf(sc[0][0], (float)((C1[1] << 8) + C1[0]), sc[0][1] * (float)((C2[1] << 8) + C2[0]));
+        const float odd = fmaf(sc[1][0], (float)((C3[3] << 8) + C3[2]), sc[1][1] * (float)((C4[3] << 8) + C4[2]));
+        return d * fmaf(a.s_e, even, a.s_o * odd);
+    }
+};
+
 // Policies whose block_dot_lane wants the format's lookup table (a copy in LDS) as a fourth argument.
 template <class F, class = void>
 struct QvTakesTable : std::false_type {};

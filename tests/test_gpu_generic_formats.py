@@ -101,7 +101,7 @@ def test_mixture_of_experts_layer(qtype, tokens):
 
 
 I8_GEMV_KERNEL = {2: "q4_0_gemv_mfma_lds", 3: "q4_1_gemv_mfma_lds", 6: "q5_0_gemv_mfma_lds", 7: "q5_1_gemv_mfma_lds",
-                  13: "q5k_gemv_mfma_lds"}
+                  13: "q5k_gemv_mfma_lds", 11: "q3k_gemv_mfma_lds"}
 
 
 @pytest.mark.parametrize("qtype", sorted(I8_GEMV_KERNEL))
