@@ -713,12 +713,36 @@ int dispatch_q4k_rows16(const uint8_t *W, size_t row_bytes, const float *X, floa
     if (col_groups > 1 && m < 3) return -1;  // two rows: the two-row GEMV walks the matrix once
     static const char *genv = getenv("JQ_Q4K_ROWS16_GRID");
     const unsigned grid = (unsigned)std::min<size_t>(tiles, genv ? (size_t)std::max(atoi(genv), 1) : (tiles + rounds - 1) / rounds);
+    // rows of 4096 columns, one after the other: the streaming form of the kernel (JQ_Q4K_ROWS16_LDS = 0: the form before
+    // it; = own: the activations quantised by every workgroup for itself instead of by the preparation launch, which
+    // measured slower: every workgroup then reads all 16 rows of activations, 57 MB through the L2 for 224 workgroups)
+    static const char *lds_env = getenv("JQ_Q4K_ROWS16_LDS");
+    const bool lds_form = col_groups == 1 && row_bytes == (size_t)jq::QD_ROW && !genv && !(lds_env && lds_env[0] == '0');
+    const size_t rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
+    if (lds_form && lds_env && !strcmp(lds_env, "own")) {
+        note_kernel("q4k_rows16_lds");
+        for (size_t g = 0; g < groups; g++)
+            hipLaunchKernelGGL(jq::q4k_rows16_lds<true>, dim3((unsigned)G), dim3(1024), 0, s, W, X + 16 * g * k, nullptr,
+                               Y + 16 * g * n, (int)std::min<size_t>(16, m - 16 * g), (int)n, (int)G, (int)(tiles / G),
+                               (int)(tiles % G), (int)k);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
     CallScratch scratch;
     uint8_t *acts = nullptr;
     const size_t cols = k / 256, group_bytes = cols * (size_t)jq::QM_REC;
     if (scratch.get(groups * group_bytes, s, &acts)) return 1;
-    note_kernel("q4k_rows16_mfma");
     hipLaunchKernelGGL(jq::q4k_acts16_prep, dim3(8, (unsigned)cols, (unsigned)groups), dim3(64), 0, s, X, (int)m, (int)k, acts);
+    if (lds_form) {
+        note_kernel("q4k_rows16_lds");
+        for (size_t g = 0; g < groups; g++)
+            hipLaunchKernelGGL(jq::q4k_rows16_lds<false>, dim3((unsigned)G), dim3(1024), 0, s, W, X, (const uint8_t *)(acts + g * group_bytes),
+                               Y + 16 * g * n, (int)std::min<size_t>(16, m - 16 * g), (int)n, (int)G, (int)(tiles / G),
+                               (int)(tiles % G), (int)k);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
+    note_kernel("q4k_rows16_mfma");
     for (size_t g = 0; g < groups; g++)
         for (size_t cg = 0; cg < col_groups; cg++)
             hipLaunchKernelGGL(jq::q4k_rows16_mfma, dim3(grid), dim3(1024), 0, s, W + cg * (size_t)jq::QD_ROW,

@@ -1079,7 +1079,7 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 1, 7168, 1536, "q4k_gemv_mfma_cols"),        # DeepSeek-V3's query down-projection
     (capi.Q4_K, 1, 16384, 7168, "q4k_gemv_mfma_cols"),       # its attention output projection
     (capi.Q4_K, 2, 2048, 768, "q4k_gemv_mfma"),
-    (capi.Q4_K, 16, 4096, 14336, "q4k_rows16_mfma"),
+    (capi.Q4_K, 16, 4096, 14336, "q4k_rows16_lds"),
     (capi.Q4_K, 16, 2048, 768, "q4k_stream_mfma"),
     (capi.Q4_K, 512, 4096, 14336, "q4k_gemm_i8"),           # 256 tiles of 256 x 112
     (capi.Q4_K, 128, 4096, 14336, "q4k_gemm_i8+splitk"),    # 224 tiles of 128 x 64, two splits
