@@ -1964,18 +1964,20 @@ int dispatch_moe_down_mfma(const jq_moe *m, const float *A, float *y, int T, int
     const jq_moe_config &c = m->cfg;
     const int k = (int)c.inter, n = (int)c.hidden, k_used = (int)c.n_expert_used, S = k_used + n_extra;
     const uint32_t type = m->down->type;
-    const int bb = moe_mfma_block_bytes(type);
+    // (Q6_K: rows of three 210-byte blocks, the down projections of a Q4_K_M file's layers with more bits)
+    const int bb = type == JQ_TYPE_Q6_K ? jq::QvQ6K::BLOCK : moe_mfma_block_bytes(type);
     uintptr_t bits = (uintptr_t)m->down->dev | (uintptr_t)A;
     if (m->fold_shared) bits |= (uintptr_t)m->sdown->dev;
     static const char *only = getenv("JQ_MOE_MFMA_ONLY");
     if (off || (only && only[0] == 'g') || !bb || k % 256 != 0 || (bits & 15) != 0 || S > 64 || T <= 0 || T > 65535) return -1;
     const int nb = k / 256;
-    if (m->down->row_bytes != (size_t)nb * bb || nb > 16 || (type != JQ_TYPE_Q4_K && nb != 8)) return -1;
+    if (m->down->row_bytes != (size_t)nb * bb || nb > 16) return -1;
+    if (type == JQ_TYPE_Q6_K ? (nb != 3 || n % 16 != 0) : (type != JQ_TYPE_Q4_K && nb != 8)) return -1;
     const jq::MoeStack wd = moe_stack(m->down, c.hidden, c.n_expert, m->fold_shared ? m->sdown : nullptr);
-#define JQ_DN(F, NB, SPP, SL, XB)                                                                                       \
+#define JQ_DN(F, NB, SPP, SL, XB, ...)                                                                                       \
     do {                                                                                                              \
-        auto kern = jq::moe_down_mfma<F, NB, SPP, SL, XB>;                                                            \
-        constexpr int lds = jq::moe_down_mfma_lds<F, NB, SPP, SL, XB>();                                              \
+        auto kern = jq::moe_down_mfma<F, NB, SPP, SL, XB, ##__VA_ARGS__>;                                                            \
+        constexpr int lds = jq::moe_down_mfma_lds<F, NB, SPP, SL, XB, ##__VA_ARGS__>();                                              \
         static_assert(lds <= 158 * 1024, "the ring fits a compute unit");                                             \
         static const int attr_rc = moe_mfma_big_lds(kern, lds);                                                       \
         if (attr_rc) return 1;                                                                                        \
@@ -1988,6 +1990,8 @@ int dispatch_moe_down_mfma(const jq_moe *m, const float *A, float *y, int T, int
     // (IQ2_XXS: two slots and one activation buffer, 74 KB, two workgroups a compute unit)
     if (type == JQ_TYPE_IQ2_XXS) JQ_DN(jq::QvI8<jq::IQ2_XXS>, 8, 2, 2, 1);
     else if (type == JQ_TYPE_MXFP4) JQ_DN(jq::QvI8<jq::MXFP4>, 8, 2, 2, 2);
+    else if (type == JQ_TYPE_Q6_K && (S + 3) / 4 == (S + 4) / 5) JQ_DN(jq::QvQ6K, 3, 4, 2, 1, true);
+    else if (type == JQ_TYPE_Q6_K) JQ_DN(jq::QvQ6K, 3, 5, 2, 1, true);
     else if (nb == 3 && (S + 3) / 4 == (S + 4) / 5) JQ_DN(jq::QvQ4K, 3, 4, 3, 2);
     else if (nb == 3) JQ_DN(jq::QvQ4K, 3, 5, 2, 2);
     else if (nb == 8) JQ_DN(jq::QvQ4K, 8, 2, 2, 2);
@@ -2307,7 +2311,8 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     // tile add into it in the down projection
     bool y_cleared = false;
     if (rc < 0 && same_gu && max_group <= 1) {
-        const bool will_split = (m->fold_shared || !m->sgate) && m->down->type == JQ_TYPE_Q4_K && c.hidden <= 2048 &&
+        const bool will_split = (m->fold_shared || !m->sgate) && c.hidden <= 2048 && c.hidden % 16 == 0 &&
+                                (m->down->type == JQ_TYPE_Q4_K || (m->down->type == JQ_TYPE_Q6_K && c.inter == 768)) &&
                                 moe_down_mfma_splits(m, (int)T, extra);
         rc = dispatch_moe_gate_up_mfma(m, x, groups, s, clamp, will_split ? y : nullptr, will_split ? (int)(T * c.hidden) : 0,
                                        gate_later.logits ? &gate_later : nullptr);

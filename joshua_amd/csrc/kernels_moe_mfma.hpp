@@ -422,10 +422,15 @@ __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     return (const uint8_t *)(((uint64_t)hi << 32) | lo);
 }
 
-template <class F, int NB, int SPP, int SLOTS, int XB>
+// bytes of a ring slot: 16 rows of SPP segments, padded row by row, or (SPAN) the segments' 16 rows as they lie in memory
+template <class F, int NB, int SPP, bool SPAN>
+constexpr int moe_down_mfma_slot() {
+    return SPAN ? SPP * 16 * NB * F::BLOCK : 16 * moe_mfma_row_lds(SPP * NB * F::BLOCK);
+}
+template <class F, int NB, int SPP, int SLOTS, int XB, bool SPAN = false>
 constexpr int moe_down_mfma_lds() {
-    return qv_table_bytes<F>() + SLOTS * 16 * moe_mfma_row_lds(SPP * NB * F::BLOCK) + XB * 16 * 1024 + 16 * moe_mfma_stage_only<F>() +
-           16 * 68 * 4;
+    return qv_table_bytes<F>() + SLOTS * moe_down_mfma_slot<F, NB, SPP, SPAN>() + XB * 16 * 1024 + 16 * moe_mfma_stage_only<F>() +
+           16 * 68 * 4 + (SPAN ? 256 : 0);
 }
 
 // One workgroup per (token, 16 rows of the result).  The token's S = k_used + n_extra pairs are the segments of
@@ -436,28 +441,35 @@ constexpr int moe_down_mfma_lds() {
 // do not fit) with the waves' activations beside them, and a lane adds its chunk sums of all passes in a register.
 // XB: buffers of the waves' raw activations (two with three slots; one is enough with two, where the next pass is
 // asked for once this one's activations are in registers).
-template <class F, int NB, int SPP, int SLOTS, int XB>
+// SPAN: rows that are not a multiple of 16 bytes (Q6_K: 210-byte blocks).  The 16 rows of a segment's tile are one
+// span of memory that starts and ends on 16 bytes whatever the row length; all 1024 lanes copy it 16 bytes each and it
+// sits in LDS as in memory (n must be a multiple of 16).
+template <class F, int NB, int SPP, int SLOTS, int XB, bool SPAN = false>
 __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *__restrict__ A,
                                                       const int *__restrict__ gexp, const float *__restrict__ wts,
                                                       float *__restrict__ Y, int n, int k_used, int n_extra, int P) {
     static_assert(NB * SPP <= 16, "a pass is at most 16 super-block columns");
     static_assert(SLOTS == 2 || SLOTS == 3, "one or two passes ahead of the arithmetic");
     static_assert(XB == 2 || (XB == 1 && SLOTS == 2), "two passes in flight keep two activation buffers");
-    constexpr int RB = NB * F::BLOCK, ROW_LDS = moe_mfma_row_lds(SPP * RB), LOADS = (RB + 1023) / 1024, STG = moe_mfma_stage_only<F>();
-    constexpr int LPF = SPP * LOADS + 1;  // loads a wave and pass: its row's segments and its activations
-    static_assert(RB % 16 == 0, "rows are copied 16 bytes a lane");
+    constexpr int RB = NB * F::BLOCK, ROW_LDS = moe_mfma_row_lds(SPP * RB), STG = moe_mfma_stage_only<F>();
+    // load instructions a wave and segment: its row's kilobytes, or its share of the 16 RB / 16 pieces of a span
+    constexpr int LOADS = SPAN ? (RB + 1023) / 1024 : (RB + 1023) / 1024;
+    constexpr int LPF = SPP * LOADS + 1;  // loads a wave and pass: the segments and the wave's activations
+    constexpr int SLOT = moe_down_mfma_slot<F, NB, SPP, SPAN>();
+    static_assert(SPAN || RB % 16 == 0, "rows are copied 16 bytes a lane");
     constexpr int MAX_S = 64;
     extern __shared__ __attribute__((aligned(16))) uint8_t moe_mfma_lds[];
     __shared__ const uint8_t *seg_base[MAX_S];
     __shared__ float seg_wt[MAX_S];
     __shared__ int seg_pair[MAX_S];
     const uint64_t *table = qv_stage_table<F>(moe_mfma_lds);
-    uint8_t *ring = moe_mfma_lds + qv_table_bytes<F>();            // [SLOTS][16][ROW_LDS]
-    float *xbuf = (float *)(ring + SLOTS * 16 * ROW_LDS);          // [XB][16][256]
+    uint8_t *ring = moe_mfma_lds + qv_table_bytes<F>();            // [SLOTS][SLOT]
+    float *xbuf = (float *)(ring + SLOTS * SLOT);                  // [XB][16][256]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, c = lane >> 4;
-    uint32_t *stage = (uint32_t *)(ring + SLOTS * 16 * ROW_LDS + XB * 16 * 1024 + wave * STG);
-    float *part = (float *)(ring + SLOTS * 16 * ROW_LDS + XB * 16 * 1024 + 16 * STG);  // [16][68]
+    uint32_t *stage = (uint32_t *)(ring + SLOTS * SLOT + XB * 16 * 1024 + wave * STG);
+    float *part = (float *)(ring + SLOTS * SLOT + XB * 16 * 1024 + 16 * STG);  // [16][68]
+    const uint32_t dump0 = lds_offset_of(part + 16 * 68);          // (SPAN) where a wave without a piece of a span points its load
     // gridDim.z workgroups share a (token, row tile): number z takes passes z, z + gridDim.z, ..
     const int t = blockIdx.y, S = k_used + n_extra, Z = gridDim.z, z = blockIdx.z;
     const int NP = ((S + SPP - 1) / SPP - z + Z - 1) / Z;
@@ -474,17 +486,31 @@ __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *
     const uint32_t ring0 = lds_offset_of(ring), xbuf0 = lds_offset_of(xbuf);
     const int inter = 256 * NB;
     auto fetch = [&](int i) __attribute__((always_inline)) {
-        const uint32_t dst = ring0 + (uint32_t)((i % SLOTS) * 16 + wave) * ROW_LDS;
+        const uint32_t slot0 = ring0 + (uint32_t)(i % SLOTS) * SLOT;
         const int first = (z + Z * i) * SPP;  // the pass's first segment
 #pragma unroll
         for (int qq = 0; qq < SPP; qq++) {
             const int s = min(first + qq, S - 1);
-            const uint8_t *src = uniform_ptr(seg_base[s]) + (size_t)row * RB;
+            if (SPAN) {
+                const uint8_t *src = uniform_ptr(seg_base[s]) + (size_t)(16 * (int)blockIdx.x) * RB;
 #pragma unroll
-            for (int j = 0; j < LOADS; j++) {
-                constexpr int full = 64;
-                const int lanes = (RB - 1024 * j) / 16 < full ? (RB - 1024 * j) / 16 : full;
-                if (lane < lanes) async_load16_s(src + 1024 * j, 16 * lane, dst + qq * RB + 1024 * j);
+                for (int j = 0; j < LOADS; j++) {
+                    const int p0 = 64 * (wave + 16 * j), left = RB - p0;  // a span is RB pieces of 16 bytes
+                    if (left > 0) {
+                        if (lane < left) async_load16_s(src + 16 * (size_t)p0, 16 * lane, slot0 + qq * (16 * RB) + 16 * p0);
+                    } else if (lane == 0) {
+                        async_load16_s(src, 0, dump0 + 16 * wave);  // so that every wave counts the same loads
+                    }
+                }
+            } else {
+                const uint8_t *src = uniform_ptr(seg_base[s]) + (size_t)row * RB;
+                const uint32_t dst = slot0 + (uint32_t)wave * ROW_LDS;
+#pragma unroll
+                for (int j = 0; j < LOADS; j++) {
+                    constexpr int full = 64;
+                    const int lanes = (RB - 1024 * j) / 16 < full ? (RB - 1024 * j) / 16 : full;
+                    if (lane < lanes) async_load16_s(src + 1024 * j, 16 * lane, dst + qq * RB + 1024 * j);
+                }
             }
         }
         const int s = min(first + min(q, SPP - 1), S - 1);
@@ -508,7 +534,11 @@ __global__ __launch_bounds__(1024) void moe_down_mfma(MoeStack Wd, const float *
         if (i + SLOTS - 1 < NP) fetch(i + SLOTS - 1);
         v = float4{v.x * w, v.y * w, v.z * w, v.w * w};
         const typename F::Acts acts = F::prepare(v, stage, lane);
-        if (live) acc += qv_dot<F>(ring + ((i % SLOTS) * 16 + r) * ROW_LDS + q * RB + blk * F::BLOCK, acts, c, table);
+        if (live) {
+            const uint8_t *at = SPAN ? ring + (i % SLOTS) * SLOT + q * (16 * RB) + r * RB + blk * F::BLOCK
+                                     : ring + (i % SLOTS) * SLOT + r * ROW_LDS + q * RB + blk * F::BLOCK;
+            acc += qv_dot<F>(at, acts, c, table);
+        }
     }
     part[r * 68 + 4 * wave + c] = acc;
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

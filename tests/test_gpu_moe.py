@@ -340,3 +340,36 @@ def test_expert_kernel_at_seeded_random_layers(monkeypatch, qtype, h, inter, E, 
     got = dev.forward(x)
     assert capi.last_kernel() == "moe_expert_dot8", (h, inter, E, k, tokens)
     assert close(got, ora.forward(x))
+
+
+@pytest.mark.parametrize("tokens,shared", [(1, False), (3, False), (1, True)])
+def test_q4k_experts_with_a_q6k_down_projection(tokens, shared):
+    """The mix of a Q4_K_M file's layers with more bits: gate and up in Q4_K, down in Q6_K, rows of 768 (three
+    210-byte blocks: 630 bytes, a multiple of neither 4 nor 16).  Decode-sized calls take the matrix-core kernels for
+    both; the 16 rows of a down tile are copied as one span, which starts and ends on 16 bytes whatever the row."""
+    h, inter, E, k = 2048, 768, 16, 4
+    rw = synth.normal(700, (E, h), sigma=0.02)
+    gate = synth.normal_quantized(capi.Q4_K, 701, E * inter * h, 0.02)
+    up = synth.normal_quantized(capi.Q4_K, 702, E * inter * h, 0.02)
+    down = synth.normal_quantized(capi.Q6_K, 703, E * h * inter, 0.02)
+    sh_o = sh_w = None
+    if shared:   # a shared expert of the same types and shape rides along as one more pair
+        sg, su = (synth.normal_quantized(capi.Q4_K, 704 + i, inter * h, 0.02) for i in range(2))
+        sd = synth.normal_quantized(capi.Q6_K, 706, h * inter, 0.02)
+        sh_w = (capi.Weight.upload(capi.Q4_K, sg, inter, h), capi.Weight.upload(capi.Q4_K, su, inter, h),
+                capi.Weight.upload(capi.Q6_K, sd, h, inter))
+    ora = MoeOracle(capi.Q4_K, h, inter, E, k, rw, gate, up, down, avx2=oracle.have_avx2(), qtype_down=capi.Q6_K)
+    cfg = capi.MoeConfig(E, k, h, inter, 0, 1, 0.0, 1, 1, 0.0, 0.0)
+    dev = capi.Moe(cfg, rw, capi.Weight.upload(capi.Q4_K, gate, E * inter, h), capi.Weight.upload(capi.Q4_K, up, E * inter, h),
+                   capi.Weight.upload(capi.Q6_K, down, E * h, inter), shared=sh_w)
+    x = synth.normal(710 + tokens, (tokens, h))
+    got = dev.forward(x)
+    assert capi.last_kernel() == "moe_down_mfma"
+    want = ora.forward(x)
+    if shared:
+        sx = np.ascontiguousarray(x, np.float32)
+        g = oracle.matmul_t(capi.Q4_K, (tokens, h, inter), sx, sg, avx2=oracle.have_avx2())
+        u = oracle.matmul_t(capi.Q4_K, (tokens, h, inter), sx, su, avx2=oracle.have_avx2())
+        from oracle.moe import silu
+        want = want + oracle.matmul_t(capi.Q6_K, (tokens, inter, h), (silu(g) * u).astype(np.float32), sd, avx2=oracle.have_avx2())
+    assert close(got, want)
