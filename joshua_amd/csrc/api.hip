@@ -2265,10 +2265,13 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     // few tokens an expert (at most six on average): the int8 kernel that takes four rows an MFMA; more: the
     // f16 ring kernel, which reads a group's weights once for up to 16 rows
     const bool few = (size_t)P <= 6 * (size_t)c.n_expert;
-    // many tokens an expert (48 on average or more): the grouped int8 GEMM, which unpacks a weight tile once for
-    // 128 rows (Qwen3-30B-A3B sizes, 2048 tokens: 1.34 ms a call against the ring kernel's 2.03; equal at 512)
+    // many tokens an expert (16 on average or more): the grouped int8 GEMM, which unpacks a weight tile once for
+    // 128 rows (Qwen3-30B-A3B sizes, evenly routed tokens: 352 us a call of 256 tokens against the ring kernel's 324,
+    // 504 against 526 at 512, 1.19 ms against 2.03 at 2048).  The ring kernel walks an expert's rows once per 16 of its
+    // pairs, so its time follows the fullest expert, which the host does not know: 512 copies of one token (8 experts
+    // with 512 pairs each) take it 2.45 ms a layer and the GEMM 0.7, hence the GEMM from where the two are level.
     static const char *gemm_from_env = getenv("JQ_MOE_GEMM_FROM_PAIRS_PER_EXPERT");
-    const size_t gemm_from = gemm_from_env ? (size_t)atoll(gemm_from_env) : 48;
+    const size_t gemm_from = gemm_from_env ? (size_t)atoll(gemm_from_env) : 16;
     const bool prefer_gemm = m->gacts && max_group > 1 && (size_t)P >= gemm_from * (size_t)c.n_expert &&
                              c.hidden % 256 == 0 && c.inter % 256 == 0 && a16 >= 16 &&
                              align_of({m->down, m->fold_shared ? m->sdown : nullptr}) >= 16;
