@@ -1896,6 +1896,15 @@ bool moe_gate_up_mfma_takes(const jq_moe *m, const float *X) {
     return nb <= 32 && c.inter % 8 == 0 && pieces <= (iq2 ? 1024u : 2048u) && slot >= (size_t)nb * 1024 && lds <= 158 * 1024;
 }
 
+// MXFP4 and Q4_K rows that are whole 16-byte pieces of at most 4 KB travel row by row into padded LDS rows
+// (JQ_MOE_GATE_UP_SPANS: as spans of 8 rows like the other shapes).
+template <class F>
+bool moe_gate_up_rows_padded(int nb) {
+    static const char *spans = getenv("JQ_MOE_GATE_UP_SPANS");
+    const int rb = nb * F::BLOCK;
+    return !spans && rb % 16 == 0 && rb <= 4096 && jq::moe_gate_up_rows_mfma_lds<F, 2, 2, 2, true>(nb) <= 158 * 1024;
+}
+
 // `gate`: the launch runs the gating of the T tokens too (the router's logits are in m->logits).
 int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStream_t s, const jq::MoeClamp &cl, float *zero,
                               int zero_n, const jq::MoeGateIn *gate) {
@@ -1915,11 +1924,12 @@ int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStr
                            m->xrow, m->yrow, m->G, n, cl, zero, zero_n, gi);                                          \
     } while (0)
     // rows of more than 8 super-blocks: 16 waves a pair and tile sequence, two columns a wave
-#define JQ_GUR(F, SL, J, GATE)                                                                                        \
+#define JQ_GUR(F, SL, J, GATE) JQ_GUR_(F, SL, J, GATE, false)
+#define JQ_GUR_(F, SL, J, GATE, ROWS)                                                                                 \
     do {                                                                                                              \
-        auto kern = jq::moe_gate_up_rows_mfma<F, 2, SL, J, GATE>;                                                     \
-        const int lds = jq::moe_gate_up_rows_mfma_lds<F, 2, SL, J>(nb);                                               \
-        const int slot = (16 * nb * F::BLOCK + 15) / 16 * 16;                                                         \
+        auto kern = jq::moe_gate_up_rows_mfma<F, 2, SL, J, GATE, ROWS>;                                               \
+        const int lds = jq::moe_gate_up_rows_mfma_lds<F, 2, SL, J, ROWS>(nb);                                         \
+        const int slot = jq::moe_gate_up_rows_slot<F, ROWS>(nb);                                                      \
         if (lds > 158 * 1024 || (SL - 1) * slot < nb * 1024 || zero) return -1;                                   \
         static const int attr_rc = moe_mfma_big_lds(kern, 158 * 1024);                                                \
         if (attr_rc) return 1;                                                                                        \
@@ -1931,8 +1941,12 @@ int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStr
     if (nb > 8) {
         if (type == JQ_TYPE_IQ2_XXS && gate) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 2, 1, true);
         else if (type == JQ_TYPE_IQ2_XXS) JQ_GUR(jq::QvI8<jq::IQ2_XXS>, 2, 1, false);
+        else if (type == JQ_TYPE_MXFP4 && moe_gate_up_rows_padded<jq::QvI8<jq::MXFP4>>(nb) && gate) JQ_GUR_(jq::QvI8<jq::MXFP4>, 2, 2, true, true);
+        else if (type == JQ_TYPE_MXFP4 && moe_gate_up_rows_padded<jq::QvI8<jq::MXFP4>>(nb)) JQ_GUR_(jq::QvI8<jq::MXFP4>, 2, 2, false, true);
         else if (type == JQ_TYPE_MXFP4 && gate) JQ_GUR(jq::QvI8<jq::MXFP4>, 2, 2, true);
         else if (type == JQ_TYPE_MXFP4) JQ_GUR(jq::QvI8<jq::MXFP4>, 2, 2, false);
+        else if (moe_gate_up_rows_padded<jq::QvQ4K>(nb) && gate) JQ_GUR_(jq::QvQ4K, 2, 2, true, true);
+        else if (moe_gate_up_rows_padded<jq::QvQ4K>(nb)) JQ_GUR_(jq::QvQ4K, 2, 2, false, true);
         else if (gate) JQ_GUR(jq::QvQ4K, 2, 2, true);
         else JQ_GUR(jq::QvQ4K, 2, 2, false);
         note_kernel(gate ? "moe_gate_up_rows_mfma+gating" : "moe_gate_up_rows_mfma");
@@ -1953,6 +1967,7 @@ int dispatch_moe_gate_up_mfma(const jq_moe *m, const float *X, int pairs, hipStr
     else JQ_GU(jq::QvQ4K, 1, false);
 #undef JQ_GU
 #undef JQ_GUR
+#undef JQ_GUR_
     note_kernel(gate ? "moe_gate_up_mfma+gating" : "moe_gate_up_mfma");
     HIP_TRY(hipGetLastError());
     return 0;

@@ -305,12 +305,19 @@ __global__ __launch_bounds__(64 * NB) void moe_gate_up_mfma(MoeStack Wa, MoeStac
 // rows (8 consecutive rows of a matrix are one span of memory, copied 16 bytes a lane by all 1024 lanes: J
 // instructions a span and wave), and a lane adds its chunk sums of its columns in a register.
 // The raw activations (1 KB a column) wait in the ring's slots behind the first until they are prepared.
-template <class F, int NG, int SLOTS, int J>
+// ROWS: rows that are whole 16-byte pieces (at most 2 J KB long) travel row by row instead, wave w copying row w of
+// the 16, and sit in LDS 16 bytes past a multiple of 256 apart, so that the 16 rows a lane group reads side by side
+// fall on all banks (MXFP4 rows of 7168: 3808 bytes, where the rows of a span collide two by two).
+template <class F, bool ROWS>
+constexpr int moe_gate_up_rows_slot(int nb) {
+    return ROWS ? 16 * moe_mfma_row_lds(nb * F::BLOCK) : (16 * nb * F::BLOCK + 15) / 16 * 16;
+}
+template <class F, int NG, int SLOTS, int J, bool ROWS = false>
 constexpr int moe_gate_up_rows_mfma_lds(int nb) {
-    return qv_table_bytes<F>() + SLOTS * ((16 * nb * F::BLOCK + 15) / 16 * 16) + 1024 + 16 * moe_mfma_stage_only<F>() + 16 * 68 * 4;
+    return qv_table_bytes<F>() + SLOTS * moe_gate_up_rows_slot<F, ROWS>(nb) + 1024 + 16 * moe_mfma_stage_only<F>() + 16 * 68 * 4;
 }
 
-template <class F, int NG, int SLOTS, int J, bool GATE>
+template <class F, int NG, int SLOTS, int J, bool GATE, bool ROWS = false>
 __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeStack Wb, const float *__restrict__ X,
                                                               const int *__restrict__ gexp, const int *__restrict__ xrow,
                                                               const int *__restrict__ yrow, float *__restrict__ G, int inter,
@@ -320,7 +327,8 @@ __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeSt
     extern __shared__ __attribute__((aligned(16))) uint8_t moe_mfma_lds[];
     __shared__ int picked;
     const uint64_t *table = qv_stage_table<F>(moe_mfma_lds);
-    const int RB = nb * F::BLOCK, span = 8 * RB, slot_bytes = (2 * span + 15) / 16 * 16;  // 8 RB is a multiple of 16
+    const int RB = nb * F::BLOCK, span = 8 * RB;  // 8 RB is a multiple of 16
+    const int RS = ROWS ? moe_mfma_row_lds(RB) : RB, slot_bytes = moe_gate_up_rows_slot<F, ROWS>(nb);
     uint8_t *ring = moe_mfma_lds + qv_table_bytes<F>();
     uint8_t *dump = ring + SLOTS * slot_bytes;                       // where a wave without a piece of a span points its load
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -366,10 +374,23 @@ __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeSt
     if (GATE) e = __builtin_amdgcn_readfirstlane(picked);
     const uint8_t *wa = moe_expert_base(Wa, e), *wb = moe_expert_base(Wb, e);
     const uint32_t ring0 = lds_offset_of(ring), dump0 = lds_offset_of(dump);
-    const int pieces = span / 16;
+    const int pieces = (ROWS ? RB : span) / 16;
     auto fetch = [&](int i) __attribute__((always_inline)) {
         const size_t row0 = (size_t)8 * (b + (size_t)min(i, nt - 1) * G_);
         const uint32_t slot0 = ring0 + (uint32_t)(i % SLOTS) * slot_bytes;
+        if (ROWS) {
+            const uint8_t *src = (wave >= 8 ? wb : wa) + (row0 + (size_t)(wave & 7)) * RB;
+#pragma unroll
+            for (int j = 0; j < 2 * J; j++) {
+                const int first = 64 * j, left = pieces - first;  // this instruction's pieces of the wave's row
+                if (left > 0) {
+                    if (lane < left) async_load16_s(src + 16 * (size_t)first, 16 * lane, slot0 + wave * RS + 16 * first);
+                } else if (lane == 0) {
+                    async_load16_s(src, 0, dump0 + 16 * wave);  // so that every wave counts the same loads
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             const uint8_t *src = (half ? wb : wa) + row0 * RB;
@@ -399,7 +420,7 @@ __global__ __launch_bounds__(1024) void moe_gate_up_rows_mfma(MoeStack Wa, MoeSt
         float acc = 0.0f;
 #pragma unroll
         for (int cg = 0; cg < NG; cg++)
-            if (16 * cg + wave < nb) acc += qv_dot<F>(slot + r * RB + (16 * cg + wave) * F::BLOCK, acts[cg], c, table);
+            if (16 * cg + wave < nb) acc += qv_dot<F>(slot + r * RS + (16 * cg + wave) * F::BLOCK, acts[cg], c, table);
         part[r * 68 + 4 * wave + c] = acc;
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
