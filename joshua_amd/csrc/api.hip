@@ -29,6 +29,7 @@
 #include "kernels_dot4_q8.hpp"
 #include "kernels_moe.hpp"
 #include "kernels_moe_mfma.hpp"
+#include "kernels_gemv_mfma_tile.hpp"
 #include "kernels_mfma_q4k_ring.hpp"
 #include "kernels_moe_q4k_quads.hpp"
 #include "kernels_mfma_q4k_rows16.hpp"
@@ -295,6 +296,25 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     static const char *mode_env = getenv("JQ_Q4K_DOT4");
     static const std::string mode = mode_env ? mode_env : "auto";
     if (mode == "0" || nb == 0 || row_bytes % 16 != 0 || ((uintptr_t)W & 15) != 0 || ((uintptr_t)X & 15) != 0) return -1;
+    // rows of 8 super-blocks (a 2048-wide hidden size), 64 weight rows or more: one workgroup of 8 waves a tile of 16
+    // rows, with the decoder's norm form (4608 x 2048, q|k of a Qwen3-30B-A3B-shaped layer with residual add and RMSNorm:
+    // one launch where there were rmsnorm_rows and the one-shot matrix-core GEMV).  JQ_Q4K_GEMV_TILE = 0 switches it off.
+    static const char *tile_env = getenv("JQ_Q4K_GEMV_TILE");
+    if (mode == "auto" && !swiglu && !(tile_env && tile_env[0] == '0') && nb == 8 && k == 2048 && row_bytes == nb * 144 &&
+        n >= 64 && n <= 0x7FFFFFF0ull) {
+        const jq::QdNorm nm = norm ? *norm : jq::QdNorm{};
+        constexpr int lds = jq::gemv_mfma_tile_lds<jq::QvQ4K, 8>();
+        static_assert(lds <= 64 * 1024, "within the default dynamic LDS limit");
+        note_kernel("q4k_gemv_mfma_tile");
+        if (norm)
+            hipLaunchKernelGGL((jq::gemv_mfma_tile<jq::QvQ4K, 8, true>), dim3((unsigned)((n + 15) / 16)), dim3(512), lds, s, W, X, Y,
+                               (int)n, nm.res, nm.w, nm.eps, nm.x_out, nm.hn_out);
+        else
+            hipLaunchKernelGGL((jq::gemv_mfma_tile<jq::QvQ4K, 8, false>), dim3((unsigned)((n + 15) / 16)), dim3(512), lds, s, W, X, Y,
+                               (int)n, nullptr, nullptr, 0.0f, nullptr, nullptr);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
     // rows of more than 16 super-blocks (up to 64: rows of 4352 to 16384 columns, contiguous), 512 weight rows or
     // more: the matrix-core kernel over two to four passes of 16 columns (4096 x 12288, a feed-forward down
     // projection: 7.2 us, where v_dot4 kernels in steps of 8 and 16 rows took 8.9; 4096 x 8192 5.6 against 6.5;
@@ -2128,9 +2148,11 @@ int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, s
 // says whether it ran)
 // `gate_later`: when the gating can run by one wave a token, it is left to the caller's next kernel (the logits are
 // in m->logits) and *gate_later holds its operands; else it is cleared.
+// `pre`: the decoder layer's residual add and RMSNorm run inside the router launch (one token; x is then pre->hn_out,
+// which that launch writes).
 int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePairGroups pg,
                   jq::ActsI8 planes = jq::ActsI8{nullptr, nullptr, nullptr, nullptr}, bool *planes_made = nullptr,
-                  jq::MoeGateIn *gate_later = nullptr) {
+                  jq::MoeGateIn *gate_later = nullptr, const jq::MoePreNormArgs *pre = nullptr) {
     const jq_moe_config &c = m->cfg;
     const unsigned token_runs = (unsigned)((T + jq::ROUTER_TOKENS_PER_WG - 1) / jq::ROUTER_TOKENS_PER_WG);
     static const char *no_tile = getenv("JQ_MOE_NO_ROUTER_TILE");
@@ -2140,13 +2162,16 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
                          (int)c.n_group, (int)c.topk_group};
     static const char *no_wave = getenv("JQ_MOE_NO_WAVE_GATE");
     const bool wave_gate = !no_wave && c.n_group <= 1 && c.n_expert <= 256 && c.n_expert_used <= 64;
-    if (T >= tile_from && !no_tile)  // many tokens: a token's activations read once per eight experts (the same bits)
+    if (pre)
+        hipLaunchKernelGGL(jq::moe_router_logits_norm, dim3(c.n_expert), dim3(256), 0, s, m->router_w, *pre, m->logits,
+                           (int)c.hidden, (int)c.n_expert);
+    else if (T >= tile_from && !no_tile)  // many tokens: a token's activations read once per eight experts (the same bits)
         hipLaunchKernelGGL(jq::moe_router_logits_tile, dim3((c.n_expert + 7) / 8, (unsigned)((T + 7) / 8)), dim3(256), 0, s,
                            m->router_w, x, m->logits, (int)T, (int)c.hidden, (int)c.n_expert);
     else
         hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert, token_runs), dim3(256), 0, s, m->router_w, x, m->logits,
                            (int)T, (int)c.hidden, (int)c.n_expert, planes);
-    if (planes_made) *planes_made = planes.xl && !(T >= tile_from && !no_tile);
+    if (planes_made) *planes_made = !pre && planes.xl && !(T >= tile_from && !no_tile);
     size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);
     if (gate_later) {
         if (wave_gate) {
@@ -2174,7 +2199,15 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
     return 0;
 }
 
-int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s) {
+// The decoder's residual add and RMSNorm in front of a layer's mixture of experts: x_out = x + res,
+// hn_out = rmsnorm(x_out) w, and the experts run over hn_out.  `fused` says whether the router launch did it
+// (then the caller's residual row is x_out) or a launch of its own in place (then it is still x).
+struct MoePreNorm {
+    jq::MoePreNormArgs a;
+    bool fused;
+};
+
+int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s, MoePreNorm *pre = nullptr) {
     const jq_moe_config &c = m->cfg;
     const int P = (int)(T * c.n_expert_used), extra = m->fold_shared ? 1 : 0;
     // the experts' SwiGLU clamp; a folded shared expert is expert number n_expert and has its own
@@ -2233,12 +2266,27 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         // the matrix-core gate and up kernel can run the gating itself
         static const char *no_late_gate = getenv("JQ_MOE_NO_GATING_IN_GATE_UP");
         const bool late = !no_late_gate && m->gate->type == m->up->type && moe_gate_up_mfma_takes(m, x);
+        // one token of a decoder layer: the norm in front of the experts runs inside the router launch
+        static const char *no_pre = getenv("JQ_MOE_NO_NORM_IN_ROUTER");
+        if (pre) {
+            pre->fused = !no_pre && T == 1 && !planes.xl && c.hidden % 4 == 0 && x == pre->a.hn_out &&
+                         (((uintptr_t)pre->a.x | (uintptr_t)pre->a.res | (uintptr_t)pre->a.w | (uintptr_t)pre->a.x_out |
+                           (uintptr_t)pre->a.hn_out | (uintptr_t)m->router_w) & 15) == 0;
+            if (!pre->fused)
+                hipLaunchKernelGGL(jq::rmsnorm_rows, dim3((unsigned)T), dim3(1024), 0, s, (float *)pre->a.x, pre->a.res, pre->a.w,
+                                   pre->a.eps, pre->a.hn_out, (int)c.hidden);
+        }
         if (moe_route_dev(m, T, x, s, jq::MoePairGroups{m->gexp, m->offsets, m->xrow, m->yrow, extra}, planes, &planes_ready,
-                          late ? &gate_later : nullptr))
+                          late ? &gate_later : nullptr, pre && pre->fused ? &pre->a : nullptr))
             return 1;
         groups = P + extra * (int)T;
         max_group = 1;
     } else {
+        if (pre) {
+            pre->fused = false;
+            hipLaunchKernelGGL(jq::rmsnorm_rows, dim3((unsigned)T), dim3(1024), 0, s, (float *)pre->a.x, pre->a.res, pre->a.w,
+                               pre->a.eps, pre->a.hn_out, (int)c.hidden);
+        }
         if (moe_route_dev(m, T, x, s, jq::MoePairGroups{nullptr, nullptr, nullptr, nullptr, 0})) return 1;
         groups = (int)c.n_expert + extra;
         max_group = (int)T;
@@ -3230,12 +3278,17 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         if (model_mm(m, p + ".attn_output.weight", m->att, m->proj, T, s)) return 1;
         if (c.n_expert) {
             // x + moe(norm(x)) (reference: src/quantized_qwen3_moe.rs:806-812)
-            hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, m->proj, w_fn, c.rms_eps, m->hn, h);
             jq_moe *moe = m->moe[l];
             if (m->moe_scratch_at >= 0 && m->moe_scratch_at != (int)l && m->moe[m->moe_scratch_at])
                 moe_swap_scratch(moe, m->moe[m->moe_scratch_at]);
             m->moe_scratch_at = (int)l;
-            if (jq_moe_forward(moe, T, m->hn, m->proj, 1, s)) return 1;
+            // (the norm: inside the router launch for a single token, else a launch of its own in place)
+            MoePreNorm pre{jq::MoePreNormArgs{xc, m->proj, w_fn, c.rms_eps, xo, m->hn}, false};
+            {
+                std::lock_guard<std::mutex> lock(moe->mu);
+                if (moe_reserve(moe, T) || moe_forward_dev(moe, T, m->hn, m->proj, s, &pre)) return 1;
+            }
+            if (pre.fused) std::swap(xc, xo);
             pending = m->proj;
             continue;
         }

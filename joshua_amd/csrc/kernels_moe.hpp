@@ -94,6 +94,57 @@ __global__ __launch_bounds__(256) void moe_router_logits(const float *__restrict
     moe_router_logits_body(Wr, X, logits, T, h, E, planes);
 }
 
+// The router's logits of ONE token with the decoder layer's residual add and RMSNorm in front
+// (reference: src/quantized_qwen3_moe.rs:806-812: x + moe(norm(x))), a launch less: every workgroup adds res to x and
+// normalises the row for itself (h floats, read twice, the second time from cache), workgroup 0 stores x + res to
+// x_out (a buffer other than x: the others are still reading x) and the normalised row to hn_out, where the expert
+// kernels behind this launch read it.  Column c of the row goes to the thread that takes it in moe_router_logits, and
+// the logit is accumulated and reduced in the same order, so given the same normalised row the two give the same bits.
+struct MoePreNormArgs {
+    const float *x, *res, *w;
+    float eps;
+    float *x_out, *hn_out;
+};
+
+__global__ __launch_bounds__(256) void moe_router_logits_norm(const float *__restrict__ Wr, MoePreNormArgs nm,
+                                                               float *__restrict__ logits, int h, int E) {
+    __shared__ float red[2][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, e = blockIdx.x;
+    const float *wr = Wr + (size_t)e * h;
+    float ss = 0.0f;
+    for (int c = threadIdx.x * 4; c < h; c += 1024) {
+        float4 v = ld<float4>((const uint8_t *)(nm.x + c));
+        if (nm.res) {
+            const float4 r = ld<float4>((const uint8_t *)(nm.res + c));
+            v.x += r.x, v.y += r.y, v.z += r.z, v.w += r.w;
+        }
+        ss = fmaf(v.x, v.x, ss), ss = fmaf(v.y, v.y, ss), ss = fmaf(v.z, v.z, ss), ss = fmaf(v.w, v.w, ss);
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) red[0][wave] = ss;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf(((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / (float)h + nm.eps);
+    float acc = 0.0f;
+    for (int c = threadIdx.x * 4; c < h; c += 1024) {
+        float4 v = ld<float4>((const uint8_t *)(nm.x + c));
+        if (nm.res) {
+            const float4 r = ld<float4>((const uint8_t *)(nm.res + c));
+            v.x += r.x, v.y += r.y, v.z += r.z, v.w += r.w;
+        }
+        const float4 g = ld<float4>((const uint8_t *)(nm.w + c)), w = ld<float4>((const uint8_t *)(wr + c));
+        const float4 hn = float4{v.x * inv * g.x, v.y * inv * g.y, v.z * inv * g.z, v.w * inv * g.w};
+        if (e == 0) *(float4 *)(nm.x_out + c) = v, *(float4 *)(nm.hn_out + c) = hn;
+        acc = fmaf(hn.x, w.x, acc);
+        acc = fmaf(hn.y, w.y, acc);
+        acc = fmaf(hn.z, w.z, acc);
+        acc = fmaf(hn.w, w.w, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) red[1][wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) logits[e] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+}
+
 // The same logits for several tokens: one workgroup per (8 router rows, 8 tokens), so a token's activations are read
 // once per eight experts instead of once per expert (512 tokens x 256 experts of 7168: 228 -> 60 us).  Every
 // logit is accumulated by the same thread over the same columns in the same order as in moe_router_logits and

@@ -152,7 +152,7 @@ def q4k_integer_case(n, k, seed, group=16, big_value=4161407, small=65535):
 
 @pytest.mark.parametrize("m", [1, 2, 5, 16])
 def test_q4k_integer_dot_products_are_bit_exact(m):
-    n, k = 160, 2048
+    n, k = 160, 2048 if m > 1 else 1792   # (one row over rows of 2048 has a kernel and a test of its own)
     if m <= 2:   # int8 MFMA GEMV: activation range 4161407 per 16-element group
         blocks, q, x = q4k_integer_case(n, k, 90 + m)
     else:        # streaming f16 MFMA kernel: 4193279 per 256-element super-block
@@ -1075,7 +1075,8 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 1, 12288, 4096, "q4k_gemv_mfma_cols"),       # a feed-forward down projection
     (capi.Q4_K, 1, 8192, 2048, "q4k_gemv_mfma_cols"),
     (capi.Q4_K, 1, 8192, 8192, "q4k_gemv_mfma_cols"),        # more than one row tile a workgroup
-    (capi.Q4_K, 1, 2048, 768, "q4k_gemv_mfma"),              # an expert's gate projection
+    (capi.Q4_K, 1, 2048, 768, "q4k_gemv_mfma_tile"),         # an expert's gate projection; a 2048-wide model's projections
+    (capi.Q4_K, 1, 1024, 768, "q4k_gemv_mfma"),
     (capi.Q4_K, 1, 7168, 1536, "q4k_gemv_mfma_cols"),        # DeepSeek-V3's query down-projection
     (capi.Q4_K, 1, 16384, 7168, "q4k_gemv_mfma_cols"),       # its attention output projection
     (capi.Q4_K, 2, 2048, 768, "q4k_gemv_mfma"),
@@ -1118,6 +1119,43 @@ def test_kernel_chosen_for_a_shape(qtype, m, k, n, kernel):
     w.matmul_t_dev(m, x.data_ptr(), x.numel(), y.data_ptr(), y.numel(), torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert capi.last_kernel() == kernel
+
+
+# ---- Q4_K, one activation row over rows of 2048 columns: one workgroup of 8 waves a tile of 16 rows ----
+
+@pytest.mark.parametrize("n", [64, 100, 768 + 5, 4608, 16 * 300 + 9])
+def test_q4k_mfma_gemv_over_rows_of_2048(n):
+    """Whole and ragged last tiles, fewer and more tiles than compute units."""
+    k = 2048
+    blocks = make_blocks(capi.Q4_K, n, k, 500 + n % 89)
+    lhs = synth.normal(501, (1, k))
+    got = capi.Weight.upload(capi.Q4_K, blocks, n, k).matmul_t(1, lhs)
+    assert capi.last_kernel() == "q4k_gemv_mfma_tile"
+    assert close(got, oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+
+
+def test_q4k_mfma_gemv_over_rows_of_2048_integer_sums_and_odd_activations():
+    n, k = 1024 + 48, 2048
+    blocks, q, x = q4k_integer_case(n, k, 19, group=32, big_value=32639, small=4000)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    got = w.matmul_t(1, x[None, :].astype(np.float32))
+    assert capi.last_kernel() == "q4k_gemv_mfma_tile"
+    assert np.array_equal(got[0], (x @ q.T).astype(np.float32))
+    rng = np.random.default_rng(11)
+    blocks = make_blocks(capi.Q4_K, n, k, 504)
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    lhs = synth.normal(502, (1, k))
+    lhs[0] *= (10.0 ** rng.integers(-6, 7, size=k // 16)).repeat(16).astype(np.float32)
+    wd = oracle.dequantize(capi.Q4_K, blocks).reshape(n, k).astype(np.float64)
+    want, mag = wd @ lhs[0].astype(np.float64), np.abs(wd) @ np.abs(lhs[0].astype(np.float64))
+    got = w.matmul_t(1, lhs)[0].astype(np.float64)
+    assert np.all(np.abs(got - want) <= 2.0 ** -16 * mag)   # 16-bit fixed point per 32 elements
+    for bad in (np.inf, -np.inf, np.nan):
+        lhs = synth.normal(503, (1, k))
+        lhs[0, 777] = bad
+        assert np.all(np.isnan(w.matmul_t(1, lhs)))
+    w.matmul_t(1, np.zeros((1, k), np.float32))
+    assert np.array_equal(w.matmul_t(1, np.zeros((1, k), np.float32)), np.zeros((1, n), np.float32))
 
 
 # ---- Q4_K, one activation row over rows of 17 to 64 super-blocks: the matrix-core GEMV in passes of 16 columns ----

@@ -70,6 +70,22 @@ def test_single_token_steps_with_4096_wide_rows(mix):
         pos += 1
 
 
+@pytest.mark.parametrize("mix", ["q4_k_m", "q4_k"])
+def test_single_token_steps_with_2048_wide_rows(mix):
+    """hidden = 2048: residual add + RMSNorm + q|k(|v) of a single-token step are one launch of the kernel
+    that takes a tile of 16 rows a workgroup; gate, up and the rest run as launches of their own."""
+    cfg = dict(CFG, n_layer=4, hidden=2048, n_head=4, n_kv_head=2, head_dim=128, ffn=768, vocab=512, n_ctx=32)
+    m, o = make(cfg, 37, mix)
+    prompt = [3, 500, 41, 41, 256, 9]
+    ok, e = close(m.forward(prompt, 0), o.forward(prompt, 0))
+    assert ok, f"prefill: {e}"
+    pos = len(prompt)
+    for t in [5, 123, 511, 0, 350]:
+        ok, e = close(m.forward([t], pos), o.forward([t], pos))
+        assert ok, f"pos {pos}: {e}"
+        pos += 1
+
+
 def test_paired_gate_up_rows_serve_prefill_and_replacement():
     """With 4096-wide Q4_K rows the gate and up matrices are stored with alternating rows (the
     single-token launch applies SwiGLU itself); multi-token steps read them as strided views, and a

@@ -54,6 +54,27 @@ def test_plugin_serves_a_qwen3moe_gguf(tmp_path):
     p.close()
 
 
+def test_single_token_steps_with_2048_wide_rows(tmp_path):
+    """hidden = 2048 (Qwen3-30B-A3B's): a single-token step runs the attention block's norm inside the q|k launch and the
+    expert block's norm inside the router launch; steps of several tokens run them as launches of their own."""
+    cfg = dict(CFG, n_layer=3, hidden=2048, n_head=4, n_kv_head=2, head_dim=128, vocab=512, n_ctx=40, n_expert=16,
+               n_expert_used=4, expert_ffn=256)
+    path = tmp_path / "moe2048.gguf"
+    tensors = write_model(path, cfg, 67)
+    o = oq.Qwen3Oracle(cfg, tensors, avx2=oracle.have_avx2())
+    p = capi.NpuPlugin(str(path), cfg["n_ctx"])
+    assert p.rc == 0, capi.last_error()
+    prompt = [3, 500, 41, 41, 256, 9, 88]
+    rc, got = p.forward(prompt, 0)
+    assert rc == 0 and close(got, o.forward(prompt, 0)), capi.last_error()
+    pos = len(prompt)
+    for step in ([5], [123], [7, 8, 9], [511], [0]):
+        rc, got = p.forward(step, pos)
+        assert rc == 0 and close(got, o.forward(step, pos)), f"pos {pos}"
+        pos += len(step)
+    p.close()
+
+
 def test_configuration_of_a_qwen3moe_file(tmp_path):
     """The expert keys land in the configuration; attention.norm_topk_prob defaults to true when the file
     leaves it out and is honoured when false (reference: src/quantized_qwen3_moe.rs:119-134)."""
