@@ -385,6 +385,40 @@ int dispatch_q4k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float 
     return 0;
 }
 
+// y1 = W1 hn and y2 = W2 hn in one launch, hn = rmsnorm(x + res) w: W1 Q4_K with 2048 rows or more of 4096 columns
+// (the streaming kernel), W2 Q6_K or Q8_0 with few enough rows that G + n2 / 16 workgroups still run side by side.
+// Returns -1 when the shapes are outside its reach.  JQ_NO_NORM_PAIR switches it off.
+int dispatch_q4k_norm_pair(const uint8_t *W1, size_t row_bytes1, size_t n1, uint32_t type2, const uint8_t *W2, size_t row_bytes2,
+                           size_t n2, size_t k, const float *X, float *Y1, float *Y2, const jq::QdNorm &nm, hipStream_t s) {
+    static const char *off = getenv("JQ_NO_NORM_PAIR");
+    static const char *dot4 = getenv("JQ_Q4K_DOT4"), *mfma = getenv("JQ_Q4K_GEMV_MFMA"), *no_norm = getenv("JQ_NO_FUSED_NORM");
+    if (off || dot4 || mfma || no_norm || k != 4096 || row_bytes1 != (size_t)jq::QvQ4K::ROW || n1 < 2048 || n1 > 0x7FFFFFF0ull ||
+        n2 == 0 || n2 % 16 != 0 || nm.hn_out || !nm.x_out || !nm.w)
+        return -1;
+    if ((((uintptr_t)W1 | (uintptr_t)W2 | (uintptr_t)X | (uintptr_t)nm.w | (uintptr_t)nm.res | (uintptr_t)nm.x_out) & 15) != 0) return -1;
+    const size_t tiles = (n1 + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
+    const size_t tiles2 = n2 / 16;
+    if (G + tiles2 > 256) return -1;  // (one workgroup a compute unit: more would queue behind the streaming ones)
+    const jq::QvWork wk{(int)n1, (int)G, (int)(tiles / G), (int)(tiles % G)};
+#define JQ_PAIR(F2)                                                                                                        \
+    do {                                                                                                                   \
+        auto kern = jq::gemv_mfma_norm_pair<jq::QvQ4K, F2>;                                                                \
+        constexpr int lds = jq::gemv_mfma_norm_pair_lds<jq::QvQ4K, F2>();                                                  \
+        static_assert(lds <= 160 * 1024, "one workgroup's LDS");                                                          \
+        static const hipError_t attr_rc = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
+        HIP_TRY(attr_rc);                                                                                                  \
+        hipLaunchKernelGGL(kern, dim3((unsigned)(G + tiles2)), dim3(1024), lds, s, W1, X, Y1, wk.n, wk.G, wk.rounds, wk.extra, \
+                           nm.res, nm.w, nm.eps, nm.x_out, W2, Y2, (int)n2);                                               \
+    } while (0)
+    if (type2 == JQ_TYPE_Q6_K && row_bytes2 == 16 * 210) JQ_PAIR(jq::QvQ6K);
+    else if (type2 == JQ_TYPE_Q8_0 && row_bytes2 == 128 * 34) JQ_PAIR(jq::QvI8<jq::Q8_0>);
+    else return -1;
+#undef JQ_PAIR
+    note_kernel("q4k_gemv_mfma_lds+pair");
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 // Q2_K, one activation row, rows of 4096: the int8 matrix-core GEMV.  Returns -1 when the shape is outside
 // its reach.  JQ_Q2K_GEMV_MFMA = 0 switches it off.
 int dispatch_q2k_mfma(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
@@ -3210,10 +3244,24 @@ int model_forward_dev(jq_model *m, uint32_t T, uint32_t pos, hipStream_t s) {
         static const char *no_fused_prefill = getenv("JQ_NO_FUSED_QKV_PREFILL");
         // (the split attention kernel of steps up to 8 tokens reads q, k and v of a token as rows of their own)
         auto fqm = T > 1 && !split && !no_fused_prefill ? m->fused.find(p + ".qkv") : m->fused.end();
-        const bool v_fused = fq != m->fused.end() && fq->second->n == (size_t)(nh + 2 * nkv) * d;
-        // single token: residual add, norm and q|k(|v) as one launch when the kernel has that form
-        const bool normed = fq != m->fused.end() &&
-                            model_norm_mm(fq->second, xc, pending, w_an, c.rms_eps, xo, v_fused ? nullptr : m->hn, m->cat, false, s);
+        bool v_fused = fq != m->fused.end() && fq->second->n == (size_t)(nh + 2 * nkv) * d;
+        // single token: residual add, norm and q|k(|v) as one launch when the kernel has that form; an attn_v of
+        // another format (Q6_K, Q8_0) rides in the same launch where its tiles fit beside the q|k workgroups
+        bool normed = false;
+        if (fq != m->fused.end() && !v_fused && fq->second->type == JQ_TYPE_Q4_K) {
+            auto vw = m->q.find(p + ".attn_v.weight");
+            if (vw != m->q.end() && vw->second->k == fq->second->k && vw->second->n == (size_t)nkv * d) {
+                const jq_weight *w1 = fq->second, *w2 = vw->second;
+                const jq::QdNorm nm{pending, w_an, c.rms_eps, xo, nullptr};
+                const int rc = dispatch_q4k_norm_pair(w1->dev, w1->row_bytes, w1->n, w2->type, w2->dev, w2->row_bytes, w2->n, w1->k, xc,
+                                                      m->cat, m->cat + w1->n, nm, s);
+                if (rc > 0) return 1;
+                if (rc == 0) normed = v_fused = true;
+            }
+        }
+        if (!normed)
+            normed = fq != m->fused.end() &&
+                     model_norm_mm(fq->second, xc, pending, w_an, c.rms_eps, xo, v_fused ? nullptr : m->hn, m->cat, false, s);
         if (normed) std::swap(xc, xo);
         else hipLaunchKernelGGL(jq::rmsnorm_rows, dim3(T), dim3(1024), 0, s, xc, pending, w_an, c.rms_eps, m->hn, h);
         if (fq != m->fused.end()) {  // one launch for q|k(|v) of a single token

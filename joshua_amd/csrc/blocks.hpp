@@ -237,6 +237,17 @@ struct Q8_0 {  // d:f16 | qs[32] i8   (reference: src/kquant_dot.rs:53-61,287-30
             for (int b = 0; b < 4; b++) w[4 * i + b] = (float)(int8_t)(q[i] >> (8 * b)) * d;
         }
     }
+    // The block as eight words of int8: the codes as they are, w = scale code.
+    static constexpr bool HAS_DECODE_I8 = true, I8_HAS_MIN = false;
+    static constexpr int I8_UNITS = 1, I8_EXTRA_ENTRIES = 0;
+    __device__ static uint64_t i8_extra_entry(int) { return 0; }
+    __device__ static void decode_i8(const uint64_t *, const uint8_t *blk, int, int *w, float &scale, float &offset) {
+        const uint4 qa = ldw<uint4>(blk + 2), qb = ldw<uint4>(blk + 18);
+        w[0] = (int)qa.x, w[1] = (int)qa.y, w[2] = (int)qa.z, w[3] = (int)qa.w;
+        w[4] = (int)qb.x, w[5] = (int)qb.y, w[6] = (int)qb.z, w[7] = (int)qb.w;
+        scale = f16_bits(ld<uint16_t>(blk));
+        offset = 0.0f;
+    }
 };
 
 // Bits 0..3 of b as bit 4 of bytes 0..3: the fifth bits of four 5-bit codes beside their nibbles.

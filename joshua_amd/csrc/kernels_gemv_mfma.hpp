@@ -369,29 +369,45 @@ __device__ __forceinline__ void async_load16_s(const uint8_t *sbase, uint32_t vo
 //     arguments of their own so that the leading ones arrive preloaded.
 //   * SWIGLU: the matrix holds gate and up rows alternately (row 2j gate_j, row 2j + 1 up_j) and
 //     Y[j] = silu(gate_j . x) * (up_j . x), n / 2 values (reference: src/quantized_qwen3_moe.rs:397-401).
-template <class F, bool NORM = false, bool SWIGLU = false>
-__global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                      float *__restrict__ Y, int n, int G, int rounds, int extra,
-                                                      const float *nm_res, const float *nm_w, float nm_eps,
-                                                      float *nm_x_out, float *nm_hn_out) {
-    constexpr int SLOTS = F::SLOTS, FL = 4;          // ring slots (three: two tiles in flight); tiles a flush
+// The kernel's LDS, one block of bytes so that a launch which runs two kernels' bodies side by side can give both the
+// same block: the ring, the partial sums [FL][16][68], the waves' staging areas where the ring has no room for
+// them, the waves' sums of squares.
+template <class F>
+struct GemvMfmaLds {
+    static constexpr int FL = 4;                     // tiles a flush
+    static constexpr int STAGE = F::STAGE_BYTES + 1024;
+    static constexpr bool STAGE_IN_RING = STAGE <= F::ROW_LDS;
+    static constexpr int RING = F::SLOTS * 16 * F::ROW_LDS, PART = FL * 16 * 68 * 4;
+    static constexpr int STAGE_AT = RING + PART, SS_AT = STAGE_AT + (STAGE_IN_RING ? 16 : 16 * ((STAGE + 15) / 16 * 16));
+    static constexpr int BYTES = SS_AT + 64;
+};
+
+// `b`: the workgroup's number among the G of this product.
+template <class F, bool NORM, bool SWIGLU>
+__device__ __forceinline__ void gemv_mfma_lds_body(uint8_t *lds, int b, const uint8_t *__restrict__ W,
+                                                   const float *__restrict__ X, float *__restrict__ Y, int n, int G,
+                                                   int rounds, int extra, const float *nm_res, const float *nm_w,
+                                                   float nm_eps, float *nm_x_out, float *nm_hn_out) {
+    typedef GemvMfmaLds<F> L;
+    constexpr int SLOTS = F::SLOTS, FL = L::FL;      // ring slots (three: two tiles in flight); tiles a flush
     static_assert(!NORM || (2048 <= F::ROW_LDS && F::SLOTS == 3), "the norm's operands wait in a wave's row of ring slot 1");
-    __shared__ float ss_lds[16];
     constexpr int FULL = F::ROW / 1024, REST = (F::ROW - 1024 * FULL) / 16, LOADS = FULL + (REST ? 1 : 0);
-    __shared__ __attribute__((aligned(16))) uint8_t ring[SLOTS][16 * F::ROW_LDS];
-    __shared__ __attribute__((aligned(16))) float part[FL][16][68];
+    constexpr int SLOT_BYTES = 16 * F::ROW_LDS;
+    uint8_t *ring = lds;                             // [SLOTS][16 * ROW_LDS]
+    float *part = (float *)(lds + L::RING);          // [FL][16][68]
+    float *ss_lds = (float *)(lds + L::SS_AT);       // [16]
     // a wave's staging area (what prepare() needs, then its 256 raw activations): its own row of the last ring
     // slot when that is long enough, which no load targets before tile 2 is asked for in the main loop; else
     // memory of its own
-    constexpr int STAGE = F::STAGE_BYTES + 1024;
-    constexpr bool STAGE_IN_RING = STAGE <= F::ROW_LDS;
-    __shared__ __attribute__((aligned(16))) uint8_t stage_mem[STAGE_IN_RING ? 16 : 16 * STAGE];
+    constexpr int STAGE = (L::STAGE + 15) / 16 * 16;
+    constexpr bool STAGE_IN_RING = L::STAGE_IN_RING;
+    uint8_t *stage_mem = lds + L::STAGE_AT;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r = lane & 15, c = lane >> 4, b = (int)blockIdx.x;
+    const int r = lane & 15, c = lane >> 4;
     const int nt = rounds + (b < extra ? 1 : 0);  // tiles of this workgroup (no division in front of the first loads)
     if (nt <= 0) return;
     auto tile_row0 = [&](int i) __attribute__((always_inline)) { return 16 * (b + i * G); };
-    const uint32_t voff = 16 * lane, ring0 = lds_offset_of(&ring[0][0]);
+    const uint32_t voff = 16 * lane, ring0 = lds_offset_of(ring);
     // fetch(i) asks for tile min(i, nt - 1) into slot i % 3 (the fetches in front of the main loop are
     // unconditional, so that every wave counts the same loads); the row's address is scalar arithmetic
     auto fetch = [&](int slot_i) __attribute__((always_inline)) {
@@ -405,12 +421,12 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
     };
     // the raw activations travel like the tiles (every global read of this kernel is an asynchronous load
     // counted by hand)
-    uint32_t *stage = (uint32_t *)(STAGE_IN_RING ? &ring[SLOTS - 1][wave * F::ROW_LDS] : &stage_mem[wave * STAGE]);
+    uint32_t *stage = (uint32_t *)(STAGE_IN_RING ? ring + (SLOTS - 1) * SLOT_BYTES + wave * F::ROW_LDS : stage_mem + wave * STAGE);
     float *x_raw = (float *)((uint8_t *)stage + F::STAGE_BYTES);
     async_load16(X + 256 * wave + 4 * lane, lds_offset_of(x_raw));
     // norm weight and residual columns wait in the wave's row of ring slot 1, which no tile enters before the
     // activations are prepared
-    float *w_raw = (float *)&ring[1][wave * F::ROW_LDS], *r_raw = w_raw + 256;
+    float *w_raw = (float *)(ring + SLOT_BYTES + wave * F::ROW_LDS), *r_raw = w_raw + 256;
     if (NORM) {
         async_load16(nm_w + 256 * wave + 4 * lane, lds_offset_of(w_raw));
         if (nm_res) async_load16(nm_res + 256 * wave + 4 * lane, lds_offset_of(r_raw));
@@ -457,7 +473,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
             F::scale(acts, inv);
             if (b == 0 && nm_hn_out) *(float4 *)(nm_hn_out + 256 * wave + 4 * lane) = float4{v.x * inv, v.y * inv, v.z * inv, v.w * inv};
         }
-        part[t & (FL - 1)][r][4 * wave + c] = F::block_dot_lane(&ring[t % SLOTS][r * F::ROW_LDS + wave * F::BLOCK], acts, c);
+        part[((t & (FL - 1)) * 16 + r) * 68 + 4 * wave + c] =
+            F::block_dot_lane(ring + (t % SLOTS) * SLOT_BYTES + r * F::ROW_LDS + wave * F::BLOCK, acts, c);
         // every wave is done with tile t - 1, whose slot tile t + 2 takes; with two slots it takes tile t's own,
         // once every wave has read it
         if (t + 2 < nt) {
@@ -471,7 +488,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             const int tt = (t & ~(FL - 1)) + c;
-            const float4 p = *(const float4 *)&part[c][wave][4 * r];
+            const float4 p = *(const float4 *)&part[(c * 16 + wave) * 68 + 4 * r];
             float sum = (p.x + p.y) + (p.z + p.w);
             sum = sum_row16(sum);
             if (!SWIGLU) {
@@ -480,7 +497,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
                     if (row < n) Y[row] = sum;
                 }
             } else if ((wave & 1) == 0) {  // an even wave takes its gate row and the up row behind it
-                const float4 q = *(const float4 *)&part[c][wave + 1][4 * r];
+                const float4 q = *(const float4 *)&part[(c * 16 + wave + 1) * 68 + 4 * r];
                 float up = (q.x + q.y) + (q.z + q.w);
                 up = sum_row16(up);
                 if (r == 0 && tt <= t) {
@@ -490,6 +507,16 @@ __global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict_
             }
         }
     }
+}
+
+template <class F, bool NORM = false, bool SWIGLU = false>
+__global__ __launch_bounds__(1024) void gemv_mfma_lds(const uint8_t *__restrict__ W, const float *__restrict__ X,
+                                                      float *__restrict__ Y, int n, int G, int rounds, int extra,
+                                                      const float *nm_res, const float *nm_w, float nm_eps,
+                                                      float *nm_x_out, float *nm_hn_out) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[GemvMfmaLds<F>::BYTES];
+    gemv_mfma_lds_body<F, NORM, SWIGLU>(lds, (int)blockIdx.x, W, X, Y, n, G, rounds, extra, nm_res, nm_w, nm_eps, nm_x_out,
+                                        nm_hn_out);
 }
 
 // The same kernel for rows of more than 16 super-blocks (up to 16 NG): a tile is 16 rows x one pass of 16

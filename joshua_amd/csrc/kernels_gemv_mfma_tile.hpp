@@ -24,16 +24,16 @@ constexpr int gemv_mfma_tile_lds() {
     return qv_table_bytes<F>() + 16 * moe_mfma_row_lds(NB * F::BLOCK) + NB * gemv_mfma_tile_stage<F, NB>() + 16 * 68 * 4 + 64;
 }
 
+// `b`: the tile's number; `first`: this workgroup stores x + res and the normalised row.
 template <class F, int NB, bool NORM>
-__global__ __launch_bounds__(64 * NB) void gemv_mfma_tile(const uint8_t *__restrict__ W, const float *__restrict__ X,
-                                                          float *__restrict__ Y, int n, const float *nm_res,
-                                                          const float *nm_w, float nm_eps, float *nm_x_out,
-                                                          float *nm_hn_out) {
-    static_assert(NB == 2 || NB == 4 || NB == 8, "a row of 2, 4 or 8 super-blocks");
+__device__ __forceinline__ void gemv_mfma_tile_body(uint8_t *gemv_tile_lds, int b, bool first, const uint8_t *__restrict__ W,
+                                                    const float *__restrict__ X, float *__restrict__ Y, int n,
+                                                    const float *nm_res, const float *nm_w, float nm_eps, float *nm_x_out,
+                                                    float *nm_hn_out) {
+    static_assert(NB == 2 || NB == 4 || NB == 8 || NB == 16, "a row of 2, 4, 8 or 16 super-blocks");
     constexpr int RB = NB * F::BLOCK, ROW_LDS = moe_mfma_row_lds(RB), LOADS = (RB + 1023) / 1024;
     constexpr int STG = gemv_mfma_tile_stage<F, NB>(), RPW = 16 / NB;  // tile rows a wave copies
     static_assert(RB % 16 == 0, "rows are copied 16 bytes a lane");
-    extern __shared__ __attribute__((aligned(16))) uint8_t gemv_tile_lds[];
     const uint64_t *table = qv_stage_table<F>(gemv_tile_lds);
     uint8_t *tile = gemv_tile_lds + qv_table_bytes<F>();  // [16][ROW_LDS]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64 * NB) void gemv_mfma_tile(const uint8_t *__restr
         async_load16(nm_w + 256 * wave + 4 * lane, lds_offset_of(w_raw));
         if (nm_res) async_load16(nm_res + 256 * wave + 4 * lane, lds_offset_of(r_raw));
     }
-    const int row0 = 16 * (int)blockIdx.x;
+    const int row0 = 16 * b;
     const uint32_t tile0 = lds_offset_of(tile);
 #pragma unroll
     for (int i = 0; i < RPW; i++) {
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(64 * NB) void gemv_mfma_tile(const uint8_t *__restr
         ss = wave_sum(ss);
         if (lane == 0) ss_lds[wave] = ss;
         const float4 g = *(const float4 *)&w_raw[4 * lane];
-        if (blockIdx.x == 0) *(float4 *)(nm_x_out + 256 * wave + 4 * lane) = v;
+        if (first) *(float4 *)(nm_x_out + 256 * wave + 4 * lane) = v;
         v = float4{v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w};
     }
     typename F::Acts acts = F::prepare(v, stage, lane);
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(64 * NB) void gemv_mfma_tile(const uint8_t *__restr
         for (int i = 0; i < NB; i++) tot += ss_lds[i];
         const float inv = 1.0f / sqrtf(tot / (float)(256 * NB) + nm_eps);
         F::scale(acts, inv);
-        if (blockIdx.x == 0 && nm_hn_out)
+        if (first && nm_hn_out)
             *(float4 *)(nm_hn_out + 256 * wave + 4 * lane) = float4{v.x * inv, v.y * inv, v.z * inv, v.w * inv};
     }
     part[r * 68 + 4 * wave + c] = qv_dot<F>(tile + r * ROW_LDS + wave * F::BLOCK, acts, c, table);
@@ -99,6 +99,39 @@ __global__ __launch_bounds__(64 * NB) void gemv_mfma_tile(const uint8_t *__restr
         sum = wave_sum(sum);
         if (lane == 0 && row0 + rr < n) Y[row0 + rr] = sum;
     }
+}
+
+template <class F, int NB, bool NORM>
+__global__ __launch_bounds__(64 * NB) void gemv_mfma_tile(const uint8_t *__restrict__ W, const float *__restrict__ X,
+                                                          float *__restrict__ Y, int n, const float *nm_res,
+                                                          const float *nm_w, float nm_eps, float *nm_x_out,
+                                                          float *nm_hn_out) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemv_tile_lds[];
+    gemv_mfma_tile_body<F, NB, NORM>(gemv_tile_lds, (int)blockIdx.x, blockIdx.x == 0, W, X, Y, n, nm_res, nm_w, nm_eps, nm_x_out,
+                                     nm_hn_out);
+}
+
+// Two products over the same normalised activation row in one launch: Y1 = W1 hn on the streaming kernel
+// (gemv_mfma_lds, workgroups 0 .. G - 1) and Y2 = W2 hn, a smaller matrix of another format, one tile of 16 rows a
+// workgroup behind them (the decoder's q|k product of Q4_K beside an attn_v kept as Q6_K or Q8_0: a launch less).
+// Rows of 4096 columns.  Workgroup 0 stores x + res.
+template <class F1, class F2>
+constexpr int gemv_mfma_norm_pair_lds() {
+    return GemvMfmaLds<F1>::BYTES > gemv_mfma_tile_lds<F2, 16>() ? GemvMfmaLds<F1>::BYTES : gemv_mfma_tile_lds<F2, 16>();
+}
+
+template <class F1, class F2>
+__global__ __launch_bounds__(1024) void gemv_mfma_norm_pair(const uint8_t *__restrict__ W1, const float *__restrict__ X,
+                                                            float *__restrict__ Y1, int n1, int G, int rounds, int extra,
+                                                            const float *nm_res, const float *nm_w, float nm_eps,
+                                                            float *nm_x_out, const uint8_t *__restrict__ W2,
+                                                            float *__restrict__ Y2, int n2) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemv_tile_lds[];
+    const int b = (int)blockIdx.x;
+    if (b < G)
+        gemv_mfma_lds_body<F1, true, false>(gemv_tile_lds, b, W1, X, Y1, n1, G, rounds, extra, nm_res, nm_w, nm_eps, nm_x_out, nullptr);
+    else
+        gemv_mfma_tile_body<F2, 16, true>(gemv_tile_lds, b - G, false, W2, X, Y2, n2, nm_res, nm_w, nm_eps, nullptr, nullptr);
 }
 
 }  // namespace jq

@@ -86,6 +86,23 @@ def test_single_token_steps_with_2048_wide_rows(mix):
         pos += 1
 
 
+def test_single_token_steps_with_attn_v_of_another_format_in_the_qk_launch():
+    """hidden = 4096 and 2560 rows of q|k: on the layers that keep attn_v as Q6_K or Q8_0 (four of these eight, two of
+    each) its tiles run in the launch of residual add + RMSNorm + q|k, behind the workgroups of the Q4_K product."""
+    cfg = dict(CFG, n_layer=8, hidden=4096, n_head=16, n_kv_head=4, head_dim=128, ffn=512, vocab=512, n_ctx=32)
+    m, o = make(cfg, 39, "q4_k_m")
+    kinds = {o.t[f"blk.{l}.attn_v.weight"][0] for l in range(8)}
+    assert {capi.Q6_K, capi.Q8_0} <= kinds
+    prompt = [3, 500, 41, 41, 256, 9]
+    ok, e = close(m.forward(prompt, 0), o.forward(prompt, 0))
+    assert ok, f"prefill: {e}"
+    pos = len(prompt)
+    for t in [5, 123, 511, 0]:
+        ok, e = close(m.forward([t], pos), o.forward([t], pos))
+        assert ok, f"pos {pos}: {e}"
+        pos += 1
+
+
 def test_paired_gate_up_rows_serve_prefill_and_replacement():
     """With 4096-wide Q4_K rows the gate and up matrices are stored with alternating rows (the
     single-token launch applies SwiGLU itself); multi-token steps read them as strided views, and a
