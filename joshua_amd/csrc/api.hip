@@ -392,10 +392,29 @@ int dispatch_q4k_norm_pair(const uint8_t *W1, size_t row_bytes1, size_t n1, uint
                            size_t n2, size_t k, const float *X, float *Y1, float *Y2, const jq::QdNorm &nm, hipStream_t s) {
     static const char *off = getenv("JQ_NO_NORM_PAIR");
     static const char *dot4 = getenv("JQ_Q4K_DOT4"), *mfma = getenv("JQ_Q4K_GEMV_MFMA"), *no_norm = getenv("JQ_NO_FUSED_NORM");
-    if (off || dot4 || mfma || no_norm || k != 4096 || row_bytes1 != (size_t)jq::QvQ4K::ROW || n1 < 2048 || n1 > 0x7FFFFFF0ull ||
-        n2 == 0 || n2 % 16 != 0 || nm.hn_out || !nm.x_out || !nm.w)
-        return -1;
+    if (off || dot4 || mfma || no_norm || n2 == 0 || n2 % 16 != 0 || nm.hn_out || !nm.x_out || !nm.w) return -1;
     if ((((uintptr_t)W1 | (uintptr_t)W2 | (uintptr_t)X | (uintptr_t)nm.w | (uintptr_t)nm.res | (uintptr_t)nm.x_out) & 15) != 0) return -1;
+    // rows of 2048 columns: both products a tile of 16 rows a workgroup of 8 waves
+    static const char *tile_env = getenv("JQ_Q4K_GEMV_TILE");
+    if (k == 2048 && row_bytes1 == 8 * 144 && n1 >= 64 && n1 <= 0x7FFFFFF0ull && !(tile_env && tile_env[0] == '0')) {
+#define JQ_TPAIR(F2)                                                                                                       \
+    do {                                                                                                                   \
+        auto kern = jq::gemv_mfma_tile_norm_pair<jq::QvQ4K, F2, 8>;                                                        \
+        constexpr int lds = jq::gemv_mfma_tile_pair_lds<jq::QvQ4K, F2, 8>();                                               \
+        static const hipError_t attr_rc = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
+        HIP_TRY(attr_rc);                                                                                                  \
+        hipLaunchKernelGGL(kern, dim3((unsigned)((n1 + 15) / 16 + n2 / 16)), dim3(512), lds, s, W1, X, Y1, (int)n1, nm.res, nm.w, \
+                           nm.eps, nm.x_out, W2, Y2, (int)n2);                                                             \
+    } while (0)
+        if (type2 == JQ_TYPE_Q6_K && row_bytes2 == 8 * 210) JQ_TPAIR(jq::QvQ6K);
+        else if (type2 == JQ_TYPE_Q8_0 && row_bytes2 == 64 * 34) JQ_TPAIR(jq::QvI8<jq::Q8_0>);
+        else return -1;
+#undef JQ_TPAIR
+        note_kernel("q4k_gemv_mfma_tile+pair");
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
+    if (k != 4096 || row_bytes1 != (size_t)jq::QvQ4K::ROW || n1 < 2048 || n1 > 0x7FFFFFF0ull) return -1;
     const size_t tiles = (n1 + 15) / 16, rounds_up = (tiles + 255) / 256, G = (tiles + rounds_up - 1) / rounds_up;
     const size_t tiles2 = n2 / 16;
     if (G + tiles2 > 256) return -1;  // (one workgroup a compute unit: more would queue behind the streaming ones)

@@ -134,4 +134,25 @@ __global__ __launch_bounds__(1024) void gemv_mfma_norm_pair(const uint8_t *__res
         gemv_mfma_tile_body<F2, 16, true>(gemv_tile_lds, b - G, false, W2, X, Y2, n2, nm_res, nm_w, nm_eps, nullptr, nullptr);
 }
 
+// The same for rows of NB super-blocks: both products a tile of 16 rows a workgroup of NB waves, the tiles of W2 behind
+// those of W1.
+template <class F1, class F2, int NB>
+constexpr int gemv_mfma_tile_pair_lds() {
+    return gemv_mfma_tile_lds<F1, NB>() > gemv_mfma_tile_lds<F2, NB>() ? gemv_mfma_tile_lds<F1, NB>() : gemv_mfma_tile_lds<F2, NB>();
+}
+
+template <class F1, class F2, int NB>
+__global__ __launch_bounds__(64 * NB) void gemv_mfma_tile_norm_pair(const uint8_t *__restrict__ W1, const float *__restrict__ X,
+                                                                    float *__restrict__ Y1, int n1, const float *nm_res,
+                                                                    const float *nm_w, float nm_eps, float *nm_x_out,
+                                                                    const uint8_t *__restrict__ W2, float *__restrict__ Y2,
+                                                                    int n2) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemv_tile_lds[];
+    const int b = (int)blockIdx.x, t1 = (n1 + 15) / 16;
+    if (b < t1)
+        gemv_mfma_tile_body<F1, NB, true>(gemv_tile_lds, b, b == 0, W1, X, Y1, n1, nm_res, nm_w, nm_eps, nm_x_out, nullptr);
+    else
+        gemv_mfma_tile_body<F2, NB, true>(gemv_tile_lds, b - t1, false, W2, X, Y2, n2, nm_res, nm_w, nm_eps, nullptr, nullptr);
+}
+
 }  // namespace jq
