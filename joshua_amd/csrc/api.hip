@@ -1515,7 +1515,7 @@ struct jq_moe {
     uint8_t *gacts = nullptr;  // activations of the grouped int8 GEMM, and its tables
     int *gtab = nullptr;
     size_t gtab_rows = 0;      // row groups (and tiles) the tables hold
-    int gtile_rgs = 8;         // row groups a tile of the current plan: 8 (waves share the rows) or 2 (the weight rows)
+    int gtile_rgs = 8;         // row groups a tile of the current plan: 8 (waves share the rows), 2 (the weight rows), 0 (both: two launches)
     jq::ActsI8 qi8{nullptr, nullptr, nullptr, nullptr};  // activations as int8 planes (decode path, long rows)
     std::mutex mu;
 };
@@ -1590,7 +1590,7 @@ int moe_reserve(jq_moe *m, size_t T) {
         // row groups of 16 pairs that never mix two experts: at most PR / 16 + one part-filled group an expert
         m->gtab_rows = PR / 16 + c.n_expert + 2;
         HIP_TRY(hipMalloc((void **)&m->gacts, m->gtab_rows * (std::max<size_t>(c.hidden, c.inter) / 256 + 1) * jq::QI_REC));
-        HIP_TRY(hipMalloc((void **)&m->gtab, (5 * m->gtab_rows + 2) * sizeof(int)));
+        HIP_TRY(hipMalloc((void **)&m->gtab, (8 * m->gtab_rows + 4) * sizeof(int)));
     }
     if (m->sgate) {
         size_t si = m->sgate->n;
@@ -2125,7 +2125,12 @@ int dispatch_moe_rows(uint32_t type, const uint8_t *const *Wptr, size_t row_byte
 // Returns -1 when the matrix is outside its reach.
 jq::QiGroupTables moe_gemm_tables(const jq_moe *m) {
     const size_t R = m->gtab_rows;
-    return jq::QiGroupTables{m->gtab, m->gtab + R, m->gtab + 2 * R, m->gtab + 3 * R, m->gtab + 4 * R, m->gtab + 5 * R};
+    return jq::QiGroupTables{m->gtab, m->gtab + R, m->gtab + 2 * R, m->gtab + 3 * R, m->gtab + 4 * R, m->gtab + 8 * R};
+}
+// (the mixed plan's tiles of two row groups; their count sits where a launch looks for it: at counts[1])
+jq::QiGroupTables moe_gemm_tables_small(const jq_moe *m) {
+    const size_t R = m->gtab_rows;
+    return jq::QiGroupTables{m->gtab, m->gtab + R, m->gtab + 5 * R, m->gtab + 6 * R, m->gtab + 7 * R, m->gtab + 8 * R + 1};
 }
 
 template <class F>
@@ -2134,15 +2139,18 @@ int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, 
     if (!m->gacts || k % 256 != 0 || row_bytes % F::ALIGN != 0 || base_align < F::ALIGN) return -1;
     constexpr int NG = 4;
     const size_t nb = (size_t)k / 256, tx = ((size_t)n + 16 * NG - 1) / (16 * NG);
-    const size_t max_rg = m->gtab_rows, max_mt = m->gtab_rows;
-    if (tx * max_mt > 0x7FFFFFFFull) return -1;
+    const size_t max_rg = m->gtab_rows;
+    if (tx * max_rg > 0x7FFFFFFFull) return -1;
     const jq::QiGroupTables t = moe_gemm_tables(m);
     if (!prepared)
         hipLaunchKernelGGL((jq::moe_gemm_i8_prep<F::SUB16>), dim3((unsigned)nb, (unsigned)max_rg), dim3(256), 0, s, X, xsel, t, k,
                            m->gacts);
     constexpr int lds = jq::qi_lds_bytes<F, NG>();
-    const jq::QiGrouped gp{wptr, m->gexp, m->yrow, t};
     hipError_t attr_rc = hipSuccess;
+    // most tiles a plan can hold: every tile of the mixed plan's first list has five row groups or more, its second
+    // list at most two tiles an expert
+    const size_t n_groups = m->cfg.n_expert + (m->fold_shared ? 1 : 0);
+    const size_t max_big = m->gtile_rgs == 0 ? max_rg / 5 + 1 : max_rg, max_small = m->gtile_rgs == 0 ? 2 * n_groups : max_rg;
 #define JQ_MOE_GEMM(NW_, NSPLIT_)                                                                                     \
     do {                                                                                                              \
         auto kern = jq::kq_gemm_i8<F, NW_, NG, true, NSPLIT_>;                                                        \
@@ -2152,16 +2160,18 @@ int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, 
             rc_once = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);       \
         });                                                                                                           \
         attr_rc = rc_once;                                                                                            \
+        const jq::QiGrouped gp{wptr, m->gexp, m->yrow, NSPLIT_ && m->gtile_rgs == 0 ? moe_gemm_tables_small(m) : t};   \
+        const size_t max_mt = NSPLIT_ ? max_small : max_big;                                                          \
         if (attr_rc == hipSuccess)                                                                                    \
             hipLaunchKernelGGL(kern, dim3((unsigned)(tx * max_mt)), dim3(64 * NW_), lds, s, (const uint8_t *)nullptr, \
                                row_bytes, (const uint8_t *)m->gacts, Y, 0, n, (int)nb, 0, (int)tx, 0, (int)nb,       \
                                (size_t)0, gp);                                                                        \
     } while (0)
-    if (m->gtile_rgs == 2) JQ_MOE_GEMM(2, true);
-    else JQ_MOE_GEMM(4, false);
+    if (m->gtile_rgs != 2) JQ_MOE_GEMM(4, false);
+    if (m->gtile_rgs != 8 && attr_rc == hipSuccess) JQ_MOE_GEMM(2, true);
 #undef JQ_MOE_GEMM
     HIP_TRY(attr_rc);
-    note_kernel(m->gtile_rgs == 2 ? "moe_gemm_i8_few" : "moe_gemm_i8");
+    note_kernel(m->gtile_rgs == 2 ? "moe_gemm_i8_few" : m->gtile_rgs == 0 ? "moe_gemm_i8_mixed" : "moe_gemm_i8");
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -2169,9 +2179,13 @@ int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, 
 // The tile plan of a bucketed call: few pairs an expert (32 on average or fewer) -> tiles of two row groups whose
 // waves share the weight rows; more -> tiles of eight row groups whose waves share the rows.
 void moe_gemm_plan(jq_moe *m, int groups, size_t pairs, hipStream_t s) {
-    static const char *env = getenv("JQ_MOE_GEMM_TILE_ROWS");  // 32 or 128: the tile for every call
-    m->gtile_rgs = env ? (atoi(env) == 32 ? 2 : 8) : (pairs <= 32 * (size_t)groups ? 2 : 8);
-    hipLaunchKernelGGL(jq::moe_gemm_i8_plan, dim3(1), dim3(256), 0, s, m->offsets, groups, m->gtile_rgs, moe_gemm_tables(m));
+    // Few pairs an expert on average (under 8): every tile two row groups.  More: the mixed plan, since the pairs of a
+    // call are seldom spread evenly (a prompt of one repeated token sends all its pairs to eight experts) and the
+    // host does not know how they fell: eight row groups a tile where an expert has them, two for the rest.
+    static const char *env = getenv("JQ_MOE_GEMM_TILE_ROWS");  // 32 or 128: that tile for every call; 0: the mixed plan
+    m->gtile_rgs = env ? (atoi(env) == 32 ? 2 : atoi(env) == 128 ? 8 : 0) : (pairs < 8 * (size_t)groups ? 2 : 0);
+    hipLaunchKernelGGL(jq::moe_gemm_i8_plan, dim3(1), dim3(256), 0, s, m->offsets, groups, m->gtile_rgs, moe_gemm_tables(m),
+                       moe_gemm_tables_small(m));
 }
 
 int dispatch_moe_gemm_i8(jq_moe *m, uint32_t type, const uint8_t *const *wptr, size_t row_bytes, int base_align,

@@ -159,11 +159,57 @@ __global__ __launch_bounds__(256) void q4k_gemm_i8_prep(const float *__restrict_
 //   counts[0], counts[1]    row groups and tiles in all
 // for at most max_rg row groups and max_mt tiles (callers size them as pairs / 16 + groups and
 // pairs / (16 tile_rgs) + groups, which always suffice).
+// tile_rgs = 0, the mixed plan: an expert's row groups go eight to a tile while five or more are left (mt_*, counts[1]
+// of them, at most row groups / 5) and the rest two to a tile (`small`'s mt_*, counts[2] of them, at most two an expert),
+// for two launches: tiles whose waves share the rows where an expert has many pairs, tiles whose waves share the weight
+// rows for the tails and for experts with few.  `small.counts` is counts + 1, so that either launch finds its tile count
+// at counts[1].
 struct QiGroupTables {
     int *rg_pair, *rg_cnt, *mt_group, *mt_rg0, *mt_nrg, *counts;
 };
 __global__ __launch_bounds__(256) void moe_gemm_i8_plan(const int *__restrict__ offsets, int groups, int tile_rgs,
-                                                         QiGroupTables t) {
+                                                         QiGroupTables t, QiGroupTables small = QiGroupTables{}) {
+    if (tile_rgs == 0) {
+        __shared__ int base[3][257], run[3];
+        if (threadIdx.x == 0) run[0] = run[1] = run[2] = 0;
+        __syncthreads();
+        for (int g0 = 0; g0 < groups; g0 += 256) {
+            const int g = g0 + (int)threadIdx.x;
+            const int cnt = g < groups ? offsets[g + 1] - offsets[g] : 0;
+            const int nrg = (cnt + 15) >> 4;
+            const int nbig = nrg / 8 + (nrg % 8 >= 5 ? 1 : 0), rest = max(nrg - 8 * nbig, 0), nsmall = (rest + 1) / 2;
+            base[0][threadIdx.x] = nrg, base[1][threadIdx.x] = nbig, base[2][threadIdx.x] = nsmall;
+            __syncthreads();
+            if (threadIdx.x < 3) {
+                int a = run[threadIdx.x];
+                for (int i = 0; i < 256; i++) {
+                    const int x = base[threadIdx.x][i];
+                    base[threadIdx.x][i] = a;
+                    a += x;
+                }
+                run[threadIdx.x] = a;
+            }
+            __syncthreads();
+            if (g < groups) {
+                const int first = offsets[g], rg0 = base[0][threadIdx.x];
+                for (int r = 0; r < nrg; r++) {
+                    t.rg_pair[rg0 + r] = first + 16 * r;
+                    t.rg_cnt[rg0 + r] = min(16, cnt - 16 * r);
+                }
+                for (int q = 0; q < nbig; q++) {
+                    const int at = base[1][threadIdx.x] + q;
+                    t.mt_group[at] = g, t.mt_rg0[at] = rg0 + 8 * q, t.mt_nrg[at] = min(8, nrg - 8 * q);
+                }
+                for (int q = 0; q < nsmall; q++) {
+                    const int at = base[2][threadIdx.x] + q;
+                    small.mt_group[at] = g, small.mt_rg0[at] = rg0 + 8 * nbig + 2 * q, small.mt_nrg[at] = min(2, rest - 2 * q);
+                }
+            }
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) t.counts[0] = run[0], t.counts[1] = run[1], t.counts[2] = run[2];
+        return;
+    }
     __shared__ int rg_base[257], mt_base[257];
     // serial prefix over the groups in chunks of 256 (a few hundred groups at most)
     __shared__ int carry[2];

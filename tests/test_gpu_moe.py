@@ -255,23 +255,23 @@ def test_few_tokens_an_expert_take_the_int8_quads_kernel(tokens):
 
 
 @pytest.mark.parametrize("qtype,h,inter,E,k,tokens,shared_inter,kw,kernel", [
-    (capi.Q4_K, 5120, 256, 8, 2, 40, 0, {}, "moe_gemm_i8_few"),      # rows too long for the Q4_K grouped kernels
+    (capi.Q4_K, 5120, 256, 8, 2, 40, 0, {}, "moe_gemm_i8_mixed"),    # rows too long for the Q4_K grouped kernels
     (capi.IQ2_XXS, 1024, 512, 8, 2, 70, 512, dict(gating="sigmoid", swiglu_clamp=0.02, swiglu_clamp_shared=0.01),
-     "moe_gemm_i8_few"),                                             # the shared expert's 70 pairs: three tiles of 32
-    (capi.MXFP4, 512, 768, 16, 4, 33, 0, {}, "moe_gemm_i8_few"),
-    (capi.Q6_K, 768, 256, 4, 2, 300, 0, {}, "moe_gemm_i8"),          # about 150 pairs an expert: two tiles of 128
-    (capi.Q2_K, 512, 256, 4, 2, 300, 0, dict(swiglu_clamp=0.02), "moe_gemm_i8"),
-    (capi.Q8_0, 256, 512, 16, 4, 64, 512, dict(gating="sigmoid", weights_scale=2.5), "moe_gemm_i8_few"),
-    (capi.MXFP4, 256, 256, 160, 6, 150, 0, {}, "moe_gemm_i8_few"),   # more experts than one pass of the tile plan
-    (capi.IQ2_XXS, 512, 512, 4, 2, 200, 0, {}, "moe_gemm_i8"),
-    (capi.Q4_K, 512, 256, 4, 2, 300, 256, dict(gating="sigmoid"), "moe_gemm_i8"),  # 48 pairs an expert or more: ahead of the ring kernel
+     "moe_gemm_i8_mixed"),                                           # the shared expert's 70 pairs: one tile of 128
+    (capi.MXFP4, 512, 768, 16, 4, 33, 0, {}, "moe_gemm_i8_mixed"),
+    (capi.Q6_K, 768, 256, 4, 2, 300, 0, {}, "moe_gemm_i8_mixed"),    # about 150 pairs an expert: a tile of 128 and one of 32
+    (capi.Q2_K, 512, 256, 4, 2, 300, 0, dict(swiglu_clamp=0.02), "moe_gemm_i8_mixed"),
+    (capi.Q8_0, 256, 512, 16, 4, 64, 512, dict(gating="sigmoid", weights_scale=2.5), "moe_gemm_i8_mixed"),
+    (capi.MXFP4, 256, 256, 160, 6, 150, 0, {}, "moe_gemm_i8_few"),   # more experts than one pass of the tile plan; under 8 pairs an expert
+    (capi.IQ2_XXS, 512, 512, 4, 2, 200, 0, {}, "moe_gemm_i8_mixed"),
+    (capi.Q4_K, 512, 256, 4, 2, 300, 256, dict(gating="sigmoid"), "moe_gemm_i8_mixed"),  # 16 pairs an expert or more: ahead of the ring kernel
 ])
 def test_many_tokens_take_the_grouped_int8_gemm(qtype, h, inter, E, k, tokens, shared_inter, kw, kernel):
     """Bucketed calls of the formats with a side of the int8 GEMM: pairs sorted by expert are laid out in row
     groups of 16 that never mix two experts, gate and up run from one preparation of the tokens, the activation
-    is applied in place (with the shared expert's own clamp on its rows) and the down projection reads it.  Up
-    to 32 pairs an expert on average: tiles of 32 rows whose waves share the weight rows; more: tiles of 128
-    rows whose waves share the rows."""
+    is applied in place (with the shared expert's own clamp on its rows) and the down projection reads it.  Under 8
+    pairs an expert on average: tiles of 32 rows whose waves share the weight rows; more: an expert's pairs in tiles of
+    128 rows whose waves share the rows while 80 or more are left, the rest in tiles of 32 (two launches)."""
     ora, dev = build(qtype, h, inter, E, k, 150 + h, shared_inter=shared_inter, **kw)
     x = synth.normal(151 + tokens, (tokens, h))
     want = ora.forward(x)
@@ -281,6 +281,27 @@ def test_many_tokens_take_the_grouped_int8_gemm(qtype, h, inter, E, k, tokens, s
     assert np.array_equal(got, dev.forward(x))
     few = synth.normal(152, (3, h))                                   # then a decode-sized call on the same layer
     assert close(dev.forward(few), ora.forward(few))
+
+
+@pytest.mark.parametrize("qtype", [capi.Q4_K, capi.MXFP4])
+def test_grouped_int8_gemm_with_pairs_that_fall_unevenly(qtype):
+    """260 of 300 tokens route alike: two experts get 260 pairs and more (two tiles of 128 and a tail of tiles of 32),
+    the others a few each (tiles of 32 only), and experts without a pair get no tile."""
+    ora, dev = build(qtype, 2048, 256, 16, 2, 171)
+    x = 0.5 * synth.normal(172, (300, 2048))      # (the magnitude a normed layer gives: the GEMM's fixed point holds 1e-3 there)
+    # a token whose second and third expert are well apart, so that its near-copies pick the same two
+    logits = x[:40] @ ora.router_w.T
+    top3 = np.sort(logits, axis=1)[:, -3:]
+    x0 = x[int(np.argmax(top3[:, 1] - top3[:, 0]))].copy()
+    x[:260] = x0 + 0.01 * x[:260]
+    ids, _ = dev.route(x)
+    assert np.array_equal(np.sort(ids, axis=1), np.sort(ora.route(x)[0], axis=1))
+    counts = np.bincount(ids.reshape(-1), minlength=16)
+    assert counts.max() >= 260 and counts.min() < 16
+    got = dev.forward(x)
+    assert capi.last_kernel() == "moe_gemm_i8_mixed"
+    assert close(got, ora.forward(x))
+    assert np.array_equal(got, dev.forward(x))
 
 
 @pytest.mark.parametrize("qtype,h,inter,E,k,tokens,shared_inter,kw", [
