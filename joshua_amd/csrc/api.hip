@@ -485,6 +485,37 @@ int dispatch_i8_gemv(uint32_t type, const uint8_t *W, size_t row_bytes, const fl
     }
 }
 
+// Q6_K, Q8_0 and Q5_K, one activation row, rows of 2048 columns, 64 weight rows or more: a tile of 16 rows a workgroup of
+// 8 waves on the int8 matrix cores (the output head of a 2048-wide model, 151936 rows of Q6_K).  Returns -1 when the
+// shape is outside its reach (then the f32 row kernel runs).
+template <class F>
+int launch_gemv_tile8(const char *name, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t n, hipStream_t s) {
+    if (row_bytes != (size_t)8 * F::BLOCK) return -1;
+    auto kern = jq::gemv_mfma_tile<F, 8, false>;
+    constexpr int lds = jq::gemv_mfma_tile_lds<F, 8>();
+    static const hipError_t attr_rc = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    HIP_TRY(attr_rc);
+    note_kernel(name);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((n + 15) / 16)), dim3(512), lds, s, W, X, Y, (int)n, nullptr, nullptr, 0.0f, nullptr,
+                       nullptr);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int dispatch_gemv_tile8(uint32_t type, const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n,
+                        hipStream_t s) {
+    static const char *off = getenv("JQ_Q4K_GEMV_TILE");
+    if ((off && off[0] == '0') || k != 2048 || n < 64 || n > 0x7FFFFFF0ull || (((uintptr_t)W | (uintptr_t)X) & 15) != 0 ||
+        row_bytes % 16 != 0)
+        return -1;
+    switch (type) {
+    case JQ_TYPE_Q6_K: return launch_gemv_tile8<jq::QvQ6K>("q6k_gemv_mfma_tile", W, row_bytes, X, Y, n, s);
+    case JQ_TYPE_Q8_0: return launch_gemv_tile8<jq::QvI8<jq::Q8_0>>("q8_0_gemv_mfma_tile", W, row_bytes, X, Y, n, s);
+    case JQ_TYPE_Q5_K: return launch_gemv_tile8<jq::QvI8<jq::Q5_K>>("q5k_gemv_mfma_tile", W, row_bytes, X, Y, n, s);
+    default: return -1;
+    }
+}
+
 // Q6_K, one activation row, rows of 4096, 8192 or 12288: the v_dot4 LDS-ring kernel.
 // Returns -1 when the shape is outside its reach.
 int dispatch_q6k_dot4(const uint8_t *W, size_t row_bytes, const float *X, float *Y, size_t k, size_t n, hipStream_t s) {
@@ -1055,7 +1086,9 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
         if (rc >= 0) return rc;
     }
     if (m == 1) {
-        const int rc = dispatch_i8_gemv(type, W, row_bytes, X, Y, k, n, s);
+        int rc = dispatch_gemv_tile8(type, W, row_bytes, X, Y, k, n, s);
+        if (rc >= 0) return rc;
+        rc = dispatch_i8_gemv(type, W, row_bytes, X, Y, k, n, s);
         if (rc >= 0) return rc;
     }
     // Q6_K and Q8_0 with two or three activation rows against a matrix of 16M weights or more: the one-row kernel

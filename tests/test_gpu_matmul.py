@@ -1134,6 +1134,22 @@ def test_q4k_mfma_gemv_over_rows_of_2048(n):
     assert close(got, oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
 
 
+@pytest.mark.parametrize("qtype,kernel", [(capi.Q6_K, "q6k_gemv_mfma_tile"), (capi.Q8_0, "q8_0_gemv_mfma_tile"),
+                                          (capi.Q5_K, "q5k_gemv_mfma_tile")])
+@pytest.mark.parametrize("n", [64, 512 + 7, 16 * 700 + 3])
+def test_other_formats_one_row_over_rows_of_2048(qtype, kernel, n):
+    """The same kernel over the Q6_K, Q8_0 and Q5_K policies (the attn_v and the output head of a 2048-wide model)."""
+    k = 2048
+    blocks = synth.random_blocks(qtype, 510 + n % 89, n * k) if qtype == capi.Q5_K else make_blocks(qtype, n, k, 510 + n % 89)
+    lhs = synth.normal(511, (1, k))
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    got = w.matmul_t(1, lhs)
+    assert capi.last_kernel() == kernel
+    assert close(got, oracle.matmul_t(qtype, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+    lhs[0, 1234] = np.nan
+    assert np.all(np.isnan(w.matmul_t(1, lhs)))
+
+
 def test_q4k_mfma_gemv_over_rows_of_2048_integer_sums_and_odd_activations():
     n, k = 1024 + 48, 2048
     blocks, q, x = q4k_integer_case(n, k, 19, group=32, big_value=32639, small=4000)
