@@ -2178,15 +2178,19 @@ int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, 
     if (!prepared)
         hipLaunchKernelGGL((jq::moe_gemm_i8_prep<F::SUB16>), dim3((unsigned)nb, (unsigned)max_rg), dim3(256), 0, s, X, xsel, t, k,
                            m->gacts);
-    constexpr int lds = jq::qi_lds_bytes<F, NG>();
     hipError_t attr_rc = hipSuccess;
+    // (the tiles of few rows on one operand buffer: four workgroups a compute unit instead of two.  JQ_MOE_GEMM_DOUBLE_BUFFER
+    // keeps the two buffers)
+    static const char *double_env = getenv("JQ_MOE_GEMM_DOUBLE_BUFFER");
     // most tiles a plan can hold: every tile of the mixed plan's first list has five row groups or more, its second
     // list at most two tiles an expert
     const size_t n_groups = m->cfg.n_expert + (m->fold_shared ? 1 : 0);
     const size_t max_big = m->gtile_rgs == 0 ? max_rg / 5 + 1 : max_rg, max_small = m->gtile_rgs == 0 ? 2 * n_groups : max_rg;
-#define JQ_MOE_GEMM(NW_, NSPLIT_)                                                                                     \
+#define JQ_MOE_GEMM(NW_, NSPLIT_) JQ_MOE_GEMM_(NW_, NSPLIT_, false)
+#define JQ_MOE_GEMM_(NW_, NSPLIT_, SINGLE_)                                                                           \
     do {                                                                                                              \
-        auto kern = jq::kq_gemm_i8<F, NW_, NG, true, NSPLIT_>;                                                        \
+        auto kern = jq::kq_gemm_i8<F, NW_, NG, true, NSPLIT_, SINGLE_>;                                               \
+        constexpr int lds = jq::qi_lds_bytes<F, NG, SINGLE_>();                                                       \
         static std::once_flag big_lds;                                                                                \
         static hipError_t rc_once = hipSuccess;                                                                       \
         std::call_once(big_lds, [&] {                                                                                 \
@@ -2201,8 +2205,12 @@ int launch_moe_gemm_i8(jq_moe *m, const uint8_t *const *wptr, size_t row_bytes, 
                                (size_t)0, gp);                                                                        \
     } while (0)
     if (m->gtile_rgs != 2) JQ_MOE_GEMM(4, false);
-    if (m->gtile_rgs != 8 && attr_rc == hipSuccess) JQ_MOE_GEMM(2, true);
+    if (m->gtile_rgs != 8 && attr_rc == hipSuccess) {
+        if (double_env) JQ_MOE_GEMM(2, true);
+        else JQ_MOE_GEMM_(2, true, true);
+    }
 #undef JQ_MOE_GEMM
+#undef JQ_MOE_GEMM_
     HIP_TRY(attr_rc);
     note_kernel(m->gtile_rgs == 2 ? "moe_gemm_i8_few" : m->gtile_rgs == 0 ? "moe_gemm_i8_mixed" : "moe_gemm_i8");
     HIP_TRY(hipGetLastError());
@@ -2315,7 +2323,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     int groups, max_group;
     // Decode-sized (one group a pair, every pair reading its expert's rows) or bucketed by expert (every expert hit
     // read once)?  A pair costs about a = 0.10 + 0.17 bytes-per-weight ns a weight on the integer-dot kernels;
-    // a bucketed expert costs g = 0.45 ns a weight on the grouped int8 GEMM (bound by the unpacking; 0.36 for Q4_K)
+    // a bucketed expert costs g = 0.30 ns a weight on the grouped int8 GEMM (bound by the unpacking; 0.36 for Q4_K)
     // and 0.28 on the Q4_K kernels for short rows.  With d(P) = E (1 - (1 - 1/E)^P) experts hit by P pairs, pairs win
     // while P a <= d(P) g (Qwen3-30B-A3B sizes: up to ~100 pairs over 128 experts).  Formats without integer-dot
     // kernels keep pairs up to the number of experts.
@@ -2343,7 +2351,7 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
         const bool short_q4k = m->gate->type == JQ_TYPE_Q4_K && c.hidden <= 2048 && c.inter <= 2048;
         // (Q4_K unpacks for less: a 256-token call of DeepSeek-V3-sized Q4_K experts, 3.8 ms, is 0.34 an expert)
         // (long rows: a = 0.07 + 0.17 bytes-per-weight; DeepSeek-V3 sizes, 8 tokens: 4.9 us a pair of IQ2_XXS, 6.7 of MXFP4)
-        const double a = (short_q4k ? 0.10 : 0.07) + 0.17 * bpw, g = short_q4k ? 0.28 : m->gate->type == JQ_TYPE_Q4_K ? 0.36 : 0.45;
+        const double a = (short_q4k ? 0.10 : 0.07) + 0.17 * bpw, g = short_q4k ? 0.28 : m->gate->type == JQ_TYPE_Q4_K ? 0.36 : 0.30;
         const double hit = (double)c.n_expert * (1.0 - std::pow(1.0 - 1.0 / (double)c.n_expert, (double)P));
         const double by_pairs = (double)P * a, by_gemm = hit * g;
         double by_expert = INFINITY;
@@ -2511,12 +2519,14 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
                                              (size_t)P + extra * T, m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out,
                                              (int)c.inter, (int)c.hidden, groups, s);
     if (rc > 0) return 1;
-    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && few)
+    // (where gate and up ran on the grouped GEMM, their rows being too long for the Q4_K kernels for short rows, so does
+    // the down projection: those kernels walk an expert's 7168 rows at DeepSeek-V3 sizes, 7.7 ms a call of 256 tokens)
+    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && few && !planned)
         rc = dispatch_moe_q4k_quads<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                            m->qi8, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                            (int)c.hidden, groups, s);
     if (rc > 0) return 1;
-    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && !prefer_gemm)
+    if (rc < 0 && fused_act && max_group > 1 && m->down->type == JQ_TYPE_Q4_K && !prefer_gemm && !planned)
         rc = dispatch_moe_q4k_ring<false>(m->pdown, nullptr, m->down->row_bytes, d16, m->G, (size_t)P + extra * T,
                                           m->qacts, m->gexp, m->offsets, m->yrow, m->yrow, m->out, (int)c.inter,
                                           (int)c.hidden, groups, s);

@@ -278,8 +278,8 @@ __global__ __launch_bounds__(256) void moe_gemm_i8_prep(const float *__restrict_
 // last 16.  With eight sub-blocks (48 bytes): m_0..7 as halves, 1024 m_0..7 as halves; with sixteen (80
 // bytes): m_0..7, m_8..15, 1024 m_0..7, 1024 m_8..15.
 constexpr int QI_TILE = 4 * 2 * 64 * 16;
-template <class F, int NG>
-constexpr int qi_lds_bytes() { return 2 * (NG * QI_TILE + 16 * NG * F::META) + F::TABLE; }
+template <class F, int NG, bool SINGLE = false>
+constexpr int qi_lds_bytes() { return (SINGLE ? 1 : 2) * (NG * QI_TILE + 16 * NG * F::META) + F::TABLE; }
 
 typedef short qi_s2 __attribute__((ext_vector_type(2)));
 
@@ -922,7 +922,10 @@ struct QiGrouped {
 // the waves share the weight-row groups instead of the activation rows: wave w takes groups w NG / NW ..
 // of them against both row groups, so that every wave has matrix work whatever the row count (with the rows
 // split, a tile of one row group leaves all waves but one only the unpacking).
-template <class F, int NW, int NG, bool GROUPED = false, bool NSPLIT = false>
+// SINGLE: one operand buffer instead of two.  A super-block is unpacked as a whole, then multiplied, with a barrier
+// after either; half the LDS lets twice the workgroups share a compute unit, and while one unpacks the others
+// multiply (for the tiles of few rows, whose two waves a workgroup leave the unpacking's lookups nothing to hide behind).
+template <class F, int NW, int NG, bool GROUPED = false, bool NSPLIT = false, bool SINGLE = false>
 __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict__ W, size_t row_bytes,
                                                       const uint8_t *__restrict__ acts, float *__restrict__ Y,
                                                       int m_rows, int n, int nb, int groups, int tx, int ty,
@@ -933,7 +936,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
     constexpr int MT = NSPLIT ? 32 : 32 * NW;   // activation rows a tile
     static_assert(!NSPLIT || (NG % NW == 0 && NGW >= 2), "two weight-row groups a wave or more");
     extern __shared__ __attribute__((aligned(16))) uint8_t qi_lds[];
-    const uint8_t *tab = qi_lds + 2 * BUF;  // the format's lookup table, behind the two buffers
+    const uint8_t *tab = qi_lds + (SINGLE ? 1 : 2) * BUF;  // the format's lookup table, behind the buffers
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
     int bx, by;
     int rg0 = 0, nrg = 0;  // GROUPED: the tile's first row group and how many it has
@@ -1000,7 +1003,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
 
     fetch_part(0, 0), fetch_part(0, 1), fetch_part(0, 2);
     if constexpr (F::TABLE > 0) {  // every workgroup that got this far: no wave has left
-        F::stage(qi_lds + 2 * BUF);
+        F::stage(qi_lds + (SINGLE ? 1 : 2) * BUF);
         __syncthreads();
     }
     take_header();
@@ -1029,8 +1032,17 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
     __syncthreads();
 
     for (int b = 0; b < nb; b++) {
-        const uint8_t *buf = qi_lds + (b & 1) * BUF;
+        const uint8_t *buf = qi_lds + (SINGLE ? 0 : (b & 1) * BUF);
         const int b_next = min(b + 1, nb - 1), b_next2 = min(b + 2, nb - 1);
+        if (SINGLE && b > 0) {
+            // (every wave is through with super-block b - 1: the barrier that ended its iteration)
+            take_header();
+#pragma unroll
+            for (int j = 0; j < 8; j++) unpack_piece(qi_lds, j);
+            unpack_meta(qi_lds);
+            fetch_part(b_next, 0), fetch_part(b_next, 1), fetch_part(b_next, 2);
+            __syncthreads();
+        }
 #pragma unroll
         for (int mg = 0; mg < 2; mg++) {
             // scales and I2 operand of this row group: wanted in the last quarter
@@ -1077,7 +1089,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                 const bool first_of_pass = s < 4 * T0 ? s % T0 == 0 : (s - 4 * T0) % (NGW - T0) == 0;
                 const bool last_of_pass = s < 4 * T0 ? s % T0 == T0 - 1 : (s - 4 * T0) % (NGW - T0) == NGW - T0 - 1;
                 const int pass = s < 4 * T0 ? c : 4 + c;  // 0..7 within the half
-                if (first_of_pass) {
+                if (!SINGLE && first_of_pass) {
                     // An eighth of the next super-block's weights becomes operands in every pass, thinly spread
                     // among the MFMAs (its bytes were asked for half an iteration or more ago); the registers of
                     // a part are refilled with the super-block after that as soon as the part is used up.
@@ -1110,7 +1122,7 @@ __global__ __launch_bounds__(64 * NW) void kq_gemm_i8(const uint8_t *__restrict_
                 __builtin_amdgcn_sched_barrier(0);
             }
             finish(NGW - 1);
-            if (mg == 1) fetch_part(b_next2, 2);
+            if (!SINGLE && mg == 1) fetch_part(b_next2, 2);
             __builtin_amdgcn_sched_barrier(0);
         }
         // every wave is done with the buffer the next super-block went into: it was read one iteration ago, in
