@@ -1108,6 +1108,15 @@ int dispatch_matmul(uint32_t type, const uint8_t *W, size_t row_bytes, const flo
     // rows on the int8 GEMV further down; from three on the streaming kernel, whose time hardly depends on
     // the row count, or, against a very long matrix (a vocabulary projection), the LDS-ring kernel, whose
     // second launch only pays off from some 100 us of streaming on.
+    // (two rows against 2048 to 8192 weight rows of 4096 columns: the one-row kernel twice, 7.6 us at 4096 rows against
+    // the 16-row kernel's 9.6 with its preparation launch; from 14336 rows on the two are level and the 16-row kernel
+    // reads the matrix once)
+    if (type == JQ_TYPE_Q4_K && m == 2 && k == 4096 && n >= 2048 && n <= 8192) {
+        static const char *no_loop = getenv("JQ_NO_ONE_ROW_LOOP");
+        int rc = no_loop ? -1 : dispatch_q4k_dot4(W, row_bytes, X, Y, k, n, s);
+        if (rc == 0) rc = dispatch_q4k_dot4(W, row_bytes, X + k, Y + n, k, n, s);
+        if (rc >= 0) return rc;
+    }
     if (type == JQ_TYPE_Q4_K && m >= 2) {
         const int rc = dispatch_q4k_rows16(W, row_bytes, X, Y, m, k, n, s);
         if (rc >= 0) return rc;

@@ -1005,6 +1005,17 @@ def test_q4k_mfma_gemv_row_counts(n):
     assert close(got, oracle.matmul_t(capi.Q4_K, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
 
 
+def test_two_rows_against_a_mid_sized_matrix_run_the_one_row_kernel_twice():
+    n, k = 4096 + 21, 4096
+    blocks = make_blocks(capi.Q4_K, n, k, 305)
+    lhs = synth.normal(306, (2, k))
+    w = capi.Weight.upload(capi.Q4_K, blocks, n, k)
+    got = w.matmul_t(2, lhs)
+    assert capi.last_kernel() == "q4k_gemv_mfma_lds"
+    assert close(got, oracle.matmul_t(capi.Q4_K, (2, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+    assert np.array_equal(got[1], w.matmul_t(1, lhs[1:])[0])
+
+
 def test_q4k_mfma_gemv_integer_dot_products_are_bit_exact():
     """Activation range 32639 per 32-element sub-block, as in the v_dot4 kernel: the sums of the low-nibble
     sub-blocks come straight from the matrix cores, those of the high-nibble sub-blocks as
@@ -1080,6 +1091,8 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 1, 7168, 1536, "q4k_gemv_mfma_cols"),        # DeepSeek-V3's query down-projection
     (capi.Q4_K, 1, 16384, 7168, "q4k_gemv_mfma_cols"),       # its attention output projection
     (capi.Q4_K, 2, 2048, 768, "q4k_gemv_mfma"),
+    (capi.Q4_K, 2, 4096, 4096, "q4k_gemv_mfma_lds"),         # two rows against a mid-sized matrix: the one-row kernel twice
+    (capi.Q4_K, 2, 4096, 14336, "q4k_rows16_lds"),
     (capi.Q4_K, 16, 4096, 14336, "q4k_rows16_lds"),
     (capi.Q4_K, 16, 2048, 768, "q4k_stream_mfma"),
     (capi.Q4_K, 512, 4096, 14336, "q4k_gemm_i8"),           # 256 tiles of 256 x 112
