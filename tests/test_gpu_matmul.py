@@ -1100,9 +1100,11 @@ KERNEL_OF_SHAPE = [  # which kernel serves the shapes the benchmarks quote: (for
     (capi.Q4_K, 128, 4096, 4096, "q4k_gemm_i8+splitk"),     # 64 tiles of 128 x 64: split over k
     (capi.Q4_K, 512, 4096, 1024, "q4k_gemm_i8+splitk"),
     (capi.Q4_K, 128, 4096, 256, "q4k_gemm_mfma+splitk"),    # a small product: the f16 kernel
-    (capi.Q8_0, 1, 4096, 4096, "q8_0_gemv_dot4_lds"),
+    (capi.Q8_0, 1, 4096, 4096, "q8_0_gemv_mfma_tile"),       # one tile of 16 rows a compute unit
+    (capi.Q8_0, 1, 4096, 8192, "q8_0_gemv_dot4_lds"),
     (capi.Q6_K, 1, 12288, 4096, "q6k_gemv_mfma_cols"),      # a feed-forward down projection
-    (capi.Q6_K, 1, 4096, 4096, "q6k_gemv_dot4_lds"),
+    (capi.Q6_K, 1, 4096, 4096, "q6k_gemv_mfma_tile"),
+    (capi.Q6_K, 1, 4096, 8192, "q6k_gemv_dot4_lds"),
     (capi.Q6_K, 1, 1024, 4096, "matmul_rows_staged"),
     (capi.Q6_K, 64, 4096, 1024, "q6k_gemm_i8+splitk"),
     (capi.Q6_K, 64, 2048, 256, "gemm_decoded_mfma+splitk"), # a small product: weights decoded in the workgroup
@@ -1160,6 +1162,22 @@ def test_other_formats_one_row_over_rows_of_2048(qtype, kernel, n):
     assert capi.last_kernel() == kernel
     assert close(got, oracle.matmul_t(qtype, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
     lhs[0, 1234] = np.nan
+    assert np.all(np.isnan(w.matmul_t(1, lhs)))
+
+
+@pytest.mark.parametrize("qtype,kernel,n", [(capi.Q8_0, "q8_0_gemv_mfma_tile", 256), (capi.Q8_0, "q8_0_gemv_mfma_tile", 2048 + 7),
+                                            (capi.Q8_0, "q8_0_gemv_mfma_tile", 4096), (capi.Q6_K, "q6k_gemv_mfma_tile", 2048),
+                                            (capi.Q6_K, "q6k_gemv_mfma_tile", 4096 - 9)])
+def test_q8_0_and_q6k_one_row_against_up_to_4096_rows_of_4096(qtype, kernel, n):
+    """At most one tile of 16 rows a compute unit: 16 waves a tile, the whole matrix asked for at once."""
+    k = 4096
+    blocks = make_blocks(qtype, n, k, 520 + n % 89)
+    lhs = synth.normal(521, (1, k))
+    w = capi.Weight.upload(qtype, blocks, n, k)
+    got = w.matmul_t(1, lhs)
+    assert capi.last_kernel() == kernel
+    assert close(got, oracle.matmul_t(qtype, (1, k, n), lhs, blocks, avx2=oracle.have_avx2()))
+    lhs[0, 3000] = np.inf
     assert np.all(np.isnan(w.matmul_t(1, lhs)))
 
 
