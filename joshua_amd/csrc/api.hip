@@ -1770,18 +1770,23 @@ int dispatch_moe_q4k_ring(const uint8_t *const *Wa, const uint8_t *const *Wb, si
 
 // Q4_K experts with a few tokens per group (four on average at batch 64 over 128 experts): the int8 kernel
 // that multiplies four activation rows an MFMA.  Returns -1 when the shape is outside its reach.
+bool moe_q4k_quads_takes(const jq::ActsI8 &xq, size_t row_bytes, int base_align, const float *X, int k) {
+    const int nb = k / 256;
+    static const char *off = getenv("JQ_MOE_NO_QUADS");
+    return !(off || !xq.xl || k % 256 != 0 || nb < 2 || nb > 16 || row_bytes != (size_t)nb * 144 || base_align < 16 ||
+             ((uintptr_t)X & 15) != 0);
+}
+
 template <bool DUAL>
 int dispatch_moe_q4k_quads(const uint8_t *const *Wa, const uint8_t *const *Wb, size_t row_bytes, int base_align,
                            const float *X, size_t x_rows, jq::ActsI8 xq, const int *gexp, const int *offsets,
                            const int *xsel, const int *yrow, float *Y, int k, int n, int groups, hipStream_t s,
-                           const jq::MoeClamp &cl = jq::MoeClamp{}) {
+                           const jq::MoeClamp &cl = jq::MoeClamp{}, bool planes_ready = false) {
     const int nb = k / 256;
-    static const char *off = getenv("JQ_MOE_NO_QUADS");
-    if (off || !xq.xl || k % 256 != 0 || nb < 2 || nb > 16 || row_bytes != (size_t)nb * 144 || base_align < 16 ||
-        ((uintptr_t)X & 15) != 0)
-        return -1;
+    if (!moe_q4k_quads_takes(xq, row_bytes, base_align, X, k)) return -1;
     const size_t words = x_rows * (size_t)(k / 4);
-    hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
+    if (!planes_ready)  // (else the router launch left X as planes in xq)
+        hipLaunchKernelGGL(jq::acts_i8_prep, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, X, x_rows, k, xq);
     const int maxnb = nb > 8 ? 16 : nb > 4 ? 8 : 4, n_tiles = (n + 15) / 16;
     // 2048 workgroups a launch (measured at 128 groups of 768 x 2048: 8 a group 184 us a layer call, 16: 173,
     // 24: 177, 48: 202; the f16 ring kernel: 204 at 8 and more above)
@@ -2321,11 +2326,12 @@ int moe_route_dev(jq_moe *m, size_t T, const float *x, hipStream_t s, jq::MoePai
                            (int)c.hidden, (int)c.n_expert);
     else if (T >= tile_from && !no_tile)  // many tokens: a token's activations read once per eight experts (the same bits)
         hipLaunchKernelGGL(jq::moe_router_logits_tile, dim3((c.n_expert + 7) / 8, (unsigned)((T + 7) / 8)), dim3(256), 0, s,
-                           m->router_w, x, m->logits, (int)T, (int)c.hidden, (int)c.n_expert);
+                           m->router_w, x, m->logits, (int)T, (int)c.hidden, (int)c.n_expert,
+                           c.hidden % 32 == 0 ? planes : jq::ActsI8{nullptr, nullptr, nullptr, nullptr});
     else
         hipLaunchKernelGGL(jq::moe_router_logits, dim3(c.n_expert, token_runs), dim3(256), 0, s, m->router_w, x, m->logits,
                            (int)T, (int)c.hidden, (int)c.n_expert, planes);
-    if (planes_made) *planes_made = !pre && planes.xl && !(T >= tile_from && !no_tile);
+    if (planes_made) *planes_made = !pre && planes.xl && (c.hidden % 32 == 0 || !(T >= tile_from && !no_tile));
     size_t sm = (2 * c.n_expert + std::max<uint32_t>(c.n_group, 1) + c.n_expert_used + 4) * sizeof(float);
     if (gate_later) {
         if (wave_gate) {
@@ -2441,7 +2447,20 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
             hipLaunchKernelGGL(jq::rmsnorm_rows, dim3((unsigned)T), dim3(1024), 0, s, (float *)pre->a.x, pre->a.res, pre->a.w,
                                pre->a.eps, pre->a.hn_out, (int)c.hidden);
         }
-        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{nullptr, nullptr, nullptr, nullptr, 0})) return 1;
+        // few pairs an expert of Q4_K with short rows: gate and up will run on the kernel that takes four rows an MFMA,
+        // which reads x as fixed-point planes; the router launch leaves them behind
+        jq::ActsI8 planes{nullptr, nullptr, nullptr, nullptr};
+        {
+            const jq_weight *ws[4] = {m->gate, m->up, m->fold_shared ? m->sgate : nullptr, m->fold_shared ? m->sup : nullptr};
+            uintptr_t bits = 0;
+            for (const jq_weight *w : ws) bits |= w ? ((uintptr_t)w->dev | (uintptr_t)w->row_bytes) : 0;
+            static const char *no_router_planes = getenv("JQ_MOE_NO_ROUTER_PLANES");
+            if (!no_router_planes && !expert_dot8 && m->gate->type == JQ_TYPE_Q4_K && m->up->type == JQ_TYPE_Q4_K &&
+                m->gate->row_bytes == m->up->row_bytes && (size_t)P <= 6 * (size_t)c.n_expert &&
+                moe_q4k_quads_takes(m->qi8, m->gate->row_bytes, (bits & 15) ? 4 : 16, x, (int)c.hidden))
+                planes = m->qi8;
+        }
+        if (moe_route_dev(m, T, x, s, jq::MoePairGroups{nullptr, nullptr, nullptr, nullptr, 0}, planes, &planes_ready)) return 1;
         groups = (int)c.n_expert + extra;
         max_group = (int)T;
         const int in_lds = (size_t)P <= 12288;
@@ -2500,7 +2519,8 @@ int moe_forward_dev(jq_moe *m, size_t T, const float *x, float *y, hipStream_t s
     if (rc > 0) return 1;
     if (rc < 0 && same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K && few)
         rc = dispatch_moe_q4k_quads<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qi8, m->gexp, m->offsets,
-                                          m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp);
+                                          m->xrow, m->yrow, m->G, (int)c.hidden, (int)c.inter, groups, s, clamp,
+                                          max_group > 1 && planes_ready);
     if (rc > 0) return 1;
     if (rc < 0 && same_gu && max_group > 1 && m->gate->type == JQ_TYPE_Q4_K && !prefer_gemm)
         rc = dispatch_moe_q4k_ring<true>(m->pgate, m->pup, m->gate->row_bytes, a16, x, T, m->qacts, m->gexp, m->offsets,

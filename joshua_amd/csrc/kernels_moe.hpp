@@ -149,11 +149,22 @@ __global__ __launch_bounds__(256) void moe_router_logits_norm(const float *__res
 // once per eight experts instead of once per expert (512 tokens x 256 experts of 7168: 228 -> 60 us).  Every
 // logit is accumulated by the same thread over the same columns in the same order as in moe_router_logits and
 // reduced the same way, so the two kernels give the same bits.
+// With `planes` (h a multiple of 32) the launch also leaves the tokens' activations as fixed-point planes for the expert
+// kernels behind it: the workgroups of a token tile share its 8 h / 32 blocks, eight lanes a block.
 __global__ __launch_bounds__(256) void moe_router_logits_tile(const float *__restrict__ Wr, const float *__restrict__ X,
-                                                               float *__restrict__ logits, int T, int h, int E) {
+                                                               float *__restrict__ logits, int T, int h, int E,
+                                                               ActsI8 planes = ActsI8{nullptr, nullptr, nullptr, nullptr}) {
     __shared__ float red[4][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int e0 = 8 * (int)blockIdx.x, t0 = 8 * (int)blockIdx.y;
+    if (planes.xl) {
+        const int bpt = h / 32, units = 8 * bpt;  // blocks a token, blocks of the tile
+        for (int u = 32 * (int)blockIdx.x + ((int)threadIdx.x >> 3); u < units; u += 32 * (int)gridDim.x) {
+            const int t = t0 + u / bpt, b = u % bpt;
+            // (the eight lanes of a block stay together: u depends on threadIdx.x >> 3 only)
+            if (t < T) acts_i8_quantize(X, (size_t)t * (size_t)(h / 4) + 8 * b + (threadIdx.x & 7), planes);
+        }
+    }
     float acc[8][8];
 #pragma unroll
     for (int i = 0; i < 8; i++)
