@@ -41,12 +41,15 @@ CALIB_BIN = os.path.join(HERE, "calib", "copy_kernel")
 
 PROBE_SRC = os.path.join(HERE, "calib", "read_probe.hip")
 PROBE_BIN = os.path.join(HERE, "calib", "read_probe")
+MIX_SRC = os.path.join(HERE, "calib", "gemm_mix_probe.hip")
+MIX_BIN = os.path.join(HERE, "calib", "gemm_mix_probe")
 
 
 def build_calibration() -> str:
-    """The copy kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters, and the plain-read probe that gives
-    the floor of one launch over a matrix of the benchmark's size."""
-    for src, out in ((CALIB_SRC, CALIB_BIN), (PROBE_SRC, PROBE_BIN)):
+    """The copy kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters, the plain-read probe that gives
+    the floor of one launch over a matrix of the benchmark's size, and the probe that runs the int8 GEMM's
+    instruction mix of a super-block iteration with nothing else around it."""
+    for src, out in ((CALIB_SRC, CALIB_BIN), (PROBE_SRC, PROBE_BIN), (MIX_SRC, MIX_BIN)):
         res = subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-o", out, src], capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"hipcc failed:\n{res.stderr}")
