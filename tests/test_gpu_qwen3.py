@@ -103,6 +103,21 @@ def test_single_token_steps_with_attn_v_of_another_format_in_the_qk_launch():
         pos += 1
 
 
+def test_single_token_steps_over_one_to_eighteen_key_chunks():
+    """32 heads of 128, four KV heads: single-token steps whose split attention covers one, two, three, five and
+    eighteen chunks of 64 keys, between prefill chunks of 61 to 830 tokens."""
+    cfg = dict(CFG, n_layer=2, hidden=512, n_head=32, n_kv_head=4, head_dim=128, ffn=512, vocab=512, n_ctx=1120)
+    m, o = make(cfg, 41, "q4_k")
+    rng = np.random.default_rng(17)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], size=1110)]
+    pos = 0
+    for step in (1, 1, 61, 1, 1, 1, 64, 1, 130, 1, 1, 830, 1, 1):   # single-token steps at 1, 2, 64..66, 131, 262, 1093.. cached tokens
+        chunk = toks[pos:pos + step]
+        ok, e = close(m.forward(chunk, pos), o.forward(chunk, pos))
+        assert ok, f"pos {pos} +{step}: {e}"
+        pos += step
+
+
 def test_paired_gate_up_rows_serve_prefill_and_replacement():
     """With 4096-wide Q4_K rows the gate and up matrices are stored with alternating rows (the
     single-token launch applies SwiGLU itself); multi-token steps read them as strided views, and a
